@@ -1,0 +1,230 @@
+"""ctypes binding of the CPU oracle (``libloken_oracle.so``). TEST INFRASTRUCTURE ONLY.
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may
+import this package, and only as the checker; the shipped ``loken_amd`` package never does.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+_HERE = Path(__file__).resolve().parent
+_LIB_PATH = _HERE / "libloken_oracle.so"
+
+Q8_0, Q8_1, Q4_K, Q6_K, Q8_K = 8, 9, 12, 14, 15
+BLOCK_LEN = {Q8_0: 32, Q8_1: 32, Q4_K: 256, Q6_K: 256, Q8_K: 256}
+BLOCK_BYTES = {Q8_0: 34, Q8_1: 36, Q4_K: 144, Q6_K: 210, Q8_K: 292}
+
+
+def build(force: bool = False) -> Path:
+    """Compile the oracle with the Makefile beside it (gcc only)."""
+    if force:
+        subprocess.run(["make", "-C", str(_HERE), "clean"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", str(_HERE)], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            build()
+        _lib = C.CDLL(str(_LIB_PATH))
+        _declare(_lib)
+    return _lib
+
+
+_sz, _i, _vp = C.c_size_t, C.c_int, C.c_void_p
+
+
+def _declare(l: C.CDLL) -> None:
+    l.lko_f16_to_f32.restype = C.c_float
+    l.lko_f16_to_f32.argtypes = [C.c_uint16]
+    l.lko_f32_to_f16.restype = C.c_uint16
+    l.lko_f32_to_f16.argtypes = [C.c_float]
+    l.lko_unpack_scales_mins.argtypes = [_vp, _vp, _vp]
+    l.lko_pack_scales_mins.argtypes = [_vp, _vp, _vp]
+    l.lko_dequantize.argtypes = [_i, _vp, _sz, _vp]
+    for name in ("lko_quantize_q8_0", "lko_quantize_q8_1", "lko_quantize_q8_k"):
+        getattr(l, name).argtypes = [_vp, _sz, _vp]
+        getattr(l, name).restype = None
+    l.oa_matmul.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _sz, _vp]
+    l.oa_matmul_fast.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _i]
+    l.oa_matmul_exact.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp]
+    l.ob_subdots.argtypes = [_i, _sz, _sz, _vp, _vp, _vp, _vp]
+    l.ob_matmul_q8_1.argtypes = [_i, _sz, _sz, _sz, _vp, _sz, _vp, _vp]
+    l.ob_matmul.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp]
+    l.ob_matmul_f64.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp]
+    l.lko_topk_softmax.argtypes = [_vp, _sz, _sz, _sz, _i, _vp, _vp]
+    l.lko_topk_softmax.restype = None
+    l.lko_group_by_expert.argtypes = [_vp, _sz, _vp, _vp]
+    l.lko_group_by_expert.restype = None
+    l.lko_moe_forward.argtypes = [_i, _i, _i, _sz, _sz, _sz, _sz, _sz] + [_vp] * 8
+    l.lko_cpu_has_avx2.restype = _i
+
+
+def _p(a: np.ndarray) -> int:
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data
+
+
+def _u8(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.uint8).reshape(-1)
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def f16_to_f32(h: int) -> float:
+    return float(lib().lko_f16_to_f32(int(h)))
+
+
+def f32_to_f16(f: float) -> int:
+    return int(lib().lko_f32_to_f16(float(f)))
+
+
+def unpack_scales_mins(packed12) -> tuple[np.ndarray, np.ndarray]:
+    p = _u8(packed12)
+    sc, mn = np.zeros(8, np.uint8), np.zeros(8, np.uint8)
+    lib().lko_unpack_scales_mins(_p(p), _p(sc), _p(mn))
+    return sc, mn
+
+
+def pack_scales_mins(scales, mins) -> np.ndarray:
+    sc, mn = _u8(scales), _u8(mins)
+    out = np.zeros(12, np.uint8)
+    lib().lko_pack_scales_mins(_p(sc), _p(mn), _p(out))
+    return out
+
+
+def dequantize(dtype: int, blocks) -> np.ndarray:
+    b = _u8(blocks)
+    n_blocks = b.size // BLOCK_BYTES[dtype]
+    out = np.empty(n_blocks * BLOCK_LEN[dtype], np.float32)
+    rc = lib().lko_dequantize(dtype, _p(b), n_blocks, _p(out))
+    if rc:
+        raise ValueError(f"dequantize: dtype {dtype} not handled")
+    return out
+
+
+def _quantize(fn: str, dtype: int, x) -> np.ndarray:
+    x = _f32(x).reshape(-1)
+    assert x.size % BLOCK_LEN[dtype] == 0
+    out = np.zeros(x.size // BLOCK_LEN[dtype] * BLOCK_BYTES[dtype], np.uint8)
+    getattr(lib(), fn)(_p(x), x.size, _p(out))
+    return out
+
+
+def quantize_q8_0(x) -> np.ndarray:
+    return _quantize("lko_quantize_q8_0", Q8_0, x)
+
+
+def quantize_q8_1(x) -> np.ndarray:
+    return _quantize("lko_quantize_q8_1", Q8_1, x)
+
+
+def quantize_q8_k(x) -> np.ndarray:
+    return _quantize("lko_quantize_q8_k", Q8_K, x)
+
+
+class OracleError(ValueError):
+    pass
+
+
+_ERR = {-1: "k is not a multiple of the block size", -2: "rhs byte length is wrong",
+        -3: "dtype not handled"}
+
+
+def _check(rc: int) -> None:
+    if rc:
+        raise OracleError(_ERR.get(rc, f"oracle error {rc}"))
+
+
+def oa_matmul(dtype: int, lhs, rhs, n: int, *, fast_threads: int = 0, exact: bool = False) -> np.ndarray:
+    lhs = _f32(lhs)
+    m, k = lhs.shape
+    rhs = _u8(rhs)
+    dst = np.empty((m, n), np.float32)
+    if exact:
+        _check(lib().oa_matmul_exact(dtype, m, k, n, _p(lhs), _p(rhs), _p(dst)))
+    elif fast_threads > 0:
+        _check(lib().oa_matmul_fast(dtype, m, k, n, _p(lhs), _p(rhs), rhs.size, _p(dst), fast_threads))
+    else:
+        _check(lib().oa_matmul(dtype, m, k, n, _p(lhs), _p(rhs), rhs.size, _p(dst)))
+    return dst
+
+
+def ob_matmul(dtype: int, lhs, rhs, n: int) -> np.ndarray:
+    lhs = _f32(lhs)
+    m, k = lhs.shape
+    rhs = _u8(rhs)
+    dst = np.empty((m, n), np.float32)
+    _check(lib().ob_matmul(dtype, m, k, n, _p(lhs), _p(rhs), _p(dst)))
+    return dst
+
+
+def ob_matmul_q8_1(dtype: int, act_q8_1, m: int, k: int, rhs, n: int, stride_blocks: int | None = None) -> np.ndarray:
+    act = _u8(act_q8_1)
+    rhs = _u8(rhs)
+    dst = np.empty((m, n), np.float32)
+    _check(lib().ob_matmul_q8_1(dtype, m, k, n, _p(act), stride_blocks or k // 32, _p(rhs), _p(dst)))
+    return dst
+
+
+def ob_matmul_f64(dtype: int, lhs, rhs, n: int) -> np.ndarray:
+    lhs = _f32(lhs)
+    m, k = lhs.shape
+    rhs = _u8(rhs)
+    dst = np.empty((m, n), np.float64)
+    _check(lib().ob_matmul_f64(dtype, m, k, n, _p(lhs), _p(rhs), _p(dst)))
+    return dst
+
+
+def ob_subdots(dtype: int, k: int, n: int, rhs, act_q8_1) -> tuple[np.ndarray, np.ndarray]:
+    """(dots[n, k/32 or k/16], sums[k/32]) of weight rows against one Q8_1 activation row."""
+    rhs, act = _u8(rhs), _u8(act_q8_1)
+    per = 16 if dtype == Q6_K else 32
+    dots = np.empty((n, k // per), np.int32)
+    sums = np.empty(k // 32, np.int32)
+    _check(lib().ob_subdots(dtype, k, n, _p(rhs), _p(act), _p(dots), _p(sums)))
+    return dots, sums
+
+
+def topk_softmax(logits, topk: int, renorm: bool = True) -> tuple[np.ndarray, np.ndarray]:
+    logits = _f32(logits)
+    t, e = logits.shape
+    ids = np.empty((t, topk), np.int32)
+    w = np.empty((t, topk), np.float32)
+    lib().lko_topk_softmax(_p(logits), t, e, topk, int(renorm), _p(ids), _p(w))
+    return ids, w
+
+
+def group_by_expert(ids) -> tuple[np.ndarray, np.ndarray]:
+    ids = np.ascontiguousarray(ids, np.int32).reshape(-1)
+    slots = np.empty(ids.size, np.int32)
+    experts = np.empty(ids.size, np.int32)
+    lib().lko_group_by_expert(_p(ids), ids.size, _p(slots), _p(experts))
+    return slots, experts
+
+
+def moe_forward(family: int, dt_gu: int, dt_down: int, x, gate, up, down, ids, weights,
+                n_experts: int, ffn: int, want_h: bool = False):
+    x = _f32(x)
+    tokens, hidden = x.shape
+    ids = np.ascontiguousarray(ids, np.int32)
+    topk = ids.shape[1]
+    weights = _f32(weights)
+    gate, up, down = _u8(gate), _u8(up), _u8(down)
+    out = np.empty((tokens, hidden), np.float32)
+    h = np.empty((tokens * topk, ffn), np.float32) if want_h else None
+    _check(lib().lko_moe_forward(family, dt_gu, dt_down, tokens, hidden, ffn, n_experts, topk,
+                                 _p(x), _p(gate), _p(up), _p(down), _p(ids), _p(weights),
+                                 _p(h) if want_h else None, _p(out)))
+    return (out, h) if want_h else out

@@ -1,0 +1,123 @@
+/*
+ * CPU oracle for the GGUF block-quantized matmul path. TEST INFRASTRUCTURE ONLY.
+ *
+ * A plain-C restatement of loken's CPU quantized-matmul path (Rust, under
+ * src/tensor/quant_cpu and src/inference/moe_cuda_cpu of the reference). Nothing in the
+ * shipped library links, loads or calls this file: only the test-suite, the smoke check and
+ * the CPU-baseline leg of the benchmark do, and there only as the checker.
+ *
+ * Two families of entry points:
+ *   oa_*  "as served": K-quant weights against Q8_K activations (256 values, f32 scale,
+ *         bsums), Q8_0 weights against Q8_0 activations. This is what loken's CPU backend
+ *         runs (format/q4_k.rs:62-88, q6_k.rs:51-82, q8_0.rs:83-97, drivers.rs:2108-2142).
+ *   ob_*  "same codes": the activation is quantized by loken's BlockQ8_1::quantize
+ *         (format/q8_1.rs:46-61), the integer sub-block dots are the inner `dot` of
+ *         q4_k.rs:138-153 / q6_k.rs:137-160 / q8_0.rs:88-95 taken per Q8_1 block, and the f32
+ *         combine is the one a Q8_1-activation kernel performs (cuda/moe/gguf.cuh:664-685,
+ *         782-816, 486-495). The GPU kernels are compared bit-for-bit on the integers and to
+ *         1e-3 relative / 1e-4 absolute on the f32 outputs against this family.
+ *
+ * Pinned by (see tests/test_oracle_*.py): ggml's own QUANT/DEQUANT records for q4_K, q6_K,
+ * q8_0, q8_K (scripts/oracle/vectors.txt) and ggml-written blocks with their decoded rows
+ * (tests/vectors/ggml_encode.json) for layouts, f16 conversion and dequantizers; exhaustive
+ * pack/unpack round-trip for the 6-bit scales; closed forms for the three activation
+ * quantizers; numpy int64 brute force for every integer sum; an f64 dot over dequantized
+ * values and the reduction to a plain int8 GEMV for the f32 combines; decomposition into
+ * single-matrix calls for the MoE routines; a textbook softmax/top-k for the router.
+ */
+#ifndef LOKEN_ORACLE_H
+#define LOKEN_ORACLE_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml type ids, src/tensor/quantized/dtype.rs:66-96 */
+enum { LKO_Q8_0 = 8, LKO_Q8_1 = 9, LKO_Q4_K = 12, LKO_Q6_K = 14, LKO_Q8_K = 15 };
+
+#define LKO_QK_K 256
+#define LKO_Q4K_BYTES 144
+#define LKO_Q6K_BYTES 210
+#define LKO_Q80_BYTES 34
+#define LKO_Q81_BYTES 36
+#define LKO_Q8K_BYTES 292
+
+/* ---- scalar helpers ---- */
+float    lko_f16_to_f32(uint16_t h);
+uint16_t lko_f32_to_f16(float f);            /* IEEE round-to-nearest-even, as the `half` crate */
+int      lko_block_len(int dtype);           /* values per block, 0 if not handled */
+int      lko_block_bytes(int dtype);         /* bytes per block, 0 if not handled */
+
+/* blocks.rs:145-158 / 167-179 */
+void lko_unpack_scales_mins(const uint8_t packed[12], uint8_t scales[8], uint8_t mins[8]);
+void lko_pack_scales_mins(const uint8_t scales[8], const uint8_t mins[8], uint8_t packed[12]);
+
+/* ---- dequantizers (pin the layouts) ---- */
+int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out);
+
+/* ---- activation quantizers ---- */
+void lko_quantize_q8_0(const float* x, size_t n, uint8_t* out);   /* q8_0.rs:51-67 */
+void lko_quantize_q8_1(const float* x, size_t n, uint8_t* out);   /* q8_1.rs:46-61 */
+void lko_quantize_q8_k(const float* x, size_t n, uint8_t* out);   /* q8_k.rs:96-119 */
+
+/* ---- O-A: the served CPU path ---- */
+/* dst[m,n] = lhs[m,k] (f32) x rhs[n, k/blk] blocks. Returns 0, or a negative code with the
+ * reference's error conditions (drivers.rs:2122-2139): -1 k not a multiple of the block,
+ * -2 rhs byte length wrong, -3 dtype not handled. */
+int oa_matmul(int dtype, size_t m, size_t k, size_t n, const float* lhs,
+              const uint8_t* rhs, size_t rhs_bytes, float* dst);
+/* The exact-fold variant, dot_exact (q4_k.rs:117-131, q6_k.rs:121-134): integer block sums,
+ * `combine`, shares added in block order from -0.0. K-quants only. */
+int oa_matmul_exact(int dtype, size_t m, size_t k, size_t n, const float* lhs,
+                    const uint8_t* rhs, float* dst);
+
+/* ---- O-B: same-codes path ---- */
+/* Integer sub-block dots of one weight row set against ONE Q8_1 activation row.
+ *   Q4_K: dots[n][k/32] = sum_32 nibble*q8 ; sums[k/32] = sum_32 q8 (weight independent)
+ *   Q6_K: dots[n][k/16] = sum_16 (code-32)*q8
+ *   Q8_0: dots[n][k/32] = sum_32 q*q8
+ * `act_q8_1` is k/32 Q8_1 blocks. `sums` may be NULL. */
+int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t* act_q8_1,
+               int32_t* dots, int32_t* sums);
+/* dst[m,n] from Q8_1 activation rows (m rows of k/32 blocks, row stride `act_stride_blocks`). */
+int ob_matmul_q8_1(int dtype, size_t m, size_t k, size_t n, const uint8_t* act_q8_1,
+                   size_t act_stride_blocks, const uint8_t* rhs, float* dst);
+/* Same, quantizing lhs[m,k] f32 first with lko_quantize_q8_1. */
+int ob_matmul(int dtype, size_t m, size_t k, size_t n, const float* lhs,
+              const uint8_t* rhs, float* dst);
+/* f64 evaluation of the same-codes product: sum over dequantized weight x dequantized Q8_1. */
+int ob_matmul_f64(int dtype, size_t m, size_t k, size_t n, const float* lhs,
+                  const uint8_t* rhs, double* dst);
+
+/* ---- router and MoE ---- */
+/* softmax -> top-k by value descending (ties: lower index first) -> optional renormalize.
+ * moe_cuda_cpu/mod.rs:2098-2113. ids[t,topk], weights[t,topk]. */
+void lko_topk_softmax(const float* logits, size_t tokens, size_t n_experts, size_t topk,
+                      int renorm, int32_t* ids, float* weights);
+/* Stable sort of the flattened (token, choice) slots by expert id:
+ * sorted_slots[i], sorted_experts[i] (generic_transformer/moe_weights.rs:27-54,102-116). */
+void lko_group_by_expert(const int32_t* ids, size_t pairs, int32_t* sorted_slots,
+                         int32_t* sorted_experts);
+/* Whole expert block, host semantics of fused_gate_up_silu_cpu + fused_down_reduce_cpu
+ * (moe_cuda_cpu/mod.rs:459-605, 1478-1660): x[tokens,hidden] -> out[tokens,hidden].
+ * gate/up: [experts, ffn, hidden/blk], down: [experts, hidden, ffn/blk]; `family` 0 = O-A
+ * activations (Q8_K / Q8_0), 1 = O-B (Q8_1). SiLU is u*(g/(1+exp(-g))); the fold adds
+ * tw[slot]*dot into the token row in expert-run order. `h_sorted` (pairs x ffn, sorted order)
+ * may be NULL. */
+int lko_moe_forward(int family, int dtype_gate_up, int dtype_down, size_t tokens, size_t hidden,
+                    size_t ffn, size_t n_experts, size_t topk, const float* x,
+                    const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+                    const int32_t* ids, const float* weights, float* h_sorted, float* out);
+
+/* ---- timed CPU baseline (cpu_baseline.c): O-A semantics, AVX2 kernels, worker pool ---- */
+int lko_cpu_has_avx2(void);
+int oa_matmul_fast(int dtype, size_t m, size_t k, size_t n, const float* lhs,
+                   const uint8_t* rhs, size_t rhs_bytes, float* dst, int threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,220 @@
+"""Pins the oracle's integer sums and f32 combines without retyping its formulas.
+
+  * integer sub-block dots: numpy int64 brute force over nibbles/codes decoded by an
+    independent numpy decoder (itself checked against ggml's DEQUANT in this file);
+  * f32 outputs: an f64 sum over dequantized weights x dequantized activations (the bound the
+    reference uses, src/tensor/quantized/tests.rs:576-632) and the special case sc=1, m=0, d=1
+    where the Q4_K product is a plain int8 GEMV;
+  * the threaded AVX2 baseline against the scalar path at the reference's vector-vs-scalar bound
+    (src/tensor/quant_cpu/avx/parity.rs:50-56).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from loken_amd import synth
+
+DT = {"q4_k": oracle.Q4_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0}
+
+
+# ---- independent numpy decoders: integer codes and float scales per value ----
+def np_codes_q4k(w):
+    """w [n, nb, 144] -> codes [n, nb*256] (0..15), sc [n, nb*8], mn [n, nb*8], d, dmin [n, nb]."""
+    n, nb, _ = w.shape
+    qs = w[:, :, 16:].reshape(n, nb, 4, 32)
+    codes = np.stack([qs & 0xF, qs >> 4], axis=3).reshape(n, nb * 256).astype(np.int64)
+    p = w[:, :, 4:16].astype(np.int64)
+    sc = np.empty((n, nb, 8), np.int64)
+    mn = np.empty((n, nb, 8), np.int64)
+    sc[..., :4] = p[..., 0:4] & 63
+    mn[..., :4] = p[..., 4:8] & 63
+    sc[..., 4:] = (p[..., 8:12] & 0xF) | ((p[..., 0:4] >> 6) << 4)
+    mn[..., 4:] = (p[..., 8:12] >> 4) | ((p[..., 4:8] >> 6) << 4)
+    d = w[:, :, 0:2].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+    dmin = w[:, :, 2:4].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+    return codes, sc.reshape(n, nb * 8), mn.reshape(n, nb * 8), d, dmin
+
+
+def np_codes_q6k(w):
+    n, nb, _ = w.shape
+    ql = w[:, :, 0:128].reshape(n, nb, 2, 2, 32).astype(np.int64)      # [half][span][l]
+    qh = w[:, :, 128:192].reshape(n, nb, 2, 32).astype(np.int64)       # [half][l]
+    codes = np.empty((n, nb, 2, 4, 32), np.int64)
+    for g in range(4):
+        low = (ql[:, :, :, g % 2, :] >> (0 if g < 2 else 4)) & 0xF
+        high = (qh >> (2 * g)) & 3
+        codes[:, :, :, g, :] = (low | (high << 4)) - 32
+    sc = w[:, :, 192:208].copy().view(np.int8).reshape(n, nb * 16).astype(np.int64)
+    d = w[:, :, 208:210].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+    return codes.reshape(n, nb * 256), sc, d
+
+
+def np_codes_q80(w):
+    n, nb, _ = w.shape
+    codes = w[:, :, 2:].copy().view(np.int8).reshape(n, nb * 32).astype(np.int64)
+    d = w[:, :, 0:2].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+    return codes, d
+
+
+def np_q81(act_bytes):
+    b = act_bytes.reshape(-1, 36)
+    d = b[:, 0:2].copy().view(np.float16).reshape(-1).astype(np.float64)
+    q = b[:, 4:].copy().view(np.int8).astype(np.int64)
+    return d, q
+
+
+def np_dequant(dtype, w):
+    n = w.shape[0]
+    if dtype == oracle.Q4_K:
+        codes, sc, mn, d, dmin = np_codes_q4k(w)
+        scale = np.repeat(sc * np.repeat(d, 8, axis=1), 32, axis=1)
+        off = np.repeat(mn * np.repeat(dmin, 8, axis=1), 32, axis=1)
+        return scale * codes - off
+    if dtype == oracle.Q6_K:
+        codes, sc, d = np_codes_q6k(w)
+        return np.repeat(sc * np.repeat(d, 16, axis=1), 16, axis=1) * codes
+    codes, d = np_codes_q80(w)
+    return np.repeat(d, 32, axis=1) * codes
+
+
+def test_numpy_decoders_agree_with_ggml(ggml_vectors):
+    for name, dtype in (("q4_K", oracle.Q4_K), ("q6_K", oracle.Q6_K), ("q8_0", oracle.Q8_0)):
+        rec = ggml_vectors[name]
+        w = rec["quant"].reshape(1, -1, rec["block_bytes"])
+        got = np_dequant(dtype, w).reshape(-1)
+        np.testing.assert_allclose(got, rec["dequant"].astype(np.float64), rtol=2e-7, atol=0)
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+def test_integer_subdots_match_numpy_brute_force(name):
+    dtype = DT[name]
+    n, k = 16, 1024
+    w = synth.weight(dtype, n, k, seed=11, stream=1)
+    x = synth.activation(1, k, seed=11)
+    act = oracle.quantize_q8_1(x)
+    dots, sums = oracle.ob_subdots(dtype, k, n, w, act)
+    _, q = np_q81(act)
+    q = q.reshape(-1)
+    assert sums.tolist() == q.reshape(-1, 32).sum(axis=1).tolist()
+    if dtype == oracle.Q4_K:
+        codes = np_codes_q4k(w)[0]
+        want = (codes * q[None, :]).reshape(n, k // 32, 32).sum(axis=2)
+    elif dtype == oracle.Q6_K:
+        codes = np_codes_q6k(w)[0]
+        want = (codes * q[None, :]).reshape(n, k // 16, 16).sum(axis=2)
+    else:
+        codes = np_codes_q80(w)[0]
+        want = (codes * q[None, :]).reshape(n, k // 32, 32).sum(axis=2)
+    assert dots.astype(np.int64).tolist() == want.tolist()
+
+
+def test_q4k_extreme_subdot_value():
+    # all-15 nibbles against all-127 activations: 15 * 127 * 32 = 60960 per sub-block
+    w = np.zeros((1, 1, 144), np.uint8)
+    w[..., 16:] = 0xFF
+    x = np.full((1, 256), 127.0, np.float32)
+    dots, sums = oracle.ob_subdots(oracle.Q4_K, 256, 1, w, oracle.quantize_q8_1(x))
+    assert dots.tolist() == [[60960] * 8] and sums.tolist() == [127 * 32] * 8
+
+
+def test_q4k_reduces_to_int8_gemv_when_scales_are_one():
+    # sc = 1, m = 0, d = 1, activations on the exact grid with d8 = 1: out = nibbles @ codes
+    rng = np.random.default_rng(12)
+    n, k = 8, 512
+    w = synth.weight(oracle.Q4_K, n, k, seed=12)
+    w[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    w[:, :, 2:4] = 0
+    w[:, :, 4:16] = oracle.pack_scales_mins([1] * 8, [0] * 8)
+    a = rng.integers(-127, 128, (2, k))
+    a[:, ::32] = 127
+    x = a.astype(np.float32)
+    want = a @ np_codes_q4k(w)[0].T
+    got_b = oracle.ob_matmul(oracle.Q4_K, x, w, n)
+    assert got_b.astype(np.int64).tolist() == want.tolist()
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+@pytest.mark.parametrize("m", [1, 4])
+def test_same_codes_f32_is_the_f64_product_up_to_rounding(name, m):
+    dtype = DT[name]
+    n, k = 24, 2048
+    w = synth.weight(dtype, n, k, seed=13, stream=2)
+    x = synth.activation(m, k, seed=13)
+    got = oracle.ob_matmul(dtype, x, w, n)
+    ref = oracle.ob_matmul_f64(dtype, x, w, n)
+    # independent f64: numpy decoders on both operands
+    d8, q8 = np_q81(oracle.quantize_q8_1(x))
+    xa = (q8 * d8[:, None]).reshape(m, k)
+    ref_np = xa @ np_dequant(dtype, w).T
+    np.testing.assert_allclose(ref, ref_np, rtol=1e-12, atol=1e-15)
+    # f32 accumulation over k/32 terms: error far below the 1e-3 parity tolerance
+    absdot = np.abs(xa) @ np.abs(np_dequant(dtype, w)).T
+    assert (np.abs(got - ref) <= 2e-6 * absdot + 1e-9).all()
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+@pytest.mark.parametrize("m", [1, 4])
+def test_served_path_matches_f64_over_dequantized_weights(name, m):
+    # the reference's own matmul-level check and tolerance (quantized/tests.rs:576-632)
+    dtype = DT[name]
+    n, k = 16, 1024
+    w = synth.weight(dtype, n, k, seed=14, stream=3)
+    x = synth.activation(m, k, seed=14)
+    got = oracle.oa_matmul(dtype, x, w, n)
+    wd = np_dequant(dtype, w)
+    ref = x.astype(np.float64) @ wd.T
+    bound = 5e-3 * (np.abs(x.astype(np.float64)) @ np.abs(wd).T) + 1e-3
+    assert (np.abs(got - ref) <= bound).all()
+    # and it is the exact-fold variant up to f32 summation order
+    if dtype != oracle.Q8_0:
+        ex = oracle.oa_matmul(dtype, x, w, n, exact=True)
+        assert (np.abs(ex - got) <= 1e-3 * np.maximum(np.abs(got), 1.0)).all()
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+def test_served_path_integer_core_with_q8k_codes(name):
+    # f64 product of dequantized weights with dequantized O-A activations: pins the Q8_K / Q8_0
+    # pairing and the bsums use, independent of the oracle's loops.
+    dtype = DT[name]
+    n, k = 8, 768
+    w = synth.weight(dtype, n, k, seed=15, stream=4)
+    x = synth.activation(2, k, seed=15)
+    if dtype == oracle.Q8_0:
+        xa = oracle.dequantize(oracle.Q8_0, oracle.quantize_q8_0(x)).reshape(2, k)
+    else:
+        xa = oracle.dequantize(oracle.Q8_K, oracle.quantize_q8_k(x)).reshape(2, k)
+    wd = np_dequant(dtype, w)
+    ref = xa.astype(np.float64) @ wd.T
+    got = oracle.oa_matmul(dtype, x, w, n)
+    absdot = np.abs(xa.astype(np.float64)) @ np.abs(wd).T
+    assert (np.abs(got - ref) <= 4e-6 * absdot + 1e-9).all()
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+@pytest.mark.parametrize("m,threads", [(1, 1), (1, 3), (5, 4), (9, 2)])
+def test_threaded_avx2_baseline_matches_scalar_path(name, m, threads):
+    dtype = DT[name]
+    n, k = 100, 1024
+    w = synth.weight(dtype, n, k, seed=16, stream=5)
+    x = synth.activation(m, k, seed=16)
+    slow = oracle.oa_matmul(dtype, x, w, n)
+    fast = oracle.oa_matmul(dtype, x, w, n, fast_threads=threads)
+    assert (np.abs(fast - slow) <= 1e-3 * np.maximum(np.abs(slow), 1.0)).all()
+
+
+def test_driver_error_conditions():
+    w = synth.weight(oracle.Q4_K, 4, 512, seed=1)
+    x = np.zeros((1, 500), np.float32)
+    with pytest.raises(oracle.OracleError, match="multiple of the block"):
+        oracle.oa_matmul(oracle.Q4_K, x, w, 4)
+    with pytest.raises(oracle.OracleError, match="byte length"):
+        oracle.oa_matmul(oracle.Q4_K, np.zeros((1, 512), np.float32), w, 5)
+    with pytest.raises(oracle.OracleError, match="not handled"):
+        oracle.oa_matmul(3, np.zeros((1, 512), np.float32), w, 4)
+
+
+def test_empty_rows_and_columns():
+    w = synth.weight(oracle.Q4_K, 4, 256, seed=1)
+    assert oracle.ob_matmul(oracle.Q4_K, np.zeros((0, 256), np.float32), w, 4).shape == (0, 4)
+    assert oracle.oa_matmul(oracle.Q4_K, np.zeros((0, 256), np.float32), w, 4).shape == (0, 4)
+    assert oracle.ob_matmul(oracle.Q4_K, np.zeros((2, 256), np.float32), w[:0], 0).shape == (2, 0)
