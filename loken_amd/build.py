@@ -1,0 +1,51 @@
+"""Builds ``libloken_gfx950.so`` in-tree with hipcc for gfx950 (cross-compiles without a GPU)."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+CSRC = HERE / "csrc"
+LIB = HERE / "libloken_gfx950.so"
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fno-fast-math",
+    # packed-FP32 instructions stay off: the compiler forms them from plain float code otherwise
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
+]
+
+
+def sources() -> list[Path]:
+    return sorted(CSRC.glob("*.hip"))
+
+
+def _compile(src: Path) -> Path:
+    obj = CSRC / (src.stem + ".o")
+    cmd = [HIPCC, *FLAGS, "-c", str(src), "-o", str(obj)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src.name}:\n{r.stderr[-6000:]}")
+    return obj
+
+
+def build(jobs: int = 8, verbose: bool = False) -> Path:
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(srcs)))) as pool:
+        objs = list(pool.map(_compile, srcs))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr[-6000:]}")
+    if verbose:
+        print(f"built {LIB} from {len(srcs)} sources")
+    return LIB
+
+
+if __name__ == "__main__":
+    build(verbose=True)
+    sys.exit(0)

@@ -1,0 +1,86 @@
+// Shared device helpers for the gfx950 quantized-matmul kernels. wave64 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#include "../../include/loken_gfx950.h"
+
+#define LK_WAVE 64
+
+// GGUF block geometry (src/tensor/quantized/dtype.rs:66-96 of the reference).
+#define Q4K_BYTES 144
+#define Q6K_BYTES 210
+#define Q80_BYTES 34
+#define Q81_BYTES 36
+
+// 16-byte loads from blocks that are only 2-byte aligned (Q6_K 210 B, Q8_0 34 B): global memory
+// on gfx950 serves unaligned dwordx4, the type only tells the compiler not to assume more.
+typedef uint4 __attribute__((aligned(2))) uint4_a2;
+typedef uint4 __attribute__((aligned(4))) uint4_a4;
+typedef uint32_t __attribute__((aligned(2))) uint32_a2;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+static __device__ __forceinline__ int dot4(int a, int b, int c) {
+    return __builtin_amdgcn_sdot4(a, b, c, false);
+}
+
+static __device__ __forceinline__ int dot16(const uint4& w, const uint4& a, int c) {
+    c = dot4((int)w.x, (int)a.x, c);
+    c = dot4((int)w.y, (int)a.y, c);
+    c = dot4((int)w.z, (int)a.z, c);
+    return dot4((int)w.w, (int)a.w, c);
+}
+
+static __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
+    return __half2float(__ushort_as_half((unsigned short)h));
+}
+
+template <int ctrl>
+static __device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xF, 0xF, true));
+}
+
+// Sum over the 64 lanes of a wave; every lane returns the total.
+static __device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);  // row_half_mirror
+    v += dpp_f32<0x140>(v);  // row_mirror
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+static __device__ __forceinline__ int wave_sum_i32(int v) {
+    for (int o = 1; o < 64; o <<= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// Output element conversion.
+template <typename T> static __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half from_f32<__half>(float v) { return __float2half_rn(v); }
+template <> __device__ __forceinline__ __hip_bfloat16 from_f32<__hip_bfloat16>(float v) { return __float2bfloat16(v); }
+
+template <typename T> static __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<__half>(__half v) { return __half2float(v); }
+template <> __device__ __forceinline__ float to_f32<__hip_bfloat16>(__hip_bfloat16 v) { return __bfloat162float(v); }
+
+// Host side: device facts fetched once.
+struct LkDevice {
+    int cus;
+    int lds_bytes;
+};
+const LkDevice& lk_device();
+
+static inline int lk_launch_status() {
+    return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;
+}

@@ -1,0 +1,55 @@
+"""Loads ``libloken_gfx950.so`` and declares the C ABI of ``include/loken_gfx950.h``.
+
+There is no fallback: a missing library raises, it is never replaced by another code path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libloken_gfx950.so"
+
+LK_OK, LK_ERR_ARG, LK_ERR_TYPE, LK_ERR_LAUNCH, LK_ERR_NOMEM = 0, 1, 2, 3, 4
+_ERR_NAMES = {1: "LK_ERR_ARG", 2: "LK_ERR_TYPE", 3: "LK_ERR_LAUNCH", 4: "LK_ERR_NOMEM"}
+
+TYPE_F32, TYPE_F16, TYPE_BF16 = 0, 1, 30
+TYPE_Q8_0, TYPE_Q8_1, TYPE_Q4_K, TYPE_Q6_K = 8, 9, 12, 14
+
+
+class LokenError(RuntimeError):
+    def __init__(self, fn: str, code: int):
+        super().__init__(f"{fn} failed: {_ERR_NAMES.get(code, code)}")
+        self.code = code
+
+
+_vp, _i, _i64, _f = C.c_void_p, C.c_int, C.c_int64, C.c_float
+
+# name -> (restype, argtypes); mirrors include/loken_gfx950.h declaration by declaration
+SIGNATURES = {
+    "lk_device_info": (_i, [_vp, _vp, _vp, _vp]),
+    "lk_quantize_q8_1": (_i, [_vp, _i, _vp, _i, _i, _i, _vp]),
+    "lk_mmvq": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp]),
+    "lk_mmvq_subdots": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m loken_amd.build` (hipcc, gfx950)")
+        lib = C.CDLL(str(LIB_PATH))
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(fn: str, code: int) -> None:
+    if code != LK_OK:
+        raise LokenError(fn, code)

@@ -1,0 +1,63 @@
+"""Host layer over the C ABI for callers that hold torch device tensors.
+
+torch is used for device memory and the current stream only; every computation goes through
+``libloken_gfx950.so``. Function names follow the reference's Rust launch surface
+(src/tensor/cuda/quant.rs of loken): ``quantize_q8_1_rows`` (:19-26,112-151), ``mmvq_f32``
+(:173-184, 3264-3298).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import lib as _lib
+from .synth import BLOCK_BYTES, BLOCK_LEN
+
+ROW_PADDING = 512
+
+_X_TYPES = {torch.float32: _lib.TYPE_F32, torch.float16: _lib.TYPE_F16, torch.bfloat16: _lib.TYPE_BF16}
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def pad_to(v: int, m: int) -> int:
+    return (v + m - 1) // m * m
+
+
+def quantize_q8_1_rows(x: torch.Tensor, k_padded: int | None = None) -> torch.Tensor:
+    """``[rows, k]`` f32/f16/bf16 -> ``[rows, k_padded/32, 36]`` uint8 Q8_1 blocks."""
+    if not x.is_cuda or x.dim() != 2 or not x.is_contiguous():
+        raise ValueError("q8_1 quantize: a contiguous 2-D device tensor is required")
+    rows, k = x.shape
+    k_padded = pad_to(k, ROW_PADDING) if k_padded is None else k_padded
+    out = torch.empty((rows, k_padded // 32, 36), dtype=torch.uint8, device=x.device)
+    _lib.check("lk_quantize_q8_1", _lib.load().lk_quantize_q8_1(
+        x.data_ptr(), _X_TYPES[x.dtype], out.data_ptr(), k, k_padded, rows, _stream()))
+    return out
+
+
+def mmvq(wtype: int, weight: torch.Tensor, q8_1: torch.Tensor, k: int, n: int, *,
+         out_dtype: torch.dtype = torch.float32, bias: torch.Tensor | None = None,
+         decode_order: bool = False) -> torch.Tensor:
+    """``weight`` (uint8 blob of ``n`` rows of ``k`` values) x ``q8_1`` ``[b, k_padded/32, 36]``
+    -> ``[b, n]``."""
+    b = q8_1.shape[0]
+    expect = n * (k // BLOCK_LEN[wtype]) * BLOCK_BYTES[wtype] if wtype in BLOCK_LEN else -1
+    if weight.numel() < expect:
+        raise ValueError(f"mmvq: weight holds {weight.numel()} bytes, {expect} needed")
+    out = torch.empty((b, n), dtype=out_dtype, device=weight.device)
+    _lib.check("lk_mmvq", _lib.load().lk_mmvq(
+        wtype, weight.data_ptr(), q8_1.data_ptr(), out.data_ptr(), _X_TYPES[out_dtype], k, n, b,
+        q8_1.shape[1], n, bias.data_ptr() if bias is not None else None, int(decode_order), _stream()))
+    return out
+
+
+def mmvq_subdots(wtype: int, weight: torch.Tensor, q8_1_row: torch.Tensor, k: int, n: int):
+    """Integer sub-block dots of every weight row against ONE Q8_1 row (parity probe)."""
+    per = 16 if wtype == _lib.TYPE_Q6_K else 32
+    dots = torch.empty((n, k // per), dtype=torch.int32, device=weight.device)
+    sums = torch.empty((k // 32,), dtype=torch.int32, device=weight.device)
+    _lib.check("lk_mmvq_subdots", _lib.load().lk_mmvq_subdots(
+        wtype, weight.data_ptr(), q8_1_row.data_ptr(), dots.data_ptr(), sums.data_ptr(), k, n, _stream()))
+    return dots, sums

@@ -1,0 +1,187 @@
+"""GPU parity of the decode path (Q8_1 quantizer + mat-vec) against the CPU oracle.
+
+Bars: Q8_1 bytes and integer sub-block dots bit-exact; f32 outputs within 1e-3 relative +
+1e-4 absolute of the same-codes oracle (O-B); and within the reference's own quantization
+envelope 1e-3 * sum|x.w| + 1e-3 (src/tensor/quantized/tests.rs:715-724) of the served CPU path
+(O-A), whose activation codes differ by design (Q8_K per 256 vs Q8_1 per 32).
+"""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+import oracle
+from loken_amd import lib, ops, synth
+
+pytestmark = pytest.mark.gpu
+
+DT = {"q4_k": lib.TYPE_Q4_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0}
+RTOL, ATOL = 1e-3, 1e-4
+
+
+def dev(a: np.ndarray) -> "torch.Tensor":
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def assert_close(got, want):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    bad = np.abs(got - want) > RTOL * np.abs(want) + ATOL
+    assert not bad.any(), f"{bad.sum()} of {bad.size} outside 1e-3 rel + 1e-4 abs; worst {np.abs(got - want).max()}"
+
+
+# ---------------------------------------------------------------- quantizer
+@pytest.mark.parametrize("rows,k", [(1, 4096), (3, 1000), (8, 14336), (2, 32), (1, 33), (5, 2048)])
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_q8_1_quantizer_is_bit_exact(rows, k, dtype):
+    x = synth.activation(rows, k, seed=31) * np.float32(2.5)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    xt = dev(x).to(tdt)
+    x_seen = xt.to(torch.float32).cpu().numpy()  # what the kernel reads, widened exactly
+    kp = ops.pad_to(k, 512)
+    got = ops.quantize_q8_1_rows(xt).cpu().numpy()
+    assert got.shape == (rows, kp // 32, 36)
+    padded = np.zeros((rows, kp), np.float32)
+    padded[:, :k] = x_seen
+    want = oracle.quantize_q8_1(padded).reshape(rows, kp // 32, 36)
+    assert np.array_equal(got, want)
+
+
+def test_q8_1_quantizer_edge_values():
+    x = np.zeros((4, 64), np.float32)
+    x[1, 0] = 127.0
+    x[1, 1:9] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, -63.5]   # exact ties at d = 1
+    x[2] = 1e-30                                                  # tiny but nonzero
+    x[3, 5] = -3.0e38                                             # near f32 max
+    got = ops.quantize_q8_1_rows(dev(x), k_padded=64).cpu().numpy()
+    want = oracle.quantize_q8_1(x).reshape(4, 2, 36)
+    assert np.array_equal(got, want)
+    assert got[1, 0, 4:13].view(np.int8).tolist() == [127, 1, 2, 3, -1, -2, -3, 64, -64]
+
+
+def test_quantizer_rejects_what_it_cannot_take():
+    x = torch.zeros((2, 64), device="cuda")
+    with pytest.raises(lib.LokenError):
+        ops.quantize_q8_1_rows(x, k_padded=48)      # not whole blocks
+    with pytest.raises(lib.LokenError):
+        ops.quantize_q8_1_rows(x, k_padded=32)      # shorter than the row
+
+
+# ---------------------------------------------------------------- integer sub-block dots
+@pytest.mark.parametrize("name,n,k", [("q4_k", 16, 1024), ("q4_k", 5, 768), ("q4_k", 64, 4096),
+                                      ("q6_k", 16, 1024), ("q6_k", 7, 2304), ("q8_0", 16, 1024),
+                                      ("q8_0", 9, 96), ("q8_0", 4, 4096)])
+def test_integer_subblock_dots_are_bit_exact(name, n, k):
+    wtype = DT[name]
+    w = synth.weight(wtype, n, k, seed=32, stream=1)
+    x = synth.activation(1, k, seed=32)
+    q = ops.quantize_q8_1_rows(dev(x))
+    dots, sums = ops.mmvq_subdots(wtype, dev(w), q[0], k, n)
+    want_dots, want_sums = oracle.ob_subdots(wtype, k, n, w, oracle.quantize_q8_1(x))
+    assert np.array_equal(dots.cpu().numpy(), want_dots)
+    assert np.array_equal(sums.cpu().numpy(), want_sums)
+
+
+def test_q4k_extreme_subdot_on_gpu():
+    w = np.zeros((1, 1, 144), np.uint8)
+    w[..., 16:] = 0xFF
+    x = np.full((1, 256), 127.0, np.float32)
+    dots, sums = ops.mmvq_subdots(lib.TYPE_Q4_K, dev(w), ops.quantize_q8_1_rows(dev(x))[0], 256, 1)
+    assert dots.cpu().tolist() == [[60960] * 8] and sums.cpu().tolist() == [127 * 32] * 8
+
+
+# ---------------------------------------------------------------- f32 outputs
+SHAPES = [
+    ("q4_k", 4096, 4096), ("q4_k", 1024, 4096), ("q4_k", 33, 768), ("q4_k", 1, 256), ("q4_k", 257, 2048),
+    ("q6_k", 4096, 2048), ("q6_k", 19, 2304), ("q6_k", 1, 256), ("q6_k", 130, 14336),
+    ("q8_0", 1000, 4096), ("q8_0", 3, 32), ("q8_0", 65, 1056),
+]
+
+
+@pytest.mark.parametrize("name,n,k", SHAPES)
+@pytest.mark.parametrize("batch", [1, 2, 3, 4, 5, 8])
+def test_matvec_matches_same_codes_oracle(name, n, k, batch):
+    wtype = DT[name]
+    w = synth.weight(wtype, n, k, seed=33, stream=2)
+    x = synth.activation(batch, k, seed=33)
+    q = ops.quantize_q8_1_rows(dev(x))
+    got = ops.mmvq(wtype, dev(w), q, k, n).cpu().numpy()
+    want = oracle.ob_matmul(wtype, x, w, n)
+    assert_close(got, want)
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+def test_matvec_within_reference_envelope_of_served_cpu_path(name):
+    wtype = DT[name]
+    n, k = 512, 4096
+    w = synth.weight(wtype, n, k, seed=34, stream=3)
+    x = synth.activation(4, k, seed=34)
+    got = ops.mmvq(wtype, dev(w), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
+    served = oracle.oa_matmul(wtype, x, w, n)
+    wd = oracle.dequantize(wtype, w).reshape(n, k).astype(np.float64)
+    envelope = 1e-3 * (np.abs(x.astype(np.float64)) @ np.abs(wd).T) + 1e-3
+    assert (np.abs(got - served) <= envelope).all()
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+def test_rows_do_not_depend_on_batch(name):
+    # decode order: a row of a batched launch carries the bits of its own batch-1 launch
+    wtype = DT[name]
+    n, k = 300, 2048
+    w = dev(synth.weight(wtype, n, k, seed=35, stream=4))
+    q = ops.quantize_q8_1_rows(dev(synth.activation(6, k, seed=35)))
+    full = ops.mmvq(wtype, w, q, k, n, decode_order=True)
+    for j in range(6):
+        one = ops.mmvq(wtype, w, q[j:j + 1], k, n)
+        assert torch.equal(one[0], full[j])
+
+
+@pytest.mark.parametrize("out", ["f16", "bf16"])
+def test_bias_and_narrow_outputs(out):
+    wtype, n, k = lib.TYPE_Q4_K, 200, 1024
+    w = synth.weight(wtype, n, k, seed=36, stream=5)
+    x = synth.activation(2, k, seed=36)
+    bias = synth.activation(1, n, seed=36, stream=9)[0]
+    q = ops.quantize_q8_1_rows(dev(x))
+    tdt = {"f16": torch.float16, "bf16": torch.bfloat16}[out]
+    f32 = ops.mmvq(wtype, dev(w), q, k, n, bias=dev(bias))
+    want = oracle.ob_matmul(wtype, x, w, n) + bias[None, :]
+    assert_close(f32.cpu().numpy(), want)
+    narrow = ops.mmvq(wtype, dev(w), q, k, n, out_dtype=tdt, bias=dev(bias))
+    assert torch.equal(narrow, f32.to(tdt))
+
+
+def test_strided_destination_and_activation():
+    # dst rows further apart than n, activation rows further apart than k/32
+    wtype, n, k = lib.TYPE_Q6_K, 40, 512
+    w = synth.weight(wtype, n, k, seed=37, stream=6)
+    x = synth.activation(3, k, seed=37)
+    q = ops.quantize_q8_1_rows(dev(x), k_padded=1024)
+    out = torch.full((3, 64), 7.0, device="cuda")
+    lib.check("lk_mmvq", lib.load().lk_mmvq(wtype, dev(w).data_ptr(), q.data_ptr(), out.data_ptr(),
+                                            lib.TYPE_F32, k, n, 3, 1024 // 32, 64, None, 0,
+                                            torch.cuda.current_stream().cuda_stream))
+    got = out.cpu().numpy()
+    assert_close(got[:, :n], oracle.ob_matmul(wtype, x, w, n))
+    assert (got[:, n:] == 7.0).all()
+
+
+# ---------------------------------------------------------------- full benchmark sizes
+@pytest.mark.parametrize("name,n,k", [("q4_k", 14336, 4096), ("q6_k", 4096, 14336), ("q8_0", 128256, 4096)])
+def test_full_size_matvec_against_oracle(name, n, k):
+    wtype = DT[name]
+    w = synth.weight(wtype, n, k, seed=0, stream=10)
+    x = synth.activation(1, k, seed=0)
+    got = ops.mmvq(wtype, dev(w), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(wtype, x, w, n))
+    # size-independent property: the product is linear in the block scale d, so doubling every
+    # d (exact in f16) doubles every output bit for bit
+    w2 = w.copy()
+    off = {"q4_k": 0, "q6_k": 208, "q8_0": 0}[name]
+    d = w2[:, :, off:off + 2].copy().view(np.float16)
+    w2[:, :, off:off + 2] = (d * np.float16(2)).view(np.uint8)
+    if name == "q4_k":
+        dm = w2[:, :, 2:4].copy().view(np.float16)
+        w2[:, :, 2:4] = (dm * np.float16(2)).view(np.uint8)
+    got2 = ops.mmvq(wtype, dev(w2), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
+    assert np.array_equal(got2, 2 * got)
