@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF block-quantized matmul hot path on one MI355X.
+
+One *step* = every quantized linear of one Llama-3-8B-shaped decode step at batch `--batch`
+(default 1): per layer q, o 4096->4096, k, v 4096->1024, gate, up 4096->14336 in Q4_K and down
+14336->4096 in Q6_K, 32 layers, then lm_head 4096->128256 in Q8_0: 225 weight matrices,
+4.97 GB of blocks, each linear preceded by the Q8_1 quantization of its activation (q/k/v and
+gate/up share one). Distinct weights per layer, so the step is cache-cold by construction.
+Weights and activations are synthetic (seeded, generated on the device) and resident in HBM
+before the timed region.
+
+`value` = weight bytes of the step / time per step (the reference's mat-vec convention: weight
+bytes only, src/tensor/cuda/quant.rs:3905,3959-3961 of loken), whole job, one GPU.
+
+Two more measurements ride in the same JSON line:
+  roofline      the dominant kernel (Q4_K mat-vec): average launch duration over the step's own
+                mix of Q4_K launches, timed with HIP events on the launch stream, against the
+                algorithmic weight bytes per launch and MI355X's 8 TB/s HBM peak.
+  cpu_baseline  the CPU oracle's served path (AVX2 + worker pool restatement of loken's CPU
+                quantized matmul) on a bounded sample of the same workload, on this host's cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+LAYERS = 32
+HIDDEN, KV, FFN, VOCAB = 4096, 1024, 14336, 128256
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=1, help="activation rows per mat-vec (1..8)")
+    ap.add_argument("--layers", type=int, default=LAYERS)
+    ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline sample")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported "
+              "(no collectives or sharding are part of it).", file=sys.stderr)
+        return 2
+
+    import torch
+    from loken_amd import lib, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    L = lib.load()  # raises if the HIP library is missing: there is no other path
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+    b = args.batch
+
+    # ------------------------------------------------------------------ synthetic blocks
+    def halfs(n, scale):
+        v = torch.randn(n, device=dev, generator=gen).abs() * scale
+        return v.to(torch.float16).view(torch.uint8).reshape(n, 2)
+
+    def make_q4k(n, k):
+        nb = n * (k // 256)
+        w = torch.randint(0, 256, (nb, 144), dtype=torch.uint8, device=dev, generator=gen)
+        w[:, 0:2] = halfs(nb, 1e-3)
+        w[:, 2:4] = halfs(nb, 5e-4)
+        return w.reshape(-1)
+
+    def make_q6k(n, k):
+        nb = n * (k // 256)
+        w = torch.randint(0, 256, (nb, 210), dtype=torch.uint8, device=dev, generator=gen)
+        sc = torch.randint(-64, 64, (nb, 16), dtype=torch.int8, device=dev, generator=gen)
+        w[:, 192:208] = sc.view(torch.uint8)
+        w[:, 208:210] = halfs(nb, 1e-3)
+        return w.reshape(-1)
+
+    def make_q80(n, k):
+        nb = n * (k // 32)
+        w = torch.empty((nb, 34), dtype=torch.uint8, device=dev)
+        w[:, 0:2] = halfs(nb, 1e-3)
+        w[:, 2:] = torch.randint(-127, 128, (nb, 32), dtype=torch.int8, device=dev, generator=gen).view(torch.uint8)
+        return w.reshape(-1)
+
+    Q4K, Q6K, Q80 = lib.TYPE_Q4_K, lib.TYPE_Q6_K, lib.TYPE_Q8_0
+    shapes = [  # (name, wtype, n, k, maker, activation group)
+        ("q", Q4K, HIDDEN, HIDDEN, make_q4k, "x"), ("k", Q4K, KV, HIDDEN, make_q4k, "x"),
+        ("v", Q4K, KV, HIDDEN, make_q4k, "x"), ("o", Q4K, HIDDEN, HIDDEN, make_q4k, "attn"),
+        ("gate", Q4K, FFN, HIDDEN, make_q4k, "x2"), ("up", Q4K, FFN, HIDDEN, make_q4k, "x2"),
+        ("down", Q6K, HIDDEN, FFN, make_q6k, "h"),
+    ]
+    stream = torch.cuda.current_stream().cuda_stream
+    acts = {g: torch.randn((b, k), device=dev, generator=gen) for g, k in
+            (("x", HIDDEN), ("attn", HIDDEN), ("x2", HIDDEN), ("h", FFN), ("final", HIDDEN))}
+    q81 = {g: torch.empty((b, -(-a.shape[1] // 512) * 512 // 32, 36), dtype=torch.uint8, device=dev)
+           for g, a in acts.items()}
+
+    plan = []       # (fn, args) in launch order: one step
+    q4k_plan = []   # the Q4_K mat-vec launches of a step
+    total_bytes = 0
+    q4k_bytes = 0
+    keep = []
+
+    def add_quant(g):
+        a, q = acts[g], q81[g]
+        plan.append((L.lk_quantize_q8_1, (a.data_ptr(), lib.TYPE_F32, q.data_ptr(), a.shape[1],
+                                          q.shape[1] * 32, b, stream)))
+
+    def add_gemv(wtype, w, g, n, k):
+        nonlocal total_bytes, q4k_bytes
+        out = torch.empty((b, n), dtype=torch.float32, device=dev)
+        keep.append(out)
+        q = q81[g]
+        item = (L.lk_mmvq, (wtype, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, b,
+                            q.shape[1], n, None, 0, stream))
+        plan.append(item)
+        nbytes = synth.weight_bytes(wtype, n, k)
+        total_bytes += nbytes
+        if wtype == Q4K:
+            q4k_plan.append(item)
+            q4k_bytes += nbytes
+        return out
+
+    first_out = None
+    first_w = None
+    for layer in range(args.layers):
+        last_group = None
+        for name, wtype, n, k, maker, g in shapes:
+            w = maker(n, k)
+            keep.append(w)
+            if g != last_group:
+                add_quant(g)
+                last_group = g
+            out = add_gemv(wtype, w, g, n, k)
+            if first_out is None:
+                first_out, first_w = out, w
+    lm_head = make_q80(VOCAB, HIDDEN)
+    keep.append(lm_head)
+    add_quant("final")
+    add_gemv(Q80, lm_head, "final", VOCAB, HIDDEN)
+    torch.cuda.synchronize()
+
+    def run(items):
+        for fn, a in items:
+            rc = fn(*a)
+            if rc:
+                raise lib.LokenError(fn.__name__, rc)
+
+    run(plan)  # eager once: first-launch set-up happens outside any capture
+    torch.cuda.synchronize()
+
+    graph = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        # the launch stream is an argument of every planned call: rebuild the plans on `side`
+        def on_stream(items, s):
+            return [(fn, a[:-1] + (s,)) for fn, a in items]
+        with torch.cuda.stream(side):
+            cap_plan = on_stream(plan, side.cuda_stream)
+            run(cap_plan)
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                run(cap_plan)
+        torch.cuda.synchronize()
+
+    def step():
+        if graph is not None:
+            graph.replay()
+        else:
+            run(plan)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = total_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ------------------------------------------------------------------ roofline leg
+    # The step's own mix of Q4_K mat-vec launches, nothing else on the stream, between two
+    # events on the launch stream.
+    reps = max(3, min(20, args.steps))
+    run(q4k_plan)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        run(q4k_plan)
+    e1.record()
+    torch.cuda.synchronize()
+    launches = reps * len(q4k_plan)
+    avg_us = e0.elapsed_time(e1) * 1e3 / launches
+    bytes_per_launch = q4k_bytes / len(q4k_plan)
+    achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": f"mmvq_q4k_kernel<{b},*,float>", "avg_launch_us": round(avg_us, 3),
+                "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches}
+
+    # ------------------------------------------------------------------ CPU baseline leg
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(args, torch, synth, lib, first_w, first_out, acts["x"], b)
+
+    line = {
+        "metric": "Q4_K GEMV weight GB/s (% HBM peak); prefill MMQ int8 TOPS (% MFMA peak)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": f"llama3-8b decode-step quantized linears (Q4_K q,k,v,o,gate,up; Q6_K down; "
+                               f"Q8_0 lm_head), batch {b}, {args.layers} layers",
+                   "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
+                   "hip_graph": graph is not None},
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+def cpu_baseline(args, torch, synth, lib, w_dev, out_dev, x_dev, b):
+    """The oracle's threaded served path on layer 0's q_proj-shaped sample, rotating copies."""
+    import numpy as np
+
+    import oracle
+
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    n, k = HIDDEN, HIDDEN
+    w = w_dev.cpu().numpy()
+    x = x_dev.cpu().numpy()
+    # parity of the benchmarked path on this very matrix, against the same-codes oracle
+    want = oracle.ob_matmul(oracle.Q4_K, x, w, n)
+    got = out_dev.cpu().numpy()
+    ok = bool((np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-4).all())
+    # working set past the last-level cache: 16 distinct copies = 151 MB
+    copies = [w.copy() for _ in range(16)]
+    oracle.oa_matmul(oracle.Q4_K, x, copies[0], n, fast_threads=threads)
+    t0 = time.perf_counter()
+    calls = 0
+    while time.perf_counter() - t0 < args.cpu_seconds:
+        for c in copies:
+            oracle.oa_matmul(oracle.Q4_K, x, c, n, fast_threads=threads)
+            calls += 1
+    dt = time.perf_counter() - t0
+    gbs = calls * synth.weight_bytes(lib.TYPE_Q4_K, n, k) / dt / 1e9
+    kind = "port"
+    return {"value": round(gbs, 2), "unit": "GB/s", "cores": threads, "kind": kind,
+            "sample": f"Q4_K mat-vec {n}x{k}, batch {b}, {calls} calls over 16 rotating copies "
+                      f"({dt:.1f} s), AVX2 + {threads}-thread pool restatement of the CPU path "
+                      f"(Q8_K activations)",
+            "gpu_parity_on_sample": "ok" if ok else "FAILED"}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -19,6 +19,10 @@
 
 #include "lk_common.h"
 
+#include <cstdlib>
+#include <mutex>
+#include <unordered_map>
+
 namespace {
 
 constexpr int WG = 256;            // threads per workgroup
@@ -30,6 +34,7 @@ constexpr int WAVES = WG / LK_WAVE;
 // --------------------------------------------------------------------------------------------
 
 // Q4_K: 16 bytes of qs = values l..l+15 of sub-block 2p (low nibbles) and of 2p+1 (high nibbles).
+// Adds their products with the matching 16 activation codes of each sub-block into d_lo / d_hi.
 static __device__ __forceinline__ void q4k_dots(const uint4& q, const uint4& a_lo, const uint4& a_hi,
                                                 int& d_lo, int& d_hi) {
     uint4 lo, hi;
@@ -37,22 +42,24 @@ static __device__ __forceinline__ void q4k_dots(const uint4& q, const uint4& a_l
     lo.y = q.y & 0x0F0F0F0Fu; hi.y = (q.y >> 4) & 0x0F0F0F0Fu;
     lo.z = q.z & 0x0F0F0F0Fu; hi.z = (q.z >> 4) & 0x0F0F0F0Fu;
     lo.w = q.w & 0x0F0F0F0Fu; hi.w = (q.w >> 4) & 0x0F0F0F0Fu;
-    d_lo = dot16(lo, a_lo, 0);
-    d_hi = dot16(hi, a_hi, 0);
+    d_lo = dot16(lo, a_lo, d_lo);
+    d_hi = dot16(hi, a_hi, d_hi);
 }
 
-// The two (scale, min) pairs of sub-blocks 2p, 2p+1 from the 12 packed bytes (words w1..w3 of the
-// block header). Returns scales in bits 0-7 / 8-15 of `sc`, mins likewise in `mn`.
-static __device__ __forceinline__ void q4k_scale_pair(uint32_t w1, uint32_t w2, uint32_t w3, int p,
-                                                      uint32_t& sc, uint32_t& mn) {
-    const int sh = 16 * (p & 1);
-    const uint32_t a = w1 >> sh, b = w2 >> sh, c = w3 >> sh;
-    const uint32_t sc_first = a & 0x3F3Fu, mn_first = b & 0x3F3Fu;
-    const uint32_t sc_last = (c & 0x0F0Fu) | (((a >> 6) & 0x0303u) << 4);
-    const uint32_t mn_last = ((c >> 4) & 0x0F0Fu) | (((b >> 6) & 0x0303u) << 4);
-    sc = p < 2 ? sc_first : sc_last;
-    mn = p < 2 ? mn_first : mn_last;
-}
+// The (scale, min) pairs of sub-blocks 2p, 2p+1 from the 12 packed bytes (words w1..w3 of the
+// block header): scales in bits 0-7 / 8-15 of `sc`, mins likewise in `mn`. Sub-blocks 0-3 keep
+// their six bits in one byte; 4-7 take a nibble from bytes 8-11 and two bits from the top of
+// bytes 0-7. The selectors depend on the lane only, so they are built once outside any loop.
+struct Q4KScaleSel {
+    uint32_t shift, first, mask_main, mask_top;
+    __device__ __forceinline__ explicit Q4KScaleSel(int p)
+        : shift(16 * (p & 1)), first(p < 2), mask_main(p < 2 ? 0x3F3Fu : 0x0F0Fu), mask_top(p < 2 ? 0u : 0x3030u) {}
+    __device__ __forceinline__ void unpack(uint32_t w1, uint32_t w2, uint32_t w3, uint32_t& sc, uint32_t& mn) const {
+        const uint32_t a = w1 >> shift, b = w2 >> shift, c = w3 >> shift;
+        sc = ((first ? a : c) & mask_main) | ((a >> 2) & mask_top);
+        mn = ((first ? b : (c >> 4)) & mask_main) | ((b >> 2) & mask_top);
+    }
+};
 
 // Q6_K: 16 bytes of ql and the 16 bytes of qh over the same l give two runs of 16 signed codes:
 // run A in group g0 (low nibbles, qh bits 2*g0), run B in group g0+2 (high nibbles, bits 2*g0+4).
@@ -81,12 +88,13 @@ static __device__ __forceinline__ void q6k_dots(const uint4& ql, const uint4& qh
 
 struct FmtQ4K {
     static constexpr int BLOCK_BYTES = Q4K_BYTES, BLOCK_LEN = 256;
-    static constexpr int VPI = 2048;   // values per wave pass
-    static constexpr int PLANES = 2, SCF = 2;
-    // j: Q8_1 block index inside the pass (0..63), lh: which 16-byte half of its codes
+    static constexpr int VPI = 4096;   // values per wave pass: 16 super-blocks, 4 lanes each
+    static constexpr int PLANES = 4, SCF = 2;
+    // j: Q8_1 block index inside the pass (0..127), lh: which 16-byte half of its codes.
+    // Lane (block lb, pair p) reads plane (2 * odd + lh) at lane * 16.
     static __device__ __forceinline__ int slot(int j, int lh) {
         const int lb = j >> 3, s = j & 7;
-        return (s & 1) * 1024 + (lb * 8 + (s >> 1) * 2 + lh) * 16;
+        return ((s & 1) * 2 + lh) * 1024 + (lb * 4 + (s >> 1)) * 16;
     }
 };
 struct FmtQ6K {
@@ -164,74 +172,111 @@ __global__ __launch_bounds__(WG) void mmvq_q4k_kernel(const uint8_t* __restrict_
                                                       int nb, int n, int stride_col_y, int stride_col_dst,
                                                       const float* __restrict__ bias) {
     extern __shared__ __align__(16) uint8_t lds[];
-    const int n_iter = (nb + 7) >> 3;
+    const int n_iter = (nb + 15) >> 4;
     const int row_bytes = lds_bytes_per_row<FmtQ4K>(n_iter);
-    stage_activation<FmtQ4K, B>(lds, vy, nb * 8, n_iter, stride_col_y);
-    __syncthreads();
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lb = lane >> 3, ch = lane & 7, p = ch >> 1;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lb = lane >> 2, p = lane & 3;
+    const Q4KScaleSel sel(p);
+    const uint32_t hdr_off = lb * Q4K_BYTES, qs_off = hdr_off + 16 + 32 * p;
     const size_t row_stride = (size_t)nb * Q4K_BYTES;
+    const int n_tiles = (n + R - 1) / R;
+    const int tile_stride = gridDim.x * WAVES;
 
-    for (int tile = blockIdx.x * WAVES + wave; tile * R < n; tile += gridDim.x * WAVES) {
-        const int row0 = tile * R;
-        float acc[R][B];
+    struct Frag {
+        uint4 hdr[R], q0[R], q1[R];
+    };
+    // One pass (16 super-blocks) of R rows into registers. Lanes past the row end hold zeros:
+    // d = dmin = 0 and the staged activation tail is zero, so they add nothing.
+    auto load = [&](Frag& f, int tile, int it) {
+        const bool valid = it * 16 + lb < nb;
+        // an out-of-range lane re-reads the row's last block and drops its d / dmin
+        const uint32_t back = valid ? 0u : (uint32_t)(it * 16 + lb - (nb - 1)) * Q4K_BYTES;
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
+        for (int r = 0; r < R; ++r) {
+            const int row = min(tile * R + r, n - 1);
+            const uint8_t* bp = vx + row * row_stride + (size_t)it * (16 * Q4K_BYTES);
+            f.hdr[r] = *(const uint4*)(bp + (hdr_off - back));
+            f.q0[r] = *(const uint4*)(bp + (qs_off - back));
+            f.q1[r] = *(const uint4*)(bp + (qs_off - back + 16));
+            if (!valid) f.hdr[r].x = 0;
+        }
+    };
 
-        for (int it = 0; it < n_iter; ++it) {
-            const int blk = it * 8 + lb;
-            const bool valid = blk < nb;
-            const int blk_c = valid ? blk : nb - 1;
-            uint4 hdr[R], q[R];
+    float acc[R][B];
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r, n - 1);
-                const uint8_t* bp = vx + row * row_stride + (size_t)blk_c * Q4K_BYTES;
-                hdr[r] = *(const uint4*)bp;
-                q[r] = *(const uint4*)(bp + 16 + 16 * ch);
-            }
-            float dsc_lo[R], dsc_hi[R], dm_lo[R], dm_hi[R];
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                uint32_t sc, mn;
-                q4k_scale_pair(hdr[r].y, hdr[r].z, hdr[r].w, p, sc, mn);
-                const float d = valid ? f16_bits_to_f32(hdr[r].x & 0xFFFFu) : 0.f;
-                // each of the two lanes sharing a sub-block carries half of its min term
-                const float dmin_h = valid ? 0.5f * f16_bits_to_f32(hdr[r].x >> 16) : 0.f;
-                dsc_lo[r] = d * (float)(sc & 0xFFu);
-                dsc_hi[r] = d * (float)(sc >> 8);
-                dm_lo[r] = dmin_h * (float)(mn & 0xFFu);
-                dm_hi[r] = dmin_h * (float)(mn >> 8);
-            }
+        for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
+
+    auto compute = [&](const Frag& f, int tile, int it) {
+        float d[R], dmin[R], scl[R], sch[R], ml[R], mh[R];
 #pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const uint8_t* rowl = lds + c * row_bytes;
-                const uint8_t* codes = rowl + it * 2048;
-                const uint4 a_lo = *(const uint4*)(codes + lane * 16);
-                const uint4 a_hi = *(const uint4*)(codes + 1024 + lane * 16);
-                const float4 s4 = *(const float4*)(rowl + n_iter * 2048 + (size_t)(blk * 8 + 2 * p) * 8);
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    int d_lo, d_hi;
-                    q4k_dots(q[r], a_lo, a_hi, d_lo, d_hi);
-                    float v = dsc_lo[r] * (s4.x * (float)d_lo);
-                    v += dsc_hi[r] * (s4.z * (float)d_hi);
-                    v -= dm_lo[r] * s4.y;
-                    v -= dm_hi[r] * s4.w;
-                    acc[r][c] += v;
-                }
-            }
+        for (int r = 0; r < R; ++r) {
+            uint32_t sc, mn;
+            sel.unpack(f.hdr[r].y, f.hdr[r].z, f.hdr[r].w, sc, mn);
+            d[r] = f16_bits_to_f32(f.hdr[r].x & 0xFFFFu);
+            dmin[r] = f16_bits_to_f32(f.hdr[r].x >> 16);
+            scl[r] = (float)(sc & 0xFFu);
+            sch[r] = (float)(sc >> 8);
+            ml[r] = (float)(mn & 0xFFu);
+            mh[r] = (float)(mn >> 8);
         }
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+        for (int c = 0; c < B; ++c) {
+            const uint8_t* rowl = lds + c * row_bytes;
+            const uint8_t* codes = rowl + it * 4096 + lane * 16;
+            const uint4 a00 = *(const uint4*)(codes);
+            const uint4 a01 = *(const uint4*)(codes + 1024);
+            const uint4 a10 = *(const uint4*)(codes + 2048);
+            const uint4 a11 = *(const uint4*)(codes + 3072);
+            const float4 s4 = *(const float4*)(rowl + n_iter * 4096 + (size_t)((it * 16 + lb) * 8 + 2 * p) * 8);
 #pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const float total = wave_sum(acc[r][c]);
-                if (lane == 0 && row0 + r < n) store_out(dst, stride_col_dst, c, row0 + r, total, bias);
+            for (int r = 0; r < R; ++r) {
+                int d_lo = 0, d_hi = 0;
+                q4k_dots(f.q0[r], a00, a10, d_lo, d_hi);
+                q4k_dots(f.q1[r], a01, a11, d_lo, d_hi);
+                const float u = (scl[r] * s4.x) * (float)d_lo + (sch[r] * s4.z) * (float)d_hi;
+                const float w = ml[r] * s4.y + mh[r] * s4.w;
+                acc[r][c] += d[r] * u - dmin[r] * w;
             }
+        }
+        if (it == n_iter - 1) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int c = 0; c < B; ++c) {
+                    const float total = wave_sum(acc[r][c]);
+                    acc[r][c] = 0.f;
+                    if (lane == 0 && tile * R + r < n) store_out(dst, stride_col_dst, c, tile * R + r, total, bias);
+                }
+        }
+    };
+
+    // Steps are (tile, pass) pairs in order; the loads of step i+1 are issued before step i is
+    // consumed, ping-ponging between two register fragments.
+    // The first weight loads go out before the activation is staged, so the two memory
+    // latencies overlap instead of adding up (it is most of a small matrix's run time).
+    int tile = blockIdx.x * WAVES + wave, it = 0;
+    Frag fa, fb;
+    if (tile < n_tiles) load(fa, tile, 0);
+    stage_activation<FmtQ4K, B>(lds, vy, nb * 8, n_iter, stride_col_y);
+    __syncthreads();
+    if (tile >= n_tiles) return;
+    for (;;) {
+        int nt = tile, ni = it + 1;
+        if (ni == n_iter) { ni = 0; nt += tile_stride; }
+        if (nt < n_tiles) load(fb, nt, ni);
+        compute(fa, tile, it);
+        tile = nt; it = ni;
+        if (tile >= n_tiles) break;
+        nt = tile; ni = it + 1;
+        if (ni == n_iter) { ni = 0; nt += tile_stride; }
+        if (nt < n_tiles) load(fa, nt, ni);
+        compute(fb, tile, it);
+        tile = nt; it = ni;
+        if (tile >= n_tiles) break;
     }
 }
 
@@ -461,33 +506,71 @@ static int n_iter_of(int nb) {
     return (nb + per - 1) / per;
 }
 
-#define LK_DEFINE_LAUNCHER(NAME, KERNEL, FMT, ROWS1, ROWSN)                                            \
+// Launch geometry. `R` rows per wave and the number of resident workgroups per CU set how many
+// bytes are in flight; both have measured optima well below "as many as fit" (HBM throughput
+// drops when too many requests are outstanding). LK_TUNE_R / LK_TUNE_WGS_PER_CU override the
+// built-in choice for measurement runs.
+static int tune_env(const char* name) {
+    const char* v = getenv(name);
+    return v ? atoi(v) : 0;
+}
+
+template <class FMT, int B, int R, typename T, typename K>
+static int launch_rows(K kernel, const MmvqArgs& a, int wgs_per_cu) {
+    const int lds_bytes = B * lds_bytes_per_row<FMT>(n_iter_of<FMT>(a.nb));
+    const LkDevice& dev = lk_device();
+    if (lds_bytes > dev.lds_bytes) return LK_ERR_ARG;
+    // Per kernel instance and LDS size: raise the dynamic-LDS limit once and ask the runtime how
+    // many workgroups a CU holds. Cached, so steady-state launches (and launches recorded into a
+    // graph) make no runtime query.
+    static std::mutex mu;
+    static std::unordered_map<int, int> resident_by_lds;
+    int resident = 0;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = resident_by_lds.find(lds_bytes);
+        if (it == resident_by_lds.end()) {
+            if (lds_bytes > 48 * 1024 &&
+                hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
+                (void)hipGetLastError();
+                return LK_ERR_LAUNCH;
+            }
+            int r = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)kernel, WG, (size_t)lds_bytes) != hipSuccess || r < 1) {
+                (void)hipGetLastError();
+                r = 1;
+            }
+            it = resident_by_lds.emplace(lds_bytes, r).first;
+        }
+        resident = it->second;
+    }
+    const int tiles = (a.n + R - 1) / R;
+    const int wgs_needed = (tiles + WAVES - 1) / WAVES;
+    // Persistent grid: exactly as many workgroups as are resident at once, so no workgroup waits
+    // for a slot and each wave walks several row tiles.
+    static const int forced = tune_env("LK_TUNE_WGS_PER_CU");
+    const int cap = forced > 0 ? forced : wgs_per_cu;
+    const int per_cu = resident > cap ? cap : resident;
+    const int grid = wgs_needed < dev.cus * per_cu ? wgs_needed : dev.cus * per_cu;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(WG), lds_bytes, a.stream, a.vx, a.vy, (T*)a.dst, a.nb,
+                       a.n, a.stride_col_y, a.stride_col_dst, a.bias);
+    return lk_launch_status();
+}
+
+#define LK_DEFINE_LAUNCHER(NAME, KERNEL, FMT, ROWS1, ROWSN, WGS_PER_CU)                                \
     template <int B, typename T>                                                                      \
     static int NAME(const MmvqArgs& a) {                                                              \
+        static const int forced_r = tune_env("LK_TUNE_R");                                            \
+        if (B == 1 && forced_r == 1) return launch_rows<FMT, B, 1, T>(KERNEL<B, 1, T>, a, WGS_PER_CU); \
+        if (B == 1 && forced_r == 2) return launch_rows<FMT, B, 2, T>(KERNEL<B, 2, T>, a, WGS_PER_CU); \
+        if (B == 1 && forced_r == 4) return launch_rows<FMT, B, 4, T>(KERNEL<B, 4, T>, a, WGS_PER_CU); \
         constexpr int R = (B == 1) ? ROWS1 : ROWSN;                                                   \
-        const int lds_bytes = B * lds_bytes_per_row<FMT>(n_iter_of<FMT>(a.nb));                        \
-        const LkDevice& dev = lk_device();                                                            \
-        if (lds_bytes > dev.lds_bytes) return LK_ERR_ARG;                                             \
-        auto kernel = KERNEL<B, R, T>;                                                                \
-        if (lds_bytes > 48 * 1024 &&                                                                  \
-            hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,      \
-                                lds_bytes) != hipSuccess) {                                           \
-            (void)hipGetLastError();                                                                  \
-            return LK_ERR_LAUNCH;                                                                     \
-        }                                                                                             \
-        const int tiles = (a.n + R - 1) / R;                                                          \
-        const int wgs_needed = (tiles + WAVES - 1) / WAVES;                                           \
-        int per_cu = dev.lds_bytes / lds_bytes;                                                       \
-        per_cu = per_cu < 1 ? 1 : (per_cu > 8 ? 8 : per_cu);                                          \
-        const int grid = wgs_needed < dev.cus * per_cu ? wgs_needed : dev.cus * per_cu;               \
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(WG), lds_bytes, a.stream, a.vx, a.vy, (T*)a.dst,  \
-                           a.nb, a.n, a.stride_col_y, a.stride_col_dst, a.bias);                      \
-        return lk_launch_status();                                                                    \
+        return launch_rows<FMT, B, R, T>(KERNEL<B, R, T>, a, WGS_PER_CU);                             \
     }
 
-LK_DEFINE_LAUNCHER(launch_q4k, mmvq_q4k_kernel, FmtQ4K, 2, 2)
-LK_DEFINE_LAUNCHER(launch_q6k, mmvq_q6k_kernel, FmtQ6K, 2, 2)
-LK_DEFINE_LAUNCHER(launch_q80, mmvq_q80_kernel, FmtQ80, 2, 2)
+LK_DEFINE_LAUNCHER(launch_q4k, mmvq_q4k_kernel, FmtQ4K, 2, 2, 8)
+LK_DEFINE_LAUNCHER(launch_q6k, mmvq_q6k_kernel, FmtQ6K, 2, 2, 8)
+LK_DEFINE_LAUNCHER(launch_q80, mmvq_q80_kernel, FmtQ80, 2, 2, 8)
 
 #define LK_BATCH_SWITCH(FN, T)                                                                         \
     switch (batch) {                                                                                  \
