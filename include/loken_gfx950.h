@@ -88,6 +88,40 @@ int lk_mmvq(int wtype, const void* vx, const void* vy_q8_1, void* dst, int dst_t
 int lk_mmvq_subdots(int wtype, const void* vx, const void* vy_q8_1, int32_t* dots, int32_t* sums,
                     int ncols_x, int nrows_x, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Prefill path: tiled quantized matmul on int8 MFMA. Names, argument lists and return
+ * conventions are loken's (src/tensor/quantized/mmq.rs:64-116 quantizers, :132-147 and
+ * cuda/mmq_gguf/mmq_launch.cuh:192-206 tile kernels), so `mmq_forward`
+ * (src/tensor/quantized/kernel_matmul/mmq.rs:21-159) links against them unchanged.
+ * ------------------------------------------------------------------------------------- */
+
+/* Activation rows -> the workspace the tile kernels read. `x` is f32, or f16 when type_x == 1;
+ * row r of the result is row ids[r] of x (ids nullable); ne00 = values per row, s01/s02/s03 =
+ * element strides of row / channel / sample, ne0 = padded row length (multiple of 512),
+ * ne1 = rows, ne2 * ne3 = channels. `vy` needs ne1 * (ne0/128) * 144 bytes per channel, the
+ * size loken allocates. D4 (scale only: Q6_K, Q8_0) and DS4 (scale and sum: Q4_K) write the
+ * same records here. D2S6 serves Q2_K alone and is not part of this library.
+ * Replaces launch_mmq_quantize_q8_1_{D4,DS4} of cuda/mmq_gguf/mmq_quantize.cu:67-166; codes
+ * follow BlockQ8_1::quantize (1/d rule), not that file's 127/amax rule, so that tiled and
+ * mat-vec products see the same integers. */
+void launch_mmq_quantize_q8_1_D4(const void* x, const int32_t* ids, void* vy, int type_x,
+                                 int64_t ne00, int64_t s01, int64_t s02, int64_t s03, int64_t ne0,
+                                 int64_t ne1, int64_t ne2, int64_t ne3, void* stream);
+void launch_mmq_quantize_q8_1_DS4(const void* x, const int32_t* ids, void* vy, int type_x,
+                                  int64_t ne00, int64_t s01, int64_t s02, int64_t s03, int64_t ne0,
+                                  int64_t ne1, int64_t ne2, int64_t ne3, void* stream);
+
+/* dst[col, row] (f32, rows `stride_col_dst` floats apart) = weight row `row` . token `col`.
+ *   x = weights [nrows_x][stride_row_x blocks], y = workspace of ncols_y rows, ncols_x = k.
+ * Returns the token-tile width launched (32, 64 or 128), 0 when nothing ran (bad sizes, or k
+ * not a multiple of 256). tmp_fixup, cc, nsm, smpbo, warp_size are accepted and unused: there
+ * is no stream-k fixup pass and one device family.
+ * Replaces launch_mmq_gguf_{q4_k,q6_k,q8_0} (cuda/mmq_gguf/mmq_launch.cuh:61-206). */
+int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,377 @@
+// Prefill / batched matmul on int8 MFMA: GGUF weight rows against Q8_1-quantized token rows.
+//
+//   out[token, n] = sum over 32-value sub-blocks s of  wscale_s[n] * d8_s[token] * D_s[n, token]
+//                   (Q4_K: minus sum_s (dmin*m_s)[n] * (d8_s*S_s)[token])
+// where D_s is the exact integer dot of a sub-block (v_mfma_i32_32x32x32_i8, K = 32 = one
+// sub-block) and S_s the integer sum of the activation codes. The integer part is what loken's
+// CPU path forms (src/tensor/quant_cpu/format/q4_k.rs:138-153, q6_k.rs:137-160, q8_0.rs:88-95);
+// the f32 combine is the Q8_1-side one (cuda/moe/gguf.cuh:664-713, 782-816, 486-495). This file
+// stands in for cuda/mmq_gguf/{mmq_quantize.cu, mmq_launch.cuh, mmq_gguf.cuh} of the reference
+// and shares nothing with them but the entry-point names and the workspace size contract.
+//
+// Workspace ("y", written by launch_mmq_quantize_q8_1_*): per (256-value block kb, row) one
+// record of 288 bytes = 2 x 144, block-major: record (kb * rows + row) holds
+//   [256 int8 codes][8 x f16 d8][8 x int16 sum of codes]   (one d8 / sum per 32 codes).
+// Same bytes per row as the reference's block_q8_1_mmq tiles (144 per 128 values), so the
+// host-side sizing rows * (k_padded/128) * 144 (+ slack) of src/tensor/quantized/kernel_matmul/
+// mmq.rs:38-41 holds unchanged. The quantization rule is the decode quantizer's (d = amax/127,
+// codes = round_half_away(x * (1/d))), so a tiled product is M mat-vec products to the integer.
+//
+// Kernel shape: workgroup tile 128 weight rows x TM tokens, K walked one 256-value block at a
+// time. Per step the workgroup expands the weight nibbles to int8 in LDS laid out
+// [sub-block][row][32 bytes] (so an MFMA operand is one conflict-free ds_read_b128 per lane),
+// copies the token codes likewise, and tables the per-sub-block scales as f32. A wave owns a
+// 32*JT x 32*IT patch of the tile: lanes <-> weight rows (coalesced stores), accumulator
+// registers <-> tokens. The Q4_K min term is a rank-8 update per block and runs on the f32
+// MFMA (v_mfma_f32_32x32x2_f32) straight into the accumulators, costing no per-element VALU.
+
+#include "lk_common.h"
+
+#include <mutex>
+#include <unordered_map>
+
+namespace {
+
+constexpr int MMQ_WG = 256;
+constexpr int TN = 128;            // weight rows per workgroup tile
+constexpr int REC_BYTES = 288;     // workspace record: 256 codes + 8 f16 + 8 i16
+
+// --------------------------------------------------------------------------------------------
+// Activation quantizer -> workspace records
+// --------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void mmq_quantize_kernel(const T* __restrict__ x,
+                                                           const int32_t* __restrict__ ids,
+                                                           uint8_t* __restrict__ vy, int64_t ne00,
+                                                           int64_t s01, int64_t s02, int64_t s03,
+                                                           int64_t ne0, int ne1, int ne2) {
+#pragma clang fp contract(off)
+    const int64_t i0 = ((int64_t)blockIdx.y * 256 + threadIdx.x) * 4;
+    if (i0 >= ne0) return;
+    const int row = blockIdx.x;
+    const int64_t channel = blockIdx.z % ne2, sample = blockIdx.z / ne2;
+    const int64_t src_row = ids ? ids[row] : row;
+    const T* xr = x + sample * s03 + channel * s02 + src_row * s01;
+
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i0 + 0 < ne00) v.x = to_f32<T>(xr[i0 + 0]);
+    if (i0 + 1 < ne00) v.y = to_f32<T>(xr[i0 + 1]);
+    if (i0 + 2 < ne00) v.z = to_f32<T>(xr[i0 + 2]);
+    if (i0 + 3 < ne00) v.w = to_f32<T>(xr[i0 + 3]);
+
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1));
+    amax = fmaxf(amax, __shfl_xor(amax, 2));
+    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    const float d = amax / 127.0f;
+    const float inv = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q0 = (int)roundf(v.x * inv), q1 = (int)roundf(v.y * inv);
+    const int q2 = (int)roundf(v.z * inv), q3 = (int)roundf(v.w * inv);
+    int sum = q0 + q1 + q2 + q3;
+    sum += __shfl_xor(sum, 1);
+    sum += __shfl_xor(sum, 2);
+    sum += __shfl_xor(sum, 4);
+
+    const int64_t kb = i0 / 256;
+    const int64_t blocks_per_channel = (ne0 / 256) * ne1;
+    uint8_t* rec = vy + ((int64_t)blockIdx.z * blocks_per_channel + kb * ne1 + row) * REC_BYTES;
+    const int in_rec = (int)(i0 % 256);
+    *(uint32_t*)(rec + in_rec) = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) |
+                                 ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
+    if ((in_rec & 31) == 0) {
+        const int s = in_rec >> 5;
+        *(uint16_t*)(rec + 256 + 2 * s) = __half_as_ushort(__float2half_rn(d));
+        *(int16_t*)(rec + 272 + 2 * s) = (int16_t)sum;
+    }
+}
+
+static void launch_quantize(const void* x, const int32_t* ids, void* vy, int type_x, int64_t ne00,
+                            int64_t s01, int64_t s02, int64_t s03, int64_t ne0, int64_t ne1,
+                            int64_t ne2, int64_t ne3, void* stream) {
+    if (!x || !vy || ne1 <= 0 || ne0 <= 0 || ne0 % 256 != 0 || ne2 <= 0 || ne3 <= 0) return;
+    const dim3 grid((unsigned)ne1, (unsigned)((ne0 + 1023) / 1024), (unsigned)(ne2 * ne3));
+    hipStream_t s = (hipStream_t)stream;
+    if (type_x == LK_TYPE_F16) {
+        hipLaunchKernelGGL(mmq_quantize_kernel<__half>, grid, dim3(256), 0, s, (const __half*)x, ids,
+                           (uint8_t*)vy, ne00, s01, s02, s03, ne0, (int)ne1, (int)ne2);
+    } else {
+        hipLaunchKernelGGL(mmq_quantize_kernel<float>, grid, dim3(256), 0, s, (const float*)x, ids,
+                           (uint8_t*)vy, ne00, s01, s02, s03, ne0, (int)ne1, (int)ne2);
+    }
+    (void)hipGetLastError();
+}
+
+// --------------------------------------------------------------------------------------------
+// Weight formats: how one 256-value block of TN rows becomes int8 sub-block tiles + scales.
+// LDS per step:  wq[8][TN][32] int8, aq[8][TM][32] int8, wsc[NS][TN] f32, wmn[8][TN] f32 (Q4_K),
+//                ad8[8][TM] f32, ads[8][TM] f32 (Q4_K).   NS = weight scales per block (8 or 16).
+// --------------------------------------------------------------------------------------------
+struct MmqQ4K {
+    static constexpr int BLOCK_BYTES = Q4K_BYTES;
+    static constexpr int NS = 8;          // one weight scale per 32 values
+    static constexpr bool HAS_MIN = true;
+    static constexpr int BLOCKS_PER_STEP = 1;
+
+    // rows [n0, n0+TN) of block kb -> LDS
+    static __device__ __forceinline__ void stage(const uint8_t* __restrict__ w, int64_t nb, int kb, int n0,
+                                                 int n, int8_t* wq, float* wsc, float* wmn) {
+        for (int idx = threadIdx.x; idx < TN * 8; idx += MMQ_WG) {
+            const int row = idx >> 3, c = idx & 7;
+            const int gn = min(n0 + row, n - 1);
+            const uint4 q = *(const uint4*)(w + ((int64_t)gn * nb + kb) * Q4K_BYTES + 16 + 16 * c);
+            uint4 lo, hi;
+            lo.x = q.x & 0x0F0F0F0Fu; hi.x = (q.x >> 4) & 0x0F0F0F0Fu;
+            lo.y = q.y & 0x0F0F0F0Fu; hi.y = (q.y >> 4) & 0x0F0F0F0Fu;
+            lo.z = q.z & 0x0F0F0F0Fu; hi.z = (q.z >> 4) & 0x0F0F0F0Fu;
+            lo.w = q.w & 0x0F0F0F0Fu; hi.w = (q.w >> 4) & 0x0F0F0F0Fu;
+            const int p = c >> 1, h = c & 1;
+            *(uint4*)(wq + ((2 * p) * TN + row) * 32 + 16 * h) = lo;
+            *(uint4*)(wq + ((2 * p + 1) * TN + row) * 32 + 16 * h) = hi;
+        }
+        for (int row = threadIdx.x; row < TN; row += MMQ_WG) {
+            const bool live = n0 + row < n;
+            const int gn = min(n0 + row, n - 1);
+            const uint4 hdr = *(const uint4*)(w + ((int64_t)gn * nb + kb) * Q4K_BYTES);
+            const float d = live ? f16_bits_to_f32(hdr.x & 0xFFFFu) : 0.f;
+            const float dmin = live ? f16_bits_to_f32(hdr.x >> 16) : 0.f;
+            const uint8_t* p = (const uint8_t*)&hdr.y;  // the 12 packed bytes
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                int sc, mn;
+                if (j < 4) {
+                    sc = p[j] & 63;
+                    mn = p[j + 4] & 63;
+                } else {
+                    sc = (p[j + 4] & 0xF) | ((p[j - 4] >> 6) << 4);
+                    mn = (p[j + 4] >> 4) | ((p[j] >> 6) << 4);
+                }
+                wsc[j * TN + row] = d * (float)sc;
+                wmn[j * TN + row] = -(dmin * (float)mn);
+            }
+        }
+    }
+};
+
+// Token rows [m0, m0+TM) of block kb (record layout above) -> LDS. Rows at or past m_end read as
+// zeros. `col_of` maps a tile row to its workspace row (identity for the dense product).
+template <int TM, bool WITH_SUMS>
+static __device__ __forceinline__ void stage_tokens(const uint8_t* __restrict__ y, int64_t rows_total, int kb,
+                                                    int m0, int m_end, int8_t* aq, float* ad8, float* ads) {
+    for (int idx = threadIdx.x; idx < TM * 18; idx += MMQ_WG) {
+        const int r = idx / 18, c = idx % 18;
+        const bool live = m0 + r < m_end;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (live) v = *(const uint4*)(y + ((int64_t)kb * rows_total + m0 + r) * REC_BYTES + 16 * c);
+        if (c < 16) {
+            *(uint4*)(aq + ((c >> 1) * TM + r) * 32 + 16 * (c & 1)) = v;
+        } else if (c == 16) {
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int s = 0; s < 8; ++s) ad8[s * TM + r] = f16_bits_to_f32((w[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
+        } else if (WITH_SUMS) {
+            // sums ride one chunk after the scales of the same record
+            const uint4 dv = live ? *(const uint4*)(y + ((int64_t)kb * rows_total + m0 + r) * REC_BYTES + 256)
+                                  : make_uint4(0, 0, 0, 0);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w}, dw[4] = {dv.x, dv.y, dv.z, dv.w};
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const float d8 = f16_bits_to_f32((dw[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
+                const int sum = (int)(int16_t)((w[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
+                ads[s * TM + r] = d8 * (float)sum;
+            }
+        }
+    }
+}
+
+// One problem = one weight slab against a contiguous run of workspace rows.
+struct MmqProblem {
+    const uint8_t* w;      // [n][nb] blocks
+    const uint8_t* y;      // workspace records
+    float* dst;
+    const int32_t* ids_dst;  // nullable: destination row of workspace row c
+    int64_t nb;            // 256-value blocks per weight row
+    int64_t rows_total;    // rows the workspace was quantized with (record stride)
+    int64_t ldd;           // floats between destination rows
+    int n, m_begin, m_end;
+};
+
+template <class F, int TM, int WAVES_M>
+static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, int m0, uint8_t* lds) {
+    constexpr int WAVES_N = 4 / WAVES_M;
+    constexpr int JT = TN / (32 * WAVES_N), IT = TM / (32 * WAVES_M);
+    static_assert(JT >= 1 && IT >= 1, "tile does not split over four waves");
+
+    int8_t* wq = (int8_t*)lds;                       // [8][TN][32]
+    int8_t* aq = wq + 8 * TN * 32;                   // [8][TM][32]
+    float* wsc = (float*)(aq + 8 * TM * 32);         // [NS][TN]
+    float* wmn = wsc + F::NS * TN;                   // [8][TN]   (HAS_MIN)
+    float* ad8 = wmn + (F::HAS_MIN ? 8 * TN : 0);    // [8][TM]
+    float* ads = ad8 + 8 * TM;                       // [8][TM]   (HAS_MIN)
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wn = wave % WAVES_N, wm = wave / WAVES_N;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    v16f acc[IT][JT];
+#pragma unroll
+    for (int it = 0; it < IT; ++it)
+#pragma unroll
+        for (int jt = 0; jt < JT; ++jt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[it][jt][v] = 0.f;
+
+    for (int kb = 0; kb < pb.nb; ++kb) {
+        __syncthreads();  // the previous step's readers are done with the tiles
+        F::stage(pb.w, pb.nb, kb, n0, pb.n, wq, wsc, wmn);
+        stage_tokens<TM, F::HAS_MIN>(pb.y, pb.rows_total, kb, m0, pb.m_end, aq, ad8, ads);
+        __syncthreads();
+
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            v4i a[IT], b[JT];
+            float ws[JT];
+#pragma unroll
+            for (int it = 0; it < IT; ++it)
+                a[it] = *(const v4i*)(aq + (s * TM + (wm * IT + it) * 32 + l32) * 32 + 16 * lh);
+#pragma unroll
+            for (int jt = 0; jt < JT; ++jt) {
+                b[jt] = *(const v4i*)(wq + (s * TN + (wn * JT + jt) * 32 + l32) * 32 + 16 * lh);
+                ws[jt] = wsc[s * TN + (wn * JT + jt) * 32 + l32];
+            }
+#pragma unroll
+            for (int it = 0; it < IT; ++it) {
+                // d8 of the 16 tokens this lane's accumulator registers stand for
+                float d8v[16];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float4 t = *(const float4*)(ad8 + s * TM + (wm * IT + it) * 32 + 8 * g + 4 * lh);
+                    d8v[4 * g + 0] = t.x; d8v[4 * g + 1] = t.y; d8v[4 * g + 2] = t.z; d8v[4 * g + 3] = t.w;
+                }
+#pragma unroll
+                for (int jt = 0; jt < JT; ++jt) {
+                    v16i c = {0};
+                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[it], b[jt], c, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        acc[it][jt][v] = fmaf((float)c[v], ws[jt] * d8v[v], acc[it][jt][v]);
+                }
+            }
+        }
+        if (F::HAS_MIN) {
+            // acc += (d8*S)[token, s] * (-dmin*m)[s, n], s = 0..7: four K=2 f32 MFMAs per patch
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                float am[IT], bm[JT];
+#pragma unroll
+                for (int it = 0; it < IT; ++it) am[it] = ads[(2 * kk + lh) * TM + (wm * IT + it) * 32 + l32];
+#pragma unroll
+                for (int jt = 0; jt < JT; ++jt) bm[jt] = wmn[(2 * kk + lh) * TN + (wn * JT + jt) * 32 + l32];
+#pragma unroll
+                for (int it = 0; it < IT; ++it)
+#pragma unroll
+                    for (int jt = 0; jt < JT; ++jt)
+                        acc[it][jt] = __builtin_amdgcn_mfma_f32_32x32x2f32(am[it], bm[jt], acc[it][jt], 0, 0, 0);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int it = 0; it < IT; ++it)
+#pragma unroll
+        for (int jt = 0; jt < JT; ++jt) {
+            const int gn = n0 + (wn * JT + jt) * 32 + l32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int col = m0 + (wm * IT + it) * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
+                if (gn < pb.n && col < pb.m_end) {
+                    const int64_t drow = pb.ids_dst ? pb.ids_dst[col] : col;
+                    pb.dst[drow * pb.ldd + gn] = acc[it][jt][v];
+                }
+            }
+        }
+}
+
+template <class F, int TM>
+static constexpr int mmq_lds_bytes() {
+    return 8 * TN * 32 + 8 * TM * 32 + (F::NS * TN + (F::HAS_MIN ? 8 * TN : 0) + 8 * TM + (F::HAS_MIN ? 8 * TM : 0)) * 4;
+}
+
+// Dense product. Workgroup id -> (n tile, m tile) so that the m tiles of one n tile (which
+// re-read the same weight rows) are issued back to back on the same XCD: ids are dealt round
+// robin over the 8 XCDs, so the XCD is id % 8 and its local sequence id / 8.
+template <class F, int TM, int WAVES_M>
+__global__ __launch_bounds__(MMQ_WG) void mmq_dense_kernel(MmqProblem pb, int n_tiles, int m_tiles) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int id = blockIdx.x;
+    const int xcd = id & 7, seq = id >> 3;
+    const int m_tile = seq % m_tiles;
+    const int n_tile = (seq / m_tiles) * 8 + xcd;
+    if (n_tile >= n_tiles) return;
+    mmq_tile<F, TM, WAVES_M>(pb, n_tile * TN, pb.m_begin + m_tile * TM, lds);
+}
+
+template <typename K>
+static int prepare_kernel(K kernel, int lds_bytes) {
+    static std::mutex mu;
+    static std::unordered_map<const void*, bool> done;
+    std::lock_guard<std::mutex> lock(mu);
+    if (done.count((const void*)kernel)) return LK_OK;
+    if (lds_bytes > lk_device().lds_bytes) return LK_ERR_ARG;
+    if (lds_bytes > 48 * 1024 &&
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return LK_ERR_LAUNCH;
+    }
+    done[(const void*)kernel] = true;
+    return LK_OK;
+}
+
+template <class F, int TM, int WAVES_M>
+static int launch_dense_tm(const MmqProblem& pb, hipStream_t s) {
+    auto kernel = mmq_dense_kernel<F, TM, WAVES_M>;
+    constexpr int lds_bytes = mmq_lds_bytes<F, TM>();
+    if (prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
+    const int n_tiles = (pb.n + TN - 1) / TN;
+    const int m_tiles = (pb.m_end - pb.m_begin + TM - 1) / TM;
+    const int n_groups = (n_tiles + 7) / 8;
+    const int grid = n_groups * 8 * m_tiles;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(MMQ_WG), lds_bytes, s, pb, n_tiles, m_tiles);
+    return hipGetLastError() == hipSuccess ? TM : 0;
+}
+
+template <class F>
+static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x, int64_t nrows_x,
+                        int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, void* stream) {
+    if (!x || !y || !dst || ncols_x <= 0 || nrows_x <= 0 || ncols_y <= 0) return 0;
+    if (ncols_x % 256 != 0 || stride_row_x != ncols_x / 256 * F::BLOCKS_PER_STEP) return 0;
+    if (stride_col_dst < nrows_x || nrows_x > INT32_MAX || ncols_y > INT32_MAX) return 0;
+    MmqProblem pb{(const uint8_t*)x, (const uint8_t*)y, (float*)dst, nullptr, ncols_x / 256, ncols_y,
+                  stride_col_dst, (int)nrows_x, 0, (int)ncols_y};
+    hipStream_t s = (hipStream_t)stream;
+    if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s);
+    if (ncols_y <= 64) return launch_dense_tm<F, 64, 2>(pb, s);
+    return launch_dense_tm<F, 128, 2>(pb, s);
+}
+
+}  // namespace
+
+extern "C" void launch_mmq_quantize_q8_1_D4(const void* x, const int32_t* ids, void* vy, int type_x,
+                                            int64_t ne00, int64_t s01, int64_t s02, int64_t s03,
+                                            int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3, void* stream) {
+    launch_quantize(x, ids, vy, type_x, ne00, s01, s02, s03, ne0, ne1, ne2, ne3, stream);
+}
+
+extern "C" void launch_mmq_quantize_q8_1_DS4(const void* x, const int32_t* ids, void* vy, int type_x,
+                                             int64_t ne00, int64_t s01, int64_t s02, int64_t s03,
+                                             int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3, void* stream) {
+    launch_quantize(x, ids, vy, type_x, ne00, s01, s02, s03, ne0, ne1, ne2, ne3, stream);
+}
+
+extern "C" int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* y, void* dst,
+                                    int64_t ncols_x, int64_t nrows_x, int64_t ncols_y,
+                                    int64_t stride_row_x, int64_t stride_col_dst, int cc, int nsm,
+                                    int64_t smpbo, int warp_size, void* stream) {
+    (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
+    return launch_dense<MmqQ4K>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
+}

@@ -61,3 +61,47 @@ def mmvq_subdots(wtype: int, weight: torch.Tensor, q8_1_row: torch.Tensor, k: in
     _lib.check("lk_mmvq_subdots", _lib.load().lk_mmvq_subdots(
         wtype, weight.data_ptr(), q8_1_row.data_ptr(), dots.data_ptr(), sums.data_ptr(), k, n, _stream()))
     return dots, sums
+
+
+# ------------------------------------------------------------------------------------ prefill
+MMQ_QUANTIZER = {_lib.TYPE_Q4_K: "launch_mmq_quantize_q8_1_DS4", _lib.TYPE_Q6_K: "launch_mmq_quantize_q8_1_D4",
+                 _lib.TYPE_Q8_0: "launch_mmq_quantize_q8_1_D4"}
+MMQ_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_gguf_q4_k", _lib.TYPE_Q6_K: "launch_mmq_gguf_q6_k",
+                _lib.TYPE_Q8_0: "launch_mmq_gguf_q8_0"}
+MMQ_DEVICE_INFO = dict(cc=0x1000950, nsm=256, smpbo=160 * 1024, warp_size=64)
+
+
+def mmq_workspace_bytes(rows: int, k: int) -> int:
+    """The reference's sizing (kernel_matmul/mmq.rs:38-41): 144 bytes per 128 padded values per
+    row, plus 128 records of slack."""
+    k_padded = pad_to(pad_to(k, 512), 128)
+    return rows * (k_padded // 128) * 144 + 128 * 144
+
+
+def mmq_quantize(wtype: int, x: torch.Tensor, gather: torch.Tensor | None = None,
+                 rows: int | None = None) -> torch.Tensor:
+    """Rows of ``x`` ``[_, k]`` (f32 or f16) into the tile kernels' workspace; row ``i`` of the
+    result is row ``gather[i]`` of ``x`` when a gather is given (MmqRouting::quantize)."""
+    k = x.shape[1]
+    rows = (gather.numel() if gather is not None else x.shape[0]) if rows is None else rows
+    k_padded = pad_to(pad_to(k, 512), 128)
+    ws = torch.empty(mmq_workspace_bytes(rows, k), dtype=torch.uint8, device=x.device)
+    fn = getattr(_lib.load(), MMQ_QUANTIZER[wtype])
+    fn(x.data_ptr(), gather.data_ptr() if gather is not None else None, ws.data_ptr(),
+       1 if x.dtype == torch.float16 else 0, k, x.stride(0), 0, 0, k_padded, rows, 1, 1, _stream())
+    return ws
+
+
+def mmq_forward(wtype: int, weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tensor:
+    """``[rows, k]`` x weight ``[n, k]`` -> ``[rows, n]`` f32 through the tiled kernels, the two
+    launches of QKernelMatMul::mmq_forward (kernel_matmul/mmq.rs:103-136)."""
+    rows, k = x.shape
+    ws = mmq_quantize(wtype, x)
+    out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
+    fn = getattr(_lib.load(), MMQ_LAUNCHER[wtype])
+    i = MMQ_DEVICE_INFO
+    launched = fn(None, weight.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, rows, k // BLOCK_LEN[wtype], n,
+                  i["cc"], i["nsm"], i["smpbo"], i["warp_size"], _stream())
+    if launched == 0:
+        raise _lib.LokenError(MMQ_LAUNCHER[wtype], _lib.LK_ERR_ARG)
+    return out

@@ -1,0 +1,156 @@
+"""GPU parity of the prefill path (workspace quantizer + int8-MFMA tiled matmul).
+
+Same bars as the decode path: workspace codes / scales / sums bit-exact with loken's
+BlockQ8_1::quantize; f32 outputs within 1e-3 relative + 1e-4 absolute of the same-codes oracle;
+and the family-vs-family check the reference runs (tiled matmul vs mat-vec on the same weights,
+src/tensor/quantized/tests.rs:848-921), here to a much tighter bound since both families see
+identical integer codes.
+"""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+import oracle
+from loken_amd import lib, ops, synth
+
+pytestmark = pytest.mark.gpu
+
+DT = {"q4_k": lib.TYPE_Q4_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0}
+SERVED = [name for name in DT if hasattr(lib.load(), ops.MMQ_LAUNCHER[DT[name]])]
+RTOL, ATOL = 1e-3, 1e-4
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def assert_close(got, want):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    bad = np.abs(got - want) > RTOL * np.abs(want) + ATOL
+    assert not bad.any(), f"{bad.sum()} of {bad.size} outside tolerance; worst {np.abs(got - want).max()}"
+
+
+def unpack_workspace(ws: np.ndarray, rows: int, k_padded: int):
+    """-> codes int8 [rows, k_padded], d f16 [rows, k_padded/32], sums int16 [rows, k_padded/32]"""
+    nkb = k_padded // 256
+    rec = ws[: nkb * rows * 288].reshape(nkb, rows, 288)
+    codes = rec[:, :, :256].copy().view(np.int8).transpose(1, 0, 2).reshape(rows, k_padded)
+    d = rec[:, :, 256:272].copy().view(np.float16).transpose(1, 0, 2).reshape(rows, nkb * 8)
+    sums = rec[:, :, 272:288].copy().view(np.int16).transpose(1, 0, 2).reshape(rows, nkb * 8)
+    return codes, d, sums
+
+
+@pytest.mark.parametrize("rows,k", [(1, 256), (7, 1000), (130, 4096), (33, 768)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_workspace_quantizer_is_bit_exact(rows, k, f16):
+    x = synth.activation(rows, k, seed=41) * np.float32(1.7)
+    xt = dev(x).to(torch.float16) if f16 else dev(x)
+    x_seen = xt.to(torch.float32).cpu().numpy()
+    kp = ops.pad_to(k, 512)
+    ws = ops.mmq_quantize(lib.TYPE_Q4_K, xt).cpu().numpy()
+    codes, d, sums = unpack_workspace(ws, rows, kp)
+    padded = np.zeros((rows, kp), np.float32)
+    padded[:, :k] = x_seen
+    want = oracle.quantize_q8_1(padded).reshape(rows, kp // 32, 36)
+    assert np.array_equal(codes.reshape(rows, kp // 32, 32), want[:, :, 4:].view(np.int8))
+    assert np.array_equal(d.view(np.uint16), want[:, :, 0:2].copy().view(np.uint16).reshape(rows, -1))
+    assert np.array_equal(sums.astype(np.int32), want[:, :, 4:].view(np.int8).astype(np.int32).sum(axis=2))
+
+
+def test_workspace_quantizer_gathers_rows():
+    x = synth.activation(9, 512, seed=42)
+    ids = np.array([3, 3, 0, 8, 1, 1, 1, 7], np.int32)
+    ws = ops.mmq_quantize(lib.TYPE_Q4_K, dev(x), gather=dev(ids)).cpu().numpy()
+    codes, d, _ = unpack_workspace(ws, len(ids), 512)
+    want = oracle.quantize_q8_1(x[ids]).reshape(len(ids), 16, 36)
+    assert np.array_equal(codes.reshape(len(ids), 16, 32), want[:, :, 4:].view(np.int8))
+    assert np.array_equal(d.view(np.uint16), want[:, :, 0:2].copy().view(np.uint16).reshape(len(ids), -1))
+
+
+SHAPES = [(6, 256, 128), (8, 512, 64), (33, 768, 130), (64, 1024, 256), (65, 1024, 129), (128, 2048, 384),
+          (200, 4096, 300), (1, 256, 1), (129, 256, 257)]
+
+
+@pytest.mark.parametrize("name", SERVED)
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_tiled_matmul_matches_same_codes_oracle(name, m, k, n):
+    wtype = DT[name]
+    w = synth.weight(wtype, n, k, seed=43, stream=1)
+    x = synth.activation(m, k, seed=43)
+    got = ops.mmq_forward(wtype, dev(w), dev(x), n).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(wtype, x, w, n))
+
+
+@pytest.mark.parametrize("name", SERVED)
+def test_tiled_matmul_agrees_with_matvec_family(name):
+    wtype = DT[name]
+    m, k, n = 40, 2048, 520
+    w = dev(synth.weight(wtype, n, k, seed=44, stream=2))
+    x = dev(synth.activation(m, k, seed=44))
+    tiled = ops.mmq_forward(wtype, w, x, n)
+    q = ops.quantize_q8_1_rows(x)
+    rows = torch.cat([ops.mmvq(wtype, w, q[i:i + 8], k, n) for i in range(0, m, 8)])
+    # same integers on both sides: only f32 summation order differs
+    scale = rows.abs().max().item()
+    assert (tiled - rows).abs().max().item() <= 2e-5 * scale
+
+
+@pytest.mark.parametrize("name", SERVED)
+def test_exact_activation_grid_leaves_only_summation_order(name):
+    # activations n * 2^-6 with one |n| = 127 per block quantize exactly
+    # (the construction of src/inference/moe_cuda/imma_reference.rs:17-29)
+    wtype = DT[name]
+    m, k, n = 16, 1024, 96
+    rng = np.random.default_rng(45)
+    a = rng.integers(-127, 128, (m, k))
+    a[:, ::32] = 127
+    x = (a * 2.0 ** -6).astype(np.float32)
+    w = synth.weight(wtype, n, k, seed=45, stream=3)
+    got = ops.mmq_forward(wtype, dev(w), dev(x), n).cpu().numpy()
+    ref = oracle.ob_matmul_f64(wtype, x, w, n)
+    wd = np.abs(oracle.dequantize(wtype, w).reshape(n, k).astype(np.float64))
+    bound = 1e-5 * (np.abs(x.astype(np.float64)) @ wd.T)
+    assert (np.abs(got - ref) <= bound + 1e-9).all()
+
+
+@pytest.mark.parametrize("name", SERVED)
+def test_launcher_declines_what_it_cannot_tile(name):
+    wtype = DT[name]
+    fn = getattr(lib.load(), ops.MMQ_LAUNCHER[wtype])
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    i = ops.MMQ_DEVICE_INFO
+    s = torch.cuda.current_stream().cuda_stream
+    p = buf.data_ptr()
+    blk = synth.BLOCK_LEN[wtype]
+    # k not a multiple of 256, a wrong block stride, no rows: 0 = nothing ran
+    assert fn(None, p, p, p, 128, 4, 4, 128 // blk, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
+    assert fn(None, p, p, p, 256, 4, 4, 256 // blk + 1, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
+    assert fn(None, p, p, p, 256, 4, 0, 256 // blk, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
+    assert fn(None, None, p, p, 256, 4, 4, 256 // blk, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
+
+
+@pytest.mark.parametrize("name,m,k,n", [("q4_k", 512, 4096, 14336), ("q6_k", 2048, 14336, 4096)])
+def test_full_benchmark_size_against_matvec_and_sampled_oracle(name, m, k, n):
+    if name not in SERVED:
+        pytest.skip(f"{name} tile kernel not built")
+    wtype = DT[name]
+    w = synth.weight(wtype, n, k, seed=0, stream=20)
+    x = synth.activation(m, k, seed=0, stream=21)
+    wd, xd = dev(w), dev(x)
+    tiled = ops.mmq_forward(wtype, wd, xd, n)
+    # 1. a sample of token rows against the mat-vec family over ALL weight rows
+    rows = [0, 1, 2, 3, m // 2, m // 2 + 1, m - 2, m - 1]
+    q = ops.quantize_q8_1_rows(xd[rows].contiguous())
+    vec = ops.mmvq(wtype, wd, q, k, n)
+    assert (tiled[rows] - vec).abs().max().item() <= 2e-5 * vec.abs().max().item()
+    # 2. a sample of (token, weight row) pairs against the CPU oracle
+    rng = np.random.default_rng(46)
+    tok = np.sort(rng.choice(m, 12, replace=False))
+    wr = np.sort(rng.choice(n, 300, replace=False))
+    want = oracle.ob_matmul(wtype, x[tok], w[wr], len(wr))
+    assert_close(tiled.cpu().numpy()[np.ix_(tok, wr)], want)
+    # 3. size-independent property: permuting token rows permutes output rows, bit for bit
+    perm = torch.randperm(m, device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+    assert torch.equal(ops.mmq_forward(wtype, wd, xd[perm].contiguous(), n), tiled[perm])
