@@ -121,6 +121,15 @@ int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* y, void* ds
                          int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
                          int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
                          void* stream);
+int launch_mmq_gguf_q6_k(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+/* Q8_0 rows are 32-value blocks (stride_row_x = k / 32); k must still be a multiple of 256. */
+int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
 
 #ifdef __cplusplus
 }

@@ -115,6 +115,7 @@ struct MmqQ4K {
     // rows [n0, n0+TN) of block kb -> LDS
     static __device__ __forceinline__ void stage(const uint8_t* __restrict__ w, int64_t nb, int kb, int n0,
                                                  int n, int8_t* wq, float* wsc, float* wmn) {
+        // nb: Q4_K blocks between consecutive rows
         for (int idx = threadIdx.x; idx < TN * 8; idx += MMQ_WG) {
             const int row = idx >> 3, c = idx & 7;
             const int gn = min(n0 + row, n - 1);
@@ -148,6 +149,74 @@ struct MmqQ4K {
                 wsc[j * TN + row] = d * (float)sc;
                 wmn[j * TN + row] = -(dmin * (float)mn);
             }
+        }
+    }
+};
+
+// Q6_K: sixteen int8 scales per block, one per 16 values, so one MFMA K (32) spans two of them;
+// the tile loop runs each 32-group as two MFMAs over half-masked weight operands.
+struct MmqQ6K {
+    static constexpr int BLOCK_BYTES = Q6K_BYTES;
+    static constexpr int NS = 16;
+    static constexpr bool HAS_MIN = false;
+    static constexpr int BLOCKS_PER_STEP = 1;
+
+    static __device__ __forceinline__ uint32_t word(uint32_t ql, uint32_t qh, int nib_shift, int hi_shift) {
+        const uint32_t code = ((ql >> nib_shift) & 0x0F0F0F0Fu) | (((qh >> hi_shift) & 0x03030303u) << 4);
+        return (code + 0x60606060u) ^ 0x80808080u;  // per byte: code - 32, signed
+    }
+    static __device__ __forceinline__ void stage(const uint8_t* __restrict__ w, int64_t nb, int kb, int n0,
+                                                 int n, int8_t* wq, float* wsc, float* wmn) {
+        (void)wmn;
+        for (int idx = threadIdx.x; idx < TN * 8; idx += MMQ_WG) {
+            const int row = idx >> 3, c = idx & 7;
+            const int h = c >> 2, g0 = (c >> 1) & 1, lh = c & 1;
+            const int gn = min(n0 + row, n - 1);
+            const uint8_t* bp = w + ((int64_t)gn * nb + kb) * Q6K_BYTES;
+            const uint4 ql = *(const uint4_a2*)(bp + 16 * c);
+            const uint4 qh = *(const uint4_a2*)(bp + 128 + 16 * (2 * h + lh));
+            uint4 ca, cb;
+            const int sh = 2 * g0;
+            ca.x = word(ql.x, qh.x, 0, sh); cb.x = word(ql.x, qh.x, 4, sh + 4);
+            ca.y = word(ql.y, qh.y, 0, sh); cb.y = word(ql.y, qh.y, 4, sh + 4);
+            ca.z = word(ql.z, qh.z, 0, sh); cb.z = word(ql.z, qh.z, 4, sh + 4);
+            ca.w = word(ql.w, qh.w, 0, sh); cb.w = word(ql.w, qh.w, 4, sh + 4);
+            *(uint4*)(wq + ((4 * h + g0) * TN + row) * 32 + 16 * lh) = ca;
+            *(uint4*)(wq + ((4 * h + g0 + 2) * TN + row) * 32 + 16 * lh) = cb;
+        }
+        for (int idx = threadIdx.x; idx < TN * 16; idx += MMQ_WG) {
+            const int row = idx >> 4, j = idx & 15;
+            const bool live = n0 + row < n;
+            const int gn = min(n0 + row, n - 1);
+            const uint8_t* bp = w + ((int64_t)gn * nb + kb) * Q6K_BYTES;
+            const float d = live ? f16_bits_to_f32(*(const uint16_t*)(bp + 208)) : 0.f;
+            wsc[j * TN + row] = d * (float)((const int8_t*)bp)[192 + j];
+        }
+    }
+};
+
+// Q8_0: eight 34-byte blocks per 256-value step, codes copied as they are.
+struct MmqQ80 {
+    static constexpr int BLOCK_BYTES = Q80_BYTES;
+    static constexpr int NS = 8;
+    static constexpr bool HAS_MIN = false;
+    static constexpr int BLOCKS_PER_STEP = 8;
+
+    static __device__ __forceinline__ void stage(const uint8_t* __restrict__ w, int64_t nb, int kb, int n0,
+                                                 int n, int8_t* wq, float* wsc, float* wmn) {
+        (void)wmn;
+        for (int idx = threadIdx.x; idx < TN * 16; idx += MMQ_WG) {
+            const int row = idx >> 4, c = idx & 15, blk = c >> 1, h = c & 1;
+            const int gn = min(n0 + row, n - 1);
+            const uint8_t* bp = w + ((int64_t)gn * nb + (int64_t)kb * 8 + blk) * Q80_BYTES;
+            *(uint4*)(wq + (blk * TN + row) * 32 + 16 * h) = *(const uint4_a2*)(bp + 2 + 16 * h);
+        }
+        for (int idx = threadIdx.x; idx < TN * 8; idx += MMQ_WG) {
+            const int row = idx >> 3, blk = idx & 7;
+            const bool live = n0 + row < n;
+            const int gn = min(n0 + row, n - 1);
+            const uint8_t* bp = w + ((int64_t)gn * nb + (int64_t)kb * 8 + blk) * Q80_BYTES;
+            wsc[blk * TN + row] = live ? f16_bits_to_f32(*(const uint16_t*)bp) : 0.f;
         }
     }
 };
@@ -189,7 +258,8 @@ struct MmqProblem {
     const uint8_t* y;      // workspace records
     float* dst;
     const int32_t* ids_dst;  // nullable: destination row of workspace row c
-    int64_t nb;            // 256-value blocks per weight row
+    int64_t nb;            // K steps: 256-value blocks per weight row
+    int64_t row_blocks;    // format blocks between consecutive weight rows
     int64_t rows_total;    // rows the workspace was quantized with (record stride)
     int64_t ldd;           // floats between destination rows
     int n, m_begin, m_end;
@@ -223,21 +293,27 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
 
     for (int kb = 0; kb < pb.nb; ++kb) {
         __syncthreads();  // the previous step's readers are done with the tiles
-        F::stage(pb.w, pb.nb, kb, n0, pb.n, wq, wsc, wmn);
+        F::stage(pb.w, pb.row_blocks, kb, n0, pb.n, wq, wsc, wmn);
         stage_tokens<TM, F::HAS_MIN>(pb.y, pb.rows_total, kb, m0, pb.m_end, aq, ad8, ads);
         __syncthreads();
 
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             v4i a[IT], b[JT];
-            float ws[JT];
+            float ws[JT], ws2[JT];
 #pragma unroll
             for (int it = 0; it < IT; ++it)
                 a[it] = *(const v4i*)(aq + (s * TM + (wm * IT + it) * 32 + l32) * 32 + 16 * lh);
 #pragma unroll
             for (int jt = 0; jt < JT; ++jt) {
                 b[jt] = *(const v4i*)(wq + (s * TN + (wn * JT + jt) * 32 + l32) * 32 + 16 * lh);
-                ws[jt] = wsc[s * TN + (wn * JT + jt) * 32 + l32];
+                if constexpr (F::NS == 16) {
+                    ws[jt] = wsc[(2 * s) * TN + (wn * JT + jt) * 32 + l32];
+                    ws2[jt] = wsc[(2 * s + 1) * TN + (wn * JT + jt) * 32 + l32];
+                } else {
+                    ws[jt] = wsc[s * TN + (wn * JT + jt) * 32 + l32];
+                    ws2[jt] = 0.f;
+                }
             }
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
@@ -250,11 +326,26 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
                 }
 #pragma unroll
                 for (int jt = 0; jt < JT; ++jt) {
-                    v16i c = {0};
-                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[it], b[jt], c, 0, 0, 0);
+                    if constexpr (F::NS == 16) {
+                        // lanes 0-31 hold k 0..15 of the operand, lanes 32-63 k 16..31: masking one
+                        // half leaves the 16-value group the other weight scale does not govern
+                        const v4i zero = {0, 0, 0, 0};
+                        const v4i b_lo = lh == 0 ? b[jt] : zero, b_hi = lh == 0 ? zero : b[jt];
+                        v16i c0 = {0}, c1 = {0};
+                        c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[it], b_lo, c0, 0, 0, 0);
+                        c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[it], b_hi, c1, 0, 0, 0);
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        acc[it][jt][v] = fmaf((float)c[v], ws[jt] * d8v[v], acc[it][jt][v]);
+                        for (int v = 0; v < 16; ++v) {
+                            const float t = fmaf(ws2[jt], (float)c1[v], ws[jt] * (float)c0[v]);
+                            acc[it][jt][v] = fmaf(t, d8v[v], acc[it][jt][v]);
+                        }
+                    } else {
+                        v16i c = {0};
+                        c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[it], b[jt], c, 0, 0, 0);
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            acc[it][jt][v] = fmaf((float)c[v], ws[jt] * d8v[v], acc[it][jt][v]);
+                    }
                 }
             }
         }
@@ -344,10 +435,10 @@ template <class F>
 static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x, int64_t nrows_x,
                         int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, void* stream) {
     if (!x || !y || !dst || ncols_x <= 0 || nrows_x <= 0 || ncols_y <= 0) return 0;
-    if (ncols_x % 256 != 0 || stride_row_x != ncols_x / 256 * F::BLOCKS_PER_STEP) return 0;
+    if (ncols_x % 256 != 0 || stride_row_x < ncols_x / 256 * F::BLOCKS_PER_STEP) return 0;
     if (stride_col_dst < nrows_x || nrows_x > INT32_MAX || ncols_y > INT32_MAX) return 0;
-    MmqProblem pb{(const uint8_t*)x, (const uint8_t*)y, (float*)dst, nullptr, ncols_x / 256, ncols_y,
-                  stride_col_dst, (int)nrows_x, 0, (int)ncols_y};
+    MmqProblem pb{(const uint8_t*)x, (const uint8_t*)y, (float*)dst, nullptr, ncols_x / 256, stride_row_x,
+                  ncols_y, stride_col_dst, (int)nrows_x, 0, (int)ncols_y};
     hipStream_t s = (hipStream_t)stream;
     if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s);
     if (ncols_y <= 64) return launch_dense_tm<F, 64, 2>(pb, s);
@@ -374,4 +465,20 @@ extern "C" int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* 
                                     int64_t smpbo, int warp_size, void* stream) {
     (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
     return launch_dense<MmqQ4K>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
+}
+
+extern "C" int launch_mmq_gguf_q6_k(void* tmp_fixup, const void* x, const void* y, void* dst,
+                                    int64_t ncols_x, int64_t nrows_x, int64_t ncols_y,
+                                    int64_t stride_row_x, int64_t stride_col_dst, int cc, int nsm,
+                                    int64_t smpbo, int warp_size, void* stream) {
+    (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
+    return launch_dense<MmqQ6K>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
+}
+
+extern "C" int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* y, void* dst,
+                                    int64_t ncols_x, int64_t nrows_x, int64_t ncols_y,
+                                    int64_t stride_row_x, int64_t stride_col_dst, int cc, int nsm,
+                                    int64_t smpbo, int warp_size, void* stream) {
+    (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
+    return launch_dense<MmqQ80>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
 }

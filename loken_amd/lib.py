@@ -33,6 +33,8 @@ SIGNATURES = {
     "launch_mmq_quantize_q8_1_D4": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),
     "launch_mmq_quantize_q8_1_DS4": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),
     "launch_mmq_gguf_q4_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
+    "launch_mmq_gguf_q6_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
+    "launch_mmq_gguf_q8_0": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
 }
 
 _lib = None

@@ -124,9 +124,9 @@ def test_launcher_declines_what_it_cannot_tile(name):
     s = torch.cuda.current_stream().cuda_stream
     p = buf.data_ptr()
     blk = synth.BLOCK_LEN[wtype]
-    # k not a multiple of 256, a wrong block stride, no rows: 0 = nothing ran
+    # k not a multiple of 256, a row stride shorter than the row, no rows: 0 = nothing ran
     assert fn(None, p, p, p, 128, 4, 4, 128 // blk, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
-    assert fn(None, p, p, p, 256, 4, 4, 256 // blk + 1, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
+    assert fn(None, p, p, p, 256, 4, 4, 256 // blk - 1, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
     assert fn(None, p, p, p, 256, 4, 0, 256 // blk, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
     assert fn(None, None, p, p, 256, 4, 4, 256 // blk, 4, i["cc"], i["nsm"], i["smpbo"], 64, s) == 0
 
