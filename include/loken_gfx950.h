@@ -131,6 +131,62 @@ int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* y, void* ds
                          int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
                          void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * MoE prefill: expert-batched tiled matmul and the steps around it. Names and argument lists are
+ * loken's (src/tensor/quantized/mmq.rs:151-173; src/inference/moe_cuda/mmq_experts.rs:42-56),
+ * called as MmqRouting::{from_choices, gate_up_over, down_fold_over} call them (:183-557).
+ * ------------------------------------------------------------------------------------- */
+
+/* For each expert e < n_experts: slab `x + e * stride_expert_x` (bytes) of nrows_x rows against
+ * the workspace rows [expert_bounds[e], expert_bounds[e+1]) of `y` (ncols_y rows in all, sorted
+ * by expert); workspace row c is written to destination row ids_dst[c] (or c when ids_dst is
+ * null), rows `stride_col_dst` floats apart. A second stack `x_second` of the same shape is
+ * multiplied in the same launch, its results `dst_second` floats after the first's in each row.
+ * ncols_max sizes the grid's column-tile axis (longer runs are still covered), ncols_hint or a
+ * non-zero mmq_x picks the tile width. Returns the tile width launched, 0 when nothing ran.
+ * Replaces launch_mmq_moe_gguf_* (cuda/mmq_gguf/mmq_launch.cuh:212-319). */
+int launch_mmq_moe_gguf_q4_k(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_q6_k(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_q8_0(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+
+/* From a routing already sorted by expert: bounds[e] = first sorted row of expert >= e
+ * (n_experts + 1 entries), slots_out = slots, src_rows[i] = slots[i] / topk.
+ * cuda/moe/moe_mmq.cu:30-55,180-188. */
+void loken_moe_mmq_plan(const int32_t* experts, const int32_t* slots, int n, int topk, int n_experts,
+                        int32_t* bounds, int32_t* slots_out, int32_t* src_rows, void* stream);
+/* From the router's choices [n = tokens * topk]: groups the pairs by expert on the device.
+ * `counts` is n_experts ints of scratch. Rows of one expert come in ascending pair order (the
+ * reference leaves that order unspecified). cuda/moe/moe_mmq.cu:57-99,190-198. */
+void loken_moe_mmq_route(const int32_t* choices, int n, int topk, int n_experts, int32_t* counts,
+                         int32_t* bounds, int32_t* slots, int32_t* src_rows, void* stream);
+/* out[r, c] = silu(gu[r, c]) * gu[r, width + c] over gu [rows, 2 * width]. moe_mmq.cu:101-114. */
+void loken_moe_mmq_silu_mul(const float* gu, float* out, int64_t rows, int width, void* stream);
+/* gpt-oss gate: x = min(g + gb, limit), u' = clamp(u + ub, -limit, limit),
+ * out = x * sigmoid(alpha x) * (1 + u'); biases [n_experts, width], nullable. moe_mmq.cu:131-153. */
+void loken_moe_mmq_swiglu_oai(const float* gu, float* out, int64_t rows, int width,
+                              const int32_t* bounds, int n_experts, const float* gate_bias,
+                              const float* up_bias, float alpha, float limit, void* stream);
+/* out[t, c] += sum over k ascending of weights[p] * (pairs[p, c] + down_bias[choices[p], c]),
+ * p = t * topk + k; bias and choices nullable together. moe_mmq.cu:155-176. */
+void loken_moe_mmq_fold(const float* pairs, const float* weights, const int32_t* choices,
+                        const float* down_bias, float* out, int64_t tokens, int topk, int cols,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

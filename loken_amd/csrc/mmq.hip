@@ -402,6 +402,24 @@ __global__ __launch_bounds__(MMQ_WG) void mmq_dense_kernel(MmqProblem pb, int n_
     mmq_tile<F, TM, WAVES_M>(pb, n_tile * TN, pb.m_begin + m_tile * TM, lds);
 }
 
+// Expert-batched product: expert e's slab against the sorted rows [bounds[e], bounds[e+1]).
+// grid = (n tiles, column tiles sized for the longest run the host expects, stacks * experts);
+// a run longer than the grid covers is walked by the same workgroups in further passes.
+template <class F, int TM, int WAVES_M>
+__global__ __launch_bounds__(MMQ_WG) void mmq_moe_kernel(MmqProblem pb, const uint8_t* w_second,
+                                                         int64_t dst_second, const int32_t* __restrict__ bounds,
+                                                         int64_t stride_expert, int n_experts) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int stack = blockIdx.z / n_experts, e = blockIdx.z % n_experts;
+    pb.m_begin = bounds[e];
+    pb.m_end = bounds[e + 1];
+    if (pb.m_end <= pb.m_begin) return;
+    pb.w = (stack ? w_second : pb.w) + (int64_t)e * stride_expert;
+    if (stack) pb.dst += dst_second;
+    for (int m0 = pb.m_begin + blockIdx.y * TM; m0 < pb.m_end; m0 += gridDim.y * TM)
+        mmq_tile<F, TM, WAVES_M>(pb, blockIdx.x * TN, m0, lds);
+}
+
 template <typename K>
 static int prepare_kernel(K kernel, int lds_bytes) {
     static std::mutex mu;
@@ -445,6 +463,41 @@ static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x
     return launch_dense_tm<F, 128, 2>(pb, s);
 }
 
+template <class F, int TM, int WAVES_M>
+static int launch_moe_tm(const MmqProblem& pb, const uint8_t* w_second, int64_t dst_second,
+                         const int32_t* bounds, int64_t stride_expert, int n_experts, int64_t ncols_max,
+                         hipStream_t s) {
+    auto kernel = mmq_moe_kernel<F, TM, WAVES_M>;
+    constexpr int lds_bytes = mmq_lds_bytes<F, TM>();
+    if (prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
+    const int64_t col_tiles = (ncols_max + TM - 1) / TM;
+    const dim3 grid((pb.n + TN - 1) / TN, (unsigned)(col_tiles < 1 ? 1 : (col_tiles > 65535 ? 65535 : col_tiles)),
+                    (unsigned)((w_second ? 2 : 1) * n_experts));
+    hipLaunchKernelGGL(kernel, grid, dim3(MMQ_WG), lds_bytes, s, pb, w_second, dst_second, bounds,
+                       stride_expert, n_experts);
+    return hipGetLastError() == hipSuccess ? TM : 0;
+}
+
+template <class F>
+static int launch_moe(const void* x, const void* x_second, int64_t dst_second, const void* y, void* dst,
+                      const int* expert_bounds, const int* ids_dst, int64_t stride_expert_x,
+                      int64_t ncols_x, int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                      int64_t stride_col_dst, int n_experts, int64_t ncols_max, int64_t ncols_hint,
+                      int mmq_x, void* stream) {
+    if (!x || !y || !dst || !expert_bounds || ncols_x <= 0 || nrows_x <= 0 || ncols_y <= 0 || n_experts <= 0) return 0;
+    if (ncols_x % 256 != 0 || stride_row_x < ncols_x / 256 * F::BLOCKS_PER_STEP) return 0;
+    if (nrows_x > INT32_MAX || ncols_y > INT32_MAX || (int64_t)n_experts * 2 > 65535) return 0;
+    MmqProblem pb{(const uint8_t*)x, (const uint8_t*)y, (float*)dst, ids_dst, ncols_x / 256, stride_row_x,
+                  ncols_y, stride_col_dst, (int)nrows_x, 0, 0};
+    hipStream_t s = (hipStream_t)stream;
+    const uint8_t* w2 = (const uint8_t*)x_second;
+    // the narrowest tile at or above what was asked for, else one sized for the expected run
+    const int64_t want = mmq_x > 0 ? mmq_x : (ncols_hint > 0 ? ncols_hint : ncols_max);
+    if (want <= 32) return launch_moe_tm<F, 32, 1>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
+    if (want <= 64) return launch_moe_tm<F, 64, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
+    return launch_moe_tm<F, 128, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
+}
+
 }  // namespace
 
 extern "C" void launch_mmq_quantize_q8_1_D4(const void* x, const int32_t* ids, void* vy, int type_x,
@@ -482,3 +535,20 @@ extern "C" int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* 
     (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
     return launch_dense<MmqQ80>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
 }
+
+#define LK_MMQ_MOE_ENTRY(NAME, FMT)                                                                     \
+    extern "C" int NAME(const void* x, const void* x_second, int64_t dst_second, const void* y,        \
+                        void* dst, const int* expert_bounds, const int* ids_dst,                       \
+                        int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x, int64_t ncols_y,    \
+                        int64_t stride_row_x, int64_t stride_col_dst, int n_experts, int64_t ncols_max, \
+                        int64_t ncols_hint, int mmq_x, int cc, int64_t smpbo, int warp_size,           \
+                        void* stream) {                                                                \
+        (void)cc; (void)smpbo; (void)warp_size;                                                        \
+        return launch_moe<FMT>(x, x_second, dst_second, y, dst, expert_bounds, ids_dst, stride_expert_x, \
+                               ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, n_experts,     \
+                               ncols_max, ncols_hint, mmq_x, stream);                                  \
+    }
+
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q4_k, MmqQ4K)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q6_k, MmqQ6K)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q8_0, MmqQ80)

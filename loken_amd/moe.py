@@ -1,0 +1,126 @@
+"""Host side of the MoE expert block, mirroring loken's ``MmqRouting``
+(src/inference/moe_cuda/mmq_experts.rs:108-736): group the routed pairs by expert, run gate and
+up as one expert-batched launch, apply the GLU, run down scattered back to slot order, fold each
+token's slots in slot order. torch holds the buffers; every computation is a C-ABI call.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import lib as _lib
+from .ops import MMQ_DEVICE_INFO, _stream, mmq_quantize
+from .synth import BLOCK_BYTES, BLOCK_LEN
+
+MMQ_MOE_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_moe_gguf_q4_k", _lib.TYPE_Q6_K: "launch_mmq_moe_gguf_q6_k",
+                    _lib.TYPE_Q8_0: "launch_mmq_moe_gguf_q8_0"}
+MMQ_X_MIN, GRID_Y_MAX = 8, 65535
+
+
+def moe_mmq_serves(wtype: int, k: int) -> bool:
+    """mmq_experts.rs:90-92; the tile kernels here walk 256 values per step."""
+    return wtype in MMQ_MOE_LAUNCHER and k % 256 == 0
+
+
+class MmqRouting:
+    """The routing in the form the expert-batched launches read it."""
+
+    def __init__(self, tokens: int, topk: int, n_experts: int, device):
+        rows = tokens * topk
+        self.tokens, self.topk, self.experts = tokens, topk, n_experts
+        self.bounds = torch.zeros(n_experts + 1, dtype=torch.int32, device=device)
+        self.slots = torch.zeros(rows, dtype=torch.int32, device=device)
+        self.src_rows = torch.zeros(rows, dtype=torch.int32, device=device)
+        self.choices = None
+        self.mmq_x = 0
+
+    @classmethod
+    def new(cls, slots: torch.Tensor, experts: torch.Tensor, topk: int, n_experts: int) -> "MmqRouting":
+        """From the stably sorted routing (mmq_experts.rs:157-176)."""
+        rows = slots.numel()
+        if rows % topk:
+            raise ValueError(f"moe mmq: {rows} routed rows is not a multiple of topk={topk}")
+        plan = cls(rows // topk, topk, n_experts, slots.device)
+        _lib.load().loken_moe_mmq_plan(experts.data_ptr(), slots.data_ptr(), rows, topk, n_experts,
+                                       plan.bounds.data_ptr(), plan.slots.data_ptr(),
+                                       plan.src_rows.data_ptr(), _stream())
+        return plan
+
+    @classmethod
+    def from_choices(cls, choices: torch.Tensor, n_experts: int) -> "MmqRouting":
+        """From the router's choices ``[tokens, topk]`` (mmq_experts.rs:183-206)."""
+        tokens, topk = choices.shape
+        choices = choices.to(torch.int32).contiguous()
+        plan = cls(tokens, topk, n_experts, choices.device)
+        counts = torch.zeros(n_experts, dtype=torch.int32, device=choices.device)
+        _lib.load().loken_moe_mmq_route(choices.data_ptr(), tokens * topk, topk, n_experts, counts.data_ptr(),
+                                        plan.bounds.data_ptr(), plan.slots.data_ptr(),
+                                        plan.src_rows.data_ptr(), _stream())
+        plan.choices = choices
+        return plan
+
+    def with_tile_width(self, mmq_x: int) -> "MmqRouting":
+        self.mmq_x = mmq_x
+        return self
+
+    @property
+    def rows(self) -> int:
+        return self.tokens * self.topk
+
+    def longest_run_expected(self) -> int:
+        """mmq_experts.rs:215-227: mean + sqrt(2 ln experts) deviations of a binomial count."""
+        experts = float(max(self.experts, 1))
+        p = min(self.topk / experts, 1.0)
+        mean = self.tokens * p
+        dev = math.sqrt(mean * (1.0 - p))
+        longest = mean + dev * math.sqrt(2.0 * math.log(experts)) if experts > 1 else mean
+        return max(1, min(int(math.ceil(longest)), max(self.tokens, 1)))
+
+    def _matmul(self, wtype: int, stack: torch.Tensor, second: torch.Tensor | None, second_offset: int,
+                n: int, k: int, y: torch.Tensor, dst: torch.Tensor, stride: int, ids_dst: torch.Tensor | None):
+        if not moe_mmq_serves(wtype, k):
+            raise ValueError(f"moe mmq: no expert-batched kernel for type {wtype} at k={k}")
+        blocks_per_row = k // BLOCK_LEN[wtype]
+        expert_bytes = n * blocks_per_row * BLOCK_BYTES[wtype]
+        longest = self.longest_run_expected()
+        i = MMQ_DEVICE_INFO
+        launched = getattr(_lib.load(), MMQ_MOE_LAUNCHER[wtype])(
+            stack.data_ptr(), second.data_ptr() if second is not None else None, second_offset, y.data_ptr(),
+            dst.data_ptr(), self.bounds.data_ptr(), ids_dst.data_ptr() if ids_dst is not None else None,
+            expert_bytes, k, n, self.rows, blocks_per_row, stride, self.experts,
+            min(longest, GRID_Y_MAX * MMQ_X_MIN), longest, self.mmq_x, i["cc"], i["smpbo"], i["warp_size"], _stream())
+        if launched == 0:
+            raise _lib.LokenError(MMQ_MOE_LAUNCHER[wtype], _lib.LK_ERR_ARG)
+
+    def gate_up_silu(self, wtype: int, xs: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, width: int) -> torch.Tensor:
+        """``silu(gate . x) * (up . x)`` for every routed row, in sorted order: ``[rows, width]``
+        (mmq_experts.rs:300-435). ``gate`` / ``up`` are stacks of ``[experts, width, k]`` blocks."""
+        tokens, k = xs.shape
+        if tokens != self.tokens:
+            raise ValueError(f"moe mmq: {tokens} tokens against a plan of {self.tokens}")
+        y = mmq_quantize(wtype, xs.to(torch.float32).contiguous(), gather=self.src_rows)
+        gu = torch.empty((self.rows, 2 * width), dtype=torch.float32, device=xs.device)
+        self._matmul(wtype, gate, up, width, width, k, y, gu, 2 * width, None)
+        out = torch.empty((self.rows, width), dtype=torch.float32, device=xs.device)
+        _lib.load().loken_moe_mmq_silu_mul(gu.data_ptr(), out.data_ptr(), self.rows, width, _stream())
+        return out
+
+    def down_fold(self, wtype: int, hs: torch.Tensor, down: torch.Tensor, hidden: int, topk_weights: torch.Tensor,
+                  residual: torch.Tensor | None = None) -> torch.Tensor:
+        """Down projection of the sorted rows ``hs`` ``[rows, k]``, each scaled by its router
+        weight and folded into its token in slot order: ``[tokens, hidden]`` (mmq_experts.rs:440-557)."""
+        rows, k = hs.shape
+        if rows != self.rows:
+            raise ValueError(f"moe mmq: {rows} rows against a plan of {self.rows}")
+        y = mmq_quantize(wtype, hs.contiguous())
+        pairs = torch.empty((rows, hidden), dtype=torch.float32, device=hs.device)
+        self._matmul(wtype, down, None, 0, hidden, k, y, pairs, hidden, self.slots)
+        out = (residual.reshape(self.tokens, hidden).to(torch.float32).clone() if residual is not None
+               else torch.zeros((self.tokens, hidden), dtype=torch.float32, device=hs.device))
+        w = topk_weights.to(torch.float32).contiguous()
+        if w.numel() != rows:
+            raise ValueError(f"moe mmq: {w.numel()} router weights for {rows} rows")
+        _lib.load().loken_moe_mmq_fold(pairs.data_ptr(), w.data_ptr(), None, None, out.data_ptr(), self.tokens,
+                                       self.topk, hidden, _stream())
+        return out

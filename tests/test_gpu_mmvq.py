@@ -158,7 +158,8 @@ def test_strided_destination_and_activation():
     x = synth.activation(3, k, seed=37)
     q = ops.quantize_q8_1_rows(dev(x), k_padded=1024)
     out = torch.full((3, 64), 7.0, device="cuda")
-    lib.check("lk_mmvq", lib.load().lk_mmvq(wtype, dev(w).data_ptr(), q.data_ptr(), out.data_ptr(),
+    wd = dev(w)
+    lib.check("lk_mmvq", lib.load().lk_mmvq(wtype, wd.data_ptr(), q.data_ptr(), out.data_ptr(),
                                             lib.TYPE_F32, k, n, 3, 1024 // 32, 64, None, 0,
                                             torch.cuda.current_stream().cuda_stream))
     got = out.cpu().numpy()
