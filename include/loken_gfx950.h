@@ -78,6 +78,33 @@ int lk_mmvq(int wtype, const void* vx, const void* vy_q8_1, void* dst, int dst_t
             int ncols_x, int nrows_x, int batch, int stride_col_y, int stride_col_dst,
             const float* bias, int decode_order, void* stream);
 
+/* Up to 4 weight matrices of one format and one k over the SAME activation rows in one launch:
+ * matrix i has nrows_x[i] rows and writes dst[i] (bias[i] nullable, `bias` itself nullable).
+ * The pointer arrays are host arrays. Every row carries the bits lk_mmvq gives it alone.
+ * Generalizes the two-matrix launch `mmvq_gguf_{tag}_f32_plain_dual_cuda1` / mmvq_f32_dual
+ * (src/inference/cuda/mmvq_gguf.cu:515-545; src/tensor/cuda/quant.rs:3369-3413), which attention
+ * uses for q and k; three matrices serve q, k, v of a layer at once. */
+int lk_mmvq_multi(int wtype, int count, const void* const* vx, const void* vy_q8_1, void* const* dst,
+                  int dst_type, int ncols_x, const int* nrows_x, int batch, int stride_col_y,
+                  int stride_col_dst, const float* const* bias, void* stream);
+
+/* dst[j, row] = act(gate row . x_j) * (up row . x_j), act 0 = SiLU g/(1+exp(-g)), 1 = tanh-GELU;
+ * gate and up have the same shape; batch 1..4; dst f32 or bf16. Replaces kernels
+ * `mmvq_gguf_pair_{g}_{u}_silu*_cuda1` and `mmvq_gguf_q4_k_{f32,bf16}_fused_{silu,gelu}_cuda1`
+ * with fast_mmvq::try_fused (src/inference/cuda/mmvq_gguf.cu:588-758;
+ * src/tensor/quantized/fast_mmvq.rs:97-282). */
+int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, const void* vy_q8_1, void* dst,
+                     int dst_type, int ncols_x, int nrows_x, int batch, int stride_col_y,
+                     int stride_col_dst, int act, void* stream);
+
+/* `groups` weights of one shape [nrows_x, ncols_x], each over its OWN Q8_1 row: weight g lives at
+ * device address table[g] (a device array), reads the blocks from g * ncols_x/32 of vy_q8_1 and
+ * writes dst from g * nrows_x. ncols_x must be a multiple of 512. Replaces kernel
+ * `mmvq_gguf_{tag}_f32_plain_grouped_cuda1` / mmvq_f32_grouped
+ * (src/inference/cuda/mmvq_gguf.cu:547-565; src/tensor/cuda/quant.rs:3418-3466). */
+int lk_mmvq_grouped(int wtype, const uint64_t* table, int groups, const void* vy_q8_1, float* dst,
+                    int ncols_x, int nrows_x, void* stream);
+
 /* Parity probe: the exact integer sub-block dot products the mat-vec kernels form, for ONE
  * activation row. dots: Q4_K int32[nrows_x][ncols_x/32] (sum over 32 of nibble*q8),
  * Q6_K int32[nrows_x][ncols_x/16] (sum over 16 of (code-32)*q8), Q8_0 int32[nrows_x][ncols_x/32].

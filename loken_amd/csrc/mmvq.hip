@@ -1,413 +1,95 @@
-// Decode mat-vec: GGUF weight rows (Q4_K / Q6_K / Q8_0) against 1..8 Q8_1 activation rows.
+// Decode mat-vec launchers: GGUF weight rows (Q4_K / Q6_K / Q8_0) against 1..8 Q8_1 activation
+// rows, plus the fused neighbours that share its engine (several matrices over one activation,
+// gate/up pairs with the activation function applied in the store, grouped launches).
 //
 // Bandwidth work, so the design is about bytes in flight, not arithmetic:
-//   * a lane loads 16 weight bytes per instruction (global_load_dwordx4) and a wave takes whole
-//     super-blocks side by side: Q4_K / Q6_K 8 lanes per 256-value block (8 blocks = 2048 values
-//     per wave pass), Q8_0 2 lanes per 32-value block (32 blocks = 1024 values per pass);
-//   * a wave owns R consecutive weight rows end to end (no cross-wave reduction), issues the
-//     loads of all R rows before it consumes any, and persists over row tiles;
+//   * a lane loads 16 weight bytes per instruction (global_load_dwordx4); a wave takes whole
+//     super-blocks side by side (Q4_K 4 lanes per 256-value block and 16 blocks = 4096 values
+//     per pass; Q6_K 8 lanes per block; Q8_0 2 lanes per 32-value block);
+//   * a wave owns R consecutive weight rows end to end (no cross-wave reduction) and persists
+//     over row tiles, with the next tile's loads in flight while the current one is consumed;
 //   * the Q8_1 activation is staged ONCE per workgroup into LDS, re-laid so that the 16 bytes a
 //     lane needs sit at lane*16 of a plane (conflict-free ds_read_b128), with its f16 scales
 //     widened to f32 and, for Q4_K, d8 * sum(codes) precomputed for the min term;
 //   * 6-bit scales / mins are unpacked in registers from the 16-byte block header;
-//   * integer products are v_dot4_i32_i8; the per-lane f32 partials meet in one wave64 DPP
+//   * integer products are v_dot4_i32_i8; per-lane f32 partials meet in one wave64 DPP
 //     reduction per row.
-//
-// What each format computes follows loken's definitions: src/tensor/quant_cpu/format/q4_k.rs:62-88,
-// q6_k.rs:51-82, q8_0.rs:83-97 for the integer sums, and the Q8_1-side combine of
-// cuda/moe/gguf.cuh:664-685 (Q4_K), 782-816 (Q6_K), 486-495 (Q8_0).
+// The engines live in mmvq_core.h.
 
-#include "lk_common.h"
+#include "mmvq_core.h"
 
 #include <cstdlib>
 #include <mutex>
 #include <unordered_map>
 
+using namespace mmvq;
+
 namespace {
 
-constexpr int WG = 256;            // threads per workgroup
-constexpr int WAVES = WG / LK_WAVE;
-
-// --------------------------------------------------------------------------------------------
-// Integer cores: what one lane forms from its 16 weight bytes. Shared by the mat-vec kernels and
-// the sub-block-dot probe, so the probe shows the integers the product is built from.
-// --------------------------------------------------------------------------------------------
-
-// Q4_K: 16 bytes of qs = values l..l+15 of sub-block 2p (low nibbles) and of 2p+1 (high nibbles).
-// Adds their products with the matching 16 activation codes of each sub-block into d_lo / d_hi.
-static __device__ __forceinline__ void q4k_dots(const uint4& q, const uint4& a_lo, const uint4& a_hi,
-                                                int& d_lo, int& d_hi) {
-    uint4 lo, hi;
-    lo.x = q.x & 0x0F0F0F0Fu; hi.x = (q.x >> 4) & 0x0F0F0F0Fu;
-    lo.y = q.y & 0x0F0F0F0Fu; hi.y = (q.y >> 4) & 0x0F0F0F0Fu;
-    lo.z = q.z & 0x0F0F0F0Fu; hi.z = (q.z >> 4) & 0x0F0F0F0Fu;
-    lo.w = q.w & 0x0F0F0F0Fu; hi.w = (q.w >> 4) & 0x0F0F0F0Fu;
-    d_lo = dot16(lo, a_lo, d_lo);
-    d_hi = dot16(hi, a_hi, d_hi);
-}
-
-// The (scale, min) pairs of sub-blocks 2p, 2p+1 from the 12 packed bytes (words w1..w3 of the
-// block header): scales in bits 0-7 / 8-15 of `sc`, mins likewise in `mn`. Sub-blocks 0-3 keep
-// their six bits in one byte; 4-7 take a nibble from bytes 8-11 and two bits from the top of
-// bytes 0-7. The selectors depend on the lane only, so they are built once outside any loop.
-struct Q4KScaleSel {
-    uint32_t shift, first, mask_main, mask_top;
-    __device__ __forceinline__ explicit Q4KScaleSel(int p)
-        : shift(16 * (p & 1)), first(p < 2), mask_main(p < 2 ? 0x3F3Fu : 0x0F0Fu), mask_top(p < 2 ? 0u : 0x3030u) {}
-    __device__ __forceinline__ void unpack(uint32_t w1, uint32_t w2, uint32_t w3, uint32_t& sc, uint32_t& mn) const {
-        const uint32_t a = w1 >> shift, b = w2 >> shift, c = w3 >> shift;
-        sc = ((first ? a : c) & mask_main) | ((a >> 2) & mask_top);
-        mn = ((first ? b : (c >> 4)) & mask_main) | ((b >> 2) & mask_top);
-    }
+// Up to four same-format, same-k matrices over one activation in one launch (q/k/v, gate/up).
+// Workgroups [wg_begin[i], wg_begin[i+1]) serve matrix i.
+constexpr int MAX_MULTI = 4;
+struct MultiArgs {
+    const uint8_t* vx[MAX_MULTI];
+    void* dst[MAX_MULTI];
+    const float* bias[MAX_MULTI];
+    int n[MAX_MULTI];
+    int wg_begin[MAX_MULTI + 1];
+    int count;
 };
 
-// Q6_K: 16 bytes of ql and the 16 bytes of qh over the same l give two runs of 16 signed codes:
-// run A in group g0 (low nibbles, qh bits 2*g0), run B in group g0+2 (high nibbles, bits 2*g0+4).
-static __device__ __forceinline__ uint32_t q6k_word(uint32_t ql, uint32_t qh, int nib_shift, int hi_shift) {
-    const uint32_t code = ((ql >> nib_shift) & 0x0F0F0F0Fu) | (((qh >> hi_shift) & 0x03030303u) << 4);
-    // per byte: code - 32 as a signed byte (code <= 63, so +0x60 cannot carry into the next byte)
-    return (code + 0x60606060u) ^ 0x80808080u;
-}
-static __device__ __forceinline__ void q6k_dots(const uint4& ql, const uint4& qh, int g0,
-                                                const uint4& a_a, const uint4& a_b, int& d_a, int& d_b) {
-    uint4 ca, cb;
-    const int s = 2 * g0;
-    ca.x = q6k_word(ql.x, qh.x, 0, s); cb.x = q6k_word(ql.x, qh.x, 4, s + 4);
-    ca.y = q6k_word(ql.y, qh.y, 0, s); cb.y = q6k_word(ql.y, qh.y, 4, s + 4);
-    ca.z = q6k_word(ql.z, qh.z, 0, s); cb.z = q6k_word(ql.z, qh.z, 4, s + 4);
-    ca.w = q6k_word(ql.w, qh.w, 0, s); cb.w = q6k_word(ql.w, qh.w, 4, s + 4);
-    d_a = dot16(ca, a_a, 0);
-    d_b = dot16(cb, a_b, 0);
-}
-
-// --------------------------------------------------------------------------------------------
-// Activation staging. Formats differ only in where a Q8_1 block's two 16-byte halves land.
-// LDS per activation row: `n_iter` passes x `PLANES` planes x 1024 bytes of codes, then the
-// scale table (SCF floats per Q8_1 block).
-// --------------------------------------------------------------------------------------------
-
-struct FmtQ4K {
-    static constexpr int BLOCK_BYTES = Q4K_BYTES, BLOCK_LEN = 256;
-    static constexpr int VPI = 4096;   // values per wave pass: 16 super-blocks, 4 lanes each
-    static constexpr int PLANES = 4, SCF = 2;
-    // j: Q8_1 block index inside the pass (0..127), lh: which 16-byte half of its codes.
-    // Lane (block lb, pair p) reads plane (2 * odd + lh) at lane * 16.
-    static __device__ __forceinline__ int slot(int j, int lh) {
-        const int lb = j >> 3, s = j & 7;
-        return ((s & 1) * 2 + lh) * 1024 + (lb * 4 + (s >> 1)) * 16;
-    }
-};
-struct FmtQ6K {
-    static constexpr int BLOCK_BYTES = Q6K_BYTES, BLOCK_LEN = 256;
-    static constexpr int VPI = 2048;
-    static constexpr int PLANES = 2, SCF = 1;
-    static __device__ __forceinline__ int slot(int j, int lh) {
-        const int lb = j >> 3, s = j & 7, h = s >> 2, g = s & 3;
-        return (g >> 1) * 1024 + (lb * 8 + h * 4 + (g & 1) * 2 + lh) * 16;
-    }
-};
-struct FmtQ80 {
-    static constexpr int BLOCK_BYTES = Q80_BYTES, BLOCK_LEN = 32;
-    static constexpr int VPI = 1024;
-    static constexpr int PLANES = 1, SCF = 1;
-    static __device__ __forceinline__ int slot(int j, int lh) { return j * 32 + lh * 16; }
-};
-
-template <class F>
-static __host__ __device__ constexpr int lds_bytes_per_row(int n_iter) {
-    return n_iter * F::VPI + n_iter * (F::VPI / 32) * F::SCF * 4;
-}
-
-// Stage `batch` Q8_1 rows. k32 = real Q8_1 blocks per row; the rest of the last pass is zeroed.
-template <class F, int B>
-static __device__ __forceinline__ void stage_activation(uint8_t* lds, const uint8_t* __restrict__ vy,
-                                                        int k32, int n_iter, int stride_col_y) {
-    const int per_pass = F::VPI / 32;
-    const int total = n_iter * per_pass;
-    const int row_bytes = lds_bytes_per_row<F>(n_iter);
-    for (int j = threadIdx.x; j < total; j += WG) {
-        const int it = j / per_pass, ji = j % per_pass;
-#pragma unroll
-        for (int c = 0; c < B; ++c) {
-            uint8_t* row = lds + c * row_bytes;
-            float* sc = (float*)(row + n_iter * F::VPI);
-            uint4 lo = make_uint4(0, 0, 0, 0), hi = make_uint4(0, 0, 0, 0);
-            float d8 = 0.f, ds = 0.f;
-            if (j < k32) {
-                const uint32_t* src = (const uint32_t*)(vy + ((size_t)c * stride_col_y + j) * Q81_BYTES);
-                const uint32_t head = src[0];
-                lo = make_uint4(src[1], src[2], src[3], src[4]);
-                hi = make_uint4(src[5], src[6], src[7], src[8]);
-                d8 = f16_bits_to_f32(head & 0xFFFFu);
-                if (F::SCF == 2) {
-                    const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
-                    ds = d8 * (float)dot16(ones, hi, dot16(ones, lo, 0));
-                }
-            }
-            uint8_t* codes = row + it * F::PLANES * 1024;
-            *(uint4*)(codes + F::slot(ji, 0)) = lo;
-            *(uint4*)(codes + F::slot(ji, 1)) = hi;
-            if (F::SCF == 2) {
-                *(float2*)(sc + 2 * j) = make_float2(d8, ds);
-            } else {
-                sc[j] = d8;
-            }
-        }
-    }
-}
-
-template <typename T>
-static __device__ __forceinline__ void store_out(T* dst, int stride_col_dst, int col, int row, float v,
-                                                 const float* bias) {
-    if (bias) v += bias[row];
-    dst[(size_t)col * stride_col_dst + row] = from_f32<T>(v);
-}
-
-// --------------------------------------------------------------------------------------------
-// Q4_K
-// --------------------------------------------------------------------------------------------
-template <int B, int R, typename T>
-__global__ __launch_bounds__(WG) void mmvq_q4k_kernel(const uint8_t* __restrict__ vx,
-                                                      const uint8_t* __restrict__ vy, T* __restrict__ dst,
-                                                      int nb, int n, int stride_col_y, int stride_col_dst,
-                                                      const float* __restrict__ bias) {
+template <class E, int B, int R, typename T>
+__global__ __launch_bounds__(WG) void mmvq_kernel(MultiArgs m, const uint8_t* __restrict__ vy, int nb,
+                                                  int stride_col_y, int stride_col_dst) {
     extern __shared__ __align__(16) uint8_t lds[];
-    const int n_iter = (nb + 15) >> 4;
-    const int row_bytes = lds_bytes_per_row<FmtQ4K>(n_iter);
-
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lb = lane >> 2, p = lane & 3;
-    const Q4KScaleSel sel(p);
-    const uint32_t hdr_off = lb * Q4K_BYTES, qs_off = hdr_off + 16 + 32 * p;
-    const size_t row_stride = (size_t)nb * Q4K_BYTES;
-    const int n_tiles = (n + R - 1) / R;
-    const int tile_stride = gridDim.x * WAVES;
-
-    struct Frag {
-        uint4 hdr[R], q0[R], q1[R];
-    };
-    // One pass (16 super-blocks) of R rows into registers. Lanes past the row end hold zeros:
-    // d = dmin = 0 and the staged activation tail is zero, so they add nothing.
-    auto load = [&](Frag& f, int tile, int it) {
-        const bool valid = it * 16 + lb < nb;
-        // an out-of-range lane re-reads the row's last block and drops its d / dmin
-        const uint32_t back = valid ? 0u : (uint32_t)(it * 16 + lb - (nb - 1)) * Q4K_BYTES;
+    int w = 0;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int row = min(tile * R + r, n - 1);
-            const uint8_t* bp = vx + row * row_stride + (size_t)it * (16 * Q4K_BYTES);
-            f.hdr[r] = *(const uint4*)(bp + (hdr_off - back));
-            f.q0[r] = *(const uint4*)(bp + (qs_off - back));
-            f.q1[r] = *(const uint4*)(bp + (qs_off - back + 16));
-            if (!valid) f.hdr[r].x = 0;
-        }
-    };
-
-    float acc[R][B];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
-
-    auto compute = [&](const Frag& f, int tile, int it) {
-        float d[R], dmin[R], scl[R], sch[R], ml[R], mh[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            uint32_t sc, mn;
-            sel.unpack(f.hdr[r].y, f.hdr[r].z, f.hdr[r].w, sc, mn);
-            d[r] = f16_bits_to_f32(f.hdr[r].x & 0xFFFFu);
-            dmin[r] = f16_bits_to_f32(f.hdr[r].x >> 16);
-            scl[r] = (float)(sc & 0xFFu);
-            sch[r] = (float)(sc >> 8);
-            ml[r] = (float)(mn & 0xFFu);
-            mh[r] = (float)(mn >> 8);
-        }
-#pragma unroll
-        for (int c = 0; c < B; ++c) {
-            const uint8_t* rowl = lds + c * row_bytes;
-            const uint8_t* codes = rowl + it * 4096 + lane * 16;
-            const uint4 a00 = *(const uint4*)(codes);
-            const uint4 a01 = *(const uint4*)(codes + 1024);
-            const uint4 a10 = *(const uint4*)(codes + 2048);
-            const uint4 a11 = *(const uint4*)(codes + 3072);
-            const float4 s4 = *(const float4*)(rowl + n_iter * 4096 + (size_t)((it * 16 + lb) * 8 + 2 * p) * 8);
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                int d_lo = 0, d_hi = 0;
-                q4k_dots(f.q0[r], a00, a10, d_lo, d_hi);
-                q4k_dots(f.q1[r], a01, a11, d_lo, d_hi);
-                const float u = (scl[r] * s4.x) * (float)d_lo + (sch[r] * s4.z) * (float)d_hi;
-                const float w = ml[r] * s4.y + mh[r] * s4.w;
-                acc[r][c] += d[r] * u - dmin[r] * w;
-            }
-        }
-        if (it == n_iter - 1) {
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int c = 0; c < B; ++c) {
-                    const float total = wave_sum(acc[r][c]);
-                    acc[r][c] = 0.f;
-                    if (lane == 0 && tile * R + r < n) store_out(dst, stride_col_dst, c, tile * R + r, total, bias);
-                }
-        }
-    };
-
-    // Steps are (tile, pass) pairs in order; the loads of step i+1 are issued before step i is
-    // consumed, ping-ponging between two register fragments.
-    // The first weight loads go out before the activation is staged, so the two memory
-    // latencies overlap instead of adding up (it is most of a small matrix's run time).
-    int tile = blockIdx.x * WAVES + wave, it = 0;
-    Frag fa, fb;
-    if (tile < n_tiles) load(fa, tile, 0);
-    stage_activation<FmtQ4K, B>(lds, vy, nb * 8, n_iter, stride_col_y);
-    __syncthreads();
-    if (tile >= n_tiles) return;
-    for (;;) {
-        int nt = tile, ni = it + 1;
-        if (ni == n_iter) { ni = 0; nt += tile_stride; }
-        if (nt < n_tiles) load(fb, nt, ni);
-        compute(fa, tile, it);
-        tile = nt; it = ni;
-        if (tile >= n_tiles) break;
-        nt = tile; ni = it + 1;
-        if (ni == n_iter) { ni = 0; nt += tile_stride; }
-        if (nt < n_tiles) load(fa, nt, ni);
-        compute(fb, tile, it);
-        tile = nt; it = ni;
-        if (tile >= n_tiles) break;
-    }
+    for (int i = 1; i < MAX_MULTI; ++i)
+        if (i < m.count && (int)blockIdx.x >= m.wg_begin[i]) w = i;
+    const int wgs = m.wg_begin[w + 1] - m.wg_begin[w];
+    RowJob<1> job{{m.vx[w]}, vy, nb, m.n[w], stride_col_y, wgs * WAVES, ((int)blockIdx.x - m.wg_begin[w]) * WAVES};
+    T* dst = (T*)m.dst[w];
+    const float* bias = m.bias[w];
+    E::template run<B, R, 1>(job, lds, [&](int row, int c, const float* tot) {
+        float v = tot[0];
+        if (bias) v += bias[row];
+        dst[(size_t)c * stride_col_dst + row] = from_f32<T>(v);
+    });
 }
 
-// --------------------------------------------------------------------------------------------
-// Q6_K
-// --------------------------------------------------------------------------------------------
-template <int B, int R, typename T>
-__global__ __launch_bounds__(WG) void mmvq_q6k_kernel(const uint8_t* __restrict__ vx,
-                                                      const uint8_t* __restrict__ vy, T* __restrict__ dst,
-                                                      int nb, int n, int stride_col_y, int stride_col_dst,
-                                                      const float* __restrict__ bias) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    const int n_iter = (nb + 7) >> 3;
-    const int row_bytes = lds_bytes_per_row<FmtQ6K>(n_iter);
-    stage_activation<FmtQ6K, B>(lds, vy, nb * 8, n_iter, stride_col_y);
-    __syncthreads();
-
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lb = lane >> 3, ch = lane & 7;
-    const int h = ch >> 2, g0 = (ch >> 1) & 1, lh = ch & 1;
-    const size_t row_stride = (size_t)nb * Q6K_BYTES;
-
-    for (int tile = blockIdx.x * WAVES + wave; tile * R < n; tile += gridDim.x * WAVES) {
-        const int row0 = tile * R;
-        float acc[R][B];
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
-
-        for (int it = 0; it < n_iter; ++it) {
-            const int blk = it * 8 + lb;
-            const bool valid = blk < nb;
-            const int blk_c = valid ? blk : nb - 1;
-            uint4 ql[R], qh[R];
-            float dsa[R], dsb[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r, n - 1);
-                const uint8_t* bp = vx + row * row_stride + (size_t)blk_c * Q6K_BYTES;
-                ql[r] = *(const uint4_a2*)(bp + 16 * ch);
-                qh[r] = *(const uint4_a2*)(bp + 128 + 16 * (2 * h + lh));
-                const int sa = ((const int8_t*)bp)[192 + 8 * h + 2 * g0 + lh];
-                const int sb = ((const int8_t*)bp)[192 + 8 * h + 2 * g0 + 4 + lh];
-                const float d = valid ? f16_bits_to_f32(*(const uint16_t*)(bp + 208)) : 0.f;
-                dsa[r] = d * (float)sa;
-                dsb[r] = d * (float)sb;
-            }
-#pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const uint8_t* rowl = lds + c * row_bytes;
-                const uint8_t* codes = rowl + it * 2048;
-                const uint4 a_a = *(const uint4*)(codes + lane * 16);
-                const uint4 a_b = *(const uint4*)(codes + 1024 + lane * 16);
-                const float* sc = (const float*)(rowl + n_iter * 2048);
-                const float d8a = sc[blk * 8 + 4 * h + g0];
-                const float d8b = sc[blk * 8 + 4 * h + g0 + 2];
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    int d_a, d_b;
-                    q6k_dots(ql[r], qh[r], g0, a_a, a_b, d_a, d_b);
-                    acc[r][c] += dsa[r] * (d8a * (float)d_a) + dsb[r] * (d8b * (float)d_b);
-                }
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const float total = wave_sum(acc[r][c]);
-                if (lane == 0 && row0 + r < n) store_out(dst, stride_col_dst, c, row0 + r, total, bias);
-            }
-    }
+// gate and up rows over one activation, out = act(gate) * up (fast_mmvq::try_fused of the
+// reference, src/tensor/quantized/fast_mmvq.rs:97-282; kernels mmvq_gguf_pair_*_silu and
+// *_fused_{silu,gelu}, src/inference/cuda/mmvq_gguf.cu:588-758).
+static __device__ __forceinline__ float act_silu(float g) { return g / (1.0f + expf(-g)); }
+static __device__ __forceinline__ float act_gelu_tanh(float g) {
+    return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * g * (1.0f + 0.044715f * g * g)));
 }
 
-// --------------------------------------------------------------------------------------------
-// Q8_0
-// --------------------------------------------------------------------------------------------
-template <int B, int R, typename T>
-__global__ __launch_bounds__(WG) void mmvq_q80_kernel(const uint8_t* __restrict__ vx,
-                                                      const uint8_t* __restrict__ vy, T* __restrict__ dst,
-                                                      int nb, int n, int stride_col_y, int stride_col_dst,
-                                                      const float* __restrict__ bias) {
+template <class E, int B, int R, typename T, int ACT>
+__global__ __launch_bounds__(WG) void mmvq_pair_kernel(const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up,
+                                                       const uint8_t* __restrict__ vy, T* __restrict__ dst, int nb,
+                                                       int n, int stride_col_y, int stride_col_dst) {
     extern __shared__ __align__(16) uint8_t lds[];
-    const int n_iter = (nb + 31) >> 5;
-    const int row_bytes = lds_bytes_per_row<FmtQ80>(n_iter);
-    stage_activation<FmtQ80, B>(lds, vy, nb, n_iter, stride_col_y);
-    __syncthreads();
+    RowJob<2> job{{gate, up}, vy, nb, n, stride_col_y, (int)gridDim.x * WAVES, (int)blockIdx.x * WAVES};
+    E::template run<B, R, 2>(job, lds, [&](int row, int c, const float* tot) {
+        const float a = ACT == 0 ? act_silu(tot[0]) : act_gelu_tanh(tot[0]);
+        dst[(size_t)c * stride_col_dst + row] = from_f32<T>(a * tot[1]);
+    });
+}
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lb = lane >> 1, lh = lane & 1;
-    const size_t row_stride = (size_t)nb * Q80_BYTES;
-
-    for (int tile = blockIdx.x * WAVES + wave; tile * R < n; tile += gridDim.x * WAVES) {
-        const int row0 = tile * R;
-        float acc[R][B];
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
-
-        for (int it = 0; it < n_iter; ++it) {
-            const int blk = it * 32 + lb;
-            const bool valid = blk < nb;
-            const int blk_c = valid ? blk : nb - 1;
-            uint4 q[R];
-            float d[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r, n - 1);
-                const uint8_t* bp = vx + row * row_stride + (size_t)blk_c * Q80_BYTES;
-                q[r] = *(const uint4_a2*)(bp + 2 + 16 * lh);
-                d[r] = valid ? f16_bits_to_f32(*(const uint16_t*)bp) : 0.f;
-            }
-#pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const uint8_t* rowl = lds + c * row_bytes;
-                const uint4 a = *(const uint4*)(rowl + it * 1024 + lane * 16);
-                const float d8 = ((const float*)(rowl + n_iter * 1024))[blk];
-#pragma unroll
-                for (int r = 0; r < R; ++r) acc[r][c] += (d[r] * d8) * (float)dot16(q[r], a, 0);
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const float total = wave_sum(acc[r][c]);
-                if (lane == 0 && row0 + r < n) store_out(dst, stride_col_dst, c, row0 + r, total, bias);
-            }
-    }
+// `groups` weights of one shape, each over its OWN activation row: weight g (address table[g])
+// reads the Q8_1 blocks from g * k/32 and writes dst from g * n (mmvq_f32_grouped,
+// src/tensor/cuda/quant.rs:3418-3466).
+template <class E, int R>
+__global__ __launch_bounds__(WG) void mmvq_grouped_kernel(const uint64_t* __restrict__ table,
+                                                          const uint8_t* __restrict__ vy, float* __restrict__ dst,
+                                                          int nb, int n, int k32) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int g = blockIdx.y;
+    RowJob<1> job{{(const uint8_t*)table[g]}, vy + (size_t)g * k32 * Q81_BYTES, nb, n, k32,
+                  (int)gridDim.x * WAVES, (int)blockIdx.x * WAVES};
+    float* out = dst + (size_t)g * n;
+    E::template run<1, R, 1>(job, lds, [&](int row, int, const float* tot) { out[row] = tot[0]; });
 }
 
 // --------------------------------------------------------------------------------------------
@@ -491,116 +173,186 @@ __global__ void act_sums_kernel(const uint8_t* __restrict__ vy, int32_t* __restr
 // --------------------------------------------------------------------------------------------
 // Host dispatch
 // --------------------------------------------------------------------------------------------
-struct MmvqArgs {
-    const uint8_t* vx;
-    const uint8_t* vy;
-    void* dst;
-    int nb, n, stride_col_y, stride_col_dst;
-    const float* bias;
-    hipStream_t stream;
-};
-
-template <class F>
-static int n_iter_of(int nb) {
-    const int per = F::VPI / F::BLOCK_LEN;
-    return (nb + per - 1) / per;
-}
 
 // Launch geometry. `R` rows per wave and the number of resident workgroups per CU set how many
-// bytes are in flight; both have measured optima well below "as many as fit" (HBM throughput
-// drops when too many requests are outstanding). LK_TUNE_R / LK_TUNE_WGS_PER_CU override the
-// built-in choice for measurement runs.
+// bytes are in flight; both have measured optima below "as many as fit" (HBM throughput drops
+// when too many requests are outstanding). LK_TUNE_WGS_PER_CU overrides the built-in cap for
+// measurement runs.
 static int tune_env(const char* name) {
     const char* v = getenv(name);
     return v ? atoi(v) : 0;
 }
 
-template <class FMT, int B, int R, typename T, typename K>
-static int launch_rows(K kernel, const MmvqArgs& a, int wgs_per_cu) {
-    const int lds_bytes = B * lds_bytes_per_row<FMT>(n_iter_of<FMT>(a.nb));
-    const LkDevice& dev = lk_device();
-    if (lds_bytes > dev.lds_bytes) return LK_ERR_ARG;
-    // Per kernel instance and LDS size: raise the dynamic-LDS limit once and ask the runtime how
-    // many workgroups a CU holds. Cached, so steady-state launches (and launches recorded into a
-    // graph) make no runtime query.
+// Per kernel instance and LDS size: raise the dynamic-LDS limit once and ask the runtime how many
+// workgroups a CU holds. Cached, so steady-state launches (and launches recorded into a graph)
+// make no runtime query. Returns workgroups resident per CU, 0 on failure.
+template <typename K>
+static int resident_per_cu(K kernel, int lds_bytes) {
     static std::mutex mu;
-    static std::unordered_map<int, int> resident_by_lds;
-    int resident = 0;
-    {
-        std::lock_guard<std::mutex> lock(mu);
-        auto it = resident_by_lds.find(lds_bytes);
-        if (it == resident_by_lds.end()) {
-            if (lds_bytes > 48 * 1024 &&
-                hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
-                (void)hipGetLastError();
-                return LK_ERR_LAUNCH;
-            }
-            int r = 0;
-            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)kernel, WG, (size_t)lds_bytes) != hipSuccess || r < 1) {
-                (void)hipGetLastError();
-                r = 1;
-            }
-            it = resident_by_lds.emplace(lds_bytes, r).first;
-        }
-        resident = it->second;
+    static std::unordered_map<int, int> by_lds;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = by_lds.find(lds_bytes);
+    if (it != by_lds.end()) return it->second;
+    if (lds_bytes > lk_device().lds_bytes) return 0;
+    if (lds_bytes > 48 * 1024 &&
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
     }
-    const int tiles = (a.n + R - 1) / R;
-    const int wgs_needed = (tiles + WAVES - 1) / WAVES;
-    // Persistent grid: exactly as many workgroups as are resident at once, so no workgroup waits
-    // for a slot and each wave walks several row tiles.
+    int r = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)kernel, WG, (size_t)lds_bytes) != hipSuccess || r < 1) {
+        (void)hipGetLastError();
+        r = 1;
+    }
     static const int forced = tune_env("LK_TUNE_WGS_PER_CU");
-    const int cap = forced > 0 ? forced : wgs_per_cu;
-    const int per_cu = resident > cap ? cap : resident;
-    const int grid = wgs_needed < dev.cus * per_cu ? wgs_needed : dev.cus * per_cu;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(WG), lds_bytes, a.stream, a.vx, a.vy, (T*)a.dst, a.nb,
-                       a.n, a.stride_col_y, a.stride_col_dst, a.bias);
+    const int cap = forced > 0 ? forced : 8;
+    r = r > cap ? cap : r;
+    by_lds.emplace(lds_bytes, r);
+    return r;
+}
+
+static inline int wgs_for_rows(int n, int rows_per_wave) {
+    const int tiles = (n + rows_per_wave - 1) / rows_per_wave;
+    return (tiles + WAVES - 1) / WAVES;
+}
+
+struct MmvqCall {
+    MultiArgs m;
+    const uint8_t* vy;
+    int nb, stride_col_y, stride_col_dst;
+    hipStream_t stream;
+};
+
+template <class E, int B, typename T>
+static int launch_plain(MmvqCall& a) {
+    constexpr int R = 2;
+    auto kernel = mmvq_kernel<E, B, R, T>;
+    const int lds_bytes = lds_bytes_for<typename E::Fmt>(a.nb, B);
+    const int per_cu = resident_per_cu(kernel, lds_bytes);
+    if (per_cu == 0) return LK_ERR_ARG;
+    // Persistent grid: no more workgroups than are resident at once, shared out over the
+    // matrices in proportion to their rows.
+    const int capacity = lk_device().cus * per_cu;
+    int need[MAX_MULTI], total = 0;
+    for (int i = 0; i < a.m.count; ++i) {
+        need[i] = wgs_for_rows(a.m.n[i], R);
+        total += need[i];
+    }
+    a.m.wg_begin[0] = 0;
+    for (int i = 0; i < a.m.count; ++i) {
+        int share = need[i];
+        if (total > capacity) {
+            share = (int)((int64_t)need[i] * capacity / total);
+            if (share < 1) share = 1;
+        }
+        a.m.wg_begin[i + 1] = a.m.wg_begin[i] + share;
+    }
+    for (int i = a.m.count; i < MAX_MULTI; ++i) a.m.wg_begin[i + 1] = a.m.wg_begin[i];
+    hipLaunchKernelGGL(kernel, dim3(a.m.wg_begin[a.m.count]), dim3(WG), lds_bytes, a.stream, a.m, a.vy, a.nb,
+                       a.stride_col_y, a.stride_col_dst);
     return lk_launch_status();
 }
 
-#define LK_DEFINE_LAUNCHER(NAME, KERNEL, FMT, ROWS1, ROWSN, WGS_PER_CU)                                \
-    template <int B, typename T>                                                                      \
-    static int NAME(const MmvqArgs& a) {                                                              \
-        static const int forced_r = tune_env("LK_TUNE_R");                                            \
-        if (B == 1 && forced_r == 1) return launch_rows<FMT, B, 1, T>(KERNEL<B, 1, T>, a, WGS_PER_CU); \
-        if (B == 1 && forced_r == 2) return launch_rows<FMT, B, 2, T>(KERNEL<B, 2, T>, a, WGS_PER_CU); \
-        if (B == 1 && forced_r == 4) return launch_rows<FMT, B, 4, T>(KERNEL<B, 4, T>, a, WGS_PER_CU); \
-        constexpr int R = (B == 1) ? ROWS1 : ROWSN;                                                   \
-        return launch_rows<FMT, B, R, T>(KERNEL<B, R, T>, a, WGS_PER_CU);                             \
-    }
-
-LK_DEFINE_LAUNCHER(launch_q4k, mmvq_q4k_kernel, FmtQ4K, 2, 2, 8)
-LK_DEFINE_LAUNCHER(launch_q6k, mmvq_q6k_kernel, FmtQ6K, 2, 2, 8)
-LK_DEFINE_LAUNCHER(launch_q80, mmvq_q80_kernel, FmtQ80, 2, 2, 8)
-
-#define LK_BATCH_SWITCH(FN, T)                                                                         \
+#define LK_BATCH_SWITCH(FN, E, T, ARG)                                                                 \
     switch (batch) {                                                                                  \
-        case 1: return FN<1, T>(a);                                                                   \
-        case 2: return FN<2, T>(a);                                                                   \
-        case 3: return FN<3, T>(a);                                                                   \
-        case 4: return FN<4, T>(a);                                                                   \
-        case 5: return FN<5, T>(a);                                                                   \
-        case 6: return FN<6, T>(a);                                                                   \
-        case 7: return FN<7, T>(a);                                                                   \
-        case 8: return FN<8, T>(a);                                                                   \
+        case 1: return FN<E, 1, T>(ARG);                                                              \
+        case 2: return FN<E, 2, T>(ARG);                                                              \
+        case 3: return FN<E, 3, T>(ARG);                                                              \
+        case 4: return FN<E, 4, T>(ARG);                                                              \
+        case 5: return FN<E, 5, T>(ARG);                                                              \
+        case 6: return FN<E, 6, T>(ARG);                                                              \
+        case 7: return FN<E, 7, T>(ARG);                                                              \
+        case 8: return FN<E, 8, T>(ARG);                                                              \
         default: return LK_ERR_ARG;                                                                   \
     }
 
 template <typename T>
-static int dispatch_type(int wtype, int batch, const MmvqArgs& a) {
+static int dispatch_plain(int wtype, int batch, MmvqCall& a) {
     switch (wtype) {
-        case LK_TYPE_Q4_K: LK_BATCH_SWITCH(launch_q4k, T)
-        case LK_TYPE_Q6_K: LK_BATCH_SWITCH(launch_q6k, T)
-        case LK_TYPE_Q8_0: LK_BATCH_SWITCH(launch_q80, T)
+        case LK_TYPE_Q4_K: LK_BATCH_SWITCH(launch_plain, EngQ4K, T, a)
+        case LK_TYPE_Q6_K: LK_BATCH_SWITCH(launch_plain, EngQ6K, T, a)
+        case LK_TYPE_Q8_0: LK_BATCH_SWITCH(launch_plain, EngQ80, T, a)
         default: return LK_ERR_TYPE;
     }
 }
 
-static int block_len_of(int wtype) {
-    switch (wtype) {
-        case LK_TYPE_Q4_K: case LK_TYPE_Q6_K: return 256;
-        case LK_TYPE_Q8_0: return 32;
-        default: return 0;
+static int check_common(int wtype, const void* vy, int ncols_x, int batch, int stride_col_y) {
+    const int bl = block_len_of(wtype);
+    if (bl == 0) return LK_ERR_TYPE;
+    if (!vy || ncols_x <= 0 || ncols_x % bl != 0) return LK_ERR_ARG;
+    if (batch < 1 || batch > 8 || stride_col_y < ncols_x / 32) return LK_ERR_ARG;
+    if (((uintptr_t)vy & 3) != 0) return LK_ERR_ARG;
+    return LK_OK;
+}
+static int check_weight(int wtype, const void* vx) {
+    if (!vx) return LK_ERR_ARG;
+    if (wtype == LK_TYPE_Q4_K && ((uintptr_t)vx & 15) != 0) return LK_ERR_ARG;
+    if (((uintptr_t)vx & 1) != 0) return LK_ERR_ARG;
+    return LK_OK;
+}
+
+static int run_multi(int wtype, int count, const void* const* vx, const void* vy, void* const* dst, int dst_type,
+                     int ncols_x, const int* nrows_x, int batch, int stride_col_y, int stride_col_dst,
+                     const float* const* bias, void* stream) {
+    if (int rc = check_common(wtype, vy, ncols_x, batch, stride_col_y)) return rc;
+    if (count < 1 || count > MAX_MULTI) return LK_ERR_ARG;
+    MmvqCall a{};
+    a.vy = (const uint8_t*)vy;
+    a.nb = ncols_x / block_len_of(wtype);
+    a.stride_col_y = stride_col_y;
+    a.stride_col_dst = stride_col_dst;
+    a.stream = (hipStream_t)stream;
+    int live = 0;
+    for (int i = 0; i < count; ++i) {
+        if (nrows_x[i] < 0) return LK_ERR_ARG;
+        if (nrows_x[i] == 0) continue;
+        if (int rc = check_weight(wtype, vx[i])) return rc;
+        if (!dst[i] || stride_col_dst < nrows_x[i]) return LK_ERR_ARG;
+        a.m.vx[live] = (const uint8_t*)vx[i];
+        a.m.dst[live] = dst[i];
+        a.m.bias[live] = bias ? bias[i] : nullptr;
+        a.m.n[live] = nrows_x[i];
+        ++live;
     }
+    if (live == 0) return LK_OK;
+    a.m.count = live;
+    switch (dst_type) {
+        case LK_TYPE_F32: return dispatch_plain<float>(wtype, batch, a);
+        case LK_TYPE_F16: return dispatch_plain<__half>(wtype, batch, a);
+        case LK_TYPE_BF16: return dispatch_plain<__hip_bfloat16>(wtype, batch, a);
+        default: return LK_ERR_TYPE;
+    }
+}
+
+template <class E, int B, typename T>
+static int launch_pair(const uint8_t* gate, const uint8_t* up, const uint8_t* vy, void* dst, int nb, int n,
+                       int stride_col_y, int stride_col_dst, int act, hipStream_t s) {
+    constexpr int R = 1;
+    const int lds_bytes = lds_bytes_for<typename E::Fmt>(nb, B);
+    auto launch = [&](auto kernel) {
+        const int per_cu = resident_per_cu(kernel, lds_bytes);
+        if (per_cu == 0) return (int)LK_ERR_ARG;
+        const int need = wgs_for_rows(n, R), cap = lk_device().cus * per_cu;
+        hipLaunchKernelGGL(kernel, dim3(need < cap ? need : cap), dim3(WG), lds_bytes, s, gate, up, vy, (T*)dst, nb, n,
+                           stride_col_y, stride_col_dst);
+        return lk_launch_status();
+    };
+    return act == 0 ? launch(mmvq_pair_kernel<E, B, R, T, 0>) : launch(mmvq_pair_kernel<E, B, R, T, 1>);
+}
+
+template <class E>
+static int launch_grouped(const uint64_t* table, int groups, const uint8_t* vy, float* dst, int nb, int n, int k32,
+                          hipStream_t s) {
+    constexpr int R = 2;
+    auto kernel = mmvq_grouped_kernel<E, R>;
+    const int lds_bytes = lds_bytes_for<typename E::Fmt>(nb, 1);
+    const int per_cu = resident_per_cu(kernel, lds_bytes);
+    if (per_cu == 0) return LK_ERR_ARG;
+    const int need = wgs_for_rows(n, R);
+    int cap = lk_device().cus * per_cu / groups;
+    if (cap < 1) cap = 1;
+    hipLaunchKernelGGL(kernel, dim3(need < cap ? need : cap, groups), dim3(WG), lds_bytes, s, table, vy, dst, nb, n, k32);
+    return lk_launch_status();
 }
 
 }  // namespace
@@ -609,21 +361,67 @@ extern "C" int lk_mmvq(int wtype, const void* vx, const void* vy_q8_1, void* dst
                        int ncols_x, int nrows_x, int batch, int stride_col_y, int stride_col_dst,
                        const float* bias, int decode_order, void* stream) {
     (void)decode_order;  // a row's sum never depends on batch here
+    if (block_len_of(wtype) == 0) return LK_ERR_TYPE;
+    if (nrows_x == 0) return LK_OK;
+    return run_multi(wtype, 1, &vx, vy_q8_1, &dst, dst_type, ncols_x, &nrows_x, batch, stride_col_y, stride_col_dst,
+                     bias ? &bias : nullptr, stream);
+}
+
+extern "C" int lk_mmvq_multi(int wtype, int count, const void* const* vx, const void* vy_q8_1, void* const* dst,
+                             int dst_type, int ncols_x, const int* nrows_x, int batch, int stride_col_y,
+                             int stride_col_dst, const float* const* bias, void* stream) {
+    if (!vx || !dst || !nrows_x) return LK_ERR_ARG;
+    return run_multi(wtype, count, vx, vy_q8_1, dst, dst_type, ncols_x, nrows_x, batch, stride_col_y, stride_col_dst,
+                     bias, stream);
+}
+
+extern "C" int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, const void* vy_q8_1, void* dst,
+                                int dst_type, int ncols_x, int nrows_x, int batch, int stride_col_y,
+                                int stride_col_dst, int act, void* stream) {
+    if (int rc = check_common(wtype, vy_q8_1, ncols_x, batch, stride_col_y)) return rc;
+    if (nrows_x == 0) return LK_OK;
+    if (int rc = check_weight(wtype, gate)) return rc;
+    if (int rc = check_weight(wtype, up)) return rc;
+    if (!dst || nrows_x < 0 || stride_col_dst < nrows_x || (act != 0 && act != 1)) return LK_ERR_ARG;
+    if (batch > 4) return LK_ERR_ARG;
+    const int nb = ncols_x / block_len_of(wtype);
+    hipStream_t s = (hipStream_t)stream;
+    const uint8_t *g = (const uint8_t*)gate, *u = (const uint8_t*)up, *y = (const uint8_t*)vy_q8_1;
+#define LK_PAIR(E, T)                                                                                          \
+    switch (batch) {                                                                                           \
+        case 1: return launch_pair<E, 1, T>(g, u, y, dst, nb, nrows_x, stride_col_y, stride_col_dst, act, s);  \
+        case 2: return launch_pair<E, 2, T>(g, u, y, dst, nb, nrows_x, stride_col_y, stride_col_dst, act, s);  \
+        case 3: return launch_pair<E, 3, T>(g, u, y, dst, nb, nrows_x, stride_col_y, stride_col_dst, act, s);  \
+        default: return launch_pair<E, 4, T>(g, u, y, dst, nb, nrows_x, stride_col_y, stride_col_dst, act, s); \
+    }
+#define LK_PAIR_TYPE(E)                                          \
+    switch (dst_type) {                                          \
+        case LK_TYPE_F32: LK_PAIR(E, float)                      \
+        case LK_TYPE_BF16: LK_PAIR(E, __hip_bfloat16)            \
+        default: return LK_ERR_TYPE;                             \
+    }
+    switch (wtype) {
+        case LK_TYPE_Q4_K: LK_PAIR_TYPE(EngQ4K)
+        case LK_TYPE_Q6_K: LK_PAIR_TYPE(EngQ6K)
+        case LK_TYPE_Q8_0: LK_PAIR_TYPE(EngQ80)
+        default: return LK_ERR_TYPE;
+    }
+}
+
+extern "C" int lk_mmvq_grouped(int wtype, const uint64_t* table, int groups, const void* vy_q8_1, float* dst,
+                               int ncols_x, int nrows_x, void* stream) {
     const int bl = block_len_of(wtype);
     if (bl == 0) return LK_ERR_TYPE;
-    if (nrows_x == 0) return LK_OK;
-    if (!vx || !vy_q8_1 || !dst || ncols_x <= 0 || nrows_x < 0 || ncols_x % bl != 0) return LK_ERR_ARG;
-    if (batch < 1 || batch > 8 || stride_col_y < ncols_x / 32 || stride_col_dst < nrows_x) return LK_ERR_ARG;
-    if (((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
-    if (wtype == LK_TYPE_Q4_K && ((uintptr_t)vx & 15) != 0) return LK_ERR_ARG;
-    if (((uintptr_t)vx & 1) != 0) return LK_ERR_ARG;
-    MmvqArgs a{(const uint8_t*)vx, (const uint8_t*)vy_q8_1, dst, ncols_x / bl, nrows_x,
-               stride_col_y, stride_col_dst, bias, (hipStream_t)stream};
-    switch (dst_type) {
-        case LK_TYPE_F32: return dispatch_type<float>(wtype, batch, a);
-        case LK_TYPE_F16: return dispatch_type<__half>(wtype, batch, a);
-        case LK_TYPE_BF16: return dispatch_type<__hip_bfloat16>(wtype, batch, a);
-        default: return LK_ERR_TYPE;
+    if (groups == 0 || nrows_x == 0) return LK_OK;
+    if (!table || !vy_q8_1 || !dst || groups < 0 || groups > 65535 || nrows_x < 0 || ncols_x <= 0) return LK_ERR_ARG;
+    if (ncols_x % LK_ROW_PADDING != 0 || ncols_x % bl != 0 || ((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
+    const int nb = ncols_x / bl, k32 = ncols_x / 32;
+    hipStream_t s = (hipStream_t)stream;
+    const uint8_t* y = (const uint8_t*)vy_q8_1;
+    switch (wtype) {
+        case LK_TYPE_Q4_K: return launch_grouped<EngQ4K>(table, groups, y, dst, nb, nrows_x, k32, s);
+        case LK_TYPE_Q6_K: return launch_grouped<EngQ6K>(table, groups, y, dst, nb, nrows_x, k32, s);
+        default: return launch_grouped<EngQ80>(table, groups, y, dst, nb, nrows_x, k32, s);
     }
 }
 

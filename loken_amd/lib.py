@@ -29,6 +29,9 @@ SIGNATURES = {
     "lk_device_info": (_i, [_vp, _vp, _vp, _vp]),
     "lk_quantize_q8_1": (_i, [_vp, _i, _vp, _i, _i, _i, _vp]),
     "lk_mmvq": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp]),
+    "lk_mmvq_multi": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _vp, _vp]),
+    "lk_mmvq_pair_act": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "lk_mmvq_grouped": (_i, [_i, _vp, _i, _vp, _vp, _i, _i, _vp]),
     "lk_mmvq_subdots": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _vp]),
     "launch_mmq_quantize_q8_1_D4": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),
     "launch_mmq_quantize_q8_1_DS4": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),

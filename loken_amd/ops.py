@@ -53,6 +53,45 @@ def mmvq(wtype: int, weight: torch.Tensor, q8_1: torch.Tensor, k: int, n: int, *
     return out
 
 
+def mmvq_multi(wtype: int, weights, q8_1: torch.Tensor, k: int, ns, *, out_dtype: torch.dtype = torch.float32):
+    """Several matrices (same format, same k) over the same Q8_1 rows in one launch -> list of
+    ``[b, n_i]`` outputs (forward_quantized_pair of the reference generalised to 4)."""
+    import ctypes as C
+    b = q8_1.shape[0]
+    count = len(weights)
+    outs = [torch.empty((b, n), dtype=out_dtype, device=q8_1.device) for n in ns]
+    stride = max(ns)
+    if any(n != stride for n in ns) and b > 1:
+        # one destination row stride serves every matrix: give each its own launch-wide stride
+        outs = [torch.empty((b, stride), dtype=out_dtype, device=q8_1.device) for _ in ns]
+    vx = (C.c_void_p * count)(*[w.data_ptr() for w in weights])
+    dst = (C.c_void_p * count)(*[o.data_ptr() for o in outs])
+    nn = (C.c_int * count)(*ns)
+    _lib.check("lk_mmvq_multi", _lib.load().lk_mmvq_multi(
+        wtype, count, vx, q8_1.data_ptr(), dst, _X_TYPES[out_dtype], k, nn, b, q8_1.shape[1], stride, None, _stream()))
+    return [o[:, :n] for o, n in zip(outs, ns)]
+
+
+def mmvq_pair_act(wtype: int, gate: torch.Tensor, up: torch.Tensor, q8_1: torch.Tensor, k: int, n: int, *,
+                  act: str = "silu", out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """``act(gate . x) * (up . x)`` in one launch (fast_mmvq::try_fused)."""
+    b = q8_1.shape[0]
+    out = torch.empty((b, n), dtype=out_dtype, device=q8_1.device)
+    _lib.check("lk_mmvq_pair_act", _lib.load().lk_mmvq_pair_act(
+        wtype, gate.data_ptr(), up.data_ptr(), q8_1.data_ptr(), out.data_ptr(), _X_TYPES[out_dtype], k, n, b,
+        q8_1.shape[1], n, {"silu": 0, "gelu": 1}[act], _stream()))
+    return out
+
+
+def mmvq_grouped(wtype: int, table: torch.Tensor, q8_1: torch.Tensor, k: int, n: int) -> torch.Tensor:
+    """``groups`` same-shape weights (device address table, uint64) each over its own Q8_1 row."""
+    groups = table.numel()
+    out = torch.empty((groups, n), dtype=torch.float32, device=q8_1.device)
+    _lib.check("lk_mmvq_grouped", _lib.load().lk_mmvq_grouped(
+        wtype, table.data_ptr(), groups, q8_1.data_ptr(), out.data_ptr(), k, n, _stream()))
+    return out
+
+
 def mmvq_subdots(wtype: int, weight: torch.Tensor, q8_1_row: torch.Tensor, k: int, n: int):
     """Integer sub-block dots of every weight row against ONE Q8_1 row (parity probe)."""
     per = 16 if wtype == _lib.TYPE_Q6_K else 32

@@ -186,3 +186,53 @@ def test_full_size_matvec_against_oracle(name, n, k):
         w2[:, :, 2:4] = (dm * np.float16(2)).view(np.uint8)
     got2 = ops.mmvq(wtype, dev(w2), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
     assert np.array_equal(got2, 2 * got)
+
+
+# ---------------------------------------------------------------- fused neighbours
+@pytest.mark.parametrize("name", sorted(DT))
+@pytest.mark.parametrize("batch", [1, 3])
+def test_multi_launch_rows_carry_the_bits_of_their_own_launch(name, batch):
+    wtype = DT[name]
+    k, ns = 2048, [512, 128, 130]
+    ws = [dev(synth.weight(wtype, n, k, seed=38, stream=10 + i)) for i, n in enumerate(ns)]
+    q = ops.quantize_q8_1_rows(dev(synth.activation(batch, k, seed=38)))
+    outs = ops.mmvq_multi(wtype, ws, q, k, ns)
+    for w, n, o in zip(ws, ns, outs):
+        assert torch.equal(o, ops.mmvq(wtype, w, q, k, n))
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+def test_gate_up_pair_with_activation_in_the_store(name, act):
+    wtype = DT[name]
+    k, n = 1024, 300
+    g = synth.weight(wtype, n, k, seed=39, stream=1)
+    u = synth.weight(wtype, n, k, seed=39, stream=2)
+    x = synth.activation(2, k, seed=39) * np.float32(20.0)
+    q = ops.quantize_q8_1_rows(dev(x))
+    got = ops.mmvq_pair_act(wtype, dev(g), dev(u), q, k, n, act=act).cpu().numpy()
+    gg = oracle.ob_matmul(wtype, x, g, n).astype(np.float64)
+    uu = oracle.ob_matmul(wtype, x, u, n).astype(np.float64)
+    if act == "silu":
+        want = gg / (1.0 + np.exp(-gg)) * uu
+    else:
+        want = 0.5 * gg * (1.0 + np.tanh(0.7978845608028654 * gg * (1.0 + 0.044715 * gg * gg))) * uu
+    # act(g)*u inherits the relative error of g and u: bound against the row scale
+    assert (np.abs(got - want) <= 2e-3 * np.abs(want) + 1e-4 * np.abs(want).max()).all()
+    # and it is exactly the two single launches combined the same way
+    gs = ops.mmvq(wtype, dev(g), q, k, n)
+    us = ops.mmvq(wtype, dev(u), q, k, n)
+    if act == "silu":
+        torch.testing.assert_close(torch.from_numpy(got).cuda(), gs / (1 + torch.exp(-gs)) * us, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", sorted(DT))
+def test_grouped_launch_each_weight_over_its_own_row(name):
+    wtype = DT[name]
+    groups, k, n = 5, 1024, 96
+    ws = [dev(synth.weight(wtype, n, k, seed=40, stream=20 + g)) for g in range(groups)]
+    table = torch.tensor([w.data_ptr() for w in ws], dtype=torch.int64, device="cuda")
+    q = ops.quantize_q8_1_rows(dev(synth.activation(groups, k, seed=40)))   # k is a multiple of 512
+    got = ops.mmvq_grouped(wtype, table, q, k, n)
+    for g in range(groups):
+        assert torch.equal(got[g], ops.mmvq(wtype, ws[g], q[g:g + 1], k, n)[0])
