@@ -214,6 +214,44 @@ void loken_moe_mmq_fold(const float* pairs, const float* weights, const int32_t*
                         const float* down_bias, float* out, int64_t tokens, int topk, int cols,
                         void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * MoE decode: one mat-vec per routed pair (few rows per expert). Names, argument lists and row
+ * conventions are loken's (src/inference/moe_cuda/mod.rs:235-262, 415-442, 473-483;
+ * cuda/moe/moe_gguf.cu:476-511, 755-860, 1049-1061). sorted_token_ids[i] is the flattened
+ * (token * topk + choice) slot of routed pair i, expert_ids[i] its expert; size_m = pairs,
+ * size_n = output rows per expert, size_k = reduction length; quant_type is loken's wire id
+ * (0 = Q8_0, 1 = Q4_K, 5 = Q6_K). Weights are stacks [num_experts][size_n][size_k / block].
+ * These launchers quantize the f32 activation themselves into a per-(device, stream)
+ * grow-only scratch (the one allocation in this library; growing is refused with
+ * LK_ERR_NOMEM while the stream is being captured). Return 0 or an LK_ERR_* code.
+ * ------------------------------------------------------------------------------------- */
+
+/* out[slot, :] = expert(slot) . x[row], times topk_weights[slot] when given; with weights the
+ * activation row is `slot` (inputs [size_m, k]), without it is slot / topk (inputs [size_m/topk, k]). */
+int loken_moe_gemm_gguf(const float* inputs, const void* weights, const int32_t* sorted_token_ids,
+                        const int32_t* expert_ids, const float* topk_weights, void* outputs,
+                        int num_experts, int topk, int size_m, int size_n, int size_k, int quant_type,
+                        void* stream);
+/* out[slot, :] = silu(gate_e . x[slot / topk]) * (up_e . x[slot / topk]); inputs [size_m/topk, k]. */
+int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const void* gate_weights,
+                                         const void* up_weights, const int32_t* sorted_token_ids,
+                                         const int32_t* expert_ids, float* outputs, int num_experts,
+                                         int topk, int size_m, int size_n, int size_k, int quant_type,
+                                         void* stream);
+/* outputs[t, :] (+)= sum over k ascending of topk_weights[p] * (down_e(p) . inputs[p] + down_bias[e(p)]),
+ * p = t * topk + k; inputs [size_m, k] in slot order. Without add_after `outputs` [size_m/topk,
+ * size_n] must be pre-filled (zeros or the residual) and is accumulated into; with it the result
+ * is written as fold + add_after. down_bias [num_experts, size_n] nullable. */
+int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,
+                                    const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                    const float* topk_weights, float* outputs, int num_experts, int topk,
+                                    int size_m, int size_n, int size_k, int gguf_dtype,
+                                    const float* down_bias, const float* add_after, void* stream);
+/* outputs[t, c] += sum over k ascending of pairs[(t * topk + k), c] (cuda/moe/moe_gguf.cu:745-752). */
+void loken_moe_sum_topk(const float* pairs, float* outputs, int tokens, int topk, int cols, void* stream);
+/* Frees the current device's MoE decode scratch (cuda/moe/moe_gguf.cu:104-118). Synchronizes. */
+void loken_stream_scratch_release(void);
+
 #ifdef __cplusplus
 }
 #endif

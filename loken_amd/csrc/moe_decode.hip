@@ -1,0 +1,295 @@
+// MoE decode: one mat-vec per routed (token, expert) pair, for batches too small to fill the
+// expert-batched tiles. Entry points, argument lists and row conventions are loken's
+// (src/inference/moe_cuda/mod.rs:235-262, 415-442, 473-483; cuda/moe/moe_gguf.cu:403-511,
+// 528-608, 755-860, 896-1060):
+//   sorted_token_ids[i] is the flattened (token * topk + choice) slot of routed pair i and
+//   expert_ids[i] its expert; gate/up read activation row slot / topk and write row slot; down
+//   reads row slot, scales by topk_weights[slot] and writes row slot of a scratch that a fold
+//   then sums per token IN SLOT ORDER (no atomics, the same sum on every run).
+// The launchers quantize the activation themselves into a per-(device, stream) grow-only
+// scratch, as the reference's do; loken_stream_scratch_release frees it.
+//
+// Kernels: grid (row tiles, pairs); each workgroup stages its pair's Q8_1 row into LDS and runs
+// the shared mat-vec row engine on the pair's expert slab. SiLU uses the accurate expf, as the
+// host path does (src/inference/moe_cuda_cpu/mod.rs:598).
+
+#include "mmvq_core.h"
+
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+using namespace mmvq;
+
+extern "C" int lk_quantize_q8_1(const void* x, int x_type, void* vy, int kx, int kx_padded, int rows, void* stream);
+
+namespace {
+
+// ---------------------------------------------------------------- stream scratch
+struct ScratchSlot {
+    int device;
+    hipStream_t stream;
+    void* ptr = nullptr;
+    size_t size = 0;
+    std::vector<void*> kept;  // outgrown buffers: queued kernels may still read them
+};
+std::mutex g_scratch_mu;
+std::vector<ScratchSlot> g_scratch;
+
+// Caller holds g_scratch_mu from the reservation until its launches are on the stream: the
+// buffer belongs to the stream, and another thread's quantize landing between a launcher's
+// two kernels is what the second would then read.
+void* reserve_scratch(size_t bytes, hipStream_t stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    ScratchSlot* slot = nullptr;
+    for (auto& s : g_scratch)
+        if (s.device == dev && s.stream == stream) slot = &s;
+    if (!slot) {
+        g_scratch.push_back(ScratchSlot{dev, stream});
+        slot = &g_scratch.back();
+    }
+    if (slot->size >= bytes) return slot->ptr;
+    // growing allocates, which a stream under capture may not do
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) return nullptr;
+    (void)hipGetLastError();
+    size_t want = bytes + bytes / 4;
+    want = (want + 255) & ~(size_t)255;
+    void* fresh = nullptr;
+    if (hipMalloc(&fresh, want) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (slot->ptr) slot->kept.push_back(slot->ptr);
+    slot->ptr = fresh;
+    slot->size = want;
+    return fresh;
+}
+
+// ---------------------------------------------------------------- kernels
+struct MoeDims {
+    int experts, topk, pairs, cols, nb, k32;  // k32: Q8_1 blocks between activation rows
+    int64_t slab_bytes;                       // one expert's weights
+};
+
+enum { MODE_PLAIN = 0, MODE_GATED = 1, MODE_DOWN = 2 };
+
+template <class E, int R, int MODE>
+__global__ __launch_bounds__(WG) void moe_rows_kernel(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1,
+                                                      const uint8_t* __restrict__ acts,
+                                                      const int32_t* __restrict__ sorted_token_ids,
+                                                      const int32_t* __restrict__ expert_ids,
+                                                      const float* __restrict__ topk_weights,
+                                                      const float* __restrict__ down_bias,
+                                                      float* __restrict__ out, MoeDims d) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int pair = blockIdx.y;
+    const int slot = sorted_token_ids[pair];
+    const int e = expert_ids[pair];
+    if (slot < 0 || slot >= d.pairs) return;
+    float* out_row = out + (size_t)slot * d.cols;
+    if (e < 0 || e >= d.experts) {
+        // a pair the routing leaves out adds nothing: its row of the fold's input reads zero
+        if (MODE == MODE_DOWN)
+            for (int r = blockIdx.x * WG + threadIdx.x; r < d.cols; r += gridDim.x * WG) out_row[r] = 0.f;
+        return;
+    }
+    const bool own_row = MODE == MODE_DOWN || (MODE == MODE_PLAIN && topk_weights != nullptr);
+    const int act_row = own_row ? slot : slot / d.topk;
+    const uint8_t* vy = acts + (size_t)act_row * d.k32 * Q81_BYTES;
+    const float scale = (MODE != MODE_GATED && topk_weights) ? topk_weights[slot] : 1.0f;
+    const uint8_t* slab0 = w0 + (int64_t)e * d.slab_bytes;
+    const int tile_stride = (int)gridDim.x * WAVES, tile_first = (int)blockIdx.x * WAVES;
+    if (MODE == MODE_GATED) {
+        const uint8_t* slab1 = w1 + (int64_t)e * d.slab_bytes;
+        RowJob<2> job{{slab0, slab1}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first};
+        E::template run<1, R, 2>(job, lds, [&](int row, int, const float* tot) {
+            const float g = tot[0];
+            out_row[row] = g / (1.0f + expf(-g)) * tot[1];
+        });
+    } else {
+        RowJob<1> job{{slab0}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first};
+        E::template run<1, R, 1>(job, lds, [&](int row, int, const float* tot) {
+            float v = tot[0] * scale;
+            if (MODE == MODE_DOWN && down_bias) v += scale * down_bias[(size_t)e * d.cols + row];
+            out_row[row] = v;
+        });
+    }
+}
+
+// outputs[t] (+)= sum over k ascending of pairs[t * topk + k]; with `add` the result is written
+// as fold + add instead of accumulated (cuda/moe/moe_gguf.cu:591-625).
+__global__ void sum_topk_kernel(const float* __restrict__ pairs, const float* __restrict__ add,
+                                float* __restrict__ outputs, int tokens, int topk, int cols) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)tokens * cols) return;
+    const size_t token = i / cols, col = i % cols;
+    float acc = add ? 0.0f : outputs[i];
+    for (int k = 0; k < topk; ++k) acc += pairs[(token * topk + k) * cols + col];
+    outputs[i] = add ? acc + add[i] : acc;
+}
+
+template <typename K>
+static int prepare(K kernel, int lds_bytes) {
+    static std::mutex mu;
+    static std::unordered_map<int, int> by_lds;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = by_lds.find(lds_bytes);
+    if (it != by_lds.end()) return it->second;
+    if (lds_bytes > lk_device().lds_bytes) return 0;
+    if (lds_bytes > 48 * 1024 &&
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    int r = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)kernel, WG, (size_t)lds_bytes) != hipSuccess || r < 1) {
+        (void)hipGetLastError();
+        r = 1;
+    }
+    r = r > 8 ? 8 : r;
+    by_lds.emplace(lds_bytes, r);
+    return r;
+}
+
+template <class E, int MODE>
+static int launch_mode(const uint8_t* w0, const uint8_t* w1, const uint8_t* acts, const int32_t* sti,
+                       const int32_t* eid, const float* tw, const float* bias, float* out, const MoeDims& d,
+                       hipStream_t s) {
+    constexpr int R = MODE == MODE_GATED ? 1 : 2;
+    auto kernel = moe_rows_kernel<E, R, MODE>;
+    const int lds_bytes = lds_bytes_for<typename E::Fmt>(d.nb, 1);
+    const int per_cu = prepare(kernel, lds_bytes);
+    if (per_cu == 0) return LK_ERR_ARG;
+    const int tiles = (d.cols + R - 1) / R;
+    const int need = (tiles + WAVES - 1) / WAVES;
+    int share = lk_device().cus * per_cu / d.pairs;
+    if (share < 1) share = 1;
+    const dim3 grid(need < share ? need : share, d.pairs);
+    if (grid.y > 65535u) return LK_ERR_ARG;
+    hipLaunchKernelGGL(kernel, grid, dim3(WG), lds_bytes, s, w0, w1, acts, sti, eid, tw, bias, out, d);
+    return lk_launch_status();
+}
+
+template <int MODE>
+static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts, const int32_t* sti,
+                         const int32_t* eid, const float* tw, const float* bias, float* out, MoeDims d, int size_k,
+                         hipStream_t s) {
+    switch (quant_type) {   // wire ids of the reference's MOE_GGUF_FORMATS table (cuda/moe/gguf.cuh:55-71)
+        case 0:
+            d.nb = size_k / 32; d.slab_bytes = (int64_t)d.cols * d.nb * Q80_BYTES;
+            return launch_mode<EngQ80, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
+        case 1:
+            d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q4K_BYTES;
+            return launch_mode<EngQ4K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
+        case 5:
+            d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q6K_BYTES;
+            return launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
+        default:
+            return LK_ERR_TYPE;
+    }
+}
+
+static int block_len_of_wire(int quant_type) {
+    return quant_type == 0 ? 32 : (quant_type == 1 || quant_type == 5) ? 256 : 0;
+}
+
+static bool bad_shape(int quant_type, int num_experts, int topk, int size_m, int size_n, int size_k) {
+    const int bl = block_len_of_wire(quant_type);
+    return bl == 0 || num_experts <= 0 || topk <= 0 || size_m < 0 || size_n <= 0 || size_k <= 0 ||
+           size_k % bl != 0 || size_m % topk != 0;
+}
+
+static inline int pad512(int k) { return (k + 511) / 512 * 512; }
+
+}  // namespace
+
+extern "C" void loken_stream_scratch_release() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    for (auto it = g_scratch.begin(); it != g_scratch.end();) {
+        if (it->device != dev) { ++it; continue; }
+        if (it->ptr) (void)hipFree(it->ptr);
+        for (void* p : it->kept) (void)hipFree(p);
+        it = g_scratch.erase(it);
+    }
+}
+
+extern "C" void loken_moe_sum_topk(const float* pairs, float* outputs, int tokens, int topk, int cols, void* stream) {
+    if (tokens <= 0 || cols <= 0) return;
+    const size_t total = (size_t)tokens * cols;
+    hipLaunchKernelGGL(sum_topk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, pairs,
+                       (const float*)nullptr, outputs, tokens, topk, cols);
+    (void)hipGetLastError();
+}
+
+extern "C" int loken_moe_gemm_gguf(const float* inputs, const void* weights, const int32_t* sorted_token_ids,
+                                   const int32_t* expert_ids, const float* topk_weights, void* outputs,
+                                   int num_experts, int topk, int size_m, int size_n, int size_k, int quant_type,
+                                   void* stream) {
+    if (block_len_of_wire(quant_type) == 0) return LK_ERR_TYPE;
+    if (size_m == 0) return LK_OK;
+    if (!inputs || !weights || !sorted_token_ids || !expert_ids || !outputs ||
+        bad_shape(quant_type, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const int kp = pad512(size_k);
+    // with routing weights every entry has its own activation row; without, topk entries share one
+    const int act_rows = topk_weights ? size_m : size_m / topk;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    uint8_t* acts = (uint8_t*)reserve_scratch((size_t)act_rows * (kp / 32) * Q81_BYTES, s);
+    if (!acts) return LK_ERR_NOMEM;
+    if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, acts, size_k, kp, act_rows, stream)) return rc;
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0};
+    return launch_format<MODE_PLAIN>(quant_type, (const uint8_t*)weights, nullptr, acts, sorted_token_ids, expert_ids,
+                                     topk_weights, nullptr, (float*)outputs, d, size_k, s);
+}
+
+extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const void* gate_weights,
+                                                    const void* up_weights, const int32_t* sorted_token_ids,
+                                                    const int32_t* expert_ids, float* outputs, int num_experts,
+                                                    int topk, int size_m, int size_n, int size_k, int quant_type,
+                                                    void* stream) {
+    if (block_len_of_wire(quant_type) == 0) return LK_ERR_TYPE;
+    if (size_m == 0) return LK_OK;
+    if (!inputs || !gate_weights || !up_weights || !sorted_token_ids || !expert_ids || !outputs ||
+        bad_shape(quant_type, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const int kp = pad512(size_k), act_rows = size_m / topk;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    uint8_t* acts = (uint8_t*)reserve_scratch((size_t)act_rows * (kp / 32) * Q81_BYTES, s);
+    if (!acts) return LK_ERR_NOMEM;
+    if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, acts, size_k, kp, act_rows, stream)) return rc;
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0};
+    return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights, acts,
+                                     sorted_token_ids, expert_ids, nullptr, nullptr, outputs, d, size_k, s);
+}
+
+extern "C" int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,
+                                               const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                               const float* topk_weights, float* outputs, int num_experts, int topk,
+                                               int size_m, int size_n, int size_k, int gguf_dtype,
+                                               const float* down_bias, const float* add_after, void* stream) {
+    if (block_len_of_wire(gguf_dtype) == 0) return LK_ERR_TYPE;
+    if (size_m == 0) return LK_OK;
+    if (!inputs || !weights || !sorted_token_ids || !expert_ids || !topk_weights || !outputs ||
+        bad_shape(gguf_dtype, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const int kp = pad512(size_k);
+    const size_t act_bytes = (((size_t)size_m * (kp / 32) * Q81_BYTES) + 255) & ~(size_t)255;
+    const size_t pair_bytes = (size_t)size_m * size_n * sizeof(float);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    uint8_t* base = (uint8_t*)reserve_scratch(act_bytes + pair_bytes, s);
+    if (!base) return LK_ERR_NOMEM;
+    float* pairs = (float*)(base + act_bytes);
+    if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, base, size_k, kp, size_m, stream)) return rc;
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0};
+    if (int rc = launch_format<MODE_DOWN>(gguf_dtype, (const uint8_t*)weights, nullptr, base, sorted_token_ids,
+                                          expert_ids, topk_weights, down_bias, pairs, d, size_k, s)) return rc;
+    const int tokens = size_m / topk;
+    const size_t total = (size_t)tokens * size_n;
+    hipLaunchKernelGGL(sum_topk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (const float*)pairs,
+                       add_after, outputs, tokens, topk, size_n);
+    return lk_launch_status();
+}

@@ -124,3 +124,87 @@ class MmqRouting:
         _lib.load().loken_moe_mmq_fold(pairs.data_ptr(), w.data_ptr(), None, None, out.data_ptr(), self.tokens,
                                        self.topk, hidden, _stream())
         return out
+
+
+# ------------------------------------------------------------------------------------ decode
+# loken's wire ids for the MoE decode launchers (EXPERT_QUANT_CODES, cuda/moe/gguf.cuh:55-71)
+EXPERT_QUANT_CODES = {_lib.TYPE_Q8_0: 0, _lib.TYPE_Q4_K: 1, _lib.TYPE_Q6_K: 5}
+
+
+class ExpertRouting:
+    """The routing grouped by expert: a stable sort of the flattened (token, choice) slots by
+    expert id (ExpertRouting::group, src/inference/generic_transformer/moe_weights.rs:27-54,102-116)."""
+
+    def __init__(self, choices: torch.Tensor):
+        flat = choices.reshape(-1).to(torch.int64)
+        order = torch.sort(flat, stable=True).indices
+        self.sorted_token_ids = order.to(torch.int32).contiguous()
+        self.expert_ids = flat[order].to(torch.int32).contiguous()
+        self.tokens, self.topk = choices.shape
+
+
+def moe_gemm_gguf_gate_up_silu_mul(wtype: int, x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                                   routing: ExpertRouting, n_experts: int, ffn: int) -> torch.Tensor:
+    """``[tokens, k]`` -> ``[tokens * topk, ffn]`` in SLOT order (src/inference/moe_cuda/gemm.rs:285-302)."""
+    tokens, k = x.shape
+    pairs = tokens * routing.topk
+    out = torch.empty((pairs, ffn), dtype=torch.float32, device=x.device)
+    _lib.check("loken_moe_gemm_gguf_gate_up_silu_mul", _lib.load().loken_moe_gemm_gguf_gate_up_silu_mul(
+        x.data_ptr(), gate.data_ptr(), up.data_ptr(), routing.sorted_token_ids.data_ptr(),
+        routing.expert_ids.data_ptr(), out.data_ptr(), n_experts, routing.topk, pairs, ffn, k,
+        EXPERT_QUANT_CODES[wtype], _stream()))
+    return out
+
+
+def moe_gemm_gguf_down_reduce(wtype: int, h: torch.Tensor, down: torch.Tensor, routing: ExpertRouting,
+                              topk_weights: torch.Tensor, n_experts: int, hidden: int,
+                              residual: torch.Tensor | None = None, down_bias: torch.Tensor | None = None,
+                              add_after: torch.Tensor | None = None) -> torch.Tensor:
+    """``[tokens * topk, k]`` in slot order -> ``[tokens, hidden]`` (src/inference/moe_cuda/mod.rs:437-441)."""
+    pairs, k = h.shape
+    tokens = pairs // routing.topk
+    out = (residual.to(torch.float32).clone() if residual is not None
+           else torch.zeros((tokens, hidden), dtype=torch.float32, device=h.device))
+    w = topk_weights.to(torch.float32).contiguous()
+    _lib.check("loken_moe_gemm_gguf_down_reduce", _lib.load().loken_moe_gemm_gguf_down_reduce(
+        h.data_ptr(), down.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+        w.data_ptr(), out.data_ptr(), n_experts, routing.topk, pairs, hidden, k, EXPERT_QUANT_CODES[wtype],
+        down_bias.data_ptr() if down_bias is not None else None,
+        add_after.data_ptr() if add_after is not None else None, _stream()))
+    return out
+
+
+def moe_gemm_gguf(wtype: int, x: torch.Tensor, weights: torch.Tensor, routing: ExpertRouting, n_experts: int, n: int,
+                  topk_weights: torch.Tensor | None = None) -> torch.Tensor:
+    """One routed product per pair, rows in slot order (src/inference/moe_cuda/gemm.rs:18-...)."""
+    k = x.shape[1]
+    pairs = routing.tokens * routing.topk
+    out = torch.empty((pairs, n), dtype=torch.float32, device=x.device)
+    _lib.check("loken_moe_gemm_gguf", _lib.load().loken_moe_gemm_gguf(
+        x.data_ptr(), weights.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+        topk_weights.data_ptr() if topk_weights is not None else None, out.data_ptr(), n_experts, routing.topk,
+        pairs, n, k, EXPERT_QUANT_CODES[wtype], _stream()))
+    return out
+
+
+def moe_mmq_pays(rows: int, experts: int) -> bool:
+    """Routed rows from which the expert-batched matmul beats the per-pair kernels
+    (mmq_experts.rs:72-86: break-even at one routed row per expert)."""
+    return rows >= max(experts, 1)
+
+
+def moe_forward(wtype_gu: int, wtype_down: int, x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                down: torch.Tensor, choices: torch.Tensor, topk_weights: torch.Tensor, n_experts: int,
+                ffn: int) -> torch.Tensor:
+    """The expert block of one layer, path chosen as the reference's layer code chooses it
+    (src/inference/generic_transformer/moe_weights.rs:2118-2152): the expert-batched tiled
+    matmuls when there is at least a routed row per expert, else one mat-vec per routed pair."""
+    tokens, hidden = x.shape
+    topk = choices.shape[1]
+    if moe_mmq_pays(tokens * topk, n_experts) and moe_mmq_serves(wtype_gu, hidden) and moe_mmq_serves(wtype_down, ffn):
+        plan = MmqRouting.from_choices(choices, n_experts)
+        h = plan.gate_up_silu(wtype_gu, x, gate, up, ffn)
+        return plan.down_fold(wtype_down, h, down, hidden, topk_weights.reshape(-1))
+    routing = ExpertRouting(choices)
+    h = moe_gemm_gguf_gate_up_silu_mul(wtype_gu, x.contiguous(), gate, up, routing, n_experts, ffn)
+    return moe_gemm_gguf_down_reduce(wtype_down, h, down, routing, topk_weights.reshape(-1), n_experts, hidden)

@@ -178,3 +178,114 @@ def test_benchmark_shape_256_tokens_against_sampled_oracle():
     # every routed pair landed somewhere: the per-expert load adds up
     bounds = plan.bounds.cpu().numpy()
     assert bounds[-1] == tokens * topk and (np.diff(bounds) >= 0).all()
+
+
+# ---------------------------------------------------------------- decode (per routed pair)
+from loken_amd.moe import (ExpertRouting, moe_forward, moe_gemm_gguf, moe_gemm_gguf_down_reduce,
+                           moe_gemm_gguf_gate_up_silu_mul)
+
+
+def slot_order(h_sorted, ids):
+    """oracle rows are in sorted order; the decode kernels write slot order"""
+    slots, _ = oracle.group_by_expert(ids)
+    out = np.empty_like(h_sorted)
+    out[slots] = h_sorted
+    return out
+
+
+@pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(1, 2048, 768, 128, 8), (3, 512, 256, 6, 2),
+                                                             (16, 1024, 768, 32, 4)])
+@pytest.mark.parametrize("dt_down", [lib.TYPE_Q4_K, lib.TYPE_Q6_K])
+def test_per_pair_decode_block_matches_oracle(tokens, hidden, ffn, n_experts, topk, dt_down):
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=57, dt_down=dt_down)
+    want, want_h = oracle.moe_forward(1, lib.TYPE_Q4_K, dt_down, x, gate, up, down, ids, w, n_experts, ffn, want_h=True)
+    routing = ExpertRouting(dev(ids))
+    slots, experts = oracle.group_by_expert(ids)
+    assert routing.sorted_token_ids.cpu().tolist() == slots.tolist()
+    assert routing.expert_ids.cpu().tolist() == experts.tolist()
+    h = moe_gemm_gguf_gate_up_silu_mul(lib.TYPE_Q4_K, dev(x), dev(gate), dev(up), routing, n_experts, ffn)
+    want_slot = slot_order(want_h, ids)
+    assert (np.abs(h.cpu().numpy() - want_slot) <= 1e-3 * np.abs(want_slot) + 1e-4 * np.abs(want_slot).max()).all()
+    out = moe_gemm_gguf_down_reduce(dt_down, h, dev(down), routing, dev(w.reshape(-1)), n_experts, hidden)
+    scale = np.abs(want).max()
+    assert (np.abs(out.cpu().numpy() - want) <= 2e-3 * np.abs(want) + 2e-4 * scale).all()
+
+
+def test_decode_down_reduce_is_tight_on_oracle_rows_and_folds_in_slot_order():
+    tokens, hidden, ffn, n_experts, topk = 4, 512, 512, 8, 3
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=58)
+    want, want_h = oracle.moe_forward(1, lib.TYPE_Q4_K, lib.TYPE_Q4_K, x, gate, up, down, ids, w, n_experts, ffn, want_h=True)
+    routing = ExpertRouting(dev(ids))
+    h = dev(slot_order(want_h, ids))
+    out = moe_gemm_gguf_down_reduce(lib.TYPE_Q4_K, h, dev(down), routing, dev(w.reshape(-1)), n_experts, hidden)
+    assert_close(out.cpu().numpy(), want, atol=1e-4 * max(1.0, np.abs(want).max()))
+    # residual as the starting value, add_after as a written sum, bias scaled by the router weight
+    res = torch.randn((tokens, hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(5))
+    with_res = moe_gemm_gguf_down_reduce(lib.TYPE_Q4_K, h, dev(down), routing, dev(w.reshape(-1)), n_experts, hidden, residual=res)
+    added = moe_gemm_gguf_down_reduce(lib.TYPE_Q4_K, h, dev(down), routing, dev(w.reshape(-1)), n_experts, hidden, add_after=res)
+    scale = out.abs().max().item() + res.abs().max().item()
+    assert (with_res - (out + res)).abs().max().item() <= 1e-6 * scale
+    assert (added - (out + res)).abs().max().item() <= 1e-6 * scale
+    bias = torch.randn((n_experts, hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(6))
+    biased = moe_gemm_gguf_down_reduce(lib.TYPE_Q4_K, h, dev(down), routing, dev(w.reshape(-1)), n_experts, hidden, down_bias=bias)
+    wt = dev(w)
+    extra = (wt.unsqueeze(-1) * bias[dev(ids).long()]).sum(dim=1)
+    assert (biased - (out + extra)).abs().max().item() <= 1e-5 * (scale + extra.abs().max().item())
+
+
+def test_generic_routed_product_with_and_without_weights():
+    tokens, k, n, n_experts, topk = 5, 512, 96, 7, 2
+    wq = synth.weight(lib.TYPE_Q8_0, n_experts * n, k, seed=59, stream=1)
+    x = synth.activation(tokens, k, seed=59)
+    ids, w = oracle.topk_softmax(synth.activation(tokens, n_experts, seed=59, stream=7), topk)
+    routing = ExpertRouting(dev(ids))
+    we = wq.reshape(n_experts, n, -1, 34)
+    plain = moe_gemm_gguf(lib.TYPE_Q8_0, dev(x), dev(wq), routing, n_experts, n).cpu().numpy()
+    for t in range(tokens):
+        for j in range(topk):
+            assert_close(plain[t * topk + j], oracle.ob_matmul(lib.TYPE_Q8_0, x[t:t + 1], we[ids[t, j]], n)[0])
+    # with routing weights: one activation row per slot, output scaled
+    xs = synth.activation(tokens * topk, k, seed=59, stream=8)
+    scaled = moe_gemm_gguf(lib.TYPE_Q8_0, dev(xs), dev(wq), routing, n_experts, n, topk_weights=dev(w.reshape(-1))).cpu().numpy()
+    for p in range(tokens * topk):
+        e = ids.reshape(-1)[p]
+        assert_close(scaled[p], w.reshape(-1)[p] * oracle.ob_matmul(lib.TYPE_Q8_0, xs[p:p + 1], we[e], n)[0])
+
+
+def test_pairs_the_routing_leaves_out_add_nothing():
+    tokens, hidden, ffn, n_experts, topk = 3, 256, 256, 4, 2
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=60)
+    routing = ExpertRouting(dev(ids))
+    h = moe_gemm_gguf_gate_up_silu_mul(lib.TYPE_Q4_K, dev(x), dev(gate), dev(up), routing, n_experts, ffn)
+    full = moe_gemm_gguf_down_reduce(lib.TYPE_Q4_K, h, dev(down), routing, dev(w.reshape(-1)), n_experts, hidden)
+    # mark the first sorted pair as belonging to no expert: the fold must see zeros for it
+    dropped = routing.sorted_token_ids[0].item()
+    routing.expert_ids[0] = n_experts + 3
+    part = moe_gemm_gguf_down_reduce(lib.TYPE_Q4_K, h, dev(down), routing, dev(w.reshape(-1)), n_experts, hidden)
+    t = dropped // topk
+    others = [i for i in range(tokens) if i != t]
+    assert torch.equal(part[others], full[others])
+    assert not torch.equal(part[t], full[t])
+
+
+def test_launchers_report_bad_arguments_and_formats():
+    l = lib.load()
+    buf = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    p, s = buf.data_ptr(), torch.cuda.current_stream().cuda_stream
+    assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 4, 8, 256, 2, s) == lib.LK_ERR_TYPE     # q2_K: not served
+    assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 4, 8, 250, 1, s) == lib.LK_ERR_ARG      # k not whole blocks
+    assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 5, 8, 256, 1, s) == lib.LK_ERR_ARG      # pairs % topk
+    assert l.loken_moe_gemm_gguf_down_reduce(p, p, p, p, None, p, 4, 2, 4, 8, 256, 1, None, None, s) == lib.LK_ERR_ARG
+    assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 0, 8, 256, 1, s) == lib.LK_OK           # nothing routed
+    l.loken_stream_scratch_release()
+
+
+@pytest.mark.parametrize("tokens", [1, 16, 256])
+def test_layer_entry_picks_a_path_and_both_agree(tokens):
+    hidden, ffn, n_experts, topk = 512, 256, 16, 4
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=61)
+    args = (lib.TYPE_Q4_K, lib.TYPE_Q4_K, dev(x), dev(gate), dev(up), dev(down), dev(ids), dev(w), n_experts, ffn)
+    got = moe_forward(*args).cpu().numpy()
+    want = oracle.moe_forward(1, lib.TYPE_Q4_K, lib.TYPE_Q4_K, x, gate, up, down, ids, w, n_experts, ffn)
+    scale = np.abs(want).max()
+    assert (np.abs(got - want) <= 2e-3 * np.abs(want) + 2e-4 * scale).all()
