@@ -4,8 +4,10 @@
 One *step* = every quantized linear of one Llama-3-8B-shaped decode step at batch `--batch`
 (default 1): per layer q, o 4096->4096, k, v 4096->1024, gate, up 4096->14336 in Q4_K and down
 14336->4096 in Q6_K, 32 layers, then lm_head 4096->128256 in Q8_0: 225 weight matrices,
-4.97 GB of blocks, each linear preceded by the Q8_1 quantization of its activation (q/k/v and
-gate/up share one). Distinct weights per layer, so the step is cache-cold by construction.
+4.97 GB of blocks. Default launch plan (`--plan fused`): the linears that share an activation go
+out as one launch (q,k,v; gate,up) and every launch quantizes its f32 activation to Q8_1 in LDS
+itself, 4 launches per layer; `--plan split` is the two-launch form per linear (Q8_1 quantizer,
+then mat-vec). Distinct weights per layer, so the step is cache-cold by construction.
 Weights and activations are synthetic (seeded, generated on the device) and resident in HBM
 before the timed region.
 
@@ -42,6 +44,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=1, help="activation rows per mat-vec (1..8)")
     ap.add_argument("--layers", type=int, default=LAYERS)
+    ap.add_argument("--plan", choices=["fused", "split"], default="fused",
+                    help="fused: shared-activation linears per launch, Q8_1 quantized in-kernel; split: quantize + mat-vec per linear")
     ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -134,9 +138,40 @@ def main() -> int:
             q4k_bytes += nbytes
         return out
 
+    import ctypes as C
+
+    def add_fused(wtype, ws, g, ns, k):
+        """One launch: the matrices `ws` (ns rows each) over activation group `g`, quantized in-kernel."""
+        nonlocal total_bytes, q4k_bytes
+        a = acts[g]
+        stride = max(ns)
+        outs = [torch.empty((b, stride), dtype=torch.float32, device=dev) for _ in ns]
+        vx = (C.c_void_p * len(ws))(*[w.data_ptr() for w in ws])
+        dst = (C.c_void_p * len(ws))(*[o.data_ptr() for o in outs])
+        nn = (C.c_int * len(ws))(*ns)
+        keep.extend(outs + [vx, dst, nn])
+        item = (L.lk_mmvq_fused, (wtype, len(ws), vx, a.data_ptr(), a.stride(0), dst, lib.TYPE_F32, k, nn, b,
+                                  stride, None, stream))
+        plan.append(item)
+        nbytes = sum(synth.weight_bytes(wtype, n, k) for n in ns)
+        total_bytes += nbytes
+        if wtype == Q4K:
+            q4k_plan.append(item)
+            q4k_bytes += nbytes
+        return outs[0]
+
     first_out = None
     first_w = None
     for layer in range(args.layers):
+        if args.plan == "fused":
+            made = {name: (maker(n, k), wtype, n, k, g) for name, wtype, n, k, maker, g in shapes}
+            keep.extend(v[0] for v in made.values())
+            for group in (("q", "k", "v"), ("o",), ("gate", "up"), ("down",)):
+                wtype, k, g = made[group[0]][1], made[group[0]][3], made[group[0]][4]
+                out = add_fused(wtype, [made[nm][0] for nm in group], g, [made[nm][2] for nm in group], k)
+                if first_out is None:
+                    first_out, first_w = out, made["q"][0]
+            continue
         last_group = None
         for name, wtype, n, k, maker, g in shapes:
             w = maker(n, k)
@@ -149,8 +184,11 @@ def main() -> int:
                 first_out, first_w = out, w
     lm_head = make_q80(VOCAB, HIDDEN)
     keep.append(lm_head)
-    add_quant("final")
-    add_gemv(Q80, lm_head, "final", VOCAB, HIDDEN)
+    if args.plan == "fused":
+        add_fused(Q80, [lm_head], "final", [VOCAB], HIDDEN)
+    else:
+        add_quant("final")
+        add_gemv(Q80, lm_head, "final", VOCAB, HIDDEN)
     torch.cuda.synchronize()
 
     def run(items):
@@ -212,7 +250,7 @@ def main() -> int:
     achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": f"mmvq_q4k_kernel<{b},*,float>", "avg_launch_us": round(avg_us, 3),
+                "kernel": f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches}
 
     # ------------------------------------------------------------------ CPU baseline leg
@@ -227,7 +265,7 @@ def main() -> int:
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"llama3-8b decode-step quantized linears (Q4_K q,k,v,o,gate,up; Q6_K down; "
                                f"Q8_0 lm_head), batch {b}, {args.layers} layers",
-                   "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
+                   "launch_plan": args.plan, "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
                    "hip_graph": graph is not None},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": roofline,

@@ -88,6 +88,17 @@ int lk_mmvq_multi(int wtype, int count, const void* const* vx, const void* vy_q8
                   int dst_type, int ncols_x, const int* nrows_x, int batch, int stride_col_y,
                   int stride_col_dst, const float* const* bias, void* stream);
 
+/* lk_mmvq_multi straight from f32 activation rows (`batch` rows, `stride_x` floats apart, 16-byte
+ * aligned, stride a multiple of 4): every workgroup quantizes the rows to Q8_1 in LDS while it
+ * stages them, with the steps of lk_quantize_q8_1, so the outputs carry the bits of the
+ * two-launch path and the quantize launch disappears. This is what QKernelMatMul::forward does
+ * for a decode row (quantize, then mat-vec: src/tensor/quantized/kernel_matmul.rs:1474-1487,
+ * 658-691) folded into one launch, in the spirit of the reference's fused Q8_1 producers
+ * (src/inference/cuda/mmvq_gguf.cu:760-1000; src/tensor/cuda/prequant.rs). */
+int lk_mmvq_fused(int wtype, int count, const void* const* vx, const float* x, int stride_x,
+                  void* const* dst, int dst_type, int ncols_x, const int* nrows_x, int batch,
+                  int stride_col_dst, const float* const* bias, void* stream);
+
 /* dst[j, row] = act(gate row . x_j) * (up row . x_j), act 0 = SiLU g/(1+exp(-g)), 1 = tanh-GELU;
  * gate and up have the same shape; batch 1..4; dst f32 or bf16. Replaces kernels
  * `mmvq_gguf_pair_{g}_{u}_silu*_cuda1` and `mmvq_gguf_q4_k_{f32,bf16}_fused_{silu,gelu}_cuda1`

@@ -40,14 +40,15 @@ struct MultiArgs {
 
 template <class E, int B, int R, typename T>
 __global__ __launch_bounds__(WG) void mmvq_kernel(MultiArgs m, const uint8_t* __restrict__ vy, int nb,
-                                                  int stride_col_y, int stride_col_dst) {
+                                                  int stride_col_y, int stride_col_dst, int act_stride_f32) {
     extern __shared__ __align__(16) uint8_t lds[];
     int w = 0;
 #pragma unroll
     for (int i = 1; i < MAX_MULTI; ++i)
         if (i < m.count && (int)blockIdx.x >= m.wg_begin[i]) w = i;
     const int wgs = m.wg_begin[w + 1] - m.wg_begin[w];
-    RowJob<1> job{{m.vx[w]}, vy, nb, m.n[w], stride_col_y, wgs * WAVES, ((int)blockIdx.x - m.wg_begin[w]) * WAVES};
+    RowJob<1> job{{m.vx[w]}, vy, nb, m.n[w], stride_col_y, wgs * WAVES, ((int)blockIdx.x - m.wg_begin[w]) * WAVES,
+                  act_stride_f32};
     T* dst = (T*)m.dst[w];
     const float* bias = m.bias[w];
     E::template run<B, R, 1>(job, lds, [&](int row, int c, const float* tot) {
@@ -220,12 +221,12 @@ struct MmvqCall {
     MultiArgs m;
     const uint8_t* vy;
     int nb, stride_col_y, stride_col_dst;
+    int act_stride_f32;  // non-zero: vy is f32 rows, quantized in the kernel
     hipStream_t stream;
 };
 
-template <class E, int B, typename T>
-static int launch_plain(MmvqCall& a) {
-    constexpr int R = 2;
+template <class E, int B, int R, typename T>
+static int launch_plain_r(MmvqCall& a) {
     auto kernel = mmvq_kernel<E, B, R, T>;
     const int lds_bytes = lds_bytes_for<typename E::Fmt>(a.nb, B);
     const int per_cu = resident_per_cu(kernel, lds_bytes);
@@ -249,8 +250,17 @@ static int launch_plain(MmvqCall& a) {
     }
     for (int i = a.m.count; i < MAX_MULTI; ++i) a.m.wg_begin[i + 1] = a.m.wg_begin[i];
     hipLaunchKernelGGL(kernel, dim3(a.m.wg_begin[a.m.count]), dim3(WG), lds_bytes, a.stream, a.m, a.vy, a.nb,
-                       a.stride_col_y, a.stride_col_dst);
+                       a.stride_col_y, a.stride_col_dst, a.act_stride_f32);
     return lk_launch_status();
+}
+
+// Rows per wave: two rows share every activation read. LK_TUNE_R=1 selects one row per tile for
+// measurement runs (batch <= 4).
+template <class E, int B, typename T>
+static int launch_plain(MmvqCall& a) {
+    static const int forced = tune_env("LK_TUNE_R");
+    if (B <= 4 && forced == 1) return launch_plain_r<E, B, 1, T>(a);
+    return launch_plain_r<E, B, 2, T>(a);
 }
 
 #define LK_BATCH_SWITCH(FN, E, T, ARG)                                                                 \
@@ -293,14 +303,16 @@ static int check_weight(int wtype, const void* vx) {
 
 static int run_multi(int wtype, int count, const void* const* vx, const void* vy, void* const* dst, int dst_type,
                      int ncols_x, const int* nrows_x, int batch, int stride_col_y, int stride_col_dst,
-                     const float* const* bias, void* stream) {
-    if (int rc = check_common(wtype, vy, ncols_x, batch, stride_col_y)) return rc;
+                     const float* const* bias, void* stream, int act_stride_f32 = 0) {
+    if (int rc = check_common(wtype, vy, ncols_x, batch, act_stride_f32 ? ncols_x / 32 : stride_col_y)) return rc;
+    if (act_stride_f32 && (act_stride_f32 < ncols_x || act_stride_f32 % 4 != 0 || ((uintptr_t)vy & 15) != 0)) return LK_ERR_ARG;
     if (count < 1 || count > MAX_MULTI) return LK_ERR_ARG;
     MmvqCall a{};
     a.vy = (const uint8_t*)vy;
     a.nb = ncols_x / block_len_of(wtype);
     a.stride_col_y = stride_col_y;
     a.stride_col_dst = stride_col_dst;
+    a.act_stride_f32 = act_stride_f32;
     a.stream = (hipStream_t)stream;
     int live = 0;
     for (int i = 0; i < count; ++i) {
@@ -373,6 +385,14 @@ extern "C" int lk_mmvq_multi(int wtype, int count, const void* const* vx, const 
     if (!vx || !dst || !nrows_x) return LK_ERR_ARG;
     return run_multi(wtype, count, vx, vy_q8_1, dst, dst_type, ncols_x, nrows_x, batch, stride_col_y, stride_col_dst,
                      bias, stream);
+}
+
+extern "C" int lk_mmvq_fused(int wtype, int count, const void* const* vx, const float* x, int stride_x,
+                             void* const* dst, int dst_type, int ncols_x, const int* nrows_x, int batch,
+                             int stride_col_dst, const float* const* bias, void* stream) {
+    if (!vx || !dst || !nrows_x || stride_x <= 0) return LK_ERR_ARG;
+    return run_multi(wtype, count, vx, x, dst, dst_type, ncols_x, nrows_x, batch, 0, stride_col_dst, bias, stream,
+                     stride_x);
 }
 
 extern "C" int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, const void* vy_q8_1, void* dst,

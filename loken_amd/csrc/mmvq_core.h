@@ -145,6 +145,65 @@ static __device__ __forceinline__ void stage_activation(uint8_t* lds, const uint
 }
 
 
+// The same staging from f32 rows: the workgroup quantizes each 32-value block itself, with the
+// steps of the stand-alone quantizer (d = amax/127 rounded to f16, codes = round_half_away(x *
+// (1/d)) with d before its rounding, integer code sum), so the staged bytes are the ones the
+// two-launch path stages. Eight lanes own a block, four values each.
+template <class F, int B>
+static __device__ __forceinline__ void stage_activation_f32(uint8_t* lds, const float* __restrict__ x, int k32,
+                                                            int n_iter, int x_stride) {
+#pragma clang fp contract(off)
+    const int per_pass = F::VPI / 32;
+    const int total = n_iter * per_pass;
+    const int row_bytes = lds_bytes_per_row<F>(n_iter);
+    constexpr int U = 4;  // loads issued together: the lane exchanges below would otherwise
+                          // serialize one memory latency per 1024 values
+    for (int t0 = threadIdx.x; t0 < total * 8; t0 += WG * U) {
+#pragma unroll
+        for (int c = 0; c < B; ++c) {
+            float4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int t = t0 + u * WG, j = t >> 3, l8 = t & 7;
+                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (t < total * 8 && j < k32) v[u] = *(const float4*)(x + (size_t)c * x_stride + j * 32 + l8 * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int t = t0 + u * WG, j = t >> 3, l8 = t & 7;
+                if (t >= total * 8) break;
+                const int it = j / per_pass, ji = j % per_pass;
+                float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
+                amax = fmaxf(amax, __shfl_xor(amax, 1));
+                amax = fmaxf(amax, __shfl_xor(amax, 2));
+                amax = fmaxf(amax, __shfl_xor(amax, 4));
+                const float d = amax / 127.0f;
+                const float inv = d != 0.0f ? 1.0f / d : 0.0f;
+                const int q0 = (int)roundf(v[u].x * inv), q1 = (int)roundf(v[u].y * inv);
+                const int q2 = (int)roundf(v[u].z * inv), q3 = (int)roundf(v[u].w * inv);
+                int sum = q0 + q1 + q2 + q3;
+                sum += __shfl_xor(sum, 1);
+                sum += __shfl_xor(sum, 2);
+                sum += __shfl_xor(sum, 4);
+                uint8_t* row = lds + c * row_bytes;
+                uint8_t* codes = row + it * F::PLANES * 1024;
+                *(uint32_t*)(codes + F::slot(ji, l8 >> 2) + 4 * (l8 & 3)) =
+                    (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
+                    ((uint32_t)(q3 & 0xFF) << 24);
+                if (l8 == 0) {
+                    float* sc = (float*)(row + n_iter * F::VPI);
+                    const float d8 = __half2float(__float2half_rn(d));
+                    if (F::SCF == 2) {
+                        *(float2*)(sc + 2 * j) = make_float2(d8, d8 * (float)sum);
+                    } else {
+                        sc[j] = d8;
+                    }
+                }
+            }
+        }
+    }
+}
+
 // What a workgroup computes: rows of `vx[0..NW)` against the B activation rows at `vy`.
 template <int NW>
 struct RowJob {
@@ -155,7 +214,18 @@ struct RowJob {
     int stride_col_y;  // Q8_1 blocks between activation rows
     int tile_stride;   // row tiles between a wave's consecutive tiles
     int tile_first;    // first row tile of wave 0 of this workgroup
+    int act_stride_f32 = 0;  // non-zero: `vy` holds f32 activation rows this many floats apart,
+                             // quantized to Q8_1 by the workgroup itself while staging
 };
+
+// The activation as the engines stage it, whichever form it arrives in.
+template <class F, int B, int NW>
+static __device__ __forceinline__ void stage_job(uint8_t* lds, const RowJob<NW>& job, int k32, int n_iter) {
+    if (job.act_stride_f32)
+        stage_activation_f32<F, B>(lds, (const float*)job.vy, k32, n_iter, job.act_stride_f32);
+    else
+        stage_activation<F, B>(lds, job.vy, k32, n_iter, job.stride_col_y);
+}
 
 // ---------------------------------------------------------------------------------------------
 // Q4_K: 4 lanes per super-block (32 bytes of qs each = two whole sub-blocks), 16 super-blocks
@@ -258,7 +328,7 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
     int tile = job.tile_first + wave, it = 0;
     Frag fa, fb;
     if (tile < n_tiles) load(fa, tile, 0);
-    stage_activation<FmtQ4K, B>(lds, job.vy, nb * 8, n_iter, job.stride_col_y);
+    stage_job<FmtQ4K, B>(lds, job, nb * 8, n_iter);
     __syncthreads();
     if (tile >= n_tiles) return;
     // Steps are (tile, pass) pairs in order; the loads of step i+1 are issued before step i is
@@ -287,7 +357,7 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
     const int nb = job.nb, n = job.n;
     const int n_iter = (nb + 7) >> 3;
     const int row_bytes = lds_bytes_per_row<FmtQ6K>(n_iter);
-    stage_activation<FmtQ6K, B>(lds, job.vy, nb * 8, n_iter, job.stride_col_y);
+    stage_job<FmtQ6K, B>(lds, job, nb * 8, n_iter);
     __syncthreads();
 
     const int lane = threadIdx.x & 63;
@@ -363,7 +433,7 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
     const int nb = job.nb, n = job.n;
     const int n_iter = (nb + 31) >> 5;
     const int row_bytes = lds_bytes_per_row<FmtQ80>(n_iter);
-    stage_activation<FmtQ80, B>(lds, job.vy, nb, n_iter, job.stride_col_y);
+    stage_job<FmtQ80, B>(lds, job, nb, n_iter);
     __syncthreads();
 
     const int lane = threadIdx.x & 63;

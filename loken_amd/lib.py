@@ -30,6 +30,7 @@ SIGNATURES = {
     "lk_quantize_q8_1": (_i, [_vp, _i, _vp, _i, _i, _i, _vp]),
     "lk_mmvq": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _i, _vp]),
     "lk_mmvq_multi": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _vp, _vp]),
+    "lk_mmvq_fused": (_i, [_i, _i, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _vp, _vp]),
     "lk_mmvq_pair_act": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "lk_mmvq_grouped": (_i, [_i, _vp, _i, _vp, _vp, _i, _i, _vp]),
     "lk_mmvq_subdots": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _vp]),

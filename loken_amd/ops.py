@@ -72,6 +72,21 @@ def mmvq_multi(wtype: int, weights, q8_1: torch.Tensor, k: int, ns, *, out_dtype
     return [o[:, :n] for o, n in zip(outs, ns)]
 
 
+def mmvq_fused(wtype: int, weights, x: torch.Tensor, ns, *, out_dtype: torch.dtype = torch.float32):
+    """Quantize-and-multiply in one launch: f32 rows ``x`` ``[b, k]`` against several matrices."""
+    import ctypes as C
+    b, k = x.shape
+    count = len(weights)
+    stride = max(ns)
+    outs = [torch.empty((b, stride), dtype=out_dtype, device=x.device) for _ in ns]
+    vx = (C.c_void_p * count)(*[w.data_ptr() for w in weights])
+    dst = (C.c_void_p * count)(*[o.data_ptr() for o in outs])
+    nn = (C.c_int * count)(*ns)
+    _lib.check("lk_mmvq_fused", _lib.load().lk_mmvq_fused(
+        wtype, count, vx, x.data_ptr(), x.stride(0), dst, _X_TYPES[out_dtype], k, nn, b, stride, None, _stream()))
+    return [o[:, :n] for o, n in zip(outs, ns)]
+
+
 def mmvq_pair_act(wtype: int, gate: torch.Tensor, up: torch.Tensor, q8_1: torch.Tensor, k: int, n: int, *,
                   act: str = "silu", out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """``act(gate . x) * (up . x)`` in one launch (fast_mmvq::try_fused)."""

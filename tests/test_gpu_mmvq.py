@@ -236,3 +236,16 @@ def test_grouped_launch_each_weight_over_its_own_row(name):
     got = ops.mmvq_grouped(wtype, table, q, k, n)
     for g in range(groups):
         assert torch.equal(got[g], ops.mmvq(wtype, ws[g], q[g:g + 1], k, n)[0])
+
+
+@pytest.mark.parametrize("name,k", [("q4_k", 4096), ("q4_k", 768), ("q6_k", 2304), ("q8_0", 1056), ("q8_0", 4096)])
+@pytest.mark.parametrize("batch", [1, 4])
+def test_quantize_in_kernel_path_carries_the_bits_of_the_two_launch_path(name, k, batch):
+    wtype = DT[name]
+    ns = [300, 64]
+    ws = [dev(synth.weight(wtype, n, k, seed=62, stream=30 + i)) for i, n in enumerate(ns)]
+    x = dev(synth.activation(batch, k, seed=62) * np.float32(3.0))
+    fused = ops.mmvq_fused(wtype, ws, x, ns)
+    q = ops.quantize_q8_1_rows(x)
+    for w, n, o in zip(ws, ns, fused):
+        assert torch.equal(o, ops.mmvq(wtype, w, q, k, n))
