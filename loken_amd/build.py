@@ -18,6 +18,9 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
 ]
+# MFMA results are consumed by VALU fix-ups right away: keep them in VGPRs instead of the
+# accumulator file, which would cost one v_accvgpr_read per value.
+PER_FILE_FLAGS = {"mmq.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def sources() -> list[Path]:
@@ -26,7 +29,7 @@ def sources() -> list[Path]:
 
 def _compile(src: Path) -> Path:
     obj = CSRC / (src.stem + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [HIPCC, *FLAGS, *PER_FILE_FLAGS.get(src.name, []), "-c", str(src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src.name}:\n{r.stderr[-6000:]}")

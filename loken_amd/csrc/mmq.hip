@@ -27,6 +27,7 @@
 
 #include "lk_common.h"
 
+#include <cstdlib>
 #include <mutex>
 #include <unordered_map>
 
@@ -105,21 +106,39 @@ static void launch_quantize(const void* x, const int32_t* ids, void* vy, int typ
 // Weight formats: how one 256-value block of TN rows becomes int8 sub-block tiles + scales.
 // LDS per step:  wq[8][TN][32] int8, aq[8][TM][32] int8, wsc[NS][TN] f32, wmn[8][TN] f32 (Q4_K),
 //                ad8[8][TM] f32, ads[8][TM] f32 (Q4_K).   NS = weight scales per block (8 or 16).
+// Staging is split in two so a step's global loads fly while the previous step is multiplied:
+// fetch() issues the loads into a register fragment, commit() expands the fragment into LDS.
 // --------------------------------------------------------------------------------------------
 struct MmqQ4K {
     static constexpr int BLOCK_BYTES = Q4K_BYTES;
     static constexpr int NS = 8;          // one weight scale per 32 values
     static constexpr bool HAS_MIN = true;
     static constexpr int BLOCKS_PER_STEP = 1;
+    static constexpr int QCH = TN * 8 / MMQ_WG;   // 16-byte qs chunks per thread per step
 
-    // rows [n0, n0+TN) of block kb -> LDS
-    static __device__ __forceinline__ void stage(const uint8_t* __restrict__ w, int64_t nb, int kb, int n0,
-                                                 int n, int8_t* wq, float* wsc, float* wmn) {
-        // nb: Q4_K blocks between consecutive rows
-        for (int idx = threadIdx.x; idx < TN * 8; idx += MMQ_WG) {
-            const int row = idx >> 3, c = idx & 7;
+    struct Frag {
+        uint4 q[QCH];
+        uint4 hdr;
+    };
+    // nb: Q4_K blocks between consecutive rows
+    static __device__ __forceinline__ void fetch(Frag& f, const uint8_t* __restrict__ w, int64_t nb, int kb,
+                                                 int n0, int n) {
+#pragma unroll
+        for (int i = 0; i < QCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, c = idx & 7;
             const int gn = min(n0 + row, n - 1);
-            const uint4 q = *(const uint4*)(w + ((int64_t)gn * nb + kb) * Q4K_BYTES + 16 + 16 * c);
+            f.q[i] = *(const uint4*)(w + ((int64_t)gn * nb + kb) * Q4K_BYTES + 16 + 16 * c);
+        }
+        if (threadIdx.x < TN) {
+            const int gn = min(n0 + (int)threadIdx.x, n - 1);
+            f.hdr = *(const uint4*)(w + ((int64_t)gn * nb + kb) * Q4K_BYTES);
+        }
+    }
+    static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
+#pragma unroll
+        for (int i = 0; i < QCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, c = idx & 7;
+            const uint4 q = f.q[i];
             uint4 lo, hi;
             lo.x = q.x & 0x0F0F0F0Fu; hi.x = (q.x >> 4) & 0x0F0F0F0Fu;
             lo.y = q.y & 0x0F0F0F0Fu; hi.y = (q.y >> 4) & 0x0F0F0F0Fu;
@@ -129,22 +148,22 @@ struct MmqQ4K {
             *(uint4*)(wq + ((2 * p) * TN + row) * 32 + 16 * h) = lo;
             *(uint4*)(wq + ((2 * p + 1) * TN + row) * 32 + 16 * h) = hi;
         }
-        for (int row = threadIdx.x; row < TN; row += MMQ_WG) {
+        if (threadIdx.x < TN) {
+            const int row = threadIdx.x;
             const bool live = n0 + row < n;
-            const int gn = min(n0 + row, n - 1);
-            const uint4 hdr = *(const uint4*)(w + ((int64_t)gn * nb + kb) * Q4K_BYTES);
-            const float d = live ? f16_bits_to_f32(hdr.x & 0xFFFFu) : 0.f;
-            const float dmin = live ? f16_bits_to_f32(hdr.x >> 16) : 0.f;
-            const uint8_t* p = (const uint8_t*)&hdr.y;  // the 12 packed bytes
+            const float d = live ? f16_bits_to_f32(f.hdr.x & 0xFFFFu) : 0.f;
+            const float dmin = live ? f16_bits_to_f32(f.hdr.x >> 16) : 0.f;
+            const uint32_t w1 = f.hdr.y, w2 = f.hdr.z, w3 = f.hdr.w;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                int sc, mn;
+                uint32_t sc, mn;
                 if (j < 4) {
-                    sc = p[j] & 63;
-                    mn = p[j + 4] & 63;
+                    sc = (w1 >> (8 * j)) & 63u;
+                    mn = (w2 >> (8 * j)) & 63u;
                 } else {
-                    sc = (p[j + 4] & 0xF) | ((p[j - 4] >> 6) << 4);
-                    mn = (p[j + 4] >> 4) | ((p[j] >> 6) << 4);
+                    const int t = j - 4;
+                    sc = ((w3 >> (8 * t)) & 0xFu) | ((((w1 >> (8 * t)) >> 6) & 3u) << 4);
+                    mn = ((w3 >> (8 * t + 4)) & 0xFu) | ((((w2 >> (8 * t)) >> 6) & 3u) << 4);
                 }
                 wsc[j * TN + row] = d * (float)sc;
                 wmn[j * TN + row] = -(dmin * (float)mn);
@@ -160,21 +179,42 @@ struct MmqQ6K {
     static constexpr int NS = 16;
     static constexpr bool HAS_MIN = false;
     static constexpr int BLOCKS_PER_STEP = 1;
+    static constexpr int QCH = TN * 8 / MMQ_WG;
 
+    struct Frag {
+        uint4 ql[QCH], qh[QCH];
+        uint4 sc;       // the sixteen scale bytes of this thread's row
+        uint32_t d;     // its f16 d
+    };
     static __device__ __forceinline__ uint32_t word(uint32_t ql, uint32_t qh, int nib_shift, int hi_shift) {
         const uint32_t code = ((ql >> nib_shift) & 0x0F0F0F0Fu) | (((qh >> hi_shift) & 0x03030303u) << 4);
         return (code + 0x60606060u) ^ 0x80808080u;  // per byte: code - 32, signed
     }
-    static __device__ __forceinline__ void stage(const uint8_t* __restrict__ w, int64_t nb, int kb, int n0,
-                                                 int n, int8_t* wq, float* wsc, float* wmn) {
-        (void)wmn;
-        for (int idx = threadIdx.x; idx < TN * 8; idx += MMQ_WG) {
-            const int row = idx >> 3, c = idx & 7;
-            const int h = c >> 2, g0 = (c >> 1) & 1, lh = c & 1;
+    static __device__ __forceinline__ void fetch(Frag& f, const uint8_t* __restrict__ w, int64_t nb, int kb,
+                                                 int n0, int n) {
+#pragma unroll
+        for (int i = 0; i < QCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, c = idx & 7;
+            const int h = c >> 2, lh = c & 1;
             const int gn = min(n0 + row, n - 1);
             const uint8_t* bp = w + ((int64_t)gn * nb + kb) * Q6K_BYTES;
-            const uint4 ql = *(const uint4_a2*)(bp + 16 * c);
-            const uint4 qh = *(const uint4_a2*)(bp + 128 + 16 * (2 * h + lh));
+            f.ql[i] = *(const uint4_a2*)(bp + 16 * c);
+            f.qh[i] = *(const uint4_a2*)(bp + 128 + 16 * (2 * h + lh));
+        }
+        if (threadIdx.x < TN) {
+            const int gn = min(n0 + (int)threadIdx.x, n - 1);
+            const uint8_t* bp = w + ((int64_t)gn * nb + kb) * Q6K_BYTES;
+            f.sc = *(const uint4_a2*)(bp + 192);
+            f.d = *(const uint16_t*)(bp + 208);
+        }
+    }
+    static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
+        (void)wmn;
+#pragma unroll
+        for (int i = 0; i < QCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, c = idx & 7;
+            const int h = c >> 2, g0 = (c >> 1) & 1, lh = c & 1;
+            const uint4 ql = f.ql[i], qh = f.qh[i];
             uint4 ca, cb;
             const int sh = 2 * g0;
             ca.x = word(ql.x, qh.x, 0, sh); cb.x = word(ql.x, qh.x, 4, sh + 4);
@@ -184,13 +224,13 @@ struct MmqQ6K {
             *(uint4*)(wq + ((4 * h + g0) * TN + row) * 32 + 16 * lh) = ca;
             *(uint4*)(wq + ((4 * h + g0 + 2) * TN + row) * 32 + 16 * lh) = cb;
         }
-        for (int idx = threadIdx.x; idx < TN * 16; idx += MMQ_WG) {
-            const int row = idx >> 4, j = idx & 15;
-            const bool live = n0 + row < n;
-            const int gn = min(n0 + row, n - 1);
-            const uint8_t* bp = w + ((int64_t)gn * nb + kb) * Q6K_BYTES;
-            const float d = live ? f16_bits_to_f32(*(const uint16_t*)(bp + 208)) : 0.f;
-            wsc[j * TN + row] = d * (float)((const int8_t*)bp)[192 + j];
+        if (threadIdx.x < TN) {
+            const int row = threadIdx.x;
+            const float d = n0 + row < n ? f16_bits_to_f32(f.d) : 0.f;
+            const uint32_t w[4] = {f.sc.x, f.sc.y, f.sc.z, f.sc.w};
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                wsc[j * TN + row] = d * (float)(int8_t)((w[j >> 2] >> (8 * (j & 3))) & 0xFFu);
         }
     }
 };
@@ -201,56 +241,83 @@ struct MmqQ80 {
     static constexpr int NS = 8;
     static constexpr bool HAS_MIN = false;
     static constexpr int BLOCKS_PER_STEP = 8;
+    static constexpr int QCH = TN * 16 / MMQ_WG, DCH = TN * 8 / MMQ_WG;
 
-    static __device__ __forceinline__ void stage(const uint8_t* __restrict__ w, int64_t nb, int kb, int n0,
-                                                 int n, int8_t* wq, float* wsc, float* wmn) {
-        (void)wmn;
-        for (int idx = threadIdx.x; idx < TN * 16; idx += MMQ_WG) {
-            const int row = idx >> 4, c = idx & 15, blk = c >> 1, h = c & 1;
+    struct Frag {
+        uint4 q[QCH];
+        uint32_t d[DCH];
+    };
+    static __device__ __forceinline__ void fetch(Frag& f, const uint8_t* __restrict__ w, int64_t nb, int kb,
+                                                 int n0, int n) {
+#pragma unroll
+        for (int i = 0; i < QCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 4, c = idx & 15, blk = c >> 1, h = c & 1;
             const int gn = min(n0 + row, n - 1);
-            const uint8_t* bp = w + ((int64_t)gn * nb + (int64_t)kb * 8 + blk) * Q80_BYTES;
-            *(uint4*)(wq + (blk * TN + row) * 32 + 16 * h) = *(const uint4_a2*)(bp + 2 + 16 * h);
+            f.q[i] = *(const uint4_a2*)(w + ((int64_t)gn * nb + (int64_t)kb * 8 + blk) * Q80_BYTES + 2 + 16 * h);
         }
-        for (int idx = threadIdx.x; idx < TN * 8; idx += MMQ_WG) {
-            const int row = idx >> 3, blk = idx & 7;
-            const bool live = n0 + row < n;
+#pragma unroll
+        for (int i = 0; i < DCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, blk = idx & 7;
             const int gn = min(n0 + row, n - 1);
-            const uint8_t* bp = w + ((int64_t)gn * nb + (int64_t)kb * 8 + blk) * Q80_BYTES;
-            wsc[blk * TN + row] = live ? f16_bits_to_f32(*(const uint16_t*)bp) : 0.f;
+            f.d[i] = *(const uint16_t*)(w + ((int64_t)gn * nb + (int64_t)kb * 8 + blk) * Q80_BYTES);
+        }
+    }
+    static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
+        (void)wmn;
+#pragma unroll
+        for (int i = 0; i < QCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 4, c = idx & 15, blk = c >> 1, h = c & 1;
+            *(uint4*)(wq + (blk * TN + row) * 32 + 16 * h) = f.q[i];
+        }
+#pragma unroll
+        for (int i = 0; i < DCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, blk = idx & 7;
+            wsc[blk * TN + row] = n0 + row < n ? f16_bits_to_f32(f.d[i]) : 0.f;
         }
     }
 };
 
-// Token rows [m0, m0+TM) of block kb (record layout above) -> LDS. Rows at or past m_end read as
-// zeros. `col_of` maps a tile row to its workspace row (identity for the dense product).
-template <int TM, bool WITH_SUMS>
-static __device__ __forceinline__ void stage_tokens(const uint8_t* __restrict__ y, int64_t rows_total, int kb,
-                                                    int m0, int m_end, int8_t* aq, float* ad8, float* ads) {
-    for (int idx = threadIdx.x; idx < TM * 18; idx += MMQ_WG) {
-        const int r = idx / 18, c = idx % 18;
-        const bool live = m0 + r < m_end;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (live) v = *(const uint4*)(y + ((int64_t)kb * rows_total + m0 + r) * REC_BYTES + 16 * c);
-        if (c < 16) {
-            *(uint4*)(aq + ((c >> 1) * TM + r) * 32 + 16 * (c & 1)) = v;
-        } else if (c == 16) {
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+// Token rows [m0, m0+TM) of block kb (record layout above). Rows at or past m_end read as zeros.
+template <int TM>
+struct TokenFrag {
+    static constexpr int CCH = (TM * 16 + MMQ_WG - 1) / MMQ_WG;   // code chunks per thread
+    uint4 codes[CCH];
+    uint4 d8, sums;   // thread r < TM: the scales and sums of row r
+
+    __device__ __forceinline__ void fetch(const uint8_t* __restrict__ y, int64_t rows_total, int kb, int m0, int m_end) {
 #pragma unroll
-            for (int s = 0; s < 8; ++s) ad8[s * TM + r] = f16_bits_to_f32((w[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
-        } else if (WITH_SUMS) {
-            // sums ride one chunk after the scales of the same record
-            const uint4 dv = live ? *(const uint4*)(y + ((int64_t)kb * rows_total + m0 + r) * REC_BYTES + 256)
-                                  : make_uint4(0, 0, 0, 0);
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w}, dw[4] = {dv.x, dv.y, dv.z, dv.w};
+        for (int i = 0; i < CCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, r = idx >> 4, c = idx & 15;
+            codes[i] = make_uint4(0, 0, 0, 0);
+            if (idx < TM * 16 && m0 + r < m_end)
+                codes[i] = *(const uint4*)(y + ((int64_t)kb * rows_total + m0 + r) * REC_BYTES + 16 * c);
+        }
+        d8 = sums = make_uint4(0, 0, 0, 0);
+        if ((int)threadIdx.x < TM && m0 + (int)threadIdx.x < m_end) {
+            const uint8_t* rec = y + ((int64_t)kb * rows_total + m0 + threadIdx.x) * REC_BYTES;
+            d8 = *(const uint4*)(rec + 256);
+            sums = *(const uint4*)(rec + 272);
+        }
+    }
+    template <bool WITH_SUMS>
+    __device__ __forceinline__ void commit(int8_t* aq, float* ad8, float* ads) const {
+#pragma unroll
+        for (int i = 0; i < CCH; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, r = idx >> 4, c = idx & 15;
+            if (idx < TM * 16) *(uint4*)(aq + ((c >> 1) * TM + r) * 32 + 16 * (c & 1)) = codes[i];
+        }
+        if ((int)threadIdx.x < TM) {
+            const int r = threadIdx.x;
+            const uint32_t dw[4] = {d8.x, d8.y, d8.z, d8.w}, sw[4] = {sums.x, sums.y, sums.z, sums.w};
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
-                const float d8 = f16_bits_to_f32((dw[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
-                const int sum = (int)(int16_t)((w[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
-                ads[s * TM + r] = d8 * (float)sum;
+                const float d = f16_bits_to_f32((dw[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
+                ad8[s * TM + r] = d;
+                if (WITH_SUMS) ads[s * TM + r] = d * (float)(int)(int16_t)((sw[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
             }
         }
     }
-}
+};
 
 // One problem = one weight slab against a contiguous run of workspace rows.
 struct MmqProblem {
@@ -291,11 +358,20 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[it][jt][v] = 0.f;
 
+    typename F::Frag wf;
+    TokenFrag<TM> tf;
+    F::fetch(wf, pb.w, pb.row_blocks, 0, n0, pb.n);
+    tf.fetch(pb.y, pb.rows_total, 0, m0, pb.m_end);
+
     for (int kb = 0; kb < pb.nb; ++kb) {
         __syncthreads();  // the previous step's readers are done with the tiles
-        F::stage(pb.w, pb.row_blocks, kb, n0, pb.n, wq, wsc, wmn);
-        stage_tokens<TM, F::HAS_MIN>(pb.y, pb.rows_total, kb, m0, pb.m_end, aq, ad8, ads);
+        F::commit(wf, n0, pb.n, wq, wsc, wmn);
+        tf.template commit<F::HAS_MIN>(aq, ad8, ads);
         __syncthreads();
+        if (kb + 1 < pb.nb) {  // next step's loads fly under this step's arithmetic
+            F::fetch(wf, pb.w, pb.row_blocks, kb + 1, n0, pb.n);
+            tf.fetch(pb.y, pb.rows_total, kb + 1, m0, pb.m_end);
+        }
 
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
@@ -392,7 +468,7 @@ static constexpr int mmq_lds_bytes() {
 // re-read the same weight rows) are issued back to back on the same XCD: ids are dealt round
 // robin over the 8 XCDs, so the XCD is id % 8 and its local sequence id / 8.
 template <class F, int TM, int WAVES_M>
-__global__ __launch_bounds__(MMQ_WG) void mmq_dense_kernel(MmqProblem pb, int n_tiles, int m_tiles) {
+__global__ __launch_bounds__(MMQ_WG, 2) void mmq_dense_kernel(MmqProblem pb, int n_tiles, int m_tiles) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int id = blockIdx.x;
     const int xcd = id & 7, seq = id >> 3;
@@ -406,7 +482,7 @@ __global__ __launch_bounds__(MMQ_WG) void mmq_dense_kernel(MmqProblem pb, int n_
 // grid = (n tiles, column tiles sized for the longest run the host expects, stacks * experts);
 // a run longer than the grid covers is walked by the same workgroups in further passes.
 template <class F, int TM, int WAVES_M>
-__global__ __launch_bounds__(MMQ_WG) void mmq_moe_kernel(MmqProblem pb, const uint8_t* w_second,
+__global__ __launch_bounds__(MMQ_WG, 2) void mmq_moe_kernel(MmqProblem pb, const uint8_t* w_second,
                                                          int64_t dst_second, const int32_t* __restrict__ bounds,
                                                          int64_t stride_expert, int n_experts) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -460,6 +536,7 @@ static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x
     hipStream_t s = (hipStream_t)stream;
     if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s);
     if (ncols_y <= 64) return launch_dense_tm<F, 64, 2>(pb, s);
+    if (getenv("LK_MMQ_TM64")) return launch_dense_tm<F, 64, 2>(pb, s);
     return launch_dense_tm<F, 128, 2>(pb, s);
 }
 
