@@ -20,6 +20,8 @@
 // on gfx950 serves unaligned dwordx4, the type only tells the compiler not to assume more.
 typedef uint4 __attribute__((aligned(2))) uint4_a2;
 typedef uint4 __attribute__((aligned(4))) uint4_a4;
+typedef uint2 __attribute__((aligned(2))) uint2_a2;
+typedef uint4 __attribute__((aligned(4))) uint4_a4;
 typedef uint32_t __attribute__((aligned(2))) uint32_a2;
 
 typedef int v4i __attribute__((ext_vector_type(4)));

@@ -328,12 +328,27 @@ static int run_multi(int wtype, int count, const void* const* vx, const void* vy
     }
     if (live == 0) return LK_OK;
     a.m.count = live;
-    switch (dst_type) {
-        case LK_TYPE_F32: return dispatch_plain<float>(wtype, batch, a);
-        case LK_TYPE_F16: return dispatch_plain<__half>(wtype, batch, a);
-        case LK_TYPE_BF16: return dispatch_plain<__hip_bfloat16>(wtype, batch, a);
-        default: return LK_ERR_TYPE;
+    if (dst_type != LK_TYPE_F32 && dst_type != LK_TYPE_F16 && dst_type != LK_TYPE_BF16) return LK_ERR_TYPE;
+    // A launch stages all its activation rows in LDS; a batch that does not fit (long rows) goes
+    // out as several launches over equal shares of the rows.
+    const int fit = lk_device().lds_bytes / lds_bytes_of(wtype, a.nb, 1);
+    if (fit < 1) return LK_ERR_ARG;
+    const int launches = (batch + fit - 1) / fit, share = (batch + launches - 1) / launches;
+    const size_t dst_elem = dst_type == LK_TYPE_F32 ? 4 : 2;
+    for (int b0 = 0; b0 < batch; b0 += share) {
+        const int b = batch - b0 < share ? batch - b0 : share;
+        MmvqCall c = a;
+        c.vy = a.vy + (act_stride_f32 ? (size_t)b0 * act_stride_f32 * sizeof(float) : (size_t)b0 * stride_col_y * Q81_BYTES);
+        for (int i = 0; i < live; ++i) c.m.dst[i] = (uint8_t*)a.m.dst[i] + (size_t)b0 * stride_col_dst * dst_elem;
+        int rc;
+        switch (dst_type) {
+            case LK_TYPE_F32: rc = dispatch_plain<float>(wtype, b, c); break;
+            case LK_TYPE_F16: rc = dispatch_plain<__half>(wtype, b, c); break;
+            default: rc = dispatch_plain<__hip_bfloat16>(wtype, b, c); break;
+        }
+        if (rc != LK_OK) return rc;
     }
+    return LK_OK;
 }
 
 template <class E, int B, typename T>
@@ -405,6 +420,19 @@ extern "C" int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, con
     if (!dst || nrows_x < 0 || stride_col_dst < nrows_x || (act != 0 && act != 1)) return LK_ERR_ARG;
     if (batch > 4) return LK_ERR_ARG;
     const int nb = ncols_x / block_len_of(wtype);
+    if (dst_type != LK_TYPE_F32 && dst_type != LK_TYPE_BF16) return LK_ERR_TYPE;
+    const int fit = lk_device().lds_bytes / lds_bytes_of(wtype, nb, 1);
+    if (fit < 1) return LK_ERR_ARG;
+    if (batch > fit) {   // rows too long to stage the whole batch: one launch per share of it
+        for (int b0 = 0; b0 < batch; b0 += fit) {
+            const int b = batch - b0 < fit ? batch - b0 : fit;
+            const int rc = lk_mmvq_pair_act(wtype, gate, up, (const uint8_t*)vy_q8_1 + (size_t)b0 * stride_col_y * Q81_BYTES,
+                                            (uint8_t*)dst + (size_t)b0 * stride_col_dst * (dst_type == LK_TYPE_F32 ? 4 : 2),
+                                            dst_type, ncols_x, nrows_x, b, stride_col_y, stride_col_dst, act, stream);
+            if (rc != LK_OK) return rc;
+        }
+        return LK_OK;
+    }
     hipStream_t s = (hipStream_t)stream;
     const uint8_t *g = (const uint8_t*)gate, *u = (const uint8_t*)up, *y = (const uint8_t*)vy_q8_1;
 #define LK_PAIR(E, T)                                                                                          \

@@ -68,10 +68,56 @@ static __device__ __forceinline__ void q6k_dots(const uint4& ql, const uint4& qh
     d_b = dot16(cb, a_b, 0);
 }
 
+// Q6_K with the codes left unsigned (0..63): 16 bytes of each half-row of ql (`ql0` = l, `ql1` =
+// l + 32) and the 16 bytes of qh over the same l give 16 codes of each of the half's four
+// 32-value groups. The caller starts each accumulator at -32 * (sum of that run's activation
+// codes), which yields the integer the signed form gives.
+static __device__ __forceinline__ void q6k_dots_biased(const uint4& ql0, const uint4& ql1, const uint4& qh,
+                                                       const uint4 (&a)[4], int (&dot)[4]) {
+    uint4 c[4];
+#define LK_Q6K_RAW(f)                                                       \
+    c[0].f = (ql0.f & 0x0F0F0F0Fu) | ((qh.f << 4) & 0x30303030u);             \
+    c[1].f = (ql1.f & 0x0F0F0F0Fu) | ((qh.f << 2) & 0x30303030u);             \
+    c[2].f = ((ql0.f >> 4) & 0x0F0F0F0Fu) | (qh.f & 0x30303030u);             \
+    c[3].f = ((ql1.f >> 4) & 0x0F0F0F0Fu) | ((qh.f >> 2) & 0x30303030u);
+    LK_Q6K_RAW(x) LK_Q6K_RAW(y) LK_Q6K_RAW(z) LK_Q6K_RAW(w)
+#undef LK_Q6K_RAW
+#pragma unroll
+    for (int g = 0; g < 4; ++g) dot[g] = dot16(c[g], a[g], dot[g]);
+}
+
+// Dword-aligned read of 16 bytes that start on any even address. A 2-byte-aligned dwordx4 load
+// runs at about three quarters of the rate of a dword-aligned one on this part, so the load is
+// made from the enclosing dwords and shifted into place. The fifth dword is the one that holds
+// the run's last two bytes (the run's own last dword when the address is already aligned), so
+// nothing outside dwords the run touches is read.
+struct Run16 {
+    uint4 w;
+    uint32_t e;
+};
+static __device__ __forceinline__ Run16 load_run16(const uint8_t* p) {
+    const uintptr_t a = (uintptr_t)p;
+    const uint8_t* b = (const uint8_t*)(a & ~(uintptr_t)3);
+    Run16 r;
+    r.w = *(const uint4_a4*)b;
+    r.e = *(const uint32_t*)(b + 12 + 2 * (a & 2));
+    return r;
+}
+static __device__ __forceinline__ uint4 run16_value(const Run16& r, uint32_t shift_bits) {
+    uint4 v;
+    v.x = __builtin_amdgcn_alignbit(r.w.y, r.w.x, shift_bits);
+    v.y = __builtin_amdgcn_alignbit(r.w.z, r.w.y, shift_bits);
+    v.z = __builtin_amdgcn_alignbit(r.w.w, r.w.z, shift_bits);
+    v.w = __builtin_amdgcn_alignbit(r.e, r.w.w, shift_bits);
+    return v;
+}
+
 // --------------------------------------------------------------------------------------------
 // Activation staging. Formats differ only in where a Q8_1 block's two 16-byte halves land.
 // LDS per activation row: `n_iter` passes x `PLANES` planes x 1024 bytes of codes, then the
-// scale table (SCF floats per Q8_1 block).
+// scale table, SCF dwords per Q8_1 block: d; with SCF 2 also d * (sum of the block's codes),
+// interleaved; with SCF 3 three arrays one after the other: d, then -32 * (sum of codes) of every
+// block's first 16 values, then of its last 16, as integers.
 // --------------------------------------------------------------------------------------------
 
 struct FmtQ4K {
@@ -87,11 +133,12 @@ struct FmtQ4K {
 };
 struct FmtQ6K {
     static constexpr int BLOCK_BYTES = Q6K_BYTES, BLOCK_LEN = 256;
-    static constexpr int VPI = 2048;
-    static constexpr int PLANES = 2, SCF = 1;
+    static constexpr int VPI = 4096;   // 16 super-blocks per wave pass, 4 lanes each
+    static constexpr int PLANES = 4, SCF = 3;
+    // Lane (block lb, half h, 16-run lh) reads plane g (the 32-value group inside the half) at lane * 16.
     static __device__ __forceinline__ int slot(int j, int lh) {
         const int lb = j >> 3, s = j & 7, h = s >> 2, g = s & 3;
-        return (g >> 1) * 1024 + (lb * 8 + h * 4 + (g & 1) * 2 + lh) * 16;
+        return g * 1024 + (lb * 4 + h * 2 + lh) * 16;
     }
 };
 struct FmtQ80 {
@@ -137,6 +184,11 @@ static __device__ __forceinline__ void stage_activation(uint8_t* lds, const uint
             *(uint4*)(codes + F::slot(ji, 1)) = hi;
             if (F::SCF == 2) {
                 *(float2*)(sc + 2 * j) = make_float2(d8, ds);
+            } else if (F::SCF == 3) {
+                const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
+                sc[j] = d8;
+                ((int*)sc)[total + j] = -32 * dot16(ones, lo, 0);
+                ((int*)sc)[2 * total + j] = -32 * dot16(ones, hi, 0);
             } else {
                 sc[j] = d8;
             }
@@ -184,6 +236,7 @@ static __device__ __forceinline__ void stage_activation_f32(uint8_t* lds, const 
                 int sum = q0 + q1 + q2 + q3;
                 sum += __shfl_xor(sum, 1);
                 sum += __shfl_xor(sum, 2);
+                const int half_sum = sum;   // lanes 0-3: the block's first 16 values, 4-7: the rest
                 sum += __shfl_xor(sum, 4);
                 uint8_t* row = lds + c * row_bytes;
                 uint8_t* codes = row + it * F::PLANES * 1024;
@@ -195,10 +248,14 @@ static __device__ __forceinline__ void stage_activation_f32(uint8_t* lds, const 
                     const float d8 = __half2float(__float2half_rn(d));
                     if (F::SCF == 2) {
                         *(float2*)(sc + 2 * j) = make_float2(d8, d8 * (float)sum);
+                    } else if (F::SCF == 3) {
+                        sc[j] = d8;
+                        ((int*)sc)[total + j] = -32 * half_sum;
                     } else {
                         sc[j] = d8;
                     }
                 }
+                if (F::SCF == 3 && l8 == 4) ((int*)(row + n_iter * F::VPI))[2 * total + j] = -32 * half_sum;
             }
         }
     }
@@ -350,79 +407,133 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Q6_K: 8 lanes per super-block (16 bytes of ql + the matching 16 of qh = two runs of 16 codes).
+// The step loop the Q6_K and Q8_0 engines share. Steps are (row tile, pass) pairs in order; the
+// loads of step i+1 are issued before step i is consumed, ping-ponging between two register
+// fragments, and the very first loads go out before the activation is staged so that the two
+// memory latencies overlap.
+// ---------------------------------------------------------------------------------------------
+template <class Frag, class Stage, class Load, class Compute>
+static __device__ __forceinline__ void step_loop(int tile, int tile_stride, int n_tiles, int n_iter, Stage&& stage,
+                                                 Load&& load, Compute&& compute) {
+    int it = 0;
+    Frag fa, fb;
+    if (tile < n_tiles) load(fa, tile, 0);
+    stage();
+    __syncthreads();
+    if (tile >= n_tiles) return;
+    for (;;) {
+        int nt = tile, ni = it + 1;
+        if (ni == n_iter) { ni = 0; nt += tile_stride; }
+        if (nt < n_tiles) load(fb, nt, ni);
+        compute(fa, tile, it);
+        tile = nt; it = ni;
+        if (tile >= n_tiles) break;
+        nt = tile; ni = it + 1;
+        if (ni == n_iter) { ni = 0; nt += tile_stride; }
+        if (nt < n_tiles) load(fa, nt, ni);
+        compute(fb, tile, it);
+        tile = nt; it = ni;
+        if (tile >= n_tiles) break;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Q6_K: 4 lanes per super-block, 16 super-blocks per wave pass. Lane (half h, run lh) takes the
+// 16 bytes of both ql half-rows and the 16 bytes of qh at l = 16 * lh, which is 16 codes of each
+// of the half's four groups and reads no byte of ql / qh twice across the wave (the load unit's
+// cycles, not HBM, bound this format). The codes stay unsigned; the -32 offset comes in through
+// the staged per-run activation sums.
 // ---------------------------------------------------------------------------------------------
 template <int B, int R, int NW, class Epi>
 static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* lds, Epi&& epi) {
     const int nb = job.nb, n = job.n;
-    const int n_iter = (nb + 7) >> 3;
+    const int n_iter = (nb + 15) >> 4;
     const int row_bytes = lds_bytes_per_row<FmtQ6K>(n_iter);
-    stage_job<FmtQ6K, B>(lds, job, nb * 8, n_iter);
-    __syncthreads();
+    const int total = n_iter * 128;   // Q8_1 blocks the staged row is padded to
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lb = lane >> 3, ch = lane & 7;
-    const int h = ch >> 2, g0 = (ch >> 1) & 1, lh = ch & 1;
+    const int lb = lane >> 2, h = (lane >> 1) & 1, lh = lane & 1;
+    const uint32_t ql_off = 64 * h + 16 * lh, qh_off = 128 + 32 * h + 16 * lh, sc_off = 192 + 8 * h;
     const size_t row_stride = (size_t)nb * Q6K_BYTES;
     const int n_tiles = (n + R - 1) / R;
     constexpr int RW = R * NW;
 
-    for (int tile = job.tile_first + wave; tile < n_tiles; tile += job.tile_stride) {
-        const int row0 = tile * R;
-        float acc[RW][B];
+    struct Frag {
+        uint4 ql0[RW], ql1[RW], qh[RW];
+        uint2 sc[RW];     // the half's 8 scale bytes
+        uint32_t d[RW];   // f16 bits, zero for a lane past the row end
+    };
+    auto load = [&](Frag& f, int tile, int it) {
+        const int blk = it * 16 + lb;
+        const bool valid = blk < nb;
+        const int blk_c = valid ? blk : nb - 1;
 #pragma unroll
-        for (int r = 0; r < RW; ++r)
+        for (int w = 0; w < NW; ++w)
 #pragma unroll
-            for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
-
-        for (int it = 0; it < n_iter; ++it) {
-            const int blk = it * 8 + lb;
-            const bool valid = blk < nb;
-            const int blk_c = valid ? blk : nb - 1;
-            uint4 ql[RW], qh[RW];
-            float dsa[RW], dsb[RW];
-#pragma unroll
-            for (int w = 0; w < NW; ++w)
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const int row = min(row0 + r, n - 1);
-                    const uint8_t* bp = job.vx[w] + row * row_stride + (size_t)blk_c * Q6K_BYTES;
-                    ql[w * R + r] = *(const uint4_a2*)(bp + 16 * ch);
-                    qh[w * R + r] = *(const uint4_a2*)(bp + 128 + 16 * (2 * h + lh));
-                    const int sa = ((const int8_t*)bp)[192 + 8 * h + 2 * g0 + lh];
-                    const int sb = ((const int8_t*)bp)[192 + 8 * h + 2 * g0 + 4 + lh];
-                    const float d = valid ? f16_bits_to_f32(*(const uint16_t*)(bp + 208)) : 0.f;
-                    dsa[w * R + r] = d * (float)sa;
-                    dsb[w * R + r] = d * (float)sb;
-                }
-#pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const uint8_t* rowl = lds + c * row_bytes;
-                const uint8_t* codes = rowl + it * 2048;
-                const uint4 a_a = *(const uint4*)(codes + lane * 16);
-                const uint4 a_b = *(const uint4*)(codes + 1024 + lane * 16);
-                const float* sc = (const float*)(rowl + n_iter * 2048);
-                const float d8a = sc[blk * 8 + 4 * h + g0];
-                const float d8b = sc[blk * 8 + 4 * h + g0 + 2];
-#pragma unroll
-                for (int r = 0; r < RW; ++r) {
-                    int d_a, d_b;
-                    q6k_dots(ql[r], qh[r], g0, a_a, a_b, d_a, d_b);
-                    acc[r][c] += dsa[r] * (d8a * (float)d_a) + dsb[r] * (d8b * (float)d_b);
-                }
+            for (int r = 0; r < R; ++r) {
+                const int row = min(tile * R + r, n - 1);
+                const uint8_t* bp = job.vx[w] + row * row_stride + (size_t)blk_c * Q6K_BYTES;
+                f.ql0[w * R + r] = *(const uint4_a2*)(bp + ql_off);
+                f.ql1[w * R + r] = *(const uint4_a2*)(bp + ql_off + 32);
+                f.qh[w * R + r] = *(const uint4_a2*)(bp + qh_off);
+                f.sc[w * R + r] = *(const uint2_a2*)(bp + sc_off);
+                f.d[w * R + r] = valid ? (uint32_t) * (const uint16_t*)(bp + 208) : 0u;
             }
+    };
+
+    float acc[RW][B];
+#pragma unroll
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+        for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
+
+    auto compute = [&](const Frag& f, int tile, int it) {
+        float ds[RW][4];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            const float d = f16_bits_to_f32(f.d[r]);
+            ds[r][0] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].x, 8 * lh, 8);
+            ds[r][1] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].x, 8 * lh + 16, 8);
+            ds[r][2] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].y, 8 * lh, 8);
+            ds[r][3] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].y, 8 * lh + 16, 8);
         }
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+        for (int c = 0; c < B; ++c) {
+            const uint8_t* rowl = lds + c * row_bytes;
+            const uint8_t* codes = rowl + it * 4096 + lane * 16;
+            uint4 a[4];
 #pragma unroll
-            for (int c = 0; c < B; ++c) {
-                float tot[NW];
+            for (int g = 0; g < 4; ++g) a[g] = *(const uint4*)(codes + g * 1024);
+            const uint8_t* sc = rowl + n_iter * 4096;
+            const int j0 = (it * 16 + lb) * 8 + 4 * h;   // the half's four Q8_1 blocks
+            const float4 d8 = *(const float4*)(sc + 4 * j0);
+            const int4 bias = *(const int4*)(sc + 4 * (total * (1 + lh) + j0));
 #pragma unroll
-                for (int w = 0; w < NW; ++w) tot[w] = wave_sum(acc[w * R + r][c]);
-                if (lane == 0 && row0 + r < n) epi(row0 + r, c, tot);
+            for (int r = 0; r < RW; ++r) {
+                int dot[4] = {bias.x, bias.y, bias.z, bias.w};
+                q6k_dots_biased(f.ql0[r], f.ql1[r], f.qh[r], a, dot);
+                acc[r][c] += ds[r][0] * (d8.x * (float)dot[0]) + ds[r][2] * (d8.z * (float)dot[2]);
+                acc[r][c] += ds[r][1] * (d8.y * (float)dot[1]) + ds[r][3] * (d8.w * (float)dot[3]);
             }
-    }
+        }
+        if (it == n_iter - 1) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int c = 0; c < B; ++c) {
+                    float tot[NW];
+#pragma unroll
+                    for (int w = 0; w < NW; ++w) {
+                        tot[w] = wave_sum(acc[w * R + r][c]);
+                        acc[w * R + r][c] = 0.f;
+                    }
+                    if (lane == 0 && tile * R + r < n) epi(tile * R + r, c, tot);
+                }
+        }
+    };
+    step_loop<Frag>(job.tile_first + wave, job.tile_stride, n_tiles, n_iter,
+                    [&] { stage_job<FmtQ6K, B>(lds, job, nb * 8, n_iter); }, load, compute);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -433,8 +544,6 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
     const int nb = job.nb, n = job.n;
     const int n_iter = (nb + 31) >> 5;
     const int row_bytes = lds_bytes_per_row<FmtQ80>(n_iter);
-    stage_job<FmtQ80, B>(lds, job, nb, n_iter);
-    __syncthreads();
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -443,49 +552,69 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
     const int n_tiles = (n + R - 1) / R;
     constexpr int RW = R * NW;
 
-    for (int tile = job.tile_first + wave; tile < n_tiles; tile += job.tile_stride) {
-        const int row0 = tile * R;
-        float acc[RW][B];
+    struct Frag {
+        Run16 q[RW];
+        uint32_t d[RW];       // f16 bits, zero for a lane past the row end
+        uint32_t shift[RW];   // bits to shift q by
+    };
+    auto load = [&](Frag& f, int tile, int it) {
+        const int blk = it * 32 + lb;
+        const bool valid = blk < nb;
+        const int blk_c = valid ? blk : nb - 1;
 #pragma unroll
-        for (int r = 0; r < RW; ++r)
+        for (int w = 0; w < NW; ++w)
 #pragma unroll
-            for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
-
-        for (int it = 0; it < n_iter; ++it) {
-            const int blk = it * 32 + lb;
-            const bool valid = blk < nb;
-            const int blk_c = valid ? blk : nb - 1;
-            uint4 q[RW];
-            float d[RW];
-#pragma unroll
-            for (int w = 0; w < NW; ++w)
-#pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const int row = min(row0 + r, n - 1);
-                    const uint8_t* bp = job.vx[w] + row * row_stride + (size_t)blk_c * Q80_BYTES;
-                    q[w * R + r] = *(const uint4_a2*)(bp + 2 + 16 * lh);
-                    d[w * R + r] = valid ? f16_bits_to_f32(*(const uint16_t*)bp) : 0.f;
-                }
-#pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const uint8_t* rowl = lds + c * row_bytes;
-                const uint4 a = *(const uint4*)(rowl + it * 1024 + lane * 16);
-                const float d8 = ((const float*)(rowl + n_iter * 1024))[blk];
-#pragma unroll
-                for (int r = 0; r < RW; ++r) acc[r][c] += (d[r] * d8) * (float)dot16(q[r], a, 0);
+            for (int r = 0; r < R; ++r) {
+                const int row = min(tile * R + r, n - 1);
+                const uint8_t* bp = job.vx[w] + row * row_stride + (size_t)blk_c * Q80_BYTES;
+                f.q[w * R + r] = load_run16(bp + 2 + 16 * lh);
+                f.shift[w * R + r] = ((uint32_t)(uintptr_t)(bp + 2) & 2u) * 8u;
+                f.d[w * R + r] = valid ? (uint32_t) * (const uint16_t*)bp : 0u;
             }
+    };
+
+    float acc[RW][B];
+#pragma unroll
+    for (int r = 0; r < RW; ++r)
+#pragma unroll
+        for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
+
+    auto compute = [&](const Frag& f, int tile, int it) {
+        const int blk = it * 32 + lb;
+        uint4 q[RW];
+        float d[RW];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            q[r] = run16_value(f.q[r], f.shift[r]);
+            d[r] = f16_bits_to_f32(f.d[r]);
         }
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+        for (int c = 0; c < B; ++c) {
+            const uint8_t* rowl = lds + c * row_bytes;
+            const uint4 a = *(const uint4*)(rowl + it * 1024 + lane * 16);
+            const float d8 = ((const float*)(rowl + n_iter * 1024))[blk];
 #pragma unroll
-            for (int c = 0; c < B; ++c) {
-                float tot[NW];
+            for (int r = 0; r < RW; ++r) acc[r][c] += (d[r] * d8) * (float)dot16(q[r], a, 0);
+        }
+        if (it == n_iter - 1) {
 #pragma unroll
-                for (int w = 0; w < NW; ++w) tot[w] = wave_sum(acc[w * R + r][c]);
-                if (lane == 0 && row0 + r < n) epi(row0 + r, c, tot);
-            }
-    }
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int c = 0; c < B; ++c) {
+                    float tot[NW];
+#pragma unroll
+                    for (int w = 0; w < NW; ++w) {
+                        tot[w] = wave_sum(acc[w * R + r][c]);
+                        acc[w * R + r][c] = 0.f;
+                    }
+                    if (lane == 0 && tile * R + r < n) epi(tile * R + r, c, tot);
+                }
+        }
+    };
+    step_loop<Frag>(job.tile_first + wave, job.tile_stride, n_tiles, n_iter,
+                    [&] { stage_job<FmtQ80, B>(lds, job, nb, n_iter); }, load, compute);
 }
+
 
 // Format tags: which engine serves a ggml type, and its LDS footprint.
 struct EngQ4K {
@@ -512,6 +641,14 @@ static inline int n_iter_of(int nb) {
 template <class F>
 static inline int lds_bytes_for(int nb, int batch) {
     return batch * lds_bytes_per_row<F>(n_iter_of<F>(nb));
+}
+
+static inline int lds_bytes_of(int wtype, int nb, int batch) {
+    switch (wtype) {
+        case LK_TYPE_Q4_K: return lds_bytes_for<FmtQ4K>(nb, batch);
+        case LK_TYPE_Q6_K: return lds_bytes_for<FmtQ6K>(nb, batch);
+        default: return lds_bytes_for<FmtQ80>(nb, batch);
+    }
 }
 
 static inline int block_len_of(int wtype) {
