@@ -4,10 +4,12 @@
 One *step* = every quantized linear of one Llama-3-8B-shaped decode step at batch `--batch`
 (default 1): per layer q, o 4096->4096, k, v 4096->1024, gate, up 4096->14336 in Q4_K and down
 14336->4096 in Q6_K, 32 layers, then lm_head 4096->128256 in Q8_0: 225 weight matrices,
-4.97 GB of blocks. Default launch plan (`--plan fused`): the linears that share an activation go
-out as one launch (q,k,v; gate,up) and every launch quantizes its f32 activation to Q8_1 in LDS
-itself, 4 launches per layer; `--plan split` is the two-launch form per linear (Q8_1 quantizer,
-then mat-vec). Distinct weights per layer, so the step is cache-cold by construction.
+4.97 GB of blocks. Launch plans: `--plan fused`: the linears that share an activation go out as
+one launch (q,k,v; gate,up) and every launch quantizes its f32 activation to Q8_1 in LDS itself,
+4 launches per layer; `--plan split`: the two-launch form per linear (Q8_1 quantizer, then
+mat-vec); `--plan auto` (default): fused, except that `down`, whose 14336-value rows are dear to
+quantize once per workgroup, keeps its own quantizer launch (5 launches per layer).
+Distinct weights per layer, so the step is cache-cold by construction.
 Weights and activations are synthetic (seeded, generated on the device) and resident in HBM
 before the timed region.
 
@@ -44,8 +46,10 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=1, help="activation rows per mat-vec (1..8)")
     ap.add_argument("--layers", type=int, default=LAYERS)
-    ap.add_argument("--plan", choices=["fused", "split"], default="fused",
-                    help="fused: shared-activation linears per launch, Q8_1 quantized in-kernel; split: quantize + mat-vec per linear")
+    ap.add_argument("--plan", choices=["auto", "fused", "split"], default="auto",
+                    help="fused: shared-activation linears per launch, Q8_1 quantized in-kernel; split: quantize + "
+                         "mat-vec per linear; auto: fused, except that rows longer than 8192 values are quantized "
+                         "by their own launch (every workgroup of a fused launch quantizes the whole row)")
     ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -163,11 +167,16 @@ def main() -> int:
     first_out = None
     first_w = None
     for layer in range(args.layers):
-        if args.plan == "fused":
+        if args.plan in ("fused", "auto"):
             made = {name: (maker(n, k), wtype, n, k, g) for name, wtype, n, k, maker, g in shapes}
             keep.extend(v[0] for v in made.values())
             for group in (("q", "k", "v"), ("o",), ("gate", "up"), ("down",)):
                 wtype, k, g = made[group[0]][1], made[group[0]][3], made[group[0]][4]
+                if args.plan == "auto" and k > 8192:
+                    add_quant(g)
+                    for nm in group:
+                        add_gemv(wtype, made[nm][0], g, made[nm][2], k)
+                    continue
                 out = add_fused(wtype, [made[nm][0] for nm in group], g, [made[nm][2] for nm in group], k)
                 if first_out is None:
                     first_out, first_w = out, made["q"][0]
@@ -184,7 +193,7 @@ def main() -> int:
                 first_out, first_w = out, w
     lm_head = make_q80(VOCAB, HIDDEN)
     keep.append(lm_head)
-    if args.plan == "fused":
+    if args.plan in ("fused", "auto"):
         add_fused(Q80, [lm_head], "final", [VOCAB], HIDDEN)
     else:
         add_quant("final")
