@@ -29,6 +29,13 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
+// A byte address typed as global memory. Weight addresses travel in this type: one rebuilt from
+// integers, read from a table or passed through an opaque statement is otherwise a generic
+// pointer and is read with flat loads, which also count against the LDS wait counter.
+typedef const __attribute__((address_space(1))) uint8_t* gbytes_t;
+static __device__ __forceinline__ gbytes_t to_gbytes(const void* p) { return (gbytes_t)p; }
+static __device__ __forceinline__ gbytes_t to_gbytes(uint64_t bits) { return (gbytes_t)bits; }
+
 static __device__ __forceinline__ int dot4(int a, int b, int c) {
     return __builtin_amdgcn_sdot4(a, b, c, false);
 }

@@ -42,15 +42,47 @@ template <class E, int B, int R, typename T>
 __global__ __launch_bounds__(WG) void mmvq_kernel(MultiArgs m, const uint8_t* __restrict__ vy, int nb,
                                                   int stride_col_y, int stride_col_dst, int act_stride_f32) {
     extern __shared__ __align__(16) uint8_t lds[];
+    // Which matrix this workgroup serves. Every field is read at a fixed index and picked with a
+    // mask, so the kernel arguments the first loads need arrive in one round of scalar loads
+    // (indexing the arrays by a computed `w`, or reading them under a branch, costs further
+    // dependent rounds before the first weight load can go out).
+    static_assert(MAX_MULTI == 4, "the pin below lists four matrices");
+    uintptr_t vxs[MAX_MULTI];
+    int ns[MAX_MULTI], begins[MAX_MULTI + 1], count = m.count;
+#pragma unroll
+    for (int i = 0; i < MAX_MULTI; ++i) {
+        vxs[i] = (uintptr_t)m.vx[i];
+        ns[i] = m.n[i];
+        begins[i] = m.wg_begin[i];
+    }
+    begins[MAX_MULTI] = m.wg_begin[MAX_MULTI];
+    // Pinned together: left alone, the compiler reads m.vx only after it has waited for the
+    // other fields, which puts a second scalar round trip in front of the first weight load.
+    asm volatile("" : "+s"(vxs[0]), "+s"(vxs[1]), "+s"(vxs[2]), "+s"(vxs[3]), "+s"(ns[0]), "+s"(ns[1]), "+s"(ns[2]),
+                 "+s"(ns[3]), "+s"(begins[1]), "+s"(begins[2]), "+s"(begins[3]), "+s"(begins[4]), "+s"(count));
     int w = 0;
 #pragma unroll
     for (int i = 1; i < MAX_MULTI; ++i)
-        if (i < m.count && (int)blockIdx.x >= m.wg_begin[i]) w = i;
-    const int wgs = m.wg_begin[w + 1] - m.wg_begin[w];
-    RowJob<1> job{{m.vx[w]}, vy, nb, m.n[w], stride_col_y, wgs * WAVES, ((int)blockIdx.x - m.wg_begin[w]) * WAVES,
+        if (i < count && (int)blockIdx.x >= begins[i]) w = i;
+    uintptr_t vx_bits = 0, dst_bits = 0, bias_bits = 0;
+    uint32_t n_bits = 0, first_bits = 0, end_bits = 0;
+#pragma unroll
+    for (int i = 0; i < MAX_MULTI; ++i) {
+        const uint32_t pick = 0u - (uint32_t)(w == i);
+        const uintptr_t pick64 = (uintptr_t)(int64_t)(int32_t)pick;
+        vx_bits |= vxs[i] & pick64;
+        dst_bits |= (uintptr_t)m.dst[i] & pick64;
+        bias_bits |= (uintptr_t)m.bias[i] & pick64;
+        n_bits |= (uint32_t)ns[i] & pick;
+        first_bits |= (uint32_t)(i ? begins[i] : 0) & pick;
+        end_bits |= (uint32_t)begins[i + 1] & pick;
+    }
+    const gbytes_t vx = to_gbytes((uint64_t)vx_bits);
+    T* dst = (T*)(uint8_t*)to_gbytes((uint64_t)dst_bits);
+    const float* bias = (const float*)to_gbytes((uint64_t)bias_bits);
+    const int n = (int)n_bits, wg_first = (int)first_bits, wg_end = (int)end_bits;
+    RowJob<1> job{{vx}, vy, nb, n, stride_col_y, (wg_end - wg_first) * WAVES, ((int)blockIdx.x - wg_first) * WAVES,
                   act_stride_f32};
-    T* dst = (T*)m.dst[w];
-    const float* bias = m.bias[w];
     E::template run<B, R, 1>(job, lds, [&](int row, int c, const float* tot) {
         float v = tot[0];
         if (bias) v += bias[row];
@@ -71,7 +103,7 @@ __global__ __launch_bounds__(WG) void mmvq_pair_kernel(const uint8_t* __restrict
                                                        const uint8_t* __restrict__ vy, T* __restrict__ dst, int nb,
                                                        int n, int stride_col_y, int stride_col_dst) {
     extern __shared__ __align__(16) uint8_t lds[];
-    RowJob<2> job{{gate, up}, vy, nb, n, stride_col_y, (int)gridDim.x * WAVES, (int)blockIdx.x * WAVES};
+    RowJob<2> job{{to_gbytes(gate), to_gbytes(up)}, vy, nb, n, stride_col_y, (int)gridDim.x * WAVES, (int)blockIdx.x * WAVES};
     E::template run<B, R, 2>(job, lds, [&](int row, int c, const float* tot) {
         const float a = ACT == 0 ? act_silu(tot[0]) : act_gelu_tanh(tot[0]);
         dst[(size_t)c * stride_col_dst + row] = from_f32<T>(a * tot[1]);
@@ -87,7 +119,7 @@ __global__ __launch_bounds__(WG) void mmvq_grouped_kernel(const uint64_t* __rest
                                                           int nb, int n, int k32) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int g = blockIdx.y;
-    RowJob<1> job{{(const uint8_t*)table[g]}, vy + (size_t)g * k32 * Q81_BYTES, nb, n, k32,
+    RowJob<1> job{{to_gbytes(table[g])}, vy + (size_t)g * k32 * Q81_BYTES, nb, n, k32,
                   (int)gridDim.x * WAVES, (int)blockIdx.x * WAVES};
     float* out = dst + (size_t)g * n;
     E::template run<1, R, 1>(job, lds, [&](int row, int, const float* tot) { out[row] = tot[0]; });

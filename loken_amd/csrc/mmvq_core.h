@@ -153,110 +153,187 @@ static __host__ __device__ constexpr int lds_bytes_per_row(int n_iter) {
     return n_iter * F::VPI + n_iter * (F::VPI / 32) * F::SCF * 4;
 }
 
+// Staging runs in two halves so that an engine can put its first weight loads between them:
+// `stage_issue` sends the loads of the first round of activation data (per thread: one Q8_1 block,
+// or 16 floats) and `stage_finish` turns them into the LDS image and walks the later rounds.
+// Loads return in issue order, so the activation (small, usually in L2) must be asked for BEFORE
+// the weights (HBM) or the staging would wait for the weights as well. Only launches of up to
+// two activation rows hoist the first round; wider ones would hold too many registers.
+template <int B>
+struct ActRegs {
+    static constexpr int ROWS = B <= 2 ? B : 0;
+    uint32_t head[ROWS ? ROWS : 1];   // a Q8_1 block: d and s, then the two halves of its codes
+    uint4 lo[ROWS ? ROWS : 1], hi[ROWS ? ROWS : 1];
+    float4 x[ROWS ? ROWS : 1][4];
+};
+
+// One Q8_1 block (j-th of its row; `real` false past the row's end) into the LDS image of `row`.
+template <class F>
+static __device__ __forceinline__ void put_q8_1_block(uint8_t* row, int n_iter, int j, bool real, uint32_t head,
+                                                      uint4 lo, uint4 hi) {
+    const int per_pass = F::VPI / 32, total = n_iter * per_pass;
+    const int it = j / per_pass, ji = j % per_pass;
+    float* sc = (float*)(row + n_iter * F::VPI);
+    const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
+    if (!real) {
+        lo = hi = make_uint4(0, 0, 0, 0);
+        head = 0;
+    }
+    const float d8 = f16_bits_to_f32(head & 0xFFFFu);
+    uint8_t* codes = row + it * F::PLANES * 1024;
+    *(uint4*)(codes + F::slot(ji, 0)) = lo;
+    *(uint4*)(codes + F::slot(ji, 1)) = hi;
+    if (F::SCF == 2) {
+        *(float2*)(sc + 2 * j) = make_float2(d8, d8 * (float)dot16(ones, hi, dot16(ones, lo, 0)));
+    } else if (F::SCF == 3) {
+        sc[j] = d8;
+        ((int*)sc)[total + j] = -32 * dot16(ones, lo, 0);
+        ((int*)sc)[2 * total + j] = -32 * dot16(ones, hi, 0);
+    } else {
+        sc[j] = d8;
+    }
+}
+
+// A Q8_1 block as three loads that land where they are used (36-byte blocks are dword aligned).
+static __device__ __forceinline__ void load_q8_1_block(const uint8_t* __restrict__ p, uint32_t& head, uint4& lo,
+                                                       uint4& hi) {
+    // The two offsets pass through an opaque statement: seen as p + 4 and p + 20 the compiler
+    // fuses the loads into 16 + 16 + 4 bytes from p and then has to wait for them on the spot to
+    // shuffle the registers back into `lo` and `hi`.
+    int off_lo = 4, off_hi = 20;
+    asm("" : "+v"(off_lo));
+    asm("" : "+v"(off_hi));
+    head = *(const uint32_t*)p;
+    lo = *(const uint4_a4*)(p + off_lo);
+    hi = *(const uint4_a4*)(p + off_hi);
+}
+
+// Every thread loads (a thread past the row's end re-reads its last block and drops it later):
+// a load under a branch would make the wave wait for it where the branch ends.
+template <class F, int B>
+static __device__ __forceinline__ void stage_issue_q8_1(ActRegs<B>& ar, const uint8_t* __restrict__ vy, int k32,
+                                                        int stride_col_y) {
+    const int j = min((int)threadIdx.x, k32 - 1);
+#pragma unroll
+    for (int c = 0; c < ActRegs<B>::ROWS; ++c)
+        load_q8_1_block(vy + ((size_t)c * stride_col_y + j) * Q81_BYTES, ar.head[c], ar.lo[c], ar.hi[c]);
+}
+
 // Stage `batch` Q8_1 rows. k32 = real Q8_1 blocks per row; the rest of the last pass is zeroed.
 template <class F, int B>
-static __device__ __forceinline__ void stage_activation(uint8_t* lds, const uint8_t* __restrict__ vy,
-                                                        int k32, int n_iter, int stride_col_y) {
-    const int per_pass = F::VPI / 32;
-    const int total = n_iter * per_pass;
+static __device__ __forceinline__ void stage_finish_q8_1(const ActRegs<B>& ar, uint8_t* lds,
+                                                         const uint8_t* __restrict__ vy, int k32, int n_iter,
+                                                         int stride_col_y) {
+    const int total = n_iter * (F::VPI / 32);
     const int row_bytes = lds_bytes_per_row<F>(n_iter);
-    for (int j = threadIdx.x; j < total; j += WG) {
-        const int it = j / per_pass, ji = j % per_pass;
+    int j = threadIdx.x;
+    if (ActRegs<B>::ROWS) {
+        if (j < total) {
+#pragma unroll
+            for (int c = 0; c < ActRegs<B>::ROWS; ++c)
+                put_q8_1_block<F>(lds + c * row_bytes, n_iter, j, j < k32, ar.head[c], ar.lo[c], ar.hi[c]);
+        }
+        j += WG;
+    }
+    for (; j < total; j += WG) {
 #pragma unroll
         for (int c = 0; c < B; ++c) {
-            uint8_t* row = lds + c * row_bytes;
-            float* sc = (float*)(row + n_iter * F::VPI);
-            uint4 lo = make_uint4(0, 0, 0, 0), hi = make_uint4(0, 0, 0, 0);
-            float d8 = 0.f, ds = 0.f;
-            if (j < k32) {
-                const uint32_t* src = (const uint32_t*)(vy + ((size_t)c * stride_col_y + j) * Q81_BYTES);
-                const uint32_t head = src[0];
-                lo = make_uint4(src[1], src[2], src[3], src[4]);
-                hi = make_uint4(src[5], src[6], src[7], src[8]);
-                d8 = f16_bits_to_f32(head & 0xFFFFu);
-                if (F::SCF == 2) {
-                    const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
-                    ds = d8 * (float)dot16(ones, hi, dot16(ones, lo, 0));
-                }
-            }
-            uint8_t* codes = row + it * F::PLANES * 1024;
-            *(uint4*)(codes + F::slot(ji, 0)) = lo;
-            *(uint4*)(codes + F::slot(ji, 1)) = hi;
-            if (F::SCF == 2) {
-                *(float2*)(sc + 2 * j) = make_float2(d8, ds);
-            } else if (F::SCF == 3) {
-                const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
-                sc[j] = d8;
-                ((int*)sc)[total + j] = -32 * dot16(ones, lo, 0);
-                ((int*)sc)[2 * total + j] = -32 * dot16(ones, hi, 0);
-            } else {
-                sc[j] = d8;
-            }
+            uint32_t head;
+            uint4 lo, hi;
+            load_q8_1_block(vy + ((size_t)c * stride_col_y + min(j, k32 - 1)) * Q81_BYTES, head, lo, hi);
+            put_q8_1_block<F>(lds + c * row_bytes, n_iter, j, j < k32, head, lo, hi);
         }
     }
 }
 
-
 // The same staging from f32 rows: the workgroup quantizes each 32-value block itself, with the
 // steps of the stand-alone quantizer (d = amax/127 rounded to f16, codes = round_half_away(x *
 // (1/d)) with d before its rounding, integer code sum), so the staged bytes are the ones the
-// two-launch path stages. Eight lanes own a block, four values each.
-template <class F, int B>
-static __device__ __forceinline__ void stage_activation_f32(uint8_t* lds, const float* __restrict__ x, int k32,
-                                                            int n_iter, int x_stride) {
+// two-launch path stages. Eight lanes own a block, four values each; item t is lane t & 7 of
+// block t >> 3. All eight lanes of a block call this together.
+template <class F>
+static __device__ __forceinline__ void put_f32_quad(uint8_t* row, int n_iter, int k32, int t, float4 v) {
 #pragma clang fp contract(off)
-    const int per_pass = F::VPI / 32;
-    const int total = n_iter * per_pass;
+    const int per_pass = F::VPI / 32, total = n_iter * per_pass;
+    const int j = t >> 3, l8 = t & 7;
+    if (j >= k32) v = make_float4(0.f, 0.f, 0.f, 0.f);   // padding of the last pass
+    const int it = j / per_pass, ji = j % per_pass;
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1));
+    amax = fmaxf(amax, __shfl_xor(amax, 2));
+    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    const float d = amax / 127.0f;
+    const float inv = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q0 = (int)roundf(v.x * inv), q1 = (int)roundf(v.y * inv);
+    const int q2 = (int)roundf(v.z * inv), q3 = (int)roundf(v.w * inv);
+    int sum = q0 + q1 + q2 + q3;
+    sum += __shfl_xor(sum, 1);
+    sum += __shfl_xor(sum, 2);
+    const int half_sum = sum;   // lanes 0-3: the block's first 16 values, 4-7: the rest
+    sum += __shfl_xor(sum, 4);
+    uint8_t* codes = row + it * F::PLANES * 1024;
+    *(uint32_t*)(codes + F::slot(ji, l8 >> 2) + 4 * (l8 & 3)) =
+        (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
+        ((uint32_t)(q3 & 0xFF) << 24);
+    float* sc = (float*)(row + n_iter * F::VPI);
+    if (l8 == 0) {
+        const float d8 = __half2float(__float2half_rn(d));
+        if (F::SCF == 2) {
+            *(float2*)(sc + 2 * j) = make_float2(d8, d8 * (float)sum);
+        } else if (F::SCF == 3) {
+            sc[j] = d8;
+            ((int*)sc)[total + j] = -32 * half_sum;
+        } else {
+            sc[j] = d8;
+        }
+    }
+    if (F::SCF == 3 && l8 == 4) ((int*)sc)[2 * total + j] = -32 * half_sum;
+}
+
+constexpr int F32_ROUND = 4;  // float4 loads a thread issues together: the lane exchanges would
+                              // otherwise serialize one memory latency per 1024 values
+
+template <class F, int B>
+static __device__ __forceinline__ void load_f32_round(float4 (&v)[F32_ROUND], const float* __restrict__ x, int t0,
+                                                      int items, int k32) {
+#pragma unroll
+    for (int u = 0; u < F32_ROUND; ++u) {
+        // past the row's end: re-read its last quad (dropped by the caller), never a branch
+        const int t = min(t0 + u * WG, k32 * 8 - 1);
+        v[u] = *(const float4*)(x + (size_t)t * 4);
+    }
+}
+
+template <class F, int B>
+static __device__ __forceinline__ void stage_issue_f32(ActRegs<B>& ar, const float* __restrict__ x, int k32,
+                                                       int n_iter, int x_stride) {
+    const int items = n_iter * (F::VPI / 32) * 8;
+#pragma unroll
+    for (int c = 0; c < ActRegs<B>::ROWS; ++c) load_f32_round<F, B>(ar.x[c], x + (size_t)c * x_stride, threadIdx.x, items, k32);
+}
+
+template <class F, int B>
+static __device__ __forceinline__ void stage_finish_f32(const ActRegs<B>& ar, uint8_t* lds, const float* __restrict__ x,
+                                                        int k32, int n_iter, int x_stride) {
+    const int items = n_iter * (F::VPI / 32) * 8;
     const int row_bytes = lds_bytes_per_row<F>(n_iter);
-    constexpr int U = 4;  // loads issued together: the lane exchanges below would otherwise
-                          // serialize one memory latency per 1024 values
-    for (int t0 = threadIdx.x; t0 < total * 8; t0 += WG * U) {
+    int t0 = threadIdx.x;
+    if (ActRegs<B>::ROWS) {
+#pragma unroll
+        for (int c = 0; c < ActRegs<B>::ROWS; ++c)
+#pragma unroll
+            for (int u = 0; u < F32_ROUND; ++u)
+                if (t0 + u * WG < items) put_f32_quad<F>(lds + c * row_bytes, n_iter, k32, t0 + u * WG, ar.x[c][u]);
+        t0 += WG * F32_ROUND;
+    }
+    for (; t0 < items; t0 += WG * F32_ROUND) {
 #pragma unroll
         for (int c = 0; c < B; ++c) {
-            float4 v[U];
+            float4 v[F32_ROUND];
+            load_f32_round<F, B>(v, x + (size_t)c * x_stride, t0, items, k32);
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int t = t0 + u * WG, j = t >> 3, l8 = t & 7;
-                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (t < total * 8 && j < k32) v[u] = *(const float4*)(x + (size_t)c * x_stride + j * 32 + l8 * 4);
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int t = t0 + u * WG, j = t >> 3, l8 = t & 7;
-                if (t >= total * 8) break;
-                const int it = j / per_pass, ji = j % per_pass;
-                float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
-                amax = fmaxf(amax, __shfl_xor(amax, 1));
-                amax = fmaxf(amax, __shfl_xor(amax, 2));
-                amax = fmaxf(amax, __shfl_xor(amax, 4));
-                const float d = amax / 127.0f;
-                const float inv = d != 0.0f ? 1.0f / d : 0.0f;
-                const int q0 = (int)roundf(v[u].x * inv), q1 = (int)roundf(v[u].y * inv);
-                const int q2 = (int)roundf(v[u].z * inv), q3 = (int)roundf(v[u].w * inv);
-                int sum = q0 + q1 + q2 + q3;
-                sum += __shfl_xor(sum, 1);
-                sum += __shfl_xor(sum, 2);
-                const int half_sum = sum;   // lanes 0-3: the block's first 16 values, 4-7: the rest
-                sum += __shfl_xor(sum, 4);
-                uint8_t* row = lds + c * row_bytes;
-                uint8_t* codes = row + it * F::PLANES * 1024;
-                *(uint32_t*)(codes + F::slot(ji, l8 >> 2) + 4 * (l8 & 3)) =
-                    (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
-                    ((uint32_t)(q3 & 0xFF) << 24);
-                if (l8 == 0) {
-                    float* sc = (float*)(row + n_iter * F::VPI);
-                    const float d8 = __half2float(__float2half_rn(d));
-                    if (F::SCF == 2) {
-                        *(float2*)(sc + 2 * j) = make_float2(d8, d8 * (float)sum);
-                    } else if (F::SCF == 3) {
-                        sc[j] = d8;
-                        ((int*)sc)[total + j] = -32 * half_sum;
-                    } else {
-                        sc[j] = d8;
-                    }
-                }
-                if (F::SCF == 3 && l8 == 4) ((int*)(row + n_iter * F::VPI))[2 * total + j] = -32 * half_sum;
-            }
+            for (int u = 0; u < F32_ROUND; ++u)
+                if (t0 + u * WG < items) put_f32_quad<F>(lds + c * row_bytes, n_iter, k32, t0 + u * WG, v[u]);
         }
     }
 }
@@ -264,7 +341,7 @@ static __device__ __forceinline__ void stage_activation_f32(uint8_t* lds, const 
 // What a workgroup computes: rows of `vx[0..NW)` against the B activation rows at `vy`.
 template <int NW>
 struct RowJob {
-    const uint8_t* vx[NW];
+    gbytes_t vx[NW];
     const uint8_t* vy;
     int nb;            // format blocks per weight row
     int n;             // weight rows
@@ -275,13 +352,34 @@ struct RowJob {
                              // quantized to Q8_1 by the workgroup itself while staging
 };
 
-// The activation as the engines stage it, whichever form it arrives in.
-template <class F, int B, int NW>
-static __device__ __forceinline__ void stage_job(uint8_t* lds, const RowJob<NW>& job, int k32, int n_iter) {
-    if (job.act_stride_f32)
-        stage_activation_f32<F, B>(lds, (const float*)job.vy, k32, n_iter, job.act_stride_f32);
-    else
-        stage_activation<F, B>(lds, job.vy, k32, n_iter, job.stride_col_y);
+// Keeps the loads written before it ahead of the loads written after it in the instruction
+// stream. Without it the compiler is free to sink an activation load towards its first use,
+// which lies past the weight loads, and loads return in issue order.
+static __device__ __forceinline__ void load_fence(const void* p) {
+    asm volatile("" : : "s"(p) : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// The activation as the engines stage it, whichever form it arrives in, with `mid` (the engine's
+// first weight loads) between the two halves. Each form runs `mid` in its own branch: merged
+// after the branch, the wait for the activation data could no longer tell how many loads are
+// ahead of the weights and would wait for part of them too.
+template <class F, int B, int NW, class Mid>
+static __device__ __forceinline__ void stage_around(uint8_t* lds, const RowJob<NW>& job, int k32, int n_iter, Mid&& mid) {
+    ActRegs<B> ar;
+    if (job.act_stride_f32) {
+        stage_issue_f32<F, B>(ar, (const float*)job.vy, k32, n_iter, job.act_stride_f32);
+        load_fence(job.vy);
+        mid();
+        load_fence(job.vy);
+        stage_finish_f32<F, B>(ar, lds, (const float*)job.vy, k32, n_iter, job.act_stride_f32);
+    } else {
+        stage_issue_q8_1<F, B>(ar, job.vy, k32, job.stride_col_y);
+        load_fence(job.vy);
+        mid();
+        load_fence(job.vy);
+        stage_finish_q8_1<F, B>(ar, lds, job.vy, k32, n_iter, job.stride_col_y);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -308,7 +406,9 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
         uint4 hdr[RW], q0[RW], q1[RW];
     };
     // One pass (16 super-blocks) of R rows of every matrix into registers. A lane past the row
-    // end re-reads the row's last block and drops its d / dmin, so it adds nothing.
+    // end re-reads the row's last block and drops its d / dmin when it consumes it, so it adds
+    // nothing (the loaded registers themselves are left alone: touching them here would make
+    // the wave wait for the load).
     auto load = [&](Frag& f, int tile, int it) {
         const bool valid = it * 16 + lb < nb;
         const uint32_t back = valid ? 0u : (uint32_t)(it * 16 + lb - (nb - 1)) * Q4K_BYTES;
@@ -317,12 +417,11 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int row = min(tile * R + r, n - 1);
-                const uint8_t* bp = job.vx[w] + row * row_stride + (size_t)it * (16 * Q4K_BYTES);
+                const uint8_t* bp = (const uint8_t*)(job.vx[w] + row * row_stride + (size_t)it * (16 * Q4K_BYTES));
                 Frag& g = f;
                 g.hdr[w * R + r] = *(const uint4*)(bp + (hdr_off - back));
                 g.q0[w * R + r] = *(const uint4*)(bp + (qs_off - back));
                 g.q1[w * R + r] = *(const uint4*)(bp + (qs_off - back + 16));
-                if (!valid) g.hdr[w * R + r].x = 0;
             }
     };
 
@@ -338,8 +437,9 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
         for (int r = 0; r < RW; ++r) {
             uint32_t sc, mn;
             sel.unpack(f.hdr[r].y, f.hdr[r].z, f.hdr[r].w, sc, mn);
-            d[r] = f16_bits_to_f32(f.hdr[r].x & 0xFFFFu);
-            dmin[r] = f16_bits_to_f32(f.hdr[r].x >> 16);
+            const uint32_t dd = it * 16 + lb < nb ? f.hdr[r].x : 0u;
+            d[r] = f16_bits_to_f32(dd & 0xFFFFu);
+            dmin[r] = f16_bits_to_f32(dd >> 16);
             scl[r] = (float)(sc & 0xFFu);
             sch[r] = (float)(sc >> 8);
             ml[r] = (float)(mn & 0xFFu);
@@ -380,12 +480,13 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
         }
     };
 
-    // The first weight loads go out before the activation is staged, so the two memory
+    // The first weight loads go out between the two halves of the staging, so the two memory
     // latencies overlap instead of adding up (most of a small matrix's run time).
     int tile = job.tile_first + wave, it = 0;
     Frag fa, fb;
-    if (tile < n_tiles) load(fa, tile, 0);
-    stage_job<FmtQ4K, B>(lds, job, nb * 8, n_iter);
+    // (a wave without a tile loads the last one rather than nothing: a load under a branch would
+    // blur the count of loads ahead of the weights and the staging would wait for some of them)
+    stage_around<FmtQ4K, B>(lds, job, nb * 8, n_iter, [&] { load(fa, min(tile, n_tiles - 1), 0); });
     __syncthreads();
     if (tile >= n_tiles) return;
     // Steps are (tile, pass) pairs in order; the loads of step i+1 are issued before step i is
@@ -409,16 +510,17 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
 // ---------------------------------------------------------------------------------------------
 // The step loop the Q6_K and Q8_0 engines share. Steps are (row tile, pass) pairs in order; the
 // loads of step i+1 are issued before step i is consumed, ping-ponging between two register
-// fragments, and the very first loads go out before the activation is staged so that the two
-// memory latencies overlap.
+// fragments, and the very first loads go out between the two halves of the activation staging so
+// that the two memory latencies overlap.
 // ---------------------------------------------------------------------------------------------
 template <class Frag, class Stage, class Load, class Compute>
 static __device__ __forceinline__ void step_loop(int tile, int tile_stride, int n_tiles, int n_iter, Stage&& stage,
                                                  Load&& load, Compute&& compute) {
     int it = 0;
     Frag fa, fb;
-    if (tile < n_tiles) load(fa, tile, 0);
-    stage();
+    // (a wave without a tile loads the last one rather than nothing: a load under a branch would
+    // blur the count of loads ahead of the weights and the staging would wait for some of them)
+    stage([&] { load(fa, min(tile, n_tiles - 1), 0); });
     __syncthreads();
     if (tile >= n_tiles) return;
     for (;;) {
@@ -462,23 +564,22 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
     struct Frag {
         uint4 ql0[RW], ql1[RW], qh[RW];
         uint2 sc[RW];     // the half's 8 scale bytes
-        uint32_t d[RW];   // f16 bits, zero for a lane past the row end
+        uint32_t d[RW];   // f16 bits
     };
+    // A lane past the row end re-reads the row's last block and drops its d when it consumes it.
     auto load = [&](Frag& f, int tile, int it) {
-        const int blk = it * 16 + lb;
-        const bool valid = blk < nb;
-        const int blk_c = valid ? blk : nb - 1;
+        const int blk_c = min(it * 16 + lb, nb - 1);
 #pragma unroll
         for (int w = 0; w < NW; ++w)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int row = min(tile * R + r, n - 1);
-                const uint8_t* bp = job.vx[w] + row * row_stride + (size_t)blk_c * Q6K_BYTES;
+                const uint8_t* bp = (const uint8_t*)(job.vx[w] + row * row_stride + (size_t)blk_c * Q6K_BYTES);
                 f.ql0[w * R + r] = *(const uint4_a2*)(bp + ql_off);
                 f.ql1[w * R + r] = *(const uint4_a2*)(bp + ql_off + 32);
                 f.qh[w * R + r] = *(const uint4_a2*)(bp + qh_off);
                 f.sc[w * R + r] = *(const uint2_a2*)(bp + sc_off);
-                f.d[w * R + r] = valid ? (uint32_t) * (const uint16_t*)(bp + 208) : 0u;
+                f.d[w * R + r] = *(const uint16_t*)(bp + 208);
             }
     };
 
@@ -492,7 +593,7 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
         float ds[RW][4];
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
-            const float d = f16_bits_to_f32(f.d[r]);
+            const float d = it * 16 + lb < nb ? f16_bits_to_f32(f.d[r]) : 0.f;
             ds[r][0] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].x, 8 * lh, 8);
             ds[r][1] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].x, 8 * lh + 16, 8);
             ds[r][2] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].y, 8 * lh, 8);
@@ -533,7 +634,7 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
         }
     };
     step_loop<Frag>(job.tile_first + wave, job.tile_stride, n_tiles, n_iter,
-                    [&] { stage_job<FmtQ6K, B>(lds, job, nb * 8, n_iter); }, load, compute);
+                    [&](auto&& mid) { stage_around<FmtQ6K, B>(lds, job, nb * 8, n_iter, mid); }, load, compute);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -554,22 +655,21 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
 
     struct Frag {
         Run16 q[RW];
-        uint32_t d[RW];       // f16 bits, zero for a lane past the row end
+        uint32_t d[RW];       // f16 bits
         uint32_t shift[RW];   // bits to shift q by
     };
+    // A lane past the row end re-reads the row's last block and drops its d when it consumes it.
     auto load = [&](Frag& f, int tile, int it) {
-        const int blk = it * 32 + lb;
-        const bool valid = blk < nb;
-        const int blk_c = valid ? blk : nb - 1;
+        const int blk_c = min(it * 32 + lb, nb - 1);
 #pragma unroll
         for (int w = 0; w < NW; ++w)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int row = min(tile * R + r, n - 1);
-                const uint8_t* bp = job.vx[w] + row * row_stride + (size_t)blk_c * Q80_BYTES;
+                const uint8_t* bp = (const uint8_t*)(job.vx[w] + row * row_stride + (size_t)blk_c * Q80_BYTES);
                 f.q[w * R + r] = load_run16(bp + 2 + 16 * lh);
                 f.shift[w * R + r] = ((uint32_t)(uintptr_t)(bp + 2) & 2u) * 8u;
-                f.d[w * R + r] = valid ? (uint32_t) * (const uint16_t*)bp : 0u;
+                f.d[w * R + r] = *(const uint16_t*)bp;
             }
     };
 
@@ -586,7 +686,7 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
             q[r] = run16_value(f.q[r], f.shift[r]);
-            d[r] = f16_bits_to_f32(f.d[r]);
+            d[r] = blk < nb ? f16_bits_to_f32(f.d[r]) : 0.f;
         }
 #pragma unroll
         for (int c = 0; c < B; ++c) {
@@ -612,7 +712,7 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
         }
     };
     step_loop<Frag>(job.tile_first + wave, job.tile_stride, n_tiles, n_iter,
-                    [&] { stage_job<FmtQ80, B>(lds, job, nb, n_iter); }, load, compute);
+                    [&](auto&& mid) { stage_around<FmtQ80, B>(lds, job, nb, n_iter, mid); }, load, compute);
 }
 
 

@@ -103,13 +103,13 @@ __global__ __launch_bounds__(WG) void moe_rows_kernel(const uint8_t* __restrict_
     const int tile_stride = (int)gridDim.x * WAVES, tile_first = (int)blockIdx.x * WAVES;
     if (MODE == MODE_GATED) {
         const uint8_t* slab1 = w1 + (int64_t)e * d.slab_bytes;
-        RowJob<2> job{{slab0, slab1}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first};
+        RowJob<2> job{{to_gbytes(slab0), to_gbytes(slab1)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first};
         E::template run<1, R, 2>(job, lds, [&](int row, int, const float* tot) {
             const float g = tot[0];
             out_row[row] = g / (1.0f + expf(-g)) * tot[1];
         });
     } else {
-        RowJob<1> job{{slab0}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first};
+        RowJob<1> job{{to_gbytes(slab0)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first};
         E::template run<1, R, 1>(job, lds, [&](int row, int, const float* tot) {
             float v = tot[0] * scale;
             if (MODE == MODE_DOWN && down_bias) v += scale * down_bias[(size_t)e * d.cols + row];
