@@ -56,15 +56,39 @@ static __device__ __forceinline__ float dpp_f32(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xF, 0xF, true));
 }
 
-// Sum over the 64 lanes of a wave; every lane returns the total.
+template <int ctrl>
+static __device__ __forceinline__ int dpp_i32(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, ctrl, 0xF, 0xF, true);
+}
+
+// Sum over the 64 lanes of a wave; every lane returns the total. Lane exchanges inside a row of
+// 16 are DPP moves; the four row totals cross through scalar registers (an LDS-crossbar
+// permute costs two orders of magnitude more latency than either).
 static __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
     v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
     v += dpp_f32<0x141>(v);  // row_half_mirror
     v += dpp_f32<0x140>(v);  // row_mirror
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
+    const int bits = __float_as_int(v);
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(bits, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(bits, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(bits, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(bits, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// Maximum / sum over each aligned group of 8 lanes; every lane of the group returns it.
+// `quad` receives the value after the first two steps (the lane's group of 4).
+static __device__ __forceinline__ float max8(float v) {
+    v = fmaxf(v, dpp_f32<0xB1>(v));
+    v = fmaxf(v, dpp_f32<0x4E>(v));
+    return fmaxf(v, dpp_f32<0x141>(v));   // quads are uniform by now, so the mirror is "the other quad"
+}
+static __device__ __forceinline__ int sum8(int v, int& quad) {
+    v += dpp_i32<0xB1>(v);
+    v += dpp_i32<0x4E>(v);
+    quad = v;
+    return v + dpp_i32<0x141>(v);
 }
 
 static __device__ __forceinline__ int wave_sum_i32(int v) {

@@ -61,17 +61,13 @@ __global__ __launch_bounds__(256) void mmq_quantize_kernel(const T* __restrict__
     if (i0 + 3 < ne00) v.w = to_f32<T>(xr[i0 + 3]);
 
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    amax = max8(amax);
     const float d = amax / 127.0f;
     const float inv = d != 0.0f ? 1.0f / d : 0.0f;
     const int q0 = (int)roundf(v.x * inv), q1 = (int)roundf(v.y * inv);
     const int q2 = (int)roundf(v.z * inv), q3 = (int)roundf(v.w * inv);
-    int sum = q0 + q1 + q2 + q3;
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
-    sum += __shfl_xor(sum, 4);
+    int quad_sum;
+    const int sum = sum8(q0 + q1 + q2 + q3, quad_sum);
 
     const int64_t kb = i0 / 256;
     const int64_t blocks_per_channel = (ne0 / 256) * ne1;

@@ -259,18 +259,13 @@ static __device__ __forceinline__ void put_f32_quad(uint8_t* row, int n_iter, in
     if (j >= k32) v = make_float4(0.f, 0.f, 0.f, 0.f);   // padding of the last pass
     const int it = j / per_pass, ji = j % per_pass;
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    amax = max8(amax);
     const float d = amax / 127.0f;
     const float inv = d != 0.0f ? 1.0f / d : 0.0f;
     const int q0 = (int)roundf(v.x * inv), q1 = (int)roundf(v.y * inv);
     const int q2 = (int)roundf(v.z * inv), q3 = (int)roundf(v.w * inv);
-    int sum = q0 + q1 + q2 + q3;
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
-    const int half_sum = sum;   // lanes 0-3: the block's first 16 values, 4-7: the rest
-    sum += __shfl_xor(sum, 4);
+    int half_sum;   // lanes 0-3: the block's first 16 values, 4-7: the rest
+    const int sum = sum8(q0 + q1 + q2 + q3, half_sum);
     uint8_t* codes = row + it * F::PLANES * 1024;
     *(uint32_t*)(codes + F::slot(ji, l8 >> 2) + 4 * (l8 & 3)) =
         (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |

@@ -62,19 +62,15 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const T* __restrict_
     }
 
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-    amax = fmaxf(amax, __shfl_xor(amax, 4));
+    amax = max8(amax);
 
     const float d = amax / 127.0f;
     const float inv = d != 0.0f ? 1.0f / d : 0.0f;
     const int q0 = round_code(v.x * inv), q1 = round_code(v.y * inv);
     const int q2 = round_code(v.z * inv), q3 = round_code(v.w * inv);
 
-    int sum = q0 + q1 + q2 + q3;
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
-    sum += __shfl_xor(sum, 4);
+    int quad_sum;
+    const int sum = sum8(q0 + q1 + q2 + q3, quad_sum);
 
     const size_t block = (size_t)row * (kx_padded / 32) + i0 / 32;
     uint32_t* out = vy + block * 9;  // 36 bytes = 9 words
