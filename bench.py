@@ -53,6 +53,12 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", choices=["decode", "gemv-4096", "mmq", "moe", "decode-1p7b"], default="decode",
+                    help="decode (default): the Llama-3-8B step described above; the others are the further measured "
+                         "workloads of loken_amd/workloads.py, one JSON line each")
+    ap.add_argument("--shape", choices=["2a", "2b"], default="2a", help="--workload mmq: 512x4096->14336 Q4_K or 2048x14336->4096 Q6_K")
+    ap.add_argument("--tokens", type=int, default=256, help="--workload moe: rows through the expert block")
+    ap.add_argument("--launches", type=int, default=200, help="timed launches of the per-launch workloads")
     return ap.parse_args()
 
 
@@ -62,6 +68,10 @@ def main() -> int:
         print("bench.py: this build runs on ONE GPU; --gpus > 1 is not supported "
               "(no collectives or sharding are part of it).", file=sys.stderr)
         return 2
+
+    if args.workload != "decode":
+        from loken_amd import workloads
+        return workloads.run(args)
 
     import torch
     from loken_amd import lib, synth

@@ -1,0 +1,431 @@
+"""The other measured workloads of `bench.py` (`--workload ...`): one JSON line each.
+
+  gemv-4096   one Q4_K 4096x4096 mat-vec at one row, over rotating copies of the weight (more
+              than twice the 256 MB last-level cache) and over one hot copy; the Q8_1 quantizer
+              launch timed by itself and the two-launch call timed as a whole
+  mmq         the tiled int8-MFMA matmul: `--shape 2a` = 512 rows x 4096 -> 14336 in Q4_K,
+              `--shape 2b` = 2048 rows x 14336 -> 4096 in Q6_K; quantizer + matmul per step
+  moe         one Qwen3-30B-A3B-shaped expert block (128 experts, 2048 -> 768 -> 2048, top-8,
+              Q4_K) at `--tokens` rows, path chosen as the layer code chooses it
+  decode-1p7b every quantized linear of a Qwen3-1.7B-shaped decode step at `--batch` rows:
+              mat-vec launches up to 8 rows, the tiled matmul above
+
+Timing: 20 warm-up launches, then `--launches` (default 200) launches each bracketed by its own
+pair of events on the launch stream; median, p10, p90, min and max are reported (the protocol of
+the reference's own kernel benchmark, src/tensor/cuda/quant.rs:3940-3957).
+"""
+from __future__ import annotations
+
+import json
+
+import numpy as np
+import torch
+
+from . import lib, moe, ops, synth
+
+HBM_PEAK_GBS = 8000.0
+INT8_PEAK_TOPS = 5000.0
+Q4K, Q6K, Q80 = lib.TYPE_Q4_K, lib.TYPE_Q6_K, lib.TYPE_Q8_0
+NAMES = {Q4K: "Q4_K", Q6K: "Q6_K", Q80: "Q8_0"}
+
+
+# ---------------------------------------------------------------------------- synthetic blocks
+class Maker:
+    """Random blocks generated on the device (field distributions of the seeded host generator
+    in synth.py, which would take minutes for gigabytes)."""
+
+    def __init__(self, dev, seed=0):
+        self.dev = dev
+        self.gen = torch.Generator(device=dev)
+        self.gen.manual_seed(seed)
+
+    def halfs(self, n, scale):
+        v = torch.randn(n, device=self.dev, generator=self.gen).abs() * scale
+        return v.to(torch.float16).view(torch.uint8).reshape(n, 2)
+
+    def q4k(self, n, k):
+        nb = n * (k // 256)
+        w = torch.randint(0, 256, (nb, 144), dtype=torch.uint8, device=self.dev, generator=self.gen)
+        w[:, 0:2] = self.halfs(nb, 1e-3)
+        w[:, 2:4] = self.halfs(nb, 5e-4)
+        return w.reshape(-1)
+
+    def q6k(self, n, k):
+        nb = n * (k // 256)
+        w = torch.randint(0, 256, (nb, 210), dtype=torch.uint8, device=self.dev, generator=self.gen)
+        sc = torch.randint(-64, 64, (nb, 16), dtype=torch.int8, device=self.dev, generator=self.gen)
+        w[:, 192:208] = sc.view(torch.uint8)
+        w[:, 208:210] = self.halfs(nb, 1e-3)
+        return w.reshape(-1)
+
+    def q80(self, n, k):
+        nb = n * (k // 32)
+        w = torch.empty((nb, 34), dtype=torch.uint8, device=self.dev)
+        w[:, 0:2] = self.halfs(nb, 1e-3)
+        w[:, 2:] = torch.randint(-127, 128, (nb, 32), dtype=torch.int8, device=self.dev,
+                                 generator=self.gen).view(torch.uint8)
+        return w.reshape(-1)
+
+    def make(self, wtype, n, k):
+        return {Q4K: self.q4k, Q6K: self.q6k, Q80: self.q80}[wtype](n, k)
+
+    def randn(self, *shape):
+        return torch.randn(shape, device=self.dev, generator=self.gen)
+
+
+# ---------------------------------------------------------------------------- timing
+def time_launches(fn, launches, warm=20):
+    """Per-launch durations in microseconds; `fn(i)` issues launch i on the current stream."""
+    for i in range(warm):
+        fn(i)
+    torch.cuda.synchronize()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
+    for i, (a, b) in enumerate(pairs):
+        a.record()
+        fn(i)
+        b.record()
+    torch.cuda.synchronize()
+    return np.array([a.elapsed_time(b) * 1e3 for a, b in pairs])
+
+
+def time_back_to_back(fn, launches, warm=20):
+    """Average microseconds per launch with the launches issued back to back between two events."""
+    for i in range(warm):
+        fn(i)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(launches):
+        fn(i)
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / launches
+
+
+def capture(fn):
+    """`fn()` (launches on the current stream) recorded once into a HIP graph on a side stream."""
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        fn()                                  # first-launch set-up happens outside the capture
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            fn()
+    torch.cuda.synchronize()
+    return graph
+
+
+def time_replays(graph, launches, warm=20):
+    """Per-replay durations in microseconds of a captured graph."""
+    return time_launches(lambda i: graph.replay(), launches, warm)
+
+
+def spread(us):
+    return {"median_us": round(float(np.median(us)), 3), "p10_us": round(float(np.percentile(us, 10)), 3),
+            "p90_us": round(float(np.percentile(us, 90)), 3), "min_us": round(float(us.min()), 3),
+            "max_us": round(float(us.max()), 3), "launches": int(us.size)}
+
+
+def line(args, metric_value, unit, ms_per_step, dtype, config, roofline, extra=None):
+    out = {"metric": "Q4_K GEMV weight GB/s (% HBM peak); prefill MMQ int8 TOPS (% MFMA peak)",
+           "value": round(metric_value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": dtype, "data": "synthetic", "config": config, "roofline": roofline, "cpu_baseline": None}
+    if extra:
+        out.update(extra)
+    print(json.dumps(out))
+    return 0
+
+
+def check(rc, what):
+    if rc:
+        raise lib.LokenError(what, rc)
+
+
+# ---------------------------------------------------------------------------- gemv-4096
+def gemv_4096(args, dev):
+    L = lib.load()
+    n = k = 4096
+    nbytes = synth.weight_bytes(Q4K, n, k)
+    base = torch.from_numpy(synth.weight(Q4K, n, k, seed=0, stream=0)).to(dev).reshape(-1)
+    copies = [base.clone() for _ in range(64)]           # 604 MB > 2 x 256 MB of last-level cache
+    x = torch.from_numpy(synth.activation(1, k, seed=0)).to(dev)
+    q = ops.quantize_q8_1_rows(x)
+    out = torch.empty((1, n), device=dev)
+    s = torch.cuda.current_stream().cuda_stream
+
+    def mv(w):
+        check(L.lk_mmvq(Q4K, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, 1, q.shape[1], n, None,
+                        0, s), "lk_mmvq")
+
+    def quant():
+        check(L.lk_quantize_q8_1(x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, q.shape[1] * 32, 1, s), "lk_quantize_q8_1")
+
+    vx = (lib.C.c_void_p * 1)()
+    dst = (lib.C.c_void_p * 1)(out.data_ptr())
+    nn = (lib.C.c_int * 1)(n)
+
+    def fused(w):
+        vx[0] = w.data_ptr()
+        check(L.lk_mmvq_fused(Q4K, 1, vx, x.data_ptr(), x.stride(0), dst, lib.TYPE_F32, k, nn, 1, n, None, s),
+              "lk_mmvq_fused")
+
+    launches = args.launches
+    rotated = time_launches(lambda i: mv(copies[i % 64]), launches)
+    hot = time_launches(lambda i: mv(copies[0]), launches)
+    quant_us = time_launches(lambda i: quant(), launches)
+    two = time_launches(lambda i: (quant(), mv(copies[i % 64])), launches)
+    one = time_launches(lambda i: fused(copies[i % 64]), launches)
+    stream_us = time_back_to_back(lambda i: mv(copies[i % 64]), launches)
+    # GPU-side rate without the host's per-launch cost: the 64 rotating launches as one graph
+    side_calls = {}
+
+    def sixty_four():
+        s2 = torch.cuda.current_stream().cuda_stream
+        for w in copies:
+            check(L.lk_mmvq(Q4K, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, 1, q.shape[1], n,
+                            None, 0, s2), "lk_mmvq")
+
+    def sixty_four_fused():
+        s2 = torch.cuda.current_stream().cuda_stream
+        for j, w in enumerate(copies):
+            vxs = side_calls.setdefault(j, (lib.C.c_void_p * 1)(w.data_ptr()))
+            check(L.lk_mmvq_fused(Q4K, 1, vxs, x.data_ptr(), x.stride(0), dst, lib.TYPE_F32, k, nn, 1, n, None, s2),
+                  "lk_mmvq_fused")
+
+    graph_us = time_replays(capture(sixty_four), 50) / 64.0
+    graph_fused_us = time_replays(capture(sixty_four_fused), 50) / 64.0
+    gbs = lambda us: nbytes / us / 1e3
+    med = float(np.median(rotated))
+    roofline = {"bound": "hbm", "achieved": round(gbs(med), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(gbs(med) / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "mmvq_kernel<EngQ4K,1,2,float>",
+                "avg_launch_us": round(float(rotated.mean()), 3), "algorithmic_bytes_per_launch": nbytes,
+                "launches_timed": launches}
+    extra = {"rotated_64_copies": dict(spread(rotated), gbs_median=round(gbs(med), 1)),
+             "hot_one_copy": dict(spread(hot), gbs_median=round(gbs(float(np.median(hot))), 1)),
+             "quantizer_launch": spread(quant_us),
+             "call_two_launches": dict(spread(two), gbs_median=round(gbs(float(np.median(two))), 1)),
+             "call_fused_one_launch": dict(spread(one), gbs_median=round(gbs(float(np.median(one))), 1)),
+             "back_to_back_us_per_launch": round(stream_us, 3), "back_to_back_gbs": round(gbs(stream_us), 1),
+             "graph_of_64_rotating_launches": {"us_per_launch_median": round(float(np.median(graph_us)), 3),
+                                               "gbs_median": round(gbs(float(np.median(graph_us))), 1)},
+             "graph_of_64_fused_launches": {"us_per_launch_median": round(float(np.median(graph_fused_us)), 3),
+                                            "gbs_median": round(gbs(float(np.median(graph_fused_us))), 1)},
+             "note": "per-launch event pairs and back-to-back eager launches are bounded by the host's launch cost; "
+                     "the graph figures are the GPU-side rate, cache-cold (604 MB of rotating copies)"}
+    g_med = float(np.median(graph_us))
+    roofline.update({"achieved": round(gbs(g_med), 1), "frac": round(gbs(g_med) / HBM_PEAK_GBS, 4),
+                     "avg_launch_us": round(float(graph_us.mean()), 3), "launches_timed": 50 * 64,
+                     "timed_as": "graph of 64 launches over rotating copies"})
+    med = g_med
+    return line(args, gbs(med), "GB/s", med * 1e-3, "int8",
+                {"workload": "Q4_K mat-vec 4096x4096, one row, 64 rotating weight copies", "weight_bytes": nbytes},
+                roofline, extra)
+
+
+# ---------------------------------------------------------------------------- mmq
+def mmq(args, dev):
+    L = lib.load()
+    wtype, m, k, n = {"2a": (Q4K, 512, 4096, 14336), "2b": (Q6K, 2048, 14336, 4096)}[args.shape]
+    mk = Maker(dev)
+    w = mk.make(wtype, n, k)
+    x = mk.randn(m, k)
+    out = torch.empty((m, n), device=dev)
+    ws = ops.mmq_quantize(wtype, x)
+    quantizer = getattr(L, ops.MMQ_QUANTIZER[wtype])
+    launcher = getattr(L, ops.MMQ_LAUNCHER[wtype])
+    info = ops.MMQ_DEVICE_INFO
+    s = torch.cuda.current_stream().cuda_stream
+    k_padded = ops.pad_to(ops.pad_to(k, 512), 128)
+
+    def quant():
+        quantizer(x.data_ptr(), None, ws.data_ptr(), 0, k, x.stride(0), 0, 0, k_padded, m, 1, 1, s)
+
+    def matmul():
+        if launcher(None, w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
+                    info["cc"], info["nsm"], info["smpbo"], info["warp_size"], s) == 0:
+            raise lib.LokenError(ops.MMQ_LAUNCHER[wtype], lib.LK_ERR_ARG)
+
+    launches = args.launches
+    mm = time_launches(lambda i: matmul(), launches)
+    qu = time_launches(lambda i: quant(), launches)
+    both = time_launches(lambda i: (quant(), matmul()), launches)
+    op_count = 2.0 * m * k * n
+    tops = lambda us: op_count / us / 1e6
+    med = float(np.median(both))
+    kern = float(np.median(mm))
+    name = {Q4K: "MmqQ4K", Q6K: "MmqQ6K"}[wtype]
+    roofline = {"bound": "mfma", "achieved": round(tops(kern), 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                "frac": round(tops(kern) / INT8_PEAK_TOPS, 4), "traffic": None,
+                "kernel": f"mmq_dense_kernel<{name},128,2>", "avg_launch_us": round(float(mm.mean()), 3),
+                "algorithmic_ops_per_launch": int(op_count), "launches_timed": launches}
+    extra = {"matmul_launch": dict(spread(mm), tops_median=round(tops(kern), 1)), "quantizer_launch": spread(qu),
+             "call_two_launches": dict(spread(both), tops_median=round(tops(med), 1))}
+    return line(args, tops(med), "TOP/s", med * 1e-3, "int8",
+                {"workload": f"tiled matmul {m} rows x {k} -> {n}, {NAMES[wtype]} weights, quantizer + matmul",
+                 "ops": int(op_count)}, roofline, extra)
+
+
+# ---------------------------------------------------------------------------- moe
+def moe_block(args, dev):
+    experts, hidden, ffn, topk, tokens = 128, 2048, 768, 8, args.tokens
+    mk = Maker(dev)
+    gate = mk.q4k(experts * ffn, hidden)
+    up = mk.q4k(experts * ffn, hidden)
+    down = mk.q4k(experts * hidden, ffn)
+    x = mk.randn(tokens, hidden)
+    logits = mk.randn(tokens, experts)
+    probs = torch.softmax(logits, dim=-1)
+    weights, choices = torch.topk(probs, topk, dim=-1)
+    weights = (weights / weights.sum(dim=-1, keepdim=True)).contiguous()
+    choices = choices.to(torch.int32).contiguous()
+
+    pairs = tokens * topk
+    tiled = moe.moe_mmq_pays(pairs, experts)
+    # The routing (the router's side of the boundary) is built once; the timed block is what the
+    # expert launchers do with it, recorded into a graph so that the host's cost stays outside.
+    flat_w = weights.reshape(-1)
+    if tiled:
+        plan = moe.MmqRouting.from_choices(choices, experts)
+
+        def block():
+            h = plan.gate_up_silu(Q4K, x, gate, up, ffn)
+            return plan.down_fold(Q4K, h, down, hidden, flat_w)
+    else:
+        routing = moe.ExpertRouting(choices)
+
+        def block():
+            h = moe.moe_gemm_gguf_gate_up_silu_mul(Q4K, x, gate, up, routing, experts, ffn)
+            return moe.moe_gemm_gguf_down_reduce(Q4K, h, down, routing, flat_w, experts, hidden)
+
+    eager = time_launches(lambda i: block(), args.launches)
+    us = time_replays(capture(block), args.launches)
+    med = float(np.median(us))
+    load = torch.bincount(choices.reshape(-1).to(torch.int64), minlength=experts).cpu().numpy()
+    distinct = int((load > 0).sum())
+    one_matrix = synth.weight_bytes(Q4K, ffn, hidden)
+    if tiled:
+        op_count = 6.0 * pairs * ffn * hidden
+        value, unit = op_count / med / 1e6, "TOP/s"
+        roofline = {"bound": "mfma", "achieved": round(value, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                    "frac": round(value / INT8_PEAK_TOPS, 4), "traffic": None, "kernel": "mmq_moe_kernel<MmqQ4K,...>",
+                    "note": "whole expert block (plan, route, quantize, two grouped matmuls, activation, fold)"}
+    else:
+        nbytes = 3 * one_matrix * distinct
+        value, unit = nbytes / med / 1e3, "GB/s"
+        roofline = {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "moe_rows_kernel<EngQ4K,...>",
+                    "note": "whole expert block (quantize, gate/up pairs, down pairs, weighted sum); bytes = 3 matrices "
+                            "per distinct expert hit"}
+    extra = {"block_graph_replay": spread(us), "block_eager_from_python": spread(eager), "path": "expert-batched tiled matmul" if tiled else "mat-vec per routed pair",
+             "routed_pairs": pairs, "distinct_experts": distinct,
+             "expert_load_histogram": {"max": int(load.max()), "mean": round(float(load.mean()), 2),
+                                       "rows_per_expert_sorted_top8": sorted(load.tolist(), reverse=True)[:8]}}
+    return line(args, value, unit, med * 1e-3, "int8",
+                {"workload": f"MoE expert block, 128 experts 2048->768->2048 Q4_K, top-8, {tokens} tokens"}, roofline,
+                extra)
+
+
+# ---------------------------------------------------------------------------- decode-1p7b
+def decode_1p7b(args, dev):
+    L = lib.load()
+    b = args.batch
+    hidden, kv, ffn, vocab, layers = 2048, 1024, 6144, 151936, 28
+    mk = Maker(dev)
+    s = torch.cuda.current_stream().cuda_stream
+    info = ops.MMQ_DEVICE_INFO
+    groups = [("x", hidden, Q4K, [hidden, kv, kv]), ("attn", hidden, Q4K, [hidden]), ("x2", hidden, Q4K, [ffn, ffn]),
+              ("h", ffn, Q6K, [hidden])]
+    acts = {g: mk.randn(b, k) for g, k, _, _ in groups}
+    acts["final"] = mk.randn(b, hidden)
+    keep, plan, total_bytes = [], [], 0
+    matvec = b <= 8
+
+    def add_group(g, k, wtype, ns):
+        nonlocal total_bytes
+        weights = [mk.make(wtype, n, k) for n in ns]
+        keep.extend(weights)
+        total_bytes += sum(synth.weight_bytes(wtype, n, k) for n in ns)
+        x = acts[g]
+        if matvec and k <= 8192:
+            stride = max(ns)
+            outs = [torch.empty((b, stride), device=dev) for _ in ns]
+            vx = (lib.C.c_void_p * len(ns))(*[w.data_ptr() for w in weights])
+            dst = (lib.C.c_void_p * len(ns))(*[o.data_ptr() for o in outs])
+            nn = (lib.C.c_int * len(ns))(*ns)
+            keep.extend(outs + [vx, dst, nn])
+            plan.append(("status", L.lk_mmvq_fused, (wtype, len(ns), vx, x.data_ptr(), x.stride(0), dst, lib.TYPE_F32, k, nn, b,
+                                           stride, None, s)))
+        elif matvec:
+            q = torch.empty((b, ops.pad_to(k, 512) // 32, 36), dtype=torch.uint8, device=dev)
+            keep.append(q)
+            plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, q.shape[1] * 32, b, s)))
+            for w, n in zip(weights, ns):
+                out = torch.empty((b, n), device=dev)
+                keep.append(out)
+                plan.append(("status", L.lk_mmvq, (wtype, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, b,
+                                         q.shape[1], n, None, 0, s)))
+        else:
+            k_padded = ops.pad_to(ops.pad_to(k, 512), 128)
+            ws = torch.empty(ops.mmq_workspace_bytes(b, k), dtype=torch.uint8, device=dev)
+            keep.append(ws)
+            plan.append(("void", getattr(L, ops.MMQ_QUANTIZER[wtype]),
+                         (x.data_ptr(), None, ws.data_ptr(), 0, k, x.stride(0), 0, 0, k_padded, b, 1, 1, s)))
+            for w, n in zip(weights, ns):
+                out = torch.empty((b, n), device=dev)
+                keep.append(out)
+                plan.append(("tile", getattr(L, ops.MMQ_LAUNCHER[wtype]),
+                             (None, w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, b, k // 256, n, info["cc"],
+                              info["nsm"], info["smpbo"], info["warp_size"], s)))
+
+    for _ in range(layers):
+        for g, k, wtype, ns in groups:
+            add_group(g, k, wtype, ns)
+    add_group("final", hidden, Q6K, [vocab])
+    def run(items):
+        for kind, fn, a in items:
+            rc = fn(*a)
+            if kind == "tile" and rc == 0:      # tile width launched; 0 = nothing ran
+                raise lib.LokenError("tiled matmul launcher", lib.LK_ERR_ARG)
+            if kind == "status" and rc:
+                raise lib.LokenError("mat-vec launcher", rc)
+
+    run(plan)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        cap = [(kind, fn, a[:-1] + (side.cuda_stream,)) for kind, fn, a in plan]
+        run(cap)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            run(cap)
+    torch.cuda.synchronize()
+    import time
+    for _ in range(args.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = total_bytes / (ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": "whole step (all launches of the graph)", "launches_per_step": len(plan)}
+    return line(args, value, "GB/s", ms, "int8",
+                {"workload": f"qwen3-1.7b decode-step quantized linears (Q4_K attention and gate/up, Q6_K down and "
+                             f"lm_head), batch {b}, 28 layers",
+                 "path": "mat-vec (fused; own quantizer launch for rows over 8192 values)" if matvec
+                         else "tiled int8-MFMA matmul (quantizer per activation, matmul per linear)",
+                 "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline)
+
+
+def run(args) -> int:
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible")
+    lib.load()  # raises if the HIP library is missing: there is no other path
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    return {"gemv-4096": gemv_4096, "mmq": mmq, "moe": moe_block, "decode-1p7b": decode_1p7b}[args.workload](args, dev)
