@@ -260,6 +260,14 @@ int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,
                                     const float* down_bias, const float* add_after, void* stream);
 /* outputs[t, c] += sum over k ascending of pairs[(t * topk + k), c] (cuda/moe/moe_gguf.cu:745-752). */
 void loken_moe_sum_topk(const float* pairs, float* outputs, int tokens, int topk, int cols, void* stream);
+/* Q4_K weight [size_n rows, size_k] x plain Q8_1 rows [size_m, size_k / 32 blocks] -> output
+ * [size_m, size_n] f32 on the int8 matrix unit, 32 activation rows per pass and no weight staging
+ * in LDS: the path for row counts between the mat-vec kernels and the tiled matmul. Replaces
+ * loken_dense_q4k_imma_m8_plain (declared src/inference/moe_cuda/mod.rs:456-458, called from
+ * dense_q4k_imma_m8_matmul, src/inference/moe_cuda/dense/imma.rs:82-135). size_k a multiple of
+ * 256; weights 16-byte aligned; nothing is launched on a bad argument (void, as the reference's). */
+void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
+                                   int size_k, void* stream);
 /* Frees the current device's MoE decode scratch (cuda/moe/moe_gguf.cu:104-118). Synchronizes. */
 void loken_stream_scratch_release(void);
 

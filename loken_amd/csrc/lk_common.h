@@ -114,6 +114,10 @@ struct LkDevice {
 };
 const LkDevice& lk_device();
 
+// Q4_K x up to any number of Q8_1 rows on the matrix unit (rows_mfma.hip); LK_* status.
+int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y,
+                     int ldd, hipStream_t stream);
+
 static inline int lk_launch_status() {
     return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;
 }

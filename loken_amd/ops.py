@@ -125,6 +125,18 @@ MMQ_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_gguf_q4_k", _lib.TYPE_Q6_K: "launch_
 MMQ_DEVICE_INFO = dict(cc=0x1000950, nsm=256, smpbo=160 * 1024, warp_size=64)
 
 
+def dense_q4k_rows(weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tensor:
+    """``[rows, k]`` f32 x Q4_K weight ``[n, k]`` -> ``[rows, n]`` f32 on the matrix unit, rows
+    quantized to plain Q8_1 first (dense_q4k_imma_m8_matmul, src/inference/moe_cuda/dense/imma.rs:82-135)."""
+    rows, k = x.shape
+    if k % 256:
+        raise ValueError("dense_q4k_rows: k must be a multiple of 256")
+    q = quantize_q8_1_rows(x, k_padded=k)
+    out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
+    _lib.load().loken_dense_q4k_imma_m8_plain(weight.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k, _stream())
+    return out
+
+
 def mmq_workspace_bytes(rows: int, k: int) -> int:
     """The reference's sizing (kernel_matmul/mmq.rs:38-41): 144 bytes per 128 padded values per
     row, plus 128 records of slack."""

@@ -365,6 +365,27 @@ def decode_1p7b(args, dev):
                 keep.append(out)
                 plan.append(("status", L.lk_mmvq, (wtype, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, b,
                                          q.shape[1], n, None, 0, s)))
+        elif wtype == Q4K and b <= 64:
+            # a handful of rows: Q4_K on the matrix unit without weight staging
+            q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
+            keep.append(q)
+            plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s)))
+            for w, n in zip(weights, ns):
+                out = torch.empty((b, n), device=dev)
+                keep.append(out)
+                plan.append(("void", L.loken_dense_q4k_imma_m8_plain, (w.data_ptr(), q.data_ptr(), out.data_ptr(), b, n, k, s)))
+        elif b <= 32 and args.mid_rows == "matvec":
+            # mat-vec launches over slices of eight rows
+            q = torch.empty((b, ops.pad_to(k, 512) // 32, 36), dtype=torch.uint8, device=dev)
+            keep.append(q)
+            plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, q.shape[1] * 32, b, s)))
+            for w, n in zip(weights, ns):
+                out = torch.empty((b, n), device=dev)
+                keep.append(out)
+                for r0 in range(0, b, 8):
+                    rows = min(8, b - r0)
+                    plan.append(("status", L.lk_mmvq, (wtype, w.data_ptr(), q[r0].data_ptr(), out[r0].data_ptr(),
+                                                        lib.TYPE_F32, k, n, rows, q.shape[1], n, None, 0, s)))
         else:
             k_padded = ops.pad_to(ops.pad_to(k, 512), 128)
             ws = torch.empty(ops.mmq_workspace_bytes(b, k), dtype=torch.uint8, device=dev)
@@ -418,7 +439,9 @@ def decode_1p7b(args, dev):
                 {"workload": f"qwen3-1.7b decode-step quantized linears (Q4_K attention and gate/up, Q6_K down and "
                              f"lm_head), batch {b}, 28 layers",
                  "path": "mat-vec (fused; own quantizer launch for rows over 8192 values)" if matvec
-                         else "tiled int8-MFMA matmul (quantizer per activation, matmul per linear)",
+                         else "Q4_K: matrix-unit rows kernel (no weight staging); Q6_K: "
+                              + ("mat-vec over slices of eight rows" if b <= 32 and args.mid_rows == "matvec"
+                                 else "tiled int8-MFMA matmul"),
                  "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline)
 
 

@@ -1,0 +1,75 @@
+"""GPU parity of the matrix-unit path for a handful of activation rows (Q4_K x plain Q8_1 rows,
+the library's loken_dense_q4k_imma_m8_plain).
+
+Bars: f32 outputs within 1e-3 relative + 1e-4 absolute of the same-codes oracle (the integer
+sub-block dots are the ones the mat-vec family is checked on bit for bit; here they come out of
+v_mfma_i32_32x32x32_i8); agreement with the mat-vec family to summation order; a row's result
+does not depend on how many other rows ride in the pass.
+"""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+import oracle
+from loken_amd import lib, ops, synth
+
+pytestmark = pytest.mark.gpu
+
+Q4K = lib.TYPE_Q4_K
+RTOL, ATOL = 1e-3, 1e-4
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def assert_close(got, want):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    bad = np.abs(got - want) > RTOL * np.abs(want) + ATOL
+    assert not bad.any(), f"{bad.sum()} of {bad.size} outside tolerance; worst {np.abs(got - want).max()}"
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (5, 256, 64), (16, 1024, 130), (32, 768, 33), (33, 512, 96),
+                                   (70, 2048, 257), (9, 14336, 40), (12, 4096, 1024)])
+def test_rows_on_the_matrix_unit_match_same_codes_oracle(m, k, n):
+    w = synth.weight(Q4K, n, k, seed=60, stream=1)
+    x = synth.activation(m, k, seed=60)
+    got = ops.dense_q4k_rows(dev(w), dev(x), n).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(Q4K, x, w, n))
+
+
+def test_rows_agree_with_matvec_family():
+    m, k, n = 24, 4096, 600
+    w = dev(synth.weight(Q4K, n, k, seed=61, stream=2))
+    x = dev(synth.activation(m, k, seed=61))
+    got = ops.dense_q4k_rows(w, x, n)
+    q = ops.quantize_q8_1_rows(x)
+    rows = torch.cat([ops.mmvq(Q4K, w, q[i:i + 8], k, n) for i in range(0, m, 8)])
+    # same integers on both sides: only f32 summation order differs
+    assert (got - rows).abs().max().item() <= 2e-5 * rows.abs().max().item()
+
+
+def test_a_row_does_not_depend_on_its_company():
+    m, k, n = 40, 1024, 200
+    w = dev(synth.weight(Q4K, n, k, seed=62, stream=3))
+    x = dev(synth.activation(m, k, seed=62))
+    full = ops.dense_q4k_rows(w, x, n)
+    for rows in ([0], [3, 4, 5], list(range(31, 40))):
+        part = ops.dense_q4k_rows(w, x[rows].contiguous(), n)
+        assert torch.equal(part, full[rows])
+
+
+def test_full_gate_shape_against_matvec_and_sampled_oracle():
+    m, k, n = 16, 4096, 14336
+    w = synth.weight(Q4K, n, k, seed=0, stream=30)
+    x = synth.activation(m, k, seed=0, stream=31)
+    wd, xd = dev(w), dev(x)
+    got = ops.dense_q4k_rows(wd, xd, n)
+    q = ops.quantize_q8_1_rows(xd)
+    vec = torch.cat([ops.mmvq(Q4K, wd, q[i:i + 8], k, n) for i in range(0, m, 8)])
+    assert (got - vec).abs().max().item() <= 2e-5 * vec.abs().max().item()
+    rng = np.random.default_rng(63)
+    wr = np.sort(rng.choice(n, 300, replace=False))
+    assert_close(got.cpu().numpy()[:, wr], oracle.ob_matmul(Q4K, x, w[wr], len(wr)))
