@@ -53,6 +53,9 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain device copy of 1 GiB before the steps: the dispatch of known size that "
+                         "scales the FETCH_SIZE / WRITE_SIZE counters of a profiled run")
     ap.add_argument("--workload", choices=["decode", "gemv-4096", "mmq", "moe", "decode-1p7b"], default="decode",
                     help="decode (default): the Llama-3-8B step described above; the others are the further measured "
                          "workloads of loken_amd/workloads.py, one JSON line each")
@@ -221,6 +224,13 @@ def main() -> int:
 
     run(plan)  # eager once: first-launch set-up happens outside any capture
     torch.cuda.synchronize()
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+        src.fill_(1.0)
+        dstc = torch.empty_like(src)
+        dstc.copy_(src)   # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dstc
 
     graph = None
     if not args.no_graph:
