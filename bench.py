@@ -35,6 +35,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel's launch mix, from the two rocprofv3 counter runs
+# (FETCH_SIZE, then WRITE_SIZE, scaled by a plain 1 GiB copy) summarized in
+# profiles/mmvq_llama3_8b_decode_b1_hbm_traffic.md. Counters cannot be read from inside this
+# process, so the figure is carried here for the configuration it was taken on:
+# (launch plan, batch, layers) -> bytes.
+MEASURED_TRAFFIC = {("auto", 1, 32): 30215800, ("fused", 1, 32): 30215800}
 LAYERS = 32
 HIDDEN, KV, FFN, VOCAB = 4096, 1024, 14336, 128256
 
@@ -281,7 +287,8 @@ def main() -> int:
     bytes_per_launch = q4k_bytes / len(q4k_plan)
     achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC.get((args.plan, b, args.layers)),
                 "kernel": f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches}
 
