@@ -7,8 +7,10 @@ One *step* = every quantized linear of one Llama-3-8B-shaped decode step at batc
 4.97 GB of blocks. Launch plans: `--plan fused`: the linears that share an activation go out as
 one launch (q,k,v; gate,up) and every launch quantizes its f32 activation to Q8_1 in LDS itself,
 4 launches per layer; `--plan split`: the two-launch form per linear (Q8_1 quantizer, then
-mat-vec); `--plan auto` (default): fused, except that `down`, whose 14336-value rows are dear to
-quantize once per workgroup, keeps its own quantizer launch (5 launches per layer).
+mat-vec); `--plan auto` (default): fused, and up to 4 rows the gate,up launch applies SiLU(gate)*up
+and writes the Q8_1 rows that `down` reads (4 launches per layer, no quantizer launch); above 4
+rows `down`, whose 14336-value rows are dear to quantize once per workgroup, keeps its own
+quantizer launch (5 launches per layer).
 Distinct weights per layer, so the step is cache-cold by construction.
 Weights and activations are synthetic (seeded, generated on the device) and resident in HBM
 before the timed region.
@@ -186,14 +188,35 @@ def main() -> int:
             q4k_bytes += nbytes
         return outs[0]
 
+    def add_pair(wtype, gate, up, g, n, k):
+        """One launch: silu(gate . x) * (up . x) as Q8_1 rows in q81["h"] (which `down` then reads)."""
+        nonlocal total_bytes, q4k_bytes
+        a, q = acts[g], q81["h"]
+        item = (L.lk_mmvq_pair_act_q8_1, (wtype, gate.data_ptr(), up.data_ptr(), a.data_ptr(), 1, a.stride(0),
+                                          q.data_ptr(), q.shape[1], k, n, b, 0, stream))
+        plan.append(item)
+        nbytes = 2 * synth.weight_bytes(wtype, n, k)
+        total_bytes += nbytes
+        if wtype == Q4K:
+            q4k_plan.append(item)
+            q4k_bytes += nbytes
+
     first_out = None
     first_w = None
     for layer in range(args.layers):
         if args.plan in ("fused", "auto"):
             made = {name: (maker(n, k), wtype, n, k, g) for name, wtype, n, k, maker, g in shapes}
             keep.extend(v[0] for v in made.values())
+            paired = args.plan == "auto" and b <= 4
             for group in (("q", "k", "v"), ("o",), ("gate", "up"), ("down",)):
                 wtype, k, g = made[group[0]][1], made[group[0]][3], made[group[0]][4]
+                if paired and group == ("gate", "up"):
+                    # act(gate . x) * (up . x) written as the Q8_1 rows `down` reads
+                    add_pair(wtype, made["gate"][0], made["up"][0], g, made["gate"][2], k)
+                    continue
+                if paired and group == ("down",):
+                    add_gemv(wtype, made["down"][0], "h", made["down"][2], k)
+                    continue
                 if args.plan == "auto" and k > 8192:
                     add_quant(g)
                     for nm in group:

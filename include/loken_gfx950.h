@@ -108,6 +108,17 @@ int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, const void* vy
                      int dst_type, int ncols_x, int nrows_x, int batch, int stride_col_y,
                      int stride_col_dst, int act, void* stream);
 
+/* The gate/up pair launch that hands its result on as Q8_1: dst = Q8_1(act(gate . x) * (up . x)),
+ * blocks of 32 consecutive output rows, written with lk_quantize_q8_1's rule, so the down
+ * projection of a decode layer reads it without a quantizer launch in between (the fused
+ * neighbours of the mat-vec: pair kernels src/inference/cuda/mmvq_gguf.cu:588-758 followed by
+ * quantize_q8_1_rows, src/tensor/cuda/quant.rs:112-151, in one launch). `act`: the activation
+ * rows, f32 (act_is_f32 != 0, stride_act floats apart, quantized to Q8_1 in the kernel) or Q8_1
+ * (stride_act blocks apart). dst: batch rows of nrows_x / 32 blocks, stride_dst_blocks apart.
+ * nrows_x a multiple of 32; batch 1..4; act_fn 0 = SiLU, 1 = tanh-GELU. */
+int lk_mmvq_pair_act_q8_1(int wtype, const void* gate, const void* up, const void* act, int act_is_f32,
+                          int stride_act, void* dst_q8_1, int stride_dst_blocks, int ncols_x, int nrows_x,
+                          int batch, int act_fn, void* stream);
 /* `groups` weights of one shape [nrows_x, ncols_x], each over its OWN Q8_1 row: weight g lives at
  * device address table[g] (a device array), reads the blocks from g * ncols_x/32 of vy_q8_1 and
  * writes dst from g * nrows_x. ncols_x must be a multiple of 512. Replaces kernel

@@ -345,6 +345,20 @@ struct RowJob {
     int tile_first;    // first row tile of wave 0 of this workgroup
     int act_stride_f32 = 0;  // non-zero: `vy` holds f32 activation rows this many floats apart,
                              // quantized to Q8_1 by the workgroup itself while staging
+    // A wave's tiles: it starts at tile_first + wave * wave_stride, walks run_len consecutive tiles
+    // (a power of two; the run starts on a multiple of it) and then jumps tile_stride from the
+    // run's last tile. The defaults give the plain round-robin tile, tile + tile_stride, ...
+    int wave_stride = 1;
+    int run_len = 1;
+};
+
+template <int NW>
+static __device__ __forceinline__ int next_tile(const RowJob<NW>& job, int t) {
+    return (job.run_len > 1 && ((t + 1) & (job.run_len - 1))) ? t + 1 : t + job.tile_stride;
+}
+
+struct NoTileHook {
+    __device__ __forceinline__ void operator()(int) const {}
 };
 
 // Keeps the loads written before it ahead of the loads written after it in the instruction
@@ -382,8 +396,9 @@ static __device__ __forceinline__ void stage_around(uint8_t* lds, const RowJob<N
 // per wave pass, loads of the next step in flight while the current one is consumed.
 // epi(row, col, totals[NW]) runs on lane 0 for every finished (row, activation row).
 // ---------------------------------------------------------------------------------------------
-template <int B, int R, int NW, class Epi>
-static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* lds, Epi&& epi) {
+// done(tile) runs on every lane of the wave once the tile's rows have been handed to epi.
+template <int B, int R, int NW, class Epi, class Done>
+static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* lds, Epi&& epi, Done&& done) {
     const int nb = job.nb, n = job.n;
     const int n_iter = (nb + 15) >> 4;
     const int row_bytes = lds_bytes_per_row<FmtQ4K>(n_iter);
@@ -472,12 +487,13 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
                     }
                     if (lane == 0 && tile * R + r < n) epi(tile * R + r, c, tot);
                 }
+            done(tile);
         }
     };
 
     // The first weight loads go out between the two halves of the staging, so the two memory
     // latencies overlap instead of adding up (most of a small matrix's run time).
-    int tile = job.tile_first + wave, it = 0;
+    int tile = job.tile_first + wave * job.wave_stride, it = 0;
     Frag fa, fb;
     // (a wave without a tile loads the last one rather than nothing: a load under a branch would
     // blur the count of loads ahead of the weights and the staging would wait for some of them)
@@ -488,13 +504,13 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
     // consumed, ping-ponging between two register fragments.
     for (;;) {
         int nt = tile, ni = it + 1;
-        if (ni == n_iter) { ni = 0; nt += job.tile_stride; }
+        if (ni == n_iter) { ni = 0; nt = next_tile(job, nt); }
         if (nt < n_tiles) load(fb, nt, ni);
         compute(fa, tile, it);
         tile = nt; it = ni;
         if (tile >= n_tiles) break;
         nt = tile; ni = it + 1;
-        if (ni == n_iter) { ni = 0; nt += job.tile_stride; }
+        if (ni == n_iter) { ni = 0; nt = next_tile(job, nt); }
         if (nt < n_tiles) load(fa, nt, ni);
         compute(fb, tile, it);
         tile = nt; it = ni;
@@ -508,8 +524,8 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
 // fragments, and the very first loads go out between the two halves of the activation staging so
 // that the two memory latencies overlap.
 // ---------------------------------------------------------------------------------------------
-template <class Frag, class Stage, class Load, class Compute>
-static __device__ __forceinline__ void step_loop(int tile, int tile_stride, int n_tiles, int n_iter, Stage&& stage,
+template <class Frag, int NW, class Stage, class Load, class Compute>
+static __device__ __forceinline__ void step_loop(const RowJob<NW>& job, int tile, int n_tiles, int n_iter, Stage&& stage,
                                                  Load&& load, Compute&& compute) {
     int it = 0;
     Frag fa, fb;
@@ -520,13 +536,13 @@ static __device__ __forceinline__ void step_loop(int tile, int tile_stride, int 
     if (tile >= n_tiles) return;
     for (;;) {
         int nt = tile, ni = it + 1;
-        if (ni == n_iter) { ni = 0; nt += tile_stride; }
+        if (ni == n_iter) { ni = 0; nt = next_tile(job, nt); }
         if (nt < n_tiles) load(fb, nt, ni);
         compute(fa, tile, it);
         tile = nt; it = ni;
         if (tile >= n_tiles) break;
         nt = tile; ni = it + 1;
-        if (ni == n_iter) { ni = 0; nt += tile_stride; }
+        if (ni == n_iter) { ni = 0; nt = next_tile(job, nt); }
         if (nt < n_tiles) load(fa, nt, ni);
         compute(fb, tile, it);
         tile = nt; it = ni;
@@ -541,8 +557,8 @@ static __device__ __forceinline__ void step_loop(int tile, int tile_stride, int 
 // cycles, not HBM, bound this format). The codes stay unsigned; the -32 offset comes in through
 // the staged per-run activation sums.
 // ---------------------------------------------------------------------------------------------
-template <int B, int R, int NW, class Epi>
-static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* lds, Epi&& epi) {
+template <int B, int R, int NW, class Epi, class Done>
+static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* lds, Epi&& epi, Done&& done) {
     const int nb = job.nb, n = job.n;
     const int n_iter = (nb + 15) >> 4;
     const int row_bytes = lds_bytes_per_row<FmtQ6K>(n_iter);
@@ -626,17 +642,18 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
                     }
                     if (lane == 0 && tile * R + r < n) epi(tile * R + r, c, tot);
                 }
+            done(tile);
         }
     };
-    step_loop<Frag>(job.tile_first + wave, job.tile_stride, n_tiles, n_iter,
+    step_loop<Frag>(job, job.tile_first + wave * job.wave_stride, n_tiles, n_iter,
                     [&](auto&& mid) { stage_around<FmtQ6K, B>(lds, job, nb * 8, n_iter, mid); }, load, compute);
 }
 
 // ---------------------------------------------------------------------------------------------
 // Q8_0: 2 lanes per 32-value block, 32 blocks per wave pass.
 // ---------------------------------------------------------------------------------------------
-template <int B, int R, int NW, class Epi>
-static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* lds, Epi&& epi) {
+template <int B, int R, int NW, class Epi, class Done>
+static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* lds, Epi&& epi, Done&& done) {
     const int nb = job.nb, n = job.n;
     const int n_iter = (nb + 31) >> 5;
     const int row_bytes = lds_bytes_per_row<FmtQ80>(n_iter);
@@ -704,9 +721,10 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
                     }
                     if (lane == 0 && tile * R + r < n) epi(tile * R + r, c, tot);
                 }
+            done(tile);
         }
     };
-    step_loop<Frag>(job.tile_first + wave, job.tile_stride, n_tiles, n_iter,
+    step_loop<Frag>(job, job.tile_first + wave * job.wave_stride, n_tiles, n_iter,
                     [&](auto&& mid) { stage_around<FmtQ80, B>(lds, job, nb, n_iter, mid); }, load, compute);
 }
 
@@ -714,18 +732,24 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
 // Format tags: which engine serves a ggml type, and its LDS footprint.
 struct EngQ4K {
     using Fmt = FmtQ4K;
-    template <int B, int R, int NW, class Epi>
-    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e) { rows_q4k<B, R, NW>(j, lds, e); }
+    template <int B, int R, int NW, class Epi, class Done = NoTileHook>
+    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
+        rows_q4k<B, R, NW>(j, lds, e, d);
+    }
 };
 struct EngQ6K {
     using Fmt = FmtQ6K;
-    template <int B, int R, int NW, class Epi>
-    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e) { rows_q6k<B, R, NW>(j, lds, e); }
+    template <int B, int R, int NW, class Epi, class Done = NoTileHook>
+    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
+        rows_q6k<B, R, NW>(j, lds, e, d);
+    }
 };
 struct EngQ80 {
     using Fmt = FmtQ80;
-    template <int B, int R, int NW, class Epi>
-    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e) { rows_q80<B, R, NW>(j, lds, e); }
+    template <int B, int R, int NW, class Epi, class Done = NoTileHook>
+    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
+        rows_q80<B, R, NW>(j, lds, e, d);
+    }
 };
 
 template <class F>

@@ -54,6 +54,7 @@ SIGNATURES.update({
     "loken_moe_gemm_gguf_down_reduce": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp, _vp]),
     "loken_moe_sum_topk": (None, [_vp, _vp, _i, _i, _i, _vp]),
     "loken_stream_scratch_release": (None, []),
+    "lk_mmvq_pair_act_q8_1": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i, _i, _vp]),
     "loken_dense_q4k_imma_m8_plain": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "loken_moe_mmq_fold": (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
 })

@@ -98,6 +98,19 @@ def mmvq_pair_act(wtype: int, gate: torch.Tensor, up: torch.Tensor, q8_1: torch.
     return out
 
 
+def mmvq_pair_act_q8_1(wtype: int, gate: torch.Tensor, up: torch.Tensor, x: torch.Tensor, k: int, n: int, *,
+                       act: str = "silu") -> torch.Tensor:
+    """``Q8_1(act(gate . x) * (up . x))`` as ``[b, n/32, 36]`` bytes; ``x`` is f32 ``[b, k]`` or Q8_1
+    ``[b, k_padded/32, 36]``."""
+    is_f32 = x.dtype == torch.float32
+    b = x.shape[0]
+    out = torch.empty((b, n // 32, 36), dtype=torch.uint8, device=gate.device)
+    _lib.check("lk_mmvq_pair_act_q8_1", _lib.load().lk_mmvq_pair_act_q8_1(
+        wtype, gate.data_ptr(), up.data_ptr(), x.data_ptr(), int(is_f32), x.stride(0) if is_f32 else x.shape[1],
+        out.data_ptr(), n // 32, k, n, b, {"silu": 0, "gelu": 1}[act], _stream()))
+    return out
+
+
 def mmvq_grouped(wtype: int, table: torch.Tensor, q8_1: torch.Tensor, k: int, n: int) -> torch.Tensor:
     """``groups`` same-shape weights (device address table, uint64) each over its own Q8_1 row."""
     groups = table.numel()

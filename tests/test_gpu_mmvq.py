@@ -249,3 +249,29 @@ def test_quantize_in_kernel_path_carries_the_bits_of_the_two_launch_path(name, k
     q = ops.quantize_q8_1_rows(x)
     for w, n, o in zip(ws, ns, fused):
         assert torch.equal(o, ops.mmvq(wtype, w, q, k, n))
+
+
+# ---------------------------------------------------------------- gate/up pair handing on Q8_1
+@pytest.mark.parametrize("name,n,k,b,act", [("q4_k", 64, 512, 1, "silu"), ("q4_k", 14336, 4096, 1, "silu"),
+                                            ("q4_k", 96, 768, 3, "gelu"), ("q6_k", 128, 1024, 2, "silu"),
+                                            ("q8_0", 160, 256, 4, "silu")])
+def test_pair_launch_writes_the_quantizers_q8_1_of_its_own_f32_result(name, n, k, b, act):
+    """The Q8_1 blocks of the pair launch are, byte for byte, what the stand-alone quantizer makes of
+    the f32 result of the same pair launch; and feeding them to a mat-vec equals the two-step path."""
+    wtype = DT[name]
+    gate = dev(synth.weight(wtype, n, k, seed=70, stream=1))
+    up = dev(synth.weight(wtype, n, k, seed=70, stream=2))
+    x = dev(synth.activation(b, k, seed=70))
+    q = ops.quantize_q8_1_rows(x)
+    h = ops.mmvq_pair_act(wtype, gate, up, q, k, n, act=act)
+    want = ops.quantize_q8_1_rows(h, k_padded=n)
+    for src in (x, q):   # f32 rows quantized in the kernel, or Q8_1 rows
+        got = ops.mmvq_pair_act_q8_1(wtype, gate, up, src, k, n, act=act)
+        assert torch.equal(got, want)
+
+
+def test_pair_q8_1_launch_declines_partial_blocks():
+    gate = dev(synth.weight(lib.TYPE_Q4_K, 40, 256, seed=71))
+    x = dev(synth.activation(1, 256, seed=71))
+    with pytest.raises(lib.LokenError):
+        ops.mmvq_pair_act_q8_1(lib.TYPE_Q4_K, gate, gate, x, 256, 40)
