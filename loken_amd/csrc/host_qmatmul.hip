@@ -1,0 +1,226 @@
+// Host mirror of loken's QKernelMatMul for the card path: see include/loken_host.hpp.
+
+#include "../../include/loken_host.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <map>
+#include <mutex>
+
+namespace loken {
+namespace {
+
+constexpr int Q81_BLOCK = 36;
+constexpr size_t MMQ_RECORD = 144;                      // bytes per 128 padded values per row
+constexpr size_t FIXUP_BYTES = 256u * 128u * 128u * 4u;  // kernel_matmul/mmq.rs:42
+
+size_t pad_to(size_t v, size_t m) { return (v + m - 1) / m * m; }
+
+// One device's buffers. `mu` is held across a quantize -> consume pair so that two host threads
+// sharing the card's stream cannot interleave their pairs (fast_mmvq.rs:15-32,
+// kernel_matmul/mmq.rs:43-86); `last_use` orders a later user on ANOTHER stream behind the
+// kernels enqueued here (the host mutex alone orders only the enqueueing).
+struct Slot {
+    std::mutex mu;
+    void* act = nullptr;      // Q8_1 rows / tiled-matmul workspace
+    size_t act_bytes = 0;
+    void* fixup = nullptr;
+    hipEvent_t last_use = nullptr;
+    bool used = false;
+};
+
+std::mutex g_slots_mu;
+std::map<int, Slot*> g_slots;
+
+Slot& slot_of(int device) {
+    std::lock_guard<std::mutex> lock(g_slots_mu);
+    auto it = g_slots.find(device);
+    if (it != g_slots.end()) return *it->second;
+    Slot* s = new Slot();
+    g_slots.emplace(device, s);
+    return *s;
+}
+
+bool capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+
+// Grow-only, zero-filled. Never grows while `stream` records a graph (an allocation is not a
+// capturable operation): the caller warms the size up outside the capture, as with the MoE scratch.
+int reserve(Slot& slot, size_t bytes, bool want_fixup, hipStream_t stream) {
+    const bool rec = capturing(stream);
+    if (slot.act_bytes < bytes) {
+        if (rec) return LK_ERR_NOMEM;
+        if (slot.act) {   // release the smaller one first: no double peak (kernel_matmul/mmq.rs:49-53)
+            if (hipStreamSynchronize(stream) != hipSuccess || hipFree(slot.act) != hipSuccess) (void)hipGetLastError();
+            slot.act = nullptr;
+            slot.act_bytes = 0;
+        }
+        if (hipMalloc(&slot.act, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            slot.act = nullptr;
+            return LK_ERR_NOMEM;
+        }
+        slot.act_bytes = bytes;
+        if (hipMemsetAsync(slot.act, 0, bytes, stream) != hipSuccess) (void)hipGetLastError();
+    }
+    if (want_fixup && !slot.fixup) {
+        if (rec) return LK_ERR_NOMEM;
+        if (hipMalloc(&slot.fixup, FIXUP_BYTES) != hipSuccess) {
+            (void)hipGetLastError();
+            slot.fixup = nullptr;
+            return LK_ERR_NOMEM;
+        }
+        if (hipMemsetAsync(slot.fixup, 0, FIXUP_BYTES, stream) != hipSuccess) (void)hipGetLastError();
+    }
+    if (!slot.last_use && !rec) {
+        if (hipEventCreateWithFlags(&slot.last_use, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            slot.last_use = nullptr;
+        }
+    }
+    // queue behind whoever used the buffers last; a graph being recorded neither waits nor marks
+    if (slot.used && slot.last_use && !rec && hipStreamWaitEvent(stream, slot.last_use, 0) != hipSuccess)
+        (void)hipGetLastError();
+    return LK_OK;
+}
+
+void mark_used(Slot& slot, hipStream_t stream) {
+    if (slot.last_use && !capturing(stream)) {
+        if (hipEventRecord(slot.last_use, stream) != hipSuccess) (void)hipGetLastError();
+        slot.used = true;
+    }
+}
+
+bool tiled_serves(int dtype, int k) {
+    return (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q6_K || dtype == LK_TYPE_Q8_0) && k % 256 == 0;
+}
+
+size_t elem_bytes(int type) { return type == LK_TYPE_F32 ? 4 : 2; }
+
+}  // namespace
+
+int matvec_rows(int dtype, int k) {
+    if (dtype == LK_TYPE_Q4_K && k % 256 == 0) return 6;
+    return tiled_serves(dtype, k) ? 32 : 8;
+}
+
+QKernelMatMul::QKernelMatMul(int dtype, int n, int k, const void* blob, int device)
+    : dtype_(dtype), n_(n), k_(k), device_(device), blob_(blob) {}
+
+int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void* stream_ptr, bool decode_order) {
+    last_path_ = Path::None;
+    hipStream_t stream = (hipStream_t)stream_ptr;
+    if (dtype_ != LK_TYPE_Q4_K && dtype_ != LK_TYPE_Q6_K && dtype_ != LK_TYPE_Q8_0) return LK_ERR_TYPE;
+    if (x_type != LK_TYPE_F32 && x_type != LK_TYPE_F16 && x_type != LK_TYPE_BF16) return LK_ERR_TYPE;
+    if (rows == 0) return LK_OK;
+    if (!x || !out || !blob_ || rows < 0 || n_ <= 0 || k_ <= 0) return LK_ERR_ARG;
+    const int block_len = dtype_ == LK_TYPE_Q8_0 ? 32 : 256;
+    if (k_ % block_len != 0) return LK_ERR_ARG;
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess || current != device_) {
+        (void)hipGetLastError();
+        return LK_ERR_ARG;   // "input on a different device" (kernel_matmul.rs:1499-1503)
+    }
+    const int mv_max = matvec_rows(dtype_, k_);
+    Slot& slot = slot_of(device_);
+
+    // --- mat-vec family: up to matvec_rows, or any count when every row must sum like a one-row call
+    if (rows <= mv_max || decode_order) {
+        if (x_type == LK_TYPE_F32 && rows <= 2 && k_ <= 8192 && ((uintptr_t)x & 15) == 0 && k_ % 4 == 0) {
+            const void* vx[1] = {blob_};
+            void* dst[1] = {out};
+            const int nn[1] = {n_};
+            last_path_ = Path::MatVecFused;
+            return lk_mmvq_fused(dtype_, 1, vx, (const float*)x, k_, dst, x_type, k_, nn, rows, n_, nullptr, stream);
+        }
+        const int k_padded = (int)pad_to((size_t)k_, 512), blocks = k_padded / 32;
+        std::lock_guard<std::mutex> pair(slot.mu);
+        if (int rc = reserve(slot, (size_t)rows * blocks * Q81_BLOCK, false, stream)) return rc;
+        if (int rc = lk_quantize_q8_1(x, x_type, slot.act, k_, k_padded, rows, stream)) return rc;
+        for (int r0 = 0; r0 < rows; r0 += 8) {
+            const int b = rows - r0 < 8 ? rows - r0 : 8;
+            const int rc = lk_mmvq(dtype_, blob_, (const uint8_t*)slot.act + (size_t)r0 * blocks * Q81_BLOCK,
+                                   (uint8_t*)out + (size_t)r0 * n_ * elem_bytes(x_type), x_type, k_, n_, b, blocks, n_,
+                                   nullptr, decode_order ? 1 : 0, stream);
+            if (rc) return rc;
+        }
+        mark_used(slot, stream);
+        last_path_ = Path::MatVec;
+        return LK_OK;
+    }
+    if (x_type != LK_TYPE_F32) return LK_ERR_TYPE;   // the matrix-unit kernels write f32
+
+    // --- Q4_K, a handful of rows: matrix unit, weights straight from HBM
+    if (dtype_ == LK_TYPE_Q4_K && rows <= 64 && ((uintptr_t)blob_ & 15) == 0) {
+        const int blocks = k_ / 32;
+        std::lock_guard<std::mutex> pair(slot.mu);
+        if (int rc = reserve(slot, (size_t)rows * blocks * Q81_BLOCK, false, stream)) return rc;
+        if (int rc = lk_quantize_q8_1(x, x_type, slot.act, k_, k_, rows, stream)) return rc;
+        loken_dense_q4k_imma_m8_plain(blob_, slot.act, (float*)out, rows, n_, k_, stream);
+        mark_used(slot, stream);
+        last_path_ = Path::RowsOnMatrixUnit;
+        return LK_OK;
+    }
+
+    // --- tiled matmul (mmq_forward, kernel_matmul/mmq.rs:21-159)
+    if (!tiled_serves(dtype_, k_)) return LK_ERR_TYPE;
+    const size_t k_padded = pad_to(pad_to((size_t)k_, 512), 128);
+    const size_t ws_bytes = (size_t)rows * (k_padded / 128) * MMQ_RECORD + 128 * MMQ_RECORD;
+    std::lock_guard<std::mutex> pair(slot.mu);
+    if (int rc = reserve(slot, ws_bytes, true, stream)) return rc;
+    auto quantizer = dtype_ == LK_TYPE_Q4_K ? launch_mmq_quantize_q8_1_DS4 : launch_mmq_quantize_q8_1_D4;
+    quantizer(x, nullptr, slot.act, 0, k_, k_, 0, 0, (int64_t)k_padded, rows, 1, 1, stream);
+    auto launcher = dtype_ == LK_TYPE_Q4_K ? launch_mmq_gguf_q4_k : dtype_ == LK_TYPE_Q6_K ? launch_mmq_gguf_q6_k : launch_mmq_gguf_q8_0;
+    int abi = 0, cus = 0, lds = 0, wave = 0;
+    (void)lk_device_info(&abi, &cus, &lds, &wave);
+    const int tile = launcher(slot.fixup, blob_, slot.act, out, k_, n_, rows, k_ / block_len, n_, 0x1000950, cus, lds, wave,
+                              stream);
+    mark_used(slot, stream);
+    if (tile == 0) return LK_ERR_ARG;   // "no tile fits, nothing ran": the reference falls back to dequantized
+    last_path_ = Path::Tiled;
+    return LK_OK;
+}
+
+void release_workspaces() {
+    std::lock_guard<std::mutex> lock(g_slots_mu);
+    int current = 0;
+    (void)hipGetDevice(&current);
+    for (auto& kv : g_slots) {
+        Slot& s = *kv.second;
+        std::lock_guard<std::mutex> pair(s.mu);
+        if (hipSetDevice(kv.first) != hipSuccess) { (void)hipGetLastError(); continue; }
+        (void)hipDeviceSynchronize();
+        if (s.act) (void)hipFree(s.act);
+        if (s.fixup) (void)hipFree(s.fixup);
+        if (s.last_use) (void)hipEventDestroy(s.last_use);
+        s.act = s.fixup = nullptr;
+        s.act_bytes = 0;
+        s.last_use = nullptr;
+        s.used = false;
+    }
+    (void)hipSetDevice(current);
+    (void)hipGetLastError();
+}
+
+}  // namespace loken
+
+extern "C" void* lkh_qkernel_matmul_new(int dtype, int n, int k, const void* blob, int device) {
+    return new loken::QKernelMatMul(dtype, n, k, blob, device);
+}
+extern "C" void lkh_qkernel_matmul_free(void* handle) { delete (loken::QKernelMatMul*)handle; }
+extern "C" int lkh_qkernel_matmul_forward(void* handle, const void* x, int x_type, int rows, void* out, void* stream,
+                                          int decode_order) {
+    if (!handle) return LK_ERR_ARG;
+    return ((loken::QKernelMatMul*)handle)->forward(x, x_type, rows, out, stream, decode_order != 0);
+}
+extern "C" int lkh_qkernel_matmul_last_path(void* handle) {
+    return handle ? (int)((loken::QKernelMatMul*)handle)->last_path() : 0;
+}
+extern "C" int lkh_matvec_rows(int dtype, int k) { return loken::matvec_rows(dtype, k); }
+extern "C" void lkh_release_workspaces(void) { loken::release_workspaces(); }

@@ -55,6 +55,12 @@ SIGNATURES.update({
     "loken_moe_sum_topk": (None, [_vp, _vp, _i, _i, _i, _vp]),
     "loken_stream_scratch_release": (None, []),
     "lk_mmvq_pair_act_q8_1": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i, _i, _vp]),
+    "lkh_qkernel_matmul_new": (_vp, [_i, _i, _i, _vp, _i]),
+    "lkh_qkernel_matmul_free": (None, [_vp]),
+    "lkh_qkernel_matmul_forward": (_i, [_vp, _vp, _i, _i, _vp, _vp, _i]),
+    "lkh_qkernel_matmul_last_path": (_i, [_vp]),
+    "lkh_matvec_rows": (_i, [_i, _i]),
+    "lkh_release_workspaces": (None, []),
     "loken_dense_q4k_imma_m8_plain": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "loken_moe_mmq_fold": (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
 })

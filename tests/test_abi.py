@@ -8,9 +8,12 @@ ROOT = Path(__file__).resolve().parent.parent
 
 
 def declared_symbols():
+    """Every function of the C ABI header, and the `extern "C"` part of the C++ host header."""
     text = (ROOT / "include" / "loken_gfx950.h").read_text()
+    host = (ROOT / "include" / "loken_host.hpp").read_text()
+    text += host[host.index('extern "C" {'):]
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(?:int|void)\s+(\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(?:int|void\s*\*?)\s*(\w+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():

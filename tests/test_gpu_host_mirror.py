@@ -1,0 +1,141 @@
+"""The C++ host mirror of QKernelMatMul (include/loken_host.hpp) through its C symbols: path chosen
+by row count, results equal to the launchers called one by one, workspace rules."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+import oracle
+from loken_amd import lib, ops, synth
+
+pytestmark = pytest.mark.gpu
+
+DT = {"q4_k": lib.TYPE_Q4_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0}
+PATH = {1: "matvec-fused", 2: "matvec", 3: "rows-on-matrix-unit", 4: "tiled"}
+X_TYPES = {torch.float32: lib.TYPE_F32, torch.float16: lib.TYPE_F16, torch.bfloat16: lib.TYPE_BF16}
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+class Linear:
+    def __init__(self, wtype, w, n, k):
+        self.l = lib.load()
+        self.w = w   # keeps the blob alive
+        self.n, self.k = n, k
+        self.h = self.l.lkh_qkernel_matmul_new(wtype, n, k, w.data_ptr(), torch.cuda.current_device())
+
+    def __call__(self, x, decode_order=False, stream=None):
+        out = torch.empty((x.shape[0], self.n), dtype=x.dtype, device=x.device)
+        s = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+        rc = self.l.lkh_qkernel_matmul_forward(self.h, x.data_ptr(), X_TYPES[x.dtype], x.shape[0], out.data_ptr(), s,
+                                               int(decode_order))
+        if rc:
+            raise lib.LokenError("lkh_qkernel_matmul_forward", rc)
+        return out
+
+    @property
+    def path(self):
+        return PATH.get(self.l.lkh_qkernel_matmul_last_path(self.h), "none")
+
+    def close(self):
+        self.l.lkh_qkernel_matmul_free(self.h)
+
+
+def close(got, want, rtol=1e-3, atol=1e-4):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    return bool((np.abs(got - want) <= rtol * np.abs(want) + atol).all())
+
+
+@pytest.mark.parametrize("name,rows,expect", [
+    ("q4_k", 1, "matvec-fused"), ("q4_k", 2, "matvec-fused"), ("q4_k", 5, "matvec"), ("q4_k", 7, "rows-on-matrix-unit"),
+    ("q4_k", 40, "rows-on-matrix-unit"), ("q4_k", 80, "tiled"), ("q6_k", 1, "matvec-fused"), ("q6_k", 20, "matvec"),
+    ("q6_k", 40, "tiled"), ("q8_0", 3, "matvec"), ("q8_0", 33, "tiled")])
+def test_forward_takes_the_path_of_its_row_count_and_matches_the_oracle(name, rows, expect):
+    wtype, n, k = DT[name], 200, 1024
+    w = synth.weight(wtype, n, k, seed=80, stream=1)
+    x = synth.activation(rows, k, seed=80)
+    lin = Linear(wtype, dev(w), n, k)
+    try:
+        got = lin(dev(x))
+        assert lin.path == expect
+        assert close(got.cpu().numpy(), oracle.ob_matmul(wtype, x, w, n))
+    finally:
+        lin.close()
+
+
+def test_decode_order_keeps_every_row_on_the_matvec_family_and_rows_independent():
+    wtype, n, k = lib.TYPE_Q4_K, 300, 2048
+    w = dev(synth.weight(wtype, n, k, seed=81, stream=1))
+    x = dev(synth.activation(20, k, seed=81))
+    lin = Linear(wtype, w, n, k)
+    try:
+        batch = lin(x, decode_order=True)
+        assert lin.path == "matvec"
+        q = ops.quantize_q8_1_rows(x)
+        for r in (0, 7, 8, 19):
+            assert torch.equal(batch[r:r + 1], ops.mmvq(wtype, w, q[r:r + 1], k, n))
+    finally:
+        lin.close()
+
+
+def test_half_inputs_stay_in_their_type_on_the_matvec_family_and_are_declined_above_it():
+    wtype, n, k = lib.TYPE_Q6_K, 64, 512
+    w = dev(synth.weight(wtype, n, k, seed=82, stream=1))
+    lin = Linear(wtype, w, n, k)
+    try:
+        x = dev(synth.activation(3, k, seed=82)).to(torch.bfloat16)
+        y = lin(x)
+        assert y.dtype == torch.bfloat16 and lin.path == "matvec"
+        want = ops.mmvq(wtype, w, ops.quantize_q8_1_rows(x), k, n, out_dtype=torch.bfloat16)
+        assert torch.equal(y, want)
+        with pytest.raises(lib.LokenError):
+            lin(dev(synth.activation(50, k, seed=82)).to(torch.float16))
+    finally:
+        lin.close()
+
+
+def test_workspace_grows_outside_a_capture_only_and_replays_then():
+    wtype, n, k = lib.TYPE_Q4_K, 128, 1024
+    w = dev(synth.weight(wtype, n, k, seed=83, stream=1))
+    lin = Linear(wtype, w, n, k)
+    lib.load().lkh_release_workspaces()
+    try:
+        x = dev(synth.activation(12, k, seed=83))
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with pytest.raises(lib.LokenError) as err:      # nothing reserved yet: refused while recording
+                with torch.cuda.graph(graph, stream=side):
+                    lin(x, stream=side.cuda_stream)
+            assert "LK_ERR_NOMEM" in str(err.value)
+        torch.cuda.synchronize()
+        eager = lin(x)                                       # reserves the workspace
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        out = torch.empty((12, n), device="cuda")
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                rc = lib.load().lkh_qkernel_matmul_forward(lin.h, x.data_ptr(), lib.TYPE_F32, 12, out.data_ptr(),
+                                                           side.cuda_stream, 0)
+                assert rc == 0
+        for _ in range(3):
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+    finally:
+        lin.close()
+
+
+def test_argument_errors_are_status_codes():
+    l = lib.load()
+    assert l.lkh_matvec_rows(lib.TYPE_Q4_K, 4096) == 6 and l.lkh_matvec_rows(lib.TYPE_Q6_K, 4096) == 32
+    h = l.lkh_qkernel_matmul_new(99, 8, 256, 16, 0)
+    assert l.lkh_qkernel_matmul_forward(h, 16, lib.TYPE_F32, 1, 16, None, 0) == lib.LK_ERR_TYPE
+    l.lkh_qkernel_matmul_free(h)
+    h = l.lkh_qkernel_matmul_new(lib.TYPE_Q4_K, 8, 250, 16, 0)
+    assert l.lkh_qkernel_matmul_forward(h, 16, lib.TYPE_F32, 1, 16, None, 0) == lib.LK_ERR_ARG
+    assert l.lkh_qkernel_matmul_forward(h, 16, lib.TYPE_F32, 0, 16, None, 0) == lib.LK_OK
+    l.lkh_qkernel_matmul_free(h)
