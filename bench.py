@@ -69,6 +69,8 @@ def parse_args():
                          "workloads of loken_amd/workloads.py, one JSON line each")
     ap.add_argument("--shape", choices=["2a", "2b"], default="2a", help="--workload mmq: 512x4096->14336 Q4_K or 2048x14336->4096 Q6_K")
     ap.add_argument("--tokens", type=int, default=256, help="--workload moe: rows through the expert block")
+    ap.add_argument("--moe-path", choices=["auto", "tiled", "pairs"], default="auto",
+                    help="--workload moe: expert-batched tiled matmul, mat-vec per routed pair, or the library's choice")
     ap.add_argument("--mid-rows", choices=["matvec", "tiled"], default="matvec",
                     help="--workload decode-1p7b, 9..32 rows: Q6_K linears as mat-vec launches over slices of eight "
                          "rows, or through the tiled matmul")

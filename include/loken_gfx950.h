@@ -279,6 +279,14 @@ void loken_moe_sum_topk(const float* pairs, float* outputs, int tokens, int topk
  * 256; weights 16-byte aligned; nothing is launched on a bad argument (void, as the reference's). */
 void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
                                    int size_k, void* stream);
+/* The router step in front of the expert block: softmax over each row of logits [n_rows,
+ * n_experts], the n_expert_used largest probabilities in descending order (ties to the lower
+ * expert id) into weights / ids [n_rows, n_expert_used], divided by their sum when with_norm != 0.
+ * Name and arguments of the reference's launcher (cuda/moe/gate_topk.cu:405-451; topk_softmax,
+ * src/inference/moe_cuda_cpu/mod.rs:2098-2113). Up to 512 experts, up to 64 used; nothing is
+ * launched outside that (the caller falls back). */
+void loken_topk_softmax(const float* logits, float* weights, uint32_t* ids, int n_rows, int n_experts,
+                        int n_expert_used, int with_norm, void* stream);
 /* Frees the current device's MoE decode scratch (cuda/moe/moe_gguf.cu:104-118). Synchronizes. */
 void loken_stream_scratch_release(void);
 

@@ -61,6 +61,7 @@ SIGNATURES.update({
     "lkh_qkernel_matmul_last_path": (_i, [_vp]),
     "lkh_matvec_rows": (_i, [_i, _i]),
     "lkh_release_workspaces": (None, []),
+    "loken_topk_softmax": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "loken_dense_q4k_imma_m8_plain": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "loken_moe_mmq_fold": (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
 })

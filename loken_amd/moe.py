@@ -187,6 +187,21 @@ def moe_gemm_gguf(wtype: int, x: torch.Tensor, weights: torch.Tensor, routing: E
     return out
 
 
+def topk_softmax(logits: torch.Tensor, topk: int, renorm: bool = True):
+    """Router: ``[tokens, experts]`` f32 logits -> (weights f32 ``[tokens, topk]``, choices int32
+    ``[tokens, topk]``), probabilities descending, ties to the lower expert id (topk_softmax,
+    src/inference/moe_cuda_cpu/mod.rs:2098-2113)."""
+    tokens, experts = logits.shape
+    if experts > 512 or topk > 64 or topk > experts:
+        raise ValueError("topk_softmax: at most 512 experts and 64 choices")
+    logits = logits.to(torch.float32).contiguous()
+    weights = torch.empty((tokens, topk), dtype=torch.float32, device=logits.device)
+    ids = torch.empty((tokens, topk), dtype=torch.int32, device=logits.device)
+    _lib.load().loken_topk_softmax(logits.data_ptr(), weights.data_ptr(), ids.data_ptr(), tokens, experts, topk,
+                                   int(renorm), _stream())
+    return weights, ids
+
+
 def moe_mmq_pays(rows: int, experts: int) -> bool:
     """Routed rows from which the expert-batched matmul beats the per-pair kernels
     (mmq_experts.rs:72-86: break-even at one routed row per expert)."""

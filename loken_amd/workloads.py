@@ -281,7 +281,7 @@ def moe_block(args, dev):
     choices = choices.to(torch.int32).contiguous()
 
     pairs = tokens * topk
-    tiled = moe.moe_mmq_pays(pairs, experts)
+    tiled = moe.moe_mmq_pays(pairs, experts) if args.moe_path == "auto" else args.moe_path == "tiled"
     # The routing (the router's side of the boundary) is built once; the timed block is what the
     # expert launchers do with it, recorded into a graph so that the host's cost stays outside.
     flat_w = weights.reshape(-1)

@@ -12,7 +12,7 @@ import pytest
 torch = pytest.importorskip("torch")
 
 import oracle
-from loken_amd import lib, synth
+from loken_amd import lib, moe, synth
 from loken_amd.moe import MmqRouting
 
 pytestmark = pytest.mark.gpu
@@ -289,3 +289,24 @@ def test_layer_entry_picks_a_path_and_both_agree(tokens):
     want = oracle.moe_forward(1, lib.TYPE_Q4_K, lib.TYPE_Q4_K, x, gate, up, down, ids, w, n_experts, ffn)
     scale = np.abs(want).max()
     assert (np.abs(got - want) <= 2e-3 * np.abs(want) + 2e-4 * scale).all()
+
+
+# ---------------------------------------------------------------- router
+@pytest.mark.parametrize("tokens,experts,topk,renorm", [(1, 128, 8, True), (16, 128, 8, True), (256, 128, 8, False),
+                                                        (7, 60, 4, True), (5, 512, 64, True), (3, 8, 8, False)])
+def test_router_topk_softmax_matches_oracle(tokens, experts, topk, renorm):
+    logits = synth.normal(90, tokens * 1000 + experts, tokens * experts).astype(np.float32).reshape(tokens, experts)
+    want_ids, want_w = oracle.topk_softmax(logits, topk, renorm)
+    w, ids = moe.topk_softmax(dev(logits), topk, renorm)
+    assert np.array_equal(ids.cpu().numpy(), want_ids)
+    assert np.allclose(w.cpu().numpy(), want_w, rtol=1e-5, atol=1e-7)
+
+
+def test_router_ties_go_to_the_lower_expert_and_weights_descend():
+    logits = np.zeros((2, 128), np.float32)
+    logits[1, [5, 40, 41, 100]] = [2.0, 3.0, 3.0, 2.0]
+    w, ids = moe.topk_softmax(dev(logits), 8, True)
+    ids, w = ids.cpu().numpy(), w.cpu().numpy()
+    assert ids[0].tolist() == list(range(8)) and np.allclose(w[0], 1.0 / 8)
+    assert ids[1, :4].tolist() == [40, 41, 5, 100] and ids[1, 4:].tolist() == [0, 1, 2, 3]
+    assert (np.diff(w[1]) <= 0).all() and abs(w[1].sum() - 1.0) < 1e-6
