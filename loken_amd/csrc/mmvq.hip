@@ -323,7 +323,7 @@ static int launch_plain_r(MmvqCall& a) {
     const int capacity = lk_device().cus * per_cu;
     int need[MAX_MULTI], total = 0;
     for (int i = 0; i < a.m.count; ++i) {
-        need[i] = wgs_for_rows(a.m.n[i], R);
+        need[i] = wgs_for_rows(a.m.n[i], R * E::rows_per_pass(a.nb));
         total += need[i];
     }
     a.m.wg_begin[0] = 0;
@@ -366,7 +366,9 @@ static int launch_plain(MmvqCall& a) {
 template <typename T>
 static int dispatch_plain(int wtype, int batch, MmvqCall& a) {
     switch (wtype) {
-        case LK_TYPE_Q4_K: LK_BATCH_SWITCH(launch_plain, EngQ4K, T, a)
+        case LK_TYPE_Q4_K:
+            if (a.nb <= 8) { LK_BATCH_SWITCH(launch_plain, EngQ4KShort, T, a) }
+            LK_BATCH_SWITCH(launch_plain, EngQ4K, T, a)
         case LK_TYPE_Q6_K: LK_BATCH_SWITCH(launch_plain, EngQ6K, T, a)
         case LK_TYPE_Q8_0: LK_BATCH_SWITCH(launch_plain, EngQ80, T, a)
         default: return LK_ERR_TYPE;
@@ -446,7 +448,7 @@ static int launch_pair(const uint8_t* gate, const uint8_t* up, const uint8_t* vy
     auto launch = [&](auto kernel) {
         const int per_cu = resident_per_cu(kernel, lds_bytes);
         if (per_cu == 0) return (int)LK_ERR_ARG;
-        const int need = wgs_for_rows(n, R), cap = lk_device().cus * per_cu;
+        const int need = wgs_for_rows(n, R * E::rows_per_pass(nb)), cap = lk_device().cus * per_cu;
         hipLaunchKernelGGL(kernel, dim3(need < cap ? need : cap), dim3(WG), lds_bytes, s, gate, up, vy, (T*)dst, nb, n,
                            stride_col_y, stride_col_dst);
         return lk_launch_status();
@@ -478,7 +480,7 @@ static int launch_grouped(const uint64_t* table, int groups, const uint8_t* vy, 
     const int lds_bytes = lds_bytes_for<typename E::Fmt>(nb, 1);
     const int per_cu = resident_per_cu(kernel, lds_bytes);
     if (per_cu == 0) return LK_ERR_ARG;
-    const int need = wgs_for_rows(n, R);
+    const int need = wgs_for_rows(n, R * E::rows_per_pass(nb));
     int cap = lk_device().cus * per_cu / groups;
     if (cap < 1) cap = 1;
     hipLaunchKernelGGL(kernel, dim3(need < cap ? need : cap, groups), dim3(WG), lds_bytes, s, table, vy, dst, nb, n, k32);
@@ -552,7 +554,9 @@ extern "C" int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, con
         default: return LK_ERR_TYPE;                             \
     }
     switch (wtype) {
-        case LK_TYPE_Q4_K: LK_PAIR_TYPE(EngQ4K)
+        case LK_TYPE_Q4_K:
+            if (nb <= 8) { LK_PAIR_TYPE(EngQ4KShort) }
+            LK_PAIR_TYPE(EngQ4K)
         case LK_TYPE_Q6_K: LK_PAIR_TYPE(EngQ6K)
         case LK_TYPE_Q8_0: LK_PAIR_TYPE(EngQ80)
         default: return LK_ERR_TYPE;
@@ -604,7 +608,9 @@ extern "C" int lk_mmvq_grouped(int wtype, const uint64_t* table, int groups, con
     hipStream_t s = (hipStream_t)stream;
     const uint8_t* y = (const uint8_t*)vy_q8_1;
     switch (wtype) {
-        case LK_TYPE_Q4_K: return launch_grouped<EngQ4K>(table, groups, y, dst, nb, nrows_x, k32, s);
+        case LK_TYPE_Q4_K:
+            return nb <= 8 ? launch_grouped<EngQ4KShort>(table, groups, y, dst, nb, nrows_x, k32, s)
+                           : launch_grouped<EngQ4K>(table, groups, y, dst, nb, nrows_x, k32, s);
         case LK_TYPE_Q6_K: return launch_grouped<EngQ6K>(table, groups, y, dst, nb, nrows_x, k32, s);
         default: return launch_grouped<EngQ80>(table, groups, y, dst, nb, nrows_x, k32, s);
     }

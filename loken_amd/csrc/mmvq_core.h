@@ -396,38 +396,64 @@ static __device__ __forceinline__ void stage_around(uint8_t* lds, const RowJob<N
 // per wave pass, loads of the next step in flight while the current one is consumed.
 // epi(row, col, totals[NW]) runs on lane 0 for every finished (row, activation row).
 // ---------------------------------------------------------------------------------------------
+// Short rows: a pass has 16 super-block slots of 4 lanes; a row of at most 8 (4) super-blocks
+// would leave half (three quarters) of the lanes idle, so 2 (4) rows share a pass, each in its
+// own 32 (16) lanes. The MoE expert matrices (k = 2048, 768) and small dense models live here.
+static __host__ __device__ __forceinline__ int q4k_rows_per_pass(int nb) { return nb <= 4 ? 4 : nb <= 8 ? 2 : 1; }
+
+// Totals of the four rows of 16 lanes, every lane returns all four.
+static __device__ __forceinline__ void row16_sums(float v, float (&q)[4]) {
+    v += dpp_f32<0xB1>(v);
+    v += dpp_f32<0x4E>(v);
+    v += dpp_f32<0x141>(v);
+    v += dpp_f32<0x140>(v);
+    const int bits = __float_as_int(v);
+    q[0] = __int_as_float(__builtin_amdgcn_readlane(bits, 0));
+    q[1] = __int_as_float(__builtin_amdgcn_readlane(bits, 16));
+    q[2] = __int_as_float(__builtin_amdgcn_readlane(bits, 32));
+    q[3] = __int_as_float(__builtin_amdgcn_readlane(bits, 48));
+}
+
 // done(tile) runs on every lane of the wave once the tile's rows have been handed to epi.
-template <int B, int R, int NW, class Epi, class Done>
+// PACK false: one row per pass, all of this a compile-time 1 / 16 (the long-row kernels pay
+// nothing for the short-row form); PACK true: rows per pass from the row length.
+template <int B, int R, int NW, bool PACK, class Epi, class Done>
 static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* lds, Epi&& epi, Done&& done) {
     const int nb = job.nb, n = job.n;
-    const int n_iter = (nb + 15) >> 4;
-    const int row_bytes = lds_bytes_per_row<FmtQ4K>(n_iter);
+    const int n_iter_lds = (nb + 15) >> 4;   // passes of the staged activation (its layout)
+    const int row_bytes = lds_bytes_per_row<FmtQ4K>(n_iter_lds);
+    // rows side by side in a pass (tile runs keep the plain form)
+    const int RP = (!PACK || job.run_len > 1) ? 1 : q4k_rows_per_pass(nb);
+    const int S = PACK ? 16 / RP : 16;       // super-block slots of one row in a pass
+    const int n_iter = (nb + S - 1) / S;     // passes per tile (1 whenever RP > 1)
+    const int TR = R * RP;                   // rows per tile
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lb = lane >> 2, p = lane & 3;
+    const int slot = lb & (S - 1), rp = lb / S;
     const Q4KScaleSel sel(p);
-    const uint32_t hdr_off = lb * Q4K_BYTES, qs_off = hdr_off + 16 + 32 * p;
+    const uint32_t hdr_off = slot * Q4K_BYTES, qs_off = hdr_off + 16 + 32 * p;
     const size_t row_stride = (size_t)nb * Q4K_BYTES;
-    const int n_tiles = (n + R - 1) / R;
+    const int n_tiles = (n + TR - 1) / TR;
     constexpr int RW = R * NW;
 
     struct Frag {
         uint4 hdr[RW], q0[RW], q1[RW];
     };
-    // One pass (16 super-blocks) of R rows of every matrix into registers. A lane past the row
-    // end re-reads the row's last block and drops its d / dmin when it consumes it, so it adds
-    // nothing (the loaded registers themselves are left alone: touching them here would make
-    // the wave wait for the load).
+    // One pass (16 super-block slots) of R rows per lane group of every matrix into registers. A
+    // lane past the row end re-reads the row's last block and drops its d / dmin when it consumes
+    // it, so it adds nothing (the loaded registers themselves are left alone: touching them here
+    // would make the wave wait for the load).
     auto load = [&](Frag& f, int tile, int it) {
-        const bool valid = it * 16 + lb < nb;
-        const uint32_t back = valid ? 0u : (uint32_t)(it * 16 + lb - (nb - 1)) * Q4K_BYTES;
+        const bool valid = it * S + slot < nb;
+        const uint32_t back = valid ? 0u : (uint32_t)(it * S + slot - (nb - 1)) * Q4K_BYTES;
 #pragma unroll
         for (int w = 0; w < NW; ++w)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const int row = min(tile * R + r, n - 1);
-                const uint8_t* bp = (const uint8_t*)(job.vx[w] + row * row_stride + (size_t)it * (16 * Q4K_BYTES));
+                const int row = min(tile * TR + rp * R + r, n - 1);
+                const uint8_t* bp = (const uint8_t*)(job.vx[w] + row * row_stride + (size_t)it * (S * Q4K_BYTES));
                 Frag& g = f;
                 g.hdr[w * R + r] = *(const uint4*)(bp + (hdr_off - back));
                 g.q0[w * R + r] = *(const uint4*)(bp + (qs_off - back));
@@ -442,12 +468,13 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
         for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
 
     auto compute = [&](const Frag& f, int tile, int it) {
+        const int block = it * S + slot;   // the lane's super-block of its row
         float d[RW], dmin[RW], scl[RW], sch[RW], ml[RW], mh[RW];
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
             uint32_t sc, mn;
             sel.unpack(f.hdr[r].y, f.hdr[r].z, f.hdr[r].w, sc, mn);
-            const uint32_t dd = it * 16 + lb < nb ? f.hdr[r].x : 0u;
+            const uint32_t dd = block < nb ? f.hdr[r].x : 0u;
             d[r] = f16_bits_to_f32(dd & 0xFFFFu);
             dmin[r] = f16_bits_to_f32(dd >> 16);
             scl[r] = (float)(sc & 0xFFu);
@@ -458,12 +485,12 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
 #pragma unroll
         for (int c = 0; c < B; ++c) {
             const uint8_t* rowl = lds + c * row_bytes;
-            const uint8_t* codes = rowl + it * 4096 + lane * 16;
+            const uint8_t* codes = rowl + (block >> 4) * 4096 + ((block & 15) * 4 + p) * 16;
             const uint4 a00 = *(const uint4*)(codes);
             const uint4 a01 = *(const uint4*)(codes + 1024);
             const uint4 a10 = *(const uint4*)(codes + 2048);
             const uint4 a11 = *(const uint4*)(codes + 3072);
-            const float4 s4 = *(const float4*)(rowl + n_iter * 4096 + (size_t)((it * 16 + lb) * 8 + 2 * p) * 8);
+            const float4 s4 = *(const float4*)(rowl + n_iter_lds * 4096 + (size_t)(block * 8 + 2 * p) * 8);
 #pragma unroll
             for (int r = 0; r < RW; ++r) {
                 int d_lo = 0, d_hi = 0;
@@ -479,13 +506,35 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int c = 0; c < B; ++c) {
-                    float tot[NW];
+                    float q[NW][4];
 #pragma unroll
                     for (int w = 0; w < NW; ++w) {
-                        tot[w] = wave_sum(acc[w * R + r][c]);
+                        row16_sums(acc[w * R + r][c], q[w]);
                         acc[w * R + r][c] = 0.f;
                     }
-                    if (lane == 0 && tile * R + r < n) epi(tile * R + r, c, tot);
+                    if (lane == 0) {
+                        float tot[NW];
+                        const int row0 = tile * TR + r;
+                        if (RP == 1) {
+#pragma unroll
+                            for (int w = 0; w < NW; ++w) tot[w] = (q[w][0] + q[w][1]) + (q[w][2] + q[w][3]);
+                            if (row0 < n) epi(row0, c, tot);
+                        } else if (RP == 2) {
+#pragma unroll
+                            for (int g = 0; g < 2; ++g) {
+#pragma unroll
+                                for (int w = 0; w < NW; ++w) tot[w] = q[w][2 * g] + q[w][2 * g + 1];
+                                if (row0 + g * R < n) epi(row0 + g * R, c, tot);
+                            }
+                        } else {
+#pragma unroll
+                            for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                                for (int w = 0; w < NW; ++w) tot[w] = q[w][g];
+                                if (row0 + g * R < n) epi(row0 + g * R, c, tot);
+                            }
+                        }
+                    }
                 }
             done(tile);
         }
@@ -497,7 +546,7 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
     Frag fa, fb;
     // (a wave without a tile loads the last one rather than nothing: a load under a branch would
     // blur the count of loads ahead of the weights and the staging would wait for some of them)
-    stage_around<FmtQ4K, B>(lds, job, nb * 8, n_iter, [&] { load(fa, min(tile, n_tiles - 1), 0); });
+    stage_around<FmtQ4K, B>(lds, job, nb * 8, n_iter_lds, [&] { load(fa, min(tile, n_tiles - 1), 0); });
     __syncthreads();
     if (tile >= n_tiles) return;
     // Steps are (tile, pass) pairs in order; the loads of step i+1 are issued before step i is
@@ -732,13 +781,24 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
 // Format tags: which engine serves a ggml type, and its LDS footprint.
 struct EngQ4K {
     using Fmt = FmtQ4K;
+    static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
-        rows_q4k<B, R, NW>(j, lds, e, d);
+        rows_q4k<B, R, NW, false>(j, lds, e, d);
+    }
+};
+// Q4_K rows of at most 8 super-blocks (k <= 2048): 2 or 4 rows share a pass.
+struct EngQ4KShort {
+    using Fmt = FmtQ4K;
+    static __host__ __device__ int rows_per_pass(int nb) { return q4k_rows_per_pass(nb); }
+    template <int B, int R, int NW, class Epi, class Done = NoTileHook>
+    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
+        rows_q4k<B, R, NW, true>(j, lds, e, d);
     }
 };
 struct EngQ6K {
     using Fmt = FmtQ6K;
+    static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
         rows_q6k<B, R, NW>(j, lds, e, d);
@@ -746,6 +806,7 @@ struct EngQ6K {
 };
 struct EngQ80 {
     using Fmt = FmtQ80;
+    static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
         rows_q80<B, R, NW>(j, lds, e, d);

@@ -162,7 +162,8 @@ static int launch_mode(const uint8_t* w0, const uint8_t* w1, const uint8_t* acts
     const int lds_bytes = lds_bytes_for<typename E::Fmt>(d.nb, 1);
     const int per_cu = prepare(kernel, lds_bytes);
     if (per_cu == 0) return LK_ERR_ARG;
-    const int tiles = (d.cols + R - 1) / R;
+    const int tile_rows = R * E::rows_per_pass(d.nb);
+    const int tiles = (d.cols + tile_rows - 1) / tile_rows;
     const int need = (tiles + WAVES - 1) / WAVES;
     int share = lk_device().cus * per_cu / d.pairs;
     if (share < 1) share = 1;
@@ -182,7 +183,8 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
             return launch_mode<EngQ80, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 1:
             d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q4K_BYTES;
-            return launch_mode<EngQ4K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
+            return d.nb <= 8 ? launch_mode<EngQ4KShort, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s)
+                             : launch_mode<EngQ4K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 5:
             d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q6K_BYTES;
             return launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);

@@ -203,9 +203,11 @@ def topk_softmax(logits: torch.Tensor, topk: int, renorm: bool = True):
 
 
 def moe_mmq_pays(rows: int, experts: int) -> bool:
-    """Routed rows from which the expert-batched matmul beats the per-pair kernels
-    (mmq_experts.rs:72-86: break-even at one routed row per expert)."""
-    return rows >= max(experts, 1)
+    """Routed rows from which the expert-batched matmul beats the per-pair kernels. The reference
+    breaks even at one routed row per expert (mmq_experts.rs:72-86); on MI355X, with this
+    library's kernels, the mat-vec per routed pair stays ahead up to three rows per expert
+    (Qwen3-30B-A3B shapes: 117 us against 162 us at 32 tokens, 176 against 168 at 48)."""
+    return rows >= 3 * max(experts, 1)
 
 
 def moe_forward(wtype_gu: int, wtype_down: int, x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
