@@ -42,7 +42,7 @@ HBM_PEAK_GBS = 8000.0
 # profiles/mmvq_llama3_8b_decode_b1_hbm_traffic.md. Counters cannot be read from inside this
 # process, so the figure is carried here for the configuration it was taken on:
 # (launch plan, batch, layers) -> bytes.
-MEASURED_TRAFFIC = {("auto", 1, 32): 30215800, ("fused", 1, 32): 30215800}
+MEASURED_TRAFFIC = {("auto", 1, 32): 30192100}
 LAYERS = 32
 HIDDEN, KV, FFN, VOCAB = 4096, 1024, 14336, 128256
 
@@ -314,7 +314,9 @@ def main() -> int:
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC.get((args.plan, b, args.layers)),
-                "kernel": f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
+                "kernel": (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
+                           f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if args.plan == "auto" and b <= 4
+                          else f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches}
 
     # ------------------------------------------------------------------ CPU baseline leg
