@@ -68,13 +68,23 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     const int n_tiles = (p.n + 31) >> 5;
     const size_t row_bytes = (size_t)p.nb * Q4K_BYTES;
 
-    // Activation scales of this pass, zero for the rows the pass does not have.
+    // Activation scales of this pass, zero for the rows the pass does not have. Eight loads are
+    // issued before the first is used: one at a time, each would cost a memory latency.
     const uint8_t* y0 = p.y + (size_t)m0 * p.stride_y * Q81_BYTES;
-    for (int idx = threadIdx.x; idx < p.nb * 8 * TOK; idx += WG) {
-        const int sub = idx >> 5, tok = idx & 31;
-        float d8 = 0.f;
-        if (tok < m_count) d8 = f16_bits_to_f32(*(const uint16_t*)(y0 + ((size_t)tok * p.stride_y + sub) * Q81_BYTES));
-        d8_table[idx] = d8;
+    const int entries = p.nb * 8 * TOK;
+    for (int base = threadIdx.x; base < entries; base += WG * 8) {
+        uint32_t bits[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int idx = min(base + u * WG, entries - 1);
+            const int sub = idx >> 5, tok = min(idx & 31, m_count - 1);
+            bits[u] = *(const uint16_t*)(y0 + ((size_t)tok * p.stride_y + sub) * Q81_BYTES);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int idx = base + u * WG;
+            if (idx < entries) d8_table[idx] = (idx & 31) < m_count ? f16_bits_to_f32(bits[u]) : 0.f;
+        }
     }
 
     // The lane's activation row (a row past the end re-reads the last one; its scales are zero).
