@@ -333,6 +333,10 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
     constexpr int WAVES_N = 4 / WAVES_M;
     constexpr int JT = TN / (32 * WAVES_N), IT = TM / (32 * WAVES_M);
     static_assert(JT >= 1 && IT >= 1, "tile does not split over four waves");
+    // Which operand's index lands on the accumulator registers. A wave with more token tiles than
+    // weight tiles puts the weight rows there (matrix instruction called as weights x tokens);
+    // not for two scales per sub-block (Q6_K), whose second set of 16 registers spills.
+    constexpr bool SWAP = IT > JT && F::NS != 16;
 
     int8_t* wq = (int8_t*)lds;                       // [8][TN][32]
     int8_t* aq = wq + 8 * TN * 32;                   // [8][TM][32]
@@ -387,6 +391,49 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
                     ws2[jt] = 0.f;
                 }
             }
+            if constexpr (SWAP) {
+                // Weight rows on the accumulator registers, tokens on the lanes: the 16 per-register
+                // scales are the weight tile's (read once and shared by the wave's token tiles), the
+                // token scale is one value per lane.
+                float wsv[JT][16], ws2v[JT][16];
+#pragma unroll
+                for (int jt = 0; jt < JT; ++jt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int at = (wn * JT + jt) * 32 + 8 * g + 4 * lh;
+                        const float4 t = *(const float4*)(wsc + (F::NS == 16 ? 2 * s : s) * TN + at);
+                        wsv[jt][4 * g + 0] = t.x; wsv[jt][4 * g + 1] = t.y; wsv[jt][4 * g + 2] = t.z; wsv[jt][4 * g + 3] = t.w;
+                        if constexpr (F::NS == 16) {
+                            const float4 u = *(const float4*)(wsc + (2 * s + 1) * TN + at);
+                            ws2v[jt][4 * g + 0] = u.x; ws2v[jt][4 * g + 1] = u.y; ws2v[jt][4 * g + 2] = u.z; ws2v[jt][4 * g + 3] = u.w;
+                        }
+                    }
+#pragma unroll
+                for (int it = 0; it < IT; ++it) {
+                    const float d8l = ad8[s * TM + (wm * IT + it) * 32 + l32];
+#pragma unroll
+                    for (int jt = 0; jt < JT; ++jt) {
+                        if constexpr (F::NS == 16) {
+                            const v4i zero = {0, 0, 0, 0};
+                            const v4i b_lo = lh == 0 ? b[jt] : zero, b_hi = lh == 0 ? zero : b[jt];
+                            v16i c0 = {0}, c1 = {0};
+                            c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(b_lo, a[it], c0, 0, 0, 0);
+                            c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(b_hi, a[it], c1, 0, 0, 0);
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) {
+                                const float t = fmaf(ws2v[jt][v], (float)c1[v], wsv[jt][v] * (float)c0[v]);
+                                acc[it][jt][v] = fmaf(t, d8l, acc[it][jt][v]);
+                            }
+                        } else {
+                            v16i c = {0};
+                            c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[jt], a[it], c, 0, 0, 0);
+#pragma unroll
+                            for (int v = 0; v < 16; ++v)
+                                acc[it][jt][v] = fmaf((float)c[v], wsv[jt][v] * d8l, acc[it][jt][v]);
+                        }
+                    }
+                }
+            } else {
 #pragma unroll
             for (int it = 0; it < IT; ++it) {
                 // d8 of the 16 tokens this lane's accumulator registers stand for
@@ -420,6 +467,7 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
                     }
                 }
             }
+            }
         }
         if (F::HAS_MIN) {
             // acc += (d8*S)[token, s] * (-dmin*m)[s, n], s = 0..7: four K=2 f32 MFMAs per patch
@@ -434,7 +482,8 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
                 for (int it = 0; it < IT; ++it)
 #pragma unroll
                     for (int jt = 0; jt < JT; ++jt)
-                        acc[it][jt] = __builtin_amdgcn_mfma_f32_32x32x2f32(am[it], bm[jt], acc[it][jt], 0, 0, 0);
+                        acc[it][jt] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x2f32(bm[jt], am[it], acc[it][jt], 0, 0, 0)
+                                           : __builtin_amdgcn_mfma_f32_32x32x2f32(am[it], bm[jt], acc[it][jt], 0, 0, 0);
             }
         }
     }
@@ -443,13 +492,25 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
     for (int it = 0; it < IT; ++it)
 #pragma unroll
         for (int jt = 0; jt < JT; ++jt) {
-            const int gn = n0 + (wn * JT + jt) * 32 + l32;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int col = m0 + (wm * IT + it) * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
-                if (gn < pb.n && col < pb.m_end) {
+            if constexpr (SWAP) {
+                const int col = m0 + (wm * IT + it) * 32 + l32;
+                if (col < pb.m_end) {
                     const int64_t drow = pb.ids_dst ? pb.ids_dst[col] : col;
-                    pb.dst[drow * pb.ldd + gn] = acc[it][jt][v];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int gn = n0 + (wn * JT + jt) * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
+                        if (gn < pb.n) pb.dst[drow * pb.ldd + gn] = acc[it][jt][v];
+                    }
+                }
+            } else {
+                const int gn = n0 + (wn * JT + jt) * 32 + l32;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int col = m0 + (wm * IT + it) * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
+                    if (gn < pb.n && col < pb.m_end) {
+                        const int64_t drow = pb.ids_dst ? pb.ids_dst[col] : col;
+                        pb.dst[drow * pb.ldd + gn] = acc[it][jt][v];
+                    }
                 }
             }
         }
