@@ -395,7 +395,7 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
                 // Weight rows on the accumulator registers, tokens on the lanes: the 16 per-register
                 // scales are the weight tile's (read once and shared by the wave's token tiles), the
                 // token scale is one value per lane.
-                float wsv[JT][16], ws2v[JT][16];
+                float wsv[JT][16], ws2v[JT][16], wso[JT][16];
 #pragma unroll
                 for (int jt = 0; jt < JT; ++jt)
 #pragma unroll
@@ -407,6 +407,8 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
                             const float4 u = *(const float4*)(wsc + (2 * s + 1) * TN + at);
                             ws2v[jt][4 * g + 0] = u.x; ws2v[jt][4 * g + 1] = u.y; ws2v[jt][4 * g + 2] = u.z; ws2v[jt][4 * g + 3] = u.w;
                         }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) wso[jt][4 * g + e] = -12582912.0f * wsv[jt][4 * g + e];
                     }
 #pragma unroll
                 for (int it = 0; it < IT; ++it) {
@@ -425,11 +427,27 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
                                 acc[it][jt][v] = fmaf(t, d8l, acc[it][jt][v]);
                             }
                         } else {
-                            v16i c = {0};
-                            c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[jt], a[it], c, 0, 0, 0);
+                            if constexpr (F::HAS_MIN) {
+                                v16i c = {0};
+                                c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[jt], a[it], c, 0, 0, 0);
 #pragma unroll
-                            for (int v = 0; v < 16; ++v)
-                                acc[it][jt][v] = fmaf((float)c[v], wsv[jt][v] * d8l, acc[it][jt][v]);
+                                for (int v = 0; v < 16; ++v)
+                                    acc[it][jt][v] = fmaf((float)c[v], wsv[jt][v] * d8l, acc[it][jt][v]);
+                            } else {
+                                // The int32 accumulators start at the bit pattern of 1.5 * 2^23, so the
+                                // dots leave the matrix unit as the floats MAGIC + dot; the offset goes
+                                // in the first fma, exactly (the weight scale is an f16: MAGIC * scale
+                                // does not round), which then rounds dot * scale once, as
+                                // convert-then-multiply would. (With a min term to carry as well, the 16
+                                // registers of offsets cost more than the conversions they save.)
+                                v16i c;
+#pragma unroll
+                                for (int v = 0; v < 16; ++v) c[v] = 0x4B400000;
+                                c = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[jt], a[it], c, 0, 0, 0);
+#pragma unroll
+                                for (int v = 0; v < 16; ++v)
+                                    acc[it][jt][v] = fmaf(fmaf(__int_as_float(c[v]), wsv[jt][v], wso[jt][v]), d8l, acc[it][jt][v]);
+                            }
                         }
                     }
                 }
@@ -594,10 +612,10 @@ static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x
     if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s);
     if (ncols_y <= 64) return launch_dense_tm<F, 64, 2>(pb, s);
     if (getenv("LK_MMQ_TM64")) return launch_dense_tm<F, 64, 2>(pb, s);
-    // 128-token tile: a wave takes all four token tiles of one 32-row weight tile (1 x 4 waves) for
-    // the K-quants, a 2 x 2 patch for Q8_0 (measured: Q4_K 350 against 334 TOP/s at 512 rows, 404
-    // against 364 at 2048; Q6_K 320 against 313; Q8_0 295 against 304)
-    constexpr int WAVES_M = (F::HAS_MIN || F::NS == 16) ? 1 : 2;
+    // 128-token tile: a wave takes all four token tiles of one 32-row weight tile (measured against
+    // a 2 x 2 patch per wave: Q4_K 366 against 334 TOP/s at 512 rows, 434 against 364 at 2048;
+    // Q6_K 320 against 313; Q8_0 305 against 304)
+    constexpr int WAVES_M = 1;
     return launch_dense_tm<F, 128, WAVES_M>(pb, s);
 }
 
@@ -633,7 +651,7 @@ static int launch_moe(const void* x, const void* x_second, int64_t dst_second, c
     const int64_t want = mmq_x > 0 ? mmq_x : (ncols_hint > 0 ? ncols_hint : ncols_max);
     if (want <= 32) return launch_moe_tm<F, 32, 1>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
     if (want <= 64) return launch_moe_tm<F, 64, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
-    constexpr int WAVES_M = (F::HAS_MIN || F::NS == 16) ? 1 : 2;
+    constexpr int WAVES_M = 1;
     return launch_moe_tm<F, 128, WAVES_M>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
 }
 
