@@ -25,17 +25,15 @@
 // registers <-> tokens. The Q4_K min term is a rank-8 update per block and runs on the f32
 // MFMA (v_mfma_f32_32x32x2_f32) straight into the accumulators, costing no per-element VALU.
 
-#include "lk_common.h"
+#include "mmq_problem.h"
 
 #include <cstdlib>
-#include <mutex>
-#include <unordered_map>
 
 namespace {
 
 constexpr int MMQ_WG = 256;
 constexpr int TN = 128;            // weight rows per workgroup tile
-constexpr int REC_BYTES = 288;     // workspace record: 256 codes + 8 f16 + 8 i16
+constexpr int REC_BYTES = MMQ_REC_BYTES;
 
 // --------------------------------------------------------------------------------------------
 // Activation quantizer -> workspace records
@@ -315,19 +313,6 @@ struct TokenFrag {
     }
 };
 
-// One problem = one weight slab against a contiguous run of workspace rows.
-struct MmqProblem {
-    const uint8_t* w;      // [n][nb] blocks
-    const uint8_t* y;      // workspace records
-    float* dst;
-    const int32_t* ids_dst;  // nullable: destination row of workspace row c
-    int64_t nb;            // K steps: 256-value blocks per weight row
-    int64_t row_blocks;    // format blocks between consecutive weight rows
-    int64_t rows_total;    // rows the workspace was quantized with (record stride)
-    int64_t ldd;           // floats between destination rows
-    int n, m_begin, m_end;
-};
-
 template <class F, int TM, int WAVES_M>
 static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, int m0, uint8_t* lds) {
     constexpr int WAVES_N = 4 / WAVES_M;
@@ -571,27 +556,11 @@ __global__ __launch_bounds__(MMQ_WG, 2) void mmq_moe_kernel(MmqProblem pb, const
         mmq_tile<F, TM, WAVES_M>(pb, blockIdx.x * TN, m0, lds);
 }
 
-template <typename K>
-static int prepare_kernel(K kernel, int lds_bytes) {
-    static std::mutex mu;
-    static std::unordered_map<const void*, bool> done;
-    std::lock_guard<std::mutex> lock(mu);
-    if (done.count((const void*)kernel)) return LK_OK;
-    if (lds_bytes > lk_device().lds_bytes) return LK_ERR_ARG;
-    if (lds_bytes > 48 * 1024 &&
-        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) {
-        (void)hipGetLastError();
-        return LK_ERR_LAUNCH;
-    }
-    done[(const void*)kernel] = true;
-    return LK_OK;
-}
-
 template <class F, int TM, int WAVES_M>
 static int launch_dense_tm(const MmqProblem& pb, hipStream_t s) {
     auto kernel = mmq_dense_kernel<F, TM, WAVES_M>;
     constexpr int lds_bytes = mmq_lds_bytes<F, TM>();
-    if (prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
+    if (mmq_prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
     const int n_tiles = (pb.n + TN - 1) / TN;
     const int m_tiles = (pb.m_end - pb.m_begin + TM - 1) / TM;
     const int n_groups = (n_tiles + 7) / 8;
@@ -611,7 +580,12 @@ static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x
     hipStream_t s = (hipStream_t)stream;
     if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s);
     if (ncols_y <= 64) return launch_dense_tm<F, 64, 2>(pb, s);
-    if (getenv("LK_MMQ_TM64")) return launch_dense_tm<F, 64, 2>(pb, s);
+    if constexpr (F::HAS_MIN) {   // Q4_K: scales folded into f16 operands
+        if (!getenv("LK_MMQ_I8")) {
+            const int tm = lk_mmq_q4k_f16_dense(pb, s);
+            if (tm >= 0) return tm;
+        }
+    }
     // 128-token tile: a wave takes all four token tiles of one 32-row weight tile (measured against
     // a 2 x 2 patch per wave: Q4_K 366 against 334 TOP/s at 512 rows, 434 against 364 at 2048;
     // Q6_K 320 against 313; Q8_0 305 against 304)
@@ -625,7 +599,7 @@ static int launch_moe_tm(const MmqProblem& pb, const uint8_t* w_second, int64_t 
                          hipStream_t s) {
     auto kernel = mmq_moe_kernel<F, TM, WAVES_M>;
     constexpr int lds_bytes = mmq_lds_bytes<F, TM>();
-    if (prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
+    if (mmq_prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
     const int64_t col_tiles = (ncols_max + TM - 1) / TM;
     const dim3 grid((pb.n + TN - 1) / TN, (unsigned)(col_tiles < 1 ? 1 : (col_tiles > 65535 ? 65535 : col_tiles)),
                     (unsigned)((w_second ? 2 : 1) * n_experts));
@@ -651,6 +625,12 @@ static int launch_moe(const void* x, const void* x_second, int64_t dst_second, c
     const int64_t want = mmq_x > 0 ? mmq_x : (ncols_hint > 0 ? ncols_hint : ncols_max);
     if (want <= 32) return launch_moe_tm<F, 32, 1>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
     if (want <= 64) return launch_moe_tm<F, 64, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
+    if constexpr (F::HAS_MIN) {
+        if (!getenv("LK_MMQ_I8")) {
+            const int tm = lk_mmq_q4k_f16_moe(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
+            if (tm >= 0) return tm;
+        }
+    }
     constexpr int WAVES_M = 1;
     return launch_moe_tm<F, 128, WAVES_M>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
 }

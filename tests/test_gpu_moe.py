@@ -114,8 +114,14 @@ def test_result_does_not_depend_on_tile_width():
         plan = MmqRouting.from_choices(dev(ids), n_experts).with_tile_width(width)
         h = plan.gate_up_silu(lib.TYPE_Q4_K, dev(x), dev(gate), dev(up), ffn)
         outs.append(plan.down_fold(lib.TYPE_Q4_K, h, dev(down), hidden, dev(w.reshape(-1))))
-    for o in outs[1:]:
+    # The narrow tiles run the same int8 kernel, to the bit. The 128-token tile of Q4_K forms the
+    # same integer dots on the f16 matrix unit and adds them up in another f32 order; the hidden
+    # state is re-quantized between the two products, so a last-bit difference there can move a
+    # code by one: a float tolerance, not equality.
+    for o in outs[1:3]:
         assert torch.equal(o, outs[0])
+    scale = outs[0].abs().max().item()
+    assert (outs[3] - outs[0]).abs().max().item() <= 1e-4 * scale
 
 
 def test_glu_kernels():
