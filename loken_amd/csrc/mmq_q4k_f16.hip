@@ -14,13 +14,16 @@
 // (< 2^24). D_s leaves the unit as a float that already carries the weight scale, and one fma by
 // the lane's d8 finishes it. Half the matrix rate of int8, a third of the vector work.
 //
-// Shape: a wave owns 32 weight rows and TT token tiles of 32; registers <-> weight rows, lanes <->
-// tokens (v_mfma_f32_32x32x16_f16 called as weights x tokens). Weight rows are private to a wave,
-// so they never touch LDS: each lane loads its row's block straight from global memory in operand
-// order and expands the nibbles in registers. Token codes are shared by the four waves of a
-// column: the workgroup expands them to f16 once per step into LDS, two stages deep, one barrier
-// per step. The min term is a rank-8 update per block on the bf16 matrix unit, with d8 * S split
-// into three bf16 pieces (24 bits, nothing lost).
+// Shape: a workgroup of eight waves takes 256 weight rows x 64 tokens; a wave owns 32 of the rows
+// and both token tiles of 32; registers <-> weight rows, lanes <-> tokens (v_mfma_f32_32x32x16_f16
+// called as weights x tokens). Per 256-value step the workgroup copies its 256 weight blocks into
+// LDS as they lie in memory (consecutive lanes read consecutive 16-byte pieces of a row's block:
+// loading them lane-per-row instead touches 64 cache lines per instruction and was a fifth of
+// the kernel's time), and each lane then picks its row's nibbles out of LDS in operand order and
+// expands them in registers. Token codes are expanded to f16 once per step into LDS. Both tiles
+// are two stages deep, filled for step k + 1 while step k is multiplied, one barrier per step.
+// The min term is a rank-8 update per block on the bf16 matrix unit, with d8 * S split into
+// three bf16 pieces (24 bits, nothing lost).
 //
 // K order inside a sub-block: lane half h (lane / 32) of MFMA hf holds values 16 h + 8 hf + i,
 // i in the order 0 2 1 3 4 6 5 7 (what masking a dword's even and odd bytes yields); weights and
@@ -39,43 +42,54 @@ static __device__ __forceinline__ uint32_t h2_bits(h2 v) { return __builtin_bit_
 
 constexpr uint32_t H1024 = 0x64006400u;   // two f16 1024.0: OR-ing an 8-bit integer into the mantissa adds it
 
-template <int TT, int WM>
 struct Wide {
-    static constexpr int WAVES = 4 * WM;              // four waves along the weight rows
+    static constexpr int WAVES = 8;                   // along the weight rows
     static constexpr int THREADS = 64 * WAVES;
-    static constexpr int TM = 32 * TT * WM;           // tokens per workgroup tile
-    static constexpr int TN = 128;                    // weight rows per workgroup tile
+    static constexpr int TT = 2;                      // token tiles of 32 per wave
+    static constexpr int TM = 32 * TT;                // tokens per workgroup tile
+    static constexpr int TN = 32 * WAVES;             // weight rows per workgroup tile
     static constexpr int CCH = TM * 16 / THREADS;     // 16-code chunks per thread per step
     static constexpr int PARTS = THREADS / TM;        // threads sharing one token's scales
-    static constexpr int SB = 8 / PARTS;              // sub-blocks per such thread
-    static_assert(TM * 16 % THREADS == 0 && THREADS % TM == 0 && (SB == 2 || SB == 4), "tile split");
-    // one LDS stage: f16 codes [plane = (s, hf, h)][token ^ swizzle][8 halves], d8 [s][token] f32,
-    // pieces [hi, mid, lo, zero][token][8 bf16]
+    static_assert(TM * 16 % THREADS == 0 && PARTS == 8, "one sub-block's scale per thread");
+    static constexpr int WCH = (TN * 9 + THREADS - 1) / THREADS;   // 16-byte weight chunks per thread per step
+    // one token stage: f16 codes [plane = (s, hf, h)][token ^ swizzle][8 halves], d8 [s][token] f32,
+    // pieces [hi, mid, lo, zero][token][8 bf16]; one weight stage: TN blocks of 144 bytes
     static constexpr int CODES = TM * 512, D8 = TM * 32, PIECES = 4 * TM * 16;
     static constexpr int STAGE = CODES + D8 + PIECES;
-    static constexpr int LDS = 2 * STAGE + WAVES * 256;   // + per wave: d and -dmin of its 32 rows
+    static constexpr int WSTAGE = TN * Q4K_BYTES;
+    static constexpr int LDS = 2 * STAGE + 2 * WSTAGE + WAVES * 256;   // + per wave: d and -dmin of its 32 rows
 };
 
-struct WeightFrag {
-    uint4 hdr;     // d, dmin, 12 scale bytes
-    uint4 q[4];    // 16 bytes of each 64-value pair: the lane half's 16 low- and 16 high-nibble codes
-};
+// The workgroup's copy of one step's weight blocks: chunk q = tid + i * THREADS is 16-byte piece
+// q % 9 of row q / 9's block, and lands at byte 16 q of the stage.
+struct WeightCopy {
+    using C = Wide;
+    const uint8_t* from[C::WCH];   // the chunk's address in step 0 (rows past the end re-read the last row)
+    uint4 data[C::WCH];
 
-// Load `i` of the five that bring in a block (every lane of these loads is a cache line of its
-// own, so the kernels issue them one at a time between other work).
-static __device__ __forceinline__ void fetch_weights_part(WeightFrag& f, const uint8_t* __restrict__ block, int h, int i) {
-    if (i == 0) f.hdr = *(const uint4*)block;
-    else f.q[i - 1] = *(const uint4*)(block + 16 + 32 * (i - 1) + 16 * h);
-}
-static __device__ __forceinline__ void fetch_weights(WeightFrag& f, const uint8_t* __restrict__ block, int h) {
+    __device__ __forceinline__ void place(const uint8_t* w, int64_t row_bytes, int n0, int n) {
 #pragma unroll
-    for (int i = 0; i < 5; ++i) fetch_weights_part(f, block, h, i);
-}
+        for (int i = 0; i < C::WCH; ++i) {
+            const int q = min((int)threadIdx.x + i * C::THREADS, C::TN * 9 - 1);
+            from[i] = w + (int64_t)min(n0 + q / 9, n - 1) * row_bytes + 16 * (q % 9);
+        }
+    }
+    // The last round has chunks for half the threads only; the others repeat the stage's last
+    // chunk (same bytes to the same place), which keeps the step free of branches.
+    __device__ __forceinline__ void fetch_part(int64_t step_bytes, int i) { data[i] = *(const uint4*)(from[i] + step_bytes); }
+    __device__ __forceinline__ void commit_part(uint8_t* wstage, int i) const {
+        *(uint4*)(wstage + min((int)threadIdx.x + i * C::THREADS, C::TN * 9 - 1) * 16) = data[i];
+    }
+    __device__ __forceinline__ void commit(uint8_t* wstage) const {
+#pragma unroll
+        for (int i = 0; i < C::WCH; ++i) commit_part(wstage, i);
+    }
+};
 
-template <class C>
 struct TokenFrag16 {
+    using C = Wide;
     uint4 codes[C::CCH];
-    uint32_t d8[C::SB / 2], sums[C::SB / 2];
+    uint16_t d8, sum;   // of sub-block tid / TM of token tid % TM
 
     // Byte offsets of this thread's loads inside one K step's slab of records (rows past the end
     // re-read the last row: their results are never stored).
@@ -88,7 +102,7 @@ struct TokenFrag16 {
             code_at[i] = (uint32_t)min(m0 + r, m_end - 1) * MMQ_REC_BYTES + 16 * c;
         }
         const int r = tid % C::TM, part = tid / C::TM;
-        scale_at = (uint32_t)min(m0 + r, m_end - 1) * MMQ_REC_BYTES + 256 + 2 * C::SB * part;
+        scale_at = (uint32_t)min(m0 + r, m_end - 1) * MMQ_REC_BYTES + 256 + 2 * part;
     }
     // Part i < CCH: a chunk of codes; part CCH: the scales and sums.
     static constexpr int FETCH_PARTS = C::CCH + 1;
@@ -96,11 +110,8 @@ struct TokenFrag16 {
         if (i < C::CCH) {
             codes[i] = *(const uint4*)(slab + code_at[i]);
         } else {
-#pragma unroll
-            for (int q = 0; q < C::SB / 2; ++q) {
-                d8[q] = *(const uint32_t*)(slab + scale_at + 4 * q);
-                sums[q] = *(const uint32_t*)(slab + scale_at + 16 + 4 * q);
-            }
+            d8 = *(const uint16_t*)(slab + scale_at);
+            sum = *(const uint16_t*)(slab + scale_at + 16);
         }
     }
     __device__ __forceinline__ void fetch(const uint8_t* __restrict__ slab) {
@@ -117,10 +128,14 @@ struct TokenFrag16 {
         odd = h2_bits(as_h2(((u >> 8) & 0x00FF00FFu) ^ 0x64806480u) - bias);
     }
 
+    // Part i of the registers into a stage (the parts of fetch_part).
     __device__ __forceinline__ void commit(uint8_t* stage) const {
-        const int tid = threadIdx.x;
 #pragma unroll
-        for (int i = 0; i < C::CCH; ++i) {
+        for (int i = 0; i < FETCH_PARTS; ++i) commit_part(stage, i);
+    }
+    __device__ __forceinline__ void commit_part(uint8_t* stage, int i) const {
+        const int tid = threadIdx.x;
+        if (i < C::CCH) {
             const int idx = tid + i * C::THREADS, r = idx >> 4, c = idx & 15;
             const int s = c >> 1, h = c & 1;
             const uint32_t u[4] = {codes[i].x, codes[i].y, codes[i].z, codes[i].w};
@@ -134,37 +149,24 @@ struct TokenFrag16 {
                 // the plane's (s, h) so that they land in 16 different bank groups
                 *(uint4*)(stage + (plane * C::TM + (r ^ c)) * 16) = out;
             }
+            return;
         }
         float* ad8 = (float*)(stage + C::CODES);
         uint8_t* ap = stage + C::CODES + C::D8;
-        const int r = tid % C::TM, part = tid / C::TM;
-        uint32_t hi[C::SB / 2], mid[C::SB / 2], lo[C::SB / 2];
-#pragma unroll
-        for (int q = 0; q < C::SB; ++q) {
-            const int s = part * C::SB + q;
-            const float d = f16_bits_to_f32((d8[q >> 1] >> (16 * (q & 1))) & 0xFFFFu);
-            const int sum = (int)(int16_t)((sums[q >> 1] >> (16 * (q & 1))) & 0xFFFFu);
-            ad8[s * C::TM + r] = d;
-            // d8 * S as three bf16 (truncations of the running remainder: 8 bits each, exact)
-            const float p0 = d * (float)sum;
-            const uint32_t b0 = __float_as_uint(p0) & 0xFFFF0000u;
-            const float p1 = p0 - __uint_as_float(b0);
-            const uint32_t b1 = __float_as_uint(p1) & 0xFFFF0000u;
-            const float p2 = p1 - __uint_as_float(b1);
-            const uint32_t b2 = __float_as_uint(p2) & 0xFFFF0000u;
-            if (q & 1) {
-                hi[q >> 1] |= b0; mid[q >> 1] |= b1; lo[q >> 1] |= b2;
-            } else {
-                hi[q >> 1] = b0 >> 16; mid[q >> 1] = b1 >> 16; lo[q >> 1] = b2 >> 16;
-            }
-        }
-#pragma unroll
-        for (int q = 0; q < C::SB / 2; ++q) {
-            const int at = r * 16 + part * C::SB * 2 + 4 * q;
-            *(uint32_t*)(ap + 0 * C::TM * 16 + at) = hi[q];
-            *(uint32_t*)(ap + 1 * C::TM * 16 + at) = mid[q];
-            *(uint32_t*)(ap + 2 * C::TM * 16 + at) = lo[q];
-        }
+        const int r = tid % C::TM, s = tid / C::TM;
+        const float d = f16_bits_to_f32(d8);
+        ad8[s * C::TM + r] = d;
+        // d8 * S as three bf16 (truncations of the running remainder: 8 bits each, exact)
+        const float p0 = d * (float)(int)(int16_t)sum;
+        const uint32_t b0 = __float_as_uint(p0) & 0xFFFF0000u;
+        const float p1 = p0 - __uint_as_float(b0);
+        const uint32_t b1 = __float_as_uint(p1) & 0xFFFF0000u;
+        const float p2 = p1 - __uint_as_float(b1);
+        const uint32_t b2 = __float_as_uint(p2) & 0xFFFF0000u;
+        const int at = r * 16 + s * 2;
+        *(uint16_t*)(ap + 0 * C::TM * 16 + at) = (uint16_t)(b0 >> 16);
+        *(uint16_t*)(ap + 1 * C::TM * 16 + at) = (uint16_t)(b1 >> 16);
+        *(uint16_t*)(ap + 2 * C::TM * 16 + at) = (uint16_t)(b2 >> 16);
     }
 };
 
@@ -203,10 +205,10 @@ static __device__ __forceinline__ void weight_operands(const uint4& q, bool high
 }
 
 // The B operands and the token scale of item (s, tt). `ad8` already points at the lane's token.
-template <class C>
 static __device__ __forceinline__ void load_item(const uint8_t* stage, const uint8_t* ad8, int s, int tt, int token0,
                                                  int h, v8h b[2], float& d8) {
     // token0 ^ (2 s + h) only changes the low four bits, so the tile offset 32 tt adds on top
+    using C = Wide;
     const uint8_t* at = stage + (token0 ^ (2 * s + h)) * 16 + h * C::TM * 16 + tt * 512;
     b[0] = *(const v8h*)(at + (s * 4 + 0) * C::TM * 16);
     b[1] = *(const v8h*)(at + (s * 4 + 2) * C::TM * 16);
@@ -221,18 +223,14 @@ static __device__ __forceinline__ void scale_item(int it, const v16f& dot, float
     for (int v = 8 * HALF; v < 8 * HALF + 8; ++v) part[tt][v] = s == 0 ? dot[v] * d8 : fmaf(dot[v], d8, part[tt][v]);
 }
 
-template <int TT, int WM>
 static __device__ __forceinline__ void q4k_f16_tile(const MmqProblem& pb, int n0, int m0, uint8_t* lds) {
-    using C = Wide<TT, WM>;
-    constexpr int TM = C::TM;
+    using C = Wide;
+    constexpr int TM = C::TM, TT = C::TT;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wn = wave & 3, wm = wave >> 2;
     const int j = lane & 31, h = lane >> 5;
-    float* wd = (float*)(lds + 2 * C::STAGE) + wave * 64;   // [0, 32) d, [32, 64) -dmin of the wave's rows
-
-    const int gn = min(n0 + 32 * wn + j, pb.n - 1);
-    const uint8_t* wrow = pb.w + (int64_t)gn * pb.row_blocks * Q4K_BYTES;
+    uint8_t* wstages = lds + 2 * C::STAGE;
+    float* wd = (float*)(wstages + 2 * C::WSTAGE) + wave * 64;   // [0, 32) d, [32, 64) -dmin of the wave's rows
     const int last = (int)pb.nb - 1;
 
     v16f acc[TT];
@@ -247,33 +245,43 @@ static __device__ __forceinline__ void q4k_f16_tile(const MmqProblem& pb, int n0
         *(uint4*)(stage + C::CODES + C::D8 + (3 * TM + i % TM) * 16) = make_uint4(0, 0, 0, 0);
     }
 
-    WeightFrag wf, wf_next;
-    TokenFrag16<C> tf;
+    WeightCopy wc;
+    TokenFrag16 tf;
     const int64_t slab_bytes = pb.rows_total * MMQ_REC_BYTES;
     tf.place(m0, pb.m_end);
+    wc.place(pb.w, pb.row_blocks * Q4K_BYTES, n0, pb.n);
     tf.fetch(pb.y);
-    fetch_weights(wf, wrow, h);
+#pragma unroll
+    for (int i = 0; i < C::WCH; ++i) wc.fetch_part(0, i);
     tf.commit(lds);
+    wc.commit(wstages);
     tf.fetch(pb.y + min(1, last) * slab_bytes);
+#pragma unroll
+    for (int i = 0; i < C::WCH; ++i) wc.fetch_part((int64_t)min(1, last) * Q4K_BYTES, i);
     __syncthreads();
 
     // 1024.0 | 1024.0 in a vector register: with the mask as the instruction's one literal,
     // (x & mask) | h1024 is a single v_and_or_b32
     uint32_t h1024 = H1024;
     asm volatile("" : "+v"(h1024));
-    const int token0 = 32 * wm * TT + j;   // the lane's token in the wave's first token tile
+    const int token0 = j;   // the lane's token in the first token tile
 
     for (int kb = 0; kb <= last; ++kb) {
         const uint8_t* stage = lds + (kb & 1) * C::STAGE;
         const uint8_t* ad8 = stage + C::CODES + token0 * 4;
         const uint8_t* ap = stage + C::CODES + C::D8 + token0 * 16;
-        const uint8_t* next_block = wrow + (int64_t)min(kb + 1, last) * Q4K_BYTES;
+        // the lane's row in the weight stage; its half of pair p's nibbles at +16 + 32 p + 16 h
+        const uint8_t* wblock = wstages + (kb & 1) * C::WSTAGE + (32 * wave + j) * Q4K_BYTES;
         const uint8_t* next_slab = pb.y + min(kb + 2, last) * slab_bytes;
+        const int64_t next_step = (int64_t)min(kb + 2, last) * Q4K_BYTES;
+
+        const uint4 hdr = *(const uint4*)wblock;
+        uint4 nib = *(const uint4*)(wblock + 16 + 16 * h);
         uint32_t sc[8], mn[8];
-        unpack_scales(wf.hdr, sc, mn);
+        unpack_scales(hdr, sc, mn);
         if (h == 0) {
-            wd[j] = f16_bits_to_f32(wf.hdr.x & 0xFFFFu);
-            wd[32 + j] = -f16_bits_to_f32(wf.hdr.x >> 16);
+            wd[j] = f16_bits_to_f32(hdr.x & 0xFFFFu);
+            wd[32 + j] = -f16_bits_to_f32(hdr.x >> 16);
         }
 
         // Items (s, tt) run through a three-deep pipeline written out by hand: the LDS reads of
@@ -283,15 +291,18 @@ static __device__ __forceinline__ void q4k_f16_tile(const MmqProblem& pb, int n0
         v8h a[2][2], b[2][2];
         float d8v[3];   // read at item i + 1's loads, used at item i - 1's fmas: three alive
         v16f dot[2], part[TT];
-        weight_operands(wf.q[0], false, sc[0], h1024, a[0]);
-        load_item<C>(stage, ad8, 0, 0, token0, h, b[0], d8v[0]);
+        weight_operands(nib, false, sc[0], h1024, a[0]);
+        load_item(stage, ad8, 0, 0, token0, h, b[0], d8v[0]);
 #pragma unroll
         for (int it = 0; it < NI; ++it) {
             const int s = it / TT;
-            if (it + 1 < NI) load_item<C>(stage, ad8, (it + 1) / TT, (it + 1) % TT, token0, h, b[(it + 1) & 1], d8v[(it + 1) % 3]);
+            if (it + 1 < NI) load_item(stage, ad8, (it + 1) / TT, (it + 1) % TT, token0, h, b[(it + 1) & 1], d8v[(it + 1) % 3]);
+            // the nibbles of the pair after this one (read one sub-block before they are expanded)
+            uint4 nib_next = nib;
+            if (it % TT == 0 && (s & 1) == 0 && s + 2 < 8) nib_next = *(const uint4*)(wblock + 16 + 32 * ((s + 2) >> 1) + 16 * h);
             // The second MFMA takes the first one's result as its accumulator and cannot issue
-            // before that is written; a wave issues in order, so whatever should run meanwhile
-            // has to sit between the two.
+            // before that is written, and a wave's own vector instructions do not issue past a
+            // waiting one: whatever should run meanwhile has to sit between the two.
             {
                 v16f zero = {0.f};
                 dot[it & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s & 1][0], b[it & 1][0], zero, 0, 0, 0);
@@ -302,15 +313,31 @@ static __device__ __forceinline__ void q4k_f16_tile(const MmqProblem& pb, int n0
             dot[it & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[s & 1][1], b[it & 1][1], dot[it & 1], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             if (it >= 1) scale_item<TT, 1>(it - 1, dot[(it - 1) & 1], d8v[(it - 1) % 3], part);
-            if (it % TT == 0 && s + 1 < 8) weight_operands(wf.q[(s + 1) >> 1], (s + 1) & 1, sc[s + 1], h1024, a[(s + 1) & 1]);
-            // The loads of later steps, one per item: the next block of weights first; the tokens
-            // of the step after next once this step's have left their registers for the other
-            // stage (whose last readers left at the barrier that ended the previous step).
-            constexpr int COMMIT_AT = NI - 1 - TokenFrag16<C>::FETCH_PARTS;
-            static_assert(COMMIT_AT >= 5, "more loads than items to spread them over");
-            if (it < 5) fetch_weights_part(wf_next, next_block, h, it);
-            if (it == COMMIT_AT) tf.commit(lds + ((kb + 1) & 1) * C::STAGE);
-            if (it > COMMIT_AT) tf.fetch_part(next_slab, it - COMMIT_AT - 1);
+            if (it % TT == 0 && s + 1 < 8) {
+                // sub-block s + 1: the high nibbles of the current pair, or the low ones of the next
+                if ((s + 1) & 1) {
+                    weight_operands(nib, true, sc[s + 1], h1024, a[(s + 1) & 1]);
+                    nib = nib_next;
+                } else {
+                    weight_operands(nib, false, sc[s + 1], h1024, a[(s + 1) & 1]);
+                }
+            }
+            // The next step's tokens and weights leave their registers for the other stages (whose
+            // last readers left at the barrier that ended the previous step) one part per item, so
+            // that eight waves' LDS writes do not arrive in one burst; each part's registers take
+            // the load of the step after next one item later.
+            constexpr int PARTS = TokenFrag16::FETCH_PARTS + C::WCH;
+            constexpr int FIRST = NI - 1 - PARTS;
+            static_assert(FIRST >= 0, "more parts than items to spread them over");
+            {
+                const int c = it - FIRST, f = it - FIRST - 1;   // the part committed / fetched at this item
+                uint8_t* to = lds + ((kb + 1) & 1) * C::STAGE;
+                uint8_t* wto = wstages + ((kb + 1) & 1) * C::WSTAGE;
+                if (c >= 0 && c < C::WCH) wc.commit_part(wto, c);
+                if (c >= C::WCH && c < PARTS) tf.commit_part(to, c - C::WCH);
+                if (f >= 0 && f < C::WCH) wc.fetch_part(next_step, f);
+                if (f >= C::WCH && f < PARTS) tf.fetch_part(next_slab, f - C::WCH);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
         scale_item<TT, 0>(NI - 1, dot[(NI - 1) & 1], d8v[(NI - 1) % 3], part);
@@ -344,21 +371,19 @@ static __device__ __forceinline__ void q4k_f16_tile(const MmqProblem& pb, int n0
             for (int v = 0; v < 16; ++v)
                 acc[tt][v] = fmaf(ndm[v], mins[v], fmaf(dv[v], part[tt][v], acc[tt][v]));
         }
-
-        wf = wf_next;
         __syncthreads();
     }
 
     const bool vec_ok = ((uintptr_t)pb.dst % 16 == 0) && (pb.ldd % 4 == 0);
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-        const int col = m0 + 32 * (wm * TT + tt) + j;
+        const int col = m0 + 32 * tt + j;
         if (col >= pb.m_end) continue;
         const int64_t drow = pb.ids_dst ? pb.ids_dst[col] : col;
         float* out = pb.dst + drow * pb.ldd;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            const int gn0 = n0 + 32 * wn + 8 * g + 4 * h;
+            const int gn0 = n0 + 32 * wave + 8 * g + 4 * h;
             if (vec_ok && gn0 + 3 < pb.n) {
                 *(float4*)(out + gn0) = make_float4(acc[tt][4 * g], acc[tt][4 * g + 1], acc[tt][4 * g + 2], acc[tt][4 * g + 3]);
             } else {
@@ -372,74 +397,58 @@ static __device__ __forceinline__ void q4k_f16_tile(const MmqProblem& pb, int n0
 
 // Workgroup id -> (n tile, m tile): the m tiles of one n tile re-read the same weight rows, so
 // they are issued back to back on one XCD (ids are dealt round robin over the 8 XCDs).
-template <int TT, int WM>
-__global__ __launch_bounds__((Wide<TT, WM>::THREADS), 1) void q4k_f16_dense_kernel(MmqProblem pb, int n_tiles, int m_tiles) {
+__global__ __launch_bounds__(Wide::THREADS, 1) void q4k_f16_dense_kernel(MmqProblem pb, int n_tiles, int m_tiles) {
     extern __shared__ __align__(16) uint8_t lds[];
-    using C = Wide<TT, WM>;
     const int id = blockIdx.x;
     const int xcd = id & 7, seq = id >> 3;
     const int m_tile = seq % m_tiles;
     const int n_tile = (seq / m_tiles) * 8 + xcd;
     if (n_tile >= n_tiles) return;
-    q4k_f16_tile<TT, WM>(pb, n_tile * C::TN, pb.m_begin + m_tile * C::TM, lds);
+    q4k_f16_tile(pb, n_tile * Wide::TN, pb.m_begin + m_tile * Wide::TM, lds);
 }
 
-template <int TT, int WM>
-__global__ __launch_bounds__((Wide<TT, WM>::THREADS), 1) void q4k_f16_moe_kernel(MmqProblem pb, const uint8_t* w_second,
-                                                                              int64_t dst_second,
-                                                                              const int32_t* __restrict__ bounds,
-                                                                              int64_t stride_expert, int n_experts) {
+// Expert-batched: expert e's slab against the sorted rows [bounds[e], bounds[e+1]).
+__global__ __launch_bounds__(Wide::THREADS, 1) void q4k_f16_moe_kernel(MmqProblem pb, const uint8_t* w_second,
+                                                                      int64_t dst_second,
+                                                                      const int32_t* __restrict__ bounds,
+                                                                      int64_t stride_expert, int n_experts) {
     extern __shared__ __align__(16) uint8_t lds[];
-    using C = Wide<TT, WM>;
     const int stack = blockIdx.z / n_experts, e = blockIdx.z % n_experts;
     pb.m_begin = bounds[e];
     pb.m_end = bounds[e + 1];
     if (pb.m_end <= pb.m_begin) return;
     pb.w = (stack ? w_second : pb.w) + (int64_t)e * stride_expert;
     if (stack) pb.dst += dst_second;
-    for (int m0 = pb.m_begin + blockIdx.y * C::TM; m0 < pb.m_end; m0 += gridDim.y * C::TM) {
-        q4k_f16_tile<TT, WM>(pb, blockIdx.x * C::TN, m0, lds);
-        __syncthreads();   // the next tile's prologue rewrites stage 0
+    for (int m0 = pb.m_begin + blockIdx.y * Wide::TM; m0 < pb.m_end; m0 += gridDim.y * Wide::TM) {
+        q4k_f16_tile(pb, blockIdx.x * Wide::TN, m0, lds);
+        __syncthreads();   // the next tile's prologue rewrites the first stages
     }
-}
-
-template <int TT, int WM>
-static int launch_dense(const MmqProblem& pb, hipStream_t s) {
-    using C = Wide<TT, WM>;
-    auto kernel = q4k_f16_dense_kernel<TT, WM>;
-    if (mmq_prepare_kernel(kernel, C::LDS) != LK_OK) return 0;
-    const int n_tiles = (pb.n + C::TN - 1) / C::TN;
-    const int m_tiles = (pb.m_end - pb.m_begin + C::TM - 1) / C::TM;
-    const int grid = (n_tiles + 7) / 8 * 8 * m_tiles;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(C::THREADS), C::LDS, s, pb, n_tiles, m_tiles);
-    return hipGetLastError() == hipSuccess ? C::TM : 0;
-}
-
-template <int TT, int WM>
-static int launch_moe(const MmqProblem& pb, const uint8_t* w_second, int64_t dst_second, const int32_t* bounds,
-                      int64_t stride_expert, int n_experts, int64_t ncols_max, hipStream_t s) {
-    using C = Wide<TT, WM>;
-    auto kernel = q4k_f16_moe_kernel<TT, WM>;
-    if (mmq_prepare_kernel(kernel, C::LDS) != LK_OK) return 0;
-    const int64_t col_tiles = (ncols_max + C::TM - 1) / C::TM;
-    const dim3 grid((pb.n + C::TN - 1) / C::TN, (unsigned)(col_tiles < 1 ? 1 : (col_tiles > 65535 ? 65535 : col_tiles)),
-                    (unsigned)((w_second ? 2 : 1) * n_experts));
-    hipLaunchKernelGGL(kernel, grid, dim3(C::THREADS), C::LDS, s, pb, w_second, dst_second, bounds, stride_expert,
-                       n_experts);
-    return hipGetLastError() == hipSuccess ? C::TM : 0;
 }
 
 }  // namespace
 
 int lk_mmq_q4k_f16_dense(const MmqProblem& pb, hipStream_t s) {
+    using C = Wide;
     if (((uintptr_t)pb.w | (uintptr_t)pb.y) % 16 != 0 || pb.rows_total > (1 << 23)) return -1;
-    return launch_dense<2, 2>(pb, s);
+    if (mmq_prepare_kernel(q4k_f16_dense_kernel, C::LDS) != LK_OK) return 0;
+    const int n_tiles = (pb.n + C::TN - 1) / C::TN;
+    const int m_tiles = (pb.m_end - pb.m_begin + C::TM - 1) / C::TM;
+    const int grid = (n_tiles + 7) / 8 * 8 * m_tiles;
+    hipLaunchKernelGGL(q4k_f16_dense_kernel, dim3(grid), dim3(C::THREADS), C::LDS, s, pb, n_tiles, m_tiles);
+    return hipGetLastError() == hipSuccess ? C::TM : 0;
 }
 
 int lk_mmq_q4k_f16_moe(const MmqProblem& pb, const uint8_t* w_second, int64_t dst_second, const int32_t* bounds,
                        int64_t stride_expert, int n_experts, int64_t ncols_max, hipStream_t s) {
+    using C = Wide;
     if (((uintptr_t)pb.w | (uintptr_t)pb.y | (uintptr_t)w_second) % 16 != 0 || stride_expert % 16 != 0 ||
         pb.rows_total > (1 << 23))
         return -1;
-    return launch_moe<2, 2>(pb, w_second, dst_second, bounds, stride_expert, n_experts, ncols_max, s);
+    if (mmq_prepare_kernel(q4k_f16_moe_kernel, C::LDS) != LK_OK) return 0;
+    const int64_t col_tiles = (ncols_max + C::TM - 1) / C::TM;
+    const dim3 grid((pb.n + C::TN - 1) / C::TN, (unsigned)(col_tiles < 1 ? 1 : (col_tiles > 65535 ? 65535 : col_tiles)),
+                    (unsigned)((w_second ? 2 : 1) * n_experts));
+    hipLaunchKernelGGL(q4k_f16_moe_kernel, grid, dim3(C::THREADS), C::LDS, s, pb, w_second, dst_second, bounds,
+                       stride_expert, n_experts);
+    return hipGetLastError() == hipSuccess ? C::TM : 0;
 }
