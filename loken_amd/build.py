@@ -20,7 +20,8 @@ FLAGS = [
 ]
 # MFMA results are consumed by VALU fix-ups right away: keep them in VGPRs instead of the
 # accumulator file, which would cost one v_accvgpr_read per value.
-PER_FILE_FLAGS = {"mmq.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+_VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
+PER_FILE_FLAGS = {"mmq.hip": _VGPR_FORM, "mmq_q4k_f16.hip": _VGPR_FORM}
 
 
 def sources() -> list[Path]:
