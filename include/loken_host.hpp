@@ -12,6 +12,10 @@
 
 #include <stdint.h>
 
+#include <string>
+#include <unordered_map>
+#include <vector>
+
 #include "loken_gfx950.h"
 
 namespace loken {
@@ -56,6 +60,102 @@ private:
 /* Frees every workspace this layer holds on every device (synchronizes those devices). */
 void release_workspaces();
 
+/* ------------------------------------------------------------------------------------------
+ * GGUF container reader and weight upload (loken's src/tensor/quantized/gguf_file.rs; the upload
+ * rule of kernel_matmul.rs:218-236 and cuda_storage.rs:27-39).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Metadata value types, by the id the file stores (gguf_file.rs:45-60). */
+enum class GgufType : int {
+    U8 = 0, I8 = 1, U16 = 2, I16 = 3, U32 = 4, I32 = 5, F32 = 6, Bool = 7, String = 8, Array = 9,
+    U64 = 10, I64 = 11, F64 = 12,
+};
+
+struct GgufValue {
+    GgufType type = GgufType::U8;
+    GgufType elem_type = GgufType::U8;   /* of an Array */
+    uint64_t u = 0;                      /* unsigned kinds and Bool */
+    int64_t i = 0;                       /* signed kinds */
+    double f = 0;                        /* F32 (widened) and F64 */
+    std::string s;
+    std::vector<GgufValue> items;
+
+    /* The reference's conversions (gguf_file.rs:314-357): any whole-number kind that fits; to_i64
+     * refuses a U64 whatever its value; floats convert among themselves only. False = not that. */
+    bool to_u64(uint64_t* out) const;
+    bool to_i64(int64_t* out) const;
+    bool to_f64(double* out) const;
+};
+
+struct GgufTensor {
+    std::string name;
+    std::vector<int64_t> dims;   /* row-major: the file's order reversed */
+    int dtype = 0;               /* block type id, as LK_TYPE_* where those exist */
+    uint64_t offset = 0;         /* from the aligned start of the payload */
+    uint64_t bytes = 0;          /* elements / block values * block bytes */
+    uint64_t elements() const;
+};
+
+/* What a model listing needs from a header without reading a tensor (gguf_file.rs:575-708).
+ * -1 = the file does not say. */
+struct GgufFacts {
+    bool has_architecture = false;
+    std::string architecture;
+    int64_t file_type = -1;
+    int64_t parameter_count = -1;   /* declared, else the sum over the tensor directory */
+    bool pools = false;             /* `<architecture>.pooling_type` is present */
+    int64_t split_parts = -1;
+};
+
+class GgufFile {
+public:
+    /* Maps `path` read-only and parses its header; nullptr and a message on any failure. */
+    static GgufFile* open(const char* path, std::string* error);
+    /* Parses an image the caller keeps alive (a mapping of its own, a test's bytes). */
+    static GgufFile* over(const void* bytes, uint64_t len, std::string* error);
+    ~GgufFile();
+
+    int version() const { return version_; }
+    uint64_t alignment() const { return alignment_; }
+    uint64_t data_offset() const { return data_offset_; }   /* first multiple of alignment after the directory */
+
+    int kv_count() const { return (int)keys_.size(); }       /* in file order */
+    const std::string& key(int index) const { return keys_[index]; }
+    const GgufValue& value(int index) const { return values_[index]; }
+    int find_key(const char* key) const;                     /* -1: absent */
+
+    int tensor_count() const { return (int)tensors_.size(); }
+    const GgufTensor& tensor(int index) const { return tensors_[index]; }
+    int find_tensor(const char* name) const;                 /* -1: absent */
+    /* The tensor's blocks inside the image; nullptr when the directory points past its end. */
+    const void* tensor_data(int index) const;
+
+    GgufFacts facts() const;
+    const GgufFacts& cached_facts() {
+        if (!facts_ready_) { facts_ = facts(); facts_ready_ = true; }
+        return facts_;
+    }
+
+    /* Device copy the kernels take: hipMalloc of bytes + 4096 on `device`, the tail zeroed, the
+     * blocks copied on `stream`; returns after the copy has left the host. nullptr on failure.
+     * The caller frees it (hipFree / lkh_gguf_free_blob). */
+    void* upload(int index, int device, void* stream, uint64_t* blob_bytes) const;
+
+private:
+    GgufFile();
+    bool parse(std::string* error);
+    struct Image;
+    Image* image_;
+    int version_ = 0;
+    uint64_t alignment_ = 32, data_offset_ = 0;
+    std::vector<std::string> keys_;
+    std::vector<GgufValue> values_;
+    std::unordered_map<std::string, int> kv_index_, tensor_index_;
+    std::vector<GgufTensor> tensors_;
+    GgufFacts facts_;
+    bool facts_ready_ = false;
+};
+
 }  // namespace loken
 
 /* The same through plain C, for callers and tests that bind by symbol. */
@@ -67,6 +167,39 @@ int lkh_qkernel_matmul_forward(void* handle, const void* x, int x_type, int rows
 int lkh_qkernel_matmul_last_path(void* handle);
 int lkh_matvec_rows(int dtype, int k);
 void lkh_release_workspaces(void);
+
+/* GgufFile by handle. `err` (nullable, `err_len` bytes) receives the message when a call that
+ * returns a handle returns NULL. Strings returned through `const char**` live as long as the
+ * handle. Status returns are LK_OK or LK_ERR_ARG (no such handle / index) / LK_ERR_TYPE (the value
+ * is not of the kind asked for). */
+void* lkh_gguf_open(const char* path, char* err, int err_len);
+void* lkh_gguf_over(const void* bytes, uint64_t len, char* err, int err_len);
+void lkh_gguf_close(void* g);
+int lkh_gguf_layout(void* g, int* version, uint64_t* alignment, uint64_t* data_offset, int* tensor_count,
+                    int* kv_count);
+int lkh_gguf_find_tensor(void* g, const char* name);
+int lkh_gguf_tensor(void* g, int index, const char** name, int* dtype, int* n_dims, int64_t* dims, int max_dims,
+                    uint64_t* offset, uint64_t* bytes);
+void* lkh_gguf_tensor_data(void* g, int index);
+int lkh_gguf_find_key(void* g, const char* key);
+int lkh_gguf_kv(void* g, int index, const char** key, int* type, int* elem_type, uint64_t* count);
+int lkh_gguf_kv_u64(void* g, int index, uint64_t* out);
+int lkh_gguf_kv_i64(void* g, int index, int64_t* out);
+int lkh_gguf_kv_f64(void* g, int index, double* out);
+int lkh_gguf_kv_bool(void* g, int index, int* out);
+int lkh_gguf_kv_str(void* g, int index, const char** out, uint64_t* len);
+int lkh_gguf_kv_item_u64(void* g, int index, uint64_t i, uint64_t* out);
+int lkh_gguf_kv_item_i64(void* g, int index, uint64_t i, int64_t* out);
+int lkh_gguf_kv_item_f64(void* g, int index, uint64_t i, double* out);
+int lkh_gguf_kv_item_str(void* g, int index, uint64_t i, const char** out, uint64_t* len);
+int lkh_gguf_facts(void* g, const char** architecture, int64_t* file_type, int64_t* parameter_count, int* pools,
+                   int64_t* split_parts);
+void* lkh_gguf_upload(void* g, int index, int device, void* stream, uint64_t* blob_bytes);
+void lkh_gguf_free_blob(void* blob);
+/* Tensor `name` (2-D, Q4_K / Q6_K / Q8_0) uploaded to `device` and wrapped as a QKernelMatMul
+ * handle (QKernelMatMul::from_qtensor_on, kernel_matmul.rs:213-275); `*blob` receives the device
+ * allocation, which the caller frees after the handle. */
+void* lkh_gguf_linear(void* g, const char* name, int device, void* stream, void** blob, char* err, int err_len);
 }
 
 #endif

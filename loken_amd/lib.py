@@ -23,6 +23,7 @@ class LokenError(RuntimeError):
 
 
 _vp, _i, _i64, _f = C.c_void_p, C.c_int, C.c_int64, C.c_float
+_cp, _u64 = C.c_char_p, C.c_uint64
 
 # name -> (restype, argtypes); mirrors include/loken_gfx950.h declaration by declaration
 SIGNATURES = {
@@ -61,6 +62,28 @@ SIGNATURES.update({
     "lkh_qkernel_matmul_last_path": (_i, [_vp]),
     "lkh_matvec_rows": (_i, [_i, _i]),
     "lkh_release_workspaces": (None, []),
+    "lkh_gguf_open": (_vp, [_cp, _vp, _i]),
+    "lkh_gguf_over": (_vp, [_vp, _u64, _vp, _i]),
+    "lkh_gguf_close": (None, [_vp]),
+    "lkh_gguf_layout": (_i, [_vp] * 6),
+    "lkh_gguf_find_tensor": (_i, [_vp, _cp]),
+    "lkh_gguf_tensor": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
+    "lkh_gguf_tensor_data": (_vp, [_vp, _i]),
+    "lkh_gguf_find_key": (_i, [_vp, _cp]),
+    "lkh_gguf_kv": (_i, [_vp, _i, _vp, _vp, _vp, _vp]),
+    "lkh_gguf_kv_u64": (_i, [_vp, _i, _vp]),
+    "lkh_gguf_kv_i64": (_i, [_vp, _i, _vp]),
+    "lkh_gguf_kv_f64": (_i, [_vp, _i, _vp]),
+    "lkh_gguf_kv_bool": (_i, [_vp, _i, _vp]),
+    "lkh_gguf_kv_str": (_i, [_vp, _i, _vp, _vp]),
+    "lkh_gguf_kv_item_u64": (_i, [_vp, _i, _u64, _vp]),
+    "lkh_gguf_kv_item_i64": (_i, [_vp, _i, _u64, _vp]),
+    "lkh_gguf_kv_item_f64": (_i, [_vp, _i, _u64, _vp]),
+    "lkh_gguf_kv_item_str": (_i, [_vp, _i, _u64, _vp, _vp]),
+    "lkh_gguf_facts": (_i, [_vp] * 6),
+    "lkh_gguf_upload": (_vp, [_vp, _i, _i, _vp, _vp]),
+    "lkh_gguf_free_blob": (None, [_vp]),
+    "lkh_gguf_linear": (_vp, [_vp, _cp, _i, _vp, _vp, _vp, _i]),
     "loken_topk_softmax": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "loken_dense_q4k_imma_m8_plain": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "loken_moe_mmq_fold": (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
