@@ -108,6 +108,33 @@ int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, const void* vy
                      int dst_type, int ncols_x, int nrows_x, int batch, int stride_col_y,
                      int stride_col_dst, int act, void* stream);
 
+/* Decode-step producers that end in the activation a mat-vec reads: the f32 row is written as
+ * before and the same row leaves as Q8_1 blocks (`vy`: rows * cols / 32 blocks of 36 bytes, byte
+ * for byte what lk_quantize_q8_1 makes of the f32 row), so the mat-vec that follows needs no
+ * quantizer launch. rows x cols f32, contiguous; cols a multiple of 512 (the quantized row has no
+ * padding), one workgroup per row. Sum of squares as the reference's wide kernels fold it (lane t
+ * of 256 over t, t + 256, ..., then a stride-halving tree); rms = 1 / sqrt(mean + eps), correctly
+ * rounded, where the reference takes the card's rsqrtf approximation.
+ * Replace kernels `rmsnorm_wide_q8_1_f32`, `add_rmsnorm_dual_wide_q8_1_f32` and
+ * `post_norm_add_norm_wide_q8_1_f32` (src/inference/cuda/mmvq_gguf.cu:805-936) with their launch
+ * sites rms_norm_f32 (src/tensor/cuda/gemm.rs:561-590) and fused_post_norm_add_norm /
+ * fused_add_rmsnorm_dual (src/inference/kernel/fused/buffers/conv.rs:990-1110). */
+int lk_rmsnorm_q8_1(const float* x, const float* weight, float* out, void* vy, float eps, int cols, int rows,
+                    void* stream);
+/* sum_out = x + residual; norm_out = rmsnorm(sum_out, weight), also as Q8_1. */
+int lk_add_rmsnorm_q8_1(const float* x, const float* residual, const float* weight, float* sum_out,
+                        float* norm_out, void* vy, float eps, int cols, int rows, void* stream);
+/* x_out = rmsnorm(a, w_post) + residual (each product rounded before it is added);
+ * norm_out = rmsnorm(x_out, w_ffn), also as Q8_1. */
+int lk_post_norm_add_norm_q8_1(const float* a, const float* w_post, const float* residual, const float* w_ffn,
+                               float* x_out, float* norm_out, void* vy, float eps_post, float eps_ffn, int cols,
+                               int rows, void* stream);
+/* out[r, i] = act(gu[r, i]) * gu[r, n + i] for rows of 2 n values (gate then up), also as Q8_1;
+ * act 0 = SiLU g / (1 + exp(-g)), 1 = tanh-GELU; n a multiple of 32. Replaces kernels
+ * `split_silu_mul_q8_1_f32` / `split_gelu_mul_q8_1_f32` (src/inference/cuda/mmvq_gguf.cu:971-999;
+ * launched from src/inference/kernel/fused/buffers/conv.rs:735,834), which take one row. */
+int lk_split_act_mul_q8_1(const float* gu, float* out, void* vy, int n, int rows, int act, void* stream);
+
 /* The gate/up pair launch that hands its result on as Q8_1: dst = Q8_1(act(gate . x) * (up . x)),
  * blocks of 32 consecutive output rows, written with lk_quantize_q8_1's rule, so the down
  * projection of a decode layer reads it without a quantizer launch in between (the fused

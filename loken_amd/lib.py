@@ -55,6 +55,10 @@ SIGNATURES.update({
     "loken_moe_gemm_gguf_down_reduce": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp, _vp]),
     "loken_moe_sum_topk": (None, [_vp, _vp, _i, _i, _i, _vp]),
     "loken_stream_scratch_release": (None, []),
+    "lk_rmsnorm_q8_1": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _vp]),
+    "lk_add_rmsnorm_q8_1": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _i, _i, _vp]),
+    "lk_post_norm_add_norm_q8_1": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _i, _i, _vp]),
+    "lk_split_act_mul_q8_1": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "lk_mmvq_pair_act_q8_1": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp, _i, _i, _i, _i, _i, _vp]),
     "lkh_qkernel_matmul_new": (_vp, [_i, _i, _i, _vp, _i]),
     "lkh_qkernel_matmul_free": (None, [_vp]),

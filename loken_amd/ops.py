@@ -37,6 +37,51 @@ def quantize_q8_1_rows(x: torch.Tensor, k_padded: int | None = None) -> torch.Te
     return out
 
 
+def _q8_1_rows(rows: int, cols: int, device) -> torch.Tensor:
+    return torch.empty((rows, cols // 32, 36), dtype=torch.uint8, device=device)
+
+
+def rmsnorm_q8_1(x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """rms_norm_f32 with the row also quantized (src/tensor/cuda/gemm.rs:561-590) -> (out, q8_1)."""
+    rows, cols = x.shape
+    out, q = torch.empty_like(x), _q8_1_rows(rows, cols, x.device)
+    _lib.check("lk_rmsnorm_q8_1", _lib.load().lk_rmsnorm_q8_1(
+        x.data_ptr(), weight.data_ptr(), out.data_ptr(), q.data_ptr(), eps, cols, rows, _stream()))
+    return out, q
+
+
+def add_rmsnorm_q8_1(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float):
+    """fused_add_rmsnorm_dual (src/inference/kernel/fused/buffers/conv.rs:1043-1110) -> (sum, norm, q8_1)."""
+    rows, cols = x.shape
+    total, out, q = torch.empty_like(x), torch.empty_like(x), _q8_1_rows(rows, cols, x.device)
+    _lib.check("lk_add_rmsnorm_q8_1", _lib.load().lk_add_rmsnorm_q8_1(
+        x.data_ptr(), residual.data_ptr(), weight.data_ptr(), total.data_ptr(), out.data_ptr(), q.data_ptr(), eps,
+        cols, rows, _stream()))
+    return total, out, q
+
+
+def post_norm_add_norm_q8_1(a: torch.Tensor, w_post: torch.Tensor, residual: torch.Tensor, w_ffn: torch.Tensor,
+                            eps_post: float, eps_ffn: float):
+    """fused_post_norm_add_norm (src/inference/kernel/fused/buffers/conv.rs:975-1035) -> (x, norm, q8_1)."""
+    rows, cols = a.shape
+    x_out, out, q = torch.empty_like(a), torch.empty_like(a), _q8_1_rows(rows, cols, a.device)
+    _lib.check("lk_post_norm_add_norm_q8_1", _lib.load().lk_post_norm_add_norm_q8_1(
+        a.data_ptr(), w_post.data_ptr(), residual.data_ptr(), w_ffn.data_ptr(), x_out.data_ptr(), out.data_ptr(),
+        q.data_ptr(), eps_post, eps_ffn, cols, rows, _stream()))
+    return x_out, out, q
+
+
+def split_act_mul_q8_1(gu: torch.Tensor, act: int = 0):
+    """``[rows, 2 n]`` gate|up -> (act(gate) * up ``[rows, n]``, its Q8_1 rows); act 0 SiLU, 1 tanh-GELU."""
+    rows, two_n = gu.shape
+    n = two_n // 2
+    out = torch.empty((rows, n), dtype=torch.float32, device=gu.device)
+    q = _q8_1_rows(rows, n, gu.device)
+    _lib.check("lk_split_act_mul_q8_1", _lib.load().lk_split_act_mul_q8_1(
+        gu.data_ptr(), out.data_ptr(), q.data_ptr(), n, rows, act, _stream()))
+    return out, q
+
+
 def mmvq(wtype: int, weight: torch.Tensor, q8_1: torch.Tensor, k: int, n: int, *,
          out_dtype: torch.dtype = torch.float32, bias: torch.Tensor | None = None,
          decode_order: bool = False) -> torch.Tensor:

@@ -67,6 +67,12 @@ def _declare(l: C.CDLL) -> None:
     l.lko_group_by_expert.restype = None
     l.lko_moe_forward.argtypes = [_i, _i, _i, _sz, _sz, _sz, _sz, _sz] + [_vp] * 8
     l.lko_cpu_has_avx2.restype = _i
+    l.lko_inv_rms_wide.restype = C.c_float
+    l.lko_inv_rms_wide.argtypes = [_vp, _sz, C.c_float]
+    l.lko_norm_rows.restype = None
+    l.lko_norm_rows.argtypes = [_i, _vp, _vp, _vp, _vp, _vp, _vp, C.c_float, C.c_float, _sz, _sz]
+    l.lko_split_act_mul.restype = None
+    l.lko_split_act_mul.argtypes = [_vp, _vp, _sz, _sz, _i]
 
 
 def _p(a: np.ndarray) -> int:
@@ -228,3 +234,31 @@ def moe_forward(family: int, dt_gu: int, dt_down: int, x, gate, up, down, ids, w
                                  _p(x), _p(gate), _p(up), _p(down), _p(ids), _p(weights),
                                  _p(h) if want_h else None, _p(out)))
     return (out, h) if want_h else out
+
+
+def inv_rms_wide(row, eps: float) -> float:
+    row = _f32(row).reshape(-1)
+    return float(lib().lko_inv_rms_wide(_p(row), row.size, eps))
+
+
+def norm_rows(mode: int, x, w, *, w_first=None, residual=None, eps: float = 1e-6, eps_first: float = 1e-6):
+    """mode 0 -> out; mode 1 (add then norm) and 2 (norm, add, norm) -> (mid, out)."""
+    x = _f32(x)
+    rows, cols = x.shape
+    w = _f32(w)
+    w_first = _f32(w_first) if w_first is not None else None
+    residual = _f32(residual) if residual is not None else None
+    out = np.empty_like(x)
+    mid = np.empty_like(x) if mode else None
+    lib().lko_norm_rows(mode, _p(x), _p(w_first) if w_first is not None else None,
+                        _p(residual) if residual is not None else None, _p(w), _p(mid) if mode else None, _p(out),
+                        eps_first, eps, cols, rows)
+    return (mid, out) if mode else out
+
+
+def split_act_mul(gu, act: int = 0) -> np.ndarray:
+    gu = _f32(gu)
+    rows, two_n = gu.shape
+    out = np.empty((rows, two_n // 2), np.float32)
+    lib().lko_split_act_mul(_p(gu), _p(out), two_n // 2, rows, act)
+    return out

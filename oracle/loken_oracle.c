@@ -756,3 +756,59 @@ int lko_moe_forward(int family, int dt_gu, int dt_down, size_t tokens, size_t hi
     free(slots); free(experts); free(xq); free(h); free(hq);
     return 0;
 }
+
+/* ------------------------------------------------------------------------------------------
+ * Decode-step producers (RMSNorm family, split activation): src/inference/cuda/mmvq_gguf.cu.
+ * ---------------------------------------------------------------------------------------- */
+
+float lko_inv_rms_wide(const float* row, size_t cols, float eps) {
+    float tree[256];
+    for (size_t t = 0; t < 256; ++t) {          /* :811-817, the build contracts sum += v * v */
+        float part = 0.0f;
+        for (size_t i = t; i < cols; i += 256) part = fmaf(row[i], row[i], part);
+        tree[t] = part;
+    }
+    for (size_t s = 128; s > 0; s >>= 1)        /* :820-823 */
+        for (size_t t = 0; t < s; ++t) tree[t] += tree[t + s];
+    return 1.0f / sqrtf(tree[0] / (float)cols + eps);
+}
+
+void lko_norm_rows(int mode, const float* x, const float* w_first, const float* residual, const float* w,
+                   float* mid, float* out, float eps_first, float eps, size_t cols, size_t rows) {
+    float* srow = (float*)malloc(sizeof(float) * cols);
+    for (size_t r = 0; r < rows; ++r) {
+        const size_t off = r * cols;
+        for (size_t i = 0; i < cols; ++i) {
+            float v = x[off + i];
+            if (mode == 1) { v = v + residual[off + i]; mid[off + i] = v; }
+            srow[i] = v;
+        }
+        if (mode == 2) {
+            const float rms_first = lko_inv_rms_wide(srow, cols, eps_first);
+            for (size_t i = 0; i < cols; ++i) {
+                const float y = (srow[i] * rms_first) * w_first[i];   /* :914-916 */
+                const float xr = y + residual[off + i];
+                srow[i] = xr;
+                mid[off + i] = xr;
+            }
+        }
+        const float rms = lko_inv_rms_wide(srow, cols, eps);
+        for (size_t i = 0; i < cols; ++i) out[off + i] = (srow[i] * rms) * w[i];
+    }
+    free(srow);
+}
+
+void lko_split_act_mul(const float* gu, float* out, size_t n, size_t rows, int act) {
+    for (size_t r = 0; r < rows; ++r)
+        for (size_t i = 0; i < n; ++i) {
+            const float g = gu[r * 2 * n + i], u = gu[r * 2 * n + n + i];
+            float a;
+            if (act == 0) {
+                a = g / (1.0f + expf(-g));
+            } else {
+                const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+                a = 0.5f * g * (1.0f + tanhf(k0 * (g + k1 * g * g * g)));
+            }
+            out[r * n + i] = a * u;
+        }
+}

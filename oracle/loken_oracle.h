@@ -112,6 +112,20 @@ int lko_moe_forward(int family, int dtype_gate_up, int dtype_down, size_t tokens
                     const uint8_t* gate, const uint8_t* up, const uint8_t* down,
                     const int32_t* ids, const float* weights, float* h_sorted, float* out);
 
+/* ---- decode-step producers that end in a Q8_1 row (src/inference/cuda/mmvq_gguf.cu:789-999) ---- */
+/* 1 / sqrt(mean of squares + eps) as the wide norm kernels accumulate it (:811-829): lane t of 256
+ * folds the squares of values t, t + 256, ... with a fused multiply-add, the 256 partial sums fold
+ * as a stride-halving tree. The reciprocal square root is 1 / sqrtf, both correctly rounded (the
+ * reference's rsqrtf approximation has no portable bits). */
+float lko_inv_rms_wide(const float* row, size_t cols, float eps);
+/* mode 0: out = (x * rms) * w (:805-837). mode 1: mid = x + residual, out = rmsnorm(mid, w)
+ * (:839-877). mode 2: mid = (x * rms_first) * w_first + residual, each product rounded before it
+ * is added; out = rmsnorm(mid, w) (:879-936). rows x cols; unused pointers may be NULL. */
+void lko_norm_rows(int mode, const float* x, const float* w_first, const float* residual, const float* w,
+                   float* mid, float* out, float eps_first, float eps, size_t cols, size_t rows);
+/* out[r, i] = act(gu[r, i]) * gu[r, n + i]; act 0 = g / (1 + exp(-g)), 1 = tanh-GELU (:971-999). */
+void lko_split_act_mul(const float* gu, float* out, size_t n, size_t rows, int act);
+
 /* ---- timed CPU baseline (cpu_baseline.c): O-A semantics, AVX2 kernels, worker pool ---- */
 int lko_cpu_has_avx2(void);
 int oa_matmul_fast(int dtype, size_t m, size_t k, size_t n, const float* lhs,
