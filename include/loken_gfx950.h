@@ -9,7 +9,7 @@
  * Each declaration cites the reference interface (loken, paths relative to its root) it
  * stands in for. Two groups:
  *   * names and signatures kept verbatim where loken links a launcher statically
- *     (launch_mmq_*, loken_moe_*): src/tensor/quantized/mmq.rs, src/inference/moe_cuda/*.rs;
+ *     (launch_mmq_*, loken_moe_*): src/tensor/quantized/mmq.rs, src/inference/moe_cuda/ (*.rs);
  *   * lk_* launchers where loken fetches a kernel BY NAME from a run-time-compiled module and
  *     launches it with a (32, nwarps) block (src/tensor/cuda/quant.rs:3581-3684): a wave64
  *     kernel cannot honour that block contract, so the launch geometry moves behind the ABI.
@@ -314,6 +314,30 @@ void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* outpu
  * launched outside that (the caller falls back). */
 void loken_topk_softmax(const float* logits, float* weights, uint32_t* ids, int n_rows, int n_experts,
                         int n_expert_used, int with_norm, void* stream);
+/* Gate mat-vec + softmax + top-k of each token in one launch: logits = gate_w [n_experts, hidden]
+ * f32 . x [n_rows, hidden] f32, then the selection of loken_topk_softmax. A token has a workgroup
+ * of 16 waves whose lanes walk each weight row together, so a logit is a 64-lane f32 sum (the
+ * reference's is one lane's serial sum: same value up to summation order). Name and arguments of
+ * the reference's launcher (cuda/moe/gate_topk.cu:366-403; called from
+ * src/inference/moe_cuda/dense/gate.rs:51). hidden up to 8192, up to 512 experts (the reference:
+ * 32/64/128/256); nothing is launched outside that (the caller falls back). */
+void loken_gate_topk_softmax(const float* x_in, const float* gate_w, float* weights_out, uint32_t* ids_out,
+                             int hidden, int n_rows, int n_experts, int n_expert_used, int with_norm, void* stream);
+/* Sigmoid router over logits [n_rows, n_experts]: p = 1 / (1 + exp(-logit)); the n_expert_used
+ * experts with the largest p + bias[expert] (bias nullable; ties to the lower id), weights = the
+ * unbiased p, divided by max(their sum, 2^-14) when with_norm != 0, then times `scale`. Name and
+ * arguments of the reference's launcher (cuda/moe/gate_topk.cu:140-200, 479-512; called from
+ * src/inference/moe_cuda/dense/gate.rs:133). exp is the accurate one (the reference's is the fast
+ * intrinsic). */
+void loken_topk_sigmoid_post(const float* logits_in, const float* bias, float* weights_out, uint32_t* ids_out,
+                             int n_rows, int n_experts, int n_expert_used, int with_norm, float scale, void* stream);
+/* Stable ascending sort of n u32 keys by rank: sorted[r] = the key, order[r] = the index it came
+ * from; equal keys keep their order. Groups the routing's (token, choice) pairs by expert on the
+ * device (cuda/moe/gate_topk.cu:515-548; called from src/inference/moe_cuda/routing.rs:223). */
+void loken_stable_sort_u32(const uint32_t* keys, uint32_t* sorted, uint32_t* order, int n, void* stream);
+/* The decode-size form (cuda/moe/gate_topk.cu:453-477; src/inference/moe_cuda/dense/gate.rs:185):
+ * same result for m keys; the reference serves m <= 32, this m <= 256, nothing is launched above. */
+void loken_argsort_small_u32(const uint32_t* in, uint32_t* sorted_out, uint32_t* index_out, int m, void* stream);
 /* Frees the current device's MoE decode scratch (cuda/moe/moe_gguf.cu:104-118). Synchronizes. */
 void loken_stream_scratch_release(void);
 

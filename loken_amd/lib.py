@@ -88,6 +88,10 @@ SIGNATURES.update({
     "lkh_gguf_upload": (_vp, [_vp, _i, _i, _vp, _vp]),
     "lkh_gguf_free_blob": (None, [_vp]),
     "lkh_gguf_linear": (_vp, [_vp, _cp, _i, _vp, _vp, _vp, _i]),
+    "loken_gate_topk_softmax": (None, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "loken_topk_sigmoid_post": (None, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _vp]),
+    "loken_stable_sort_u32": (None, [_vp, _vp, _vp, _i, _vp]),
+    "loken_argsort_small_u32": (None, [_vp, _vp, _vp, _i, _vp]),
     "loken_topk_softmax": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "loken_dense_q4k_imma_m8_plain": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "loken_moe_mmq_fold": (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),

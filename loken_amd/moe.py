@@ -202,6 +202,51 @@ def topk_softmax(logits: torch.Tensor, topk: int, renorm: bool = True):
     return weights, ids
 
 
+def _router_out(tokens: int, topk: int, device):
+    return (torch.empty((tokens, topk), dtype=torch.float32, device=device),
+            torch.empty((tokens, topk), dtype=torch.int32, device=device))
+
+
+def gate_topk_softmax(x: torch.Tensor, gate_w: torch.Tensor, topk: int, renorm: bool = True):
+    """Gate mat-vec + softmax + top-k in one launch: ``x [tokens, hidden]`` f32, ``gate_w [experts,
+    hidden]`` f32 -> (weights, choices) as ``topk_softmax`` (gate_topk_softmax,
+    src/inference/moe_cuda/dense/gate.rs:20-75)."""
+    tokens, hidden = x.shape
+    experts = gate_w.shape[0]
+    if hidden > 8192 or experts > 512 or topk > 64 or topk > experts or gate_w.shape[1] != hidden:
+        raise ValueError("gate_topk_softmax: hidden <= 8192, at most 512 experts and 64 choices")
+    weights, ids = _router_out(tokens, topk, x.device)
+    _lib.load().loken_gate_topk_softmax(x.data_ptr(), gate_w.data_ptr(), weights.data_ptr(), ids.data_ptr(), hidden,
+                                        tokens, experts, topk, int(renorm), _stream())
+    return weights, ids
+
+
+def topk_sigmoid_post(logits: torch.Tensor, topk: int, bias: torch.Tensor | None = None, renorm: bool = True,
+                      scale: float = 1.0):
+    """Sigmoid router: chosen on probability + bias, weighted by the probability alone
+    (topk_sigmoid_post, src/inference/moe_cuda/dense/gate.rs:100-160)."""
+    tokens, experts = logits.shape
+    if experts > 512 or topk > 64 or topk > experts:
+        raise ValueError("topk_sigmoid_post: at most 512 experts and 64 choices")
+    weights, ids = _router_out(tokens, topk, logits.device)
+    _lib.load().loken_topk_sigmoid_post(logits.data_ptr(), bias.data_ptr() if bias is not None else None,
+                                        weights.data_ptr(), ids.data_ptr(), tokens, experts, topk, int(renorm), scale,
+                                        _stream())
+    return weights, ids
+
+
+def stable_sort_u32(keys: torch.Tensor, small: bool = False):
+    """-> (sorted keys, the index each came from), equal keys in their original order
+    (loken_stable_sort_u32 / loken_argsort_small_u32, src/inference/moe_cuda/routing.rs:200-242)."""
+    n = keys.numel()
+    if small and n > 256:
+        raise ValueError("argsort_small: at most 256 keys")
+    out, order = torch.empty_like(keys), torch.empty_like(keys)
+    fn = _lib.load().loken_argsort_small_u32 if small else _lib.load().loken_stable_sort_u32
+    fn(keys.data_ptr(), out.data_ptr(), order.data_ptr(), n, _stream())
+    return out, order
+
+
 def moe_mmq_pays(rows: int, experts: int) -> bool:
     """Routed rows from which the expert-batched matmul beats the per-pair kernels. The reference
     breaks even at one routed row per expert (mmq_experts.rs:72-86); on MI355X, with this

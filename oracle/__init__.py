@@ -63,6 +63,8 @@ def _declare(l: C.CDLL) -> None:
     l.ob_matmul_f64.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp]
     l.lko_topk_softmax.argtypes = [_vp, _sz, _sz, _sz, _i, _vp, _vp]
     l.lko_topk_softmax.restype = None
+    l.lko_topk_sigmoid.argtypes = [_vp, _vp, _sz, _sz, _sz, _i, C.c_float, _vp, _vp]
+    l.lko_topk_sigmoid.restype = None
     l.lko_group_by_expert.argtypes = [_vp, _sz, _vp, _vp]
     l.lko_group_by_expert.restype = None
     l.lko_moe_forward.argtypes = [_i, _i, _i, _sz, _sz, _sz, _sz, _sz] + [_vp] * 8
@@ -262,3 +264,14 @@ def split_act_mul(gu, act: int = 0) -> np.ndarray:
     out = np.empty((rows, two_n // 2), np.float32)
     lib().lko_split_act_mul(_p(gu), _p(out), two_n // 2, rows, act)
     return out
+
+
+def topk_sigmoid(logits, topk: int, bias=None, renorm: bool = True, scale: float = 1.0):
+    logits = _f32(logits)
+    t, e = logits.shape
+    bias = _f32(bias) if bias is not None else None
+    ids = np.empty((t, topk), np.int32)
+    w = np.empty((t, topk), np.float32)
+    lib().lko_topk_sigmoid(_p(logits), _p(bias) if bias is not None else None, t, e, topk, int(renorm), scale,
+                           _p(ids), _p(w))
+    return ids, w

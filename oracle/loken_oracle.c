@@ -812,3 +812,29 @@ void lko_split_act_mul(const float* gu, float* out, size_t n, size_t rows, int a
             out[r * n + i] = a * u;
         }
 }
+
+void lko_topk_sigmoid(const float* logits, const float* bias, size_t tokens, size_t n_experts, size_t topk,
+                      int renorm, float scale, int32_t* ids, float* weights) {
+    float* p = (float*)malloc(sizeof(float) * n_experts);
+    float* sel = (float*)malloc(sizeof(float) * n_experts);
+    for (size_t t = 0; t < tokens; ++t) {
+        const float* row = logits + t * n_experts;
+        for (size_t e = 0; e < n_experts; ++e) {
+            p[e] = 1.0f / (1.0f + expf(-row[e]));
+            sel[e] = p[e] + (bias ? bias[e] : 0.0f);
+        }
+        float sum = 0.0f;
+        for (size_t j = 0; j < topk; ++j) {
+            size_t best = 0;
+            for (size_t e = 1; e < n_experts; ++e)
+                if (sel[e] > sel[best]) best = e;          /* strict: the lower index wins a tie */
+            ids[t * topk + j] = (int32_t)best;
+            weights[t * topk + j] = p[best];
+            sum += p[best];
+            sel[best] = -INFINITY;
+        }
+        const float inv = renorm ? 1.0f / fmaxf(sum, 6.103515625e-5f) : 1.0f;
+        for (size_t j = 0; j < topk; ++j) weights[t * topk + j] = weights[t * topk + j] * inv * scale;
+    }
+    free(p); free(sel);
+}

@@ -97,6 +97,11 @@ int ob_matmul_f64(int dtype, size_t m, size_t k, size_t n, const float* lhs,
  * moe_cuda_cpu/mod.rs:2098-2113. ids[t,topk], weights[t,topk]. */
 void lko_topk_softmax(const float* logits, size_t tokens, size_t n_experts, size_t topk,
                       int renorm, int32_t* ids, float* weights);
+/* Sigmoid router (cuda/moe/gate_topk.cu:140-200, 329-364): p = 1 / (1 + exp(-logit)); top-k on
+ * p + bias (bias nullable; ties: lower index first); weights = p of the chosen, divided by
+ * max(sum, 2^-14) if renorm, times scale. */
+void lko_topk_sigmoid(const float* logits, const float* bias, size_t tokens, size_t n_experts, size_t topk,
+                      int renorm, float scale, int32_t* ids, float* weights);
 /* Stable sort of the flattened (token, choice) slots by expert id:
  * sorted_slots[i], sorted_experts[i] (generic_transformer/moe_weights.rs:27-54,102-116). */
 void lko_group_by_expert(const int32_t* ids, size_t pairs, int32_t* sorted_slots,
