@@ -20,9 +20,9 @@ from __future__ import annotations
 
 import numpy as np
 
-GGML_Q8_0, GGML_Q8_1, GGML_Q4_K, GGML_Q6_K = 8, 9, 12, 14
-BLOCK_LEN = {GGML_Q8_0: 32, GGML_Q8_1: 32, GGML_Q4_K: 256, GGML_Q6_K: 256}
-BLOCK_BYTES = {GGML_Q8_0: 34, GGML_Q8_1: 36, GGML_Q4_K: 144, GGML_Q6_K: 210}
+GGML_Q8_0, GGML_Q8_1, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K = 8, 9, 12, 13, 14
+BLOCK_LEN = {GGML_Q8_0: 32, GGML_Q8_1: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256}
+BLOCK_BYTES = {GGML_Q8_0: 34, GGML_Q8_1: 36, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210}
 
 _G = np.uint64(0x9E3779B97F4A7C15)
 _M1 = np.uint64(0xBF58476D1CE4E5B9)
@@ -91,6 +91,19 @@ def q4k_blocks(n_blocks: int, seed: int = 0, stream: int = 0) -> np.ndarray:
     return out
 
 
+def q5k_blocks(n_blocks: int, seed: int = 0, stream: int = 0) -> np.ndarray:
+    """``[n_blocks, 176]`` random Q5_K super-blocks: the Q4_K fields plus 32 bytes of fifth bits."""
+    s = stream * 8
+    out = np.empty((n_blocks, 176), np.uint8)
+    out[:, 0:2] = _f16_bytes(np.abs(normal(seed, s + 0, n_blocks)) * np.float32(1e-3))
+    out[:, 2:4] = _f16_bytes(np.abs(normal(seed, s + 1, n_blocks)) * np.float32(5e-4))
+    fields = rand_ints(seed, s + 2, n_blocks * 16, 64).reshape(n_blocks, 16)
+    out[:, 4:16] = pack_scales_mins(fields[:, :8], fields[:, 8:])
+    out[:, 16:48] = rand_bytes(seed, s + 4, n_blocks * 32).reshape(n_blocks, 32)
+    out[:, 48:176] = rand_bytes(seed, s + 3, n_blocks * 128).reshape(n_blocks, 128)
+    return out
+
+
 def q6k_blocks(n_blocks: int, seed: int = 0, stream: int = 0) -> np.ndarray:
     """``[n_blocks, 210]`` random Q6_K super-blocks."""
     s = stream * 8
@@ -112,7 +125,7 @@ def q80_blocks(n_blocks: int, seed: int = 0, stream: int = 0) -> np.ndarray:
     return out
 
 
-_MAKERS = {GGML_Q4_K: q4k_blocks, GGML_Q6_K: q6k_blocks, GGML_Q8_0: q80_blocks}
+_MAKERS = {GGML_Q4_K: q4k_blocks, GGML_Q5_K: q5k_blocks, GGML_Q6_K: q6k_blocks, GGML_Q8_0: q80_blocks}
 
 
 def weight(dtype: int, n: int, k: int, seed: int = 0, stream: int = 0) -> np.ndarray:

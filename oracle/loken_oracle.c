@@ -80,7 +80,7 @@ uint16_t lko_f32_to_f16(float f) {
 int lko_block_len(int dtype) {
     switch (dtype) {
         case LKO_Q8_0: case LKO_Q8_1: return 32;
-        case LKO_Q4_K: case LKO_Q6_K: case LKO_Q8_K: return 256;
+        case LKO_Q4_K: case LKO_Q5_K: case LKO_Q6_K: case LKO_Q8_K: return 256;
         default: return 0;
     }
 }
@@ -90,6 +90,7 @@ int lko_block_bytes(int dtype) {
         case LKO_Q8_0: return LKO_Q80_BYTES;
         case LKO_Q8_1: return LKO_Q81_BYTES;
         case LKO_Q4_K: return LKO_Q4K_BYTES;
+        case LKO_Q5_K: return LKO_Q5K_BYTES;
         case LKO_Q6_K: return LKO_Q6K_BYTES;
         case LKO_Q8_K: return LKO_Q8K_BYTES;
         default: return 0;
@@ -144,6 +145,8 @@ void lko_pack_scales_mins(const uint8_t scales[8], const uint8_t mins[8], uint8_
 }
 
 /* Field offsets. Q4_K: d@0 dmin@2 scales@4 qs@16 (q4_k.rs:12-20).
+ * Q5_K: d@0 dmin@2 scales@4 qh@16 qs@48 (q5_k.rs:10-16); a value is its Q4_K nibble plus bit s of
+ * qh[l] as the fifth bit (q5_k.rs:66-71, 105-106).
  * Q6_K: ql@0 qh@128 scales@192 d@208 (q6_k.rs:8-16). Q8_0: d@0 qs@2. Q8_1: d@0 s@2 qs@4.
  * Q8_K: d(f32)@0 qs@4 bsums@260 (q8_k.rs:13-20). */
 
@@ -156,6 +159,14 @@ static inline int q6k_code(const uint8_t* blk, int h, int g, int l) {
     const int low = (ql[span + l] >> nibble) & 0x0F;
     const int high = (qh[l] >> (2 * g)) & 0x03;
     return (low | (high << 4)) - 32;
+}
+
+/* The five-bit code of element `l` of sub-block `s` (q5_k.rs:66-71). */
+static inline int q5k_code(const uint8_t* blk, int s, int l) {
+    const uint8_t packed = blk[48 + (s / 2) * 32 + l];
+    const int shift = (s % 2 == 0) ? 0 : 4;
+    const int fifth = (blk[16 + l] >> s) & 1;
+    return ((packed >> shift) & 0x0F) | (fifth << 4);
 }
 
 int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out) {
@@ -176,6 +187,21 @@ int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out
                 for (int l = 0; l < 32; ++l) {
                     y[s * 32 + l] = scale * (float)((group[l] >> shift) & 0x0F) - offset;
                 }
+            }
+        }
+        return 0;
+    case LKO_Q5_K: /* q5_k.rs:95-112 */
+        for (size_t b = 0; b < n_blocks; ++b) {
+            const uint8_t* blk = blocks + b * LKO_Q5K_BYTES;
+            float* y = out + b * 256;
+            const float d = lko_f16_to_f32(rd_u16(blk));
+            const float dmin = lko_f16_to_f32(rd_u16(blk + 2));
+            uint8_t sc[8], mn[8];
+            lko_unpack_scales_mins(blk + 4, sc, mn);
+            for (int s = 0; s < 8; ++s) {
+                const float scale = d * (float)sc[s];
+                const float offset = dmin * (float)mn[s];
+                for (int l = 0; l < 32; ++l) y[s * 32 + l] = scale * (float)q5k_code(blk, s, l) - offset;
             }
         }
         return 0;
@@ -295,6 +321,13 @@ static inline int32_t q4k_sub_dot(const uint8_t* blk, int s, const int8_t* acts)
     return dot;
 }
 
+/* q5_k.rs:62-73 inner `dot`: the same with the fifth bit. */
+static inline int32_t q5k_sub_dot(const uint8_t* blk, int s, const int8_t* acts) {
+    int32_t dot = 0;
+    for (int l = 0; l < 32; ++l) dot += (int32_t)q5k_code(blk, s, l) * (int32_t)acts[l];
+    return dot;
+}
+
 /* q6_k.rs:137-160: the sixteen per-16 sums of a Q6_K block against 256 activation codes. */
 static inline void q6k_sub_dots(const uint8_t* blk, const int8_t* acts256, int32_t per_sub[16]) {
     for (int j = 0; j < 16; ++j) per_sub[j] = 0;
@@ -327,6 +360,28 @@ static float oa_dot_q4k(const uint8_t* w, const uint8_t* y, size_t nb) {
         float scaled = 0.0f, offset = 0.0f;
         for (int s = 0; s < 8; ++s) {
             const int32_t dot = q4k_sub_dot(x, s, yq + 32 * s);
+            const int32_t bs = (int32_t)(int16_t)rd_u16(yb + 260 + 4 * s) +
+                               (int32_t)(int16_t)rd_u16(yb + 260 + 4 * s + 2);
+            scaled += (float)sc[s] * (float)dot;
+            offset += (float)mn[s] * (float)bs;
+        }
+        total += rd_f32(yb) * (lko_f16_to_f32(rd_u16(x)) * scaled - lko_f16_to_f32(rd_u16(x + 2)) * offset);
+    }
+    return total;
+}
+
+/* q5_k.rs:51-80 */
+static float oa_dot_q5k(const uint8_t* w, const uint8_t* y, size_t nb) {
+    float total = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * LKO_Q5K_BYTES;
+        const uint8_t* yb = y + b * LKO_Q8K_BYTES;
+        const int8_t* yq = (const int8_t*)(yb + 4);
+        uint8_t sc[8], mn[8];
+        lko_unpack_scales_mins(x + 4, sc, mn);
+        float scaled = 0.0f, offset = 0.0f;
+        for (int s = 0; s < 8; ++s) {
+            const int32_t dot = q5k_sub_dot(x, s, yq + 32 * s);
             const int32_t bs = (int32_t)(int16_t)rd_u16(yb + 260 + 4 * s) +
                                (int32_t)(int16_t)rd_u16(yb + 260 + 4 * s + 2);
             scaled += (float)sc[s] * (float)dot;
@@ -428,6 +483,29 @@ static float ob_dot_q4k(const uint8_t* w, const uint8_t* y, size_t nb) {
     return total;
 }
 
+/* gguf.cuh:723-748 (vec_dot_q5_K_q8_1_impl_vmmq): the Q4_K combine over the five-bit codes. */
+static float ob_dot_q5k(const uint8_t* w, const uint8_t* y, size_t nb) {
+    float total = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * LKO_Q5K_BYTES;
+        uint8_t sc[8], mn[8];
+        lko_unpack_scales_mins(x + 4, sc, mn);
+        float scaled = 0.0f, offset = 0.0f;
+        for (int s = 0; s < 8; ++s) {
+            const uint8_t* yb = y + (b * 8 + s) * LKO_Q81_BYTES;
+            const int8_t* yq = (const int8_t*)(yb + 4);
+            const float d8 = lko_f16_to_f32(rd_u16(yb));
+            const int32_t dot = q5k_sub_dot(x, s, yq);
+            int32_t sum = 0;
+            for (int l = 0; l < 32; ++l) sum += yq[l];
+            scaled += d8 * (float)(dot * (int32_t)sc[s]);
+            offset += d8 * (float)(sum * (int32_t)mn[s]);
+        }
+        total += lko_f16_to_f32(rd_u16(x)) * scaled - lko_f16_to_f32(rd_u16(x + 2)) * offset;
+    }
+    return total;
+}
+
 /* gguf.cuh:782-816: sum over the sixteen runs of d8*(dot*sc), times d. */
 static float ob_dot_q6k(const uint8_t* w, const uint8_t* y, size_t nb) {
     float total = 0.0f;
@@ -467,6 +545,7 @@ typedef float (*row_dot_fn)(const uint8_t* w, const uint8_t* y, size_t nb);
 static row_dot_fn oa_dot_of(int dtype) {
     switch (dtype) {
         case LKO_Q4_K: return oa_dot_q4k;
+        case LKO_Q5_K: return oa_dot_q5k;
         case LKO_Q6_K: return oa_dot_q6k;
         case LKO_Q8_0: return oa_dot_q80;
         default: return NULL;
@@ -475,6 +554,7 @@ static row_dot_fn oa_dot_of(int dtype) {
 static row_dot_fn ob_dot_of(int dtype) {
     switch (dtype) {
         case LKO_Q4_K: return ob_dot_q4k;
+        case LKO_Q5_K: return ob_dot_q5k;
         case LKO_Q6_K: return ob_dot_q6k;
         case LKO_Q8_0: return ob_dot_q80;
         default: return NULL;
@@ -531,7 +611,7 @@ int oa_matmul_exact(int dtype, size_t m, size_t k, size_t n, const float* lhs,
 int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t* act,
                int32_t* dots, int32_t* sums) {
     const size_t blk = (size_t)lko_block_len(dtype);
-    if (blk == 0 || (dtype != LKO_Q4_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
+    if (blk == 0 || (dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
     if (k % blk != 0) return -1;
     const size_t nb = k / blk;
     const size_t wrow = nb * (size_t)lko_block_bytes(dtype);
@@ -550,6 +630,11 @@ int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t*
                 for (int s = 0; s < 8; ++s)
                     dots[c * (k / 32) + b * 8 + s] = q4k_sub_dot(
                         w + b * LKO_Q4K_BYTES, s, (const int8_t*)(act + (b * 8 + s) * LKO_Q81_BYTES + 4));
+        } else if (dtype == LKO_Q5_K) {
+            for (size_t b = 0; b < nb; ++b)
+                for (int s = 0; s < 8; ++s)
+                    dots[c * (k / 32) + b * 8 + s] = q5k_sub_dot(
+                        w + b * LKO_Q5K_BYTES, s, (const int8_t*)(act + (b * 8 + s) * LKO_Q81_BYTES + 4));
         } else if (dtype == LKO_Q6_K) {
             for (size_t b = 0; b < nb; ++b) {
                 int8_t acts[256];
@@ -605,6 +690,18 @@ static int dequant_row_f64(int dtype, const uint8_t* w, size_t nb, double* out) 
                 for (int l = 0; l < 32; ++l)
                     out[b * 256 + s * 32 + l] = d * sc[s] * (double)((group[l] >> shift) & 0x0F) - dmin * mn[s];
             }
+        }
+        return 0;
+    }
+    if (dtype == LKO_Q5_K) {
+        for (size_t b = 0; b < nb; ++b) {
+            const uint8_t* x = w + b * LKO_Q5K_BYTES;
+            const double d = lko_f16_to_f32(rd_u16(x)), dmin = lko_f16_to_f32(rd_u16(x + 2));
+            uint8_t sc[8], mn[8];
+            lko_unpack_scales_mins(x + 4, sc, mn);
+            for (int s = 0; s < 8; ++s)
+                for (int l = 0; l < 32; ++l)
+                    out[b * 256 + s * 32 + l] = d * sc[s] * (double)q5k_code(x, s, l) - dmin * mn[s];
         }
         return 0;
     }

@@ -36,10 +36,11 @@ extern "C" {
 #endif
 
 /* ggml type ids, src/tensor/quantized/dtype.rs:66-96 */
-enum { LKO_Q8_0 = 8, LKO_Q8_1 = 9, LKO_Q4_K = 12, LKO_Q6_K = 14, LKO_Q8_K = 15 };
+enum { LKO_Q8_0 = 8, LKO_Q8_1 = 9, LKO_Q4_K = 12, LKO_Q5_K = 13, LKO_Q6_K = 14, LKO_Q8_K = 15 };
 
 #define LKO_QK_K 256
 #define LKO_Q4K_BYTES 144
+#define LKO_Q5K_BYTES 176
 #define LKO_Q6K_BYTES 210
 #define LKO_Q80_BYTES 34
 #define LKO_Q81_BYTES 36

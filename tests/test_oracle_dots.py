@@ -14,7 +14,8 @@ import pytest
 import oracle
 from loken_amd import synth
 
-DT = {"q4_k": oracle.Q4_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0}
+DT = {"q4_k": oracle.Q4_K, "q5_k": oracle.Q5_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0}
+FAST = sorted(set(DT) - {"q5_k"})   # formats the timed AVX2 baseline serves
 
 
 # ---- independent numpy decoders: integer codes and float scales per value ----
@@ -33,6 +34,16 @@ def np_codes_q4k(w):
     d = w[:, :, 0:2].copy().view(np.float16).reshape(n, nb).astype(np.float64)
     dmin = w[:, :, 2:4].copy().view(np.float16).reshape(n, nb).astype(np.float64)
     return codes, sc.reshape(n, nb * 8), mn.reshape(n, nb * 8), d, dmin
+
+
+def np_codes_q5k(w):
+    """w [n, nb, 176]: the Q4_K decoding of the same fields, plus bit s of qh[l] worth sixteen."""
+    n, nb, _ = w.shape
+    as_q4k = np.concatenate([w[:, :, :16], w[:, :, 48:]], axis=2)
+    codes, sc, mn, d, dmin = np_codes_q4k(as_q4k)
+    qh = w[:, :, 16:48].astype(np.int64)                                  # [n, nb, l]
+    fifth = (qh[:, :, None, :] >> np.arange(8)[None, None, :, None]) & 1  # [n, nb, s, l]
+    return codes + 16 * fifth.reshape(n, nb * 256), sc, mn, d, dmin
 
 
 def np_codes_q6k(w):
@@ -65,8 +76,8 @@ def np_q81(act_bytes):
 
 def np_dequant(dtype, w):
     n = w.shape[0]
-    if dtype == oracle.Q4_K:
-        codes, sc, mn, d, dmin = np_codes_q4k(w)
+    if dtype in (oracle.Q4_K, oracle.Q5_K):
+        codes, sc, mn, d, dmin = (np_codes_q4k if dtype == oracle.Q4_K else np_codes_q5k)(w)
         scale = np.repeat(sc * np.repeat(d, 8, axis=1), 32, axis=1)
         off = np.repeat(mn * np.repeat(dmin, 8, axis=1), 32, axis=1)
         return scale * codes - off
@@ -78,7 +89,7 @@ def np_dequant(dtype, w):
 
 
 def test_numpy_decoders_agree_with_ggml(ggml_vectors):
-    for name, dtype in (("q4_K", oracle.Q4_K), ("q6_K", oracle.Q6_K), ("q8_0", oracle.Q8_0)):
+    for name, dtype in (("q4_K", oracle.Q4_K), ("q5_K", oracle.Q5_K), ("q6_K", oracle.Q6_K), ("q8_0", oracle.Q8_0)):
         rec = ggml_vectors[name]
         w = rec["quant"].reshape(1, -1, rec["block_bytes"])
         got = np_dequant(dtype, w).reshape(-1)
@@ -96,8 +107,8 @@ def test_integer_subdots_match_numpy_brute_force(name):
     _, q = np_q81(act)
     q = q.reshape(-1)
     assert sums.tolist() == q.reshape(-1, 32).sum(axis=1).tolist()
-    if dtype == oracle.Q4_K:
-        codes = np_codes_q4k(w)[0]
+    if dtype in (oracle.Q4_K, oracle.Q5_K):
+        codes = (np_codes_q4k if dtype == oracle.Q4_K else np_codes_q5k)(w)[0]
         want = (codes * q[None, :]).reshape(n, k // 32, 32).sum(axis=2)
     elif dtype == oracle.Q6_K:
         codes = np_codes_q6k(w)[0]
@@ -166,7 +177,7 @@ def test_served_path_matches_f64_over_dequantized_weights(name, m):
     bound = 5e-3 * (np.abs(x.astype(np.float64)) @ np.abs(wd).T) + 1e-3
     assert (np.abs(got - ref) <= bound).all()
     # and it is the exact-fold variant up to f32 summation order
-    if dtype != oracle.Q8_0:
+    if dtype in (oracle.Q4_K, oracle.Q6_K):   # the formats the reference states an exact fold for
         ex = oracle.oa_matmul(dtype, x, w, n, exact=True)
         assert (np.abs(ex - got) <= 1e-3 * np.maximum(np.abs(got), 1.0)).all()
 
@@ -190,7 +201,7 @@ def test_served_path_integer_core_with_q8k_codes(name):
     assert (np.abs(got - ref) <= 4e-6 * absdot + 1e-9).all()
 
 
-@pytest.mark.parametrize("name", sorted(DT))
+@pytest.mark.parametrize("name", FAST)
 @pytest.mark.parametrize("m,threads", [(1, 1), (1, 3), (5, 4), (9, 2)])
 def test_threaded_avx2_baseline_matches_scalar_path(name, m, threads):
     dtype = DT[name]
