@@ -33,6 +33,7 @@ extern "C" {
 #define LK_TYPE_Q8_0 8
 #define LK_TYPE_Q8_1 9
 #define LK_TYPE_Q4_K 12
+#define LK_TYPE_Q5_K 13
 #define LK_TYPE_Q6_K 14
 #define LK_TYPE_BF16 30
 
@@ -64,7 +65,7 @@ int lk_quantize_q8_1(const void* x, int x_type, void* vy, int kx, int kx_padded,
                      void* stream);
 
 /* dst[j, row] = weight row `row` . activation row j, j < batch (1..8).
- *   wtype          LK_TYPE_Q4_K | LK_TYPE_Q6_K | LK_TYPE_Q8_0
+ *   wtype          LK_TYPE_Q4_K | LK_TYPE_Q5_K | LK_TYPE_Q6_K | LK_TYPE_Q8_0
  *   vx             nrows_x rows of ncols_x / block_len blocks
  *   vy_q8_1        batch rows of Q8_1 blocks, `stride_col_y` blocks apart (k_padded / 32)
  *   dst            `dst_type` LK_TYPE_F32 | F16 | BF16, rows `stride_col_dst` elements apart
@@ -192,8 +193,12 @@ void launch_mmq_quantize_q8_1_DS4(const void* x, const int32_t* ids, void* vy, i
  * Returns the token-tile width launched (32, 64 or 128), 0 when nothing ran (bad sizes, or k
  * not a multiple of 256). tmp_fixup, cc, nsm, smpbo, warp_size are accepted and unused: there
  * is no stream-k fixup pass and one device family.
- * Replaces launch_mmq_gguf_{q4_k,q6_k,q8_0} (cuda/mmq_gguf/mmq_launch.cuh:61-206). */
+ * Replaces launch_mmq_gguf_{q4_k,q5_k,q6_k,q8_0} (cuda/mmq_gguf/mmq_launch.cuh:61-206). */
 int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+int launch_mmq_gguf_q5_k(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
                          int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
                          int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
                          void* stream);
@@ -222,6 +227,12 @@ int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* y, void* ds
  * non-zero mmq_x picks the tile width. Returns the tile width launched, 0 when nothing ran.
  * Replaces launch_mmq_moe_gguf_* (cuda/mmq_gguf/mmq_launch.cuh:212-319). */
 int launch_mmq_moe_gguf_q4_k(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_q5_k(const void* x, const void* x_second, int64_t dst_second, const void* y,
                              void* dst, const int* expert_bounds, const int* ids_dst,
                              int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
                              int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,

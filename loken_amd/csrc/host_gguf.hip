@@ -507,7 +507,7 @@ extern "C" void* lkh_gguf_linear(void* g, const char* name, int device, void* st
         put_error(err, err_len, "QKernelMatMul: weight must be 2-D, got " + std::to_string(t.dims.size()) + " dims");
         return nullptr;
     }
-    if (t.dtype != LK_TYPE_Q4_K && t.dtype != LK_TYPE_Q6_K && t.dtype != LK_TYPE_Q8_0) {
+    if (t.dtype != LK_TYPE_Q4_K && t.dtype != LK_TYPE_Q5_K && t.dtype != LK_TYPE_Q6_K && t.dtype != LK_TYPE_Q8_0) {
         put_error(err, err_len, "QKernelMatMul: block type " + std::to_string(t.dtype) + " is not served on the card");
         return nullptr;
     }

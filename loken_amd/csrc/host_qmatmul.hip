@@ -98,7 +98,7 @@ void mark_used(Slot& slot, hipStream_t stream) {
 }
 
 bool tiled_serves(int dtype, int k) {
-    return (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q6_K || dtype == LK_TYPE_Q8_0) && k % 256 == 0;
+    return (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K || dtype == LK_TYPE_Q6_K || dtype == LK_TYPE_Q8_0) && k % 256 == 0;
 }
 
 size_t elem_bytes(int type) { return type == LK_TYPE_F32 ? 4 : 2; }
@@ -116,7 +116,7 @@ QKernelMatMul::QKernelMatMul(int dtype, int n, int k, const void* blob, int devi
 int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void* stream_ptr, bool decode_order) {
     last_path_ = Path::None;
     hipStream_t stream = (hipStream_t)stream_ptr;
-    if (dtype_ != LK_TYPE_Q4_K && dtype_ != LK_TYPE_Q6_K && dtype_ != LK_TYPE_Q8_0) return LK_ERR_TYPE;
+    if (dtype_ != LK_TYPE_Q4_K && dtype_ != LK_TYPE_Q5_K && dtype_ != LK_TYPE_Q6_K && dtype_ != LK_TYPE_Q8_0) return LK_ERR_TYPE;
     if (x_type != LK_TYPE_F32 && x_type != LK_TYPE_F16 && x_type != LK_TYPE_BF16) return LK_ERR_TYPE;
     if (rows == 0) return LK_OK;
     if (!x || !out || !blob_ || rows < 0 || n_ <= 0 || k_ <= 0) return LK_ERR_ARG;
@@ -174,9 +174,9 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     const size_t ws_bytes = (size_t)rows * (k_padded / 128) * MMQ_RECORD + 128 * MMQ_RECORD;
     std::lock_guard<std::mutex> pair(slot.mu);
     if (int rc = reserve(slot, ws_bytes, true, stream)) return rc;
-    auto quantizer = dtype_ == LK_TYPE_Q4_K ? launch_mmq_quantize_q8_1_DS4 : launch_mmq_quantize_q8_1_D4;
+    auto quantizer = dtype_ == LK_TYPE_Q4_K || dtype_ == LK_TYPE_Q5_K ? launch_mmq_quantize_q8_1_DS4 : launch_mmq_quantize_q8_1_D4;
     quantizer(x, nullptr, slot.act, 0, k_, k_, 0, 0, (int64_t)k_padded, rows, 1, 1, stream);
-    auto launcher = dtype_ == LK_TYPE_Q4_K ? launch_mmq_gguf_q4_k : dtype_ == LK_TYPE_Q6_K ? launch_mmq_gguf_q6_k : launch_mmq_gguf_q8_0;
+    auto launcher = dtype_ == LK_TYPE_Q4_K ? launch_mmq_gguf_q4_k : dtype_ == LK_TYPE_Q5_K ? launch_mmq_gguf_q5_k : dtype_ == LK_TYPE_Q6_K ? launch_mmq_gguf_q6_k : launch_mmq_gguf_q8_0;
     int abi = 0, cus = 0, lds = 0, wave = 0;
     (void)lk_device_info(&abi, &cus, &lds, &wave);
     const int tile = launcher(slot.fixup, blob_, slot.act, out, k_, n_, rows, k_ / block_len, n_, 0x1000950, cus, lds, wave,

@@ -12,6 +12,7 @@
 
 // GGUF block geometry (src/tensor/quantized/dtype.rs:66-96 of the reference).
 #define Q4K_BYTES 144
+#define Q5K_BYTES 176
 #define Q6K_BYTES 210
 #define Q80_BYTES 34
 #define Q81_BYTES 36

@@ -103,8 +103,14 @@ static void launch_quantize(const void* x, const int32_t* ids, void* vy, int typ
 // Staging is split in two so a step's global loads fly while the previous step is multiplied:
 // fetch() issues the loads into a register fragment, commit() expands the fragment into LDS.
 // --------------------------------------------------------------------------------------------
-struct MmqQ4K {
-    static constexpr int BLOCK_BYTES = Q4K_BYTES;
+// Q5 = false: Q4_K. Q5 = true: Q5_K, the same header followed by 32 bytes of fifth bits (bit s of
+// byte l belongs to value l of sub-block s, worth 16: src/tensor/quant_cpu/format/q5_k.rs:66-71) and
+// then the nibbles; the int8 tiles take codes 0..31 as they take 0..15.
+template <bool Q5>
+struct MmqQ45K {
+    static constexpr int BLOCK_BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES;
+    static constexpr int QS0 = Q5 ? 48 : 16;
+    static constexpr bool F16_TILES = !Q5;   // Q4_K above 64 tokens: the f16 tile kernel
     static constexpr int NS = 8;          // one weight scale per 32 values
     static constexpr bool HAS_MIN = true;
     static constexpr int BLOCKS_PER_STEP = 1;
@@ -112,6 +118,7 @@ struct MmqQ4K {
 
     struct Frag {
         uint4 q[QCH];
+        uint4 qh[Q5 ? QCH : 1];
         uint4 hdr;
     };
     // nb: Q4_K blocks between consecutive rows
@@ -121,11 +128,13 @@ struct MmqQ4K {
         for (int i = 0; i < QCH; ++i) {
             const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, c = idx & 7;
             const int gn = min(n0 + row, n - 1);
-            f.q[i] = *(const uint4*)(w + ((int64_t)gn * nb + kb) * Q4K_BYTES + 16 + 16 * c);
+            const uint8_t* block = w + ((int64_t)gn * nb + kb) * BLOCK_BYTES;
+            f.q[i] = *(const uint4*)(block + QS0 + 16 * c);
+            if (Q5) f.qh[i] = *(const uint4*)(block + 16 + 16 * (c & 1));
         }
         if (threadIdx.x < TN) {
             const int gn = min(n0 + (int)threadIdx.x, n - 1);
-            f.hdr = *(const uint4*)(w + ((int64_t)gn * nb + kb) * Q4K_BYTES);
+            f.hdr = *(const uint4*)(w + ((int64_t)gn * nb + kb) * BLOCK_BYTES);
         }
     }
     static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
@@ -139,6 +148,14 @@ struct MmqQ4K {
             lo.z = q.z & 0x0F0F0F0Fu; hi.z = (q.z >> 4) & 0x0F0F0F0Fu;
             lo.w = q.w & 0x0F0F0F0Fu; hi.w = (q.w >> 4) & 0x0F0F0F0Fu;
             const int p = c >> 1, h = c & 1;
+            if (Q5) {
+                const uint4 b = f.qh[i];
+                const int s0 = 2 * p;
+                lo.x |= ((b.x >> s0) << 4) & 0x10101010u; hi.x |= ((b.x >> s0) << 3) & 0x10101010u;
+                lo.y |= ((b.y >> s0) << 4) & 0x10101010u; hi.y |= ((b.y >> s0) << 3) & 0x10101010u;
+                lo.z |= ((b.z >> s0) << 4) & 0x10101010u; hi.z |= ((b.z >> s0) << 3) & 0x10101010u;
+                lo.w |= ((b.w >> s0) << 4) & 0x10101010u; hi.w |= ((b.w >> s0) << 3) & 0x10101010u;
+            }
             *(uint4*)(wq + ((2 * p) * TN + row) * 32 + 16 * h) = lo;
             *(uint4*)(wq + ((2 * p + 1) * TN + row) * 32 + 16 * h) = hi;
         }
@@ -165,6 +182,8 @@ struct MmqQ4K {
         }
     }
 };
+using MmqQ4K = MmqQ45K<false>;
+using MmqQ5K = MmqQ45K<true>;
 
 // Q6_K: sixteen int8 scales per block, one per 16 values, so one MFMA K (32) spans two of them;
 // the tile loop runs each 32-group as two MFMAs over half-masked weight operands.
@@ -172,6 +191,7 @@ struct MmqQ6K {
     static constexpr int BLOCK_BYTES = Q6K_BYTES;
     static constexpr int NS = 16;
     static constexpr bool HAS_MIN = false;
+    static constexpr bool F16_TILES = false;
     static constexpr int BLOCKS_PER_STEP = 1;
     static constexpr int QCH = TN * 8 / MMQ_WG;
 
@@ -234,6 +254,7 @@ struct MmqQ80 {
     static constexpr int BLOCK_BYTES = Q80_BYTES;
     static constexpr int NS = 8;
     static constexpr bool HAS_MIN = false;
+    static constexpr bool F16_TILES = false;
     static constexpr int BLOCKS_PER_STEP = 8;
     static constexpr int QCH = TN * 16 / MMQ_WG, DCH = TN * 8 / MMQ_WG;
 
@@ -580,7 +601,7 @@ static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x
     hipStream_t s = (hipStream_t)stream;
     if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s);
     if (ncols_y <= 64) return launch_dense_tm<F, 64, 2>(pb, s);
-    if constexpr (F::HAS_MIN) {   // Q4_K: scales folded into f16 operands
+    if constexpr (F::F16_TILES) {   // Q4_K: scales folded into f16 operands
         if (!getenv("LK_MMQ_I8")) {
             const int tm = lk_mmq_q4k_f16_dense(pb, s);
             if (tm >= 0) return tm;
@@ -625,7 +646,7 @@ static int launch_moe(const void* x, const void* x_second, int64_t dst_second, c
     const int64_t want = mmq_x > 0 ? mmq_x : (ncols_hint > 0 ? ncols_hint : ncols_max);
     if (want <= 32) return launch_moe_tm<F, 32, 1>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
     if (want <= 64) return launch_moe_tm<F, 64, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
-    if constexpr (F::HAS_MIN) {
+    if constexpr (F::F16_TILES) {
         if (!getenv("LK_MMQ_I8")) {
             const int tm = lk_mmq_q4k_f16_moe(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
             if (tm >= 0) return tm;
@@ -655,6 +676,14 @@ extern "C" int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* 
                                     int64_t smpbo, int warp_size, void* stream) {
     (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
     return launch_dense<MmqQ4K>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
+}
+
+extern "C" int launch_mmq_gguf_q5_k(void* tmp_fixup, const void* x, const void* y, void* dst,
+                                    int64_t ncols_x, int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                                    int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                                    void* stream) {
+    (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
+    return launch_dense<MmqQ5K>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
 }
 
 extern "C" int launch_mmq_gguf_q6_k(void* tmp_fixup, const void* x, const void* y, void* dst,
@@ -687,5 +716,6 @@ extern "C" int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* 
     }
 
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q4_k, MmqQ4K)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q5_k, MmqQ5K)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q6_k, MmqQ6K)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q8_0, MmqQ80)

@@ -211,6 +211,30 @@ __global__ __launch_bounds__(64) void subdots_q4k_kernel(const uint8_t* __restri
     }
 }
 
+__global__ __launch_bounds__(64) void subdots_q5k_kernel(const uint8_t* __restrict__ vx,
+                                                         const uint8_t* __restrict__ vy,
+                                                         int32_t* __restrict__ dots, int nb) {
+    const int row = blockIdx.y, lane = threadIdx.x;
+    const int blk = blockIdx.x * 8 + (lane >> 3), ch = lane & 7, p = ch >> 1, lh = ch & 1;
+    int d_lo = 0, d_hi = 0;
+    if (blk < nb) {
+        const uint8_t* bp = vx + ((size_t)row * nb + blk) * Q5K_BYTES;
+        const uint4 q = *(const uint4*)(bp + 48 + 16 * ch);
+        const uint4 qh = *(const uint4*)(bp + 16 + 16 * lh);
+        uint4 a_lo, a_hi;
+        load_act16(vy, blk * 8 + 2 * p, lh, a_lo);
+        load_act16(vy, blk * 8 + 2 * p + 1, lh, a_hi);
+        q5k_dots(q, shr4(qh, 2 * p), a_lo, a_hi, d_lo, d_hi);
+    }
+    d_lo += __shfl_xor(d_lo, 1);
+    d_hi += __shfl_xor(d_hi, 1);
+    if (blk < nb && lh == 0) {
+        int32_t* out = dots + (size_t)row * nb * 8 + blk * 8 + 2 * p;
+        out[0] = d_lo;
+        out[1] = d_hi;
+    }
+}
+
 __global__ __launch_bounds__(64) void subdots_q6k_kernel(const uint8_t* __restrict__ vx,
                                                          const uint8_t* __restrict__ vy,
                                                          int32_t* __restrict__ dots, int nb) {
@@ -369,6 +393,7 @@ static int dispatch_plain(int wtype, int batch, MmvqCall& a) {
         case LK_TYPE_Q4_K:
             if (a.nb <= 8) { LK_BATCH_SWITCH(launch_plain, EngQ4KShort, T, a) }
             LK_BATCH_SWITCH(launch_plain, EngQ4K, T, a)
+        case LK_TYPE_Q5_K: LK_BATCH_SWITCH(launch_plain, EngQ5K, T, a)
         case LK_TYPE_Q6_K: LK_BATCH_SWITCH(launch_plain, EngQ6K, T, a)
         case LK_TYPE_Q8_0: LK_BATCH_SWITCH(launch_plain, EngQ80, T, a)
         default: return LK_ERR_TYPE;
@@ -385,7 +410,7 @@ static int check_common(int wtype, const void* vy, int ncols_x, int batch, int s
 }
 static int check_weight(int wtype, const void* vx) {
     if (!vx) return LK_ERR_ARG;
-    if (wtype == LK_TYPE_Q4_K && ((uintptr_t)vx & 15) != 0) return LK_ERR_ARG;
+    if ((wtype == LK_TYPE_Q4_K || wtype == LK_TYPE_Q5_K) && ((uintptr_t)vx & 15) != 0) return LK_ERR_ARG;
     if (((uintptr_t)vx & 1) != 0) return LK_ERR_ARG;
     return LK_OK;
 }
@@ -557,6 +582,7 @@ extern "C" int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, con
         case LK_TYPE_Q4_K:
             if (nb <= 8) { LK_PAIR_TYPE(EngQ4KShort) }
             LK_PAIR_TYPE(EngQ4K)
+        case LK_TYPE_Q5_K: LK_PAIR_TYPE(EngQ5K)
         case LK_TYPE_Q6_K: LK_PAIR_TYPE(EngQ6K)
         case LK_TYPE_Q8_0: LK_PAIR_TYPE(EngQ80)
         default: return LK_ERR_TYPE;
@@ -591,6 +617,7 @@ extern "C" int lk_mmvq_pair_act_q8_1(int wtype, const void* gate, const void* up
     }
     switch (wtype) {
         case LK_TYPE_Q4_K: LK_PAIR_Q(EngQ4K)
+        case LK_TYPE_Q5_K: LK_PAIR_Q(EngQ5K)
         case LK_TYPE_Q6_K: LK_PAIR_Q(EngQ6K)
         case LK_TYPE_Q8_0: LK_PAIR_Q(EngQ80)
         default: return LK_ERR_TYPE;
@@ -611,6 +638,7 @@ extern "C" int lk_mmvq_grouped(int wtype, const uint64_t* table, int groups, con
         case LK_TYPE_Q4_K:
             return nb <= 8 ? launch_grouped<EngQ4KShort>(table, groups, y, dst, nb, nrows_x, k32, s)
                            : launch_grouped<EngQ4K>(table, groups, y, dst, nb, nrows_x, k32, s);
+        case LK_TYPE_Q5_K: return launch_grouped<EngQ5K>(table, groups, y, dst, nb, nrows_x, k32, s);
         case LK_TYPE_Q6_K: return launch_grouped<EngQ6K>(table, groups, y, dst, nb, nrows_x, k32, s);
         default: return launch_grouped<EngQ80>(table, groups, y, dst, nb, nrows_x, k32, s);
     }
@@ -628,6 +656,8 @@ extern "C" int lk_mmvq_subdots(int wtype, const void* vx, const void* vy_q8_1, i
     const uint8_t* y = (const uint8_t*)vy_q8_1;
     if (wtype == LK_TYPE_Q4_K) {
         hipLaunchKernelGGL(subdots_q4k_kernel, dim3((nb + 7) / 8, nrows_x), dim3(64), 0, s, w, y, dots, nb);
+    } else if (wtype == LK_TYPE_Q5_K) {
+        hipLaunchKernelGGL(subdots_q5k_kernel, dim3((nb + 7) / 8, nrows_x), dim3(64), 0, s, w, y, dots, nb);
     } else if (wtype == LK_TYPE_Q6_K) {
         hipLaunchKernelGGL(subdots_q6k_kernel, dim3((nb + 7) / 8, nrows_x), dim3(64), 0, s, w, y, dots, nb);
     } else {

@@ -34,6 +34,23 @@ static __device__ __forceinline__ void q4k_dots(const uint4& q, const uint4& a_l
     d_hi = dot16(hi, a_hi, d_hi);
 }
 
+// Q5_K: the same 16 bytes of qs plus the 16 bytes of qh over the same l; bit 2p of a qh byte is
+// the fifth bit (worth 16) of that value in sub-block 2p, bit 2p+1 in sub-block 2p+1
+// (src/tensor/quant_cpu/format/q5_k.rs:66-71). `hs` arrives already shifted right by 2p.
+static __device__ __forceinline__ void q5k_dots(const uint4& q, const uint4& hs, const uint4& a_lo, const uint4& a_hi,
+                                                int& d_lo, int& d_hi) {
+    uint4 lo, hi;
+    lo.x = (q.x & 0x0F0F0F0Fu) | ((hs.x << 4) & 0x10101010u); hi.x = ((q.x >> 4) & 0x0F0F0F0Fu) | ((hs.x << 3) & 0x10101010u);
+    lo.y = (q.y & 0x0F0F0F0Fu) | ((hs.y << 4) & 0x10101010u); hi.y = ((q.y >> 4) & 0x0F0F0F0Fu) | ((hs.y << 3) & 0x10101010u);
+    lo.z = (q.z & 0x0F0F0F0Fu) | ((hs.z << 4) & 0x10101010u); hi.z = ((q.z >> 4) & 0x0F0F0F0Fu) | ((hs.z << 3) & 0x10101010u);
+    lo.w = (q.w & 0x0F0F0F0Fu) | ((hs.w << 4) & 0x10101010u); hi.w = ((q.w >> 4) & 0x0F0F0F0Fu) | ((hs.w << 3) & 0x10101010u);
+    d_lo = dot16(lo, a_lo, d_lo);
+    d_hi = dot16(hi, a_hi, d_hi);
+}
+static __device__ __forceinline__ uint4 shr4(const uint4& v, int s) {
+    return make_uint4(v.x >> s, v.y >> s, v.z >> s, v.w >> s);
+}
+
 // The (scale, min) pairs of sub-blocks 2p, 2p+1 from the 12 packed bytes (words w1..w3 of the
 // block header): scales in bits 0-7 / 8-15 of `sc`, mins likewise in `mn`. Sub-blocks 0-3 keep
 // their six bits in one byte; 4-7 take a nibble from bytes 8-11 and two bits from the top of
@@ -130,6 +147,10 @@ struct FmtQ4K {
         const int lb = j >> 3, s = j & 7;
         return ((s & 1) * 2 + lh) * 1024 + (lb * 4 + (s >> 1)) * 16;
     }
+};
+// Q5_K stages its activation as Q4_K does: the two formats share sub-blocks, scales and mins.
+struct FmtQ5K : FmtQ4K {
+    static constexpr int BLOCK_BYTES = Q5K_BYTES;
 };
 struct FmtQ6K {
     static constexpr int BLOCK_BYTES = Q6K_BYTES, BLOCK_LEN = 256;
@@ -417,8 +438,10 @@ static __device__ __forceinline__ void row16_sums(float v, float (&q)[4]) {
 // done(tile) runs on every lane of the wave once the tile's rows have been handed to epi.
 // PACK false: one row per pass, all of this a compile-time 1 / 16 (the long-row kernels pay
 // nothing for the short-row form); PACK true: rows per pass from the row length.
-template <int B, int R, int NW, bool PACK, class Epi, class Done>
+template <int B, int R, int NW, bool PACK, bool Q5, class Epi, class Done>
 static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* lds, Epi&& epi, Done&& done) {
+    // Q5_K: the Q4_K header, then 32 bytes of fifth bits, then the nibbles
+    constexpr int BB = Q5 ? Q5K_BYTES : Q4K_BYTES, QS0 = Q5 ? 48 : 16;
     const int nb = job.nb, n = job.n;
     const int n_iter_lds = (nb + 15) >> 4;   // passes of the staged activation (its layout)
     const int row_bytes = lds_bytes_per_row<FmtQ4K>(n_iter_lds);
@@ -433,13 +456,14 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
     const int lb = lane >> 2, p = lane & 3;
     const int slot = lb & (S - 1), rp = lb / S;
     const Q4KScaleSel sel(p);
-    const uint32_t hdr_off = slot * Q4K_BYTES, qs_off = hdr_off + 16 + 32 * p;
-    const size_t row_stride = (size_t)nb * Q4K_BYTES;
+    const uint32_t hdr_off = slot * BB, qs_off = hdr_off + QS0 + 32 * p;
+    const size_t row_stride = (size_t)nb * BB;
     const int n_tiles = (n + TR - 1) / TR;
     constexpr int RW = R * NW;
 
     struct Frag {
         uint4 hdr[RW], q0[RW], q1[RW];
+        uint4 h0[Q5 ? RW : 1], h1[Q5 ? RW : 1];   // Q5_K: qh over l 0..15 and 16..31 (every pair's lane reads both)
     };
     // One pass (16 super-block slots) of R rows per lane group of every matrix into registers. A
     // lane past the row end re-reads the row's last block and drops its d / dmin when it consumes
@@ -447,17 +471,21 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
     // would make the wave wait for the load).
     auto load = [&](Frag& f, int tile, int it) {
         const bool valid = it * S + slot < nb;
-        const uint32_t back = valid ? 0u : (uint32_t)(it * S + slot - (nb - 1)) * Q4K_BYTES;
+        const uint32_t back = valid ? 0u : (uint32_t)(it * S + slot - (nb - 1)) * BB;
 #pragma unroll
         for (int w = 0; w < NW; ++w)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int row = min(tile * TR + rp * R + r, n - 1);
-                const uint8_t* bp = (const uint8_t*)(job.vx[w] + row * row_stride + (size_t)it * (S * Q4K_BYTES));
+                const uint8_t* bp = (const uint8_t*)(job.vx[w] + row * row_stride + (size_t)it * (S * BB));
                 Frag& g = f;
                 g.hdr[w * R + r] = *(const uint4*)(bp + (hdr_off - back));
                 g.q0[w * R + r] = *(const uint4*)(bp + (qs_off - back));
                 g.q1[w * R + r] = *(const uint4*)(bp + (qs_off - back + 16));
+                if (Q5) {
+                    g.h0[w * R + r] = *(const uint4*)(bp + (hdr_off - back + 16));
+                    g.h1[w * R + r] = *(const uint4*)(bp + (hdr_off - back + 32));
+                }
             }
     };
 
@@ -494,8 +522,13 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
 #pragma unroll
             for (int r = 0; r < RW; ++r) {
                 int d_lo = 0, d_hi = 0;
-                q4k_dots(f.q0[r], a00, a10, d_lo, d_hi);
-                q4k_dots(f.q1[r], a01, a11, d_lo, d_hi);
+                if (Q5) {
+                    q5k_dots(f.q0[r], shr4(f.h0[r], 2 * p), a00, a10, d_lo, d_hi);
+                    q5k_dots(f.q1[r], shr4(f.h1[r], 2 * p), a01, a11, d_lo, d_hi);
+                } else {
+                    q4k_dots(f.q0[r], a00, a10, d_lo, d_hi);
+                    q4k_dots(f.q1[r], a01, a11, d_lo, d_hi);
+                }
                 const float u = (scl[r] * s4.x) * (float)d_lo + (sch[r] * s4.z) * (float)d_hi;
                 const float w = ml[r] * s4.y + mh[r] * s4.w;
                 acc[r][c] += d[r] * u - dmin[r] * w;
@@ -784,7 +817,7 @@ struct EngQ4K {
     static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
-        rows_q4k<B, R, NW, false>(j, lds, e, d);
+        rows_q4k<B, R, NW, false, false>(j, lds, e, d);
     }
 };
 // Q4_K rows of at most 8 super-blocks (k <= 2048): 2 or 4 rows share a pass.
@@ -793,7 +826,24 @@ struct EngQ4KShort {
     static __host__ __device__ int rows_per_pass(int nb) { return q4k_rows_per_pass(nb); }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
-        rows_q4k<B, R, NW, true>(j, lds, e, d);
+        rows_q4k<B, R, NW, true, false>(j, lds, e, d);
+    }
+};
+// Q5_K: the Q4_K engine with the fifth-bit plane (long and short rows alike).
+struct EngQ5K {
+    using Fmt = FmtQ5K;
+    static __host__ __device__ int rows_per_pass(int) { return 1; }
+    template <int B, int R, int NW, class Epi, class Done = NoTileHook>
+    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
+        rows_q4k<B, R, NW, false, true>(j, lds, e, d);
+    }
+};
+struct EngQ5KShort {
+    using Fmt = FmtQ5K;
+    static __host__ __device__ int rows_per_pass(int nb) { return q4k_rows_per_pass(nb); }
+    template <int B, int R, int NW, class Epi, class Done = NoTileHook>
+    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
+        rows_q4k<B, R, NW, true, true>(j, lds, e, d);
     }
 };
 struct EngQ6K {
@@ -825,7 +875,7 @@ static inline int lds_bytes_for(int nb, int batch) {
 
 static inline int lds_bytes_of(int wtype, int nb, int batch) {
     switch (wtype) {
-        case LK_TYPE_Q4_K: return lds_bytes_for<FmtQ4K>(nb, batch);
+        case LK_TYPE_Q4_K: case LK_TYPE_Q5_K: return lds_bytes_for<FmtQ4K>(nb, batch);
         case LK_TYPE_Q6_K: return lds_bytes_for<FmtQ6K>(nb, batch);
         default: return lds_bytes_for<FmtQ80>(nb, batch);
     }
@@ -833,7 +883,7 @@ static inline int lds_bytes_of(int wtype, int nb, int batch) {
 
 static inline int block_len_of(int wtype) {
     switch (wtype) {
-        case LK_TYPE_Q4_K: case LK_TYPE_Q6_K: return 256;
+        case LK_TYPE_Q4_K: case LK_TYPE_Q5_K: case LK_TYPE_Q6_K: return 256;
         case LK_TYPE_Q8_0: return 32;
         default: return 0;
     }
@@ -841,6 +891,7 @@ static inline int block_len_of(int wtype) {
 static inline int block_bytes_of(int wtype) {
     switch (wtype) {
         case LK_TYPE_Q4_K: return Q4K_BYTES;
+        case LK_TYPE_Q5_K: return Q5K_BYTES;
         case LK_TYPE_Q6_K: return Q6K_BYTES;
         case LK_TYPE_Q8_0: return Q80_BYTES;
         default: return 0;

@@ -13,7 +13,7 @@ LK_OK, LK_ERR_ARG, LK_ERR_TYPE, LK_ERR_LAUNCH, LK_ERR_NOMEM = 0, 1, 2, 3, 4
 _ERR_NAMES = {1: "LK_ERR_ARG", 2: "LK_ERR_TYPE", 3: "LK_ERR_LAUNCH", 4: "LK_ERR_NOMEM"}
 
 TYPE_F32, TYPE_F16, TYPE_BF16 = 0, 1, 30
-TYPE_Q8_0, TYPE_Q8_1, TYPE_Q4_K, TYPE_Q6_K = 8, 9, 12, 14
+TYPE_Q8_0, TYPE_Q8_1, TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K = 8, 9, 12, 13, 14
 
 
 class LokenError(RuntimeError):
@@ -38,12 +38,14 @@ SIGNATURES = {
     "launch_mmq_quantize_q8_1_D4": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),
     "launch_mmq_quantize_q8_1_DS4": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),
     "launch_mmq_gguf_q4_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
+    "launch_mmq_gguf_q5_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
     "launch_mmq_gguf_q6_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
     "launch_mmq_gguf_q8_0": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
 }
 _MOE_MMQ = (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _vp] + [_i64] * 6 + [_i, _i64, _i64, _i, _i, _i64, _i, _vp])
 SIGNATURES.update({
     "launch_mmq_moe_gguf_q4_k": _MOE_MMQ,
+    "launch_mmq_moe_gguf_q5_k": _MOE_MMQ,
     "launch_mmq_moe_gguf_q6_k": _MOE_MMQ,
     "launch_mmq_moe_gguf_q8_0": _MOE_MMQ,
     "loken_moe_mmq_plan": (None, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),

@@ -13,7 +13,8 @@ from . import lib as _lib
 from .ops import MMQ_DEVICE_INFO, _stream, mmq_quantize
 from .synth import BLOCK_BYTES, BLOCK_LEN
 
-MMQ_MOE_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_moe_gguf_q4_k", _lib.TYPE_Q6_K: "launch_mmq_moe_gguf_q6_k",
+MMQ_MOE_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_moe_gguf_q4_k", _lib.TYPE_Q5_K: "launch_mmq_moe_gguf_q5_k",
+                    _lib.TYPE_Q6_K: "launch_mmq_moe_gguf_q6_k",
                     _lib.TYPE_Q8_0: "launch_mmq_moe_gguf_q8_0"}
 MMQ_X_MIN, GRID_Y_MAX = 8, 65535
 

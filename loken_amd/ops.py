@@ -176,9 +176,11 @@ def mmvq_subdots(wtype: int, weight: torch.Tensor, q8_1_row: torch.Tensor, k: in
 
 
 # ------------------------------------------------------------------------------------ prefill
-MMQ_QUANTIZER = {_lib.TYPE_Q4_K: "launch_mmq_quantize_q8_1_DS4", _lib.TYPE_Q6_K: "launch_mmq_quantize_q8_1_D4",
+MMQ_QUANTIZER = {_lib.TYPE_Q4_K: "launch_mmq_quantize_q8_1_DS4", _lib.TYPE_Q5_K: "launch_mmq_quantize_q8_1_DS4",
+                 _lib.TYPE_Q6_K: "launch_mmq_quantize_q8_1_D4",
                  _lib.TYPE_Q8_0: "launch_mmq_quantize_q8_1_D4"}
-MMQ_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_gguf_q4_k", _lib.TYPE_Q6_K: "launch_mmq_gguf_q6_k",
+MMQ_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_gguf_q4_k", _lib.TYPE_Q5_K: "launch_mmq_gguf_q5_k",
+                _lib.TYPE_Q6_K: "launch_mmq_gguf_q6_k",
                 _lib.TYPE_Q8_0: "launch_mmq_gguf_q8_0"}
 MMQ_DEVICE_INFO = dict(cc=0x1000950, nsm=256, smpbo=160 * 1024, warp_size=64)
 
