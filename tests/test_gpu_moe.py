@@ -65,7 +65,7 @@ def test_route_with_experts_nobody_chose_and_one_token():
 
 @pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(5, 512, 256, 6, 2), (40, 1024, 512, 8, 3),
                                                              (1, 256, 256, 4, 2), (70, 512, 768, 16, 4)])
-@pytest.mark.parametrize("dt_down", [lib.TYPE_Q4_K, lib.TYPE_Q6_K])
+@pytest.mark.parametrize("dt_down", [lib.TYPE_Q4_K, lib.TYPE_Q5_K, lib.TYPE_Q6_K])
 def test_expert_batched_block_matches_oracle(tokens, hidden, ffn, n_experts, topk, dt_down):
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=51, dt_down=dt_down)
     want, want_h = oracle.moe_forward(1, lib.TYPE_Q4_K, dt_down, x, gate, up, down, ids, w, n_experts, ffn, want_h=True)
