@@ -8,9 +8,9 @@ One *step* = every quantized linear of one Llama-3-8B-shaped decode step at batc
 one launch (q,k,v; gate,up) and every launch quantizes its f32 activation to Q8_1 in LDS itself,
 4 launches per layer; `--plan split`: the two-launch form per linear (Q8_1 quantizer, then
 mat-vec); `--plan auto` (default): fused, and up to 4 rows the gate,up launch applies SiLU(gate)*up
-and writes the Q8_1 rows that `down` reads (4 launches per layer, no quantizer launch); above 4
-rows `down`, whose 14336-value rows are dear to quantize once per workgroup, keeps its own
-quantizer launch (5 launches per layer).
+and writes the Q8_1 rows that `down` reads (4 launches per layer, no quantizer launch); at 5 rows
+the split plan, and from 6 rows `--plan rows`: split, with the Q4_K matrices of 2048 rows or more
+on the matrix-unit rows kernel (loken_dense_q4k_imma_m8_plain), as measured on MI355X.
 Distinct weights per layer, so the step is cache-cold by construction.
 Weights and activations are synthetic (seeded, generated on the device) and resident in HBM
 before the timed region.
@@ -54,7 +54,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=1, help="activation rows per mat-vec (1..8)")
     ap.add_argument("--layers", type=int, default=LAYERS)
-    ap.add_argument("--plan", choices=["auto", "fused", "split"], default="auto",
+    ap.add_argument("--plan", choices=["auto", "fused", "split", "rows"], default="auto",
                     help="fused: shared-activation linears per launch, Q8_1 quantized in-kernel; split: quantize + "
                          "mat-vec per linear; auto: fused, except that rows longer than 8192 values are quantized "
                          "by their own launch (every workgroup of a fused launch quantizes the whole row)")
@@ -101,6 +101,9 @@ def main() -> int:
     gen = torch.Generator(device=dev)
     gen.manual_seed(0)
     b = args.batch
+    # `auto` above four rows (measured on MI355X): two launches per linear at 5 rows, and from 6 rows the
+    # Q4_K matrices of 2048 rows or more on the matrix-unit rows kernel
+    kind = args.plan if args.plan != "auto" or b <= 4 else ("split" if b == 5 else "rows")
 
     # ------------------------------------------------------------------ synthetic blocks
     def halfs(n, scale):
@@ -203,13 +206,28 @@ def main() -> int:
             q4k_plan.append(item)
             q4k_bytes += nbytes
 
+    def add_rows(w, g, n, k):
+        """Q4_K x the Q8_1 rows of group `g` on the matrix unit (the activation staged in LDS up to 8 rows)."""
+        nonlocal total_bytes, q4k_bytes
+        out = torch.empty((b, n), dtype=torch.float32, device=dev)
+        keep.append(out)
+        q = q81[g]
+        assert q.shape[1] * 32 == k
+        item = (L.loken_dense_q4k_imma_m8_plain, (w.data_ptr(), q.data_ptr(), out.data_ptr(), b, n, k, stream))
+        plan.append(item)
+        nbytes = synth.weight_bytes(Q4K, n, k)
+        total_bytes += nbytes
+        q4k_plan.append(item)
+        q4k_bytes += nbytes
+        return out
+
     first_out = None
     first_w = None
     for layer in range(args.layers):
-        if args.plan in ("fused", "auto"):
+        if kind in ("fused", "auto"):
             made = {name: (maker(n, k), wtype, n, k, g) for name, wtype, n, k, maker, g in shapes}
             keep.extend(v[0] for v in made.values())
-            paired = args.plan == "auto" and b <= 4
+            paired = kind == "auto" and b <= 4
             for group in (("q", "k", "v"), ("o",), ("gate", "up"), ("down",)):
                 wtype, k, g = made[group[0]][1], made[group[0]][3], made[group[0]][4]
                 if paired and group == ("gate", "up"):
@@ -219,7 +237,7 @@ def main() -> int:
                 if paired and group == ("down",):
                     add_gemv(wtype, made["down"][0], "h", made["down"][2], k)
                     continue
-                if args.plan == "auto" and k > 8192:
+                if kind == "auto" and k > 8192:
                     add_quant(g)
                     for nm in group:
                         add_gemv(wtype, made[nm][0], g, made[nm][2], k)
@@ -235,12 +253,17 @@ def main() -> int:
             if g != last_group:
                 add_quant(g)
                 last_group = g
-            out = add_gemv(wtype, w, g, n, k)
+            # the matrix-unit rows kernel gives a workgroup 32 weight rows: below a few thousand
+            # rows it leaves most of the chip idle and the mat-vec is the faster launch
+            if kind == "rows" and wtype == Q4K and n >= 2048:
+                out = add_rows(w, g, n, k)
+            else:
+                out = add_gemv(wtype, w, g, n, k)
             if first_out is None:
                 first_out, first_w = out, w
     lm_head = make_q80(VOCAB, HIDDEN)
     keep.append(lm_head)
-    if args.plan in ("fused", "auto"):
+    if kind in ("fused", "auto"):
         add_fused(Q80, [lm_head], "final", [VOCAB], HIDDEN)
     else:
         add_quant("final")
@@ -315,8 +338,9 @@ def main() -> int:
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC.get((args.plan, b, args.layers)),
                 "kernel": (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
-                           f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if args.plan == "auto" and b <= 4
-                          else f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
+                           f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if kind == "auto"
+                          else ("q4k_rows_staged_kernel<1> (q, o, gate, up), " if kind == "rows" else "")
+                          + f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches}
 
     # ------------------------------------------------------------------ CPU baseline leg
@@ -331,7 +355,7 @@ def main() -> int:
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"llama3-8b decode-step quantized linears (Q4_K q,k,v,o,gate,up; Q6_K down; "
                                f"Q8_0 lm_head), batch {b}, {args.layers} layers",
-                   "launch_plan": args.plan, "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
+                   "launch_plan": args.plan if kind == args.plan else f"{args.plan} -> {kind}", "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
                    "hip_graph": graph is not None},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": roofline,

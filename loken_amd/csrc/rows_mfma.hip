@@ -19,7 +19,16 @@
 // The four waves of a workgroup split the super-blocks of the same 32 rows between them and
 // add their partial tiles through LDS, which keeps small matrices spread over the chip.
 //
-// The min term -dmin * m[s] * d8 * S[s] is rank one per sub-block and goes through
+// Registers stand for activation rows (register v = row (v / 4) * 8 + 4 * (l / 32) + v % 4) and lanes
+// for weight rows, so a launch of at most 8 (16) activation rows only ever needs registers 0..3
+// (0..7) of each tile: the kernel is compiled for G = 1, 2 or 4 groups of eight rows and spends the
+// per-sub-block fix-up on those registers alone. That fix-up is most of the kernel's vector work,
+// and with it cut to a quarter the weights stream near the memory rate.
+//
+// The min term -dmin * m[s] * d8 * S[s] is rank one per sub-block. With G < 4 it is vector work on
+// the live registers: d8 * S of every (sub-block, activation row) is tabled in LDS beside d8 when
+// the workgroup starts (S summed from the codes there), and a register's row reads it as a
+// broadcast. With G = 4 it goes through
 // v_mfma_f32_32x32x2_f32 with K = the two halves of the sub-block: A = d8 * (sum of the lane's
 // own 16 codes), B = -dmin * m[s] in both halves. No lane exchange is needed for the sum.
 
@@ -53,12 +62,18 @@ struct Frag {
     v4i a[8];
 };
 
-static __device__ __forceinline__ int lds_floats_table(int nb) { return nb * 8 * TOK; }
+// Floats of the scale tables: d8 [nb * 8][8 G], and with G < 4 also d8 * S in the same shape.
+template <int G>
+static __host__ __device__ constexpr int lds_floats_table(int nb) { return nb * 8 * 8 * G * (G < 4 ? 2 : 1); }
 
+template <int G>
 __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
+    constexpr int TW = 8 * G;   // activation rows a table row holds
+    constexpr int NV = 4 * G;   // live accumulator registers
     extern __shared__ __align__(16) uint8_t lds[];
-    float* d8_table = (float*)lds;                                   // [nb * 8][TOK]
-    float* reduce = d8_table + lds_floats_table(p.nb);               // [WAVES][16][64]
+    float* d8_table = (float*)lds;                                   // [nb * 8][TW]
+    float* ds_table = d8_table + p.nb * 8 * TW;                      // [nb * 8][TW], G < 4 only
+    float* reduce = d8_table + lds_floats_table<G>(p.nb);            // [WAVES][NV][64]
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -71,19 +86,47 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     // Activation scales of this pass, zero for the rows the pass does not have. Eight loads are
     // issued before the first is used: one at a time, each would cost a memory latency.
     const uint8_t* y0 = p.y + (size_t)m0 * p.stride_y * Q81_BYTES;
-    const int entries = p.nb * 8 * TOK;
-    for (int base = threadIdx.x; base < entries; base += WG * 8) {
-        uint32_t bits[8];
+    const int entries = p.nb * 8 * TW;
+    if constexpr (G == 4) {
+        for (int base = threadIdx.x; base < entries; base += WG * 8) {
+            uint32_t bits[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int idx = min(base + u * WG, entries - 1);
-            const int sub = idx >> 5, tok = min(idx & 31, m_count - 1);
-            bits[u] = *(const uint16_t*)(y0 + ((size_t)tok * p.stride_y + sub) * Q81_BYTES);
+            for (int u = 0; u < 8; ++u) {
+                const int idx = min(base + u * WG, entries - 1);
+                const int sub = idx >> 5, tok = min(idx & 31, m_count - 1);
+                bits[u] = *(const uint16_t*)(y0 + ((size_t)tok * p.stride_y + sub) * Q81_BYTES);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = base + u * WG;
+                if (idx < entries) d8_table[idx] = (idx & 31) < m_count ? f16_bits_to_f32(bits[u]) : 0.f;
+            }
         }
+    } else {
+        // whole blocks: the scale and the integer sum of the 32 codes (four entries in flight)
+        for (int base = threadIdx.x; base < entries; base += WG * 4) {
+            uint32_t head[4];
+            uint4 lo[4], hi[4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int idx = base + u * WG;
-            if (idx < entries) d8_table[idx] = (idx & 31) < m_count ? f16_bits_to_f32(bits[u]) : 0.f;
+            for (int u = 0; u < 4; ++u) {
+                const int idx = min(base + u * WG, entries - 1);
+                const int sub = idx / TW, tok = min(idx % TW, m_count - 1);
+                const uint8_t* b = y0 + ((size_t)tok * p.stride_y + sub) * Q81_BYTES;
+                head[u] = *(const uint32_t*)b;
+                lo[u] = *(const uint4_a4*)(b + 4);
+                hi[u] = *(const uint4_a4*)(b + 20);
+            }
+            const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * WG;
+                if (idx < entries) {
+                    const bool real = idx % TW < m_count;
+                    const float d8 = real ? f16_bits_to_f32(head[u] & 0xFFFFu) : 0.f;
+                    d8_table[idx] = d8;
+                    ds_table[idx] = d8 * (float)dot16(ones, hi[u], dot16(ones, lo[u], 0));
+                }
+            }
         }
     }
 
@@ -106,6 +149,7 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
 
     // Two accumulators: the scale term is vector arithmetic on `acc`, the min term a chain of
     // matrix instructions on `acc_min`; kept apart, neither waits for the other's latency.
+    // (With G < 4 both are vector arithmetic on the live registers.)
     v16f acc, acc_min;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = acc_min[v] = 0.f;
@@ -149,20 +193,29 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) c[v] = MAGIC_BITS;
             c = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a[s], b, c, 0, 0, 0);
-            const float* d8_sub = d8_table + (kb * 8 + s) * TOK;
-            // min term: this lane's activation row and half of the sub-block
-            const uint4 au = make_uint4((uint32_t)f.a[s][0], (uint32_t)f.a[s][1], (uint32_t)f.a[s][2], (uint32_t)f.a[s][3]);
-            const float half_sum = d8_sub[l32] * (float)dot16(ones, au, 0);
-            acc_min = __builtin_amdgcn_mfma_f32_32x32x2f32(half_sum, dmm[s], acc_min, 0, 0, 0);
+            const float* d8_sub = d8_table + (kb * 8 + s) * TW;
+            if constexpr (G == 4) {
+                // min term: this lane's activation row and half of the sub-block
+                const uint4 au = make_uint4((uint32_t)f.a[s][0], (uint32_t)f.a[s][1], (uint32_t)f.a[s][2], (uint32_t)f.a[s][3]);
+                const float half_sum = d8_sub[l32] * (float)dot16(ones, au, 0);
+                acc_min = __builtin_amdgcn_mfma_f32_32x32x2f32(half_sum, dmm[s], acc_min, 0, 0, 0);
+            }
             // scale term: register v stands for activation row (v / 4) * 8 + lh * 4 + v % 4
             const float off = -MAGIC * dsc[s];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+            for (int g = 0; g < G; ++g) {
                 const float4 t = *(const float4*)(d8_sub + 8 * g + 4 * lh);
                 acc[4 * g + 0] = fmaf(fmaf(__int_as_float(c[4 * g + 0]), dsc[s], off), t.x, acc[4 * g + 0]);
                 acc[4 * g + 1] = fmaf(fmaf(__int_as_float(c[4 * g + 1]), dsc[s], off), t.y, acc[4 * g + 1]);
                 acc[4 * g + 2] = fmaf(fmaf(__int_as_float(c[4 * g + 2]), dsc[s], off), t.z, acc[4 * g + 2]);
                 acc[4 * g + 3] = fmaf(fmaf(__int_as_float(c[4 * g + 3]), dsc[s], off), t.w, acc[4 * g + 3]);
+                if constexpr (G < 4) {
+                    const float4 u = *(const float4*)(ds_table + (kb * 8 + s) * TW + 8 * g + 4 * lh);
+                    acc_min[4 * g + 0] = fmaf(dmm[s], u.x, acc_min[4 * g + 0]);
+                    acc_min[4 * g + 1] = fmaf(dmm[s], u.y, acc_min[4 * g + 1]);
+                    acc_min[4 * g + 2] = fmaf(dmm[s], u.z, acc_min[4 * g + 2]);
+                    acc_min[4 * g + 3] = fmaf(dmm[s], u.w, acc_min[4 * g + 3]);
+                }
             }
         }
     };
@@ -177,18 +230,18 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
 
     auto finish_tile = [&](int t) {
         // add the four partial tiles and write the activation rows this pass has
-        float* mine = reduce + wave * (16 * 64);
+        float* mine = reduce + wave * (NV * 64);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
+        for (int v = 0; v < NV; ++v) {
             mine[v * 64 + lane] = acc[v] + acc_min[v];
             acc[v] = acc_min[v] = 0.f;
         }
         __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int v = wave * 4 + r;
-            const float sum = (reduce[v * 64 + lane] + reduce[(16 + v) * 64 + lane]) +
-                              (reduce[(32 + v) * 64 + lane] + reduce[(48 + v) * 64 + lane]);
+        for (int r = 0; r < G; ++r) {
+            const int v = wave * G + r;
+            const float sum = (reduce[v * 64 + lane] + reduce[(NV + v) * 64 + lane]) +
+                              (reduce[(2 * NV + v) * 64 + lane] + reduce[(3 * NV + v) * 64 + lane]);
             const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = t * 32 + l32;
             if (tok < m_count && row < p.n) p.dst[(size_t)(m0 + tok) * p.ldd + row] = sum;
         }
@@ -221,6 +274,191 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// At most 16 activation rows whose codes fit in LDS: the workgroup stages the codes once (in the
+// order the A operand wants them) beside the two scale tables, so the only global loads of a step
+// are the weight row's five 16-byte pieces, and a wave keeps three or four steps of them in flight. With the
+// activation read from memory per step as above, two steps in flight left a decode-sized matrix
+// (one 32-row tile per workgroup, four steps per wave) waiting on memory latency most of its time.
+// ---------------------------------------------------------------------------------------------
+struct WFrag {
+    uint4 hdr, q[4];
+};
+
+template <int G>
+static __host__ __device__ constexpr int lds_bytes_staged(int nb) {
+    // codes [nb * 8][8 G][32], d8 and d8 * S [nb * 8][8 G] floats each, reduce [WAVES][4 G][64] floats
+    return nb * 8 * 8 * G * 32 + 2 * nb * 8 * 8 * G * 4 + WAVES * 4 * G * 64 * 4;
+}
+
+template <int G>
+__global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Args p) {
+    constexpr int TW = 8 * G, NV = 4 * G;
+    extern __shared__ __align__(16) uint8_t lds[];
+    uint8_t* codes = lds;                                            // [nb * 8][TW][32]
+    float* d8_table = (float*)(codes + (size_t)p.nb * 8 * TW * 32);  // [nb * 8][TW]
+    float* ds_table = d8_table + p.nb * 8 * TW;                      // [nb * 8][TW]
+    float* reduce = ds_table + p.nb * 8 * TW;                        // [WAVES][NV][64]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int m_count = p.m;   // one pass: the launcher sends at most TW rows here
+    const int n_tiles = (p.n + 31) >> 5;
+    const size_t row_bytes = (size_t)p.nb * Q4K_BYTES;
+    const int entries = p.nb * 8 * TW;
+
+    // Steps of this wave: (tile, super-block) pairs, super-blocks wave, wave + 4, ... of each tile
+    // of this workgroup in turn.
+    const int my_blocks = (p.nb - wave + WAVES - 1) / WAVES;
+    const int my_tiles = (int)blockIdx.x < n_tiles ? (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    const int total = my_tiles * my_blocks;
+    auto loadw = [&](WFrag& f, int j) {
+        const int tile = blockIdx.x + (j / my_blocks) * gridDim.x, kb = wave + (j % my_blocks) * WAVES;
+        const int row = min(tile * 32 + l32, p.n - 1);
+        const uint8_t* bp = (const uint8_t*)(to_gbytes(p.w) + row * row_bytes + (size_t)kb * Q4K_BYTES);
+        f.hdr = *(const uint4*)bp;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) f.q[c] = *(const uint4*)(bp + 16 + 32 * c + 16 * lh);
+    };
+
+    // The activation: every (sub-block, row) entry is one Q8_1 block; its codes go to LDS as they
+    // are, its scale and scale * (sum of codes) into the tables. The first round's loads are issued
+    // before the first weight loads and consumed after them (loads return in issue order: asked for
+    // after the weights, the activation, which sits in L2, would wait for HBM).
+    constexpr int PER = 4;
+    uint32_t head[PER];
+    uint4 lo[PER], hi[PER];
+    auto issue = [&](int base) {
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int idx = min(base + u * WG, entries - 1);
+            const int sub = idx / TW, tok = min(idx % TW, m_count - 1);
+            const uint8_t* b = p.y + ((size_t)tok * p.stride_y + sub) * Q81_BYTES;
+            head[u] = *(const uint32_t*)b;
+            lo[u] = *(const uint4_a4*)(b + 4);
+            hi[u] = *(const uint4_a4*)(b + 20);
+        }
+    };
+    auto place = [&](int base) {
+        const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int idx = base + u * WG;
+            if (idx < entries) {
+                const bool real = idx % TW < m_count;
+                const float d8 = real ? f16_bits_to_f32(head[u] & 0xFFFFu) : 0.f;
+                d8_table[idx] = d8;
+                ds_table[idx] = d8 * (float)dot16(ones, hi[u], dot16(ones, lo[u], 0));
+                *(uint4*)(codes + (size_t)idx * 32) = lo[u];
+                *(uint4*)(codes + (size_t)idx * 32 + 16) = hi[u];
+            }
+        }
+    };
+    constexpr int DEPTH = G == 1 ? 4 : 3;   // steps of weight loads a wave keeps in flight (registers)
+    WFrag f[DEPTH];
+    issue(threadIdx.x);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+        if (d < total) loadw(f[d], d);
+    place(threadIdx.x);
+    for (int r = WG * PER; r < entries; r += WG * PER) {
+        issue(r + threadIdx.x);
+        place(r + threadIdx.x);
+    }
+    __syncthreads();
+
+    float acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = 0.f;
+
+    // the lane's A operand: activation row l32 (rows the launch does not have repeat the live
+    // ones; their results sit in registers nobody reads), codes 16 lh .. 16 lh + 15 of the sub-block
+    const uint8_t* a_lane = codes + (l32 % TW) * 32 + 16 * lh;
+
+    auto compute = [&](const WFrag& w, int kb) {
+        const uint32_t w1 = w.hdr.y, w2 = w.hdr.z, w3 = w.hdr.w;
+        const uint32_t sc_lo = w1 & 0x3F3F3F3Fu, mn_lo = w2 & 0x3F3F3F3Fu;
+        const uint32_t sc_hi = (w3 & 0x0F0F0F0Fu) | ((w1 >> 2) & 0x30303030u);
+        const uint32_t mn_hi = ((w3 >> 4) & 0x0F0F0F0Fu) | ((w2 >> 2) & 0x30303030u);
+        const float d = f16_bits_to_f32(w.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(w.hdr.x >> 16);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint32_t scs = ((s < 4 ? sc_lo : sc_hi) >> (8 * (s & 3))) & 0xFFu;
+            const uint32_t mns = ((s < 4 ? mn_lo : mn_hi) >> (8 * (s & 3))) & 0xFFu;
+            const float dsc = d * (float)scs, dmm = -(dmin * (float)mns);
+            const uint4 q = w.q[s >> 1];
+            v4i b;
+            if (s & 1) {
+                b = v4i{(int)((q.x >> 4) & 0x0F0F0F0Fu), (int)((q.y >> 4) & 0x0F0F0F0Fu),
+                        (int)((q.z >> 4) & 0x0F0F0F0Fu), (int)((q.w >> 4) & 0x0F0F0F0Fu)};
+            } else {
+                b = v4i{(int)(q.x & 0x0F0F0F0Fu), (int)(q.y & 0x0F0F0F0Fu), (int)(q.z & 0x0F0F0F0Fu),
+                        (int)(q.w & 0x0F0F0F0Fu)};
+            }
+            const int sub = kb * 8 + s;
+            const v4i a = *(const v4i*)(a_lane + (size_t)sub * TW * 32);
+            // the accumulators start at the bit pattern of 1.5 * 2^23, so the dots leave the matrix
+            // unit as floats (see the kernel above)
+            constexpr int MAGIC_BITS = 0x4B400000;
+            constexpr float MAGIC = 12582912.0f;
+            v16i c;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) c[v] = MAGIC_BITS;
+            c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+            const float off = -MAGIC * dsc;
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float4 t = *(const float4*)(d8_table + sub * TW + 8 * g + 4 * lh);
+                const float4 u = *(const float4*)(ds_table + sub * TW + 8 * g + 4 * lh);
+                acc[4 * g + 0] = fmaf(fmaf(__int_as_float(c[4 * g + 0]), dsc, off), t.x, fmaf(dmm, u.x, acc[4 * g + 0]));
+                acc[4 * g + 1] = fmaf(fmaf(__int_as_float(c[4 * g + 1]), dsc, off), t.y, fmaf(dmm, u.y, acc[4 * g + 1]));
+                acc[4 * g + 2] = fmaf(fmaf(__int_as_float(c[4 * g + 2]), dsc, off), t.z, fmaf(dmm, u.z, acc[4 * g + 2]));
+                acc[4 * g + 3] = fmaf(fmaf(__int_as_float(c[4 * g + 3]), dsc, off), t.w, fmaf(dmm, u.w, acc[4 * g + 3]));
+            }
+            // one sub-block's tile at a time: left free, the scheduler starts all eight matrix
+            // instructions of a step first and holds 8 x 16 result registers
+            if (s & 1) __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    auto finish_tile = [&](int t) {
+        float* mine = reduce + wave * (NV * 64);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            mine[v * 64 + lane] = acc[v];
+            acc[v] = 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < G; ++r) {
+            const int v = wave * G + r;
+            const float sum = (reduce[v * 64 + lane] + reduce[(NV + v) * 64 + lane]) +
+                              (reduce[(2 * NV + v) * 64 + lane] + reduce[(3 * NV + v) * 64 + lane]);
+            const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = t * 32 + l32;
+            if (tok < m_count && row < p.n) p.dst[(size_t)tok * p.ldd + row] = sum;
+        }
+        __syncthreads();   // the partial tiles may be overwritten
+    };
+
+    if (my_blocks == 0) {   // rows shorter than four super-blocks: this wave only keeps the barriers
+        for (int t = 0; t < my_tiles; ++t) finish_tile(blockIdx.x + t * gridDim.x);
+        return;
+    }
+    for (int j0 = 0; j0 < total; j0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int j = j0 + d;
+            if (j < total) {
+                compute(f[d], wave + (j % my_blocks) * WAVES);
+                if (j + DEPTH < total) loadw(f[d], j + DEPTH);
+                if ((j + 1) % my_blocks == 0) finish_tile(blockIdx.x + (j / my_blocks) * gridDim.x);
+            }
+        }
+    }
+}
+
+template <int G>
 int resident_cap(int lds_bytes) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -231,17 +469,63 @@ int resident_cap(int lds_bytes) {
     if (lds_bytes > lk_device().lds_bytes) {
         r = 0;
     } else if (lds_bytes > 48 * 1024 &&
-               hipFuncSetAttribute((const void*)q4k_rows_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+               hipFuncSetAttribute((const void*)q4k_rows_mfma_kernel<G>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         r = 0;
-    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_mfma_kernel, WG,
+    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_mfma_kernel<G>, WG,
                                                             (size_t)lds_bytes) != hipSuccess || r < 1) {
         (void)hipGetLastError();
         r = 1;
     }
     by_lds.emplace(lds_bytes, r);
     return r;
+}
+
+template <int G>
+int launch_rows(const Args& a, hipStream_t stream) {
+    const int lds_bytes = (lds_floats_table<G>(a.nb) + WAVES * 4 * G * 64) * (int)sizeof(float);
+    const int per_cu = resident_cap<G>(lds_bytes);
+    if (per_cu == 0) return LK_ERR_ARG;   // rows too long for the scale tables
+    const int n_tiles = (a.n + 31) / 32, groups = (a.m + TOK - 1) / TOK;
+    if (groups > 65535) return LK_ERR_ARG;
+    int cap = lk_device().cus * per_cu / groups;
+    if (cap < 1) cap = 1;
+    hipLaunchKernelGGL(q4k_rows_mfma_kernel<G>, dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
+    return lk_launch_status();
+}
+
+// The staged kernel for `a.m` <= 8 G rows, if its LDS image fits; -1 when it does not.
+template <int G>
+int launch_staged(const Args& a, hipStream_t stream) {
+    static std::mutex mu;
+    static std::unordered_map<int, int> by_lds;
+    const int lds_bytes = lds_bytes_staged<G>(a.nb);
+    if (lds_bytes > lk_device().lds_bytes) return -1;
+    int per_cu;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = by_lds.find(lds_bytes);
+        if (it == by_lds.end()) {
+            int r = 0;
+            if (lds_bytes > 48 * 1024 &&
+                hipFuncSetAttribute((const void*)q4k_rows_staged_kernel<G>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    lds_bytes) != hipSuccess) {
+                (void)hipGetLastError();
+                r = 0;
+            } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_staged_kernel<G>, WG,
+                                                                    (size_t)lds_bytes) != hipSuccess || r < 1) {
+                (void)hipGetLastError();
+                r = 1;
+            }
+            it = by_lds.emplace(lds_bytes, r).first;
+        }
+        per_cu = it->second;
+    }
+    if (per_cu == 0) return -1;
+    const int n_tiles = (a.n + 31) / 32, cap = lk_device().cus * per_cu;
+    hipLaunchKernelGGL(q4k_rows_staged_kernel<G>, dim3(n_tiles < cap ? n_tiles : cap), dim3(WG), lds_bytes, stream, a);
+    return lk_launch_status();
 }
 
 }  // namespace
@@ -253,17 +537,18 @@ int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m,
     if (!w || !q8_1 || !output || size_m < 0 || size_n < 0 || size_k <= 0 || size_k % 256 != 0) return LK_ERR_ARG;
     if (stride_y < size_k / 32 || ldd < size_n) return LK_ERR_ARG;
     if ((((uintptr_t)w) & 15) != 0 || (((uintptr_t)q8_1) & 3) != 0) return LK_ERR_ARG;
-    const int nb = size_k / 256;
-    const int lds_bytes = (nb * 8 * TOK + WAVES * 16 * 64) * (int)sizeof(float);
-    const int per_cu = resident_cap(lds_bytes);
-    if (per_cu == 0) return LK_ERR_ARG;   // rows too long for the scale table
-    const int n_tiles = (size_n + 31) / 32, groups = (size_m + TOK - 1) / TOK;
-    if (groups > 65535) return LK_ERR_ARG;
-    int cap = lk_device().cus * per_cu / groups;
-    if (cap < 1) cap = 1;
-    Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, nb, size_n, size_m, stride_y, ldd};
-    hipLaunchKernelGGL(q4k_rows_mfma_kernel, dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
-    return lk_launch_status();
+    Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd};
+    // at most 8 / 16 activation rows in all: the fix-up runs on the registers those rows live in,
+    // and the activation is staged in LDS when it fits there
+    if (size_m <= 8) {
+        const int rc = launch_staged<1>(a, stream);
+        return rc >= 0 ? rc : launch_rows<1>(a, stream);
+    }
+    if (size_m <= 16) {
+        const int rc = launch_staged<2>(a, stream);
+        return rc >= 0 ? rc : launch_rows<2>(a, stream);
+    }
+    return launch_rows<4>(a, stream);
 }
 
 extern "C" void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
