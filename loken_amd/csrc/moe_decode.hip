@@ -71,6 +71,8 @@ void* reserve_scratch(size_t bytes, hipStream_t stream) {
 struct MoeDims {
     int experts, topk, pairs, cols, nb, k32;  // k32: Q8_1 blocks between activation rows
     int64_t slab_bytes;                       // one expert's weights
+    int act_f32 = 0;                          // non-zero: `acts` holds f32 rows this many floats apart and
+                                              // every workgroup quantizes its pair's row while staging it
 };
 
 enum { MODE_PLAIN = 0, MODE_GATED = 1, MODE_DOWN = 2 };
@@ -97,19 +99,20 @@ __global__ __launch_bounds__(WG) void moe_rows_kernel(const uint8_t* __restrict_
     }
     const bool own_row = MODE == MODE_DOWN || (MODE == MODE_PLAIN && topk_weights != nullptr);
     const int act_row = own_row ? slot : slot / d.topk;
-    const uint8_t* vy = acts + (size_t)act_row * d.k32 * Q81_BYTES;
+    const uint8_t* vy = d.act_f32 ? acts + (size_t)act_row * d.act_f32 * sizeof(float)
+                                  : acts + (size_t)act_row * d.k32 * Q81_BYTES;
     const float scale = (MODE != MODE_GATED && topk_weights) ? topk_weights[slot] : 1.0f;
     const uint8_t* slab0 = w0 + (int64_t)e * d.slab_bytes;
     const int tile_stride = (int)gridDim.x * WAVES, tile_first = (int)blockIdx.x * WAVES;
     if (MODE == MODE_GATED) {
         const uint8_t* slab1 = w1 + (int64_t)e * d.slab_bytes;
-        RowJob<2> job{{to_gbytes(slab0), to_gbytes(slab1)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first};
+        RowJob<2> job{{to_gbytes(slab0), to_gbytes(slab1)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first, d.act_f32};
         E::template run<1, R, 2>(job, lds, [&](int row, int, const float* tot) {
             const float g = tot[0];
             out_row[row] = g / (1.0f + expf(-g)) * tot[1];
         });
     } else {
-        RowJob<1> job{{to_gbytes(slab0)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first};
+        RowJob<1> job{{to_gbytes(slab0)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first, d.act_f32};
         E::template run<1, R, 1>(job, lds, [&](int row, int, const float* tot) {
             float v = tot[0] * scale;
             if (MODE == MODE_DOWN && down_bias) v += scale * down_bias[(size_t)e * d.cols + row];
@@ -205,6 +208,13 @@ static bool bad_shape(int quant_type, int num_experts, int topk, int size_m, int
 
 static inline int pad512(int k) { return (k + 511) / 512 * 512; }
 
+// f32 rows a workgroup can quantize while it stages them (what lk_mmvq_fused asks of its input): a
+// pair's row is a few KB, so reading it as floats costs less than a quantizer launch ahead of the
+// kernel and the scratch round trip between the two.
+static inline bool rows_stage_as_f32(const float* inputs, int size_k) {
+    return ((uintptr_t)inputs & 15) == 0 && size_k % 4 == 0 && size_k <= 8192;
+}
+
 }  // namespace
 
 extern "C" void loken_stream_scratch_release() {
@@ -239,6 +249,11 @@ extern "C" int loken_moe_gemm_gguf(const float* inputs, const void* weights, con
     const int kp = pad512(size_k);
     // with routing weights every entry has its own activation row; without, topk entries share one
     const int act_rows = topk_weights ? size_m : size_m / topk;
+    if (rows_stage_as_f32(inputs, size_k)) {
+        MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k};
+        return launch_format<MODE_PLAIN>(quant_type, (const uint8_t*)weights, nullptr, (const uint8_t*)inputs,
+                                         sorted_token_ids, expert_ids, topk_weights, nullptr, (float*)outputs, d, size_k, s);
+    }
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     uint8_t* acts = (uint8_t*)reserve_scratch((size_t)act_rows * (kp / 32) * Q81_BYTES, s);
     if (!acts) return LK_ERR_NOMEM;
@@ -259,6 +274,12 @@ extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const v
         bad_shape(quant_type, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k), act_rows = size_m / topk;
+    if (rows_stage_as_f32(inputs, size_k)) {
+        MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k};
+        return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights,
+                                         (const uint8_t*)inputs, sorted_token_ids, expert_ids, nullptr, nullptr, outputs,
+                                         d, size_k, s);
+    }
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     uint8_t* acts = (uint8_t*)reserve_scratch((size_t)act_rows * (kp / 32) * Q81_BYTES, s);
     if (!acts) return LK_ERR_NOMEM;
@@ -279,15 +300,18 @@ extern "C" int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* 
         bad_shape(gguf_dtype, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k);
-    const size_t act_bytes = (((size_t)size_m * (kp / 32) * Q81_BYTES) + 255) & ~(size_t)255;
+    const bool as_f32 = rows_stage_as_f32(inputs, size_k);
+    const size_t act_bytes = as_f32 ? 0 : (((size_t)size_m * (kp / 32) * Q81_BYTES) + 255) & ~(size_t)255;
     const size_t pair_bytes = (size_t)size_m * size_n * sizeof(float);
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     uint8_t* base = (uint8_t*)reserve_scratch(act_bytes + pair_bytes, s);
     if (!base) return LK_ERR_NOMEM;
     float* pairs = (float*)(base + act_bytes);
-    if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, base, size_k, kp, size_m, stream)) return rc;
-    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0};
-    if (int rc = launch_format<MODE_DOWN>(gguf_dtype, (const uint8_t*)weights, nullptr, base, sorted_token_ids,
+    if (!as_f32)
+        if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, base, size_k, kp, size_m, stream)) return rc;
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, as_f32 ? size_k : 0};
+    if (int rc = launch_format<MODE_DOWN>(gguf_dtype, (const uint8_t*)weights, nullptr,
+                                          as_f32 ? (const uint8_t*)inputs : base, sorted_token_ids,
                                           expert_ids, topk_weights, down_bias, pairs, d, size_k, s)) return rc;
     const int tokens = size_m / topk;
     const size_t total = (size_t)tokens * size_n;
