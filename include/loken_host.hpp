@@ -3,7 +3,7 @@
  * kernel_matmul/mmq.rs:21-159): which kernel family a call takes by its row count, the grow-only
  * per-device workspaces with the host mutex held across a quantize -> consume pair of launches,
  * and the event that orders workspace reuse between streams. Rust is what the reference's host is
- * written in; this is the same logic for a C++ caller, and what the Rust shim of INTEGRATION.md
+ * written in; this is the same logic for a C++ caller, and what a Rust binding to this library
  * would keep doing on its own side.
  *
  * Device pointers in, device pointers out; nothing here synchronizes the host with the device. */
