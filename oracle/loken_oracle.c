@@ -79,7 +79,7 @@ uint16_t lko_f32_to_f16(float f) {
 
 int lko_block_len(int dtype) {
     switch (dtype) {
-        case LKO_Q8_0: case LKO_Q8_1: return 32;
+        case LKO_Q8_0: case LKO_Q8_1: case LKO_Q4_0: case LKO_Q4_1: case LKO_Q5_0: case LKO_Q5_1: return 32;
         case LKO_Q4_K: case LKO_Q5_K: case LKO_Q6_K: case LKO_Q8_K: return 256;
         default: return 0;
     }
@@ -88,6 +88,10 @@ int lko_block_len(int dtype) {
 int lko_block_bytes(int dtype) {
     switch (dtype) {
         case LKO_Q8_0: return LKO_Q80_BYTES;
+        case LKO_Q4_0: return 18;
+        case LKO_Q4_1: return 20;
+        case LKO_Q5_0: return 22;
+        case LKO_Q5_1: return 24;
         case LKO_Q8_1: return LKO_Q81_BYTES;
         case LKO_Q4_K: return LKO_Q4K_BYTES;
         case LKO_Q5_K: return LKO_Q5K_BYTES;
@@ -169,6 +173,8 @@ static inline int q5k_code(const uint8_t* blk, int s, int l) {
     return ((packed >> shift) & 0x0F) | (fifth << 4);
 }
 
+static int legacy_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out);
+
 int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out) {
     switch (dtype) {
     case LKO_Q4_K: /* q4_k.rs:98-114 */
@@ -241,7 +247,7 @@ int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out
         }
         return 0;
     default:
-        return -3;
+        return legacy_dequantize(dtype, blocks, n_blocks, out);
     }
 }
 
@@ -540,6 +546,113 @@ static float ob_dot_q80(const uint8_t* w, const uint8_t* y, size_t nb) {
     return total;
 }
 
+
+/* ------------------------------------------------------------------------------------------
+ * The 32-value formats with nibble codes (q4_0.rs, q4_1.rs, q5_0.rs, q5_1.rs): byte j of `qs`
+ * holds value j in its low nibble and value j + 16 in its high one; the five-bit formats keep
+ * bit v of the little-endian word `qh` as value v's fifth bit. Q4_0 {d, qs} and Q5_0 {d, qh, qs}
+ * mean (code - 8 / 16) * d; Q4_1 {d, m, qs} and Q5_1 {d, m, qh, qs} mean code * d + m.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct { int bytes, m_at, qh_at, qs_at, bias; } legacy_layout;
+
+static int legacy_layout_of(int dtype, legacy_layout* l) {
+    switch (dtype) {
+        case LKO_Q4_0: *l = (legacy_layout){18, -1, -1, 2, 8}; return 1;
+        case LKO_Q4_1: *l = (legacy_layout){20, 2, -1, 4, 0}; return 1;
+        case LKO_Q5_0: *l = (legacy_layout){22, -1, 2, 6, 16}; return 1;
+        case LKO_Q5_1: *l = (legacy_layout){24, 2, 4, 8, 0}; return 1;
+        default: return 0;
+    }
+}
+
+/* The unsigned code of value v (q5_0.rs:43-48). */
+static inline int legacy_code(const uint8_t* blk, const legacy_layout* l, int v) {
+    const uint8_t packed = blk[l->qs_at + (v & 15)];
+    int code = v < 16 ? (packed & 0x0F) : (packed >> 4);
+    if (l->qh_at >= 0) {
+        const uint32_t qh = (uint32_t)blk[l->qh_at] | ((uint32_t)blk[l->qh_at + 1] << 8) |
+                            ((uint32_t)blk[l->qh_at + 2] << 16) | ((uint32_t)blk[l->qh_at + 3] << 24);
+        code |= (int)((qh >> v) & 1u) << 4;
+    }
+    return code;
+}
+
+/* The integer the CPU dots form (q4_0.rs:104-113, q4_1.rs:104-111): sum of (code - bias) * a. */
+static inline int32_t legacy_sub_dot(const uint8_t* blk, const legacy_layout* l, const int8_t* acts) {
+    int32_t dot = 0;
+    for (int v = 0; v < 32; ++v) dot += (int32_t)(legacy_code(blk, l, v) - l->bias) * (int32_t)acts[v];
+    return dot;
+}
+
+static int legacy_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out) {
+    legacy_layout l;
+    if (!legacy_layout_of(dtype, &l)) return -3;
+    for (size_t b = 0; b < n_blocks; ++b) {
+        const uint8_t* blk = blocks + b * (size_t)l.bytes;
+        const float d = lko_f16_to_f32(rd_u16(blk));
+        const float m = l.m_at >= 0 ? lko_f16_to_f32(rd_u16(blk + l.m_at)) : 0.0f;
+        for (int v = 0; v < 32; ++v) {
+            const int code = legacy_code(blk, &l, v);
+            out[b * 32 + v] = l.m_at >= 0 ? (float)code * d + m : (float)(code - l.bias) * d;
+        }
+    }
+    return 0;
+}
+
+/* Served CPU path: Q4_0 / Q5_0 against Q8_0 blocks, dot * d * y.d (q4_0.rs:96-117); Q4_1 / Q5_1
+ * against Q8_1 blocks, dot * d * y.d + m * y.s (q4_1.rs:95-115). */
+static float oa_dot_legacy(int dtype, const uint8_t* w, const uint8_t* y, size_t nb) {
+    legacy_layout l;
+    legacy_layout_of(dtype, &l);
+    float total = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * (size_t)l.bytes;
+        if (l.m_at < 0) {
+            const uint8_t* yb = y + b * LKO_Q80_BYTES;
+            const int32_t dot = legacy_sub_dot(x, &l, (const int8_t*)(yb + 2));
+            total += (float)dot * lko_f16_to_f32(rd_u16(x)) * lko_f16_to_f32(rd_u16(yb));
+        } else {
+            const uint8_t* yb = y + b * LKO_Q81_BYTES;
+            const int32_t dot = legacy_sub_dot(x, &l, (const int8_t*)(yb + 4));
+            total += (float)dot * lko_f16_to_f32(rd_u16(x)) * lko_f16_to_f32(rd_u16(yb)) +
+                     lko_f16_to_f32(rd_u16(x + l.m_at)) * lko_f16_to_f32(rd_u16(yb + 2));
+        }
+    }
+    return total;
+}
+
+/* Same codes on the Q8_1 side, the sum of the activation codes taken as the integer it is
+ * (cuda/moe/gguf.cuh:436-441 total_biased_codes; :400-405 with the minimum): d * d8 * dot, plus
+ * m * (d8 * sum of codes) for the formats with a minimum. */
+static float ob_dot_legacy(int dtype, const uint8_t* w, const uint8_t* y, size_t nb) {
+    legacy_layout l;
+    legacy_layout_of(dtype, &l);
+    float total = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * (size_t)l.bytes;
+        const uint8_t* yb = y + b * LKO_Q81_BYTES;
+        const int8_t* yq = (const int8_t*)(yb + 4);
+        const float d8 = lko_f16_to_f32(rd_u16(yb));
+        const int32_t dot = legacy_sub_dot(x, &l, yq);
+        float part = lko_f16_to_f32(rd_u16(x)) * d8 * (float)dot;
+        if (l.m_at >= 0) {
+            int32_t sum = 0;
+            for (int v = 0; v < 32; ++v) sum += yq[v];
+            part += lko_f16_to_f32(rd_u16(x + l.m_at)) * (d8 * (float)sum);
+        }
+        total += part;
+    }
+    return total;
+}
+static float oa_dot_q40(const uint8_t* w, const uint8_t* y, size_t nb) { return oa_dot_legacy(LKO_Q4_0, w, y, nb); }
+static float oa_dot_q41(const uint8_t* w, const uint8_t* y, size_t nb) { return oa_dot_legacy(LKO_Q4_1, w, y, nb); }
+static float oa_dot_q50(const uint8_t* w, const uint8_t* y, size_t nb) { return oa_dot_legacy(LKO_Q5_0, w, y, nb); }
+static float oa_dot_q51(const uint8_t* w, const uint8_t* y, size_t nb) { return oa_dot_legacy(LKO_Q5_1, w, y, nb); }
+static float ob_dot_q40(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_Q4_0, w, y, nb); }
+static float ob_dot_q41(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_Q4_1, w, y, nb); }
+static float ob_dot_q50(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_Q5_0, w, y, nb); }
+static float ob_dot_q51(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_Q5_1, w, y, nb); }
+
 typedef float (*row_dot_fn)(const uint8_t* w, const uint8_t* y, size_t nb);
 
 static row_dot_fn oa_dot_of(int dtype) {
@@ -548,6 +661,10 @@ static row_dot_fn oa_dot_of(int dtype) {
         case LKO_Q5_K: return oa_dot_q5k;
         case LKO_Q6_K: return oa_dot_q6k;
         case LKO_Q8_0: return oa_dot_q80;
+        case LKO_Q4_0: return oa_dot_q40;
+        case LKO_Q4_1: return oa_dot_q41;
+        case LKO_Q5_0: return oa_dot_q50;
+        case LKO_Q5_1: return oa_dot_q51;
         default: return NULL;
     }
 }
@@ -557,16 +674,23 @@ static row_dot_fn ob_dot_of(int dtype) {
         case LKO_Q5_K: return ob_dot_q5k;
         case LKO_Q6_K: return ob_dot_q6k;
         case LKO_Q8_0: return ob_dot_q80;
+        case LKO_Q4_0: return ob_dot_q40;
+        case LKO_Q4_1: return ob_dot_q41;
+        case LKO_Q5_0: return ob_dot_q50;
+        case LKO_Q5_1: return ob_dot_q51;
         default: return NULL;
     }
 }
 
 /* O-A activation: Q8_K for K-quants, Q8_0 for Q8_0 (BlockFormat::ActivationBlock). */
 static size_t oa_act_row_bytes(int dtype, size_t k) {
-    return dtype == LKO_Q8_0 ? (k / 32) * LKO_Q80_BYTES : (k / 256) * LKO_Q8K_BYTES;
+    if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0) return (k / 32) * LKO_Q80_BYTES;
+    if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1) return (k / 32) * LKO_Q81_BYTES;   /* q4_1.rs: BlockQ8_1 */
+    return (k / 256) * LKO_Q8K_BYTES;
 }
 static void oa_quantize_act(int dtype, const float* x, size_t k, uint8_t* out) {
-    if (dtype == LKO_Q8_0) lko_quantize_q8_0(x, k, out);
+    if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0) lko_quantize_q8_0(x, k, out);
+    else if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1) lko_quantize_q8_1(x, k, out);
     else lko_quantize_q8_k(x, k, out);
 }
 
@@ -611,7 +735,9 @@ int oa_matmul_exact(int dtype, size_t m, size_t k, size_t n, const float* lhs,
 int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t* act,
                int32_t* dots, int32_t* sums) {
     const size_t blk = (size_t)lko_block_len(dtype);
-    if (blk == 0 || (dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
+    legacy_layout ll;
+    const int legacy = legacy_layout_of(dtype, &ll);
+    if (blk == 0 || (!legacy && dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
     if (k % blk != 0) return -1;
     const size_t nb = k / blk;
     const size_t wrow = nb * (size_t)lko_block_bytes(dtype);
@@ -641,6 +767,10 @@ int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t*
                 for (int s = 0; s < 8; ++s) memcpy(acts + 32 * s, act + (b * 8 + s) * LKO_Q81_BYTES + 4, 32);
                 q6k_sub_dots(w + b * LKO_Q6K_BYTES, acts, dots + c * (k / 16) + b * 16);
             }
+        } else if (legacy) {
+            for (size_t b = 0; b < nb; ++b)
+                dots[c * nb + b] = legacy_sub_dot(w + b * (size_t)ll.bytes, &ll,
+                                                  (const int8_t*)(act + b * LKO_Q81_BYTES + 4));
         } else {
             for (size_t b = 0; b < nb; ++b)
                 dots[c * nb + b] = i8_dot32((const int8_t*)(w + b * LKO_Q80_BYTES + 2),
@@ -723,6 +853,16 @@ static int dequant_row_f64(int dtype, const uint8_t* w, size_t nb, double* out) 
             const uint8_t* x = w + b * LKO_Q80_BYTES;
             const double d = lko_f16_to_f32(rd_u16(x));
             for (int l = 0; l < 32; ++l) out[b * 32 + l] = d * (double)(int8_t)x[2 + l];
+        }
+        return 0;
+    }
+    legacy_layout ll;
+    if (legacy_layout_of(dtype, &ll)) {
+        for (size_t b = 0; b < nb; ++b) {
+            const uint8_t* x = w + b * (size_t)ll.bytes;
+            const double d = lko_f16_to_f32(rd_u16(x));
+            const double m = ll.m_at >= 0 ? lko_f16_to_f32(rd_u16(x + ll.m_at)) : 0.0;
+            for (int v = 0; v < 32; ++v) out[b * 32 + v] = d * (double)(legacy_code(x, &ll, v) - ll.bias) + m;
         }
         return 0;
     }

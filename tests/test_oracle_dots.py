@@ -14,8 +14,9 @@ import pytest
 import oracle
 from loken_amd import synth
 
-DT = {"q4_k": oracle.Q4_K, "q5_k": oracle.Q5_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0}
-FAST = sorted(set(DT) - {"q5_k"})   # formats the timed AVX2 baseline serves
+LEGACY = {"q4_0": oracle.Q4_0, "q4_1": oracle.Q4_1, "q5_0": oracle.Q5_0, "q5_1": oracle.Q5_1}
+DT = {"q4_k": oracle.Q4_K, "q5_k": oracle.Q5_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0, **LEGACY}
+FAST = sorted(set(DT) - {"q5_k"} - set(LEGACY))   # formats the timed AVX2 baseline serves
 
 
 # ---- independent numpy decoders: integer codes and float scales per value ----
@@ -67,6 +68,22 @@ def np_codes_q80(w):
     return codes, d
 
 
+def np_codes_legacy(dtype, w):
+    """w [n, nb, bytes] of a 32-value nibble format -> codes less their bias [n, nb*32], d, m [n, nb]."""
+    n, nb, _ = w.shape
+    qs_at = {oracle.Q4_0: 2, oracle.Q4_1: 4, oracle.Q5_0: 6, oracle.Q5_1: 8}[dtype]
+    qs = w[:, :, qs_at:qs_at + 16].astype(np.int64)
+    codes = np.concatenate([qs & 0xF, qs >> 4], axis=2)                       # value v at [..., v]
+    if dtype in (oracle.Q5_0, oracle.Q5_1):
+        qh = w[:, :, qs_at - 4:qs_at].copy().view(np.uint32).reshape(n, nb, 1).astype(np.int64)
+        codes = codes | (((qh >> np.arange(32)[None, None, :]) & 1) << 4)
+    codes = codes - {oracle.Q4_0: 8, oracle.Q5_0: 16}.get(dtype, 0)
+    d = w[:, :, 0:2].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+    m = (w[:, :, 2:4].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+         if dtype in (oracle.Q4_1, oracle.Q5_1) else np.zeros((n, nb)))
+    return codes.reshape(n, nb * 32), d, m
+
+
 def np_q81(act_bytes):
     b = act_bytes.reshape(-1, 36)
     d = b[:, 0:2].copy().view(np.float16).reshape(-1).astype(np.float64)
@@ -84,12 +101,16 @@ def np_dequant(dtype, w):
     if dtype == oracle.Q6_K:
         codes, sc, d = np_codes_q6k(w)
         return np.repeat(sc * np.repeat(d, 16, axis=1), 16, axis=1) * codes
+    if dtype in LEGACY.values():
+        codes, d, m = np_codes_legacy(dtype, w)
+        return np.repeat(d, 32, axis=1) * codes + np.repeat(m, 32, axis=1)
     codes, d = np_codes_q80(w)
     return np.repeat(d, 32, axis=1) * codes
 
 
 def test_numpy_decoders_agree_with_ggml(ggml_vectors):
-    for name, dtype in (("q4_K", oracle.Q4_K), ("q5_K", oracle.Q5_K), ("q6_K", oracle.Q6_K), ("q8_0", oracle.Q8_0)):
+    for name, dtype in (("q4_K", oracle.Q4_K), ("q5_K", oracle.Q5_K), ("q6_K", oracle.Q6_K), ("q8_0", oracle.Q8_0),
+                        ("q4_0", oracle.Q4_0), ("q4_1", oracle.Q4_1), ("q5_0", oracle.Q5_0), ("q5_1", oracle.Q5_1)):
         rec = ggml_vectors[name]
         w = rec["quant"].reshape(1, -1, rec["block_bytes"])
         got = np_dequant(dtype, w).reshape(-1)
@@ -114,7 +135,7 @@ def test_integer_subdots_match_numpy_brute_force(name):
         codes = np_codes_q6k(w)[0]
         want = (codes * q[None, :]).reshape(n, k // 16, 16).sum(axis=2)
     else:
-        codes = np_codes_q80(w)[0]
+        codes = np_codes_legacy(dtype, w)[0] if dtype in LEGACY.values() else np_codes_q80(w)[0]
         want = (codes * q[None, :]).reshape(n, k // 32, 32).sum(axis=2)
     assert dots.astype(np.int64).tolist() == want.tolist()
 
@@ -190,15 +211,24 @@ def test_served_path_integer_core_with_q8k_codes(name):
     n, k = 8, 768
     w = synth.weight(dtype, n, k, seed=15, stream=4)
     x = synth.activation(2, k, seed=15)
-    if dtype == oracle.Q8_0:
+    slack = 0.0
+    if dtype in (oracle.Q8_0, oracle.Q4_0, oracle.Q5_0):
         xa = oracle.dequantize(oracle.Q8_0, oracle.quantize_q8_0(x)).reshape(2, k)
+    elif dtype in (oracle.Q4_1, oracle.Q5_1):
+        # these pair with Q8_1 and take the block's sum from its f16 `s` field: the minimum's term
+        # carries that field's rounding (2^-11 of |m * s| per block)
+        d8, q = np_q81(oracle.quantize_q8_1(x))
+        xa = (d8[:, None] * q).reshape(2, k)
+        m = np.abs(np_codes_legacy(dtype, w)[2])                                   # [n, nb]
+        s_abs = np.abs(xa.reshape(2, k // 32, 32).sum(axis=2))                     # [rows, nb]
+        slack = 2.0 ** -11 * (s_abs @ m.T)
     else:
         xa = oracle.dequantize(oracle.Q8_K, oracle.quantize_q8_k(x)).reshape(2, k)
     wd = np_dequant(dtype, w)
     ref = xa.astype(np.float64) @ wd.T
     got = oracle.oa_matmul(dtype, x, w, n)
     absdot = np.abs(xa.astype(np.float64)) @ np.abs(wd).T
-    assert (np.abs(got - ref) <= 4e-6 * absdot + 1e-9).all()
+    assert (np.abs(got - ref) <= 4e-6 * absdot + 1e-9 + slack).all()
 
 
 @pytest.mark.parametrize("name", FAST)
@@ -221,7 +251,7 @@ def test_driver_error_conditions():
     with pytest.raises(oracle.OracleError, match="byte length"):
         oracle.oa_matmul(oracle.Q4_K, np.zeros((1, 512), np.float32), w, 5)
     with pytest.raises(oracle.OracleError, match="not handled"):
-        oracle.oa_matmul(3, np.zeros((1, 512), np.float32), w, 4)
+        oracle.oa_matmul(10, np.zeros((1, 512), np.float32), w, 4)   # Q2_K: no statement of it here
 
 
 def test_empty_rows_and_columns():
