@@ -30,6 +30,10 @@ extern "C" {
 /* ggml type ids (src/tensor/quantized/dtype.rs:66-96) */
 #define LK_TYPE_F32 0
 #define LK_TYPE_F16 1
+#define LK_TYPE_Q4_0 2
+#define LK_TYPE_Q4_1 3
+#define LK_TYPE_Q5_0 6
+#define LK_TYPE_Q5_1 7
 #define LK_TYPE_Q8_0 8
 #define LK_TYPE_Q8_1 9
 #define LK_TYPE_Q4_K 12
@@ -65,7 +69,8 @@ int lk_quantize_q8_1(const void* x, int x_type, void* vy, int kx, int kx_padded,
                      void* stream);
 
 /* dst[j, row] = weight row `row` . activation row j, j < batch (1..8).
- *   wtype          LK_TYPE_Q4_K | LK_TYPE_Q5_K | LK_TYPE_Q6_K | LK_TYPE_Q8_0
+ *   wtype          LK_TYPE_Q4_K | LK_TYPE_Q5_K | LK_TYPE_Q6_K | LK_TYPE_Q8_0, and (this launcher and
+ *                  lk_mmvq_subdots only) the 32-value nibble formats LK_TYPE_Q4_0 | Q4_1 | Q5_0 | Q5_1
  *   vx             nrows_x rows of ncols_x / block_len blocks
  *   vy_q8_1        batch rows of Q8_1 blocks, `stride_col_y` blocks apart (k_padded / 32)
  *   dst            `dst_type` LK_TYPE_F32 | F16 | BF16, rows `stride_col_dst` elements apart

@@ -119,6 +119,13 @@ const LkDevice& lk_device();
 int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y,
                      int ldd, hipStream_t stream);
 
+// The 32-value nibble formats (mmvq_legacy.hip); status LK_*.
+bool lk_is_legacy_type(int wtype);
+int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, int dst_type, int ncols_x, int nrows_x,
+                   int batch, int stride_col_y, int stride_col_dst, const float* bias, hipStream_t stream);
+int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32_t* dots, int ncols_x, int nrows_x,
+                           hipStream_t stream);
+
 static inline int lk_launch_status() {
     return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;
 }

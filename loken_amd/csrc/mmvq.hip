@@ -518,6 +518,9 @@ extern "C" int lk_mmvq(int wtype, const void* vx, const void* vy_q8_1, void* dst
                        int ncols_x, int nrows_x, int batch, int stride_col_y, int stride_col_dst,
                        const float* bias, int decode_order, void* stream) {
     (void)decode_order;  // a row's sum never depends on batch here
+    if (lk_is_legacy_type(wtype))   // Q4_0, Q4_1, Q5_0, Q5_1: the plain kernel of mmvq_legacy.hip
+        return lk_mmvq_legacy(wtype, vx, vy_q8_1, dst, dst_type, ncols_x, nrows_x, batch, stride_col_y, stride_col_dst,
+                              bias, (hipStream_t)stream);
     if (block_len_of(wtype) == 0) return LK_ERR_TYPE;
     if (nrows_x == 0) return LK_OK;
     return run_multi(wtype, 1, &vx, vy_q8_1, &dst, dst_type, ncols_x, &nrows_x, batch, stride_col_y, stride_col_dst,
@@ -646,6 +649,15 @@ extern "C" int lk_mmvq_grouped(int wtype, const uint64_t* table, int groups, con
 
 extern "C" int lk_mmvq_subdots(int wtype, const void* vx, const void* vy_q8_1, int32_t* dots,
                                int32_t* sums, int ncols_x, int nrows_x, void* stream) {
+    if (lk_is_legacy_type(wtype)) {
+        if (int rc = lk_mmvq_subdots_legacy(wtype, vx, vy_q8_1, dots, ncols_x, nrows_x, (hipStream_t)stream)) return rc;
+        if (sums) {
+            const int k32 = ncols_x / 32;
+            hipLaunchKernelGGL(act_sums_kernel, dim3((k32 + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                               (const uint8_t*)vy_q8_1, sums, k32);
+        }
+        return lk_launch_status();
+    }
     const int bl = block_len_of(wtype);
     if (bl == 0) return LK_ERR_TYPE;
     if (!vx || !vy_q8_1 || !dots || ncols_x <= 0 || nrows_x <= 0 || ncols_x % bl != 0) return LK_ERR_ARG;

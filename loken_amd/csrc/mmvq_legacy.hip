@@ -1,0 +1,187 @@
+// Mat-vec for the 32-value nibble formats Q4_0, Q4_1, Q5_0, Q5_1 against Q8_1 activation rows.
+//
+// Formats as loken states them (src/tensor/quant_cpu/format/q4_0.rs, q4_1.rs, q5_0.rs, q5_1.rs): byte
+// j of `qs` holds value j in its low nibble and value j + 16 in its high one; the five-bit formats
+// keep bit v of the little-endian word `qh` as value v's fifth bit. Q4_0 {d, qs} and Q5_0 {d, qh,
+// qs} mean (code - 8 / 16) * d; Q4_1 {d, m, qs} and Q5_1 {d, m, qh, qs} mean code * d + m.
+// Per block the product with a Q8_1 block {d8, codes a} is, as the reference's mat-vec forms it
+// (cuda/moe/gguf.cuh:392-441: total_biased_codes, total_with_minimum), with the sum of the
+// activation codes taken as the integer it is (as every kernel of this library takes it):
+//     d * d8 * (sum code * a - bias * sum a)            Q4_0 (bias 8), Q5_0 (bias 16)
+//     d * d8 * (sum code * a) + m * (d8 * sum a)        Q4_1, Q5_1
+// Replaces kernels `mmvq_gguf_{q4_0,q4_1,q5_0,q5_1}_{f32,f16,bf16}_plain_cuda{1..8}`
+// (src/inference/cuda/mmvq_gguf.cu:338-363) behind lk_mmvq.
+//
+// Shape: a wave owns a weight row; its lanes walk the row's blocks 64 at a time (consecutive lanes
+// read consecutive 18..24-byte blocks, so a wave's loads cover one contiguous run), each lane forms
+// its block's integers against every activation row of the batch and the wave folds once per row.
+// The activation blocks come straight from memory: a row of them is a few KB and stays in cache.
+// These formats are the long tail of the reference's table; this kernel is the plain statement,
+// without the LDS staging and register pipelines of the K-quant engines.
+
+#include "lk_common.h"
+
+namespace {
+
+constexpr int LWG = 256, LWAVES = 4;
+
+template <int ID> struct Legacy;
+template <> struct Legacy<2> { static constexpr int BYTES = 18, M_AT = -1, QH_AT = -1, QS_AT = 2, BIAS = 8; };
+template <> struct Legacy<3> { static constexpr int BYTES = 20, M_AT = 2, QH_AT = -1, QS_AT = 4, BIAS = 0; };
+template <> struct Legacy<6> { static constexpr int BYTES = 22, M_AT = -1, QH_AT = 2, QS_AT = 6, BIAS = 16; };
+template <> struct Legacy<7> { static constexpr int BYTES = 24, M_AT = 2, QH_AT = 4, QS_AT = 8, BIAS = 0; };
+
+// Four bits of `x` (bits 0..3) to bit 4 of four bytes: byte i receives bit i. The multiplier lays
+// the nibble down at shifts 0, 7, 14, 21, which puts bit i at position 8 i; the copies do not overlap.
+static __device__ __forceinline__ uint32_t fifth_bits(uint32_t x) {
+    return (((x & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+}
+
+// A block's unsigned codes: lo = values 0..15, hi = values 16..31, four per dword.
+template <class F>
+static __device__ __forceinline__ void block_codes(const uint8_t* __restrict__ bp, uint4& lo, uint4& hi) {
+    const uint4 q = *(const uint4_a2*)(bp + F::QS_AT);
+    lo = make_uint4(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu, q.z & 0x0F0F0F0Fu, q.w & 0x0F0F0F0Fu);
+    hi = make_uint4((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu, (q.z >> 4) & 0x0F0F0F0Fu, (q.w >> 4) & 0x0F0F0F0Fu);
+    if (F::QH_AT >= 0) {
+        const uint32_t qh = (uint32_t)*(const uint16_t*)(bp + F::QH_AT) | ((uint32_t)*(const uint16_t*)(bp + F::QH_AT + 2) << 16);
+        lo.x |= fifth_bits(qh);       lo.y |= fifth_bits(qh >> 4);  lo.z |= fifth_bits(qh >> 8);  lo.w |= fifth_bits(qh >> 12);
+        hi.x |= fifth_bits(qh >> 16); hi.y |= fifth_bits(qh >> 20); hi.z |= fifth_bits(qh >> 24); hi.w |= fifth_bits(qh >> 28);
+    }
+}
+
+// The block's integer against one Q8_1 block: sum (code - bias) * a, and the sum of a.
+static __device__ __forceinline__ void block_dot(const uint4& lo, const uint4& hi, const uint8_t* __restrict__ yb, int bias,
+                                                 int& dot, int& asum) {
+    const uint4 a_lo = *(const uint4_a4*)(yb + 4), a_hi = *(const uint4_a4*)(yb + 20);
+    const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
+    asum = dot16(ones, a_hi, dot16(ones, a_lo, 0));
+    dot = dot16(hi, a_hi, dot16(lo, a_lo, 0)) - bias * asum;
+}
+
+template <int ID, int B, typename T>
+__global__ __launch_bounds__(LWG) void mmvq_legacy_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
+                                                          T* __restrict__ dst, const float* __restrict__ bias, int nb, int n,
+                                                          int stride_col_y, int stride_col_dst) {
+    using F = Legacy<ID>;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    for (int row = blockIdx.x * LWAVES + wave; row < n; row += gridDim.x * LWAVES) {
+        const uint8_t* wrow = vx + (size_t)row * nb * F::BYTES;
+        float acc[B];
+#pragma unroll
+        for (int c = 0; c < B; ++c) acc[c] = 0.f;
+        for (int b = lane; b < nb; b += 64) {
+            const uint8_t* bp = wrow + (size_t)b * F::BYTES;
+            uint4 lo, hi;
+            block_codes<F>(bp, lo, hi);
+            const float d = f16_bits_to_f32(*(const uint16_t*)bp);
+            const float m = F::M_AT >= 0 ? f16_bits_to_f32(*(const uint16_t*)(bp + (F::M_AT >= 0 ? F::M_AT : 0))) : 0.f;
+#pragma unroll
+            for (int c = 0; c < B; ++c) {
+                const uint8_t* yb = vy + ((size_t)c * stride_col_y + b) * Q81_BYTES;
+                const float d8 = f16_bits_to_f32(*(const uint16_t*)yb);
+                int dot, asum;
+                block_dot(lo, hi, yb, F::BIAS, dot, asum);
+                float part = d * d8 * (float)dot;
+                if (F::M_AT >= 0) part += m * (d8 * (float)asum);
+                acc[c] += part;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < B; ++c) {
+            const float total = wave_sum(acc[c]);
+            if (lane == 0) dst[(size_t)c * stride_col_dst + row] = from_f32<T>(bias ? total + bias[row] : total);
+        }
+    }
+}
+
+// The parity probe: every block's integer (sum (code - bias) * a) against ONE Q8_1 row.
+template <int ID>
+__global__ __launch_bounds__(64) void subdots_legacy_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
+                                                            int32_t* __restrict__ dots, int nb) {
+    using F = Legacy<ID>;
+    const int row = blockIdx.y, b = blockIdx.x * 64 + threadIdx.x;
+    if (b >= nb) return;
+    uint4 lo, hi;
+    block_codes<F>(vx + ((size_t)row * nb + b) * F::BYTES, lo, hi);
+    int dot, asum;
+    block_dot(lo, hi, vy + (size_t)b * Q81_BYTES, F::BIAS, dot, asum);
+    dots[(size_t)row * nb + b] = dot;
+}
+
+template <int ID, int B, typename T>
+static int launch(const void* vx, const void* vy, void* dst, const float* bias, int nb, int n, int stride_col_y,
+                  int stride_col_dst, hipStream_t s) {
+    const int need = (n + LWAVES - 1) / LWAVES, cap = lk_device().cus * 8;
+    hipLaunchKernelGGL((mmvq_legacy_kernel<ID, B, T>), dim3(need < cap ? need : cap), dim3(LWG), 0, s, (const uint8_t*)vx,
+                       (const uint8_t*)vy, (T*)dst, bias, nb, n, stride_col_y, stride_col_dst);
+    return lk_launch_status();
+}
+
+template <int ID, typename T>
+static int by_batch(int batch, const void* vx, const void* vy, void* dst, const float* bias, int nb, int n,
+                    int stride_col_y, int stride_col_dst, hipStream_t s) {
+    // batches above four go out as two launches: the per-lane accumulators stay few
+    if (batch > 4) {
+        if (int rc = by_batch<ID, T>(4, vx, vy, dst, bias, nb, n, stride_col_y, stride_col_dst, s)) return rc;
+        return by_batch<ID, T>(batch - 4, vx, (const uint8_t*)vy + (size_t)4 * stride_col_y * Q81_BYTES,
+                               (T*)dst + (size_t)4 * stride_col_dst, bias, nb, n, stride_col_y, stride_col_dst, s);
+    }
+    switch (batch) {
+        case 1: return launch<ID, 1, T>(vx, vy, dst, bias, nb, n, stride_col_y, stride_col_dst, s);
+        case 2: return launch<ID, 2, T>(vx, vy, dst, bias, nb, n, stride_col_y, stride_col_dst, s);
+        case 3: return launch<ID, 3, T>(vx, vy, dst, bias, nb, n, stride_col_y, stride_col_dst, s);
+        default: return launch<ID, 4, T>(vx, vy, dst, bias, nb, n, stride_col_y, stride_col_dst, s);
+    }
+}
+
+template <int ID>
+static int by_type(int dst_type, int batch, const void* vx, const void* vy, void* dst, const float* bias, int nb, int n,
+                   int stride_col_y, int stride_col_dst, hipStream_t s) {
+    switch (dst_type) {
+        case LK_TYPE_F32: return by_batch<ID, float>(batch, vx, vy, dst, bias, nb, n, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_F16: return by_batch<ID, __half>(batch, vx, vy, dst, bias, nb, n, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_BF16: return by_batch<ID, __hip_bfloat16>(batch, vx, vy, dst, bias, nb, n, stride_col_y, stride_col_dst, s);
+        default: return LK_ERR_TYPE;
+    }
+}
+
+}  // namespace
+
+bool lk_is_legacy_type(int wtype) {
+    return wtype == LK_TYPE_Q4_0 || wtype == LK_TYPE_Q4_1 || wtype == LK_TYPE_Q5_0 || wtype == LK_TYPE_Q5_1;
+}
+
+// lk_mmvq for the 32-value nibble formats (the caller has told them apart with lk_is_legacy_type).
+int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, int dst_type, int ncols_x, int nrows_x,
+                   int batch, int stride_col_y, int stride_col_dst, const float* bias, hipStream_t s) {
+    if (nrows_x == 0) return LK_OK;
+    if (!vx || !vy_q8_1 || !dst || ncols_x <= 0 || ncols_x % 32 != 0 || nrows_x < 0) return LK_ERR_ARG;
+    if (batch < 1 || batch > 8 || stride_col_y < ncols_x / 32 || stride_col_dst < nrows_x) return LK_ERR_ARG;
+    if (((uintptr_t)vx & 1) != 0 || ((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
+    const int nb = ncols_x / 32;
+    switch (wtype) {
+        case LK_TYPE_Q4_0: return by_type<2>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_Q4_1: return by_type<3>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_Q5_0: return by_type<6>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_Q5_1: return by_type<7>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        default: return LK_ERR_TYPE;
+    }
+}
+
+int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32_t* dots, int ncols_x, int nrows_x,
+                           hipStream_t s) {
+    if (!vx || !vy_q8_1 || !dots || ncols_x <= 0 || ncols_x % 32 != 0 || nrows_x <= 0 || nrows_x > 65535) return LK_ERR_ARG;
+    const int nb = ncols_x / 32;
+    const dim3 grid((nb + 63) / 64, nrows_x);
+    const uint8_t *w = (const uint8_t*)vx, *y = (const uint8_t*)vy_q8_1;
+    switch (wtype) {
+        case LK_TYPE_Q4_0: hipLaunchKernelGGL(subdots_legacy_kernel<2>, grid, dim3(64), 0, s, w, y, dots, nb); break;
+        case LK_TYPE_Q4_1: hipLaunchKernelGGL(subdots_legacy_kernel<3>, grid, dim3(64), 0, s, w, y, dots, nb); break;
+        case LK_TYPE_Q5_0: hipLaunchKernelGGL(subdots_legacy_kernel<6>, grid, dim3(64), 0, s, w, y, dots, nb); break;
+        case LK_TYPE_Q5_1: hipLaunchKernelGGL(subdots_legacy_kernel<7>, grid, dim3(64), 0, s, w, y, dots, nb); break;
+        default: return LK_ERR_TYPE;
+    }
+    return lk_launch_status();
+}

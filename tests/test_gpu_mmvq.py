@@ -16,6 +16,8 @@ from loken_amd import lib, ops, synth
 pytestmark = pytest.mark.gpu
 
 DT = {"q4_k": lib.TYPE_Q4_K, "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0}
+# the 32-value nibble formats: served by lk_mmvq and the sub-dot probe only
+LEGACY = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1}
 RTOL, ATOL = 1e-3, 1e-4
 
 
@@ -89,6 +91,63 @@ def test_q4k_extreme_subdot_on_gpu():
     x = np.full((1, 256), 127.0, np.float32)
     dots, sums = ops.mmvq_subdots(lib.TYPE_Q4_K, dev(w), ops.quantize_q8_1_rows(dev(x))[0], 256, 1)
     assert dots.cpu().tolist() == [[60960] * 8] and sums.cpu().tolist() == [127 * 32] * 8
+
+
+@pytest.mark.parametrize("name", sorted(LEGACY))
+@pytest.mark.parametrize("n,k", [(16, 1024), (5, 96), (3, 32), (70, 4096)])
+def test_legacy_integer_block_dots_are_bit_exact(name, n, k):
+    wtype = LEGACY[name]
+    w = synth.weight(wtype, n, k, seed=70, stream=1)
+    x = synth.activation(1, k, seed=70)
+    q = ops.quantize_q8_1_rows(dev(x))
+    dots, sums = ops.mmvq_subdots(wtype, dev(w), q[0], k, n)
+    want_dots, want_sums = oracle.ob_subdots(wtype, k, n, w, oracle.quantize_q8_1(x))
+    assert np.array_equal(dots.cpu().numpy(), want_dots)
+    assert np.array_equal(sums.cpu().numpy(), want_sums)
+
+
+@pytest.mark.parametrize("name", sorted(LEGACY))
+@pytest.mark.parametrize("n,k", [(4096, 4096), (33, 96), (1, 32), (257, 2080), (1000, 14336)])
+@pytest.mark.parametrize("batch", [1, 3, 4, 7, 8])
+def test_legacy_matvec_matches_same_codes_oracle(name, n, k, batch):
+    wtype = LEGACY[name]
+    w = synth.weight(wtype, n, k, seed=71, stream=2)
+    x = synth.activation(batch, k, seed=71)
+    got = ops.mmvq(wtype, dev(w), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(wtype, x, w, n))
+
+
+@pytest.mark.parametrize("name", sorted(LEGACY))
+def test_legacy_matvec_extremes_bias_and_half_outputs(name):
+    wtype = LEGACY[name]
+    n, k = 40, 256
+    # every code at its maximum against every activation code at +-127
+    w = synth.weight(wtype, n, k, seed=72, stream=3)
+    qs_at = {"q4_0": 2, "q4_1": 4, "q5_0": 6, "q5_1": 8}[name]
+    w[:, :, qs_at - (4 if name.startswith("q5") else 0):] = 0xFF
+    x = np.where(np.arange(k) % 2 == 0, 127.0, -127.0).astype(np.float32).reshape(1, k) * np.float32(0.5)
+    q = ops.quantize_q8_1_rows(dev(x))
+    got = ops.mmvq(wtype, dev(w), q, k, n)
+    assert_close(got.cpu().numpy(), oracle.ob_matmul(wtype, x, w, n))
+    bias = dev(synth.normal(72, 9, n))
+    with_bias = ops.mmvq(wtype, dev(w), q, k, n, bias=bias)
+    assert torch.equal(with_bias, got + bias)
+    for t in (torch.float16, torch.bfloat16):
+        assert torch.equal(ops.mmvq(wtype, dev(w), q, k, n, out_dtype=t), got.to(t))
+
+
+@pytest.mark.parametrize("name", sorted(LEGACY))
+def test_legacy_matvec_within_the_reference_envelope(name):
+    wtype = LEGACY[name]
+    n, k = 256, 4096
+    w = synth.weight(wtype, n, k, seed=73, stream=4)
+    x = synth.activation(2, k, seed=73)
+    got = ops.mmvq(wtype, dev(w), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
+    wd = oracle.dequantize(wtype, w).reshape(n, k).astype(np.float64)
+    truth = x.astype(np.float64) @ wd.T
+    envelope = 1e-3 * (np.abs(x.astype(np.float64)) @ np.abs(wd).T) + 1e-3
+    assert (np.abs(got - truth) <= envelope).all()
+    assert (np.abs(oracle.oa_matmul(wtype, x, w, n) - truth) <= envelope).all()
 
 
 # ---------------------------------------------------------------- f32 outputs
