@@ -21,9 +21,10 @@ from __future__ import annotations
 import numpy as np
 
 GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1 = 2, 3, 6, 7
+GGML_IQ4_NL, GGML_MXFP4 = 20, 39
 GGML_Q8_0, GGML_Q8_1, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K = 8, 9, 12, 13, 14
-BLOCK_LEN = {GGML_Q4_0: 32, GGML_Q4_1: 32, GGML_Q5_0: 32, GGML_Q5_1: 32, GGML_Q8_0: 32, GGML_Q8_1: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256}
-BLOCK_BYTES = {GGML_Q4_0: 18, GGML_Q4_1: 20, GGML_Q5_0: 22, GGML_Q5_1: 24, GGML_Q8_0: 34, GGML_Q8_1: 36, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210}
+BLOCK_LEN = {GGML_IQ4_NL: 32, GGML_MXFP4: 32, GGML_Q4_0: 32, GGML_Q4_1: 32, GGML_Q5_0: 32, GGML_Q5_1: 32, GGML_Q8_0: 32, GGML_Q8_1: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256}
+BLOCK_BYTES = {GGML_IQ4_NL: 18, GGML_MXFP4: 17, GGML_Q4_0: 18, GGML_Q4_1: 20, GGML_Q5_0: 22, GGML_Q5_1: 24, GGML_Q8_0: 34, GGML_Q8_1: 36, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210}
 
 _G = np.uint64(0x9E3779B97F4A7C15)
 _M1 = np.uint64(0xBF58476D1CE4E5B9)
@@ -134,10 +135,17 @@ def legacy_blocks(dtype: int, n_blocks: int, seed: int = 0, stream: int = 0) -> 
     out[:, 0:2] = _f16_bytes(np.abs(normal(seed, s + 1, n_blocks)) * np.float32(2e-3))
     if dtype in (GGML_Q4_1, GGML_Q5_1):
         out[:, 2:4] = _f16_bytes(normal(seed, s + 2, n_blocks) * np.float32(1e-2))
+    if dtype == GGML_IQ4_NL:
+        out[:, 0:2] = _f16_bytes(np.abs(normal(seed, s + 1, n_blocks)) * np.float32(2e-4))
+    if dtype == GGML_MXFP4:   # the scale is one E8M0 byte: 0.5 * 2^(e - 127), here 2^-12 .. 2^-5
+        out[:, 1:2] = out[:, 2:3]   # (byte 1 is a code byte again)
+        out[:, 0] = 116 + rand_ints(seed, s + 3, n_blocks, 8)
     return out
 
 
-_MAKERS = {GGML_Q4_0: lambda n, seed=0, stream=0: legacy_blocks(GGML_Q4_0, n, seed, stream),
+_MAKERS = {GGML_IQ4_NL: lambda n, seed=0, stream=0: legacy_blocks(GGML_IQ4_NL, n, seed, stream),
+           GGML_MXFP4: lambda n, seed=0, stream=0: legacy_blocks(GGML_MXFP4, n, seed, stream),
+           GGML_Q4_0: lambda n, seed=0, stream=0: legacy_blocks(GGML_Q4_0, n, seed, stream),
            GGML_Q4_1: lambda n, seed=0, stream=0: legacy_blocks(GGML_Q4_1, n, seed, stream),
            GGML_Q5_0: lambda n, seed=0, stream=0: legacy_blocks(GGML_Q5_0, n, seed, stream),
            GGML_Q5_1: lambda n, seed=0, stream=0: legacy_blocks(GGML_Q5_1, n, seed, stream),

@@ -79,7 +79,8 @@ uint16_t lko_f32_to_f16(float f) {
 
 int lko_block_len(int dtype) {
     switch (dtype) {
-        case LKO_Q8_0: case LKO_Q8_1: case LKO_Q4_0: case LKO_Q4_1: case LKO_Q5_0: case LKO_Q5_1: return 32;
+        case LKO_Q8_0: case LKO_Q8_1: case LKO_Q4_0: case LKO_Q4_1: case LKO_Q5_0: case LKO_Q5_1:
+        case LKO_IQ4_NL: case LKO_MXFP4: return 32;
         case LKO_Q4_K: case LKO_Q5_K: case LKO_Q6_K: case LKO_Q8_K: return 256;
         default: return 0;
     }
@@ -92,6 +93,8 @@ int lko_block_bytes(int dtype) {
         case LKO_Q4_1: return 20;
         case LKO_Q5_0: return 22;
         case LKO_Q5_1: return 24;
+        case LKO_IQ4_NL: return 18;
+        case LKO_MXFP4: return 17;
         case LKO_Q8_1: return LKO_Q81_BYTES;
         case LKO_Q4_K: return LKO_Q4K_BYTES;
         case LKO_Q5_K: return LKO_Q5K_BYTES;
@@ -553,19 +556,38 @@ static float ob_dot_q80(const uint8_t* w, const uint8_t* y, size_t nb) {
  * bit v of the little-endian word `qh` as value v's fifth bit. Q4_0 {d, qs} and Q5_0 {d, qh, qs}
  * mean (code - 8 / 16) * d; Q4_1 {d, m, qs} and Q5_1 {d, m, qh, qs} mean code * d + m.
  * ---------------------------------------------------------------------------------------- */
-typedef struct { int bytes, m_at, qh_at, qs_at, bias; } legacy_layout;
+/* IQ4_NL {d, qs} and MXFP4 {e, qs} pack their nibbles the same way but a code names a level of a
+ * table: iq4_nl.rs:11-13 (d * LEVELS[code]), mxfp4.rs / blocks.rs:24-42 (KVALUES_MXFP4[code] * the
+ * block's E8M0 scale as e8m0_to_fp32_half gives it: 0.5 * 2^(e - 127), denormal patterns below 2). */
+static const int8_t LEVELS_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+static const int8_t LEVELS_MXFP4[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+
+static float e8m0_to_f32_half(uint8_t e) {
+    const uint32_t bits = e < 2 ? (0x00200000u << e) : ((uint32_t)(e - 1) << 23);
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+typedef struct { int bytes, m_at, qh_at, qs_at, bias; const int8_t* levels; } legacy_layout;
 
 static int legacy_layout_of(int dtype, legacy_layout* l) {
     switch (dtype) {
-        case LKO_Q4_0: *l = (legacy_layout){18, -1, -1, 2, 8}; return 1;
-        case LKO_Q4_1: *l = (legacy_layout){20, 2, -1, 4, 0}; return 1;
-        case LKO_Q5_0: *l = (legacy_layout){22, -1, 2, 6, 16}; return 1;
-        case LKO_Q5_1: *l = (legacy_layout){24, 2, 4, 8, 0}; return 1;
+        case LKO_Q4_0: *l = (legacy_layout){18, -1, -1, 2, 8, NULL}; return 1;
+        case LKO_Q4_1: *l = (legacy_layout){20, 2, -1, 4, 0, NULL}; return 1;
+        case LKO_Q5_0: *l = (legacy_layout){22, -1, 2, 6, 16, NULL}; return 1;
+        case LKO_Q5_1: *l = (legacy_layout){24, 2, 4, 8, 0, NULL}; return 1;
+        case LKO_IQ4_NL: *l = (legacy_layout){18, -1, -1, 2, 0, LEVELS_IQ4NL}; return 1;
+        case LKO_MXFP4: *l = (legacy_layout){17, -1, -1, 1, 0, LEVELS_MXFP4}; return 1;
         default: return 0;
     }
 }
 
-/* The unsigned code of value v (q5_0.rs:43-48). */
+/* The unsigned code of value v (q5_0.rs:43-48), or the level it names in a table format. */
+static inline float legacy_scale(const uint8_t* blk, int dtype) {
+    return dtype == LKO_MXFP4 ? e8m0_to_f32_half(blk[0]) : lko_f16_to_f32(rd_u16(blk));
+}
+
 static inline int legacy_code(const uint8_t* blk, const legacy_layout* l, int v) {
     const uint8_t packed = blk[l->qs_at + (v & 15)];
     int code = v < 16 ? (packed & 0x0F) : (packed >> 4);
@@ -574,7 +596,7 @@ static inline int legacy_code(const uint8_t* blk, const legacy_layout* l, int v)
                             ((uint32_t)blk[l->qh_at + 2] << 16) | ((uint32_t)blk[l->qh_at + 3] << 24);
         code |= (int)((qh >> v) & 1u) << 4;
     }
-    return code;
+    return l->levels ? (int)l->levels[code] : code;   /* a table format's "code" is its level */
 }
 
 /* The integer the CPU dots form (q4_0.rs:104-113, q4_1.rs:104-111): sum of (code - bias) * a. */
@@ -589,7 +611,7 @@ static int legacy_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, 
     if (!legacy_layout_of(dtype, &l)) return -3;
     for (size_t b = 0; b < n_blocks; ++b) {
         const uint8_t* blk = blocks + b * (size_t)l.bytes;
-        const float d = lko_f16_to_f32(rd_u16(blk));
+        const float d = legacy_scale(blk, dtype);
         const float m = l.m_at >= 0 ? lko_f16_to_f32(rd_u16(blk + l.m_at)) : 0.0f;
         for (int v = 0; v < 32; ++v) {
             const int code = legacy_code(blk, &l, v);
@@ -610,7 +632,7 @@ static float oa_dot_legacy(int dtype, const uint8_t* w, const uint8_t* y, size_t
         if (l.m_at < 0) {
             const uint8_t* yb = y + b * LKO_Q80_BYTES;
             const int32_t dot = legacy_sub_dot(x, &l, (const int8_t*)(yb + 2));
-            total += (float)dot * lko_f16_to_f32(rd_u16(x)) * lko_f16_to_f32(rd_u16(yb));
+            total += (float)dot * legacy_scale(x, dtype) * lko_f16_to_f32(rd_u16(yb));
         } else {
             const uint8_t* yb = y + b * LKO_Q81_BYTES;
             const int32_t dot = legacy_sub_dot(x, &l, (const int8_t*)(yb + 4));
@@ -634,7 +656,7 @@ static float ob_dot_legacy(int dtype, const uint8_t* w, const uint8_t* y, size_t
         const int8_t* yq = (const int8_t*)(yb + 4);
         const float d8 = lko_f16_to_f32(rd_u16(yb));
         const int32_t dot = legacy_sub_dot(x, &l, yq);
-        float part = lko_f16_to_f32(rd_u16(x)) * d8 * (float)dot;
+        float part = legacy_scale(x, dtype) * d8 * (float)dot;
         if (l.m_at >= 0) {
             int32_t sum = 0;
             for (int v = 0; v < 32; ++v) sum += yq[v];
@@ -652,6 +674,10 @@ static float ob_dot_q40(const uint8_t* w, const uint8_t* y, size_t nb) { return 
 static float ob_dot_q41(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_Q4_1, w, y, nb); }
 static float ob_dot_q50(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_Q5_0, w, y, nb); }
 static float ob_dot_q51(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_Q5_1, w, y, nb); }
+static float oa_dot_iq4nl(const uint8_t* w, const uint8_t* y, size_t nb) { return oa_dot_legacy(LKO_IQ4_NL, w, y, nb); }
+static float oa_dot_mxfp4(const uint8_t* w, const uint8_t* y, size_t nb) { return oa_dot_legacy(LKO_MXFP4, w, y, nb); }
+static float ob_dot_iq4nl(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_IQ4_NL, w, y, nb); }
+static float ob_dot_mxfp4(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_MXFP4, w, y, nb); }
 
 typedef float (*row_dot_fn)(const uint8_t* w, const uint8_t* y, size_t nb);
 
@@ -665,6 +691,8 @@ static row_dot_fn oa_dot_of(int dtype) {
         case LKO_Q4_1: return oa_dot_q41;
         case LKO_Q5_0: return oa_dot_q50;
         case LKO_Q5_1: return oa_dot_q51;
+        case LKO_IQ4_NL: return oa_dot_iq4nl;
+        case LKO_MXFP4: return oa_dot_mxfp4;
         default: return NULL;
     }
 }
@@ -678,18 +706,22 @@ static row_dot_fn ob_dot_of(int dtype) {
         case LKO_Q4_1: return ob_dot_q41;
         case LKO_Q5_0: return ob_dot_q50;
         case LKO_Q5_1: return ob_dot_q51;
+        case LKO_IQ4_NL: return ob_dot_iq4nl;
+        case LKO_MXFP4: return ob_dot_mxfp4;
         default: return NULL;
     }
 }
 
 /* O-A activation: Q8_K for K-quants, Q8_0 for Q8_0 (BlockFormat::ActivationBlock). */
 static size_t oa_act_row_bytes(int dtype, size_t k) {
-    if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0) return (k / 32) * LKO_Q80_BYTES;
+    if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0 || dtype == LKO_IQ4_NL || dtype == LKO_MXFP4)
+        return (k / 32) * LKO_Q80_BYTES;
     if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1) return (k / 32) * LKO_Q81_BYTES;   /* q4_1.rs: BlockQ8_1 */
     return (k / 256) * LKO_Q8K_BYTES;
 }
 static void oa_quantize_act(int dtype, const float* x, size_t k, uint8_t* out) {
-    if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0) lko_quantize_q8_0(x, k, out);
+    if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0 || dtype == LKO_IQ4_NL || dtype == LKO_MXFP4)
+        lko_quantize_q8_0(x, k, out);
     else if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1) lko_quantize_q8_1(x, k, out);
     else lko_quantize_q8_k(x, k, out);
 }
@@ -860,7 +892,7 @@ static int dequant_row_f64(int dtype, const uint8_t* w, size_t nb, double* out) 
     if (legacy_layout_of(dtype, &ll)) {
         for (size_t b = 0; b < nb; ++b) {
             const uint8_t* x = w + b * (size_t)ll.bytes;
-            const double d = lko_f16_to_f32(rd_u16(x));
+            const double d = legacy_scale(x, dtype);
             const double m = ll.m_at >= 0 ? lko_f16_to_f32(rd_u16(x + ll.m_at)) : 0.0;
             for (int v = 0; v < 32; ++v) out[b * 32 + v] = d * (double)(legacy_code(x, &ll, v) - ll.bias) + m;
         }

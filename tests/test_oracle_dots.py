@@ -14,7 +14,10 @@ import pytest
 import oracle
 from loken_amd import synth
 
-LEGACY = {"q4_0": oracle.Q4_0, "q4_1": oracle.Q4_1, "q5_0": oracle.Q5_0, "q5_1": oracle.Q5_1}
+LEGACY = {"q4_0": oracle.Q4_0, "q4_1": oracle.Q4_1, "q5_0": oracle.Q5_0, "q5_1": oracle.Q5_1, "iq4_nl": oracle.IQ4_NL,
+          "mxfp4": oracle.MXFP4}
+LEVELS = {oracle.IQ4_NL: np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64),
+          oracle.MXFP4: np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], np.int64)}
 DT = {"q4_k": oracle.Q4_K, "q5_k": oracle.Q5_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0, **LEGACY}
 FAST = sorted(set(DT) - {"q5_k"} - set(LEGACY))   # formats the timed AVX2 baseline serves
 
@@ -71,14 +74,19 @@ def np_codes_q80(w):
 def np_codes_legacy(dtype, w):
     """w [n, nb, bytes] of a 32-value nibble format -> codes less their bias [n, nb*32], d, m [n, nb]."""
     n, nb, _ = w.shape
-    qs_at = {oracle.Q4_0: 2, oracle.Q4_1: 4, oracle.Q5_0: 6, oracle.Q5_1: 8}[dtype]
+    qs_at = {oracle.Q4_0: 2, oracle.Q4_1: 4, oracle.Q5_0: 6, oracle.Q5_1: 8, oracle.IQ4_NL: 2, oracle.MXFP4: 1}[dtype]
     qs = w[:, :, qs_at:qs_at + 16].astype(np.int64)
     codes = np.concatenate([qs & 0xF, qs >> 4], axis=2)                       # value v at [..., v]
     if dtype in (oracle.Q5_0, oracle.Q5_1):
         qh = w[:, :, qs_at - 4:qs_at].copy().view(np.uint32).reshape(n, nb, 1).astype(np.int64)
         codes = codes | (((qh >> np.arange(32)[None, None, :]) & 1) << 4)
     codes = codes - {oracle.Q4_0: 8, oracle.Q5_0: 16}.get(dtype, 0)
-    d = w[:, :, 0:2].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+    if dtype in LEVELS:
+        codes = LEVELS[dtype][codes]
+    if dtype == oracle.MXFP4:   # E8M0 scale, halved: 2^(e - 128) (the generator keeps e well above 1)
+        d = np.exp2(w[:, :, 0].astype(np.float64) - 128.0)
+    else:
+        d = w[:, :, 0:2].copy().view(np.float16).reshape(n, nb).astype(np.float64)
     m = (w[:, :, 2:4].copy().view(np.float16).reshape(n, nb).astype(np.float64)
          if dtype in (oracle.Q4_1, oracle.Q5_1) else np.zeros((n, nb)))
     return codes.reshape(n, nb * 32), d, m
@@ -110,7 +118,8 @@ def np_dequant(dtype, w):
 
 def test_numpy_decoders_agree_with_ggml(ggml_vectors):
     for name, dtype in (("q4_K", oracle.Q4_K), ("q5_K", oracle.Q5_K), ("q6_K", oracle.Q6_K), ("q8_0", oracle.Q8_0),
-                        ("q4_0", oracle.Q4_0), ("q4_1", oracle.Q4_1), ("q5_0", oracle.Q5_0), ("q5_1", oracle.Q5_1)):
+                        ("q4_0", oracle.Q4_0), ("q4_1", oracle.Q4_1), ("q5_0", oracle.Q5_0), ("q5_1", oracle.Q5_1),
+                        ("mxfp4", oracle.MXFP4)):
         rec = ggml_vectors[name]
         w = rec["quant"].reshape(1, -1, rec["block_bytes"])
         got = np_dequant(dtype, w).reshape(-1)
@@ -212,7 +221,7 @@ def test_served_path_integer_core_with_q8k_codes(name):
     w = synth.weight(dtype, n, k, seed=15, stream=4)
     x = synth.activation(2, k, seed=15)
     slack = 0.0
-    if dtype in (oracle.Q8_0, oracle.Q4_0, oracle.Q5_0):
+    if dtype in (oracle.Q8_0, oracle.Q4_0, oracle.Q5_0, oracle.IQ4_NL, oracle.MXFP4):
         xa = oracle.dequantize(oracle.Q8_0, oracle.quantize_q8_0(x)).reshape(2, k)
     elif dtype in (oracle.Q4_1, oracle.Q5_1):
         # these pair with Q8_1 and take the block's sum from its f16 `s` field: the minimum's term
