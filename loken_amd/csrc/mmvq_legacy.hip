@@ -1,4 +1,5 @@
-// Mat-vec for the 32-value nibble formats Q4_0, Q4_1, Q5_0, Q5_1 against Q8_1 activation rows.
+// Mat-vec for the 32-value nibble formats Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, MXFP4 against Q8_1
+// activation rows.
 //
 // Formats as loken states them (src/tensor/quant_cpu/format/q4_0.rs, q4_1.rs, q5_0.rs, q5_1.rs): byte
 // j of `qs` holds value j in its low nibble and value j + 16 in its high one; the five-bit formats
@@ -9,7 +10,12 @@
 // activation codes taken as the integer it is (as every kernel of this library takes it):
 //     d * d8 * (sum code * a - bias * sum a)            Q4_0 (bias 8), Q5_0 (bias 16)
 //     d * d8 * (sum code * a) + m * (d8 * sum a)        Q4_1, Q5_1
-// Replaces kernels `mmvq_gguf_{q4_0,q4_1,q5_0,q5_1}_{f32,f16,bf16}_plain_cuda{1..8}`
+// IQ4_NL {d, qs} and MXFP4 {e, qs} pack their nibbles the same way, but a code names a level of a
+// 16-entry int8 table (src/tensor/quant_cpu/format/iq4_nl.rs:11-13; KVALUES_MXFP4 and the E8M0 scale
+// 0.5 * 2^(e - 127), src/tensor/quant_cpu/blocks.rs:24-42): scale * d8 * (sum level * a). Four
+// levels at a time come out of the table with two byte permutes (entries 0..7, 8..15) and a select
+// on the code's top bit.
+// Replaces kernels `mmvq_gguf_{q4_0,q4_1,q5_0,q5_1,iq4_nl,mxfp4}_{f32,f16,bf16}_plain_cuda{1..8}`
 // (src/inference/cuda/mmvq_gguf.cu:338-363) behind lk_mmvq.
 //
 // Shape: a wave owns a weight row; its lanes walk the row's blocks 64 at a time (consecutive lanes
@@ -25,11 +31,40 @@ namespace {
 
 constexpr int LWG = 256, LWAVES = 4;
 
+// TABLE: 0 = the code is the value (less BIAS); 1 = IQ4_NL's levels; 2 = MXFP4's levels, E8M0 scale.
 template <int ID> struct Legacy;
-template <> struct Legacy<2> { static constexpr int BYTES = 18, M_AT = -1, QH_AT = -1, QS_AT = 2, BIAS = 8; };
-template <> struct Legacy<3> { static constexpr int BYTES = 20, M_AT = 2, QH_AT = -1, QS_AT = 4, BIAS = 0; };
-template <> struct Legacy<6> { static constexpr int BYTES = 22, M_AT = -1, QH_AT = 2, QS_AT = 6, BIAS = 16; };
-template <> struct Legacy<7> { static constexpr int BYTES = 24, M_AT = 2, QH_AT = 4, QS_AT = 8, BIAS = 0; };
+template <> struct Legacy<2> { static constexpr int BYTES = 18, M_AT = -1, QH_AT = -1, QS_AT = 2, BIAS = 8, TABLE = 0; };
+template <> struct Legacy<3> { static constexpr int BYTES = 20, M_AT = 2, QH_AT = -1, QS_AT = 4, BIAS = 0, TABLE = 0; };
+template <> struct Legacy<6> { static constexpr int BYTES = 22, M_AT = -1, QH_AT = 2, QS_AT = 6, BIAS = 16, TABLE = 0; };
+template <> struct Legacy<7> { static constexpr int BYTES = 24, M_AT = 2, QH_AT = 4, QS_AT = 8, BIAS = 0, TABLE = 0; };
+template <> struct Legacy<20> { static constexpr int BYTES = 18, M_AT = -1, QH_AT = -1, QS_AT = 2, BIAS = 0, TABLE = 1; };
+template <> struct Legacy<39> { static constexpr int BYTES = 17, M_AT = -1, QH_AT = -1, QS_AT = 1, BIAS = 0, TABLE = 2; };
+
+typedef uint4 __attribute__((aligned(1))) uint4_a1;
+
+// The levels of four codes (one per byte of `codes`, 0..15) from a 16-entry int8 table held as
+// four dwords: a byte permute picks among eight entries, so two of them and the code's bit 3.
+template <int TABLE>
+static __device__ __forceinline__ uint32_t levels_of(uint32_t codes) {
+    // IQ4_NL: -127 -104 -83 -65 | -49 -35 -22 -10 | 1 13 25 38 | 53 69 89 113
+    // MXFP4:  0 1 2 3 | 4 6 8 12 | 0 -1 -2 -3 | -4 -6 -8 -12
+    constexpr uint32_t T0 = TABLE == 1 ? 0xBFAD9881u : 0x03020100u, T1 = TABLE == 1 ? 0xF6EADDCFu : 0x0C080604u;
+    constexpr uint32_t T2 = TABLE == 1 ? 0x26190D01u : 0xFDFEFF00u, T3 = TABLE == 1 ? 0x71594535u : 0xF4F8FAFCu;
+    const uint32_t idx = codes & 0x07070707u;
+    const uint32_t low = __builtin_amdgcn_perm(T1, T0, idx), high = __builtin_amdgcn_perm(T3, T2, idx);
+    const uint32_t top = ((codes >> 3) & 0x01010101u) * 0xFFu;   // 0xFF in the bytes whose code is 8..15
+    return (high & top) | (low & ~top);
+}
+
+// The block's scale: an f16, or MXFP4's E8M0 byte as 0.5 * 2^(e - 127) (denormal patterns below 2).
+template <class F>
+static __device__ __forceinline__ float block_scale(const uint8_t* __restrict__ bp) {
+    if (F::TABLE == 2) {
+        const uint32_t e = bp[0];
+        return __uint_as_float(e < 2 ? (0x00200000u << e) : ((e - 1) << 23));
+    }
+    return f16_bits_to_f32(*(const uint16_t*)bp);
+}
 
 // Four bits of `x` (bits 0..3) to bit 4 of four bytes: byte i receives bit i. The multiplier lays
 // the nibble down at shifts 0, 7, 14, 21, which puts bit i at position 8 i; the copies do not overlap.
@@ -40,9 +75,15 @@ static __device__ __forceinline__ uint32_t fifth_bits(uint32_t x) {
 // A block's unsigned codes: lo = values 0..15, hi = values 16..31, four per dword.
 template <class F>
 static __device__ __forceinline__ void block_codes(const uint8_t* __restrict__ bp, uint4& lo, uint4& hi) {
-    const uint4 q = *(const uint4_a2*)(bp + F::QS_AT);
+    uint4 q;
+    if (F::BYTES % 2) q = *(const uint4_a1*)(bp + F::QS_AT);   // 17-byte blocks start on any byte
+    else q = *(const uint4_a2*)(bp + F::QS_AT);
     lo = make_uint4(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu, q.z & 0x0F0F0F0Fu, q.w & 0x0F0F0F0Fu);
     hi = make_uint4((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu, (q.z >> 4) & 0x0F0F0F0Fu, (q.w >> 4) & 0x0F0F0F0Fu);
+    if (F::TABLE) {
+        lo = make_uint4(levels_of<F::TABLE>(lo.x), levels_of<F::TABLE>(lo.y), levels_of<F::TABLE>(lo.z), levels_of<F::TABLE>(lo.w));
+        hi = make_uint4(levels_of<F::TABLE>(hi.x), levels_of<F::TABLE>(hi.y), levels_of<F::TABLE>(hi.z), levels_of<F::TABLE>(hi.w));
+    }
     if (F::QH_AT >= 0) {
         const uint32_t qh = (uint32_t)*(const uint16_t*)(bp + F::QH_AT) | ((uint32_t)*(const uint16_t*)(bp + F::QH_AT + 2) << 16);
         lo.x |= fifth_bits(qh);       lo.y |= fifth_bits(qh >> 4);  lo.z |= fifth_bits(qh >> 8);  lo.w |= fifth_bits(qh >> 12);
@@ -75,7 +116,7 @@ __global__ __launch_bounds__(LWG) void mmvq_legacy_kernel(const uint8_t* __restr
             const uint8_t* bp = wrow + (size_t)b * F::BYTES;
             uint4 lo, hi;
             block_codes<F>(bp, lo, hi);
-            const float d = f16_bits_to_f32(*(const uint16_t*)bp);
+            const float d = block_scale<F>(bp);
             const float m = F::M_AT >= 0 ? f16_bits_to_f32(*(const uint16_t*)(bp + (F::M_AT >= 0 ? F::M_AT : 0))) : 0.f;
 #pragma unroll
             for (int c = 0; c < B; ++c) {
@@ -150,7 +191,8 @@ static int by_type(int dst_type, int batch, const void* vx, const void* vy, void
 }  // namespace
 
 bool lk_is_legacy_type(int wtype) {
-    return wtype == LK_TYPE_Q4_0 || wtype == LK_TYPE_Q4_1 || wtype == LK_TYPE_Q5_0 || wtype == LK_TYPE_Q5_1;
+    return wtype == LK_TYPE_Q4_0 || wtype == LK_TYPE_Q4_1 || wtype == LK_TYPE_Q5_0 || wtype == LK_TYPE_Q5_1 ||
+           wtype == LK_TYPE_IQ4_NL || wtype == LK_TYPE_MXFP4;
 }
 
 // lk_mmvq for the 32-value nibble formats (the caller has told them apart with lk_is_legacy_type).
@@ -159,13 +201,15 @@ int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, in
     if (nrows_x == 0) return LK_OK;
     if (!vx || !vy_q8_1 || !dst || ncols_x <= 0 || ncols_x % 32 != 0 || nrows_x < 0) return LK_ERR_ARG;
     if (batch < 1 || batch > 8 || stride_col_y < ncols_x / 32 || stride_col_dst < nrows_x) return LK_ERR_ARG;
-    if (((uintptr_t)vx & 1) != 0 || ((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
+    if ((wtype != LK_TYPE_MXFP4 && ((uintptr_t)vx & 1) != 0) || ((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
     const int nb = ncols_x / 32;
     switch (wtype) {
         case LK_TYPE_Q4_0: return by_type<2>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q4_1: return by_type<3>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q5_0: return by_type<6>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q5_1: return by_type<7>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_IQ4_NL: return by_type<20>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_MXFP4: return by_type<39>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         default: return LK_ERR_TYPE;
     }
 }
@@ -181,6 +225,8 @@ int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32
         case LK_TYPE_Q4_1: hipLaunchKernelGGL(subdots_legacy_kernel<3>, grid, dim3(64), 0, s, w, y, dots, nb); break;
         case LK_TYPE_Q5_0: hipLaunchKernelGGL(subdots_legacy_kernel<6>, grid, dim3(64), 0, s, w, y, dots, nb); break;
         case LK_TYPE_Q5_1: hipLaunchKernelGGL(subdots_legacy_kernel<7>, grid, dim3(64), 0, s, w, y, dots, nb); break;
+        case LK_TYPE_IQ4_NL: hipLaunchKernelGGL(subdots_legacy_kernel<20>, grid, dim3(64), 0, s, w, y, dots, nb); break;
+        case LK_TYPE_MXFP4: hipLaunchKernelGGL(subdots_legacy_kernel<39>, grid, dim3(64), 0, s, w, y, dots, nb); break;
         default: return LK_ERR_TYPE;
     }
     return lk_launch_status();

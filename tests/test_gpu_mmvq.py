@@ -17,7 +17,8 @@ pytestmark = pytest.mark.gpu
 
 DT = {"q4_k": lib.TYPE_Q4_K, "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0}
 # the 32-value nibble formats: served by lk_mmvq and the sub-dot probe only
-LEGACY = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1}
+LEGACY = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
+          "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4}
 RTOL, ATOL = 1e-3, 1e-4
 
 
@@ -123,7 +124,7 @@ def test_legacy_matvec_extremes_bias_and_half_outputs(name):
     n, k = 40, 256
     # every code at its maximum against every activation code at +-127
     w = synth.weight(wtype, n, k, seed=72, stream=3)
-    qs_at = {"q4_0": 2, "q4_1": 4, "q5_0": 6, "q5_1": 8}[name]
+    qs_at = {"q4_0": 2, "q4_1": 4, "q5_0": 6, "q5_1": 8, "iq4_nl": 2, "mxfp4": 1}[name]
     w[:, :, qs_at - (4 if name.startswith("q5") else 0):] = 0xFF
     x = np.where(np.arange(k) % 2 == 0, 127.0, -127.0).astype(np.float32).reshape(1, k) * np.float32(0.5)
     q = ops.quantize_q8_1_rows(dev(x))
