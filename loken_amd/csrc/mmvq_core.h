@@ -103,32 +103,6 @@ static __device__ __forceinline__ void q6k_dots_biased(const uint4& ql0, const u
     for (int g = 0; g < 4; ++g) dot[g] = dot16(c[g], a[g], dot[g]);
 }
 
-// Dword-aligned read of 16 bytes that start on any even address. A 2-byte-aligned dwordx4 load
-// runs at about three quarters of the rate of a dword-aligned one on this part, so the load is
-// made from the enclosing dwords and shifted into place. The fifth dword is the one that holds
-// the run's last two bytes (the run's own last dword when the address is already aligned), so
-// nothing outside dwords the run touches is read.
-struct Run16 {
-    uint4 w;
-    uint32_t e;
-};
-static __device__ __forceinline__ Run16 load_run16(const uint8_t* p) {
-    const uintptr_t a = (uintptr_t)p;
-    const uint8_t* b = (const uint8_t*)(a & ~(uintptr_t)3);
-    Run16 r;
-    r.w = *(const uint4_a4*)b;
-    r.e = *(const uint32_t*)(b + 12 + 2 * (a & 2));
-    return r;
-}
-static __device__ __forceinline__ uint4 run16_value(const Run16& r, uint32_t shift_bits) {
-    uint4 v;
-    v.x = __builtin_amdgcn_alignbit(r.w.y, r.w.x, shift_bits);
-    v.y = __builtin_amdgcn_alignbit(r.w.z, r.w.y, shift_bits);
-    v.z = __builtin_amdgcn_alignbit(r.w.w, r.w.z, shift_bits);
-    v.w = __builtin_amdgcn_alignbit(r.e, r.w.w, shift_bits);
-    return v;
-}
-
 // --------------------------------------------------------------------------------------------
 // Activation staging. Formats differ only in where a Q8_1 block's two 16-byte halves land.
 // LDS per activation row: `n_iter` passes x `PLANES` planes x 1024 bytes of codes, then the

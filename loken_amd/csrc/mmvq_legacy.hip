@@ -76,8 +76,17 @@ static __device__ __forceinline__ uint32_t fifth_bits(uint32_t x) {
 template <class F>
 static __device__ __forceinline__ void block_codes(const uint8_t* __restrict__ bp, uint4& lo, uint4& hi) {
     uint4 q;
-    if (F::BYTES % 2) q = *(const uint4_a1*)(bp + F::QS_AT);   // 17-byte blocks start on any byte
-    else q = *(const uint4_a2*)(bp + F::QS_AT);
+    if (F::BYTES % 2) {
+        q = *(const uint4_a1*)(bp + F::QS_AT);   // 17-byte blocks start on any byte
+    } else if (F::BYTES % 4) {
+        // blocks of 18 and 22 bytes put every other run of codes two bytes off a dword, where a
+        // 16-byte load runs at three quarters of its rate: read the enclosing dwords and shift
+        // (Q4_0 14336 x 4096: 12.8 -> 11.4 us)
+        const uint8_t* qs = bp + F::QS_AT;
+        q = run16_value(load_run16(qs), 8 * (uint32_t)((uintptr_t)qs & 3));
+    } else {
+        q = *(const uint4_a2*)(bp + F::QS_AT);   // 20- and 24-byte blocks keep the alignment of the blob
+    }
     lo = make_uint4(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu, q.z & 0x0F0F0F0Fu, q.w & 0x0F0F0F0Fu);
     hi = make_uint4((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu, (q.z >> 4) & 0x0F0F0F0Fu, (q.w >> 4) & 0x0F0F0F0Fu);
     if (F::TABLE) {

@@ -1,5 +1,7 @@
 """The other measured workloads of `bench.py` (`--workload ...`): one JSON line each.
 
+  gemv        one mat-vec of any served format (`--wtype`, `--rows-n`, `--cols-k`, `--batch`) over rotating
+              copies of the weight, as one graph
   gemv-4096   one Q4_K 4096x4096 mat-vec at one row, over rotating copies of the weight (more
               than twice the 256 MB last-level cache) and over one hot copy; the Q8_1 quantizer
               launch timed by itself and the two-launch call timed as a whole
@@ -141,6 +143,44 @@ def line(args, metric_value, unit, ms_per_step, dtype, config, roofline, extra=N
 def check(rc, what):
     if rc:
         raise lib.LokenError(what, rc)
+
+
+# ---------------------------------------------------------------------------- gemv (any format)
+WTYPES = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
+          "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "q8_0": lib.TYPE_Q8_0, "q4_k": lib.TYPE_Q4_K,
+          "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K}
+
+
+def gemv(args, dev):
+    """One `--wtype` mat-vec of `--rows-n` x `--cols-k` at `--batch` rows through lk_mmvq, over rotating
+    copies of the weight (together past twice the last-level cache), replayed as one HIP graph."""
+    L = lib.load()
+    wtype, n, k, b = WTYPES[args.wtype], args.rows_n, args.cols_k, args.batch
+    nbytes = synth.weight_bytes(wtype, n, k)
+    n_copies = max(2, min(64, int(600e6 // nbytes) + 1))
+    seed_rows = min(n, 256)   # a few generated rows repeated: the kernels do not care what the blocks hold
+    base = torch.from_numpy(synth.weight(wtype, seed_rows, k, seed=0)).to(dev).reshape(seed_rows, -1)
+    base = base.repeat((n + seed_rows - 1) // seed_rows, 1)[:n].contiguous().reshape(-1)
+    copies = [base.clone() for _ in range(n_copies)]
+    q = ops.quantize_q8_1_rows(torch.from_numpy(synth.activation(b, k, seed=0)).to(dev))
+    out = torch.empty((b, n), device=dev)
+
+    def all_copies():
+        s2 = torch.cuda.current_stream().cuda_stream
+        for w in copies:
+            check(L.lk_mmvq(wtype, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, b, q.shape[1], n,
+                            None, 0, s2), "lk_mmvq")
+
+    us = time_replays(capture(all_copies), max(10, args.launches // n_copies)) / n_copies
+    med = float(np.median(us))
+    value = nbytes / med / 1e3
+    roofline = {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None, "kernel": f"lk_mmvq, {args.wtype}",
+                "avg_launch_us": round(float(us.mean()), 3), "algorithmic_bytes_per_launch": nbytes}
+    return line(args, value, "GB/s", med / 1e3, "int8",
+                {"workload": f"{args.wtype} mat-vec {n} x {k}, {b} activation row(s), graph of {n_copies} launches over "
+                             f"{n_copies} rotating copies ({n_copies * nbytes / 1e6:.0f} MB)", "hip_graph": True}, roofline,
+                {"per_launch": spread(us)})
 
 
 # ---------------------------------------------------------------------------- gemv-4096
@@ -458,4 +498,4 @@ def run(args) -> int:
     lib.load()  # raises if the HIP library is missing: there is no other path
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    return {"gemv-4096": gemv_4096, "mmq": mmq, "moe": moe_block, "decode-1p7b": decode_1p7b}[args.workload](args, dev)
+    return {"gemv": gemv, "gemv-4096": gemv_4096, "mmq": mmq, "moe": moe_block, "decode-1p7b": decode_1p7b}[args.workload](args, dev)
