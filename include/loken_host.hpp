@@ -196,7 +196,7 @@ int lkh_gguf_facts(void* g, const char** architecture, int64_t* file_type, int64
                    int64_t* split_parts);
 void* lkh_gguf_upload(void* g, int index, int device, void* stream, uint64_t* blob_bytes);
 void lkh_gguf_free_blob(void* blob);
-/* Tensor `name` (2-D, Q4_K / Q5_K / Q6_K / Q8_0) uploaded to `device` and wrapped as a QKernelMatMul
+/* Tensor `name` (2-D; Q4_K / Q5_K / Q6_K / Q8_0, or a 32-value nibble format, which runs as mat-vec launches at any row count) uploaded to `device` and wrapped as a QKernelMatMul
  * handle (QKernelMatMul::from_qtensor_on, kernel_matmul.rs:213-275); `*blob` receives the device
  * allocation, which the caller frees after the handle. */
 void* lkh_gguf_linear(void* g, const char* name, int device, void* stream, void** blob, char* err, int err_len);

@@ -97,6 +97,12 @@ void mark_used(Slot& slot, hipStream_t stream) {
     }
 }
 
+// The 32-value nibble formats: served by the plain mat-vec only, whatever the row count.
+bool matvec_only(int dtype) {
+    return dtype == LK_TYPE_Q4_0 || dtype == LK_TYPE_Q4_1 || dtype == LK_TYPE_Q5_0 || dtype == LK_TYPE_Q5_1 ||
+           dtype == LK_TYPE_IQ4_NL || dtype == LK_TYPE_MXFP4;
+}
+
 bool tiled_serves(int dtype, int k) {
     return (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K || dtype == LK_TYPE_Q6_K || dtype == LK_TYPE_Q8_0) && k % 256 == 0;
 }
@@ -116,11 +122,12 @@ QKernelMatMul::QKernelMatMul(int dtype, int n, int k, const void* blob, int devi
 int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void* stream_ptr, bool decode_order) {
     last_path_ = Path::None;
     hipStream_t stream = (hipStream_t)stream_ptr;
-    if (dtype_ != LK_TYPE_Q4_K && dtype_ != LK_TYPE_Q5_K && dtype_ != LK_TYPE_Q6_K && dtype_ != LK_TYPE_Q8_0) return LK_ERR_TYPE;
+    const bool plain = matvec_only(dtype_);
+    if (!plain && dtype_ != LK_TYPE_Q4_K && dtype_ != LK_TYPE_Q5_K && dtype_ != LK_TYPE_Q6_K && dtype_ != LK_TYPE_Q8_0) return LK_ERR_TYPE;
     if (x_type != LK_TYPE_F32 && x_type != LK_TYPE_F16 && x_type != LK_TYPE_BF16) return LK_ERR_TYPE;
     if (rows == 0) return LK_OK;
     if (!x || !out || !blob_ || rows < 0 || n_ <= 0 || k_ <= 0) return LK_ERR_ARG;
-    const int block_len = dtype_ == LK_TYPE_Q8_0 ? 32 : 256;
+    const int block_len = dtype_ == LK_TYPE_Q8_0 || plain ? 32 : 256;
     if (k_ % block_len != 0) return LK_ERR_ARG;
     int current = -1;
     if (hipGetDevice(&current) != hipSuccess || current != device_) {
@@ -131,8 +138,8 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     Slot& slot = slot_of(device_);
 
     // --- mat-vec family: up to matvec_rows, or any count when every row must sum like a one-row call
-    if (rows <= mv_max || decode_order) {
-        if (x_type == LK_TYPE_F32 && rows <= 2 && k_ <= 8192 && ((uintptr_t)x & 15) == 0 && k_ % 4 == 0) {
+    if (rows <= mv_max || decode_order || plain) {
+        if (!plain && x_type == LK_TYPE_F32 && rows <= 2 && k_ <= 8192 && ((uintptr_t)x & 15) == 0 && k_ % 4 == 0) {
             const void* vx[1] = {blob_};
             void* dst[1] = {out};
             const int nn[1] = {n_};

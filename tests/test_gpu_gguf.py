@@ -18,7 +18,8 @@ HIP_D2H = 2
 
 def model_file(tmp_path):
     shapes = {"blk.0.attn_q.weight": (lib.TYPE_Q4_K, 192, 1024), "blk.0.ffn_down.weight": (lib.TYPE_Q6_K, 160, 768),
-              "output.weight": (lib.TYPE_Q8_0, 320, 512), "blk.0.attn_v.weight": (lib.TYPE_Q5_K, 96, 1024)}
+              "output.weight": (lib.TYPE_Q8_0, 320, 512), "blk.0.attn_v.weight": (lib.TYPE_Q5_K, 96, 1024),
+              "blk.0.attn_k.weight": (lib.TYPE_Q4_0, 64, 1024), "blk.0.ffn_up.weight": (lib.TYPE_MXFP4, 128, 512)}
     blocks = {name: synth.weight(dt, n, k, seed=90, stream=i) for i, (name, (dt, n, k)) in enumerate(shapes.items())}
     norm = np.arange(1024, dtype=np.float32)
     tensors = [(name, (n, k), dt, blocks[name].tobytes()) for name, (dt, n, k) in shapes.items()]
