@@ -81,7 +81,7 @@ int lko_block_len(int dtype) {
     switch (dtype) {
         case LKO_Q8_0: case LKO_Q8_1: case LKO_Q4_0: case LKO_Q4_1: case LKO_Q5_0: case LKO_Q5_1:
         case LKO_IQ4_NL: case LKO_MXFP4: return 32;
-        case LKO_Q4_K: case LKO_Q5_K: case LKO_Q6_K: case LKO_Q8_K: return 256;
+        case LKO_Q2_K: case LKO_Q3_K: case LKO_Q4_K: case LKO_Q5_K: case LKO_Q6_K: case LKO_Q8_K: return 256;
         default: return 0;
     }
 }
@@ -96,6 +96,8 @@ int lko_block_bytes(int dtype) {
         case LKO_IQ4_NL: return 18;
         case LKO_MXFP4: return 17;
         case LKO_Q8_1: return LKO_Q81_BYTES;
+        case LKO_Q2_K: return 84;
+        case LKO_Q3_K: return 110;
         case LKO_Q4_K: return LKO_Q4K_BYTES;
         case LKO_Q5_K: return LKO_Q5K_BYTES;
         case LKO_Q6_K: return LKO_Q6K_BYTES;
@@ -177,6 +179,7 @@ static inline int q5k_code(const uint8_t* blk, int s, int l) {
 }
 
 static int legacy_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out);
+static int lowbit_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out);
 
 int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out) {
     switch (dtype) {
@@ -249,6 +252,8 @@ int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out
             for (int l = 0; l < 256; ++l) out[b * 256 + l] = (float)(int8_t)blk[4 + l] * d;
         }
         return 0;
+    case LKO_Q2_K: case LKO_Q3_K:
+        return lowbit_dequantize(dtype, blocks, n_blocks, out);
     default:
         return legacy_dequantize(dtype, blocks, n_blocks, out);
     }
@@ -679,10 +684,142 @@ static float oa_dot_mxfp4(const uint8_t* w, const uint8_t* y, size_t nb) { retur
 static float ob_dot_iq4nl(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_IQ4_NL, w, y, nb); }
 static float ob_dot_mxfp4(const uint8_t* w, const uint8_t* y, size_t nb) { return ob_dot_legacy(LKO_MXFP4, w, y, nb); }
 
+
+/* ------------------------------------------------------------------------------------------
+ * Q2_K {scales[16], qs[64], d, dmin} = 84 bytes (q2_k.rs:15-20) and Q3_K {hmask[32], qs[64],
+ * scales[12], d} = 110 bytes (q3_k.rs:10-15): sixteen sub-blocks of sixteen two-bit codes.
+ * Sub-block s reads byte 32 * (s / 8) + 16 * (s % 2) + l at shift 2 * ((s % 8) / 2)
+ * (q2_k.rs:30-33, q3_k.rs:132-140); positions run 16 s + l, so the 32 values of Q8_1 block j are
+ * sub-blocks 2 j and 2 j + 1. Q2_K: d * (sc & 15) * q - dmin * (sc >> 4). Q3_K: d * scale * (q + third),
+ * third = -4 where bit j of hmask[16 * (s % 2) + l] is clear; scales six bits less 32 (q3_k.rs:27-37).
+ * ---------------------------------------------------------------------------------------- */
+static inline int q23k_low(const uint8_t* qs, int s, int l) {
+    return (qs[32 * (s / 8) + 16 * (s % 2) + l] >> (2 * ((s % 8) / 2))) & 3;
+}
+static inline int q3k_value(const uint8_t* blk, int s, int l) {
+    const int bit = 4 * (s / 8) + (s % 8) / 2;
+    return q23k_low(blk + 32, s, l) + (((blk[16 * (s % 2) + l] >> bit) & 1) ? 0 : -4);
+}
+static void q3k_scales(const uint8_t* packed, int8_t out[16]) {
+    for (int i = 0; i < 16; ++i) {
+        const int group = i / 4, j = i % 4;
+        const uint8_t byte = packed[j + 4 * (group % 2)];
+        const int low = group < 2 ? (byte & 0x0F) : (byte >> 4);
+        const int high = (packed[8 + j] >> (2 * group)) & 0x03;
+        out[i] = (int8_t)((low | (high << 4)) - 32);
+    }
+}
+/* Sub-block s against its sixteen activation codes: the integers the CPU dots form
+ * (q2_k.rs:98-102; q3_k.rs block_sum). */
+static inline int32_t q2k_sub_dot(const uint8_t* blk, int s, const int8_t* acts) {
+    int32_t dot = 0;
+    for (int l = 0; l < 16; ++l) dot += q23k_low(blk + 16, s, l) * (int32_t)acts[l];
+    return dot;
+}
+static inline int32_t q3k_sub_dot(const uint8_t* blk, int s, const int8_t* acts) {
+    int32_t dot = 0;
+    for (int l = 0; l < 16; ++l) dot += q3k_value(blk, s, l) * (int32_t)acts[l];
+    return dot;
+}
+
+static int lowbit_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out) {
+    for (size_t b = 0; b < n_blocks; ++b) {
+        float* y = out + b * 256;
+        if (dtype == LKO_Q2_K) {                                    /* q2_k.rs:51-64 */
+            const uint8_t* blk = blocks + b * 84;
+            const float d = lko_f16_to_f32(rd_u16(blk + 80)), dmin = lko_f16_to_f32(rd_u16(blk + 82));
+            for (int s = 0; s < 16; ++s) {
+                const float scale = d * (float)(blk[s] & 0x0F), offset = dmin * (float)(blk[s] >> 4);
+                for (int l = 0; l < 16; ++l) y[16 * s + l] = scale * (float)q23k_low(blk + 16, s, l) - offset;
+            }
+        } else {                                                    /* q3_k.rs:127-146 */
+            const uint8_t* blk = blocks + b * 110;
+            const float d = lko_f16_to_f32(rd_u16(blk + 108));
+            int8_t sc[16];
+            q3k_scales(blk + 96, sc);
+            for (int s = 0; s < 16; ++s) {
+                const float scale = d * (float)sc[s];
+                for (int l = 0; l < 16; ++l) y[16 * s + l] = scale * (float)q3k_value(blk, s, l);
+            }
+        }
+    }
+    return 0;
+}
+
+/* Served CPU path against Q8_K (q2_k.rs:88-109, 124-126; q3_k.rs:161-167 with its combine
+ * y.d * (x.d * sum)): integer sums per block, shares added in block order from -0. */
+static float oa_dot_q2k(const uint8_t* w, const uint8_t* y, size_t nb) {
+    float total = -0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * 84;
+        const uint8_t* yb = y + b * LKO_Q8K_BYTES;
+        const int8_t* yq = (const int8_t*)(yb + 4);
+        int32_t scaled = 0, offset = 0;
+        for (int s = 0; s < 16; ++s) {
+            scaled += (int32_t)(x[s] & 0x0F) * q2k_sub_dot(x, s, yq + 16 * s);
+            offset += (int32_t)(x[s] >> 4) * (int32_t)(int16_t)rd_u16(yb + 260 + 2 * s);
+        }
+        total += rd_f32(yb) * (lko_f16_to_f32(rd_u16(x + 80)) * (float)scaled - lko_f16_to_f32(rd_u16(x + 82)) * (float)offset);
+    }
+    return total;
+}
+static float oa_dot_q3k(const uint8_t* w, const uint8_t* y, size_t nb) {
+    float total = -0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * 110;
+        const uint8_t* yb = y + b * LKO_Q8K_BYTES;
+        const int8_t* yq = (const int8_t*)(yb + 4);
+        int8_t sc[16];
+        q3k_scales(x + 96, sc);
+        int32_t sum = 0;
+        for (int s = 0; s < 16; ++s) sum += (int32_t)sc[s] * q3k_sub_dot(x, s, yq + 16 * s);
+        total += rd_f32(yb) * (lko_f16_to_f32(rd_u16(x + 108)) * (float)sum);
+    }
+    return total;
+}
+/* Same codes on the Q8_1 side (cuda/moe/gguf.cuh:524-546 for Q2_K: d * sum d8 * (dot * scale) -
+ * dmin * sum d8 * (sum of codes * minimum); Q3_K likewise without a minimum, vec_dot_plane_q3_K). */
+static float ob_dot_q2k(const uint8_t* w, const uint8_t* y, size_t nb) {
+    float total = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * 84;
+        float scaled = 0.0f, offset = 0.0f;
+        for (int s = 0; s < 16; ++s) {
+            const uint8_t* yb = y + (b * 8 + s / 2) * LKO_Q81_BYTES;
+            const int8_t* yq = (const int8_t*)(yb + 4) + 16 * (s % 2);
+            const float d8 = lko_f16_to_f32(rd_u16(yb));
+            int32_t sum = 0;
+            for (int l = 0; l < 16; ++l) sum += yq[l];
+            scaled += d8 * (float)(q2k_sub_dot(x, s, yq) * (int32_t)(x[s] & 0x0F));
+            offset += d8 * (float)(sum * (int32_t)(x[s] >> 4));
+        }
+        total += lko_f16_to_f32(rd_u16(x + 80)) * scaled - lko_f16_to_f32(rd_u16(x + 82)) * offset;
+    }
+    return total;
+}
+static float ob_dot_q3k(const uint8_t* w, const uint8_t* y, size_t nb) {
+    float total = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * 110;
+        int8_t sc[16];
+        q3k_scales(x + 96, sc);
+        float scaled = 0.0f;
+        for (int s = 0; s < 16; ++s) {
+            const uint8_t* yb = y + (b * 8 + s / 2) * LKO_Q81_BYTES;
+            const int8_t* yq = (const int8_t*)(yb + 4) + 16 * (s % 2);
+            scaled += lko_f16_to_f32(rd_u16(yb)) * (float)(q3k_sub_dot(x, s, yq) * (int32_t)sc[s]);
+        }
+        total += lko_f16_to_f32(rd_u16(x + 108)) * scaled;
+    }
+    return total;
+}
+
 typedef float (*row_dot_fn)(const uint8_t* w, const uint8_t* y, size_t nb);
 
 static row_dot_fn oa_dot_of(int dtype) {
     switch (dtype) {
+        case LKO_Q2_K: return oa_dot_q2k;
+        case LKO_Q3_K: return oa_dot_q3k;
         case LKO_Q4_K: return oa_dot_q4k;
         case LKO_Q5_K: return oa_dot_q5k;
         case LKO_Q6_K: return oa_dot_q6k;
@@ -698,6 +835,8 @@ static row_dot_fn oa_dot_of(int dtype) {
 }
 static row_dot_fn ob_dot_of(int dtype) {
     switch (dtype) {
+        case LKO_Q2_K: return ob_dot_q2k;
+        case LKO_Q3_K: return ob_dot_q3k;
         case LKO_Q4_K: return ob_dot_q4k;
         case LKO_Q5_K: return ob_dot_q5k;
         case LKO_Q6_K: return ob_dot_q6k;
@@ -769,7 +908,7 @@ int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t*
     const size_t blk = (size_t)lko_block_len(dtype);
     legacy_layout ll;
     const int legacy = legacy_layout_of(dtype, &ll);
-    if (blk == 0 || (!legacy && dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
+    if (blk == 0 || (!legacy && dtype != LKO_Q2_K && dtype != LKO_Q3_K && dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
     if (k % blk != 0) return -1;
     const size_t nb = k / blk;
     const size_t wrow = nb * (size_t)lko_block_bytes(dtype);
@@ -788,6 +927,13 @@ int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t*
                 for (int s = 0; s < 8; ++s)
                     dots[c * (k / 32) + b * 8 + s] = q4k_sub_dot(
                         w + b * LKO_Q4K_BYTES, s, (const int8_t*)(act + (b * 8 + s) * LKO_Q81_BYTES + 4));
+        } else if (dtype == LKO_Q2_K || dtype == LKO_Q3_K) {
+            for (size_t b = 0; b < nb; ++b)
+                for (int s = 0; s < 16; ++s) {
+                    const int8_t* a = (const int8_t*)(act + (b * 8 + s / 2) * LKO_Q81_BYTES + 4) + 16 * (s % 2);
+                    dots[c * (k / 16) + b * 16 + s] = dtype == LKO_Q2_K ? q2k_sub_dot(w + b * 84, s, a)
+                                                                        : q3k_sub_dot(w + b * 110, s, a);
+                }
         } else if (dtype == LKO_Q5_K) {
             for (size_t b = 0; b < nb; ++b)
                 for (int s = 0; s < 8; ++s)
@@ -885,6 +1031,22 @@ static int dequant_row_f64(int dtype, const uint8_t* w, size_t nb, double* out) 
             const uint8_t* x = w + b * LKO_Q80_BYTES;
             const double d = lko_f16_to_f32(rd_u16(x));
             for (int l = 0; l < 32; ++l) out[b * 32 + l] = d * (double)(int8_t)x[2 + l];
+        }
+        return 0;
+    }
+    if (dtype == LKO_Q2_K || dtype == LKO_Q3_K) {
+        for (size_t b = 0; b < nb; ++b) {
+            const uint8_t* x = w + b * (size_t)(dtype == LKO_Q2_K ? 84 : 110);
+            int8_t sc3[16];
+            if (dtype == LKO_Q3_K) q3k_scales(x + 96, sc3);
+            for (int s = 0; s < 16; ++s)
+                for (int l = 0; l < 16; ++l) {
+                    if (dtype == LKO_Q2_K)
+                        out[b * 256 + 16 * s + l] = (double)lko_f16_to_f32(rd_u16(x + 80)) * (x[s] & 0x0F) * q23k_low(x + 16, s, l) -
+                                                    (double)lko_f16_to_f32(rd_u16(x + 82)) * (x[s] >> 4);
+                    else
+                        out[b * 256 + 16 * s + l] = (double)lko_f16_to_f32(rd_u16(x + 108)) * sc3[s] * q3k_value(x, s, l);
+                }
         }
         return 0;
     }

@@ -6,7 +6,7 @@ Run once in the authoring container (the reference is not present on the GPU box
 
 Only data records are copied, no source text:
   * scripts/oracle/vectors.txt -> ggml_vectors.txt: the N / INPUT records and the
-    TYPE / QUANT / DEQUANT records of q4_0, q4_1, q5_0, q5_1, q8_0, q4_K, q5_K, q6_K, q8_K, mxfp4 (ggml's own scalar quantize and
+    TYPE / QUANT / DEQUANT records of q4_0, q4_1, q5_0, q5_1, q8_0, q2_K, q3_K, q4_K, q5_K, q6_K, q8_K, mxfp4 (ggml's own scalar quantize and
     dequantize outputs on a 1024-value input; floats are 8-hex-digit bit patterns).
   * tests/vectors/ggml_encode.json -> ggml_encode_subset.json: rows, cols, read, x and the
     `blocks` / `expected` hex strings of q4_0, q4_1, q5_0, q5_1, q4_k, q5_k, q6_k, q8_0, iq4_nl, mxfp4 (ggml-written blocks of an 8x512
@@ -16,7 +16,7 @@ import json
 import sys
 from pathlib import Path
 
-KEEP_TYPES = {"q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q4_K", "q5_K", "q6_K", "q8_K", "mxfp4"}
+KEEP_TYPES = {"q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_K", "q3_K", "q4_K", "q5_K", "q6_K", "q8_K", "mxfp4"}
 
 
 def main(ref: str) -> None:
@@ -43,7 +43,7 @@ def main(ref: str) -> None:
     sub = {k: j[k] for k in ("rows", "cols", "read", "x")}
     sub["formats"] = {
         f: {"blocks": j["formats"][f]["blocks"], "expected": j["formats"][f]["expected"]}
-        for f in ("q4_0", "q4_1", "q5_0", "q5_1", "q4_k", "q5_k", "q6_k", "q8_0", "iq4_nl", "mxfp4")
+        for f in ("q4_0", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k", "q8_0", "iq4_nl", "mxfp4")
     }
     (here / "ggml_encode_subset.json").write_text(json.dumps(sub))
 

@@ -18,8 +18,9 @@ LEGACY = {"q4_0": oracle.Q4_0, "q4_1": oracle.Q4_1, "q5_0": oracle.Q5_0, "q5_1":
           "mxfp4": oracle.MXFP4}
 LEVELS = {oracle.IQ4_NL: np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64),
           oracle.MXFP4: np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], np.int64)}
-DT = {"q4_k": oracle.Q4_K, "q5_k": oracle.Q5_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0, **LEGACY}
-FAST = sorted(set(DT) - {"q5_k"} - set(LEGACY))   # formats the timed AVX2 baseline serves
+LOWBIT = {"q2_k": oracle.Q2_K, "q3_k": oracle.Q3_K}
+DT = {"q4_k": oracle.Q4_K, "q5_k": oracle.Q5_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0, **LEGACY, **LOWBIT}
+FAST = sorted(set(DT) - {"q5_k"} - set(LEGACY) - set(LOWBIT))   # formats the timed AVX2 baseline serves
 
 
 # ---- independent numpy decoders: integer codes and float scales per value ----
@@ -92,6 +93,38 @@ def np_codes_legacy(dtype, w):
     return codes.reshape(n, nb * 32), d, m
 
 
+def np_codes_lowbit(dtype, w):
+    """Q2_K [n, nb, 84] / Q3_K [n, nb, 110] -> values [n, nb*256], scales, mins [n, nb*16], d, dmin [n, nb]."""
+    n, nb, _ = w.shape
+    q2 = dtype == oracle.Q2_K
+    qs = w[:, :, 16:80] if q2 else w[:, :, 32:96]
+    qs = qs.reshape(n, nb, 2, 2, 16).astype(np.int64)                          # [half of block][byte half][l]
+    vals = np.empty((n, nb, 16, 16), np.int64)
+    for sb in range(16):
+        half, t = sb // 8, sb % 8
+        vals[:, :, sb, :] = (qs[:, :, half, t % 2, :] >> (2 * (t // 2))) & 3
+        if not q2:
+            hm = w[:, :, 16 * (t % 2):16 * (t % 2) + 16].astype(np.int64)
+            vals[:, :, sb, :] -= 4 * (1 - ((hm >> (4 * half + t // 2)) & 1))
+    if q2:
+        sc = (w[:, :, 0:16] & 0xF).astype(np.int64)
+        mn = (w[:, :, 0:16] >> 4).astype(np.int64)
+        d = w[:, :, 80:82].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+        dmin = w[:, :, 82:84].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+    else:
+        p = w[:, :, 96:108].astype(np.int64)
+        sc = np.empty((n, nb, 16), np.int64)
+        for i in range(16):
+            group, j = i // 4, i % 4
+            byte = p[:, :, j + 4 * (group % 2)]
+            low = (byte & 0xF) if group < 2 else (byte >> 4)
+            sc[:, :, i] = (low | (((p[:, :, 8 + j] >> (2 * group)) & 3) << 4)) - 32
+        mn = np.zeros((n, nb, 16), np.int64)
+        d = w[:, :, 108:110].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+        dmin = np.zeros((n, nb))
+    return vals.reshape(n, nb * 256), sc.reshape(n, nb * 16), mn.reshape(n, nb * 16), d, dmin
+
+
 def np_q81(act_bytes):
     b = act_bytes.reshape(-1, 36)
     d = b[:, 0:2].copy().view(np.float16).reshape(-1).astype(np.float64)
@@ -112,6 +145,10 @@ def np_dequant(dtype, w):
     if dtype in LEGACY.values():
         codes, d, m = np_codes_legacy(dtype, w)
         return np.repeat(d, 32, axis=1) * codes + np.repeat(m, 32, axis=1)
+    if dtype in LOWBIT.values():
+        vals, sc, mn, d, dmin = np_codes_lowbit(dtype, w)
+        return (np.repeat(sc * np.repeat(d, 16, axis=1), 16, axis=1) * vals
+                - np.repeat(mn * np.repeat(dmin, 16, axis=1), 16, axis=1))
     codes, d = np_codes_q80(w)
     return np.repeat(d, 32, axis=1) * codes
 
@@ -119,7 +156,7 @@ def np_dequant(dtype, w):
 def test_numpy_decoders_agree_with_ggml(ggml_vectors):
     for name, dtype in (("q4_K", oracle.Q4_K), ("q5_K", oracle.Q5_K), ("q6_K", oracle.Q6_K), ("q8_0", oracle.Q8_0),
                         ("q4_0", oracle.Q4_0), ("q4_1", oracle.Q4_1), ("q5_0", oracle.Q5_0), ("q5_1", oracle.Q5_1),
-                        ("mxfp4", oracle.MXFP4)):
+                        ("mxfp4", oracle.MXFP4), ("q2_K", oracle.Q2_K), ("q3_K", oracle.Q3_K)):
         rec = ggml_vectors[name]
         w = rec["quant"].reshape(1, -1, rec["block_bytes"])
         got = np_dequant(dtype, w).reshape(-1)
@@ -143,6 +180,8 @@ def test_integer_subdots_match_numpy_brute_force(name):
     elif dtype == oracle.Q6_K:
         codes = np_codes_q6k(w)[0]
         want = (codes * q[None, :]).reshape(n, k // 16, 16).sum(axis=2)
+    elif dtype in LOWBIT.values():
+        want = (np_codes_lowbit(dtype, w)[0] * q[None, :]).reshape(n, k // 16, 16).sum(axis=2)
     else:
         codes = np_codes_legacy(dtype, w)[0] if dtype in LEGACY.values() else np_codes_q80(w)[0]
         want = (codes * q[None, :]).reshape(n, k // 32, 32).sum(axis=2)
@@ -260,7 +299,7 @@ def test_driver_error_conditions():
     with pytest.raises(oracle.OracleError, match="byte length"):
         oracle.oa_matmul(oracle.Q4_K, np.zeros((1, 512), np.float32), w, 5)
     with pytest.raises(oracle.OracleError, match="not handled"):
-        oracle.oa_matmul(10, np.zeros((1, 512), np.float32), w, 4)   # Q2_K: no statement of it here
+        oracle.oa_matmul(16, np.zeros((1, 512), np.float32), w, 4)   # IQ2_XXS: no statement of it here
 
 
 def test_empty_rows_and_columns():
