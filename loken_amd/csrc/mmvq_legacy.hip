@@ -1,5 +1,5 @@
-// Mat-vec for the 32-value nibble formats Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, MXFP4 against Q8_1
-// activation rows.
+// Mat-vec for the 32-value nibble formats Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, MXFP4 and the two-bit
+// K-quants Q2_K, Q3_K against Q8_1 activation rows.
 //
 // Formats as loken states them (src/tensor/quant_cpu/format/q4_0.rs, q4_1.rs, q5_0.rs, q5_1.rs): byte
 // j of `qs` holds value j in its low nibble and value j + 16 in its high one; the five-bit formats
@@ -160,12 +160,131 @@ __global__ __launch_bounds__(64) void subdots_legacy_kernel(const uint8_t* __res
     dots[(size_t)row * nb + b] = dot;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Q2_K {scales[16], qs[64], d, dmin} (84 bytes) and Q3_K {hmask[32], qs[64], scales[12], d} (110
+// bytes): sixteen sub-blocks of sixteen two-bit codes (src/tensor/quant_cpu/format/q2_k.rs:15-33,
+// q3_k.rs:10-37, 127-146). The 32 values of Q8_1 block j of a super-block are sub-blocks 2 j and
+// 2 j + 1: bytes 32 (j / 4) .. + 32 of qs at shift 2 (j % 4), and for Q3_K bit j of the 32 hmask
+// bytes (clear = the value is four less). Q2_K: d * (sc & 15) * q - dmin * (sc >> 4); Q3_K:
+// d * (six-bit scale - 32) * (q - 4 * !h). Combined as the reference's mat-vec combines them
+// (cuda/moe/gguf.cuh:524-546, 937-959). A lane owns one Q8_1 block of the row; eight lanes share a
+// super-block (and re-read its header bytes from cache). The plain statement, as above.
+// ---------------------------------------------------------------------------------------------
+struct LowbitBlock {
+    uint4 lo, hi;         // the block's codes 0..3, values 0..15 and 16..31
+    uint4 nlo, nhi;       // Q3_K: 1 where the high bit is clear
+    int sc0, sc1, mn0, mn1;
+    float d, dmin;
+};
+
+template <int ID>
+static __device__ __forceinline__ LowbitBlock lowbit_block(const uint8_t* __restrict__ bp, int j) {
+    LowbitBlock r;
+    const int shift = 2 * (j & 3);
+    const uint8_t* qs = bp + (ID == 10 ? 16 : 32) + 32 * (j >> 2);
+    const uint4 q0 = *(const uint4_a2*)qs, q1 = *(const uint4_a2*)(qs + 16);
+    r.lo = make_uint4((q0.x >> shift) & 0x03030303u, (q0.y >> shift) & 0x03030303u, (q0.z >> shift) & 0x03030303u, (q0.w >> shift) & 0x03030303u);
+    r.hi = make_uint4((q1.x >> shift) & 0x03030303u, (q1.y >> shift) & 0x03030303u, (q1.z >> shift) & 0x03030303u, (q1.w >> shift) & 0x03030303u);
+    if (ID == 10) {
+        const uint32_t s0 = bp[2 * j], s1 = bp[2 * j + 1];
+        r.sc0 = s0 & 15; r.mn0 = s0 >> 4; r.sc1 = s1 & 15; r.mn1 = s1 >> 4;
+        r.d = f16_bits_to_f32(*(const uint16_t*)(bp + 80));
+        r.dmin = f16_bits_to_f32(*(const uint16_t*)(bp + 82));
+        r.nlo = r.nhi = make_uint4(0, 0, 0, 0);
+    } else {
+        const uint4 h0 = *(const uint4_a2*)bp, h1 = *(const uint4_a2*)(bp + 16);
+        r.nlo = make_uint4((~h0.x >> j) & 0x01010101u, (~h0.y >> j) & 0x01010101u, (~h0.z >> j) & 0x01010101u, (~h0.w >> j) & 0x01010101u);
+        r.nhi = make_uint4((~h1.x >> j) & 0x01010101u, (~h1.y >> j) & 0x01010101u, (~h1.z >> j) & 0x01010101u, (~h1.w >> j) & 0x01010101u);
+        // scales 2 j and 2 j + 1 of the sixteen packed in twelve bytes
+        const uint8_t* p = bp + 96;
+        const int group = j >> 1, jj = 2 * (j & 1);
+        const uint32_t b0 = p[jj + 4 * (group & 1)], b1 = p[jj + 1 + 4 * (group & 1)];
+        const uint32_t t0 = p[8 + jj], t1 = p[9 + jj];
+        r.sc0 = (int)((group < 2 ? (b0 & 15) : (b0 >> 4)) | (((t0 >> (2 * group)) & 3) << 4)) - 32;
+        r.sc1 = (int)((group < 2 ? (b1 & 15) : (b1 >> 4)) | (((t1 >> (2 * group)) & 3) << 4)) - 32;
+        r.mn0 = r.mn1 = 0;
+        r.d = f16_bits_to_f32(*(const uint16_t*)(bp + 108));
+        r.dmin = 0.f;
+    }
+    return r;
+}
+
+// The two sub-block integers of the block against a Q8_1 block, and the two activation sums.
+template <int ID>
+static __device__ __forceinline__ void lowbit_dots(const LowbitBlock& w, const uint8_t* __restrict__ yb, int& dot0, int& dot1,
+                                                   int& sum0, int& sum1) {
+    const uint4 a_lo = *(const uint4_a4*)(yb + 4), a_hi = *(const uint4_a4*)(yb + 20);
+    dot0 = dot16(w.lo, a_lo, 0);
+    dot1 = dot16(w.hi, a_hi, 0);
+    if (ID == 10) {
+        const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
+        sum0 = dot16(ones, a_lo, 0);
+        sum1 = dot16(ones, a_hi, 0);
+    } else {
+        dot0 -= 4 * dot16(w.nlo, a_lo, 0);
+        dot1 -= 4 * dot16(w.nhi, a_hi, 0);
+        sum0 = sum1 = 0;
+    }
+}
+
+template <int ID, int B, typename T>
+__global__ __launch_bounds__(LWG) void mmvq_lowbit_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
+                                                          T* __restrict__ dst, const float* __restrict__ bias, int nb, int n,
+                                                          int stride_col_y, int stride_col_dst) {
+    constexpr int BYTES = ID == 10 ? 84 : 110;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int k32 = nb * 8;
+    for (int row = blockIdx.x * LWAVES + wave; row < n; row += gridDim.x * LWAVES) {
+        const uint8_t* wrow = vx + (size_t)row * nb * BYTES;
+        float acc[B];
+#pragma unroll
+        for (int c = 0; c < B; ++c) acc[c] = 0.f;
+        for (int idx = lane; idx < k32; idx += 64) {
+            const LowbitBlock w = lowbit_block<ID>(wrow + (size_t)(idx >> 3) * BYTES, idx & 7);
+#pragma unroll
+            for (int c = 0; c < B; ++c) {
+                const uint8_t* yb = vy + ((size_t)c * stride_col_y + idx) * Q81_BYTES;
+                const float d8 = f16_bits_to_f32(*(const uint16_t*)yb);
+                int dot0, dot1, sum0, sum1;
+                lowbit_dots<ID>(w, yb, dot0, dot1, sum0, sum1);
+                float part = w.d * (d8 * (float)(dot0 * w.sc0 + dot1 * w.sc1));
+                if (ID == 10) part -= w.dmin * (d8 * (float)(sum0 * w.mn0 + sum1 * w.mn1));
+                acc[c] += part;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < B; ++c) {
+            const float total = wave_sum(acc[c]);
+            if (lane == 0) dst[(size_t)c * stride_col_dst + row] = from_f32<T>(bias ? total + bias[row] : total);
+        }
+    }
+}
+
+template <int ID>
+__global__ __launch_bounds__(64) void subdots_lowbit_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
+                                                            int32_t* __restrict__ dots, int nb) {
+    constexpr int BYTES = ID == 10 ? 84 : 110;
+    const int row = blockIdx.y, idx = blockIdx.x * 64 + threadIdx.x;
+    if (idx >= nb * 8) return;
+    const LowbitBlock w = lowbit_block<ID>(vx + ((size_t)row * nb + (idx >> 3)) * BYTES, idx & 7);
+    int dot0, dot1, sum0, sum1;
+    lowbit_dots<ID>(w, vy + (size_t)idx * Q81_BYTES, dot0, dot1, sum0, sum1);
+    int32_t* out = dots + (size_t)row * nb * 16 + 2 * idx;
+    out[0] = dot0;
+    out[1] = dot1;
+}
+
 template <int ID, int B, typename T>
 static int launch(const void* vx, const void* vy, void* dst, const float* bias, int nb, int n, int stride_col_y,
                   int stride_col_dst, hipStream_t s) {
     const int need = (n + LWAVES - 1) / LWAVES, cap = lk_device().cus * 8;
-    hipLaunchKernelGGL((mmvq_legacy_kernel<ID, B, T>), dim3(need < cap ? need : cap), dim3(LWG), 0, s, (const uint8_t*)vx,
-                       (const uint8_t*)vy, (T*)dst, bias, nb, n, stride_col_y, stride_col_dst);
+    if constexpr (ID == 10 || ID == 11)
+        hipLaunchKernelGGL((mmvq_lowbit_kernel<ID, B, T>), dim3(need < cap ? need : cap), dim3(LWG), 0, s, (const uint8_t*)vx,
+                           (const uint8_t*)vy, (T*)dst, bias, nb, n, stride_col_y, stride_col_dst);
+    else
+        hipLaunchKernelGGL((mmvq_legacy_kernel<ID, B, T>), dim3(need < cap ? need : cap), dim3(LWG), 0, s, (const uint8_t*)vx,
+                           (const uint8_t*)vy, (T*)dst, bias, nb, n, stride_col_y, stride_col_dst);
     return lk_launch_status();
 }
 
@@ -201,18 +320,21 @@ static int by_type(int dst_type, int batch, const void* vx, const void* vy, void
 
 bool lk_is_legacy_type(int wtype) {
     return wtype == LK_TYPE_Q4_0 || wtype == LK_TYPE_Q4_1 || wtype == LK_TYPE_Q5_0 || wtype == LK_TYPE_Q5_1 ||
-           wtype == LK_TYPE_IQ4_NL || wtype == LK_TYPE_MXFP4;
+           wtype == LK_TYPE_IQ4_NL || wtype == LK_TYPE_MXFP4 || wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K;
 }
 
 // lk_mmvq for the 32-value nibble formats (the caller has told them apart with lk_is_legacy_type).
 int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, int dst_type, int ncols_x, int nrows_x,
                    int batch, int stride_col_y, int stride_col_dst, const float* bias, hipStream_t s) {
     if (nrows_x == 0) return LK_OK;
-    if (!vx || !vy_q8_1 || !dst || ncols_x <= 0 || ncols_x % 32 != 0 || nrows_x < 0) return LK_ERR_ARG;
+    const int block_len = wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K ? 256 : 32;
+    if (!vx || !vy_q8_1 || !dst || ncols_x <= 0 || ncols_x % block_len != 0 || nrows_x < 0) return LK_ERR_ARG;
     if (batch < 1 || batch > 8 || stride_col_y < ncols_x / 32 || stride_col_dst < nrows_x) return LK_ERR_ARG;
     if ((wtype != LK_TYPE_MXFP4 && ((uintptr_t)vx & 1) != 0) || ((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
-    const int nb = ncols_x / 32;
+    const int nb = ncols_x / block_len;
     switch (wtype) {
+        case LK_TYPE_Q2_K: return by_type<10>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_Q3_K: return by_type<11>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q4_0: return by_type<2>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q4_1: return by_type<3>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q5_0: return by_type<6>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
@@ -226,9 +348,17 @@ int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, in
 int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32_t* dots, int ncols_x, int nrows_x,
                            hipStream_t s) {
     if (!vx || !vy_q8_1 || !dots || ncols_x <= 0 || ncols_x % 32 != 0 || nrows_x <= 0 || nrows_x > 65535) return LK_ERR_ARG;
+    const uint8_t *w = (const uint8_t*)vx, *y = (const uint8_t*)vy_q8_1;
+    if (wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K) {   // sixteen sub-block integers per super-block
+        if (ncols_x % 256 != 0) return LK_ERR_ARG;
+        const int nbk = ncols_x / 256;
+        const dim3 gridk((nbk * 8 + 63) / 64, nrows_x);
+        if (wtype == LK_TYPE_Q2_K) hipLaunchKernelGGL(subdots_lowbit_kernel<10>, gridk, dim3(64), 0, s, w, y, dots, nbk);
+        else hipLaunchKernelGGL(subdots_lowbit_kernel<11>, gridk, dim3(64), 0, s, w, y, dots, nbk);
+        return lk_launch_status();
+    }
     const int nb = ncols_x / 32;
     const dim3 grid((nb + 63) / 64, nrows_x);
-    const uint8_t *w = (const uint8_t*)vx, *y = (const uint8_t*)vy_q8_1;
     switch (wtype) {
         case LK_TYPE_Q4_0: hipLaunchKernelGGL(subdots_legacy_kernel<2>, grid, dim3(64), 0, s, w, y, dots, nb); break;
         case LK_TYPE_Q4_1: hipLaunchKernelGGL(subdots_legacy_kernel<3>, grid, dim3(64), 0, s, w, y, dots, nb); break;

@@ -167,7 +167,7 @@ def mmvq_grouped(wtype: int, table: torch.Tensor, q8_1: torch.Tensor, k: int, n:
 
 def mmvq_subdots(wtype: int, weight: torch.Tensor, q8_1_row: torch.Tensor, k: int, n: int):
     """Integer sub-block dots of every weight row against ONE Q8_1 row (parity probe)."""
-    per = 16 if wtype == _lib.TYPE_Q6_K else 32
+    per = 16 if wtype in (_lib.TYPE_Q6_K, _lib.TYPE_Q2_K, _lib.TYPE_Q3_K) else 32
     dots = torch.empty((n, k // per), dtype=torch.int32, device=weight.device)
     sums = torch.empty((k // 32,), dtype=torch.int32, device=weight.device)
     _lib.check("lk_mmvq_subdots", _lib.load().lk_mmvq_subdots(

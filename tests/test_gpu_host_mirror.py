@@ -11,7 +11,7 @@ from loken_amd import lib, ops, synth
 pytestmark = pytest.mark.gpu
 
 DT = {"q4_k": lib.TYPE_Q4_K, "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0,
-      "q4_0": lib.TYPE_Q4_0, "q5_1": lib.TYPE_Q5_1, "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4}
+      "q4_0": lib.TYPE_Q4_0, "q5_1": lib.TYPE_Q5_1, "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K}
 PATH = {1: "matvec-fused", 2: "matvec", 3: "rows-on-matrix-unit", 4: "tiled"}
 X_TYPES = {torch.float32: lib.TYPE_F32, torch.float16: lib.TYPE_F16, torch.bfloat16: lib.TYPE_BF16}
 
@@ -54,7 +54,7 @@ def close(got, want, rtol=1e-3, atol=1e-4):
     ("q4_k", 40, "rows-on-matrix-unit"), ("q4_k", 80, "tiled"), ("q6_k", 1, "matvec-fused"), ("q6_k", 20, "matvec"),
     ("q6_k", 40, "tiled"), ("q8_0", 3, "matvec"), ("q8_0", 33, "tiled"), ("q5_k", 1, "matvec-fused"),
     ("q5_k", 20, "matvec"), ("q5_k", 40, "tiled"), ("q5_k", 200, "tiled"), ("q4_0", 1, "matvec"), ("q4_0", 50, "matvec"),
-    ("q5_1", 9, "matvec"), ("iq4_nl", 3, "matvec"), ("mxfp4", 17, "matvec")])
+    ("q5_1", 9, "matvec"), ("iq4_nl", 3, "matvec"), ("mxfp4", 17, "matvec"), ("q2_k", 12, "matvec"), ("q3_k", 1, "matvec")])
 def test_forward_takes_the_path_of_its_row_count_and_matches_the_oracle(name, rows, expect):
     wtype, n, k = DT[name], 200, 1024
     w = synth.weight(wtype, n, k, seed=80, stream=1)

@@ -151,6 +151,52 @@ def test_legacy_matvec_within_the_reference_envelope(name):
     assert (np.abs(oracle.oa_matmul(wtype, x, w, n) - truth) <= envelope).all()
 
 
+LOWBIT = {"q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K}
+
+
+@pytest.mark.parametrize("name", sorted(LOWBIT))
+@pytest.mark.parametrize("n,k", [(16, 1024), (5, 768), (3, 256), (40, 4096)])
+def test_two_bit_integer_subblock_dots_are_bit_exact(name, n, k):
+    wtype = LOWBIT[name]
+    w = synth.weight(wtype, n, k, seed=74, stream=1)
+    x = synth.activation(1, k, seed=74)
+    q = ops.quantize_q8_1_rows(dev(x))
+    dots, sums = ops.mmvq_subdots(wtype, dev(w), q[0], k, n)
+    want_dots, want_sums = oracle.ob_subdots(wtype, k, n, w, oracle.quantize_q8_1(x))
+    assert np.array_equal(dots.cpu().numpy(), want_dots)
+    assert np.array_equal(sums.cpu().numpy(), want_sums)
+
+
+@pytest.mark.parametrize("name", sorted(LOWBIT))
+@pytest.mark.parametrize("n,k", [(4096, 4096), (33, 768), (1, 256), (257, 2048), (500, 14336)])
+@pytest.mark.parametrize("batch", [1, 3, 4, 8])
+def test_two_bit_matvec_matches_same_codes_oracle(name, n, k, batch):
+    wtype = LOWBIT[name]
+    w = synth.weight(wtype, n, k, seed=75, stream=2)
+    x = synth.activation(batch, k, seed=75)
+    got = ops.mmvq(wtype, dev(w), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(wtype, x, w, n))
+
+
+@pytest.mark.parametrize("name", sorted(LOWBIT))
+def test_two_bit_matvec_within_the_reference_envelope_and_outputs(name):
+    wtype = LOWBIT[name]
+    n, k = 256, 4096
+    w = synth.weight(wtype, n, k, seed=76, stream=4)
+    x = synth.activation(2, k, seed=76)
+    q = ops.quantize_q8_1_rows(dev(x))
+    got_t = ops.mmvq(wtype, dev(w), q, k, n)
+    got = got_t.cpu().numpy()
+    wd = oracle.dequantize(wtype, w).reshape(n, k).astype(np.float64)
+    truth = x.astype(np.float64) @ wd.T
+    envelope = 1e-3 * (np.abs(x.astype(np.float64)) @ np.abs(wd).T) + 1e-3
+    assert (np.abs(got - truth) <= envelope).all()
+    assert (np.abs(oracle.oa_matmul(wtype, x, w, n) - truth) <= envelope).all()
+    bias = dev(synth.normal(76, 9, n))
+    assert torch.equal(ops.mmvq(wtype, dev(w), q, k, n, bias=bias), got_t + bias)
+    assert torch.equal(ops.mmvq(wtype, dev(w), q, k, n, out_dtype=torch.bfloat16), got_t.to(torch.bfloat16))
+
+
 # ---------------------------------------------------------------- f32 outputs
 SHAPES = [
     ("q4_k", 4096, 4096), ("q4_k", 1024, 4096), ("q4_k", 33, 768), ("q4_k", 1, 256), ("q4_k", 257, 2048),
