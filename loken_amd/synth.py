@@ -23,9 +23,10 @@ import numpy as np
 GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1 = 2, 3, 6, 7
 GGML_IQ4_NL, GGML_MXFP4 = 20, 39
 GGML_Q2_K, GGML_Q3_K = 10, 11
+GGML_IQ4_XS = 23
 GGML_Q8_0, GGML_Q8_1, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K = 8, 9, 12, 13, 14
-BLOCK_LEN = {GGML_Q2_K: 256, GGML_Q3_K: 256, GGML_IQ4_NL: 32, GGML_MXFP4: 32, GGML_Q4_0: 32, GGML_Q4_1: 32, GGML_Q5_0: 32, GGML_Q5_1: 32, GGML_Q8_0: 32, GGML_Q8_1: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256}
-BLOCK_BYTES = {GGML_Q2_K: 84, GGML_Q3_K: 110, GGML_IQ4_NL: 18, GGML_MXFP4: 17, GGML_Q4_0: 18, GGML_Q4_1: 20, GGML_Q5_0: 22, GGML_Q5_1: 24, GGML_Q8_0: 34, GGML_Q8_1: 36, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210}
+BLOCK_LEN = {GGML_IQ4_XS: 256, GGML_Q2_K: 256, GGML_Q3_K: 256, GGML_IQ4_NL: 32, GGML_MXFP4: 32, GGML_Q4_0: 32, GGML_Q4_1: 32, GGML_Q5_0: 32, GGML_Q5_1: 32, GGML_Q8_0: 32, GGML_Q8_1: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256}
+BLOCK_BYTES = {GGML_IQ4_XS: 136, GGML_Q2_K: 84, GGML_Q3_K: 110, GGML_IQ4_NL: 18, GGML_MXFP4: 17, GGML_Q4_0: 18, GGML_Q4_1: 20, GGML_Q5_0: 22, GGML_Q5_1: 24, GGML_Q8_0: 34, GGML_Q8_1: 36, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210}
 
 _G = np.uint64(0x9E3779B97F4A7C15)
 _M1 = np.uint64(0xBF58476D1CE4E5B9)
@@ -133,6 +134,9 @@ def lowbit_blocks(dtype: int, n_blocks: int, seed: int = 0, stream: int = 0) -> 
     s = stream * 8
     nbytes = BLOCK_BYTES[dtype]
     out = rand_bytes(seed, s + 0, n_blocks * nbytes).reshape(n_blocks, nbytes).copy()
+    if dtype == GGML_IQ4_XS:   # d leads the block; everything else is codes and scale bits
+        out[:, 0:2] = _f16_bytes(np.abs(normal(seed, s + 1, n_blocks)) * np.float32(2e-5))
+        return out
     out[:, nbytes - 2:] = _f16_bytes(np.abs(normal(seed, s + 1, n_blocks)) * np.float32(1e-3))
     if dtype == GGML_Q2_K:
         out[:, 80:82] = _f16_bytes(np.abs(normal(seed, s + 2, n_blocks)) * np.float32(2e-3))   # d; dmin is the tail
@@ -155,7 +159,8 @@ def legacy_blocks(dtype: int, n_blocks: int, seed: int = 0, stream: int = 0) -> 
     return out
 
 
-_MAKERS = {GGML_Q2_K: lambda n, seed=0, stream=0: lowbit_blocks(GGML_Q2_K, n, seed, stream),
+_MAKERS = {GGML_IQ4_XS: lambda n, seed=0, stream=0: lowbit_blocks(GGML_IQ4_XS, n, seed, stream),
+           GGML_Q2_K: lambda n, seed=0, stream=0: lowbit_blocks(GGML_Q2_K, n, seed, stream),
            GGML_Q3_K: lambda n, seed=0, stream=0: lowbit_blocks(GGML_Q3_K, n, seed, stream),
            GGML_IQ4_NL: lambda n, seed=0, stream=0: legacy_blocks(GGML_IQ4_NL, n, seed, stream),
            GGML_MXFP4: lambda n, seed=0, stream=0: legacy_blocks(GGML_MXFP4, n, seed, stream),

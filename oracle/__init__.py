@@ -17,9 +17,10 @@ _LIB_PATH = _HERE / "libloken_oracle.so"
 Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 IQ4_NL, MXFP4 = 20, 39
 Q2_K, Q3_K = 10, 11
+IQ4_XS = 23
 Q8_0, Q8_1, Q4_K, Q5_K, Q6_K, Q8_K = 8, 9, 12, 13, 14, 15
-BLOCK_LEN = {Q2_K: 256, Q3_K: 256, IQ4_NL: 32, MXFP4: 32, Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
-BLOCK_BYTES = {Q2_K: 84, Q3_K: 110, IQ4_NL: 18, MXFP4: 17, Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
+BLOCK_LEN = {IQ4_XS: 256, Q2_K: 256, Q3_K: 256, IQ4_NL: 32, MXFP4: 32, Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
+BLOCK_BYTES = {IQ4_XS: 136, Q2_K: 84, Q3_K: 110, IQ4_NL: 18, MXFP4: 17, Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
 
 
 def build(force: bool = False) -> Path:

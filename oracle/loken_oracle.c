@@ -81,7 +81,7 @@ int lko_block_len(int dtype) {
     switch (dtype) {
         case LKO_Q8_0: case LKO_Q8_1: case LKO_Q4_0: case LKO_Q4_1: case LKO_Q5_0: case LKO_Q5_1:
         case LKO_IQ4_NL: case LKO_MXFP4: return 32;
-        case LKO_Q2_K: case LKO_Q3_K: case LKO_Q4_K: case LKO_Q5_K: case LKO_Q6_K: case LKO_Q8_K: return 256;
+        case LKO_Q2_K: case LKO_Q3_K: case LKO_Q4_K: case LKO_Q5_K: case LKO_Q6_K: case LKO_Q8_K: case LKO_IQ4_XS: return 256;
         default: return 0;
     }
 }
@@ -97,6 +97,7 @@ int lko_block_bytes(int dtype) {
         case LKO_MXFP4: return 17;
         case LKO_Q8_1: return LKO_Q81_BYTES;
         case LKO_Q2_K: return 84;
+        case LKO_IQ4_XS: return 136;
         case LKO_Q3_K: return 110;
         case LKO_Q4_K: return LKO_Q4K_BYTES;
         case LKO_Q5_K: return LKO_Q5K_BYTES;
@@ -180,6 +181,7 @@ static inline int q5k_code(const uint8_t* blk, int s, int l) {
 
 static int legacy_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out);
 static int lowbit_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out);
+static int iq4xs_dequantize(const uint8_t* blocks, size_t n_blocks, float* out);
 
 int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out) {
     switch (dtype) {
@@ -254,6 +256,8 @@ int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out
         return 0;
     case LKO_Q2_K: case LKO_Q3_K:
         return lowbit_dequantize(dtype, blocks, n_blocks, out);
+    case LKO_IQ4_XS:
+        return iq4xs_dequantize(blocks, n_blocks, out);
     default:
         return legacy_dequantize(dtype, blocks, n_blocks, out);
     }
@@ -814,11 +818,62 @@ static float ob_dot_q3k(const uint8_t* w, const uint8_t* y, size_t nb) {
     return total;
 }
 
+
+/* IQ4_XS {d, scales_h u16, scales_l[4], qs[128]} = 136 bytes (iq4_xs.rs:5-10): eight runs of 32
+ * values, run ib = bytes 16 ib .. + 16 of qs (byte j: value j low, value j + 16 high) as IQ4_NL
+ * levels, times d * (six-bit scale - 32), the scale's low four bits in scales_l, top two in
+ * scales_h (iq4_xs.rs:24-37). Its CPU dot pairs it with per-32 activation runs quantized as Q8_1
+ * quantizes (q8_k32.rs:44-57) and adds run_scale * dot * y.d per run (iq4_xs.rs:50-62). */
+static inline int iq4xs_scale(const uint8_t* blk, int ib) {
+    const int low = (blk[4 + ib / 2] >> (4 * (ib % 2))) & 0x0F;
+    const int high = (rd_u16(blk + 2) >> (2 * ib)) & 3;
+    return (low | (high << 4)) - 32;
+}
+static inline int32_t iq4xs_sub_dot(const uint8_t* blk, int ib, const int8_t* acts) {
+    const uint8_t* q = blk + 8 + 16 * ib;
+    int32_t dot = 0;
+    for (int j = 0; j < 16; ++j)
+        dot += (int32_t)LEVELS_IQ4NL[q[j] & 0x0F] * acts[j] + (int32_t)LEVELS_IQ4NL[q[j] >> 4] * acts[j + 16];
+    return dot;
+}
+static int iq4xs_dequantize(const uint8_t* blocks, size_t n_blocks, float* out) {
+    for (size_t b = 0; b < n_blocks; ++b) {
+        const uint8_t* blk = blocks + b * 136;
+        const float d = lko_f16_to_f32(rd_u16(blk));
+        for (int ib = 0; ib < 8; ++ib) {
+            const float dl = d * (float)iq4xs_scale(blk, ib);
+            const uint8_t* q = blk + 8 + 16 * ib;
+            for (int j = 0; j < 16; ++j) {
+                out[b * 256 + 32 * ib + j] = dl * (float)LEVELS_IQ4NL[q[j] & 0x0F];
+                out[b * 256 + 32 * ib + j + 16] = dl * (float)LEVELS_IQ4NL[q[j] >> 4];
+            }
+        }
+    }
+    return 0;
+}
+/* Both families read Q8_1-quantized runs (the served path's run quantizer is Q8_1's). */
+static float dot_iq4xs(const uint8_t* w, const uint8_t* y, size_t nb) {
+    float total = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * 136;
+        const float d = lko_f16_to_f32(rd_u16(x));
+        float block = 0.0f;
+        for (int ib = 0; ib < 8; ++ib) {
+            const uint8_t* yb = y + (b * 8 + ib) * LKO_Q81_BYTES;
+            const int32_t dot = iq4xs_sub_dot(x, ib, (const int8_t*)(yb + 4));
+            block += d * (float)iq4xs_scale(x, ib) * (float)dot * lko_f16_to_f32(rd_u16(yb));
+        }
+        total += block;
+    }
+    return total;
+}
+
 typedef float (*row_dot_fn)(const uint8_t* w, const uint8_t* y, size_t nb);
 
 static row_dot_fn oa_dot_of(int dtype) {
     switch (dtype) {
         case LKO_Q2_K: return oa_dot_q2k;
+        case LKO_IQ4_XS: return dot_iq4xs;
         case LKO_Q3_K: return oa_dot_q3k;
         case LKO_Q4_K: return oa_dot_q4k;
         case LKO_Q5_K: return oa_dot_q5k;
@@ -836,6 +891,7 @@ static row_dot_fn oa_dot_of(int dtype) {
 static row_dot_fn ob_dot_of(int dtype) {
     switch (dtype) {
         case LKO_Q2_K: return ob_dot_q2k;
+        case LKO_IQ4_XS: return dot_iq4xs;
         case LKO_Q3_K: return ob_dot_q3k;
         case LKO_Q4_K: return ob_dot_q4k;
         case LKO_Q5_K: return ob_dot_q5k;
@@ -855,13 +911,13 @@ static row_dot_fn ob_dot_of(int dtype) {
 static size_t oa_act_row_bytes(int dtype, size_t k) {
     if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0 || dtype == LKO_IQ4_NL || dtype == LKO_MXFP4)
         return (k / 32) * LKO_Q80_BYTES;
-    if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1) return (k / 32) * LKO_Q81_BYTES;   /* q4_1.rs: BlockQ8_1 */
+    if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1 || dtype == LKO_IQ4_XS) return (k / 32) * LKO_Q81_BYTES;   /* q4_1.rs: BlockQ8_1 */
     return (k / 256) * LKO_Q8K_BYTES;
 }
 static void oa_quantize_act(int dtype, const float* x, size_t k, uint8_t* out) {
     if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0 || dtype == LKO_IQ4_NL || dtype == LKO_MXFP4)
         lko_quantize_q8_0(x, k, out);
-    else if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1) lko_quantize_q8_1(x, k, out);
+    else if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1 || dtype == LKO_IQ4_XS) lko_quantize_q8_1(x, k, out);
     else lko_quantize_q8_k(x, k, out);
 }
 
@@ -908,7 +964,7 @@ int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t*
     const size_t blk = (size_t)lko_block_len(dtype);
     legacy_layout ll;
     const int legacy = legacy_layout_of(dtype, &ll);
-    if (blk == 0 || (!legacy && dtype != LKO_Q2_K && dtype != LKO_Q3_K && dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
+    if (blk == 0 || (!legacy && dtype != LKO_IQ4_XS && dtype != LKO_Q2_K && dtype != LKO_Q3_K && dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
     if (k % blk != 0) return -1;
     const size_t nb = k / blk;
     const size_t wrow = nb * (size_t)lko_block_bytes(dtype);
@@ -927,6 +983,11 @@ int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t*
                 for (int s = 0; s < 8; ++s)
                     dots[c * (k / 32) + b * 8 + s] = q4k_sub_dot(
                         w + b * LKO_Q4K_BYTES, s, (const int8_t*)(act + (b * 8 + s) * LKO_Q81_BYTES + 4));
+        } else if (dtype == LKO_IQ4_XS) {
+            for (size_t b = 0; b < nb; ++b)
+                for (int s = 0; s < 8; ++s)
+                    dots[c * (k / 32) + b * 8 + s] = iq4xs_sub_dot(
+                        w + b * 136, s, (const int8_t*)(act + (b * 8 + s) * LKO_Q81_BYTES + 4));
         } else if (dtype == LKO_Q2_K || dtype == LKO_Q3_K) {
             for (size_t b = 0; b < nb; ++b)
                 for (int s = 0; s < 16; ++s) {
@@ -1031,6 +1092,19 @@ static int dequant_row_f64(int dtype, const uint8_t* w, size_t nb, double* out) 
             const uint8_t* x = w + b * LKO_Q80_BYTES;
             const double d = lko_f16_to_f32(rd_u16(x));
             for (int l = 0; l < 32; ++l) out[b * 32 + l] = d * (double)(int8_t)x[2 + l];
+        }
+        return 0;
+    }
+    if (dtype == LKO_IQ4_XS) {
+        for (size_t b = 0; b < nb; ++b) {
+            const uint8_t* x = w + b * 136;
+            const double d = lko_f16_to_f32(rd_u16(x));
+            for (int ib = 0; ib < 8; ++ib)
+                for (int j = 0; j < 16; ++j) {
+                    const uint8_t q = x[8 + 16 * ib + j];
+                    out[b * 256 + 32 * ib + j] = d * iq4xs_scale(x, ib) * LEVELS_IQ4NL[q & 0x0F];
+                    out[b * 256 + 32 * ib + j + 16] = d * iq4xs_scale(x, ib) * LEVELS_IQ4NL[q >> 4];
+                }
         }
         return 0;
     }

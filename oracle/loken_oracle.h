@@ -38,7 +38,7 @@ extern "C" {
 /* ggml type ids, src/tensor/quantized/dtype.rs:66-96 */
 enum { LKO_Q4_0 = 2, LKO_Q4_1 = 3, LKO_Q5_0 = 6, LKO_Q5_1 = 7, LKO_Q8_0 = 8, LKO_Q8_1 = 9, LKO_Q2_K = 10, LKO_Q3_K = 11,
        LKO_Q4_K = 12, LKO_Q5_K = 13,
-       LKO_Q6_K = 14, LKO_Q8_K = 15, LKO_IQ4_NL = 20, LKO_MXFP4 = 39 };
+       LKO_Q6_K = 14, LKO_Q8_K = 15, LKO_IQ4_NL = 20, LKO_IQ4_XS = 23, LKO_MXFP4 = 39 };
 
 #define LKO_QK_K 256
 #define LKO_Q4K_BYTES 144

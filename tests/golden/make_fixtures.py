@@ -43,7 +43,7 @@ def main(ref: str) -> None:
     sub = {k: j[k] for k in ("rows", "cols", "read", "x")}
     sub["formats"] = {
         f: {"blocks": j["formats"][f]["blocks"], "expected": j["formats"][f]["expected"]}
-        for f in ("q4_0", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k", "q8_0", "iq4_nl", "mxfp4")
+        for f in ("q4_0", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k", "q8_0", "iq4_nl", "iq4_xs", "mxfp4")
     }
     (here / "ggml_encode_subset.json").write_text(json.dumps(sub))
 

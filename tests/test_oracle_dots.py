@@ -19,8 +19,9 @@ LEGACY = {"q4_0": oracle.Q4_0, "q4_1": oracle.Q4_1, "q5_0": oracle.Q5_0, "q5_1":
 LEVELS = {oracle.IQ4_NL: np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int64),
           oracle.MXFP4: np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], np.int64)}
 LOWBIT = {"q2_k": oracle.Q2_K, "q3_k": oracle.Q3_K}
-DT = {"q4_k": oracle.Q4_K, "q5_k": oracle.Q5_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0, **LEGACY, **LOWBIT}
-FAST = sorted(set(DT) - {"q5_k"} - set(LEGACY) - set(LOWBIT))   # formats the timed AVX2 baseline serves
+DT = {"q4_k": oracle.Q4_K, "q5_k": oracle.Q5_K, "q6_k": oracle.Q6_K, "q8_0": oracle.Q8_0, "iq4_xs": oracle.IQ4_XS, **LEGACY,
+      **LOWBIT}
+FAST = sorted(set(DT) - {"q5_k", "iq4_xs"} - set(LEGACY) - set(LOWBIT))   # formats the timed AVX2 baseline serves
 
 
 # ---- independent numpy decoders: integer codes and float scales per value ----
@@ -125,6 +126,19 @@ def np_codes_lowbit(dtype, w):
     return vals.reshape(n, nb * 256), sc.reshape(n, nb * 16), mn.reshape(n, nb * 16), d, dmin
 
 
+def np_codes_iq4xs(w):
+    """w [n, nb, 136] -> levels [n, nb*256], run scales (six bits less 32) [n, nb*8], d [n, nb]."""
+    n, nb, _ = w.shape
+    q = w[:, :, 8:136].reshape(n, nb, 8, 16).astype(np.int64)
+    lv = LEVELS[oracle.IQ4_NL]
+    vals = np.concatenate([lv[q & 0xF], lv[q >> 4]], axis=3)                         # [n, nb, run, 32]
+    sl = w[:, :, 4:8].astype(np.int64)
+    sh = w[:, :, 2:4].copy().view(np.uint16).reshape(n, nb).astype(np.int64)
+    ls = np.stack([((sl[:, :, ib // 2] >> (4 * (ib % 2))) & 0xF) | (((sh >> (2 * ib)) & 3) << 4) for ib in range(8)], axis=2) - 32
+    d = w[:, :, 0:2].copy().view(np.float16).reshape(n, nb).astype(np.float64)
+    return vals.reshape(n, nb * 256), ls.reshape(n, nb * 8), d
+
+
 def np_q81(act_bytes):
     b = act_bytes.reshape(-1, 36)
     d = b[:, 0:2].copy().view(np.float16).reshape(-1).astype(np.float64)
@@ -145,6 +159,9 @@ def np_dequant(dtype, w):
     if dtype in LEGACY.values():
         codes, d, m = np_codes_legacy(dtype, w)
         return np.repeat(d, 32, axis=1) * codes + np.repeat(m, 32, axis=1)
+    if dtype == oracle.IQ4_XS:
+        vals, ls, d = np_codes_iq4xs(w)
+        return np.repeat(ls * np.repeat(d, 8, axis=1), 32, axis=1) * vals
     if dtype in LOWBIT.values():
         vals, sc, mn, d, dmin = np_codes_lowbit(dtype, w)
         return (np.repeat(sc * np.repeat(d, 16, axis=1), 16, axis=1) * vals
@@ -182,6 +199,8 @@ def test_integer_subdots_match_numpy_brute_force(name):
         want = (codes * q[None, :]).reshape(n, k // 16, 16).sum(axis=2)
     elif dtype in LOWBIT.values():
         want = (np_codes_lowbit(dtype, w)[0] * q[None, :]).reshape(n, k // 16, 16).sum(axis=2)
+    elif dtype == oracle.IQ4_XS:
+        want = (np_codes_iq4xs(w)[0] * q[None, :]).reshape(n, k // 32, 32).sum(axis=2)
     else:
         codes = np_codes_legacy(dtype, w)[0] if dtype in LEGACY.values() else np_codes_q80(w)[0]
         want = (codes * q[None, :]).reshape(n, k // 32, 32).sum(axis=2)
@@ -262,6 +281,9 @@ def test_served_path_integer_core_with_q8k_codes(name):
     slack = 0.0
     if dtype in (oracle.Q8_0, oracle.Q4_0, oracle.Q5_0, oracle.IQ4_NL, oracle.MXFP4):
         xa = oracle.dequantize(oracle.Q8_0, oracle.quantize_q8_0(x)).reshape(2, k)
+    elif dtype == oracle.IQ4_XS:   # per-32 runs quantized as Q8_1 quantizes; no sum field is read
+        d8, q = np_q81(oracle.quantize_q8_1(x))
+        xa = (d8[:, None] * q).reshape(2, k)
     elif dtype in (oracle.Q4_1, oracle.Q5_1):
         # these pair with Q8_1 and take the block's sum from its f16 `s` field: the minimum's term
         # carries that field's rounding (2^-11 of |m * s| per block)

@@ -20,7 +20,7 @@ def test_dequantize_matches_ggml_bits(ggml_vectors, name):
     assert got.view(np.uint32).tolist() == rec["dequant"].view(np.uint32).tolist()
 
 
-@pytest.mark.parametrize("name,dtype", [("q2_k", oracle.Q2_K), ("q3_k", oracle.Q3_K), ("iq4_nl", oracle.IQ4_NL), ("mxfp4", oracle.MXFP4), ("q4_0", oracle.Q4_0), ("q4_1", oracle.Q4_1), ("q5_0", oracle.Q5_0), ("q5_1", oracle.Q5_1),
+@pytest.mark.parametrize("name,dtype", [("q2_k", oracle.Q2_K), ("q3_k", oracle.Q3_K), ("iq4_nl", oracle.IQ4_NL), ("iq4_xs", oracle.IQ4_XS), ("mxfp4", oracle.MXFP4), ("q4_0", oracle.Q4_0), ("q4_1", oracle.Q4_1), ("q5_0", oracle.Q5_0), ("q5_1", oracle.Q5_1),
                                         ("q4_k", oracle.Q4_K), ("q5_k", oracle.Q5_K), ("q6_k", oracle.Q6_K), ("q8_0", oracle.Q8_0)])
 def test_ggml_written_blocks_decode_to_ggml_rows(ggml_encode, name, dtype):
     f = ggml_encode["formats"][name]
