@@ -42,6 +42,7 @@ extern "C" {
 #define LK_TYPE_Q5_K 13
 #define LK_TYPE_Q6_K 14
 #define LK_TYPE_IQ4_NL 20
+#define LK_TYPE_IQ4_XS 23
 #define LK_TYPE_BF16 30
 #define LK_TYPE_MXFP4 39
 
@@ -74,7 +75,7 @@ int lk_quantize_q8_1(const void* x, int x_type, void* vy, int kx, int kx_padded,
 
 /* dst[j, row] = weight row `row` . activation row j, j < batch (1..8).
  *   wtype          LK_TYPE_Q4_K | LK_TYPE_Q5_K | LK_TYPE_Q6_K | LK_TYPE_Q8_0, and (this launcher and
- *                  lk_mmvq_subdots only) the 32-value nibble formats LK_TYPE_Q4_0 | Q4_1 | Q5_0 | Q5_1 | IQ4_NL | MXFP4 and Q2_K | Q3_K
+ *                  lk_mmvq_subdots only) the 32-value nibble formats LK_TYPE_Q4_0 | Q4_1 | Q5_0 | Q5_1 | IQ4_NL | MXFP4 and Q2_K | Q3_K | IQ4_XS
  *   vx             nrows_x rows of ncols_x / block_len blocks
  *   vy_q8_1        batch rows of Q8_1 blocks, `stride_col_y` blocks apart (k_padded / 32)
  *   dst            `dst_type` LK_TYPE_F32 | F16 | BF16, rows `stride_col_dst` elements apart

@@ -509,7 +509,7 @@ extern "C" void* lkh_gguf_linear(void* g, const char* name, int device, void* st
     }
     const bool nibble32 = t.dtype == LK_TYPE_Q4_0 || t.dtype == LK_TYPE_Q4_1 || t.dtype == LK_TYPE_Q5_0 ||
                           t.dtype == LK_TYPE_Q5_1 || t.dtype == LK_TYPE_IQ4_NL || t.dtype == LK_TYPE_MXFP4 ||
-                          t.dtype == LK_TYPE_Q2_K || t.dtype == LK_TYPE_Q3_K;   // (the mat-vec-only formats)
+                          t.dtype == LK_TYPE_Q2_K || t.dtype == LK_TYPE_Q3_K || t.dtype == LK_TYPE_IQ4_XS;   // (the mat-vec-only formats)
     if (!nibble32 && t.dtype != LK_TYPE_Q4_K && t.dtype != LK_TYPE_Q5_K && t.dtype != LK_TYPE_Q6_K && t.dtype != LK_TYPE_Q8_0) {
         put_error(err, err_len, "QKernelMatMul: block type " + std::to_string(t.dtype) + " is not served on the card");
         return nullptr;

@@ -101,7 +101,8 @@ void mark_used(Slot& slot, hipStream_t stream) {
 // the row count.
 bool matvec_only(int dtype) {
     return dtype == LK_TYPE_Q4_0 || dtype == LK_TYPE_Q4_1 || dtype == LK_TYPE_Q5_0 || dtype == LK_TYPE_Q5_1 ||
-           dtype == LK_TYPE_IQ4_NL || dtype == LK_TYPE_MXFP4 || dtype == LK_TYPE_Q2_K || dtype == LK_TYPE_Q3_K;
+           dtype == LK_TYPE_IQ4_NL || dtype == LK_TYPE_MXFP4 || dtype == LK_TYPE_Q2_K || dtype == LK_TYPE_Q3_K ||
+           dtype == LK_TYPE_IQ4_XS;
 }
 
 bool tiled_serves(int dtype, int k) {
@@ -128,7 +129,7 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     if (x_type != LK_TYPE_F32 && x_type != LK_TYPE_F16 && x_type != LK_TYPE_BF16) return LK_ERR_TYPE;
     if (rows == 0) return LK_OK;
     if (!x || !out || !blob_ || rows < 0 || n_ <= 0 || k_ <= 0) return LK_ERR_ARG;
-    const int block_len = dtype_ == LK_TYPE_Q8_0 || (plain && dtype_ != LK_TYPE_Q2_K && dtype_ != LK_TYPE_Q3_K) ? 32 : 256;
+    const int block_len = dtype_ == LK_TYPE_Q8_0 || (plain && dtype_ != LK_TYPE_Q2_K && dtype_ != LK_TYPE_Q3_K && dtype_ != LK_TYPE_IQ4_XS) ? 32 : 256;
     if (k_ % block_len != 0) return LK_ERR_ARG;
     int current = -1;
     if (hipGetDevice(&current) != hipSuccess || current != device_) {

@@ -1,5 +1,5 @@
 // Mat-vec for the 32-value nibble formats Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, MXFP4 and the two-bit
-// K-quants Q2_K, Q3_K against Q8_1 activation rows.
+// K-quants Q2_K, Q3_K (and IQ4_XS) against Q8_1 activation rows.
 //
 // Formats as loken states them (src/tensor/quant_cpu/format/q4_0.rs, q4_1.rs, q5_0.rs, q5_1.rs): byte
 // j of `qs` holds value j in its low nibble and value j + 16 in its high one; the five-bit formats
@@ -169,6 +169,9 @@ __global__ __launch_bounds__(64) void subdots_legacy_kernel(const uint8_t* __res
 // d * (six-bit scale - 32) * (q - 4 * !h). Combined as the reference's mat-vec combines them
 // (cuda/moe/gguf.cuh:524-546, 937-959). A lane owns one Q8_1 block of the row; eight lanes share a
 // super-block (and re-read its header bytes from cache). The plain statement, as above.
+// IQ4_XS {d, scales_h, scales_l[4], qs[128]} (136 bytes, iq4_xs.rs:5-37) rides the same kernel: run
+// j = bytes 16 j .. + 16 of qs as IQ4_NL levels (low nibbles values 0..15, high 16..31), one
+// six-bit scale less 32 for the run.
 // ---------------------------------------------------------------------------------------------
 struct LowbitBlock {
     uint4 lo, hi;         // the block's codes 0..3, values 0..15 and 16..31
@@ -180,6 +183,21 @@ struct LowbitBlock {
 template <int ID>
 static __device__ __forceinline__ LowbitBlock lowbit_block(const uint8_t* __restrict__ bp, int j) {
     LowbitBlock r;
+    if (ID == 23) {
+        const uint4 q = *(const uint4_a4*)(bp + 8 + 16 * j);
+        r.lo = make_uint4(levels_of<1>(q.x & 0x0F0F0F0Fu), levels_of<1>(q.y & 0x0F0F0F0Fu), levels_of<1>(q.z & 0x0F0F0F0Fu),
+                          levels_of<1>(q.w & 0x0F0F0F0Fu));
+        r.hi = make_uint4(levels_of<1>((q.x >> 4) & 0x0F0F0F0Fu), levels_of<1>((q.y >> 4) & 0x0F0F0F0Fu),
+                          levels_of<1>((q.z >> 4) & 0x0F0F0F0Fu), levels_of<1>((q.w >> 4) & 0x0F0F0F0Fu));
+        const uint32_t low = ((uint32_t)bp[4 + (j >> 1)] >> (4 * (j & 1))) & 15u;
+        const uint32_t high = ((uint32_t)*(const uint16_t*)(bp + 2) >> (2 * j)) & 3u;
+        r.sc0 = r.sc1 = (int)(low | (high << 4)) - 32;
+        r.mn0 = r.mn1 = 0;
+        r.d = f16_bits_to_f32(*(const uint16_t*)bp);
+        r.dmin = 0.f;
+        r.nlo = r.nhi = make_uint4(0, 0, 0, 0);
+        return r;
+    }
     const int shift = 2 * (j & 3);
     const uint8_t* qs = bp + (ID == 10 ? 16 : 32) + 32 * (j >> 2);
     const uint4 q0 = *(const uint4_a2*)qs, q1 = *(const uint4_a2*)(qs + 16);
@@ -220,9 +238,11 @@ static __device__ __forceinline__ void lowbit_dots(const LowbitBlock& w, const u
         const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
         sum0 = dot16(ones, a_lo, 0);
         sum1 = dot16(ones, a_hi, 0);
-    } else {
+    } else if (ID == 11) {
         dot0 -= 4 * dot16(w.nlo, a_lo, 0);
         dot1 -= 4 * dot16(w.nhi, a_hi, 0);
+        sum0 = sum1 = 0;
+    } else {
         sum0 = sum1 = 0;
     }
 }
@@ -231,7 +251,7 @@ template <int ID, int B, typename T>
 __global__ __launch_bounds__(LWG) void mmvq_lowbit_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
                                                           T* __restrict__ dst, const float* __restrict__ bias, int nb, int n,
                                                           int stride_col_y, int stride_col_dst) {
-    constexpr int BYTES = ID == 10 ? 84 : 110;
+    constexpr int BYTES = ID == 10 ? 84 : ID == 11 ? 110 : 136;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int k32 = nb * 8;
@@ -264,12 +284,16 @@ __global__ __launch_bounds__(LWG) void mmvq_lowbit_kernel(const uint8_t* __restr
 template <int ID>
 __global__ __launch_bounds__(64) void subdots_lowbit_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
                                                             int32_t* __restrict__ dots, int nb) {
-    constexpr int BYTES = ID == 10 ? 84 : 110;
+    constexpr int BYTES = ID == 10 ? 84 : ID == 11 ? 110 : 136;
     const int row = blockIdx.y, idx = blockIdx.x * 64 + threadIdx.x;
     if (idx >= nb * 8) return;
     const LowbitBlock w = lowbit_block<ID>(vx + ((size_t)row * nb + (idx >> 3)) * BYTES, idx & 7);
     int dot0, dot1, sum0, sum1;
     lowbit_dots<ID>(w, vy + (size_t)idx * Q81_BYTES, dot0, dot1, sum0, sum1);
+    if (ID == 23) {   // one integer per run of 32
+        dots[(size_t)row * nb * 8 + idx] = dot0 + dot1;
+        return;
+    }
     int32_t* out = dots + (size_t)row * nb * 16 + 2 * idx;
     out[0] = dot0;
     out[1] = dot1;
@@ -279,7 +303,7 @@ template <int ID, int B, typename T>
 static int launch(const void* vx, const void* vy, void* dst, const float* bias, int nb, int n, int stride_col_y,
                   int stride_col_dst, hipStream_t s) {
     const int need = (n + LWAVES - 1) / LWAVES, cap = lk_device().cus * 8;
-    if constexpr (ID == 10 || ID == 11)
+    if constexpr (ID == 10 || ID == 11 || ID == 23)
         hipLaunchKernelGGL((mmvq_lowbit_kernel<ID, B, T>), dim3(need < cap ? need : cap), dim3(LWG), 0, s, (const uint8_t*)vx,
                            (const uint8_t*)vy, (T*)dst, bias, nb, n, stride_col_y, stride_col_dst);
     else
@@ -320,14 +344,15 @@ static int by_type(int dst_type, int batch, const void* vx, const void* vy, void
 
 bool lk_is_legacy_type(int wtype) {
     return wtype == LK_TYPE_Q4_0 || wtype == LK_TYPE_Q4_1 || wtype == LK_TYPE_Q5_0 || wtype == LK_TYPE_Q5_1 ||
-           wtype == LK_TYPE_IQ4_NL || wtype == LK_TYPE_MXFP4 || wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K;
+           wtype == LK_TYPE_IQ4_NL || wtype == LK_TYPE_MXFP4 || wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K ||
+           wtype == LK_TYPE_IQ4_XS;
 }
 
 // lk_mmvq for the 32-value nibble formats (the caller has told them apart with lk_is_legacy_type).
 int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, int dst_type, int ncols_x, int nrows_x,
                    int batch, int stride_col_y, int stride_col_dst, const float* bias, hipStream_t s) {
     if (nrows_x == 0) return LK_OK;
-    const int block_len = wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K ? 256 : 32;
+    const int block_len = wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K || wtype == LK_TYPE_IQ4_XS ? 256 : 32;
     if (!vx || !vy_q8_1 || !dst || ncols_x <= 0 || ncols_x % block_len != 0 || nrows_x < 0) return LK_ERR_ARG;
     if (batch < 1 || batch > 8 || stride_col_y < ncols_x / 32 || stride_col_dst < nrows_x) return LK_ERR_ARG;
     if ((wtype != LK_TYPE_MXFP4 && ((uintptr_t)vx & 1) != 0) || ((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
@@ -335,6 +360,7 @@ int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, in
     switch (wtype) {
         case LK_TYPE_Q2_K: return by_type<10>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q3_K: return by_type<11>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_IQ4_XS: return by_type<23>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q4_0: return by_type<2>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q4_1: return by_type<3>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q5_0: return by_type<6>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
@@ -349,12 +375,14 @@ int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32
                            hipStream_t s) {
     if (!vx || !vy_q8_1 || !dots || ncols_x <= 0 || ncols_x % 32 != 0 || nrows_x <= 0 || nrows_x > 65535) return LK_ERR_ARG;
     const uint8_t *w = (const uint8_t*)vx, *y = (const uint8_t*)vy_q8_1;
-    if (wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K) {   // sixteen sub-block integers per super-block
+    if (wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K || wtype == LK_TYPE_IQ4_XS) {
+        // sixteen sub-block integers per super-block (IQ4_XS: eight, one per run of 32)
         if (ncols_x % 256 != 0) return LK_ERR_ARG;
         const int nbk = ncols_x / 256;
         const dim3 gridk((nbk * 8 + 63) / 64, nrows_x);
         if (wtype == LK_TYPE_Q2_K) hipLaunchKernelGGL(subdots_lowbit_kernel<10>, gridk, dim3(64), 0, s, w, y, dots, nbk);
-        else hipLaunchKernelGGL(subdots_lowbit_kernel<11>, gridk, dim3(64), 0, s, w, y, dots, nbk);
+        else if (wtype == LK_TYPE_Q3_K) hipLaunchKernelGGL(subdots_lowbit_kernel<11>, gridk, dim3(64), 0, s, w, y, dots, nbk);
+        else hipLaunchKernelGGL(subdots_lowbit_kernel<23>, gridk, dim3(64), 0, s, w, y, dots, nbk);
         return lk_launch_status();
     }
     const int nb = ncols_x / 32;

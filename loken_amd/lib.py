@@ -16,6 +16,7 @@ TYPE_F32, TYPE_F16, TYPE_BF16 = 0, 1, 30
 TYPE_Q4_0, TYPE_Q4_1, TYPE_Q5_0, TYPE_Q5_1 = 2, 3, 6, 7
 TYPE_IQ4_NL, TYPE_MXFP4 = 20, 39
 TYPE_Q2_K, TYPE_Q3_K = 10, 11
+TYPE_IQ4_XS = 23
 TYPE_Q8_0, TYPE_Q8_1, TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K = 8, 9, 12, 13, 14
 
 

@@ -148,7 +148,7 @@ def check(rc, what):
 # ---------------------------------------------------------------------------- gemv (any format)
 WTYPES = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
           "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "q8_0": lib.TYPE_Q8_0, "q4_k": lib.TYPE_Q4_K,
-          "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K}
+          "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "iq4_xs": lib.TYPE_IQ4_XS}
 
 
 def gemv(args, dev):

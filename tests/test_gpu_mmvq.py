@@ -151,7 +151,7 @@ def test_legacy_matvec_within_the_reference_envelope(name):
     assert (np.abs(oracle.oa_matmul(wtype, x, w, n) - truth) <= envelope).all()
 
 
-LOWBIT = {"q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K}
+LOWBIT = {"q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "iq4_xs": lib.TYPE_IQ4_XS}
 
 
 @pytest.mark.parametrize("name", sorted(LOWBIT))
