@@ -188,6 +188,9 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
             d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q4K_BYTES;
             return d.nb <= 8 ? launch_mode<EngQ4KShort, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s)
                              : launch_mode<EngQ4K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
+        case 4:
+            d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q5K_BYTES;
+            return launch_mode<EngQ5K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 5:
             d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q6K_BYTES;
             return launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
@@ -197,7 +200,7 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
 }
 
 static int block_len_of_wire(int quant_type) {
-    return quant_type == 0 ? 32 : (quant_type == 1 || quant_type == 5) ? 256 : 0;
+    return quant_type == 0 ? 32 : (quant_type == 1 || quant_type == 4 || quant_type == 5) ? 256 : 0;
 }
 
 static bool bad_shape(int quant_type, int num_experts, int topk, int size_m, int size_n, int size_k) {

@@ -129,7 +129,7 @@ class MmqRouting:
 
 # ------------------------------------------------------------------------------------ decode
 # loken's wire ids for the MoE decode launchers (EXPERT_QUANT_CODES, cuda/moe/gguf.cuh:55-71)
-EXPERT_QUANT_CODES = {_lib.TYPE_Q8_0: 0, _lib.TYPE_Q4_K: 1, _lib.TYPE_Q6_K: 5}
+EXPERT_QUANT_CODES = {_lib.TYPE_Q8_0: 0, _lib.TYPE_Q4_K: 1, _lib.TYPE_Q5_K: 4, _lib.TYPE_Q6_K: 5}
 
 
 class ExpertRouting:

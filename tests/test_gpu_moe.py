@@ -201,7 +201,7 @@ def slot_order(h_sorted, ids):
 
 @pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(1, 2048, 768, 128, 8), (3, 512, 256, 6, 2),
                                                              (16, 1024, 768, 32, 4)])
-@pytest.mark.parametrize("dt_down", [lib.TYPE_Q4_K, lib.TYPE_Q6_K])
+@pytest.mark.parametrize("dt_down", [lib.TYPE_Q4_K, lib.TYPE_Q5_K, lib.TYPE_Q6_K])
 def test_per_pair_decode_block_matches_oracle(tokens, hidden, ffn, n_experts, topk, dt_down):
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=57, dt_down=dt_down)
     want, want_h = oracle.moe_forward(1, lib.TYPE_Q4_K, dt_down, x, gate, up, down, ids, w, n_experts, ffn, want_h=True)
