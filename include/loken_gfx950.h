@@ -76,7 +76,8 @@ int lk_quantize_q8_1(const void* x, int x_type, void* vy, int kx, int kx_padded,
 /* dst[j, row] = weight row `row` . activation row j, j < batch (1..8).
  *   wtype          LK_TYPE_Q4_K | LK_TYPE_Q5_K | LK_TYPE_Q6_K | LK_TYPE_Q8_0, and (this launcher and
  *                  lk_mmvq_subdots only) the 32-value nibble formats LK_TYPE_Q4_0 | Q4_1 | Q5_0 | Q5_1 | IQ4_NL | MXFP4 and Q2_K | Q3_K | IQ4_XS
- *   vx             nrows_x rows of ncols_x / block_len blocks
+ *   vx             nrows_x rows of ncols_x / block_len blocks (Q4_K / Q5_K 16-byte aligned, Q2_K / IQ4_XS
+ *                  4-byte, MXFP4 any address, every other format 2-byte; else LK_ERR_ARG)
  *   vy_q8_1        batch rows of Q8_1 blocks, `stride_col_y` blocks apart (k_padded / 32)
  *   dst            `dst_type` LK_TYPE_F32 | F16 | BF16, rows `stride_col_dst` elements apart
  *   bias           nullable f32[nrows_x], added in the store

@@ -21,9 +21,11 @@
 // Shape: a wave owns a weight row; its lanes walk the row's blocks 64 at a time (consecutive lanes
 // read consecutive 18..24-byte blocks, so a wave's loads cover one contiguous run), each lane forms
 // its block's integers against every activation row of the batch and the wave folds once per row.
-// The activation blocks come straight from memory: a row of them is a few KB and stays in cache.
-// These formats are the long tail of the reference's table; this kernel is the plain statement,
-// without the LDS staging and register pipelines of the K-quant engines.
+// The workgroup first copies the activation rows into LDS (codes in two planes of 16-byte halves,
+// scales as f32, the halves' code sums as integers), so the load unit carries weight bytes only: a
+// two-bit format has four activation bytes to the weight byte. Rows too long for 48 KB of LDS are
+// read from memory block by block instead. These formats are the long tail of the reference's
+// table; the kernels are plain statements without the register pipelines of the K-quant engines.
 
 #include "lk_common.h"
 
@@ -100,22 +102,73 @@ static __device__ __forceinline__ void block_codes(const uint8_t* __restrict__ b
     }
 }
 
-// The block's integer against one Q8_1 block: sum (code - bias) * a, and the sum of a.
-static __device__ __forceinline__ void block_dot(const uint4& lo, const uint4& hi, const uint8_t* __restrict__ yb, int bias,
-                                                 int& dot, int& asum) {
-    const uint4 a_lo = *(const uint4_a4*)(yb + 4), a_hi = *(const uint4_a4*)(yb + 20);
+// One Q8_1 block of the activation as the dots take it: the two halves of its codes, its scale and
+// the integer sums of the halves.
+struct ActBlock {
+    uint4 lo, hi;
+    float d8;
+    int sum0, sum1;
+};
+
+static __device__ __forceinline__ ActBlock act_from_memory(const uint8_t* __restrict__ yb) {
+    ActBlock a;
+    a.lo = *(const uint4_a4*)(yb + 4);
+    a.hi = *(const uint4_a4*)(yb + 20);
+    a.d8 = f16_bits_to_f32(*(const uint16_t*)yb);
     const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
-    asum = dot16(ones, a_hi, dot16(ones, a_lo, 0));
-    dot = dot16(hi, a_hi, dot16(lo, a_lo, 0)) - bias * asum;
+    a.sum0 = dot16(ones, a.lo, 0);
+    a.sum1 = dot16(ones, a.hi, 0);
+    return a;
 }
 
-template <int ID, int B, typename T>
+// LDS copy of `batch` activation rows of `k32` blocks: plane of low halves, plane of high halves
+// (16 bytes per block each, so consecutive lanes read consecutive 16-byte slots), the scales as
+// f32, the two sums packed as 16-bit halves of a dword (|sum| <= 16 * 127).
+constexpr int ACT_LDS_PER_BLOCK = 40;
+
+static __device__ __forceinline__ void stage_acts(uint8_t* lds, const uint8_t* __restrict__ vy, int batch, int k32,
+                                                  int stride_col_y) {
+    const int total = batch * k32;
+    for (int i = threadIdx.x; i < total; i += LWG) {
+        const int c = i / k32, b = i - c * k32;
+        const ActBlock a = act_from_memory(vy + ((size_t)c * stride_col_y + b) * Q81_BYTES);
+        ((uint4*)lds)[i] = a.lo;
+        ((uint4*)lds)[total + i] = a.hi;
+        ((float*)(lds + (size_t)total * 32))[i] = a.d8;
+        ((int*)(lds + (size_t)total * 36))[i] = (a.sum0 & 0xFFFF) | (a.sum1 << 16);
+    }
+    __syncthreads();
+}
+
+template <bool STAGED>
+static __device__ __forceinline__ ActBlock act_block(const uint8_t* lds, const uint8_t* __restrict__ vy, int total, int k32,
+                                                     int stride_col_y, int c, int b) {
+    if (!STAGED) return act_from_memory(vy + ((size_t)c * stride_col_y + b) * Q81_BYTES);
+    const int i = c * k32 + b;
+    ActBlock a;
+    a.lo = ((const uint4*)lds)[i];
+    a.hi = ((const uint4*)lds)[total + i];
+    a.d8 = ((const float*)(lds + (size_t)total * 32))[i];
+    const int packed = ((const int*)(lds + (size_t)total * 36))[i];
+    a.sum0 = (packed << 16) >> 16;
+    a.sum1 = packed >> 16;
+    return a;
+}
+
+// The block's integer against one Q8_1 block: sum (code - bias) * a.
+static __device__ __forceinline__ int block_dot(const uint4& lo, const uint4& hi, const ActBlock& a, int bias) {
+    return dot16(hi, a.hi, dot16(lo, a.lo, 0)) - bias * (a.sum0 + a.sum1);
+}
+
+template <int ID, int B, typename T, bool STAGED>
 __global__ __launch_bounds__(LWG) void mmvq_legacy_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
                                                           T* __restrict__ dst, const float* __restrict__ bias, int nb, int n,
                                                           int stride_col_y, int stride_col_dst) {
     using F = Legacy<ID>;
+    extern __shared__ __align__(16) uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (STAGED) stage_acts(lds, vy, B, nb, stride_col_y);
     for (int row = blockIdx.x * LWAVES + wave; row < n; row += gridDim.x * LWAVES) {
         const uint8_t* wrow = vx + (size_t)row * nb * F::BYTES;
         float acc[B];
@@ -129,12 +182,9 @@ __global__ __launch_bounds__(LWG) void mmvq_legacy_kernel(const uint8_t* __restr
             const float m = F::M_AT >= 0 ? f16_bits_to_f32(*(const uint16_t*)(bp + (F::M_AT >= 0 ? F::M_AT : 0))) : 0.f;
 #pragma unroll
             for (int c = 0; c < B; ++c) {
-                const uint8_t* yb = vy + ((size_t)c * stride_col_y + b) * Q81_BYTES;
-                const float d8 = f16_bits_to_f32(*(const uint16_t*)yb);
-                int dot, asum;
-                block_dot(lo, hi, yb, F::BIAS, dot, asum);
-                float part = d * d8 * (float)dot;
-                if (F::M_AT >= 0) part += m * (d8 * (float)asum);
+                const ActBlock a = act_block<STAGED>(lds, vy, B * nb, nb, stride_col_y, c, b);
+                float part = d * a.d8 * (float)block_dot(lo, hi, a, F::BIAS);
+                if (F::M_AT >= 0) part += m * (a.d8 * (float)(a.sum0 + a.sum1));
                 acc[c] += part;
             }
         }
@@ -155,9 +205,7 @@ __global__ __launch_bounds__(64) void subdots_legacy_kernel(const uint8_t* __res
     if (b >= nb) return;
     uint4 lo, hi;
     block_codes<F>(vx + ((size_t)row * nb + b) * F::BYTES, lo, hi);
-    int dot, asum;
-    block_dot(lo, hi, vy + (size_t)b * Q81_BYTES, F::BIAS, dot, asum);
-    dots[(size_t)row * nb + b] = dot;
+    dots[(size_t)row * nb + b] = block_dot(lo, hi, act_from_memory(vy + (size_t)b * Q81_BYTES), F::BIAS);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -180,6 +228,22 @@ struct LowbitBlock {
     float d, dmin;
 };
 
+// 32 bytes at a 2-byte-aligned address, made from the enclosing dwords like a Run16: two 16-byte
+// loads and the dword that holds the run's last two bytes. Q3_K's 110-byte super-blocks put every
+// other one two bytes off a dword, and its mat-vec ran at half the rate of Q2_K's on 16-byte loads
+// from such addresses.
+static __device__ __forceinline__ void load_run32(const uint8_t* p, uint4& lo, uint4& hi) {
+    const uintptr_t a = (uintptr_t)p;
+    const uint8_t* b = (const uint8_t*)(a & ~(uintptr_t)3);
+    const uint4 x = *(const uint4_a4*)b, y = *(const uint4_a4*)(b + 16);
+    const uint32_t e = *(const uint32_t*)(b + 28 + 2 * (a & 2));
+    const uint32_t sh = 8 * (uint32_t)(a & 3);
+    lo = make_uint4(__builtin_amdgcn_alignbit(x.y, x.x, sh), __builtin_amdgcn_alignbit(x.z, x.y, sh),
+                    __builtin_amdgcn_alignbit(x.w, x.z, sh), __builtin_amdgcn_alignbit(y.x, x.w, sh));
+    hi = make_uint4(__builtin_amdgcn_alignbit(y.y, y.x, sh), __builtin_amdgcn_alignbit(y.z, y.y, sh),
+                    __builtin_amdgcn_alignbit(y.w, y.z, sh), __builtin_amdgcn_alignbit(e, y.w, sh));
+}
+
 template <int ID>
 static __device__ __forceinline__ LowbitBlock lowbit_block(const uint8_t* __restrict__ bp, int j) {
     LowbitBlock r;
@@ -189,37 +253,51 @@ static __device__ __forceinline__ LowbitBlock lowbit_block(const uint8_t* __rest
                           levels_of<1>(q.w & 0x0F0F0F0Fu));
         r.hi = make_uint4(levels_of<1>((q.x >> 4) & 0x0F0F0F0Fu), levels_of<1>((q.y >> 4) & 0x0F0F0F0Fu),
                           levels_of<1>((q.z >> 4) & 0x0F0F0F0Fu), levels_of<1>((q.w >> 4) & 0x0F0F0F0Fu));
-        const uint32_t low = ((uint32_t)bp[4 + (j >> 1)] >> (4 * (j & 1))) & 15u;
-        const uint32_t high = ((uint32_t)*(const uint16_t*)(bp + 2) >> (2 * j)) & 3u;
+        const uint2 head = *(const uint2_a2*)bp;   // d, scales_h | scales_l[4]
+        const uint32_t low = (head.y >> (4 * j)) & 15u;
+        const uint32_t high = (head.x >> (16 + 2 * j)) & 3u;
         r.sc0 = r.sc1 = (int)(low | (high << 4)) - 32;
         r.mn0 = r.mn1 = 0;
-        r.d = f16_bits_to_f32(*(const uint16_t*)bp);
+        r.d = f16_bits_to_f32(head.x & 0xFFFFu);
         r.dmin = 0.f;
         r.nlo = r.nhi = make_uint4(0, 0, 0, 0);
         return r;
     }
     const int shift = 2 * (j & 3);
     const uint8_t* qs = bp + (ID == 10 ? 16 : 32) + 32 * (j >> 2);
-    const uint4 q0 = *(const uint4_a2*)qs, q1 = *(const uint4_a2*)(qs + 16);
+    uint4 q0, q1;
+    if (ID == 11) {
+        load_run32(qs, q0, q1);
+    } else {
+        q0 = *(const uint4_a4*)qs;
+        q1 = *(const uint4_a4*)(qs + 16);
+    }
     r.lo = make_uint4((q0.x >> shift) & 0x03030303u, (q0.y >> shift) & 0x03030303u, (q0.z >> shift) & 0x03030303u, (q0.w >> shift) & 0x03030303u);
     r.hi = make_uint4((q1.x >> shift) & 0x03030303u, (q1.y >> shift) & 0x03030303u, (q1.z >> shift) & 0x03030303u, (q1.w >> shift) & 0x03030303u);
     if (ID == 10) {
-        const uint32_t s0 = bp[2 * j], s1 = bp[2 * j + 1];
-        r.sc0 = s0 & 15; r.mn0 = s0 >> 4; r.sc1 = s1 & 15; r.mn1 = s1 >> 4;
-        r.d = f16_bits_to_f32(*(const uint16_t*)(bp + 80));
-        r.dmin = f16_bits_to_f32(*(const uint16_t*)(bp + 82));
+        const uint32_t sm = *(const uint16_t*)(bp + 2 * j);   // scale | min << 4 of sub-blocks 2 j, 2 j + 1
+        r.sc0 = sm & 15; r.mn0 = (sm >> 4) & 15; r.sc1 = (sm >> 8) & 15; r.mn1 = sm >> 12;
+        const uint32_t dm = *(const uint32_a2*)(bp + 80);
+        r.d = f16_bits_to_f32(dm & 0xFFFFu);
+        r.dmin = f16_bits_to_f32(dm >> 16);
         r.nlo = r.nhi = make_uint4(0, 0, 0, 0);
     } else {
-        const uint4 h0 = *(const uint4_a2*)bp, h1 = *(const uint4_a2*)(bp + 16);
+        uint4 h0, h1;
+        load_run32(bp, h0, h1);
         r.nlo = make_uint4((~h0.x >> j) & 0x01010101u, (~h0.y >> j) & 0x01010101u, (~h0.z >> j) & 0x01010101u, (~h0.w >> j) & 0x01010101u);
         r.nhi = make_uint4((~h1.x >> j) & 0x01010101u, (~h1.y >> j) & 0x01010101u, (~h1.z >> j) & 0x01010101u, (~h1.w >> j) & 0x01010101u);
         // scales 2 j and 2 j + 1 of the sixteen packed in twelve bytes
-        const uint8_t* p = bp + 96;
+        // (scale i: low four bits = nibble i / 8 of byte i % 8, top two = bits 2 (i / 4) of byte 8 + i % 4)
+        const uintptr_t sa = (uintptr_t)(bp + 96);
+        const uint32_t* sb = (const uint32_t*)(sa & ~(uintptr_t)3);
+        const uint32_t x0 = sb[0], x1 = sb[1], x2 = sb[2], x3 = sb[2 + ((sa & 2) >> 1)], sh = 8 * (uint32_t)(sa & 3);
+        const uint32_t w0 = __builtin_amdgcn_alignbit(x1, x0, sh), w1 = __builtin_amdgcn_alignbit(x2, x1, sh),
+                       w2 = __builtin_amdgcn_alignbit(x3, x2, sh);
         const int group = j >> 1, jj = 2 * (j & 1);
-        const uint32_t b0 = p[jj + 4 * (group & 1)], b1 = p[jj + 1 + 4 * (group & 1)];
-        const uint32_t t0 = p[8 + jj], t1 = p[9 + jj];
-        r.sc0 = (int)((group < 2 ? (b0 & 15) : (b0 >> 4)) | (((t0 >> (2 * group)) & 3) << 4)) - 32;
-        r.sc1 = (int)((group < 2 ? (b1 & 15) : (b1 >> 4)) | (((t1 >> (2 * group)) & 3) << 4)) - 32;
+        const uint32_t low = ((group & 1) ? w1 : w0) >> (8 * jj + (group < 2 ? 0 : 4));
+        const uint32_t top = w2 >> (8 * jj + 2 * group);
+        r.sc0 = (int)((low & 15u) | ((top & 3u) << 4)) - 32;
+        r.sc1 = (int)(((low >> 8) & 15u) | (((top >> 8) & 3u) << 4)) - 32;
         r.mn0 = r.mn1 = 0;
         r.d = f16_bits_to_f32(*(const uint16_t*)(bp + 108));
         r.dmin = 0.f;
@@ -227,34 +305,37 @@ static __device__ __forceinline__ LowbitBlock lowbit_block(const uint8_t* __rest
     return r;
 }
 
-// The two sub-block integers of the block against a Q8_1 block, and the two activation sums.
+// The two sub-block integers of the block against a Q8_1 block.
 template <int ID>
-static __device__ __forceinline__ void lowbit_dots(const LowbitBlock& w, const uint8_t* __restrict__ yb, int& dot0, int& dot1,
-                                                   int& sum0, int& sum1) {
-    const uint4 a_lo = *(const uint4_a4*)(yb + 4), a_hi = *(const uint4_a4*)(yb + 20);
-    dot0 = dot16(w.lo, a_lo, 0);
-    dot1 = dot16(w.hi, a_hi, 0);
-    if (ID == 10) {
-        const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
-        sum0 = dot16(ones, a_lo, 0);
-        sum1 = dot16(ones, a_hi, 0);
-    } else if (ID == 11) {
-        dot0 -= 4 * dot16(w.nlo, a_lo, 0);
-        dot1 -= 4 * dot16(w.nhi, a_hi, 0);
-        sum0 = sum1 = 0;
-    } else {
-        sum0 = sum1 = 0;
+static __device__ __forceinline__ void lowbit_dots(const LowbitBlock& w, const ActBlock& a, int& dot0, int& dot1) {
+    dot0 = dot16(w.lo, a.lo, 0);
+    dot1 = dot16(w.hi, a.hi, 0);
+    if (ID == 11) {
+        dot0 -= 4 * dot16(w.nlo, a.lo, 0);
+        dot1 -= 4 * dot16(w.nhi, a.hi, 0);
     }
 }
 
-template <int ID, int B, typename T>
+// The block's share of the row's result.
+template <int ID>
+static __device__ __forceinline__ float lowbit_share(const LowbitBlock& w, const ActBlock& a) {
+    int dot0, dot1;
+    lowbit_dots<ID>(w, a, dot0, dot1);
+    float part = w.d * (a.d8 * (float)(dot0 * w.sc0 + dot1 * w.sc1));
+    if (ID == 10) part -= w.dmin * (a.d8 * (float)(a.sum0 * w.mn0 + a.sum1 * w.mn1));
+    return part;
+}
+
+template <int ID, int B, typename T, bool STAGED>
 __global__ __launch_bounds__(LWG) void mmvq_lowbit_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
                                                           T* __restrict__ dst, const float* __restrict__ bias, int nb, int n,
                                                           int stride_col_y, int stride_col_dst) {
     constexpr int BYTES = ID == 10 ? 84 : ID == 11 ? 110 : 136;
+    extern __shared__ __align__(16) uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int k32 = nb * 8;
+    if (STAGED) stage_acts(lds, vy, B, k32, stride_col_y);
     for (int row = blockIdx.x * LWAVES + wave; row < n; row += gridDim.x * LWAVES) {
         const uint8_t* wrow = vx + (size_t)row * nb * BYTES;
         float acc[B];
@@ -263,15 +344,8 @@ __global__ __launch_bounds__(LWG) void mmvq_lowbit_kernel(const uint8_t* __restr
         for (int idx = lane; idx < k32; idx += 64) {
             const LowbitBlock w = lowbit_block<ID>(wrow + (size_t)(idx >> 3) * BYTES, idx & 7);
 #pragma unroll
-            for (int c = 0; c < B; ++c) {
-                const uint8_t* yb = vy + ((size_t)c * stride_col_y + idx) * Q81_BYTES;
-                const float d8 = f16_bits_to_f32(*(const uint16_t*)yb);
-                int dot0, dot1, sum0, sum1;
-                lowbit_dots<ID>(w, yb, dot0, dot1, sum0, sum1);
-                float part = w.d * (d8 * (float)(dot0 * w.sc0 + dot1 * w.sc1));
-                if (ID == 10) part -= w.dmin * (d8 * (float)(sum0 * w.mn0 + sum1 * w.mn1));
-                acc[c] += part;
-            }
+            for (int c = 0; c < B; ++c)
+                acc[c] += lowbit_share<ID>(w, act_block<STAGED>(lds, vy, B * k32, k32, stride_col_y, c, idx));
         }
 #pragma unroll
         for (int c = 0; c < B; ++c) {
@@ -288,8 +362,8 @@ __global__ __launch_bounds__(64) void subdots_lowbit_kernel(const uint8_t* __res
     const int row = blockIdx.y, idx = blockIdx.x * 64 + threadIdx.x;
     if (idx >= nb * 8) return;
     const LowbitBlock w = lowbit_block<ID>(vx + ((size_t)row * nb + (idx >> 3)) * BYTES, idx & 7);
-    int dot0, dot1, sum0, sum1;
-    lowbit_dots<ID>(w, vy + (size_t)idx * Q81_BYTES, dot0, dot1, sum0, sum1);
+    int dot0, dot1;
+    lowbit_dots<ID>(w, act_from_memory(vy + (size_t)idx * Q81_BYTES), dot0, dot1);
     if (ID == 23) {   // one integer per run of 32
         dots[(size_t)row * nb * 8 + idx] = dot0 + dot1;
         return;
@@ -303,12 +377,22 @@ template <int ID, int B, typename T>
 static int launch(const void* vx, const void* vy, void* dst, const float* bias, int nb, int n, int stride_col_y,
                   int stride_col_dst, hipStream_t s) {
     const int need = (n + LWAVES - 1) / LWAVES, cap = lk_device().cus * 8;
-    if constexpr (ID == 10 || ID == 11 || ID == 23)
-        hipLaunchKernelGGL((mmvq_lowbit_kernel<ID, B, T>), dim3(need < cap ? need : cap), dim3(LWG), 0, s, (const uint8_t*)vx,
-                           (const uint8_t*)vy, (T*)dst, bias, nb, n, stride_col_y, stride_col_dst);
-    else
-        hipLaunchKernelGGL((mmvq_legacy_kernel<ID, B, T>), dim3(need < cap ? need : cap), dim3(LWG), 0, s, (const uint8_t*)vx,
-                           (const uint8_t*)vy, (T*)dst, bias, nb, n, stride_col_y, stride_col_dst);
+    const dim3 grid(need < cap ? need : cap);
+    constexpr bool LOWBIT = ID == 10 || ID == 11 || ID == 23;
+    const int k32 = LOWBIT ? nb * 8 : nb;
+    const size_t lds_bytes = (size_t)B * k32 * ACT_LDS_PER_BLOCK;
+    const auto run = [&](auto kernel, size_t lds) {
+        hipLaunchKernelGGL(kernel, grid, dim3(LWG), lds, s, (const uint8_t*)vx, (const uint8_t*)vy, (T*)dst, bias, nb, n,
+                           stride_col_y, stride_col_dst);
+    };
+    // the activation rows in LDS while they fit the 48 KB every kernel may ask for; from memory beyond
+    if (lds_bytes <= 48 * 1024) {
+        if constexpr (LOWBIT) run(mmvq_lowbit_kernel<ID, B, T, true>, lds_bytes);
+        else run(mmvq_legacy_kernel<ID, B, T, true>, lds_bytes);
+    } else {
+        if constexpr (LOWBIT) run(mmvq_lowbit_kernel<ID, B, T, false>, 0);
+        else run(mmvq_legacy_kernel<ID, B, T, false>, 0);
+    }
     return lk_launch_status();
 }
 
@@ -356,6 +440,8 @@ int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, in
     if (!vx || !vy_q8_1 || !dst || ncols_x <= 0 || ncols_x % block_len != 0 || nrows_x < 0) return LK_ERR_ARG;
     if (batch < 1 || batch > 8 || stride_col_y < ncols_x / 32 || stride_col_dst < nrows_x) return LK_ERR_ARG;
     if ((wtype != LK_TYPE_MXFP4 && ((uintptr_t)vx & 1) != 0) || ((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
+    // super-blocks of 84 and 136 bytes are read with dword-aligned 16-byte loads
+    if ((wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_IQ4_XS) && ((uintptr_t)vx & 3) != 0) return LK_ERR_ARG;
     const int nb = ncols_x / block_len;
     switch (wtype) {
         case LK_TYPE_Q2_K: return by_type<10>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
@@ -377,7 +463,7 @@ int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32
     const uint8_t *w = (const uint8_t*)vx, *y = (const uint8_t*)vy_q8_1;
     if (wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K || wtype == LK_TYPE_IQ4_XS) {
         // sixteen sub-block integers per super-block (IQ4_XS: eight, one per run of 32)
-        if (ncols_x % 256 != 0) return LK_ERR_ARG;
+        if (ncols_x % 256 != 0 || ((uintptr_t)vx & (wtype == LK_TYPE_Q3_K ? 1 : 3)) != 0) return LK_ERR_ARG;
         const int nbk = ncols_x / 256;
         const dim3 gridk((nbk * 8 + 63) / 64, nrows_x);
         if (wtype == LK_TYPE_Q2_K) hipLaunchKernelGGL(subdots_lowbit_kernel<10>, gridk, dim3(64), 0, s, w, y, dots, nbk);
