@@ -291,7 +291,8 @@ void loken_moe_mmq_fold(const float* pairs, const float* weights, const int32_t*
  * cuda/moe/moe_gguf.cu:476-511, 755-860, 1049-1061). sorted_token_ids[i] is the flattened
  * (token * topk + choice) slot of routed pair i, expert_ids[i] its expert; size_m = pairs,
  * size_n = output rows per expert, size_k = reduction length; quant_type is loken's wire id
- * (0 = Q8_0, 1 = Q4_K, 4 = Q5_K, 5 = Q6_K). Weights are stacks [num_experts][size_n][size_k / block].
+ * (0 = Q8_0, 1 = Q4_K, 2 = Q2_K, 3 = Q3_K, 4 = Q5_K, 5 = Q6_K, 6 = Q5_0, 7 = MXFP4, 8 = Q5_1, 9 = IQ4_NL,
+ * 10 = IQ4_XS; the codebook formats 11..15 return LK_ERR_TYPE). Weights are stacks [num_experts][size_n][size_k / block].
  * These launchers quantize the f32 activation themselves into a per-(device, stream)
  * grow-only scratch (the one allocation in this library; growing is refused with
  * LK_ERR_NOMEM while the stream is being captured). Return 0 or an LK_ERR_* code.

@@ -151,6 +151,13 @@ int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, in
                    int batch, int stride_col_y, int stride_col_dst, const float* bias, hipStream_t stream);
 int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32_t* dots, int ncols_x, int nrows_x,
                            hipStream_t stream);
+// MoE decode for the expert formats the K-quant engines do not serve (mmvq_legacy.hip): block length
+// of a wire id (0: not one of them), and the per-pair launch over Q8_1 activation rows.
+int lk_moe_wire_block_len_legacy(int quant_type);
+int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts_q8_1,
+                       const int32_t* sorted_token_ids, const int32_t* expert_ids, const float* topk_weights,
+                       const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
+                       int k32_stride, hipStream_t s);
 
 static inline int lk_launch_status() {
     return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;

@@ -373,6 +373,117 @@ __global__ __launch_bounds__(64) void subdots_lowbit_kernel(const uint8_t* __res
     out[1] = dot1;
 }
 
+// ---------------------------------------------------------------------------------------------
+// MoE decode over these formats: the per-pair mat-vec of loken's expert launchers
+// (cuda/moe/moe_gguf.cu:476-511, 755-860, 1049-1061) for the rows of its format table that the
+// K-quant engines do not serve. Workgroups (x, pair): the pair's Q8_1 row goes to LDS once, each
+// wave then takes weight rows of the pair's expert. MODE 0: out = w . x (times the routing weight
+// when given), 1: silu(gate . x) * (up . x), 2: routing weight * (w . x + bias).
+// ---------------------------------------------------------------------------------------------
+struct MoeLegacyDims {
+    int experts, topk, pairs, cols, nb, k32, k32_stride;
+    int64_t slab_bytes;
+};
+
+// A lane's share of one weight row against the activation row in LDS.
+template <int ID>
+static __device__ __forceinline__ float staged_row_share(const uint8_t* __restrict__ wrow, int nb, const uint8_t* lds,
+                                                         int k32, int lane) {
+    float acc = 0.f;
+    if constexpr (ID == 10 || ID == 11 || ID == 23) {
+        constexpr int BYTES = ID == 10 ? 84 : ID == 11 ? 110 : 136;
+        for (int idx = lane; idx < k32; idx += 64) {
+            const LowbitBlock w = lowbit_block<ID>(wrow + (size_t)(idx >> 3) * BYTES, idx & 7);
+            acc += lowbit_share<ID>(w, act_block<true>(lds, nullptr, k32, k32, 0, 0, idx));
+        }
+    } else {
+        using F = Legacy<ID>;
+        for (int b = lane; b < nb; b += 64) {
+            const uint8_t* bp = wrow + (size_t)b * F::BYTES;
+            uint4 lo, hi;
+            block_codes<F>(bp, lo, hi);
+            const float d = block_scale<F>(bp);
+            const float m = F::M_AT >= 0 ? f16_bits_to_f32(*(const uint16_t*)(bp + (F::M_AT >= 0 ? F::M_AT : 0))) : 0.f;
+            const ActBlock a = act_block<true>(lds, nullptr, nb, nb, 0, 0, b);
+            float part = d * a.d8 * (float)block_dot(lo, hi, a, F::BIAS);
+            if (F::M_AT >= 0) part += m * (a.d8 * (float)(a.sum0 + a.sum1));
+            acc += part;
+        }
+    }
+    return acc;
+}
+
+template <int ID> struct BytesOf { static constexpr int V = Legacy<ID>::BYTES; };
+template <> struct BytesOf<10> { static constexpr int V = 84; };
+template <> struct BytesOf<11> { static constexpr int V = 110; };
+template <> struct BytesOf<23> { static constexpr int V = 136; };
+
+template <int ID, int MODE>
+__global__ __launch_bounds__(LWG) void moe_rows_legacy_kernel(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1,
+                                                              const uint8_t* __restrict__ acts,
+                                                              const int32_t* __restrict__ sorted_token_ids,
+                                                              const int32_t* __restrict__ expert_ids,
+                                                              const float* __restrict__ topk_weights,
+                                                              const float* __restrict__ down_bias, float* __restrict__ out,
+                                                              MoeLegacyDims d) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int pair = blockIdx.y;
+    const int slot = sorted_token_ids[pair];
+    const int e = expert_ids[pair];
+    if (slot < 0 || slot >= d.pairs) return;   // the whole workgroup leaves together
+    float* out_row = out + (size_t)slot * d.cols;
+    if (e < 0 || e >= d.experts) {
+        // a pair the routing leaves out adds nothing: its row of the fold's input reads zero
+        if (MODE == 2)
+            for (int r = blockIdx.x * LWG + threadIdx.x; r < d.cols; r += gridDim.x * LWG) out_row[r] = 0.f;
+        return;
+    }
+    const bool own_row = MODE == 2 || (MODE == 0 && topk_weights != nullptr);
+    const int act_row = own_row ? slot : slot / d.topk;
+    stage_acts(lds, acts + (size_t)act_row * d.k32_stride * Q81_BYTES, 1, d.k32, 0);
+    const float scale = (MODE != 1 && topk_weights) ? topk_weights[slot] : 1.0f;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const size_t row_bytes = (size_t)d.nb * BytesOf<ID>::V;
+    const uint8_t* slab0 = w0 + (int64_t)e * d.slab_bytes;
+    for (int row = blockIdx.x * LWAVES + wave; row < d.cols; row += gridDim.x * LWAVES) {
+        const float first = wave_sum(staged_row_share<ID>(slab0 + row * row_bytes, d.nb, lds, d.k32, lane));
+        if (MODE == 1) {
+            const uint8_t* slab1 = w1 + (int64_t)e * d.slab_bytes;
+            const float second = wave_sum(staged_row_share<ID>(slab1 + row * row_bytes, d.nb, lds, d.k32, lane));
+            if (lane == 0) out_row[row] = first / (1.0f + expf(-first)) * second;
+        } else {
+            float v = first * scale;
+            if (MODE == 2 && down_bias) v += scale * down_bias[(size_t)e * d.cols + row];
+            if (lane == 0) out_row[row] = v;
+        }
+    }
+}
+
+template <int ID>
+static int launch_moe(int mode, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts, const int32_t* sti,
+                      const int32_t* eid, const float* tw, const float* bias, float* out, MoeLegacyDims d, hipStream_t s) {
+    constexpr bool LOWBIT = ID == 10 || ID == 11 || ID == 23;
+    d.k32 = LOWBIT ? d.nb * 8 : d.nb;
+    d.slab_bytes = (int64_t)d.cols * d.nb * BytesOf<ID>::V;
+    const size_t lds_bytes = (size_t)d.k32 * ACT_LDS_PER_BLOCK;
+    if (lds_bytes > 48 * 1024 || d.pairs > 65535) return LK_ERR_ARG;
+    const int need = (d.cols + LWAVES - 1) / LWAVES;
+    int share = lk_device().cus * 8 / d.pairs;
+    if (share < 1) share = 1;
+    const dim3 grid(need < share ? need : share, d.pairs);
+    const auto run = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(LWG), lds_bytes, s, w0, w1, acts, sti, eid, tw, bias, out, d);
+    };
+    switch (mode) {
+        case 0: run(moe_rows_legacy_kernel<ID, 0>); break;
+        case 1: run(moe_rows_legacy_kernel<ID, 1>); break;
+        case 2: run(moe_rows_legacy_kernel<ID, 2>); break;
+        default: return LK_ERR_ARG;
+    }
+    return lk_launch_status();
+}
+
 template <int ID, int B, typename T>
 static int launch(const void* vx, const void* vy, void* dst, const float* bias, int nb, int n, int stride_col_y,
                   int stride_col_dst, hipStream_t s) {
@@ -483,4 +594,35 @@ int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32
         default: return LK_ERR_TYPE;
     }
     return lk_launch_status();
+}
+
+// Wire ids of the reference's expert table (src/inference/moe_cuda/gemm.rs:23-39) served here.
+int lk_moe_wire_block_len_legacy(int quant_type) {
+    switch (quant_type) {
+        case 2: case 3: case 10: return 256;       // Q2_K, Q3_K, IQ4_XS
+        case 6: case 7: case 8: case 9: return 32; // Q5_0, MXFP4, Q5_1, IQ4_NL
+        default: return 0;
+    }
+}
+
+int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts_q8_1,
+                       const int32_t* sorted_token_ids, const int32_t* expert_ids, const float* topk_weights,
+                       const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
+                       int k32_stride, hipStream_t s) {
+    const int bl = lk_moe_wire_block_len_legacy(quant_type);
+    if (bl == 0) return LK_ERR_TYPE;
+    if (size_k % bl != 0 || ((uintptr_t)acts_q8_1 & 3) != 0) return LK_ERR_ARG;
+    const uintptr_t both = (uintptr_t)w0 | (uintptr_t)w1;
+    const uintptr_t mask = (quant_type == 2 || quant_type == 10) ? 3 : quant_type == 7 ? 0 : 1;
+    if ((both & mask) != 0) return LK_ERR_ARG;
+    MoeLegacyDims d{experts, topk, pairs, cols, size_k / bl, 0, k32_stride, 0};
+    switch (quant_type) {
+        case 2: return launch_moe<10>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 3: return launch_moe<11>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 6: return launch_moe<6>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 7: return launch_moe<39>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 8: return launch_moe<7>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 9: return launch_moe<20>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        default: return launch_moe<23>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+    }
 }

@@ -195,12 +195,17 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
             d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q6K_BYTES;
             return launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         default:
-            return LK_ERR_TYPE;
+            // Q2_K, Q3_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS: the wave-per-row kernels over Q8_1 rows
+            if (d.act_f32) return LK_ERR_ARG;
+            return lk_moe_rows_legacy(MODE, quant_type, w0, w1, acts, sti, eid, tw, bias, out, d.experts, d.topk,
+                                      d.pairs, d.cols, size_k, d.k32, s);
     }
 }
 
 static int block_len_of_wire(int quant_type) {
-    return quant_type == 0 ? 32 : (quant_type == 1 || quant_type == 4 || quant_type == 5) ? 256 : 0;
+    if (quant_type == 0) return 32;
+    if (quant_type == 1 || quant_type == 4 || quant_type == 5) return 256;
+    return lk_moe_wire_block_len_legacy(quant_type);
 }
 
 static bool bad_shape(int quant_type, int num_experts, int topk, int size_m, int size_n, int size_k) {
@@ -214,7 +219,8 @@ static inline int pad512(int k) { return (k + 511) / 512 * 512; }
 // f32 rows a workgroup can quantize while it stages them (what lk_mmvq_fused asks of its input): a
 // pair's row is a few KB, so reading it as floats costs less than a quantizer launch ahead of the
 // kernel and the scratch round trip between the two.
-static inline bool rows_stage_as_f32(const float* inputs, int size_k) {
+static inline bool rows_stage_as_f32(const float* inputs, int size_k, int quant_type) {
+    if (lk_moe_wire_block_len_legacy(quant_type) != 0) return false;   // those kernels read Q8_1 rows
     return ((uintptr_t)inputs & 15) == 0 && size_k % 4 == 0 && size_k <= 8192;
 }
 
@@ -252,7 +258,7 @@ extern "C" int loken_moe_gemm_gguf(const float* inputs, const void* weights, con
     const int kp = pad512(size_k);
     // with routing weights every entry has its own activation row; without, topk entries share one
     const int act_rows = topk_weights ? size_m : size_m / topk;
-    if (rows_stage_as_f32(inputs, size_k)) {
+    if (rows_stage_as_f32(inputs, size_k, quant_type)) {
         MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k};
         return launch_format<MODE_PLAIN>(quant_type, (const uint8_t*)weights, nullptr, (const uint8_t*)inputs,
                                          sorted_token_ids, expert_ids, topk_weights, nullptr, (float*)outputs, d, size_k, s);
@@ -277,7 +283,7 @@ extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const v
         bad_shape(quant_type, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k), act_rows = size_m / topk;
-    if (rows_stage_as_f32(inputs, size_k)) {
+    if (rows_stage_as_f32(inputs, size_k, quant_type)) {
         MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k};
         return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights,
                                          (const uint8_t*)inputs, sorted_token_ids, expert_ids, nullptr, nullptr, outputs,
@@ -303,7 +309,7 @@ extern "C" int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* 
         bad_shape(gguf_dtype, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k);
-    const bool as_f32 = rows_stage_as_f32(inputs, size_k);
+    const bool as_f32 = rows_stage_as_f32(inputs, size_k, gguf_dtype);
     const size_t act_bytes = as_f32 ? 0 : (((size_t)size_m * (kp / 32) * Q81_BYTES) + 255) & ~(size_t)255;
     const size_t pair_bytes = (size_t)size_m * size_n * sizeof(float);
     std::lock_guard<std::mutex> lock(g_scratch_mu);

@@ -129,7 +129,9 @@ class MmqRouting:
 
 # ------------------------------------------------------------------------------------ decode
 # loken's wire ids for the MoE decode launchers (EXPERT_QUANT_CODES, cuda/moe/gguf.cuh:55-71)
-EXPERT_QUANT_CODES = {_lib.TYPE_Q8_0: 0, _lib.TYPE_Q4_K: 1, _lib.TYPE_Q5_K: 4, _lib.TYPE_Q6_K: 5}
+EXPERT_QUANT_CODES = {_lib.TYPE_Q8_0: 0, _lib.TYPE_Q4_K: 1, _lib.TYPE_Q2_K: 2, _lib.TYPE_Q3_K: 3, _lib.TYPE_Q5_K: 4,
+                      _lib.TYPE_Q6_K: 5, _lib.TYPE_Q5_0: 6, _lib.TYPE_MXFP4: 7, _lib.TYPE_Q5_1: 8, _lib.TYPE_IQ4_NL: 9,
+                      _lib.TYPE_IQ4_XS: 10}
 
 
 class ExpertRouting:

@@ -29,8 +29,8 @@ def assert_close(got, want, rtol=RTOL, atol=ATOL):
     assert not bad.any(), f"{bad.sum()} of {bad.size} outside tolerance; worst {np.abs(got - want).max()}"
 
 
-def make_layer(tokens, hidden, ffn, n_experts, topk, seed, dt_down=lib.TYPE_Q4_K, x_scale=30.0):
-    dt = lib.TYPE_Q4_K
+def make_layer(tokens, hidden, ffn, n_experts, topk, seed, dt_down=lib.TYPE_Q4_K, x_scale=30.0, dt_gu=lib.TYPE_Q4_K):
+    dt = dt_gu
     gate = synth.weight(dt, n_experts * ffn, hidden, seed=seed, stream=1)
     up = synth.weight(dt, n_experts * ffn, hidden, seed=seed, stream=2)
     down = synth.weight(dt_down, n_experts * hidden, ffn, seed=seed, stream=3)
@@ -217,6 +217,53 @@ def test_per_pair_decode_block_matches_oracle(tokens, hidden, ffn, n_experts, to
     assert (np.abs(out.cpu().numpy() - want) <= 2e-3 * np.abs(want) + 2e-4 * scale).all()
 
 
+# the rows of the reference's expert table (src/inference/moe_cuda/gemm.rs:23-39) beyond the K-quant engines
+TABLE_TAIL = {"q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "q5_0": lib.TYPE_Q5_0, "mxfp4": lib.TYPE_MXFP4,
+              "q5_1": lib.TYPE_Q5_1, "iq4_nl": lib.TYPE_IQ4_NL, "iq4_xs": lib.TYPE_IQ4_XS}
+
+
+@pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(1, 1024, 768, 16, 4), (3, 512, 256, 6, 2)])
+@pytest.mark.parametrize("name", sorted(TABLE_TAIL))
+def test_per_pair_decode_block_in_the_tail_formats_matches_oracle(name, tokens, hidden, ffn, n_experts, topk):
+    dt = TABLE_TAIL[name]
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=61, dt_down=dt, dt_gu=dt, x_scale=4.0)
+    want, want_h = oracle.moe_forward(1, dt, dt, x, gate, up, down, ids, w, n_experts, ffn, want_h=True)
+    routing = ExpertRouting(dev(ids))
+    h = moe_gemm_gguf_gate_up_silu_mul(dt, dev(x), dev(gate), dev(up), routing, n_experts, ffn)
+    want_slot = slot_order(want_h, ids)
+    assert (np.abs(h.cpu().numpy() - want_slot) <= 1e-3 * np.abs(want_slot) + 1e-4 * np.abs(want_slot).max()).all()
+    # down from the oracle's own intermediate rows, so the two stages are checked apart
+    bias = torch.randn((n_experts, hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(7))
+    out = moe_gemm_gguf_down_reduce(dt, dev(want_slot), dev(down), routing, dev(w.reshape(-1)), n_experts, hidden)
+    scale = np.abs(want).max()
+    assert (np.abs(out.cpu().numpy() - want) <= 1e-3 * np.abs(want) + 1e-4 * scale).all()
+    with_bias = moe_gemm_gguf_down_reduce(dt, dev(want_slot), dev(down), routing, dev(w.reshape(-1)), n_experts, hidden,
+                                          down_bias=bias)
+    add = (dev(w).unsqueeze(-1) * bias[dev(ids).long()]).sum(1)
+    assert (with_bias - (out + add)).abs().max().item() <= 1e-5 * (scale + add.abs().max().item())
+    # the plain launcher over the same pairs: the gate product alone
+    plain = moe_gemm_gguf(dt, dev(x), dev(gate), routing, n_experts, ffn)
+    slots, experts = oracle.group_by_expert(ids)
+    gate_rows = gate.reshape(n_experts, ffn, -1)
+    for j in range(len(slots)):
+        want_row = oracle.ob_matmul(dt, x[slots[j] // topk][None, :], gate_rows[experts[j]].reshape(-1), ffn)[0]
+        got_row = plain[slots[j]].cpu().numpy()
+        assert (np.abs(got_row - want_row) <= 1e-3 * np.abs(want_row) + 1e-4 * np.abs(want_row).max()).all()
+
+
+def test_decode_launchers_refuse_the_codebook_formats():
+    tokens, hidden, ffn, n_experts, topk = 2, 512, 256, 4, 2
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=62)
+    routing = ExpertRouting(dev(ids))
+    L = lib.load()
+    out = torch.empty((tokens * topk, ffn), device="cuda")
+    for wire in (11, 12, 13, 14, 15, 16, -1):
+        rc = L.loken_moe_gemm_gguf(dev(x).data_ptr(), dev(gate).data_ptr(), routing.sorted_token_ids.data_ptr(),
+                                   routing.expert_ids.data_ptr(), None, out.data_ptr(), n_experts, topk,
+                                   tokens * topk, ffn, hidden, wire, None)
+        assert rc == lib.LK_ERR_TYPE
+
+
 def test_decode_down_reduce_is_tight_on_oracle_rows_and_folds_in_slot_order():
     tokens, hidden, ffn, n_experts, topk = 4, 512, 512, 8, 3
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=58)
@@ -278,7 +325,7 @@ def test_launchers_report_bad_arguments_and_formats():
     l = lib.load()
     buf = torch.zeros(4096, dtype=torch.uint8, device="cuda")
     p, s = buf.data_ptr(), torch.cuda.current_stream().cuda_stream
-    assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 4, 8, 256, 2, s) == lib.LK_ERR_TYPE     # q2_K: not served
+    assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 4, 8, 256, 11, s) == lib.LK_ERR_TYPE    # IQ3_XXS: not served
     assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 4, 8, 250, 1, s) == lib.LK_ERR_ARG      # k not whole blocks
     assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 5, 8, 256, 1, s) == lib.LK_ERR_ARG      # pairs % topk
     assert l.loken_moe_gemm_gguf_down_reduce(p, p, p, p, None, p, 4, 2, 4, 8, 256, 1, None, None, s) == lib.LK_ERR_ARG
