@@ -72,6 +72,7 @@ def parse_args():
     ap.add_argument("--rows-n", type=int, default=14336, help="--workload gemv: weight rows")
     ap.add_argument("--cols-k", type=int, default=4096, help="--workload gemv: values per row")
     ap.add_argument("--tokens", type=int, default=256, help="--workload moe: rows through the expert block")
+    ap.add_argument("--moe-wtype", default="q4_k", help="--workload moe: the experts' format (as --wtype)")
     ap.add_argument("--moe-path", choices=["auto", "tiled", "pairs"], default="auto",
                     help="--workload moe: expert-batched tiled matmul, mat-vec per routed pair, or the library's choice")
     ap.add_argument("--mid-rows", choices=["matvec", "tiled"], default="matvec",

@@ -393,7 +393,9 @@ static int dispatch_plain(int wtype, int batch, MmvqCall& a) {
         case LK_TYPE_Q4_K:
             if (a.nb <= 8) { LK_BATCH_SWITCH(launch_plain, EngQ4KShort, T, a) }
             LK_BATCH_SWITCH(launch_plain, EngQ4K, T, a)
-        case LK_TYPE_Q5_K: LK_BATCH_SWITCH(launch_plain, EngQ5K, T, a)
+        case LK_TYPE_Q5_K:
+            if (a.nb <= 8) { LK_BATCH_SWITCH(launch_plain, EngQ5KShort, T, a) }
+            LK_BATCH_SWITCH(launch_plain, EngQ5K, T, a)
         case LK_TYPE_Q6_K: LK_BATCH_SWITCH(launch_plain, EngQ6K, T, a)
         case LK_TYPE_Q8_0: LK_BATCH_SWITCH(launch_plain, EngQ80, T, a)
         default: return LK_ERR_TYPE;

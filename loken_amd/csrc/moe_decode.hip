@@ -190,7 +190,8 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
                              : launch_mode<EngQ4K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 4:
             d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q5K_BYTES;
-            return launch_mode<EngQ5K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
+            return d.nb <= 8 ? launch_mode<EngQ5KShort, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s)
+                             : launch_mode<EngQ5K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 5:
             d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q6K_BYTES;
             return launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);

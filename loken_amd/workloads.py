@@ -317,9 +317,18 @@ def mmq(args, dev):
 def moe_block(args, dev):
     experts, hidden, ffn, topk, tokens = 128, 2048, 768, 8, args.tokens
     mk = Maker(dev)
-    gate = mk.q4k(experts * ffn, hidden)
-    up = mk.q4k(experts * ffn, hidden)
-    down = mk.q4k(experts * hidden, ffn)
+    # `--moe-wtype` other than q4_k: the same block with every expert matrix in that format
+    name = args.moe_wtype
+    wt = WTYPES[name]
+    if wt == Q4K:
+        gate = mk.q4k(experts * ffn, hidden)
+        up = mk.q4k(experts * ffn, hidden)
+        down = mk.q4k(experts * hidden, ffn)
+    else:
+        def stack(n, k, stream):   # a few generated rows repeated: the kernels do not care what the blocks hold
+            base = torch.from_numpy(synth.weight(wt, 256, k, seed=0, stream=stream)).to(dev).reshape(256, -1)
+            return base.repeat(n // 256, 1).contiguous().reshape(-1)
+        gate, up, down = stack(experts * ffn, hidden, 1), stack(experts * ffn, hidden, 2), stack(experts * hidden, ffn, 3)
     x = mk.randn(tokens, hidden)
     logits = mk.randn(tokens, experts)
     probs = torch.softmax(logits, dim=-1)
@@ -329,6 +338,7 @@ def moe_block(args, dev):
 
     pairs = tokens * topk
     tiled = moe.moe_mmq_pays(pairs, experts) if args.moe_path == "auto" else args.moe_path == "tiled"
+    tiled = tiled and moe.moe_mmq_serves(wt, hidden) and moe.moe_mmq_serves(wt, ffn)
     # The routing (the router's side of the boundary) is built once; the timed block is what the
     # expert launchers do with it, recorded into a graph so that the host's cost stays outside.
     flat_w = weights.reshape(-1)
@@ -336,32 +346,32 @@ def moe_block(args, dev):
         plan = moe.MmqRouting.from_choices(choices, experts)
 
         def block():
-            h = plan.gate_up_silu(Q4K, x, gate, up, ffn)
-            return plan.down_fold(Q4K, h, down, hidden, flat_w)
+            h = plan.gate_up_silu(wt, x, gate, up, ffn)
+            return plan.down_fold(wt, h, down, hidden, flat_w)
     else:
         routing = moe.ExpertRouting(choices)
 
         def block():
-            h = moe.moe_gemm_gguf_gate_up_silu_mul(Q4K, x, gate, up, routing, experts, ffn)
-            return moe.moe_gemm_gguf_down_reduce(Q4K, h, down, routing, flat_w, experts, hidden)
+            h = moe.moe_gemm_gguf_gate_up_silu_mul(wt, x, gate, up, routing, experts, ffn)
+            return moe.moe_gemm_gguf_down_reduce(wt, h, down, routing, flat_w, experts, hidden)
 
     eager = time_launches(lambda i: block(), args.launches)
     us = time_replays(capture(block), args.launches)
     med = float(np.median(us))
     load = torch.bincount(choices.reshape(-1).to(torch.int64), minlength=experts).cpu().numpy()
     distinct = int((load > 0).sum())
-    one_matrix = synth.weight_bytes(Q4K, ffn, hidden)
+    one_matrix = synth.weight_bytes(wt, ffn, hidden)
     if tiled:
         op_count = 6.0 * pairs * ffn * hidden
         value, unit = op_count / med / 1e6, "TOP/s"
         roofline = {"bound": "mfma", "achieved": round(value, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                    "frac": round(value / INT8_PEAK_TOPS, 4), "traffic": None, "kernel": "mmq_moe_kernel<MmqQ4K,...>",
+                    "frac": round(value / INT8_PEAK_TOPS, 4), "traffic": None, "kernel": f"mmq_moe_kernel, {name}",
                     "note": "whole expert block (plan, route, quantize, two grouped matmuls, activation, fold)"}
     else:
         nbytes = 3 * one_matrix * distinct
         value, unit = nbytes / med / 1e3, "GB/s"
         roofline = {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "moe_rows_kernel<EngQ4K,...>",
+                    "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None, "kernel": f"moe_rows_kernel / moe_rows_legacy_kernel, {name}",
                     "note": "whole expert block (quantize, gate/up pairs, down pairs, weighted sum); bytes = 3 matrices "
                             "per distinct expert hit"}
     extra = {"block_graph_replay": spread(us), "block_eager_from_python": spread(eager), "path": "expert-batched tiled matmul" if tiled else "mat-vec per routed pair",
@@ -369,7 +379,7 @@ def moe_block(args, dev):
              "expert_load_histogram": {"max": int(load.max()), "mean": round(float(load.mean()), 2),
                                        "rows_per_expert_sorted_top8": sorted(load.tolist(), reverse=True)[:8]}}
     return line(args, value, unit, med * 1e-3, "int8",
-                {"workload": f"MoE expert block, 128 experts 2048->768->2048 Q4_K, top-8, {tokens} tokens"}, roofline,
+                {"workload": f"MoE expert block, 128 experts 2048->768->2048 {name}, top-8, {tokens} tokens"}, roofline,
                 extra)
 
 

@@ -219,10 +219,11 @@ def test_per_pair_decode_block_matches_oracle(tokens, hidden, ffn, n_experts, to
 
 # the rows of the reference's expert table (src/inference/moe_cuda/gemm.rs:23-39) beyond the K-quant engines
 TABLE_TAIL = {"q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "q5_0": lib.TYPE_Q5_0, "mxfp4": lib.TYPE_MXFP4,
-              "q5_1": lib.TYPE_Q5_1, "iq4_nl": lib.TYPE_IQ4_NL, "iq4_xs": lib.TYPE_IQ4_XS}
+              "q5_1": lib.TYPE_Q5_1, "iq4_nl": lib.TYPE_IQ4_NL, "iq4_xs": lib.TYPE_IQ4_XS,
+              "q5_k": lib.TYPE_Q5_K}   # and Q5_K on the K-quant engine, short rows and long
 
 
-@pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(1, 1024, 768, 16, 4), (3, 512, 256, 6, 2)])
+@pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(1, 1024, 768, 16, 4), (3, 512, 256, 6, 2), (2, 2560, 512, 4, 2)])
 @pytest.mark.parametrize("name", sorted(TABLE_TAIL))
 def test_per_pair_decode_block_in_the_tail_formats_matches_oracle(name, tokens, hidden, ffn, n_experts, topk):
     dt = TABLE_TAIL[name]
