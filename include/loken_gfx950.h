@@ -310,6 +310,29 @@ int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const void* gate_w
                                          const int32_t* expert_ids, float* outputs, int num_experts,
                                          int topk, int size_m, int size_n, int size_k, int quant_type,
                                          void* stream);
+/* The same launch with the other gated activations of the reference's expert kernels
+ * (cuda/moe/moe_gguf.cu:960-1003, 1101-1118; 1146-1184, 1196-...; 1243-1289, 1301-...;
+ * src/inference/moe_cuda/gemm.rs:596-747), g = gate_e . x, u = up_e . x:
+ *   swiglu_oai      g += gate_bias[e], u += up_bias[e] ([num_experts, size_n] f32, nullable);
+ *                   x = min(g, limit); out = x * sigmoid(alpha x) * (1 + clamp(u, -limit, limit))
+ *   swiglu_limited  g = min(g, limit), u = clamp(u, -limit, limit); out = silu(g) * u
+ *   gelu_mul_concat one tensor [num_experts, 2 size_n, k] per layer, an expert's gate rows then its
+ *                   up rows; out = gelu_tanh(g) * u */
+int loken_moe_gemm_gguf_gate_up_swiglu_oai(const float* inputs, const void* gate_weights,
+                                           const void* up_weights, const int32_t* sorted_token_ids,
+                                           const int32_t* expert_ids, const float* gate_bias,
+                                           const float* up_bias, float* outputs, int num_experts, int topk,
+                                           int size_m, int size_n, int size_k, int quant_type, float alpha,
+                                           float limit, void* stream);
+int loken_moe_gemm_gguf_gate_up_swiglu_limited(const float* inputs, const void* gate_weights,
+                                               const void* up_weights, const int32_t* sorted_token_ids,
+                                               const int32_t* expert_ids, float* outputs, int num_experts,
+                                               int topk, int size_m, int size_n, int size_k, int quant_type,
+                                               float limit, void* stream);
+int loken_moe_gemm_gguf_gate_up_gelu_mul_concat(const float* inputs, const void* gate_up_weights,
+                                                const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                                float* outputs, int num_experts, int topk, int size_m,
+                                                int size_n, int size_k, int quant_type, void* stream);
 /* outputs[t, :] (+)= sum over k ascending of topk_weights[p] * (down_e(p) . inputs[p] + down_bias[e(p)]),
  * p = t * topk + k; inputs [size_m, k] in slot order. Without add_after `outputs` [size_m/topk,
  * size_n] must be pre-filled (zeros or the residual) and is accumulated into; with it the result

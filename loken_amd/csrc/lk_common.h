@@ -151,13 +151,49 @@ int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, in
                    int batch, int stride_col_y, int stride_col_dst, const float* bias, hipStream_t stream);
 int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32_t* dots, int ncols_x, int nrows_x,
                            hipStream_t stream);
+// What the gated MoE decode launch makes of a row's gate product g and up product u
+// (cuda/moe/moe_gguf.cu:994-1003, 1178-1184, 1280-1289 of the reference):
+//   SILU      g / (1 + exp(-g)) * u
+//   OAI       g += gate_bias, u += up_bias (per expert, nullable); x = min(g, limit); u' = clamp(u, +-limit);
+//             x * sigmoid(alpha x) * (1 + u')
+//   LIMITED   g = min(g, limit), u = clamp(u, +-limit); g / (1 + exp(-g)) * u
+//   GELU      0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u
+enum { LK_GATE_SILU = 0, LK_GATE_OAI = 1, LK_GATE_LIMITED = 2, LK_GATE_GELU = 3 };
+struct LkGateAct {
+    int kind = LK_GATE_SILU;
+    float alpha = 0.f, limit = 0.f;
+    const float* gate_bias = nullptr;
+    const float* up_bias = nullptr;
+};
+static __device__ __forceinline__ float lk_gated(const LkGateAct& a, float g, float u, size_t bias_at) {
+    switch (a.kind) {
+        case LK_GATE_OAI: {
+            if (a.gate_bias) g += a.gate_bias[bias_at];
+            if (a.up_bias) u += a.up_bias[bias_at];
+            const float x = fminf(g, a.limit);
+            const float uc = fminf(fmaxf(u, -a.limit), a.limit);
+            return (x * (1.0f / (1.0f + expf(-a.alpha * x)))) * (1.0f + uc);
+        }
+        case LK_GATE_LIMITED: {
+            g = fminf(g, a.limit);
+            u = fminf(fmaxf(u, -a.limit), a.limit);
+            return g / (1.0f + expf(-g)) * u;
+        }
+        case LK_GATE_GELU:
+            return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * (g * g * g)))) * u;
+        default:
+            return g / (1.0f + expf(-g)) * u;
+    }
+}
+
 // MoE decode for the expert formats the K-quant engines do not serve (mmvq_legacy.hip): block length
-// of a wire id (0: not one of them), and the per-pair launch over Q8_1 activation rows.
+// of a wire id (0: not one of them), and the per-pair launch over Q8_1 activation rows. An expert's
+// slab is `slab_rows` weight rows (cols, or twice that where gate and up share a tensor).
 int lk_moe_wire_block_len_legacy(int quant_type);
 int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts_q8_1,
                        const int32_t* sorted_token_ids, const int32_t* expert_ids, const float* topk_weights,
                        const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
-                       int k32_stride, hipStream_t s);
+                       int k32_stride, const LkGateAct& act, int slab_rows, hipStream_t s);
 
 static inline int lk_launch_status() {
     return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;

@@ -378,11 +378,13 @@ __global__ __launch_bounds__(64) void subdots_lowbit_kernel(const uint8_t* __res
 // (cuda/moe/moe_gguf.cu:476-511, 755-860, 1049-1061) for the rows of its format table that the
 // K-quant engines do not serve. Workgroups (x, pair): the pair's Q8_1 row goes to LDS once, each
 // wave then takes weight rows of the pair's expert. MODE 0: out = w . x (times the routing weight
-// when given), 1: silu(gate . x) * (up . x), 2: routing weight * (w . x + bias).
+// when given), 1: the gated activation of (gate . x, up . x), 2: routing weight * (w . x + bias).
 // ---------------------------------------------------------------------------------------------
 struct MoeLegacyDims {
     int experts, topk, pairs, cols, nb, k32, k32_stride;
     int64_t slab_bytes;
+    int slab_rows;
+    LkGateAct act;
 };
 
 // A lane's share of one weight row against the activation row in LDS.
@@ -451,7 +453,7 @@ __global__ __launch_bounds__(LWG) void moe_rows_legacy_kernel(const uint8_t* __r
         if (MODE == 1) {
             const uint8_t* slab1 = w1 + (int64_t)e * d.slab_bytes;
             const float second = wave_sum(staged_row_share<ID>(slab1 + row * row_bytes, d.nb, lds, d.k32, lane));
-            if (lane == 0) out_row[row] = first / (1.0f + expf(-first)) * second;
+            if (lane == 0) out_row[row] = lk_gated(d.act, first, second, (size_t)e * d.cols + row);
         } else {
             float v = first * scale;
             if (MODE == 2 && down_bias) v += scale * down_bias[(size_t)e * d.cols + row];
@@ -465,7 +467,7 @@ static int launch_moe(int mode, const uint8_t* w0, const uint8_t* w1, const uint
                       const int32_t* eid, const float* tw, const float* bias, float* out, MoeLegacyDims d, hipStream_t s) {
     constexpr bool LOWBIT = ID == 10 || ID == 11 || ID == 23;
     d.k32 = LOWBIT ? d.nb * 8 : d.nb;
-    d.slab_bytes = (int64_t)d.cols * d.nb * BytesOf<ID>::V;
+    d.slab_bytes = (int64_t)d.slab_rows * d.nb * BytesOf<ID>::V;
     const size_t lds_bytes = (size_t)d.k32 * ACT_LDS_PER_BLOCK;
     if (lds_bytes > 48 * 1024 || d.pairs > 65535) return LK_ERR_ARG;
     const int need = (d.cols + LWAVES - 1) / LWAVES;
@@ -608,14 +610,14 @@ int lk_moe_wire_block_len_legacy(int quant_type) {
 int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts_q8_1,
                        const int32_t* sorted_token_ids, const int32_t* expert_ids, const float* topk_weights,
                        const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
-                       int k32_stride, hipStream_t s) {
+                       int k32_stride, const LkGateAct& act, int slab_rows, hipStream_t s) {
     const int bl = lk_moe_wire_block_len_legacy(quant_type);
     if (bl == 0) return LK_ERR_TYPE;
     if (size_k % bl != 0 || ((uintptr_t)acts_q8_1 & 3) != 0) return LK_ERR_ARG;
     const uintptr_t both = (uintptr_t)w0 | (uintptr_t)w1;
     const uintptr_t mask = (quant_type == 2 || quant_type == 10) ? 3 : quant_type == 7 ? 0 : 1;
     if ((both & mask) != 0) return LK_ERR_ARG;
-    MoeLegacyDims d{experts, topk, pairs, cols, size_k / bl, 0, k32_stride, 0};
+    MoeLegacyDims d{experts, topk, pairs, cols, size_k / bl, 0, k32_stride, 0, slab_rows, act};
     switch (quant_type) {
         case 2: return launch_moe<10>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
         case 3: return launch_moe<11>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);

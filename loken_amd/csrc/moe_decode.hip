@@ -73,6 +73,8 @@ struct MoeDims {
     int64_t slab_bytes;                       // one expert's weights
     int act_f32 = 0;                          // non-zero: `acts` holds f32 rows this many floats apart and
                                               // every workgroup quantizes its pair's row while staging it
+    int slab_rows = 0;                        // weight rows per expert when not `cols` (gate and up in one tensor)
+    LkGateAct act;                            // MODE_GATED: what becomes of (gate . x, up . x)
 };
 
 enum { MODE_PLAIN = 0, MODE_GATED = 1, MODE_DOWN = 2 };
@@ -108,8 +110,7 @@ __global__ __launch_bounds__(WG) void moe_rows_kernel(const uint8_t* __restrict_
         const uint8_t* slab1 = w1 + (int64_t)e * d.slab_bytes;
         RowJob<2> job{{to_gbytes(slab0), to_gbytes(slab1)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first, d.act_f32};
         E::template run<1, R, 2>(job, lds, [&](int row, int, const float* tot) {
-            const float g = tot[0];
-            out_row[row] = g / (1.0f + expf(-g)) * tot[1];
+            out_row[row] = lk_gated(d.act, tot[0], tot[1], (size_t)e * d.cols + row);
         });
     } else {
         RowJob<1> job{{to_gbytes(slab0)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first, d.act_f32};
@@ -180,26 +181,27 @@ template <int MODE>
 static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts, const int32_t* sti,
                          const int32_t* eid, const float* tw, const float* bias, float* out, MoeDims d, int size_k,
                          hipStream_t s) {
+    const int64_t slab_rows = d.slab_rows ? d.slab_rows : d.cols;
     switch (quant_type) {   // wire ids of the reference's MOE_GGUF_FORMATS table (cuda/moe/gguf.cuh:55-71)
         case 0:
-            d.nb = size_k / 32; d.slab_bytes = (int64_t)d.cols * d.nb * Q80_BYTES;
+            d.nb = size_k / 32; d.slab_bytes = slab_rows * d.nb * Q80_BYTES;
             return launch_mode<EngQ80, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 1:
-            d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q4K_BYTES;
+            d.nb = size_k / 256; d.slab_bytes = slab_rows * d.nb * Q4K_BYTES;
             return d.nb <= 8 ? launch_mode<EngQ4KShort, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s)
                              : launch_mode<EngQ4K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 4:
-            d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q5K_BYTES;
+            d.nb = size_k / 256; d.slab_bytes = slab_rows * d.nb * Q5K_BYTES;
             return d.nb <= 8 ? launch_mode<EngQ5KShort, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s)
                              : launch_mode<EngQ5K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 5:
-            d.nb = size_k / 256; d.slab_bytes = (int64_t)d.cols * d.nb * Q6K_BYTES;
+            d.nb = size_k / 256; d.slab_bytes = slab_rows * d.nb * Q6K_BYTES;
             return launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         default:
             // Q2_K, Q3_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS: the wave-per-row kernels over Q8_1 rows
             if (d.act_f32) return LK_ERR_ARG;
             return lk_moe_rows_legacy(MODE, quant_type, w0, w1, acts, sti, eid, tw, bias, out, d.experts, d.topk,
-                                      d.pairs, d.cols, size_k, d.k32, s);
+                                      d.pairs, d.cols, size_k, d.k32, d.act, (int)slab_rows, s);
     }
 }
 
@@ -273,11 +275,12 @@ extern "C" int loken_moe_gemm_gguf(const float* inputs, const void* weights, con
                                      topk_weights, nullptr, (float*)outputs, d, size_k, s);
 }
 
-extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const void* gate_weights,
-                                                    const void* up_weights, const int32_t* sorted_token_ids,
-                                                    const int32_t* expert_ids, float* outputs, int num_experts,
-                                                    int topk, int size_m, int size_n, int size_k, int quant_type,
-                                                    void* stream) {
+// The gated launch: act(gate . x, up . x) per routed pair. `slab_rows` = weight rows per expert in
+// both stacks (size_n, or 2 size_n when `up_weights` points size_n rows into the gate's tensor).
+static int gate_up_impl(const float* inputs, const void* gate_weights, const void* up_weights,
+                        const int32_t* sorted_token_ids, const int32_t* expert_ids, float* outputs, int num_experts,
+                        int topk, int size_m, int size_n, int size_k, int quant_type, const LkGateAct& act,
+                        int slab_rows, void* stream) {
     if (block_len_of_wire(quant_type) == 0) return LK_ERR_TYPE;
     if (size_m == 0) return LK_OK;
     if (!inputs || !gate_weights || !up_weights || !sorted_token_ids || !expert_ids || !outputs ||
@@ -285,7 +288,7 @@ extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const v
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k), act_rows = size_m / topk;
     if (rows_stage_as_f32(inputs, size_k, quant_type)) {
-        MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k};
+        MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k, slab_rows, act};
         return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights,
                                          (const uint8_t*)inputs, sorted_token_ids, expert_ids, nullptr, nullptr, outputs,
                                          d, size_k, s);
@@ -294,9 +297,59 @@ extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const v
     uint8_t* acts = (uint8_t*)reserve_scratch((size_t)act_rows * (kp / 32) * Q81_BYTES, s);
     if (!acts) return LK_ERR_NOMEM;
     if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, acts, size_k, kp, act_rows, stream)) return rc;
-    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0};
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, 0, slab_rows, act};
     return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights, acts,
                                      sorted_token_ids, expert_ids, nullptr, nullptr, outputs, d, size_k, s);
+}
+
+extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const void* gate_weights,
+                                                    const void* up_weights, const int32_t* sorted_token_ids,
+                                                    const int32_t* expert_ids, float* outputs, int num_experts,
+                                                    int topk, int size_m, int size_n, int size_k, int quant_type,
+                                                    void* stream) {
+    return gate_up_impl(inputs, gate_weights, up_weights, sorted_token_ids, expert_ids, outputs, num_experts, topk,
+                        size_m, size_n, size_k, quant_type, LkGateAct{}, 0, stream);
+}
+
+extern "C" int loken_moe_gemm_gguf_gate_up_swiglu_oai(const float* inputs, const void* gate_weights,
+                                                      const void* up_weights, const int32_t* sorted_token_ids,
+                                                      const int32_t* expert_ids, const float* gate_bias,
+                                                      const float* up_bias, float* outputs, int num_experts, int topk,
+                                                      int size_m, int size_n, int size_k, int quant_type, float alpha,
+                                                      float limit, void* stream) {
+    LkGateAct act;
+    act.kind = LK_GATE_OAI; act.alpha = alpha; act.limit = limit; act.gate_bias = gate_bias; act.up_bias = up_bias;
+    return gate_up_impl(inputs, gate_weights, up_weights, sorted_token_ids, expert_ids, outputs, num_experts, topk,
+                        size_m, size_n, size_k, quant_type, act, 0, stream);
+}
+
+extern "C" int loken_moe_gemm_gguf_gate_up_swiglu_limited(const float* inputs, const void* gate_weights,
+                                                          const void* up_weights, const int32_t* sorted_token_ids,
+                                                          const int32_t* expert_ids, float* outputs, int num_experts,
+                                                          int topk, int size_m, int size_n, int size_k, int quant_type,
+                                                          float limit, void* stream) {
+    LkGateAct act;
+    act.kind = LK_GATE_LIMITED; act.limit = limit;
+    return gate_up_impl(inputs, gate_weights, up_weights, sorted_token_ids, expert_ids, outputs, num_experts, topk,
+                        size_m, size_n, size_k, quant_type, act, 0, stream);
+}
+
+extern "C" int loken_moe_gemm_gguf_gate_up_gelu_mul_concat(const float* inputs, const void* gate_up_weights,
+                                                           const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                                           float* outputs, int num_experts, int topk, int size_m,
+                                                           int size_n, int size_k, int quant_type, void* stream) {
+    const int bl = block_len_of_wire(quant_type);
+    if (bl == 0) return LK_ERR_TYPE;
+    if (!gate_up_weights || size_n <= 0 || size_k <= 0 || size_k % bl != 0) return size_m == 0 ? LK_OK : LK_ERR_ARG;
+    // an expert's slab holds the gate's size_n rows, then the up's
+    // block bytes by wire id: Q8_0, Q4_K, Q2_K, Q3_K, Q5_K, Q6_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS
+    static const int bytes_of_wire[] = {34, 144, 84, 110, 176, 210, 22, 17, 24, 18, 136};
+    const int64_t row_bytes = (int64_t)(size_k / bl) * bytes_of_wire[quant_type];
+    const uint8_t* up = (const uint8_t*)gate_up_weights + (int64_t)size_n * row_bytes;
+    LkGateAct act;
+    act.kind = LK_GATE_GELU;
+    return gate_up_impl(inputs, gate_up_weights, up, sorted_token_ids, expert_ids, outputs, num_experts, topk, size_m,
+                        size_n, size_k, quant_type, act, 2 * size_n, stream);
 }
 
 extern "C" int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,

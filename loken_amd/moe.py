@@ -159,6 +159,47 @@ def moe_gemm_gguf_gate_up_silu_mul(wtype: int, x: torch.Tensor, gate: torch.Tens
     return out
 
 
+def moe_gemm_gguf_gate_up_swiglu_oai(wtype: int, x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                                     routing: ExpertRouting, n_experts: int, n: int, alpha: float, limit: float,
+                                     gate_bias: torch.Tensor | None = None,
+                                     up_bias: torch.Tensor | None = None) -> torch.Tensor:
+    """gpt-oss's clamped SwiGLU with per-expert biases in the gated launch
+    (src/inference/moe_cuda/gemm.rs:596-651)."""
+    k = x.shape[1]
+    pairs = routing.tokens * routing.topk
+    out = torch.empty((pairs, n), dtype=torch.float32, device=x.device)
+    _lib.check("loken_moe_gemm_gguf_gate_up_swiglu_oai", _lib.load().loken_moe_gemm_gguf_gate_up_swiglu_oai(
+        x.data_ptr(), gate.data_ptr(), up.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+        gate_bias.data_ptr() if gate_bias is not None else None, up_bias.data_ptr() if up_bias is not None else None,
+        out.data_ptr(), n_experts, routing.topk, pairs, n, k, EXPERT_QUANT_CODES[wtype], alpha, limit, _stream()))
+    return out
+
+
+def moe_gemm_gguf_gate_up_swiglu_limited(wtype: int, x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                                         routing: ExpertRouting, n_experts: int, n: int, limit: float) -> torch.Tensor:
+    """The bounded SwiGLU (src/inference/moe_cuda/gemm.rs:656-704)."""
+    k = x.shape[1]
+    pairs = routing.tokens * routing.topk
+    out = torch.empty((pairs, n), dtype=torch.float32, device=x.device)
+    _lib.check("loken_moe_gemm_gguf_gate_up_swiglu_limited", _lib.load().loken_moe_gemm_gguf_gate_up_swiglu_limited(
+        x.data_ptr(), gate.data_ptr(), up.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+        out.data_ptr(), n_experts, routing.topk, pairs, n, k, EXPERT_QUANT_CODES[wtype], limit, _stream()))
+    return out
+
+
+def moe_gemm_gguf_gate_up_gelu_mul_concat(wtype: int, x: torch.Tensor, gate_up: torch.Tensor, routing: ExpertRouting,
+                                          n_experts: int, n: int) -> torch.Tensor:
+    """gelu(gate) * up over one ``[experts, 2 n, k]`` tensor, an expert's gate rows then its up rows
+    (src/inference/moe_cuda/gemm.rs:706-747)."""
+    k = x.shape[1]
+    pairs = routing.tokens * routing.topk
+    out = torch.empty((pairs, n), dtype=torch.float32, device=x.device)
+    _lib.check("loken_moe_gemm_gguf_gate_up_gelu_mul_concat", _lib.load().loken_moe_gemm_gguf_gate_up_gelu_mul_concat(
+        x.data_ptr(), gate_up.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+        out.data_ptr(), n_experts, routing.topk, pairs, n, k, EXPERT_QUANT_CODES[wtype], _stream()))
+    return out
+
+
 def moe_gemm_gguf_down_reduce(wtype: int, h: torch.Tensor, down: torch.Tensor, routing: ExpertRouting,
                               topk_weights: torch.Tensor, n_experts: int, hidden: int,
                               residual: torch.Tensor | None = None, down_bias: torch.Tensor | None = None,

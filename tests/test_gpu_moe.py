@@ -252,6 +252,51 @@ def test_per_pair_decode_block_in_the_tail_formats_matches_oracle(name, tokens, 
         assert (np.abs(got_row - want_row) <= 1e-3 * np.abs(want_row) + 1e-4 * np.abs(want_row).max()).all()
 
 
+@pytest.mark.parametrize("name", ["q4_k", "q6_k", "q8_0", "mxfp4", "q5_0", "q3_k"])
+def test_gated_decode_launch_with_the_other_activations(name):
+    """The gate and up products are the same-codes oracle's; the activation on top of them is the
+    closed form the reference's kernels state (cuda/moe/moe_gguf.cu:994-1003, 1178-1184, 1280-1289)."""
+    from loken_amd.moe import (moe_gemm_gguf_gate_up_gelu_mul_concat, moe_gemm_gguf_gate_up_swiglu_limited,
+                               moe_gemm_gguf_gate_up_swiglu_oai)
+    dt = {"q4_k": lib.TYPE_Q4_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0, **TABLE_TAIL}[name]
+    tokens, hidden, ffn, n_experts, topk = 3, 512, 256, 5, 2
+    gate, up, _, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=63, dt_gu=dt, x_scale=4.0)
+    routing = ExpertRouting(dev(ids))
+    slots, experts = oracle.group_by_expert(ids)
+    gate_rows, up_rows = gate.reshape(n_experts, ffn, -1), up.reshape(n_experts, ffn, -1)
+    g = np.empty((tokens * topk, ffn), np.float64)
+    u = np.empty((tokens * topk, ffn), np.float64)
+    for j in range(len(slots)):
+        row = x[slots[j] // topk][None, :]
+        g[slots[j]] = oracle.ob_matmul(dt, row, gate_rows[experts[j]].reshape(-1), ffn)[0]
+        u[slots[j]] = oracle.ob_matmul(dt, row, up_rows[experts[j]].reshape(-1), ffn)[0]
+    e_of_slot = ids.reshape(-1)
+
+    def close(got, want):
+        got = got.cpu().numpy()
+        assert (np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-4 * np.abs(want).max()).all()
+
+    limit = float(np.quantile(np.abs(g), 0.7))   # so that both sides of every clamp occur
+    alpha = 1.702
+    gb = synth.normal(63, 11, n_experts * ffn).reshape(n_experts, ffn) * np.float32(0.1 * limit)
+    ub = synth.normal(63, 12, n_experts * ffn).reshape(n_experts, ffn) * np.float32(0.1 * limit)
+    for biased in (False, True):
+        gg = g + (gb[e_of_slot] if biased else 0.0)
+        uu = u + (ub[e_of_slot] if biased else 0.0)
+        xx = np.minimum(gg, limit)
+        want = xx / (1.0 + np.exp(-alpha * xx)) * (1.0 + np.clip(uu, -limit, limit))
+        got = moe_gemm_gguf_gate_up_swiglu_oai(dt, dev(x), dev(gate), dev(up), routing, n_experts, ffn, alpha, limit,
+                                               dev(gb) if biased else None, dev(ub) if biased else None)
+        close(got, want)
+    gl = np.minimum(g, limit)
+    close(moe_gemm_gguf_gate_up_swiglu_limited(dt, dev(x), dev(gate), dev(up), routing, n_experts, ffn, limit),
+          gl / (1.0 + np.exp(-gl)) * np.clip(u, -limit, limit))
+    # one tensor per layer: every expert's gate rows, then its up rows
+    both = np.concatenate([gate_rows, up_rows], axis=1)
+    want = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3))) * u
+    close(moe_gemm_gguf_gate_up_gelu_mul_concat(dt, dev(x), dev(np.ascontiguousarray(both)), routing, n_experts, ffn), want)
+
+
 def test_decode_launchers_refuse_the_codebook_formats():
     tokens, hidden, ffn, n_experts, topk = 2, 512, 256, 4, 2
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=62)
