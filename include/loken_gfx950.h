@@ -333,6 +333,22 @@ int loken_moe_gemm_gguf_gate_up_gelu_mul_concat(const float* inputs, const void*
                                                 const int32_t* sorted_token_ids, const int32_t* expert_ids,
                                                 float* outputs, int num_experts, int topk, int size_m,
                                                 int size_n, int size_k, int quant_type, void* stream);
+/* loken_moe_gemm_gguf_gate_up_silu_mul over the first `*live` routed pairs, the count read on the
+ * card when the kernel runs (a captured step whose routing changes between replays); the rows of
+ * the other pairs are not written (cuda/moe/moe_gguf.cu:1063-1075; moe_cuda/gemm.rs:424-474). */
+int loken_moe_gemm_gguf_gate_up_silu_mul_live(const float* inputs, const void* gate_weights,
+                                              const void* up_weights, const int32_t* sorted_token_ids,
+                                              const int32_t* expert_ids, float* outputs, int num_experts,
+                                              int topk, int size_m, int size_n, int size_k, int quant_type,
+                                              const unsigned int* live, void* stream);
+/* The down launch up to the pairs' rows: pair_rows[slot, :] = topk_weights[slot] * (down_e . inputs[slot])
+ * for the first `*live` routed pairs, zero rows for the others; the caller sums a token's topk rows
+ * (cuda/moe/moe_gguf.cu:838-852; moe_cuda/gemm.rs:550-590). */
+int loken_moe_gemm_gguf_down_pairs_live(const float* inputs, const void* weights,
+                                        const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                        const float* topk_weights, float* pair_rows, int num_experts,
+                                        int topk, int size_m, int size_n, int size_k, int quant_type,
+                                        const unsigned int* live, void* stream);
 /* outputs[t, :] (+)= sum over k ascending of topk_weights[p] * (down_e(p) . inputs[p] + down_bias[e(p)]),
  * p = t * topk + k; inputs [size_m, k] in slot order. Without add_after `outputs` [size_m/topk,
  * size_n] must be pre-filled (zeros or the residual) and is accumulated into; with it the result

@@ -188,12 +188,13 @@ static __device__ __forceinline__ float lk_gated(const LkGateAct& a, float g, fl
 
 // MoE decode for the expert formats the K-quant engines do not serve (mmvq_legacy.hip): block length
 // of a wire id (0: not one of them), and the per-pair launch over Q8_1 activation rows. An expert's
-// slab is `slab_rows` weight rows (cols, or twice that where gate and up share a tensor).
+// slab is `slab_rows` weight rows (cols, or twice that where gate and up share a tensor); with `live`
+// only the first *live pairs run (the count is read on the card).
 int lk_moe_wire_block_len_legacy(int quant_type);
 int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts_q8_1,
                        const int32_t* sorted_token_ids, const int32_t* expert_ids, const float* topk_weights,
                        const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
-                       int k32_stride, const LkGateAct& act, int slab_rows, hipStream_t s);
+                       int k32_stride, const LkGateAct& act, int slab_rows, const unsigned int* live, hipStream_t s);
 
 static inline int lk_launch_status() {
     return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;

@@ -385,6 +385,7 @@ struct MoeLegacyDims {
     int64_t slab_bytes;
     int slab_rows;
     LkGateAct act;
+    const unsigned int* live;
 };
 
 // A lane's share of one weight row against the activation row in LDS.
@@ -430,6 +431,7 @@ __global__ __launch_bounds__(LWG) void moe_rows_legacy_kernel(const uint8_t* __r
                                                               MoeLegacyDims d) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int pair = blockIdx.y;
+    if (d.live != nullptr && pair >= (int)*d.live) return;
     const int slot = sorted_token_ids[pair];
     const int e = expert_ids[pair];
     if (slot < 0 || slot >= d.pairs) return;   // the whole workgroup leaves together
@@ -610,14 +612,14 @@ int lk_moe_wire_block_len_legacy(int quant_type) {
 int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts_q8_1,
                        const int32_t* sorted_token_ids, const int32_t* expert_ids, const float* topk_weights,
                        const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
-                       int k32_stride, const LkGateAct& act, int slab_rows, hipStream_t s) {
+                       int k32_stride, const LkGateAct& act, int slab_rows, const unsigned int* live, hipStream_t s) {
     const int bl = lk_moe_wire_block_len_legacy(quant_type);
     if (bl == 0) return LK_ERR_TYPE;
     if (size_k % bl != 0 || ((uintptr_t)acts_q8_1 & 3) != 0) return LK_ERR_ARG;
     const uintptr_t both = (uintptr_t)w0 | (uintptr_t)w1;
     const uintptr_t mask = (quant_type == 2 || quant_type == 10) ? 3 : quant_type == 7 ? 0 : 1;
     if ((both & mask) != 0) return LK_ERR_ARG;
-    MoeLegacyDims d{experts, topk, pairs, cols, size_k / bl, 0, k32_stride, 0, slab_rows, act};
+    MoeLegacyDims d{experts, topk, pairs, cols, size_k / bl, 0, k32_stride, 0, slab_rows, act, live};
     switch (quant_type) {
         case 2: return launch_moe<10>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
         case 3: return launch_moe<11>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);

@@ -75,6 +75,7 @@ struct MoeDims {
                                               // every workgroup quantizes its pair's row while staging it
     int slab_rows = 0;                        // weight rows per expert when not `cols` (gate and up in one tensor)
     LkGateAct act;                            // MODE_GATED: what becomes of (gate . x, up . x)
+    const unsigned int* live = nullptr;       // when given: only the first *live pairs run
 };
 
 enum { MODE_PLAIN = 0, MODE_GATED = 1, MODE_DOWN = 2 };
@@ -89,6 +90,7 @@ __global__ __launch_bounds__(WG) void moe_rows_kernel(const uint8_t* __restrict_
                                                       float* __restrict__ out, MoeDims d) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int pair = blockIdx.y;
+    if (d.live != nullptr && pair >= (int)*d.live) return;
     const int slot = sorted_token_ids[pair];
     const int e = expert_ids[pair];
     if (slot < 0 || slot >= d.pairs) return;
@@ -201,7 +203,7 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
             // Q2_K, Q3_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS: the wave-per-row kernels over Q8_1 rows
             if (d.act_f32) return LK_ERR_ARG;
             return lk_moe_rows_legacy(MODE, quant_type, w0, w1, acts, sti, eid, tw, bias, out, d.experts, d.topk,
-                                      d.pairs, d.cols, size_k, d.k32, d.act, (int)slab_rows, s);
+                                      d.pairs, d.cols, size_k, d.k32, d.act, (int)slab_rows, d.live, s);
     }
 }
 
@@ -280,7 +282,7 @@ extern "C" int loken_moe_gemm_gguf(const float* inputs, const void* weights, con
 static int gate_up_impl(const float* inputs, const void* gate_weights, const void* up_weights,
                         const int32_t* sorted_token_ids, const int32_t* expert_ids, float* outputs, int num_experts,
                         int topk, int size_m, int size_n, int size_k, int quant_type, const LkGateAct& act,
-                        int slab_rows, void* stream) {
+                        int slab_rows, void* stream, const unsigned int* live = nullptr) {
     if (block_len_of_wire(quant_type) == 0) return LK_ERR_TYPE;
     if (size_m == 0) return LK_OK;
     if (!inputs || !gate_weights || !up_weights || !sorted_token_ids || !expert_ids || !outputs ||
@@ -288,7 +290,7 @@ static int gate_up_impl(const float* inputs, const void* gate_weights, const voi
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k), act_rows = size_m / topk;
     if (rows_stage_as_f32(inputs, size_k, quant_type)) {
-        MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k, slab_rows, act};
+        MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k, slab_rows, act, live};
         return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights,
                                          (const uint8_t*)inputs, sorted_token_ids, expert_ids, nullptr, nullptr, outputs,
                                          d, size_k, s);
@@ -297,7 +299,7 @@ static int gate_up_impl(const float* inputs, const void* gate_weights, const voi
     uint8_t* acts = (uint8_t*)reserve_scratch((size_t)act_rows * (kp / 32) * Q81_BYTES, s);
     if (!acts) return LK_ERR_NOMEM;
     if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, acts, size_k, kp, act_rows, stream)) return rc;
-    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, 0, slab_rows, act};
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, 0, slab_rows, act, live};
     return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights, acts,
                                      sorted_token_ids, expert_ids, nullptr, nullptr, outputs, d, size_k, s);
 }
@@ -309,6 +311,15 @@ extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const v
                                                     void* stream) {
     return gate_up_impl(inputs, gate_weights, up_weights, sorted_token_ids, expert_ids, outputs, num_experts, topk,
                         size_m, size_n, size_k, quant_type, LkGateAct{}, 0, stream);
+}
+
+extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul_live(const float* inputs, const void* gate_weights,
+                                                         const void* up_weights, const int32_t* sorted_token_ids,
+                                                         const int32_t* expert_ids, float* outputs, int num_experts,
+                                                         int topk, int size_m, int size_n, int size_k, int quant_type,
+                                                         const unsigned int* live, void* stream) {
+    return gate_up_impl(inputs, gate_weights, up_weights, sorted_token_ids, expert_ids, outputs, num_experts, topk,
+                        size_m, size_n, size_k, quant_type, LkGateAct{}, 0, stream, live);
 }
 
 extern "C" int loken_moe_gemm_gguf_gate_up_swiglu_oai(const float* inputs, const void* gate_weights,
@@ -352,33 +363,68 @@ extern "C" int loken_moe_gemm_gguf_gate_up_gelu_mul_concat(const float* inputs, 
                         size_n, size_k, quant_type, act, 2 * size_n, stream);
 }
 
-extern "C" int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,
-                                               const int32_t* sorted_token_ids, const int32_t* expert_ids,
-                                               const float* topk_weights, float* outputs, int num_experts, int topk,
-                                               int size_m, int size_n, int size_k, int gguf_dtype,
-                                               const float* down_bias, const float* add_after, void* stream) {
+__global__ void zero_f32_kernel(float* __restrict__ p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+
+// Down per routed pair, then the fold over a token's pairs; with `pair_rows` the weighted rows go to
+// the caller's [size_m, size_n] buffer and the sum is the caller's (cuda/moe/moe_gguf.cu:755-820).
+static int down_impl(const float* inputs, const void* weights, const int32_t* sorted_token_ids,
+                     const int32_t* expert_ids, const float* topk_weights, float* outputs, int num_experts, int topk,
+                     int size_m, int size_n, int size_k, int gguf_dtype, const float* down_bias,
+                     const float* add_after, const unsigned int* live, float* pair_rows, void* stream) {
     if (block_len_of_wire(gguf_dtype) == 0) return LK_ERR_TYPE;
     if (size_m == 0) return LK_OK;
-    if (!inputs || !weights || !sorted_token_ids || !expert_ids || !topk_weights || !outputs ||
+    if (!inputs || !weights || !sorted_token_ids || !expert_ids || !topk_weights || (!outputs && !pair_rows) ||
         bad_shape(gguf_dtype, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k);
     const bool as_f32 = rows_stage_as_f32(inputs, size_k, gguf_dtype);
     const size_t act_bytes = as_f32 ? 0 : (((size_t)size_m * (kp / 32) * Q81_BYTES) + 255) & ~(size_t)255;
-    const size_t pair_bytes = (size_t)size_m * size_n * sizeof(float);
+    const size_t pair_bytes = pair_rows ? 0 : (size_t)size_m * size_n * sizeof(float);
     std::lock_guard<std::mutex> lock(g_scratch_mu);
-    uint8_t* base = (uint8_t*)reserve_scratch(act_bytes + pair_bytes, s);
-    if (!base) return LK_ERR_NOMEM;
-    float* pairs = (float*)(base + act_bytes);
+    uint8_t* base = nullptr;
+    if (act_bytes + pair_bytes) {
+        base = (uint8_t*)reserve_scratch(act_bytes + pair_bytes, s);
+        if (!base) return LK_ERR_NOMEM;
+    }
+    float* pairs = pair_rows ? pair_rows : (float*)(base + act_bytes);
     if (!as_f32)
         if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, base, size_k, kp, size_m, stream)) return rc;
-    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, as_f32 ? size_k : 0};
+    if (live) {
+        // the pairs past the count leave their rows to the sum: zero (a fill kernel, so that a
+        // caller may capture the launch)
+        const size_t n = (size_t)size_m * size_n;
+        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, pairs, n);
+    }
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, as_f32 ? size_k : 0, 0, LkGateAct{}, live};
     if (int rc = launch_format<MODE_DOWN>(gguf_dtype, (const uint8_t*)weights, nullptr,
                                           as_f32 ? (const uint8_t*)inputs : base, sorted_token_ids,
                                           expert_ids, topk_weights, down_bias, pairs, d, size_k, s)) return rc;
+    if (pair_rows) return lk_launch_status();
     const int tokens = size_m / topk;
     const size_t total = (size_t)tokens * size_n;
     hipLaunchKernelGGL(sum_topk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (const float*)pairs,
                        add_after, outputs, tokens, topk, size_n);
     return lk_launch_status();
+}
+
+extern "C" int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,
+                                               const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                               const float* topk_weights, float* outputs, int num_experts, int topk,
+                                               int size_m, int size_n, int size_k, int gguf_dtype,
+                                               const float* down_bias, const float* add_after, void* stream) {
+    return down_impl(inputs, weights, sorted_token_ids, expert_ids, topk_weights, outputs, num_experts, topk, size_m,
+                     size_n, size_k, gguf_dtype, down_bias, add_after, nullptr, nullptr, stream);
+}
+
+extern "C" int loken_moe_gemm_gguf_down_pairs_live(const float* inputs, const void* weights,
+                                                   const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                                   const float* topk_weights, float* pair_rows, int num_experts,
+                                                   int topk, int size_m, int size_n, int size_k, int quant_type,
+                                                   const unsigned int* live, void* stream) {
+    if (!pair_rows) return size_m == 0 ? LK_OK : LK_ERR_ARG;
+    return down_impl(inputs, weights, sorted_token_ids, expert_ids, topk_weights, nullptr, num_experts, topk, size_m,
+                     size_n, size_k, quant_type, nullptr, nullptr, live, pair_rows, stream);
 }

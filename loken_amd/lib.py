@@ -61,6 +61,8 @@ SIGNATURES.update({
     "loken_moe_gemm_gguf_gate_up_swiglu_oai": (_i, [_vp] * 8 + [_i] * 6 + [_f, _f, _vp]),
     "loken_moe_gemm_gguf_gate_up_swiglu_limited": (_i, [_vp] * 6 + [_i] * 6 + [_f, _vp]),
     "loken_moe_gemm_gguf_gate_up_gelu_mul_concat": (_i, [_vp] * 5 + [_i] * 6 + [_vp]),
+    "loken_moe_gemm_gguf_gate_up_silu_mul_live": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp]),
+    "loken_moe_gemm_gguf_down_pairs_live": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp]),
     "loken_moe_gemm_gguf_down_reduce": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp, _vp]),
     "loken_moe_sum_topk": (None, [_vp, _vp, _i, _i, _i, _vp]),
     "loken_stream_scratch_release": (None, []),

@@ -200,6 +200,35 @@ def moe_gemm_gguf_gate_up_gelu_mul_concat(wtype: int, x: torch.Tensor, gate_up: 
     return out
 
 
+def moe_gemm_gguf_gate_up_silu_mul_live(wtype: int, x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                                        routing: ExpertRouting, n_experts: int, n: int, live: torch.Tensor,
+                                        out: torch.Tensor | None = None) -> torch.Tensor:
+    """The gated launch over the first ``live[0]`` routed pairs (a uint32 on the card); the other
+    pairs' rows of ``out`` keep what they held (src/inference/moe_cuda/gemm.rs:424-474)."""
+    k = x.shape[1]
+    pairs = routing.tokens * routing.topk
+    if out is None:
+        out = torch.zeros((pairs, n), dtype=torch.float32, device=x.device)
+    _lib.check("loken_moe_gemm_gguf_gate_up_silu_mul_live", _lib.load().loken_moe_gemm_gguf_gate_up_silu_mul_live(
+        x.data_ptr(), gate.data_ptr(), up.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+        out.data_ptr(), n_experts, routing.topk, pairs, n, k, EXPERT_QUANT_CODES[wtype], live.data_ptr(), _stream()))
+    return out
+
+
+def moe_gemm_gguf_down_pairs_live(wtype: int, h: torch.Tensor, down: torch.Tensor, routing: ExpertRouting,
+                                  topk_weights: torch.Tensor, n_experts: int, hidden: int,
+                                  live: torch.Tensor) -> torch.Tensor:
+    """Each of the first ``live[0]`` routed pairs' down rows at its weight, ``[pairs, hidden]`` in slot
+    order, zero rows for the rest (src/inference/moe_cuda/gemm.rs:550-590)."""
+    pairs, k = h.shape
+    out = torch.empty((pairs, hidden), dtype=torch.float32, device=h.device)
+    _lib.check("loken_moe_gemm_gguf_down_pairs_live", _lib.load().loken_moe_gemm_gguf_down_pairs_live(
+        h.data_ptr(), down.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+        topk_weights.data_ptr(), out.data_ptr(), n_experts, routing.topk, pairs, hidden, k, EXPERT_QUANT_CODES[wtype],
+        live.data_ptr(), _stream()))
+    return out
+
+
 def moe_gemm_gguf_down_reduce(wtype: int, h: torch.Tensor, down: torch.Tensor, routing: ExpertRouting,
                               topk_weights: torch.Tensor, n_experts: int, hidden: int,
                               residual: torch.Tensor | None = None, down_bias: torch.Tensor | None = None,

@@ -297,6 +297,36 @@ def test_gated_decode_launch_with_the_other_activations(name):
     close(moe_gemm_gguf_gate_up_gelu_mul_concat(dt, dev(x), dev(np.ascontiguousarray(both)), routing, n_experts, ffn), want)
 
 
+@pytest.mark.parametrize("name", ["q4_k", "mxfp4"])
+def test_live_count_variants_run_the_first_pairs_only(name):
+    from loken_amd.moe import moe_gemm_gguf_down_pairs_live, moe_gemm_gguf_gate_up_silu_mul_live
+    dt = {"q4_k": lib.TYPE_Q4_K, **TABLE_TAIL}[name]
+    tokens, hidden, ffn, n_experts, topk = 4, 512, 256, 5, 2
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=64, dt_down=dt, dt_gu=dt, x_scale=4.0)
+    routing = ExpertRouting(dev(ids))
+    slots = routing.sorted_token_ids.cpu().numpy()
+    pairs = tokens * topk
+    full_h = moe_gemm_gguf_gate_up_silu_mul(dt, dev(x), dev(gate), dev(up), routing, n_experts, ffn)
+    flat_w = dev(w.reshape(-1))
+    for count in (5, pairs, 0):
+        live = torch.tensor([count], dtype=torch.int32, device="cuda")   # the card reads it as a uint32
+        marker = torch.full((pairs, ffn), -7.0, device="cuda")
+        h = moe_gemm_gguf_gate_up_silu_mul_live(dt, dev(x), dev(gate), dev(up), routing, n_experts, ffn, live, out=marker)
+        ran, idle = slots[:count], slots[count:]
+        assert torch.equal(h[ran], full_h[ran])
+        assert (h[idle] == -7.0).all()
+        rows = moe_gemm_gguf_down_pairs_live(dt, full_h, dev(down), routing, flat_w, n_experts, hidden, live)
+        assert (rows[idle] == 0).all()
+        if count == pairs:
+            want = moe_gemm_gguf_down_reduce(dt, full_h, dev(down), routing, flat_w, n_experts, hidden)
+            got = rows.reshape(tokens, topk, hidden).sum(1)
+            assert (got - want).abs().max().item() <= 1e-6 * want.abs().max().item()
+            all_rows = rows
+    live = torch.tensor([5], dtype=torch.int32, device="cuda")
+    rows5 = moe_gemm_gguf_down_pairs_live(dt, full_h, dev(down), routing, flat_w, n_experts, hidden, live)
+    assert torch.equal(rows5[slots[:5]], all_rows[slots[:5]])
+
+
 def test_decode_launchers_refuse_the_codebook_formats():
     tokens, hidden, ffn, n_experts, topk = 2, 512, 256, 4, 2
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=62)
