@@ -349,6 +349,29 @@ int loken_moe_gemm_gguf_down_pairs_live(const float* inputs, const void* weights
                                         const float* topk_weights, float* pair_rows, int num_experts,
                                         int topk, int size_m, int size_n, int size_k, int quant_type,
                                         const unsigned int* live, void* stream);
+/* A layer's experts over two tensors: the slots from `alt_from` on are slot (expert - alt_from) of
+ * the `alt_*` tensor (same format and row count per expert). `alt_at`, when not NULL, is an array
+ * of two addresses ON THE CARD read when the kernel runs and used in place of alt_gate / alt_up
+ * (for the down launch: [0] in place of alt_weights). Otherwise as the launch each is named after
+ * (cuda/moe/moe_gguf.cu:239-257, 824-836, 868-880, 1078-1091; moe_cuda/gemm.rs:319-419, 479-545, 778-...). */
+int loken_moe_gemm_gguf_gate_up_silu_mul_two(const float* inputs, const void* gate_weights,
+                                             const void* up_weights, const void* alt_gate,
+                                             const void* alt_up, int alt_from, const void* const* alt_at,
+                                             const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                             float* outputs, int num_experts, int topk, int size_m,
+                                             int size_n, int size_k, int quant_type, void* stream);
+int loken_moe_gemm_gguf_down_reduce_two(const float* inputs, const void* weights, const void* alt_weights,
+                                        int alt_from, const int32_t* sorted_token_ids,
+                                        const int32_t* expert_ids, const float* topk_weights, float* outputs,
+                                        int num_experts, int topk, int size_m, int size_n, int size_k,
+                                        int quant_type, const float* down_bias, const float* add_after,
+                                        void* stream);
+int loken_moe_gemm_gguf_down_pairs_two(const float* inputs, const void* weights, const void* alt_weights,
+                                       int alt_from, const void* const* alt_at,
+                                       const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                       const float* topk_weights, float* pair_rows, int num_experts,
+                                       int topk, int size_m, int size_n, int size_k, int quant_type,
+                                       void* stream);
 /* outputs[t, :] (+)= sum over k ascending of topk_weights[p] * (down_e(p) . inputs[p] + down_bias[e(p)]),
  * p = t * topk + k; inputs [size_m, k] in slot order. Without add_after `outputs` [size_m/topk,
  * size_n] must be pre-filled (zeros or the residual) and is accumulated into; with it the result

@@ -186,6 +186,22 @@ static __device__ __forceinline__ float lk_gated(const LkGateAct& a, float g, fl
     }
 }
 
+// A layer's experts over two tensors (cuda/moe/moe_gguf.cu:239-257 of the reference): the slots from
+// `alt_from` on are slot (expert - alt_from) of the second tensor; `alt_at`, when given, is a pair of
+// addresses on the card read when the kernel runs (gate / down at [0], up at [1]).
+struct LkMoeAlt {
+    const uint8_t* alt0 = nullptr;
+    const uint8_t* alt1 = nullptr;
+    int alt_from = 0;
+    const void* const* alt_at = nullptr;
+};
+static __device__ __forceinline__ const uint8_t* lk_expert_slab(const uint8_t* base, int which, const LkMoeAlt& alt, int e,
+                                                                int64_t slab_bytes) {
+    const uint8_t* second = alt.alt_at ? (const uint8_t*)alt.alt_at[which] : (which ? alt.alt1 : alt.alt0);
+    if (second != nullptr && e >= alt.alt_from) return second + (int64_t)(e - alt.alt_from) * slab_bytes;
+    return base + (int64_t)e * slab_bytes;
+}
+
 // MoE decode for the expert formats the K-quant engines do not serve (mmvq_legacy.hip): block length
 // of a wire id (0: not one of them), and the per-pair launch over Q8_1 activation rows. An expert's
 // slab is `slab_rows` weight rows (cols, or twice that where gate and up share a tensor); with `live`
@@ -194,7 +210,8 @@ int lk_moe_wire_block_len_legacy(int quant_type);
 int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts_q8_1,
                        const int32_t* sorted_token_ids, const int32_t* expert_ids, const float* topk_weights,
                        const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
-                       int k32_stride, const LkGateAct& act, int slab_rows, const unsigned int* live, hipStream_t s);
+                       int k32_stride, const LkGateAct& act, int slab_rows, const unsigned int* live,
+                       const LkMoeAlt& alt, hipStream_t s);
 
 static inline int lk_launch_status() {
     return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;

@@ -386,6 +386,7 @@ struct MoeLegacyDims {
     int slab_rows;
     LkGateAct act;
     const unsigned int* live;
+    LkMoeAlt alt;
 };
 
 // A lane's share of one weight row against the activation row in LDS.
@@ -449,11 +450,11 @@ __global__ __launch_bounds__(LWG) void moe_rows_legacy_kernel(const uint8_t* __r
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const size_t row_bytes = (size_t)d.nb * BytesOf<ID>::V;
-    const uint8_t* slab0 = w0 + (int64_t)e * d.slab_bytes;
+    const uint8_t* slab0 = lk_expert_slab(w0, 0, d.alt, e, d.slab_bytes);
     for (int row = blockIdx.x * LWAVES + wave; row < d.cols; row += gridDim.x * LWAVES) {
         const float first = wave_sum(staged_row_share<ID>(slab0 + row * row_bytes, d.nb, lds, d.k32, lane));
         if (MODE == 1) {
-            const uint8_t* slab1 = w1 + (int64_t)e * d.slab_bytes;
+            const uint8_t* slab1 = lk_expert_slab(w1, 1, d.alt, e, d.slab_bytes);
             const float second = wave_sum(staged_row_share<ID>(slab1 + row * row_bytes, d.nb, lds, d.k32, lane));
             if (lane == 0) out_row[row] = lk_gated(d.act, first, second, (size_t)e * d.cols + row);
         } else {
@@ -612,14 +613,15 @@ int lk_moe_wire_block_len_legacy(int quant_type) {
 int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts_q8_1,
                        const int32_t* sorted_token_ids, const int32_t* expert_ids, const float* topk_weights,
                        const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
-                       int k32_stride, const LkGateAct& act, int slab_rows, const unsigned int* live, hipStream_t s) {
+                       int k32_stride, const LkGateAct& act, int slab_rows, const unsigned int* live,
+                       const LkMoeAlt& alt, hipStream_t s) {
     const int bl = lk_moe_wire_block_len_legacy(quant_type);
     if (bl == 0) return LK_ERR_TYPE;
     if (size_k % bl != 0 || ((uintptr_t)acts_q8_1 & 3) != 0) return LK_ERR_ARG;
-    const uintptr_t both = (uintptr_t)w0 | (uintptr_t)w1;
+    const uintptr_t both = (uintptr_t)w0 | (uintptr_t)w1 | (uintptr_t)alt.alt0 | (uintptr_t)alt.alt1;
     const uintptr_t mask = (quant_type == 2 || quant_type == 10) ? 3 : quant_type == 7 ? 0 : 1;
     if ((both & mask) != 0) return LK_ERR_ARG;
-    MoeLegacyDims d{experts, topk, pairs, cols, size_k / bl, 0, k32_stride, 0, slab_rows, act, live};
+    MoeLegacyDims d{experts, topk, pairs, cols, size_k / bl, 0, k32_stride, 0, slab_rows, act, live, alt};
     switch (quant_type) {
         case 2: return launch_moe<10>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
         case 3: return launch_moe<11>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);

@@ -76,6 +76,7 @@ struct MoeDims {
     int slab_rows = 0;                        // weight rows per expert when not `cols` (gate and up in one tensor)
     LkGateAct act;                            // MODE_GATED: what becomes of (gate . x, up . x)
     const unsigned int* live = nullptr;       // when given: only the first *live pairs run
+    LkMoeAlt alt;                             // the experts from alt.alt_from on live in a second tensor
 };
 
 enum { MODE_PLAIN = 0, MODE_GATED = 1, MODE_DOWN = 2 };
@@ -106,10 +107,10 @@ __global__ __launch_bounds__(WG) void moe_rows_kernel(const uint8_t* __restrict_
     const uint8_t* vy = d.act_f32 ? acts + (size_t)act_row * d.act_f32 * sizeof(float)
                                   : acts + (size_t)act_row * d.k32 * Q81_BYTES;
     const float scale = (MODE != MODE_GATED && topk_weights) ? topk_weights[slot] : 1.0f;
-    const uint8_t* slab0 = w0 + (int64_t)e * d.slab_bytes;
+    const uint8_t* slab0 = lk_expert_slab(w0, 0, d.alt, e, d.slab_bytes);
     const int tile_stride = (int)gridDim.x * WAVES, tile_first = (int)blockIdx.x * WAVES;
     if (MODE == MODE_GATED) {
-        const uint8_t* slab1 = w1 + (int64_t)e * d.slab_bytes;
+        const uint8_t* slab1 = lk_expert_slab(w1, 1, d.alt, e, d.slab_bytes);
         RowJob<2> job{{to_gbytes(slab0), to_gbytes(slab1)}, vy, d.nb, d.cols, d.k32, tile_stride, tile_first, d.act_f32};
         E::template run<1, R, 2>(job, lds, [&](int row, int, const float* tot) {
             out_row[row] = lk_gated(d.act, tot[0], tot[1], (size_t)e * d.cols + row);
@@ -203,7 +204,7 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
             // Q2_K, Q3_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS: the wave-per-row kernels over Q8_1 rows
             if (d.act_f32) return LK_ERR_ARG;
             return lk_moe_rows_legacy(MODE, quant_type, w0, w1, acts, sti, eid, tw, bias, out, d.experts, d.topk,
-                                      d.pairs, d.cols, size_k, d.k32, d.act, (int)slab_rows, d.live, s);
+                                      d.pairs, d.cols, size_k, d.k32, d.act, (int)slab_rows, d.live, d.alt, s);
     }
 }
 
@@ -282,7 +283,7 @@ extern "C" int loken_moe_gemm_gguf(const float* inputs, const void* weights, con
 static int gate_up_impl(const float* inputs, const void* gate_weights, const void* up_weights,
                         const int32_t* sorted_token_ids, const int32_t* expert_ids, float* outputs, int num_experts,
                         int topk, int size_m, int size_n, int size_k, int quant_type, const LkGateAct& act,
-                        int slab_rows, void* stream, const unsigned int* live = nullptr) {
+                        int slab_rows, void* stream, const unsigned int* live = nullptr, const LkMoeAlt& alt = LkMoeAlt{}) {
     if (block_len_of_wire(quant_type) == 0) return LK_ERR_TYPE;
     if (size_m == 0) return LK_OK;
     if (!inputs || !gate_weights || !up_weights || !sorted_token_ids || !expert_ids || !outputs ||
@@ -290,7 +291,7 @@ static int gate_up_impl(const float* inputs, const void* gate_weights, const voi
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k), act_rows = size_m / topk;
     if (rows_stage_as_f32(inputs, size_k, quant_type)) {
-        MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k, slab_rows, act, live};
+        MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k, slab_rows, act, live, alt};
         return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights,
                                          (const uint8_t*)inputs, sorted_token_ids, expert_ids, nullptr, nullptr, outputs,
                                          d, size_k, s);
@@ -299,7 +300,7 @@ static int gate_up_impl(const float* inputs, const void* gate_weights, const voi
     uint8_t* acts = (uint8_t*)reserve_scratch((size_t)act_rows * (kp / 32) * Q81_BYTES, s);
     if (!acts) return LK_ERR_NOMEM;
     if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, acts, size_k, kp, act_rows, stream)) return rc;
-    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, 0, slab_rows, act, live};
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, 0, slab_rows, act, live, alt};
     return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights, acts,
                                      sorted_token_ids, expert_ids, nullptr, nullptr, outputs, d, size_k, s);
 }
@@ -320,6 +321,18 @@ extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul_live(const float* inputs, co
                                                          const unsigned int* live, void* stream) {
     return gate_up_impl(inputs, gate_weights, up_weights, sorted_token_ids, expert_ids, outputs, num_experts, topk,
                         size_m, size_n, size_k, quant_type, LkGateAct{}, 0, stream, live);
+}
+
+extern "C" int loken_moe_gemm_gguf_gate_up_silu_mul_two(const float* inputs, const void* gate_weights,
+                                                        const void* up_weights, const void* alt_gate,
+                                                        const void* alt_up, int alt_from, const void* const* alt_at,
+                                                        const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                                        float* outputs, int num_experts, int topk, int size_m,
+                                                        int size_n, int size_k, int quant_type, void* stream) {
+    LkMoeAlt alt;
+    alt.alt0 = (const uint8_t*)alt_gate; alt.alt1 = (const uint8_t*)alt_up; alt.alt_from = alt_from; alt.alt_at = alt_at;
+    return gate_up_impl(inputs, gate_weights, up_weights, sorted_token_ids, expert_ids, outputs, num_experts, topk,
+                        size_m, size_n, size_k, quant_type, LkGateAct{}, 0, stream, nullptr, alt);
 }
 
 extern "C" int loken_moe_gemm_gguf_gate_up_swiglu_oai(const float* inputs, const void* gate_weights,
@@ -373,7 +386,8 @@ __global__ void zero_f32_kernel(float* __restrict__ p, size_t n) {
 static int down_impl(const float* inputs, const void* weights, const int32_t* sorted_token_ids,
                      const int32_t* expert_ids, const float* topk_weights, float* outputs, int num_experts, int topk,
                      int size_m, int size_n, int size_k, int gguf_dtype, const float* down_bias,
-                     const float* add_after, const unsigned int* live, float* pair_rows, void* stream) {
+                     const float* add_after, const unsigned int* live, float* pair_rows, void* stream,
+                     const LkMoeAlt& alt = LkMoeAlt{}) {
     if (block_len_of_wire(gguf_dtype) == 0) return LK_ERR_TYPE;
     if (size_m == 0) return LK_OK;
     if (!inputs || !weights || !sorted_token_ids || !expert_ids || !topk_weights || (!outputs && !pair_rows) ||
@@ -398,7 +412,7 @@ static int down_impl(const float* inputs, const void* weights, const int32_t* so
         const size_t n = (size_t)size_m * size_n;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, pairs, n);
     }
-    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, as_f32 ? size_k : 0, 0, LkGateAct{}, live};
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, as_f32 ? size_k : 0, 0, LkGateAct{}, live, alt};
     if (int rc = launch_format<MODE_DOWN>(gguf_dtype, (const uint8_t*)weights, nullptr,
                                           as_f32 ? (const uint8_t*)inputs : base, sorted_token_ids,
                                           expert_ids, topk_weights, down_bias, pairs, d, size_k, s)) return rc;
@@ -427,4 +441,29 @@ extern "C" int loken_moe_gemm_gguf_down_pairs_live(const float* inputs, const vo
     if (!pair_rows) return size_m == 0 ? LK_OK : LK_ERR_ARG;
     return down_impl(inputs, weights, sorted_token_ids, expert_ids, topk_weights, nullptr, num_experts, topk, size_m,
                      size_n, size_k, quant_type, nullptr, nullptr, live, pair_rows, stream);
+}
+
+extern "C" int loken_moe_gemm_gguf_down_reduce_two(const float* inputs, const void* weights, const void* alt_weights,
+                                                   int alt_from, const int32_t* sorted_token_ids,
+                                                   const int32_t* expert_ids, const float* topk_weights, float* outputs,
+                                                   int num_experts, int topk, int size_m, int size_n, int size_k,
+                                                   int quant_type, const float* down_bias, const float* add_after,
+                                                   void* stream) {
+    LkMoeAlt alt;
+    alt.alt0 = (const uint8_t*)alt_weights; alt.alt_from = alt_from;
+    return down_impl(inputs, weights, sorted_token_ids, expert_ids, topk_weights, outputs, num_experts, topk, size_m,
+                     size_n, size_k, quant_type, down_bias, add_after, nullptr, nullptr, stream, alt);
+}
+
+extern "C" int loken_moe_gemm_gguf_down_pairs_two(const float* inputs, const void* weights, const void* alt_weights,
+                                                  int alt_from, const void* const* alt_at,
+                                                  const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                                  const float* topk_weights, float* pair_rows, int num_experts,
+                                                  int topk, int size_m, int size_n, int size_k, int quant_type,
+                                                  void* stream) {
+    if (!pair_rows) return size_m == 0 ? LK_OK : LK_ERR_ARG;
+    LkMoeAlt alt;
+    alt.alt0 = (const uint8_t*)alt_weights; alt.alt_from = alt_from; alt.alt_at = alt_at;
+    return down_impl(inputs, weights, sorted_token_ids, expert_ids, topk_weights, nullptr, num_experts, topk, size_m,
+                     size_n, size_k, quant_type, nullptr, nullptr, nullptr, pair_rows, stream, alt);
 }

@@ -63,6 +63,9 @@ SIGNATURES.update({
     "loken_moe_gemm_gguf_gate_up_gelu_mul_concat": (_i, [_vp] * 5 + [_i] * 6 + [_vp]),
     "loken_moe_gemm_gguf_gate_up_silu_mul_live": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp]),
     "loken_moe_gemm_gguf_down_pairs_live": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp]),
+    "loken_moe_gemm_gguf_gate_up_silu_mul_two": (_i, [_vp] * 5 + [_i] + [_vp] * 4 + [_i] * 6 + [_vp]),
+    "loken_moe_gemm_gguf_down_reduce_two": (_i, [_vp] * 3 + [_i] + [_vp] * 4 + [_i] * 6 + [_vp, _vp, _vp]),
+    "loken_moe_gemm_gguf_down_pairs_two": (_i, [_vp] * 3 + [_i] + [_vp] * 5 + [_i] * 6 + [_vp]),
     "loken_moe_gemm_gguf_down_reduce": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp, _vp]),
     "loken_moe_sum_topk": (None, [_vp, _vp, _i, _i, _i, _vp]),
     "loken_stream_scratch_release": (None, []),

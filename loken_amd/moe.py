@@ -229,6 +229,52 @@ def moe_gemm_gguf_down_pairs_live(wtype: int, h: torch.Tensor, down: torch.Tenso
     return out
 
 
+def moe_gemm_gguf_gate_up_silu_mul_over(wtype: int, x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                                        more_gate: torch.Tensor, more_up: torch.Tensor, more_from: int,
+                                        routing: ExpertRouting, n_experts: int, n: int,
+                                        more_at: torch.Tensor | None = None) -> torch.Tensor:
+    """The gated launch with the experts from ``more_from`` on in a second pair of tensors; ``more_at``
+    (two int64 addresses on the card) names them at run time instead
+    (src/inference/moe_cuda/gemm.rs:319-419)."""
+    k = x.shape[1]
+    pairs = routing.tokens * routing.topk
+    out = torch.empty((pairs, n), dtype=torch.float32, device=x.device)
+    _lib.check("loken_moe_gemm_gguf_gate_up_silu_mul_two", _lib.load().loken_moe_gemm_gguf_gate_up_silu_mul_two(
+        x.data_ptr(), gate.data_ptr(), up.data_ptr(), more_gate.data_ptr(), more_up.data_ptr(), more_from,
+        more_at.data_ptr() if more_at is not None else None, routing.sorted_token_ids.data_ptr(),
+        routing.expert_ids.data_ptr(), out.data_ptr(), n_experts, routing.topk, pairs, n, k, EXPERT_QUANT_CODES[wtype],
+        _stream()))
+    return out
+
+
+def moe_gemm_gguf_down_reduce_over(wtype: int, h: torch.Tensor, down: torch.Tensor, more_down: torch.Tensor,
+                                   more_from: int, routing: ExpertRouting, topk_weights: torch.Tensor, n_experts: int,
+                                   hidden: int, down_bias: torch.Tensor | None = None) -> torch.Tensor:
+    """Down + fold with the experts from ``more_from`` on in a second tensor
+    (src/inference/moe_cuda/gemm.rs:778-...)."""
+    pairs, k = h.shape
+    out = torch.zeros((pairs // routing.topk, hidden), dtype=torch.float32, device=h.device)
+    _lib.check("loken_moe_gemm_gguf_down_reduce_two", _lib.load().loken_moe_gemm_gguf_down_reduce_two(
+        h.data_ptr(), down.data_ptr(), more_down.data_ptr(), more_from, routing.sorted_token_ids.data_ptr(),
+        routing.expert_ids.data_ptr(), topk_weights.data_ptr(), out.data_ptr(), n_experts, routing.topk, pairs, hidden, k,
+        EXPERT_QUANT_CODES[wtype], down_bias.data_ptr() if down_bias is not None else None, None, _stream()))
+    return out
+
+
+def moe_gemm_gguf_down_pairs_over(wtype: int, h: torch.Tensor, down: torch.Tensor, more_down: torch.Tensor,
+                                  more_from: int, routing: ExpertRouting, topk_weights: torch.Tensor, n_experts: int,
+                                  hidden: int, more_at: torch.Tensor | None = None) -> torch.Tensor:
+    """The same up to the pairs' weighted rows, ``[pairs, hidden]`` (src/inference/moe_cuda/gemm.rs:479-545)."""
+    pairs, k = h.shape
+    out = torch.empty((pairs, hidden), dtype=torch.float32, device=h.device)
+    _lib.check("loken_moe_gemm_gguf_down_pairs_two", _lib.load().loken_moe_gemm_gguf_down_pairs_two(
+        h.data_ptr(), down.data_ptr(), more_down.data_ptr(), more_from,
+        more_at.data_ptr() if more_at is not None else None, routing.sorted_token_ids.data_ptr(),
+        routing.expert_ids.data_ptr(), topk_weights.data_ptr(), out.data_ptr(), n_experts, routing.topk, pairs, hidden, k,
+        EXPERT_QUANT_CODES[wtype], _stream()))
+    return out
+
+
 def moe_gemm_gguf_down_reduce(wtype: int, h: torch.Tensor, down: torch.Tensor, routing: ExpertRouting,
                               topk_weights: torch.Tensor, n_experts: int, hidden: int,
                               residual: torch.Tensor | None = None, down_bias: torch.Tensor | None = None,

@@ -327,6 +327,39 @@ def test_live_count_variants_run_the_first_pairs_only(name):
     assert torch.equal(rows5[slots[:5]], all_rows[slots[:5]])
 
 
+@pytest.mark.parametrize("name", ["q4_k", "q6_k", "mxfp4"])
+def test_experts_over_two_tensors_match_the_one_tensor_launch(name):
+    from loken_amd.moe import (moe_gemm_gguf_down_pairs_over, moe_gemm_gguf_down_reduce_over,
+                               moe_gemm_gguf_gate_up_silu_mul_over)
+    dt = {"q4_k": lib.TYPE_Q4_K, "q6_k": lib.TYPE_Q6_K, **TABLE_TAIL}[name]
+    tokens, hidden, ffn, n_experts, topk, cut = 5, 512, 256, 6, 3, 4
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=65, dt_down=dt, dt_gu=dt, x_scale=4.0)
+    routing = ExpertRouting(dev(ids))
+    flat_w = dev(w.reshape(-1))
+    want_h = moe_gemm_gguf_gate_up_silu_mul(dt, dev(x), dev(gate), dev(up), routing, n_experts, ffn)
+    want = moe_gemm_gguf_down_reduce(dt, want_h, dev(down), routing, flat_w, n_experts, hidden)
+
+    def halves(stack):   # experts 0..cut-1 in one allocation, cut.. in another
+        per = stack.reshape(n_experts, -1)
+        return dev(np.ascontiguousarray(per[:cut])), dev(np.ascontiguousarray(per[cut:]))
+
+    (g0, g1), (u0, u1), (d0, d1) = halves(gate), halves(up), halves(down)
+    h = moe_gemm_gguf_gate_up_silu_mul_over(dt, dev(x), g0, u0, g1, u1, cut, routing, n_experts, ffn)
+    assert torch.equal(h, want_h)
+    # the second pair named by addresses on the card; the host-side ones are then ignored
+    at = torch.tensor([g1.data_ptr(), u1.data_ptr()], dtype=torch.int64, device="cuda")
+    h2 = moe_gemm_gguf_gate_up_silu_mul_over(dt, dev(x), g0, u0, g0, u0, cut, routing, n_experts, ffn, more_at=at)
+    assert torch.equal(h2, want_h)
+    bias = torch.randn((n_experts, hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
+    assert torch.equal(moe_gemm_gguf_down_reduce_over(dt, want_h, d0, d1, cut, routing, flat_w, n_experts, hidden), want)
+    assert torch.equal(moe_gemm_gguf_down_reduce_over(dt, want_h, d0, d1, cut, routing, flat_w, n_experts, hidden, down_bias=bias),
+                       moe_gemm_gguf_down_reduce(dt, want_h, dev(down), routing, flat_w, n_experts, hidden, down_bias=bias))
+    rows = moe_gemm_gguf_down_pairs_over(dt, want_h, d0, d1, cut, routing, flat_w, n_experts, hidden)
+    assert (rows.reshape(tokens, topk, hidden).sum(1) - want).abs().max().item() <= 1e-6 * want.abs().max().item()
+    at_d = torch.tensor([d1.data_ptr(), 0], dtype=torch.int64, device="cuda")
+    assert torch.equal(moe_gemm_gguf_down_pairs_over(dt, want_h, d0, d0, cut, routing, flat_w, n_experts, hidden, more_at=at_d), rows)
+
+
 def test_decode_launchers_refuse_the_codebook_formats():
     tokens, hidden, ffn, n_experts, topk = 2, 512, 256, 4, 2
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=62)
