@@ -432,9 +432,15 @@ __global__ __launch_bounds__(LWG) void moe_rows_legacy_kernel(const uint8_t* __r
                                                               MoeLegacyDims d) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int pair = blockIdx.y;
-    if (d.live != nullptr && pair >= (int)*d.live) return;
+    // the pair's routing and the live count in one round of scalar loads, the launch's fields in the
+    // round before it (asked for where each is first used they arrive in many dependent rounds)
     const int slot = sorted_token_ids[pair];
     const int e = expert_ids[pair];
+    const unsigned int live = d.live != nullptr ? *d.live : 0xFFFFFFFFu;
+    asm volatile("" ::"s"(slot), "s"(e), "s"(live), "s"(d.pairs), "s"(d.experts), "s"(d.cols), "s"(d.nb), "s"(d.k32),
+                 "s"(d.k32_stride), "s"(d.topk), "s"(w0), "s"(w1), "s"(acts), "s"(out), "s"(topk_weights),
+                 "s"(d.slab_bytes), "s"(d.alt.alt0), "s"(d.alt.alt_at), "s"(d.alt.alt_from), "s"(d.act.kind));
+    if ((unsigned int)pair >= live) return;
     if (slot < 0 || slot >= d.pairs) return;   // the whole workgroup leaves together
     float* out_row = out + (size_t)slot * d.cols;
     if (e < 0 || e >= d.experts) {
