@@ -139,7 +139,18 @@ __global__ void sum_topk_kernel(const float* __restrict__ pairs, const float* __
     if (i >= (size_t)tokens * cols) return;
     const size_t token = i / cols, col = i % cols;
     float acc = add ? 0.0f : outputs[i];
-    for (int k = 0; k < topk; ++k) acc += pairs[(token * topk + k) * cols + col];
+    const float* p = pairs + token * topk * cols + col;
+    // four rows' loads in flight at a time; the additions stay in k order
+    int k = 0;
+    for (; k + 4 <= topk; k += 4) {
+        const float p0 = p[(size_t)k * cols], p1 = p[(size_t)(k + 1) * cols], p2 = p[(size_t)(k + 2) * cols],
+                    p3 = p[(size_t)(k + 3) * cols];
+        acc += p0;
+        acc += p1;
+        acc += p2;
+        acc += p3;
+    }
+    for (; k < topk; ++k) acc += p[(size_t)k * cols];
     outputs[i] = add ? acc + add[i] : acc;
 }
 
