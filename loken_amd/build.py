@@ -28,8 +28,18 @@ def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
-def _compile(src: Path) -> Path:
+def _fresh(src: Path, obj: Path) -> bool:
+    """True when `obj` is newer than `src` and every header it may include."""
+    if not obj.exists():
+        return False
+    deps = [src, *CSRC.glob("*.h"), *(HERE.parent / "include").glob("*.h*"), Path(__file__)]
+    return obj.stat().st_mtime > max(d.stat().st_mtime for d in deps)
+
+
+def _compile(src: Path, incremental: bool = False) -> Path:
     obj = CSRC / (src.stem + ".o")
+    if incremental and _fresh(src, obj):
+        return obj
     cmd = [HIPCC, *FLAGS, *PER_FILE_FLAGS.get(src.name, []), "-c", str(src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -37,10 +47,11 @@ def _compile(src: Path) -> Path:
     return obj
 
 
-def build(jobs: int = 8, verbose: bool = False) -> Path:
+def build(jobs: int = 8, verbose: bool = False, incremental: bool = False) -> Path:
+    """Compiles every source (always, unless `incremental`: then only those older than their object)."""
     srcs = sources()
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(srcs)))) as pool:
-        objs = list(pool.map(_compile, srcs))
+        objs = list(pool.map(lambda s: _compile(s, incremental), srcs))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -51,5 +62,5 @@ def build(jobs: int = 8, verbose: bool = False) -> Path:
 
 
 if __name__ == "__main__":
-    build(verbose=True)
+    build(verbose=True, incremental="--incremental" in sys.argv)
     sys.exit(0)

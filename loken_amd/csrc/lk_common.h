@@ -78,6 +78,46 @@ static __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// The sum over each aligned group of LANES (16, 32 or 64) lanes, every lane of the group returns
+// it. Same order of additions as wave_sum: pairs, quads, the two quads of a half row, the two half
+// rows, then rows 0+1 and 2+3, then the two halves of the wave. The rows cross through the two
+// row-swap instructions (v_permlane16_swap, v_permlane32_swap), which stay in the vector unit.
+static __device__ __forceinline__ float swap_add16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+static __device__ __forceinline__ float swap_add32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+template <int LANES>
+static __device__ __forceinline__ float group_sum(float v) {
+    v += dpp_f32<0xB1>(v);
+    v += dpp_f32<0x4E>(v);
+    v += dpp_f32<0x141>(v);
+    v += dpp_f32<0x140>(v);
+    if (LANES >= 32) v = swap_add16(v);
+    if (LANES >= 64) v = swap_add32(v);
+    return v;
+}
+// Two values at once: the even lanes of a group return the group's sum of `x0`, the odd lanes that
+// of `x1`, each with the additions of group_sum in the same order as far as lanes 0 and 1 of the
+// group are concerned, the only lanes whose result is defined (the first step hands every lane its
+// neighbour's value of the row it keeps, the later steps move by even distances only: shifts by 4
+// and 8 inside a row of 16, so lane 0 adds (Q0 + Q1) + (Q2 + Q3) over the row's quads as
+// group_sum's mirrors do).
+template <int LANES>
+static __device__ __forceinline__ float group_sum2(float x0, float x1, bool odd) {
+    const float keep = odd ? x1 : x0, send = odd ? x0 : x1;
+    float v = keep + dpp_f32<0xB1>(send);
+    v += dpp_f32<0x4E>(v);
+    v += dpp_f32<0x104>(v);   // row_shl:4: lane i takes lane i + 4 (the next quad; nothing past the row)
+    v += dpp_f32<0x108>(v);   // row_shl:8
+    if (LANES >= 32) v = swap_add16(v);
+    if (LANES >= 64) v = swap_add32(v);
+    return v;
+}
+
 // Maximum / sum over each aligned group of 8 lanes; every lane of the group returns it.
 // `quad` receives the value after the first two steps (the lane's group of 4).
 static __device__ __forceinline__ float max8(float v) {
@@ -144,6 +184,23 @@ const LkDevice& lk_device();
 // Q4_K x up to any number of Q8_1 rows on the matrix unit (rows_mfma.hip); LK_* status.
 int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y,
                      int ldd, hipStream_t stream);
+
+// Q4_K x ONE activation row with the row's codes held in registers (mmvq_reg.hip): rows of at most
+// 16 super-blocks. Up to four matrices over one activation; `act_f32` non-zero: `act` is the f32
+// row, quantized by every workgroup itself. LK_* status.
+struct LkRegMulti {
+    const uint8_t* vx[4];
+    void* dst[4];
+    const float* bias[4];
+    int n[4];
+    int count;
+};
+bool lk_q4k_reg_serves(int nb);
+int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, int dst_type, hipStream_t stream);
+// The gate/up pair over one activation row: dst = act(gate . x) * (up . x) as f32 / bf16
+// (`dst_q8_1` false) or as Q8_1 blocks of 32 consecutive rows (true; n a multiple of 32).
+int lk_q4k_reg_pair(const uint8_t* gate, const uint8_t* up, const void* act, int act_f32, void* dst, int dst_type,
+                    bool dst_q8_1, int nb, int n, int act_fn, hipStream_t stream);
 
 // The 32-value nibble formats (mmvq_legacy.hip); status LK_*.
 bool lk_is_legacy_type(int wtype);

@@ -34,6 +34,38 @@ static __device__ __forceinline__ void q4k_dots(const uint4& q, const uint4& a_l
     d_hi = dot16(hi, a_hi, d_hi);
 }
 
+// The same with the high nibbles left in place: a byte of (q & 0xF0) ^ 0x80, read as signed, is
+// 16 * nibble - 128, so the dot product with the activation codes is 16 * d_hi - 128 * sum(codes).
+// The caller starts `x_hi` at 128 * (sum of the sub-block's activation codes) and receives
+// 16 * d_hi exactly; the mask and the flip are one three-operand bit instruction per dword where
+// the shift and mask of q4k_dots are two.
+static __device__ __forceinline__ void q4k_dots_biased(const uint4& q, const uint4& a_lo, const uint4& a_hi,
+                                                       uint32_t flip, int& d_lo, int& x_hi) {
+    uint4 lo, hx;
+    lo.x = q.x & 0x0F0F0F0Fu; hx.x = (q.x & 0xF0F0F0F0u) ^ flip;
+    lo.y = q.y & 0x0F0F0F0Fu; hx.y = (q.y & 0xF0F0F0F0u) ^ flip;
+    lo.z = q.z & 0x0F0F0F0Fu; hx.z = (q.z & 0xF0F0F0F0u) ^ flip;
+    lo.w = q.w & 0x0F0F0F0Fu; hx.w = (q.w & 0xF0F0F0F0u) ^ flip;
+    d_lo = dot16(lo, a_lo, d_lo);
+    x_hi = dot16(hx, a_hi, x_hi);
+}
+
+// A lane's share of a Q4_K row from one pair of sub-blocks (2p: low nibbles, 2p + 1: high):
+//   d * (scl * d8a * d_lo + sch * d8b * d_hi) - dmin * (ml * sa + mh * sb),  sa = d8a * sum(codes of 2p), sb likewise.
+// Every engine forms it here, with the roundings written out, so that a row carries the same
+// bits whichever engine served it. `d8b` and `d_hi` may arrive as d8b / 16 and 16 * d_hi
+// (q4k_dots_biased): powers of two move through the roundings unchanged.
+static __device__ __forceinline__ float q4k_pair_share(float d, float dmin, float scl, float sch, float ml, float mh,
+                                                       float d8a, float d8b, float sa, float sb, float d_lo, float d_hi) {
+#pragma clang fp contract(off)
+    const float ka = scl * d8a, kb = sch * d8b;
+    const float hi = kb * d_hi, mb = mh * sb;
+    const float u = __builtin_fmaf(ka, d_lo, hi);
+    const float w = __builtin_fmaf(ml, sa, mb);
+    const float off = dmin * w;
+    return __builtin_fmaf(d, u, -off);
+}
+
 // Q5_K: the same 16 bytes of qs plus the 16 bytes of qh over the same l; bit 2p of a qh byte is
 // the fifth bit (worth 16) of that value in sub-block 2p, bit 2p+1 in sub-block 2p+1
 // (src/tensor/quant_cpu/format/q5_k.rs:66-71). `hs` arrives already shifted right by 2p.
@@ -503,9 +535,8 @@ static __device__ __forceinline__ void rows_q4k(const RowJob<NW>& job, uint8_t* 
                     q4k_dots(f.q0[r], a00, a10, d_lo, d_hi);
                     q4k_dots(f.q1[r], a01, a11, d_lo, d_hi);
                 }
-                const float u = (scl[r] * s4.x) * (float)d_lo + (sch[r] * s4.z) * (float)d_hi;
-                const float w = ml[r] * s4.y + mh[r] * s4.w;
-                acc[r][c] += d[r] * u - dmin[r] * w;
+                acc[r][c] += q4k_pair_share(d[r], dmin[r], scl[r], sch[r], ml[r], mh[r], s4.x, s4.z, s4.y,
+                                            s4.w, (float)d_lo, (float)d_hi);
             }
         }
         if (it == n_iter - 1) {

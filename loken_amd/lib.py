@@ -108,6 +108,9 @@ SIGNATURES.update({
     "loken_argsort_small_u32": (None, [_vp, _vp, _vp, _i, _vp]),
     "loken_topk_softmax": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "loken_dense_q4k_imma_m8_plain": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "lk_probe_empty": (_i, [_i, _vp]),
+    "lk_probe_read": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
+    "lk_probe_mfma": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "loken_moe_mmq_fold": (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
 })
 
