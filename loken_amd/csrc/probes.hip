@@ -94,7 +94,7 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(int iters, int valu, in
 #pragma unroll
     for (int t = 0; t < ACCS; ++t)
 #pragma unroll
-        for (int e = 0; e < (int)(sizeof(typename M::Acc) / 4); ++e) c[t][e] = 0;
+        for (int e = 0; e < (int)(sizeof(typename M::Acc) / 4); ++e) c[t][e] = t + 1;   // distinct, or the four chains are one
     float f[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t) f[t] = (float)(lane + t);
@@ -102,7 +102,10 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(int iters, int valu, in
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
         for (int t = 0; t < ACCS; ++t) {
-            if (matrix_wave) c[t] = M::step(a, b, c[t]);
+            if (matrix_wave) {
+                c[t] = M::step(a, b, c[t]);
+                asm volatile("" : "+v"(c[t]));   // the chain stays as written: nothing folds across rounds
+            }
             if (vector_wave) {
                 for (int v = 0; v < valu; v += 8) {
 #pragma unroll
