@@ -51,6 +51,10 @@ extern "C" {
 #define LK_ERR_TYPE 2       /* weight / activation / output type not served */
 #define LK_ERR_LAUNCH 3     /* the HIP runtime refused the launch */
 #define LK_ERR_NOMEM 4      /* scratch could not be reserved (MoE decode launchers only) */
+#define LK_ERR_SIZE 5       /* the call needs more than the fixed scratch of an entry point that allocates nothing */
+
+/* Bytes of the per-device fixed scratch array behind loken_moe_gemm_gguf_down_reduce_static. */
+#define LK_STATIC_SCRATCH_BYTES (8u << 20)
 
 /* Row padding of a quantized activation, in values (MATRIX_ROW_PADDING,
  * src/tensor/quantized/mod.rs:29-35). */
@@ -381,6 +385,21 @@ int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,
                                     const float* topk_weights, float* outputs, int num_experts, int topk,
                                     int size_m, int size_n, int size_k, int gguf_dtype,
                                     const float* down_bias, const float* add_after, void* stream);
+/* loken_moe_gemm_gguf_down_reduce for callers that cannot allocate device memory (code recording a
+ * HIP graph, serving loops and harnesses that forbid it): same arguments, same kernels, same
+ * result, but the pairs' rows (and the Q8_1 rows of the formats that read them) live in a fixed
+ * array of LK_STATIC_SCRATCH_BYTES that every GPU's copy of the library holds from load until the
+ * process ends. No hipMalloc, hipFree or other allocating call is made. A call that needs more,
+ * size_m * size_n * 4 bytes plus, for the formats that read Q8_1 rows,
+ * size_m * pad512(size_k) / 32 * 36 bytes rounded up to 256, returns LK_ERR_SIZE and launches
+ * nothing. Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
+ * streams, or two host threads) race; calls on one stream are ordered and safe. No counterpart in
+ * the reference. */
+int loken_moe_gemm_gguf_down_reduce_static(const float* inputs, const void* weights,
+                                           const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                           const float* topk_weights, float* outputs, int num_experts,
+                                           int topk, int size_m, int size_n, int size_k, int gguf_dtype,
+                                           const float* down_bias, const float* add_after, void* stream);
 /* outputs[t, c] += sum over k ascending of pairs[(t * topk + k), c] (cuda/moe/moe_gguf.cu:745-752). */
 void loken_moe_sum_topk(const float* pairs, float* outputs, int tokens, int topk, int cols, void* stream);
 /* Q4_K weight [size_n rows, size_k] x plain Q8_1 rows [size_m, size_k / 32 blocks] -> output

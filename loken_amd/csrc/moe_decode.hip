@@ -67,6 +67,32 @@ void* reserve_scratch(size_t bytes, hipStream_t stream) {
     return fresh;
 }
 
+// ---------------------------------------------------------------- static scratch
+// Scratch of the entry point that allocates nothing (loken_moe_gemm_gguf_down_reduce_static): a
+// fixed array in every device's copy of the library image. Each GPU holds its own copy at its own
+// address; the name below is only the host's handle for it, so host code asks the runtime for the
+// device address once per device and passes that.
+constexpr size_t STATIC_SCRATCH_BYTES = LK_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
+
+std::mutex g_static_mu;
+std::vector<std::pair<int, uint8_t*>> g_static_ptr;   // (device, address of `scratch` there)
+
+uint8_t* static_scratch() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    for (const auto& e : g_static_ptr)
+        if (e.first == dev) return e.second;
+    uint8_t* ptr = nullptr;
+    if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    g_static_ptr.emplace_back(dev, ptr);
+    return ptr;
+}
+
 // ---------------------------------------------------------------- kernels
 struct MoeDims {
     int experts, topk, pairs, cols, nb, k32;  // k32: Q8_1 blocks between activation rows
@@ -404,7 +430,7 @@ static int down_impl(const float* inputs, const void* weights, const int32_t* so
                      const int32_t* expert_ids, const float* topk_weights, float* outputs, int num_experts, int topk,
                      int size_m, int size_n, int size_k, int gguf_dtype, const float* down_bias,
                      const float* add_after, const unsigned int* live, float* pair_rows, void* stream,
-                     const LkMoeAlt& alt = LkMoeAlt{}) {
+                     const LkMoeAlt& alt = LkMoeAlt{}, bool from_static = false) {
     if (block_len_of_wire(gguf_dtype) == 0) return LK_ERR_TYPE;
     if (size_m == 0) return LK_OK;
     if (!inputs || !weights || !sorted_token_ids || !expert_ids || !topk_weights || (!outputs && !pair_rows) ||
@@ -416,11 +442,21 @@ static int down_impl(const float* inputs, const void* weights, const int32_t* so
     const size_t pair_bytes = pair_rows ? 0 : (size_t)size_m * size_n * sizeof(float);
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     uint8_t* base = nullptr;
-    if (act_bytes + pair_bytes) {
+    if (from_static) {
+        // nothing is allocated: the device's fixed array, or an error when the call does not fit it
+        if (act_bytes + pair_bytes > STATIC_SCRATCH_BYTES) return LK_ERR_SIZE;
+        base = static_scratch();
+        if (!base) return LK_ERR_LAUNCH;
+    } else if (act_bytes + pair_bytes) {
         base = (uint8_t*)reserve_scratch(act_bytes + pair_bytes, s);
         if (!base) return LK_ERR_NOMEM;
     }
     float* pairs = pair_rows ? pair_rows : (float*)(base + act_bytes);
+    if (from_static && !live) {
+        // the array keeps the last call's rows: a pair the routing leaves out must read as zero
+        const size_t n = (size_t)size_m * size_n;
+        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, pairs, n);
+    }
     if (!as_f32)
         if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, base, size_k, kp, size_m, stream)) return rc;
     if (live) {
@@ -448,6 +484,15 @@ extern "C" int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* 
                                                const float* down_bias, const float* add_after, void* stream) {
     return down_impl(inputs, weights, sorted_token_ids, expert_ids, topk_weights, outputs, num_experts, topk, size_m,
                      size_n, size_k, gguf_dtype, down_bias, add_after, nullptr, nullptr, stream);
+}
+
+extern "C" int loken_moe_gemm_gguf_down_reduce_static(const float* inputs, const void* weights,
+                                                      const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                                      const float* topk_weights, float* outputs, int num_experts,
+                                                      int topk, int size_m, int size_n, int size_k, int gguf_dtype,
+                                                      const float* down_bias, const float* add_after, void* stream) {
+    return down_impl(inputs, weights, sorted_token_ids, expert_ids, topk_weights, outputs, num_experts, topk, size_m,
+                     size_n, size_k, gguf_dtype, down_bias, add_after, nullptr, nullptr, stream, LkMoeAlt{}, true);
 }
 
 extern "C" int loken_moe_gemm_gguf_down_pairs_live(const float* inputs, const void* weights,

@@ -9,8 +9,9 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libloken_gfx950.so"
 
-LK_OK, LK_ERR_ARG, LK_ERR_TYPE, LK_ERR_LAUNCH, LK_ERR_NOMEM = 0, 1, 2, 3, 4
-_ERR_NAMES = {1: "LK_ERR_ARG", 2: "LK_ERR_TYPE", 3: "LK_ERR_LAUNCH", 4: "LK_ERR_NOMEM"}
+LK_OK, LK_ERR_ARG, LK_ERR_TYPE, LK_ERR_LAUNCH, LK_ERR_NOMEM, LK_ERR_SIZE = 0, 1, 2, 3, 4, 5
+_ERR_NAMES = {1: "LK_ERR_ARG", 2: "LK_ERR_TYPE", 3: "LK_ERR_LAUNCH", 4: "LK_ERR_NOMEM", 5: "LK_ERR_SIZE"}
+STATIC_SCRATCH_BYTES = 8 << 20
 
 TYPE_F32, TYPE_F16, TYPE_BF16 = 0, 1, 30
 TYPE_Q4_0, TYPE_Q4_1, TYPE_Q5_0, TYPE_Q5_1 = 2, 3, 6, 7
@@ -67,6 +68,7 @@ SIGNATURES.update({
     "loken_moe_gemm_gguf_down_reduce_two": (_i, [_vp] * 3 + [_i] + [_vp] * 4 + [_i] * 6 + [_vp, _vp, _vp]),
     "loken_moe_gemm_gguf_down_pairs_two": (_i, [_vp] * 3 + [_i] + [_vp] * 5 + [_i] * 6 + [_vp]),
     "loken_moe_gemm_gguf_down_reduce": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp, _vp]),
+    "loken_moe_gemm_gguf_down_reduce_static": (_i, [_vp] * 6 + [_i] * 6 + [_vp, _vp, _vp]),
     "loken_moe_sum_topk": (None, [_vp, _vp, _i, _i, _i, _vp]),
     "loken_stream_scratch_release": (None, []),
     "lk_rmsnorm_q8_1": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _vp]),
