@@ -410,6 +410,12 @@ void loken_moe_sum_topk(const float* pairs, float* outputs, int tokens, int topk
  * 256; weights 16-byte aligned; nothing is launched on a bad argument (void, as the reference's). */
 void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
                                    int size_k, void* stream);
+/* The same launch with a status: LK_ERR_ARG (and nothing launched) for rows too long for the kernel's
+ * scale tables in LDS (beyond roughly 36 thousand values) or a misaligned buffer, where the void
+ * form above can only stay silent. What the host mirror calls, so that such a call goes on to the
+ * tiled matmul instead of returning an untouched buffer. */
+int lk_dense_q4k_rows(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
+                      void* stream);
 /* The router step in front of the expert block: softmax over each row of logits [n_rows,
  * n_experts], the n_expert_used largest probabilities in descending order (ties to the lower
  * expert id) into weights / ids [n_rows, n_expert_used], divided by their sum when with_norm != 0.

@@ -15,7 +15,10 @@
 
 #include <hip/hip_runtime.h>
 
+#include <climits>
+#include <cstdint>
 #include <cstdio>
+#include <exception>
 #include <cstring>
 #include <fcntl.h>
 #include <string>
@@ -101,7 +104,9 @@ GgufValue read_value(Cursor& c, uint32_t type, int depth = 0) {
             const uint64_t count = c.scalar<uint64_t>();
             if (depth > 8) throw Failure{"gguf: arrays nested too deep"};
             v.elem_type = (GgufType)elem;
-            v.items.reserve((size_t)(count < (1u << 20) ? count : (1u << 20)));
+            // an array cannot hold more items than the file has bytes left (every item is at least one)
+            if (count > c.len - c.at) throw Failure{"gguf: array longer than the file"};
+            v.items.reserve((size_t)(count < 4096 ? count : 4096));
             for (uint64_t i = 0; i < count; ++i) v.items.push_back(read_value(c, elem, depth + 1));
             break;
         }
@@ -186,14 +191,25 @@ bool GgufFile::parse(std::string* error) {
             GgufTensor t;
             t.name = c.string();
             const uint32_t n_dims = c.scalar<uint32_t>();
-            for (uint32_t d = 0; d < n_dims; ++d) t.dims.push_back((int64_t)c.scalar<uint64_t>());
+            if (n_dims > 8) throw Failure{"gguf: tensor `" + t.name + "` has " + std::to_string(n_dims) + " dimensions"};
+            uint64_t elements = 1;
+            for (uint32_t d = 0; d < n_dims; ++d) {
+                const uint64_t dim = c.scalar<uint64_t>();
+                if (dim == 0 || dim > (uint64_t)INT64_MAX || __builtin_mul_overflow(elements, dim, &elements) ||
+                    elements > (uint64_t)INT64_MAX)
+                    throw Failure{"gguf: tensor `" + t.name + "` has a dimension the format cannot mean"};
+                t.dims.push_back((int64_t)dim);
+            }
             // stored innermost-first; the rest of the stack states shapes row-major
             for (size_t a = 0, b = t.dims.size(); a + 1 < b; ++a, --b) std::swap(t.dims[a], t.dims[b - 1]);
             t.dtype = (int)c.scalar<uint32_t>();
             t.offset = c.scalar<uint64_t>();
             const DtypeRow* row = dtype_row(t.dtype);
             if (!row) throw Failure{"unsupported ggml dtype id " + std::to_string(t.dtype)};
-            t.bytes = t.elements() / (uint64_t)row->values * (uint64_t)row->bytes;
+            if (elements % (uint64_t)row->values != 0)
+                throw Failure{"gguf: tensor `" + t.name + "` is not whole blocks of its type"};
+            if (__builtin_mul_overflow(elements / (uint64_t)row->values, (uint64_t)row->bytes, &t.bytes))
+                throw Failure{"gguf: tensor `" + t.name + "` is larger than an address"};
             tensor_index_[t.name] = (int)tensors_.size();
             tensors_.push_back(std::move(t));
         }
@@ -202,10 +218,15 @@ bool GgufFile::parse(std::string* error) {
         uint64_t a;
         if (it != kv_index_.end() && values_[it->second].to_u64(&a)) alignment_ = a;
         if (alignment_ == 0) throw Failure{"gguf: general.alignment is zero"};
+        if ((alignment_ & (alignment_ - 1)) != 0 || alignment_ > image_->len)
+            throw Failure{"gguf: general.alignment " + std::to_string(alignment_) + " is not a power of two inside the file"};
         data_offset_ = (c.at + alignment_ - 1) / alignment_ * alignment_;
         return true;
     } catch (const Failure& f) {
         if (error) *error = f.what;
+        return false;
+    } catch (const std::exception& e) {   // a length the standard library refuses, or no memory: never out of an extern "C" call
+        if (error) *error = std::string("gguf: ") + e.what();
         return false;
     }
 }
@@ -514,7 +535,7 @@ extern "C" void* lkh_gguf_linear(void* g, const char* name, int device, void* st
         put_error(err, err_len, "QKernelMatMul: block type " + std::to_string(t.dtype) + " is not served on the card");
         return nullptr;
     }
-    if (t.dims[0] > INT32_MAX || t.dims[1] > INT32_MAX) {
+    if (t.dims[0] <= 0 || t.dims[1] <= 0 || t.dims[0] > INT32_MAX || t.dims[1] > INT32_MAX) {
         put_error(err, err_len, "QKernelMatMul: dimension beyond 2^31");
         return nullptr;
     }

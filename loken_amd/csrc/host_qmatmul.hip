@@ -171,10 +171,15 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
         std::lock_guard<std::mutex> pair(slot.mu);
         if (int rc = reserve(slot, (size_t)rows * blocks * Q81_BLOCK, false, stream)) return rc;
         if (int rc = lk_quantize_q8_1(x, x_type, slot.act, k_, k_, rows, stream)) return rc;
-        loken_dense_q4k_imma_m8_plain(blob_, slot.act, (float*)out, rows, n_, k_, stream);
+        // the launcher with a status (the exported void form drops it): rows too long for its scale
+        // tables in LDS launch nothing, and the call goes on to the tiled matmul below
+        const int rc = lk_dense_q4k_rows(blob_, slot.act, (float*)out, rows, n_, k_, stream);
         mark_used(slot, stream);
-        last_path_ = Path::RowsOnMatrixUnit;
-        return LK_OK;
+        if (rc == LK_OK) {
+            last_path_ = Path::RowsOnMatrixUnit;
+            return LK_OK;
+        }
+        if (rc != LK_ERR_ARG) return rc;
     }
 
     // --- tiled matmul (mmq_forward, kernel_matmul/mmq.rs:21-159)

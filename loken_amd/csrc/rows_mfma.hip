@@ -551,6 +551,11 @@ int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m,
     return launch_rows<4>(a, stream);
 }
 
+extern "C" int lk_dense_q4k_rows(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
+                                 void* stream) {
+    return lk_q4k_rows_mfma(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, (hipStream_t)stream);
+}
+
 extern "C" void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
                                               int size_k, void* stream) {
     (void)lk_q4k_rows_mfma(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, (hipStream_t)stream);

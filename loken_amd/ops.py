@@ -193,7 +193,10 @@ def dense_q4k_rows(weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tenso
         raise ValueError("dense_q4k_rows: k must be a multiple of 256")
     q = quantize_q8_1_rows(x, k_padded=k)
     out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
-    _lib.load().loken_dense_q4k_imma_m8_plain(weight.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k, _stream())
+    # the status-returning form of loken_dense_q4k_imma_m8_plain: a launch it declines must not
+    # come back as an untouched buffer
+    _lib.check("lk_dense_q4k_rows",
+               _lib.load().lk_dense_q4k_rows(weight.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k, _stream()))
     return out
 
 

@@ -185,3 +185,29 @@ def test_tensor_bytes_follow_the_block_table():
 def test_a_repeated_name_finds_the_later_entry_and_keeps_file_order():
     g = gguf.GgufFile(data=gguf.write_bytes([("k", gguf.U32, 1), ("k", gguf.U32, 2)], []))
     assert g.keys() == ["k", "k"] and g.get("k") == 2
+
+
+def test_header_arithmetic_from_the_file_is_not_trusted():
+    q4k = synth.weight(lib.TYPE_Q4_K, 1, 256).tobytes()
+    # dimensions that are zero, negative as int64, or whose product wraps
+    for dims in ((0, 256), (2 ** 63, 2), (2 ** 62, 4), (2 ** 32, 2 ** 32)):
+        with pytest.raises(gguf.GgufError, match="dimension"):
+            gguf.GgufFile(data=gguf.write_bytes([], [("w", dims, 12, q4k)]))
+    with pytest.raises(gguf.GgufError, match="dimensions"):
+        gguf.GgufFile(data=gguf.write_bytes([], [("w", (1,) * 9, 0, b"")]))
+    # a row that is not whole blocks of its type
+    with pytest.raises(gguf.GgufError, match="not whole blocks"):
+        gguf.GgufFile(data=gguf.write_bytes([], [("w", (1, 250), 12, q4k)]))
+    # an alignment that is not a power of two, or larger than the file
+    with pytest.raises(gguf.GgufError, match="power of two"):
+        gguf.GgufFile(data=gguf.write_bytes([("general.alignment", gguf.U32, 48)], []))
+    with pytest.raises(gguf.GgufError, match="power of two"):
+        gguf.GgufFile(data=_with_u64_alignment(2 ** 62))
+    # a 30-byte file that claims an array of 2^60 items: refused before anything is reserved
+    head = b"GGUF" + struct.pack("<IQQ", 3, 0, 1) + s("a") + struct.pack("<IIQ", 9, 4, 2 ** 60)
+    with pytest.raises(gguf.GgufError, match="longer than the file"):
+        gguf.GgufFile(data=head)
+
+
+def _with_u64_alignment(value):
+    return b"GGUF" + struct.pack("<IQQ", 3, 0, 1) + s("general.alignment") + struct.pack("<IQ", 10, value) + b"\0" * 64

@@ -142,3 +142,25 @@ def test_argument_errors_are_status_codes():
     assert l.lkh_qkernel_matmul_forward(h, 16, lib.TYPE_F32, 1, 16, None, 0) == lib.LK_ERR_ARG
     assert l.lkh_qkernel_matmul_forward(h, 16, lib.TYPE_F32, 0, 16, None, 0) == lib.LK_OK
     l.lkh_qkernel_matmul_free(h)
+
+
+def test_rows_too_long_for_the_matrix_unit_rows_kernel_go_to_the_tiles():
+    # 12 rows of 40960 values: the rows kernel's scale tables do not fit LDS; the call must end on the
+    # tiled matmul with a written buffer, and the direct wrapper must raise instead of returning
+    wtype, n, k, rows = lib.TYPE_Q4_K, 64, 40960, 12
+    w = synth.weight(wtype, n, k, seed=84, stream=1)
+    x = synth.activation(rows, k, seed=84)
+    lin = Linear(wtype, dev(w), n, k)
+    try:
+        out = torch.full((rows, n), float("nan"), device="cuda")
+        rc = lib.load().lkh_qkernel_matmul_forward(lin.h, dev(x).data_ptr(), lib.TYPE_F32, rows, out.data_ptr(),
+                                                   torch.cuda.current_stream().cuda_stream, 0)
+        assert rc == 0 and lin.path == "tiled"
+        # 160 blocks per row summed one after the other in f32: held to the row scale, not element by
+        # element (the test is about which kernel ran and that it wrote the buffer)
+        want = oracle.ob_matmul(wtype, x, w, n)
+        assert np.abs(out.cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max() + 1e-4
+    finally:
+        lin.close()
+    with pytest.raises(lib.LokenError):
+        ops.dense_q4k_rows(dev(w), dev(x), n)
