@@ -22,8 +22,13 @@ Two more measurements ride in the same JSON line:
   roofline      the dominant kernel (Q4_K mat-vec): average launch duration over the step's own
                 mix of Q4_K launches, timed with HIP events on the launch stream, against the
                 algorithmic weight bytes per launch and MI355X's 8 TB/s HBM peak.
-  cpu_baseline  the CPU oracle's served path (AVX2 + worker pool restatement of loken's CPU
-                quantized matmul) on a bounded sample of the same workload, on this host's cores.
+  cpu_baseline  loken's served CPU decode path for Q4_K, restated (Q8_K activation, weights repacked
+                eight rows at a time, persistent worker pool), on a bounded sample of the same
+                workload, on this host's cores.
+  gemv_4096     BASELINE config 0 (Q4_K 4096 x 4096, one row) over rotating copies.
+  mmq           BASELINE configs 2a / 2b, the tiled matmul, against the int8 matrix peak.
+  roofline.peak_measured / mmq.peak_measured: what a read-only launch and a register-resident
+                matrix-instruction loop reach on this card (loken_amd/probes.py).
 """
 from __future__ import annotations
 
@@ -61,6 +66,8 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--brief", action="store_true",
+                    help="the decode step and its roofline leg only: no config 0, tiled-matmul or ceiling measurements")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of 1 GiB before the steps: the dispatch of known size that "
                          "scales the FETCH_SIZE / WRITE_SIZE counters of a profiled run")
@@ -151,6 +158,7 @@ def main() -> int:
 
     plan = []       # (fn, args) in launch order: one step
     q4k_plan = []   # the Q4_K mat-vec launches of a step
+    q4k_launch_sizes = []   # their weight bytes, launch by launch
     total_bytes = 0
     q4k_bytes = 0
     keep = []
@@ -173,6 +181,7 @@ def main() -> int:
         if wtype == Q4K:
             q4k_plan.append(item)
             q4k_bytes += nbytes
+            q4k_launch_sizes.append(nbytes)
         return out
 
     import ctypes as C
@@ -195,6 +204,7 @@ def main() -> int:
         if wtype == Q4K:
             q4k_plan.append(item)
             q4k_bytes += nbytes
+            q4k_launch_sizes.append(nbytes)
         return outs[0]
 
     def add_pair(wtype, gate, up, g, n, k):
@@ -209,6 +219,7 @@ def main() -> int:
         if wtype == Q4K:
             q4k_plan.append(item)
             q4k_bytes += nbytes
+            q4k_launch_sizes.append(nbytes)
 
     def add_rows(w, g, n, k):
         """Q4_K x the Q8_1 rows of group `g` on the matrix unit (the activation staged in LDS up to 8 rows)."""
@@ -223,6 +234,7 @@ def main() -> int:
         total_bytes += nbytes
         q4k_plan.append(item)
         q4k_bytes += nbytes
+        q4k_launch_sizes.append(nbytes)
         return out
 
     first_out = None
@@ -323,15 +335,31 @@ def main() -> int:
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
 
     # ------------------------------------------------------------------ roofline leg
-    # The step's own mix of Q4_K mat-vec launches, nothing else on the stream, between two
-    # events on the launch stream.
+    # The step's own mix of Q4_K mat-vec launches, nothing else, recorded into one graph and
+    # replayed between two events on the replaying stream (the stream the kernels run on).
     reps = max(3, min(20, args.steps))
     run(q4k_plan)
     torch.cuda.synchronize()
+    q4k_graph = None
+    if not args.no_graph:
+        side2 = torch.cuda.Stream()
+        q4k_graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side2):
+            cap_q4k = [(fn, a[:-1] + (side2.cuda_stream,)) for fn, a in q4k_plan]
+            run(cap_q4k)
+            side2.synchronize()
+            with torch.cuda.graph(q4k_graph, stream=side2):
+                run(cap_q4k)
+        torch.cuda.synchronize()
+        q4k_graph.replay()
+        torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(reps):
-        run(q4k_plan)
+        if q4k_graph is not None:
+            q4k_graph.replay()
+        else:
+            run(q4k_plan)
     e1.record()
     torch.cuda.synchronize()
     launches = reps * len(q4k_plan)
@@ -341,11 +369,44 @@ def main() -> int:
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC.get((args.plan, b, args.layers)),
-                "kernel": (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
-                           f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if kind == "auto"
+                "kernel": (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<1,1,true> (q+k+v), q4k_reg_kernel<2,1,true> (o), "
+                           f"q4k_reg_pair_kernel<1,true,true> (gate+up)") if kind == "auto" and b == 1
+                          else (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
+                                f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if kind == "auto"
                           else ("q4k_rows_staged_kernel<1> (q, o, gate, up), " if kind == "rows" else "")
                           + f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
-                "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches}
+                "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches,
+                "timed_as": "graph replay of the mix" if q4k_graph is not None else "eager launches"}
+    q4k_launch_bytes = sorted({int(a_bytes) for a_bytes in q4k_launch_sizes})
+
+    # ------------------------------------------------------------------ the rest of the metric, and measured denominators
+    extras = {}
+    used_graph = graph is not None
+    if not args.brief:
+        from loken_amd import probes, workloads
+        used_graph = graph is not None
+        graph = q4k_graph = None   # the step's 5 GB of weights make room for the other workloads
+        keep.clear()
+        torch.cuda.empty_cache()
+        ceil, rb = probes.ceilings()
+        # what a launch that only READS as many bytes as each Q4_K launch of the mix takes (best of a
+        # few grid shapes): the floor a dependent launch of that size has on this card
+        floors = {}
+        for nbytes in q4k_launch_bytes:
+            floors[str(nbytes)] = round(min(rb.rate(nbytes, wgs, pat)[0] for wgs, pat in ((1024, 2), (2048, 4), (2048, 8), (1024, 4))), 3)
+        del rb
+        torch.cuda.empty_cache()
+        mix_floor_us = sum(floors[str(int(sz))] for sz in q4k_launch_sizes) / len(q4k_launch_sizes)
+        roofline["peak_measured"] = {"hbm_read_1gib_gbs": ceil["hbm_read_1gib_gbs"], "empty_launch_us": ceil["empty_launch_us"],
+                                     "read_only_launch_us_by_bytes": floors,
+                                     "read_only_mix_avg_us": round(mix_floor_us, 3),
+                                     "read_only_mix_gbs": round(bytes_per_launch / mix_floor_us / 1e3, 1),
+                                     "frac_of_read_only_mix": round(mix_floor_us / avg_us, 4)}
+        extras["gemv_4096"] = workloads.brief_gemv_4096()
+        extras["mmq"] = {"2a": workloads.brief_mmq("2a"), "2b": workloads.brief_mmq("2b"),
+                         "peak": 5000.0, "unit": "TOP/s",
+                         "peak_measured": {"mfma_i8_32x32x32_tops": ceil["mfma_i8_32x32x32_tops"],
+                                           "mfma_f16_32x32x16_tflops": ceil["mfma_f16_32x32x16_tflops"]}}
 
     # ------------------------------------------------------------------ CPU baseline leg
     cpu = None
@@ -360,22 +421,40 @@ def main() -> int:
         "config": {"workload": f"llama3-8b decode-step quantized linears (Q4_K q,k,v,o,gate,up; Q6_K down; "
                                f"Q8_0 lm_head), batch {b}, {args.layers} layers",
                    "launch_plan": args.plan if kind == args.plan else f"{args.plan} -> {kind}", "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
-                   "hip_graph": graph is not None},
+                   "hip_graph": used_graph},
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "q4k_gemv_gbs": round(achieved, 1), "q4k_gemv_pct_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBS, 2),
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
+    line.update(extras)
     print(json.dumps(line))
     return 0
 
 
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(args, torch, synth, lib, w_dev, out_dev, x_dev, b):
-    """The oracle's threaded served path on layer 0's q_proj-shaped sample, rotating copies."""
+    """loken's served CPU path for Q4_K decode, restated (oracle/cpu_baseline.c): Q8_K activation,
+    weights repacked eight rows at a time, one group dot per eight columns, on a persistent pool of
+    one worker per physical core of this process's CPU set (or OMP_NUM_THREADS when the host sets
+    it: the GPU box gives a job a share of its cores). Layer 0's q_proj-shaped sample, rotating
+    copies past the last-level cache."""
     import numpy as np
 
     import oracle
 
-    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    physical, logical = oracle.cpu_counts()
+    asked = int(os.environ.get("OMP_NUM_THREADS", "0"))
+    threads = oracle.pool_start(min(asked, physical) if asked > 0 else 0)
     n, k = HIDDEN, HIDDEN
     w = w_dev.cpu().numpy()
     x = x_dev.cpu().numpy()
@@ -383,22 +462,27 @@ def cpu_baseline(args, torch, synth, lib, w_dev, out_dev, x_dev, b):
     want = oracle.ob_matmul(oracle.Q4_K, x, w, n)
     got = out_dev.cpu().numpy()
     ok = bool((np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-4).all())
-    # working set past the last-level cache: 16 distinct copies = 151 MB
-    copies = [w.copy() for _ in range(16)]
-    oracle.oa_matmul(oracle.Q4_K, x, copies[0], n, fast_threads=threads)
+    x8 = oracle.repack_q4k_x8(w, n, k)
+    served_ok = bool((np.abs(oracle.oa_matmul_q4k_x8(x, x8, n) - oracle.oa_matmul(oracle.Q4_K, x, w, n))
+                      <= 1e-3 * np.maximum(np.abs(oracle.oa_matmul(oracle.Q4_K, x, w, n)), 1.0)).all())
+    # working set past the last-level cache: 32 distinct copies = 302 MB
+    copies = [x8.copy() for _ in range(32)]
+    oracle.oa_matmul_q4k_x8(x, copies[0], n)
     t0 = time.perf_counter()
     calls = 0
     while time.perf_counter() - t0 < args.cpu_seconds:
         for c in copies:
-            oracle.oa_matmul(oracle.Q4_K, x, c, n, fast_threads=threads)
+            oracle.oa_matmul_q4k_x8(x, c, n)
             calls += 1
     dt = time.perf_counter() - t0
     gbs = calls * synth.weight_bytes(lib.TYPE_Q4_K, n, k) / dt / 1e9
-    kind = "port"
-    return {"value": round(gbs, 2), "unit": "GB/s", "cores": threads, "kind": kind,
-            "sample": f"Q4_K mat-vec {n}x{k}, batch {b}, {calls} calls over 16 rotating copies "
-                      f"({dt:.1f} s), AVX2 + {threads}-thread pool restatement of the CPU path "
-                      f"(Q8_K activations)",
+    return {"value": round(gbs, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model(), "physical_cores": physical, "logical_cpus": logical,
+            "threads_source": "OMP_NUM_THREADS" if asked > 0 else "one per physical core",
+            "sample": f"Q4_K mat-vec {n}x{k}, batch {b}, {calls} calls over 32 rotating copies of the repacked weights "
+                      f"({dt:.1f} s): Q8_K activation, eight-row repacked weights, group dot per eight columns "
+                      f"(loken's served decode path, restated in C with AVX2), persistent pool of {threads} threads",
+            "served_path_vs_scalar_oracle": "ok" if served_ok else "FAILED",
             "gpu_parity_on_sample": "ok" if ok else "FAILED"}
 
 

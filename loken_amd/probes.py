@@ -104,7 +104,7 @@ def mfma_rate(kind=0, workgroups=2048, iters=2000, valu_per_mfma=0, mode=0):
 def ceilings(quick=True):
     """The denominators bench.py reports: streaming read over 1 GiB and the int8 matrix loop."""
     rb = ReadBuffers()
-    best = max(rb.rate(1 << 30, wgs, pat)[1] for wgs, pat in ((2048, 4), (4096, 4), (2048, 8)))
+    best = max(rb.rate(1 << 30, wgs, pat)[1] for wgs, pat in ((2048, 1), (4096, 1), (1024, 2)))
     tops, _ = mfma_rate(0)
     f16, _ = mfma_rate(1)
     return {"hbm_read_1gib_gbs": round(best, 1), "hbm_read_frac_of_8tbs": round(best / HBM_PEAK_GBS, 4),

@@ -502,6 +502,83 @@ def decode_1p7b(args, dev):
                  "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline)
 
 
+# ---------------------------------------------------------------------------- short forms for the default line
+def brief_gemv_4096(launches=64, replays=30):
+    """Config 0 for the default benchmark line: the Q4_K 4096 x 4096 mat-vec at one row as a graph of
+    `launches` launches over that many rotating copies (604 MB at 64: past twice the last-level
+    cache), from a Q8_1 row and from the f32 row quantized in the kernel."""
+    L = lib.load()
+    dev = torch.device("cuda:0")
+    n = k = 4096
+    nbytes = synth.weight_bytes(Q4K, n, k)
+    base = torch.from_numpy(synth.weight(Q4K, n, k, seed=0, stream=0)).to(dev).reshape(-1)
+    copies = [base.clone() for _ in range(launches)]
+    x = torch.from_numpy(synth.activation(1, k, seed=0)).to(dev)
+    q = ops.quantize_q8_1_rows(x)
+    out = torch.empty((1, n), device=dev)
+    keep = []
+
+    def plain():
+        s2 = torch.cuda.current_stream().cuda_stream
+        for w in copies:
+            check(L.lk_mmvq(Q4K, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, 1, q.shape[1], n, None, 0,
+                            s2), "lk_mmvq")
+
+    def fused():
+        s2 = torch.cuda.current_stream().cuda_stream
+        dst = (lib.C.c_void_p * 1)(out.data_ptr())
+        nn = (lib.C.c_int * 1)(n)
+        for w in copies:
+            vx = (lib.C.c_void_p * 1)(w.data_ptr())
+            keep.append(vx)
+            check(L.lk_mmvq_fused(Q4K, 1, vx, x.data_ptr(), x.stride(0), dst, lib.TYPE_F32, k, nn, 1, n, None, s2),
+                  "lk_mmvq_fused")
+
+    us = float(np.median(time_replays(capture(plain), replays))) / launches
+    us_fused = float(np.median(time_replays(capture(fused), replays))) / launches
+    want = None
+    return {"workload": "Q4_K 4096x4096 mat-vec, one row, seed 0, graph of %d launches over %d rotating copies" % (launches, launches),
+            "weight_bytes": nbytes, "us_per_launch": round(us, 3), "gbs": round(nbytes / us / 1e3, 1),
+            "frac_of_8tbs": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+            "f32_activation_quantized_in_kernel": {"us_per_launch": round(us_fused, 3),
+                                                   "gbs": round(nbytes / us_fused / 1e3, 1)}}
+
+
+def brief_mmq(shape, launches=30):
+    """Configs 2a / 2b for the default benchmark line: median of event-bracketed launches of the tiled
+    matmul alone and of quantizer + matmul."""
+    L = lib.load()
+    dev = torch.device("cuda:0")
+    wtype, m, k, n = {"2a": (Q4K, 512, 4096, 14336), "2b": (Q6K, 2048, 14336, 4096)}[shape]
+    mk = Maker(dev)
+    w = mk.make(wtype, n, k)
+    x = mk.randn(m, k)
+    out = torch.empty((m, n), device=dev)
+    ws = ops.mmq_quantize(wtype, x)
+    quantizer = getattr(L, ops.MMQ_QUANTIZER[wtype])
+    launcher = getattr(L, ops.MMQ_LAUNCHER[wtype])
+    info = ops.MMQ_DEVICE_INFO
+    s = torch.cuda.current_stream().cuda_stream
+    k_padded = ops.pad_to(ops.pad_to(k, 512), 128)
+
+    def quant():
+        quantizer(x.data_ptr(), None, ws.data_ptr(), 0, k, x.stride(0), 0, 0, k_padded, m, 1, 1, s)
+
+    def matmul():
+        if launcher(None, w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
+                    info["cc"], info["nsm"], info["smpbo"], info["warp_size"], s) == 0:
+            raise lib.LokenError(ops.MMQ_LAUNCHER[wtype], lib.LK_ERR_ARG)
+
+    mm = float(np.median(time_launches(lambda i: matmul(), launches, warm=5)))
+    both = float(np.median(time_launches(lambda i: (quant(), matmul()), launches, warm=5)))
+    op_count = 2.0 * m * k * n
+    return {"workload": f"tiled matmul {m} rows x {k} -> {n}, {NAMES[wtype]}", "ops": int(op_count),
+            "kernel": "q4k_f16_dense_kernel (exact integers on f16 operands)" if wtype == Q4K else "mmq_dense_kernel<MmqQ6K,128,1>",
+            "matmul_us": round(mm, 2), "tops": round(op_count / mm / 1e6, 1),
+            "frac_of_int8_peak": round(op_count / mm / 1e6 / INT8_PEAK_TOPS, 4),
+            "quantize_plus_matmul_us": round(both, 2), "tops_with_quantizer": round(op_count / both / 1e6, 1)}
+
+
 def run(args) -> int:
     if not torch.cuda.is_available():
         raise SystemExit("bench.py: no GPU visible")

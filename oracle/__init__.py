@@ -73,6 +73,10 @@ def _declare(l: C.CDLL) -> None:
     l.lko_group_by_expert.restype = None
     l.lko_moe_forward.argtypes = [_i, _i, _i, _sz, _sz, _sz, _sz, _sz] + [_vp] * 8
     l.lko_cpu_has_avx2.restype = _i
+    l.lko_pool_start.argtypes = [_i]
+    l.lko_repack_q4k_x8.argtypes = [_vp, _sz, _sz, _vp]
+    l.lko_repack_q4k_x8.restype = None
+    l.oa_matmul_q4k_x8.argtypes = [_sz, _sz, _sz, _vp, _vp, _vp]
     l.lko_inv_rms_wide.restype = C.c_float
     l.lko_inv_rms_wide.argtypes = [_vp, _sz, C.c_float]
     l.lko_norm_rows.restype = None
@@ -171,6 +175,33 @@ def oa_matmul(dtype: int, lhs, rhs, n: int, *, fast_threads: int = 0, exact: boo
     else:
         _check(lib().oa_matmul(dtype, m, k, n, _p(lhs), _p(rhs), rhs.size, _p(dst)))
     return dst
+
+
+def repack_q4k_x8(rhs, n: int, k: int) -> np.ndarray:
+    """Q4_K rows `[n, k/256]` (n a multiple of 8) -> the eight-row group blocks the served CPU path reads."""
+    rhs = _u8(rhs)
+    nb = k // 256
+    out = np.empty((n // 8) * nb * 1152, np.uint8)
+    lib().lko_repack_q4k_x8(_p(rhs), n, nb, _p(out))
+    return out
+
+
+def oa_matmul_q4k_x8(lhs, x8: np.ndarray, n: int) -> np.ndarray:
+    """The served Q4_K CPU path: Q8_K activations against repacked weights on the persistent pool."""
+    lhs = _f32(lhs)
+    m, k = lhs.shape
+    dst = np.empty((m, n), np.float32)
+    _check(lib().oa_matmul_q4k_x8(m, k, n, _p(lhs), _p(x8), _p(dst)))
+    return dst
+
+
+def pool_start(threads: int = 0) -> int:
+    return lib().lko_pool_start(threads)
+
+
+def cpu_counts() -> tuple[int, int]:
+    """(physical cores, logical CPUs) this process may run on."""
+    return lib().lko_physical_cores(), lib().lko_logical_cpus()
 
 
 def ob_matmul(dtype: int, lhs, rhs, n: int) -> np.ndarray:

@@ -13,6 +13,10 @@
  * only by float summation order; tests hold it to the reference's own vector-vs-scalar bound
  * 1e-3 * max(|ref|, 1) (avx/parity.rs:50-56).
  *
+ * Two drivers: the per-column dot above for every format (oa_matmul_fast), and the path loken
+ * actually serves Q4_K with (oa_matmul_q4k_x8): rows repacked eight at a time and one group dot per
+ * eight output columns. Both run on ONE persistent pool of workers (no thread is created per call).
+ *
  * Falls back to the scalar oracle when the CPU lacks AVX2.
  */
 #define _GNU_SOURCE
@@ -20,7 +24,9 @@
 
 #include <immintrin.h>
 #include <pthread.h>
+#include <sched.h>
 #include <stdatomic.h>
+#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -135,6 +141,280 @@ static float dot_q80_q80_avx2(const uint8_t* w, const uint8_t* y, size_t nb) {
     return _mm_cvtss_f32(s);
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * Persistent worker pool (the shape of gemv_pool::Pool, src/tensor/quant_cpu/gemv_pool.rs:74-365):
+ * workers are created once, one per physical core the process may run on (:186-203), and stay
+ * alive; a job is published by bumping a generation counter, workers spin on it for a bounded
+ * budget and then sleep on a condition variable; chunks are grabbed from one atomic counter and the
+ * caller works alongside the workers and returns when every chunk has been finished.
+ * ------------------------------------------------------------------------------------------- */
+typedef void (*chunk_fn)(void* ctx, size_t chunk);
+
+typedef struct {
+    pthread_t* tid;
+    int workers;                 /* threads beside the caller */
+    atomic_uint generation;      /* bumped once per job */
+    atomic_size_t next, done;    /* next chunk to grab; chunks finished */
+    size_t n_chunks;
+    chunk_fn fn;
+    void* ctx;
+    pthread_mutex_t mu;
+    pthread_cond_t wake;
+    atomic_int sleepers;
+    atomic_int stop;
+} pool_t;
+
+static pool_t g_pool;
+static pthread_mutex_t g_pool_mu = PTHREAD_MUTEX_INITIALIZER;
+static int g_pool_threads = 0;
+#define POOL_SPIN 20000   /* polls of the generation counter before a worker goes to sleep */
+
+static void pool_drain(pool_t* p) {
+    for (;;) {
+        const size_t c = atomic_fetch_add(&p->next, 1);
+        if (c >= p->n_chunks) break;
+        p->fn(p->ctx, c);
+        atomic_fetch_add(&p->done, 1);
+    }
+}
+
+static void* pool_worker(void* arg) {
+    pool_t* p = (pool_t*)arg;
+    unsigned seen = atomic_load(&p->generation);
+    for (;;) {
+        int spins = 0;
+        while (atomic_load_explicit(&p->generation, memory_order_acquire) == seen && !atomic_load(&p->stop)) {
+            if (++spins < POOL_SPIN) {
+                _mm_pause();
+                continue;
+            }
+            pthread_mutex_lock(&p->mu);
+            atomic_fetch_add(&p->sleepers, 1);
+            while (atomic_load(&p->generation) == seen && !atomic_load(&p->stop)) pthread_cond_wait(&p->wake, &p->mu);
+            atomic_fetch_sub(&p->sleepers, 1);
+            pthread_mutex_unlock(&p->mu);
+        }
+        if (atomic_load(&p->stop)) return NULL;
+        seen = atomic_load(&p->generation);
+        pool_drain(p);
+    }
+}
+
+/* Physical cores this process may run on: distinct first entries of the siblings lists of the
+ * CPUs in the affinity mask. Falls back to the number of CPUs in the mask. */
+int lko_physical_cores(void) {
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    if (sched_getaffinity(0, sizeof set, &set) != 0) return 1;
+    int cores = 0, logical = 0;
+    for (int cpu = 0; cpu < CPU_SETSIZE; ++cpu) {
+        if (!CPU_ISSET(cpu, &set)) continue;
+        ++logical;
+        char path[128];
+        snprintf(path, sizeof path, "/sys/devices/system/cpu/cpu%d/topology/thread_siblings_list", cpu);
+        FILE* f = fopen(path, "r");
+        int first = cpu;
+        if (f) {
+            if (fscanf(f, "%d", &first) != 1) first = cpu;
+            fclose(f);
+        }
+        if (first == cpu) ++cores;   /* a core is counted at its lowest-numbered sibling */
+    }
+    return cores > 0 ? cores : (logical > 0 ? logical : 1);
+}
+int lko_logical_cpus(void) {
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    if (sched_getaffinity(0, sizeof set, &set) != 0) return 1;
+    return CPU_COUNT(&set);
+}
+
+/* Starts (or resizes) the pool: `threads` callers-plus-workers in all; 0 = one per physical core.
+ * Returns the thread count in use. */
+int lko_pool_start(int threads) {
+    if (threads <= 0) threads = lko_physical_cores();
+    pthread_mutex_lock(&g_pool_mu);
+    if (g_pool_threads != threads) {
+        if (g_pool_threads > 0) {   /* stop the old workers */
+            atomic_store(&g_pool.stop, 1);
+            pthread_mutex_lock(&g_pool.mu);
+            pthread_cond_broadcast(&g_pool.wake);
+            pthread_mutex_unlock(&g_pool.mu);
+            for (int t = 0; t < g_pool.workers; ++t) pthread_join(g_pool.tid[t], NULL);
+            free(g_pool.tid);
+            pthread_mutex_destroy(&g_pool.mu);
+            pthread_cond_destroy(&g_pool.wake);
+        }
+        memset(&g_pool, 0, sizeof g_pool);
+        pthread_mutex_init(&g_pool.mu, NULL);
+        pthread_cond_init(&g_pool.wake, NULL);
+        g_pool.workers = threads - 1;
+        g_pool.tid = (pthread_t*)calloc((size_t)(threads > 1 ? threads - 1 : 1), sizeof(pthread_t));
+        int started = 0;
+        if (g_pool.tid)
+            for (; started < g_pool.workers; ++started)
+                if (pthread_create(&g_pool.tid[started], NULL, pool_worker, &g_pool) != 0) break;
+        g_pool.workers = started;
+        g_pool_threads = started + 1;
+    }
+    const int n = g_pool_threads;
+    pthread_mutex_unlock(&g_pool_mu);
+    return n;
+}
+
+/* Runs fn(ctx, c) for c in [0, n_chunks) on the pool; returns when all are done. One job at a time. */
+static void pool_run(size_t n_chunks, chunk_fn fn, void* ctx) {
+    pool_t* p = &g_pool;
+    p->fn = fn;
+    p->ctx = ctx;
+    p->n_chunks = n_chunks;
+    atomic_store(&p->next, 0);
+    atomic_store(&p->done, 0);
+    atomic_fetch_add_explicit(&p->generation, 1, memory_order_release);
+    if (atomic_load(&p->sleepers) > 0) {
+        pthread_mutex_lock(&p->mu);
+        pthread_cond_broadcast(&p->wake);
+        pthread_mutex_unlock(&p->mu);
+    }
+    pool_drain(p);
+    while (atomic_load_explicit(&p->done, memory_order_acquire) < n_chunks) _mm_pause();
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * The served Q4_K path: rows repacked eight at a time (BlockQ4Kx8, repack_q4k.rs:17-68) and one
+ * group dot per eight output columns (gemv_group_scalar states the sums, :174-219; the AVX2
+ * form is gemv_group_avx2_plain, :913-...; driver matmul_q4k_plain_pre, drivers.rs:61-95).
+ *
+ * Group block (2*8 f16 d and dmin, 8 x 12 packed scale bytes, 1024 bytes of nibbles): source byte
+ * p of row j of the eight sits at qs[(p / 8) * 64 + j * 8 + p % 8], so step kk of the sixteen
+ * holds eight bytes of every row side by side: values 8 (kk % 4) .. + 8 of sub-blocks 2 (kk / 4)
+ * (low nibbles) and 2 (kk / 4) + 1 (high nibbles).
+ *   out[j] = sum over blocks of  d_j * act.d * sum_s sc_js * dot_js  -  dmin_j * act.d * sum_s m_js * bsum_s
+ * with every integer exact and the two float sums kept apart until the end, as the reference's.
+ * ------------------------------------------------------------------------------------------- */
+#define LKO_Q4KX8_BYTES (32 + 96 + 1024)
+
+void lko_repack_q4k_x8(const uint8_t* rhs, size_t n, size_t nb, uint8_t* out) {
+    for (size_t g = 0; g < n / 8; ++g)
+        for (size_t b = 0; b < nb; ++b) {
+            uint8_t* dst = out + (g * nb + b) * LKO_Q4KX8_BYTES;
+            for (size_t j = 0; j < 8; ++j) {
+                const uint8_t* src = rhs + ((g * 8 + j) * nb + b) * LKO_Q4K_BYTES;
+                memcpy(dst + 2 * j, src, 2);             /* d */
+                memcpy(dst + 16 + 2 * j, src + 2, 2);    /* dmin */
+                memcpy(dst + 32 + 12 * j, src + 4, 12);  /* the row's own packed scales */
+                for (size_t p = 0; p < 128; ++p) dst[128 + (p / 8) * 64 + j * 8 + (p % 8)] = src[16 + p];
+            }
+        }
+}
+
+/* Eight output columns from one group's `nb` blocks against one Q8_K row. */
+static void gemv_group_q4k_x8(const uint8_t* grp, const uint8_t* y, size_t nb, float out[8]) {
+    const __m256i nib = _mm256_set1_epi8(0x0F);
+    __m256 acc = _mm256_setzero_ps(), acc_min = _mm256_setzero_ps();
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* blk = grp + b * LKO_Q4KX8_BYTES;
+        const uint8_t* yb = y + b * LKO_Q8K_BYTES;
+        float yd;
+        memcpy(&yd, yb, 4);
+        const int8_t* acts = (const int8_t*)(yb + 4);
+        const int16_t* bsums = (const int16_t*)(yb + 260);
+        /* the eight rows' scales and mins, sub-block major: tab[s][j] */
+        int16_t sc[8][8], mn[8][8];
+        for (int j = 0; j < 8; ++j) {
+            uint8_t s8[8], m8[8];
+            lko_unpack_scales_mins(blk + 32 + 12 * j, s8, m8);
+            for (int s = 0; s < 8; ++s) { sc[s][j] = s8[s]; mn[s][j] = m8[s]; }
+        }
+        /* rows 0-3 in `ia`, rows 4-7 in `ib`: two int32 partials per row */
+        __m256i ia = _mm256_setzero_si256(), ib = _mm256_setzero_si256();
+        const uint8_t* qs = blk + 128;
+        for (int pair = 0; pair < 4; ++pair) {
+            __m256i lo_a = _mm256_setzero_si256(), lo_b = lo_a, hi_a = lo_a, hi_b = lo_a;
+            for (int kk = 0; kk < 4; ++kk) {
+                const __m256i qa = _mm256_loadu_si256((const __m256i*)(qs + (pair * 4 + kk) * 64));
+                const __m256i qb = _mm256_loadu_si256((const __m256i*)(qs + (pair * 4 + kk) * 64 + 32));
+                int64_t a_lo8, a_hi8;   /* the same eight activation codes against every row */
+                memcpy(&a_lo8, acts + pair * 64 + kk * 8, 8);
+                memcpy(&a_hi8, acts + pair * 64 + 32 + kk * 8, 8);
+                const __m256i a_lo = _mm256_set1_epi64x(a_lo8), a_hi = _mm256_set1_epi64x(a_hi8);
+                /* sixteen-bit partials: at most 4 steps x 2 products x 15 x 127, inside int16 */
+                lo_a = _mm256_add_epi16(lo_a, _mm256_maddubs_epi16(_mm256_and_si256(qa, nib), a_lo));
+                lo_b = _mm256_add_epi16(lo_b, _mm256_maddubs_epi16(_mm256_and_si256(qb, nib), a_lo));
+                hi_a = _mm256_add_epi16(hi_a, _mm256_maddubs_epi16(_mm256_and_si256(_mm256_srli_epi16(qa, 4), nib), a_hi));
+                hi_b = _mm256_add_epi16(hi_b, _mm256_maddubs_epi16(_mm256_and_si256(_mm256_srli_epi16(qb, 4), nib), a_hi));
+            }
+            /* each row's scale over its four sixteen-bit lanes: multiply, widen and pair-add in one */
+            const int16_t* s0 = sc[2 * pair];
+            const int16_t* s1 = sc[2 * pair + 1];
+#define ROWS4(t, o) _mm256_setr_epi16(t[o], t[o], t[o], t[o], t[o + 1], t[o + 1], t[o + 1], t[o + 1], t[o + 2], t[o + 2], \
+                                      t[o + 2], t[o + 2], t[o + 3], t[o + 3], t[o + 3], t[o + 3])
+            ia = _mm256_add_epi32(ia, _mm256_add_epi32(_mm256_madd_epi16(lo_a, ROWS4(s0, 0)), _mm256_madd_epi16(hi_a, ROWS4(s1, 0))));
+            ib = _mm256_add_epi32(ib, _mm256_add_epi32(_mm256_madd_epi16(lo_b, ROWS4(s0, 4)), _mm256_madd_epi16(hi_b, ROWS4(s1, 4))));
+#undef ROWS4
+        }
+        /* [r0 r0 r1 r1 | r2 r2 r3 r3] and [r4 ..] -> one int32 per row, rows in lane order */
+        const __m256i h = _mm256_hadd_epi32(ia, ib);   /* r0 r1 r4 r5 | r2 r3 r6 r7 */
+        const __m256i sums = _mm256_permutevar8x32_epi32(h, _mm256_setr_epi32(0, 1, 4, 5, 2, 3, 6, 7));
+        /* the min term: sum_s m_js * (bsums[2s] + bsums[2s+1]) */
+        __m256i im = _mm256_setzero_si256();
+        for (int s = 0; s < 8; ++s) {
+            const int32_t bs = (int32_t)bsums[2 * s] + bsums[2 * s + 1];
+            const __m256i m = _mm256_cvtepi16_epi32(_mm_loadu_si128((const __m128i*)mn[s]));
+            im = _mm256_add_epi32(im, _mm256_mullo_epi32(m, _mm256_set1_epi32(bs)));
+        }
+        const __m256 d = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)blk));
+        const __m256 dmin = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)(blk + 16)));
+        const __m256 ydv = _mm256_set1_ps(yd);
+        acc = _mm256_fmadd_ps(_mm256_cvtepi32_ps(sums), _mm256_mul_ps(d, ydv), acc);
+        acc_min = _mm256_fmadd_ps(_mm256_cvtepi32_ps(im), _mm256_mul_ps(dmin, ydv), acc_min);
+    }
+    _mm256_storeu_ps(out, _mm256_sub_ps(acc, acc_min));
+}
+
+typedef struct {
+    size_t m, n, nb, groups, chunk;
+    const uint8_t* x8;
+    const uint8_t* act;   /* m rows of nb Q8_K blocks */
+    float* dst;
+} x8_job_t;
+
+static void x8_chunk(void* ctx, size_t c) {
+    const x8_job_t* j = (const x8_job_t*)ctx;
+    const size_t g1 = (c + 1) * j->chunk < j->groups ? (c + 1) * j->chunk : j->groups;
+    for (size_t g = c * j->chunk; g < g1; ++g) {
+        const uint8_t* grp = j->x8 + g * j->nb * LKO_Q4KX8_BYTES;
+        /* every activation row against the group while its blocks are in cache */
+        for (size_t r = 0; r < j->m; ++r) {
+            float out8[8];
+            gemv_group_q4k_x8(grp, j->act + r * j->nb * LKO_Q8K_BYTES, j->nb, out8);
+            memcpy(j->dst + r * j->n + g * 8, out8, sizeof out8);
+        }
+    }
+}
+
+/* dst[m, n] = lhs[m, k] x repacked Q4_K weights (`x8` from lko_repack_q4k_x8; n a multiple of 8),
+ * Q8_K activations, on the persistent pool (started on first use, one worker per physical core
+ * unless lko_pool_start chose otherwise). Column groups are dealt one chunk per thread
+ * (drivers.rs:71-76). Returns 0, -1 (k not whole blocks), -4 (n not a multiple of 8), -5 (no memory). */
+int oa_matmul_q4k_x8(size_t m, size_t k, size_t n, const float* lhs, const uint8_t* x8, float* dst) {
+    if (k % LKO_QK_K != 0) return -1;
+    if (n % 8 != 0) return -4;
+    if (!lko_cpu_has_avx2()) return -3;
+    const int threads = lko_pool_start(g_pool_threads > 0 ? g_pool_threads : 0);
+    x8_job_t job;
+    job.m = m; job.n = n; job.nb = k / LKO_QK_K; job.groups = n / 8; job.x8 = x8; job.dst = dst;
+    uint8_t* act = (uint8_t*)malloc(job.nb * LKO_Q8K_BYTES * (m ? m : 1));
+    if (!act) return -5;
+    for (size_t r = 0; r < m; ++r) lko_quantize_q8_k(lhs + r * k, k, act + r * job.nb * LKO_Q8K_BYTES);
+    job.act = act;
+    job.chunk = (job.groups + (size_t)threads - 1) / (size_t)threads;
+    if (job.chunk < 1) job.chunk = 1;
+    pool_run((job.groups + job.chunk - 1) / job.chunk, x8_chunk, &job);
+    free(act);
+    return 0;
+}
+
 typedef float (*row_dot_fn)(const uint8_t*, const uint8_t*, size_t);
 
 typedef struct {
@@ -143,24 +423,18 @@ typedef struct {
     const uint8_t* rhs;
     const uint8_t* act;
     float* dst;
-    atomic_size_t next;
 } job_t;
 
-static void* worker(void* arg) {
-    job_t* j = (job_t*)arg;
-    for (;;) {
-        const size_t c = atomic_fetch_add(&j->next, 1);
-        if (c >= j->n_chunks) break;
-        const size_t col0 = c * j->chunk_cols;
-        const size_t col1 = col0 + j->chunk_cols < j->n ? col0 + j->chunk_cols : j->n;
-        for (size_t r0 = 0; r0 < j->m; r0 += 8) {
-            const size_t r1 = r0 + 8 < j->m ? r0 + 8 : j->m;
-            for (size_t col = col0; col < col1; ++col)
-                for (size_t r = r0; r < r1; ++r)
-                    j->dst[r * j->n + col] = j->dot(j->rhs + col * j->wrow, j->act + r * j->arow, j->nb);
-        }
+static void column_chunk(void* ctx, size_t c) {
+    const job_t* j = (const job_t*)ctx;
+    const size_t col0 = c * j->chunk_cols;
+    const size_t col1 = col0 + j->chunk_cols < j->n ? col0 + j->chunk_cols : j->n;
+    for (size_t r0 = 0; r0 < j->m; r0 += 8) {
+        const size_t r1 = r0 + 8 < j->m ? r0 + 8 : j->m;
+        for (size_t col = col0; col < col1; ++col)
+            for (size_t r = r0; r < r1; ++r)
+                j->dst[r * j->n + col] = j->dot(j->rhs + col * j->wrow, j->act + r * j->arow, j->nb);
     }
-    return NULL;
 }
 
 int lko_cpu_has_avx2(void) {
@@ -182,11 +456,12 @@ int oa_matmul_fast(int dtype, size_t m, size_t k, size_t n, const float* lhs,
     }
     if (k % blk != 0) return -1;
     if (rhs_bytes != n * (k / blk) * wblk) return -2;
-    if (threads < 1) threads = 1;
+    threads = lko_pool_start(threads < 1 ? 1 : threads);
     job_t job;
     job.dot = dot; job.m = m; job.n = n; job.nb = k / blk; job.wrow = job.nb * wblk;
     job.arow = (k / aval) * ablk; job.rhs = rhs; job.dst = dst;
     uint8_t* act = (uint8_t*)malloc(job.arow * (m ? m : 1));
+    if (!act) return -5;
     for (size_t r = 0; r < m; ++r) {
         if (dtype == LKO_Q8_0) lko_quantize_q8_0(lhs + r * k, k, act + r * job.arow);
         else lko_quantize_q8_k(lhs + r * k, k, act + r * job.arow);
@@ -198,12 +473,7 @@ int oa_matmul_fast(int dtype, size_t m, size_t k, size_t n, const float* lhs,
     if (chunk > n) chunk = n ? n : 1;
     job.chunk_cols = chunk;
     job.n_chunks = (n + chunk - 1) / chunk;
-    atomic_init(&job.next, 0);
-    pthread_t* tid = (pthread_t*)malloc(sizeof(pthread_t) * (size_t)threads);
-    for (int t = 1; t < threads; ++t) pthread_create(&tid[t], NULL, worker, &job);
-    worker(&job);
-    for (int t = 1; t < threads; ++t) pthread_join(tid[t], NULL);
-    free(tid);
+    pool_run(job.n_chunks, column_chunk, &job);
     free(act);
     return 0;
 }

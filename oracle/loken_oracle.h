@@ -136,6 +136,16 @@ void lko_split_act_mul(const float* gu, float* out, size_t n, size_t rows, int a
 
 /* ---- timed CPU baseline (cpu_baseline.c): O-A semantics, AVX2 kernels, worker pool ---- */
 int lko_cpu_has_avx2(void);
+/* The worker pool both drivers run on: persistent, one worker per physical core of the affinity
+ * mask unless `threads` says otherwise (gemv_pool.rs:186-203). Returns the threads in use. */
+int lko_pool_start(int threads);
+int lko_physical_cores(void);
+int lko_logical_cpus(void);
+/* BlockQ4Kx8::repack (repack_q4k.rs:44-68): n rows (a multiple of 8) of nb Q4_K blocks into
+ * n / 8 * nb group blocks of 1152 bytes; `out` holds that many. */
+void lko_repack_q4k_x8(const uint8_t* rhs, size_t n, size_t nb, uint8_t* out);
+/* The served Q4_K path over the repacked weights (matmul_q4k_plain_pre, drivers.rs:61-95). */
+int oa_matmul_q4k_x8(size_t m, size_t k, size_t n, const float* lhs, const uint8_t* x8, float* dst);
 int oa_matmul_fast(int dtype, size_t m, size_t k, size_t n, const float* lhs,
                    const uint8_t* rhs, size_t rhs_bytes, float* dst, int threads);
 

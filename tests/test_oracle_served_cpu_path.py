@@ -1,0 +1,94 @@
+"""The timed CPU baseline's served Q4_K path (rows repacked eight at a time, one group dot per eight
+columns, persistent worker pool) against the scalar oracle it is a faster statement of.
+
+  * the repack is the reference's index map (repack_q4k.rs:44-68), checked byte by byte;
+  * on inputs whose every factor is exactly representable the group dot returns the exact integer
+    combination of the scalar definition (gemv_group_scalar, repack_q4k.rs:174-219): max abs 0;
+  * on random inputs it stays inside the reference's own vector-vs-scalar bound
+    1e-3 * max(|ref|, 1) (avx/parity.rs:50-56), for one row and for several;
+  * the pool gives the same bits whatever its size (every output is one thread's own sum).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from loken_amd import synth
+
+Q4K = oracle.Q4_K
+pytestmark = pytest.mark.skipif(not oracle.lib().lko_cpu_has_avx2(), reason="needs AVX2")
+
+
+def test_repack_places_every_byte_where_the_reference_puts_it():
+    n, k = 16, 512
+    nb = k // 256
+    w = synth.weight(Q4K, n, k, seed=5)
+    x8 = oracle.repack_q4k_x8(w, n, k).reshape(n // 8, nb, 1152)
+    for g in range(n // 8):
+        for b in range(nb):
+            blk = x8[g, b]
+            for j in range(8):
+                src = w[g * 8 + j, b]
+                assert np.array_equal(blk[2 * j:2 * j + 2], src[0:2])
+                assert np.array_equal(blk[16 + 2 * j:18 + 2 * j], src[2:4])
+                assert np.array_equal(blk[32 + 12 * j:44 + 12 * j], src[4:16])
+                for p in range(128):
+                    assert blk[128 + (p // 8) * 64 + j * 8 + p % 8] == src[16 + p]
+
+
+def test_group_dot_is_the_exact_integer_combination():
+    # d = dmin = 1, scales and mins small, activations integers with extreme -127: Q8_K's d is 1 and
+    # its codes are the values, so every product and sum is an integer below 2^24
+    rng = np.random.default_rng(11)
+    n, k = 24, 1024
+    nb = k // 256
+    w = synth.weight(Q4K, n, k, seed=6)
+    sc = rng.integers(0, 8, (n, nb, 8)).astype(np.uint8)
+    mn = rng.integers(0, 8, (n, nb, 8)).astype(np.uint8)
+    w[..., 4:16] = synth.pack_scales_mins(sc, mn)
+    one = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    w[..., 0:2] = one
+    w[..., 2:4] = one
+    x = rng.integers(-127, 128, (3, k)).astype(np.float32)
+    x[:, ::256] = -127.0
+    qs = w[..., 16:144].reshape(n, nb, 4, 32)
+    nibbles = np.stack([qs & 15, qs >> 4], axis=3).reshape(n, nb, 8, 32).astype(np.int64)   # [n, nb, sub-block, 32]
+    a = x.astype(np.int64).reshape(3, nb, 8, 32)
+    dots = np.einsum("nbsl,tbsl->tnbs", nibbles, a)
+    want = (dots * sc[None].astype(np.int64)).sum(axis=(2, 3)) - (a.sum(axis=3)[:, None] * mn[None].astype(np.int64)).sum(axis=(2, 3))
+    got = oracle.oa_matmul_q4k_x8(x, oracle.repack_q4k_x8(w, n, k), n)
+    assert np.abs(want).max() < 2 ** 24
+    assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("m", [1, 5])
+def test_served_path_stays_inside_the_reference_bound(m):
+    n, k = 264, 4096
+    w = synth.weight(Q4K, n, k, seed=7)
+    x = synth.activation(m, k, seed=7)
+    ref = oracle.oa_matmul(Q4K, x, w, n)
+    got = oracle.oa_matmul_q4k_x8(x, oracle.repack_q4k_x8(w, n, k), n)
+    assert (np.abs(got - ref) <= 1e-3 * np.maximum(np.abs(ref), 1.0)).all()
+    # the per-column vector driver shares the pool and the bound
+    fast = oracle.oa_matmul(Q4K, x, w, n, fast_threads=3)
+    assert (np.abs(fast - ref) <= 1e-3 * np.maximum(np.abs(ref), 1.0)).all()
+
+
+def test_results_do_not_depend_on_the_pool_size():
+    n, k = 512, 2048
+    w = synth.weight(Q4K, n, k, seed=8)
+    x = synth.activation(2, k, seed=8)
+    x8 = oracle.repack_q4k_x8(w, n, k)
+    outs = []
+    for threads in (1, 2, 5, 0):
+        assert oracle.pool_start(threads) >= 1
+        outs.append(oracle.oa_matmul_q4k_x8(x, x8, n))
+    for o in outs[1:]:
+        assert np.array_equal(o, outs[0])
+    physical, logical = oracle.cpu_counts()
+    assert 1 <= physical <= logical
+
+
+def test_argument_errors():
+    x = synth.activation(1, 256, seed=9)
+    with pytest.raises(oracle.OracleError):
+        oracle.oa_matmul_q4k_x8(x, np.zeros(1152 * 2, np.uint8), 12)   # n not a multiple of 8
