@@ -416,6 +416,39 @@ void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* outpu
  * tiled matmul instead of returning an untouched buffer. */
 int lk_dense_q4k_rows(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
                       void* stream);
+/* Gate and up over the same plain Q8_1 rows in one launch: output[m, n] = act(gate[n] . x[m]) *
+ * (up[n] . x[m]), act = SiLU (use_gelu == 0) or the tanh-form GELU. Replaces
+ * loken_dense_q4k_imma_m8_actmul (declared src/inference/moe_cuda/mod.rs:452-455; launcher
+ * cuda/moe/dense_q4k_imma_m8.cu:272-286; called from dense_q4k_imma_m8_gate_up_actmul,
+ * src/inference/moe_cuda/dense/imma.rs:320-400). Same limits as the plain form. */
+void loken_dense_q4k_imma_m8_actmul(const void* gate, const void* up, const void* q8_1, float* output,
+                                    int size_m, int size_n, int size_k, int use_gelu, void* stream);
+/* The same launch with a status, as lk_dense_q4k_rows is to the plain form. */
+int lk_dense_q4k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
+                             int size_n, int size_k, int use_gelu, void* stream);
+/* Q4_K expert rows for a handful of routed pairs per expert, over Q8_1 rows the caller quantized.
+ * gate_up: gate_up_weights [num_experts, 2 size_n, size_k] (an expert's gate rows, then its up
+ * rows); q8_1 one row per token [size_m / topk, size_k / 32 blocks]; expert_ids one expert PER PAIR;
+ * output[sorted_token_ids[pair], :] = gelu_tanh(gate . x) * (up . x). Replaces
+ * loken_moe_q4k_imma_m8_gate_up (declared src/inference/moe_cuda/mod.rs:444-447; launcher
+ * cuda/moe/moe_q4k_imma_m8.cu:312-335; caller src/inference/moe_cuda/dense/imma.rs:140-190). A pair
+ * whose expert is out of range leaves its row untouched, as there. */
+void loken_moe_q4k_imma_m8_gate_up(const void* gate_up_weights, const void* q8_1,
+                                   const int32_t* sorted_token_ids, const int32_t* expert_ids, float* output,
+                                   int num_experts, int topk, int size_m, int size_n, int size_k, void* stream);
+/* The same launch with a status. */
+int lk_moe_q4k_rows_gate_up(const void* gate_up_weights, const void* q8_1, const int32_t* sorted_token_ids,
+                            const int32_t* expert_ids, float* output, int num_experts, int topk, int size_m,
+                            int size_n, int size_k, void* stream);
+/* down: weights [num_experts, hidden, size_k]; q8_1 one row per routed pair at the pair's slot
+ * [size_m, size_k / 32 blocks]; each pair's row is scaled by topk_weights[slot] and the rows of a
+ * token are added into output [size_m / topk, hidden] in slot order (output is accumulated into, as
+ * loken_moe_sum_topk does). Replaces loken_moe_q4k_imma_m8_down (declared
+ * src/inference/moe_cuda/mod.rs:448-451; launcher cuda/moe/moe_q4k_imma_m8_down.cu:238-276). Returns 0,
+ * or non-zero when the pair rows' scratch cannot be had (the reference returns 1 there). */
+int loken_moe_q4k_imma_m8_down(const void* weights, const void* q8_1, const int32_t* sorted_token_ids,
+                               const int32_t* expert_ids, const float* topk_weights, float* output,
+                               int num_experts, int topk, int size_m, int hidden, int size_k, void* stream);
 /* The router step in front of the expert block: softmax over each row of logits [n_rows,
  * n_experts], the n_expert_used largest probabilities in descending order (ties to the lower
  * expert id) into weights / ids [n_rows, n_expert_used], divided by their sum when with_norm != 0.

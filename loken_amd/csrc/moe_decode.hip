@@ -529,3 +529,58 @@ extern "C" int loken_moe_gemm_gguf_down_pairs_two(const float* inputs, const voi
     return down_impl(inputs, weights, sorted_token_ids, expert_ids, topk_weights, nullptr, num_experts, topk, size_m,
                      size_n, size_k, quant_type, nullptr, nullptr, nullptr, pair_rows, stream, alt);
 }
+
+// ---------------------------------------------------------------- Q4_K expert rows over the caller's Q8_1
+// The reference's matrix-unit pair kernels for a handful of rows per expert
+// (loken_moe_q4k_imma_m8_gate_up, cuda/moe/moe_q4k_imma_m8.cu:312-335; loken_moe_q4k_imma_m8_down,
+// cuda/moe/moe_q4k_imma_m8_down.cu:238-276; declared src/inference/moe_cuda/mod.rs:443-451). Their
+// contract differs from the launchers above in three ways: the activation arrives as plain block_q8_1
+// rows (size_k / 32 blocks apart, no padding), `expert_ids` holds one expert per routed pair, and the
+// gate's rows and the up's share one tensor per expert, closed with the tanh-form GELU. At the loads
+// these calls are made for, a pair's rows are a mat-vec: they run on the per-pair kernels above.
+// (A tile of eight pairs that spans more than four experts loses rows in the reference; here every
+// pair with an expert in range gets its row.)
+extern "C" int lk_moe_q4k_rows_gate_up(const void* gate_up_weights, const void* q8_1, const int32_t* sorted_token_ids,
+                                       const int32_t* expert_ids, float* output, int num_experts, int topk, int size_m,
+                                       int size_n, int size_k, void* stream) {
+    if (size_m == 0) return LK_OK;
+    if (!gate_up_weights || !q8_1 || !sorted_token_ids || !expert_ids || !output ||
+        bad_shape(1, num_experts, topk, size_m, size_n, size_k) || (((uintptr_t)q8_1) & 3) != 0) return LK_ERR_ARG;
+    const uint8_t* gate = (const uint8_t*)gate_up_weights;
+    const uint8_t* up = gate + (int64_t)size_n * (size_k / 256) * Q4K_BYTES;
+    LkGateAct act;
+    act.kind = LK_GATE_GELU;
+    MoeDims d{num_experts, topk, size_m, size_n, 0, size_k / 32, 0, 0, 2 * size_n, act, nullptr, LkMoeAlt{}};
+    return launch_format<MODE_GATED>(1, gate, up, (const uint8_t*)q8_1, sorted_token_ids, expert_ids, nullptr, nullptr,
+                                     output, d, size_k, (hipStream_t)stream);
+}
+
+extern "C" void loken_moe_q4k_imma_m8_gate_up(const void* gate_up_weights, const void* q8_1,
+                                              const int32_t* sorted_token_ids, const int32_t* expert_ids, float* output,
+                                              int num_experts, int topk, int size_m, int size_n, int size_k,
+                                              void* stream) {
+    (void)lk_moe_q4k_rows_gate_up(gate_up_weights, q8_1, sorted_token_ids, expert_ids, output, num_experts, topk, size_m,
+                                  size_n, size_k, stream);
+}
+
+// One Q8_1 row per routed pair (at the pair's slot); pair rows weighted by topk_weights[slot], then
+// added into output[token] in slot order.
+extern "C" int loken_moe_q4k_imma_m8_down(const void* weights, const void* q8_1, const int32_t* sorted_token_ids,
+                                          const int32_t* expert_ids, const float* topk_weights, float* output,
+                                          int num_experts, int topk, int size_m, int hidden, int size_k, void* stream) {
+    if (size_m <= 0 || hidden <= 0 || size_k <= 0) return LK_OK;
+    if (!weights || !q8_1 || !sorted_token_ids || !expert_ids || !topk_weights || !output ||
+        bad_shape(1, num_experts, topk, size_m, hidden, size_k) || (((uintptr_t)q8_1) & 3) != 0) return LK_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    float* pairs = (float*)reserve_scratch((size_t)size_m * hidden * sizeof(float), s);
+    if (!pairs) return LK_ERR_NOMEM;
+    // a pair whose slot is out of range writes nothing: its row of the sum must read zero
+    const size_t n = (size_t)size_m * hidden;
+    hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, pairs, n);
+    MoeDims d{num_experts, topk, size_m, hidden, 0, size_k / 32, 0, 0, 0, LkGateAct{}, nullptr, LkMoeAlt{}};
+    if (int rc = launch_format<MODE_DOWN>(1, (const uint8_t*)weights, nullptr, (const uint8_t*)q8_1, sorted_token_ids,
+                                          expert_ids, topk_weights, nullptr, pairs, d, size_k, s)) return rc;
+    loken_moe_sum_topk(pairs, output, size_m / topk, topk, hidden, stream);
+    return lk_launch_status();
+}

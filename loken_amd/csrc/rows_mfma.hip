@@ -55,7 +55,18 @@ struct Args {
     int m;                // activation rows in all
     int stride_y;         // Q8_1 blocks between activation rows
     int ldd;              // floats between output rows
+    const uint8_t* w2;    // DUAL: the second matrix (same shape); the output is act(w . x) * (w2 . x)
+    int gelu;             // DUAL: 0 SiLU, 1 tanh-form GELU
 };
+
+// With DUAL a workgroup walks "virtual" tiles: 2 t is row tile t of the first matrix, 2 t + 1 the same
+// rows of the second. The first's reduced sums wait in registers for the second's.
+template <bool DUAL>
+static __device__ __forceinline__ int first_tile(int wg) { return DUAL ? 2 * wg : wg; }
+template <bool DUAL>
+static __device__ __forceinline__ int next_tile(int vt, int wgs) {
+    return DUAL ? ((vt & 1) ? vt - 1 + 2 * wgs : vt + 1) : vt + wgs;
+}
 
 struct Frag {
     uint4 hdr, q[4];
@@ -66,7 +77,7 @@ struct Frag {
 template <int G>
 static __host__ __device__ constexpr int lds_floats_table(int nb) { return nb * 8 * 8 * G * (G < 4 ? 2 : 1); }
 
-template <int G>
+template <int G, bool DUAL>
 __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     constexpr int TW = 8 * G;   // activation rows a table row holds
     constexpr int NV = 4 * G;   // live accumulator registers
@@ -134,8 +145,9 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     const uint8_t* y_lane = y0 + (size_t)min(l32, m_count - 1) * p.stride_y * Q81_BYTES + 4 + 16 * lh;
 
     auto load = [&](Frag& f, int tile, int kb) {
-        const int row = min(tile * 32 + l32, p.n - 1);
-        const uint8_t* bp = (const uint8_t*)(to_gbytes(p.w) + row * row_bytes + (size_t)kb * Q4K_BYTES);
+        const int row = min((DUAL ? tile >> 1 : tile) * 32 + l32, p.n - 1);
+        const uint8_t* mat = DUAL && (tile & 1) ? p.w2 : p.w;
+        const uint8_t* bp = (const uint8_t*)(to_gbytes(mat) + row * row_bytes + (size_t)kb * Q4K_BYTES);
         f.hdr = *(const uint4*)bp;
 #pragma unroll
         for (int c = 0; c < 4; ++c) f.q[c] = *(const uint4*)(bp + 16 + 32 * c + 16 * lh);
@@ -223,11 +235,13 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     // Steps are (row tile, super-block) pairs: wave w takes super-blocks w, w + 4, ... of every
     // tile of this workgroup; the loads of the next step fly under the arithmetic of this one.
     const int my_blocks = (p.nb - wave + WAVES - 1) / WAVES;   // may be zero for short rows
-    int tile = blockIdx.x, kb = wave;
+    const int wgs = (int)gridDim.x, n_vt = DUAL ? 2 * n_tiles : n_tiles;
+    int tile = first_tile<DUAL>(blockIdx.x), kb = wave;
     Frag fa, fb;
-    if (tile < n_tiles && my_blocks > 0) load(fa, tile, kb);
+    if (tile < n_vt && my_blocks > 0) load(fa, tile, kb);
     __syncthreads();   // the scale table is complete
 
+    float gate_keep[G];
     auto finish_tile = [&](int t) {
         // add the four partial tiles and write the activation rows this pass has
         float* mine = reduce + wave * (NV * 64);
@@ -240,36 +254,42 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
 #pragma unroll
         for (int r = 0; r < G; ++r) {
             const int v = wave * G + r;
-            const float sum = (reduce[v * 64 + lane] + reduce[(NV + v) * 64 + lane]) +
-                              (reduce[(2 * NV + v) * 64 + lane] + reduce[(3 * NV + v) * 64 + lane]);
-            const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = t * 32 + l32;
+            float sum = (reduce[v * 64 + lane] + reduce[(NV + v) * 64 + lane]) +
+                        (reduce[(2 * NV + v) * 64 + lane] + reduce[(3 * NV + v) * 64 + lane]);
+            if (DUAL && !(t & 1)) { gate_keep[r] = sum; continue; }
+            if (DUAL) {
+                LkGateAct act;
+                act.kind = p.gelu ? LK_GATE_GELU : LK_GATE_SILU;
+                sum = lk_gated(act, gate_keep[r], sum, 0);
+            }
+            const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = (DUAL ? t >> 1 : t) * 32 + l32;
             if (tok < m_count && row < p.n) p.dst[(size_t)(m0 + tok) * p.ldd + row] = sum;
         }
         __syncthreads();   // the partial tiles may be overwritten
     };
 
-    while (tile < n_tiles) {
+    while (tile < n_vt) {
         if (my_blocks > 0) {
             for (;;) {
                 int nt = tile, nk = kb + WAVES;
                 const bool last = nk >= p.nb;
-                if (last) { nk = wave; nt += gridDim.x; }
-                if (nt < n_tiles) load(fb, nt, nk);
+                if (last) { nk = wave; nt = next_tile<DUAL>(nt, wgs); }
+                if (nt < n_vt) load(fb, nt, nk);
                 compute(fa, kb);
-                if (last) { finish_tile(tile); tile = nt; kb = nk; if (tile >= n_tiles) return; }
+                if (last) { finish_tile(tile); tile = nt; kb = nk; if (tile >= n_vt) return; }
                 else kb = nk;
                 // second half of the ping-pong
                 nt = tile; nk = kb + WAVES;
                 const bool last2 = nk >= p.nb;
-                if (last2) { nk = wave; nt += gridDim.x; }
-                if (nt < n_tiles) load(fa, nt, nk);
+                if (last2) { nk = wave; nt = next_tile<DUAL>(nt, wgs); }
+                if (nt < n_vt) load(fa, nt, nk);
                 compute(fb, kb);
-                if (last2) { finish_tile(tile); tile = nt; kb = nk; if (tile >= n_tiles) return; }
+                if (last2) { finish_tile(tile); tile = nt; kb = nk; if (tile >= n_vt) return; }
                 else kb = nk;
             }
         } else {
             finish_tile(tile);   // nothing of its own to add, but the barriers are the workgroup's
-            tile += gridDim.x;
+            tile = next_tile<DUAL>(tile, wgs);
         }
     }
 }
@@ -291,7 +311,7 @@ static __host__ __device__ constexpr int lds_bytes_staged(int nb) {
     return nb * 8 * 8 * G * 32 + 2 * nb * 8 * 8 * G * 4 + WAVES * 4 * G * 64 * 4;
 }
 
-template <int G>
+template <int G, bool DUAL>
 __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Args p) {
     constexpr int TW = 8 * G, NV = 4 * G;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -311,12 +331,16 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
     // Steps of this wave: (tile, super-block) pairs, super-blocks wave, wave + 4, ... of each tile
     // of this workgroup in turn.
     const int my_blocks = (p.nb - wave + WAVES - 1) / WAVES;
-    const int my_tiles = (int)blockIdx.x < n_tiles ? (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    // (with DUAL every row tile counts twice: the first matrix's rows, then the second's)
+    const int my_tiles = ((int)blockIdx.x < n_tiles ? (n_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0) *
+                         (DUAL ? 2 : 1);
     const int total = my_tiles * my_blocks;
+    auto tile_of = [&](int ordinal) { return (int)blockIdx.x + (DUAL ? ordinal >> 1 : ordinal) * (int)gridDim.x; };
     auto loadw = [&](WFrag& f, int j) {
-        const int tile = blockIdx.x + (j / my_blocks) * gridDim.x, kb = wave + (j % my_blocks) * WAVES;
-        const int row = min(tile * 32 + l32, p.n - 1);
-        const uint8_t* bp = (const uint8_t*)(to_gbytes(p.w) + row * row_bytes + (size_t)kb * Q4K_BYTES);
+        const int ordinal = j / my_blocks, kb = wave + (j % my_blocks) * WAVES;
+        const int row = min(tile_of(ordinal) * 32 + l32, p.n - 1);
+        const uint8_t* mat = DUAL && (ordinal & 1) ? p.w2 : p.w;
+        const uint8_t* bp = (const uint8_t*)(to_gbytes(mat) + row * row_bytes + (size_t)kb * Q4K_BYTES);
         f.hdr = *(const uint4*)bp;
 #pragma unroll
         for (int c = 0; c < 4; ++c) f.q[c] = *(const uint4*)(bp + 16 + 32 * c + 16 * lh);
@@ -422,7 +446,8 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
         }
     };
 
-    auto finish_tile = [&](int t) {
+    float gate_keep[G];
+    auto finish_tile = [&](int ordinal) {
         float* mine = reduce + wave * (NV * 64);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
@@ -433,16 +458,22 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
 #pragma unroll
         for (int r = 0; r < G; ++r) {
             const int v = wave * G + r;
-            const float sum = (reduce[v * 64 + lane] + reduce[(NV + v) * 64 + lane]) +
-                              (reduce[(2 * NV + v) * 64 + lane] + reduce[(3 * NV + v) * 64 + lane]);
-            const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = t * 32 + l32;
+            float sum = (reduce[v * 64 + lane] + reduce[(NV + v) * 64 + lane]) +
+                        (reduce[(2 * NV + v) * 64 + lane] + reduce[(3 * NV + v) * 64 + lane]);
+            if (DUAL && !(ordinal & 1)) { gate_keep[r] = sum; continue; }
+            if (DUAL) {
+                LkGateAct act;
+                act.kind = p.gelu ? LK_GATE_GELU : LK_GATE_SILU;
+                sum = lk_gated(act, gate_keep[r], sum, 0);
+            }
+            const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = tile_of(ordinal) * 32 + l32;
             if (tok < m_count && row < p.n) p.dst[(size_t)tok * p.ldd + row] = sum;
         }
         __syncthreads();   // the partial tiles may be overwritten
     };
 
     if (my_blocks == 0) {   // rows shorter than four super-blocks: this wave only keeps the barriers
-        for (int t = 0; t < my_tiles; ++t) finish_tile(blockIdx.x + t * gridDim.x);
+        for (int t = 0; t < my_tiles; ++t) finish_tile(t);
         return;
     }
     for (int j0 = 0; j0 < total; j0 += DEPTH) {
@@ -452,13 +483,13 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
             if (j < total) {
                 compute(f[d], wave + (j % my_blocks) * WAVES);
                 if (j + DEPTH < total) loadw(f[d], j + DEPTH);
-                if ((j + 1) % my_blocks == 0) finish_tile(blockIdx.x + (j / my_blocks) * gridDim.x);
+                if ((j + 1) % my_blocks == 0) finish_tile(j / my_blocks);
             }
         }
     }
 }
 
-template <int G>
+template <int G, bool DUAL>
 int resident_cap(int lds_bytes) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -469,11 +500,11 @@ int resident_cap(int lds_bytes) {
     if (lds_bytes > lk_device().lds_bytes) {
         r = 0;
     } else if (lds_bytes > 48 * 1024 &&
-               hipFuncSetAttribute((const void*)q4k_rows_mfma_kernel<G>, hipFuncAttributeMaxDynamicSharedMemorySize,
+               hipFuncSetAttribute((const void*)q4k_rows_mfma_kernel<G, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         r = 0;
-    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_mfma_kernel<G>, WG,
+    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_mfma_kernel<G, DUAL>, WG,
                                                             (size_t)lds_bytes) != hipSuccess || r < 1) {
         (void)hipGetLastError();
         r = 1;
@@ -482,21 +513,21 @@ int resident_cap(int lds_bytes) {
     return r;
 }
 
-template <int G>
+template <int G, bool DUAL>
 int launch_rows(const Args& a, hipStream_t stream) {
     const int lds_bytes = (lds_floats_table<G>(a.nb) + WAVES * 4 * G * 64) * (int)sizeof(float);
-    const int per_cu = resident_cap<G>(lds_bytes);
+    const int per_cu = resident_cap<G, DUAL>(lds_bytes);
     if (per_cu == 0) return LK_ERR_ARG;   // rows too long for the scale tables
     const int n_tiles = (a.n + 31) / 32, groups = (a.m + TOK - 1) / TOK;
     if (groups > 65535) return LK_ERR_ARG;
     int cap = lk_device().cus * per_cu / groups;
     if (cap < 1) cap = 1;
-    hipLaunchKernelGGL(q4k_rows_mfma_kernel<G>, dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
+    hipLaunchKernelGGL((q4k_rows_mfma_kernel<G, DUAL>), dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
     return lk_launch_status();
 }
 
 // The staged kernel for `a.m` <= 8 G rows, if its LDS image fits; -1 when it does not.
-template <int G>
+template <int G, bool DUAL>
 int launch_staged(const Args& a, hipStream_t stream) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -509,11 +540,11 @@ int launch_staged(const Args& a, hipStream_t stream) {
         if (it == by_lds.end()) {
             int r = 0;
             if (lds_bytes > 48 * 1024 &&
-                hipFuncSetAttribute((const void*)q4k_rows_staged_kernel<G>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                hipFuncSetAttribute((const void*)q4k_rows_staged_kernel<G, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     lds_bytes) != hipSuccess) {
                 (void)hipGetLastError();
                 r = 0;
-            } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_staged_kernel<G>, WG,
+            } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_staged_kernel<G, DUAL>, WG,
                                                                     (size_t)lds_bytes) != hipSuccess || r < 1) {
                 (void)hipGetLastError();
                 r = 1;
@@ -524,8 +555,28 @@ int launch_staged(const Args& a, hipStream_t stream) {
     }
     if (per_cu == 0) return -1;
     const int n_tiles = (a.n + 31) / 32, cap = lk_device().cus * per_cu;
-    hipLaunchKernelGGL(q4k_rows_staged_kernel<G>, dim3(n_tiles < cap ? n_tiles : cap), dim3(WG), lds_bytes, stream, a);
+    hipLaunchKernelGGL((q4k_rows_staged_kernel<G, DUAL>), dim3(n_tiles < cap ? n_tiles : cap), dim3(WG), lds_bytes, stream, a);
     return lk_launch_status();
+}
+
+template <bool DUAL>
+int launch_any(const Args& a, hipStream_t stream) {
+    // at most 8 / 16 activation rows in all: the fix-up runs on the registers those rows live in,
+    // and the activation is staged in LDS when it fits there
+    if (a.m <= 8) {
+        const int rc = launch_staged<1, DUAL>(a, stream);
+        return rc >= 0 ? rc : launch_rows<1, DUAL>(a, stream);
+    }
+    if (a.m <= 16) {
+        const int rc = launch_staged<2, DUAL>(a, stream);
+        return rc >= 0 ? rc : launch_rows<2, DUAL>(a, stream);
+    }
+    return launch_rows<4, DUAL>(a, stream);
+}
+
+bool bad_rows_call(const void* w, const void* q8_1, const float* output, int size_m, int size_n, int size_k) {
+    return !w || !q8_1 || !output || size_m < 0 || size_n < 0 || size_k <= 0 || size_k % 256 != 0 ||
+           (((uintptr_t)w) & 15) != 0 || (((uintptr_t)q8_1) & 3) != 0;
 }
 
 }  // namespace
@@ -534,21 +585,10 @@ int launch_staged(const Args& a, hipStream_t stream) {
 int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
                      int stride_y, int ldd, hipStream_t stream) {
     if (size_m == 0 || size_n == 0) return LK_OK;
-    if (!w || !q8_1 || !output || size_m < 0 || size_n < 0 || size_k <= 0 || size_k % 256 != 0) return LK_ERR_ARG;
+    if (bad_rows_call(w, q8_1, output, size_m, size_n, size_k)) return LK_ERR_ARG;
     if (stride_y < size_k / 32 || ldd < size_n) return LK_ERR_ARG;
-    if ((((uintptr_t)w) & 15) != 0 || (((uintptr_t)q8_1) & 3) != 0) return LK_ERR_ARG;
-    Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd};
-    // at most 8 / 16 activation rows in all: the fix-up runs on the registers those rows live in,
-    // and the activation is staged in LDS when it fits there
-    if (size_m <= 8) {
-        const int rc = launch_staged<1>(a, stream);
-        return rc >= 0 ? rc : launch_rows<1>(a, stream);
-    }
-    if (size_m <= 16) {
-        const int rc = launch_staged<2>(a, stream);
-        return rc >= 0 ? rc : launch_rows<2>(a, stream);
-    }
-    return launch_rows<4>(a, stream);
+    Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd, nullptr, 0};
+    return launch_any<false>(a, stream);
 }
 
 extern "C" int lk_dense_q4k_rows(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
@@ -559,4 +599,21 @@ extern "C" int lk_dense_q4k_rows(const void* w, const void* q8_1, float* output,
 extern "C" void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
                                               int size_k, void* stream) {
     (void)lk_q4k_rows_mfma(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, (hipStream_t)stream);
+}
+
+// Gate and up in one launch: output[m, n] = act(gate[n] . x[m]) * (up[n] . x[m]), act = SiLU or the
+// tanh-form GELU. Replaces loken_dense_q4k_imma_m8_actmul (declared src/inference/moe_cuda/mod.rs:452-455,
+// launcher cuda/moe/dense_q4k_imma_m8.cu:272-286).
+extern "C" int lk_dense_q4k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
+                                        int size_n, int size_k, int use_gelu, void* stream) {
+    if (size_m == 0 || size_n == 0) return LK_OK;
+    if (bad_rows_call(gate, q8_1, output, size_m, size_n, size_k) || !up || (((uintptr_t)up) & 15) != 0) return LK_ERR_ARG;
+    Args a{(const uint8_t*)gate, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, size_k / 32, size_n,
+           (const uint8_t*)up, use_gelu ? 1 : 0};
+    return launch_any<true>(a, (hipStream_t)stream);
+}
+
+extern "C" void loken_dense_q4k_imma_m8_actmul(const void* gate, const void* up, const void* q8_1, float* output,
+                                               int size_m, int size_n, int size_k, int use_gelu, void* stream) {
+    (void)lk_dense_q4k_rows_actmul(gate, up, q8_1, output, size_m, size_n, size_k, use_gelu, stream);
 }

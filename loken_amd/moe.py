@@ -389,3 +389,35 @@ def moe_forward(wtype_gu: int, wtype_down: int, x: torch.Tensor, gate: torch.Ten
     routing = ExpertRouting(choices)
     h = moe_gemm_gguf_gate_up_silu_mul(wtype_gu, x.contiguous(), gate, up, routing, n_experts, ffn)
     return moe_gemm_gguf_down_reduce(wtype_down, h, down, routing, topk_weights.reshape(-1), n_experts, hidden)
+
+
+def moe_q4k_imma_m8_gate_up(x: torch.Tensor, gate_up: torch.Tensor, sorted_token_ids: torch.Tensor,
+                            expert_of_pair: torch.Tensor, n_experts: int, topk: int, n: int) -> torch.Tensor:
+    """``gelu(gate . x) * (up . x)`` per routed pair over Q8_1 rows quantized here, one expert id
+    per pair, ``[tokens * topk, n]`` in slot order, zero where a pair's expert is out of range
+    (moe_q4k_imma_m8_gate_up, src/inference/moe_cuda/dense/imma.rs:140-190)."""
+    from . import ops
+    tokens, k = x.shape
+    pairs = tokens * topk
+    q = ops.quantize_q8_1_rows(x, k_padded=k)
+    out = torch.zeros((pairs, n), dtype=torch.float32, device=x.device)
+    _lib.check("lk_moe_q4k_rows_gate_up", _lib.load().lk_moe_q4k_rows_gate_up(
+        gate_up.data_ptr(), q.data_ptr(), sorted_token_ids.data_ptr(), expert_of_pair.data_ptr(), out.data_ptr(),
+        n_experts, topk, pairs, n, k, _stream()))
+    return out
+
+
+def moe_q4k_imma_m8_down_reduce(h: torch.Tensor, down: torch.Tensor, sorted_token_ids: torch.Tensor,
+                                expert_of_pair: torch.Tensor, topk_weights: torch.Tensor, n_experts: int, topk: int,
+                                hidden: int) -> torch.Tensor:
+    """Down over one Q8_1 row per routed pair (quantized here, at the pair's slot), weighted and
+    folded into ``[tokens, hidden]`` (moe_q4k_imma_m8_down_reduce, src/inference/moe_cuda/dense/imma.rs:
+    200-300)."""
+    from . import ops
+    pairs, k = h.shape
+    q = ops.quantize_q8_1_rows(h, k_padded=k)
+    out = torch.zeros((pairs // topk, hidden), dtype=torch.float32, device=h.device)
+    _lib.check("loken_moe_q4k_imma_m8_down", _lib.load().loken_moe_q4k_imma_m8_down(
+        down.data_ptr(), q.data_ptr(), sorted_token_ids.data_ptr(), expert_of_pair.data_ptr(),
+        topk_weights.data_ptr(), out.data_ptr(), n_experts, topk, pairs, hidden, k, _stream()))
+    return out

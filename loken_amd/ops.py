@@ -234,3 +234,17 @@ def mmq_forward(wtype: int, weight: torch.Tensor, x: torch.Tensor, n: int) -> to
     if launched == 0:
         raise _lib.LokenError(MMQ_LAUNCHER[wtype], _lib.LK_ERR_ARG)
     return out
+
+
+def dense_q4k_rows_actmul(gate: torch.Tensor, up: torch.Tensor, x: torch.Tensor, n: int, use_gelu: bool) -> torch.Tensor:
+    """``act(gate . x) * (up . x)`` for ``[rows, k]`` f32 x two Q4_K weights ``[n, k]`` in one launch
+    on the matrix unit (dense_q4k_imma_m8_act_mul, src/inference/moe_cuda/dense/imma.rs:320-400)."""
+    rows, k = x.shape
+    if k % 256:
+        raise ValueError("dense_q4k_rows_actmul: k must be a multiple of 256")
+    q = quantize_q8_1_rows(x, k_padded=k)
+    out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
+    _lib.check("lk_dense_q4k_rows_actmul",
+               _lib.load().lk_dense_q4k_rows_actmul(gate.data_ptr(), up.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k,
+                                                    1 if use_gelu else 0, _stream()))
+    return out

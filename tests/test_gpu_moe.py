@@ -472,3 +472,46 @@ def test_router_ties_go_to_the_lower_expert_and_weights_descend():
     assert ids[0].tolist() == list(range(8)) and np.allclose(w[0], 1.0 / 8)
     assert ids[1, :4].tolist() == [40, 41, 5, 100] and ids[1, 4:].tolist() == [0, 1, 2, 3]
     assert (np.diff(w[1]) <= 0).all() and abs(w[1].sum() - 1.0) < 1e-6
+
+
+@pytest.mark.parametrize("tokens,topk,n_experts", [(3, 2, 5), (8, 4, 16), (1, 8, 128)])
+def test_q4k_pair_rows_over_caller_quantized_rows_with_one_expert_per_pair(tokens, topk, n_experts):
+    """loken_moe_q4k_imma_m8_gate_up and loken_moe_q4k_imma_m8_down: Q8_1 rows from the caller,
+    expert ids per pair (one of them out of range), GELU on the gate. The products are the
+    same-codes oracle's (cuda/moe/moe_q4k_imma_m8.cu:273-296, moe_q4k_imma_m8_down.cu:196-230)."""
+    from loken_amd.moe import moe_q4k_imma_m8_down_reduce, moe_q4k_imma_m8_gate_up
+    hidden, ffn = 512, 256
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=66, x_scale=4.0)
+    slots, experts = oracle.group_by_expert(ids)
+    experts = experts.copy()
+    dropped = len(slots) // 2
+    experts[dropped] = n_experts + 3          # a pair the routing leaves out
+    gate_rows, up_rows = gate.reshape(n_experts, ffn, -1), up.reshape(n_experts, ffn, -1)
+    both = np.ascontiguousarray(np.concatenate([gate_rows, up_rows], axis=1))
+    pairs = tokens * topk
+    want_h = np.zeros((pairs, ffn), np.float64)
+    for j in range(pairs):
+        if experts[j] >= n_experts:
+            continue
+        row = x[slots[j] // topk][None, :]
+        g = oracle.ob_matmul(lib.TYPE_Q4_K, row, gate_rows[experts[j]].reshape(-1), ffn)[0].astype(np.float64)
+        u = oracle.ob_matmul(lib.TYPE_Q4_K, row, up_rows[experts[j]].reshape(-1), ffn)[0].astype(np.float64)
+        want_h[slots[j]] = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3))) * u
+    sd, ed = dev(slots.astype(np.int32)), dev(experts.astype(np.int32))
+    h = moe_q4k_imma_m8_gate_up(dev(x), dev(both), sd, ed, n_experts, topk, ffn)
+    got_h = h.cpu().numpy()
+    assert (got_h[slots[dropped]] == 0).all()
+    assert (np.abs(got_h - want_h) <= 1e-3 * np.abs(want_h) + 1e-4 * np.abs(want_h).max()).all()
+
+    # down from the device's own h, so that the two sides quantize the same rows
+    down_rows = down.reshape(n_experts, hidden, -1)
+    flat_w = w.reshape(-1).astype(np.float32)
+    want = np.zeros((tokens, hidden), np.float64)
+    for slot in range(pairs):                 # slot order: the fold's order
+        j = int(np.nonzero(slots == slot)[0][0])
+        if experts[j] >= n_experts:
+            continue
+        y = oracle.ob_matmul(lib.TYPE_Q4_K, got_h[slot][None, :], down_rows[experts[j]].reshape(-1), hidden)[0]
+        want[slot // topk] += (y * flat_w[slot]).astype(np.float64)
+    got = moe_q4k_imma_m8_down_reduce(h, dev(down), sd, ed, dev(flat_w), n_experts, topk, hidden).cpu().numpy()
+    assert (np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-4 * np.abs(want).max()).all()

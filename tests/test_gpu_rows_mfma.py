@@ -84,3 +84,40 @@ def test_full_gate_shape_against_matvec_and_sampled_oracle():
     rng = np.random.default_rng(63)
     wr = np.sort(rng.choice(n, 300, replace=False))
     assert_close(got.cpu().numpy()[:, wr], oracle.ob_matmul(Q4K, x, w[wr], len(wr)))
+
+
+def gelu_tanh(g):
+    return 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+
+
+def silu(g):
+    return g / (1.0 + np.exp(-g))
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (5, 512, 70), (8, 2048, 257), (13, 1024, 130), (16, 768, 33), (33, 512, 96),
+                                   (70, 2048, 64), (3, 14336, 40)])
+@pytest.mark.parametrize("use_gelu", [False, True])
+def test_gate_and_up_in_one_launch_match_the_closed_form_over_the_oracles_products(m, k, n, use_gelu):
+    """loken_dense_q4k_imma_m8_actmul: the two products are the same-codes oracle's, the activation
+    on top of them the closed form the reference's epilogue states (cuda/moe/dense_q4k_imma_m8.cu:
+    33-58)."""
+    gate = synth.weight(Q4K, n, k, seed=61, stream=1)
+    up = synth.weight(Q4K, n, k, seed=61, stream=2)
+    x = synth.activation(m, k, seed=61) * np.float32(4.0)
+    g = oracle.ob_matmul(Q4K, x, gate, n).astype(np.float64)
+    u = oracle.ob_matmul(Q4K, x, up, n).astype(np.float64)
+    want = (gelu_tanh(g) if use_gelu else silu(g)) * u
+    got = ops.dense_q4k_rows_actmul(dev(gate), dev(up), dev(x), n, use_gelu).cpu().numpy()
+    assert (np.abs(got - want) <= RTOL * np.abs(want) + ATOL * max(1.0, np.abs(want).max())).all()
+
+
+def test_gate_and_up_in_one_launch_carry_the_plain_launches_bits():
+    """The dual launch's products are the plain launch's, bit for bit: SiLU(g) * u recomputed in f32
+    from the two plain outputs differs only by the device's exp."""
+    m, k, n = 7, 4096, 1024
+    gate, up = dev(synth.weight(Q4K, n, k, seed=62, stream=1)), dev(synth.weight(Q4K, n, k, seed=62, stream=2))
+    x = dev(synth.activation(m, k, seed=62))
+    g, u = ops.dense_q4k_rows(gate, x, n).double(), ops.dense_q4k_rows(up, x, n).double()
+    want = g / (1.0 + torch.exp(-g)) * u
+    got = ops.dense_q4k_rows_actmul(gate, up, x, n, False).double()
+    assert ((got - want).abs() <= 2e-6 * want.abs() + 1e-30).all()
