@@ -426,6 +426,17 @@ void loken_dense_q4k_imma_m8_actmul(const void* gate, const void* up, const void
 /* The same launch with a status, as lk_dense_q4k_rows is to the plain form. */
 int lk_dense_q4k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
                              int size_n, int size_k, int use_gelu, void* stream);
+/* The Q5_K siblings of the four launches above (block_q5_K = block_q4_K plus a plane of fifth bits):
+ * loken_dense_q5k_imma_m8_plain / _actmul, declared src/inference/moe_cuda/mod.rs:459-466 and picked
+ * by weight dtype at src/inference/moe_cuda/dense/imma.rs:113-116 and 362-365. */
+void loken_dense_q5k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
+                                   int size_k, void* stream);
+int lk_dense_q5k_rows(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
+                      void* stream);
+void loken_dense_q5k_imma_m8_actmul(const void* gate, const void* up, const void* q8_1, float* output,
+                                    int size_m, int size_n, int size_k, int use_gelu, void* stream);
+int lk_dense_q5k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
+                             int size_n, int size_k, int use_gelu, void* stream);
 /* Q4_K expert rows for a handful of routed pairs per expert, over Q8_1 rows the caller quantized.
  * gate_up: gate_up_weights [num_experts, 2 size_n, size_k] (an expert's gate rows, then its up
  * rows); q8_1 one row per token [size_m / topk, size_k / 32 blocks]; expert_ids one expert PER PAIR;

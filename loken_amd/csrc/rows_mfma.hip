@@ -69,15 +69,37 @@ static __device__ __forceinline__ int next_tile(int vt, int wgs) {
 }
 
 struct Frag {
-    uint4 hdr, q[4];
+    uint4 hdr, q[4], qh;   // qh: Q5_K only, the lane's 16 bytes of fifth bits (bit s = sub-block s)
     v4i a[8];
 };
+
+// Q5_K is Q4_K with a plane of fifth bits between the header and the nibbles
+// (block_q5_K: d, dmin, scales[12], qh[32], qs[128]).
+template <bool Q5>
+struct Blk {
+    static constexpr int BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES;
+    static constexpr int QS = Q5 ? 48 : 16;
+};
+
+// The B operand of sub-block s from the lane's 16 bytes of its pair's nibbles (and fifth bits).
+template <bool Q5>
+static __device__ __forceinline__ v4i codes_of(const uint4& q, const uint4& qh, int s) {
+    const uint32_t u[4] = {q.x, q.y, q.z, q.w}, h[4] = {qh.x, qh.y, qh.z, qh.w};
+    v4i b;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        uint32_t x = ((s & 1) ? u[e] >> 4 : u[e]) & 0x0F0F0F0Fu;
+        if (Q5) x |= ((h[e] >> s) & 0x01010101u) << 4;
+        b[e] = (int)x;
+    }
+    return b;
+}
 
 // Floats of the scale tables: d8 [nb * 8][8 G], and with G < 4 also d8 * S in the same shape.
 template <int G>
 static __host__ __device__ constexpr int lds_floats_table(int nb) { return nb * 8 * 8 * G * (G < 4 ? 2 : 1); }
 
-template <int G, bool DUAL>
+template <int G, bool DUAL, bool Q5>
 __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     constexpr int TW = 8 * G;   // activation rows a table row holds
     constexpr int NV = 4 * G;   // live accumulator registers
@@ -92,7 +114,7 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     const int m0 = blockIdx.y * TOK;
     const int m_count = min(TOK, p.m - m0);
     const int n_tiles = (p.n + 31) >> 5;
-    const size_t row_bytes = (size_t)p.nb * Q4K_BYTES;
+    const size_t row_bytes = (size_t)p.nb * Blk<Q5>::BYTES;
 
     // Activation scales of this pass, zero for the rows the pass does not have. Eight loads are
     // issued before the first is used: one at a time, each would cost a memory latency.
@@ -147,10 +169,11 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     auto load = [&](Frag& f, int tile, int kb) {
         const int row = min((DUAL ? tile >> 1 : tile) * 32 + l32, p.n - 1);
         const uint8_t* mat = DUAL && (tile & 1) ? p.w2 : p.w;
-        const uint8_t* bp = (const uint8_t*)(to_gbytes(mat) + row * row_bytes + (size_t)kb * Q4K_BYTES);
+        const uint8_t* bp = (const uint8_t*)(to_gbytes(mat) + row * row_bytes + (size_t)kb * Blk<Q5>::BYTES);
         f.hdr = *(const uint4*)bp;
+        if (Q5) f.qh = *(const uint4*)(bp + 16 + 16 * lh);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) f.q[c] = *(const uint4*)(bp + 16 + 32 * c + 16 * lh);
+        for (int c = 0; c < 4; ++c) f.q[c] = *(const uint4*)(bp + Blk<Q5>::QS + 32 * c + 16 * lh);
         const uint8_t* ap = y_lane + (size_t)kb * 8 * Q81_BYTES;
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
@@ -184,15 +207,7 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
         const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
-            const uint4 q = f.q[s >> 1];
-            v4i b;
-            if (s & 1) {
-                b = v4i{(int)((q.x >> 4) & 0x0F0F0F0Fu), (int)((q.y >> 4) & 0x0F0F0F0Fu),
-                        (int)((q.z >> 4) & 0x0F0F0F0Fu), (int)((q.w >> 4) & 0x0F0F0F0Fu)};
-            } else {
-                b = v4i{(int)(q.x & 0x0F0F0F0Fu), (int)(q.y & 0x0F0F0F0Fu), (int)(q.z & 0x0F0F0F0Fu),
-                        (int)(q.w & 0x0F0F0F0Fu)};
-            }
+            const v4i b = codes_of<Q5>(f.q[s >> 1], f.qh, s);
             // The int32 accumulators start at the bit pattern of 1.5 * 2^23: adding an integer of
             // magnitude below 2^22 to that pattern yields the float 1.5 * 2^23 + integer, so the
             // dots leave the matrix unit as floats and no conversion is spent on them. The offset
@@ -302,7 +317,7 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
 // (one 32-row tile per workgroup, four steps per wave) waiting on memory latency most of its time.
 // ---------------------------------------------------------------------------------------------
 struct WFrag {
-    uint4 hdr, q[4];
+    uint4 hdr, q[4], qh;
 };
 
 template <int G>
@@ -311,7 +326,7 @@ static __host__ __device__ constexpr int lds_bytes_staged(int nb) {
     return nb * 8 * 8 * G * 32 + 2 * nb * 8 * 8 * G * 4 + WAVES * 4 * G * 64 * 4;
 }
 
-template <int G, bool DUAL>
+template <int G, bool DUAL, bool Q5>
 __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Args p) {
     constexpr int TW = 8 * G, NV = 4 * G;
     extern __shared__ __align__(16) uint8_t lds[];
@@ -325,7 +340,7 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
     const int l32 = lane & 31, lh = lane >> 5;
     const int m_count = p.m;   // one pass: the launcher sends at most TW rows here
     const int n_tiles = (p.n + 31) >> 5;
-    const size_t row_bytes = (size_t)p.nb * Q4K_BYTES;
+    const size_t row_bytes = (size_t)p.nb * Blk<Q5>::BYTES;
     const int entries = p.nb * 8 * TW;
 
     // Steps of this wave: (tile, super-block) pairs, super-blocks wave, wave + 4, ... of each tile
@@ -340,10 +355,11 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
         const int ordinal = j / my_blocks, kb = wave + (j % my_blocks) * WAVES;
         const int row = min(tile_of(ordinal) * 32 + l32, p.n - 1);
         const uint8_t* mat = DUAL && (ordinal & 1) ? p.w2 : p.w;
-        const uint8_t* bp = (const uint8_t*)(to_gbytes(mat) + row * row_bytes + (size_t)kb * Q4K_BYTES);
+        const uint8_t* bp = (const uint8_t*)(to_gbytes(mat) + row * row_bytes + (size_t)kb * Blk<Q5>::BYTES);
         f.hdr = *(const uint4*)bp;
+        if (Q5) f.qh = *(const uint4*)(bp + 16 + 16 * lh);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) f.q[c] = *(const uint4*)(bp + 16 + 32 * c + 16 * lh);
+        for (int c = 0; c < 4; ++c) f.q[c] = *(const uint4*)(bp + Blk<Q5>::QS + 32 * c + 16 * lh);
     };
 
     // The activation: every (sub-block, row) entry is one Q8_1 block; its codes go to LDS as they
@@ -379,7 +395,7 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
             }
         }
     };
-    constexpr int DEPTH = G == 1 ? 4 : 3;   // steps of weight loads a wave keeps in flight (registers)
+    constexpr int DEPTH = G == 1 && !Q5 ? 4 : 3;   // steps of weight loads a wave keeps in flight (registers)
     WFrag f[DEPTH];
     issue(threadIdx.x);
 #pragma unroll
@@ -411,15 +427,7 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
             const uint32_t scs = ((s < 4 ? sc_lo : sc_hi) >> (8 * (s & 3))) & 0xFFu;
             const uint32_t mns = ((s < 4 ? mn_lo : mn_hi) >> (8 * (s & 3))) & 0xFFu;
             const float dsc = d * (float)scs, dmm = -(dmin * (float)mns);
-            const uint4 q = w.q[s >> 1];
-            v4i b;
-            if (s & 1) {
-                b = v4i{(int)((q.x >> 4) & 0x0F0F0F0Fu), (int)((q.y >> 4) & 0x0F0F0F0Fu),
-                        (int)((q.z >> 4) & 0x0F0F0F0Fu), (int)((q.w >> 4) & 0x0F0F0F0Fu)};
-            } else {
-                b = v4i{(int)(q.x & 0x0F0F0F0Fu), (int)(q.y & 0x0F0F0F0Fu), (int)(q.z & 0x0F0F0F0Fu),
-                        (int)(q.w & 0x0F0F0F0Fu)};
-            }
+            const v4i b = codes_of<Q5>(w.q[s >> 1], w.qh, s);
             const int sub = kb * 8 + s;
             const v4i a = *(const v4i*)(a_lane + (size_t)sub * TW * 32);
             // the accumulators start at the bit pattern of 1.5 * 2^23, so the dots leave the matrix
@@ -489,7 +497,7 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
     }
 }
 
-template <int G, bool DUAL>
+template <int G, bool DUAL, bool Q5>
 int resident_cap(int lds_bytes) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -500,11 +508,11 @@ int resident_cap(int lds_bytes) {
     if (lds_bytes > lk_device().lds_bytes) {
         r = 0;
     } else if (lds_bytes > 48 * 1024 &&
-               hipFuncSetAttribute((const void*)q4k_rows_mfma_kernel<G, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+               hipFuncSetAttribute((const void*)q4k_rows_mfma_kernel<G, DUAL, Q5>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         r = 0;
-    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_mfma_kernel<G, DUAL>, WG,
+    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_mfma_kernel<G, DUAL, Q5>, WG,
                                                             (size_t)lds_bytes) != hipSuccess || r < 1) {
         (void)hipGetLastError();
         r = 1;
@@ -513,21 +521,21 @@ int resident_cap(int lds_bytes) {
     return r;
 }
 
-template <int G, bool DUAL>
+template <int G, bool DUAL, bool Q5>
 int launch_rows(const Args& a, hipStream_t stream) {
     const int lds_bytes = (lds_floats_table<G>(a.nb) + WAVES * 4 * G * 64) * (int)sizeof(float);
-    const int per_cu = resident_cap<G, DUAL>(lds_bytes);
+    const int per_cu = resident_cap<G, DUAL, Q5>(lds_bytes);
     if (per_cu == 0) return LK_ERR_ARG;   // rows too long for the scale tables
     const int n_tiles = (a.n + 31) / 32, groups = (a.m + TOK - 1) / TOK;
     if (groups > 65535) return LK_ERR_ARG;
     int cap = lk_device().cus * per_cu / groups;
     if (cap < 1) cap = 1;
-    hipLaunchKernelGGL((q4k_rows_mfma_kernel<G, DUAL>), dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
+    hipLaunchKernelGGL((q4k_rows_mfma_kernel<G, DUAL, Q5>), dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
     return lk_launch_status();
 }
 
 // The staged kernel for `a.m` <= 8 G rows, if its LDS image fits; -1 when it does not.
-template <int G, bool DUAL>
+template <int G, bool DUAL, bool Q5>
 int launch_staged(const Args& a, hipStream_t stream) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -540,11 +548,11 @@ int launch_staged(const Args& a, hipStream_t stream) {
         if (it == by_lds.end()) {
             int r = 0;
             if (lds_bytes > 48 * 1024 &&
-                hipFuncSetAttribute((const void*)q4k_rows_staged_kernel<G, DUAL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                hipFuncSetAttribute((const void*)q4k_rows_staged_kernel<G, DUAL, Q5>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     lds_bytes) != hipSuccess) {
                 (void)hipGetLastError();
                 r = 0;
-            } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_staged_kernel<G, DUAL>, WG,
+            } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_staged_kernel<G, DUAL, Q5>, WG,
                                                                     (size_t)lds_bytes) != hipSuccess || r < 1) {
                 (void)hipGetLastError();
                 r = 1;
@@ -555,23 +563,23 @@ int launch_staged(const Args& a, hipStream_t stream) {
     }
     if (per_cu == 0) return -1;
     const int n_tiles = (a.n + 31) / 32, cap = lk_device().cus * per_cu;
-    hipLaunchKernelGGL((q4k_rows_staged_kernel<G, DUAL>), dim3(n_tiles < cap ? n_tiles : cap), dim3(WG), lds_bytes, stream, a);
+    hipLaunchKernelGGL((q4k_rows_staged_kernel<G, DUAL, Q5>), dim3(n_tiles < cap ? n_tiles : cap), dim3(WG), lds_bytes, stream, a);
     return lk_launch_status();
 }
 
-template <bool DUAL>
+template <bool DUAL, bool Q5>
 int launch_any(const Args& a, hipStream_t stream) {
     // at most 8 / 16 activation rows in all: the fix-up runs on the registers those rows live in,
     // and the activation is staged in LDS when it fits there
     if (a.m <= 8) {
-        const int rc = launch_staged<1, DUAL>(a, stream);
-        return rc >= 0 ? rc : launch_rows<1, DUAL>(a, stream);
+        const int rc = launch_staged<1, DUAL, Q5>(a, stream);
+        return rc >= 0 ? rc : launch_rows<1, DUAL, Q5>(a, stream);
     }
     if (a.m <= 16) {
-        const int rc = launch_staged<2, DUAL>(a, stream);
-        return rc >= 0 ? rc : launch_rows<2, DUAL>(a, stream);
+        const int rc = launch_staged<2, DUAL, Q5>(a, stream);
+        return rc >= 0 ? rc : launch_rows<2, DUAL, Q5>(a, stream);
     }
-    return launch_rows<4, DUAL>(a, stream);
+    return launch_rows<4, DUAL, Q5>(a, stream);
 }
 
 bool bad_rows_call(const void* w, const void* q8_1, const float* output, int size_m, int size_n, int size_k) {
@@ -582,38 +590,71 @@ bool bad_rows_call(const void* w, const void* q8_1, const float* output, int siz
 }  // namespace
 
 // Returns LK_OK, or the reason nothing was launched.
-int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
-                     int stride_y, int ldd, hipStream_t stream) {
+static int rows_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y,
+                      int ldd, bool q5, hipStream_t stream) {
     if (size_m == 0 || size_n == 0) return LK_OK;
     if (bad_rows_call(w, q8_1, output, size_m, size_n, size_k)) return LK_ERR_ARG;
     if (stride_y < size_k / 32 || ldd < size_n) return LK_ERR_ARG;
     Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd, nullptr, 0};
-    return launch_any<false>(a, stream);
+    return q5 ? launch_any<false, true>(a, stream) : launch_any<false, false>(a, stream);
+}
+
+int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
+                     int stride_y, int ldd, hipStream_t stream) {
+    return rows_plain(w, q8_1, output, size_m, size_n, size_k, stride_y, ldd, false, stream);
 }
 
 extern "C" int lk_dense_q4k_rows(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
                                  void* stream) {
-    return lk_q4k_rows_mfma(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, (hipStream_t)stream);
+    return rows_plain(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, false, (hipStream_t)stream);
 }
 
 extern "C" void loken_dense_q4k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
                                               int size_k, void* stream) {
-    (void)lk_q4k_rows_mfma(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, (hipStream_t)stream);
+    (void)rows_plain(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, false, (hipStream_t)stream);
 }
 
 // Gate and up in one launch: output[m, n] = act(gate[n] . x[m]) * (up[n] . x[m]), act = SiLU or the
 // tanh-form GELU. Replaces loken_dense_q4k_imma_m8_actmul (declared src/inference/moe_cuda/mod.rs:452-455,
 // launcher cuda/moe/dense_q4k_imma_m8.cu:272-286).
-extern "C" int lk_dense_q4k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
-                                        int size_n, int size_k, int use_gelu, void* stream) {
+static int rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m, int size_n,
+                       int size_k, int use_gelu, bool q5, hipStream_t stream) {
     if (size_m == 0 || size_n == 0) return LK_OK;
     if (bad_rows_call(gate, q8_1, output, size_m, size_n, size_k) || !up || (((uintptr_t)up) & 15) != 0) return LK_ERR_ARG;
     Args a{(const uint8_t*)gate, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, size_k / 32, size_n,
            (const uint8_t*)up, use_gelu ? 1 : 0};
-    return launch_any<true>(a, (hipStream_t)stream);
+    return q5 ? launch_any<true, true>(a, stream) : launch_any<true, false>(a, stream);
+}
+
+extern "C" int lk_dense_q4k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
+                                        int size_n, int size_k, int use_gelu, void* stream) {
+    return rows_actmul(gate, up, q8_1, output, size_m, size_n, size_k, use_gelu, false, (hipStream_t)stream);
 }
 
 extern "C" void loken_dense_q4k_imma_m8_actmul(const void* gate, const void* up, const void* q8_1, float* output,
                                                int size_m, int size_n, int size_k, int use_gelu, void* stream) {
-    (void)lk_dense_q4k_rows_actmul(gate, up, q8_1, output, size_m, size_n, size_k, use_gelu, stream);
+    (void)rows_actmul(gate, up, q8_1, output, size_m, size_n, size_k, use_gelu, false, (hipStream_t)stream);
+}
+
+// The Q5_K siblings (loken_dense_q5k_imma_m8_plain / _actmul, declared src/inference/moe_cuda/mod.rs:459-466,
+// picked by dtype at src/inference/moe_cuda/dense/imma.rs:113-116,362-365): the same kernels with the
+// fifth-bit plane folded into the codes.
+extern "C" int lk_dense_q5k_rows(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
+                                 void* stream) {
+    return rows_plain(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, true, (hipStream_t)stream);
+}
+
+extern "C" void loken_dense_q5k_imma_m8_plain(const void* w, const void* q8_1, float* output, int size_m, int size_n,
+                                              int size_k, void* stream) {
+    (void)rows_plain(w, q8_1, output, size_m, size_n, size_k, size_k / 32, size_n, true, (hipStream_t)stream);
+}
+
+extern "C" int lk_dense_q5k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
+                                        int size_n, int size_k, int use_gelu, void* stream) {
+    return rows_actmul(gate, up, q8_1, output, size_m, size_n, size_k, use_gelu, true, (hipStream_t)stream);
+}
+
+extern "C" void loken_dense_q5k_imma_m8_actmul(const void* gate, const void* up, const void* q8_1, float* output,
+                                               int size_m, int size_n, int size_k, int use_gelu, void* stream) {
+    (void)rows_actmul(gate, up, q8_1, output, size_m, size_n, size_k, use_gelu, true, (hipStream_t)stream);
 }

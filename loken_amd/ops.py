@@ -185,8 +185,8 @@ MMQ_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_gguf_q4_k", _lib.TYPE_Q5_K: "launch_
 MMQ_DEVICE_INFO = dict(cc=0x1000950, nsm=256, smpbo=160 * 1024, warp_size=64)
 
 
-def dense_q4k_rows(weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tensor:
-    """``[rows, k]`` f32 x Q4_K weight ``[n, k]`` -> ``[rows, n]`` f32 on the matrix unit, rows
+def dense_q4k_rows(weight: torch.Tensor, x: torch.Tensor, n: int, q5: bool = False) -> torch.Tensor:
+    """``[rows, k]`` f32 x Q4_K (``q5``: Q5_K) weight ``[n, k]`` -> ``[rows, n]`` f32 on the matrix unit, rows
     quantized to plain Q8_1 first (dense_q4k_imma_m8_matmul, src/inference/moe_cuda/dense/imma.rs:82-135)."""
     rows, k = x.shape
     if k % 256:
@@ -195,8 +195,9 @@ def dense_q4k_rows(weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tenso
     out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
     # the status-returning form of loken_dense_q4k_imma_m8_plain: a launch it declines must not
     # come back as an untouched buffer
-    _lib.check("lk_dense_q4k_rows",
-               _lib.load().lk_dense_q4k_rows(weight.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k, _stream()))
+    fn = _lib.load().lk_dense_q5k_rows if q5 else _lib.load().lk_dense_q4k_rows
+    _lib.check("lk_dense_q5k_rows" if q5 else "lk_dense_q4k_rows",
+               fn(weight.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k, _stream()))
     return out
 
 
@@ -236,15 +237,16 @@ def mmq_forward(wtype: int, weight: torch.Tensor, x: torch.Tensor, n: int) -> to
     return out
 
 
-def dense_q4k_rows_actmul(gate: torch.Tensor, up: torch.Tensor, x: torch.Tensor, n: int, use_gelu: bool) -> torch.Tensor:
-    """``act(gate . x) * (up . x)`` for ``[rows, k]`` f32 x two Q4_K weights ``[n, k]`` in one launch
+def dense_q4k_rows_actmul(gate: torch.Tensor, up: torch.Tensor, x: torch.Tensor, n: int, use_gelu: bool,
+                          q5: bool = False) -> torch.Tensor:
+    """``act(gate . x) * (up . x)`` for ``[rows, k]`` f32 x two Q4_K (``q5``: Q5_K) weights ``[n, k]`` in one launch
     on the matrix unit (dense_q4k_imma_m8_act_mul, src/inference/moe_cuda/dense/imma.rs:320-400)."""
     rows, k = x.shape
     if k % 256:
         raise ValueError("dense_q4k_rows_actmul: k must be a multiple of 256")
     q = quantize_q8_1_rows(x, k_padded=k)
     out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
-    _lib.check("lk_dense_q4k_rows_actmul",
-               _lib.load().lk_dense_q4k_rows_actmul(gate.data_ptr(), up.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k,
-                                                    1 if use_gelu else 0, _stream()))
+    fn = _lib.load().lk_dense_q5k_rows_actmul if q5 else _lib.load().lk_dense_q4k_rows_actmul
+    _lib.check("lk_dense_q5k_rows_actmul" if q5 else "lk_dense_q4k_rows_actmul",
+               fn(gate.data_ptr(), up.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k, 1 if use_gelu else 0, _stream()))
     return out

@@ -121,3 +121,33 @@ def test_gate_and_up_in_one_launch_carry_the_plain_launches_bits():
     want = g / (1.0 + torch.exp(-g)) * u
     got = ops.dense_q4k_rows_actmul(gate, up, x, n, False).double()
     assert ((got - want).abs() <= 2e-6 * want.abs() + 1e-30).all()
+
+
+Q5K = lib.TYPE_Q5_K
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (6, 512, 70), (8, 2048, 257), (16, 1024, 130), (33, 768, 96), (70, 2048, 64),
+                                   (4, 14336, 40)])
+def test_q5k_rows_on_the_matrix_unit_match_same_codes_oracle(m, k, n):
+    """loken_dense_q5k_imma_m8_plain: the fifth bit joins the nibble before the matrix instruction."""
+    w = synth.weight(Q5K, n, k, seed=63, stream=1)
+    x = synth.activation(m, k, seed=63)
+    got = ops.dense_q4k_rows(dev(w), dev(x), n, q5=True).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(Q5K, x, w, n))
+    # the mat-vec family reads the same blocks another way: same integers, different summation order
+    if m <= 8:
+        other = ops.mmvq(Q5K, dev(w), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
+        assert (np.abs(got - other) <= 2e-5 * np.abs(other) + 1e-5 * np.abs(other).max()).all()
+
+
+@pytest.mark.parametrize("m,k,n", [(3, 512, 70), (8, 2048, 130), (20, 1024, 64)])
+@pytest.mark.parametrize("use_gelu", [False, True])
+def test_q5k_gate_and_up_in_one_launch(m, k, n, use_gelu):
+    gate = synth.weight(Q5K, n, k, seed=64, stream=1)
+    up = synth.weight(Q5K, n, k, seed=64, stream=2)
+    x = synth.activation(m, k, seed=64) * np.float32(4.0)
+    g = oracle.ob_matmul(Q5K, x, gate, n).astype(np.float64)
+    u = oracle.ob_matmul(Q5K, x, up, n).astype(np.float64)
+    want = (gelu_tanh(g) if use_gelu else silu(g)) * u
+    got = ops.dense_q4k_rows_actmul(dev(gate), dev(up), dev(x), n, use_gelu, q5=True).cpu().numpy()
+    assert (np.abs(got - want) <= RTOL * np.abs(want) + ATOL * max(1.0, np.abs(want).max())).all()
