@@ -437,6 +437,11 @@ void loken_dense_q5k_imma_m8_actmul(const void* gate, const void* up, const void
                                     int size_m, int size_n, int size_k, int use_gelu, void* stream);
 int lk_dense_q5k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
                              int size_n, int size_k, int use_gelu, void* stream);
+/* Q4_K weight [nrows_x, ncols_x] x ONE plain Q8_1 row -> dst [nrows_x] f32. Name and arguments of the
+ * reference's batch-1 matrix-unit mat-vec (cuda/q4k_mmvq_imma.cu:149-175; AMD twin cuda/moe/imma_amd.cu:476;
+ * declared src/inference/quantized_cuda/mod.rs:29-40, call site quantize.rs:50-60, switched off there);
+ * served by the Q4_K mat-vec launch. ncols_x a multiple of 256; nothing is launched otherwise. */
+void q4k_mmvq_imma(const void* vx, const void* vy, void* dst, int ncols_x, int nrows_x, void* stream);
 /* Q4_K expert rows for a handful of routed pairs per expert, over Q8_1 rows the caller quantized.
  * gate_up: gate_up_weights [num_experts, 2 size_n, size_k] (an expert's gate rows, then its up
  * rows); q8_1 one row per token [size_m / topk, size_k / 32 blocks]; expert_ids one expert PER PAIR;

@@ -138,7 +138,7 @@ static int dispatch_plain(int wtype, int dst_type, int batch, MmvqCall& a) {
     switch (wtype) {
         case LK_TYPE_Q4_K: return a.nb <= 8 ? lk_eng_plain_q4k_short(batch, dst_type, a) : lk_eng_plain_q4k(batch, dst_type, a);
         case LK_TYPE_Q5_K: return a.nb <= 8 ? lk_eng_plain_q5k_short(batch, dst_type, a) : lk_eng_plain_q5k(batch, dst_type, a);
-        case LK_TYPE_Q6_K: return lk_eng_plain_q6k(batch, dst_type, a);
+        case LK_TYPE_Q6_K: return a.nb <= 8 ? lk_eng_plain_q6k_short(batch, dst_type, a) : lk_eng_plain_q6k(batch, dst_type, a);
         case LK_TYPE_Q8_0: return lk_eng_plain_q80(batch, dst_type, a);
         default: return LK_ERR_TYPE;
     }
@@ -230,6 +230,16 @@ extern "C" int lk_mmvq(int wtype, const void* vx, const void* vy_q8_1, void* dst
                      bias ? &bias : nullptr, stream);
 }
 
+// The reference's batch-1 Q4_K mat-vec on the matrix unit (cuda/q4k_mmvq_imma.cu:149-175, AMD twin
+// cuda/moe/imma_amd.cu:476; declared src/inference/quantized_cuda/mod.rs:29-40). One activation row
+// gives a matrix instruction one useful column in thirty-two, and the reference itself no longer
+// takes that path (src/inference/quantized_cuda/quantize.rs:35-47): here the name is the Q4_K
+// mat-vec launch, which computes the same sums.
+extern "C" void q4k_mmvq_imma(const void* vx, const void* vy, void* dst, int ncols_x, int nrows_x, void* stream) {
+    if (ncols_x <= 0 || nrows_x <= 0 || ncols_x % 256 != 0) return;
+    (void)lk_mmvq(LK_TYPE_Q4_K, vx, vy, dst, LK_TYPE_F32, ncols_x, nrows_x, 1, ncols_x / 32, nrows_x, nullptr, 0, stream);
+}
+
 extern "C" int lk_mmvq_multi(int wtype, int count, const void* const* vx, const void* vy_q8_1, void* const* dst,
                              int dst_type, int ncols_x, const int* nrows_x, int batch, int stride_col_y,
                              int stride_col_dst, const float* const* bias, void* stream) {
@@ -277,7 +287,7 @@ extern "C" int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, con
     switch (wtype) {
         case LK_TYPE_Q4_K: return nb <= 8 ? lk_eng_pair_q4k_short(batch, dst_type, c) : lk_eng_pair_q4k(batch, dst_type, c);
         case LK_TYPE_Q5_K: return lk_eng_pair_q5k(batch, dst_type, c);
-        case LK_TYPE_Q6_K: return lk_eng_pair_q6k(batch, dst_type, c);
+        case LK_TYPE_Q6_K: return nb <= 8 ? lk_eng_pair_q6k_short(batch, dst_type, c) : lk_eng_pair_q6k(batch, dst_type, c);
         case LK_TYPE_Q8_0: return lk_eng_pair_q80(batch, dst_type, c);
         default: return LK_ERR_TYPE;
     }
@@ -307,7 +317,7 @@ extern "C" int lk_mmvq_pair_act_q8_1(int wtype, const void* gate, const void* up
     switch (wtype) {
         case LK_TYPE_Q4_K: return lk_eng_pair_q8_1_q4k(batch, c);
         case LK_TYPE_Q5_K: return lk_eng_pair_q8_1_q5k(batch, c);
-        case LK_TYPE_Q6_K: return lk_eng_pair_q8_1_q6k(batch, c);
+        case LK_TYPE_Q6_K: return nb <= 8 ? lk_eng_pair_q8_1_q6k_short(batch, c) : lk_eng_pair_q8_1_q6k(batch, c);
         case LK_TYPE_Q8_0: return lk_eng_pair_q8_1_q80(batch, c);
         default: return LK_ERR_TYPE;
     }
@@ -328,7 +338,9 @@ extern "C" int lk_mmvq_grouped(int wtype, const uint64_t* table, int groups, con
             return nb <= 8 ? lk_eng_grouped_q4k_short(table, groups, y, dst, nb, nrows_x, k32, s)
                            : lk_eng_grouped_q4k(table, groups, y, dst, nb, nrows_x, k32, s);
         case LK_TYPE_Q5_K: return lk_eng_grouped_q5k(table, groups, y, dst, nb, nrows_x, k32, s);
-        case LK_TYPE_Q6_K: return lk_eng_grouped_q6k(table, groups, y, dst, nb, nrows_x, k32, s);
+        case LK_TYPE_Q6_K:
+            return nb <= 8 ? lk_eng_grouped_q6k_short(table, groups, y, dst, nb, nrows_x, k32, s)
+                           : lk_eng_grouped_q6k(table, groups, y, dst, nb, nrows_x, k32, s);
         default: return lk_eng_grouped_q80(table, groups, y, dst, nb, nrows_x, k32, s);
     }
 }

@@ -644,19 +644,26 @@ static __device__ __forceinline__ void step_loop(const RowJob<NW>& job, int tile
 // cycles, not HBM, bound this format). The codes stay unsigned; the -32 offset comes in through
 // the staged per-run activation sums.
 // ---------------------------------------------------------------------------------------------
-template <int B, int R, int NW, class Epi, class Done>
+// PACK: rows of at most 8 (4) super-blocks share a pass two (four) at a time, each in its own 32 (16)
+// lanes, as the short Q4_K rows do.
+template <int B, int R, int NW, bool PACK, class Epi, class Done>
 static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* lds, Epi&& epi, Done&& done) {
     const int nb = job.nb, n = job.n;
-    const int n_iter = (nb + 15) >> 4;
-    const int row_bytes = lds_bytes_per_row<FmtQ6K>(n_iter);
-    const int total = n_iter * 128;   // Q8_1 blocks the staged row is padded to
+    const int n_iter_lds = (nb + 15) >> 4;   // passes of the staged activation (its layout)
+    const int row_bytes = lds_bytes_per_row<FmtQ6K>(n_iter_lds);
+    const int total = n_iter_lds * 128;   // Q8_1 blocks the staged row is padded to
+    const int RP = (!PACK || job.run_len > 1) ? 1 : q4k_rows_per_pass(nb);
+    const int S = PACK ? 16 / RP : 16;       // super-block slots of one row in a pass
+    const int n_iter = (nb + S - 1) / S;     // passes per tile (1 whenever RP > 1)
+    const int TR = R * RP;                   // rows per tile
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lb = lane >> 2, h = (lane >> 1) & 1, lh = lane & 1;
+    const int slot = lb & (S - 1), rp = lb / S;
     const uint32_t ql_off = 64 * h + 16 * lh, qh_off = 128 + 32 * h + 16 * lh, sc_off = 192 + 8 * h;
     const size_t row_stride = (size_t)nb * Q6K_BYTES;
-    const int n_tiles = (n + R - 1) / R;
+    const int n_tiles = (n + TR - 1) / TR;
     constexpr int RW = R * NW;
 
     struct Frag {
@@ -666,12 +673,12 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
     };
     // A lane past the row end re-reads the row's last block and drops its d when it consumes it.
     auto load = [&](Frag& f, int tile, int it) {
-        const int blk_c = min(it * 16 + lb, nb - 1);
+        const int blk_c = min(it * S + slot, nb - 1);
 #pragma unroll
         for (int w = 0; w < NW; ++w)
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const int row = min(tile * R + r, n - 1);
+                const int row = min(tile * TR + rp * R + r, n - 1);
                 const uint8_t* bp = (const uint8_t*)(job.vx[w] + row * row_stride + (size_t)blk_c * Q6K_BYTES);
                 f.ql0[w * R + r] = *(const uint4_a2*)(bp + ql_off);
                 f.ql1[w * R + r] = *(const uint4_a2*)(bp + ql_off + 32);
@@ -688,10 +695,11 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
         for (int c = 0; c < B; ++c) acc[r][c] = 0.f;
 
     auto compute = [&](const Frag& f, int tile, int it) {
+        const int block = it * S + slot;   // the lane's super-block of its row
         float ds[RW][4];
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
-            const float d = it * 16 + lb < nb ? f16_bits_to_f32(f.d[r]) : 0.f;
+            const float d = block < nb ? f16_bits_to_f32(f.d[r]) : 0.f;
             ds[r][0] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].x, 8 * lh, 8);
             ds[r][1] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].x, 8 * lh + 16, 8);
             ds[r][2] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].y, 8 * lh, 8);
@@ -700,12 +708,13 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
 #pragma unroll
         for (int c = 0; c < B; ++c) {
             const uint8_t* rowl = lds + c * row_bytes;
-            const uint8_t* codes = rowl + it * 4096 + lane * 16;
+            const int blk_l = min(block, n_iter_lds * 16 - 1);   // (a lane past a packed row's end: any staged block)
+            const uint8_t* codes = rowl + (blk_l >> 4) * 4096 + ((blk_l & 15) * 4 + (lane & 3)) * 16;
             uint4 a[4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) a[g] = *(const uint4*)(codes + g * 1024);
-            const uint8_t* sc = rowl + n_iter * 4096;
-            const int j0 = (it * 16 + lb) * 8 + 4 * h;   // the half's four Q8_1 blocks
+            const uint8_t* sc = rowl + n_iter_lds * 4096;
+            const int j0 = blk_l * 8 + 4 * h;   // the half's four Q8_1 blocks
             const float4 d8 = *(const float4*)(sc + 4 * j0);
             const int4 bias = *(const int4*)(sc + 4 * (total * (1 + lh) + j0));
 #pragma unroll
@@ -722,18 +731,45 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
 #pragma unroll
                 for (int c = 0; c < B; ++c) {
                     float tot[NW];
+                    if (RP == 1) {
 #pragma unroll
-                    for (int w = 0; w < NW; ++w) {
-                        tot[w] = wave_sum(acc[w * R + r][c]);
-                        acc[w * R + r][c] = 0.f;
+                        for (int w = 0; w < NW; ++w) {
+                            tot[w] = wave_sum(acc[w * R + r][c]);
+                            acc[w * R + r][c] = 0.f;
+                        }
+                        if (lane == 0 && tile * R + r < n) epi(tile * R + r, c, tot);
+                    } else {
+                        float q[NW][4];
+#pragma unroll
+                        for (int w = 0; w < NW; ++w) {
+                            row16_sums(acc[w * R + r][c], q[w]);
+                            acc[w * R + r][c] = 0.f;
+                        }
+                        if (lane == 0) {
+                            const int row0 = tile * TR + r;
+                            if (RP == 2) {
+#pragma unroll
+                                for (int g = 0; g < 2; ++g) {
+#pragma unroll
+                                    for (int w = 0; w < NW; ++w) tot[w] = q[w][2 * g] + q[w][2 * g + 1];
+                                    if (row0 + g * R < n) epi(row0 + g * R, c, tot);
+                                }
+                            } else {
+#pragma unroll
+                                for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                                    for (int w = 0; w < NW; ++w) tot[w] = q[w][g];
+                                    if (row0 + g * R < n) epi(row0 + g * R, c, tot);
+                                }
+                            }
+                        }
                     }
-                    if (lane == 0 && tile * R + r < n) epi(tile * R + r, c, tot);
                 }
             done(tile);
         }
     };
     step_loop<Frag>(job, job.tile_first + wave * job.wave_stride, n_tiles, n_iter,
-                    [&](auto&& mid) { stage_around<FmtQ6K, B>(lds, job, nb * 8, n_iter, mid); }, load, compute);
+                    [&](auto&& mid) { stage_around<FmtQ6K, B>(lds, job, nb * 8, n_iter_lds, mid); }, load, compute);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -856,7 +892,16 @@ struct EngQ6K {
     static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
-        rows_q6k<B, R, NW>(j, lds, e, d);
+        rows_q6k<B, R, NW, false>(j, lds, e, d);
+    }
+};
+// Q6_K rows of at most 8 super-blocks: 2 or 4 rows share a pass.
+struct EngQ6KShort {
+    using Fmt = FmtQ6K;
+    static __host__ __device__ int rows_per_pass(int nb) { return q4k_rows_per_pass(nb); }
+    template <int B, int R, int NW, class Epi, class Done = NoTileHook>
+    static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
+        rows_q6k<B, R, NW, true>(j, lds, e, d);
     }
 };
 struct EngQ80 {

@@ -389,4 +389,5 @@ LK_DECLARE_ENGINE(q4k_short)
 LK_DECLARE_ENGINE(q5k)
 LK_DECLARE_ENGINE(q5k_short)
 LK_DECLARE_ENGINE(q6k)
+LK_DECLARE_ENGINE(q6k_short)
 LK_DECLARE_ENGINE(q80)

@@ -242,7 +242,8 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
                              : launch_mode<EngQ5K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         case 5:
             d.nb = size_k / 256; d.slab_bytes = slab_rows * d.nb * Q6K_BYTES;
-            return launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
+            return d.nb <= 8 ? launch_mode<EngQ6KShort, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s)
+                             : launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         default:
             // Q2_K, Q3_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS: the wave-per-row kernels over Q8_1 rows
             if (d.act_f32) return LK_ERR_ARG;

@@ -390,3 +390,17 @@ def test_pair_q8_1_launch_declines_partial_blocks():
     x = dev(synth.activation(1, 256, seed=71))
     with pytest.raises(lib.LokenError):
         ops.mmvq_pair_act_q8_1(lib.TYPE_Q4_K, gate, gate, x, 256, 40)
+
+
+def test_the_reference_batch1_matrix_unit_name_is_the_q4k_matvec():
+    """q4k_mmvq_imma (cuda/q4k_mmvq_imma.cu:149-175): same arguments, the mat-vec family's bits."""
+    n, k = 300, 2048
+    w = synth.weight(lib.TYPE_Q4_K, n, k, seed=71, stream=1)
+    x = synth.activation(1, k, seed=71)
+    wd = torch.from_numpy(w).cuda()
+    q = ops.quantize_q8_1_rows(torch.from_numpy(x).cuda(), k_padded=k)
+    out = torch.full((n,), -3.0, dtype=torch.float32, device="cuda")
+    lib.load().q4k_mmvq_imma(wd.data_ptr(), q.data_ptr(), out.data_ptr(), k, n, torch.cuda.current_stream().cuda_stream)
+    assert torch.equal(out, ops.mmvq(lib.TYPE_Q4_K, wd, q, k, n)[0])
+    want = oracle.ob_matmul(lib.TYPE_Q4_K, x, w, n)[0]
+    assert (np.abs(out.cpu().numpy() - want) <= 1e-3 * np.abs(want) + 1e-4).all()
