@@ -437,6 +437,14 @@ void loken_dense_q5k_imma_m8_actmul(const void* gate, const void* up, const void
                                     int size_m, int size_n, int size_k, int use_gelu, void* stream);
 int lk_dense_q5k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
                              int size_n, int size_k, int use_gelu, void* stream);
+/* Q6_K weight [size_n rows, size_k] x plain Q8_1 rows [size_m, size_k / 32 blocks] -> output
+ * [size_m, size_n] f32 on the int8 matrix unit: the Q6_K member of the family above. The reference
+ * has no launcher of this shape (its Q6_K rows go one at a time through vec_dot_q6_K_q8_1,
+ * cuda/moe/gguf.cuh:782-816); the host mirror of QKernelMatMul::forward uses it between the mat-vec
+ * kernels and the tiled matmul. LK_ERR_ARG, and nothing launched, for rows too long for the kernel's
+ * scale table in LDS. */
+int lk_dense_q6k_rows(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k,
+                      void* stream);
 /* Q4_K weight [nrows_x, ncols_x] x ONE plain Q8_1 row -> dst [nrows_x] f32. Name and arguments of the
  * reference's batch-1 matrix-unit mat-vec (cuda/q4k_mmvq_imma.cu:149-175; AMD twin cuda/moe/imma_amd.cu:476;
  * declared src/inference/quantized_cuda/mod.rs:29-40, call site quantize.rs:50-60, switched off there);

@@ -25,14 +25,16 @@ enum class Path : int {
     None = 0,
     MatVecFused = 1,   /* lk_mmvq_fused: f32 rows quantized inside the mat-vec launch */
     MatVec = 2,        /* lk_quantize_q8_1 + lk_mmvq (slices of eight rows) */
-    RowsOnMatrixUnit = 3, /* lk_quantize_q8_1 + loken_dense_q4k_imma_m8_plain */
+    RowsOnMatrixUnit = 3, /* lk_quantize_q8_1 + lk_dense_q4k_rows / lk_dense_q5k_rows / lk_dense_q6k_rows */
     Tiled = 4,         /* launch_mmq_quantize_q8_1_* + launch_mmq_gguf_* */
 };
 
 /* The most rows the mat-vec family takes for this weight before the call moves to a matrix-unit
  * kernel (matvec_rows of the reference, kernel_matmul.rs:27-33, with the crossovers measured on
- * MI355X: Q4_K 6 rows, then the rows kernel up to 64, then the tiled matmul; Q6_K / Q8_0 mat-vec
- * slices up to 32 rows, then the tiled matmul). */
+ * MI355X: Q4_K / Q5_K 6 rows and Q6_K 8, then the matrix-unit rows kernels while n x rows is small
+ * enough that a tiled launch would leave the chip idle (1.75 M for Q4_K / Q5_K and never under 64
+ * rows, 4 M for Q6_K), then the tiled matmul; Q8_0 mat-vec slices up to 32 rows, then the tiled
+ * matmul). */
 int matvec_rows(int dtype, int k);
 
 class QKernelMatMul {

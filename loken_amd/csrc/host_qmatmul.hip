@@ -114,8 +114,22 @@ size_t elem_bytes(int type) { return type == LK_TYPE_F32 ? 4 : 2; }
 }  // namespace
 
 int matvec_rows(int dtype, int k) {
-    if (dtype == LK_TYPE_Q4_K && k % 256 == 0) return 6;
+    if ((dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K) && k % 256 == 0) return 6;
+    if (dtype == LK_TYPE_Q6_K && k % 256 == 0) return 8;
     return tiled_serves(dtype, k) ? 32 : 8;
+}
+
+// Rows the matrix-unit rows kernels take before the tiled matmul does. Measured on MI355X over
+// n = 2048 ... 151936 and k = 2048 ... 14336: a rows kernel re-reads the weights for every 32
+// activation rows but fills the chip from the first pass; a tiled launch holds a 128- or 256-row weight
+// block per workgroup and leaves most of the chip idle until n x rows gives it enough tiles. The two
+// meet near n x rows = 1.75 M for Q4_K / Q5_K (4096 x 4096: 480 rows; 14336 x 4096: 110) and 4 M for
+// Q6_K (4096 x 14336: 1000 rows; 151936 x 2048: under 32).
+static bool rows_kernel_serves(int dtype, int n, int rows) {
+    const long long work = (long long)n * rows;
+    if (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K) return rows <= 64 || work <= 1750000;
+    if (dtype == LK_TYPE_Q6_K) return work <= (4ll << 20);
+    return false;
 }
 
 QKernelMatMul::QKernelMatMul(int dtype, int n, int k, const void* blob, int device)
@@ -165,15 +179,18 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     }
     if (x_type != LK_TYPE_F32) return LK_ERR_TYPE;   // the matrix-unit kernels write f32
 
-    // --- Q4_K, a handful of rows: matrix unit, weights straight from HBM
-    if (dtype_ == LK_TYPE_Q4_K && rows <= 64 && ((uintptr_t)blob_ & 15) == 0) {
+    // --- a handful of rows (or a matrix too small to fill the chip with tiles): matrix unit, weights
+    //     straight from HBM
+    if (rows_kernel_serves(dtype_, n_, rows) && k_ % 256 == 0 && ((uintptr_t)blob_ & (dtype_ == LK_TYPE_Q6_K ? 1 : 15)) == 0) {
         const int blocks = k_ / 32;
         std::lock_guard<std::mutex> pair(slot.mu);
         if (int rc = reserve(slot, (size_t)rows * blocks * Q81_BLOCK, false, stream)) return rc;
         if (int rc = lk_quantize_q8_1(x, x_type, slot.act, k_, k_, rows, stream)) return rc;
-        // the launcher with a status (the exported void form drops it): rows too long for its scale
+        // the launchers with a status (the exported void forms drop it): rows too long for their scale
         // tables in LDS launch nothing, and the call goes on to the tiled matmul below
-        const int rc = lk_dense_q4k_rows(blob_, slot.act, (float*)out, rows, n_, k_, stream);
+        const int rc = dtype_ == LK_TYPE_Q4_K   ? lk_dense_q4k_rows(blob_, slot.act, (float*)out, rows, n_, k_, stream)
+                       : dtype_ == LK_TYPE_Q5_K ? lk_dense_q5k_rows(blob_, slot.act, (float*)out, rows, n_, k_, stream)
+                                                : lk_dense_q6k_rows(blob_, slot.act, (float*)out, rows, n_, k_, stream);
         mark_used(slot, stream);
         if (rc == LK_OK) {
             last_path_ = Path::RowsOnMatrixUnit;

@@ -250,3 +250,16 @@ def dense_q4k_rows_actmul(gate: torch.Tensor, up: torch.Tensor, x: torch.Tensor,
     _lib.check("lk_dense_q5k_rows_actmul" if q5 else "lk_dense_q4k_rows_actmul",
                fn(gate.data_ptr(), up.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k, 1 if use_gelu else 0, _stream()))
     return out
+
+
+def dense_q6k_rows(weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tensor:
+    """``[rows, k]`` f32 x Q6_K weight ``[n, k]`` -> ``[rows, n]`` f32 on the matrix unit, rows
+    quantized to plain Q8_1 first."""
+    rows, k = x.shape
+    if k % 256:
+        raise ValueError("dense_q6k_rows: k must be a multiple of 256")
+    q = quantize_q8_1_rows(x, k_padded=k)
+    out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
+    _lib.check("lk_dense_q6k_rows",
+               _lib.load().lk_dense_q6k_rows(weight.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n, k, _stream()))
+    return out

@@ -151,3 +151,50 @@ def test_q5k_gate_and_up_in_one_launch(m, k, n, use_gelu):
     want = (gelu_tanh(g) if use_gelu else silu(g)) * u
     got = ops.dense_q4k_rows_actmul(dev(gate), dev(up), dev(x), n, use_gelu, q5=True).cpu().numpy()
     assert (np.abs(got - want) <= RTOL * np.abs(want) + ATOL * max(1.0, np.abs(want).max())).all()
+
+
+Q6K = lib.TYPE_Q6_K
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 256, 32), (3, 512, 70), (8, 2048, 257), (8, 14336, 40), (9, 768, 64), (16, 1024, 130),
+                                   (16, 14336, 33), (17, 512, 64), (32, 768, 33), (33, 512, 96), (70, 2048, 100)])
+def test_q6k_rows_on_the_matrix_unit_match_same_codes_oracle(m, k, n):
+    """Signed 6-bit codes through v_mfma_i32_32x32x32_i8, one 16-value group per lane half."""
+    w = synth.weight(Q6K, n, k, seed=65, stream=1)
+    x = synth.activation(m, k, seed=65)
+    got = ops.dense_q6k_rows(dev(w), dev(x), n).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(Q6K, x, w, n))
+    if m <= 8:   # the mat-vec family: the same integers, another summation order
+        other = ops.mmvq(Q6K, dev(w), ops.quantize_q8_1_rows(dev(x)), k, n).cpu().numpy()
+        assert (np.abs(got - other) <= 2e-5 * np.abs(other) + 1e-5 * np.abs(other).max()).all()
+
+
+def test_q6k_rows_emit_the_exact_integers_on_crafted_inputs():
+    """Activations on an integer grid with 127 in every block (d8 = 1), weights with d = 1 and scale
+    1 in one group of each super-block and 0 elsewhere: the f32 output is that group's integer dot."""
+    rng = np.random.default_rng(66)
+    m, k, n = 8, 1024, 64
+    nb = k // 256
+    x = rng.integers(-127, 128, size=(m, k)).astype(np.float32)
+    x.reshape(m, k // 32, 32)[:, :, 0] = 127.0
+    w = np.zeros((n, nb, 210), np.uint8)
+    w[:, :, :192] = rng.integers(0, 256, size=(n, nb, 192), dtype=np.uint8)
+    group = rng.integers(0, 16, size=(n, nb))
+    scales = np.zeros((n, nb, 16), np.int8)
+    np.put_along_axis(scales, group[:, :, None], 1, axis=2)
+    w[:, :, 192:208] = scales.view(np.uint8)
+    w[:, :, 208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    got = ops.dense_q6k_rows(dev(w.reshape(n, -1)), dev(x), n).cpu().numpy()
+    # the integer dot, from the format's layout
+    ql, qh = w[:, :, :128].astype(np.int32), w[:, :, 128:192].astype(np.int32)
+    codes = np.zeros((n, nb, 256), np.int32)
+    for half in range(2):
+        for qt in range(4):
+            l = np.arange(32)
+            nib = ql[:, :, 64 * half + 32 * (qt & 1) + l]
+            nib = (nib >> 4) if qt & 2 else (nib & 15)
+            hi = (qh[:, :, 32 * half + l] >> (2 * qt)) & 3
+            codes[:, :, 128 * half + 32 * qt + l] = (nib | (hi << 4)) - 32
+    mask = (np.arange(256)[None, None, :] // 16) == group[:, :, None]
+    want = np.einsum("nbk,mbk->mn", (codes * mask).astype(np.int64), x.reshape(m, nb, 256).astype(np.int64))
+    assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, got.astype(np.int64))
