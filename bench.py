@@ -27,6 +27,8 @@ Two more measurements ride in the same JSON line:
                 workload, on this host's cores.
   gemv_4096     BASELINE config 0 (Q4_K 4096 x 4096, one row) over rotating copies.
   mmq           BASELINE configs 2a / 2b, the tiled matmul, against the int8 matrix peak.
+  rows-sweep    one --wtype q4_k|q6_k matrix (--rows-n x --cols-k) at 16..2048 rows: the matrix-unit
+                rows kernel against the tiled matmul, and the path QKernelMatMul::forward's mirror takes.
   roofline.peak_measured / mmq.peak_measured: what a read-only launch and a register-resident
                 matrix-instruction loop reach on this card (loken_amd/probes.py).
 """
@@ -47,7 +49,7 @@ HBM_PEAK_GBS = 8000.0
 # profiles/mmvq_llama3_8b_decode_b1_hbm_traffic.md. Counters cannot be read from inside this
 # process, so the figure is carried here for the configuration it was taken on:
 # (launch plan, batch, layers) -> bytes.
-MEASURED_TRAFFIC = {("auto", 1, 32): 30192100}
+MEASURED_TRAFFIC = {("auto", 1, 32): 30123486}
 LAYERS = 32
 HIDDEN, KV, FFN, VOCAB = 4096, 1024, 14336, 128256
 
@@ -71,7 +73,7 @@ def parse_args():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of 1 GiB before the steps: the dispatch of known size that "
                          "scales the FETCH_SIZE / WRITE_SIZE counters of a profiled run")
-    ap.add_argument("--workload", choices=["decode", "gemv", "gemv-4096", "mmq", "moe", "decode-1p7b"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemv", "gemv-4096", "mmq", "moe", "decode-1p7b", "rows-sweep"], default="decode",
                     help="decode (default): the Llama-3-8B step described above; the others are the further measured "
                          "workloads of loken_amd/workloads.py, one JSON line each")
     ap.add_argument("--shape", choices=["2a", "2b"], default="2a", help="--workload mmq: 512x4096->14336 Q4_K or 2048x14336->4096 Q6_K")
@@ -369,11 +371,11 @@ def main() -> int:
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC.get((args.plan, b, args.layers)),
-                "kernel": (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<1,1,true> (q+k+v), q4k_reg_kernel<2,1,true> (o), "
+                "kernel": (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<2,1,true> (q+k+v, 768 workgroups; o, 512), "
                            f"q4k_reg_pair_kernel<1,true,true> (gate+up)") if kind == "auto" and b == 1
                           else (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
                                 f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if kind == "auto"
-                          else ("q4k_rows_staged_kernel<1> (q, o, gate, up), " if kind == "rows" else "")
+                          else ("q4k_rows_staged_kernel<1,false,false> (q, o, gate, up), " if kind == "rows" else "")
                           + f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches,
                 "timed_as": "graph replay of the mix" if q4k_graph is not None else "eager launches"}

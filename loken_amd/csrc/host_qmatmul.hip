@@ -123,11 +123,12 @@ int matvec_rows(int dtype, int k) {
 // n = 2048 ... 151936 and k = 2048 ... 14336: a rows kernel re-reads the weights for every 32
 // activation rows but fills the chip from the first pass; a tiled launch holds a 128- or 256-row weight
 // block per workgroup and leaves most of the chip idle until n x rows gives it enough tiles. The two
-// meet near n x rows = 1.75 M for Q4_K / Q5_K (4096 x 4096: 480 rows; 14336 x 4096: 110) and 4 M for
-// Q6_K (4096 x 14336: 1000 rows; 151936 x 2048: under 32).
+// meet near n x rows = 1.75 M for Q4_K / Q5_K (4096 x 4096: 480 rows; 14336 x 4096: 110; 128256 x 4096:
+// the rows kernel still wins at 16) and 4 M for Q6_K (4096 x 14336: 1000 rows; 151936 x 2048: under 32).
+// `bench.py --workload rows-sweep` prints the table for a shape.
 static bool rows_kernel_serves(int dtype, int n, int rows) {
     const long long work = (long long)n * rows;
-    if (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K) return rows <= 64 || work <= 1750000;
+    if (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K) return rows <= 16 || work <= 1750000;
     if (dtype == LK_TYPE_Q6_K) return work <= (4ll << 20);
     return false;
 }

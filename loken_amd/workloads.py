@@ -579,10 +579,65 @@ def brief_mmq(shape, launches=30):
             "quantize_plus_matmul_us": round(both, 2), "tops_with_quantizer": round(op_count / both / 1e6, 1)}
 
 
+# ---------------------------------------------------------------------------- rows kernels against tiles
+def rows_sweep(args, dev):
+    """One weight matrix at a ladder of row counts: quantizer + matrix-unit rows kernel against
+    quantizer + tiled matmul, each as a graph replay of the two launches, and the path the host
+    mirror of QKernelMatMul::forward takes. The crossover constants in host_qmatmul.hip come from
+    these tables."""
+    L = lib.load()
+    wtype = {"q4_k": Q4K, "q6_k": Q6K}.get(args.wtype)
+    if wtype is None:
+        raise SystemExit("--workload rows-sweep: --wtype q4_k or q6_k")
+    n, k = args.rows_n, args.cols_k
+    mk = Maker(dev)
+    w = mk.make(wtype, n, k)
+    quantizer = getattr(L, ops.MMQ_QUANTIZER[wtype])
+    launcher = getattr(L, ops.MMQ_LAUNCHER[wtype])
+    rows_fn = L.lk_dense_q4k_rows if wtype == Q4K else L.lk_dense_q6k_rows
+    info = ops.MMQ_DEVICE_INFO
+    k_padded = ops.pad_to(ops.pad_to(k, 512), 128)
+    handle = L.lkh_qkernel_matmul_new(wtype, n, k, w.data_ptr(), dev.index or 0)
+    paths = {1: "matvec-fused", 2: "matvec", 3: "rows-on-matrix-unit", 4: "tiled"}
+    table = []
+    for m in (16, 32, 64, 128, 256, 512, 1024, 2048):
+        x = mk.randn(m, k)
+        out = torch.empty((m, n), device=dev)
+        ws = torch.empty(ops.mmq_workspace_bytes(m, k), dtype=torch.uint8, device=dev)
+        q = torch.empty((m, k // 32, 36), dtype=torch.uint8, device=dev)
+
+        def tiled():
+            s = torch.cuda.current_stream().cuda_stream
+            quantizer(x.data_ptr(), None, ws.data_ptr(), 0, k, x.stride(0), 0, 0, k_padded, m, 1, 1, s)
+            if launcher(None, w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
+                        info["cc"], info["nsm"], info["smpbo"], info["warp_size"], s) == 0:
+                raise lib.LokenError(ops.MMQ_LAUNCHER[wtype], lib.LK_ERR_ARG)
+
+        def rows():
+            s = torch.cuda.current_stream().cuda_stream
+            check(L.lk_quantize_q8_1(x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, m, s), "lk_quantize_q8_1")
+            check(rows_fn(w.data_ptr(), q.data_ptr(), out.data_ptr(), m, n, k, s), "rows kernel")
+
+        t_tiled = float(np.median(time_replays(capture(tiled), 12, warm=3)))
+        t_rows = float(np.median(time_replays(capture(rows), 12, warm=3)))
+        check(L.lkh_qkernel_matmul_forward(handle, x.data_ptr(), lib.TYPE_F32, m, out.data_ptr(),
+                                           torch.cuda.current_stream().cuda_stream, 0), "lkh_qkernel_matmul_forward")
+        table.append({"rows": m, "rows_kernel_us": round(t_rows, 1), "tiled_us": round(t_tiled, 1),
+                      "forward_takes": paths.get(L.lkh_qkernel_matmul_last_path(handle), "none")})
+    L.lkh_qkernel_matmul_free(handle)
+    best = min(table, key=lambda r: min(r["rows_kernel_us"], r["tiled_us"]) / r["rows"])
+    op_count = 2.0 * best["rows"] * k * n
+    us = min(best["rows_kernel_us"], best["tiled_us"])
+    return line(args, op_count / us / 1e6, "TOP/s", us * 1e-3, "int8",
+                {"workload": f"{NAMES[wtype]} {n} x {k}: quantizer + rows kernel against quantizer + tiled matmul, graph replays"},
+                None, {"table": table})
+
+
 def run(args) -> int:
     if not torch.cuda.is_available():
         raise SystemExit("bench.py: no GPU visible")
     lib.load()  # raises if the HIP library is missing: there is no other path
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    return {"gemv": gemv, "gemv-4096": gemv_4096, "mmq": mmq, "moe": moe_block, "decode-1p7b": decode_1p7b}[args.workload](args, dev)
+    return {"gemv": gemv, "gemv-4096": gemv_4096, "mmq": mmq, "moe": moe_block, "decode-1p7b": decode_1p7b,
+            "rows-sweep": rows_sweep}[args.workload](args, dev)
