@@ -84,9 +84,10 @@ def parse_args():
     ap.add_argument("--moe-wtype", default="q4_k", help="--workload moe: the experts' format (as --wtype)")
     ap.add_argument("--moe-path", choices=["auto", "tiled", "pairs"], default="auto",
                     help="--workload moe: expert-batched tiled matmul, mat-vec per routed pair, or the library's choice")
-    ap.add_argument("--mid-rows", choices=["matvec", "tiled"], default="matvec",
-                    help="--workload decode-1p7b, 9..32 rows: Q6_K linears as mat-vec launches over slices of eight "
-                         "rows, or through the tiled matmul")
+    ap.add_argument("--mid-rows", choices=["auto", "matvec", "tiled"], default="auto",
+                    help="--workload decode-1p7b above 8 rows: auto = the host mirror's choice between the matrix-unit "
+                         "rows kernels and the tiled matmul; matvec = mat-vec launches over slices of eight rows up to "
+                         "32 rows; tiled = the tiled matmul")
     ap.add_argument("--launches", type=int, default=200, help="timed launches of the per-launch workloads")
     return ap.parse_args()
 

@@ -397,6 +397,10 @@ def decode_1p7b(args, dev):
     acts["final"] = mk.randn(b, hidden)
     keep, plan, total_bytes = [], [], 0
     matvec = b <= 8
+    used = {"rows": 0, "matvec": 0, "tiled": 0}
+
+    def rows_kernel_serves(wtype, n, rows):   # the rule of host_qmatmul.hip
+        return (rows <= 16 or n * rows <= 1750000) if wtype == Q4K else n * rows <= (4 << 20)
 
     def add_group(g, k, wtype, ns):
         nonlocal total_bytes
@@ -422,17 +426,20 @@ def decode_1p7b(args, dev):
                 keep.append(out)
                 plan.append(("status", L.lk_mmvq, (wtype, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, b,
                                          q.shape[1], n, None, 0, s)))
-        elif wtype == Q4K and b <= 64:
-            # a handful of rows: Q4_K on the matrix unit without weight staging
+        elif args.mid_rows == "auto" and all(rows_kernel_serves(wtype, n, b) for n in ns):
+            # the host mirror's choice (host_qmatmul.hip): the matrix-unit rows kernels, no weight staging
             q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
             keep.append(q)
             plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s)))
             for w, n in zip(weights, ns):
                 out = torch.empty((b, n), device=dev)
                 keep.append(out)
-                plan.append(("void", L.loken_dense_q4k_imma_m8_plain, (w.data_ptr(), q.data_ptr(), out.data_ptr(), b, n, k, s)))
+                plan.append(("status", L.lk_dense_q4k_rows if wtype == Q4K else L.lk_dense_q6k_rows,
+                             (w.data_ptr(), q.data_ptr(), out.data_ptr(), b, n, k, s)))
+                used["rows"] += 1
         elif b <= 32 and args.mid_rows == "matvec":
             # mat-vec launches over slices of eight rows
+            used["matvec"] += len(ns)
             q = torch.empty((b, ops.pad_to(k, 512) // 32, 36), dtype=torch.uint8, device=dev)
             keep.append(q)
             plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, q.shape[1] * 32, b, s)))
@@ -444,6 +451,7 @@ def decode_1p7b(args, dev):
                     plan.append(("status", L.lk_mmvq, (wtype, w.data_ptr(), q[r0].data_ptr(), out[r0].data_ptr(),
                                                         lib.TYPE_F32, k, n, rows, q.shape[1], n, None, 0, s)))
         else:
+            used["tiled"] += len(ns)
             k_padded = ops.pad_to(ops.pad_to(k, 512), 128)
             ws = torch.empty(ops.mmq_workspace_bytes(b, k), dtype=torch.uint8, device=dev)
             keep.append(ws)
@@ -496,9 +504,8 @@ def decode_1p7b(args, dev):
                 {"workload": f"qwen3-1.7b decode-step quantized linears (Q4_K attention and gate/up, Q6_K down and "
                              f"lm_head), batch {b}, 28 layers",
                  "path": "mat-vec (fused; own quantizer launch for rows over 8192 values)" if matvec
-                         else "Q4_K: matrix-unit rows kernel (no weight staging); Q6_K: "
-                              + ("mat-vec over slices of eight rows" if b <= 32 and args.mid_rows == "matvec"
-                                 else "tiled int8-MFMA matmul"),
+                         else f"linears on the matrix-unit rows kernels: {used['rows']}, as mat-vec slices of eight rows: "
+                              f"{used['matvec']}, on the tiled matmul: {used['tiled']}",
                  "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline)
 
 

@@ -23,7 +23,11 @@
  * pack/unpack round-trip for the 6-bit scales; closed forms for the three activation
  * quantizers; numpy int64 brute force for every integer sum; an f64 dot over dequantized
  * values and the reduction to a plain int8 GEMV for the f32 combines; decomposition into
- * single-matrix calls for the MoE routines; a textbook softmax/top-k for the router.
+ * single-matrix calls for the MoE routines; a textbook softmax/top-k for the router; for the
+ * served Q4_K path of cpu_baseline.c (eight-row repack, group dot, persistent pool:
+ * tests/test_oracle_served_cpu_path.py) the reference's index map byte by byte, the exact integer
+ * combination of the scalar definition on crafted inputs, the reference's own vector-vs-scalar
+ * bound on random ones, and the same bits whatever the pool size. No function is parity unpinned.
  */
 #ifndef LOKEN_ORACLE_H
 #define LOKEN_ORACLE_H
