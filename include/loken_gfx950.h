@@ -521,7 +521,7 @@ int lk_probe_empty(int workgroups, void* stream);
 int lk_probe_read(const void* src, int64_t bytes, int workgroups, int pattern, void* sink, void* stream);
 /* Register-resident matrix-unit loop: each of a workgroup's four matrix waves issues `iters` x 4
  * independent instructions of `kind` (0 v_mfma_i32_32x32x32_i8, 1 v_mfma_f32_32x32x16_f16,
- * 2 v_mfma_i32_16x16x64_i8). valu_per_mfma (a multiple of 8) independent f32 fmas ride along per
+ * 2 v_mfma_i32_16x16x64_i8, 3 v_mfma_i32_32x32x16_i8). valu_per_mfma (a multiple of 8) independent f32 fmas ride along per
  * matrix instruction: in the same wave (mode 0), or in four further waves, one beside each matrix
  * wave on its SIMD (mode 1). *ops (nullable, host memory) receives the matrix operations launched. */
 int lk_probe_mfma(int kind, int workgroups, int iters, int valu_per_mfma, int mode, void* sink, double* ops,

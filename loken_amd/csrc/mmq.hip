@@ -474,12 +474,19 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
                         // half leaves the 16-value group the other weight scale does not govern
                         const v4i zero = {0, 0, 0, 0};
                         const v4i b_lo = lh == 0 ? b[jt] : zero, b_hi = lh == 0 ? zero : b[jt];
-                        v16i c0 = {0}, c1 = {0};
+                        // The accumulators start at the bit pattern of 1.5 * 2^23, so the dots leave
+                        // the matrix unit as the floats MAGIC + dot and no conversion is spent; the
+                        // offset comes off inside the fma, exactly (the weight scale is an f16 times
+                        // an int8, 18 significant bits: MAGIC * scale does not round).
+                        v16i c0, c1;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) c0[v] = c1[v] = 0x4B400000;
                         c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[it], b_lo, c0, 0, 0, 0);
                         c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[it], b_hi, c1, 0, 0, 0);
+                        const float off0 = -12582912.0f * ws[jt], off1 = -12582912.0f * ws2[jt];
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            const float t = fmaf(ws2[jt], (float)c1[v], ws[jt] * (float)c0[v]);
+                            const float t = fmaf(__int_as_float(c0[v]), ws[jt], off0) + fmaf(__int_as_float(c1[v]), ws2[jt], off1);
                             acc[it][jt][v] = fmaf(t, d8v[v], acc[it][jt][v]);
                         }
                     } else {

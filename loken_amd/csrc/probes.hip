@@ -81,6 +81,16 @@ struct Mfma<2> {   // v_mfma_i32_16x16x64_i8
     static __device__ __forceinline__ Acc step(v4i a, v4i b, Acc c) { return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0); }
 };
 
+template <>
+struct Mfma<3> {   // v_mfma_i32_32x32x16_i8: the K = 16 form (8 bytes per lane and operand)
+    using Acc = v16i;
+    static constexpr double OPS = 2.0 * 32 * 32 * 16;
+    static __device__ __forceinline__ Acc step(v4i a, v4i b, Acc c) {
+        const long a8 = ((long)(unsigned)a[0]) | ((long)a[1] << 32), b8 = ((long)(unsigned)b[0]) | ((long)b[1] << 32);
+        return __builtin_amdgcn_mfma_i32_32x32x16_i8(a8, b8, c, 0, 0, 0);
+    }
+};
+
 template <int KIND>
 __global__ __launch_bounds__(512) void probe_mfma_kernel(int iters, int valu, int mode, uint32_t* sink) {
     using M = Mfma<KIND>;
@@ -163,6 +173,7 @@ extern "C" int lk_probe_mfma(int kind, int workgroups, int iters, int valu_per_m
         case 0: hipLaunchKernelGGL(probe_mfma_kernel<0>, dim3(workgroups), dim3(threads), 0, s, iters, valu_per_mfma, mode, out); per = Mfma<0>::OPS; break;
         case 1: hipLaunchKernelGGL(probe_mfma_kernel<1>, dim3(workgroups), dim3(threads), 0, s, iters, valu_per_mfma, mode, out); per = Mfma<1>::OPS; break;
         case 2: hipLaunchKernelGGL(probe_mfma_kernel<2>, dim3(workgroups), dim3(threads), 0, s, iters, valu_per_mfma, mode, out); per = Mfma<2>::OPS; break;
+        case 3: hipLaunchKernelGGL(probe_mfma_kernel<3>, dim3(workgroups), dim3(threads), 0, s, iters, valu_per_mfma, mode, out); per = Mfma<3>::OPS; break;
         default: return LK_ERR_ARG;
     }
     if (ops) *ops = per * ACCS * (double)iters * 4.0 * (double)workgroups;

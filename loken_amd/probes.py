@@ -17,8 +17,9 @@ import torch
 from . import lib
 
 HBM_PEAK_GBS = 8000.0
-PEAK_TOPS = {0: 5000.0, 1: 2500.0, 2: 5000.0}
-MFMA_NAMES = {0: "v_mfma_i32_32x32x32_i8", 1: "v_mfma_f32_32x32x16_f16", 2: "v_mfma_i32_16x16x64_i8"}
+PEAK_TOPS = {0: 5000.0, 1: 2500.0, 2: 5000.0, 3: 5000.0}
+MFMA_NAMES = {0: "v_mfma_i32_32x32x32_i8", 1: "v_mfma_f32_32x32x16_f16", 2: "v_mfma_i32_16x16x64_i8",
+              3: "v_mfma_i32_32x32x16_i8"}
 
 
 def _check(rc, what):
@@ -132,7 +133,7 @@ def sweep():
                                                "pattern": best[3], "frac_of_8tbs": round(best[1] / HBM_PEAK_GBS, 4)}
     del rb
     out["mfma"] = {}
-    for kind in (0, 1, 2):
+    for kind in (0, 1, 2, 3):
         tops, us = mfma_rate(kind)
         out["mfma"][MFMA_NAMES[kind]] = {"tops": round(tops, 1), "frac_of_nominal": round(tops / PEAK_TOPS[kind], 4), "us": round(us, 1)}
     # vector work beside matrix work: the same wave, or a second wave on the same SIMD

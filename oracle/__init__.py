@@ -61,6 +61,13 @@ def _declare(l: C.CDLL) -> None:
     l.oa_matmul.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _sz, _vp]
     l.oa_matmul_fast.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _i]
     l.oa_matmul_exact.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp]
+    l.lko_dot_q4k_q8k.argtypes = [_i, _vp, _vp, _sz]
+    l.lko_dot_q4k_q8k.restype = C.c_float
+    l.lko_dot_q4k_q8k_many.argtypes = [_vp, _vp, _sz, _sz, _vp]
+    l.lko_dot_q4k_q8k_many.restype = None
+    for fn in (l.oa_matmul_multi, l.oa_matmul_grouped):
+        fn.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp]
+        fn.restype = _i
     l.ob_subdots.argtypes = [_i, _sz, _sz, _vp, _vp, _vp, _vp]
     l.ob_matmul_q8_1.argtypes = [_i, _sz, _sz, _sz, _vp, _sz, _vp, _vp]
     l.ob_matmul.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp]
@@ -155,7 +162,7 @@ class OracleError(ValueError):
 
 
 _ERR = {-1: "k is not a multiple of the block size", -2: "rhs byte length is wrong",
-        -3: "dtype not handled"}
+        -3: "dtype not handled", -4: "an lhs entry has the wrong length", -5: "an outs entry has the wrong length"}
 
 
 def _check(rc: int) -> None:
@@ -175,6 +182,57 @@ def oa_matmul(dtype: int, lhs, rhs, n: int, *, fast_threads: int = 0, exact: boo
     else:
         _check(lib().oa_matmul(dtype, m, k, n, _p(lhs), _p(rhs), rhs.size, _p(dst)))
     return dst
+
+
+def _per_expert(fn, dtype: int, k: int, n: int, rhs_list, lhs_list, out_shapes):
+    import ctypes as C
+    ne = len(rhs_list)
+    rhs = [_u8(r) for r in rhs_list]
+    lhs = [_f32(x).reshape(-1) for x in lhs_list]
+    outs = [np.empty(int(np.prod(s)), np.float32) for s in out_shapes]
+    ptrs = lambda arrs: (C.c_void_p * max(ne, 1))(*[a.ctypes.data for a in arrs])
+    sizes = lambda arrs: (C.c_size_t * max(ne, 1))(*[a.size for a in arrs])
+    _check(fn(dtype, k, n, ne, ptrs(rhs), sizes(rhs), ptrs(lhs), sizes(lhs), ptrs(outs), sizes(outs)))
+    return [o.reshape(s) for o, s in zip(outs, out_shapes)]
+
+
+def oa_matmul_multi(dtype: int, k: int, n: int, rhs_list, lhs_list, out_lens=None):
+    """matmul_bytes_multi: expert e's one row against its own weight -> a list of ``[n]`` outputs."""
+    shapes = [(n,)] * len(rhs_list) if out_lens is None else [(l,) for l in out_lens]
+    return _per_expert(lib().oa_matmul_multi, dtype, k, n, rhs_list, lhs_list, shapes)
+
+
+def oa_matmul_grouped(dtype: int, k: int, n: int, rhs_list, lhs_list, out_shapes=None):
+    """matmul_bytes_grouped: expert e's rows ``[rows_e, k]`` against its own weight -> ``[rows_e, n]`` each."""
+    if out_shapes is None:
+        out_shapes = [(np.asarray(x).size // k, n) for x in lhs_list]
+    return _per_expert(lib().oa_matmul_grouped, dtype, k, n, rhs_list, lhs_list, out_shapes)
+
+
+def dot_q4k_q8k(w_row, x_row, wide: bool = False) -> float:
+    """One Q4_K row against one f32 row quantized to Q8_K, through the 256-bit or the 512-bit kernel."""
+    w = _u8(w_row)
+    x = _f32(x_row).reshape(-1)
+    nb = x.size // 256
+    act = np.empty(nb * 292, np.uint8)
+    lib().lko_quantize_q8_k(_p(x), x.size, _p(act))
+    return float(lib().lko_dot_q4k_q8k(1 if wide else 0, _p(w), _p(act), nb))
+
+
+def dot_q4k_q8k_many(w_row, x_rows) -> np.ndarray:
+    """One Q4_K row against several f32 rows (each quantized to Q8_K) in passes of four."""
+    import ctypes as C
+    w = _u8(w_row)
+    x = _f32(x_rows)
+    rows, k = x.shape
+    nb = k // 256
+    acts = [np.empty(nb * 292, np.uint8) for _ in range(rows)]
+    for r in range(rows):
+        lib().lko_quantize_q8_k(_p(np.ascontiguousarray(x[r])), k, _p(acts[r]))
+    ptrs = (C.c_void_p * max(rows, 1))(*[a.ctypes.data for a in acts])
+    out = np.empty(rows, np.float32)
+    lib().lko_dot_q4k_q8k_many(_p(w), ptrs, rows, nb, _p(out))
+    return out
 
 
 def repack_q4k_x8(rhs, n: int, k: int) -> np.ndarray:

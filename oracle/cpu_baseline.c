@@ -75,6 +75,110 @@ static float dot_q4k_q8k_avx2(const uint8_t* w, const uint8_t* y, size_t nb) {
     return total;
 }
 
+/* The same dot for up to four activation rows in one pass over the weight row
+ * (vec_dot_q4k_q8k_many, avx/superblock.rs:425-490): a block's scales and nibble vectors are
+ * formed once and spent on every row; each row then runs the one-row kernel's own operations in
+ * its order, so out[t] carries the bits of dot_q4k_q8k_avx2(w, ys[t]). */
+#define LKO_MANY_ROWS 4
+static void dot_q4k_q8k_many4_avx2(const uint8_t* w, const uint8_t* const* ys, size_t rows, size_t nb, float* out) {
+    const __m256i nib = _mm256_set1_epi8(0x0F);
+    const __m256i ones = _mm256_set1_epi16(1);
+    float total[LKO_MANY_ROWS] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * LKO_Q4K_BYTES;
+        uint8_t sc[8], mn[8];
+        lko_unpack_scales_mins(x + 4, sc, mn);
+        const float d = f16_to_f32_hw(rd16(x)), dmin = f16_to_f32_hw(rd16(x + 2));
+        __m256i code[8], scale[8];
+        for (int j = 0; j < 4; ++j) {
+            const __m256i packed = _mm256_loadu_si256((const __m256i*)(x + 16 + 32 * j));
+            code[2 * j] = _mm256_and_si256(packed, nib);
+            code[2 * j + 1] = _mm256_and_si256(_mm256_srli_epi16(packed, 4), nib);
+            scale[2 * j] = _mm256_set1_epi32(sc[2 * j]);
+            scale[2 * j + 1] = _mm256_set1_epi32(sc[2 * j + 1]);
+        }
+        for (size_t t = 0; t < rows; ++t) {
+            const uint8_t* yb = ys[t] + b * LKO_Q8K_BYTES;
+            float yd;
+            memcpy(&yd, yb, 4);
+            const int8_t* acts = (const int8_t*)(yb + 4);
+            const int16_t* bsums = (const int16_t*)(yb + 260);
+            __m256i acc = _mm256_setzero_si256();
+            int32_t offset = 0;
+            for (int j = 0; j < 4; ++j) {
+                const __m256i a_lo = _mm256_loadu_si256((const __m256i*)(acts + 64 * j));
+                const __m256i a_hi = _mm256_loadu_si256((const __m256i*)(acts + 64 * j + 32));
+                const __m256i p_lo = _mm256_madd_epi16(_mm256_maddubs_epi16(code[2 * j], a_lo), ones);
+                const __m256i p_hi = _mm256_madd_epi16(_mm256_maddubs_epi16(code[2 * j + 1], a_hi), ones);
+                acc = _mm256_add_epi32(acc, _mm256_mullo_epi32(p_lo, scale[2 * j]));
+                acc = _mm256_add_epi32(acc, _mm256_mullo_epi32(p_hi, scale[2 * j + 1]));
+                offset += (int32_t)mn[2 * j] * ((int32_t)bsums[4 * j] + bsums[4 * j + 1]);
+                offset += (int32_t)mn[2 * j + 1] * ((int32_t)bsums[4 * j + 2] + bsums[4 * j + 3]);
+            }
+            total[t] += yd * (d * (float)hsum_i32_8(acc) - dmin * (float)offset);
+        }
+    }
+    for (size_t t = 0; t < rows; ++t) out[t] = total[t];
+}
+void lko_dot_q4k_q8k_many(const uint8_t* w, const uint8_t* const* ys, size_t rows, size_t nb, float* out) {
+    for (size_t t0 = 0; t0 < rows; t0 += LKO_MANY_ROWS)
+        dot_q4k_q8k_many4_avx2(w, ys + t0, rows - t0 < LKO_MANY_ROWS ? rows - t0 : LKO_MANY_ROWS, nb, out + t0);
+}
+
+/* The 512-bit twin (avx512/superblock.rs:20-90): a 64-byte load holds two of the block's 32-byte runs,
+ * one VNNI byte dot-product covers the low (or high) nibbles of both against their activations, and
+ * the integer sums are those of the 256-bit kernel, so the folded result carries its bits. */
+__attribute__((target("avx2,fma,f16c,avx512f,avx512bw,avx512vl,avx512dq,avx512vnni")))
+static float dot_q4k_q8k_avx512(const uint8_t* w, const uint8_t* y, size_t nb) {
+    const __m512i nib = _mm512_set1_epi8(0x0F);
+    float total = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+        const uint8_t* x = w + b * LKO_Q4K_BYTES;
+        const uint8_t* yb = y + b * LKO_Q8K_BYTES;
+        uint8_t sc[8], mn[8];
+        lko_unpack_scales_mins(x + 4, sc, mn);
+        float yd;
+        memcpy(&yd, yb, 4);
+        const int8_t* acts = (const int8_t*)(yb + 4);
+        const int16_t* bsums = (const int16_t*)(yb + 260);
+        __m512i acc = _mm512_setzero_si512();
+        int32_t offset = 0;
+        for (int h = 0; h < 2; ++h) {
+            /* runs 2h and 2h + 1 of the nibbles; a run's low nibbles meet activations 64 j .. 64 j + 31,
+             * its high nibbles 64 j + 32 .. 64 j + 63 */
+            const __m512i packed = _mm512_loadu_si512((const void*)(x + 16 + 64 * h));
+            const __m512i lo = _mm512_and_si512(packed, nib);
+            const __m512i hi = _mm512_and_si512(_mm512_srli_epi16(packed, 4), nib);
+            const __m256i a0 = _mm256_loadu_si256((const __m256i*)(acts + 128 * h));
+            const __m256i a1 = _mm256_loadu_si256((const __m256i*)(acts + 128 * h + 32));
+            const __m256i a2 = _mm256_loadu_si256((const __m256i*)(acts + 128 * h + 64));
+            const __m256i a3 = _mm256_loadu_si256((const __m256i*)(acts + 128 * h + 96));
+            const __m512i a_lo = _mm512_inserti64x4(_mm512_castsi256_si512(a0), a2, 1);
+            const __m512i a_hi = _mm512_inserti64x4(_mm512_castsi256_si512(a1), a3, 1);
+            const __m512i s_lo = _mm512_inserti64x4(_mm512_set1_epi32(sc[4 * h]), _mm256_set1_epi32(sc[4 * h + 2]), 1);
+            const __m512i s_hi = _mm512_inserti64x4(_mm512_set1_epi32(sc[4 * h + 1]), _mm256_set1_epi32(sc[4 * h + 3]), 1);
+            acc = _mm512_add_epi32(acc, _mm512_mullo_epi32(_mm512_dpbusd_epi32(_mm512_setzero_si512(), lo, a_lo), s_lo));
+            acc = _mm512_add_epi32(acc, _mm512_mullo_epi32(_mm512_dpbusd_epi32(_mm512_setzero_si512(), hi, a_hi), s_hi));
+            for (int r = 0; r < 2; ++r) {
+                const int j = 2 * h + r;
+                offset += (int32_t)mn[2 * j] * ((int32_t)bsums[4 * j] + bsums[4 * j + 1]);
+                offset += (int32_t)mn[2 * j + 1] * ((int32_t)bsums[4 * j + 2] + bsums[4 * j + 3]);
+            }
+        }
+        const int32_t scaled = _mm512_reduce_add_epi32(acc);
+        total += yd * (f16_to_f32_hw(rd16(x)) * (float)scaled - f16_to_f32_hw(rd16(x + 2)) * (float)offset);
+    }
+    return total;
+}
+int lko_cpu_has_avx512(void) {
+    return __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw") && __builtin_cpu_supports("avx512vl") &&
+           __builtin_cpu_supports("avx512dq") && __builtin_cpu_supports("avx512vnni");
+}
+/* One Q4_K row against one Q8_K row through the 256-bit (wide = 0) or 512-bit (wide = 1) kernel. */
+float lko_dot_q4k_q8k(int wide, const uint8_t* w, const uint8_t* y, size_t nb) {
+    return wide ? dot_q4k_q8k_avx512(w, y, nb) : dot_q4k_q8k_avx2(w, y, nb);
+}
+
 /* Q6_K row against Q8_K row: codes kept unsigned 0..63, the 32 folded in through bsums. */
 static float dot_q6k_q8k_avx2(const uint8_t* w, const uint8_t* y, size_t nb) {
     const __m256i nib = _mm256_set1_epi8(0x0F);

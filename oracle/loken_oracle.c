@@ -941,6 +941,59 @@ int oa_matmul(int dtype, size_t m, size_t k, size_t n, const float* lhs,
     return 0;
 }
 
+/* drivers.rs:2144-2316 `matmul_bytes_multi` (and its `_serial` twin, 2182-2240): expert e's ONE
+ * activation row lhs[e] [k] against its own weight rhs[e] [n, k/blk] into outs[e] [n]. The reference
+ * shards (expert x column chunk) over its pool; each output is the same `dot` as `matmul_bytes` gives
+ * that row alone, so the schedule is not restated. */
+int oa_matmul_multi(int dtype, size_t k, size_t n, size_t ne, const uint8_t* const* rhs, const size_t* rhs_bytes,
+                    const float* const* lhs, const size_t* lhs_len, float* const* outs, const size_t* outs_len) {
+    if (ne == 0) return 0;
+    const row_dot_fn dot = oa_dot_of(dtype);
+    if (!dot) return -3;
+    const size_t blk = (size_t)lko_block_len(dtype);
+    if (k == 0 || k % blk != 0) return -1;
+    const size_t nb = k / blk, wrow = nb * (size_t)lko_block_bytes(dtype);
+    for (size_t e = 0; e < ne; ++e) {
+        if (lhs_len[e] != k) return -4;
+        if (outs_len[e] != n) return -5;
+        if (rhs_bytes[e] != n * wrow) return -2;
+    }
+    uint8_t* act = (uint8_t*)malloc(oa_act_row_bytes(dtype, k));
+    for (size_t e = 0; e < ne; ++e) {
+        oa_quantize_act(dtype, lhs[e], k, act);
+        for (size_t c = 0; c < n; ++c) outs[e][c] = dot(rhs[e] + c * wrow, act, nb);
+    }
+    free(act);
+    return 0;
+}
+
+/* drivers.rs:2318-2425 `matmul_bytes_grouped`: expert e's weight against its lhs_len[e] / k rows into
+ * outs[e] [rows, n]; every row quantized once, every output the same `dot` as one GEMV per
+ * (expert, row). */
+int oa_matmul_grouped(int dtype, size_t k, size_t n, size_t ne, const uint8_t* const* rhs, const size_t* rhs_bytes,
+                      const float* const* lhs, const size_t* lhs_len, float* const* outs, const size_t* outs_len) {
+    if (ne == 0) return 0;
+    const row_dot_fn dot = oa_dot_of(dtype);
+    if (!dot) return -3;
+    const size_t blk = (size_t)lko_block_len(dtype);
+    if (k == 0 || k % blk != 0) return -1;
+    const size_t nb = k / blk, wrow = nb * (size_t)lko_block_bytes(dtype), arow = oa_act_row_bytes(dtype, k);
+    for (size_t e = 0; e < ne; ++e) {
+        if (lhs_len[e] % k != 0) return -4;
+        if (outs_len[e] != lhs_len[e] / k * n) return -5;
+        if (rhs_bytes[e] != n * wrow) return -2;
+    }
+    for (size_t e = 0; e < ne; ++e) {
+        const size_t rows = lhs_len[e] / k;
+        uint8_t* act = (uint8_t*)malloc(arow * (rows ? rows : 1));
+        for (size_t r = 0; r < rows; ++r) oa_quantize_act(dtype, lhs[e] + r * k, k, act + r * arow);
+        for (size_t c = 0; c < n; ++c)   /* a weight column meets every row of its expert before the next is read */
+            for (size_t r = 0; r < rows; ++r) outs[e][r * n + c] = dot(rhs[e] + c * wrow, act + r * arow, nb);
+        free(act);
+    }
+    return 0;
+}
+
 int oa_matmul_exact(int dtype, size_t m, size_t k, size_t n, const float* lhs,
                     const uint8_t* rhs, float* dst) {
     row_dot_fn dot;

@@ -76,6 +76,16 @@ void lko_quantize_q8_k(const float* x, size_t n, uint8_t* out);   /* q8_k.rs:96-
  * -2 rhs byte length wrong, -3 dtype not handled. */
 int oa_matmul(int dtype, size_t m, size_t k, size_t n, const float* lhs,
               const uint8_t* rhs, size_t rhs_bytes, float* dst);
+/* matmul_bytes_multi (drivers.rs:2144-2316): expert e's one row lhs[e] [k] x rhs[e] [n, k/blk] ->
+ * outs[e] [n]; bit for bit one oa_matmul((1,k,n)) per expert. Further codes: -4 an lhs entry is not
+ * k floats, -5 an outs entry is not n floats. ne == 0 is a no-op. */
+int oa_matmul_multi(int dtype, size_t k, size_t n, size_t ne, const uint8_t* const* rhs, const size_t* rhs_bytes,
+                    const float* const* lhs, const size_t* lhs_len, float* const* outs, const size_t* outs_len);
+/* matmul_bytes_grouped (drivers.rs:2318-2425): expert e's lhs_len[e] / k rows x rhs[e] -> outs[e]
+ * [rows, n]; bit for bit one GEMV per (expert, row). -4: an lhs entry is not whole rows of k; -5: an
+ * outs entry is not rows x n. */
+int oa_matmul_grouped(int dtype, size_t k, size_t n, size_t ne, const uint8_t* const* rhs, const size_t* rhs_bytes,
+                      const float* const* lhs, const size_t* lhs_len, float* const* outs, const size_t* outs_len);
 /* The exact-fold variant, dot_exact (q4_k.rs:117-131, q6_k.rs:121-134): integer block sums,
  * `combine`, shares added in block order from -0.0. K-quants only. */
 int oa_matmul_exact(int dtype, size_t m, size_t k, size_t n, const float* lhs,
@@ -140,6 +150,14 @@ void lko_split_act_mul(const float* gu, float* out, size_t n, size_t rows, int a
 
 /* ---- timed CPU baseline (cpu_baseline.c): O-A semantics, AVX2 kernels, worker pool ---- */
 int lko_cpu_has_avx2(void);
+int lko_cpu_has_avx512(void);   /* f, bw, vl, dq and vnni */
+/* The vector dots of one Q4_K row (nb super-blocks) against Q8_K rows, for the tests: the 256-bit
+ * kernel (wide = 0; avx/superblock.rs:327-350) or its 512-bit VNNI twin (wide = 1;
+ * avx512/superblock.rs:20-90), and the several-rows-per-pass form (avx/superblock.rs:425-490), each of
+ * whose outputs carries the bits of the one-row kernel. Call only where lko_cpu_has_avx2 /
+ * lko_cpu_has_avx512 say so. */
+float lko_dot_q4k_q8k(int wide, const uint8_t* w, const uint8_t* y, size_t nb);
+void lko_dot_q4k_q8k_many(const uint8_t* w, const uint8_t* const* ys, size_t rows, size_t nb, float* out);
 /* The worker pool both drivers run on: persistent, one worker per physical core of the affinity
  * mask unless `threads` says otherwise (gemv_pool.rs:186-203). Returns the threads in use. */
 int lko_pool_start(int threads);

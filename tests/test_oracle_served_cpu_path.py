@@ -92,3 +92,35 @@ def test_argument_errors():
     x = synth.activation(1, 256, seed=9)
     with pytest.raises(oracle.OracleError):
         oracle.oa_matmul_q4k_x8(x, np.zeros(1152 * 2, np.uint8), 12)   # n not a multiple of 8
+
+
+def test_several_rows_per_pass_carry_the_one_row_kernels_bits():
+    """vec_dot_q4k_q8k_many (avx/superblock.rs:425-490): out[t] is bit for bit the one-row kernel's."""
+    k = 2048
+    w = synth.weight(Q4K, 3, k, seed=12)
+    x = synth.activation(7, k, seed=12)          # a pass of four, then a ragged one of three
+    for row in range(3):
+        many = oracle.dot_q4k_q8k_many(w[row], x)
+        for t in range(7):
+            one = np.float32(oracle.dot_q4k_q8k(w[row], x[t]))
+            assert many[t] == one
+    # and the one-row kernel is the scalar oracle's dot to the reference's vector-vs-scalar bound
+    ref = oracle.oa_matmul(Q4K, x, w, 3)
+    got = np.stack([oracle.dot_q4k_q8k_many(w[row], x) for row in range(3)], axis=1)
+    assert (np.abs(got - ref) <= 1e-3 * np.maximum(np.abs(ref), 1.0)).all()
+
+
+@pytest.mark.skipif(not oracle.lib().lko_cpu_has_avx512(), reason="needs AVX-512 with VNNI")
+def test_the_512_bit_twin_returns_the_256_bit_kernels_bits():
+    """avx512/superblock.rs:20-90: the same integer sums in wider registers, so the same float."""
+    k = 4096
+    w = synth.weight(Q4K, 16, k, seed=13)
+    x = synth.activation(3, k, seed=13) * np.float32(5.0)
+    for row in range(16):
+        for t in range(3):
+            assert oracle.dot_q4k_q8k(w[row], x[t], wide=True) == oracle.dot_q4k_q8k(w[row], x[t], wide=False)
+    # extreme codes: every nibble 15, every activation at the quantizer's extreme
+    w_hot = synth.weight(Q4K, 1, 512, seed=14)
+    w_hot.reshape(-1, 144)[:, 16:] = 0xFF
+    x_hot = np.full((1, 512), -3.0, np.float32)
+    assert oracle.dot_q4k_q8k(w_hot[0], x_hot[0], wide=True) == oracle.dot_q4k_q8k(w_hot[0], x_hot[0], wide=False)
