@@ -19,6 +19,7 @@
 
 #include "lk_common.h"
 
+#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 #include <unordered_map>
@@ -30,7 +31,8 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef u32x4 __attribute__((aligned(4))) u32x4_a4;
 
-constexpr int WG = 256, WAVES = 4;
+// Waves per workgroup: four, or eight for a matrix of so few 32-row tiles that every workgroup has a
+// CU to itself (the waves then split a row's super-blocks eight ways instead of four).
 constexpr int TOK = 32;   // activation rows per pass (the matrix instruction's M)
 
 struct Args {
@@ -138,7 +140,7 @@ static __device__ __forceinline__ void block_step(const WFrag& w, bool live, int
     quarter(I1{}, I0{}); quarter(I1{}, I1{}); quarter(I1{}, I2{}); quarter(I1{}, I3{});
 }
 
-template <int G, bool STAGED>
+template <int G, bool STAGED, int WAVES>
 static __host__ __device__ constexpr int lds_bytes_for(int nb) {
     // [codes [nb * 8][8 G][32] when staged,] d8 [nb * 8][8 G] floats, reduce [WAVES][4 G][64] floats
     return (STAGED ? nb * 8 * 8 * G * 32 : 0) + nb * 8 * 8 * G * 4 + WAVES * 4 * G * 64 * 4;
@@ -148,9 +150,9 @@ static __host__ __device__ constexpr int lds_bytes_for(int nb) {
 // them once and a wave keeps DEPTH steps of weight loads in flight. Otherwise the lane reads its
 // activation row's codes from memory with every step's weights (two steps in flight), 32 rows per
 // pass, grid y over the passes.
-template <int G, bool STAGED>
-__global__ __launch_bounds__(WG, 2) void q6k_rows_kernel(Args p) {
-    constexpr int TW = 8 * G, NV = 4 * G;
+template <int G, bool STAGED, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void q6k_rows_kernel(Args p) {
+    constexpr int TW = 8 * G, NV = 4 * G, WG = 64 * WAVES;
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t* codes = lds;                                                              // STAGED: [nb * 8][TW][32]
     float* d8_table = (float*)(lds + (STAGED ? (size_t)p.nb * 8 * TW * 32 : 0));       // [nb * 8][TW]
@@ -190,9 +192,13 @@ __global__ __launch_bounds__(WG, 2) void q6k_rows_kernel(Args p) {
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < G; ++r) {
+            if (wave >= 4) break;   // the first four waves write the NV registers' rows, G each
             const int v = wave * G + r;
-            const float sum = (reduce[v * 64 + lane] + reduce[(NV + v) * 64 + lane]) +
-                              (reduce[(2 * NV + v) * 64 + lane] + reduce[(3 * NV + v) * 64 + lane]);
+            float sum = (reduce[v * 64 + lane] + reduce[(NV + v) * 64 + lane]) +
+                        (reduce[(2 * NV + v) * 64 + lane] + reduce[(3 * NV + v) * 64 + lane]);
+            if (WAVES == 8)
+                sum += (reduce[(4 * NV + v) * 64 + lane] + reduce[(5 * NV + v) * 64 + lane]) +
+                       (reduce[(6 * NV + v) * 64 + lane] + reduce[(7 * NV + v) * 64 + lane]);
             const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = ((int)blockIdx.x + ordinal * (int)gridDim.x) * 32 + l32;
             if (tok < m_count && row < p.n) p.dst[(size_t)(m0 + tok) * p.ldd + row] = sum;
         }
@@ -316,7 +322,13 @@ __global__ __launch_bounds__(WG, 2) void q6k_rows_kernel(Args p) {
     }
 }
 
-template <int G, bool STAGED>
+// Measurement runs: an integer from the environment (0 when unset).
+static int tune_env(const char* name) {
+    const char* v = getenv(name);
+    return v ? atoi(v) : 0;
+}
+
+template <int G, bool STAGED, int WAVES>
 int resident_cap(int lds_bytes) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -327,11 +339,11 @@ int resident_cap(int lds_bytes) {
     if (lds_bytes > lk_device().lds_bytes) {
         r = 0;
     } else if (lds_bytes > 48 * 1024 &&
-               hipFuncSetAttribute((const void*)q6k_rows_kernel<G, STAGED>, hipFuncAttributeMaxDynamicSharedMemorySize,
+               hipFuncSetAttribute((const void*)q6k_rows_kernel<G, STAGED, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         r = 0;
-    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q6k_rows_kernel<G, STAGED>, WG,
+    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q6k_rows_kernel<G, STAGED, WAVES>, 64 * WAVES,
                                                             (size_t)lds_bytes) != hipSuccess || r < 1) {
         (void)hipGetLastError();
         r = 1;
@@ -341,17 +353,31 @@ int resident_cap(int lds_bytes) {
 }
 
 // -1: the kernel's LDS image does not fit (the caller tries the next form).
-template <int G, bool STAGED>
-int launch(const Args& a, hipStream_t stream) {
-    const int lds_bytes = lds_bytes_for<G, STAGED>(a.nb);
-    const int per_cu = resident_cap<G, STAGED>(lds_bytes);
+template <int G, bool STAGED, int WAVES>
+int launch_waves(const Args& a, hipStream_t stream) {
+    const int lds_bytes = lds_bytes_for<G, STAGED, WAVES>(a.nb);
+    const int per_cu = resident_cap<G, STAGED, WAVES>(lds_bytes);
     if (per_cu == 0) return -1;
     const int n_tiles = (a.n + 31) / 32, groups = STAGED ? 1 : (a.m + TOK - 1) / TOK;
     if (groups > 65535) return LK_ERR_ARG;
     int cap = lk_device().cus * per_cu / groups;
     if (cap < 1) cap = 1;
-    hipLaunchKernelGGL((q6k_rows_kernel<G, STAGED>), dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
+    hipLaunchKernelGGL((q6k_rows_kernel<G, STAGED, WAVES>), dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(64 * WAVES), lds_bytes, stream, a);
     return lk_launch_status();
+}
+
+template <int G, bool STAGED>
+int launch(const Args& a, hipStream_t stream) {
+    // eight waves when the tiles (times the passes of 32 rows) do not fill the CUs and a wave would
+    // otherwise walk eight super-blocks or more in turn
+    const int n_tiles = (a.n + 31) / 32, groups = STAGED ? 1 : (a.m + TOK - 1) / TOK;
+    static const int forced = tune_env("LK_TUNE_ROWS_WAVES");
+    const bool eight = forced ? forced == 8 : (n_tiles * groups <= lk_device().cus && a.nb >= 32);
+    if (eight) {
+        const int rc = launch_waves<G, STAGED, 8>(a, stream);
+        if (rc >= 0) return rc;
+    }
+    return launch_waves<G, STAGED, 4>(a, stream);
 }
 
 }  // namespace
