@@ -82,8 +82,9 @@ def parse_args():
     ap.add_argument("--cols-k", type=int, default=4096, help="--workload gemv: values per row")
     ap.add_argument("--tokens", type=int, default=256, help="--workload moe: rows through the expert block")
     ap.add_argument("--moe-wtype", default="q4_k", help="--workload moe: the experts' format (as --wtype)")
-    ap.add_argument("--moe-path", choices=["auto", "tiled", "pairs"], default="auto",
-                    help="--workload moe: expert-batched tiled matmul, mat-vec per routed pair, or the library's choice")
+    ap.add_argument("--moe-path", choices=["auto", "tiled", "rows", "pairs"], default="auto",
+                    help="--workload moe: expert-batched tiled matmul, expert-batched rows on the matrix unit, mat-vec per "
+                         "routed pair, or the library's choice")
     ap.add_argument("--mid-rows", choices=["auto", "matvec", "tiled"], default="auto",
                     help="--workload decode-1p7b above 8 rows: auto = the host mirror's choice between the matrix-unit "
                          "rows kernels and the tiled matmul; matvec = mat-vec launches over slices of eight rows up to "

@@ -437,6 +437,20 @@ void loken_dense_q5k_imma_m8_actmul(const void* gate, const void* up, const void
                                     int size_m, int size_n, int size_k, int use_gelu, void* stream);
 int lk_dense_q5k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
                              int size_n, int size_k, int use_gelu, void* stream);
+/* Expert-batched Q4_K rows on the matrix unit, for routings that give an expert a handful of rows:
+ * expert e's matrix (weights + e * expert_bytes, size_n rows of size_k) against the sorted rows
+ * [bounds[e], bounds[e + 1]) of the routing, 8, 16 or 32 of them per pass over the weights (rows_hint,
+ * the run length expected per expert, picks the width; any count is served). Sorted row i reads the
+ * plain Q8_1 row src_rows[i] (or i) of q8_1 (stride_blocks blocks apart) and writes row dst_rows[i]
+ * (or i) of output (ldd floats apart). With weights_second (same layout) the result is
+ * act(w . x) * (w2 . x), act 0 SiLU / 1 tanh-form GELU, else w . x. The reference reaches these
+ * loads through launch_mmq_moe_gguf_q4_k (src/tensor/quantized/mmq.rs:274-286; MmqRouting,
+ * src/inference/moe_cuda/mmq_experts.rs:300-557) or one mat-vec per routed pair; it has no launcher of
+ * this shape. The host mirror of MmqRouting uses it while an expert's run stays short. */
+int lk_moe_q4k_rows_grouped(const void* weights, const void* weights_second, int act, const void* q8_1,
+                            int stride_blocks, const int32_t* bounds, const int32_t* src_rows,
+                            const int32_t* dst_rows, float* output, int ldd, int n_experts,
+                            int64_t expert_bytes, int size_n, int size_k, int rows_hint, void* stream);
 /* Q6_K weight [size_n rows, size_k] x plain Q8_1 rows [size_m, size_k / 32 blocks] -> output
  * [size_m, size_n] f32 on the int8 matrix unit: the Q6_K member of the family above. The reference
  * has no launcher of this shape (its Q6_K rows go one at a time through vec_dot_q6_K_q8_1,

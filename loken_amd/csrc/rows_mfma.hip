@@ -99,11 +99,39 @@ static __device__ __forceinline__ v4i codes_of(const uint4& q, const uint4& qh, 
 template <int G>
 static __host__ __device__ constexpr int lds_floats_table(int nb) { return nb * 8 * 8 * G * (G < 4 ? 2 : 1); }
 
-template <int G, bool DUAL, bool Q5>
-__global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
+// Where the activation rows of a pass live and where their results go. Dense: consecutive rows.
+// Expert-batched: row i of the pass is sorted row first + i of the routing; its activation is row
+// src[first + i] of the Q8_1 rows (the token), its result goes to row dst_map[first + i] (or
+// first + i) of the output.
+struct PassRows {
+    const uint8_t* y;        // Q8_1 rows
+    float* dst;
+    const int32_t* src;      // nullable: activation row of a sorted row
+    const int32_t* dst_map;  // nullable: output row of a sorted row
+    int first;               // first row of the pass
+    int stride_y, ldd;
+    __device__ __forceinline__ const uint8_t* y_row(int i) const {
+        const int r = src ? src[first + i] : first + i;
+        return y + (size_t)r * stride_y * Q81_BYTES;
+    }
+    __device__ __forceinline__ float* out_row(int i) const {
+        const int r = dst_map ? dst_map[first + i] : first + i;
+        return dst + (size_t)r * ldd;
+    }
+};
+
+// One pass: every row tile of this workgroup's share of matrix `p.w` (and `p.w2`) against the
+// `m_count` activation rows of `rows` (at most 8 G). Every wave of the workgroup must call it, and
+// all leave it past the same barriers, so passes can follow one another.
+// KSPLIT: the four waves of the workgroup share each row tile and split its super-blocks (long rows:
+// every wave has blocks to stream, and the partial tiles meet in LDS). Without it a wave owns whole
+// row tiles, all of a row's super-blocks in turn, and nothing crosses waves but the tables: rows of
+// at most eight super-blocks, where a four-way split leaves a wave one or two blocks per tile and
+// most of its time in the reduction's barriers.
+template <int G, bool DUAL, bool Q5, bool KSPLIT = true>
+static __device__ __forceinline__ void q4k_rows_pass(const Args& p, const PassRows& rows, int m_count, uint8_t* lds) {
     constexpr int TW = 8 * G;   // activation rows a table row holds
     constexpr int NV = 4 * G;   // live accumulator registers
-    extern __shared__ __align__(16) uint8_t lds[];
     float* d8_table = (float*)lds;                                   // [nb * 8][TW]
     float* ds_table = d8_table + p.nb * 8 * TW;                      // [nb * 8][TW], G < 4 only
     float* reduce = d8_table + lds_floats_table<G>(p.nb);            // [WAVES][NV][64]
@@ -111,14 +139,11 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
-    const int m0 = blockIdx.y * TOK;
-    const int m_count = min(TOK, p.m - m0);
     const int n_tiles = (p.n + 31) >> 5;
     const size_t row_bytes = (size_t)p.nb * Blk<Q5>::BYTES;
 
     // Activation scales of this pass, zero for the rows the pass does not have. Eight loads are
     // issued before the first is used: one at a time, each would cost a memory latency.
-    const uint8_t* y0 = p.y + (size_t)m0 * p.stride_y * Q81_BYTES;
     const int entries = p.nb * 8 * TW;
     if constexpr (G == 4) {
         for (int base = threadIdx.x; base < entries; base += WG * 8) {
@@ -127,7 +152,7 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
             for (int u = 0; u < 8; ++u) {
                 const int idx = min(base + u * WG, entries - 1);
                 const int sub = idx >> 5, tok = min(idx & 31, m_count - 1);
-                bits[u] = *(const uint16_t*)(y0 + ((size_t)tok * p.stride_y + sub) * Q81_BYTES);
+                bits[u] = *(const uint16_t*)(rows.y_row(tok) + (size_t)sub * Q81_BYTES);
             }
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
@@ -144,7 +169,7 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
             for (int u = 0; u < 4; ++u) {
                 const int idx = min(base + u * WG, entries - 1);
                 const int sub = idx / TW, tok = min(idx % TW, m_count - 1);
-                const uint8_t* b = y0 + ((size_t)tok * p.stride_y + sub) * Q81_BYTES;
+                const uint8_t* b = rows.y_row(tok) + (size_t)sub * Q81_BYTES;
                 head[u] = *(const uint32_t*)b;
                 lo[u] = *(const uint4_a4*)(b + 4);
                 hi[u] = *(const uint4_a4*)(b + 20);
@@ -164,7 +189,7 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     }
 
     // The lane's activation row (a row past the end re-reads the last one; its scales are zero).
-    const uint8_t* y_lane = y0 + (size_t)min(l32, m_count - 1) * p.stride_y * Q81_BYTES + 4 + 16 * lh;
+    const uint8_t* y_lane = rows.y_row(min(l32, m_count - 1)) + 4 + 16 * lh;
 
     auto load = [&](Frag& f, int tile, int kb) {
         const int row = min((DUAL ? tile >> 1 : tile) * 32 + l32, p.n - 1);
@@ -247,10 +272,55 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
         }
     };
 
+    const int n_vt = DUAL ? 2 * n_tiles : n_tiles;
+    if constexpr (!KSPLIT) {
+        // a wave's own tiles: unit = workgroup * 4 + wave, then every (workgroups * 4)-th
+        const int units = (int)gridDim.x * WAVES;
+        int tile = first_tile<DUAL>((int)blockIdx.x * WAVES + wave), kb = 0;
+        Frag fa, fb;
+        if (tile < n_vt) load(fa, tile, 0);
+        __syncthreads();   // the scale table is complete
+        float gate_keep[NV];
+        auto finish_own = [&](int t) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                float sum = acc[v] + acc_min[v];
+                acc[v] = acc_min[v] = 0.f;
+                if (DUAL && !(t & 1)) { gate_keep[v] = sum; continue; }
+                if (DUAL) {
+                    LkGateAct act;
+                    act.kind = p.gelu ? LK_GATE_GELU : LK_GATE_SILU;
+                    sum = lk_gated(act, gate_keep[v], sum, 0);
+                }
+                const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = (DUAL ? t >> 1 : t) * 32 + l32;
+                if (tok < m_count && row < p.n) rows.out_row(tok)[row] = sum;
+            }
+        };
+        while (tile < n_vt) {
+            int nt = tile, nk = kb + 1;
+            const bool last = nk >= p.nb;
+            if (last) { nk = 0; nt = next_tile<DUAL>(nt, units); }
+            if (nt < n_vt) load(fb, nt, nk);
+            compute(fa, kb);
+            if (last) finish_own(tile);
+            tile = nt; kb = nk;
+            if (tile >= n_vt) break;
+            nt = tile; nk = kb + 1;
+            const bool last2 = nk >= p.nb;
+            if (last2) { nk = 0; nt = next_tile<DUAL>(nt, units); }
+            if (nt < n_vt) load(fa, nt, nk);
+            compute(fb, kb);
+            if (last2) finish_own(tile);
+            tile = nt; kb = nk;
+        }
+        __syncthreads();   // every wave is done with the tables: the next pass may rebuild them
+        return;
+    }
+
     // Steps are (row tile, super-block) pairs: wave w takes super-blocks w, w + 4, ... of every
     // tile of this workgroup; the loads of the next step fly under the arithmetic of this one.
     const int my_blocks = (p.nb - wave + WAVES - 1) / WAVES;   // may be zero for short rows
-    const int wgs = (int)gridDim.x, n_vt = DUAL ? 2 * n_tiles : n_tiles;
+    const int wgs = (int)gridDim.x;
     int tile = first_tile<DUAL>(blockIdx.x), kb = wave;
     Frag fa, fb;
     if (tile < n_vt && my_blocks > 0) load(fa, tile, kb);
@@ -278,9 +348,9 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
                 sum = lk_gated(act, gate_keep[r], sum, 0);
             }
             const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = (DUAL ? t >> 1 : t) * 32 + l32;
-            if (tok < m_count && row < p.n) p.dst[(size_t)(m0 + tok) * p.ldd + row] = sum;
+            if (tok < m_count && row < p.n) rows.out_row(tok)[row] = sum;
         }
-        __syncthreads();   // the partial tiles may be overwritten
+        __syncthreads();   // the partial tiles may be overwritten (and, past the last tile, the tables)
     };
 
     while (tile < n_vt) {
@@ -306,6 +376,38 @@ __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
             finish_tile(tile);   // nothing of its own to add, but the barriers are the workgroup's
             tile = next_tile<DUAL>(tile, wgs);
         }
+    }
+}
+
+// Dense: grid y walks the activation in passes of 32 rows.
+template <int G, bool DUAL, bool Q5>
+__global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int m0 = blockIdx.y * TOK;
+    const PassRows rows{p.y, p.dst, nullptr, nullptr, m0, p.stride_y, p.ldd};
+    q4k_rows_pass<G, DUAL, Q5>(p, rows, min(TOK, p.m - m0), lds);
+}
+
+// Expert-batched: grid y is the expert; its sorted rows [bounds[e], bounds[e + 1]) go through in
+// passes of 8 G, each a walk over the expert's row tiles (the tables in LDS are rebuilt per pass).
+struct MoeRows {
+    const int32_t* bounds;    // [experts + 1]
+    const int32_t* src;       // sorted row -> activation row; nullable (the sorted row itself)
+    const int32_t* dst_map;   // sorted row -> output row; nullable
+    int64_t expert_bytes;     // between consecutive experts' matrices (both stacks)
+};
+
+template <int G, bool DUAL, bool Q5, bool KSPLIT>
+__global__ __launch_bounds__(WG, 2) void q4k_rows_moe_kernel(Args p, MoeRows m) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int e = blockIdx.y;
+    const int begin = m.bounds[e], end = m.bounds[e + 1];
+    if (end <= begin) return;
+    p.w += (int64_t)e * m.expert_bytes;
+    if (DUAL) p.w2 += (int64_t)e * m.expert_bytes;
+    for (int first = begin; first < end; first += 8 * G) {
+        const PassRows rows{p.y, p.dst, m.src, m.dst_map, first, p.stride_y, p.ldd};
+        q4k_rows_pass<G, DUAL, Q5, KSPLIT>(p, rows, min(8 * G, end - first), lds);
     }
 }
 
@@ -567,6 +669,59 @@ int launch_staged(const Args& a, hipStream_t stream) {
     return lk_launch_status();
 }
 
+// The expert-batched launch: grid (workgroups per expert, experts). A workgroup walks several row
+// tiles per pass so that the tables of an expert's rows are staged by a few workgroups, not by one
+// per tile.
+template <int G, bool DUAL, bool Q5, bool KSPLIT>
+int launch_moe(const Args& a, const MoeRows& m, int n_experts, hipStream_t stream) {
+    static std::mutex mu;
+    static std::unordered_map<int, int> by_lds;
+    const int lds_bytes = (lds_floats_table<G>(a.nb) + WAVES * 4 * G * 64) * (int)sizeof(float);
+    if (lds_bytes > lk_device().lds_bytes) return LK_ERR_ARG;
+    int per_cu;
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = by_lds.find(lds_bytes);
+        if (it == by_lds.end()) {
+            int r = 0;
+            if (lds_bytes > 48 * 1024 &&
+                hipFuncSetAttribute((const void*)q4k_rows_moe_kernel<G, DUAL, Q5, KSPLIT>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    lds_bytes) != hipSuccess) {
+                (void)hipGetLastError();
+                r = 0;
+            } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_moe_kernel<G, DUAL, Q5, KSPLIT>, WG,
+                                                                    (size_t)lds_bytes) != hipSuccess || r < 1) {
+                (void)hipGetLastError();
+                r = 1;
+            }
+            it = by_lds.emplace(lds_bytes, r).first;
+        }
+        per_cu = it->second;
+    }
+    if (per_cu == 0) return LK_ERR_ARG;
+    const int n_tiles = (a.n + 31) / 32, units = KSPLIT ? n_tiles : (n_tiles + WAVES - 1) / WAVES;
+    int per_expert = (2 * lk_device().cus * per_cu + n_experts - 1) / n_experts;
+    if (per_expert < 2) per_expert = 2;
+    if (per_expert > units) per_expert = units;
+    hipLaunchKernelGGL((q4k_rows_moe_kernel<G, DUAL, Q5, KSPLIT>), dim3(per_expert, n_experts), dim3(WG), lds_bytes, stream, a, m);
+    return lk_launch_status();
+}
+
+template <bool DUAL, bool KSPLIT>
+int launch_moe_width(const Args& a, const MoeRows& m, int n_experts, int rows_hint, hipStream_t stream) {
+    if (rows_hint <= 8) return launch_moe<1, DUAL, false, KSPLIT>(a, m, n_experts, stream);
+    if (rows_hint <= 16) return launch_moe<2, DUAL, false, KSPLIT>(a, m, n_experts, stream);
+    return launch_moe<4, DUAL, false, KSPLIT>(a, m, n_experts, stream);
+}
+
+template <bool DUAL>
+int launch_moe_any(const Args& a, const MoeRows& m, int n_experts, int rows_hint, hipStream_t stream) {
+    // rows of at most eight super-blocks (the expert matrices of the MoE models: k = 2048, 768): a wave per
+    // row tile; longer rows: the four waves split a tile's super-blocks
+    return a.nb <= 8 ? launch_moe_width<DUAL, false>(a, m, n_experts, rows_hint, stream)
+                     : launch_moe_width<DUAL, true>(a, m, n_experts, rows_hint, stream);
+}
+
 template <bool DUAL, bool Q5>
 int launch_any(const Args& a, hipStream_t stream) {
     // at most 8 / 16 activation rows in all: the fix-up runs on the registers those rows live in,
@@ -657,4 +812,33 @@ extern "C" int lk_dense_q5k_rows_actmul(const void* gate, const void* up, const 
 extern "C" void loken_dense_q5k_imma_m8_actmul(const void* gate, const void* up, const void* q8_1, float* output,
                                                int size_m, int size_n, int size_k, int use_gelu, void* stream) {
     (void)rows_actmul(gate, up, q8_1, output, size_m, size_n, size_k, use_gelu, true, (hipStream_t)stream);
+}
+
+// Expert-batched Q4_K rows on the matrix unit, for routings that give an expert a handful of rows: the
+// shape of lk_dense_q4k_rows per expert, every expert's weights read once per 8 / 16 / 32 of its rows.
+// The reference reaches these loads through its tiled expert kernel (launch_mmq_moe_gguf_q4_k,
+// src/tensor/quantized/mmq.rs:274-286) or one mat-vec per pair; it has no launcher of this shape.
+//   weights        [n_experts] matrices of size_n rows, expert_bytes apart
+//   weights_second nullable; when given (same layout) the output is act(w . x) * (w2 . x), act 0 SiLU / 1 GELU
+//   q8_1           plain Q8_1 rows, stride_blocks blocks apart
+//   bounds         [n_experts + 1]: expert e owns sorted rows [bounds[e], bounds[e + 1])
+//   src_rows       nullable: sorted row -> row of q8_1 (else the sorted row itself)
+//   dst_rows       nullable: sorted row -> row of output (else the sorted row itself)
+//   rows_hint      rows an expert is expected to own (picks the pass width; any count is served)
+extern "C" int lk_moe_q4k_rows_grouped(const void* weights, const void* weights_second, int act, const void* q8_1,
+                                       int stride_blocks, const int32_t* bounds, const int32_t* src_rows,
+                                       const int32_t* dst_rows, float* output, int ldd, int n_experts,
+                                       int64_t expert_bytes, int size_n, int size_k, int rows_hint, void* stream) {
+    if (n_experts == 0 || size_n == 0) return LK_OK;
+    if (!weights || !q8_1 || !bounds || !output || n_experts < 0 || n_experts > 65535 || size_n < 0 || size_k <= 0 ||
+        size_k % 256 != 0 || stride_blocks < size_k / 32 || ldd < size_n || expert_bytes % 16 != 0)
+        return LK_ERR_ARG;
+    if ((((uintptr_t)weights) & 15) != 0 || (((uintptr_t)weights_second) & 15) != 0 || (((uintptr_t)q8_1) & 3) != 0)
+        return LK_ERR_ARG;
+    Args a{(const uint8_t*)weights, (const uint8_t*)q8_1, output, size_k / 256, size_n, 0, stride_blocks, ldd,
+           (const uint8_t*)weights_second, act ? 1 : 0};
+    const MoeRows m{bounds, src_rows, dst_rows, expert_bytes};
+    if (rows_hint < 1) rows_hint = 1;
+    return weights_second ? launch_moe_any<true>(a, m, n_experts, rows_hint, (hipStream_t)stream)
+                          : launch_moe_any<false>(a, m, n_experts, rows_hint, (hipStream_t)stream);
 }

@@ -119,6 +119,7 @@ SIGNATURES.update({
     "lk_dense_q5k_rows_actmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "q4k_mmvq_imma": (None, [_vp, _vp, _vp, _i, _i, _vp]),
     "lk_dense_q6k_rows": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "lk_moe_q4k_rows_grouped": (_i, [_vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, C.c_int64, _i, _i, _i, _vp]),
     "loken_moe_q4k_imma_m8_gate_up": (None, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "lk_moe_q4k_rows_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "loken_moe_q4k_imma_m8_down": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

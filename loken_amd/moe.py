@@ -35,6 +35,7 @@ class MmqRouting:
         self.src_rows = torch.zeros(rows, dtype=torch.int32, device=device)
         self.choices = None
         self.mmq_x = 0
+        self.path = "auto"   # "tiled" / "rows" pin the launch family (measurement and tests)
 
     @classmethod
     def new(cls, slots: torch.Tensor, experts: torch.Tensor, topk: int, n_experts: int) -> "MmqRouting":
@@ -63,6 +64,12 @@ class MmqRouting:
 
     def with_tile_width(self, mmq_x: int) -> "MmqRouting":
         self.mmq_x = mmq_x
+        return self
+
+    def with_path(self, path: str) -> "MmqRouting":
+        if path not in ("auto", "tiled", "rows"):
+            raise ValueError(f"moe mmq: unknown path {path!r}")
+        self.path = path
         return self
 
     @property
@@ -94,12 +101,39 @@ class MmqRouting:
         if launched == 0:
             raise _lib.LokenError(MMQ_MOE_LAUNCHER[wtype], _lib.LK_ERR_ARG)
 
+    # Rows an expert is expected to own up to which the matrix-unit rows launch (weights straight from
+    # HBM into the operand, one pass per 8 / 16 / 32 rows) beats the tiled one (weights expanded into
+    # LDS per 32 tokens). Measured on MI355X at 128 experts of 2048 -> 768 -> 2048, top-8: 64 tokens
+    # 136 us against 167, 128 tokens 168 against 170, 256 tokens 193 against 182 (the expected longest
+    # run is 17 at 128 tokens).
+    ROWS_LAUNCH_MAX_RUN = 17
+
+    def takes_rows_launch(self, wtype: int, k: int) -> bool:
+        return (self.path != "tiled" and wtype == _lib.TYPE_Q4_K and k % 256 == 0
+                and (self.path == "rows" or self.longest_run_expected() <= self.ROWS_LAUNCH_MAX_RUN))
+
+    def _rows_launch(self, weights: torch.Tensor, second: torch.Tensor | None, q: torch.Tensor, src, dst_map,
+                     out: torch.Tensor, n: int, k: int):
+        expert_bytes = n * (k // 256) * 144
+        _lib.check("lk_moe_q4k_rows_grouped", _lib.load().lk_moe_q4k_rows_grouped(
+            weights.data_ptr(), second.data_ptr() if second is not None else None, 0, q.data_ptr(), q.shape[1],
+            self.bounds.data_ptr(), src.data_ptr() if src is not None else None,
+            dst_map.data_ptr() if dst_map is not None else None, out.data_ptr(), out.shape[1], self.experts,
+            expert_bytes, n, k, self.longest_run_expected(), _stream()))
+
     def gate_up_silu(self, wtype: int, xs: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, width: int) -> torch.Tensor:
         """``silu(gate . x) * (up . x)`` for every routed row, in sorted order: ``[rows, width]``
         (mmq_experts.rs:300-435). ``gate`` / ``up`` are stacks of ``[experts, width, k]`` blocks."""
         tokens, k = xs.shape
         if tokens != self.tokens:
             raise ValueError(f"moe mmq: {tokens} tokens against a plan of {self.tokens}")
+        if self.takes_rows_launch(wtype, k):
+            # one Q8_1 row per token; a sorted row reads its token's; gate, up and the activation in one launch
+            from . import ops
+            q = ops.quantize_q8_1_rows(xs.to(torch.float32).contiguous(), k_padded=k)
+            out = torch.empty((self.rows, width), dtype=torch.float32, device=xs.device)
+            self._rows_launch(gate, up, q, self.src_rows, None, out, width, k)
+            return out
         y = mmq_quantize(wtype, xs.to(torch.float32).contiguous(), gather=self.src_rows)
         gu = torch.empty((self.rows, 2 * width), dtype=torch.float32, device=xs.device)
         self._matmul(wtype, gate, up, width, width, k, y, gu, 2 * width, None)
@@ -114,9 +148,14 @@ class MmqRouting:
         rows, k = hs.shape
         if rows != self.rows:
             raise ValueError(f"moe mmq: {rows} rows against a plan of {self.rows}")
-        y = mmq_quantize(wtype, hs.contiguous())
         pairs = torch.empty((rows, hidden), dtype=torch.float32, device=hs.device)
-        self._matmul(wtype, down, None, 0, hidden, k, y, pairs, hidden, self.slots)
+        if self.takes_rows_launch(wtype, k):
+            from . import ops
+            q = ops.quantize_q8_1_rows(hs.contiguous(), k_padded=k)
+            self._rows_launch(down, None, q, None, self.slots, pairs, hidden, k)
+        else:
+            y = mmq_quantize(wtype, hs.contiguous())
+            self._matmul(wtype, down, None, 0, hidden, k, y, pairs, hidden, self.slots)
         out = (residual.reshape(self.tokens, hidden).to(torch.float32).clone() if residual is not None
                else torch.zeros((self.tokens, hidden), dtype=torch.float32, device=hs.device))
         w = topk_weights.to(torch.float32).contiguous()
@@ -366,11 +405,15 @@ def stable_sort_u32(keys: torch.Tensor, small: bool = False):
     return out, order
 
 
-def moe_mmq_pays(rows: int, experts: int) -> bool:
-    """Routed rows from which the expert-batched matmul beats the per-pair kernels. The reference
+def moe_mmq_pays(rows: int, experts: int, wtype: int | None = None) -> bool:
+    """Routed rows from which the expert-batched launches beat the per-pair kernels. The reference
     breaks even at one routed row per expert (mmq_experts.rs:72-86); on MI355X, with this
-    library's kernels, the mat-vec per routed pair stays ahead up to three rows per expert
-    (Qwen3-30B-A3B shapes: 117 us against 162 us at 32 tokens, 176 against 168 at 48)."""
+    library's kernels, the mat-vec per routed pair stays ahead of the tiled matmul up to three rows
+    per expert (Qwen3-30B-A3B shapes: 117 us against 162 us at 32 tokens, 176 against 168 at 48), and
+    of the matrix-unit rows launch that Q4_K stacks take at short runs up to 2.25 (32 tokens: 114 us
+    against 120; 48: 174 against 133; 96: 321 against 141)."""
+    if wtype == _lib.TYPE_Q4_K:
+        return 4 * rows >= 9 * max(experts, 1)
     return rows >= 3 * max(experts, 1)
 
 
@@ -382,7 +425,8 @@ def moe_forward(wtype_gu: int, wtype_down: int, x: torch.Tensor, gate: torch.Ten
     matmuls when there is at least a routed row per expert, else one mat-vec per routed pair."""
     tokens, hidden = x.shape
     topk = choices.shape[1]
-    if moe_mmq_pays(tokens * topk, n_experts) and moe_mmq_serves(wtype_gu, hidden) and moe_mmq_serves(wtype_down, ffn):
+    if (moe_mmq_pays(tokens * topk, n_experts, wtype_gu if wtype_gu == wtype_down else None)
+            and moe_mmq_serves(wtype_gu, hidden) and moe_mmq_serves(wtype_down, ffn)):
         plan = MmqRouting.from_choices(choices, n_experts)
         h = plan.gate_up_silu(wtype_gu, x, gate, up, ffn)
         return plan.down_fold(wtype_down, h, down, hidden, topk_weights.reshape(-1))

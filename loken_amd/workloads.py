@@ -337,13 +337,15 @@ def moe_block(args, dev):
     choices = choices.to(torch.int32).contiguous()
 
     pairs = tokens * topk
-    tiled = moe.moe_mmq_pays(pairs, experts) if args.moe_path == "auto" else args.moe_path == "tiled"
+    tiled = moe.moe_mmq_pays(pairs, experts, wt) if args.moe_path == "auto" else args.moe_path in ("tiled", "rows")
     tiled = tiled and moe.moe_mmq_serves(wt, hidden) and moe.moe_mmq_serves(wt, ffn)
     # The routing (the router's side of the boundary) is built once; the timed block is what the
     # expert launchers do with it, recorded into a graph so that the host's cost stays outside.
     flat_w = weights.reshape(-1)
+    rows_launch = False
     if tiled:
-        plan = moe.MmqRouting.from_choices(choices, experts)
+        plan = moe.MmqRouting.from_choices(choices, experts).with_path(args.moe_path if args.moe_path in ("tiled", "rows") else "auto")
+        rows_launch = plan.takes_rows_launch(wt, hidden)
 
         def block():
             h = plan.gate_up_silu(wt, x, gate, up, ffn)
@@ -365,8 +367,10 @@ def moe_block(args, dev):
         op_count = 6.0 * pairs * ffn * hidden
         value, unit = op_count / med / 1e6, "TOP/s"
         roofline = {"bound": "mfma", "achieved": round(value, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                    "frac": round(value / INT8_PEAK_TOPS, 4), "traffic": None, "kernel": f"mmq_moe_kernel, {name}",
-                    "note": "whole expert block (plan, route, quantize, two grouped matmuls, activation, fold)"}
+                    "frac": round(value / INT8_PEAK_TOPS, 4), "traffic": None,
+                    "kernel": f"q4k_rows_moe_kernel, {name}" if rows_launch else f"mmq_moe_kernel, {name}",
+                    "note": "whole expert block (quantize, two grouped matmuls with the activation in the first, fold)"
+                            if rows_launch else "whole expert block (plan, route, quantize, two grouped matmuls, activation, fold)"}
     else:
         nbytes = 3 * one_matrix * distinct
         value, unit = nbytes / med / 1e3, "GB/s"
@@ -374,7 +378,7 @@ def moe_block(args, dev):
                     "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None, "kernel": f"moe_rows_kernel / moe_rows_legacy_kernel, {name}",
                     "note": "whole expert block (quantize, gate/up pairs, down pairs, weighted sum); bytes = 3 matrices "
                             "per distinct expert hit"}
-    extra = {"block_graph_replay": spread(us), "block_eager_from_python": spread(eager), "path": "expert-batched tiled matmul" if tiled else "mat-vec per routed pair",
+    extra = {"block_graph_replay": spread(us), "block_eager_from_python": spread(eager), "path": ("expert-batched rows on the matrix unit" if rows_launch else "expert-batched tiled matmul") if tiled else "mat-vec per routed pair",
              "routed_pairs": pairs, "distinct_experts": distinct,
              "expert_load_histogram": {"max": int(load.max()), "mean": round(float(load.mean()), 2),
                                        "rows_per_expert_sorted_top8": sorted(load.tolist(), reverse=True)[:8]}}

@@ -12,7 +12,7 @@ import pytest
 torch = pytest.importorskip("torch")
 
 import oracle
-from loken_amd import lib, moe, synth
+from loken_amd import lib, moe, ops, synth
 from loken_amd.moe import MmqRouting
 
 pytestmark = pytest.mark.gpu
@@ -66,10 +66,14 @@ def test_route_with_experts_nobody_chose_and_one_token():
 @pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(5, 512, 256, 6, 2), (40, 1024, 512, 8, 3),
                                                              (1, 256, 256, 4, 2), (70, 512, 768, 16, 4)])
 @pytest.mark.parametrize("dt_down", [lib.TYPE_Q4_K, lib.TYPE_Q5_K, lib.TYPE_Q6_K])
-def test_expert_batched_block_matches_oracle(tokens, hidden, ffn, n_experts, topk, dt_down):
+@pytest.mark.parametrize("path", ["tiled", "rows"])
+def test_expert_batched_block_matches_oracle(tokens, hidden, ffn, n_experts, topk, dt_down, path):
+    """Both launch families of the expert-batched block: the tiled matmul, and (Q4_K stacks) the
+    matrix-unit rows launch that serves short runs per expert."""
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=51, dt_down=dt_down)
     want, want_h = oracle.moe_forward(1, lib.TYPE_Q4_K, dt_down, x, gate, up, down, ids, w, n_experts, ffn, want_h=True)
-    plan = MmqRouting.from_choices(dev(ids), n_experts)
+    plan = MmqRouting.from_choices(dev(ids), n_experts).with_path(path)
+    assert plan.takes_rows_launch(lib.TYPE_Q4_K, hidden) == (path == "rows")
     h = plan.gate_up_silu(lib.TYPE_Q4_K, dev(x), dev(gate), dev(up), ffn)
     # GLU rows in sorted order; expf differs from libm's in the last place, and silu(g)*u inherits
     # the relative error of g and u where they nearly cancel: compare against the scale of a row
@@ -515,3 +519,46 @@ def test_q4k_pair_rows_over_caller_quantized_rows_with_one_expert_per_pair(token
         want[slot // topk] += (y * flat_w[slot]).astype(np.float64)
     got = moe_q4k_imma_m8_down_reduce(h, dev(down), sd, ed, dev(flat_w), n_experts, topk, hidden).cpu().numpy()
     assert (np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-4 * np.abs(want).max()).all()
+
+
+@pytest.mark.parametrize("hint", [1, 9, 40])
+@pytest.mark.parametrize("k", [512, 2560])   # a wave per row tile (at most 8 super-blocks), or four waves splitting a tile's
+def test_rows_launch_serves_any_run_length_whatever_the_hint(hint, k):
+    """lk_moe_q4k_rows_grouped: the hint only picks the pass width (8, 16 or 32 rows); an expert with
+    more rows takes more passes, one without rows none, and gather / scatter follow the routing."""
+    rng = np.random.default_rng(67)
+    n_experts, n, tokens = 5, 96, 30
+    counts = [37, 0, 1, 9, 13]                              # sorted rows per expert
+    rows = sum(counts)
+    bounds = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    src = rng.integers(0, tokens, rows).astype(np.int32)    # sorted row -> token
+    dst_map = rng.permutation(rows).astype(np.int32)        # sorted row -> output row
+    w = synth.weight(lib.TYPE_Q4_K, n_experts * n, k, seed=67, stream=1)
+    w2 = synth.weight(lib.TYPE_Q4_K, n_experts * n, k, seed=67, stream=2)
+    x = synth.activation(tokens, k, seed=67) * np.float32(4.0)
+    q = ops.quantize_q8_1_rows(dev(x), k_padded=k)
+    expert_of = np.repeat(np.arange(n_experts), counts)
+    per = w.reshape(n_experts, n, -1), w2.reshape(n_experts, n, -1)
+    prod = [np.stack([oracle.ob_matmul(lib.TYPE_Q4_K, x[src[i]][None, :], m[expert_of[i]].reshape(-1), n)[0]
+                      for i in range(rows)]).astype(np.float64) for m in per]
+    L = lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    wd, w2d, bd, sd, dd = dev(w), dev(w2), dev(bounds), dev(src), dev(dst_map)
+    # plain product, scattered
+    out = torch.full((rows, n), -9.0, device="cuda")
+    lib.check("lk_moe_q4k_rows_grouped", L.lk_moe_q4k_rows_grouped(
+        wd.data_ptr(), None, 0, q.data_ptr(), k // 32, bd.data_ptr(), sd.data_ptr(), dd.data_ptr(), out.data_ptr(), n,
+        n_experts, n * (k // 256) * 144, n, k, hint, s))
+    got = out.cpu().numpy()
+    want = np.empty_like(prod[0])
+    want[dst_map] = prod[0]
+    assert (np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-4).all()
+    # gate and up with SiLU, rows left in sorted order
+    out2 = torch.full((rows, n), -9.0, device="cuda")
+    lib.check("lk_moe_q4k_rows_grouped", L.lk_moe_q4k_rows_grouped(
+        wd.data_ptr(), w2d.data_ptr(), 0, q.data_ptr(), k // 32, bd.data_ptr(), sd.data_ptr(), None, out2.data_ptr(), n,
+        n_experts, n * (k // 256) * 144, n, k, hint, s))
+    g, u = prod
+    want2 = g / (1.0 + np.exp(-g)) * u
+    got2 = out2.cpu().numpy()
+    assert (np.abs(got2 - want2) <= 1e-3 * np.abs(want2) + 1e-4 * np.abs(want2).max()).all()
