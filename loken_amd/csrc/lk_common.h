@@ -5,6 +5,7 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_bf16.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/loken_gfx950.h"
 
@@ -269,6 +270,13 @@ int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_
                        const float* down_bias, float* out, int experts, int topk, int pairs, int cols, int size_k,
                        int k32_stride, const LkGateAct& act, int slab_rows, const unsigned int* live,
                        const LkMoeAlt& alt, hipStream_t s);
+
+// Measurement runs: an integer from the environment (0 when unset). Every LK_TUNE_* variable only
+// overrides a launch-shape choice; none changes a result.
+static inline int lk_tune_env(const char* name) {
+    const char* v = getenv(name);
+    return v ? atoi(v) : 0;
+}
 
 static inline int lk_launch_status() {
     return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;

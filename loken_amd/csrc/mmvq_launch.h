@@ -175,10 +175,6 @@ __global__ __launch_bounds__(WG) void mmvq_grouped_kernel(const uint64_t* __rest
 // bytes are in flight; both have measured optima below "as many as fit" (HBM throughput drops
 // when too many requests are outstanding). LK_TUNE_WGS_PER_CU overrides the built-in cap for
 // measurement runs.
-static inline int tune_env(const char* name) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : 0;
-}
 
 // Per kernel instance and LDS size: raise the dynamic-LDS limit once and ask the runtime how many
 // workgroups a CU holds. Cached, so steady-state launches (and launches recorded into a graph)
@@ -201,7 +197,7 @@ static int resident_per_cu(K kernel, int lds_bytes) {
         (void)hipGetLastError();
         r = 1;
     }
-    static const int forced = tune_env("LK_TUNE_WGS_PER_CU");
+    static const int forced = lk_tune_env("LK_TUNE_WGS_PER_CU");
     const int cap = forced > 0 ? forced : 8;
     r = r > cap ? cap : r;
     by_lds.emplace(lds_bytes, r);
@@ -254,7 +250,7 @@ static int launch_plain_r(MmvqCall& a) {
 // measurement runs (batch <= 4).
 template <class E, int B, typename T>
 static int launch_plain(MmvqCall& a) {
-    static const int forced = tune_env("LK_TUNE_R");
+    static const int forced = lk_tune_env("LK_TUNE_R");
     if (B <= 4 && forced == 1) return launch_plain_r<E, B, 1, T>(a);
     return launch_plain_r<E, B, 2, T>(a);
 }

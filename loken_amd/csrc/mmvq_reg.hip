@@ -348,10 +348,6 @@ __global__ __launch_bounds__(RT) void q4k_reg_pair_kernel(const uint8_t* __restr
     }
 }
 
-static int tune_env(const char* name) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : 0;
-}
 // Launch shape. f32 activation: workgroups of RW waves (the row is quantized once per workgroup), two
 // per CU. Q8_1 activation: nothing is shared inside a workgroup, four waves each, four per CU.
 // LK_TUNE_REG_WAVES / LK_TUNE_REG_WGS_PER_CU override both for measurement runs.
@@ -359,7 +355,7 @@ struct Shape {
     int waves, cap;   // waves per workgroup, most workgroups launched
 };
 static Shape shape_for(bool act_f32) {
-    static const int forced_waves = tune_env("LK_TUNE_REG_WAVES"), forced_per_cu = tune_env("LK_TUNE_REG_WGS_PER_CU");
+    static const int forced_waves = lk_tune_env("LK_TUNE_REG_WAVES"), forced_per_cu = lk_tune_env("LK_TUNE_REG_WGS_PER_CU");
     const int waves = act_f32 ? RW : (forced_waves == 4 || forced_waves == 8 ? forced_waves : 4);
     const int per_cu = forced_per_cu > 0 ? forced_per_cu : 16 / waves;
     return Shape{waves, lk_device().cus * per_cu};
@@ -381,7 +377,7 @@ static int launch_multi(const LkRegMulti& m, const void* act, int act_f32, int n
     }
     const Shape sh = shape_for(act_f32 != 0);
     const int need = (total + sh.waves - 1) / sh.waves;
-    static const int forced_grid = tune_env("LK_TUNE_REG_GRID");
+    static const int forced_grid = lk_tune_env("LK_TUNE_REG_GRID");
     const dim3 grid(forced_grid > 0 ? (forced_grid < need ? forced_grid : need) : need < sh.cap ? need : sh.cap), block(sh.waves * 64);
     if (act_f32)
         hipLaunchKernelGGL((q4k_reg_kernel<R, RP, true>), grid, block, 0, s, a, (const uint8_t*)act, nb, dst_type, sh.waves);
@@ -418,7 +414,7 @@ static int launch_pair(const uint8_t* gate, const uint8_t* up, const void* act, 
 }  // namespace
 
 bool lk_q4k_reg_serves(int nb) {
-    static const int off = tune_env("LK_TUNE_NO_REG");   // measurement runs: the staged engine for everything
+    static const int off = lk_tune_env("LK_TUNE_NO_REG");   // measurement runs: the staged engine for everything
     return nb >= 1 && nb <= MAX_NB && !off;
 }
 
@@ -429,9 +425,12 @@ int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, 
     // of loads and a tail: fewer, fatter waves), one row per tile when waves stream several.
     int rows = 0;
     for (int i = 0; i < m.count; ++i) rows += m.n[i];
-    static const int forced = tune_env("LK_TUNE_REG_R");
+    static const int forced = lk_tune_env("LK_TUNE_REG_R");
     const Shape sh = shape_for(act_f32 != 0);
-    const bool two = forced ? forced == 2 : (rows + rp - 1) / rp <= sh.cap * sh.waves * 2;
+    // (from f32 rows the bound is one workgroup per CU: q + k + v of a Llama-sized layer, 6144 rows, is
+    // faster as single rows over two workgroups per CU, 5.7 against 6.1 us; o, 4096 rows, as pairs)
+    const int waves_at_once = (act_f32 ? lk_device().cus : sh.cap) * sh.waves;
+    const bool two = forced ? forced == 2 : (rows + rp - 1) / rp <= waves_at_once * 2;
     switch (rp) {
         case 1: return two ? launch_multi<2, 1>(m, act, act_f32, nb, dst_type, stream) : launch_multi<1, 1>(m, act, act_f32, nb, dst_type, stream);
         case 2: return two ? launch_multi<2, 2>(m, act, act_f32, nb, dst_type, stream) : launch_multi<1, 2>(m, act, act_f32, nb, dst_type, stream);

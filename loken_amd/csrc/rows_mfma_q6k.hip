@@ -322,12 +322,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void q6k_rows_kerne
     }
 }
 
-// Measurement runs: an integer from the environment (0 when unset).
-static int tune_env(const char* name) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : 0;
-}
-
 template <int G, bool STAGED, int WAVES>
 int resident_cap(int lds_bytes) {
     static std::mutex mu;
@@ -371,7 +365,7 @@ int launch(const Args& a, hipStream_t stream) {
     // eight waves when the tiles (times the passes of 32 rows) do not fill the CUs and a wave would
     // otherwise walk eight super-blocks or more in turn
     const int n_tiles = (a.n + 31) / 32, groups = STAGED ? 1 : (a.m + TOK - 1) / TOK;
-    static const int forced = tune_env("LK_TUNE_ROWS_WAVES");
+    static const int forced = lk_tune_env("LK_TUNE_ROWS_WAVES");
     const bool eight = forced ? forced == 8 : (n_tiles * groups <= lk_device().cus && a.nb >= 32);
     if (eight) {
         const int rc = launch_waves<G, STAGED, 8>(a, stream);
