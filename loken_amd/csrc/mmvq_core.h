@@ -855,6 +855,8 @@ static __device__ __forceinline__ void rows_q80(const RowJob<NW>& job, uint8_t* 
 // Format tags: which engine serves a ggml type, and its LDS footprint.
 struct EngQ4K {
     using Fmt = FmtQ4K;
+    static constexpr bool ONE_ROW_TILES = false;   // one row per wave tile at one activation row
+    static constexpr int WGS_PER_CU_ONE_ROW = 8;
     static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
@@ -864,6 +866,8 @@ struct EngQ4K {
 // Q4_K rows of at most 8 super-blocks (k <= 2048): 2 or 4 rows share a pass.
 struct EngQ4KShort {
     using Fmt = FmtQ4K;
+    static constexpr bool ONE_ROW_TILES = false;   // one row per wave tile at one activation row
+    static constexpr int WGS_PER_CU_ONE_ROW = 8;
     static __host__ __device__ int rows_per_pass(int nb) { return q4k_rows_per_pass(nb); }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
@@ -873,6 +877,8 @@ struct EngQ4KShort {
 // Q5_K: the Q4_K engine with the fifth-bit plane (long and short rows alike).
 struct EngQ5K {
     using Fmt = FmtQ5K;
+    static constexpr bool ONE_ROW_TILES = false;   // one row per wave tile at one activation row
+    static constexpr int WGS_PER_CU_ONE_ROW = 8;
     static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
@@ -881,6 +887,8 @@ struct EngQ5K {
 };
 struct EngQ5KShort {
     using Fmt = FmtQ5K;
+    static constexpr bool ONE_ROW_TILES = false;   // one row per wave tile at one activation row
+    static constexpr int WGS_PER_CU_ONE_ROW = 8;
     static __host__ __device__ int rows_per_pass(int nb) { return q4k_rows_per_pass(nb); }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
@@ -889,6 +897,8 @@ struct EngQ5KShort {
 };
 struct EngQ6K {
     using Fmt = FmtQ6K;
+    static constexpr bool ONE_ROW_TILES = true;   // one row per wave tile at one activation row
+    static constexpr int WGS_PER_CU_ONE_ROW = 3;
     static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
@@ -898,6 +908,8 @@ struct EngQ6K {
 // Q6_K rows of at most 8 super-blocks: 2 or 4 rows share a pass.
 struct EngQ6KShort {
     using Fmt = FmtQ6K;
+    static constexpr bool ONE_ROW_TILES = false;   // one row per wave tile at one activation row
+    static constexpr int WGS_PER_CU_ONE_ROW = 8;
     static __host__ __device__ int rows_per_pass(int nb) { return q4k_rows_per_pass(nb); }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {
@@ -906,6 +918,8 @@ struct EngQ6KShort {
 };
 struct EngQ80 {
     using Fmt = FmtQ80;
+    static constexpr bool ONE_ROW_TILES = false;   // one row per wave tile at one activation row
+    static constexpr int WGS_PER_CU_ONE_ROW = 8;
     static __host__ __device__ int rows_per_pass(int) { return 1; }
     template <int B, int R, int NW, class Epi, class Done = NoTileHook>
     static __device__ __forceinline__ void run(const RowJob<NW>& j, uint8_t* lds, Epi&& e, Done&& d = Done()) {

@@ -180,7 +180,7 @@ __global__ __launch_bounds__(WG) void mmvq_grouped_kernel(const uint64_t* __rest
 // workgroups a CU holds. Cached, so steady-state launches (and launches recorded into a graph)
 // make no runtime query. Returns workgroups resident per CU, 0 on failure.
 template <typename K>
-static int resident_per_cu(K kernel, int lds_bytes) {
+static int resident_per_cu(K kernel, int lds_bytes, int engine_cap = 8) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
     std::lock_guard<std::mutex> lock(mu);
@@ -198,7 +198,7 @@ static int resident_per_cu(K kernel, int lds_bytes) {
         r = 1;
     }
     static const int forced = lk_tune_env("LK_TUNE_WGS_PER_CU");
-    const int cap = forced > 0 ? forced : 8;
+    const int cap = forced > 0 ? forced : engine_cap;
     r = r > cap ? cap : r;
     by_lds.emplace(lds_bytes, r);
     return r;
@@ -221,7 +221,7 @@ template <class E, int B, int R, typename T>
 static int launch_plain_r(MmvqCall& a) {
     auto kernel = mmvq_kernel<E, B, R, T>;
     const int lds_bytes = lds_bytes_for<typename E::Fmt>(a.nb, B);
-    const int per_cu = resident_per_cu(kernel, lds_bytes);
+    const int per_cu = resident_per_cu(kernel, lds_bytes, B == 1 && R == 1 ? E::WGS_PER_CU_ONE_ROW : 8);
     if (per_cu == 0) return LK_ERR_ARG;
     // Persistent grid: no more workgroups than are resident at once, shared out over the
     // matrices in proportion to their rows.
@@ -246,12 +246,16 @@ static int launch_plain_r(MmvqCall& a) {
     return lk_launch_status();
 }
 
-// Rows per wave: two rows share every activation read. LK_TUNE_R=1 selects one row per tile for
-// measurement runs (batch <= 4).
+// Rows per wave: two rows share every activation read, except where an engine measured faster with
+// one row per tile at one activation row (E::ONE_ROW_TILES: Q6_K long rows, with three workgroups per
+// CU: 4096 x 14336 12.8 against 13.7 us, 2048 x 6144 5.0 against 5.8; Q4_K / Q5_K / Q8_0 lose with it).
+// LK_TUNE_R = 1 / 2 selects the form for measurement runs (batch <= 4).
 template <class E, int B, typename T>
 static int launch_plain(MmvqCall& a) {
     static const int forced = lk_tune_env("LK_TUNE_R");
-    if (B <= 4 && forced == 1) return launch_plain_r<E, B, 1, T>(a);
+    // (not from f32 rows: there every workgroup quantizes the row first, and more, lighter workgroups pay that more often)
+    const bool one = forced ? forced == 1 : (B == 1 && E::ONE_ROW_TILES && a.act_stride_f32 == 0);
+    if (B <= 4 && one) return launch_plain_r<E, B, 1, T>(a);
     return launch_plain_r<E, B, 2, T>(a);
 }
 
