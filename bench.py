@@ -49,7 +49,7 @@ HBM_PEAK_GBS = 8000.0
 # profiles/mmvq_llama3_8b_decode_b1_hbm_traffic.md. Counters cannot be read from inside this
 # process, so the figure is carried here for the configuration it was taken on:
 # (launch plan, batch, layers) -> bytes.
-MEASURED_TRAFFIC = {("auto", 1, 32): 30123486}
+MEASURED_TRAFFIC = {("auto", 1, 32): 30120755}
 LAYERS = 32
 HIDDEN, KV, FFN, VOCAB = 4096, 1024, 14336, 128256
 
@@ -373,7 +373,7 @@ def main() -> int:
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC.get((args.plan, b, args.layers)),
-                "kernel": (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<2,1,true> (q+k+v, 768 workgroups; o, 512), "
+                "kernel": (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<1,1,true> (q+k+v, 512 workgroups), q4k_reg_kernel<2,1,true> (o, 256), "
                            f"q4k_reg_pair_kernel<1,true,true> (gate+up)") if kind == "auto" and b == 1
                           else (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
                                 f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if kind == "auto"
