@@ -63,8 +63,10 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=LAYERS)
     ap.add_argument("--plan", choices=["auto", "fused", "split", "rows"], default="auto",
                     help="fused: shared-activation linears per launch, Q8_1 quantized in-kernel; split: quantize + "
-                         "mat-vec per linear; auto: fused, except that rows longer than 8192 values are quantized "
-                         "by their own launch (every workgroup of a fused launch quantizes the whole row)")
+                         "mat-vec per linear; rows: the Q4_K matrices on the matrix-unit rows kernel (q + k + v in one "
+                         "launch, gate + up in one); auto: fused at one or two rows, except that rows longer than 8192 "
+                         "values are quantized by their own launch (every workgroup of a fused launch quantizes the "
+                         "whole row), and rows from three rows on")
     ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -116,9 +118,9 @@ def main() -> int:
     gen = torch.Generator(device=dev)
     gen.manual_seed(0)
     b = args.batch
-    # `auto` above four rows (measured on MI355X): two launches per linear at 5 rows, and from 6 rows the
-    # Q4_K matrices of 2048 rows or more on the matrix-unit rows kernel
-    kind = args.plan if args.plan != "auto" or b <= 4 else ("split" if b == 5 else "rows")
+    # `auto` from three rows on (measured on MI355X: 2.03 against 2.10 ms at 3 rows, 2.70 against 3.44 at 8):
+    # the Q4_K matrices on the matrix-unit rows kernel, q + k + v in one launch and gate + up in one
+    kind = args.plan if args.plan != "auto" or b <= 2 else "rows"
 
     # ------------------------------------------------------------------ synthetic blocks
     def halfs(n, scale):
@@ -241,6 +243,35 @@ def main() -> int:
         q4k_launch_sizes.append(nbytes)
         return out
 
+    def count_q4k(item, nbytes):
+        nonlocal total_bytes, q4k_bytes
+        plan.append(item)
+        total_bytes += nbytes
+        q4k_plan.append(item)
+        q4k_bytes += nbytes
+        q4k_launch_sizes.append(nbytes)
+
+    def add_rows_multi(ws, g, ns, k):
+        """Q4_K matrices sharing the Q8_1 rows of group `g`, one launch on the matrix unit."""
+        outs = [torch.empty((b, n), dtype=torch.float32, device=dev) for n in ns]
+        q = q81[g]
+        assert q.shape[1] * 32 == k
+        vx = (C.c_void_p * len(ws))(*[w.data_ptr() for w in ws])
+        dst = (C.c_void_p * len(ws))(*[o.data_ptr() for o in outs])
+        nn = (C.c_int * len(ws))(*ns)
+        keep.extend(outs + [vx, dst, nn])
+        count_q4k((L.lk_dense_q4k_rows_multi, (vx, dst, nn, len(ws), q.data_ptr(), b, k, 0, stream)),
+                  sum(synth.weight_bytes(Q4K, n, k) for n in ns))
+        return outs[0]
+
+    def add_rows_actmul(gate, up, g, n, k):
+        """silu(gate . x) * (up . x) over the Q8_1 rows of group `g`, one launch on the matrix unit; f32
+        out into the rows the next quantizer launch reads."""
+        q = q81[g]
+        assert q.shape[1] * 32 == k
+        count_q4k((L.lk_dense_q4k_rows_actmul, (gate.data_ptr(), up.data_ptr(), q.data_ptr(), acts["h"].data_ptr(), b, n, k, 0,
+                                                stream)), 2 * synth.weight_bytes(Q4K, n, k))
+
     first_out = None
     first_w = None
     for layer in range(args.layers):
@@ -266,6 +297,23 @@ def main() -> int:
                 if first_out is None:
                     first_out, first_w = out, made["q"][0]
             continue
+        if kind == "rows":
+            # a handful of rows on the matrix unit: q + k + v in one launch, o, gate + up with the
+            # activation in one launch, each over Q8_1 rows a quantizer launch wrote; `down` (Q6_K)
+            # through the mat-vec kernels
+            made = {name: (maker(n, k), wtype, n, k, g) for name, wtype, n, k, maker, g in shapes}
+            keep.extend(v[0] for v in made.values())
+            add_quant("x")
+            out = add_rows_multi([made[nm][0] for nm in ("q", "k", "v")], "x", [made[nm][2] for nm in ("q", "k", "v")], HIDDEN)
+            if first_out is None:
+                first_out, first_w = out, made["q"][0]
+            add_quant("attn")
+            add_rows(made["o"][0], "attn", HIDDEN, HIDDEN)
+            add_quant("x2")
+            add_rows_actmul(made["gate"][0], made["up"][0], "x2", FFN, HIDDEN)
+            add_quant("h")
+            add_gemv(Q6K, made["down"][0], "h", HIDDEN, FFN)
+            continue
         last_group = None
         for name, wtype, n, k, maker, g in shapes:
             w = maker(n, k)
@@ -273,12 +321,7 @@ def main() -> int:
             if g != last_group:
                 add_quant(g)
                 last_group = g
-            # the matrix-unit rows kernel gives a workgroup 32 weight rows: below a few thousand
-            # rows it leaves most of the chip idle and the mat-vec is the faster launch
-            if kind == "rows" and wtype == Q4K and n >= 2048:
-                out = add_rows(w, g, n, k)
-            else:
-                out = add_gemv(wtype, w, g, n, k)
+            out = add_gemv(wtype, w, g, n, k)
             if first_out is None:
                 first_out, first_w = out, w
     lm_head = make_q80(VOCAB, HIDDEN)
@@ -377,8 +420,9 @@ def main() -> int:
                            f"q4k_reg_pair_kernel<1,true,true> (gate+up)") if kind == "auto" and b == 1
                           else (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
                                 f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if kind == "auto"
-                          else ("q4k_rows_staged_kernel<1,false,false> (q, o, gate, up), " if kind == "rows" else "")
-                          + f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
+                          else ("Q4_K launches of a layer on the matrix unit, 16-row tiles: q4k_rows16_kernel<false,false,4,2> (q+k+v; o), "
+                                "q4k_rows16_kernel<true,false,4,4> (gate+up)") if kind == "rows"
+                          else f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches,
                 "timed_as": "graph replay of the mix" if q4k_graph is not None else "eager launches"}
     q4k_launch_bytes = sorted({int(a_bytes) for a_bytes in q4k_launch_sizes})

@@ -426,6 +426,13 @@ void loken_dense_q4k_imma_m8_actmul(const void* gate, const void* up, const void
 /* The same launch with a status, as lk_dense_q4k_rows is to the plain form. */
 int lk_dense_q4k_rows_actmul(const void* gate, const void* up, const void* q8_1, float* output, int size_m,
                              int size_n, int size_k, int use_gelu, void* stream);
+/* Up to three Q4_K (q5 != 0: Q5_K) matrices over the same plain Q8_1 rows (q + k + v of a decode step) in
+ * one launch: outputs[i] is [size_m, sizes_n[i]] f32. The reference issues one
+ * loken_dense_q4k_imma_m8_plain per matrix (dense_q4k_imma_m8_matmul, src/inference/moe_cuda/dense/
+ * imma.rs:82-135); results equal those launches' bit for bit. `weights`, `outputs` and `sizes_n`
+ * are host arrays of `count` (1..3) entries. */
+int lk_dense_q4k_rows_multi(const void* const* weights, float* const* outputs, const int* sizes_n, int count,
+                            const void* q8_1, int size_m, int size_k, int q5, void* stream);
 /* The Q5_K siblings of the four launches above (block_q5_K = block_q4_K plus a plane of fifth bits):
  * loken_dense_q5k_imma_m8_plain / _actmul, declared src/inference/moe_cuda/mod.rs:459-466 and picked
  * by weight dtype at src/inference/moe_cuda/dense/imma.rs:113-116 and 362-365. */

@@ -114,8 +114,7 @@ size_t elem_bytes(int type) { return type == LK_TYPE_F32 ? 4 : 2; }
 }  // namespace
 
 int matvec_rows(int dtype, int k) {
-    if ((dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K) && k % 256 == 0) return 6;
-    if (dtype == LK_TYPE_Q6_K && k % 256 == 0) return 8;
+    if ((dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K || dtype == LK_TYPE_Q6_K) && k % 256 == 0) return 8;
     return tiled_serves(dtype, k) ? 32 : 8;
 }
 
@@ -131,6 +130,17 @@ static bool rows_kernel_serves(int dtype, int n, int rows) {
     if (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K) return rows <= 16 || work <= 1750000;
     if (dtype == LK_TYPE_Q6_K) return work <= (4ll << 20);
     return false;
+}
+
+// Q4_K / Q5_K at 3 to 8 f32 rows: the 16-row tiles of the matrix-unit kernel (its time hardly moves with
+// the row count) against mat-vec launches (whose dot work grows with every row). Every workgroup of
+// the rows kernel stages all the rows, so the matrix has to be large enough to pay for that: measured
+// on MI355X, k = 4096: 14336 rows from 4 activation rows, 4096 rows from 8, 1024 rows never;
+// k = 2048: 2048 rows from 4, 6144 and 151936 rows from 3.
+static bool small_rows_kernel_pays(int dtype, int n, int k, int rows) {
+    if (dtype != LK_TYPE_Q4_K && dtype != LK_TYPE_Q5_K) return false;
+    if (rows < 3 || rows > 8 || k % 256 != 0) return false;
+    return (long long)n * rows >= (k <= 2048 ? 8192 : 57344);
 }
 
 QKernelMatMul::QKernelMatMul(int dtype, int n, int k, const void* blob, int device)
@@ -155,7 +165,8 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     Slot& slot = slot_of(device_);
 
     // --- mat-vec family: up to matvec_rows, or any count when every row must sum like a one-row call
-    if (rows <= mv_max || decode_order || plain) {
+    const bool to_rows_kernel = x_type == LK_TYPE_F32 && small_rows_kernel_pays(dtype_, n_, k_, rows);
+    if ((rows <= mv_max && !to_rows_kernel) || decode_order || plain) {
         if (!plain && x_type == LK_TYPE_F32 && rows <= 2 && k_ <= 8192 && ((uintptr_t)x & 15) == 0 && k_ % 4 == 0) {
             const void* vx[1] = {blob_};
             void* dst[1] = {out};

@@ -1,0 +1,17 @@
+// Q4_K / Q5_K x at most eight Q8_1 rows in 16-row tiles on the matrix unit (rows16_mfma.hip).
+#pragma once
+#include "lk_common.h"
+
+struct LkRows16 {
+    const uint8_t* w[3];   // matrices sharing the activation (gate and up when `dual`)
+    float* dst[3];         // their outputs (`dual`: dst[0] alone)
+    int n[3];              // weight rows of each
+    int ldd[3];            // floats between output rows
+    int count;
+    const uint8_t* y;      // Q8_1 rows, stride_y blocks apart
+    int nb, m, stride_y;
+    int gelu;              // `dual`: 0 SiLU, 1 tanh-form GELU
+};
+// True when the launch takes `size_m` activation rows of `nb` super-blocks (their codes fit in LDS).
+bool lk_rows16_serves(int size_m, int nb);
+int lk_rows16_launch(const LkRows16& a, bool dual, bool q5, hipStream_t stream);

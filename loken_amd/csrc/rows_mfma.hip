@@ -33,6 +33,7 @@
 // own 16 codes), B = -dmin * m[s] in both halves. No lane exchange is needed for the sum.
 
 #include "lk_common.h"
+#include "rows16.h"
 
 #include <mutex>
 #include <unordered_map>
@@ -727,6 +728,17 @@ int launch_any(const Args& a, hipStream_t stream) {
     // at most 8 / 16 activation rows in all: the fix-up runs on the registers those rows live in,
     // and the activation is staged in LDS when it fits there
     if (a.m <= 8) {
+        // 16-row tiles (rows16_mfma.hip): half the matrix-unit time per weight, twice the tiles
+        if (lk_rows16_serves(a.m, a.nb) && lk_tune_env("LK_TUNE_ROWS16_OFF") == 0) {
+            LkRows16 r{};
+            r.w[0] = a.w; r.w[1] = a.w2;
+            r.dst[0] = a.dst;
+            r.n[0] = r.n[1] = a.n;
+            r.ldd[0] = a.ldd;
+            r.count = DUAL ? 2 : 1;
+            r.y = a.y; r.nb = a.nb; r.m = a.m; r.stride_y = a.stride_y; r.gelu = a.gelu;
+            return lk_rows16_launch(r, DUAL, Q5, stream);
+        }
         const int rc = launch_staged<1, DUAL, Q5>(a, stream);
         return rc >= 0 ? rc : launch_rows<1, DUAL, Q5>(a, stream);
     }
@@ -789,6 +801,39 @@ extern "C" int lk_dense_q4k_rows_actmul(const void* gate, const void* up, const 
 extern "C" void loken_dense_q4k_imma_m8_actmul(const void* gate, const void* up, const void* q8_1, float* output,
                                                int size_m, int size_n, int size_k, int use_gelu, void* stream) {
     (void)rows_actmul(gate, up, q8_1, output, size_m, size_n, size_k, use_gelu, false, (hipStream_t)stream);
+}
+
+// Up to three Q4_K (q5 != 0: Q5_K) matrices over the same plain Q8_1 rows in one launch (q + k + v of a
+// decode step): outputs[i] is [size_m, sizes_n[i]] f32. The reference issues one
+// loken_dense_q4k_imma_m8_plain per matrix (dense_q4k_imma_m8_matmul, src/inference/moe_cuda/dense/
+// imma.rs:82-135); the results equal those launches' bit for bit. At most 8 rows go out as one
+// launch; more rows (or rows whose codes do not fit in LDS) fall back to one launch per matrix.
+extern "C" int lk_dense_q4k_rows_multi(const void* const* weights, float* const* outputs, const int* sizes_n, int count,
+                                       const void* q8_1, int size_m, int size_k, int q5, void* stream) {
+    if (!weights || !outputs || !sizes_n || count < 1 || count > 3) return LK_ERR_ARG;
+    if (size_m == 0) return LK_OK;
+    for (int i = 0; i < count; ++i)
+        if (sizes_n[i] > 0 && bad_rows_call(weights[i], q8_1, outputs[i], size_m, sizes_n[i], size_k)) return LK_ERR_ARG;
+    const int nb = size_k / 256;
+    if (lk_rows16_serves(size_m, nb) && lk_tune_env("LK_TUNE_ROWS16_OFF") == 0) {
+        LkRows16 r{};
+        for (int i = 0; i < count; ++i) {
+            if (sizes_n[i] <= 0) continue;
+            r.w[r.count] = (const uint8_t*)weights[i];
+            r.dst[r.count] = outputs[i];
+            r.n[r.count] = r.ldd[r.count] = sizes_n[i];
+            ++r.count;
+        }
+        if (r.count == 0) return LK_OK;
+        r.y = (const uint8_t*)q8_1; r.nb = nb; r.m = size_m; r.stride_y = size_k / 32;
+        return lk_rows16_launch(r, false, q5 != 0, (hipStream_t)stream);
+    }
+    for (int i = 0; i < count; ++i) {
+        const int rc = rows_plain(weights[i], q8_1, outputs[i], size_m, sizes_n[i], size_k, size_k / 32, sizes_n[i], q5 != 0,
+                                  (hipStream_t)stream);
+        if (rc != LK_OK) return rc;
+    }
+    return LK_OK;
 }
 
 // The Q5_K siblings (loken_dense_q5k_imma_m8_plain / _actmul, declared src/inference/moe_cuda/mod.rs:459-466,

@@ -201,6 +201,25 @@ def dense_q4k_rows(weight: torch.Tensor, x: torch.Tensor, n: int, q5: bool = Fal
     return out
 
 
+def dense_q4k_rows_multi(weights, x: torch.Tensor, sizes_n, q5: bool = False, q8_1: torch.Tensor | None = None):
+    """Up to three Q4_K (``q5``: Q5_K) weights ``[n_i, k]`` over the same ``[rows, k]`` f32 rows in one
+    launch on the matrix unit (q + k + v); a list of ``[rows, n_i]`` f32 outputs. ``q8_1``: the rows
+    already quantized (then ``x`` only gives the shape)."""
+    import ctypes as C
+    rows, k = x.shape
+    if k % 256:
+        raise ValueError("dense_q4k_rows_multi: k must be a multiple of 256")
+    q = quantize_q8_1_rows(x, k_padded=k) if q8_1 is None else q8_1
+    outs = [torch.empty((rows, n), dtype=torch.float32, device=x.device) for n in sizes_n]
+    count = len(weights)
+    wp = (C.c_void_p * count)(*[w.data_ptr() for w in weights])
+    op = (C.c_void_p * count)(*[o.data_ptr() for o in outs])
+    ns = (C.c_int * count)(*[int(n) for n in sizes_n])
+    _lib.check("lk_dense_q4k_rows_multi",
+               _lib.load().lk_dense_q4k_rows_multi(wp, op, ns, count, q.data_ptr(), rows, k, 1 if q5 else 0, _stream()))
+    return outs
+
+
 def mmq_workspace_bytes(rows: int, k: int) -> int:
     """The reference's sizing (kernel_matmul/mmq.rs:38-41): 144 bytes per 128 padded values per
     row, plus 128 records of slack."""

@@ -51,12 +51,15 @@ def close(got, want, rtol=1e-3, atol=1e-4):
 
 @pytest.mark.parametrize("name,rows,n,expect", [
     ("q4_k", 1, 200, "matvec-fused"), ("q4_k", 2, 200, "matvec-fused"), ("q4_k", 5, 200, "matvec"),
-    ("q4_k", 7, 200, "rows-on-matrix-unit"), ("q4_k", 40, 200, "rows-on-matrix-unit"),
+    ("q4_k", 8, 200, "matvec"), ("q4_k", 9, 200, "rows-on-matrix-unit"), ("q4_k", 40, 200, "rows-on-matrix-unit"),
+    # a handful of rows over a matrix large enough to pay for staging them in every workgroup
+    ("q4_k", 2, 4000, "matvec-fused"), ("q4_k", 3, 4000, "rows-on-matrix-unit"), ("q4_k", 8, 1100, "rows-on-matrix-unit"),
+    ("q5_k", 4, 2100, "rows-on-matrix-unit"), ("q5_k", 4, 2000, "matvec"),
     # above 64 rows the rows kernel keeps a matrix too small to fill the chip with tiles (n x rows up to 1.75 M)
     ("q4_k", 80, 200, "rows-on-matrix-unit"), ("q4_k", 80, 24000, "tiled"),
     ("q6_k", 1, 200, "matvec-fused"), ("q6_k", 8, 200, "matvec"), ("q6_k", 20, 200, "rows-on-matrix-unit"),
     ("q6_k", 40, 200, "rows-on-matrix-unit"), ("q6_k", 200, 24000, "tiled"),
-    ("q8_0", 3, 200, "matvec"), ("q8_0", 33, 200, "tiled"), ("q5_k", 1, 200, "matvec-fused"), ("q5_k", 6, 200, "matvec"),
+    ("q8_0", 3, 200, "matvec"), ("q8_0", 33, 200, "tiled"), ("q5_k", 1, 200, "matvec-fused"), ("q5_k", 8, 200, "matvec"),
     ("q5_k", 20, 200, "rows-on-matrix-unit"), ("q5_k", 200, 200, "rows-on-matrix-unit"), ("q5_k", 80, 24000, "tiled"),
     ("q4_0", 1, 200, "matvec"), ("q4_0", 50, 200, "matvec"), ("q5_1", 9, 200, "matvec"), ("iq4_nl", 3, 200, "matvec"),
     ("mxfp4", 17, 200, "matvec"), ("q2_k", 12, 200, "matvec"), ("q3_k", 1, 200, "matvec")])
@@ -140,7 +143,7 @@ def test_workspace_grows_outside_a_capture_only_and_replays_then():
 
 def test_argument_errors_are_status_codes():
     l = lib.load()
-    assert l.lkh_matvec_rows(lib.TYPE_Q4_K, 4096) == 6 and l.lkh_matvec_rows(lib.TYPE_Q6_K, 4096) == 8
+    assert l.lkh_matvec_rows(lib.TYPE_Q4_K, 4096) == 8 and l.lkh_matvec_rows(lib.TYPE_Q6_K, 4096) == 8
     assert l.lkh_matvec_rows(lib.TYPE_Q8_0, 4096) == 32
     h = l.lkh_qkernel_matmul_new(99, 8, 256, 16, 0)
     assert l.lkh_qkernel_matmul_forward(h, 16, lib.TYPE_F32, 1, 16, None, 0) == lib.LK_ERR_TYPE

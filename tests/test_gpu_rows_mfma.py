@@ -198,3 +198,73 @@ def test_q6k_rows_emit_the_exact_integers_on_crafted_inputs():
     mask = (np.arange(256)[None, None, :] // 16) == group[:, :, None]
     want = np.einsum("nbk,mbk->mn", (codes * mask).astype(np.int64), x.reshape(m, nb, 256).astype(np.int64))
     assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, got.astype(np.int64))
+
+
+# ---------------------------------------------------------------------------------------------
+# At most eight rows: 16-row tiles on v_mfma_i32_16x16x64_i8 (rows16_mfma.hip)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("m,k,n", [(1, 256, 1), (2, 256, 15), (3, 512, 17), (4, 768, 16), (7, 1024, 31), (8, 1280, 48),
+                                   (8, 4096, 1000), (6, 4096, 4096), (8, 11008, 50), (5, 2048, 16400), (3, 256, 16500)])
+@pytest.mark.parametrize("wtype", [Q4K, lib.TYPE_Q5_K])
+def test_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n, wtype):
+    """Ragged tile edges (n not a multiple of 16), rows of one to 43 super-blocks (waves with no
+    block of their own), every row count of the launch, and matrices of more than 1024 row tiles
+    (four tiles per workgroup instead of two)."""
+    w = synth.weight(wtype, n, k, seed=70, stream=1)
+    x = synth.activation(m, k, seed=70)
+    got = ops.dense_q4k_rows(dev(w), dev(x), n, q5=wtype != Q4K).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(wtype, x, w, n))
+
+
+def test_eight_rows_emit_the_exact_integers_on_crafted_inputs():
+    """Activations on an integer grid with 127 in every block (d8 = 1); weights with d = 1, dmin = 0
+    and scale 1 in ONE sub-block of each super-block, 0 in the others: the f32 output is that
+    sub-block's integer dot, so a code that strays into the neighbouring sub-block of its
+    instruction (or a lane that should hold zeros and does not) shows."""
+    rng = np.random.default_rng(71)
+    m, k, n = 8, 1024, 80
+    nb = k // 256
+    x = rng.integers(-127, 128, size=(m, k)).astype(np.float32)
+    x.reshape(m, k // 32, 32)[:, :, 0] = 127.0
+    w = np.zeros((n, nb, 144), np.uint8)
+    w[:, :, 16:] = rng.integers(0, 256, size=(n, nb, 128), dtype=np.uint8)
+    pick = rng.integers(0, 8, size=(n, nb))
+    sc = (np.arange(8)[None, None, :] == pick[:, :, None]).astype(np.uint8)   # six-bit scales, mins 0
+    # get_scale_min_k4: j < 4: sc = q[j] & 63; j >= 4: sc = (q[j + 4] & 15) | ((q[j - 4] >> 6) << 4)
+    w[:, :, 4:8] = sc[:, :, 0:4]
+    w[:, :, 12:16] = sc[:, :, 4:8]
+    w[:, :, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    got = ops.dense_q4k_rows(dev(w.reshape(n, -1)), dev(x), n).cpu().numpy()
+    qs = w[:, :, 16:].astype(np.int64).reshape(n, nb, 4, 32)
+    codes = np.stack([qs & 15, qs >> 4], axis=3).reshape(n, nb, 8, 32)       # sub-block 2 p, 2 p + 1
+    xs = x.reshape(m, nb, 8, 32).astype(np.int64)
+    want = np.einsum("nbsk,mbsk,nbs->mn", codes, xs, sc.astype(np.int64))
+    assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, got.astype(np.int64))
+
+
+@pytest.mark.parametrize("m", [1, 5, 8, 11])
+@pytest.mark.parametrize("q5", [False, True])
+def test_three_matrices_in_one_launch_carry_the_single_launches_bits(m, q5):
+    """q + k + v: lk_dense_q4k_rows_multi against one lk_dense_q4k_rows per matrix."""
+    k, sizes = 2048, (520, 130, 7)
+    wtype = lib.TYPE_Q5_K if q5 else Q4K
+    ws = [dev(synth.weight(wtype, n, k, seed=72, stream=i)) for i, n in enumerate(sizes)]
+    x = dev(synth.activation(m, k, seed=72))
+    outs = ops.dense_q4k_rows_multi(ws, x, sizes, q5=q5)
+    for w, n, out in zip(ws, sizes, outs):
+        assert torch.equal(out, ops.dense_q4k_rows(w, x, n, q5=q5))
+    two = ops.dense_q4k_rows_multi(ws[:2], x, sizes[:2], q5=q5)
+    assert torch.equal(two[0], outs[0]) and torch.equal(two[1], outs[1])
+
+
+@pytest.mark.parametrize("m,k,n", [(8, 4096, 8200), (2, 512, 9000)])
+def test_gate_and_up_of_many_row_tiles(m, k, n):
+    """The dual launch with four tiles (two gate, two up) per workgroup: bits of the plain launches."""
+    gate, up = dev(synth.weight(Q4K, n, k, seed=73, stream=1)), dev(synth.weight(Q4K, n, k, seed=73, stream=2))
+    x = dev(synth.activation(m, k, seed=73))
+    g, u = ops.dense_q4k_rows(gate, x, n).double(), ops.dense_q4k_rows(up, x, n).double()
+    want = g / (1.0 + torch.exp(-g)) * u
+    got = ops.dense_q4k_rows_actmul(gate, up, x, n, False).double()
+    assert ((got - want).abs() <= 2e-6 * want.abs() + 1e-30).all()
+    w = synth.weight(Q4K, 64, k, seed=73, stream=1)
+    assert_close(ops.dense_q4k_rows(gate[:64 * (k // 256) * 144], x, 64).cpu().numpy(), oracle.ob_matmul(Q4K, x.cpu().numpy(), w, 64))
