@@ -272,6 +272,16 @@ def main() -> int:
         count_q4k((L.lk_dense_q4k_rows_actmul, (gate.data_ptr(), up.data_ptr(), q.data_ptr(), acts["h"].data_ptr(), b, n, k, 0,
                                                 stream)), 2 * synth.weight_bytes(Q4K, n, k))
 
+    def add_rows_q6k(w, g, n, k):
+        """Q6_K x the Q8_1 rows of group `g` on the matrix unit."""
+        nonlocal total_bytes
+        out = torch.empty((b, n), dtype=torch.float32, device=dev)
+        keep.append(out)
+        q = q81[g]
+        assert q.shape[1] * 32 == k
+        plan.append((L.lk_dense_q6k_rows, (w.data_ptr(), q.data_ptr(), out.data_ptr(), b, n, k, stream)))
+        total_bytes += synth.weight_bytes(Q6K, n, k)
+
     first_out = None
     first_w = None
     for layer in range(args.layers):
@@ -299,8 +309,8 @@ def main() -> int:
             continue
         if kind == "rows":
             # a handful of rows on the matrix unit: q + k + v in one launch, o, gate + up with the
-            # activation in one launch, each over Q8_1 rows a quantizer launch wrote; `down` (Q6_K)
-            # through the mat-vec kernels
+            # activation in one launch, `down` (Q6_K) on the matrix unit too, each over Q8_1 rows a
+            # quantizer launch wrote
             made = {name: (maker(n, k), wtype, n, k, g) for name, wtype, n, k, maker, g in shapes}
             keep.extend(v[0] for v in made.values())
             add_quant("x")
@@ -312,7 +322,7 @@ def main() -> int:
             add_quant("x2")
             add_rows_actmul(made["gate"][0], made["up"][0], "x2", FFN, HIDDEN)
             add_quant("h")
-            add_gemv(Q6K, made["down"][0], "h", HIDDEN, FFN)
+            add_rows_q6k(made["down"][0], "h", HIDDEN, FFN)
             continue
         last_group = None
         for name, wtype, n, k, maker, g in shapes:

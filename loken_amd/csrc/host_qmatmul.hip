@@ -132,14 +132,17 @@ static bool rows_kernel_serves(int dtype, int n, int rows) {
     return false;
 }
 
-// Q4_K / Q5_K at 3 to 8 f32 rows: the 16-row tiles of the matrix-unit kernel (its time hardly moves with
-// the row count) against mat-vec launches (whose dot work grows with every row). Every workgroup of
-// the rows kernel stages all the rows, so the matrix has to be large enough to pay for that: measured
-// on MI355X, k = 4096: 14336 rows from 4 activation rows, 4096 rows from 8, 1024 rows never;
-// k = 2048: 2048 rows from 4, 6144 and 151936 rows from 3.
+// The K-quants at 3 to 8 f32 rows: the 16-row tiles of the matrix-unit kernels (their time hardly moves
+// with the row count) against mat-vec launches (whose dot work grows with every row). Every workgroup of
+// a rows kernel stages all the rows, so the matrix has to be large enough to pay for that. Measured on
+// MI355X, Q4_K / Q5_K, k = 4096: 14336 rows from 4 activation rows, 4096 rows from 8, 1024 rows never;
+// k = 2048: 2048 rows from 4, 6144 and 151936 rows from 3. Q6_K (k a multiple of 2048: its rows are loaded
+// in granules of eight super-blocks): 4096 x 14336 and 151936 x 2048 from 3 rows, 14336 x 4096 from 4,
+// 4096 x 4096 and 2048 x 6144 never.
 static bool small_rows_kernel_pays(int dtype, int n, int k, int rows) {
-    if (dtype != LK_TYPE_Q4_K && dtype != LK_TYPE_Q5_K) return false;
     if (rows < 3 || rows > 8 || k % 256 != 0) return false;
+    if (dtype == LK_TYPE_Q6_K) return k % 2048 == 0 && (long long)n * k >= (48ll << 20);
+    if (dtype != LK_TYPE_Q4_K && dtype != LK_TYPE_Q5_K) return false;
     return (long long)n * rows >= (k <= 2048 ? 8192 : 57344);
 }
 

@@ -18,6 +18,7 @@
 //     qh half-rows at 16 lh, the 16 scales and d: every byte of ql and qh once per wave.
 
 #include "lk_common.h"
+#include "rows16.h"
 
 #include <cstdlib>
 #include <mutex>
@@ -388,6 +389,9 @@ int lk_q6k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m,
     Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd};
     int rc = -1;
     if (size_m <= 8) {
+        // 16-row tiles (rows16_q6k.hip): a quarter of the matrix-unit time per weight, and every CU a tile
+        rc = lk_rows16_q6k(w, q8_1, output, size_m, size_n, size_k, stride_y, ldd, stream);
+        if (rc >= 0) return rc;
         rc = launch<1, true>(a, stream);
         if (rc < 0) rc = launch<1, false>(a, stream);
     } else if (size_m <= 16) {

@@ -268,3 +268,48 @@ def test_gate_and_up_of_many_row_tiles(m, k, n):
     assert ((got - want).abs() <= 2e-6 * want.abs() + 1e-30).all()
     w = synth.weight(Q4K, 64, k, seed=73, stream=1)
     assert_close(ops.dense_q4k_rows(gate[:64 * (k // 256) * 144], x, 64).cpu().numpy(), oracle.ob_matmul(Q4K, x.cpu().numpy(), w, 64))
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 256, 1), (2, 512, 15), (3, 768, 17), (4, 1024, 33), (4, 14336, 48), (5, 256, 16), (7, 1280, 100),
+                                   (8, 6144, 500), (6, 2048, 8300), (3, 512, 8300), (8, 512, 16500), (4, 256, 16500)])
+def test_q6k_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n):
+    """rows16_q6k.hip: both slot layouts (up to four rows, up to eight), ragged tile edges, rows of
+    one super-block (waves with nothing to add), one, two and four tiles per workgroup."""
+    w = synth.weight(Q6K, n, k, seed=74, stream=1)
+    x = synth.activation(m, k, seed=74)
+    got = ops.dense_q6k_rows(dev(w), dev(x), n).cpu().numpy()
+    assert_close(got, oracle.ob_matmul(Q6K, x, w, n))
+
+
+@pytest.mark.parametrize("k", [1024, 4096])
+@pytest.mark.parametrize("m", [3, 4, 7])
+def test_q6k_few_rows_emit_the_exact_integers_on_crafted_inputs(m, k):
+    """As test_q6k_rows_emit_the_exact_integers_on_crafted_inputs, for the launches of at most four
+    and at most eight rows: one group of each super-block has scale 1, the others 0, so a code that
+    strays into a neighbouring group of its instruction shows. k = 4096: rows of whole eight-block
+    granules, whose super-blocks are read back from LDS at eight different byte offsets."""
+    rng = np.random.default_rng(75 + m)
+    n = 80
+    nb = k // 256
+    x = rng.integers(-127, 128, size=(m, k)).astype(np.float32)
+    x.reshape(m, k // 32, 32)[:, :, 0] = 127.0
+    w = np.zeros((n, nb, 210), np.uint8)
+    w[:, :, :192] = rng.integers(0, 256, size=(n, nb, 192), dtype=np.uint8)
+    group = rng.integers(0, 16, size=(n, nb))
+    scales = np.zeros((n, nb, 16), np.int8)
+    np.put_along_axis(scales, group[:, :, None], 1, axis=2)
+    w[:, :, 192:208] = scales.view(np.uint8)
+    w[:, :, 208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    got = ops.dense_q6k_rows(dev(w.reshape(n, -1)), dev(x), n).cpu().numpy()
+    ql, qh = w[:, :, :128].astype(np.int32), w[:, :, 128:192].astype(np.int32)
+    codes = np.zeros((n, nb, 256), np.int32)
+    for half in range(2):
+        for qt in range(4):
+            l = np.arange(32)
+            nib = ql[:, :, 64 * half + 32 * (qt & 1) + l]
+            nib = (nib >> 4) if qt & 2 else (nib & 15)
+            hi = (qh[:, :, 32 * half + l] >> (2 * qt)) & 3
+            codes[:, :, 128 * half + 32 * qt + l] = (nib | (hi << 4)) - 32
+    mask = (np.arange(256)[None, None, :] // 16) == group[:, :, None]
+    want = np.einsum("nbk,mbk->mn", (codes * mask).astype(np.int64), x.reshape(m, nb, 256).astype(np.int64))
+    assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, got.astype(np.int64))
