@@ -1,4 +1,4 @@
-// Q4_K / Q5_K x at most eight Q8_1 rows in 16-row tiles on the matrix unit (rows16_mfma.hip).
+// Q4_K / Q5_K x at most sixteen Q8_1 rows in 16-row tiles on the matrix unit (rows16_mfma.hip).
 #pragma once
 #include "lk_common.h"
 
@@ -16,7 +16,7 @@ struct LkRows16 {
 bool lk_rows16_serves(int size_m, int nb);
 int lk_rows16_launch(const LkRows16& a, bool dual, bool q5, hipStream_t stream);
 
-// Q6_K x at most eight Q8_1 rows in 16-row tiles (rows16_q6k.hip). LK_* status, or -1 when the launch
-// does not serve the call (more than eight rows, or rows whose codes do not fit in LDS).
+// Q6_K x at most sixteen Q8_1 rows in 16-row tiles (rows16_q6k.hip). LK_* status, or -1 when the launch
+// does not serve the call (more rows, k not a multiple of 2048, or rows whose codes do not fit in LDS).
 int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y, int ldd,
                   hipStream_t stream);

@@ -43,9 +43,9 @@
 namespace {
 
 constexpr int KSPLIT = 4;   // waves that share a row tile
-constexpr int TOKS = 8;     // activation rows a launch serves
+constexpr int MAX_TOKS = 16;   // activation rows a launch serves: kernels for up to 8 and up to 16
 constexpr int TILE = 16;    // weight rows of a wave's tile
-constexpr int ZERO_BYTES = 2048;
+static __host__ __device__ constexpr int zero_bytes(int toks) { return toks * 256; }   // the zero lanes' run
 
 struct WFrag {
     uint4 hdr, q[2], qh;   // qh: Q5_K only
@@ -57,9 +57,9 @@ struct Blk {
     static constexpr int QS = Q5 ? 48 : 16;
 };
 
-static __host__ __device__ constexpr int lds_bytes_for(int nb, int tiles) {
-    // codes [nb * 8][8][32], zeros, d8 and d8 * S [nb * 8][2][8] floats, reduce [4 tiles][4][64] floats
-    return nb * 8 * TOKS * 32 + ZERO_BYTES + nb * 8 * 2 * TOKS * 4 + KSPLIT * tiles * 4 * 64 * 4;
+static __host__ __device__ constexpr int lds_bytes_for(int nb, int tiles, int toks) {
+    // codes [nb * 8][toks][32], zeros, d8 and d8 * S [nb * 8][2][toks] floats, reduce [4 tiles][4][64] floats
+    return nb * 8 * toks * 32 + zero_bytes(toks) + nb * 8 * 2 * toks * 4 + KSPLIT * tiles * 4 * 64 * 4;
 }
 
 // Element `i` of a three-entry kernel argument without indexing it by a register (which would
@@ -86,13 +86,19 @@ static __device__ __forceinline__ TileRef tile_ref(const LkRows16& p, int vt) {
 
 // TW: row tiles a workgroup takes at a time (four waves each). STEPS: super-blocks a wave owns of
 // every tile when that is the same for all waves (rows of 4 STEPS super-blocks), 0 for any row length.
-template <bool DUAL, bool Q5, int STEPS, int TW>
+// T16: up to sixteen activation rows. The sixteen slots are then all rows, and every set of weight codes
+// runs twice: once against sub-block s (the activation live in lane groups 0, 1) and once against s + 2
+// (live in groups 2, 3). Lane l, register v is (weight row l % 16, activation row 4 (l / 16) + v) for
+// both, so every lane unpacks all eight scales of its row and its sums are complete across sub-blocks.
+template <bool DUAL, bool Q5, int STEPS, int TW, bool T16>
 __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(LkRows16 p, int n_vt) {
     constexpr int WG = 256 * TW;
+    constexpr int TOKS = T16 ? 16 : 8;
+    constexpr int ZERO_BYTES = zero_bytes(TOKS);
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t* codes = lds;                                               // [nb * 8][8][32]
     uint8_t* zeros = codes + (size_t)p.nb * 8 * TOKS * 32;              // ZERO_BYTES
-    float* table = (float*)(zeros + ZERO_BYTES);                        // [nb * 8][2][8]: d8, d8 * S
+    float* table = (float*)(zeros + ZERO_BYTES);                        // [nb * 8][2][TOKS]: d8, d8 * S
     float* reduce = table + p.nb * 8 * 2 * TOKS;                        // [4 TW][4][64]
 
     const int lane = threadIdx.x & 63;
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
 #pragma unroll
         for (int u = 0; u < PER; ++u) {
             const int idx = min(base + u * WG, entries - 1);
-            const int sub = idx >> 3, tok = min(idx & 7, p.m - 1);
+            const int sub = idx / TOKS, tok = min(idx % TOKS, p.m - 1);
             const uint8_t* b = p.y + ((size_t)tok * p.stride_y + sub) * Q81_BYTES;
             head[u] = *(const uint32_t*)b;
             lo[u] = *(const uint4_a4*)(b + 4);
@@ -143,11 +149,11 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
         for (int u = 0; u < PER; ++u) {
             const int idx = base + u * WG;
             if (idx < entries) {
-                const bool real = (idx & 7) < p.m;
+                const int sub = idx / TOKS, tok = idx % TOKS;
+                const bool real = tok < p.m;
                 const float d8 = real ? f16_bits_to_f32(head[u] & 0xFFFFu) : 0.f;
-                const int sub = idx >> 3, tok = idx & 7;
-                table[sub * 16 + tok] = d8;
-                table[sub * 16 + 8 + tok] = d8 * (float)dot16(ones, hi[u], dot16(ones, lo[u], 0));
+                table[sub * 2 * TOKS + tok] = d8;
+                table[sub * 2 * TOKS + TOKS + tok] = d8 * (float)dot16(ones, hi[u], dot16(ones, lo[u], 0));
                 const uint32_t keep = real ? 0xFFFFFFFFu : 0u;   // rows the launch does not have: zeros
                 *(uint4*)(codes + (size_t)idx * 32) = make_uint4(lo[u].x & keep, lo[u].y & keep, lo[u].z & keep, lo[u].w & keep);
                 *(uint4*)(codes + (size_t)idx * 32 + 16) = make_uint4(hi[u].x & keep, hi[u].y & keep, hi[u].z & keep, hi[u].w & keep);
@@ -155,15 +161,21 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
         }
     };
 
-    // The lane's piece of the activation operand: slot l16 is (sub-block l16 / 8 of the two, row
-    // l16 % 8); the lane's K group belongs to sub-block par. Where the two differ the piece is zeros:
-    // those lanes read the run of zeros, at a stride of nothing.
-    const bool live = (l16 >> 3) == par;
-    const uint8_t* a_lane = live ? codes + (2 * par * TOKS + (l16 & 7)) * 32 + 16 * half : zeros;
+    // The lane's piece of the activation operand. Up to eight rows: slot l16 is (sub-block l16 / 8 of the
+    // two, row l16 % 8); the lane's K group belongs to sub-block par; where the two differ the piece is
+    // zeros: those lanes read the run of zeros, at a stride of nothing. Up to sixteen rows: slot l16 is row
+    // l16, and there are two pieces, one per run of the instruction: live for the lanes of sub-block 0
+    // (groups 0, 1) in the first, for those of sub-block 1 in the second.
+    const bool live = T16 ? par == 0 : (l16 >> 3) == par;
+    const bool live2 = T16 && par == 1;
+    const uint8_t* a_lane = live ? codes + (T16 ? l16 : 2 * par * TOKS + (l16 & 7)) * 32 + 16 * half : zeros;
+    const uint8_t* a_lane2 = live2 ? codes + (2 * TOKS + l16) * 32 + 16 * half : zeros;
     const int a_step = live ? 8 * TOKS * 32 : 0;   // bytes per super-block
-    // the lane's results: sub-blocks 2 par + {0, 1, 4, 5}, activation rows 4 half .. 4 half + 3
-    const float* t_lane = table + 2 * par * 16 + 4 * half;
-    const int sh16 = 16 * par, sh2 = 2 * par;
+    const int a_step2 = live2 ? 8 * TOKS * 32 : 0;
+    // the lane's results: up to eight rows: sub-blocks 2 par + {0, 1, 4, 5}, rows 4 half .. 4 half + 3;
+    // up to sixteen: every sub-block, rows 4 grp .. 4 grp + 3
+    const float* t_lane = T16 ? table + 4 * grp : table + 2 * par * 2 * TOKS + 4 * half;
+    const int sh16 = T16 ? 0 : 16 * par, sh2 = 2 * par;
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
 
@@ -181,16 +193,31 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
             for (int e = 0; e < 4; ++e) hp[e] >>= sh2;
         }
         const uint8_t* a_blk = a_lane + (size_t)kb * a_step;
-        const float* t_blk = t_lane + kb * 8 * 16;
+        const uint8_t* a_blk2 = a_lane2 + (size_t)kb * a_step2;
+        const float* t_blk = t_lane + kb * 8 * 2 * TOKS;
+        // The accumulators start at the bit pattern of 1.5 * 2^23: adding an integer of magnitude below
+        // 2^22 to that pattern yields the float 1.5 * 2^23 + integer, so the dots leave the matrix unit
+        // as floats. The offset goes in the first fused multiply-add, exactly: d * sc is an f16 times a
+        // six-bit integer (17 significant bits), MAGIC * d * sc has 19, neither product rounds, and the
+        // fma rounds dot * d * sc once, as convert-then-multiply would.
+        constexpr int MAGIC_BITS = 0x4B400000;
+        constexpr float MAGIC = 12582912.0f;
+        const v4i magic = {MAGIC_BITS, MAGIC_BITS, MAGIC_BITS, MAGIC_BITS};
+        // one instruction's four results into the sums: sub-block `sub` of the super-block
+        auto fold = [&](const v4i& c, float dsc, float dmm, int sub) {
+            const float off = -MAGIC * dsc;
+            const float4 t = *(const float4*)(t_blk + sub * 2 * TOKS);
+            const float4 s = *(const float4*)(t_blk + sub * 2 * TOKS + TOKS);
+            acc[0] = fmaf(fmaf(__int_as_float(c[0]), dsc, off), t.x, fmaf(dmm, s.x, acc[0]));
+            acc[1] = fmaf(fmaf(__int_as_float(c[1]), dsc, off), t.y, fmaf(dmm, s.y, acc[1]));
+            acc[2] = fmaf(fmaf(__int_as_float(c[2]), dsc, off), t.z, fmaf(dmm, s.z, acc[2]));
+            acc[3] = fmaf(fmaf(__int_as_float(c[3]), dsc, off), t.w, fmaf(dmm, s.w, acc[3]));
+        };
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {
             const uint32_t u[4] = {w.q[c2].x, w.q[c2].y, w.q[c2].z, w.q[c2].w};
 #pragma unroll
             for (int nib = 0; nib < 2; ++nib) {
-                // this lane's sub-block: 4 c2 + 2 par + nib
-                const uint32_t scs = ((c2 ? sc_hi : sc_lo) >> (8 * nib)) & 0xFFu;
-                const uint32_t mns = ((c2 ? mn_hi : mn_lo) >> (8 * nib)) & 0xFFu;
-                const float dsc = d * (float)scs, dmm = -(dmin * (float)mns);
                 v4i b;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -198,24 +225,22 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
                     if (Q5) x |= ((hp[e] >> (4 * c2 + nib)) & 0x01010101u) << 4;
                     b[e] = (int)x;
                 }
-                const v4i a = *(const v4i*)(a_blk + (4 * c2 + nib) * TOKS * 32);
-                // The accumulators start at the bit pattern of 1.5 * 2^23: adding an integer of
-                // magnitude below 2^22 to that pattern yields the float 1.5 * 2^23 + integer, so the
-                // dots leave the matrix unit as floats. The offset goes in the first fused
-                // multiply-add, exactly: d * sc is an f16 times a six-bit integer (17 significant
-                // bits), MAGIC * d * sc has 19, neither product rounds, and the fma rounds
-                // dot * d * sc once, as convert-then-multiply would.
-                constexpr int MAGIC_BITS = 0x4B400000;
-                constexpr float MAGIC = 12582912.0f;
-                v4i c = {MAGIC_BITS, MAGIC_BITS, MAGIC_BITS, MAGIC_BITS};
-                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
-                const float off = -MAGIC * dsc;
-                const float4 t = *(const float4*)(t_blk + (4 * c2 + nib) * 16);
-                const float4 s = *(const float4*)(t_blk + (4 * c2 + nib) * 16 + 8);
-                acc[0] = fmaf(fmaf(__int_as_float(c[0]), dsc, off), t.x, fmaf(dmm, s.x, acc[0]));
-                acc[1] = fmaf(fmaf(__int_as_float(c[1]), dsc, off), t.y, fmaf(dmm, s.y, acc[1]));
-                acc[2] = fmaf(fmaf(__int_as_float(c[2]), dsc, off), t.z, fmaf(dmm, s.z, acc[2]));
-                acc[3] = fmaf(fmaf(__int_as_float(c[3]), dsc, off), t.w, fmaf(dmm, s.w, acc[3]));
+                const uint32_t scw = c2 ? sc_hi : sc_lo, mnw = c2 ? mn_hi : mn_lo;
+                if constexpr (T16) {
+                    // sub-blocks 4 c2 + nib (lane groups 0, 1) and 4 c2 + 2 + nib (groups 2, 3)
+                    const v4i a0 = *(const v4i*)(a_blk + (4 * c2 + nib) * TOKS * 32);
+                    const v4i a1 = *(const v4i*)(a_blk2 + (4 * c2 + nib) * TOKS * 32);
+                    const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, magic, 0, 0, 0);
+                    const v4i c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b, magic, 0, 0, 0);
+                    fold(c0, d * (float)((scw >> (8 * nib)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib)) & 0xFFu)), 4 * c2 + nib);
+                    fold(c1, d * (float)((scw >> (8 * nib + 16)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib + 16)) & 0xFFu)),
+                         4 * c2 + 2 + nib);
+                } else {
+                    // this lane's sub-block: 4 c2 + 2 par + nib (its scale words are shifted to it)
+                    const v4i a = *(const v4i*)(a_blk + (4 * c2 + nib) * TOKS * 32);
+                    const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, magic, 0, 0, 0);
+                    fold(c, d * (float)((scw >> (8 * nib)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib)) & 0xFFu)), 4 * c2 + nib);
+                }
             }
         }
     };
@@ -229,13 +254,16 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
             acc[v] = 0.f;
         }
         __syncthreads();
-        // thread (tile ts, register v, lane l < 32): the four shares of the tile's super-blocks and
-        // the two sub-blocks of an instruction (lanes l and l + 32)
+        // Up to eight rows: thread (tile ts, register v, lane l < 32) adds the four shares of the tile's
+        // super-blocks and the two sub-blocks of an instruction (lanes l and l + 32). Up to sixteen: thread
+        // (ts, v, l < 64) adds the four shares.
+        constexpr int LANES = T16 ? 64 : 32, PER_TILE = 4 * LANES;
         const int t = threadIdx.x;
-        if (t < (DUAL ? 64 * TW : 128 * TW)) {
-            const int ts = (t >> 7) * (DUAL ? 2 : 1), v = (t >> 5) & 3, l = t & 31;
+        if (t < (DUAL ? PER_TILE * TW / 2 : PER_TILE * TW)) {
+            const int ts = (t / PER_TILE) * (DUAL ? 2 : 1), v = (t / LANES) & 3, l = t % LANES;
             auto total_of = [&](int which) {
                 const float* col = reduce + which * (KSPLIT * 256) + v * 64 + l;
+                if (T16) return (col[0] + col[256]) + (col[512] + col[768]);
                 return ((col[0] + col[32]) + (col[256] + col[288])) + ((col[512] + col[544]) + (col[768] + col[800]));
             };
             float sum = total_of(ts);
@@ -248,7 +276,7 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
             if (vt < n_vt) {
                 const TileRef tr = tile_ref<DUAL>(p, vt);
                 const int out = DUAL ? 0 : tr.mat;
-                const int tok = 4 * ((l >> 4) & 1) + v, row = tr.row0 + (l & 15);
+                const int tok = (T16 ? 4 * (l >> 4) : 4 * ((l >> 4) & 1)) + v, row = tr.row0 + (l & 15);
                 if (tok < p.m && row < pick3(p.n, out)) pick3(p.dst, out)[(size_t)tok * pick3(p.ldd, out) + row] = sum;
             }
         }
@@ -333,7 +361,7 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
 }
 
 // Workgroups per CU the kernel can keep resident with `lds_bytes` of LDS each; 0: does not fit.
-template <bool DUAL, bool Q5, int STEPS, int TW>
+template <bool DUAL, bool Q5, int STEPS, int TW, bool T16>
 int resident_cap(int lds_bytes) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -344,11 +372,11 @@ int resident_cap(int lds_bytes) {
     if (lds_bytes > lk_device().lds_bytes) {
         r = 0;
     } else if (lds_bytes > 48 * 1024 &&
-               hipFuncSetAttribute((const void*)q4k_rows16_kernel<DUAL, Q5, STEPS, TW>, hipFuncAttributeMaxDynamicSharedMemorySize,
+               hipFuncSetAttribute((const void*)q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         r = 0;
-    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows16_kernel<DUAL, Q5, STEPS, TW>, 256 * TW,
+    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16>, 256 * TW,
                                                             (size_t)lds_bytes) != hipSuccess || r < 1) {
         (void)hipGetLastError();
         r = 1;
@@ -357,10 +385,10 @@ int resident_cap(int lds_bytes) {
     return r;
 }
 
-template <bool DUAL, bool Q5, int STEPS, int TW>
+template <bool DUAL, bool Q5, int STEPS, int TW, bool T16>
 int launch_shape(const LkRows16& a, int n_vt, hipStream_t stream) {
-    const int lds_bytes = lds_bytes_for(a.nb, TW);
-    const int per_cu = resident_cap<DUAL, Q5, STEPS, TW>(lds_bytes);
+    const int lds_bytes = lds_bytes_for(a.nb, TW, T16 ? 16 : 8);
+    const int per_cu = resident_cap<DUAL, Q5, STEPS, TW, T16>(lds_bytes);
     if (per_cu == 0) return -1;
     const int units = (n_vt + TW - 1) / TW;   // tile groups
     // Every workgroup stages the activation, so a workgroup should walk a few tile groups; all of
@@ -370,11 +398,11 @@ int launch_shape(const LkRows16& a, int n_vt, hipStream_t stream) {
     if (forced > 0) cap = forced;
     const int passes = (units + cap - 1) / cap;
     const int wgs = (units + passes - 1) / passes;
-    hipLaunchKernelGGL((q4k_rows16_kernel<DUAL, Q5, STEPS, TW>), dim3(wgs), dim3(256 * TW), lds_bytes, stream, a, n_vt);
+    hipLaunchKernelGGL((q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16>), dim3(wgs), dim3(256 * TW), lds_bytes, stream, a, n_vt);
     return lk_launch_status();
 }
 
-template <bool DUAL, bool Q5, int STEPS>
+template <bool DUAL, bool Q5, int STEPS, bool T16>
 int launch_steps(const LkRows16& a, hipStream_t stream) {
     int n_vt = 0;
     if (DUAL) {
@@ -389,28 +417,33 @@ int launch_steps(const LkRows16& a, hipStream_t stream) {
     const int forced = lk_tune_env("LK_TUNE_ROWS16_TW");
     if (forced == 2 || forced == 4) tw = forced;
     if (tw == 4) {
-        const int rc = launch_shape<DUAL, Q5, STEPS, 4>(a, n_vt, stream);
+        const int rc = launch_shape<DUAL, Q5, STEPS, 4, T16>(a, n_vt, stream);
         if (rc >= 0) return rc;
     }
-    return launch_shape<DUAL, Q5, STEPS, 2>(a, n_vt, stream);
+    return launch_shape<DUAL, Q5, STEPS, 2, T16>(a, n_vt, stream);
+}
+
+template <bool DUAL, bool Q5, bool T16>
+int launch_rows(const LkRows16& a, hipStream_t stream) {
+    const int forced = lk_tune_env("LK_TUNE_ROWS16_GENERIC");
+    if (a.nb == 16 && !forced) return launch_steps<DUAL, Q5, 4, T16>(a, stream);
+    if (a.nb == 8 && !forced) return launch_steps<DUAL, Q5, 2, T16>(a, stream);
+    return launch_steps<DUAL, Q5, 0, T16>(a, stream);
 }
 
 template <bool DUAL, bool Q5>
 int launch(const LkRows16& a, hipStream_t stream) {
-    const int forced = lk_tune_env("LK_TUNE_ROWS16_GENERIC");
-    if (a.nb == 16 && !forced) return launch_steps<DUAL, Q5, 4>(a, stream);
-    if (a.nb == 8 && !forced) return launch_steps<DUAL, Q5, 2>(a, stream);
-    return launch_steps<DUAL, Q5, 0>(a, stream);
+    return a.m <= 8 ? launch_rows<DUAL, Q5, false>(a, stream) : launch_rows<DUAL, Q5, true>(a, stream);
 }
 
 }  // namespace
 
 bool lk_rows16_serves(int size_m, int nb) {
-    return size_m >= 1 && size_m <= TOKS && nb >= 1 && lds_bytes_for(nb, 2) <= lk_device().lds_bytes;
+    return size_m >= 1 && size_m <= MAX_TOKS && nb >= 1 && lds_bytes_for(nb, 2, size_m <= 8 ? 8 : 16) <= lk_device().lds_bytes;
 }
 
 int lk_rows16_launch(const LkRows16& a, bool dual, bool q5, hipStream_t stream) {
-    if (a.m < 1 || a.m > TOKS || a.nb < 1 || a.count < 1 || a.count > 3 || (dual && a.count != 2)) return LK_ERR_ARG;
+    if (a.m < 1 || a.m > MAX_TOKS || a.nb < 1 || a.count < 1 || a.count > 3 || (dual && a.count != 2)) return LK_ERR_ARG;
     if (dual && a.n[0] != a.n[1]) return LK_ERR_ARG;
     int rc;
     if (dual) rc = q5 ? launch<true, true>(a, stream) : launch<true, false>(a, stream);

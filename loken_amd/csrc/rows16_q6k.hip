@@ -44,7 +44,6 @@ namespace {
 
 constexpr int MAX_WAVES = 16;
 constexpr int TILE = 16;
-constexpr int ZERO_BYTES = 2048;
 constexpr int GRAN = 8;                 // super-blocks of a wave's granule
 constexpr int BLOCK_PIECES = 14;        // 16-byte pieces that hold one super-block of a granule
 constexpr int WPITCH = BLOCK_PIECES * 16 + 16;   // bytes between rows of a wave's buffer: 16 rows on 16 bank groups
@@ -86,15 +85,19 @@ template <int TOKS>
 static __host__ __device__ constexpr int lds_bytes_for(int nb, int waves) {
     // codes [nb * 8][TOKS][32], zeros, d8 [nb * 8][TOKS] floats, a buffer per wave (which also holds the
     // wave's partial tile of the reduction)
-    return nb * 8 * TOKS * 32 + ZERO_BYTES + nb * 8 * TOKS * 4 + waves * WBUF;
+    return nb * 8 * TOKS * 32 + TOKS * 256 + nb * 8 * TOKS * 4 + waves * WBUF;
 }
 
-// T8: up to eight activation rows (two instructions per set of weight registers), else up to four.
+// TOKS: the activation rows a launch serves. 4: one instruction per set of weight registers (slots =
+// group x row). 8: two (slots = one of two groups x row). 16: four (slots = rows; the activation live in
+// one lane group per instruction; lane l, register v is (weight row l % 16, activation row 4 (l / 16) + v)
+// for each of the four groups, so a lane's sums are complete across groups).
 // D: super-blocks of loads a wave keeps in flight (4 in workgroups of at most eight waves, else 2).
 // tw: row tiles of a workgroup; a tile's nb / 8 granules go to as many waves.
-template <bool T8, int D>
+template <int TOKS, int D>
 __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args p, int n_tiles, int tw) {
-    constexpr int TOKS = T8 ? 8 : 4;
+    constexpr bool T8 = TOKS == 8, T16 = TOKS == 16;
+    constexpr int ZERO_BYTES = TOKS * 256;   // the zero lanes' run: the largest offset a step adds, and 16
     constexpr int BLK = TOKS * 32;       // LDS bytes of one Q8_1 block's codes, all rows
     extern __shared__ __align__(16) uint8_t lds[];
     uint8_t* codes = lds;                                               // [nb * 8][TOKS][32]
@@ -205,7 +208,11 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
     // ---- the lane's pieces of the activation operand (zeros where its lane group is not the slot's)
     const uint8_t *pa, *pb = zeros;
     int step_a, step_b = 0;
-    if constexpr (T8) {
+    if constexpr (T16) {
+        // slot l16 is row l16; the lane's group is live in the instruction of that group alone
+        pa = codes + (grp >> 1) * BLK + l16 * 32 + 16 * (grp & 1);
+        step_a = 8 * BLK;
+    } else if constexpr (T8) {
         const int sel = l16 >> 3, tok = l16 & 7;
         const bool live_a = grp < 2 && grp == sel, live_b = grp >= 2 && grp - 2 == sel;
         pa = live_a ? codes + tok * 32 + 16 * grp : zeros;
@@ -218,9 +225,10 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
         pa = live ? codes + (grp >> 1) * BLK + tok * 32 + 16 * (grp & 1) : zeros;
         step_a = live ? 8 * BLK : 0;
     }
-    // the lane's results: T8: groups grp / 2 and 2 + grp / 2, rows 4 (grp % 2) + v; else group grp, row v
-    const float* t_lane = T8 ? table + 4 * (grp & 1) : table + (grp >> 1) * TOKS;
-    const int sh_sc = T8 ? 8 * (grp >> 1) : 8 * grp;
+    // the lane's results: 8 rows: groups grp / 2 and 2 + grp / 2, rows 4 (grp % 2) + v; 4 rows: group grp,
+    // row v; 16 rows: every group, rows 4 grp + v
+    const float* t_lane = T16 ? table + 4 * grp : T8 ? table + 4 * (grp & 1) : table + (grp >> 1) * TOKS;
+    const int sh_sc = T16 ? 0 : T8 ? 8 * (grp >> 1) : 8 * grp;
     const int sh_qh = 2 * (grp >> 1);
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -253,7 +261,23 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
                 // exactly: d * scale is an f16 times an int8 (18 significant bits), MAGIC * d * scale
                 // has 20, neither product rounds, and the fma rounds dot * d * scale once.
                 const v4i magic = {MAGIC_BITS, MAGIC_BITS, MAGIC_BITS, MAGIC_BITS};
-                if constexpr (T8) {
+                if constexpr (T16) {
+                    // instruction g: the activation of group g alone (zeros in the other lane groups)
+                    const v4i a_live = *(const v4i*)(a_blk + blk * BLK);
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        v4i a;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) a[e] = grp == g ? a_live[e] : 0;
+                        const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, magic, 0, 0, 0);
+                        const float dsc = d * (float)(int)__builtin_amdgcn_sbfe(scw, 8 * g, 8);
+                        const float off = -MAGIC * dsc;
+                        const float4 t = *(const float4*)(t_blk + (blk + (g >> 1)) * TOKS);
+                        const float d8[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) acc[v] = fmaf(fmaf(__int_as_float(c[v]), dsc, off), d8[v], acc[v]);
+                    }
+                } else if constexpr (T8) {
                     const v4i a0 = *(const v4i*)(a_blk + blk * BLK);
                     const v4i a1 = *(const v4i*)(b_blk + blk * BLK);
                     const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, magic, 0, 0, 0);
@@ -300,19 +324,21 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
             acc[v] = 0.f;
         }
         __syncthreads();
-        // T8: output (tile ts, register v, lane l < 32) adds the S waves' lanes l and l + 32; else
-        // output (ts, v, l < 16) adds their lanes l, l + 16, l + 32, l + 48
-        constexpr int PER_TILE = T8 ? 128 : 64, LANES = T8 ? 32 : 16;
+        // 8 rows: output (tile ts, register v, lane l < 32) adds the S waves' lanes l and l + 32; 4 rows:
+        // output (ts, v, l < 16) adds their lanes l, l + 16, l + 32, l + 48; 16 rows: output (ts, v, l < 64)
+        // adds their lanes l
+        constexpr int LANES = T16 ? 64 : T8 ? 32 : 16, PER_TILE = 4 * LANES;
         for (int o = threadIdx.x; o < PER_TILE * tw; o += WG) {
             const int ts = o / PER_TILE, v = (o / LANES) & 3, l = o % LANES;
             float sum = 0.f;
             for (int sw = 0; sw < S; ++sw) {
                 const float* col = (const float*)(wbufs + (size_t)(ts * S + sw) * WBUF) + v * 64 + l;
-                if (T8) sum += col[0] + col[32];
+                if (T16) sum += col[0];
+                else if (T8) sum += col[0] + col[32];
                 else sum += (col[0] + col[16]) + (col[32] + col[48]);
             }
             const int tile = ((int)blockIdx.x + pass * stride) * tw + ts;
-            const int tok = T8 ? 4 * ((l >> 4) & 1) + v : v, row = tile * TILE + (l & 15);
+            const int tok = T16 ? 4 * (l >> 4) + v : T8 ? 4 * ((l >> 4) & 1) + v : v, row = tile * TILE + (l & 15);
             if (tile < n_tiles && tok < p.m && row < p.n) p.dst[(size_t)tok * p.ldd + row] = sum;
         }
         __syncthreads();   // the buffers may be overwritten
@@ -360,11 +386,10 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
     }
 }
 
-template <bool T8, int D>
+template <int TOKS, int D>
 int launch_shape(const Args& a, int tw, hipStream_t stream) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
-    constexpr int TOKS = T8 ? 8 : 4;
     const int waves = tw * (a.nb / GRAN);
     const int lds_bytes = lds_bytes_for<TOKS>(a.nb, waves);
     if (lds_bytes > lk_device().lds_bytes) return -1;
@@ -374,7 +399,7 @@ int launch_shape(const Args& a, int tw, hipStream_t stream) {
         if (it == by_lds.end()) {
             int ok = 1;
             if (lds_bytes > 48 * 1024 &&
-                hipFuncSetAttribute((const void*)q6k_rows16_kernel<T8, D>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                hipFuncSetAttribute((const void*)q6k_rows16_kernel<TOKS, D>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     lds_bytes) != hipSuccess) {
                 (void)hipGetLastError();
                 ok = 0;
@@ -390,30 +415,30 @@ int launch_shape(const Args& a, int tw, hipStream_t stream) {
     if (forced > 0) cap = forced;
     const int passes = (groups + cap - 1) / cap;
     const int wgs = (groups + passes - 1) / passes;
-    hipLaunchKernelGGL((q6k_rows16_kernel<T8, D>), dim3(wgs), dim3(64 * waves), lds_bytes, stream, a, n_tiles, tw);
+    hipLaunchKernelGGL((q6k_rows16_kernel<TOKS, D>), dim3(wgs), dim3(64 * waves), lds_bytes, stream, a, n_tiles, tw);
     return lk_launch_status();
 }
 
-template <bool T8>
+template <int TOKS>
 int launch(const Args& a, hipStream_t stream) {
     // Tiles per workgroup: as many as its sixteen waves and LDS hold while every CU still gets a workgroup.
-    constexpr int TOKS = T8 ? 8 : 4;
     const int s = a.nb / GRAN, n_tiles = (a.n + TILE - 1) / TILE, cus = lk_device().cus;
     int tw = 1;
     while (2 * tw * s <= MAX_WAVES && n_tiles >= 2 * tw * cus && lds_bytes_for<TOKS>(a.nb, 2 * tw * s) <= lk_device().lds_bytes) tw *= 2;
     const int forced = lk_tune_env("LK_TUNE_ROWS16_TW");
     if (forced > 0 && forced * s <= MAX_WAVES) tw = forced;
-    return tw * s <= 8 ? launch_shape<T8, 4>(a, tw, stream) : launch_shape<T8, 2>(a, tw, stream);
+    return tw * s <= 8 ? launch_shape<TOKS, 4>(a, tw, stream) : launch_shape<TOKS, 2>(a, tw, stream);
 }
 
 }  // namespace
 
 int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y, int ldd,
                   hipStream_t stream) {
-    if (size_m < 1 || size_m > 8 || size_n < 1 || size_k < 256) return -1;
+    if (size_m < 1 || size_m > 16 || size_n < 1 || size_k < 256) return -1;
     // rows of whole granules, on 16-byte boundaries; a tile's granules within one workgroup
     if (size_k % (256 * GRAN) != 0 || size_k / (256 * GRAN) > MAX_WAVES || (((uintptr_t)w) & 15) != 0) return -1;
     if (lk_tune_env("LK_TUNE_ROWS16_OFF") != 0) return -1;
     const Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd};
-    return size_m <= 4 ? launch<false>(a, stream) : launch<true>(a, stream);
+    if (size_m > 8 && lk_tune_env("LK_TUNE_ROWS16_MAX8") != 0) return -1;
+    return size_m <= 4 ? launch<4>(a, stream) : size_m <= 8 ? launch<8>(a, stream) : launch<16>(a, stream);
 }

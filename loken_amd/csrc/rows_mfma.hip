@@ -727,9 +727,10 @@ template <bool DUAL, bool Q5>
 int launch_any(const Args& a, hipStream_t stream) {
     // at most 8 / 16 activation rows in all: the fix-up runs on the registers those rows live in,
     // and the activation is staged in LDS when it fits there
-    if (a.m <= 8) {
+    if (a.m <= 16) {
         // 16-row tiles (rows16_mfma.hip): half the matrix-unit time per weight, twice the tiles
-        if (lk_rows16_serves(a.m, a.nb) && lk_tune_env("LK_TUNE_ROWS16_OFF") == 0) {
+        if (lk_rows16_serves(a.m, a.nb) && lk_tune_env("LK_TUNE_ROWS16_OFF") == 0 &&
+            (a.m <= 8 || lk_tune_env("LK_TUNE_ROWS16_MAX8") == 0)) {
             LkRows16 r{};
             r.w[0] = a.w; r.w[1] = a.w2;
             r.dst[0] = a.dst;
@@ -739,6 +740,8 @@ int launch_any(const Args& a, hipStream_t stream) {
             r.y = a.y; r.nb = a.nb; r.m = a.m; r.stride_y = a.stride_y; r.gelu = a.gelu;
             return lk_rows16_launch(r, DUAL, Q5, stream);
         }
+    }
+    if (a.m <= 8) {
         const int rc = launch_staged<1, DUAL, Q5>(a, stream);
         return rc >= 0 ? rc : launch_rows<1, DUAL, Q5>(a, stream);
     }
@@ -806,7 +809,7 @@ extern "C" void loken_dense_q4k_imma_m8_actmul(const void* gate, const void* up,
 // Up to three Q4_K (q5 != 0: Q5_K) matrices over the same plain Q8_1 rows in one launch (q + k + v of a
 // decode step): outputs[i] is [size_m, sizes_n[i]] f32. The reference issues one
 // loken_dense_q4k_imma_m8_plain per matrix (dense_q4k_imma_m8_matmul, src/inference/moe_cuda/dense/
-// imma.rs:82-135); the results equal those launches' bit for bit. At most 8 rows go out as one
+// imma.rs:82-135); the results equal those launches' bit for bit. At most 16 rows go out as one
 // launch; more rows (or rows whose codes do not fit in LDS) fall back to one launch per matrix.
 extern "C" int lk_dense_q4k_rows_multi(const void* const* weights, float* const* outputs, const int* sizes_n, int count,
                                        const void* q8_1, int size_m, int size_k, int q5, void* stream) {
@@ -815,7 +818,8 @@ extern "C" int lk_dense_q4k_rows_multi(const void* const* weights, float* const*
     for (int i = 0; i < count; ++i)
         if (sizes_n[i] > 0 && bad_rows_call(weights[i], q8_1, outputs[i], size_m, sizes_n[i], size_k)) return LK_ERR_ARG;
     const int nb = size_k / 256;
-    if (lk_rows16_serves(size_m, nb) && lk_tune_env("LK_TUNE_ROWS16_OFF") == 0) {
+    if (lk_rows16_serves(size_m, nb) && lk_tune_env("LK_TUNE_ROWS16_OFF") == 0 &&
+        (size_m <= 8 || lk_tune_env("LK_TUNE_ROWS16_MAX8") == 0)) {
         LkRows16 r{};
         for (int i = 0; i < count; ++i) {
             if (sizes_n[i] <= 0) continue;

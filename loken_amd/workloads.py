@@ -406,8 +406,44 @@ def decode_1p7b(args, dev):
     def rows_kernel_serves(wtype, n, rows):   # the rule of host_qmatmul.hip
         return (rows <= 16 or n * rows <= 1750000) if wtype == Q4K else n * rows <= (4 << 20)
 
+    # 3 to 16 rows: the 16-row-tile kernels on the matrix unit, the matrices that share an activation in
+    # one launch (q + k + v; gate + up with the activation on top, as dense_q4k_imma_m8_act_mul of the
+    # reference does)
+    fused_rows = 3 <= b <= 16 and args.mid_rows == "auto"
+    matvec = matvec and not fused_rows
+
+    def add_fused_rows(g, k, wtype, ns):
+        nonlocal total_bytes
+        weights = [mk.make(wtype, n, k) for n in ns]
+        keep.extend(weights)
+        total_bytes += sum(synth.weight_bytes(wtype, n, k) for n in ns)
+        x = acts[g]
+        q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
+        keep.append(q)
+        plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s)))
+        used["rows"] += len(ns)
+        if wtype == Q6K:
+            for w, n in zip(weights, ns):
+                out = torch.empty((b, n), device=dev)
+                keep.append(out)
+                plan.append(("status", L.lk_dense_q6k_rows, (w.data_ptr(), q.data_ptr(), out.data_ptr(), b, n, k, s)))
+        elif g == "x2":
+            out = torch.empty((b, ns[0]), device=dev)
+            keep.append(out)
+            plan.append(("status", L.lk_dense_q4k_rows_actmul,
+                         (weights[0].data_ptr(), weights[1].data_ptr(), q.data_ptr(), out.data_ptr(), b, ns[0], k, 0, s)))
+        else:
+            outs = [torch.empty((b, n), device=dev) for n in ns]
+            vx = (lib.C.c_void_p * len(ns))(*[w.data_ptr() for w in weights])
+            dst = (lib.C.c_void_p * len(ns))(*[o.data_ptr() for o in outs])
+            nn = (lib.C.c_int * len(ns))(*ns)
+            keep.extend(outs + [vx, dst, nn])
+            plan.append(("status", L.lk_dense_q4k_rows_multi, (vx, dst, nn, len(ns), q.data_ptr(), b, k, 0, s)))
+
     def add_group(g, k, wtype, ns):
         nonlocal total_bytes
+        if fused_rows:
+            return add_fused_rows(g, k, wtype, ns)
         weights = [mk.make(wtype, n, k) for n in ns]
         keep.extend(weights)
         total_bytes += sum(synth.weight_bytes(wtype, n, k) for n in ns)
@@ -508,6 +544,8 @@ def decode_1p7b(args, dev):
                 {"workload": f"qwen3-1.7b decode-step quantized linears (Q4_K attention and gate/up, Q6_K down and "
                              f"lm_head), batch {b}, 28 layers",
                  "path": "mat-vec (fused; own quantizer launch for rows over 8192 values)" if matvec
+                         else "16-row tiles on the matrix unit: q + k + v in one launch, o, gate + up with SiLU in one, down, lm_head, "
+                              "each after a Q8_1 quantizer launch" if fused_rows
                          else f"linears on the matrix-unit rows kernels: {used['rows']}, as mat-vec slices of eight rows: "
                               f"{used['matvec']}, on the tiled matmul: {used['tiled']}",
                  "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline)

@@ -204,7 +204,9 @@ def test_q6k_rows_emit_the_exact_integers_on_crafted_inputs():
 # At most eight rows: 16-row tiles on v_mfma_i32_16x16x64_i8 (rows16_mfma.hip)
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("m,k,n", [(1, 256, 1), (2, 256, 15), (3, 512, 17), (4, 768, 16), (7, 1024, 31), (8, 1280, 48),
-                                   (8, 4096, 1000), (6, 4096, 4096), (8, 11008, 50), (5, 2048, 16400), (3, 256, 16500)])
+                                   (8, 4096, 1000), (6, 4096, 4096), (8, 11008, 50), (5, 2048, 16400), (3, 256, 16500),
+                                   (9, 256, 1), (10, 512, 17), (13, 1024, 31), (16, 1280, 48), (16, 4096, 1000), (12, 2048, 4096),
+                                   (15, 11008, 50), (11, 2048, 16400), (16, 256, 16500)])
 @pytest.mark.parametrize("wtype", [Q4K, lib.TYPE_Q5_K])
 def test_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n, wtype):
     """Ragged tile edges (n not a multiple of 16), rows of one to 43 super-blocks (waves with no
@@ -216,13 +218,14 @@ def test_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n, wtype):
     assert_close(got, oracle.ob_matmul(wtype, x, w, n))
 
 
-def test_eight_rows_emit_the_exact_integers_on_crafted_inputs():
+@pytest.mark.parametrize("m", [8, 16])
+def test_eight_rows_emit_the_exact_integers_on_crafted_inputs(m):
     """Activations on an integer grid with 127 in every block (d8 = 1); weights with d = 1, dmin = 0
     and scale 1 in ONE sub-block of each super-block, 0 in the others: the f32 output is that
     sub-block's integer dot, so a code that strays into the neighbouring sub-block of its
     instruction (or a lane that should hold zeros and does not) shows."""
     rng = np.random.default_rng(71)
-    m, k, n = 8, 1024, 80
+    k, n = 1024, 80
     nb = k // 256
     x = rng.integers(-127, 128, size=(m, k)).astype(np.float32)
     x.reshape(m, k // 32, 32)[:, :, 0] = 127.0
@@ -242,7 +245,7 @@ def test_eight_rows_emit_the_exact_integers_on_crafted_inputs():
     assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, got.astype(np.int64))
 
 
-@pytest.mark.parametrize("m", [1, 5, 8, 11])
+@pytest.mark.parametrize("m", [1, 5, 8, 11, 16, 19])
 @pytest.mark.parametrize("q5", [False, True])
 def test_three_matrices_in_one_launch_carry_the_single_launches_bits(m, q5):
     """q + k + v: lk_dense_q4k_rows_multi against one lk_dense_q4k_rows per matrix."""
@@ -257,7 +260,7 @@ def test_three_matrices_in_one_launch_carry_the_single_launches_bits(m, q5):
     assert torch.equal(two[0], outs[0]) and torch.equal(two[1], outs[1])
 
 
-@pytest.mark.parametrize("m,k,n", [(8, 4096, 8200), (2, 512, 9000)])
+@pytest.mark.parametrize("m,k,n", [(8, 4096, 8200), (2, 512, 9000), (14, 2048, 8200)])
 def test_gate_and_up_of_many_row_tiles(m, k, n):
     """The dual launch with four tiles (two gate, two up) per workgroup: bits of the plain launches."""
     gate, up = dev(synth.weight(Q4K, n, k, seed=73, stream=1)), dev(synth.weight(Q4K, n, k, seed=73, stream=2))
@@ -271,7 +274,8 @@ def test_gate_and_up_of_many_row_tiles(m, k, n):
 
 
 @pytest.mark.parametrize("m,k,n", [(1, 256, 1), (2, 512, 15), (3, 768, 17), (4, 1024, 33), (4, 14336, 48), (5, 256, 16), (7, 1280, 100),
-                                   (8, 6144, 500), (6, 2048, 8300), (3, 512, 8300), (8, 512, 16500), (4, 256, 16500)])
+                                   (8, 6144, 500), (6, 2048, 8300), (3, 512, 8300), (8, 512, 16500), (4, 256, 16500),
+                                   (9, 2048, 17), (12, 6144, 500), (16, 4096, 100), (16, 2048, 8300), (13, 2048, 16500)])
 def test_q6k_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n):
     """rows16_q6k.hip: both slot layouts (up to four rows, up to eight), ragged tile edges, rows of
     one super-block (waves with nothing to add), one, two and four tiles per workgroup."""
@@ -282,7 +286,7 @@ def test_q6k_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n):
 
 
 @pytest.mark.parametrize("k", [1024, 4096])
-@pytest.mark.parametrize("m", [3, 4, 7])
+@pytest.mark.parametrize("m", [3, 4, 7, 11, 16])
 def test_q6k_few_rows_emit_the_exact_integers_on_crafted_inputs(m, k):
     """As test_q6k_rows_emit_the_exact_integers_on_crafted_inputs, for the launches of at most four
     and at most eight rows: one group of each super-block has scale 1, the others 0, so a code that
