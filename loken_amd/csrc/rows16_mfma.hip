@@ -36,6 +36,7 @@
 
 #include "lk_common.h"
 #include "rows16.h"
+#include "rows16_core.h"
 
 #include <mutex>
 #include <unordered_map>
@@ -44,22 +45,13 @@ namespace {
 
 constexpr int KSPLIT = 4;   // waves that share a row tile
 constexpr int MAX_TOKS = 16;   // activation rows a launch serves: kernels for up to 8 and up to 16
-constexpr int TILE = 16;    // weight rows of a wave's tile
-static __host__ __device__ constexpr int zero_bytes(int toks) { return toks * 256; }   // the zero lanes' run
-
-struct WFrag {
-    uint4 hdr, q[2], qh;   // qh: Q5_K only
-};
-
-template <bool Q5>
-struct Blk {
-    static constexpr int BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES;
-    static constexpr int QS = Q5 ? 48 : 16;
-};
+using rows16::Blk;
+using rows16::TILE;
+using rows16::WFrag;
 
 static __host__ __device__ constexpr int lds_bytes_for(int nb, int tiles, int toks) {
-    // codes [nb * 8][toks][32], zeros, d8 and d8 * S [nb * 8][2][toks] floats, reduce [4 tiles][4][64] floats
-    return nb * 8 * toks * 32 + zero_bytes(toks) + nb * 8 * 2 * toks * 4 + KSPLIT * tiles * 4 * 64 * 4;
+    // the staged activation, reduce [4 tiles][4][64] floats
+    return rows16::staged_bytes(nb, toks) + KSPLIT * tiles * 4 * 64 * 4;
 }
 
 // Element `i` of a three-entry kernel argument without indexing it by a register (which would
@@ -93,22 +85,16 @@ static __device__ __forceinline__ TileRef tile_ref(const LkRows16& p, int vt) {
 template <bool DUAL, bool Q5, int STEPS, int TW, bool T16>
 __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(LkRows16 p, int n_vt) {
     constexpr int WG = 256 * TW;
-    constexpr int TOKS = T16 ? 16 : 8;
-    constexpr int ZERO_BYTES = zero_bytes(TOKS);
     extern __shared__ __align__(16) uint8_t lds[];
-    uint8_t* codes = lds;                                               // [nb * 8][8][32]
-    uint8_t* zeros = codes + (size_t)p.nb * 8 * TOKS * 32;              // ZERO_BYTES
-    float* table = (float*)(zeros + ZERO_BYTES);                        // [nb * 8][2][TOKS]: d8, d8 * S
-    float* reduce = table + p.nb * 8 * 2 * TOKS;                        // [4 TW][4][64]
+    rows16::Core<Q5, T16> core;
+    float* reduce = (float*)core.init(lds, p.nb);                       // [4 TW][4][64]
+    const rows16::RowsIn rows{p.y, p.stride_y, nullptr, 0};
 
-    const int lane = threadIdx.x & 63;
+    const int lane = core.lane, l16 = core.l16;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int tsel = wave >> 2, kq = wave & 3;   // which tile of the workgroup's TW, which share of its super-blocks
-    const int l16 = lane & 15, grp = lane >> 4;
-    const int half = grp & 1;   // which sixteen values of a sub-block (operands), which four rows (results)
-    const int par = grp >> 1;   // which of an instruction's two sub-blocks
     const size_t row_bytes = (size_t)p.nb * Blk<Q5>::BYTES;
-    const int entries = p.nb * 8 * TOKS;
+    const int entries = p.nb * 8 * core.TOKS;
     const int n_pairs = (n_vt + TW - 1) / TW;   // tile groups of the launch
     const int my_blocks = STEPS ? STEPS : (p.nb - kq + KSPLIT - 1) / KSPLIT;
 
@@ -118,132 +104,15 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
         const int row = min(t.row0 + l16, (DUAL ? p.n[0] : pick3(p.n, t.mat)) - 1);
         return (const uint8_t*)(to_gbytes(pick3(p.w, t.mat)) + row * row_bytes + (size_t)kq * Blk<Q5>::BYTES);
     };
-    auto loadw = [&](WFrag& f, const uint8_t* bp) {
-        f.hdr = *(const uint4*)bp;
-        if (Q5) f.qh = *(const uint4*)(bp + 16 + 16 * half);
-        f.q[0] = *(const uint4*)(bp + Blk<Q5>::QS + 16 * grp);
-        f.q[1] = *(const uint4*)(bp + Blk<Q5>::QS + 64 + 16 * grp);
-    };
+    auto loadw = [&](WFrag& f, const uint8_t* bp) { core.loadw(f, bp); };
     constexpr size_t STEP_BYTES = (size_t)KSPLIT * Blk<Q5>::BYTES;   // between a wave's consecutive super-blocks
-
-    // The activation: entry (sub-block, row) is one Q8_1 block. Its loads go out before the first
-    // weight loads and are consumed after them (loads return in issue order: asked for after the
-    // weights, the activation, which sits in L2, would wait for HBM).
-    constexpr int PER = 2;
-    uint32_t head[PER];
-    uint4 lo[PER], hi[PER];
-    auto issue = [&](int base) {
-#pragma unroll
-        for (int u = 0; u < PER; ++u) {
-            const int idx = min(base + u * WG, entries - 1);
-            const int sub = idx / TOKS, tok = min(idx % TOKS, p.m - 1);
-            const uint8_t* b = p.y + ((size_t)tok * p.stride_y + sub) * Q81_BYTES;
-            head[u] = *(const uint32_t*)b;
-            lo[u] = *(const uint4_a4*)(b + 4);
-            hi[u] = *(const uint4_a4*)(b + 20);
-        }
-    };
-    auto place = [&](int base) {
-        const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
-#pragma unroll
-        for (int u = 0; u < PER; ++u) {
-            const int idx = base + u * WG;
-            if (idx < entries) {
-                const int sub = idx / TOKS, tok = idx % TOKS;
-                const bool real = tok < p.m;
-                const float d8 = real ? f16_bits_to_f32(head[u] & 0xFFFFu) : 0.f;
-                table[sub * 2 * TOKS + tok] = d8;
-                table[sub * 2 * TOKS + TOKS + tok] = d8 * (float)dot16(ones, hi[u], dot16(ones, lo[u], 0));
-                const uint32_t keep = real ? 0xFFFFFFFFu : 0u;   // rows the launch does not have: zeros
-                *(uint4*)(codes + (size_t)idx * 32) = make_uint4(lo[u].x & keep, lo[u].y & keep, lo[u].z & keep, lo[u].w & keep);
-                *(uint4*)(codes + (size_t)idx * 32 + 16) = make_uint4(hi[u].x & keep, hi[u].y & keep, hi[u].z & keep, hi[u].w & keep);
-            }
-        }
-    };
-
-    // The lane's piece of the activation operand. Up to eight rows: slot l16 is (sub-block l16 / 8 of the
-    // two, row l16 % 8); the lane's K group belongs to sub-block par; where the two differ the piece is
-    // zeros: those lanes read the run of zeros, at a stride of nothing. Up to sixteen rows: slot l16 is row
-    // l16, and there are two pieces, one per run of the instruction: live for the lanes of sub-block 0
-    // (groups 0, 1) in the first, for those of sub-block 1 in the second.
-    const bool live = T16 ? par == 0 : (l16 >> 3) == par;
-    const bool live2 = T16 && par == 1;
-    const uint8_t* a_lane = live ? codes + (T16 ? l16 : 2 * par * TOKS + (l16 & 7)) * 32 + 16 * half : zeros;
-    const uint8_t* a_lane2 = live2 ? codes + (2 * TOKS + l16) * 32 + 16 * half : zeros;
-    const int a_step = live ? 8 * TOKS * 32 : 0;   // bytes per super-block
-    const int a_step2 = live2 ? 8 * TOKS * 32 : 0;
-    // the lane's results: up to eight rows: sub-blocks 2 par + {0, 1, 4, 5}, rows 4 half .. 4 half + 3;
-    // up to sixteen: every sub-block, rows 4 grp .. 4 grp + 3
-    const float* t_lane = T16 ? table + 4 * grp : table + 2 * par * 2 * TOKS + 4 * half;
-    const int sh16 = T16 ? 0 : 16 * par, sh2 = 2 * par;
+    // The activation's first loads go out before the first weight loads and are consumed after them
+    // (loads return in issue order: asked for after the weights, the activation, which sits in L2, would
+    // wait for HBM).
+    auto issue = [&](int base) { core.issue(rows, p.m, entries, base, WG); };
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-
-    auto compute = [&](const WFrag& w, int kb) {
-        // the row's (scale, min) pairs of sub-blocks 2 par, 2 par + 1, 4 + 2 par, 5 + 2 par, six bits
-        // each (get_scale_min_k4 of the format)
-        const uint32_t w1 = w.hdr.y, w2 = w.hdr.z, w3 = w.hdr.w;
-        const uint32_t sc_lo = (w1 & 0x3F3F3F3Fu) >> sh16, mn_lo = (w2 & 0x3F3F3F3Fu) >> sh16;
-        const uint32_t sc_hi = ((w3 & 0x0F0F0F0Fu) | ((w1 >> 2) & 0x30303030u)) >> sh16;
-        const uint32_t mn_hi = (((w3 >> 4) & 0x0F0F0F0Fu) | ((w2 >> 2) & 0x30303030u)) >> sh16;
-        const float d = f16_bits_to_f32(w.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(w.hdr.x >> 16);
-        uint32_t hp[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
-        if (Q5) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) hp[e] >>= sh2;
-        }
-        const uint8_t* a_blk = a_lane + (size_t)kb * a_step;
-        const uint8_t* a_blk2 = a_lane2 + (size_t)kb * a_step2;
-        const float* t_blk = t_lane + kb * 8 * 2 * TOKS;
-        // The accumulators start at the bit pattern of 1.5 * 2^23: adding an integer of magnitude below
-        // 2^22 to that pattern yields the float 1.5 * 2^23 + integer, so the dots leave the matrix unit
-        // as floats. The offset goes in the first fused multiply-add, exactly: d * sc is an f16 times a
-        // six-bit integer (17 significant bits), MAGIC * d * sc has 19, neither product rounds, and the
-        // fma rounds dot * d * sc once, as convert-then-multiply would.
-        constexpr int MAGIC_BITS = 0x4B400000;
-        constexpr float MAGIC = 12582912.0f;
-        const v4i magic = {MAGIC_BITS, MAGIC_BITS, MAGIC_BITS, MAGIC_BITS};
-        // one instruction's four results into the sums: sub-block `sub` of the super-block
-        auto fold = [&](const v4i& c, float dsc, float dmm, int sub) {
-            const float off = -MAGIC * dsc;
-            const float4 t = *(const float4*)(t_blk + sub * 2 * TOKS);
-            const float4 s = *(const float4*)(t_blk + sub * 2 * TOKS + TOKS);
-            acc[0] = fmaf(fmaf(__int_as_float(c[0]), dsc, off), t.x, fmaf(dmm, s.x, acc[0]));
-            acc[1] = fmaf(fmaf(__int_as_float(c[1]), dsc, off), t.y, fmaf(dmm, s.y, acc[1]));
-            acc[2] = fmaf(fmaf(__int_as_float(c[2]), dsc, off), t.z, fmaf(dmm, s.z, acc[2]));
-            acc[3] = fmaf(fmaf(__int_as_float(c[3]), dsc, off), t.w, fmaf(dmm, s.w, acc[3]));
-        };
-#pragma unroll
-        for (int c2 = 0; c2 < 2; ++c2) {
-            const uint32_t u[4] = {w.q[c2].x, w.q[c2].y, w.q[c2].z, w.q[c2].w};
-#pragma unroll
-            for (int nib = 0; nib < 2; ++nib) {
-                v4i b;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    uint32_t x = (nib ? u[e] >> 4 : u[e]) & 0x0F0F0F0Fu;
-                    if (Q5) x |= ((hp[e] >> (4 * c2 + nib)) & 0x01010101u) << 4;
-                    b[e] = (int)x;
-                }
-                const uint32_t scw = c2 ? sc_hi : sc_lo, mnw = c2 ? mn_hi : mn_lo;
-                if constexpr (T16) {
-                    // sub-blocks 4 c2 + nib (lane groups 0, 1) and 4 c2 + 2 + nib (groups 2, 3)
-                    const v4i a0 = *(const v4i*)(a_blk + (4 * c2 + nib) * TOKS * 32);
-                    const v4i a1 = *(const v4i*)(a_blk2 + (4 * c2 + nib) * TOKS * 32);
-                    const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, magic, 0, 0, 0);
-                    const v4i c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b, magic, 0, 0, 0);
-                    fold(c0, d * (float)((scw >> (8 * nib)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib)) & 0xFFu)), 4 * c2 + nib);
-                    fold(c1, d * (float)((scw >> (8 * nib + 16)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib + 16)) & 0xFFu)),
-                         4 * c2 + 2 + nib);
-                } else {
-                    // this lane's sub-block: 4 c2 + 2 par + nib (its scale words are shifted to it)
-                    const v4i a = *(const v4i*)(a_blk + (4 * c2 + nib) * TOKS * 32);
-                    const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, magic, 0, 0, 0);
-                    fold(c, d * (float)((scw >> (8 * nib)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib)) & 0xFFu)), 4 * c2 + nib);
-                }
-            }
-        }
-    };
+    auto compute = [&](const WFrag& w, int kb) { core.compute(w, kb, acc); };
 
     // Adds the partial tiles of the workgroup's row tiles (tiles vt0 .. vt0 + TW - 1) and writes them.
     auto finish_pair = [&](int vt0) {
@@ -284,12 +153,7 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
     };
 
     auto stage = [&]() {
-        place(threadIdx.x);
-        for (int r = WG * PER; r < entries; r += WG * PER) {
-            issue(r + threadIdx.x);
-            place(r + threadIdx.x);
-        }
-        for (int i = threadIdx.x * 16; i < ZERO_BYTES; i += WG * 16) *(uint4*)(zeros + i) = make_uint4(0, 0, 0, 0);
+        core.finish_staging(rows, p.m, p.nb, WG);
         __syncthreads();
     };
 
@@ -416,9 +280,11 @@ int launch_steps(const LkRows16& a, hipStream_t stream) {
     int tw = n_vt >= 4 * lk_device().cus ? 4 : 2;
     const int forced = lk_tune_env("LK_TUNE_ROWS16_TW");
     if (forced == 2 || forced == 4) tw = forced;
-    if (tw == 4) {
-        const int rc = launch_shape<DUAL, Q5, STEPS, 4, T16>(a, n_vt, stream);
-        if (rc >= 0) return rc;
+    if constexpr (STEPS != 0) {   // (the any-row-length path at sixteen waves would not fit the register file)
+        if (tw == 4) {
+            const int rc = launch_shape<DUAL, Q5, STEPS, 4, T16>(a, n_vt, stream);
+            if (rc >= 0) return rc;
+        }
     }
     return launch_shape<DUAL, Q5, STEPS, 2, T16>(a, n_vt, stream);
 }
