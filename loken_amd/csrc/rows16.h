@@ -16,6 +16,21 @@ struct LkRows16 {
 bool lk_rows16_serves(int size_m, int nb);
 int lk_rows16_launch(const LkRows16& a, bool dual, bool q5, hipStream_t stream);
 
+// Q4_K per expert over a sorted routing, a wave per 16-row tile (rows16_moe.hip): expert e's matrices are
+// a.w[..] + e * expert_bytes (a.n[0] rows each, a.w[1] with `dual`), its rows the sorted rows
+// [bounds[e], bounds[e + 1]) (`src`: sorted row -> row of a.y, `dst_map`: sorted row -> output row; either
+// may be null: the sorted row itself). `rows_hint`: the rows an expert is expected to own (up to 8: passes
+// of 8; up to 16: passes of 16). LK_* status, or -1 when the launch does not serve the call (rows of a
+// super-block count it is not compiled for, more rows expected).
+struct LkRows16Experts {
+    const int32_t* bounds;
+    const int32_t* src;
+    const int32_t* dst_map;
+    int64_t expert_bytes;
+};
+int lk_rows16_launch_experts(const LkRows16& a, const LkRows16Experts& m, int n_experts, bool dual, int rows_hint,
+                             hipStream_t stream);
+
 // Q6_K x at most sixteen Q8_1 rows in 16-row tiles (rows16_q6k.hip). LK_* status, or -1 when the launch
 // does not serve the call (more rows, k not a multiple of 2048, or rows whose codes do not fit in LDS).
 int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y, int ldd,

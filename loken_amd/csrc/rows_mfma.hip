@@ -888,6 +888,19 @@ extern "C" int lk_moe_q4k_rows_grouped(const void* weights, const void* weights_
            (const uint8_t*)weights_second, act ? 1 : 0};
     const MoeRows m{bounds, src_rows, dst_rows, expert_bytes};
     if (rows_hint < 1) rows_hint = 1;
+    {
+        // rows of at most eight super-blocks: a wave per 16-row tile, passes of 8 or 16 rows (rows16_moe.hip)
+        LkRows16 r{};
+        r.w[0] = (const uint8_t*)weights; r.w[1] = (const uint8_t*)weights_second;
+        r.dst[0] = output;
+        r.n[0] = r.n[1] = size_n;
+        r.ldd[0] = ldd;
+        r.count = weights_second ? 2 : 1;
+        r.y = (const uint8_t*)q8_1; r.nb = size_k / 256; r.stride_y = stride_blocks; r.gelu = act ? 1 : 0;
+        const LkRows16Experts ex{bounds, src_rows, dst_rows, expert_bytes};
+        const int rc = lk_rows16_launch_experts(r, ex, n_experts, weights_second != nullptr, rows_hint, (hipStream_t)stream);
+        if (rc >= 0) return rc;
+    }
     return weights_second ? launch_moe_any<true>(a, m, n_experts, rows_hint, (hipStream_t)stream)
                           : launch_moe_any<false>(a, m, n_experts, rows_hint, (hipStream_t)stream);
 }

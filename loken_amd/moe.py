@@ -102,11 +102,12 @@ class MmqRouting:
             raise _lib.LokenError(MMQ_MOE_LAUNCHER[wtype], _lib.LK_ERR_ARG)
 
     # Rows an expert is expected to own up to which the matrix-unit rows launch (weights straight from
-    # HBM into the operand, one pass per 8 / 16 / 32 rows) beats the tiled one (weights expanded into
-    # LDS per 32 tokens). Measured on MI355X at 128 experts of 2048 -> 768 -> 2048, top-8: 64 tokens
-    # 136 us against 167, 128 tokens 168 against 170, 256 tokens 193 against 182 (the expected longest
-    # run is 17 at 128 tokens).
-    ROWS_LAUNCH_MAX_RUN = 17
+    # HBM into the operand, a wave per 16-row tile, one pass per 16 rows) beats the tiled one (weights
+    # expanded into LDS per 32 tokens). Measured on MI355X at 128 experts of 2048 -> 768 -> 2048, top-8:
+    # 64 tokens 112 us against 173, 128 tokens 117 against 170, 256 tokens 173 against 182, 384 tokens
+    # 232 against 259, 512 tokens 273 against 271, 1024 tokens 444 against 408 (the expected longest run
+    # is 17 at 128 tokens, 39 at 384, 50 at 512).
+    ROWS_LAUNCH_MAX_RUN = 40
 
     def takes_rows_launch(self, wtype: int, k: int) -> bool:
         return (self.path != "tiled" and wtype == _lib.TYPE_Q4_K and k % 256 == 0
@@ -410,10 +411,10 @@ def moe_mmq_pays(rows: int, experts: int, wtype: int | None = None) -> bool:
     breaks even at one routed row per expert (mmq_experts.rs:72-86); on MI355X, with this
     library's kernels, the mat-vec per routed pair stays ahead of the tiled matmul up to three rows
     per expert (Qwen3-30B-A3B shapes: 117 us against 162 us at 32 tokens, 176 against 168 at 48), and
-    of the matrix-unit rows launch that Q4_K stacks take at short runs up to 2.25 (32 tokens: 114 us
-    against 120; 48: 174 against 133; 96: 321 against 141)."""
+    of the matrix-unit rows launch that Q4_K stacks take at short runs up to 1.125 (16 tokens: 69 us
+    against 77; 20: 89 against 81; 32: 113 against 94)."""
     if wtype == _lib.TYPE_Q4_K:
-        return 4 * rows >= 9 * max(experts, 1)
+        return 8 * rows >= 9 * max(experts, 1)
     return rows >= 3 * max(experts, 1)
 
 

@@ -522,12 +522,14 @@ def test_q4k_pair_rows_over_caller_quantized_rows_with_one_expert_per_pair(token
 
 
 @pytest.mark.parametrize("hint", [1, 9, 40])
-@pytest.mark.parametrize("k", [512, 2560])   # a wave per row tile (at most 8 super-blocks), or four waves splitting a tile's
+# a wave per 16-row tile (1, 2, 3, 4, 6, 8 super-blocks: every load depth), a wave per 32-row tile (5), or four
+# waves splitting a tile's super-blocks (10)
+@pytest.mark.parametrize("k", [256, 512, 768, 1024, 1280, 1536, 2048, 2560])
 def test_rows_launch_serves_any_run_length_whatever_the_hint(hint, k):
     """lk_moe_q4k_rows_grouped: the hint only picks the pass width (8, 16 or 32 rows); an expert with
     more rows takes more passes, one without rows none, and gather / scatter follow the routing."""
     rng = np.random.default_rng(67)
-    n_experts, n, tokens = 5, 96, 30
+    n_experts, n, tokens = 5, 100, 30
     counts = [37, 0, 1, 9, 13]                              # sorted rows per expert
     rows = sum(counts)
     bounds = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
