@@ -19,9 +19,10 @@ namespace rows16 {
 
 constexpr int TILE = 16;   // weight rows of a wave's tile
 static __host__ __device__ constexpr int zero_bytes(int toks) { return toks * 256; }   // the zero lanes' run
-// LDS bytes of the staged activation: codes [nb * 8][toks][32], zeros, d8 and d8 * S [nb * 8][2][toks] floats
-static __host__ __device__ constexpr int staged_bytes(int nb, int toks) {
-    return nb * 8 * toks * 32 + zero_bytes(toks) + nb * 8 * 2 * toks * 4;
+// LDS bytes of the staged activation, `chunks` groups of `toks` rows: codes [chunks][nb * 8][toks][32], zeros,
+// d8 and d8 * S [chunks][nb * 8][2][toks] floats
+static __host__ __device__ constexpr int staged_bytes(int nb, int toks, int chunks = 1) {
+    return chunks * nb * 8 * toks * 32 + zero_bytes(toks) + chunks * nb * 8 * 2 * toks * 4;
 }
 
 struct WFrag {
@@ -56,18 +57,21 @@ struct Core {
     float* table;
     int lane, l16, grp, half, par;
     const uint8_t *a_lane, *a_lane2;
-    int a_step, a_step2;
+    int a_step, a_step2;       // bytes per super-block (nothing for the zero lanes)
+    int a_chunk, a_chunk2;     // bytes per chunk of rows (nothing for the zero lanes)
+    int t_chunk;               // floats per chunk of rows
     const float* t_lane;
     int sh16, sh2;
     // staging registers
     uint32_t head[PER];
     uint4 lo[PER], hi[PER];
 
-    // Sets the pointers for rows of `nb` super-blocks; returns the first LDS byte past the staged activation.
-    __device__ __forceinline__ uint8_t* init(uint8_t* lds, int nb) {
-        codes = lds;                                             // [nb * 8][TOKS][32]
-        zeros = codes + (size_t)nb * 8 * TOKS * 32;              // zero_bytes(TOKS)
-        table = (float*)(zeros + zero_bytes(TOKS));              // [nb * 8][2][TOKS]: d8, d8 * S
+    // Sets the pointers for `chunks` groups of TOKS rows of `nb` super-blocks; returns the first LDS byte
+    // past the staged activation.
+    __device__ __forceinline__ uint8_t* init(uint8_t* lds, int nb, int chunks = 1) {
+        codes = lds;                                             // [chunks][nb * 8][TOKS][32]
+        zeros = codes + (size_t)chunks * nb * 8 * TOKS * 32;     // zero_bytes(TOKS)
+        table = (float*)(zeros + zero_bytes(TOKS));              // [chunks][nb * 8][2][TOKS]: d8, d8 * S
         lane = threadIdx.x & 63;
         l16 = lane & 15;
         grp = lane >> 4;
@@ -82,40 +86,47 @@ struct Core {
         const bool live2 = T16 && par == 1;
         a_lane = live ? codes + (T16 ? l16 : 2 * par * TOKS + (l16 & 7)) * 32 + 16 * half : zeros;
         a_lane2 = live2 ? codes + (2 * TOKS + l16) * 32 + 16 * half : zeros;
-        a_step = live ? 8 * TOKS * 32 : 0;   // bytes per super-block
+        a_step = live ? 8 * TOKS * 32 : 0;
         a_step2 = live2 ? 8 * TOKS * 32 : 0;
+        a_chunk = live ? nb * 8 * TOKS * 32 : 0;
+        a_chunk2 = live2 ? nb * 8 * TOKS * 32 : 0;
+        t_chunk = nb * 8 * 2 * TOKS;
         // the lane's results: up to eight rows: sub-blocks 2 par + {0, 1, 4, 5}, rows 4 half .. 4 half + 3;
         // up to sixteen: every sub-block, rows 4 grp .. 4 grp + 3
         t_lane = T16 ? table + 4 * grp : table + 2 * par * 2 * TOKS + 4 * half;
         sh16 = T16 ? 0 : 16 * par;
         sh2 = 2 * par;
-        return (uint8_t*)(table + nb * 8 * 2 * TOKS);
+        return (uint8_t*)(table + chunks * nb * 8 * 2 * TOKS);
     }
 
-    // The activation: entry (sub-block, row) is one Q8_1 block. `issue` puts the loads of the entries
-    // base + u * threads in flight, `place` writes them to LDS (rows past m_count: zeros).
-    __device__ __forceinline__ void issue(const RowsIn& rows, int m_count, int entries, int base, int threads) {
+    // The activation: entry (chunk, sub-block, row of the chunk) is one Q8_1 block; `per_chunk` entries to a
+    // chunk. `issue` puts the loads of the entries base + u * threads in flight, `place` writes them to LDS
+    // (rows past m_count: zeros).
+    __device__ __forceinline__ void issue(const RowsIn& rows, int m_count, int entries, int per_chunk, int base, int threads) {
 #pragma unroll
         for (int u = 0; u < PER; ++u) {
             const int idx = min(base + u * threads, entries - 1);
-            const int sub = idx / TOKS, tok = min(idx % TOKS, m_count - 1);
+            const int chunk = idx / per_chunk, in_chunk = idx % per_chunk;
+            const int sub = in_chunk / TOKS, tok = min(chunk * TOKS + in_chunk % TOKS, m_count - 1);
             const uint8_t* b = rows.block(tok, sub);
             head[u] = *(const uint32_t*)b;
             lo[u] = *(const uint4_a4*)(b + 4);
             hi[u] = *(const uint4_a4*)(b + 20);
         }
     }
-    __device__ __forceinline__ void place(int m_count, int entries, int base, int threads) {
+    __device__ __forceinline__ void place(int m_count, int entries, int per_chunk, int base, int threads) {
         const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
 #pragma unroll
         for (int u = 0; u < PER; ++u) {
             const int idx = base + u * threads;
             if (idx < entries) {
-                const int sub = idx / TOKS, tok = idx % TOKS;
-                const bool real = tok < m_count;
+                const int chunk = idx / per_chunk, in_chunk = idx % per_chunk;
+                const int sub = in_chunk / TOKS, tok = in_chunk % TOKS;
+                const bool real = chunk * TOKS + tok < m_count;
                 const float d8 = real ? f16_bits_to_f32(head[u] & 0xFFFFu) : 0.f;
-                table[sub * 2 * TOKS + tok] = d8;
-                table[sub * 2 * TOKS + TOKS + tok] = d8 * (float)dot16(ones, hi[u], dot16(ones, lo[u], 0));
+                float* t = table + chunk * t_chunk + sub * 2 * TOKS + tok;
+                t[0] = d8;
+                t[TOKS] = d8 * (float)dot16(ones, hi[u], dot16(ones, lo[u], 0));
                 const uint32_t keep = real ? 0xFFFFFFFFu : 0u;   // rows the launch does not have: zeros
                 *(uint4*)(codes + (size_t)idx * 32) = make_uint4(lo[u].x & keep, lo[u].y & keep, lo[u].z & keep, lo[u].w & keep);
                 *(uint4*)(codes + (size_t)idx * 32 + 16) = make_uint4(hi[u].x & keep, hi[u].y & keep, hi[u].z & keep, hi[u].w & keep);
@@ -124,12 +135,12 @@ struct Core {
     }
     // The entries after the first round (whose loads the caller issued ahead of its weight loads), and the
     // run of zeros. The caller's barrier follows.
-    __device__ __forceinline__ void finish_staging(const RowsIn& rows, int m_count, int nb, int threads) {
-        const int entries = nb * 8 * TOKS;
-        place(m_count, entries, threadIdx.x, threads);
+    __device__ __forceinline__ void finish_staging(const RowsIn& rows, int m_count, int nb, int threads, int chunks = 1) {
+        const int per_chunk = nb * 8 * TOKS, entries = chunks * per_chunk;
+        place(m_count, entries, per_chunk, threadIdx.x, threads);
         for (int r = threads * PER; r < entries; r += threads * PER) {
-            issue(rows, m_count, entries, r + threadIdx.x, threads);
-            place(m_count, entries, r + threadIdx.x, threads);
+            issue(rows, m_count, entries, per_chunk, r + threadIdx.x, threads);
+            place(m_count, entries, per_chunk, r + threadIdx.x, threads);
         }
         for (int i = threadIdx.x * 16; i < zero_bytes(TOKS); i += threads * 16) *(uint4*)(zeros + i) = make_uint4(0, 0, 0, 0);
     }
@@ -144,6 +155,12 @@ struct Core {
 
     // Super-block kb of the lane's weight row against the staged activation, into the lane's four sums.
     __device__ __forceinline__ void compute(const WFrag& w, int kb, float (&acc)[4]) const {
+        float (&one)[1][4] = reinterpret_cast<float (&)[1][4]>(acc);
+        compute_chunks<1>(w, kb, one);
+    }
+    // The same against CHUNKS groups of rows: the weight codes and scales are unpacked once.
+    template <int CHUNKS>
+    __device__ __forceinline__ void compute_chunks(const WFrag& w, int kb, float (&acc)[CHUNKS][4]) const {
         // the row's (scale, min) pairs, six bits each (get_scale_min_k4 of the format); up to eight rows:
         // the words shifted to sub-blocks 2 par, 2 par + 1, 4 + 2 par, 5 + 2 par
         const uint32_t w1 = w.hdr.y, w2 = w.hdr.z, w3 = w.hdr.w;
@@ -167,15 +184,15 @@ struct Core {
         constexpr int MAGIC_BITS = 0x4B400000;
         constexpr float MAGIC = 12582912.0f;
         const v4i magic = {MAGIC_BITS, MAGIC_BITS, MAGIC_BITS, MAGIC_BITS};
-        // one instruction's four results into the sums: sub-block `sub` of the super-block
-        auto fold = [&](const v4i& c, float dsc, float dmm, int sub) {
+        // one instruction's four results into the sums of chunk ch: sub-block `sub` of the super-block
+        auto fold = [&](int ch, const v4i& c, float dsc, float dmm, int sub) {
             const float off = -MAGIC * dsc;
-            const float4 t = *(const float4*)(t_blk + sub * 2 * TOKS);
-            const float4 s = *(const float4*)(t_blk + sub * 2 * TOKS + TOKS);
-            acc[0] = fmaf(fmaf(__int_as_float(c[0]), dsc, off), t.x, fmaf(dmm, s.x, acc[0]));
-            acc[1] = fmaf(fmaf(__int_as_float(c[1]), dsc, off), t.y, fmaf(dmm, s.y, acc[1]));
-            acc[2] = fmaf(fmaf(__int_as_float(c[2]), dsc, off), t.z, fmaf(dmm, s.z, acc[2]));
-            acc[3] = fmaf(fmaf(__int_as_float(c[3]), dsc, off), t.w, fmaf(dmm, s.w, acc[3]));
+            const float4 t = *(const float4*)(t_blk + ch * t_chunk + sub * 2 * TOKS);
+            const float4 s = *(const float4*)(t_blk + ch * t_chunk + sub * 2 * TOKS + TOKS);
+            acc[ch][0] = fmaf(fmaf(__int_as_float(c[0]), dsc, off), t.x, fmaf(dmm, s.x, acc[ch][0]));
+            acc[ch][1] = fmaf(fmaf(__int_as_float(c[1]), dsc, off), t.y, fmaf(dmm, s.y, acc[ch][1]));
+            acc[ch][2] = fmaf(fmaf(__int_as_float(c[2]), dsc, off), t.z, fmaf(dmm, s.z, acc[ch][2]));
+            acc[ch][3] = fmaf(fmaf(__int_as_float(c[3]), dsc, off), t.w, fmaf(dmm, s.w, acc[ch][3]));
         };
 #pragma unroll
         for (int c2 = 0; c2 < 2; ++c2) {
@@ -190,20 +207,24 @@ struct Core {
                     b[e] = (int)x;
                 }
                 const uint32_t scw = c2 ? sc_hi : sc_lo, mnw = c2 ? mn_hi : mn_lo;
-                if constexpr (T16) {
-                    // sub-blocks 4 c2 + nib (lane groups 0, 1) and 4 c2 + 2 + nib (groups 2, 3)
-                    const v4i a0 = *(const v4i*)(a_blk + (4 * c2 + nib) * TOKS * 32);
-                    const v4i a1 = *(const v4i*)(a_blk2 + (4 * c2 + nib) * TOKS * 32);
-                    const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, magic, 0, 0, 0);
-                    const v4i c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b, magic, 0, 0, 0);
-                    fold(c0, d * (float)((scw >> (8 * nib)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib)) & 0xFFu)), 4 * c2 + nib);
-                    fold(c1, d * (float)((scw >> (8 * nib + 16)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib + 16)) & 0xFFu)),
-                         4 * c2 + 2 + nib);
-                } else {
-                    // this lane's sub-block: 4 c2 + 2 par + nib (its scale words are shifted to it)
-                    const v4i a = *(const v4i*)(a_blk + (4 * c2 + nib) * TOKS * 32);
-                    const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, magic, 0, 0, 0);
-                    fold(c, d * (float)((scw >> (8 * nib)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib)) & 0xFFu)), 4 * c2 + nib);
+                const float dsc0 = d * (float)((scw >> (8 * nib)) & 0xFFu), dmm0 = -(dmin * (float)((mnw >> (8 * nib)) & 0xFFu));
+#pragma unroll
+                for (int ch = 0; ch < CHUNKS; ++ch) {
+                    if constexpr (T16) {
+                        // sub-blocks 4 c2 + nib (lane groups 0, 1) and 4 c2 + 2 + nib (groups 2, 3)
+                        const v4i a0 = *(const v4i*)(a_blk + ch * a_chunk + (4 * c2 + nib) * TOKS * 32);
+                        const v4i a1 = *(const v4i*)(a_blk2 + ch * a_chunk2 + (4 * c2 + nib) * TOKS * 32);
+                        const v4i c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, magic, 0, 0, 0);
+                        const v4i c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b, magic, 0, 0, 0);
+                        fold(ch, c0, dsc0, dmm0, 4 * c2 + nib);
+                        fold(ch, c1, d * (float)((scw >> (8 * nib + 16)) & 0xFFu), -(dmin * (float)((mnw >> (8 * nib + 16)) & 0xFFu)),
+                             4 * c2 + 2 + nib);
+                    } else {
+                        // this lane's sub-block: 4 c2 + 2 par + nib (its scale words are shifted to it)
+                        const v4i a = *(const v4i*)(a_blk + ch * a_chunk + (4 * c2 + nib) * TOKS * 32);
+                        const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, magic, 0, 0, 0);
+                        fold(ch, c, dsc0, dmm0, 4 * c2 + nib);
+                    }
                 }
             }
         }

@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
     // The activation's first loads go out before the first weight loads and are consumed after them
     // (loads return in issue order: asked for after the weights, the activation, which sits in L2, would
     // wait for HBM).
-    auto issue = [&](int base) { core.issue(rows, p.m, entries, base, WG); };
+    auto issue = [&](int base) { core.issue(rows, p.m, entries, entries, base, WG); };
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     auto compute = [&](const WFrag& w, int kb) { core.compute(w, kb, acc); };

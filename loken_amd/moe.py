@@ -102,12 +102,12 @@ class MmqRouting:
             raise _lib.LokenError(MMQ_MOE_LAUNCHER[wtype], _lib.LK_ERR_ARG)
 
     # Rows an expert is expected to own up to which the matrix-unit rows launch (weights straight from
-    # HBM into the operand, a wave per 16-row tile, one pass per 16 rows) beats the tiled one (weights
-    # expanded into LDS per 32 tokens). Measured on MI355X at 128 experts of 2048 -> 768 -> 2048, top-8:
-    # 64 tokens 112 us against 173, 128 tokens 117 against 170, 256 tokens 173 against 182, 384 tokens
-    # 232 against 259, 512 tokens 273 against 271, 1024 tokens 444 against 408 (the expected longest run
-    # is 17 at 128 tokens, 39 at 384, 50 at 512).
-    ROWS_LAUNCH_MAX_RUN = 40
+    # HBM into the operand, a wave per 16-row tile, a pass per 8, 16 or 48 rows) beats the tiled one
+    # (weights expanded into LDS per 32 tokens). Measured on MI355X at 128 experts of 2048 -> 768 -> 2048,
+    # top-8: 64 tokens 112 us against 173, 128 tokens 121 against 170, 256 tokens 159 against 183, 512
+    # tokens 228 against 271, 1024 tokens 394 against 408, 1536 tokens 537 against 463 (the expected
+    # longest run is 17 at 128 tokens, 29 at 256, 88 at 1024, 126 at 1536).
+    ROWS_LAUNCH_MAX_RUN = 90
 
     def takes_rows_launch(self, wtype: int, k: int) -> bool:
         return (self.path != "tiled" and wtype == _lib.TYPE_Q4_K and k % 256 == 0

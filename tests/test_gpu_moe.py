@@ -522,7 +522,7 @@ def test_q4k_pair_rows_over_caller_quantized_rows_with_one_expert_per_pair(token
 
 
 @pytest.mark.parametrize("hint", [1, 9, 40])
-# a wave per 16-row tile (1, 2, 3, 4, 6, 8 super-blocks: every load depth), a wave per 32-row tile (5), or four
+# a wave per 16-row tile (2, 3, 4, 8 super-blocks: every load depth), a wave per 32-row tile (1, 5, 6), or four
 # waves splitting a tile's super-blocks (10)
 @pytest.mark.parametrize("k", [256, 512, 768, 1024, 1280, 1536, 2048, 2560])
 def test_rows_launch_serves_any_run_length_whatever_the_hint(hint, k):
