@@ -7,10 +7,10 @@ One *step* = every quantized linear of one Llama-3-8B-shaped decode step at batc
 4.97 GB of blocks. Launch plans: `--plan fused`: the linears that share an activation go out as
 one launch (q,k,v; gate,up) and every launch quantizes its f32 activation to Q8_1 in LDS itself,
 4 launches per layer; `--plan split`: the two-launch form per linear (Q8_1 quantizer, then
-mat-vec); `--plan auto` (default): fused, and up to 4 rows the gate,up launch applies SiLU(gate)*up
-and writes the Q8_1 rows that `down` reads (4 launches per layer, no quantizer launch); at 5 rows
-the split plan, and from 6 rows `--plan rows`: split, with the Q4_K matrices of 2048 rows or more
-on the matrix-unit rows kernel (loken_dense_q4k_imma_m8_plain), as measured on MI355X.
+mat-vec); `--plan rows`: the matrices on the matrix-unit kernels of 16-row tiles (q + k + v in one
+launch, o, gate + up with SiLU in one launch, down, each after a Q8_1 quantizer launch); `--plan auto`
+(default): at 1 and 2 rows fused, the gate,up launch applying SiLU(gate)*up and writing the Q8_1 rows
+that `down` reads (4 launches per layer, no quantizer launch); from 3 rows `rows`, as measured on MI355X.
 Distinct weights per layer, so the step is cache-cold by construction.
 Weights and activations are synthetic (seeded, generated on the device) and resident in HBM
 before the timed region.
@@ -29,6 +29,8 @@ Two more measurements ride in the same JSON line:
   mmq           BASELINE configs 2a / 2b, the tiled matmul, against the int8 matrix peak.
   rows-sweep    one --wtype q4_k|q6_k matrix (--rows-n x --cols-k) at 16..2048 rows: the matrix-unit
                 rows kernel against the tiled matmul, and the path QKernelMatMul::forward's mirror takes.
+  other_configs the step at 4 and 8 rows, the MoE block at 1 / 16 / 256 tokens and the Qwen3-1.7B step at
+                1 / 16 / 64 rows (BASELINE configs 1, 3, 4), each from a child run of this file.
   roofline.peak_measured / mmq.peak_measured: what a read-only launch and a register-resident
                 matrix-instruction loop reach on this card (loken_amd/probes.py).
 """
@@ -93,6 +95,26 @@ def parse_args():
                          "32 rows; tiled = the tiled matmul")
     ap.add_argument("--launches", type=int, default=200, help="timed launches of the per-launch workloads")
     return ap.parse_args()
+
+
+def other_configs():
+    """ms per step (or per block) of the other configured workloads, from child runs of this file."""
+    import subprocess
+
+    def child(flags):
+        r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--steps", "20", *flags],
+                           capture_output=True, text=True, timeout=300)
+        for ln in reversed(r.stdout.splitlines()):
+            if ln.startswith("{"):
+                d = json.loads(ln)
+                return {"ms_per_step": d["ms_per_step"], "value": d["value"], "unit": d["unit"]}
+        return {"error": (r.stderr or r.stdout)[-200:]}
+
+    return {
+        "llama3_8b_step_by_rows": {str(b): child(["--brief", "--batch", str(b)]) for b in (4, 8)},
+        "moe_block_128x2048x768_top8_by_tokens": {str(t): child(["--workload", "moe", "--tokens", str(t)]) for t in (1, 16, 256)},
+        "qwen3_1p7b_step_by_rows": {str(b): child(["--workload", "decode-1p7b", "--batch", str(b)]) for b in (1, 16, 64)},
+    }
 
 
 def main() -> int:
@@ -465,6 +487,12 @@ def main() -> int:
                          "peak": 5000.0, "unit": "TOP/s",
                          "peak_measured": {"mfma_i8_32x32x32_tops": ceil["mfma_i8_32x32x32_tops"],
                                            "mfma_f16_32x32x16_tflops": ceil["mfma_f16_32x32x16_tflops"]}}
+
+        # The other configured workloads, each as a child process running this file (their weights
+        # do not fit beside one another's): the step at 4 and 8 rows, the MoE block, the Qwen3-1.7B step.
+        del ceil
+        torch.cuda.empty_cache()
+        extras["other_configs"] = other_configs()
 
     # ------------------------------------------------------------------ CPU baseline leg
     cpu = None
