@@ -471,6 +471,14 @@ def decode_1p7b(args, dev):
             q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
             keep.append(q)
             plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s)))
+            if g == "x2" and wtype == Q4K:
+                # gate and up with the activation on top in one launch (dense_q4k_imma_m8_act_mul of the reference)
+                out = torch.empty((b, ns[0]), device=dev)
+                keep.append(out)
+                plan.append(("status", L.lk_dense_q4k_rows_actmul,
+                             (weights[0].data_ptr(), weights[1].data_ptr(), q.data_ptr(), out.data_ptr(), b, ns[0], k, 0, s)))
+                used["rows"] += 2
+                return
             for w, n in zip(weights, ns):
                 out = torch.empty((b, n), device=dev)
                 keep.append(out)
