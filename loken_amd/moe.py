@@ -322,8 +322,12 @@ def moe_gemm_gguf_down_reduce(wtype: int, h: torch.Tensor, down: torch.Tensor, r
     """``[tokens * topk, k]`` in slot order -> ``[tokens, hidden]`` (src/inference/moe_cuda/mod.rs:437-441)."""
     pairs, k = h.shape
     tokens = pairs // routing.topk
-    out = (residual.to(torch.float32).clone() if residual is not None
-           else torch.zeros((tokens, hidden), dtype=torch.float32, device=h.device))
+    if residual is not None:
+        out = residual.to(torch.float32).clone()
+    elif add_after is not None:   # the sum is written, not added to what `out` holds
+        out = torch.empty((tokens, hidden), dtype=torch.float32, device=h.device)
+    else:
+        out = torch.zeros((tokens, hidden), dtype=torch.float32, device=h.device)
     w = topk_weights.to(torch.float32).contiguous()
     _lib.check("loken_moe_gemm_gguf_down_reduce", _lib.load().loken_moe_gemm_gguf_down_reduce(
         h.data_ptr(), down.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),

@@ -341,27 +341,51 @@ def moe_block(args, dev):
     tiled = tiled and moe.moe_mmq_serves(wt, hidden) and moe.moe_mmq_serves(wt, ffn)
     # The routing (the router's side of the boundary) is built once; the timed block is what the
     # expert launchers do with it, recorded into a graph so that the host's cost stays outside.
-    flat_w = weights.reshape(-1)
     rows_launch = False
-    if tiled:
-        plan = moe.MmqRouting.from_choices(choices, experts).with_path(args.moe_path if args.moe_path in ("tiled", "rows") else "auto")
-        rows_launch = plan.takes_rows_launch(wt, hidden)
 
-        def block():
-            h = plan.gate_up_silu(wt, x, gate, up, ffn)
-            return plan.down_fold(wt, h, down, hidden, flat_w)
-    else:
-        routing = moe.ExpertRouting(choices)
+    def block_of(gate, up, down, choices, weights):
+        nonlocal rows_launch
+        flat_w = weights.reshape(-1)
+        if tiled:
+            plan = moe.MmqRouting.from_choices(choices, experts).with_path(args.moe_path if args.moe_path in ("tiled", "rows") else "auto")
+            rows_launch = plan.takes_rows_launch(wt, hidden)
 
-        def block():
-            h = moe.moe_gemm_gguf_gate_up_silu_mul(wt, x, gate, up, routing, experts, ffn)
-            return moe.moe_gemm_gguf_down_reduce(wt, h, down, routing, flat_w, experts, hidden)
+            def block():
+                h = plan.gate_up_silu(wt, x, gate, up, ffn)
+                return plan.down_fold(wt, h, down, hidden, flat_w)
+        else:
+            routing = moe.ExpertRouting(choices)
 
+            def block():   # x + experts(x): the residual enters where the fold writes its sum
+                h = moe.moe_gemm_gguf_gate_up_silu_mul(wt, x, gate, up, routing, experts, ffn)
+                return moe.moe_gemm_gguf_down_reduce(wt, h, down, routing, flat_w, experts, hidden, add_after=x)
+        return block
+
+    block = block_of(gate, up, down, choices, weights)
     eager = time_launches(lambda i: block(), args.launches)
-    us = time_replays(capture(block), args.launches)
+    single = time_replays(capture(block), args.launches)
+    # The block as a decode step holds it: one graph of `layers` blocks, each layer with its own copy of
+    # the expert tensors and its own routing, so that no replay finds a layer's experts in a cache (a
+    # graph of one block also carries the whole cost of starting a graph, some microseconds, which a
+    # step of many layers pays once). More layers at few tokens: a layer then touches few experts.
+    layers = 24 if pairs <= 512 else 4
+    blocks, layer_choices = [block], [choices]
+    for layer in range(1, layers):
+        lg = mk.randn(tokens, experts)
+        lw, lc = torch.topk(torch.softmax(lg, dim=-1), topk, dim=-1)
+        lw = (lw / lw.sum(dim=-1, keepdim=True)).contiguous()
+        layer_choices.append(lc.to(torch.int32).contiguous())
+        blocks.append(block_of(gate.clone(), up.clone(), down.clone(), layer_choices[-1], lw))
+
+    def step():
+        for b in blocks:
+            b()
+
+    us = time_replays(capture(step), max(10, args.launches // 4)) / layers
     med = float(np.median(us))
     load = torch.bincount(choices.reshape(-1).to(torch.int64), minlength=experts).cpu().numpy()
-    distinct = int((load > 0).sum())
+    distinct = float(np.mean([int((torch.bincount(c.reshape(-1).to(torch.int64), minlength=experts) > 0).sum())
+                              for c in layer_choices]))   # experts a layer's block reads, mean over the layers
     one_matrix = synth.weight_bytes(wt, ffn, hidden)
     if tiled:
         op_count = 6.0 * pairs * ffn * hidden
@@ -378,7 +402,8 @@ def moe_block(args, dev):
                     "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None, "kernel": f"moe_rows_kernel / moe_rows_legacy_kernel, {name}",
                     "note": "whole expert block (quantize, gate/up pairs, down pairs, weighted sum); bytes = 3 matrices "
                             "per distinct expert hit"}
-    extra = {"block_graph_replay": spread(us), "block_eager_from_python": spread(eager), "path": ("expert-batched rows on the matrix unit" if rows_launch else "expert-batched tiled matmul") if tiled else "mat-vec per routed pair",
+    extra = {"block_in_step_graph": dict(spread(us), blocks_per_graph=layers), "block_graph_replay": spread(single),
+             "block_eager_from_python": spread(eager), "path": ("expert-batched rows on the matrix unit" if rows_launch else "expert-batched tiled matmul") if tiled else "mat-vec per routed pair",
              "routed_pairs": pairs, "distinct_experts": distinct,
              "expert_load_histogram": {"max": int(load.max()), "mean": round(float(load.mean()), 2),
                                        "rows_per_expert_sorted_top8": sorted(load.tolist(), reverse=True)[:8]}}

@@ -418,6 +418,45 @@ def test_generic_routed_product_with_and_without_weights():
         assert_close(scaled[p], w.reshape(-1)[p] * oracle.ob_matmul(lib.TYPE_Q8_0, xs[p:p + 1], we[e], n)[0])
 
 
+@pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(1, 2048, 768, 128, 8), (16, 2048, 768, 128, 8),
+                                                              (5, 100, 512, 9, 4), (7, 264, 1024, 12, 6),
+                                                              (3, 77, 768, 5, 1), (40, 96, 512, 16, 8), (64, 64, 512, 16, 8)])
+def test_down_and_fold_in_one_launch_gives_the_bits_of_the_two_launches(tokens, hidden, ffn, n_experts, topk, monkeypatch):
+    """Short Q4_K rows at a handful of tokens take one launch (down + fold); with that launch switched
+    off the same call takes the per-pair mat-vec and the fold kernel. Same bits, and both on the oracle."""
+    down = synth.weight(lib.TYPE_Q4_K, n_experts * hidden, ffn, seed=61, stream=3)
+    ids, w = oracle.topk_softmax(synth.activation(tokens, n_experts, seed=61, stream=7), topk)
+    h = synth.activation(tokens * topk, ffn, seed=61, stream=4) * np.float32(5.0)
+    routing = ExpertRouting(dev(ids))
+    bias = torch.randn((n_experts, hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(9))
+    res = torch.randn((tokens, hidden), device="cuda", generator=torch.Generator(device="cuda").manual_seed(10))
+    down_d, h_d, w_d = dev(down), dev(h), dev(w.reshape(-1))
+
+    def run(**kw):
+        return moe_gemm_gguf_down_reduce(lib.TYPE_Q4_K, h_d, down_d, routing, w_d, n_experts, hidden, **kw)
+
+    cases = ({}, {"residual": res}, {"add_after": res}, {"down_bias": bias}, {"down_bias": bias, "add_after": res})
+    one = [run(**kw) for kw in cases]
+    # a pair whose expert is out of range, in the one launch
+    keep = routing.expert_ids[0].item()
+    routing.expert_ids[0] = -1
+    one_dropped = run()
+    monkeypatch.setenv("LK_TUNE_DOWN_FOLD_OFF", "1")
+    two_dropped = run()
+    routing.expert_ids[0] = keep
+    two = [run(**kw) for kw in cases]
+    for a, b in zip(one, two):
+        assert torch.equal(a, b)
+    assert torch.equal(one_dropped, two_dropped)
+    we = down.reshape(n_experts, hidden, -1, 144)
+    want = np.zeros((tokens, hidden), np.float32)
+    for t in range(tokens):
+        for j in range(topk):
+            p = t * topk + j
+            want[t] += w[t, j] * oracle.ob_matmul(lib.TYPE_Q4_K, h[p:p + 1], we[ids[t, j]], hidden)[0]
+    assert_close(one[0].cpu().numpy(), want, atol=1e-4 * max(1.0, np.abs(want).max()))
+
+
 def test_pairs_the_routing_leaves_out_add_nothing():
     tokens, hidden, ffn, n_experts, topk = 3, 256, 256, 4, 2
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=60)
