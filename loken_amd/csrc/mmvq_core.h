@@ -135,6 +135,22 @@ static __device__ __forceinline__ void q6k_dots_biased(const uint4& ql0, const u
     for (int g = 0; g < 4; ++g) dot[g] = dot16(c[g], a[g], dot[g]);
 }
 
+// Q6_K: the scales of the four groups of a half (`sc`: the half's 8 scale bytes) for run `lh` (0: the
+// groups' first 16 values, 1: their last 16), times the super-block's d.
+static __device__ __forceinline__ void q6k_run_scales(float d, const uint2& sc, int lh, float (&ds)[4]) {
+    ds[0] = d * (float)(int)__builtin_amdgcn_sbfe(sc.x, 8 * lh, 8);
+    ds[1] = d * (float)(int)__builtin_amdgcn_sbfe(sc.x, 8 * lh + 16, 8);
+    ds[2] = d * (float)(int)__builtin_amdgcn_sbfe(sc.y, 8 * lh, 8);
+    ds[3] = d * (float)(int)__builtin_amdgcn_sbfe(sc.y, 8 * lh + 16, 8);
+}
+// A lane's share of a Q6_K row from its runs of the four groups, added to `acc`. Every kernel that
+// must give a row the same bits forms the share here.
+static __device__ __forceinline__ void q6k_half_share(float& acc, const float (&ds)[4], const float4& d8,
+                                                      const int (&dot)[4]) {
+    acc += ds[0] * (d8.x * (float)dot[0]) + ds[2] * (d8.z * (float)dot[2]);
+    acc += ds[1] * (d8.y * (float)dot[1]) + ds[3] * (d8.w * (float)dot[3]);
+}
+
 // --------------------------------------------------------------------------------------------
 // Activation staging. Formats differ only in where a Q8_1 block's two 16-byte halves land.
 // LDS per activation row: `n_iter` passes x `PLANES` planes x 1024 bytes of codes, then the
@@ -700,10 +716,7 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
             const float d = block < nb ? f16_bits_to_f32(f.d[r]) : 0.f;
-            ds[r][0] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].x, 8 * lh, 8);
-            ds[r][1] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].x, 8 * lh + 16, 8);
-            ds[r][2] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].y, 8 * lh, 8);
-            ds[r][3] = d * (float)(int)__builtin_amdgcn_sbfe(f.sc[r].y, 8 * lh + 16, 8);
+            q6k_run_scales(d, f.sc[r], lh, ds[r]);
         }
 #pragma unroll
         for (int c = 0; c < B; ++c) {
@@ -721,8 +734,7 @@ static __device__ __forceinline__ void rows_q6k(const RowJob<NW>& job, uint8_t* 
             for (int r = 0; r < RW; ++r) {
                 int dot[4] = {bias.x, bias.y, bias.z, bias.w};
                 q6k_dots_biased(f.ql0[r], f.ql1[r], f.qh[r], a, dot);
-                acc[r][c] += ds[r][0] * (d8.x * (float)dot[0]) + ds[r][2] * (d8.z * (float)dot[2]);
-                acc[r][c] += ds[r][1] * (d8.y * (float)dot[1]) + ds[r][3] * (d8.w * (float)dot[3]);
+                q6k_half_share(acc[r][c], ds[r], d8, dot);
             }
         }
         if (it == n_iter - 1) {

@@ -22,11 +22,11 @@
 using namespace mmvq;
 
 extern "C" int lk_quantize_q8_1(const void* x, int x_type, void* vy, int kx, int kx_padded, int rows, void* stream);
-// moe_down_fold.hip: down + fold of short-row Q4_K experts in one launch; -1: not served
-int lk_moe_down_fold_q4k(const float* inputs, const void* weights, const int32_t* sorted_token_ids,
-                         const int32_t* expert_ids, const float* topk_weights, float* outputs, int num_experts, int topk,
-                         int size_m, int size_n, int size_k, const float* down_bias, const float* add_after,
-                         hipStream_t stream);
+// moe_down_fold.hip: down + fold of short-row Q4_K / Q5_K / Q6_K experts in one launch; -1: not served
+int lk_moe_down_fold(int quant_type, const float* inputs, const void* weights, const int32_t* sorted_token_ids,
+                     const int32_t* expert_ids, const float* topk_weights, float* outputs, int num_experts, int topk,
+                     int size_m, int size_n, int size_k, const float* down_bias, const float* add_after,
+                     hipStream_t stream);
 
 namespace {
 
@@ -442,11 +442,11 @@ static int down_impl(const float* inputs, const void* weights, const int32_t* so
     if (!inputs || !weights || !sorted_token_ids || !expert_ids || !topk_weights || (!outputs && !pair_rows) ||
         bad_shape(gguf_dtype, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
-    // a handful of tokens over short Q4_K rows: one launch that needs no pair rows at all (the entry
+    // a handful of tokens over short K-quant rows: one launch that needs no pair rows at all (the entry
     // point that allocates nothing keeps the two launches over its fixed array)
-    if (gguf_dtype == 1 && !from_static && !live && !pair_rows && !alt.alt0 && !alt.alt_at) {
-        const int rc = lk_moe_down_fold_q4k(inputs, weights, sorted_token_ids, expert_ids, topk_weights, outputs,
-                                            num_experts, topk, size_m, size_n, size_k, down_bias, add_after, s);
+    if (!from_static && !live && !pair_rows && !alt.alt0 && !alt.alt_at) {
+        const int rc = lk_moe_down_fold(gguf_dtype, inputs, weights, sorted_token_ids, expert_ids, topk_weights, outputs,
+                                        num_experts, topk, size_m, size_n, size_k, down_bias, add_after, s);
         if (rc >= 0) return rc;
     }
     const int kp = pad512(size_k);

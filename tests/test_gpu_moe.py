@@ -421,10 +421,12 @@ def test_generic_routed_product_with_and_without_weights():
 @pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(1, 2048, 768, 128, 8), (16, 2048, 768, 128, 8),
                                                               (5, 100, 512, 9, 4), (7, 264, 1024, 12, 6),
                                                               (3, 77, 768, 5, 1), (40, 96, 512, 16, 8), (64, 64, 512, 16, 8)])
-def test_down_and_fold_in_one_launch_gives_the_bits_of_the_two_launches(tokens, hidden, ffn, n_experts, topk, monkeypatch):
-    """Short Q4_K rows at a handful of tokens take one launch (down + fold); with that launch switched
+@pytest.mark.parametrize("name", ["q4_k", "q5_k", "q6_k"])
+def test_down_and_fold_in_one_launch_gives_the_bits_of_the_two_launches(name, tokens, hidden, ffn, n_experts, topk, monkeypatch):
+    """Short K-quant rows at a handful of tokens take one launch (down + fold); with that launch switched
     off the same call takes the per-pair mat-vec and the fold kernel. Same bits, and both on the oracle."""
-    down = synth.weight(lib.TYPE_Q4_K, n_experts * hidden, ffn, seed=61, stream=3)
+    dt, block_bytes = {"q4_k": (lib.TYPE_Q4_K, 144), "q5_k": (lib.TYPE_Q5_K, 176), "q6_k": (lib.TYPE_Q6_K, 210)}[name]
+    down = synth.weight(dt, n_experts * hidden, ffn, seed=61, stream=3)
     ids, w = oracle.topk_softmax(synth.activation(tokens, n_experts, seed=61, stream=7), topk)
     h = synth.activation(tokens * topk, ffn, seed=61, stream=4) * np.float32(5.0)
     routing = ExpertRouting(dev(ids))
@@ -433,7 +435,7 @@ def test_down_and_fold_in_one_launch_gives_the_bits_of_the_two_launches(tokens, 
     down_d, h_d, w_d = dev(down), dev(h), dev(w.reshape(-1))
 
     def run(**kw):
-        return moe_gemm_gguf_down_reduce(lib.TYPE_Q4_K, h_d, down_d, routing, w_d, n_experts, hidden, **kw)
+        return moe_gemm_gguf_down_reduce(dt, h_d, down_d, routing, w_d, n_experts, hidden, **kw)
 
     cases = ({}, {"residual": res}, {"add_after": res}, {"down_bias": bias}, {"down_bias": bias, "add_after": res})
     one = [run(**kw) for kw in cases]
@@ -448,12 +450,12 @@ def test_down_and_fold_in_one_launch_gives_the_bits_of_the_two_launches(tokens, 
     for a, b in zip(one, two):
         assert torch.equal(a, b)
     assert torch.equal(one_dropped, two_dropped)
-    we = down.reshape(n_experts, hidden, -1, 144)
+    we = down.reshape(n_experts, hidden, -1, block_bytes)
     want = np.zeros((tokens, hidden), np.float32)
     for t in range(tokens):
         for j in range(topk):
             p = t * topk + j
-            want[t] += w[t, j] * oracle.ob_matmul(lib.TYPE_Q4_K, h[p:p + 1], we[ids[t, j]], hidden)[0]
+            want[t] += w[t, j] * oracle.ob_matmul(dt, h[p:p + 1], we[ids[t, j]], hidden)[0]
     assert_close(one[0].cpu().numpy(), want, atol=1e-4 * max(1.0, np.abs(want).max()))
 
 
