@@ -260,6 +260,13 @@ static __device__ __forceinline__ const uint8_t* lk_expert_slab(const uint8_t* b
     return base + (int64_t)e * slab_bytes;
 }
 
+// The Q4_K gate / up pair per routed pair of an MoE layer with the activation row's codes in
+// registers (mmvq_reg.hip): f32 activation rows `acts` [tokens][256 nb], output rows in slot order.
+// -1: not served (rows longer than 16 super-blocks, more than 65535 pairs, misaligned), else LK_*.
+int lk_q4k_reg_moe_pair(const uint8_t* gate, const uint8_t* up, const float* acts, const int32_t* sorted_token_ids,
+                        const int32_t* expert_ids, float* out, int experts, int topk, int pairs, int n, int nb,
+                        int64_t slab_bytes, const LkGateAct& act, hipStream_t stream);
+
 // MoE decode for the expert formats the K-quant engines do not serve (mmvq_legacy.hip): block length
 // of a wire id (0: not one of them), and the per-pair launch over Q8_1 activation rows. An expert's
 // slab is `slab_rows` weight rows (cols, or twice that where gate and up share a tensor); with `live`

@@ -348,6 +348,58 @@ __global__ __launch_bounds__(RT) void q4k_reg_pair_kernel(const uint8_t* __restr
     }
 }
 
+// The gate / up pair per routed (token, expert) pair of an MoE layer: grid.y names the pair, whose
+// expert picks the two slabs, whose token picks the f32 activation row and whose slot picks the
+// output row (the conventions of loken_moe_gemm_gguf_gate_up_silu_mul, cuda/moe/moe_gguf.cu:896-1060
+// of the reference). Everything else is the pair kernel above.
+struct RegMoeArgs {
+    const int32_t* sorted_token_ids;
+    const int32_t* expert_ids;
+    int experts, topk, pairs;
+    int64_t slab_bytes;
+    LkGateAct act;
+};
+template <int RP>
+__global__ __launch_bounds__(RT) void q4k_reg_moe_pair_kernel(const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up,
+                                                              const float* __restrict__ acts, float* __restrict__ out, int nb,
+                                                              int n, RegMoeArgs m, int waves) {
+#pragma clang fp contract(off)
+    __shared__ __align__(16) uint8_t lds[LDS_BYTES];
+    const int pair = blockIdx.y;
+    const int slot = m.sorted_token_ids[pair], e = m.expert_ids[pair];
+    asm volatile("" ::"s"(slot), "s"(e), "s"(m.pairs), "s"(m.experts), "s"(m.topk), "s"(m.slab_bytes), "s"(gate), "s"(up),
+                 "s"(acts), "s"(out), "s"(nb), "s"(n), "s"(waves), "s"(m.act.kind));
+    if (slot < 0 || slot >= m.pairs || e < 0 || e >= m.experts) return;   // a pair the routing leaves out writes nothing
+    const Geo<RP> g(nb);
+    const Q4KScaleSel sel(g.p);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const size_t row_stride = (size_t)nb * Q4K_BYTES;
+    const gbytes_t wg = to_gbytes(gate) + (int64_t)e * m.slab_bytes, wu = to_gbytes(up) + (int64_t)e * m.slab_bytes;
+    const gbytes_t act = to_gbytes(acts) + (size_t)(slot / m.topk) * nb * (256 * sizeof(float));
+    float* dst = out + (size_t)slot * n;
+    uint32_t flip = 0x80808080u;
+    asm volatile("" : "+v"(flip));
+    const bool odd = g.lane & 1;
+    RowFrag fg, fu;
+    auto load = [&](int row) {
+        const size_t at = (size_t)min(row, n - 1) * row_stride;
+        row_load(fg, wg + at, g.hdr_off, g.qs_off);
+        row_load(fu, wu + at, g.hdr_off, g.qs_off);
+    };
+    const int tiles = (n + RP - 1) / RP, step = (int)gridDim.x * waves;
+    int t = (int)blockIdx.x * waves + wave;
+    Slice s;
+    slice_load<true>(s, act, nb, g.unit, g.valid, lds, [&] { load(min(t, tiles - 1) * RP + g.rp); });
+    while (t < tiles) {
+        const int row = t * RP + g.rp;
+        const float both = group_sum2<Geo<RP>::GROUP>(row_share(fg, s, sel, g.valid, flip), row_share(fu, s, sel, g.valid, flip), odd);
+        const float u = dpp_f32<0xB1>(both);   // the odd neighbour's total
+        if ((g.lane & (Geo<RP>::GROUP - 1)) == 0 && row < n) dst[row] = lk_gated(m.act, both, u, (size_t)e * n + row);
+        t += step;
+        if (t < tiles) load(t * RP + g.rp);
+    }
+}
+
 // Launch shape. f32 activation: workgroups of RW waves (the row is quantized once per workgroup), two
 // per CU. Q8_1 activation: nothing is shared inside a workgroup, four waves each, four per CU.
 // LK_TUNE_REG_WAVES / LK_TUNE_REG_WGS_PER_CU override both for measurement runs.
@@ -435,6 +487,32 @@ int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, 
         case 1: return two ? launch_multi<2, 1>(m, act, act_f32, nb, dst_type, stream) : launch_multi<1, 1>(m, act, act_f32, nb, dst_type, stream);
         case 2: return two ? launch_multi<2, 2>(m, act, act_f32, nb, dst_type, stream) : launch_multi<1, 2>(m, act, act_f32, nb, dst_type, stream);
         default: return launch_multi<1, 4>(m, act, act_f32, nb, dst_type, stream);
+    }
+}
+
+template <int RP>
+static int launch_moe_pair(const uint8_t* gate, const uint8_t* up, const float* acts, float* out, int nb, int n,
+                           const RegMoeArgs& m, hipStream_t s) {
+    static const int forced_per_cu = lk_tune_env("LK_TUNE_REG_MOE_PER_CU");
+    const int tiles = (n + RP - 1) / RP, need = (tiles + RW - 1) / RW;
+    int share = lk_device().cus * (forced_per_cu > 0 ? forced_per_cu : 4) / m.pairs;
+    if (share < 1) share = 1;
+    const dim3 grid(need < share ? need : share, m.pairs);
+    hipLaunchKernelGGL((q4k_reg_moe_pair_kernel<RP>), grid, dim3(RT), 0, s, gate, up, acts, out, nb, n, m, RW);
+    return lk_launch_status();
+}
+
+int lk_q4k_reg_moe_pair(const uint8_t* gate, const uint8_t* up, const float* acts, const int32_t* sorted_token_ids,
+                        const int32_t* expert_ids, float* out, int experts, int topk, int pairs, int n, int nb,
+                        int64_t slab_bytes, const LkGateAct& act, hipStream_t stream) {
+    static const int off = lk_tune_env("LK_TUNE_NO_REG_MOE");
+    if (off || !lk_q4k_reg_serves(nb) || pairs < 1 || pairs > 65535 || n < 1) return -1;
+    if ((((uintptr_t)gate) | ((uintptr_t)up) | ((uintptr_t)acts)) & 15) return -1;
+    const RegMoeArgs m{sorted_token_ids, expert_ids, experts, topk, pairs, slab_bytes, act};
+    switch (q4k_rows_per_pass(nb)) {
+        case 1: return launch_moe_pair<1>(gate, up, acts, out, nb, n, m, stream);
+        case 2: return launch_moe_pair<2>(gate, up, acts, out, nb, n, m, stream);
+        default: return launch_moe_pair<4>(gate, up, acts, out, nb, n, m, stream);
     }
 }
 

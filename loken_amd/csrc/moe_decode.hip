@@ -339,6 +339,14 @@ static int gate_up_impl(const float* inputs, const void* gate_weights, const voi
         bad_shape(quant_type, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
     hipStream_t s = (hipStream_t)stream;
     const int kp = pad512(size_k), act_rows = size_m / topk;
+    // Q4_K rows of at most 16 super-blocks: the engine that keeps the activation's codes in registers
+    if (quant_type == 1 && !live && !alt.alt0 && !alt.alt1 && !alt.alt_at && rows_stage_as_f32(inputs, size_k, quant_type)) {
+        const int nb = size_k / 256;
+        const int rc = lk_q4k_reg_moe_pair((const uint8_t*)gate_weights, (const uint8_t*)up_weights, inputs, sorted_token_ids,
+                                           expert_ids, outputs, num_experts, topk, size_m, size_n, nb,
+                                           (int64_t)(slab_rows ? slab_rows : size_n) * nb * Q4K_BYTES, act, s);
+        if (rc >= 0) return rc;
+    }
     if (rows_stage_as_f32(inputs, size_k, quant_type)) {
         MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0, size_k, slab_rows, act, live, alt};
         return launch_format<MODE_GATED>(quant_type, (const uint8_t*)gate_weights, (const uint8_t*)up_weights,
