@@ -379,7 +379,9 @@ int loken_moe_gemm_gguf_down_pairs_two(const float* inputs, const void* weights,
 /* outputs[t, :] (+)= sum over k ascending of topk_weights[p] * (down_e(p) . inputs[p] + down_bias[e(p)]),
  * p = t * topk + k; inputs [size_m, k] in slot order. Without add_after `outputs` [size_m/topk,
  * size_n] must be pre-filled (zeros or the residual) and is accumulated into; with it the result
- * is written as fold + add_after. down_bias [num_experts, size_n] nullable. */
+ * is written as fold + add_after. down_bias [num_experts, size_n] nullable. Q4_K / Q5_K / Q6_K rows of
+ * 512, 768 or 1024 values with at most 512 routed pairs and topk <= 8 run as one launch that needs no
+ * scratch (same bits as the mat-vec launch + fold every other call takes). */
 int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,
                                     const int32_t* sorted_token_ids, const int32_t* expert_ids,
                                     const float* topk_weights, float* outputs, int num_experts, int topk,
