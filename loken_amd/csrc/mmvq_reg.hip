@@ -267,7 +267,7 @@ static __device__ __forceinline__ float act_gelu_tanh(float g) {
 
 // The gate / up pair: a tile is RP rows (one per lane group) of both matrices; the two shares of a
 // row are summed together (even lanes gate, odd lanes up) and lane 0 of the group combines them.
-// Q81_OUT: a workgroup owns whole blocks of 32 consecutive rows (wave w rows 4w .. 4w + 3, RP = 1),
+// Q81_OUT: a workgroup owns whole blocks of 32 consecutive rows (wave w rows 4w .. 4w + 3),
 // the 32 results meet in LDS and eight lanes write them as one Q8_1 block with the quantizer's steps.
 template <int RP, bool ACT_F32, bool Q81_OUT>
 __global__ __launch_bounds__(RT) void q4k_reg_pair_kernel(const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up,
@@ -311,17 +311,39 @@ __global__ __launch_bounds__(RT) void q4k_reg_pair_kernel(const uint8_t* __restr
         }
         return;
     }
+    // A wave's four rows of a block go through in PASSES = 4 / RP passes of RP rows side by side, with
+    // the loads of D passes in flight (two rows of both matrices at RP = 1: more would cost the second
+    // workgroup per CU its registers): a pass's loads go out D passes ahead, into the registers of the
+    // pass just consumed, across block boundaries too.
+    constexpr int PASSES = 4 / RP, D = PASSES < 2 ? PASSES : 2;
     const int blocks = n / 32;
     int b = blockIdx.x;
-    slice_load<ACT_F32>(s, to_gbytes(act), nb, g.unit, g.valid, lds, [&] { load(32 * min(b, blocks - 1) + 4 * wave); });
+    RowFrag bg[D], bu[D];
+    auto load_pass = [&](int slot, int blk, int i) {
+        const size_t at = (size_t)min(32 * blk + 4 * wave + i * RP + g.rp, n - 1) * row_stride;
+        row_load(bg[slot], wg + at, g.hdr_off, g.qs_off);
+        row_load(bu[slot], wu + at, g.hdr_off, g.qs_off);
+    };
+    slice_load<ACT_F32>(s, to_gbytes(act), nb, g.unit, g.valid, lds, [&] {
+#pragma unroll
+        for (int i = 0; i < D; ++i) load_pass(i, min(b, blocks - 1), i);
+    });
     int half = 0;
     for (; b < blocks; b += gridDim.x) {
-#pragma unroll 1
-        for (int i = 0; i < 4; ++i) {
-            const float v = value(s);
-            if (g.lane == 0) meet[half * 32 + 4 * wave + i] = v;
-            const int next = i < 3 ? 32 * b + 4 * wave + i + 1 : 32 * (b + (int)gridDim.x) + 4 * wave;
-            if (next < n) load(next);
+        float val[PASSES];
+        const int nb_next = b + (int)gridDim.x;
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) {
+            const float both = group_sum2<Geo<RP>::GROUP>(row_share(bg[i % D], s, sel, g.valid, flip),
+                                                          row_share(bu[i % D], s, sel, g.valid, flip), odd);
+            const float u = dpp_f32<0xB1>(both);   // the odd neighbour's total
+            val[i] = (act_fn == 0 ? act_silu(both) : act_gelu_tanh(both)) * u;
+            if (i + D < PASSES) load_pass(i % D, b, i + D);
+            else if (nb_next < blocks) load_pass(i % D, nb_next, i + D - PASSES);
+        }
+        if ((g.lane & (Geo<RP>::GROUP - 1)) == 0) {
+#pragma unroll
+            for (int i = 0; i < PASSES; ++i) meet[half * 32 + 4 * wave + i * RP + g.rp] = val[i];
         }
         __syncthreads();   // every wave of the workgroup has delivered its four
         if (wave == 0 && g.lane < 8) {
@@ -448,9 +470,9 @@ static int launch_pair(const uint8_t* gate, const uint8_t* up, const void* act, 
         const int blocks = n / 32, cap = sh.cap;
         const dim3 grid(blocks < cap ? blocks : cap);
         if (act_f32)
-            hipLaunchKernelGGL((q4k_reg_pair_kernel<1, true, true>), grid, dim3(RT), 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves);
+            hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, true, true>), grid, dim3(RT), 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves);
         else
-            hipLaunchKernelGGL((q4k_reg_pair_kernel<1, false, true>), grid, dim3(RT), 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves);
+            hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, false, true>), grid, dim3(RT), 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves);
         return lk_launch_status();
     }
     const Shape sh = shape_for(act_f32 != 0);
@@ -519,10 +541,9 @@ int lk_q4k_reg_moe_pair(const uint8_t* gate, const uint8_t* up, const float* act
 int lk_q4k_reg_pair(const uint8_t* gate, const uint8_t* up, const void* act, int act_f32, void* dst, int dst_type,
                     bool dst_q8_1, int nb, int n, int act_fn, hipStream_t stream) {
     if (!lk_q4k_reg_serves(nb) || n < 1 || (dst_q8_1 && n % 32 != 0)) return LK_ERR_ARG;
-    if (dst_q8_1) return launch_pair<1>(gate, up, act, act_f32, dst, dst_type, true, nb, n, act_fn, stream);
     switch (q4k_rows_per_pass(nb)) {
-        case 1: return launch_pair<1>(gate, up, act, act_f32, dst, dst_type, false, nb, n, act_fn, stream);
-        case 2: return launch_pair<2>(gate, up, act, act_f32, dst, dst_type, false, nb, n, act_fn, stream);
-        default: return launch_pair<4>(gate, up, act, act_f32, dst, dst_type, false, nb, n, act_fn, stream);
+        case 1: return launch_pair<1>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, stream);
+        case 2: return launch_pair<2>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, stream);
+        default: return launch_pair<4>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, stream);
     }
 }

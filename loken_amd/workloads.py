@@ -465,6 +465,11 @@ def decode_1p7b(args, dev):
             keep.extend(outs + [vx, dst, nn])
             plan.append(("status", L.lk_dense_q4k_rows_multi, (vx, dst, nn, len(ns), q.data_ptr(), b, k, 0, s)))
 
+    # one or two rows: gate + up as the pair launch that applies SiLU and writes the Q8_1 rows `down`
+    # reads (the default plan of the Llama step), so `down` needs neither the f32 rows nor a quantizer
+    paired = matvec and b <= 2
+    h_q81 = torch.empty((b, ops.pad_to(ffn, 512) // 32, 36), dtype=torch.uint8, device=dev) if paired else None
+
     def add_group(g, k, wtype, ns):
         nonlocal total_bytes
         if fused_rows:
@@ -473,7 +478,15 @@ def decode_1p7b(args, dev):
         keep.extend(weights)
         total_bytes += sum(synth.weight_bytes(wtype, n, k) for n in ns)
         x = acts[g]
-        if matvec and k <= 8192:
+        if paired and g == "x2":
+            plan.append(("status", L.lk_mmvq_pair_act_q8_1, (wtype, weights[0].data_ptr(), weights[1].data_ptr(), x.data_ptr(), 1,
+                                                              x.stride(0), h_q81.data_ptr(), h_q81.shape[1], k, ns[0], b, 0, s)))
+        elif paired and g == "h":
+            out = torch.empty((b, ns[0]), device=dev)
+            keep.append(out)
+            plan.append(("status", L.lk_mmvq, (wtype, weights[0].data_ptr(), h_q81.data_ptr(), out.data_ptr(), lib.TYPE_F32, k,
+                                               ns[0], b, h_q81.shape[1], ns[0], None, 0, s)))
+        elif matvec and k <= 8192:
             stride = max(ns)
             outs = [torch.empty((b, stride), device=dev) for _ in ns]
             vx = (lib.C.c_void_p * len(ns))(*[w.data_ptr() for w in weights])
@@ -576,7 +589,8 @@ def decode_1p7b(args, dev):
     return line(args, value, "GB/s", ms, "int8",
                 {"workload": f"qwen3-1.7b decode-step quantized linears (Q4_K attention and gate/up, Q6_K down and "
                              f"lm_head), batch {b}, 28 layers",
-                 "path": "mat-vec (fused; own quantizer launch for rows over 8192 values)" if matvec
+                 "path": "mat-vec (fused: q + k + v, o from f32 rows; gate + up as the pair launch that writes down's Q8_1 rows)" if paired
+                         else "mat-vec (fused; own quantizer launch for rows over 8192 values)" if matvec
                          else "16-row tiles on the matrix unit: q + k + v in one launch, o, gate + up with SiLU in one, down, lm_head, "
                               "each after a Q8_1 quantizer launch" if fused_rows
                          else f"linears on the matrix-unit rows kernels: {used['rows']}, as mat-vec slices of eight rows: "
