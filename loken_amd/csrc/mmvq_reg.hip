@@ -504,7 +504,9 @@ int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, 
     // (from f32 rows the bound is one workgroup per CU: q + k + v of a Llama-sized layer, 6144 rows, is
     // faster as single rows over two workgroups per CU, 5.7 against 6.1 us; o, 4096 rows, as pairs)
     const int waves_at_once = (act_f32 ? lk_device().cus : sh.cap) * sh.waves;
-    const bool two = forced ? forced == 2 : (rows + rp - 1) / rp <= waves_at_once * 2;
+    // (rows short enough to go side by side already give a wave two or four rows per pass: two such
+    // tiles per wave measured slower, Qwen3-1.7B step 0.598 against 0.586 ms)
+    const bool two = forced ? forced == 2 : rp == 1 && rows <= waves_at_once * 2;
     switch (rp) {
         case 1: return two ? launch_multi<2, 1>(m, act, act_f32, nb, dst_type, stream) : launch_multi<1, 1>(m, act, act_f32, nb, dst_type, stream);
         case 2: return two ? launch_multi<2, 2>(m, act, act_f32, nb, dst_type, stream) : launch_multi<1, 2>(m, act, act_f32, nb, dst_type, stream);
