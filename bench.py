@@ -342,8 +342,14 @@ def main() -> int:
             add_quant("attn")
             add_rows(made["o"][0], "attn", HIDDEN, HIDDEN)
             add_quant("x2")
-            add_rows_actmul(made["gate"][0], made["up"][0], "x2", FFN, HIDDEN)
-            add_quant("h")
+            if b <= 16:
+                # gate + up hands its result on as the Q8_1 rows `down` reads: no f32 round trip, no quantizer launch
+                count_q4k((L.lk_dense_q4k_rows_actmul_q8_1, (made["gate"][0].data_ptr(), made["up"][0].data_ptr(), q81["x2"].data_ptr(),
+                                                             q81["h"].data_ptr(), b, FFN, HIDDEN, 0, 0, stream)),
+                          2 * synth.weight_bytes(Q4K, FFN, HIDDEN))
+            else:
+                add_rows_actmul(made["gate"][0], made["up"][0], "x2", FFN, HIDDEN)
+                add_quant("h")
             add_rows_q6k(made["down"][0], "h", HIDDEN, FFN)
             continue
         last_group = None

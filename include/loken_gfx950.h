@@ -435,6 +435,14 @@ int lk_dense_q4k_rows_actmul(const void* gate, const void* up, const void* q8_1,
  * are host arrays of `count` (1..3) entries. */
 int lk_dense_q4k_rows_multi(const void* const* weights, float* const* outputs, const int* sizes_n, int count,
                             const void* q8_1, int size_m, int size_k, int q5, void* stream);
+/* Gate and up in one launch with the result handed on as Q8_1 rows: q8_1_out [size_m][size_n / 32 blocks]
+ * = lk_quantize_q8_1(act(gate . x) * (up . x)) byte for byte, which the layer's down projection reads
+ * with no f32 round trip and no quantizer launch in between. At most 16 rows, size_k 2048 or 4096, size_n
+ * a multiple of 32 (anything else: LK_ERR_ARG; take lk_dense_q4k_rows_actmul and the quantizer). q5 != 0:
+ * Q5_K weights. No counterpart in the reference, whose dense_q4k_imma_m8_act_mul writes f32
+ * (src/inference/moe_cuda/dense/imma.rs:320-400); the mat-vec sibling is lk_mmvq_pair_act_q8_1. */
+int lk_dense_q4k_rows_actmul_q8_1(const void* gate, const void* up, const void* q8_1, void* q8_1_out, int size_m,
+                                  int size_n, int size_k, int use_gelu, int q5, void* stream);
 /* The Q5_K siblings of the four launches above (block_q5_K = block_q4_K plus a plane of fifth bits):
  * loken_dense_q5k_imma_m8_plain / _actmul, declared src/inference/moe_cuda/mod.rs:459-466 and picked
  * by weight dtype at src/inference/moe_cuda/dense/imma.rs:113-116 and 362-365. */

@@ -133,6 +133,29 @@ static __device__ __forceinline__ int sum8(int v, int& quad) {
     return v + dpp_i32<0x141>(v);
 }
 
+// Thirty-two f32 values as one Q8_1 block, by the eight lanes of an aligned group (lane l8 brings values
+// 4 l8 .. 4 l8 + 3): the steps of the stand-alone quantizer (d = amax / 127, stored as f16; codes =
+// round-half-away(x * (1 / d)) with d before its rounding; s = f16(f32(sum of codes * d))), so the bytes
+// are those lk_quantize_q8_1 writes. `out`: the block's nine words.
+static __device__ __forceinline__ void lk_store_q8_1_block(float4 v, int l8, uint32_t* out) {
+#pragma clang fp contract(off)
+    const float amax = max8(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    const float d = amax / 127.0f;
+    const float inv = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q0 = (int)roundf(v.x * inv), q1 = (int)roundf(v.y * inv);
+    const int q2 = (int)roundf(v.z * inv), q3 = (int)roundf(v.w * inv);
+    int quad;
+    const int sum = sum8(q0 + q1 + q2 + q3, quad);
+    out[1 + l8] = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
+                  ((uint32_t)(q3 & 0xFF) << 24);
+    if (l8 == 0) {
+        const uint32_t dh = __half_as_ushort(__float2half_rn(d));
+        float scaled_sum = (float)sum * d;
+        asm volatile("" : "+v"(scaled_sum));   // two roundings, as the quantizer's
+        out[0] = dh | ((uint32_t)__half_as_ushort(__float2half_rn(scaled_sum)) << 16);
+    }
+}
+
 static __device__ __forceinline__ int wave_sum_i32(int v) {
     for (int o = 1; o < 64; o <<= 1) v += __shfl_xor(v, o);
     return v;

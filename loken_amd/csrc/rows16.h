@@ -11,6 +11,8 @@ struct LkRows16 {
     const uint8_t* y;      // Q8_1 rows, stride_y blocks apart
     int nb, m, stride_y;
     int gelu;              // `dual`: 0 SiLU, 1 tanh-form GELU
+    uint8_t* q81_dst;      // `dual` only, when given: the result as Q8_1 rows (blocks of 32 consecutive output
+    int q81_stride;        // rows, q81_stride blocks between rows) instead of f32 in dst[0]; n a multiple of 32
 };
 // True when the launch takes `size_m` activation rows of `nb` super-blocks (their codes fit in LDS).
 bool lk_rows16_serves(int size_m, int nb);

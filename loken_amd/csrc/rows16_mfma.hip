@@ -49,9 +49,9 @@ using rows16::Blk;
 using rows16::TILE;
 using rows16::WFrag;
 
-static __host__ __device__ constexpr int lds_bytes_for(int nb, int tiles, int toks) {
-    // the staged activation, reduce [4 tiles][4][64] floats
-    return rows16::staged_bytes(nb, toks) + KSPLIT * tiles * 4 * 64 * 4;
+static __host__ __device__ constexpr int lds_bytes_for(int nb, int tiles, int toks, bool q81 = false) {
+    // the staged activation, reduce [4 tiles][4][64] floats, with Q8_1 output the 32 results of every row
+    return rows16::staged_bytes(nb, toks) + KSPLIT * tiles * 4 * 64 * 4 + (q81 ? toks * 32 * 4 : 0);
 }
 
 // Element `i` of a three-entry kernel argument without indexing it by a register (which would
@@ -82,12 +82,16 @@ static __device__ __forceinline__ TileRef tile_ref(const LkRows16& p, int vt) {
 // runs twice: once against sub-block s (the activation live in lane groups 0, 1) and once against s + 2
 // (live in groups 2, 3). Lane l, register v is (weight row l % 16, activation row 4 (l / 16) + v) for
 // both, so every lane unpacks all eight scales of its row and its sums are complete across sub-blocks.
-template <bool DUAL, bool Q5, int STEPS, int TW, bool T16>
+// Q81 (gate + up, four tiles per workgroup: the 32 consecutive output rows of a Q8_1 block): the result
+// leaves as the Q8_1 rows the next linear reads, with the quantizer's steps.
+template <bool DUAL, bool Q5, int STEPS, int TW, bool T16, bool Q81 = false>
 __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(LkRows16 p, int n_vt) {
+    static_assert(!Q81 || (DUAL && TW == 4), "Q8_1 output: the dual launch with four tiles per workgroup");
     constexpr int WG = 256 * TW;
     extern __shared__ __align__(16) uint8_t lds[];
     rows16::Core<Q5, T16> core;
     float* reduce = (float*)core.init(lds, p.nb);                       // [4 TW][4][64]
+    float* meet = reduce + KSPLIT * TW * 4 * 64;                        // Q81: [TOKS][32]
     const rows16::RowsIn rows{p.y, p.stride_y, nullptr, 0};
 
     const int lane = core.lane, l16 = core.l16;
@@ -142,7 +146,11 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
                 act.kind = p.gelu ? LK_GATE_GELU : LK_GATE_SILU;
                 sum = lk_gated(act, sum, total_of(ts + 1), 0);
             }
-            if (vt < n_vt) {
+            if (Q81) {
+                // (n is a multiple of 32 here: every tile of the launch is whole)
+                const int tok = (T16 ? 4 * (l >> 4) : 4 * ((l >> 4) & 1)) + v;
+                meet[tok * 32 + 8 * ts + (l & 15)] = sum;
+            } else if (vt < n_vt) {
                 const TileRef tr = tile_ref<DUAL>(p, vt);
                 const int out = DUAL ? 0 : tr.mat;
                 const int tok = (T16 ? 4 * (l >> 4) : 4 * ((l >> 4) & 1)) + v, row = tr.row0 + (l & 15);
@@ -150,6 +158,15 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
             }
         }
         __syncthreads();   // the partial tiles may be overwritten
+        if (Q81) {
+            // eight lanes per activation row write its block; the next group's results reach `meet` only
+            // after the barrier these lanes pass next
+            if (t < 8 * p.m && vt0 < n_vt) {
+                const int tok = t >> 3, l8 = t & 7;
+                const float4 v4 = *(const float4*)(meet + tok * 32 + 4 * l8);
+                lk_store_q8_1_block(v4, l8, (uint32_t*)(p.q81_dst + ((size_t)tok * p.q81_stride + vt0 / 4) * Q81_BYTES));
+            }
+        }
     };
 
     auto stage = [&]() {
@@ -225,7 +242,7 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
 }
 
 // Workgroups per CU the kernel can keep resident with `lds_bytes` of LDS each; 0: does not fit.
-template <bool DUAL, bool Q5, int STEPS, int TW, bool T16>
+template <bool DUAL, bool Q5, int STEPS, int TW, bool T16, bool Q81 = false>
 int resident_cap(int lds_bytes) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -236,11 +253,11 @@ int resident_cap(int lds_bytes) {
     if (lds_bytes > lk_device().lds_bytes) {
         r = 0;
     } else if (lds_bytes > 48 * 1024 &&
-               hipFuncSetAttribute((const void*)q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16>, hipFuncAttributeMaxDynamicSharedMemorySize,
+               hipFuncSetAttribute((const void*)q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16, Q81>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         r = 0;
-    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16>, 256 * TW,
+    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16, Q81>, 256 * TW,
                                                             (size_t)lds_bytes) != hipSuccess || r < 1) {
         (void)hipGetLastError();
         r = 1;
@@ -249,10 +266,10 @@ int resident_cap(int lds_bytes) {
     return r;
 }
 
-template <bool DUAL, bool Q5, int STEPS, int TW, bool T16>
+template <bool DUAL, bool Q5, int STEPS, int TW, bool T16, bool Q81 = false>
 int launch_shape(const LkRows16& a, int n_vt, hipStream_t stream) {
-    const int lds_bytes = lds_bytes_for(a.nb, TW, T16 ? 16 : 8);
-    const int per_cu = resident_cap<DUAL, Q5, STEPS, TW, T16>(lds_bytes);
+    const int lds_bytes = lds_bytes_for(a.nb, TW, T16 ? 16 : 8, Q81);
+    const int per_cu = resident_cap<DUAL, Q5, STEPS, TW, T16, Q81>(lds_bytes);
     if (per_cu == 0) return -1;
     const int units = (n_vt + TW - 1) / TW;   // tile groups
     // Every workgroup stages the activation, so a workgroup should walk a few tile groups; all of
@@ -262,7 +279,7 @@ int launch_shape(const LkRows16& a, int n_vt, hipStream_t stream) {
     if (forced > 0) cap = forced;
     const int passes = (units + cap - 1) / cap;
     const int wgs = (units + passes - 1) / passes;
-    hipLaunchKernelGGL((q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16>), dim3(wgs), dim3(256 * TW), lds_bytes, stream, a, n_vt);
+    hipLaunchKernelGGL((q4k_rows16_kernel<DUAL, Q5, STEPS, TW, T16, Q81>), dim3(wgs), dim3(256 * TW), lds_bytes, stream, a, n_vt);
     return lk_launch_status();
 }
 
@@ -275,6 +292,10 @@ int launch_steps(const LkRows16& a, hipStream_t stream) {
         for (int i = 0; i < a.count; ++i) n_vt += (a.n[i] + TILE - 1) / TILE;
     }
     if (n_vt == 0) return LK_OK;
+    if (a.q81_dst) {   // Q8_1 output: the straight-line dual launch at four tiles per workgroup, or nothing
+        if constexpr (DUAL && STEPS != 0) return launch_shape<DUAL, Q5, STEPS, 4, T16, true>(a, n_vt, stream);
+        return -1;
+    }
     // Four tiles per workgroup (sixteen waves, one workgroup per CU) once that still gives every CU
     // a workgroup: half the copies of the activation staged.
     int tw = n_vt >= 4 * lk_device().cus ? 4 : 2;
@@ -311,6 +332,7 @@ bool lk_rows16_serves(int size_m, int nb) {
 int lk_rows16_launch(const LkRows16& a, bool dual, bool q5, hipStream_t stream) {
     if (a.m < 1 || a.m > MAX_TOKS || a.nb < 1 || a.count < 1 || a.count > 3 || (dual && a.count != 2)) return LK_ERR_ARG;
     if (dual && a.n[0] != a.n[1]) return LK_ERR_ARG;
+    if (a.q81_dst && (!dual || a.n[0] % 32 != 0 || (a.nb != 8 && a.nb != 16) || a.q81_stride < a.n[0] / 32)) return LK_ERR_ARG;
     int rc;
     if (dual) rc = q5 ? launch<true, true>(a, stream) : launch<true, false>(a, stream);
     else rc = q5 ? launch<false, true>(a, stream) : launch<false, false>(a, stream);

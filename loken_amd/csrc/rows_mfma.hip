@@ -840,6 +840,31 @@ extern "C" int lk_dense_q4k_rows_multi(const void* const* weights, float* const*
     return LK_OK;
 }
 
+// Gate and up in one launch with the result handed on as Q8_1: q8_1_out[m][size_n / 32] blocks =
+// lk_quantize_q8_1(act(gate . x) * (up . x)), byte for byte, so the down projection of a layer reads it
+// without the f32 round trip and the quantizer launch in between (what lk_mmvq_pair_act_q8_1 is to the
+// mat-vec pair launch). The 16-row-tile kernel at four tiles per workgroup: at most 16 rows, rows of 2048
+// or 4096 values, size_n a multiple of 32; anything else returns LK_ERR_ARG (take the f32 form and the
+// quantizer). q5 != 0: Q5_K. No counterpart in the reference, whose dense_q4k_imma_m8_act_mul writes f32
+// (src/inference/moe_cuda/dense/imma.rs:320-400).
+extern "C" int lk_dense_q4k_rows_actmul_q8_1(const void* gate, const void* up, const void* q8_1, void* q8_1_out, int size_m,
+                                             int size_n, int size_k, int use_gelu, int q5, void* stream) {
+    if (size_m == 0 || size_n == 0) return LK_OK;
+    if (!gate || !up || !q8_1 || !q8_1_out || size_m < 0 || size_n < 0 || size_n % 32 != 0 || size_k <= 0 ||
+        size_k % 256 != 0 || ((((uintptr_t)gate) | ((uintptr_t)up)) & 15) != 0 ||
+        ((((uintptr_t)q8_1) | ((uintptr_t)q8_1_out)) & 3) != 0)
+        return LK_ERR_ARG;
+    const int nb = size_k / 256;
+    if ((nb != 8 && nb != 16) || !lk_rows16_serves(size_m, nb)) return LK_ERR_ARG;
+    LkRows16 r{};
+    r.w[0] = (const uint8_t*)gate; r.w[1] = (const uint8_t*)up;
+    r.n[0] = r.n[1] = size_n;
+    r.count = 2;
+    r.y = (const uint8_t*)q8_1; r.nb = nb; r.m = size_m; r.stride_y = size_k / 32; r.gelu = use_gelu ? 1 : 0;
+    r.q81_dst = (uint8_t*)q8_1_out; r.q81_stride = size_n / 32;
+    return lk_rows16_launch(r, true, q5 != 0, (hipStream_t)stream);
+}
+
 // The Q5_K siblings (loken_dense_q5k_imma_m8_plain / _actmul, declared src/inference/moe_cuda/mod.rs:459-466,
 // picked by dtype at src/inference/moe_cuda/dense/imma.rs:113-116,362-365): the same kernels with the
 // fifth-bit plane folded into the codes.

@@ -271,6 +271,19 @@ def dense_q4k_rows_actmul(gate: torch.Tensor, up: torch.Tensor, x: torch.Tensor,
     return out
 
 
+def dense_q4k_rows_actmul_q8_1(gate: torch.Tensor, up: torch.Tensor, x: torch.Tensor, n: int, use_gelu: bool,
+                               q5: bool = False) -> torch.Tensor:
+    """dense_q4k_rows_actmul with the result as Q8_1 rows ``[rows, n / 32, 36]`` (what the down projection
+    reads): at most 16 rows, k 2048 or 4096, n a multiple of 32."""
+    rows, k = x.shape
+    q = quantize_q8_1_rows(x, k_padded=k)
+    out = torch.empty((rows, n // 32, 36), dtype=torch.uint8, device=x.device)
+    _lib.check("lk_dense_q4k_rows_actmul_q8_1",
+               _lib.load().lk_dense_q4k_rows_actmul_q8_1(gate.data_ptr(), up.data_ptr(), q.data_ptr(), out.data_ptr(), rows, n,
+                                                         k, 1 if use_gelu else 0, 1 if q5 else 0, _stream()))
+    return out
+
+
 def dense_q6k_rows(weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tensor:
     """``[rows, k]`` f32 x Q6_K weight ``[n, k]`` -> ``[rows, n]`` f32 on the matrix unit, rows
     quantized to plain Q8_1 first."""

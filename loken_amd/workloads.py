@@ -437,26 +437,31 @@ def decode_1p7b(args, dev):
     fused_rows = 3 <= b <= 16 and args.mid_rows == "auto"
     matvec = matvec and not fused_rows
 
+    rows_h_q81 = torch.empty((b, ffn // 32, 36), dtype=torch.uint8, device=dev) if fused_rows else None
+
     def add_fused_rows(g, k, wtype, ns):
         nonlocal total_bytes
         weights = [mk.make(wtype, n, k) for n in ns]
         keep.extend(weights)
         total_bytes += sum(synth.weight_bytes(wtype, n, k) for n in ns)
         x = acts[g]
+        used["rows"] += len(ns)
+        if g == "h":   # `down` reads the Q8_1 rows the gate + up launch wrote
+            out = torch.empty((b, ns[0]), device=dev)
+            keep.append(out)
+            plan.append(("status", L.lk_dense_q6k_rows, (weights[0].data_ptr(), rows_h_q81.data_ptr(), out.data_ptr(), b, ns[0], k, s)))
+            return
         q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
         keep.append(q)
         plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s)))
-        used["rows"] += len(ns)
         if wtype == Q6K:
             for w, n in zip(weights, ns):
                 out = torch.empty((b, n), device=dev)
                 keep.append(out)
                 plan.append(("status", L.lk_dense_q6k_rows, (w.data_ptr(), q.data_ptr(), out.data_ptr(), b, n, k, s)))
         elif g == "x2":
-            out = torch.empty((b, ns[0]), device=dev)
-            keep.append(out)
-            plan.append(("status", L.lk_dense_q4k_rows_actmul,
-                         (weights[0].data_ptr(), weights[1].data_ptr(), q.data_ptr(), out.data_ptr(), b, ns[0], k, 0, s)))
+            plan.append(("status", L.lk_dense_q4k_rows_actmul_q8_1,
+                         (weights[0].data_ptr(), weights[1].data_ptr(), q.data_ptr(), rows_h_q81.data_ptr(), b, ns[0], k, 0, 0, s)))
         else:
             outs = [torch.empty((b, n), device=dev) for n in ns]
             vx = (lib.C.c_void_p * len(ns))(*[w.data_ptr() for w in weights])
@@ -591,8 +596,8 @@ def decode_1p7b(args, dev):
                              f"lm_head), batch {b}, 28 layers",
                  "path": "mat-vec (fused: q + k + v, o from f32 rows; gate + up as the pair launch that writes down's Q8_1 rows)" if paired
                          else "mat-vec (fused; own quantizer launch for rows over 8192 values)" if matvec
-                         else "16-row tiles on the matrix unit: q + k + v in one launch, o, gate + up with SiLU in one, down, lm_head, "
-                              "each after a Q8_1 quantizer launch" if fused_rows
+                         else "16-row tiles on the matrix unit: q + k + v in one launch, o, gate + up with SiLU in one launch that writes "
+                              "the Q8_1 rows down reads, down, lm_head; a Q8_1 quantizer launch before the others" if fused_rows
                          else f"linears on the matrix-unit rows kernels: {used['rows']}, as mat-vec slices of eight rows: "
                               f"{used['matvec']}, on the tiled matmul: {used['tiled']}",
                  "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline)

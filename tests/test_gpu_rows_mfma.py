@@ -273,6 +273,33 @@ def test_gate_and_up_of_many_row_tiles(m, k, n):
     assert_close(ops.dense_q4k_rows(gate[:64 * (k // 256) * 144], x, 64).cpu().numpy(), oracle.ob_matmul(Q4K, x.cpu().numpy(), w, 64))
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 2048, 32), (3, 4096, 96), (4, 2048, 6144), (8, 4096, 14336), (8, 2048, 160),
+                                   (9, 4096, 64), (13, 2048, 6144), (16, 4096, 4128)])
+@pytest.mark.parametrize("q5", [False, True])
+def test_gate_and_up_handed_on_as_q8_1_rows_are_the_quantizers_bytes(m, k, n, q5):
+    """lk_dense_q4k_rows_actmul_q8_1 against lk_dense_q4k_rows_actmul followed by lk_quantize_q8_1, SiLU and GELU."""
+    wt = lib.TYPE_Q5_K if q5 else Q4K
+    gate, up = dev(synth.weight(wt, n, k, seed=77, stream=1)), dev(synth.weight(wt, n, k, seed=77, stream=2))
+    x = dev(synth.activation(m, k, seed=77) * np.float32(3.0))
+    for gelu in (False, True):
+        h = ops.dense_q4k_rows_actmul(gate, up, x, n, gelu, q5=q5)
+        want = ops.quantize_q8_1_rows(h, k_padded=n)
+        got = ops.dense_q4k_rows_actmul_q8_1(gate, up, x, n, gelu, q5=q5)
+        assert torch.equal(got.reshape(-1), want.reshape(-1))
+
+
+def test_gate_and_up_as_q8_1_refuses_what_its_kernel_does_not_take():
+    gate = dev(synth.weight(Q4K, 64, 1024, seed=78, stream=1))
+    with pytest.raises(lib.LokenError):   # rows of 1024 values
+        ops.dense_q4k_rows_actmul_q8_1(gate, gate, dev(synth.activation(4, 1024, seed=78)), 64, False)
+    gate = dev(synth.weight(Q4K, 48, 2048, seed=78, stream=1))
+    with pytest.raises(lib.LokenError):   # 48 output rows: not whole blocks
+        ops.dense_q4k_rows_actmul_q8_1(gate, gate, dev(synth.activation(4, 2048, seed=78)), 48, False)
+    gate = dev(synth.weight(Q4K, 64, 2048, seed=78, stream=1))
+    with pytest.raises(lib.LokenError):   # 17 rows
+        ops.dense_q4k_rows_actmul_q8_1(gate, gate, dev(synth.activation(17, 2048, seed=78)), 64, False)
+
+
 @pytest.mark.parametrize("m,k,n", [(1, 256, 1), (2, 512, 15), (3, 768, 17), (4, 1024, 33), (4, 14336, 48), (5, 256, 16), (7, 1280, 100),
                                    (8, 6144, 500), (6, 2048, 8300), (3, 512, 8300), (8, 512, 16500), (4, 256, 16500),
                                    (9, 2048, 17), (12, 6144, 500), (16, 4096, 100), (16, 2048, 8300), (13, 2048, 16500)])
