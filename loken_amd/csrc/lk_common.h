@@ -209,9 +209,11 @@ const LkDevice& lk_device();
 int lk_q4k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y,
                      int ldd, hipStream_t stream);
 
-// Q4_K x ONE activation row with the row's codes held in registers (mmvq_reg.hip): rows of at most
-// 16 super-blocks. Up to four matrices over one activation; `act_f32` non-zero: `act` is the f32
-// row, quantized by every workgroup itself. LK_* status.
+// Q4_K x one or two activation rows with the rows' codes held in registers (mmvq_reg.hip): weight rows of
+// at most 16 super-blocks. Up to four matrices over the activation; `act_f32` non-zero: `act` holds f32
+// rows, quantized by every workgroup itself. `batch` rows, act_stride Q8_1 blocks (floats) apart, their
+// outputs dst_stride elements apart. LK_* status.
+#define LK_REG_MAX_BATCH 2
 struct LkRegMulti {
     const uint8_t* vx[4];
     void* dst[4];
@@ -220,11 +222,13 @@ struct LkRegMulti {
     int count;
 };
 bool lk_q4k_reg_serves(int nb);
-int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, int dst_type, hipStream_t stream);
-// The gate/up pair over one activation row: dst = act(gate . x) * (up . x) as f32 / bf16
-// (`dst_q8_1` false) or as Q8_1 blocks of 32 consecutive rows (true; n a multiple of 32).
+int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, int dst_type, int batch, int act_stride,
+                     int dst_stride, hipStream_t stream);
+// The gate/up pair over the activation rows: dst = act(gate . x) * (up . x) as f32 / bf16 (`dst_q8_1`
+// false; rows dst_stride elements apart) or as Q8_1 blocks of 32 consecutive rows (true; n a multiple of
+// 32; rows dst_stride blocks apart).
 int lk_q4k_reg_pair(const uint8_t* gate, const uint8_t* up, const void* act, int act_f32, void* dst, int dst_type,
-                    bool dst_q8_1, int nb, int n, int act_fn, hipStream_t stream);
+                    bool dst_q8_1, int nb, int n, int act_fn, int batch, int act_stride, int dst_stride, hipStream_t stream);
 
 // The 32-value nibble formats (mmvq_legacy.hip); status LK_*.
 bool lk_is_legacy_type(int wtype);

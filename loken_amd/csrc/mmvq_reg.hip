@@ -80,56 +80,74 @@ static __device__ __forceinline__ float row_share(const RowFrag& f, const Slice&
 // issued behind the activation's loads and ahead of everything that waits for them: loads return in
 // issue order, so the small activation must go first and must not wait for weights.
 // unit = 4 * slot + p: which 72 bytes of the Q8_1 row (64 bytes of the LDS image) are the lane's.
-template <bool ACT_F32, class First>
-static __device__ __forceinline__ void slice_load(Slice& s, gbytes_t act, int nb, int unit, bool valid, uint8_t* lds,
-                                                  First&& first_loads) {
+// B activation rows, `act_stride` bytes apart, into B slices (the f32 form: B images of LDS_BYTES).
+template <bool ACT_F32, int B, class First>
+static __device__ __forceinline__ void slice_load(Slice (&s)[B], gbytes_t act, size_t act_stride, int nb, int unit, bool valid,
+                                                  uint8_t* lds, First&& first_loads) {
 #pragma clang fp contract(off)
     if (!ACT_F32) {
         // (cast back from the global address space: the compiler keeps track of where it came from)
-        const uint8_t* ap = (const uint8_t*)(act + (valid ? 72 * unit : 0));
-        const uint32_t head0 = *(const uint32_t*)ap;
-        s.a00 = *(const uint4_a4*)(ap + 4);
-        s.a01 = *(const uint4_a4*)(ap + 20);
-        const uint32_t head1 = *(const uint32_t*)(ap + 36);
-        s.a10 = *(const uint4_a4*)(ap + 40);
-        s.a11 = *(const uint4_a4*)(ap + 56);
+        uint32_t head0[B], head1[B];
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            const uint8_t* ap = (const uint8_t*)(act + b * act_stride + (valid ? 72 * unit : 0));
+            head0[b] = *(const uint32_t*)ap;
+            s[b].a00 = *(const uint4_a4*)(ap + 4);
+            s[b].a01 = *(const uint4_a4*)(ap + 20);
+            head1[b] = *(const uint32_t*)(ap + 36);
+            s[b].a10 = *(const uint4_a4*)(ap + 40);
+            s[b].a11 = *(const uint4_a4*)(ap + 56);
+        }
         load_fence((const void*)lds);
         first_loads();
         load_fence((const void*)lds);
-        slice_finish(s, f16_bits_to_f32(head0 & 0xFFFFu), f16_bits_to_f32(head1 & 0xFFFFu));
+#pragma unroll
+        for (int b = 0; b < B; ++b) slice_finish(s[b], f16_bits_to_f32(head0[b] & 0xFFFFu), f16_bits_to_f32(head1[b] & 0xFFFFu));
         return;
     }
     // f32 row: item t is four values, eight consecutive items (lanes) are one Q8_1 block
     const int items = nb * 64;
-    float4 v[2];
+    float4 v[B][2];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) v[u] = *(const float4*)(const uint8_t*)(act + 16 * min((int)threadIdx.x + u * RT, items - 1));
+    for (int b = 0; b < B; ++b)
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            v[b][u] = *(const float4*)(const uint8_t*)(act + b * act_stride + 16 * min((int)threadIdx.x + u * RT, items - 1));
     load_fence((const void*)lds);
     first_loads();
     load_fence((const void*)lds);
-    float* scales = (float*)(lds + LDS_CODES);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        const int item = threadIdx.x + u * RT;
-        if (item < items) {   // whole waves: items is a multiple of 64
-            const float amax = max8(fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w))));
-            const float d = amax / 127.0f;
-            const float inv = d != 0.0f ? 1.0f / d : 0.0f;
-            const int q0 = (int)roundf(v[u].x * inv), q1 = (int)roundf(v[u].y * inv);
-            const int q2 = (int)roundf(v[u].z * inv), q3 = (int)roundf(v[u].w * inv);
-            *(uint32_t*)(lds + 4 * item) = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) |
-                                           ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
-            if ((item & 7) == 0) scales[item >> 3] = __half2float(__float2half_rn(d));
+    for (int b = 0; b < B; ++b) {
+        uint8_t* img = lds + b * LDS_BYTES;
+        float* scales = (float*)(img + LDS_CODES);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int item = threadIdx.x + u * RT;
+            if (item < items) {   // whole waves: items is a multiple of 64
+                const float4 x = v[b][u];
+                const float amax = max8(fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+                const float d = amax / 127.0f;
+                const float inv = d != 0.0f ? 1.0f / d : 0.0f;
+                const int q0 = (int)roundf(x.x * inv), q1 = (int)roundf(x.y * inv);
+                const int q2 = (int)roundf(x.z * inv), q3 = (int)roundf(x.w * inv);
+                *(uint32_t*)(img + 4 * item) = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) |
+                                               ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
+                if ((item & 7) == 0) scales[item >> 3] = __half2float(__float2half_rn(d));
+            }
         }
     }
     __syncthreads();
-    const uint8_t* ap = lds + (valid ? 64 * unit : 0);
-    s.a00 = *(const uint4*)(ap);
-    s.a01 = *(const uint4*)(ap + 16);
-    s.a10 = *(const uint4*)(ap + 32);
-    s.a11 = *(const uint4*)(ap + 48);
-    const float2 dd = *(const float2*)(scales + (valid ? 2 * unit : 0));
-    slice_finish(s, dd.x, dd.y);
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+        const uint8_t* img = lds + b * LDS_BYTES;
+        const uint8_t* ap = img + (valid ? 64 * unit : 0);
+        s[b].a00 = *(const uint4*)(ap);
+        s[b].a01 = *(const uint4*)(ap + 16);
+        s[b].a10 = *(const uint4*)(ap + 32);
+        s[b].a11 = *(const uint4*)(ap + 48);
+        const float2 dd = *(const float2*)((const float*)(img + LDS_CODES) + (valid ? 2 * unit : 0));
+        slice_finish(s[b], dd.x, dd.y);
+    }
 }
 
 static __device__ __forceinline__ void store_out(void* dst, int dst_type, size_t at, float v) {
@@ -161,10 +179,11 @@ struct Geo {
 
 // Up to four matrices over one activation row. A tile is R * RP consecutive rows of one matrix;
 // wave g of the grid takes tiles g, g + waves, ...
-template <int R, int RP, bool ACT_F32>
+// B: activation rows (1 or 2), act_stride bytes apart; their outputs dst_stride elements apart.
+template <int R, int RP, bool ACT_F32, int B>
 __global__ __launch_bounds__(RT) void q4k_reg_kernel(RegArgs a, const uint8_t* __restrict__ act, int nb, int dst_type,
-                                                     int waves) {
-    __shared__ __align__(16) uint8_t lds[ACT_F32 ? LDS_BYTES : 16];
+                                                     int waves, int act_stride, int dst_stride) {
+    __shared__ __align__(16) uint8_t lds[ACT_F32 ? B * LDS_BYTES : 16];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     constexpr int TR = R * RP;
     uint32_t flip = 0x80808080u;
@@ -227,29 +246,33 @@ __global__ __launch_bounds__(RT) void q4k_reg_kernel(RegArgs a, const uint8_t* _
     };
 
     int t = (int)blockIdx.x * waves + wave;
-    Slice s;
+    Slice s[B];
     // (a wave without a tile loads the last one rather than nothing: the count of loads ahead of
     // the weights stays the same for every wave)
     relocate(min(t, total - 1));
-    slice_load<ACT_F32>(s, act_g, nb, g.unit, g.valid, lds, [&] { load(min(t, total - 1)); });
+    slice_load<ACT_F32, B>(s, act_g, (size_t)act_stride, nb, g.unit, g.valid, lds, [&] { load(min(t, total - 1)); });
     const bool odd = g.lane & 1;
     while (t < total) {
         void* dst = (void*)(uint8_t*)to_gbytes((uint64_t)cur_dst);
         const float* bias = (const float*)to_gbytes((uint64_t)cur_bias);
         const int row = (t - cur_begin) * TR + g.rp * R, n = cur_n;   // the lane group's first row of the tile
-        if (R == 2) {
-            // even lanes end with the first row's total, odd lanes with the second's
-            float v = group_sum2<Geo<RP>::GROUP>(row_share(f[0], s, sel, g.valid, flip), row_share(f[R - 1], s, sel, g.valid, flip), odd);
-            const int mine = row + (int)odd;
-            if ((g.lane & (Geo<RP>::GROUP - 1)) < 2 && mine < n) {
-                if (bias) v += bias[mine];
-                store_out(dst, dst_type, mine, v);
-            }
-        } else {
-            float v = group_sum<Geo<RP>::GROUP>(row_share(f[0], s, sel, g.valid, flip));
-            if ((g.lane & (Geo<RP>::GROUP - 1)) == 0 && row < n) {
-                if (bias) v += bias[row];
-                store_out(dst, dst_type, row, v);
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            if (R == 2) {
+                // even lanes end with the first row's total, odd lanes with the second's
+                float v = group_sum2<Geo<RP>::GROUP>(row_share(f[0], s[b], sel, g.valid, flip),
+                                                     row_share(f[R - 1], s[b], sel, g.valid, flip), odd);
+                const int mine = row + (int)odd;
+                if ((g.lane & (Geo<RP>::GROUP - 1)) < 2 && mine < n) {
+                    if (bias) v += bias[mine];
+                    store_out(dst, dst_type, (size_t)b * dst_stride + mine, v);
+                }
+            } else {
+                float v = group_sum<Geo<RP>::GROUP>(row_share(f[0], s[b], sel, g.valid, flip));
+                if ((g.lane & (Geo<RP>::GROUP - 1)) == 0 && row < n) {
+                    if (bias) v += bias[row];
+                    store_out(dst, dst_type, (size_t)b * dst_stride + row, v);
+                }
             }
         }
         t += step;
@@ -269,13 +292,16 @@ static __device__ __forceinline__ float act_gelu_tanh(float g) {
 // row are summed together (even lanes gate, odd lanes up) and lane 0 of the group combines them.
 // Q81_OUT: a workgroup owns whole blocks of 32 consecutive rows (wave w rows 4w .. 4w + 3),
 // the 32 results meet in LDS and eight lanes write them as one Q8_1 block with the quantizer's steps.
-template <int RP, bool ACT_F32, bool Q81_OUT>
+// (the two-row forms with Q8_1 output take 135-169 registers, one workgroup per CU; bounded to 128 they
+// spill and measured slower: Llama step at two rows 1.70 against 1.62 ms)
+template <int RP, bool ACT_F32, bool Q81_OUT, int B>
 __global__ __launch_bounds__(RT) void q4k_reg_pair_kernel(const uint8_t* __restrict__ gate, const uint8_t* __restrict__ up,
                                                           const uint8_t* __restrict__ act, void* __restrict__ dst, int nb,
-                                                          int n, int dst_type, int act_fn, int waves) {
+                                                          int n, int dst_type, int act_fn, int waves, int act_stride,
+                                                          int dst_stride) {
 #pragma clang fp contract(off)
-    __shared__ __align__(16) uint8_t lds[(ACT_F32 ? LDS_BYTES : 0) + (Q81_OUT ? 2 * 32 * 4 : 16)];
-    float* meet = (float*)(lds + (ACT_F32 ? LDS_BYTES : 0));   // [2][32]: two blocks in flight
+    __shared__ __align__(16) uint8_t lds[(ACT_F32 ? B * LDS_BYTES : 0) + (Q81_OUT ? B * 2 * 32 * 4 : 16)];
+    float* meet = (float*)(lds + (ACT_F32 ? B * LDS_BYTES : 0));   // [B][2][32]: two blocks in flight
     const Geo<RP> g(nb);
     const Q4KScaleSel sel(g.p);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -296,16 +322,20 @@ __global__ __launch_bounds__(RT) void q4k_reg_pair_kernel(const uint8_t* __restr
         const float u = dpp_f32<0xB1>(both);   // the odd neighbour's total
         return (act_fn == 0 ? act_silu(both) : act_gelu_tanh(both)) * u;
     };
-    Slice s;
+    Slice s[B];
     if (!Q81_OUT) {
         // tiles of RP rows, wave-strided
         const int tiles = (n + RP - 1) / RP, step = (int)gridDim.x * waves;
         int t = (int)blockIdx.x * waves + wave;
-        slice_load<ACT_F32>(s, to_gbytes(act), nb, g.unit, g.valid, lds, [&] { load(min(t, tiles - 1) * RP + g.rp); });
+        slice_load<ACT_F32, B>(s, to_gbytes(act), (size_t)act_stride, nb, g.unit, g.valid, lds,
+                               [&] { load(min(t, tiles - 1) * RP + g.rp); });
         while (t < tiles) {
             const int row = t * RP + g.rp;
-            const float v = value(s);
-            if ((g.lane & (Geo<RP>::GROUP - 1)) == 0 && row < n) store_out(dst, dst_type, row, v);
+#pragma unroll
+            for (int b = 0; b < B; ++b) {
+                const float v = value(s[b]);
+                if ((g.lane & (Geo<RP>::GROUP - 1)) == 0 && row < n) store_out(dst, dst_type, (size_t)b * dst_stride + row, v);
+            }
             t += step;
             if (t < tiles) load(t * RP + g.rp);
         }
@@ -324,31 +354,36 @@ __global__ __launch_bounds__(RT) void q4k_reg_pair_kernel(const uint8_t* __restr
         row_load(bg[slot], wg + at, g.hdr_off, g.qs_off);
         row_load(bu[slot], wu + at, g.hdr_off, g.qs_off);
     };
-    slice_load<ACT_F32>(s, to_gbytes(act), nb, g.unit, g.valid, lds, [&] {
+    slice_load<ACT_F32, B>(s, to_gbytes(act), (size_t)act_stride, nb, g.unit, g.valid, lds, [&] {
 #pragma unroll
         for (int i = 0; i < D; ++i) load_pass(i, min(b, blocks - 1), i);
     });
     int half = 0;
     for (; b < blocks; b += gridDim.x) {
-        float val[PASSES];
+        float val[B][PASSES];
         const int nb_next = b + (int)gridDim.x;
 #pragma unroll
         for (int i = 0; i < PASSES; ++i) {
-            const float both = group_sum2<Geo<RP>::GROUP>(row_share(bg[i % D], s, sel, g.valid, flip),
-                                                          row_share(bu[i % D], s, sel, g.valid, flip), odd);
-            const float u = dpp_f32<0xB1>(both);   // the odd neighbour's total
-            val[i] = (act_fn == 0 ? act_silu(both) : act_gelu_tanh(both)) * u;
+#pragma unroll
+            for (int r = 0; r < B; ++r) {
+                const float both = group_sum2<Geo<RP>::GROUP>(row_share(bg[i % D], s[r], sel, g.valid, flip),
+                                                              row_share(bu[i % D], s[r], sel, g.valid, flip), odd);
+                const float u = dpp_f32<0xB1>(both);   // the odd neighbour's total
+                val[r][i] = (act_fn == 0 ? act_silu(both) : act_gelu_tanh(both)) * u;
+            }
             if (i + D < PASSES) load_pass(i % D, b, i + D);
             else if (nb_next < blocks) load_pass(i % D, nb_next, i + D - PASSES);
         }
         if ((g.lane & (Geo<RP>::GROUP - 1)) == 0) {
 #pragma unroll
-            for (int i = 0; i < PASSES; ++i) meet[half * 32 + 4 * wave + i * RP + g.rp] = val[i];
+            for (int r = 0; r < B; ++r)
+#pragma unroll
+                for (int i = 0; i < PASSES; ++i) meet[(r * 2 + half) * 32 + 4 * wave + i * RP + g.rp] = val[r][i];
         }
         __syncthreads();   // every wave of the workgroup has delivered its four
-        if (wave == 0 && g.lane < 8) {
-            const int l8 = g.lane;
-            const float4 v = *(const float4*)(meet + half * 32 + 4 * l8);
+        if (wave == 0 && g.lane < 8 * B) {
+            const int l8 = g.lane & 7, r = g.lane >> 3;
+            const float4 v = *(const float4*)(meet + (r * 2 + half) * 32 + 4 * l8);
             const float amax = max8(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
             const float d = amax / 127.0f;
             const float inv = d != 0.0f ? 1.0f / d : 0.0f;
@@ -356,7 +391,7 @@ __global__ __launch_bounds__(RT) void q4k_reg_pair_kernel(const uint8_t* __restr
             const int q2 = (int)roundf(v.z * inv), q3 = (int)roundf(v.w * inv);
             int quad;
             const int sum = sum8(q0 + q1 + q2 + q3, quad);
-            uint32_t* out = (uint32_t*)dst + (size_t)b * 9;
+            uint32_t* out = (uint32_t*)dst + ((size_t)r * dst_stride + b) * 9;
             out[1 + l8] = (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) |
                           ((uint32_t)(q3 & 0xFF) << 24);
             if (l8 == 0) {
@@ -410,11 +445,11 @@ __global__ __launch_bounds__(RT) void q4k_reg_moe_pair_kernel(const uint8_t* __r
     };
     const int tiles = (n + RP - 1) / RP, step = (int)gridDim.x * waves;
     int t = (int)blockIdx.x * waves + wave;
-    Slice s;
-    slice_load<true>(s, act, nb, g.unit, g.valid, lds, [&] { load(min(t, tiles - 1) * RP + g.rp); });
+    Slice s[1];
+    slice_load<true, 1>(s, act, 0, nb, g.unit, g.valid, lds, [&] { load(min(t, tiles - 1) * RP + g.rp); });
     while (t < tiles) {
         const int row = t * RP + g.rp;
-        const float both = group_sum2<Geo<RP>::GROUP>(row_share(fg, s, sel, g.valid, flip), row_share(fu, s, sel, g.valid, flip), odd);
+        const float both = group_sum2<Geo<RP>::GROUP>(row_share(fg, s[0], sel, g.valid, flip), row_share(fu, s[0], sel, g.valid, flip), odd);
         const float u = dpp_f32<0xB1>(both);   // the odd neighbour's total
         if ((g.lane & (Geo<RP>::GROUP - 1)) == 0 && row < n) dst[row] = lk_gated(m.act, both, u, (size_t)e * n + row);
         t += step;
@@ -435,8 +470,9 @@ static Shape shape_for(bool act_f32) {
     return Shape{waves, lk_device().cus * per_cu};
 }
 
-template <int R, int RP>
-static int launch_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, int dst_type, hipStream_t s) {
+template <int R, int RP, int B>
+static int launch_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, int dst_type, int act_stride, int dst_stride,
+                        hipStream_t s) {
     RegArgs a{};
     int total = 0;
     for (int i = 0; i < 4; ++i) {
@@ -454,15 +490,17 @@ static int launch_multi(const LkRegMulti& m, const void* act, int act_f32, int n
     static const int forced_grid = lk_tune_env("LK_TUNE_REG_GRID");
     const dim3 grid(forced_grid > 0 ? (forced_grid < need ? forced_grid : need) : need < sh.cap ? need : sh.cap), block(sh.waves * 64);
     if (act_f32)
-        hipLaunchKernelGGL((q4k_reg_kernel<R, RP, true>), grid, block, 0, s, a, (const uint8_t*)act, nb, dst_type, sh.waves);
+        hipLaunchKernelGGL((q4k_reg_kernel<R, RP, true, B>), grid, block, 0, s, a, (const uint8_t*)act, nb, dst_type, sh.waves,
+                           act_stride, dst_stride);
     else
-        hipLaunchKernelGGL((q4k_reg_kernel<R, RP, false>), grid, block, 0, s, a, (const uint8_t*)act, nb, dst_type, sh.waves);
+        hipLaunchKernelGGL((q4k_reg_kernel<R, RP, false, B>), grid, block, 0, s, a, (const uint8_t*)act, nb, dst_type, sh.waves,
+                           act_stride, dst_stride);
     return lk_launch_status();
 }
 
-template <int RP>
+template <int RP, int B>
 static int launch_pair(const uint8_t* gate, const uint8_t* up, const void* act, int act_f32, void* dst, int dst_type,
-                       bool q81, int nb, int n, int act_fn, hipStream_t s) {
+                       bool q81, int nb, int n, int act_fn, int act_stride, int dst_stride, hipStream_t s) {
     const uint8_t* y = (const uint8_t*)act;
     if (q81) {
         // a workgroup of RW waves per block of 32 rows
@@ -470,18 +508,22 @@ static int launch_pair(const uint8_t* gate, const uint8_t* up, const void* act, 
         const int blocks = n / 32, cap = sh.cap;
         const dim3 grid(blocks < cap ? blocks : cap);
         if (act_f32)
-            hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, true, true>), grid, dim3(RT), 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves);
+            hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, true, true, B>), grid, dim3(RT), 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves,
+                               act_stride, dst_stride);
         else
-            hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, false, true>), grid, dim3(RT), 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves);
+            hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, false, true, B>), grid, dim3(RT), 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves,
+                               act_stride, dst_stride);
         return lk_launch_status();
     }
     const Shape sh = shape_for(act_f32 != 0);
     const int tiles = (n + RP - 1) / RP, need = (tiles + sh.waves - 1) / sh.waves;
     const dim3 grid(need < sh.cap ? need : sh.cap), block(sh.waves * 64);
     if (act_f32)
-        hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, true, false>), grid, block, 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves);
+        hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, true, false, B>), grid, block, 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves,
+                           act_stride, dst_stride);
     else
-        hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, false, false>), grid, block, 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves);
+        hipLaunchKernelGGL((q4k_reg_pair_kernel<RP, false, false, B>), grid, block, 0, s, gate, up, y, dst, nb, n, dst_type, act_fn, sh.waves,
+                           act_stride, dst_stride);
     return lk_launch_status();
 }
 
@@ -492,8 +534,9 @@ bool lk_q4k_reg_serves(int nb) {
     return nb >= 1 && nb <= MAX_NB && !off;
 }
 
-int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, int dst_type, hipStream_t stream) {
-    if (!lk_q4k_reg_serves(nb) || m.count < 1 || m.count > 4) return LK_ERR_ARG;
+template <int B>
+static int multi_rows(const LkRegMulti& m, const void* act, int act_f32, int nb, int dst_type, int act_bytes, int dst_stride,
+                      hipStream_t stream) {
     const int rp = q4k_rows_per_pass(nb);
     // Two rows per wave tile while every wave still gets at most one tile (the launch is one round
     // of loads and a tail: fewer, fatter waves), one row per tile when waves stream several.
@@ -508,10 +551,20 @@ int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, 
     // tiles per wave measured slower, Qwen3-1.7B step 0.598 against 0.586 ms)
     const bool two = forced ? forced == 2 : rp == 1 && rows <= waves_at_once * 2;
     switch (rp) {
-        case 1: return two ? launch_multi<2, 1>(m, act, act_f32, nb, dst_type, stream) : launch_multi<1, 1>(m, act, act_f32, nb, dst_type, stream);
-        case 2: return two ? launch_multi<2, 2>(m, act, act_f32, nb, dst_type, stream) : launch_multi<1, 2>(m, act, act_f32, nb, dst_type, stream);
-        default: return launch_multi<1, 4>(m, act, act_f32, nb, dst_type, stream);
+        case 1: return two ? launch_multi<2, 1, B>(m, act, act_f32, nb, dst_type, act_bytes, dst_stride, stream)
+                           : launch_multi<1, 1, B>(m, act, act_f32, nb, dst_type, act_bytes, dst_stride, stream);
+        case 2: return two ? launch_multi<2, 2, B>(m, act, act_f32, nb, dst_type, act_bytes, dst_stride, stream)
+                           : launch_multi<1, 2, B>(m, act, act_f32, nb, dst_type, act_bytes, dst_stride, stream);
+        default: return launch_multi<1, 4, B>(m, act, act_f32, nb, dst_type, act_bytes, dst_stride, stream);
     }
+}
+
+int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, int dst_type, int batch, int act_stride,
+                     int dst_stride, hipStream_t stream) {
+    if (!lk_q4k_reg_serves(nb) || m.count < 1 || m.count > 4 || batch < 1 || batch > LK_REG_MAX_BATCH) return LK_ERR_ARG;
+    const int act_bytes = act_stride * (act_f32 ? (int)sizeof(float) : Q81_BYTES);
+    return batch == 1 ? multi_rows<1>(m, act, act_f32, nb, dst_type, act_bytes, dst_stride, stream)
+                      : multi_rows<2>(m, act, act_f32, nb, dst_type, act_bytes, dst_stride, stream);
 }
 
 template <int RP>
@@ -540,12 +593,20 @@ int lk_q4k_reg_moe_pair(const uint8_t* gate, const uint8_t* up, const float* act
     }
 }
 
-int lk_q4k_reg_pair(const uint8_t* gate, const uint8_t* up, const void* act, int act_f32, void* dst, int dst_type,
-                    bool dst_q8_1, int nb, int n, int act_fn, hipStream_t stream) {
-    if (!lk_q4k_reg_serves(nb) || n < 1 || (dst_q8_1 && n % 32 != 0)) return LK_ERR_ARG;
+template <int B>
+static int pair_rows(const uint8_t* gate, const uint8_t* up, const void* act, int act_f32, void* dst, int dst_type, bool dst_q8_1,
+                     int nb, int n, int act_fn, int act_bytes, int dst_stride, hipStream_t stream) {
     switch (q4k_rows_per_pass(nb)) {
-        case 1: return launch_pair<1>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, stream);
-        case 2: return launch_pair<2>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, stream);
-        default: return launch_pair<4>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, stream);
+        case 1: return launch_pair<1, B>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, act_bytes, dst_stride, stream);
+        case 2: return launch_pair<2, B>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, act_bytes, dst_stride, stream);
+        default: return launch_pair<4, B>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, act_bytes, dst_stride, stream);
     }
+}
+
+int lk_q4k_reg_pair(const uint8_t* gate, const uint8_t* up, const void* act, int act_f32, void* dst, int dst_type,
+                    bool dst_q8_1, int nb, int n, int act_fn, int batch, int act_stride, int dst_stride, hipStream_t stream) {
+    if (!lk_q4k_reg_serves(nb) || n < 1 || (dst_q8_1 && n % 32 != 0) || batch < 1 || batch > LK_REG_MAX_BATCH) return LK_ERR_ARG;
+    const int act_bytes = act_stride * (act_f32 ? (int)sizeof(float) : Q81_BYTES);
+    return batch == 1 ? pair_rows<1>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, act_bytes, dst_stride, stream)
+                      : pair_rows<2>(gate, up, act, act_f32, dst, dst_type, dst_q8_1, nb, n, act_fn, act_bytes, dst_stride, stream);
 }
