@@ -454,8 +454,8 @@ def main() -> int:
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC.get((args.plan, b, args.layers)),
-                "kernel": (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<1,1,true> (q+k+v, 512 workgroups), q4k_reg_kernel<2,1,true> (o, 256), "
-                           f"q4k_reg_pair_kernel<1,true,true> (gate+up)") if kind == "auto" and b == 1
+                "kernel": (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<1,1,true,1> (q+k+v, 512 workgroups), q4k_reg_kernel<2,1,true,1> (o, 256), "
+                           f"q4k_reg_pair_kernel<1,true,true,1> (gate+up)") if kind == "auto" and b == 1
                           else (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
                                 f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if kind == "auto"
                           else ("Q4_K launches of a layer on the matrix unit, 16-row tiles: q4k_rows16_kernel<false,false,4,2> (q+k+v; o), "
