@@ -456,7 +456,7 @@ def main() -> int:
                 "traffic": MEASURED_TRAFFIC.get((args.plan, b, args.layers)),
                 "kernel": (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<1,1,true,1> (q+k+v, 512 workgroups), q4k_reg_kernel<2,1,true,1> (o, 256), "
                            f"q4k_reg_pair_kernel<1,true,true,1> (gate+up)") if kind == "auto" and b == 1
-                          else (f"Q4_K mat-vec launches of a layer: mmvq_kernel<EngQ4K,{b},2,float> (q+k+v; o), "
+                          else (f"Q4_K mat-vec launches of a layer: q4k_reg_kernel<1,1,true,2> (q+k+v), q4k_reg_kernel<2,1,true,2> (o), "
                                 f"mmvq_pair_q8_1_kernel<EngQ4K,{b},1,0> (gate+up)") if kind == "auto"
                           else ("Q4_K launches of a layer on the matrix unit, 16-row tiles: q4k_rows16_kernel<false,false,4,2> (q+k+v; o), "
                                 "q4k_rows16_kernel<true,false,4,4> (gate+up)") if kind == "rows"
