@@ -25,12 +25,12 @@ Two more measurements ride in the same JSON line:
   cpu_baseline  loken's served CPU decode path for Q4_K, restated (Q8_K activation, weights repacked
                 eight rows at a time, persistent worker pool), on a bounded sample of the same
                 workload, on this host's cores.
-  gemv_4096     BASELINE config 0 (Q4_K 4096 x 4096, one row) over rotating copies.
-  mmq           BASELINE configs 2a / 2b, the tiled matmul, against the int8 matrix peak.
+  gemv_4096     the benchmark set's configuration 0 (Q4_K 4096 x 4096, one row) over rotating copies.
+  mmq           configurations 2a / 2b, the tiled matmul, against the int8 matrix peak.
   rows-sweep    one --wtype q4_k|q6_k matrix (--rows-n x --cols-k) at 16..2048 rows: the matrix-unit
                 rows kernel against the tiled matmul, and the path QKernelMatMul::forward's mirror takes.
   other_configs the step at 4 and 8 rows, the MoE block at 1 / 16 / 256 tokens and the Qwen3-1.7B step at
-                1 / 16 / 64 rows (BASELINE configs 1, 3, 4), each from a child run of this file.
+                1 / 16 / 64 rows (configurations 1, 3, 4), each from a child run of this file.
   roofline.peak_measured / mmq.peak_measured: what a read-only launch and a register-resident
                 matrix-instruction loop reach on this card (loken_amd/probes.py).
 """
