@@ -58,7 +58,29 @@ struct Args {
     int ldd;              // floats between output rows
     const uint8_t* w2;    // DUAL: the second matrix (same shape); the output is act(w . x) * (w2 . x)
     int gelu;             // DUAL: 0 SiLU, 1 tanh-form GELU
+    // MULTI (the dense launch only): up to two more matrices over the same activation rows, each with its
+    // own output; their row tiles follow the first matrix's in the launch's tile order
+    const uint8_t* w_b = nullptr;
+    const uint8_t* w_c = nullptr;
+    float* dst_b = nullptr;
+    float* dst_c = nullptr;
+    int n_b = 0, n_c = 0, ldd_b = 0, ldd_c = 0;
 };
+
+// Row tile `t` of a launch: which matrix it belongs to, and which of that matrix's tiles it is.
+struct MatRef {
+    const uint8_t* w;
+    float* dst;
+    int n, ldd, tile;
+};
+template <bool MULTI>
+static __device__ __forceinline__ MatRef mat_of(const Args& p, float* dst, int ldd, int t) {
+    if (!MULTI) return {p.w, dst, p.n, ldd, t};
+    const int ta = (p.n + 31) >> 5, tb = (p.n_b + 31) >> 5;
+    if (t < ta) return {p.w, dst, p.n, ldd, t};
+    if (t < ta + tb) return {p.w_b, p.dst_b, p.n_b, p.ldd_b, t - ta};
+    return {p.w_c, p.dst_c, p.n_c, p.ldd_c, t - ta - tb};
+}
 
 // With DUAL a workgroup walks "virtual" tiles: 2 t is row tile t of the first matrix, 2 t + 1 the same
 // rows of the second. The first's reduced sums wait in registers for the second's.
@@ -129,8 +151,9 @@ struct PassRows {
 // row tiles, all of a row's super-blocks in turn, and nothing crosses waves but the tables: rows of
 // at most eight super-blocks, where a four-way split leaves a wave one or two blocks per tile and
 // most of its time in the reduction's barriers.
-template <int G, bool DUAL, bool Q5, bool KSPLIT = true>
+template <int G, bool DUAL, bool Q5, bool KSPLIT = true, bool MULTI = false>
 static __device__ __forceinline__ void q4k_rows_pass(const Args& p, const PassRows& rows, int m_count, uint8_t* lds) {
+    static_assert(!MULTI || (!DUAL && KSPLIT), "several matrices: the dense launch with the super-blocks split over the waves");
     constexpr int TW = 8 * G;   // activation rows a table row holds
     constexpr int NV = 4 * G;   // live accumulator registers
     float* d8_table = (float*)lds;                                   // [nb * 8][TW]
@@ -140,7 +163,7 @@ static __device__ __forceinline__ void q4k_rows_pass(const Args& p, const PassRo
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
-    const int n_tiles = (p.n + 31) >> 5;
+    const int n_tiles = ((p.n + 31) >> 5) + (MULTI ? ((p.n_b + 31) >> 5) + ((p.n_c + 31) >> 5) : 0);
     const size_t row_bytes = (size_t)p.nb * Blk<Q5>::BYTES;
 
     // Activation scales of this pass, zero for the rows the pass does not have. Eight loads are
@@ -193,8 +216,9 @@ static __device__ __forceinline__ void q4k_rows_pass(const Args& p, const PassRo
     const uint8_t* y_lane = rows.y_row(min(l32, m_count - 1)) + 4 + 16 * lh;
 
     auto load = [&](Frag& f, int tile, int kb) {
-        const int row = min((DUAL ? tile >> 1 : tile) * 32 + l32, p.n - 1);
-        const uint8_t* mat = DUAL && (tile & 1) ? p.w2 : p.w;
+        const MatRef mr = mat_of<MULTI>(p, rows.dst, rows.ldd, DUAL ? tile >> 1 : tile);
+        const int row = min(mr.tile * 32 + l32, mr.n - 1);
+        const uint8_t* mat = DUAL && (tile & 1) ? p.w2 : mr.w;
         const uint8_t* bp = (const uint8_t*)(to_gbytes(mat) + row * row_bytes + (size_t)kb * Blk<Q5>::BYTES);
         f.hdr = *(const uint4*)bp;
         if (Q5) f.qh = *(const uint4*)(bp + 16 + 16 * lh);
@@ -348,8 +372,15 @@ static __device__ __forceinline__ void q4k_rows_pass(const Args& p, const PassRo
                 act.kind = p.gelu ? LK_GATE_GELU : LK_GATE_SILU;
                 sum = lk_gated(act, gate_keep[r], sum, 0);
             }
-            const int tok = (v >> 2) * 8 + lh * 4 + (v & 3), row = (DUAL ? t >> 1 : t) * 32 + l32;
-            if (tok < m_count && row < p.n) rows.out_row(tok)[row] = sum;
+            const int tok = (v >> 2) * 8 + lh * 4 + (v & 3);
+            if (MULTI) {   // (dense rows: the pass's row i is row first + i of every output)
+                const MatRef mr = mat_of<MULTI>(p, rows.dst, rows.ldd, t);
+                const int row = mr.tile * 32 + l32;
+                if (tok < m_count && row < mr.n) mr.dst[(size_t)(rows.first + tok) * mr.ldd + row] = sum;
+            } else {
+                const int row = (DUAL ? t >> 1 : t) * 32 + l32;
+                if (tok < m_count && row < p.n) rows.out_row(tok)[row] = sum;
+            }
         }
         __syncthreads();   // the partial tiles may be overwritten (and, past the last tile, the tables)
     };
@@ -381,12 +412,12 @@ static __device__ __forceinline__ void q4k_rows_pass(const Args& p, const PassRo
 }
 
 // Dense: grid y walks the activation in passes of 32 rows.
-template <int G, bool DUAL, bool Q5>
+template <int G, bool DUAL, bool Q5, bool MULTI = false>
 __global__ __launch_bounds__(WG, 2) void q4k_rows_mfma_kernel(Args p) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int m0 = blockIdx.y * TOK;
     const PassRows rows{p.y, p.dst, nullptr, nullptr, m0, p.stride_y, p.ldd};
-    q4k_rows_pass<G, DUAL, Q5>(p, rows, min(TOK, p.m - m0), lds);
+    q4k_rows_pass<G, DUAL, Q5, true, MULTI>(p, rows, min(TOK, p.m - m0), lds);
 }
 
 // Expert-batched: grid y is the expert; its sorted rows [bounds[e], bounds[e + 1]) go through in
@@ -600,7 +631,7 @@ __global__ __launch_bounds__(WG, G == 1 ? 2 : 1) void q4k_rows_staged_kernel(Arg
     }
 }
 
-template <int G, bool DUAL, bool Q5>
+template <int G, bool DUAL, bool Q5, bool MULTI = false>
 int resident_cap(int lds_bytes) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
@@ -611,11 +642,11 @@ int resident_cap(int lds_bytes) {
     if (lds_bytes > lk_device().lds_bytes) {
         r = 0;
     } else if (lds_bytes > 48 * 1024 &&
-               hipFuncSetAttribute((const void*)q4k_rows_mfma_kernel<G, DUAL, Q5>, hipFuncAttributeMaxDynamicSharedMemorySize,
+               hipFuncSetAttribute((const void*)q4k_rows_mfma_kernel<G, DUAL, Q5, MULTI>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    lds_bytes) != hipSuccess) {
         (void)hipGetLastError();
         r = 0;
-    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_mfma_kernel<G, DUAL, Q5>, WG,
+    } else if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, (const void*)q4k_rows_mfma_kernel<G, DUAL, Q5, MULTI>, WG,
                                                             (size_t)lds_bytes) != hipSuccess || r < 1) {
         (void)hipGetLastError();
         r = 1;
@@ -624,16 +655,16 @@ int resident_cap(int lds_bytes) {
     return r;
 }
 
-template <int G, bool DUAL, bool Q5>
+template <int G, bool DUAL, bool Q5, bool MULTI = false>
 int launch_rows(const Args& a, hipStream_t stream) {
     const int lds_bytes = (lds_floats_table<G>(a.nb) + WAVES * 4 * G * 64) * (int)sizeof(float);
-    const int per_cu = resident_cap<G, DUAL, Q5>(lds_bytes);
+    const int per_cu = resident_cap<G, DUAL, Q5, MULTI>(lds_bytes);
     if (per_cu == 0) return LK_ERR_ARG;   // rows too long for the scale tables
-    const int n_tiles = (a.n + 31) / 32, groups = (a.m + TOK - 1) / TOK;
+    const int n_tiles = (a.n + 31) / 32 + (MULTI ? (a.n_b + 31) / 32 + (a.n_c + 31) / 32 : 0), groups = (a.m + TOK - 1) / TOK;
     if (groups > 65535) return LK_ERR_ARG;
     int cap = lk_device().cus * per_cu / groups;
     if (cap < 1) cap = 1;
-    hipLaunchKernelGGL((q4k_rows_mfma_kernel<G, DUAL, Q5>), dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
+    hipLaunchKernelGGL((q4k_rows_mfma_kernel<G, DUAL, Q5, MULTI>), dim3(n_tiles < cap ? n_tiles : cap, groups), dim3(WG), lds_bytes, stream, a);
     return lk_launch_status();
 }
 
@@ -809,8 +840,9 @@ extern "C" void loken_dense_q4k_imma_m8_actmul(const void* gate, const void* up,
 // Up to three Q4_K (q5 != 0: Q5_K) matrices over the same plain Q8_1 rows in one launch (q + k + v of a
 // decode step): outputs[i] is [size_m, sizes_n[i]] f32. The reference issues one
 // loken_dense_q4k_imma_m8_plain per matrix (dense_q4k_imma_m8_matmul, src/inference/moe_cuda/dense/
-// imma.rs:82-135); the results equal those launches' bit for bit. At most 16 rows go out as one
-// launch; more rows (or rows whose codes do not fit in LDS) fall back to one launch per matrix.
+// imma.rs:82-135); the results equal those launches' bit for bit. One launch at any row count (the 16-row
+// tiles up to 16 rows, the 32-row tiles above); rows too long for the kernels' LDS tables fall back to one
+// launch per matrix.
 extern "C" int lk_dense_q4k_rows_multi(const void* const* weights, float* const* outputs, const int* sizes_n, int count,
                                        const void* q8_1, int size_m, int size_k, int q5, void* stream) {
     if (!weights || !outputs || !sizes_n || count < 1 || count > 3) return LK_ERR_ARG;
@@ -831,6 +863,24 @@ extern "C" int lk_dense_q4k_rows_multi(const void* const* weights, float* const*
         if (r.count == 0) return LK_OK;
         r.y = (const uint8_t*)q8_1; r.nb = nb; r.m = size_m; r.stride_y = size_k / 32;
         return lk_rows16_launch(r, false, q5 != 0, (hipStream_t)stream);
+    }
+    if (size_m > 16 && lk_tune_env("LK_TUNE_ROWS_MULTI_OFF") == 0) {
+        // more rows: the 32-row-tile kernel walks the tiles of all the matrices in one launch
+        Args a{};
+        int live = 0;
+        for (int i = 0; i < count; ++i) {
+            if (sizes_n[i] <= 0) continue;
+            if (live == 0) { a.w = (const uint8_t*)weights[i]; a.dst = outputs[i]; a.n = a.ldd = sizes_n[i]; }
+            else if (live == 1) { a.w_b = (const uint8_t*)weights[i]; a.dst_b = outputs[i]; a.n_b = a.ldd_b = sizes_n[i]; }
+            else { a.w_c = (const uint8_t*)weights[i]; a.dst_c = outputs[i]; a.n_c = a.ldd_c = sizes_n[i]; }
+            ++live;
+        }
+        if (live == 0) return LK_OK;
+        a.y = (const uint8_t*)q8_1; a.nb = nb; a.m = size_m; a.stride_y = size_k / 32;
+        if (live > 1) {
+            const int rc = q5 ? launch_rows<4, false, true, true>(a, (hipStream_t)stream) : launch_rows<4, false, false, true>(a, (hipStream_t)stream);
+            if (rc == LK_OK) return rc;
+        }
     }
     for (int i = 0; i < count; ++i) {
         const int rc = rows_plain(weights[i], q8_1, outputs[i], size_m, sizes_n[i], size_k, size_k / 32, sizes_n[i], q5 != 0,

@@ -522,6 +522,15 @@ def decode_1p7b(args, dev):
                              (weights[0].data_ptr(), weights[1].data_ptr(), q.data_ptr(), out.data_ptr(), b, ns[0], k, 0, s)))
                 used["rows"] += 2
                 return
+            if wtype == Q4K and len(ns) > 1:   # q + k + v: one launch over the three matrices
+                outs = [torch.empty((b, n), device=dev) for n in ns]
+                vx = (lib.C.c_void_p * len(ns))(*[w.data_ptr() for w in weights])
+                dst = (lib.C.c_void_p * len(ns))(*[o.data_ptr() for o in outs])
+                nn = (lib.C.c_int * len(ns))(*ns)
+                keep.extend(outs + [vx, dst, nn])
+                plan.append(("status", L.lk_dense_q4k_rows_multi, (vx, dst, nn, len(ns), q.data_ptr(), b, k, 0, s)))
+                used["rows"] += len(ns)
+                return
             for w, n in zip(weights, ns):
                 out = torch.empty((b, n), device=dev)
                 keep.append(out)

@@ -245,7 +245,7 @@ def test_eight_rows_emit_the_exact_integers_on_crafted_inputs(m):
     assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, got.astype(np.int64))
 
 
-@pytest.mark.parametrize("m", [1, 5, 8, 11, 16, 19])
+@pytest.mark.parametrize("m", [1, 5, 8, 11, 16, 19, 32, 33, 70])
 @pytest.mark.parametrize("q5", [False, True])
 def test_three_matrices_in_one_launch_carry_the_single_launches_bits(m, q5):
     """q + k + v: lk_dense_q4k_rows_multi against one lk_dense_q4k_rows per matrix."""
