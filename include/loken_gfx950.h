@@ -437,8 +437,8 @@ int lk_dense_q4k_rows_multi(const void* const* weights, float* const* outputs, c
                             const void* q8_1, int size_m, int size_k, int q5, void* stream);
 /* Gate and up in one launch with the result handed on as Q8_1 rows: q8_1_out [size_m][size_n / 32 blocks]
  * = lk_quantize_q8_1(act(gate . x) * (up . x)) byte for byte, which the layer's down projection reads
- * with no f32 round trip and no quantizer launch in between. At most 16 rows, size_k 2048 or 4096, size_n
- * a multiple of 32 (anything else: LK_ERR_ARG; take lk_dense_q4k_rows_actmul and the quantizer). q5 != 0:
+ * with no f32 round trip and no quantizer launch in between. size_n a multiple of 32; up to 16 rows also
+ * size_k 2048 or 4096 (anything else: LK_ERR_ARG; take lk_dense_q4k_rows_actmul and the quantizer). q5 != 0:
  * Q5_K weights. No counterpart in the reference, whose dense_q4k_imma_m8_act_mul writes f32
  * (src/inference/moe_cuda/dense/imma.rs:320-400); the mat-vec sibling is lk_mmvq_pair_act_q8_1. */
 int lk_dense_q4k_rows_actmul_q8_1(const void* gate, const void* up, const void* q8_1, void* q8_1_out, int size_m,

@@ -101,6 +101,34 @@ static __device__ __forceinline__ float group_sum(float v) {
     if (LANES >= 64) v = swap_add32(v);
     return v;
 }
+// The maximum over each aligned group of 32 lanes (every lane of the group returns it).
+static __device__ __forceinline__ float group_max32(float v) {
+    v = fmaxf(v, dpp_f32<0xB1>(v));
+    v = fmaxf(v, dpp_f32<0x4E>(v));
+    v = fmaxf(v, dpp_f32<0x141>(v));
+    v = fmaxf(v, dpp_f32<0x140>(v));
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+// Thirty-two f32 values, one per lane of an aligned group of 32, as one Q8_1 block at `out` (36 bytes, 4-byte
+// aligned): the stand-alone quantizer's steps, as lk_store_q8_1_block. `l32`: the lane's place in the group.
+// Every lane of the wave calls it (the lane exchanges want them all); `store` false: nothing is written.
+static __device__ __forceinline__ void lk_store_q8_1_block_by_lane(float x, int l32, uint8_t* out, bool store) {
+#pragma clang fp contract(off)
+    const float amax = group_max32(fabsf(x));
+    const float d = amax / 127.0f;
+    const float inv = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q = (int)roundf(x * inv);
+    const float sum = group_sum<32>((float)q);   // an integer below 2^12: exact whatever the order
+    if (store) out[4 + l32] = (uint8_t)(q & 0xFF);
+    if (store && l32 == 0) {
+        const uint32_t dh = __half_as_ushort(__float2half_rn(d));
+        float scaled_sum = sum * d;
+        asm volatile("" : "+v"(scaled_sum));   // two roundings, as the quantizer's
+        *(uint32_t*)out = dh | ((uint32_t)__half_as_ushort(__float2half_rn(scaled_sum)) << 16);
+    }
+}
+
 // Two values at once: the even lanes of a group return the group's sum of `x0`, the odd lanes that
 // of `x1`, each with the additions of group_sum in the same order as far as lanes 0 and 1 of the
 // group are concerned, the only lanes whose result is defined (the first step hands every lane its

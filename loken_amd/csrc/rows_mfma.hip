@@ -65,6 +65,10 @@ struct Args {
     float* dst_b = nullptr;
     float* dst_c = nullptr;
     int n_b = 0, n_c = 0, ldd_b = 0, ldd_c = 0;
+    // DUAL, the dense launch only, when given: the result leaves as Q8_1 rows (a row tile's 32 rows are one
+    // block; q81_stride blocks between activation rows) instead of f32 in `dst`; n a multiple of 32
+    uint8_t* q81_dst = nullptr;
+    int q81_stride = 0;
 };
 
 // Row tile `t` of a launch: which matrix it belongs to, and which of that matrix's tiles it is.
@@ -373,6 +377,13 @@ static __device__ __forceinline__ void q4k_rows_pass(const Args& p, const PassRo
                 sum = lk_gated(act, gate_keep[r], sum, 0);
             }
             const int tok = (v >> 2) * 8 + lh * 4 + (v & 3);
+            if (DUAL && p.q81_dst) {
+                // the 32 lanes of a half wave hold one activation row's results for the tile's 32 rows: a block
+                // (every lane takes part in the exchanges; a row the pass does not have stores nothing)
+                uint8_t* blk = p.q81_dst + ((size_t)(rows.first + min(tok, m_count - 1)) * p.q81_stride + (t >> 1)) * Q81_BYTES;
+                lk_store_q8_1_block_by_lane(sum, l32, blk, tok < m_count);
+                continue;
+            }
             if (MULTI) {   // (dense rows: the pass's row i is row first + i of every output)
                 const MatRef mr = mat_of<MULTI>(p, rows.dst, rows.ldd, t);
                 const int row = mr.tile * 32 + l32;
@@ -893,9 +904,9 @@ extern "C" int lk_dense_q4k_rows_multi(const void* const* weights, float* const*
 // Gate and up in one launch with the result handed on as Q8_1: q8_1_out[m][size_n / 32] blocks =
 // lk_quantize_q8_1(act(gate . x) * (up . x)), byte for byte, so the down projection of a layer reads it
 // without the f32 round trip and the quantizer launch in between (what lk_mmvq_pair_act_q8_1 is to the
-// mat-vec pair launch). The 16-row-tile kernel at four tiles per workgroup: at most 16 rows, rows of 2048
-// or 4096 values, size_n a multiple of 32; anything else returns LK_ERR_ARG (take the f32 form and the
-// quantizer). q5 != 0: Q5_K. No counterpart in the reference, whose dense_q4k_imma_m8_act_mul writes f32
+// mat-vec pair launch). Up to 16 rows the 16-row-tile kernel at four tiles per workgroup (rows of 2048 or
+// 4096 values), above them the 32-row tiles (a tile's rows are one block; any row length its tables hold);
+// size_n a multiple of 32; anything else returns LK_ERR_ARG (take the f32 form and the quantizer). q5 != 0: Q5_K. No counterpart in the reference, whose dense_q4k_imma_m8_act_mul writes f32
 // (src/inference/moe_cuda/dense/imma.rs:320-400).
 extern "C" int lk_dense_q4k_rows_actmul_q8_1(const void* gate, const void* up, const void* q8_1, void* q8_1_out, int size_m,
                                              int size_n, int size_k, int use_gelu, int q5, void* stream) {
@@ -905,6 +916,13 @@ extern "C" int lk_dense_q4k_rows_actmul_q8_1(const void* gate, const void* up, c
         ((((uintptr_t)q8_1) | ((uintptr_t)q8_1_out)) & 3) != 0)
         return LK_ERR_ARG;
     const int nb = size_k / 256;
+    if (size_m > 16) {   // the 32-row tiles: a tile's rows are one block
+        Args a{(const uint8_t*)gate, (const uint8_t*)q8_1, nullptr, nb, size_n, size_m, size_k / 32, size_n,
+               (const uint8_t*)up, use_gelu ? 1 : 0};
+        a.q81_dst = (uint8_t*)q8_1_out;
+        a.q81_stride = size_n / 32;
+        return q5 ? launch_rows<4, true, true>(a, (hipStream_t)stream) : launch_rows<4, true, false>(a, (hipStream_t)stream);
+    }
     if ((nb != 8 && nb != 16) || !lk_rows16_serves(size_m, nb)) return LK_ERR_ARG;
     LkRows16 r{};
     r.w[0] = (const uint8_t*)gate; r.w[1] = (const uint8_t*)up;

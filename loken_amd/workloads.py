@@ -438,6 +438,10 @@ def decode_1p7b(args, dev):
     matvec = matvec and not fused_rows
 
     rows_h_q81 = torch.empty((b, ffn // 32, 36), dtype=torch.uint8, device=dev) if fused_rows else None
+    # above 16 rows, while the rows kernels serve gate + up and down: the same hand-over
+    mid_h_q81 = (torch.empty((b, ffn // 32, 36), dtype=torch.uint8, device=dev)
+                 if (not fused_rows and not matvec and args.mid_rows == "auto" and rows_kernel_serves(Q4K, ffn, b)
+                     and rows_kernel_serves(Q6K, hidden, b)) else None)
 
     def add_fused_rows(g, k, wtype, ns):
         nonlocal total_bytes
@@ -511,15 +515,20 @@ def decode_1p7b(args, dev):
                                          q.shape[1], n, None, 0, s)))
         elif args.mid_rows == "auto" and all(rows_kernel_serves(wtype, n, b) for n in ns):
             # the host mirror's choice (host_qmatmul.hip): the matrix-unit rows kernels, no weight staging
+            if g == "h" and mid_h_q81 is not None:   # `down` reads the Q8_1 rows the gate + up launch wrote
+                out = torch.empty((b, ns[0]), device=dev)
+                keep.append(out)
+                plan.append(("status", L.lk_dense_q6k_rows, (weights[0].data_ptr(), mid_h_q81.data_ptr(), out.data_ptr(), b, ns[0], k, s)))
+                used["rows"] += 1
+                return
             q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
             keep.append(q)
             plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s)))
             if g == "x2" and wtype == Q4K:
-                # gate and up with the activation on top in one launch (dense_q4k_imma_m8_act_mul of the reference)
-                out = torch.empty((b, ns[0]), device=dev)
-                keep.append(out)
-                plan.append(("status", L.lk_dense_q4k_rows_actmul,
-                             (weights[0].data_ptr(), weights[1].data_ptr(), q.data_ptr(), out.data_ptr(), b, ns[0], k, 0, s)))
+                # gate and up with the activation on top in one launch (dense_q4k_imma_m8_act_mul of the reference),
+                # its result handed on as the Q8_1 rows `down` reads
+                plan.append(("status", L.lk_dense_q4k_rows_actmul_q8_1,
+                             (weights[0].data_ptr(), weights[1].data_ptr(), q.data_ptr(), mid_h_q81.data_ptr(), b, ns[0], k, 0, 0, s)))
                 used["rows"] += 2
                 return
             if wtype == Q4K and len(ns) > 1:   # q + k + v: one launch over the three matrices
