@@ -280,9 +280,12 @@ template <class L, int NB, int TKP>
 int launch(const FoldCall& c, FoldDims d) {
     constexpr int RPG = 64 / (4 * TKP) * WAVES;
     const int groups = (d.cols + RPG - 1) / RPG;
-    // enough workgroups for three per CU; past that a workgroup takes more rows, so that the
-    // token's activation rows are quantized by fewer of them
-    int passes = (int)(((int64_t)c.tokens * groups + 3 * lk_device().cus - 1) / (3 * lk_device().cus));
+    // enough workgroups for two per CU; past that a workgroup takes more rows, so that the token's
+    // activation rows are quantized by fewer of them. An even count: the passes go two to a turn of
+    // the loop, and an odd last turn loads a pass nobody computes (measured at 8 tokens: 3 passes
+    // 35.5 us per block, 4 passes 32.9; at 16 tokens 6: 54.7, 8: 51.3).
+    int passes = (int)(((int64_t)c.tokens * groups + 2 * lk_device().cus - 1) / (2 * lk_device().cus));
+    passes = passes <= 1 ? 1 : passes <= 2 ? 2 : passes <= 5 ? 4 : 8;   // (12 passes: 57 us at 16 tokens, 88 at 24 against 81)
     if (const int t = lk_tune_env("LK_TUNE_DOWN_FOLD_PASSES")) passes = t;
     passes = passes < 1 ? 1 : passes > 16 ? 16 : passes;
     d.passes = passes;

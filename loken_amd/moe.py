@@ -416,7 +416,7 @@ def moe_mmq_pays(rows: int, experts: int, wtype: int | None = None) -> bool:
     library's kernels, the mat-vec per routed pair stays ahead of the tiled matmul up to three rows
     per expert (Qwen3-30B-A3B shapes: 117 us against 162 us at 32 tokens, 176 against 168 at 48), and
     of the matrix-unit rows launch that Q4_K stacks take at short runs up to 1.625 (per block inside
-    a step's graph, 16 tokens: 54 us against 74; 24: 81 against 83; 32: 92 against 88; 48: 139
+    a step's graph, 16 tokens: 51 us against 74; 24: 81 against 83; 32: 92 against 88; 48: 139
     against 106)."""
     if wtype == _lib.TYPE_Q4_K:
         return 8 * rows >= 13 * max(experts, 1)
