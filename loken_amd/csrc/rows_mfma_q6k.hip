@@ -364,10 +364,12 @@ int launch_waves(const Args& a, hipStream_t stream) {
 template <int G, bool STAGED>
 int launch(const Args& a, hipStream_t stream) {
     // eight waves when the tiles (times the passes of 32 rows) do not fill the CUs and a wave would
-    // otherwise walk eight super-blocks or more in turn
+    // otherwise walk four super-blocks or more in turn (measured at 32 / 64 rows, four against eight waves:
+    // 2048 x 6144 41.8 / 42.6 -> 36.5 / 37.6 us, 4096 x 4096 34.6 / 35.8 -> 31.9 / 33.4; rows of eight
+    // super-blocks lose, 25.8 -> 27.4)
     const int n_tiles = (a.n + 31) / 32, groups = STAGED ? 1 : (a.m + TOK - 1) / TOK;
     static const int forced = lk_tune_env("LK_TUNE_ROWS_WAVES");
-    const bool eight = forced ? forced == 8 : (n_tiles * groups <= lk_device().cus && a.nb >= 32);
+    const bool eight = forced ? forced == 8 : (n_tiles * groups <= lk_device().cus && a.nb >= 16);
     if (eight) {
         const int rc = launch_waves<G, STAGED, 8>(a, stream);
         if (rc >= 0) return rc;
