@@ -180,6 +180,15 @@ int lk_mmvq_grouped(int wtype, const uint64_t* table, int groups, const void* vy
 int lk_mmvq_subdots(int wtype, const void* vx, const void* vy_q8_1, int32_t* dots, int32_t* sums,
                     int ncols_x, int nrows_x, void* stream);
 
+/* The exact mode: Q4_K / Q6_K weight rows x `batch` Q8_K activation rows (292-byte blocks {f32 d, 256 x i8,
+ * 16 x i16 sums}, batch rows of ncols_x / 256 blocks, 4-byte aligned) -> dst[batch][nrows_x] f32 with the
+ * reference's cross-device contract (ExactDot, src/tensor/quant_cpu/format/blocks.rs:80-96; dot_exact,
+ * format/q4_k.rs:117-156, q6_k.rs:121-163): exact integer sums per super-block, then a fixed f32 fold,
+ * total += d8 * (d * f32(scaled) - dmin * f32(offset)) from -0.0 in block order, one rounding per
+ * operation. The result carries the bits of the CPU's dot_exact. A parity path, not a fast one. */
+int lk_mmvq_exact(int wtype, const void* vx, const void* vy_q8_k, float* dst, int ncols_x, int nrows_x, int batch,
+                  void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Prefill path: tiled quantized matmul on int8 MFMA. Names, argument lists and return
  * conventions are loken's (src/tensor/quantized/mmq.rs:64-116 quantizers, :132-147 and

@@ -114,6 +114,7 @@ SIGNATURES.update({
     "loken_dense_q4k_imma_m8_actmul": (None, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "lk_dense_q4k_rows_actmul": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "lk_dense_q4k_rows_multi": (_i, [_vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
+    "lk_mmvq_exact": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "lk_dense_q4k_rows_actmul_q8_1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "loken_dense_q5k_imma_m8_plain": (None, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "lk_dense_q5k_rows": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),

@@ -284,6 +284,17 @@ def dense_q4k_rows_actmul_q8_1(gate: torch.Tensor, up: torch.Tensor, x: torch.Te
     return out
 
 
+def mmvq_exact(wtype: int, weight: torch.Tensor, q8_k: torch.Tensor, n: int) -> torch.Tensor:
+    """Q4_K / Q6_K weight ``[n, k]`` x Q8_K rows ``[rows, k / 256, 292]`` uint8 -> ``[rows, n]`` f32 with the
+    reference's exact fold (dot_exact, src/tensor/quant_cpu/format/q4_k.rs:117-156, q6_k.rs:121-163): the bits
+    of the CPU path."""
+    rows, nb, _ = q8_k.shape
+    out = torch.empty((rows, n), dtype=torch.float32, device=q8_k.device)
+    _lib.check("lk_mmvq_exact", _lib.load().lk_mmvq_exact(wtype, weight.data_ptr(), q8_k.data_ptr(), out.data_ptr(),
+                                                          nb * 256, n, rows, _stream()))
+    return out
+
+
 def dense_q6k_rows(weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tensor:
     """``[rows, k]`` f32 x Q6_K weight ``[n, k]`` -> ``[rows, n]`` f32 on the matrix unit, rows
     quantized to plain Q8_1 first."""

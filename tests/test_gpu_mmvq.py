@@ -404,3 +404,27 @@ def test_the_reference_batch1_matrix_unit_name_is_the_q4k_matvec():
     assert torch.equal(out, ops.mmvq(lib.TYPE_Q4_K, wd, q, k, n)[0])
     want = oracle.ob_matmul(lib.TYPE_Q4_K, x, w, n)[0]
     assert (np.abs(out.cpu().numpy() - want) <= 1e-3 * np.abs(want) + 1e-4).all()
+
+
+@pytest.mark.parametrize("name,n,k,rows", [("q4_k", 33, 1024, 3), ("q4_k", 5, 256, 1), ("q4_k", 64, 4096, 2), ("q4_k", 7, 17408, 1),
+                                           ("q6_k", 33, 1024, 3), ("q6_k", 5, 256, 1), ("q6_k", 40, 14336, 2), ("q6_k", 7, 17408, 1)])
+def test_exact_mode_carries_the_bits_of_the_cpu_exact_fold(name, n, k, rows):
+    """lk_mmvq_exact over Q8_K rows quantized on the host against dot_exact of the CPU statement (the reference's
+    cross-device contract, blocks.rs:80-96): bit for bit, rows of more than 64 super-blocks included."""
+    wtype = {"q4_k": lib.TYPE_Q4_K, "q6_k": lib.TYPE_Q6_K}[name]
+    w = synth.weight(wtype, n, k, seed=80, stream=1)
+    x = synth.activation(rows, k, seed=80) * np.float32(9.0)
+    x[0, :256] = 0.0   # a super-block of zeros: d8 = 0
+    want = oracle.oa_matmul(wtype, x, w, n, exact=True)
+    q8k = np.stack([oracle.quantize_q8_k(x[r]).reshape(-1, 292) for r in range(rows)])
+    got = ops.mmvq_exact(wtype, dev(w), dev(q8k), n).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_exact_mode_refuses_other_formats():
+    buf = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    out = torch.zeros(4, device="cuda")
+    rc = lib.load().lk_mmvq_exact(lib.TYPE_Q8_0, buf.data_ptr(), buf.data_ptr(), out.data_ptr(), 256, 4, 1,
+                                  torch.cuda.current_stream().cuda_stream)
+    assert rc == lib.LK_ERR_TYPE
+

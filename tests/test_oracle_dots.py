@@ -270,6 +270,49 @@ def test_served_path_matches_f64_over_dequantized_weights(name, m):
         assert (np.abs(ex - got) <= 1e-3 * np.maximum(np.abs(got), 1.0)).all()
 
 
+def crafted_exact_case(dtype, n, nb, seed):
+    """Weights with d = dmin = 1 and small scales, activations on the integer grid with -127 leading every
+    super-block (Q8_K then has d = 1 and the codes are the values): every f32 operation of the exact fold is
+    exact, so the result is the integer product of the dequantized weights with the activations."""
+    rng = np.random.default_rng(seed)
+    one = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    if dtype == oracle.Q4_K:
+        w = np.zeros((n, nb, 144), np.uint8)
+        w[:, :, 0:2] = one
+        w[:, :, 2:4] = one
+        sc = rng.integers(0, 8, size=(n, nb, 8), dtype=np.uint8)
+        mn = rng.integers(0, 8, size=(n, nb, 8), dtype=np.uint8)
+        w[:, :, 4:8] = sc[:, :, 0:4]
+        w[:, :, 8:12] = mn[:, :, 0:4]
+        w[:, :, 12:16] = sc[:, :, 4:8] | (mn[:, :, 4:8] << 4)   # six-bit values below 16: no high bits to place
+        w[:, :, 16:] = rng.integers(0, 256, size=(n, nb, 128), dtype=np.uint8)
+    else:
+        w = np.zeros((n, nb, 210), np.uint8)
+        w[:, :, 0:192] = rng.integers(0, 256, size=(n, nb, 192), dtype=np.uint8)
+        w[:, :, 192:208] = rng.integers(-7, 8, size=(n, nb, 16)).astype(np.int8).view(np.uint8)
+        w[:, :, 208:210] = one
+    x = rng.integers(-126, 127, size=(3, nb * 256)).astype(np.float32)
+    x.reshape(3, nb, 256)[:, :, 0] = -127.0
+    return w.reshape(n, -1), x
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+def test_exact_fold_is_the_integer_product_where_every_step_is_exact(name):
+    # pins oa_matmul_exact (dot_exact, q4_k.rs:117-156, q6_k.rs:121-163) without retyping its loops: a dropped
+    # min term, a wrong bsum index or a sign would change the integer
+    dtype = DT[name]
+    n, nb = 12, 4
+    w, x = crafted_exact_case(dtype, n, nb, seed=16)
+    got = oracle.oa_matmul(dtype, x, w, n, exact=True)
+    wd = np_dequant(dtype, w.reshape(n, nb, -1))
+    want = x.astype(np.int64) @ np.rint(wd).astype(np.int64).T
+    assert np.abs(want).max() < 2 ** 24
+    assert np.array_equal(got.astype(np.int64), want) and np.array_equal(got, np.rint(got))
+    # all-zero activations: the fold starts from -0.0 and every block adds +0.0 or -0.0 terms to it
+    z = oracle.oa_matmul(dtype, np.zeros((1, nb * 256), np.float32), w, n, exact=True)
+    assert np.array_equal(z, np.zeros_like(z))
+
+
 @pytest.mark.parametrize("name", sorted(DT))
 def test_served_path_integer_core_with_q8k_codes(name):
     # f64 product of dequantized weights with dequantized O-A activations: pins the Q8_K / Q8_0
