@@ -236,6 +236,27 @@ int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* y, void* ds
                          int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
                          void* stream);
 
+/* The 32-value nibble formats on the Q8_0 tile (stride_row_x = k / 32 blocks; weights 2-byte aligned):
+ * codes expanded to int8 less the format's bias on the way into the tile, Q4_1 / Q5_1 with the
+ * block minimum as + m * (d8 * sum of the token's codes).
+ * Replaces launch_mmq_gguf_{q4_0,q4_1,q5_0,q5_1} (src/tensor/quantized/mmq.rs:274-279). */
+int launch_mmq_gguf_q4_0(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+int launch_mmq_gguf_q4_1(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+int launch_mmq_gguf_q5_0(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+int launch_mmq_gguf_q5_1(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * MoE prefill: expert-batched tiled matmul and the steps around it. Names and argument lists are
  * loken's (src/tensor/quantized/mmq.rs:151-173; src/inference/moe_cuda/mmq_experts.rs:42-56),
@@ -274,6 +295,47 @@ int launch_mmq_moe_gguf_q8_0(const void* x, const void* x_second, int64_t dst_se
                              int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
                              int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
                              int64_t smpbo, int warp_size, void* stream);
+
+/* The same launch for the 32-value nibble formats, and for the two that only mixtures store and that
+ * have no dense entry point (IQ4_NL: the 16 levels as int8 codes; MXFP4: its levels, E8M0 scale, 17-byte
+ * blocks at any byte address). Replaces launch_mmq_moe_gguf_{q4_0,q4_1,q5_0,q5_1} and the expert-only
+ * launch_mmq_moe_gguf_{iq4_nl,mxfp4} (src/tensor/quantized/mmq.rs:274-279, 326-334). */
+int launch_mmq_moe_gguf_q4_0(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_q4_1(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_q5_0(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_q5_1(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_iq4_nl(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                               void* dst, const int* expert_bounds, const int* ids_dst,
+                               int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                               int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                               int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                               int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_mxfp4(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                              void* dst, const int* expert_bounds, const int* ids_dst,
+                              int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                              int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                              int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                              int64_t smpbo, int warp_size, void* stream);
 
 /* From a routing already sorted by expert: bounds[e] = first sorted row of expert >= e
  * (n_experts + 1 entries), slots_out = slots, src_rows[i] = slots[i] / topk.

@@ -97,16 +97,28 @@ void mark_used(Slot& slot, hipStream_t stream) {
     }
 }
 
-// The 32-value nibble formats and the two-bit K-quants: served by the plain mat-vec only, whatever
-// the row count.
+// The 32-value nibble formats and the two-bit K-quants: served by the plain mat-vec (four of them by the
+// tiled matmul as well, from the row counts of nibble_tiles_pay below).
 bool matvec_only(int dtype) {
     return dtype == LK_TYPE_Q4_0 || dtype == LK_TYPE_Q4_1 || dtype == LK_TYPE_Q5_0 || dtype == LK_TYPE_Q5_1 ||
            dtype == LK_TYPE_IQ4_NL || dtype == LK_TYPE_MXFP4 || dtype == LK_TYPE_Q2_K || dtype == LK_TYPE_Q3_K ||
            dtype == LK_TYPE_IQ4_XS;
 }
 
+bool nibble_tiles(int dtype) {
+    return dtype == LK_TYPE_Q4_0 || dtype == LK_TYPE_Q4_1 || dtype == LK_TYPE_Q5_0 || dtype == LK_TYPE_Q5_1;
+}
+
 bool tiled_serves(int dtype, int k) {
-    return (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K || dtype == LK_TYPE_Q6_K || dtype == LK_TYPE_Q8_0) && k % 256 == 0;
+    return (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K || dtype == LK_TYPE_Q6_K || dtype == LK_TYPE_Q8_0 || nibble_tiles(dtype)) &&
+           k % 256 == 0;
+}
+
+// Q4_0 / Q4_1 / Q5_0 / Q5_1: rows from which one tiled launch beats mat-vec launches of eight rows each.
+// Measured on MI355X (Q4_0 and Q5_1 alike): 2048 x 2048 and 4096 x 4096 from 56-64 rows (48 rows: 67 us
+// against 77), 4096 x 14336 likewise, 14336 x 4096 from 24 (74 us against 60; 16 rows: 50 against 60).
+bool nibble_tiles_pay(int dtype, int n, int k, int rows) {
+    return nibble_tiles(dtype) && k % 256 == 0 && (rows > 48 || (long long)rows * n >= 300000);
 }
 
 size_t elem_bytes(int type) { return type == LK_TYPE_F32 ? 4 : 2; }
@@ -115,7 +127,7 @@ size_t elem_bytes(int type) { return type == LK_TYPE_F32 ? 4 : 2; }
 
 int matvec_rows(int dtype, int k) {
     if ((dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K || dtype == LK_TYPE_Q6_K) && k % 256 == 0) return 8;
-    return tiled_serves(dtype, k) ? 32 : 8;
+    return dtype == LK_TYPE_Q8_0 && tiled_serves(dtype, k) ? 32 : 8;
 }
 
 // Rows the matrix-unit rows kernels take before the tiled matmul does. Measured on MI355X over
@@ -169,7 +181,9 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
 
     // --- mat-vec family: up to matvec_rows, or any count when every row must sum like a one-row call
     const bool to_rows_kernel = x_type == LK_TYPE_F32 && small_rows_kernel_pays(dtype_, n_, k_, rows);
-    if ((rows <= mv_max && !to_rows_kernel) || decode_order || plain) {
+    const bool to_nibble_tiles = x_type == LK_TYPE_F32 && !decode_order && nibble_tiles_pay(dtype_, n_, k_, rows) &&
+                                 ((uintptr_t)blob_ & 1) == 0;
+    if ((rows <= mv_max && !to_rows_kernel) || decode_order || (plain && !to_nibble_tiles)) {
         if (!plain && x_type == LK_TYPE_F32 && rows <= 2 && k_ <= 8192 && ((uintptr_t)x & 15) == 0 && k_ % 4 == 0) {
             const void* vx[1] = {blob_};
             void* dst[1] = {out};
@@ -220,9 +234,18 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     const size_t ws_bytes = (size_t)rows * (k_padded / 128) * MMQ_RECORD + 128 * MMQ_RECORD;
     std::lock_guard<std::mutex> pair(slot.mu);
     if (int rc = reserve(slot, ws_bytes, true, stream)) return rc;
-    auto quantizer = dtype_ == LK_TYPE_Q4_K || dtype_ == LK_TYPE_Q5_K ? launch_mmq_quantize_q8_1_DS4 : launch_mmq_quantize_q8_1_D4;
+    // the layouts of the reference's table (quantized/mmq.rs:274-285)
+    auto quantizer = dtype_ == LK_TYPE_Q6_K || dtype_ == LK_TYPE_Q8_0 || dtype_ == LK_TYPE_Q5_0 ? launch_mmq_quantize_q8_1_D4
+                                                                                               : launch_mmq_quantize_q8_1_DS4;
     quantizer(x, nullptr, slot.act, 0, k_, k_, 0, 0, (int64_t)k_padded, rows, 1, 1, stream);
-    auto launcher = dtype_ == LK_TYPE_Q4_K ? launch_mmq_gguf_q4_k : dtype_ == LK_TYPE_Q5_K ? launch_mmq_gguf_q5_k : dtype_ == LK_TYPE_Q6_K ? launch_mmq_gguf_q6_k : launch_mmq_gguf_q8_0;
+    auto launcher = dtype_ == LK_TYPE_Q4_K   ? launch_mmq_gguf_q4_k
+                    : dtype_ == LK_TYPE_Q5_K ? launch_mmq_gguf_q5_k
+                    : dtype_ == LK_TYPE_Q6_K ? launch_mmq_gguf_q6_k
+                    : dtype_ == LK_TYPE_Q4_0 ? launch_mmq_gguf_q4_0
+                    : dtype_ == LK_TYPE_Q4_1 ? launch_mmq_gguf_q4_1
+                    : dtype_ == LK_TYPE_Q5_0 ? launch_mmq_gguf_q5_0
+                    : dtype_ == LK_TYPE_Q5_1 ? launch_mmq_gguf_q5_1
+                                             : launch_mmq_gguf_q8_0;
     int abi = 0, cus = 0, lds = 0, wave = 0;
     (void)lk_device_info(&abi, &cus, &lds, &wave);
     const int tile = launcher(slot.fixup, blob_, slot.act, out, k_, n_, rows, k_ / block_len, n_, 0x1000950, cus, lds, wave,

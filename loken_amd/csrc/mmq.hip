@@ -26,6 +26,7 @@
 // MFMA (v_mfma_f32_32x32x2_f32) straight into the accumulators, costing no per-element VALU.
 
 #include "mmq_problem.h"
+#include "legacy_blocks.h"
 
 #include <cstdlib>
 
@@ -108,6 +109,7 @@ static void launch_quantize(const void* x, const int32_t* ids, void* vy, int typ
 // then the nibbles; the int8 tiles take codes 0..31 as they take 0..15.
 template <bool Q5>
 struct MmqQ45K {
+    static constexpr int ALIGN = 4;   // whole-header reads
     static constexpr int BLOCK_BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES;
     static constexpr int QS0 = Q5 ? 48 : 16;
     static constexpr bool F16_TILES = !Q5;   // Q4_K above 64 tokens: the f16 tile kernel
@@ -188,6 +190,7 @@ using MmqQ5K = MmqQ45K<true>;
 // Q6_K: sixteen int8 scales per block, one per 16 values, so one MFMA K (32) spans two of them;
 // the tile loop runs each 32-group as two MFMAs over half-masked weight operands.
 struct MmqQ6K {
+    static constexpr int ALIGN = 2;
     static constexpr int BLOCK_BYTES = Q6K_BYTES;
     static constexpr int NS = 16;
     static constexpr bool HAS_MIN = false;
@@ -252,6 +255,7 @@ struct MmqQ6K {
 // Q8_0: eight 34-byte blocks per 256-value step, codes copied as they are.
 struct MmqQ80 {
     static constexpr int BLOCK_BYTES = Q80_BYTES;
+    static constexpr int ALIGN = 2;
     static constexpr int NS = 8;
     static constexpr bool HAS_MIN = false;
     static constexpr bool F16_TILES = false;
@@ -291,6 +295,70 @@ struct MmqQ80 {
         }
     }
 };
+
+// The 32-value nibble formats (Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, MXFP4): eight blocks per 256-value step,
+// one scale each, so the tile is Q8_0's with the codes expanded on the way into LDS. Codes leave as
+// int8 less the format's bias (a table format's as its levels); Q4_1 / Q5_1 keep unsigned codes and
+// table the block minimum, which rides the rank-8 update that serves Q4_K's: + m * (d8 * sum of codes).
+// A thread takes whole blocks (row = idx / 8, block = idx % 8: a row's eight blocks are one
+// contiguous run of 136..192 bytes).
+template <int ID>
+struct MmqLegacy {
+    using L = Legacy<ID>;
+    static constexpr int BLOCK_BYTES = L::BYTES;
+    static constexpr int NS = 8;
+    static constexpr bool HAS_MIN = L::M_AT >= 0;
+    static constexpr bool F16_TILES = false;
+    static constexpr int BLOCKS_PER_STEP = 8;
+    static constexpr int ALIGN = L::BYTES % 2 ? 1 : 2;
+    static constexpr int PER = TN * 8 / MMQ_WG;
+
+    struct Frag {
+        uint4 q[PER];
+        uint32_t qh[PER];
+        float d[PER], m[PER];
+    };
+    static __device__ __forceinline__ void fetch(Frag& f, const uint8_t* __restrict__ w, int64_t nb, int kb,
+                                                 int n0, int n) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, blk = idx & 7;
+            const int gn = min(n0 + row, n - 1);
+            const uint8_t* bp = w + ((int64_t)gn * nb + (int64_t)kb * 8 + blk) * L::BYTES;
+            f.q[i] = block_code_bytes<L>(bp);
+            f.qh[i] = block_fifth_word<L>(bp);
+            f.d[i] = block_scale<L>(bp);
+            f.m[i] = HAS_MIN ? f16_bits_to_f32(*(const uint16_t*)(bp + (HAS_MIN ? L::M_AT : 0))) : 0.f;
+        }
+    }
+    static __device__ __forceinline__ uint32_t less_bias(uint32_t codes) {
+        // per byte code - BIAS as int8: code + (0x80 - BIAS) never carries (code <= 31), and flipping
+        // bit 7 takes the 0x80 off again in two's complement
+        if (L::BIAS == 0) return codes;
+        return (codes + 0x01010101u * (uint32_t)(0x80 - L::BIAS)) ^ 0x80808080u;
+    }
+    static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, blk = idx & 7;
+            uint4 lo, hi;
+            expand_codes<L>(f.q[i], f.qh[i], lo, hi);
+            lo = make_uint4(less_bias(lo.x), less_bias(lo.y), less_bias(lo.z), less_bias(lo.w));
+            hi = make_uint4(less_bias(hi.x), less_bias(hi.y), less_bias(hi.z), less_bias(hi.w));
+            *(uint4*)(wq + (blk * TN + row) * 32) = lo;
+            *(uint4*)(wq + (blk * TN + row) * 32 + 16) = hi;
+            const bool live = n0 + row < n;
+            wsc[blk * TN + row] = live ? f.d[i] : 0.f;
+            if (HAS_MIN) wmn[blk * TN + row] = live ? f.m[i] : 0.f;
+        }
+    }
+};
+using MmqQ40 = MmqLegacy<LK_TYPE_Q4_0>;
+using MmqQ41 = MmqLegacy<LK_TYPE_Q4_1>;
+using MmqQ50 = MmqLegacy<LK_TYPE_Q5_0>;
+using MmqQ51 = MmqLegacy<LK_TYPE_Q5_1>;
+using MmqIq4Nl = MmqLegacy<LK_TYPE_IQ4_NL>;
+using MmqMxfp4 = MmqLegacy<LK_TYPE_MXFP4>;
 
 // Token rows [m0, m0+TM) of block kb (record layout above). Rows at or past m_end read as zeros.
 template <int TM>
@@ -601,6 +669,7 @@ template <class F>
 static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x, int64_t nrows_x,
                         int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, void* stream) {
     if (!x || !y || !dst || ncols_x <= 0 || nrows_x <= 0 || ncols_y <= 0) return 0;
+    if ((uintptr_t)x % F::ALIGN != 0) return 0;
     if (ncols_x % 256 != 0 || stride_row_x < ncols_x / 256 * F::BLOCKS_PER_STEP) return 0;
     if (stride_col_dst < nrows_x || nrows_x > INT32_MAX || ncols_y > INT32_MAX) return 0;
     MmqProblem pb{(const uint8_t*)x, (const uint8_t*)y, (float*)dst, nullptr, ncols_x / 256, stride_row_x,
@@ -643,6 +712,7 @@ static int launch_moe(const void* x, const void* x_second, int64_t dst_second, c
                       int64_t stride_col_dst, int n_experts, int64_t ncols_max, int64_t ncols_hint,
                       int mmq_x, void* stream) {
     if (!x || !y || !dst || !expert_bounds || ncols_x <= 0 || nrows_x <= 0 || ncols_y <= 0 || n_experts <= 0) return 0;
+    if ((uintptr_t)x % F::ALIGN != 0 || (uintptr_t)x_second % F::ALIGN != 0 || stride_expert_x % F::ALIGN != 0) return 0;
     if (ncols_x % 256 != 0 || stride_row_x < ncols_x / 256 * F::BLOCKS_PER_STEP) return 0;
     if (nrows_x > INT32_MAX || ncols_y > INT32_MAX || (int64_t)n_experts * 2 > 65535) return 0;
     MmqProblem pb{(const uint8_t*)x, (const uint8_t*)y, (float*)dst, ids_dst, ncols_x / 256, stride_row_x,
@@ -709,6 +779,19 @@ extern "C" int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* 
     return launch_dense<MmqQ80>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
 }
 
+#define LK_MMQ_DENSE_ENTRY(NAME, FMT)                                                                   \
+    extern "C" int NAME(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,     \
+                        int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, \
+                        int cc, int nsm, int64_t smpbo, int warp_size, void* stream) {                 \
+        (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;                            \
+        return launch_dense<FMT>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream); \
+    }
+
+LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q4_0, MmqQ40)
+LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q4_1, MmqQ41)
+LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q5_0, MmqQ50)
+LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q5_1, MmqQ51)
+
 #define LK_MMQ_MOE_ENTRY(NAME, FMT)                                                                     \
     extern "C" int NAME(const void* x, const void* x_second, int64_t dst_second, const void* y,        \
                         void* dst, const int* expert_bounds, const int* ids_dst,                       \
@@ -726,3 +809,9 @@ LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q4_k, MmqQ4K)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q5_k, MmqQ5K)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q6_k, MmqQ6K)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q8_0, MmqQ80)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q4_0, MmqQ40)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q4_1, MmqQ41)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q5_0, MmqQ50)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q5_1, MmqQ51)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq4_nl, MmqIq4Nl)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_mxfp4, MmqMxfp4)

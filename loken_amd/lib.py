@@ -46,6 +46,10 @@ SIGNATURES = {
     "launch_mmq_gguf_q5_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
     "launch_mmq_gguf_q6_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
     "launch_mmq_gguf_q8_0": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
+    "launch_mmq_gguf_q4_0": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
+    "launch_mmq_gguf_q4_1": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
+    "launch_mmq_gguf_q5_0": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
+    "launch_mmq_gguf_q5_1": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
 }
 _MOE_MMQ = (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _vp] + [_i64] * 6 + [_i, _i64, _i64, _i, _i, _i64, _i, _vp])
 SIGNATURES.update({
@@ -53,6 +57,12 @@ SIGNATURES.update({
     "launch_mmq_moe_gguf_q5_k": _MOE_MMQ,
     "launch_mmq_moe_gguf_q6_k": _MOE_MMQ,
     "launch_mmq_moe_gguf_q8_0": _MOE_MMQ,
+    "launch_mmq_moe_gguf_q4_0": _MOE_MMQ,
+    "launch_mmq_moe_gguf_q4_1": _MOE_MMQ,
+    "launch_mmq_moe_gguf_q5_0": _MOE_MMQ,
+    "launch_mmq_moe_gguf_q5_1": _MOE_MMQ,
+    "launch_mmq_moe_gguf_iq4_nl": _MOE_MMQ,
+    "launch_mmq_moe_gguf_mxfp4": _MOE_MMQ,
     "loken_moe_mmq_plan": (None, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "loken_moe_mmq_route": (None, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "loken_moe_mmq_silu_mul": (None, [_vp, _vp, _i64, _i, _vp]),

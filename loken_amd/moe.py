@@ -15,7 +15,11 @@ from .synth import BLOCK_BYTES, BLOCK_LEN
 
 MMQ_MOE_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_moe_gguf_q4_k", _lib.TYPE_Q5_K: "launch_mmq_moe_gguf_q5_k",
                     _lib.TYPE_Q6_K: "launch_mmq_moe_gguf_q6_k",
-                    _lib.TYPE_Q8_0: "launch_mmq_moe_gguf_q8_0"}
+                    _lib.TYPE_Q8_0: "launch_mmq_moe_gguf_q8_0",
+                    _lib.TYPE_Q4_0: "launch_mmq_moe_gguf_q4_0", _lib.TYPE_Q4_1: "launch_mmq_moe_gguf_q4_1",
+                    _lib.TYPE_Q5_0: "launch_mmq_moe_gguf_q5_0", _lib.TYPE_Q5_1: "launch_mmq_moe_gguf_q5_1",
+                    # the formats only mixtures store (quantized/mmq.rs:326-334)
+                    _lib.TYPE_IQ4_NL: "launch_mmq_moe_gguf_iq4_nl", _lib.TYPE_MXFP4: "launch_mmq_moe_gguf_mxfp4"}
 MMQ_X_MIN, GRID_Y_MAX = 8, 65535
 
 

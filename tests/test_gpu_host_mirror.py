@@ -11,7 +11,7 @@ from loken_amd import lib, ops, synth
 pytestmark = pytest.mark.gpu
 
 DT = {"q4_k": lib.TYPE_Q4_K, "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0,
-      "q4_0": lib.TYPE_Q4_0, "q5_1": lib.TYPE_Q5_1, "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K}
+      "q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1, "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K}
 PATH = {1: "matvec-fused", 2: "matvec", 3: "rows-on-matrix-unit", 4: "tiled"}
 X_TYPES = {torch.float32: lib.TYPE_F32, torch.float16: lib.TYPE_F16, torch.bfloat16: lib.TYPE_BF16}
 
@@ -61,7 +61,10 @@ def close(got, want, rtol=1e-3, atol=1e-4):
     ("q6_k", 40, 200, "rows-on-matrix-unit"), ("q6_k", 200, 24000, "tiled"),
     ("q8_0", 3, 200, "matvec"), ("q8_0", 33, 200, "tiled"), ("q5_k", 1, 200, "matvec-fused"), ("q5_k", 8, 200, "matvec"),
     ("q5_k", 20, 200, "rows-on-matrix-unit"), ("q5_k", 200, 200, "rows-on-matrix-unit"), ("q5_k", 80, 24000, "tiled"),
-    ("q4_0", 1, 200, "matvec"), ("q4_0", 50, 200, "matvec"), ("q5_1", 9, 200, "matvec"), ("iq4_nl", 3, 200, "matvec"),
+    ("q4_0", 1, 200, "matvec"), ("q4_0", 40, 200, "matvec"), ("q5_1", 9, 200, "matvec"), ("iq4_nl", 3, 200, "matvec"),
+    # four of the 32-value formats have tiles: from 49 rows, or n x rows of 300 thousand
+    ("q4_0", 50, 200, "tiled"), ("q5_0", 64, 200, "tiled"), ("q5_1", 30, 12000, "tiled"), ("q4_1", 20, 12000, "matvec"),
+    ("q4_1", 130, 300, "tiled"), ("iq4_nl", 60, 200, "matvec"),
     ("mxfp4", 17, 200, "matvec"), ("q2_k", 12, 200, "matvec"), ("q3_k", 1, 200, "matvec")])
 def test_forward_takes_the_path_of_its_row_count_and_matches_the_oracle(name, rows, n, expect):
     wtype, k = DT[name], 1024

@@ -87,6 +87,30 @@ def test_expert_batched_block_matches_oracle(tokens, hidden, ffn, n_experts, top
     assert (np.abs(got - want) <= 2e-3 * np.abs(want) + 2e-4 * scale).all()
 
 
+NIBBLE_TILES = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
+                "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4}
+
+
+@pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(40, 1024, 512, 8, 3), (70, 512, 768, 16, 4),
+                                                             (1, 256, 256, 4, 2), (300, 512, 256, 3, 2)])
+@pytest.mark.parametrize("name", sorted(NIBBLE_TILES))
+def test_expert_batched_block_in_the_nibble_formats_matches_oracle(name, tokens, hidden, ffn, n_experts, topk):
+    """The tiled launch for the 32-value formats, IQ4_NL and MXFP4 among them (which have no dense entry
+    point); the last shape runs the 128-token tiles."""
+    dt = NIBBLE_TILES[name]
+    assert moe.moe_mmq_serves(dt, hidden)
+    gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=53, dt_down=dt, dt_gu=dt, x_scale=4.0)
+    want, want_h = oracle.moe_forward(1, dt, dt, x, gate, up, down, ids, w, n_experts, ffn, want_h=True)
+    plan = MmqRouting.from_choices(dev(ids), n_experts).with_path("tiled")
+    h = plan.gate_up_silu(dt, dev(x), dev(gate), dev(up), ffn)
+    got_h = h.cpu().numpy()
+    assert (np.abs(got_h - want_h) <= 1e-3 * np.abs(want_h) + 1e-4 * np.abs(want_h).max()).all()
+    # down from the oracle's own rows, so that a code flipped by the last place of h does not enter
+    out = plan.down_fold(dt, dev(want_h), dev(down), hidden, dev(w.reshape(-1)))
+    scale = np.abs(want).max()
+    assert (np.abs(out.cpu().numpy() - want) <= 1e-3 * np.abs(want) + 1e-4 * scale).all()
+
+
 def test_down_fold_alone_is_tight_when_fed_the_oracle_rows():
     # feeding the oracle's own GLU rows removes the re-quantization ambiguity: 1e-3 rel + 1e-4 abs
     tokens, hidden, ffn, n_experts, topk = 24, 512, 512, 8, 2

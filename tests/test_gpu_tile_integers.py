@@ -31,7 +31,8 @@ pytestmark = pytest.mark.gpu
 
 Q4K, Q5K, Q6K, Q80 = lib.TYPE_Q4_K, lib.TYPE_Q5_K, lib.TYPE_Q6_K, lib.TYPE_Q8_0
 ONE = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
-SUBS = {Q4K: 8, Q5K: 8, Q6K: 16, Q80: 8}
+NIBBLE32 = {lib.TYPE_Q4_0: (18, None), lib.TYPE_Q4_1: (20, 2), lib.TYPE_Q5_0: (22, None), lib.TYPE_Q5_1: (24, 2)}
+SUBS = {Q4K: 8, Q5K: 8, Q6K: 16, Q80: 8, **{t: 8 for t in NIBBLE32}}
 
 
 def dev(a):
@@ -63,6 +64,14 @@ def isolate(wtype, w, s, min_term=False):
         w[..., 192:208] = 0
         w[..., 192 + s] = 1
         w[..., 208:210] = ONE
+    elif wtype in NIBBLE32:
+        # [n, blocks of 32, bytes]: scale 1 on every eighth block, no minimum (or the reverse)
+        m_at = NIBBLE32[wtype][1]
+        w[..., 0:2] = 0
+        if m_at is not None:
+            w[..., m_at:m_at + 2] = 0
+        at = m_at if min_term else 0
+        w[:, s::8, at:at + 2] = ONE
     else:
         w[..., 0:2] = 0
         w[:, s::8, 0:2] = ONE
@@ -78,7 +87,9 @@ def expected(wtype, w, x, s, min_term=False):
         q = oracle.quantize_q8_1(x[t])
         dots, sums = oracle.ob_subdots(wtype, k, n, w, q)
         if min_term:
-            out[t, :] = -float(sums.reshape(-1, 8)[:, s].astype(np.int64).sum())
+            # K-quants subtract dmin * m * sum, the 32-value formats add m * sum
+            sign = 1.0 if wtype in NIBBLE32 else -1.0
+            out[t, :] = sign * float(sums.reshape(-1, 8)[:, s].astype(np.int64).sum())
         else:
             out[t] = dots.reshape(n, -1, per)[:, :, s].astype(np.int64).sum(axis=1)
     return out
@@ -94,14 +105,14 @@ def check(run, wtype, n, k, m, seed, subs=None):
     for s in (range(SUBS[wtype]) if subs is None else subs):
         got = run(dev(isolate(wtype, w, s)), xd).cpu().numpy().astype(np.float64)
         assert np.array_equal(got, expected(wtype, w, x, s)), f"sub-block {s}"
-    if wtype in (Q4K, Q5K):
+    if wtype in (Q4K, Q5K) or NIBBLE32.get(wtype, (0, None))[1] is not None:
         for s in ((0, 3, 4, 7) if subs is None else subs[:1]):
             got = run(dev(isolate(wtype, w, s, min_term=True)), xd).cpu().numpy().astype(np.float64)
             assert np.array_equal(got, expected(wtype, w, x, s, min_term=True)), f"min term of sub-block {s}"
 
 
 # m <= 64: the int8 tiles (TM 32 / 64); above: TM 128, and for Q4_K the f16-operand tiles
-@pytest.mark.parametrize("wtype", [Q4K, Q5K, Q6K, Q80])
+@pytest.mark.parametrize("wtype", [Q4K, Q5K, Q6K, Q80] + sorted(NIBBLE32))
 @pytest.mark.parametrize("m", [5, 40, 64, 65, 130])
 def test_tiled_matmul_emits_the_exact_subblock_integers(wtype, m):
     n, k = 96, 1024
