@@ -257,6 +257,14 @@ int launch_mmq_gguf_q5_1(void* tmp_fixup, const void* x, const void* y, void* ds
                          int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
                          void* stream);
 
+/* Q3_K (110-byte super-blocks, stride_row_x = k / 256; weights 2-byte aligned) on the Q6_K tile shape:
+ * codes -4..3, one six-bit scale less 32 per 16 values.
+ * Replaces launch_mmq_gguf_q3_k (src/tensor/quantized/mmq.rs:281). */
+int launch_mmq_gguf_q3_k(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * MoE prefill: expert-batched tiled matmul and the steps around it. Names and argument lists are
  * loken's (src/tensor/quantized/mmq.rs:151-173; src/inference/moe_cuda/mmq_experts.rs:42-56),
@@ -336,6 +344,22 @@ int launch_mmq_moe_gguf_mxfp4(const void* x, const void* x_second, int64_t dst_s
                               int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
                               int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
                               int64_t smpbo, int warp_size, void* stream);
+
+/* Q3_K, and IQ4_XS (expert-only in the reference: eight runs of IQ4_NL levels under six-bit scales
+ * less 32; weights 4-byte aligned). Replaces launch_mmq_moe_gguf_{q3_k,iq4_xs}
+ * (src/tensor/quantized/mmq.rs:281, 329). */
+int launch_mmq_moe_gguf_q3_k(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_iq4_xs(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                               void* dst, const int* expert_bounds, const int* ids_dst,
+                               int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                               int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                               int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                               int64_t smpbo, int warp_size, void* stream);
 
 /* From a routing already sorted by expert: bounds[e] = first sorted row of expert >= e
  * (n_experts + 1 entries), slots_out = slots, src_rows[i] = slots[i] / topk.

@@ -360,6 +360,119 @@ using MmqQ51 = MmqLegacy<LK_TYPE_Q5_1>;
 using MmqIq4Nl = MmqLegacy<LK_TYPE_IQ4_NL>;
 using MmqMxfp4 = MmqLegacy<LK_TYPE_MXFP4>;
 
+// Q3_K {hmask[32], qs[64], scales[12], d} (110 bytes; src/tensor/quant_cpu/format/q3_k.rs:10-37, 127-146):
+// sixteen six-bit scales (less 32), one per 16 values, over codes (two bits, less four where the hmask
+// bit is clear) in -4..3: Q6_K's tile shape, two scales per 32-value sub-block. A thread takes one half
+// (128 values) of a row's super-block: its four sub-blocks share the same 32 code bytes at four shifts.
+struct MmqQ3K {
+    static constexpr int ALIGN = 2;
+    static constexpr int BLOCK_BYTES = 110;
+    static constexpr int NS = 16;
+    static constexpr bool HAS_MIN = false;
+    static constexpr bool F16_TILES = false;
+    static constexpr int BLOCKS_PER_STEP = 1;
+    static_assert(TN * 2 == MMQ_WG, "one (row, half) per thread");
+
+    struct Frag {
+        uint4 q0, q1, h0, h1;
+        uint32_t s0, s1, s2, d;
+    };
+    static __device__ __forceinline__ void fetch(Frag& f, const uint8_t* __restrict__ w, int64_t nb, int kb,
+                                                 int n0, int n) {
+        const int row = threadIdx.x >> 1, half = threadIdx.x & 1;
+        const int gn = min(n0 + row, n - 1);
+        const uint8_t* bp = w + ((int64_t)gn * nb + kb) * BLOCK_BYTES;
+        f.q0 = *(const uint4_a2*)(bp + 32 + 32 * half);
+        f.q1 = *(const uint4_a2*)(bp + 48 + 32 * half);
+        f.h0 = *(const uint4_a2*)bp;
+        f.h1 = *(const uint4_a2*)(bp + 16);
+        f.s0 = *(const uint32_a2*)(bp + 96);
+        f.s1 = *(const uint32_a2*)(bp + 100);
+        f.s2 = *(const uint32_a2*)(bp + 104);
+        f.d = *(const uint16_t*)(bp + 108);
+    }
+    // two-bit codes less four where `clear` holds a 1, as int8: 0x80 + q - 4 never borrows
+    static __device__ __forceinline__ uint32_t signed_codes(uint32_t q, uint32_t clear) {
+        return ((q | 0x80808080u) - (clear << 2)) ^ 0x80808080u;
+    }
+    static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
+        (void)wmn;
+        const int row = threadIdx.x >> 1, half = threadIdx.x & 1;
+        const float d = n0 + row < n ? f16_bits_to_f32(f.d) : 0.f;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int j = 4 * half + jj, shift = 2 * jj;
+            const uint32_t m2 = 0x03030303u, m1 = 0x01010101u;
+            uint4 lo, hi;
+            lo.x = signed_codes((f.q0.x >> shift) & m2, (~f.h0.x >> j) & m1);
+            lo.y = signed_codes((f.q0.y >> shift) & m2, (~f.h0.y >> j) & m1);
+            lo.z = signed_codes((f.q0.z >> shift) & m2, (~f.h0.z >> j) & m1);
+            lo.w = signed_codes((f.q0.w >> shift) & m2, (~f.h0.w >> j) & m1);
+            hi.x = signed_codes((f.q1.x >> shift) & m2, (~f.h1.x >> j) & m1);
+            hi.y = signed_codes((f.q1.y >> shift) & m2, (~f.h1.y >> j) & m1);
+            hi.z = signed_codes((f.q1.z >> shift) & m2, (~f.h1.z >> j) & m1);
+            hi.w = signed_codes((f.q1.w >> shift) & m2, (~f.h1.w >> j) & m1);
+            *(uint4*)(wq + (j * TN + row) * 32) = lo;
+            *(uint4*)(wq + (j * TN + row) * 32 + 16) = hi;
+            // scales 2 j and 2 j + 1 of the sixteen packed in twelve bytes (scale i: low four bits =
+            // nibble i / 8 of byte i % 8, top two = bits 2 (i / 4) of byte 8 + i % 4)
+            const int group = j >> 1, at = 2 * (j & 1);
+            const uint32_t low = ((group & 1) ? f.s1 : f.s0) >> (8 * at + (group < 2 ? 0 : 4));
+            const uint32_t top = f.s2 >> (8 * at + 2 * group);
+            const int sc0 = (int)((low & 15u) | ((top & 3u) << 4)) - 32;
+            const int sc1 = (int)(((low >> 8) & 15u) | (((top >> 8) & 3u) << 4)) - 32;
+            wsc[(2 * j) * TN + row] = d * (float)sc0;
+            wsc[(2 * j + 1) * TN + row] = d * (float)sc1;
+        }
+    }
+};
+
+// IQ4_XS {d, scales_h, scales_l[4], qs[128]} (136 bytes; src/tensor/quant_cpu/format/iq4_xs.rs:5-37): eight
+// runs of 32 values, each IQ4_NL levels under one six-bit scale less 32: the Q4_K tile shape without a
+// minimum. A thread takes (row, run) items.
+struct MmqIq4Xs {
+    static constexpr int ALIGN = 4;
+    static constexpr int BLOCK_BYTES = 136;
+    static constexpr int NS = 8;
+    static constexpr bool HAS_MIN = false;
+    static constexpr bool F16_TILES = false;
+    static constexpr int BLOCKS_PER_STEP = 1;
+    static constexpr int PER = TN * 8 / MMQ_WG;
+
+    struct Frag {
+        uint4 q[PER];
+        uint2 head[PER];
+    };
+    static __device__ __forceinline__ void fetch(Frag& f, const uint8_t* __restrict__ w, int64_t nb, int kb,
+                                                 int n0, int n) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, j = idx & 7;
+            const int gn = min(n0 + row, n - 1);
+            const uint8_t* bp = w + ((int64_t)gn * nb + kb) * BLOCK_BYTES;
+            f.q[i] = *(const uint4_a4*)(bp + 8 + 16 * j);
+            f.head[i] = *(const uint2_a2*)bp;   // d, scales_h | scales_l[4]
+        }
+    }
+    static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
+        (void)wmn;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, j = idx & 7;
+            const uint4 q = f.q[i];
+            const uint4 lo = make_uint4(levels_of<1>(q.x & 0x0F0F0F0Fu), levels_of<1>(q.y & 0x0F0F0F0Fu),
+                                        levels_of<1>(q.z & 0x0F0F0F0Fu), levels_of<1>(q.w & 0x0F0F0F0Fu));
+            const uint4 hi = make_uint4(levels_of<1>((q.x >> 4) & 0x0F0F0F0Fu), levels_of<1>((q.y >> 4) & 0x0F0F0F0Fu),
+                                        levels_of<1>((q.z >> 4) & 0x0F0F0F0Fu), levels_of<1>((q.w >> 4) & 0x0F0F0F0Fu));
+            *(uint4*)(wq + (j * TN + row) * 32) = lo;
+            *(uint4*)(wq + (j * TN + row) * 32 + 16) = hi;
+            const uint32_t low = (f.head[i].y >> (4 * j)) & 15u, high = (f.head[i].x >> (16 + 2 * j)) & 3u;
+            const int sc = (int)(low | (high << 4)) - 32;
+            wsc[j * TN + row] = n0 + row < n ? f16_bits_to_f32(f.head[i].x & 0xFFFFu) * (float)sc : 0.f;
+        }
+    }
+};
+
 // Token rows [m0, m0+TM) of block kb (record layout above). Rows at or past m_end read as zeros.
 template <int TM>
 struct TokenFrag {
@@ -791,6 +904,7 @@ LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q4_0, MmqQ40)
 LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q4_1, MmqQ41)
 LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q5_0, MmqQ50)
 LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q5_1, MmqQ51)
+LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q3_k, MmqQ3K)
 
 #define LK_MMQ_MOE_ENTRY(NAME, FMT)                                                                     \
     extern "C" int NAME(const void* x, const void* x_second, int64_t dst_second, const void* y,        \
@@ -815,3 +929,5 @@ LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q5_0, MmqQ50)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q5_1, MmqQ51)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq4_nl, MmqIq4Nl)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_mxfp4, MmqMxfp4)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q3_k, MmqQ3K)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq4_xs, MmqIq4Xs)

@@ -88,15 +88,15 @@ def test_expert_batched_block_matches_oracle(tokens, hidden, ffn, n_experts, top
 
 
 NIBBLE_TILES = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
-                "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4}
+                "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "iq4_xs": lib.TYPE_IQ4_XS, "q3_k": lib.TYPE_Q3_K}
 
 
 @pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(40, 1024, 512, 8, 3), (70, 512, 768, 16, 4),
                                                              (1, 256, 256, 4, 2), (300, 512, 256, 3, 2)])
 @pytest.mark.parametrize("name", sorted(NIBBLE_TILES))
 def test_expert_batched_block_in_the_nibble_formats_matches_oracle(name, tokens, hidden, ffn, n_experts, topk):
-    """The tiled launch for the 32-value formats, IQ4_NL and MXFP4 among them (which have no dense entry
-    point); the last shape runs the 128-token tiles."""
+    """The tiled launch for the 32-value formats, IQ4_XS and Q3_K; IQ4_NL, MXFP4 and IQ4_XS have no dense
+    entry point. The last shape runs the 128-token tiles."""
     dt = NIBBLE_TILES[name]
     assert moe.moe_mmq_serves(dt, hidden)
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=53, dt_down=dt, dt_gu=dt, x_scale=4.0)

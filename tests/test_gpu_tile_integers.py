@@ -32,7 +32,8 @@ pytestmark = pytest.mark.gpu
 Q4K, Q5K, Q6K, Q80 = lib.TYPE_Q4_K, lib.TYPE_Q5_K, lib.TYPE_Q6_K, lib.TYPE_Q8_0
 ONE = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
 NIBBLE32 = {lib.TYPE_Q4_0: (18, None), lib.TYPE_Q4_1: (20, 2), lib.TYPE_Q5_0: (22, None), lib.TYPE_Q5_1: (24, 2)}
-SUBS = {Q4K: 8, Q5K: 8, Q6K: 16, Q80: 8, **{t: 8 for t in NIBBLE32}}
+Q3K = lib.TYPE_Q3_K
+SUBS = {Q4K: 8, Q5K: 8, Q6K: 16, Q80: 8, Q3K: 16, **{t: 8 for t in NIBBLE32}}
 
 
 def dev(a):
@@ -64,6 +65,13 @@ def isolate(wtype, w, s, min_term=False):
         w[..., 192:208] = 0
         w[..., 192 + s] = 1
         w[..., 208:210] = ONE
+    elif wtype == Q3K:
+        # six-bit scales less 32: 33 for sub-block s, 32 for the rest (low nibble i / 8 of byte i % 8,
+        # top two bits in field i / 4 of byte 8 + i % 4)
+        w[..., 96:104] = 0
+        w[..., 104:108] = 0xAA
+        w[..., 96 + s % 8] = 1 << (4 * (s // 8))
+        w[..., 108:110] = ONE
     elif wtype in NIBBLE32:
         # [n, blocks of 32, bytes]: scale 1 on every eighth block, no minimum (or the reverse)
         m_at = NIBBLE32[wtype][1]
@@ -112,7 +120,7 @@ def check(run, wtype, n, k, m, seed, subs=None):
 
 
 # m <= 64: the int8 tiles (TM 32 / 64); above: TM 128, and for Q4_K the f16-operand tiles
-@pytest.mark.parametrize("wtype", [Q4K, Q5K, Q6K, Q80] + sorted(NIBBLE32))
+@pytest.mark.parametrize("wtype", [Q4K, Q5K, Q6K, Q80, Q3K] + sorted(NIBBLE32))
 @pytest.mark.parametrize("m", [5, 40, 64, 65, 130])
 def test_tiled_matmul_emits_the_exact_subblock_integers(wtype, m):
     n, k = 96, 1024
