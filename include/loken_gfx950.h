@@ -200,9 +200,10 @@ int lk_mmvq_exact(int wtype, const void* vx, const void* vy_q8_k, float* dst, in
  * row r of the result is row ids[r] of x (ids nullable); ne00 = values per row, s01/s02/s03 =
  * element strides of row / channel / sample, ne0 = padded row length (multiple of 512),
  * ne1 = rows, ne2 * ne3 = channels. `vy` needs ne1 * (ne0/128) * 144 bytes per channel, the
- * size loken allocates. D4 (scale only: Q6_K, Q8_0) and DS4 (scale and sum: Q4_K) write the
- * same records here. D2S6 serves Q2_K alone and is not part of this library.
- * Replaces launch_mmq_quantize_q8_1_{D4,DS4} of cuda/mmq_gguf/mmq_quantize.cu:67-166; codes
+ * size loken allocates. D4 (scale only: Q6_K, Q8_0), DS4 (scale and sum: Q4_K) and D2S6 (Q2_K: in
+ * the reference a scale per 64 values and sums per 16) write the same records here: a scale and a
+ * sum per 32 values, the Q2_K tile forming its sums per 16 from the codes.
+ * Replaces launch_mmq_quantize_q8_1_{D4,DS4,D2S6} of cuda/mmq_gguf/mmq_quantize.cu:67-166; codes
  * follow BlockQ8_1::quantize (1/d rule), not that file's 127/amax rule, so that tiled and
  * mat-vec products see the same integers. */
 void launch_mmq_quantize_q8_1_D4(const void* x, const int32_t* ids, void* vy, int type_x,
@@ -211,6 +212,9 @@ void launch_mmq_quantize_q8_1_D4(const void* x, const int32_t* ids, void* vy, in
 void launch_mmq_quantize_q8_1_DS4(const void* x, const int32_t* ids, void* vy, int type_x,
                                   int64_t ne00, int64_t s01, int64_t s02, int64_t s03, int64_t ne0,
                                   int64_t ne1, int64_t ne2, int64_t ne3, void* stream);
+void launch_mmq_quantize_q8_1_D2S6(const void* x, const int32_t* ids, void* vy, int type_x,
+                                   int64_t ne00, int64_t s01, int64_t s02, int64_t s03, int64_t ne0,
+                                   int64_t ne1, int64_t ne2, int64_t ne3, void* stream);
 
 /* dst[col, row] (f32, rows `stride_col_dst` floats apart) = weight row `row` . token `col`.
  *   x = weights [nrows_x][stride_row_x blocks], y = workspace of ncols_y rows, ncols_x = k.
@@ -261,6 +265,14 @@ int launch_mmq_gguf_q5_1(void* tmp_fixup, const void* x, const void* y, void* ds
  * codes -4..3, one six-bit scale less 32 per 16 values.
  * Replaces launch_mmq_gguf_q3_k (src/tensor/quantized/mmq.rs:281). */
 int launch_mmq_gguf_q3_k(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
+                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
+                         int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
+                         void* stream);
+
+/* Q2_K (84-byte super-blocks, weights 4-byte aligned): unsigned two-bit codes, a four-bit scale and a
+ * four-bit minimum per 16 values, the minimum against the token's sums per 16 codes.
+ * Replaces launch_mmq_gguf_q2_k (src/tensor/quantized/mmq.rs:280). */
+int launch_mmq_gguf_q2_k(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
                          int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
                          int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
                          void* stream);
@@ -360,6 +372,14 @@ int launch_mmq_moe_gguf_iq4_xs(const void* x, const void* x_second, int64_t dst_
                                int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
                                int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
                                int64_t smpbo, int warp_size, void* stream);
+
+/* Replaces launch_mmq_moe_gguf_q2_k (src/tensor/quantized/mmq.rs:280). */
+int launch_mmq_moe_gguf_q2_k(const void* x, const void* x_second, int64_t dst_second, const void* y,
+                             void* dst, const int* expert_bounds, const int* ids_dst,
+                             int64_t stride_expert_x, int64_t ncols_x, int64_t nrows_x,
+                             int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst,
+                             int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
+                             int64_t smpbo, int warp_size, void* stream);
 
 /* From a routing already sorted by expert: bounds[e] = first sorted row of expert >= e
  * (n_experts + 1 entries), slots_out = slots, src_rows[i] = slots[i] / topk.

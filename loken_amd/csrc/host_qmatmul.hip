@@ -98,7 +98,7 @@ void mark_used(Slot& slot, hipStream_t stream) {
 }
 
 // The 32-value nibble formats and the two-bit K-quants: served by the plain mat-vec (four of them by the
-// tiled matmul as well, and Q3_K, from the row counts of nibble_tiles_pay below).
+// tiled matmul as well, and Q2_K / Q3_K, from the row counts of nibble_tiles_pay below).
 bool matvec_only(int dtype) {
     return dtype == LK_TYPE_Q4_0 || dtype == LK_TYPE_Q4_1 || dtype == LK_TYPE_Q5_0 || dtype == LK_TYPE_Q5_1 ||
            dtype == LK_TYPE_IQ4_NL || dtype == LK_TYPE_MXFP4 || dtype == LK_TYPE_Q2_K || dtype == LK_TYPE_Q3_K ||
@@ -106,7 +106,8 @@ bool matvec_only(int dtype) {
 }
 
 bool nibble_tiles(int dtype) {
-    return dtype == LK_TYPE_Q4_0 || dtype == LK_TYPE_Q4_1 || dtype == LK_TYPE_Q5_0 || dtype == LK_TYPE_Q5_1 || dtype == LK_TYPE_Q3_K;
+    return dtype == LK_TYPE_Q4_0 || dtype == LK_TYPE_Q4_1 || dtype == LK_TYPE_Q5_0 || dtype == LK_TYPE_Q5_1 || dtype == LK_TYPE_Q3_K ||
+           dtype == LK_TYPE_Q2_K;
 }
 
 bool tiled_serves(int dtype, int k) {
@@ -117,11 +118,11 @@ bool tiled_serves(int dtype, int k) {
 // Q4_0 / Q4_1 / Q5_0 / Q5_1: rows from which one tiled launch beats mat-vec launches of eight rows each.
 // Measured on MI355X (Q4_0 and Q5_1 alike): 2048 x 2048 and 4096 x 4096 from 56-64 rows (48 rows: 67 us
 // against 77), 4096 x 14336 likewise, 14336 x 4096 from 24 (74 us against 60; 16 rows: 50 against 60).
-// Q3_K, whose mat-vec is slower: 4096 x 4096 from 48 rows (89 us against 85; 32 rows: 60 against 61),
+// Q3_K (and Q2_K, taken alike), whose mat-vec is slower: 4096 x 4096 from 48 rows (89 us against 85; 32 rows: 60 against 61),
 // 14336 x 4096 from 16 (78 against 61; 9 rows: 52 against 60).
 bool nibble_tiles_pay(int dtype, int n, int k, int rows) {
     if (!nibble_tiles(dtype) || k % 256 != 0) return false;
-    if (dtype == LK_TYPE_Q3_K) return rows > 40 || (long long)rows * n >= 200000;
+    if (dtype == LK_TYPE_Q3_K || dtype == LK_TYPE_Q2_K) return rows > 40 || (long long)rows * n >= 200000;
     return rows > 48 || (long long)rows * n >= 300000;
 }
 
@@ -186,7 +187,7 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     // --- mat-vec family: up to matvec_rows, or any count when every row must sum like a one-row call
     const bool to_rows_kernel = x_type == LK_TYPE_F32 && small_rows_kernel_pays(dtype_, n_, k_, rows);
     const bool to_nibble_tiles = x_type == LK_TYPE_F32 && !decode_order && nibble_tiles_pay(dtype_, n_, k_, rows) &&
-                                 ((uintptr_t)blob_ & 1) == 0;
+                                 ((uintptr_t)blob_ & (dtype_ == LK_TYPE_Q2_K ? 3 : 1)) == 0;
     if ((rows <= mv_max && !to_rows_kernel) || decode_order || (plain && !to_nibble_tiles)) {
         if (!plain && x_type == LK_TYPE_F32 && rows <= 2 && k_ <= 8192 && ((uintptr_t)x & 15) == 0 && k_ % 4 == 0) {
             const void* vx[1] = {blob_};
@@ -239,8 +240,10 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     std::lock_guard<std::mutex> pair(slot.mu);
     if (int rc = reserve(slot, ws_bytes, true, stream)) return rc;
     // the layouts of the reference's table (quantized/mmq.rs:274-285)
-    auto quantizer = dtype_ == LK_TYPE_Q6_K || dtype_ == LK_TYPE_Q8_0 || dtype_ == LK_TYPE_Q5_0 || dtype_ == LK_TYPE_Q3_K ? launch_mmq_quantize_q8_1_D4
-                                                                                               : launch_mmq_quantize_q8_1_DS4;
+    auto quantizer = dtype_ == LK_TYPE_Q2_K ? launch_mmq_quantize_q8_1_D2S6
+                     : dtype_ == LK_TYPE_Q6_K || dtype_ == LK_TYPE_Q8_0 || dtype_ == LK_TYPE_Q5_0 || dtype_ == LK_TYPE_Q3_K
+                         ? launch_mmq_quantize_q8_1_D4
+                         : launch_mmq_quantize_q8_1_DS4;
     quantizer(x, nullptr, slot.act, 0, k_, k_, 0, 0, (int64_t)k_padded, rows, 1, 1, stream);
     auto launcher = dtype_ == LK_TYPE_Q4_K   ? launch_mmq_gguf_q4_k
                     : dtype_ == LK_TYPE_Q5_K ? launch_mmq_gguf_q5_k
@@ -250,6 +253,7 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
                     : dtype_ == LK_TYPE_Q5_0 ? launch_mmq_gguf_q5_0
                     : dtype_ == LK_TYPE_Q5_1 ? launch_mmq_gguf_q5_1
                     : dtype_ == LK_TYPE_Q3_K ? launch_mmq_gguf_q3_k
+                    : dtype_ == LK_TYPE_Q2_K ? launch_mmq_gguf_q2_k
                                              : launch_mmq_gguf_q8_0;
     int abi = 0, cus = 0, lds = 0, wave = 0;
     (void)lk_device_info(&abi, &cus, &lds, &wave);

@@ -115,6 +115,7 @@ struct MmqQ45K {
     static constexpr bool F16_TILES = !Q5;   // Q4_K above 64 tokens: the f16 tile kernel
     static constexpr int NS = 8;          // one weight scale per 32 values
     static constexpr bool HAS_MIN = true;
+    static constexpr int MIN_RANK = 8;   // one minimum per 32 values
     static constexpr int BLOCKS_PER_STEP = 1;
     static constexpr int QCH = TN * 8 / MMQ_WG;   // 16-byte qs chunks per thread per step
 
@@ -194,6 +195,7 @@ struct MmqQ6K {
     static constexpr int BLOCK_BYTES = Q6K_BYTES;
     static constexpr int NS = 16;
     static constexpr bool HAS_MIN = false;
+    static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
     static constexpr int BLOCKS_PER_STEP = 1;
     static constexpr int QCH = TN * 8 / MMQ_WG;
@@ -258,6 +260,7 @@ struct MmqQ80 {
     static constexpr int ALIGN = 2;
     static constexpr int NS = 8;
     static constexpr bool HAS_MIN = false;
+    static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
     static constexpr int BLOCKS_PER_STEP = 8;
     static constexpr int QCH = TN * 16 / MMQ_WG, DCH = TN * 8 / MMQ_WG;
@@ -308,6 +311,7 @@ struct MmqLegacy {
     static constexpr int BLOCK_BYTES = L::BYTES;
     static constexpr int NS = 8;
     static constexpr bool HAS_MIN = L::M_AT >= 0;
+    static constexpr int MIN_RANK = HAS_MIN ? 8 : 0;
     static constexpr bool F16_TILES = false;
     static constexpr int BLOCKS_PER_STEP = 8;
     static constexpr int ALIGN = L::BYTES % 2 ? 1 : 2;
@@ -369,6 +373,7 @@ struct MmqQ3K {
     static constexpr int BLOCK_BYTES = 110;
     static constexpr int NS = 16;
     static constexpr bool HAS_MIN = false;
+    static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
     static constexpr int BLOCKS_PER_STEP = 1;
     static_assert(TN * 2 == MMQ_WG, "one (row, half) per thread");
@@ -427,6 +432,57 @@ struct MmqQ3K {
     }
 };
 
+// Q2_K {scales[16], qs[64], d, dmin} (84 bytes; src/tensor/quant_cpu/format/q2_k.rs:15-33): sixteen groups of
+// sixteen two-bit codes, byte g of scales = scale (low nibble) and minimum (high nibble) of group g:
+// d * scale * q - dmin * minimum. Q3_K's tile shape with unsigned codes, and the minimum as a rank-16
+// update against the token's sums per 16 codes (cuda/moe/gguf.cuh:524-546 combines per group likewise).
+struct MmqQ2K {
+    static constexpr int ALIGN = 4;
+    static constexpr int BLOCK_BYTES = 84;
+    static constexpr int NS = 16;
+    static constexpr bool HAS_MIN = true;
+    static constexpr int MIN_RANK = 16;
+    static constexpr bool F16_TILES = false;
+    static constexpr int BLOCKS_PER_STEP = 1;
+    static_assert(TN * 2 == MMQ_WG, "one (row, half) per thread");
+
+    struct Frag {
+        uint4 q0, q1;
+        uint2 sm;       // the half's eight scale | minimum bytes
+        uint32_t dm;    // d | dmin << 16
+    };
+    static __device__ __forceinline__ void fetch(Frag& f, const uint8_t* __restrict__ w, int64_t nb, int kb,
+                                                 int n0, int n) {
+        const int row = threadIdx.x >> 1, half = threadIdx.x & 1;
+        const int gn = min(n0 + row, n - 1);
+        const uint8_t* bp = w + ((int64_t)gn * nb + kb) * BLOCK_BYTES;
+        f.q0 = *(const uint4_a4*)(bp + 16 + 32 * half);
+        f.q1 = *(const uint4_a4*)(bp + 32 + 32 * half);
+        f.sm = make_uint2(*(const uint32_t*)(bp + 8 * half), *(const uint32_t*)(bp + 8 * half + 4));
+        f.dm = *(const uint32_t*)(bp + 80);
+    }
+    static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
+        const int row = threadIdx.x >> 1, half = threadIdx.x & 1;
+        const bool live = n0 + row < n;
+        const float d = live ? f16_bits_to_f32(f.dm & 0xFFFFu) : 0.f;
+        const float dmin = live ? f16_bits_to_f32(f.dm >> 16) : 0.f;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int j = 4 * half + jj, shift = 2 * jj;
+            const uint32_t m2 = 0x03030303u;
+            *(uint4*)(wq + (j * TN + row) * 32) =
+                make_uint4((f.q0.x >> shift) & m2, (f.q0.y >> shift) & m2, (f.q0.z >> shift) & m2, (f.q0.w >> shift) & m2);
+            *(uint4*)(wq + (j * TN + row) * 32 + 16) =
+                make_uint4((f.q1.x >> shift) & m2, (f.q1.y >> shift) & m2, (f.q1.z >> shift) & m2, (f.q1.w >> shift) & m2);
+            const uint32_t pair = ((jj < 2 ? f.sm.x : f.sm.y) >> (16 * (jj & 1))) & 0xFFFFu;   // bytes 2 j, 2 j + 1
+            wsc[(2 * j) * TN + row] = d * (float)(pair & 15u);
+            wsc[(2 * j + 1) * TN + row] = d * (float)((pair >> 8) & 15u);
+            wmn[(2 * j) * TN + row] = -(dmin * (float)((pair >> 4) & 15u));
+            wmn[(2 * j + 1) * TN + row] = -(dmin * (float)(pair >> 12));
+        }
+    }
+};
+
 // IQ4_XS {d, scales_h, scales_l[4], qs[128]} (136 bytes; src/tensor/quant_cpu/format/iq4_xs.rs:5-37): eight
 // runs of 32 values, each IQ4_NL levels under one six-bit scale less 32: the Q4_K tile shape without a
 // minimum. A thread takes (row, run) items.
@@ -435,6 +491,7 @@ struct MmqIq4Xs {
     static constexpr int BLOCK_BYTES = 136;
     static constexpr int NS = 8;
     static constexpr bool HAS_MIN = false;
+    static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
     static constexpr int BLOCKS_PER_STEP = 1;
     static constexpr int PER = TN * 8 / MMQ_WG;
@@ -474,10 +531,13 @@ struct MmqIq4Xs {
 };
 
 // Token rows [m0, m0+TM) of block kb (record layout above). Rows at or past m_end read as zeros.
-template <int TM>
+// S16: the weight format has a minimum per 16 values (Q2_K), so the sums are formed per chunk of 16
+// codes from the codes themselves (the record holds them per 32) and each chunk's thread reads its scale.
+template <int TM, bool S16 = false>
 struct TokenFrag {
     static constexpr int CCH = (TM * 16 + MMQ_WG - 1) / MMQ_WG;   // code chunks per thread
     uint4 codes[CCH];
+    uint32_t chunk_d8[S16 ? CCH : 1];
     uint4 d8, sums;   // thread r < TM: the scales and sums of row r
 
     __device__ __forceinline__ void fetch(const uint8_t* __restrict__ y, int64_t rows_total, int kb, int m0, int m_end) {
@@ -485,8 +545,12 @@ struct TokenFrag {
         for (int i = 0; i < CCH; ++i) {
             const int idx = threadIdx.x + i * MMQ_WG, r = idx >> 4, c = idx & 15;
             codes[i] = make_uint4(0, 0, 0, 0);
-            if (idx < TM * 16 && m0 + r < m_end)
-                codes[i] = *(const uint4*)(y + ((int64_t)kb * rows_total + m0 + r) * REC_BYTES + 16 * c);
+            if (S16) chunk_d8[i] = 0;
+            if (idx < TM * 16 && m0 + r < m_end) {
+                const uint8_t* rec = y + ((int64_t)kb * rows_total + m0 + r) * REC_BYTES;
+                codes[i] = *(const uint4*)(rec + 16 * c);
+                if (S16) chunk_d8[i] = *(const uint16_t*)(rec + 256 + 2 * (c >> 1));
+            }
         }
         d8 = sums = make_uint4(0, 0, 0, 0);
         if ((int)threadIdx.x < TM && m0 + (int)threadIdx.x < m_end) {
@@ -500,7 +564,13 @@ struct TokenFrag {
 #pragma unroll
         for (int i = 0; i < CCH; ++i) {
             const int idx = threadIdx.x + i * MMQ_WG, r = idx >> 4, c = idx & 15;
-            if (idx < TM * 16) *(uint4*)(aq + ((c >> 1) * TM + r) * 32 + 16 * (c & 1)) = codes[i];
+            if (idx < TM * 16) {
+                *(uint4*)(aq + ((c >> 1) * TM + r) * 32 + 16 * (c & 1)) = codes[i];
+                if (S16) {
+                    const uint4 ones = make_uint4(0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u);
+                    ads[c * TM + r] = f16_bits_to_f32(chunk_d8[i]) * (float)dot16(ones, codes[i], 0);
+                }
+            }
         }
         if ((int)threadIdx.x < TM) {
             const int r = threadIdx.x;
@@ -509,7 +579,7 @@ struct TokenFrag {
             for (int s = 0; s < 8; ++s) {
                 const float d = f16_bits_to_f32((dw[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
                 ad8[s * TM + r] = d;
-                if (WITH_SUMS) ads[s * TM + r] = d * (float)(int)(int16_t)((sw[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
+                if (WITH_SUMS && !S16) ads[s * TM + r] = d * (float)(int)(int16_t)((sw[s >> 1] >> (16 * (s & 1))) & 0xFFFFu);
             }
         }
     }
@@ -528,9 +598,9 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
     int8_t* wq = (int8_t*)lds;                       // [8][TN][32]
     int8_t* aq = wq + 8 * TN * 32;                   // [8][TM][32]
     float* wsc = (float*)(aq + 8 * TM * 32);         // [NS][TN]
-    float* wmn = wsc + F::NS * TN;                   // [8][TN]   (HAS_MIN)
-    float* ad8 = wmn + (F::HAS_MIN ? 8 * TN : 0);    // [8][TM]
-    float* ads = ad8 + 8 * TM;                       // [8][TM]   (HAS_MIN)
+    float* wmn = wsc + F::NS * TN;                   // [MIN_RANK][TN]
+    float* ad8 = wmn + F::MIN_RANK * TN;             // [8][TM]
+    float* ads = ad8 + 8 * TM;                       // [MIN_RANK][TM]
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -546,7 +616,7 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
             for (int v = 0; v < 16; ++v) acc[it][jt][v] = 0.f;
 
     typename F::Frag wf;
-    TokenFrag<TM> tf;
+    TokenFrag<TM, F::MIN_RANK == 16> tf;
     F::fetch(wf, pb.w, pb.row_blocks, 0, n0, pb.n);
     tf.fetch(pb.y, pb.rows_total, 0, m0, pb.m_end);
 
@@ -682,9 +752,9 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
             }
         }
         if (F::HAS_MIN) {
-            // acc += (d8*S)[token, s] * (-dmin*m)[s, n], s = 0..7: four K=2 f32 MFMAs per patch
+            // acc += (d8*S)[token, s] * (-dmin*m)[s, n], s = 0..MIN_RANK-1: K=2 f32 MFMAs, two s each
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
+            for (int kk = 0; kk < F::MIN_RANK / 2; ++kk) {
                 float am[IT], bm[JT];
 #pragma unroll
                 for (int it = 0; it < IT; ++it) am[it] = ads[(2 * kk + lh) * TM + (wm * IT + it) * 32 + l32];
@@ -730,7 +800,7 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
 
 template <class F, int TM>
 static constexpr int mmq_lds_bytes() {
-    return 8 * TN * 32 + 8 * TM * 32 + (F::NS * TN + (F::HAS_MIN ? 8 * TN : 0) + 8 * TM + (F::HAS_MIN ? 8 * TM : 0)) * 4;
+    return 8 * TN * 32 + 8 * TM * 32 + (F::NS * TN + F::MIN_RANK * TN + 8 * TM + F::MIN_RANK * TM) * 4;
 }
 
 // Dense product. Workgroup id -> (n tile, m tile) so that the m tiles of one n tile (which
@@ -860,6 +930,12 @@ extern "C" void launch_mmq_quantize_q8_1_DS4(const void* x, const int32_t* ids, 
     launch_quantize(x, ids, vy, type_x, ne00, s01, s02, s03, ne0, ne1, ne2, ne3, stream);
 }
 
+extern "C" void launch_mmq_quantize_q8_1_D2S6(const void* x, const int32_t* ids, void* vy, int type_x,
+                                              int64_t ne00, int64_t s01, int64_t s02, int64_t s03,
+                                              int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3, void* stream) {
+    launch_quantize(x, ids, vy, type_x, ne00, s01, s02, s03, ne0, ne1, ne2, ne3, stream);
+}
+
 extern "C" int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* y, void* dst,
                                     int64_t ncols_x, int64_t nrows_x, int64_t ncols_y,
                                     int64_t stride_row_x, int64_t stride_col_dst, int cc, int nsm,
@@ -905,6 +981,7 @@ LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q4_1, MmqQ41)
 LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q5_0, MmqQ50)
 LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q5_1, MmqQ51)
 LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q3_k, MmqQ3K)
+LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q2_k, MmqQ2K)
 
 #define LK_MMQ_MOE_ENTRY(NAME, FMT)                                                                     \
     extern "C" int NAME(const void* x, const void* x_second, int64_t dst_second, const void* y,        \
@@ -931,3 +1008,4 @@ LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq4_nl, MmqIq4Nl)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_mxfp4, MmqMxfp4)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q3_k, MmqQ3K)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq4_xs, MmqIq4Xs)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q2_k, MmqQ2K)

@@ -42,6 +42,7 @@ SIGNATURES = {
     "lk_mmvq_subdots": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _vp]),
     "launch_mmq_quantize_q8_1_D4": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),
     "launch_mmq_quantize_q8_1_DS4": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),
+    "launch_mmq_quantize_q8_1_D2S6": (None, [_vp, _vp, _vp, _i] + [_i64] * 8 + [_vp]),
     "launch_mmq_gguf_q4_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
     "launch_mmq_gguf_q5_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
     "launch_mmq_gguf_q6_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
@@ -51,6 +52,7 @@ SIGNATURES = {
     "launch_mmq_gguf_q5_0": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
     "launch_mmq_gguf_q5_1": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
     "launch_mmq_gguf_q3_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
+    "launch_mmq_gguf_q2_k": (_i, [_vp, _vp, _vp, _vp] + [_i64] * 5 + [_i, _i, _i64, _i, _vp]),
 }
 _MOE_MMQ = (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _vp] + [_i64] * 6 + [_i, _i64, _i64, _i, _i, _i64, _i, _vp])
 SIGNATURES.update({
@@ -65,6 +67,7 @@ SIGNATURES.update({
     "launch_mmq_moe_gguf_iq4_nl": _MOE_MMQ,
     "launch_mmq_moe_gguf_mxfp4": _MOE_MMQ,
     "launch_mmq_moe_gguf_q3_k": _MOE_MMQ,
+    "launch_mmq_moe_gguf_q2_k": _MOE_MMQ,
     "launch_mmq_moe_gguf_iq4_xs": _MOE_MMQ,
     "loken_moe_mmq_plan": (None, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "loken_moe_mmq_route": (None, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),

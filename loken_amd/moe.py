@@ -21,7 +21,7 @@ MMQ_MOE_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_moe_gguf_q4_k", _lib.TYPE_Q5_K: 
                     # the formats only mixtures store (quantized/mmq.rs:326-334)
                     _lib.TYPE_IQ4_NL: "launch_mmq_moe_gguf_iq4_nl", _lib.TYPE_MXFP4: "launch_mmq_moe_gguf_mxfp4",
                     _lib.TYPE_IQ4_XS: "launch_mmq_moe_gguf_iq4_xs",
-                    _lib.TYPE_Q3_K: "launch_mmq_moe_gguf_q3_k"}
+                    _lib.TYPE_Q3_K: "launch_mmq_moe_gguf_q3_k", _lib.TYPE_Q2_K: "launch_mmq_moe_gguf_q2_k"}
 MMQ_X_MIN, GRID_Y_MAX = 8, 65535
 
 

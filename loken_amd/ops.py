@@ -184,13 +184,14 @@ MMQ_QUANTIZER = {_lib.TYPE_Q4_K: "launch_mmq_quantize_q8_1_DS4", _lib.TYPE_Q5_K:
                  _lib.TYPE_Q4_0: "launch_mmq_quantize_q8_1_DS4", _lib.TYPE_Q4_1: "launch_mmq_quantize_q8_1_DS4",
                  _lib.TYPE_Q5_0: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_Q5_1: "launch_mmq_quantize_q8_1_DS4",
                  _lib.TYPE_IQ4_NL: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_MXFP4: "launch_mmq_quantize_q8_1_D4",
-                 _lib.TYPE_Q3_K: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_IQ4_XS: "launch_mmq_quantize_q8_1_D4"}
+                 _lib.TYPE_Q3_K: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_IQ4_XS: "launch_mmq_quantize_q8_1_D4",
+                 _lib.TYPE_Q2_K: "launch_mmq_quantize_q8_1_D2S6"}
 MMQ_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_gguf_q4_k", _lib.TYPE_Q5_K: "launch_mmq_gguf_q5_k",
                 _lib.TYPE_Q6_K: "launch_mmq_gguf_q6_k",
                 _lib.TYPE_Q8_0: "launch_mmq_gguf_q8_0",
                 _lib.TYPE_Q4_0: "launch_mmq_gguf_q4_0", _lib.TYPE_Q4_1: "launch_mmq_gguf_q4_1",
                 _lib.TYPE_Q5_0: "launch_mmq_gguf_q5_0", _lib.TYPE_Q5_1: "launch_mmq_gguf_q5_1",
-                _lib.TYPE_Q3_K: "launch_mmq_gguf_q3_k"}
+                _lib.TYPE_Q3_K: "launch_mmq_gguf_q3_k", _lib.TYPE_Q2_K: "launch_mmq_gguf_q2_k"}
 MMQ_DEVICE_INFO = dict(cc=0x1000950, nsm=256, smpbo=160 * 1024, warp_size=64)
 
 

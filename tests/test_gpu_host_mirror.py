@@ -65,6 +65,7 @@ def close(got, want, rtol=1e-3, atol=1e-4):
     # four of the 32-value formats have tiles: from 49 rows, or n x rows of 300 thousand
     ("q4_0", 50, 200, "tiled"), ("q5_0", 64, 200, "tiled"), ("q5_1", 30, 12000, "tiled"), ("q4_1", 20, 12000, "matvec"),
     ("q4_1", 130, 300, "tiled"), ("iq4_nl", 60, 200, "matvec"), ("q3_k", 41, 200, "tiled"), ("q3_k", 17, 12000, "tiled"),
+    ("q2_k", 50, 200, "tiled"),
     ("mxfp4", 17, 200, "matvec"), ("q2_k", 12, 200, "matvec"), ("q3_k", 1, 200, "matvec")])
 def test_forward_takes_the_path_of_its_row_count_and_matches_the_oracle(name, rows, n, expect):
     wtype, k = DT[name], 1024

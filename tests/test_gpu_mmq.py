@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 DT = {"q4_k": lib.TYPE_Q4_K, "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0,
       "q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
-      "q3_k": lib.TYPE_Q3_K}
+      "q3_k": lib.TYPE_Q3_K, "q2_k": lib.TYPE_Q2_K}
 SERVED = [name for name in DT if hasattr(lib.load(), ops.MMQ_LAUNCHER[DT[name]])]
 RTOL, ATOL = 1e-3, 1e-4
 

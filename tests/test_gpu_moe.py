@@ -88,7 +88,8 @@ def test_expert_batched_block_matches_oracle(tokens, hidden, ffn, n_experts, top
 
 
 NIBBLE_TILES = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
-                "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "iq4_xs": lib.TYPE_IQ4_XS, "q3_k": lib.TYPE_Q3_K}
+                "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "iq4_xs": lib.TYPE_IQ4_XS, "q3_k": lib.TYPE_Q3_K,
+                "q2_k": lib.TYPE_Q2_K}
 
 
 @pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(40, 1024, 512, 8, 3), (70, 512, 768, 16, 4),

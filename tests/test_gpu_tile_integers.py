@@ -32,8 +32,8 @@ pytestmark = pytest.mark.gpu
 Q4K, Q5K, Q6K, Q80 = lib.TYPE_Q4_K, lib.TYPE_Q5_K, lib.TYPE_Q6_K, lib.TYPE_Q8_0
 ONE = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
 NIBBLE32 = {lib.TYPE_Q4_0: (18, None), lib.TYPE_Q4_1: (20, 2), lib.TYPE_Q5_0: (22, None), lib.TYPE_Q5_1: (24, 2)}
-Q3K = lib.TYPE_Q3_K
-SUBS = {Q4K: 8, Q5K: 8, Q6K: 16, Q80: 8, Q3K: 16, **{t: 8 for t in NIBBLE32}}
+Q3K, Q2K = lib.TYPE_Q3_K, lib.TYPE_Q2_K
+SUBS = {Q4K: 8, Q5K: 8, Q6K: 16, Q80: 8, Q3K: 16, Q2K: 16, **{t: 8 for t in NIBBLE32}}
 
 
 def dev(a):
@@ -72,6 +72,12 @@ def isolate(wtype, w, s, min_term=False):
         w[..., 104:108] = 0xAA
         w[..., 96 + s % 8] = 1 << (4 * (s // 8))
         w[..., 108:110] = ONE
+    elif wtype == Q2K:
+        # byte g of the header: scale | minimum << 4 of group g
+        w[..., 0:16] = 0
+        w[..., s] = 16 if min_term else 1
+        w[..., 80:82] = 0 if min_term else ONE
+        w[..., 82:84] = ONE if min_term else 0
     elif wtype in NIBBLE32:
         # [n, blocks of 32, bytes]: scale 1 on every eighth block, no minimum (or the reverse)
         m_at = NIBBLE32[wtype][1]
@@ -94,7 +100,11 @@ def expected(wtype, w, x, s, min_term=False):
     for t in range(x.shape[0]):
         q = oracle.quantize_q8_1(x[t])
         dots, sums = oracle.ob_subdots(wtype, k, n, w, q)
-        if min_term:
+        if min_term and wtype == Q2K:
+            # the sums per 16 codes, which the Q8_1 row does not carry: from its codes
+            codes = q.reshape(-1, 36)[:, 4:].view(np.int8).astype(np.int64).reshape(-1, 16, 16)
+            out[t, :] = -float(codes[:, s, :].sum())
+        elif min_term:
             # K-quants subtract dmin * m * sum, the 32-value formats add m * sum
             sign = 1.0 if wtype in NIBBLE32 else -1.0
             out[t, :] = sign * float(sums.reshape(-1, 8)[:, s].astype(np.int64).sum())
@@ -113,14 +123,14 @@ def check(run, wtype, n, k, m, seed, subs=None):
     for s in (range(SUBS[wtype]) if subs is None else subs):
         got = run(dev(isolate(wtype, w, s)), xd).cpu().numpy().astype(np.float64)
         assert np.array_equal(got, expected(wtype, w, x, s)), f"sub-block {s}"
-    if wtype in (Q4K, Q5K) or NIBBLE32.get(wtype, (0, None))[1] is not None:
-        for s in ((0, 3, 4, 7) if subs is None else subs[:1]):
+    if wtype in (Q4K, Q5K, Q2K) or NIBBLE32.get(wtype, (0, None))[1] is not None:
+        for s in (((0, 3, 4, 7, 9, 15) if wtype == Q2K else (0, 3, 4, 7)) if subs is None else subs[:1]):
             got = run(dev(isolate(wtype, w, s, min_term=True)), xd).cpu().numpy().astype(np.float64)
             assert np.array_equal(got, expected(wtype, w, x, s, min_term=True)), f"min term of sub-block {s}"
 
 
 # m <= 64: the int8 tiles (TM 32 / 64); above: TM 128, and for Q4_K the f16-operand tiles
-@pytest.mark.parametrize("wtype", [Q4K, Q5K, Q6K, Q80, Q3K] + sorted(NIBBLE32))
+@pytest.mark.parametrize("wtype", [Q4K, Q5K, Q6K, Q80, Q3K, Q2K] + sorted(NIBBLE32))
 @pytest.mark.parametrize("m", [5, 40, 64, 65, 130])
 def test_tiled_matmul_emits_the_exact_subblock_integers(wtype, m):
     n, k = 96, 1024
