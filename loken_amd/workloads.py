@@ -29,7 +29,8 @@ HBM_PEAK_GBS = 8000.0
 INT8_PEAK_TOPS = 5000.0
 F16_PEAK_TFLOPS = 2500.0
 Q4K, Q6K, Q80 = lib.TYPE_Q4_K, lib.TYPE_Q6_K, lib.TYPE_Q8_0
-NAMES = {Q4K: "Q4_K", Q6K: "Q6_K", Q80: "Q8_0"}
+NAMES = {Q4K: "Q4_K", Q6K: "Q6_K", Q80: "Q8_0", lib.TYPE_Q5_K: "Q5_K", lib.TYPE_Q2_K: "Q2_K", lib.TYPE_Q3_K: "Q3_K",
+         lib.TYPE_Q4_0: "Q4_0", lib.TYPE_Q4_1: "Q4_1", lib.TYPE_Q5_0: "Q5_0", lib.TYPE_Q5_1: "Q5_1"}
 
 
 # ---------------------------------------------------------------------------- synthetic blocks
@@ -70,7 +71,12 @@ class Maker:
         return w.reshape(-1)
 
     def make(self, wtype, n, k):
-        return {Q4K: self.q4k, Q6K: self.q6k, Q80: self.q80}[wtype](n, k)
+        if wtype in (Q4K, Q6K, Q80):
+            return {Q4K: self.q4k, Q6K: self.q6k, Q80: self.q80}[wtype](n, k)
+        # any other format: 256 rows of the seeded host generator, repeated (the kernels do not care what
+        # the blocks hold)
+        base = torch.from_numpy(synth.weight(wtype, 256, k, seed=0, stream=wtype)).to(self.dev).reshape(256, -1)
+        return base.repeat((n + 255) // 256, 1)[:n].contiguous().reshape(-1)
 
     def randn(self, *shape):
         return torch.randn(shape, device=self.dev, generator=self.gen)
@@ -268,6 +274,10 @@ def gemv_4096(args, dev):
 def mmq(args, dev):
     L = lib.load()
     wtype, m, k, n = {"2a": (Q4K, 512, 4096, 14336), "2b": (Q6K, 2048, 14336, 4096)}[args.shape]
+    if args.mmq_wtype:   # the same shape in another format of the tiled matmul's table
+        wtype = WTYPES[args.mmq_wtype]
+        if wtype not in ops.MMQ_LAUNCHER:
+            raise SystemExit(f"--mmq-wtype {args.mmq_wtype}: no dense tiled matmul for this format")
     mk = Maker(dev)
     w = mk.make(wtype, n, k)
     x = mk.randn(m, k)
@@ -300,8 +310,10 @@ def mmq(args, dev):
     # it because the target is quoted on the int8 peak.
     if wtype == Q4K:
         kernel, peak, dtype = "q4k_f16_dense_kernel", F16_PEAK_TFLOPS, "f16 operands (exact integers), f32 accumulate"
-    else:
+    elif wtype == Q6K:
         kernel, peak, dtype = "mmq_dense_kernel<MmqQ6K,128,1>", INT8_PEAK_TOPS, "int8"
+    else:
+        kernel, peak, dtype = f"mmq_dense_kernel<{NAMES[wtype]} tile policy,128,1>", INT8_PEAK_TOPS, "int8"
     roofline = {"bound": "mfma", "achieved": round(tops(kern), 1), "peak": peak, "unit": "TOP/s",
                 "frac": round(tops(kern) / peak, 4), "frac_of_int8_peak": round(tops(kern) / INT8_PEAK_TOPS, 4),
                 "traffic": None, "kernel": kernel, "avg_launch_us": round(float(mm.mean()), 3),
