@@ -906,14 +906,29 @@ static int launch_moe(const void* x, const void* x_second, int64_t dst_second, c
     const int64_t want = mmq_x > 0 ? mmq_x : (ncols_hint > 0 ? ncols_hint : ncols_max);
     if (want <= 32) return launch_moe_tm<F, 32, 1>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
     if (want <= 64) return launch_moe_tm<F, 64, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
-    if constexpr (F::F16_TILES) {
-        if (!getenv("LK_MMQ_I8")) {
-            const int tm = lk_mmq_q4k_f16_moe(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
-            if (tm >= 0) return tm;
+    // The 128-token tile of this kernel (the routing's bounds and destination map on top of the dense
+    // tile's registers) runs out of registers for the formats with a minimum or two scales per sub-block
+    // and loses to the 64-token tile: 128 experts of 2048 -> 768 -> 2048, top-8, gate + up and down,
+    // 2048 tokens: Q6_K 954 us against 1352, Q5_K 739 against 1231; 4096 tokens: 1608 against 1991, 1297
+    // against 1787 (Q8_0 and Q4_0 go either way by a tenth and keep the wide tile).
+    if constexpr (!F::F16_TILES && (F::HAS_MIN || F::NS == 16))
+        return launch_moe_tm<F, 64, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
+    else {
+        // Left to choose (no mmq_x), the narrower tile where it pads the expected longest run a fifth
+        // less: a run of 150 rows is three tiles of 64 or two of 128, the second nearly empty (2048
+        // tokens, as above: Q8_0 1198 us against 1300, Q4_0 742 against 983; at 1024 and 4096 tokens the
+        // runs fill the wide tiles and those win by a tenth).
+        if (!F::F16_TILES && mmq_x <= 0 && 5 * ((want + 63) / 64 * 64) <= 4 * ((want + 127) / 128 * 128))
+            return launch_moe_tm<F, 64, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
+        if constexpr (F::F16_TILES) {
+            if (!getenv("LK_MMQ_I8")) {
+                const int tm = lk_mmq_q4k_f16_moe(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
+                if (tm >= 0) return tm;
+            }
         }
+        constexpr int WAVES_M = 1;
+        return launch_moe_tm<F, 128, WAVES_M>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
     }
-    constexpr int WAVES_M = 1;
-    return launch_moe_tm<F, 128, WAVES_M>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
 }
 
 }  // namespace
