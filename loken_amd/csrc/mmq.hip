@@ -859,7 +859,10 @@ static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x
                   ncols_y, stride_col_dst, (int)nrows_x, 0, (int)ncols_y};
     hipStream_t s = (hipStream_t)stream;
     if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s);
-    if (ncols_y <= 64) return launch_dense_tm<F, 64, 2>(pb, s);
+    // (Q2_K stays on 64-token tiles: with the rank-16 minimum its 128-token tile spills and runs 512 x
+    // 4096 -> 14336 in 344 us against 240, 2048 x 14336 -> 4096 in 1155 against 742; every other format
+    // is 3 to 40 % faster on the wide tile)
+    if (ncols_y <= 64 || F::MIN_RANK == 16) return launch_dense_tm<F, 64, 2>(pb, s);
     if constexpr (F::F16_TILES) {   // Q4_K: scales folded into f16 operands
         if (!getenv("LK_MMQ_I8")) {
             const int tm = lk_mmq_q4k_f16_dense(pb, s);
