@@ -440,5 +440,19 @@ int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, in
     if (lk_tune_env("LK_TUNE_ROWS16_OFF") != 0) return -1;
     const Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd};
     if (size_m > 8 && lk_tune_env("LK_TUNE_ROWS16_MAX8") != 0) return -1;
-    return size_m <= 4 ? launch<4>(a, stream) : size_m <= 8 ? launch<8>(a, stream) : launch<16>(a, stream);
+    if (size_m <= 8) return size_m <= 4 ? launch<4>(a, stream) : launch<8>(a, stream);
+    const int rc = launch<16>(a, stream);
+    if (rc != -1) return rc;
+    // Rows too long for sixteen activation rows in LDS (k = 14336: 229 KB) but not for eight: two launches,
+    // the first eight rows and the rest (4096 x 14336 at 16 rows: 2 x 16.8 us against 37.4 us on the 32-row
+    // tiles that would take the call otherwise; at 12 rows 16.8 + 13.4 against 36.8).
+    Args lo = a, hi = a;
+    lo.m = 8;
+    hi.m = size_m - 8;
+    hi.y += (size_t)8 * stride_y * Q81_BYTES;
+    hi.dst += (size_t)8 * ldd;
+    const int rc_lo = launch<8>(lo, stream);
+    if (rc_lo != LK_OK) return rc_lo;   // -1: nothing ran, the caller takes the other kernel
+    const int rc_hi = hi.m <= 4 ? launch<4>(hi, stream) : launch<8>(hi, stream);
+    return rc_hi == -1 ? LK_ERR_LAUNCH : rc_hi;   // (needs less LDS than the first: does not happen)
 }
