@@ -97,6 +97,13 @@ static __host__ __device__ constexpr int lds_bytes_for(int nb, int waves) {
 template <int TOKS, int D>
 __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args p, int n_tiles, int tw) {
     constexpr bool T8 = TOKS == 8, T16 = TOKS == 16;
+    // grid.y: the activation rows in sets of TOKS, a set per workgroup (the weights are read once per set)
+    if (gridDim.y > 1) {
+        const int set = (int)blockIdx.y;
+        p.y += (size_t)set * TOKS * p.stride_y * Q81_BYTES;
+        p.dst += (size_t)set * TOKS * p.ldd;
+        p.m = min(TOKS, p.m - set * TOKS);
+    }
     constexpr int ZERO_BYTES = TOKS * 256;   // the zero lanes' run: the largest offset a step adds, and 16
     constexpr int BLK = TOKS * 32;       // LDS bytes of one Q8_1 block's codes, all rows
     extern __shared__ __align__(16) uint8_t lds[];
@@ -387,7 +394,7 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
 }
 
 template <int TOKS, int D>
-int launch_shape(const Args& a, int tw, hipStream_t stream) {
+int launch_shape(const Args& a, int tw, int sets, hipStream_t stream) {
     static std::mutex mu;
     static std::unordered_map<int, int> by_lds;
     const int waves = tw * (a.nb / GRAN);
@@ -410,49 +417,50 @@ int launch_shape(const Args& a, int tw, hipStream_t stream) {
     }
     const int n_tiles = (a.n + TILE - 1) / TILE, groups = (n_tiles + tw - 1) / tw;
     // every workgroup as equal a share of the tile groups as the count allows
-    int cap = lk_device().cus * (lds_bytes <= lk_device().lds_bytes / 2 && waves <= 8 ? 2 : 1);
+    int cap = lk_device().cus * (lds_bytes <= lk_device().lds_bytes / 2 && waves <= 8 ? 2 : 1) / sets;
     const int forced = lk_tune_env("LK_TUNE_ROWS16_WGS");
     if (forced > 0) cap = forced;
     const int passes = (groups + cap - 1) / cap;
     const int wgs = (groups + passes - 1) / passes;
-    hipLaunchKernelGGL((q6k_rows16_kernel<TOKS, D>), dim3(wgs), dim3(64 * waves), lds_bytes, stream, a, n_tiles, tw);
+    hipLaunchKernelGGL((q6k_rows16_kernel<TOKS, D>), dim3(wgs, sets), dim3(64 * waves), lds_bytes, stream, a, n_tiles, tw);
     return lk_launch_status();
 }
 
 template <int TOKS>
-int launch(const Args& a, hipStream_t stream) {
+int launch(const Args& a, hipStream_t stream, int sets = 1) {
     // Tiles per workgroup: as many as its sixteen waves and LDS hold while every CU still gets a workgroup.
     const int s = a.nb / GRAN, n_tiles = (a.n + TILE - 1) / TILE, cus = lk_device().cus;
     int tw = 1;
-    while (2 * tw * s <= MAX_WAVES && n_tiles >= 2 * tw * cus && lds_bytes_for<TOKS>(a.nb, 2 * tw * s) <= lk_device().lds_bytes) tw *= 2;
+    while (2 * tw * s <= MAX_WAVES && n_tiles * sets >= 2 * tw * cus && lds_bytes_for<TOKS>(a.nb, 2 * tw * s) <= lk_device().lds_bytes) tw *= 2;
     const int forced = lk_tune_env("LK_TUNE_ROWS16_TW");
     if (forced > 0 && forced * s <= MAX_WAVES) tw = forced;
-    return tw * s <= 8 ? launch_shape<TOKS, 4>(a, tw, stream) : launch_shape<TOKS, 2>(a, tw, stream);
+    return tw * s <= 8 ? launch_shape<TOKS, 4>(a, tw, sets, stream) : launch_shape<TOKS, 2>(a, tw, sets, stream);
 }
 
 }  // namespace
 
 int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y, int ldd,
                   hipStream_t stream) {
-    if (size_m < 1 || size_m > 16 || size_n < 1 || size_k < 256) return -1;
+    if (size_m < 1 || size_m > 32 || size_n < 1 || size_k < 256) return -1;
     // rows of whole granules, on 16-byte boundaries; a tile's granules within one workgroup
     if (size_k % (256 * GRAN) != 0 || size_k / (256 * GRAN) > MAX_WAVES || (((uintptr_t)w) & 15) != 0) return -1;
     if (lk_tune_env("LK_TUNE_ROWS16_OFF") != 0) return -1;
     const Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd};
     if (size_m > 8 && lk_tune_env("LK_TUNE_ROWS16_MAX8") != 0) return -1;
     if (size_m <= 8) return size_m <= 4 ? launch<4>(a, stream) : launch<8>(a, stream);
-    const int rc = launch<16>(a, stream);
-    if (rc != -1) return rc;
-    // Rows too long for sixteen activation rows in LDS (k = 14336: 229 KB) but not for eight: two launches,
-    // the first eight rows and the rest (4096 x 14336 at 16 rows: 2 x 16.8 us against 37.4 us on the 32-row
-    // tiles that would take the call otherwise; at 12 rows 16.8 + 13.4 against 36.8).
-    Args lo = a, hi = a;
-    lo.m = 8;
-    hi.m = size_m - 8;
-    hi.y += (size_t)8 * stride_y * Q81_BYTES;
-    hi.dst += (size_t)8 * ldd;
-    const int rc_lo = launch<8>(lo, stream);
-    if (rc_lo != LK_OK) return rc_lo;   // -1: nothing ran, the caller takes the other kernel
-    const int rc_hi = hi.m <= 4 ? launch<4>(hi, stream) : launch<8>(hi, stream);
-    return rc_hi == -1 ? LK_ERR_LAUNCH : rc_hi;   // (needs less LDS than the first: does not happen)
+    // 9..32 rows. Sixteen at once when their codes fit LDS and the row tiles fill the chip; else the rows
+    // in sets of eight, a set per workgroup (grid.y), in one launch: rows too long for sixteen in LDS (k =
+    // 14336: 229 KB; 4096 x 14336 at 16 rows 25.7 us against 37.4 on the 32-row tiles that would take the
+    // call otherwise), so few tiles that a workgroup per tile leaves half the CUs idle (2048 x 6144 at 16
+    // rows: 11.1 us against 15.9), or 17..32 rows (2048 x 6144 at 32 rows 13.5 us against 22.4 on the 32-row
+    // tiles, 4096 x 4096 13.8 against 17.4, 4096 x 14336 42.7 against 47.4). Every set reads the weights
+    // again, from L2 while they fit there: above 16 rows a matrix of more than 64 MB stays with the 32-row
+    // tiles (151936 x 2048 at 32 rows: 173 us against 99).
+    const int n_tiles = (size_n + TILE - 1) / TILE;
+    if (size_m > 16 && (size_t)size_n * a.nb * Q6K_BYTES > ((size_t)64 << 20)) return -1;
+    if (size_m <= 16 && 2 * n_tiles > lk_device().cus) {
+        const int rc = launch<16>(a, stream);
+        if (rc != -1) return rc;
+    }
+    return launch<8>(a, stream, (size_m + 7) / 8);
 }

@@ -301,11 +301,13 @@ def test_gate_and_up_as_q8_1_refuses_what_its_kernel_does_not_take():
 @pytest.mark.parametrize("m,k,n", [(1, 256, 1), (2, 512, 15), (3, 768, 17), (4, 1024, 33), (4, 14336, 48), (5, 256, 16), (7, 1280, 100),
                                    (8, 6144, 500), (6, 2048, 8300), (3, 512, 8300), (8, 512, 16500), (4, 256, 16500),
                                    (9, 2048, 17), (12, 6144, 500), (16, 4096, 100), (16, 2048, 8300), (13, 2048, 16500),
-                                   (9, 14336, 48), (12, 14336, 100), (16, 14336, 33)])
+                                   (9, 14336, 48), (12, 14336, 100), (16, 14336, 33),
+                                   (17, 2048, 100), (24, 6144, 500), (32, 4096, 33), (31, 14336, 48), (25, 2048, 8300)])
 def test_q6k_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n):
     """rows16_q6k.hip: both slot layouts (up to four rows, up to eight), ragged tile edges, rows of
     one super-block (waves with nothing to add), one, two and four tiles per workgroup; k = 14336 above
-    eight rows: sixteen rows do not fit LDS and the call goes out as two launches."""
+    eight rows: sixteen rows do not fit LDS and the rows go out as sets of eight over the launch's second grid
+    axis, as do 17..32 rows of a matrix that L2 holds."""
     w = synth.weight(Q6K, n, k, seed=74, stream=1)
     x = synth.activation(m, k, seed=74)
     got = ops.dense_q6k_rows(dev(w), dev(x), n).cpu().numpy()
@@ -313,7 +315,7 @@ def test_q6k_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n):
 
 
 @pytest.mark.parametrize("k", [1024, 4096])
-@pytest.mark.parametrize("m", [3, 4, 7, 11, 16])
+@pytest.mark.parametrize("m", [3, 4, 7, 11, 16, 21, 32])
 def test_q6k_few_rows_emit_the_exact_integers_on_crafted_inputs(m, k):
     """As test_q6k_rows_emit_the_exact_integers_on_crafted_inputs, for the launches of at most four
     and at most eight rows: one group of each super-block has scale 1, the others 0, so a code that
