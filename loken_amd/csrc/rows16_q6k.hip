@@ -447,7 +447,11 @@ int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, in
     if (lk_tune_env("LK_TUNE_ROWS16_OFF") != 0) return -1;
     const Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd};
     if (size_m > 8 && lk_tune_env("LK_TUNE_ROWS16_MAX8") != 0) return -1;
-    if (size_m <= 8) return size_m <= 4 ? launch<4>(a, stream) : launch<8>(a, stream);
+    if (size_m <= 4) return launch<4>(a, stream);
+    const int n_tiles = (size_n + TILE - 1) / TILE;
+    // 5..8 rows over so few tiles that a workgroup per tile leaves half the CUs idle: two sets of four rows
+    // (2048 x 6144: 8.9 us against 10.7 as eight at once; sets: below)
+    if (size_m <= 8) return 2 * n_tiles <= lk_device().cus ? launch<4>(a, stream, 2) : launch<8>(a, stream);
     // 9..32 rows. Sixteen at once when their codes fit LDS and the row tiles fill the chip; else the rows
     // in sets of eight, a set per workgroup (grid.y), in one launch: rows too long for sixteen in LDS (k =
     // 14336: 229 KB; 4096 x 14336 at 16 rows 25.7 us against 37.4 on the 32-row tiles that would take the
@@ -456,7 +460,6 @@ int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, in
     // tiles, 4096 x 4096 13.8 against 17.4, 4096 x 14336 42.7 against 47.4). Every set reads the weights
     // again, from L2 while they fit there: above 16 rows a matrix of more than 64 MB stays with the 32-row
     // tiles (151936 x 2048 at 32 rows: 173 us against 99).
-    const int n_tiles = (size_n + TILE - 1) / TILE;
     if (size_m > 16 && (size_t)size_n * a.nb * Q6K_BYTES > ((size_t)64 << 20)) return -1;
     if (size_m <= 16 && 2 * n_tiles > lk_device().cus) {
         const int rc = launch<16>(a, stream);

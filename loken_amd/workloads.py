@@ -465,7 +465,13 @@ def decode_1p7b(args, dev):
         if g == "h":   # `down` reads the Q8_1 rows the gate + up launch wrote
             out = torch.empty((b, ns[0]), device=dev)
             keep.append(out)
-            plan.append(("status", L.lk_dense_q6k_rows, (weights[0].data_ptr(), rows_h_q81.data_ptr(), out.data_ptr(), b, ns[0], k, s)))
+            if b <= 6 and ns[0] * k < (48 << 20):   # a small matrix at few rows: the mat-vec (host_qmatmul.hip's rule)
+                plan.append(("status", L.lk_mmvq, (wtype, weights[0].data_ptr(), rows_h_q81.data_ptr(), out.data_ptr(), lib.TYPE_F32,
+                                                   k, ns[0], b, k // 32, ns[0], None, 0, s)))
+                used["rows"] -= 1
+                used["matvec"] += 1
+            else:
+                plan.append(("status", L.lk_dense_q6k_rows, (weights[0].data_ptr(), rows_h_q81.data_ptr(), out.data_ptr(), b, ns[0], k, s)))
             return
         q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
         keep.append(q)
