@@ -98,12 +98,10 @@ template <int TOKS, int D>
 __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args p, int n_tiles, int tw) {
     constexpr bool T8 = TOKS == 8, T16 = TOKS == 16;
     // grid.y: the activation rows in sets of TOKS, a set per workgroup (the weights are read once per set)
-    if (gridDim.y > 1) {
-        const int set = (int)blockIdx.y;
-        p.y += (size_t)set * TOKS * p.stride_y * Q81_BYTES;
-        p.dst += (size_t)set * TOKS * p.ldd;
-        p.m = min(TOKS, p.m - set * TOKS);
-    }
+    const int set = (int)blockIdx.y;
+    const uint8_t* const act_rows = p.y + (size_t)set * TOKS * p.stride_y * Q81_BYTES;
+    float* const out_rows = p.dst + (size_t)set * TOKS * p.ldd;
+    const int m_rows = min(TOKS, p.m - set * TOKS);
     constexpr int ZERO_BYTES = TOKS * 256;   // the zero lanes' run: the largest offset a step adds, and 16
     constexpr int BLK = TOKS * 32;       // LDS bytes of one Q8_1 block's codes, all rows
     extern __shared__ __align__(16) uint8_t lds[];
@@ -133,8 +131,8 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
 #pragma unroll
         for (int u = 0; u < PER; ++u) {
             const int idx = min(base + u * WG, entries - 1);
-            const int sub = idx / TOKS, tok = min(idx % TOKS, p.m - 1);
-            const uint8_t* b = p.y + ((size_t)tok * p.stride_y + sub) * Q81_BYTES;
+            const int sub = idx / TOKS, tok = min(idx % TOKS, m_rows - 1);
+            const uint8_t* b = act_rows + ((size_t)tok * p.stride_y + sub) * Q81_BYTES;
             head[u] = *(const uint32_t*)b;
             lo[u] = *(const uint4_a4*)(b + 4);
             hi[u] = *(const uint4_a4*)(b + 20);
@@ -145,7 +143,7 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
         for (int u = 0; u < PER; ++u) {
             const int idx = base + u * WG;
             if (idx < entries) {
-                const bool real = idx % TOKS < p.m;
+                const bool real = idx % TOKS < m_rows;
                 table[idx] = real ? f16_bits_to_f32(head[u] & 0xFFFFu) : 0.f;
                 const uint32_t keep = real ? 0xFFFFFFFFu : 0u;   // rows the launch does not have: zeros
                 *(uint4*)(codes + (size_t)idx * 32) = make_uint4(lo[u].x & keep, lo[u].y & keep, lo[u].z & keep, lo[u].w & keep);
@@ -346,7 +344,7 @@ __global__ __launch_bounds__(D == 4 ? 512 : 1024, 1) void q6k_rows16_kernel(Args
             }
             const int tile = ((int)blockIdx.x + pass * stride) * tw + ts;
             const int tok = T16 ? 4 * (l >> 4) + v : T8 ? 4 * ((l >> 4) & 1) + v : v, row = tile * TILE + (l & 15);
-            if (tile < n_tiles && tok < p.m && row < p.n) p.dst[(size_t)tok * p.ldd + row] = sum;
+            if (tile < n_tiles && tok < m_rows && row < p.n) out_rows[(size_t)tok * p.ldd + row] = sum;
         }
         __syncthreads();   // the buffers may be overwritten
     };
