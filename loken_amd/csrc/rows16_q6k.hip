@@ -457,10 +457,12 @@ int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, in
     // finish sooner (16 rows: 2048 x 6144 11.1 us against 15.9, 4096 x 4096 10.8 against 14.7, 8192 x 2048
     // 10.4 against 13.2, 8192 x 4096 14.5 against 15.7; 11008 x 4096 28.2 against 23.8 and 14336 x 4096 27.2
     // against 25.7 stay with sixteen at once), or 17..32 rows (2048 x 6144 at 32 rows 13.5 us against 22.4 on the 32-row
-    // tiles, 4096 x 4096 13.8 against 17.4, 4096 x 14336 42.7 against 47.4). Every set reads the weights
-    // again, from L2 while they fit there: above 16 rows a matrix of more than 64 MB stays with the 32-row
-    // tiles (151936 x 2048 at 32 rows: 173 us against 99).
-    if (size_m > 16 && (size_t)size_n * a.nb * Q6K_BYTES > ((size_t)64 << 20)) return -1;
+    // tiles, 4096 x 4096 13.8 against 17.4, 4096 x 14336 42.7 against 47.4, 4096 x 8192 24.8 against 31.1).
+    // Every set reads the weights again, from L2 while they fit there, and three or four sets of more than a
+    // tile to the CU are too many workgroups: above 16 rows a matrix of more than 64 MB or of more tiles
+    // than CUs stays with the 32-row tiles (at 32 rows 151936 x 2048 173 us against 99, 6144 x 4096 25.8
+    // against 18.4, 14336 x 4096 39.7 against 32.4).
+    if (size_m > 16 && (n_tiles > lk_device().cus || (size_t)size_n * a.nb * Q6K_BYTES > ((size_t)64 << 20))) return -1;
     if (size_m <= 16 && n_tiles > 2 * lk_device().cus) {
         const int rc = launch<16>(a, stream);
         if (rc != -1) return rc;
