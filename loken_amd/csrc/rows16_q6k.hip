@@ -447,9 +447,14 @@ int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, in
     if (size_m > 8 && lk_tune_env("LK_TUNE_ROWS16_MAX8") != 0) return -1;
     if (size_m <= 4) return launch<4>(a, stream);
     const int n_tiles = (size_n + TILE - 1) / TILE;
-    // 5..8 rows over so few tiles that a workgroup per tile leaves half the CUs idle: two sets of four rows
-    // (2048 x 6144: 8.9 us against 10.7 as eight at once; sets: below)
-    if (size_m <= 8) return 2 * n_tiles <= lk_device().cus ? launch<4>(a, stream, 2) : launch<8>(a, stream);
+    // 5..8 rows as two sets of four where that fills the chip sooner than eight at once: so few tiles that a
+    // workgroup per tile leaves half the CUs idle (2048 x 6144: 8.9 us against 10.7; 2048 x 14336 12.9 against
+    // 16.3), or a matrix small enough for its second reading to come from L2 at no cost (4096 x 4096 9.1 us
+    // against 10.3, 8192 x 2048 8.8 against 9.5, 6144 x 4096 11.7 against 12.7; 8192 x 4096, 27.5 MB, 12.2
+    // against 11.1 and stays with eight). (Sets: below.)
+    const size_t weight_bytes = (size_t)size_n * a.nb * Q6K_BYTES;
+    if (size_m <= 8)
+        return 2 * n_tiles <= lk_device().cus || weight_bytes <= ((size_t)22 << 20) ? launch<4>(a, stream, 2) : launch<8>(a, stream);
     // 9..32 rows. Sixteen at once when their codes fit LDS and the row tiles are several to the CU; else the
     // rows in sets of eight, a set per workgroup (grid.y), in one launch: rows too long for sixteen in LDS (k =
     // 14336: 229 KB; 4096 x 14336 at 16 rows 25.7 us against 37.4 on the 32-row tiles that would take the
@@ -462,7 +467,7 @@ int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, in
     // tile to the CU are too many workgroups: above 16 rows a matrix of more than 64 MB or of more tiles
     // than CUs stays with the 32-row tiles (at 32 rows 151936 x 2048 173 us against 99, 6144 x 4096 25.8
     // against 18.4, 14336 x 4096 39.7 against 32.4).
-    if (size_m > 16 && (n_tiles > lk_device().cus || (size_t)size_n * a.nb * Q6K_BYTES > ((size_t)64 << 20))) return -1;
+    if (size_m > 16 && (n_tiles > lk_device().cus || weight_bytes > ((size_t)64 << 20))) return -1;
     if (size_m <= 16 && n_tiles > 2 * lk_device().cus) {
         const int rc = launch<16>(a, stream);
         if (rc != -1) return rc;
