@@ -33,8 +33,9 @@ struct LkRows16Experts {
 int lk_rows16_launch_experts(const LkRows16& a, const LkRows16Experts& m, int n_experts, bool dual, int rows_hint,
                              hipStream_t stream);
 
-// Q6_K x at most 32 Q8_1 rows in 16-row tiles (rows16_q6k.hip; above eight rows possibly as sets of eight rows
+// Q6_K x at most 64 Q8_1 rows in 16-row tiles (rows16_q6k.hip; above eight rows possibly as sets of eight rows
 // over the same weights). LK_* status, or -1 when the launch does not serve the call (more rows, k not a
-// multiple of 2048, rows whose codes do not fit in LDS, above 16 rows a matrix of more than 64 MB or of more 16-row tiles than CUs).
+// multiple of 2048, rows whose codes do not fit in LDS, above 16 rows a matrix of more than 64 MB or of more 16-row tiles than CUs, above 32 rows
+// anything but whole rounds of resident workgroups).
 int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y, int ldd,
                   hipStream_t stream);

@@ -439,7 +439,7 @@ int launch(const Args& a, hipStream_t stream, int sets = 1) {
 
 int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, int size_n, int size_k, int stride_y, int ldd,
                   hipStream_t stream) {
-    if (size_m < 1 || size_m > 32 || size_n < 1 || size_k < 256) return -1;
+    if (size_m < 1 || size_m > 64 || size_n < 1 || size_k < 256) return -1;
     // rows of whole granules, on 16-byte boundaries; a tile's granules within one workgroup
     if (size_k % (256 * GRAN) != 0 || size_k / (256 * GRAN) > MAX_WAVES || (((uintptr_t)w) & 15) != 0) return -1;
     if (lk_tune_env("LK_TUNE_ROWS16_OFF") != 0) return -1;
@@ -468,6 +468,15 @@ int lk_rows16_q6k(const void* w, const void* q8_1, float* output, int size_m, in
     // than CUs stays with the 32-row tiles (at 32 rows 151936 x 2048 173 us against 99, 6144 x 4096 25.8
     // against 18.4, 14336 x 4096 39.7 against 32.4).
     if (size_m > 16 && (n_tiles > lk_device().cus || weight_bytes > ((size_t)64 << 20))) return -1;
+    // 33..64 rows: only as whole rounds of workgroups that are all resident at two to the CU, one round or
+    // exactly two (2048 x 6144 at 64 rows, 128 tiles x 8 sets: 18.7 us against 22.3 on the 32-row tiles; at
+    // 40..56 rows, a second round partly filled, 24 against 22.2; 1024 x 2048, 64 tiles, 9.5 against 12.0 at 64
+    // rows and 10.3 against 11.8 at 40)
+    if (size_m > 32) {
+        const int total = n_tiles * ((size_m + 7) / 8), cus = lk_device().cus;
+        const bool two_per_cu = lds_bytes_for<8>(a.nb, a.nb / GRAN) <= lk_device().lds_bytes / 2 && a.nb / GRAN <= 8;
+        if (!two_per_cu || (total > 2 * cus && total != 4 * cus)) return -1;
+    }
     if (size_m <= 16 && n_tiles > 2 * lk_device().cus) {
         const int rc = launch<16>(a, stream);
         if (rc != -1) return rc;

@@ -390,9 +390,9 @@ int lk_q6k_rows_mfma(const void* w, const void* q8_1, float* output, int size_m,
     if ((((uintptr_t)w) & 1) != 0 || (((uintptr_t)q8_1) & 3) != 0) return LK_ERR_ARG;
     Args a{(const uint8_t*)w, (const uint8_t*)q8_1, output, size_k / 256, size_n, size_m, stride_y, ldd};
     int rc = -1;
-    if (size_m <= 32) {
+    if (size_m <= 64) {
         // 16-row tiles (rows16_q6k.hip): a quarter of the matrix-unit time per weight, and every CU a tile
-        // (above 16 rows: sets of eight rows, for a matrix that L2 holds)
+        // (above 16 rows: sets of eight rows, for a small matrix that L2 holds; the launcher declines the rest)
         rc = lk_rows16_q6k(w, q8_1, output, size_m, size_n, size_k, stride_y, ldd, stream);
         if (rc >= 0) return rc;
     }

@@ -302,7 +302,8 @@ def test_gate_and_up_as_q8_1_refuses_what_its_kernel_does_not_take():
                                    (8, 6144, 500), (6, 2048, 8300), (3, 512, 8300), (8, 512, 16500), (4, 256, 16500),
                                    (9, 2048, 17), (12, 6144, 500), (16, 4096, 100), (16, 2048, 8300), (13, 2048, 16500),
                                    (9, 14336, 48), (12, 14336, 100), (16, 14336, 33),
-                                   (17, 2048, 100), (24, 6144, 500), (32, 4096, 33), (31, 14336, 48), (25, 2048, 8300)])
+                                   (17, 2048, 100), (24, 6144, 500), (32, 4096, 33), (31, 14336, 48), (25, 2048, 8300),
+                                   (64, 6144, 2048), (57, 2048, 1000), (40, 2048, 1024)])
 def test_q6k_eight_rows_or_fewer_in_sixteen_row_tiles(m, k, n):
     """rows16_q6k.hip: both slot layouts (up to four rows, up to eight), ragged tile edges, rows of
     one super-block (waves with nothing to add), one, two and four tiles per workgroup; k = 14336 above
