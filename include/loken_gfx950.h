@@ -654,24 +654,11 @@ void loken_argsort_small_u32(const uint32_t* in, uint32_t* sorted_out, uint32_t*
 /* Frees the current device's MoE decode scratch (cuda/moe/moe_gguf.cu:104-118). Synchronizes. */
 void loken_stream_scratch_release(void);
 
-/* ---------------------------------------------------------------------------------------
- * Measurement aids. No counterpart in the reference and nothing on the product path calls them:
- * they give the measured denominators reported beside the nominal MI355X peaks.
- * ------------------------------------------------------------------------------------- */
-
-/* `workgroups` workgroups of 256 threads that end at once: the floor of one launch. */
-int lk_probe_empty(int workgroups, void* stream);
-/* Reads `bytes` (a multiple of 16, 16-byte aligned) from `src` and writes nothing. pattern 1, 2,
- * 4, 8: grid-strided, that many 16-byte loads per thread in flight; 0: every workgroup walks its
- * own contiguous share. `sink` is 4 bytes of device memory (never written in practice). */
-int lk_probe_read(const void* src, int64_t bytes, int workgroups, int pattern, void* sink, void* stream);
-/* Register-resident matrix-unit loop: each of a workgroup's four matrix waves issues `iters` x 4
- * independent instructions of `kind` (0 v_mfma_i32_32x32x32_i8, 1 v_mfma_f32_32x32x16_f16,
- * 2 v_mfma_i32_16x16x64_i8, 3 v_mfma_i32_32x32x16_i8). valu_per_mfma (a multiple of 8) independent f32 fmas ride along per
- * matrix instruction: in the same wave (mode 0), or in four further waves, one beside each matrix
- * wave on its SIMD (mode 1). *ops (nullable, host memory) receives the matrix operations launched. */
-int lk_probe_mfma(int kind, int workgroups, int iters, int valu_per_mfma, int mode, void* sink, double* ops,
-                  void* stream);
+/* Makes every LK_TUNE_* / LK_MMQ_* environment override (launch shapes and path choices of
+ * measurement runs and A/B tests; none changes what a result means) be read again. The launchers
+ * read each once and keep it; a process that changes its environment while it runs calls this.
+ * No counterpart in the reference. */
+void lk_tune_refresh(void);
 
 #ifdef __cplusplus
 }

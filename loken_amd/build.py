@@ -10,6 +10,9 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIB = HERE / "libloken_gfx950.so"
+# measurement kernels: a library of their own that only the benchmark loads
+PROBES_SRC = HERE / "probes_csrc" / "probes.hip"
+PROBES_LIB = HERE / "libloken_probes.so"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -21,7 +24,7 @@ FLAGS = [
 # MFMA results are consumed by VALU fix-ups right away: keep them in VGPRs instead of the
 # accumulator file, which would cost one v_accvgpr_read per value.
 _VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form"]
-PER_FILE_FLAGS = {"mmq.hip": _VGPR_FORM, "mmq_q4k_f16.hip": _VGPR_FORM}
+PER_FILE_FLAGS = {"mmq.hip": _VGPR_FORM, "mmq_q4k_f16.hip": _VGPR_FORM, "mmq_q4k_wide.hip": _VGPR_FORM}
 
 
 def sources() -> list[Path]:
@@ -56,8 +59,18 @@ def build(jobs: int = 8, verbose: bool = False, incremental: bool = False) -> Pa
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr[-6000:]}")
+    probes_obj = PROBES_SRC.with_suffix(".o")
+    if not (incremental and _fresh(PROBES_SRC, probes_obj)):
+        r = subprocess.run([HIPCC, *FLAGS, "-c", str(PROBES_SRC), "-o", str(probes_obj)], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {PROBES_SRC.name}:\n{r.stderr[-6000:]}")
+    # lk_launch_status and the knob reader live in the product's objects: the probes link the one they use
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(PROBES_LIB), str(probes_obj),
+                        str(CSRC / "device.o")], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr[-6000:]}")
     if verbose:
-        print(f"built {LIB} from {len(srcs)} sources")
+        print(f"built {LIB} from {len(srcs)} sources and {PROBES_LIB.name}")
     return LIB
 
 

@@ -1,6 +1,8 @@
 // Device facts the launchers size their grids and LDS budgets by.
 #include "lk_common.h"
 
+#include <atomic>
+#include <cstdlib>
 #include <mutex>
 
 const LkDevice& lk_device() {
@@ -29,3 +31,20 @@ extern "C" int lk_device_info(int* abi_version, int* compute_units, int* lds_byt
     if (wave_size) *wave_size = LK_WAVE;
     return LK_OK;
 }
+
+// ---------------------------------------------------------------- environment knobs
+namespace {
+std::atomic<unsigned> g_tune_epoch{1};
+}
+
+unsigned lk_tune_epoch() { return g_tune_epoch.load(std::memory_order_relaxed); }
+
+int lk_tune_read(LkTuneSite& site) {
+    const unsigned now = g_tune_epoch.load(std::memory_order_acquire);
+    const char* v = getenv(site.name);
+    site.value = v ? atoi(v) : 0;
+    site.epoch = now;   // two threads racing here write the same pair
+    return site.value;
+}
+
+extern "C" void lk_tune_refresh(void) { g_tune_epoch.fetch_add(1, std::memory_order_acq_rel); }

@@ -333,12 +333,25 @@ int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_
                        int k32_stride, const LkGateAct& act, int slab_rows, const unsigned int* live,
                        const LkMoeAlt& alt, hipStream_t s);
 
-// Measurement runs: an integer from the environment (0 when unset). Every LK_TUNE_* variable only
-// overrides a launch-shape choice; none changes a result.
-static inline int lk_tune_env(const char* name) {
-    const char* v = getenv(name);
-    return v ? atoi(v) : 0;
-}
+// Measurement runs and A/B tests: an integer from the environment (0 when unset). Every LK_TUNE_* /
+// LK_MMQ_* variable only overrides a launch-shape or path choice; none changes what a result means.
+// A call site reads the environment once and keeps the value: the launch path pays one relaxed load
+// and a compare. lk_tune_refresh() (device.hip) makes every site read again, for a process that
+// changes its environment while it runs.
+struct LkTuneSite {
+    const char* name;
+    unsigned epoch;   // the refresh count this value was read at (0: never)
+    int value;
+};
+unsigned lk_tune_epoch();
+int lk_tune_read(LkTuneSite& site);
+#define lk_tune_env(NAME)                                                        \
+    ([]() -> int {                                                               \
+        static LkTuneSite site{NAME, 0u, 0};                                     \
+        return site.epoch == lk_tune_epoch() ? site.value : lk_tune_read(site);  \
+    }())
+static inline bool lk_env_flag_site(int v) { return v != 0; }
+#define lk_env_flag(NAME) lk_env_flag_site(lk_tune_env(NAME))
 
 static inline int lk_launch_status() {
     return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;

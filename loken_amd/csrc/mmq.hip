@@ -864,7 +864,14 @@ static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x
     // is 3 to 40 % faster on the wide tile)
     if (ncols_y <= 64 || F::MIN_RANK == 16) return launch_dense_tm<F, 64, 2>(pb, s);
     if constexpr (F::F16_TILES) {   // Q4_K: scales folded into f16 operands
-        if (!getenv("LK_MMQ_I8")) {
+        if (!lk_env_flag("LK_MMQ_I8")) {
+            // 128-token tiles with the token side expanded once per call, where they pad the rows at most a
+            // tenth more than the 64-token tiles would (512 x 4096 -> 14336: 105 us against 123)
+            const int64_t pad128 = (ncols_y + 127) / 128 * 128, pad64 = (ncols_y + 63) / 64 * 64;
+            if (ncols_y > 128 && 10 * pad128 <= 11 * pad64 && !lk_env_flag("LK_MMQ_NO_WIDE")) {
+                const int tm = lk_mmq_q4k_wide_dense(pb, s);
+                if (tm >= 0) return tm;
+            }
             const int tm = lk_mmq_q4k_f16_dense(pb, s);
             if (tm >= 0) return tm;
         }
@@ -924,7 +931,7 @@ static int launch_moe(const void* x, const void* x_second, int64_t dst_second, c
         if (!F::F16_TILES && mmq_x <= 0 && 5 * ((want + 63) / 64 * 64) <= 4 * ((want + 127) / 128 * 128))
             return launch_moe_tm<F, 64, 2>(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
         if constexpr (F::F16_TILES) {
-            if (!getenv("LK_MMQ_I8")) {
+            if (!lk_env_flag("LK_MMQ_I8")) {
                 const int tm = lk_mmq_q4k_f16_moe(pb, w2, dst_second, expert_bounds, stride_expert_x, n_experts, ncols_max, s);
                 if (tm >= 0) return tm;
             }

@@ -42,5 +42,8 @@ static int mmq_prepare_kernel(K kernel, int lds_bytes) {
 // 0 when the launch failed, -1 when the operands do not suit these kernels (16-byte alignment,
 // 32-bit record offsets) and the caller should take the int8 tiles.
 int lk_mmq_q4k_f16_dense(const MmqProblem& pb, hipStream_t s);
+// Q4_K against 129 or more token rows on the f16 tiles with four token tiles per wave (mmq_q4k_wide.hip); same returns.
+int lk_mmq_q4k_wide_dense(const MmqProblem& pb, hipStream_t s);
+void lk_mmq_q4k_wide_release(int device);
 int lk_mmq_q4k_f16_moe(const MmqProblem& pb, const uint8_t* w_second, int64_t dst_second, const int32_t* bounds,
                        int64_t stride_expert, int n_experts, int64_t ncols_max, hipStream_t s);

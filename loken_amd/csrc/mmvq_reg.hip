@@ -464,7 +464,7 @@ struct Shape {
     int waves, cap;   // waves per workgroup, most workgroups launched
 };
 static Shape shape_for(bool act_f32) {
-    static const int forced_waves = lk_tune_env("LK_TUNE_REG_WAVES"), forced_per_cu = lk_tune_env("LK_TUNE_REG_WGS_PER_CU");
+    const int forced_waves = lk_tune_env("LK_TUNE_REG_WAVES"), forced_per_cu = lk_tune_env("LK_TUNE_REG_WGS_PER_CU");
     const int waves = act_f32 ? RW : (forced_waves == 4 || forced_waves == 8 ? forced_waves : 4);
     const int per_cu = forced_per_cu > 0 ? forced_per_cu : 16 / waves;
     return Shape{waves, lk_device().cus * per_cu};
@@ -487,7 +487,7 @@ static int launch_multi(const LkRegMulti& m, const void* act, int act_f32, int n
     }
     const Shape sh = shape_for(act_f32 != 0);
     const int need = (total + sh.waves - 1) / sh.waves;
-    static const int forced_grid = lk_tune_env("LK_TUNE_REG_GRID");
+    const int forced_grid = lk_tune_env("LK_TUNE_REG_GRID");
     const dim3 grid(forced_grid > 0 ? (forced_grid < need ? forced_grid : need) : need < sh.cap ? need : sh.cap), block(sh.waves * 64);
     if (act_f32)
         hipLaunchKernelGGL((q4k_reg_kernel<R, RP, true, B>), grid, block, 0, s, a, (const uint8_t*)act, nb, dst_type, sh.waves,
@@ -530,7 +530,7 @@ static int launch_pair(const uint8_t* gate, const uint8_t* up, const void* act, 
 }  // namespace
 
 bool lk_q4k_reg_serves(int nb) {
-    static const int off = lk_tune_env("LK_TUNE_NO_REG");   // measurement runs: the staged engine for everything
+    const int off = lk_tune_env("LK_TUNE_NO_REG");   // measurement runs: the staged engine for everything
     return nb >= 1 && nb <= MAX_NB && !off;
 }
 
@@ -542,7 +542,7 @@ static int multi_rows(const LkRegMulti& m, const void* act, int act_f32, int nb,
     // of loads and a tail: fewer, fatter waves), one row per tile when waves stream several.
     int rows = 0;
     for (int i = 0; i < m.count; ++i) rows += m.n[i];
-    static const int forced = lk_tune_env("LK_TUNE_REG_R");
+    const int forced = lk_tune_env("LK_TUNE_REG_R");
     const Shape sh = shape_for(act_f32 != 0);
     // (from f32 rows the bound is one workgroup per CU: q + k + v of a Llama-sized layer, 6144 rows, is
     // faster as single rows over two workgroups per CU, 5.7 against 6.1 us; o, 4096 rows, as pairs)
@@ -570,7 +570,7 @@ int lk_q4k_reg_multi(const LkRegMulti& m, const void* act, int act_f32, int nb, 
 template <int RP>
 static int launch_moe_pair(const uint8_t* gate, const uint8_t* up, const float* acts, float* out, int nb, int n,
                            const RegMoeArgs& m, hipStream_t s) {
-    static const int forced_per_cu = lk_tune_env("LK_TUNE_REG_MOE_PER_CU");
+    const int forced_per_cu = lk_tune_env("LK_TUNE_REG_MOE_PER_CU");
     const int tiles = (n + RP - 1) / RP, need = (tiles + RW - 1) / RW;
     int share = lk_device().cus * (forced_per_cu > 0 ? forced_per_cu : 4) / m.pairs;
     if (share < 1) share = 1;
@@ -582,7 +582,7 @@ static int launch_moe_pair(const uint8_t* gate, const uint8_t* up, const float* 
 int lk_q4k_reg_moe_pair(const uint8_t* gate, const uint8_t* up, const float* acts, const int32_t* sorted_token_ids,
                         const int32_t* expert_ids, float* out, int experts, int topk, int pairs, int n, int nb,
                         int64_t slab_bytes, const LkGateAct& act, hipStream_t stream) {
-    static const int off = lk_tune_env("LK_TUNE_NO_REG_MOE");
+    const int off = lk_tune_env("LK_TUNE_NO_REG_MOE");
     if (off || !lk_q4k_reg_serves(nb) || pairs < 1 || pairs > 65535 || n < 1) return -1;
     if ((((uintptr_t)gate) | ((uintptr_t)up) | ((uintptr_t)acts)) & 15) return -1;
     const RegMoeArgs m{sorted_token_ids, expert_ids, experts, topk, pairs, slab_bytes, act};

@@ -281,9 +281,13 @@ static inline bool rows_stage_as_f32(const float* inputs, int size_k, int quant_
 
 }  // namespace
 
+void lk_mmq_q4k_wide_release(int device);   // mmq_q4k_wide.hip: the token-side operand buffers of the wide Q4_K tiles
+
 extern "C" void loken_stream_scratch_release() {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return;
+    (void)hipDeviceSynchronize();   // queued kernels may still read what is freed below
+    lk_mmq_q4k_wide_release(dev);
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     for (auto it = g_scratch.begin(); it != g_scratch.end();) {
         if (it->device != dev) { ++it; continue; }

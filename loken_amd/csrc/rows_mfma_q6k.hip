@@ -368,7 +368,7 @@ int launch(const Args& a, hipStream_t stream) {
     // 2048 x 6144 41.8 / 42.6 -> 36.5 / 37.6 us, 4096 x 4096 34.6 / 35.8 -> 31.9 / 33.4; rows of eight
     // super-blocks lose, 25.8 -> 27.4)
     const int n_tiles = (a.n + 31) / 32, groups = STAGED ? 1 : (a.m + TOK - 1) / TOK;
-    static const int forced = lk_tune_env("LK_TUNE_ROWS_WAVES");
+    const int forced = lk_tune_env("LK_TUNE_ROWS_WAVES");
     const bool eight = forced ? forced == 8 : (n_tiles * groups <= lk_device().cus && a.nb >= 16);
     if (eight) {
         const int rc = launch_waves<G, STAGED, 8>(a, stream);

@@ -142,9 +142,7 @@ SIGNATURES.update({
     "loken_moe_q4k_imma_m8_gate_up": (None, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "lk_moe_q4k_rows_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "loken_moe_q4k_imma_m8_down": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "lk_probe_empty": (_i, [_i, _vp]),
-    "lk_probe_read": (_i, [_vp, _i64, _i, _i, _vp, _vp]),
-    "lk_probe_mfma": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "lk_tune_refresh": (None, []),
     "loken_moe_mmq_fold": (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
 })
 

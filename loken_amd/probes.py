@@ -10,11 +10,33 @@ from __future__ import annotations
 
 import ctypes as C
 import json
+from pathlib import Path
 
 import numpy as np
 import torch
 
 from . import lib
+
+PROBES_PATH = Path(__file__).resolve().parent / "libloken_probes.so"
+_probes = None
+
+
+def load() -> C.CDLL:
+    """The measurement library (include/loken_probes.h): a library of its own, not the product's."""
+    global _probes
+    if _probes is None:
+        if not PROBES_PATH.exists():
+            raise ImportError(f"{PROBES_PATH} is missing: build it with `python -m loken_amd.build`")
+        L = C.CDLL(str(PROBES_PATH))
+        vp, i, i64 = C.c_void_p, C.c_int, C.c_int64
+        for name, args in {"lk_probe_empty": [i, vp], "lk_probe_read": [vp, i64, i, i, vp, vp],
+                           "lk_probe_mfma": [i, i, i, i, i, vp, vp, vp],
+                           "lk_probe_overlap": [i, i, i, i, i, i, vp, vp]}.items():
+            fn = getattr(L, name)
+            fn.restype = i
+            fn.argtypes = args
+        _probes = L
+    return _probes
 
 HBM_PEAK_GBS = 8000.0
 PEAK_TOPS = {0: 5000.0, 1: 2500.0, 2: 5000.0, 3: 5000.0}
@@ -52,7 +74,7 @@ def _graph_us(record, launches_in_graph, replays=20, warm=3):
 
 def launch_floor(workgroups=512, launches=256):
     """Microseconds per launch of a graph of empty 256-thread kernels of `workgroups` workgroups."""
-    L = lib.load()
+    L = load()
 
     def record(s):
         for _ in range(launches):
@@ -73,7 +95,7 @@ class ReadBuffers:
     def rate(self, nbytes, workgroups, pattern, launches=None):
         """(microseconds per launch, GB/s) of launches that each read `nbytes`, walking through the
         allocation so that a launch never re-reads what the last-level cache may still hold."""
-        L = lib.load()
+        L = load()
         nbytes -= nbytes % 16
         copies = max(1, self.total // nbytes)
         if launches is None:
@@ -91,7 +113,7 @@ class ReadBuffers:
 
 def mfma_rate(kind=0, workgroups=2048, iters=2000, valu_per_mfma=0, mode=0):
     """TOP/s of the register-resident matrix-unit loop (and microseconds per launch)."""
-    L = lib.load()
+    L = load()
     sink = torch.zeros(4, dtype=torch.uint8, device="cuda")
     ops = C.c_double(0)
 
@@ -100,6 +122,38 @@ def mfma_rate(kind=0, workgroups=2048, iters=2000, valu_per_mfma=0, mode=0):
 
     us = _graph_us(record, 1, replays=10)
     return ops.value / us / 1e6, us
+
+
+def overlap_ns(kind, valu, dep=0, waves_per_simd=1, iters=20000):
+    """Nanoseconds per slot of one wave of lk_probe_overlap (a SIMD runs `waves_per_simd` of them): one
+    matrix instruction and `valu` fmas; kind 4: the chained item, two instructions and 2 x valu fmas."""
+    L = load()
+    sink = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    s = torch.cuda.current_stream().cuda_stream
+    _check(L.lk_probe_overlap(kind, valu, dep, waves_per_simd, cus, 200, sink.data_ptr(), s), "lk_probe_overlap")
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    _check(L.lk_probe_overlap(kind, valu, dep, waves_per_simd, cus, iters, sink.data_ptr(), s), "lk_probe_overlap")
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e6 / (iters * 4.0)
+
+
+def overlap_table():
+    """Vector work beside matrix work, with nothing waiting on an instruction in flight."""
+    names = {0: "v_mfma_f32_32x32x16_f16", 1: "v_mfma_i32_32x32x32_i8", 2: "v_mfma_i32_16x16x64_i8", 3: "no matrix instruction",
+             4: "item: 2 chained f16 + fmas of the previous item"}
+    out = {}
+    for kind in (3, 0, 1, 2):
+        for dep in ((0, 1) if kind in (0, 1) else (0,)):
+            row = {}
+            for valu in (0, 4, 8, 12, 16, 24, 32):
+                row[f"V{valu}"] = {f"{w}_wave_per_simd_ns": round(overlap_ns(kind, valu, dep, w), 2) for w in (1, 2)}
+            out[f"{names[kind]}, fmas {'read an older result tile' if dep else 'on their own registers'}"] = row
+    out[names[4]] = {f"V{2 * v}": {f"{w}_wave_per_simd_ns": round(overlap_ns(4, v, 0, w), 2) for w in (1, 2)} for v in (4, 8, 12, 16)}
+    return out
 
 
 def ceilings(quick=True):
@@ -142,7 +196,8 @@ def sweep():
         for mode in (0, 1):
             tops, us = mfma_rate(0, valu_per_mfma=valu, mode=mode)
             ov[f"i8_valu{valu}_{'same_wave' if mode == 0 else 'other_wave'}"] = {"tops": round(tops, 1), "us": round(us, 1)}
-    out["mfma_with_vector_work"] = ov
+    out["mfma_with_vector_work_old_probe"] = ov
+    out["overlap_ns_per_slot"] = overlap_table()
     return out
 
 

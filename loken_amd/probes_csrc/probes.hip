@@ -1,9 +1,10 @@
-// Measurement aids: the small kernels that give the measured denominators reported beside the
-// nominal MI355X peaks (launch floor, streaming-read ceiling, matrix-unit issue ceiling, and how
-// vector work overlaps matrix work inside one wave and between two waves of a SIMD).
-// Nothing on the product path calls these; they have no counterpart in the reference.
+// Measurement aids, built into a library of their own (libloken_probes.so) that only the benchmark
+// loads: the small kernels that give the measured denominators reported beside the nominal MI355X
+// peaks (launch floor, streaming-read ceiling, matrix-unit issue ceiling, and how vector work
+// overlaps matrix work inside one wave and between two waves of a SIMD).
+// No product path calls these; they have no counterpart in the reference.
 
-#include "lk_common.h"
+#include "../csrc/lk_common.h"
 
 namespace {
 
@@ -134,6 +135,107 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(int iters, int valu, in
     if (x == 0x9E3779B9u) sink[0] = x;
 }
 
+
+// How vector instructions issue beside matrix instructions. A wave runs `iters` rounds of four slots;
+// a slot is one matrix instruction (KIND: 0 v_mfma_f32_32x32x16_f16, 1 v_mfma_i32_32x32x32_i8,
+// 2 v_mfma_i32_16x16x64_i8, 3 none) into one of four independent accumulator tiles followed by V
+// f32 fmas. DEP 0: the fmas work on registers of their own; DEP 1: they read the accumulator tile
+// whose matrix instruction was issued two slots earlier (finished by then). Nothing forces a wait on
+// an instruction in flight: the order in the source is the order in the binary (sched_barrier), and
+// the compiler adds only the wait states the hardware asks for.
+template <int KIND, int V, int DEP>
+__global__ __launch_bounds__(512) void probe_overlap_kernel(int iters, float s, uint32_t* sink) {
+    const int lane = threadIdx.x & 63;
+    const v4i a = {lane, lane + 1, lane + 2, lane + 3};
+    const v4i b = {lane * 3, 5, lane, 7};
+    typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+    v16f cf[4];
+    v16i ci[4];
+    v4i c4[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { cf[t][e] = 0.f; ci[t][e] = t; if (e < 4) c4[t][e] = t; }
+    float p[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) p[i] = lane + i;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if (KIND == 0) cf[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), cf[t], 0, 0, 0);
+            if (KIND == 1) ci[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, ci[t], 0, 0, 0);
+            if (KIND == 2) c4[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c4[t], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                if (DEP == 0 || KIND >= 2) p[v % 32] = __builtin_fmaf(p[v % 32], s, 1.0f);
+                else if (KIND == 0) p[v % 32] = __builtin_fmaf(cf[(t + 2) & 3][v % 16], s, p[v % 32]);
+                else p[v % 32] = __builtin_fmaf(__builtin_bit_cast(float, ci[(t + 2) & 3][v % 16]), s, p[v % 32]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    float x = 0;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) x += p[i];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { x += cf[t][e] + (float)ci[t][e]; if (e < 4) x += (float)c4[t][e]; }
+    if (x == 12345.678f) sink[0] = 1;
+}
+
+// The tile kernels' item: two chained v_mfma_f32_32x32x16_f16 from a zero accumulator with V fmas of
+// the PREVIOUS item's result behind each (two result tiles alternate), so no fma waits for an
+// instruction in flight. V = 8 is the per-sub-block scale fix-up of a 32 x 32 tile.
+template <int V>
+__global__ __launch_bounds__(512) void probe_item_kernel(int iters, float s, uint32_t* sink) {
+    const int lane = threadIdx.x & 63;
+    typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+    const v4i a = {lane, lane + 1, lane + 2, lane + 3};
+    const v4i b = {lane * 3, 5, lane, 7};
+    v16f dot[2], part;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) { dot[0][e] = 0; dot[1][e] = 0; part[e] = 0; }
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const v16f zero = {0.f};
+            dot[t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), zero, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 0; v < V; ++v) part[v % 16] = __builtin_fmaf(dot[(t + 1) & 1][v % 16], s, part[v % 16]);
+            __builtin_amdgcn_sched_barrier(0);
+            dot[t & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, b), __builtin_bit_cast(v8h, a), dot[t & 1], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = V; v < 2 * V; ++v) part[v % 16] = __builtin_fmaf(dot[(t + 1) & 1][v % 16], s, part[v % 16]);
+            // the sums are complete here and the next item starts from here (the instruction selector
+            // orders only what has side effects)
+            asm volatile("" : "+v"(part));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    float x = 0;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) x += part[e] + dot[0][e] + dot[1][e];
+    if (x == 12345.678f) sink[0] = 1;
+}
+
+typedef void (*OverlapKernel)(int, float, uint32_t*);
+template <int KIND, int DEP>
+static OverlapKernel overlap_kernel(int valu) {
+    switch (valu) {
+        case 0: return probe_overlap_kernel<KIND, 0, DEP>;
+        case 4: return probe_overlap_kernel<KIND, 4, DEP>;
+        case 8: return probe_overlap_kernel<KIND, 8, DEP>;
+        case 12: return probe_overlap_kernel<KIND, 12, DEP>;
+        case 16: return probe_overlap_kernel<KIND, 16, DEP>;
+        case 24: return probe_overlap_kernel<KIND, 24, DEP>;
+        case 32: return probe_overlap_kernel<KIND, 32, DEP>;
+        default: return nullptr;
+    }
+}
 }  // namespace
 
 extern "C" int lk_probe_empty(int workgroups, void* stream) {
@@ -177,5 +279,33 @@ extern "C" int lk_probe_mfma(int kind, int workgroups, int iters, int valu_per_m
         default: return LK_ERR_ARG;
     }
     if (ops) *ops = per * ACCS * (double)iters * 4.0 * (double)workgroups;
+    return lk_launch_status();
+}
+
+// kind 0..3 as probe_overlap_kernel, 4: the chained item (valu = fmas behind EACH of its two matrix
+// instructions: 4, 8, 12 or 16). valu in {0, 4, 8, 12, 16, 24, 32}; dep 0 / 1; waves_per_simd 1 or 2
+// (workgroups of 256 or 512 threads, one workgroup to a CU at `workgroups` <= the CU count).
+extern "C" int lk_probe_overlap(int kind, int valu, int dep, int waves_per_simd, int workgroups, int iters, void* sink,
+                                void* stream) {
+    if (!sink || workgroups < 1 || iters < 1 || (waves_per_simd != 1 && waves_per_simd != 2) || (dep != 0 && dep != 1))
+        return LK_ERR_ARG;
+    OverlapKernel k = nullptr;
+    if (kind == 4) {
+        if (valu == 4) k = probe_item_kernel<4>;
+        if (valu == 8) k = probe_item_kernel<8>;
+        if (valu == 12) k = probe_item_kernel<12>;
+        if (valu == 16) k = probe_item_kernel<16>;
+    } else if (dep == 0) {
+        if (kind == 0) k = overlap_kernel<0, 0>(valu);
+        if (kind == 1) k = overlap_kernel<1, 0>(valu);
+        if (kind == 2) k = overlap_kernel<2, 0>(valu);
+        if (kind == 3) k = overlap_kernel<3, 0>(valu);
+    } else {
+        if (kind == 0) k = overlap_kernel<0, 1>(valu);
+        if (kind == 1) k = overlap_kernel<1, 1>(valu);
+    }
+    if (!k) return LK_ERR_ARG;
+    hipLaunchKernelGGL(k, dim3(workgroups), dim3(256 * waves_per_simd), 0, (hipStream_t)stream, iters, 1.0000001f,
+                       (uint32_t*)sink);
     return lk_launch_status();
 }

@@ -16,6 +16,27 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu on the GPU box)")
 
 
+@pytest.fixture
+def knobs(monkeypatch):
+    """Sets or clears the library's environment overrides (LK_MMQ_I8, LK_TUNE_*) for one test: the
+    library keeps what it read, so every change is followed by lk_tune_refresh, and so is the
+    restoring of the environment when the test ends."""
+    from loken_amd import lib
+
+    class Knobs:
+        def set(self, name, value="1"):
+            monkeypatch.setenv(name, value)
+            lib.load().lk_tune_refresh()
+
+        def clear(self, name):
+            monkeypatch.delenv(name, raising=False)
+            lib.load().lk_tune_refresh()
+
+    yield Knobs()
+    monkeypatch.undo()
+    lib.load().lk_tune_refresh()
+
+
 def _bits_to_f32(hex_words: str) -> np.ndarray:
     """8-hex-digit IEEE bit patterns, most significant digit first."""
     n = len(hex_words) // 8

@@ -100,7 +100,7 @@ def test_tiled_matmul_agrees_with_matvec_family(name):
 
 
 @pytest.mark.parametrize("m,k,n", [(65, 256, 33), (130, 2048, 520), (300, 1024, 128)])
-def test_q4k_wide_tiles_agree_with_int8_tiles_and_matvec(m, k, n, monkeypatch):
+def test_q4k_wide_tiles_agree_with_int8_tiles_and_matvec(m, k, n, knobs):
     # Above 64 token rows Q4_K forms its sub-block dots on the f16 matrix unit (scale folded into
     # the weight operand); LK_MMQ_I8 sends the same call to the int8 tiles. Same integers either
     # way, so only the f32 summation order may differ.
@@ -108,9 +108,9 @@ def test_q4k_wide_tiles_agree_with_int8_tiles_and_matvec(m, k, n, monkeypatch):
     w = dev(synth.weight(wtype, n, k, seed=46, stream=4))
     x = dev(synth.activation(m, k, seed=46))
     wide = ops.mmq_forward(wtype, w, x, n)
-    monkeypatch.setenv("LK_MMQ_I8", "1")
+    knobs.set("LK_MMQ_I8")
     int8 = ops.mmq_forward(wtype, w, x, n)
-    monkeypatch.delenv("LK_MMQ_I8")
+    knobs.clear("LK_MMQ_I8")
     q = ops.quantize_q8_1_rows(x)
     rows = torch.cat([ops.mmvq(wtype, w, q[i:i + 8], k, n) for i in range(0, m, 8)])
     scale = rows.abs().max().item()

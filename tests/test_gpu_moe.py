@@ -447,7 +447,7 @@ def test_generic_routed_product_with_and_without_weights():
                                                               (5, 100, 512, 9, 4), (7, 264, 1024, 12, 6),
                                                               (3, 77, 768, 5, 1), (40, 96, 512, 16, 8), (64, 64, 512, 16, 8)])
 @pytest.mark.parametrize("name", ["q4_k", "q5_k", "q6_k"])
-def test_down_and_fold_in_one_launch_gives_the_bits_of_the_two_launches(name, tokens, hidden, ffn, n_experts, topk, monkeypatch):
+def test_down_and_fold_in_one_launch_gives_the_bits_of_the_two_launches(name, tokens, hidden, ffn, n_experts, topk, knobs):
     """Short K-quant rows at a handful of tokens take one launch (down + fold); with that launch switched
     off the same call takes the per-pair mat-vec and the fold kernel. Same bits, and both on the oracle."""
     dt, block_bytes = {"q4_k": (lib.TYPE_Q4_K, 144), "q5_k": (lib.TYPE_Q5_K, 176), "q6_k": (lib.TYPE_Q6_K, 210)}[name]
@@ -468,7 +468,7 @@ def test_down_and_fold_in_one_launch_gives_the_bits_of_the_two_launches(name, to
     keep = routing.expert_ids[0].item()
     routing.expert_ids[0] = -1
     one_dropped = run()
-    monkeypatch.setenv("LK_TUNE_DOWN_FOLD_OFF", "1")
+    knobs.set("LK_TUNE_DOWN_FOLD_OFF")
     two_dropped = run()
     routing.expert_ids[0] = keep
     two = [run(**kw) for kw in cases]

@@ -137,8 +137,8 @@ def test_tiled_matmul_emits_the_exact_subblock_integers(wtype, m):
     check(lambda w, x: ops.mmq_forward(wtype, w, x, n), wtype, n, k, m, seed=80 + m)
 
 
-def test_q4k_int8_tiles_above_64_rows_emit_the_exact_integers(monkeypatch):
-    monkeypatch.setenv("LK_MMQ_I8", "1")
+def test_q4k_int8_tiles_above_64_rows_emit_the_exact_integers(knobs):
+    knobs.set("LK_MMQ_I8")
     n, k, m = 96, 1024, 130
     check(lambda w, x: ops.mmq_forward(Q4K, w, x, n), Q4K, n, k, m, seed=91)
 
