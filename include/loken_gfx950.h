@@ -137,6 +137,16 @@ int lk_mmvq_pair_act(int wtype, const void* gate, const void* up, const void* vy
  * fused_add_rmsnorm_dual (src/inference/kernel/fused/buffers/conv.rs:990-1110). */
 int lk_rmsnorm_q8_1(const float* x, const float* weight, float* out, void* vy, float eps, int cols, int rows,
                     void* stream);
+/* The reference's own single-row launchers in front of a mat-vec, names and arguments kept
+ * (cuda/moe/rms_qmatmul.cu:152-169 f32 row, :221-238 bf16 row; declared src/inference/moe_cuda/mod.rs:
+ * 117-119, 468-471; called from src/inference/moe_cuda/norm.rs:154, 206): y = Q8_1(rmsnorm(x, w_norm)),
+ * hidden a multiple of 32, no f32 copy. The blocks are lk_rmsnorm_q8_1's (wide-kernel order of the
+ * sum of squares, correctly rounded 1 / sqrt, lk_quantize_q8_1's block rule). Void: nothing is
+ * launched on a bad argument. */
+void loken_rms_quantize_q8_1(const float* x, const float* w_norm, void* y_q8_1, int hidden, float rms_eps,
+                             void* stream);
+void loken_rms_quantize_q8_1_bf16(const void* x, const float* w_norm, void* y_q8_1, int hidden, float rms_eps,
+                                  void* stream);
 /* sum_out = x + residual; norm_out = rmsnorm(sum_out, weight), also as Q8_1. */
 int lk_add_rmsnorm_q8_1(const float* x, const float* residual, const float* weight, float* sum_out,
                         float* norm_out, void* vy, float eps, int cols, int rows, void* stream);
@@ -423,6 +433,17 @@ int loken_moe_gemm_gguf(const float* inputs, const void* weights, const int32_t*
                         const int32_t* expert_ids, const float* topk_weights, void* outputs,
                         int num_experts, int topk, int size_m, int size_n, int size_k, int quant_type,
                         void* stream);
+/* The prefill form (declared src/inference/moe_cuda/mod.rs:478-483; called from moe_gemm_gguf when
+ * the card has matrix instructions, src/inference/moe_cuda/gemm.rs:221-258; AMD body
+ * cuda/moe/moe_wmma_amd.cu:311-339): activation rows at the model's own width, input_dtype 0 = f16,
+ * 1 = bf16 (anything else: LK_ERR_TYPE); the other arguments, the row conventions and the status as
+ * loken_moe_gemm_gguf. Rows are quantized to Q8_1 from that width and served by the same kernels, so
+ * results carry the decode path's integers (the reference multiplies dequantized weights on bf16
+ * fragments instead: both approximate the f32 product). */
+int loken_moe_gemm_gguf_prefill(const void* input, const uint8_t* weights, const int32_t* sorted_token_ids,
+                                const int32_t* expert_ids, const float* topk_weights, void* output,
+                                int num_experts, int topk, int size_m, int size_n, int size_k, int input_dtype,
+                                int gguf_dtype, void* stream);
 /* out[slot, :] = silu(gate_e . x[slot / topk]) * (up_e . x[slot / topk]); inputs [size_m/topk, k]. */
 int loken_moe_gemm_gguf_gate_up_silu_mul(const float* inputs, const void* gate_weights,
                                          const void* up_weights, const int32_t* sorted_token_ids,

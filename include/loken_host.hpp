@@ -44,8 +44,10 @@ public:
      * Q6_K / Q8_0), owned by the caller, on device `device`. */
     QKernelMatMul(int dtype, int n, int k, const void* blob, int device);
 
-    /* x [rows, k] (LK_TYPE_F32; F16 / BF16 for calls that stay on the mat-vec family) ->
-     * out [rows, n] in x's type, on `stream`. `decode_order` keeps every row on the mat-vec
+    /* x [rows, k] (LK_TYPE_F32, F16 or BF16) -> out [rows, n] in x's type, on `stream`. The
+     * matrix-unit kernels write f32 rows; for f16 / bf16 rows they write into a buffer of the device's
+     * slot and one more launch rounds them into `out` (the reference narrows the f32 rows its
+     * mmq_forward returns the same way, kernel_matmul.rs:1086-1714). `decode_order` keeps every row on the mat-vec
      * kernels whatever the count (DecodeOrder of the reference, kernel_matmul.rs:34-75).
      * Returns LK_OK or an LK_ERR_* code; never throws, never aborts. */
     int forward(const void* x, int x_type, int rows, void* out, void* stream, bool decode_order = false);

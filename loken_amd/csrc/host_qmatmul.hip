@@ -3,8 +3,11 @@
 #include "../../include/loken_host.hpp"
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
 
 #include <map>
+#include <type_traits>
 #include <mutex>
 
 namespace loken {
@@ -25,6 +28,8 @@ struct Slot {
     void* act = nullptr;      // Q8_1 rows / tiled-matmul workspace
     size_t act_bytes = 0;
     void* fixup = nullptr;
+    void* out32 = nullptr;    // f32 result rows of a call whose rows came in f16 / bf16 (the matrix-unit kernels write f32)
+    size_t out32_bytes = 0;
     hipEvent_t last_use = nullptr;
     bool used = false;
 };
@@ -88,6 +93,41 @@ int reserve(Slot& slot, size_t bytes, bool want_fixup, hipStream_t stream) {
     if (slot.used && slot.last_use && !rec && hipStreamWaitEvent(stream, slot.last_use, 0) != hipSuccess)
         (void)hipGetLastError();
     return LK_OK;
+}
+
+// The f32 rows a half-precision call's kernels write before they are narrowed into the caller's buffer.
+int reserve_out32(Slot& slot, size_t bytes, hipStream_t stream) {
+    if (slot.out32_bytes >= bytes) return LK_OK;
+    if (capturing(stream)) return LK_ERR_NOMEM;
+    if (slot.out32) {
+        if (hipStreamSynchronize(stream) != hipSuccess || hipFree(slot.out32) != hipSuccess) (void)hipGetLastError();
+        slot.out32 = nullptr;
+        slot.out32_bytes = 0;
+    }
+    if (hipMalloc(&slot.out32, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        slot.out32 = nullptr;
+        return LK_ERR_NOMEM;
+    }
+    slot.out32_bytes = bytes;
+    return LK_OK;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void narrow_rows_kernel(const float* __restrict__ from, T* __restrict__ to, size_t count) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    if constexpr (sizeof(T) == 2 && std::is_same<T, __half>::value) to[i] = __float2half_rn(from[i]);
+    else to[i] = __float2bfloat16(from[i]);
+}
+
+// out (f16 / bf16) = the f32 rows, rounded to nearest: the conversion the reference applies to the
+// f32 rows mmq_forward returns (src/tensor/quantized/kernel_matmul.rs:1086-1714, output dtype follows input).
+int narrow_rows(const float* from, void* to, int type, size_t count, hipStream_t stream) {
+    const unsigned grid = (unsigned)((count + 255) / 256);
+    if (type == LK_TYPE_F16) hipLaunchKernelGGL(narrow_rows_kernel<__half>, dim3(grid), dim3(256), 0, stream, from, (__half*)to, count);
+    else hipLaunchKernelGGL(narrow_rows_kernel<__hip_bfloat16>, dim3(grid), dim3(256), 0, stream, from, (__hip_bfloat16*)to, count);
+    return hipGetLastError() == hipSuccess ? LK_OK : LK_ERR_LAUNCH;
 }
 
 void mark_used(Slot& slot, hipStream_t stream) {
@@ -158,7 +198,7 @@ static bool rows_kernel_serves(int dtype, int n, int rows) {
 // 4096 x 4096 and 2048 x 6144 from 7 (as two sets of four rows: 8.9 us against 9.5 at 8 rows, 8.1 as mat-vec at 6).
 static bool small_rows_kernel_pays(int dtype, int n, int k, int rows) {
     if (rows < 3 || rows > 8 || k % 256 != 0) return false;
-    if (dtype == LK_TYPE_Q6_K) return k % 2048 == 0 && ((long long)n * k >= (48ll << 20) || rows >= 7);
+    if (dtype == LK_TYPE_Q6_K) return k % 2048 == 0 && ((long long)n * k >= (48ll << 20) || (rows >= 7 && n >= 1024));
     if (dtype != LK_TYPE_Q4_K && dtype != LK_TYPE_Q5_K) return false;
     return (long long)n * rows >= (k <= 2048 ? 8192 : 57344);
 }
@@ -185,10 +225,11 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     Slot& slot = slot_of(device_);
 
     // --- mat-vec family: up to matvec_rows, or any count when every row must sum like a one-row call
-    const bool to_rows_kernel = x_type == LK_TYPE_F32 && small_rows_kernel_pays(dtype_, n_, k_, rows);
-    const bool to_nibble_tiles = x_type == LK_TYPE_F32 && !decode_order && nibble_tiles_pay(dtype_, n_, k_, rows) &&
+    const bool rows_kernel_fits = k_ % 256 == 0 && ((uintptr_t)blob_ & (dtype_ == LK_TYPE_Q6_K ? 1 : 15)) == 0;
+    const bool to_rows_kernel = rows_kernel_fits && small_rows_kernel_pays(dtype_, n_, k_, rows);
+    const bool to_nibble_tiles = !decode_order && nibble_tiles_pay(dtype_, n_, k_, rows) &&
                                  ((uintptr_t)blob_ & (dtype_ == LK_TYPE_Q2_K ? 3 : 1)) == 0;
-    if ((rows <= mv_max && !to_rows_kernel) || decode_order || (plain && !to_nibble_tiles)) {
+    auto matvec = [&]() -> int {
         if (!plain && x_type == LK_TYPE_F32 && rows <= 2 && k_ <= 8192 && ((uintptr_t)x & 15) == 0 && k_ % 4 == 0) {
             const void* vx[1] = {blob_};
             void* dst[1] = {out};
@@ -210,27 +251,42 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
         mark_used(slot, stream);
         last_path_ = Path::MatVec;
         return LK_OK;
-    }
-    if (x_type != LK_TYPE_F32) return LK_ERR_TYPE;   // the matrix-unit kernels write f32
+    };
+    if ((rows <= mv_max && !to_rows_kernel) || decode_order || (plain && !to_nibble_tiles)) return matvec();
+
+    // The matrix-unit kernels write f32 rows. Rows that came in f16 / bf16 leave in that type, as the
+    // reference's do (the f32 rows its mmq_forward returns are narrowed by the caller,
+    // src/tensor/quantized/kernel_matmul.rs:1086-1714): the kernels write into a buffer of the
+    // device's slot and one more launch rounds them into `out`.
+    const bool half_rows = x_type != LK_TYPE_F32;
+    const size_t out_count = (size_t)rows * n_;
 
     // --- a handful of rows (or a matrix too small to fill the chip with tiles): matrix unit, weights
     //     straight from HBM
-    if (rows_kernel_serves(dtype_, n_, rows) && k_ % 256 == 0 && ((uintptr_t)blob_ & (dtype_ == LK_TYPE_Q6_K ? 1 : 15)) == 0) {
+    if (rows_kernel_serves(dtype_, n_, rows) && rows_kernel_fits) {
         const int blocks = k_ / 32;
-        std::lock_guard<std::mutex> pair(slot.mu);
-        if (int rc = reserve(slot, (size_t)rows * blocks * Q81_BLOCK, false, stream)) return rc;
-        if (int rc = lk_quantize_q8_1(x, x_type, slot.act, k_, k_, rows, stream)) return rc;
-        // the launchers with a status (the exported void forms drop it): rows too long for their scale
-        // tables in LDS launch nothing, and the call goes on to the tiled matmul below
-        const int rc = dtype_ == LK_TYPE_Q4_K   ? lk_dense_q4k_rows(blob_, slot.act, (float*)out, rows, n_, k_, stream)
-                       : dtype_ == LK_TYPE_Q5_K ? lk_dense_q5k_rows(blob_, slot.act, (float*)out, rows, n_, k_, stream)
-                                                : lk_dense_q6k_rows(blob_, slot.act, (float*)out, rows, n_, k_, stream);
-        mark_used(slot, stream);
+        int rc;
+        {
+            std::lock_guard<std::mutex> pair(slot.mu);
+            if (int r = reserve(slot, (size_t)rows * blocks * Q81_BLOCK, false, stream)) return r;
+            if (half_rows)
+                if (int r = reserve_out32(slot, out_count * 4, stream)) return r;
+            float* dst = half_rows ? (float*)slot.out32 : (float*)out;
+            if (int r = lk_quantize_q8_1(x, x_type, slot.act, k_, k_, rows, stream)) return r;
+            // the launchers with a status (the exported void forms drop it): rows too long for their scale
+            // tables in LDS launch nothing, and the call goes on to the mat-vec or the tiled matmul below
+            rc = dtype_ == LK_TYPE_Q4_K   ? lk_dense_q4k_rows(blob_, slot.act, dst, rows, n_, k_, stream)
+                 : dtype_ == LK_TYPE_Q5_K ? lk_dense_q5k_rows(blob_, slot.act, dst, rows, n_, k_, stream)
+                                          : lk_dense_q6k_rows(blob_, slot.act, dst, rows, n_, k_, stream);
+            if (rc == LK_OK && half_rows) rc = narrow_rows(dst, out, x_type, out_count, stream);
+            mark_used(slot, stream);
+        }
         if (rc == LK_OK) {
             last_path_ = Path::RowsOnMatrixUnit;
             return LK_OK;
         }
         if (rc != LK_ERR_ARG) return rc;
+        if (rows <= mv_max) return matvec();   // a few rows the rows kernel declined: not worth a tile
     }
 
     // --- tiled matmul (mmq_forward, kernel_matmul/mmq.rs:21-159)
@@ -239,12 +295,15 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     const size_t ws_bytes = (size_t)rows * (k_padded / 128) * MMQ_RECORD + 128 * MMQ_RECORD;
     std::lock_guard<std::mutex> pair(slot.mu);
     if (int rc = reserve(slot, ws_bytes, true, stream)) return rc;
+    if (half_rows)
+        if (int rc = reserve_out32(slot, out_count * 4, stream)) return rc;
+    void* dst = half_rows ? slot.out32 : out;
     // the layouts of the reference's table (quantized/mmq.rs:274-285)
     auto quantizer = dtype_ == LK_TYPE_Q2_K ? launch_mmq_quantize_q8_1_D2S6
                      : dtype_ == LK_TYPE_Q6_K || dtype_ == LK_TYPE_Q8_0 || dtype_ == LK_TYPE_Q5_0 || dtype_ == LK_TYPE_Q3_K
                          ? launch_mmq_quantize_q8_1_D4
                          : launch_mmq_quantize_q8_1_DS4;
-    quantizer(x, nullptr, slot.act, 0, k_, k_, 0, 0, (int64_t)k_padded, rows, 1, 1, stream);
+    quantizer(x, nullptr, slot.act, x_type, k_, k_, 0, 0, (int64_t)k_padded, rows, 1, 1, stream);
     auto launcher = dtype_ == LK_TYPE_Q4_K   ? launch_mmq_gguf_q4_k
                     : dtype_ == LK_TYPE_Q5_K ? launch_mmq_gguf_q5_k
                     : dtype_ == LK_TYPE_Q6_K ? launch_mmq_gguf_q6_k
@@ -257,10 +316,13 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
                                              : launch_mmq_gguf_q8_0;
     int abi = 0, cus = 0, lds = 0, wave = 0;
     (void)lk_device_info(&abi, &cus, &lds, &wave);
-    const int tile = launcher(slot.fixup, blob_, slot.act, out, k_, n_, rows, k_ / block_len, n_, 0x1000950, cus, lds, wave,
+    const int tile = launcher(slot.fixup, blob_, slot.act, dst, k_, n_, rows, k_ / block_len, n_, 0x1000950, cus, lds, wave,
                               stream);
+    int narrowed = LK_OK;
+    if (tile != 0 && half_rows) narrowed = narrow_rows((const float*)dst, out, x_type, out_count, stream);
     mark_used(slot, stream);
     if (tile == 0) return LK_ERR_ARG;   // "no tile fits, nothing ran": the reference falls back to dequantized
+    if (narrowed != LK_OK) return narrowed;
     last_path_ = Path::Tiled;
     return LK_OK;
 }
@@ -276,6 +338,9 @@ void release_workspaces() {
         (void)hipDeviceSynchronize();
         if (s.act) (void)hipFree(s.act);
         if (s.fixup) (void)hipFree(s.fixup);
+        if (s.out32) (void)hipFree(s.out32);
+        s.out32 = nullptr;
+        s.out32_bytes = 0;
         if (s.last_use) (void)hipEventDestroy(s.last_use);
         s.act = s.fixup = nullptr;
         s.act_bytes = 0;

@@ -90,6 +90,9 @@ static void launch_quantize(const void* x, const int32_t* ids, void* vy, int typ
     if (type_x == LK_TYPE_F16) {
         hipLaunchKernelGGL(mmq_quantize_kernel<__half>, grid, dim3(256), 0, s, (const __half*)x, ids,
                            (uint8_t*)vy, ne00, s01, s02, s03, ne0, (int)ne1, (int)ne2);
+    } else if (type_x == LK_TYPE_BF16) {
+        hipLaunchKernelGGL(mmq_quantize_kernel<__hip_bfloat16>, grid, dim3(256), 0, s, (const __hip_bfloat16*)x, ids,
+                           (uint8_t*)vy, ne00, s01, s02, s03, ne0, (int)ne1, (int)ne2);
     } else {
         hipLaunchKernelGGL(mmq_quantize_kernel<float>, grid, dim3(256), 0, s, (const float*)x, ids,
                            (uint8_t*)vy, ne00, s01, s02, s03, ne0, (int)ne1, (int)ne2);

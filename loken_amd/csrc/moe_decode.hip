@@ -331,6 +331,37 @@ extern "C" int loken_moe_gemm_gguf(const float* inputs, const void* weights, con
                                      topk_weights, nullptr, (float*)outputs, d, size_k, s);
 }
 
+// The prefill form of the launch above (declared src/inference/moe_cuda/mod.rs:478-483; called from
+// moe_gemm_gguf whenever the card has matrix instructions, src/inference/moe_cuda/gemm.rs:221-258;
+// the reference's body for AMD cards: cuda/moe/moe_wmma_amd.cu:311-339): the activation rows arrive
+// at the model's own width (input_dtype 0 = f16, 1 = bf16), everything else as loken_moe_gemm_gguf.
+// The rows are quantized to Q8_1 from that width (the value an f16 / bf16 holds is exact in f32, so
+// the codes are those lk_quantize_q8_1 gives the same values as f32) and run through the same
+// per-pair kernels: same integers, same combine, same row conventions. The reference's kernel
+// dequantizes the weights to the activation's width instead and multiplies on bf16 fragments; both
+// approximate the f32 product of the dequantized operands, this one to the decode path's bound.
+extern "C" int loken_moe_gemm_gguf_prefill(const void* inputs, const uint8_t* weights, const int32_t* sorted_token_ids,
+                                           const int32_t* expert_ids, const float* topk_weights, void* outputs,
+                                           int num_experts, int topk, int size_m, int size_n, int size_k,
+                                           int input_dtype, int quant_type, void* stream) {
+    if (block_len_of_wire(quant_type) == 0) return LK_ERR_TYPE;
+    if (input_dtype != 0 && input_dtype != 1) return LK_ERR_TYPE;
+    if (size_m == 0) return LK_OK;
+    if (!inputs || !weights || !sorted_token_ids || !expert_ids || !outputs ||
+        bad_shape(quant_type, num_experts, topk, size_m, size_n, size_k)) return LK_ERR_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const int kp = pad512(size_k);
+    const int act_rows = topk_weights ? size_m : size_m / topk;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    uint8_t* acts = (uint8_t*)reserve_scratch((size_t)act_rows * (kp / 32) * Q81_BYTES, s);
+    if (!acts) return LK_ERR_NOMEM;
+    if (int rc = lk_quantize_q8_1(inputs, input_dtype == 0 ? LK_TYPE_F16 : LK_TYPE_BF16, acts, size_k, kp, act_rows, stream))
+        return rc;
+    MoeDims d{num_experts, topk, size_m, size_n, 0, kp / 32, 0};
+    return launch_format<MODE_PLAIN>(quant_type, weights, nullptr, acts, sorted_token_ids, expert_ids, topk_weights, nullptr,
+                                     (float*)outputs, d, size_k, s);
+}
+
 // The gated launch: act(gate . x, up . x) per routed pair. `slab_rows` = weight rows per expert in
 // both stacks (size_n, or 2 size_n when `up_weights` points size_n rows into the gate's tensor).
 static int gate_up_impl(const float* inputs, const void* gate_weights, const void* up_weights,

@@ -76,8 +76,12 @@ static __device__ __forceinline__ float inv_rms(const float* srow, float* tree, 
 
 // MODE 0: out = rmsnorm(x, w).  MODE 1: sum = x + residual; out = rmsnorm(sum, w).
 // MODE 2: x_out = rmsnorm(x, w_first) + residual; out = rmsnorm(x_out, w).
-template <int MODE>
-__global__ __launch_bounds__(NORM_WG) void norm_q8_1_kernel(const float* __restrict__ x, const float* __restrict__ w_first,
+static __device__ __forceinline__ float row_value(const float* x, size_t i) { return x[i]; }
+static __device__ __forceinline__ float row_value(const __hip_bfloat16* x, size_t i) { return __bfloat162float(x[i]); }
+
+// `out` may be null (MODE 0 only): the row then leaves as Q8_1 alone.
+template <int MODE, typename XT = float>
+__global__ __launch_bounds__(NORM_WG) void norm_q8_1_kernel(const XT* __restrict__ x, const float* __restrict__ w_first,
                                                             const float* __restrict__ residual,
                                                             const float* __restrict__ w, float* __restrict__ mid_out,
                                                             float* __restrict__ out, uint8_t* __restrict__ vy,
@@ -87,7 +91,7 @@ __global__ __launch_bounds__(NORM_WG) void norm_q8_1_kernel(const float* __restr
     const int t = threadIdx.x;
     const size_t offset = (size_t)blockIdx.x * cols;
     for (int i = t; i < cols; i += NORM_WG) {
-        float v = x[offset + i];
+        float v = row_value(x, offset + i);
         if (MODE == 1) {
             v = v + residual[offset + i];
             mid_out[offset + i] = v;
@@ -107,7 +111,7 @@ __global__ __launch_bounds__(NORM_WG) void norm_q8_1_kernel(const float* __restr
     uint8_t* row_blocks = vy + (size_t)blockIdx.x * (cols / 32) * Q81_BYTES;
     for (int i = t; i < cols; i += NORM_WG) {
         const float v = (srow[i] * rms) * w[i];
-        out[offset + i] = v;
+        if (out) out[offset + i] = v;
         quantize_lane(row_blocks, i, v);
     }
 }
@@ -194,4 +198,31 @@ extern "C" int lk_split_act_mul_q8_1(const float* gu, float* out, void* vy, int 
     else
         hipLaunchKernelGGL(split_act_mul_q8_1_kernel<1>, grid, dim3(NORM_WG), 0, (hipStream_t)stream, gu, out, (uint8_t*)vy, n);
     return lk_launch_status();
+}
+
+// The reference's own names for the single-row launch in front of a mat-vec (cuda/moe/rms_qmatmul.cu:
+// 152-169 f32 row, :221-238 bf16 row; declared src/inference/moe_cuda/mod.rs:117-119, 468-471; called
+// from src/inference/moe_cuda/norm.rs:154, 206): y = Q8_1(rmsnorm(x, w_norm)), no f32 copy. Served
+// by the kernel above, so the blocks are those of lk_rmsnorm_q8_1 (the sum of squares in the wide
+// kernels' order, 1 / sqrt correctly rounded, lk_quantize_q8_1's block rule); hidden a multiple of
+// 32 whose f32 row fits LDS. Void, as the reference's: nothing is launched on a bad argument.
+extern "C" void loken_rms_quantize_q8_1(const float* x, const float* w_norm, void* y_q8_1, int hidden, float rms_eps,
+                                        void* stream) {
+    if (!x || !w_norm || !y_q8_1 || ((uintptr_t)y_q8_1 & 3) || hidden <= 0 || hidden % 32 != 0 ||
+        (int64_t)hidden * 4 + NORM_WG * 4 > lk_device().lds_bytes)
+        return;
+    if (prepare_lds(norm_q8_1_kernel<0, float>, hidden * 4) != LK_OK) return;
+    hipLaunchKernelGGL((norm_q8_1_kernel<0, float>), dim3(1), dim3(NORM_WG), hidden * 4, (hipStream_t)stream, x, nullptr, nullptr,
+                       w_norm, nullptr, nullptr, (uint8_t*)y_q8_1, 0.0f, rms_eps, hidden);
+}
+
+extern "C" void loken_rms_quantize_q8_1_bf16(const void* x, const float* w_norm, void* y_q8_1, int hidden, float rms_eps,
+                                             void* stream) {
+    if (!x || !w_norm || !y_q8_1 || ((uintptr_t)y_q8_1 & 3) || ((uintptr_t)x & 1) || hidden <= 0 || hidden % 32 != 0 ||
+        (int64_t)hidden * 4 + NORM_WG * 4 > lk_device().lds_bytes)
+        return;
+    if (prepare_lds(norm_q8_1_kernel<0, __hip_bfloat16>, hidden * 4) != LK_OK) return;
+    hipLaunchKernelGGL((norm_q8_1_kernel<0, __hip_bfloat16>), dim3(1), dim3(NORM_WG), hidden * 4, (hipStream_t)stream,
+                       (const __hip_bfloat16*)x, nullptr, nullptr, w_norm, nullptr, nullptr, (uint8_t*)y_q8_1, 0.0f, rms_eps,
+                       hidden);
 }

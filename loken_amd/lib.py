@@ -143,6 +143,9 @@ SIGNATURES.update({
     "lk_moe_q4k_rows_gate_up": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "loken_moe_q4k_imma_m8_down": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "lk_tune_refresh": (None, []),
+    "loken_moe_gemm_gguf_prefill": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "loken_rms_quantize_q8_1": (None, [_vp, _vp, _vp, _i, _f, _vp]),
+    "loken_rms_quantize_q8_1_bf16": (None, [_vp, _vp, _vp, _i, _f, _vp]),
     "loken_moe_mmq_fold": (None, [_vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
 })
 

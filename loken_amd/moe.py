@@ -356,6 +356,21 @@ def moe_gemm_gguf(wtype: int, x: torch.Tensor, weights: torch.Tensor, routing: E
     return out
 
 
+def moe_gemm_gguf_prefill(wtype: int, x: torch.Tensor, weights: torch.Tensor, routing: ExpertRouting, n_experts: int,
+                          n: int, topk_weights: torch.Tensor | None = None) -> torch.Tensor:
+    """The same product from f16 / bf16 activation rows: what moe_gemm_gguf calls for a prefill on a card
+    with matrix instructions (src/inference/moe_cuda/gemm.rs:221-258)."""
+    k = x.shape[1]
+    pairs = routing.tokens * routing.topk
+    out = torch.empty((pairs, n), dtype=torch.float32, device=x.device)
+    input_dtype = {torch.float16: 0, torch.bfloat16: 1}[x.dtype]
+    _lib.check("loken_moe_gemm_gguf_prefill", _lib.load().loken_moe_gemm_gguf_prefill(
+        x.data_ptr(), weights.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+        topk_weights.data_ptr() if topk_weights is not None else None, out.data_ptr(), n_experts, routing.topk,
+        pairs, n, k, input_dtype, EXPERT_QUANT_CODES[wtype], _stream()))
+    return out
+
+
 def topk_softmax(logits: torch.Tensor, topk: int, renorm: bool = True):
     """Router: ``[tokens, experts]`` f32 logits -> (weights f32 ``[tokens, topk]``, choices int32
     ``[tokens, topk]``), probabilities descending, ties to the lower expert id (topk_softmax,

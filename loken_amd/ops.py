@@ -50,6 +50,16 @@ def rmsnorm_q8_1(x: torch.Tensor, weight: torch.Tensor, eps: float):
     return out, q
 
 
+def rms_quantize_q8_1(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """loken_rms_quantize_q8_1 / _bf16 (src/inference/moe_cuda/norm.rs:154, 206): one f32 or bf16 row of
+    `hidden` values -> its RMS-normed Q8_1 blocks ``[hidden / 32, 36]`` (no f32 copy)."""
+    hidden = x.numel()
+    q = torch.zeros((hidden // 32, 36), dtype=torch.uint8, device=x.device)
+    fn = {torch.float32: "loken_rms_quantize_q8_1", torch.bfloat16: "loken_rms_quantize_q8_1_bf16"}[x.dtype]
+    getattr(_lib.load(), fn)(x.data_ptr(), weight.data_ptr(), q.data_ptr(), hidden, eps, _stream())
+    return q
+
+
 def add_rmsnorm_q8_1(x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float):
     """fused_add_rmsnorm_dual (src/inference/kernel/fused/buffers/conv.rs:1043-1110) -> (sum, norm, q8_1)."""
     rows, cols = x.shape

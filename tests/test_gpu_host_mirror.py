@@ -96,7 +96,7 @@ def test_decode_order_keeps_every_row_on_the_matvec_family_and_rows_independent(
         lin.close()
 
 
-def test_half_inputs_stay_in_their_type_on_the_matvec_family_and_are_declined_above_it():
+def test_half_inputs_stay_in_their_type_on_the_matvec_family():
     wtype, n, k = lib.TYPE_Q6_K, 64, 512
     w = dev(synth.weight(wtype, n, k, seed=82, stream=1))
     lin = Linear(wtype, w, n, k)
@@ -106,8 +106,35 @@ def test_half_inputs_stay_in_their_type_on_the_matvec_family_and_are_declined_ab
         assert y.dtype == torch.bfloat16 and lin.path == "matvec"
         want = ops.mmvq(wtype, w, ops.quantize_q8_1_rows(x), k, n, out_dtype=torch.bfloat16)
         assert torch.equal(y, want)
-        with pytest.raises(lib.LokenError):
-            lin(dev(synth.activation(50, k, seed=82)).to(torch.float16))
+    finally:
+        lin.close()
+
+
+@pytest.mark.parametrize("half", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("name,rows,n,expect", [
+    ("q6_k", 50, 64, "rows-on-matrix-unit"), ("q4_k", 20, 200, "rows-on-matrix-unit"), ("q4_k", 4, 4000, "rows-on-matrix-unit"),
+    ("q4_k", 130, 24000, "tiled"), ("q4_k", 300, 6000, "tiled"), ("q6_k", 200, 24000, "tiled"), ("q8_0", 40, 200, "tiled"),
+    ("q5_1", 60, 200, "tiled"), ("q5_k", 90, 24000, "tiled")])
+def test_half_rows_above_the_matvec_family_follow_the_oracle_and_leave_in_their_type(name, rows, n, expect, half):
+    # the reference's forward serves f16 / bf16 rows at every row count and returns their type
+    # (src/tensor/quantized/kernel_matmul.rs:1086-1714): the oracle is fed the values the rows hold, and
+    # the result is the f32 call's result rounded once to the narrow type
+    wtype, k = DT[name], 1024
+    w = synth.weight(wtype, n, k, seed=83, stream=1)
+    xh = dev(synth.activation(rows, k, seed=83)).to(half)
+    x_seen = xh.to(torch.float32)
+    lin = Linear(wtype, dev(w), n, k)
+    try:
+        got = lin(xh)
+        assert got.dtype == half and lin.path == expect
+        wide = lin(x_seen)
+        assert lin.path == expect
+        assert torch.equal(got, wide.to(half))
+        pick = np.arange(n) if n <= 400 else np.sort(np.random.default_rng(83).choice(n, 300, replace=False))
+        want = oracle.ob_matmul(wtype, x_seen.cpu().numpy(), w[pick], len(pick))
+        eps = 2.0 ** -8 if half == torch.bfloat16 else 2.0 ** -11   # one rounding to the narrow type
+        gotf = got.to(torch.float32).cpu().numpy()[:, pick].astype(np.float64)
+        assert (np.abs(gotf - want) <= (1e-3 + eps) * np.abs(want) + 1e-4).all()
     finally:
         lin.close()
 

@@ -443,6 +443,40 @@ def test_generic_routed_product_with_and_without_weights():
         assert_close(scaled[p], w.reshape(-1)[p] * oracle.ob_matmul(lib.TYPE_Q8_0, xs[p:p + 1], we[e], n)[0])
 
 
+@pytest.mark.parametrize("half", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("name", ["q4_k", "q6_k", "q8_0", "q5_1"])
+def test_prefill_form_takes_half_precision_rows(name, half):
+    # loken_moe_gemm_gguf_prefill: the rows arrive as f16 / bf16; the oracle is fed the values they hold
+    from loken_amd.moe import moe_gemm_gguf_prefill
+    wtype = {"q4_k": lib.TYPE_Q4_K, "q6_k": lib.TYPE_Q6_K, "q8_0": lib.TYPE_Q8_0, "q5_1": lib.TYPE_Q5_1}[name]
+    tokens, k, n, n_experts, topk = 9, 512, 96, 6, 2
+    wq = synth.weight(wtype, n_experts * n, k, seed=61, stream=1)
+    ids, w = oracle.topk_softmax(synth.activation(tokens, n_experts, seed=61, stream=7), topk)
+    routing = ExpertRouting(dev(ids))
+    we = wq.reshape(n_experts, -1)   # an expert's n rows of blocks
+    xh = dev(synth.activation(tokens, k, seed=61)).to(half)
+    x_seen = xh.to(torch.float32).cpu().numpy()
+    got = moe_gemm_gguf_prefill(wtype, xh, dev(wq), routing, n_experts, n).cpu().numpy()
+    for t in range(tokens):
+        for j in range(topk):
+            assert_close(got[t * topk + j], oracle.ob_matmul(wtype, x_seen[t:t + 1], we[ids[t, j]], n)[0])
+    # the same values as f32 rows through the decode-form launch: the same bits
+    same = moe_gemm_gguf(wtype, xh.to(torch.float32), dev(wq), routing, n_experts, n).cpu().numpy()
+    assert np.array_equal(got, same)
+    # with routing weights: one activation row per slot, output scaled
+    xs = dev(synth.activation(tokens * topk, k, seed=61, stream=8)).to(half)
+    scaled = moe_gemm_gguf_prefill(wtype, xs, dev(wq), routing, n_experts, n, topk_weights=dev(w.reshape(-1))).cpu().numpy()
+    xs_seen = xs.to(torch.float32).cpu().numpy()
+    for p in range(tokens * topk):
+        e = ids.reshape(-1)[p]
+        assert_close(scaled[p], w.reshape(-1)[p] * oracle.ob_matmul(wtype, xs_seen[p:p + 1], we[e], n)[0])
+    # an input width the launch does not know is a status, not a launch
+    L = lib.load()
+    assert L.loken_moe_gemm_gguf_prefill(xh.data_ptr(), dev(wq).data_ptr(), routing.sorted_token_ids.data_ptr(),
+                                         routing.expert_ids.data_ptr(), None, dev(np.zeros(4, np.float32)).data_ptr(),
+                                         n_experts, topk, tokens * topk, n, k, 2, 1, None) == lib.LK_ERR_TYPE
+
+
 @pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(1, 2048, 768, 128, 8), (16, 2048, 768, 128, 8),
                                                               (5, 100, 512, 9, 4), (7, 264, 1024, 12, 6),
                                                               (3, 77, 768, 5, 1), (40, 96, 512, 16, 8), (64, 64, 512, 16, 8)])

@@ -47,6 +47,28 @@ def test_rmsnorm_row_and_its_q8_1(rows, cols):
     assert torch.equal(q, ops.quantize_q8_1_rows(out))
 
 
+@pytest.mark.parametrize("hidden", [512, 2048, 4096, 2080, 96, 14336])
+def test_reference_named_single_row_launch_writes_the_same_blocks(hidden):
+    # loken_rms_quantize_q8_1 / _bf16: Q8_1 only, any multiple of 32
+    x, _, w, _ = inputs(1, hidden, 150 + hidden)
+    want = oracle.norm_rows(0, x, w, eps=1e-5)
+    q = ops.rms_quantize_q8_1(dev(x[0]), dev(w), 1e-5)
+    assert np.array_equal(host(q), q8_1_of(want)[0])
+    xb = dev(x[0]).to(torch.bfloat16)
+    x_seen = xb.to(torch.float32).cpu().numpy()[None, :]
+    qb = ops.rms_quantize_q8_1(xb, dev(w), 1e-5)
+    assert np.array_equal(host(qb), q8_1_of(oracle.norm_rows(0, x_seen, w, eps=1e-5))[0])
+
+
+def test_reference_named_single_row_launch_declines_bad_arguments():
+    q = torch.full((4, 36), 7, dtype=torch.uint8, device="cuda")
+    x = torch.ones(100, device="cuda")
+    lib.load().loken_rms_quantize_q8_1(x.data_ptr(), x.data_ptr(), q.data_ptr(), 100, 1e-5, None)   # not a multiple of 32
+    lib.load().loken_rms_quantize_q8_1(None, x.data_ptr(), q.data_ptr(), 96, 1e-5, None)
+    torch.cuda.synchronize()
+    assert (q == 7).all()
+
+
 @pytest.mark.parametrize("rows,cols", SHAPES)
 def test_add_then_rmsnorm(rows, cols):
     x, res, w, _ = inputs(rows, cols, 200 + cols)
