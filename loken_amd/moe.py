@@ -446,20 +446,27 @@ def moe_mmq_pays(rows: int, experts: int, wtype: int | None = None) -> bool:
 
 def moe_forward(wtype_gu: int, wtype_down: int, x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
                 down: torch.Tensor, choices: torch.Tensor, topk_weights: torch.Tensor, n_experts: int,
-                ffn: int) -> torch.Tensor:
+                ffn: int, return_rows: bool = False):
     """The expert block of one layer, path chosen as the reference's layer code chooses it
     (src/inference/generic_transformer/moe_weights.rs:2118-2152): the expert-batched tiled
-    matmuls when there is at least a routed row per expert, else one mat-vec per routed pair."""
+    matmuls when there is at least a routed row per expert, else one mat-vec per routed pair.
+    `return_rows`: also the gated rows the second product read, in slot order (token * topk + choice)."""
     tokens, hidden = x.shape
     topk = choices.shape[1]
     if (moe_mmq_pays(tokens * topk, n_experts, wtype_gu if wtype_gu == wtype_down else None)
             and moe_mmq_serves(wtype_gu, hidden) and moe_mmq_serves(wtype_down, ffn)):
         plan = MmqRouting.from_choices(choices, n_experts)
         h = plan.gate_up_silu(wtype_gu, x, gate, up, ffn)
-        return plan.down_fold(wtype_down, h, down, hidden, topk_weights.reshape(-1))
+        out = plan.down_fold(wtype_down, h, down, hidden, topk_weights.reshape(-1))
+        if not return_rows:
+            return out
+        rows = torch.empty_like(h)
+        rows[plan.slots.long()] = h   # sorted order -> slot order
+        return out, rows
     routing = ExpertRouting(choices)
     h = moe_gemm_gguf_gate_up_silu_mul(wtype_gu, x.contiguous(), gate, up, routing, n_experts, ffn)
-    return moe_gemm_gguf_down_reduce(wtype_down, h, down, routing, topk_weights.reshape(-1), n_experts, hidden)
+    out = moe_gemm_gguf_down_reduce(wtype_down, h, down, routing, topk_weights.reshape(-1), n_experts, hidden)
+    return (out, h) if return_rows else out
 
 
 def moe_q4k_imma_m8_gate_up(x: torch.Tensor, gate_up: torch.Tensor, sorted_token_ids: torch.Tensor,

@@ -17,6 +17,7 @@ import pytest
 torch = pytest.importorskip("torch")
 
 import oracle
+from moe_block_check import check_block
 from loken_amd import lib, moe, ops, synth
 
 pytestmark = pytest.mark.gpu
@@ -94,19 +95,27 @@ def test_config3_expert_block_at_16_tokens_full_shape():
     down = synth.weight(Q4K, n_experts * hidden, ffn, seed=0, stream=3)
     x = synth.activation(tokens, hidden, seed=0) * np.float32(30.0)
     ids, w = oracle.topk_softmax(synth.activation(tokens, n_experts, seed=0, stream=7), topk)
-    want = oracle.moe_forward(1, Q4K, Q4K, x, gate, up, down, ids, w, n_experts, ffn)
-    scale = np.abs(want).max()
+    want, want_h = oracle.moe_forward(1, Q4K, Q4K, x, gate, up, down, ids, w, n_experts, ffn, want_h=True)
+    slots = oracle.group_by_expert(ids)[0]
+    want_slot = np.empty_like(want_h)
+    want_slot[slots] = want_h   # the oracle's gated rows are in sorted order; the checks read slot order
     gd, ud, dd, xd, wd = dev(gate), dev(up), dev(down), dev(x), dev(w.reshape(-1))
     # per routed pair (what the layer code picks at this load: one row per expert on average)
     routing = moe.ExpertRouting(dev(ids))
     h = moe.moe_gemm_gguf_gate_up_silu_mul(Q4K, xd, gd, ud, routing, n_experts, ffn)
+    assert (np.abs(h.cpu().numpy() - want_slot) <= 1e-3 * np.abs(want_slot) + 1e-4 * np.abs(want_slot).max()).all()
     out = moe.moe_gemm_gguf_down_reduce(Q4K, h, dd, routing, wd, n_experts, hidden).cpu().numpy()
-    assert (np.abs(out - want) <= 2e-3 * np.abs(want) + 2e-4 * scale).all()
+    # 1e-3 / 1e-4 with the oracle's second stage fed the card's own gated rows; end to end, anything
+    # outside that bound is attributed to a flipped Q8_1 code of those rows (tests/moe_block_check.py)
+    check_block(out, h.cpu().numpy(), want, want_slot, Q4K, down, ids, w, n_experts, hidden)
     # and the expert-batched tiles over the same routing
     plan = moe.MmqRouting.from_choices(dev(ids), n_experts)
     h2 = plan.gate_up_silu(Q4K, xd, gd, ud, ffn)
     out2 = plan.down_fold(Q4K, h2, dd, hidden, wd).cpu().numpy()
-    assert (np.abs(out2 - want) <= 2e-3 * np.abs(want) + 2e-4 * scale).all()
+    h2_slot = np.empty_like(want_h)
+    h2_slot[plan.slots.cpu().numpy()] = h2.cpu().numpy()
+    assert (np.abs(h2_slot - want_slot) <= 1e-3 * np.abs(want_slot) + 1e-4 * np.abs(want_slot).max()).all()
+    check_block(out2, h2_slot, want, want_slot, Q4K, down, ids, w, n_experts, hidden)
 
 
 # ---------------------------------------------------------------- config 4
