@@ -15,8 +15,12 @@ Distinct weights per layer, so the step is cache-cold by construction.
 Weights and activations are synthetic (seeded, generated on the device) and resident in HBM
 before the timed region.
 
-`value` = weight bytes of the step / time per step (the reference's mat-vec convention: weight
-bytes only, src/tensor/cuda/quant.rs:3905,3959-3961 of loken), whole job, one GPU.
+`value` = the figure the metric names: Q4_K weight bytes of the step / time of the step's Q4_K mat-vec
+launches (the reference's mat-vec convention: weight bytes only, src/tensor/cuda/quant.rs:3905,
+3959-3961 of loken), whole job, one GPU; it is the roofline leg's `achieved`. `ms_per_step` and
+`whole_step` are the whole step (Q4_K, Q6_K down, Q8_0 lm_head): EXACTLY `--steps` replays after
+`--warmup` untimed ones between two synchronizations, and, beside that, 200 replays after 20 warm-ups
+each between its own pair of events (median, p10, p90, min, max).
 
 Two more measurements ride in the same JSON line:
   roofline      the dominant kernel (Q4_K mat-vec): average launch duration over the step's own
@@ -24,7 +28,9 @@ Two more measurements ride in the same JSON line:
                 algorithmic weight bytes per launch and MI355X's 8 TB/s HBM peak.
   cpu_baseline  loken's served CPU decode path for Q4_K, restated (Q8_K activation, weights repacked
                 eight rows at a time, persistent worker pool), on a bounded sample of the same
-                workload, on this host's cores.
+                workload, on this host's cores, over copies that together exceed twice the host's
+                last-level cache (its size is printed); `legs` adds the served CPU prefill path on
+                configuration 2a and the expert block of configuration 3 on the pool.
   gemv_4096     the benchmark set's configuration 0 (Q4_K 4096 x 4096, one row) over rotating copies.
   mmq           configurations 2a / 2b, the tiled matmul, against the int8 matrix peak.
   rows-sweep    one --wtype q4_k|q6_k matrix (--rows-n x --cols-k) at 16..2048 rows: the matrix-unit
@@ -70,7 +76,8 @@ def parse_args():
                          "values are quantized by their own launch (every workgroup of a fused launch quantizes the "
                          "whole row), and rows from three rows on")
     ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="wall-clock budget of the CPU baseline sample")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0,
+                    help="wall-clock budget of the CPU baseline samples together (mat-vec 40 %, prefill 30 %, expert block 30 %)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--brief", action="store_true",
                     help="the decode step and its roofline leg only: no config 0, tiled-matmul or ceiling measurements")
@@ -104,13 +111,28 @@ def other_configs():
     import subprocess
 
     def child(flags):
-        r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--steps", "20", *flags],
-                           capture_output=True, text=True, timeout=300)
-        for ln in reversed(r.stdout.splitlines()):
-            if ln.startswith("{"):
-                d = json.loads(ln)
-                return {"ms_per_step": d["ms_per_step"], "value": d["value"], "unit": d["unit"]}
-        return {"error": (r.stderr or r.stdout)[-200:]}
+        # a child that hangs, dies or prints something else costs its own entry, never the parent's line
+        try:
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--steps", "20", *flags],
+                               capture_output=True, text=True, timeout=300)
+            for ln in reversed(r.stdout.splitlines()):
+                if ln.startswith("{"):
+                    d = json.loads(ln)
+                    out = {"ms_per_step": d["ms_per_step"], "value": d["value"], "unit": d["unit"]}
+                    if "whole_step" in d:
+                        out["whole_step_gbs"] = d["whole_step"]["gbs"]
+                        out["spread"] = d["whole_step"]["per_step"]
+                    for key in ("step_spread", "block_in_step_graph"):
+                        if key in d:
+                            out["spread"] = d[key]
+                    if d.get("roofline"):
+                        out["roofline"] = {k: d["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac") if k in d["roofline"]}
+                    return out
+            return {"error": (r.stderr or r.stdout)[-200:]}
+        except subprocess.TimeoutExpired:
+            return {"error": "child run exceeded 300 s and was ended"}
+        except (OSError, ValueError, KeyError) as e:
+            return {"error": f"{type(e).__name__}: {e}"[:200]}
 
     return {
         "llama3_8b_step_by_rows": {str(b): child(["--brief", "--batch", str(b)]) for b in (4, 8)},
@@ -419,12 +441,15 @@ def main() -> int:
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    value = total_bytes / (ms_per_step * 1e-3) / 1e9
+    step_gbs = total_bytes / (ms_per_step * 1e-3) / 1e9
+    from loken_amd import workloads as wl
+    # beside the K-step wall clock: 200 steps after 20 warm-ups, each between its own events
+    step_us = wl.time_launches(lambda i: step(), 200, warm=20)
 
     # ------------------------------------------------------------------ roofline leg
     # The step's own mix of Q4_K mat-vec launches, nothing else, recorded into one graph and
     # replayed between two events on the replaying stream (the stream the kernels run on).
-    reps = max(3, min(20, args.steps))
+    reps = 200
     run(q4k_plan)
     torch.cuda.synchronize()
     q4k_graph = None
@@ -440,17 +465,11 @@ def main() -> int:
         torch.cuda.synchronize()
         q4k_graph.replay()
         torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        if q4k_graph is not None:
-            q4k_graph.replay()
-        else:
-            run(q4k_plan)
-    e1.record()
-    torch.cuda.synchronize()
+    # 20 warm-up passes over the mix, then 200 timed ones, each between its own pair of events on the
+    # stream the kernels run on; the average launch duration is the mean over all of them
+    mix_us = wl.time_launches(lambda i: q4k_graph.replay() if q4k_graph is not None else run(q4k_plan), reps, warm=20) / len(q4k_plan)
     launches = reps * len(q4k_plan)
-    avg_us = e0.elapsed_time(e1) * 1e3 / launches
+    avg_us = float(mix_us.mean())
     bytes_per_launch = q4k_bytes / len(q4k_plan)
     achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -464,7 +483,9 @@ def main() -> int:
                                 "q4k_rows16_kernel<true,false,4,4> (gate+up)") if kind == "rows"
                           else f"mmvq_kernel<EngQ4K,{b},2,float>", "avg_launch_us": round(avg_us, 3),
                 "algorithmic_bytes_per_launch": int(bytes_per_launch), "launches_timed": launches,
-                "timed_as": "graph replay of the mix" if q4k_graph is not None else "eager launches"}
+                "per_launch": wl.spread(mix_us),
+                "timed_as": (f"{reps} graph replays of the mix of {len(q4k_plan)} launches, each replay between its own events; "
+                             f"per-launch figures are a replay's time over its launches") if q4k_graph is not None else "eager launches"}
     q4k_launch_bytes = sorted({int(a_bytes) for a_bytes in q4k_launch_sizes})
 
     # ------------------------------------------------------------------ the rest of the metric, and measured denominators
@@ -509,15 +530,20 @@ def main() -> int:
 
     line = {
         "metric": "Q4_K GEMV weight GB/s (% HBM peak); prefill MMQ int8 TOPS (% MFMA peak)",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "value": round(achieved, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"llama3-8b decode-step quantized linears (Q4_K q,k,v,o,gate,up; Q6_K down; "
                                f"Q8_0 lm_head), batch {b}, {args.layers} layers",
                    "launch_plan": args.plan if kind == args.plan else f"{args.plan} -> {kind}", "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
                    "hip_graph": used_graph},
-        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
-        "q4k_gemv_gbs": round(achieved, 1), "q4k_gemv_pct_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBS, 2),
+        "value_is": "Q4_K weight bytes of the step over the time of its Q4_K mat-vec launches (the roofline leg); "
+                    "ms_per_step and whole_step are the whole step, Q6_K and Q8_0 matrices included",
+        "pct_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBS, 2),
+        "whole_step": {"gbs": round(step_gbs, 1), "pct_hbm_peak": round(100.0 * step_gbs / HBM_PEAK_GBS, 2),
+                       "ms_per_step": round(ms_per_step, 4), "weight_bytes": total_bytes,
+                       "per_step": wl.spread(step_us),
+                       "gbs_at_median": round(total_bytes / float(__import__("numpy").median(step_us)) / 1e3, 1)},
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
@@ -536,12 +562,71 @@ def cpu_model():
     return "unknown"
 
 
+def host_last_level_cache():
+    """(bytes, domains) of the L3 slices the CPUs of this process's affinity set sit under, from sysfs;
+    (0, 0) when the host does not say."""
+    seen = {}
+    try:
+        cpus = sorted(os.sched_getaffinity(0))
+    except AttributeError:
+        cpus = list(range(os.cpu_count() or 1))
+    for c in cpus:
+        base = f"/sys/devices/system/cpu/cpu{c}/cache/index3/"
+        try:
+            shared = open(base + "shared_cpu_list").read().strip()
+            size = open(base + "size").read().strip()
+        except OSError:
+            continue
+        mult = {"K": 1 << 10, "M": 1 << 20, "G": 1 << 30}.get(size[-1:].upper(), 1)
+        seen[shared] = int(size.rstrip("KMGkmg")) * mult
+    return sum(seen.values()), len(seen)
+
+
+def rotating_copies(arr, llc_bytes, cap_bytes=3 << 30):
+    """Copies of `arr` that together exceed twice the last-level cache (512 MB assumed when the host
+    does not say), at least 2 and at most `cap_bytes` in all."""
+    want = 2 * (llc_bytes or (256 << 20)) + arr.nbytes
+    count = max(2, min(-(-want // arr.nbytes), max(2, cap_bytes // arr.nbytes)))
+    return [arr.copy() for _ in range(count)]
+
+
+def timed_calls(fn, copies, seconds):
+    """Calls `fn(copy)` over the copies in turn for about `seconds`; returns (calls, elapsed, per-call seconds)."""
+    import numpy as np
+    fn(copies[0])
+    per = []
+    t0 = time.perf_counter()
+    i = 0
+    while True:
+        a = time.perf_counter()
+        fn(copies[i % len(copies)])
+        bnow = time.perf_counter()
+        per.append(bnow - a)
+        i += 1
+        if bnow - t0 >= seconds and i >= 3:
+            break
+    return i, bnow - t0, np.array(per)
+
+
+def cpu_spread(per_s):
+    import numpy as np
+    us = per_s * 1e6
+    return {"median_us": round(float(np.median(us)), 1), "p10_us": round(float(np.percentile(us, 10)), 1),
+            "p90_us": round(float(np.percentile(us, 90)), 1), "min_us": round(float(us.min()), 1),
+            "max_us": round(float(us.max()), 1), "calls": int(us.size)}
+
+
 def cpu_baseline(args, torch, synth, lib, w_dev, out_dev, x_dev, b):
-    """loken's served CPU path for Q4_K decode, restated (oracle/cpu_baseline.c): Q8_K activation,
-    weights repacked eight rows at a time, one group dot per eight columns, on a persistent pool of
-    one worker per physical core of this process's CPU set (or OMP_NUM_THREADS when the host sets
-    it: the GPU box gives a job a share of its cores). Layer 0's q_proj-shaped sample, rotating
-    copies past the last-level cache."""
+    """loken's served CPU paths, restated (oracle/cpu_baseline.c), on a persistent pool of one worker
+    per physical core of this process's CPU set (or OMP_NUM_THREADS when the host sets it: the GPU
+    box gives a job a share of its cores):
+      * decode: Q8_K activation, weights repacked eight rows at a time, one group dot per eight
+        columns, on layer 0's q_proj-shaped sample (the headline leg);
+      * prefill (configuration 2a, 512 rows x 4096 -> 14336 Q4_K): the tiled driver over the same
+        repacked weights (matmul_q4k_repacked_tiled, src/tensor/quant_cpu/drivers.rs:231-339);
+      * the expert block of configuration 3 (128 experts 2048 -> 768 -> 2048 Q4_K, top-8, 256 tokens):
+        the scalar oracle's block with the tokens spread over the pool.
+    Every leg rotates copies of its weights that together exceed twice the host's last-level cache."""
     import numpy as np
 
     import oracle
@@ -549,6 +634,8 @@ def cpu_baseline(args, torch, synth, lib, w_dev, out_dev, x_dev, b):
     physical, logical = oracle.cpu_counts()
     asked = int(os.environ.get("OMP_NUM_THREADS", "0"))
     threads = oracle.pool_start(min(asked, physical) if asked > 0 else 0)
+    llc, llc_domains = host_last_level_cache()
+    budget = max(args.cpu_seconds, 1.0)
     n, k = HIDDEN, HIDDEN
     w = w_dev.cpu().numpy()
     x = x_dev.cpu().numpy()
@@ -557,27 +644,77 @@ def cpu_baseline(args, torch, synth, lib, w_dev, out_dev, x_dev, b):
     got = out_dev.cpu().numpy()
     ok = bool((np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-4).all())
     x8 = oracle.repack_q4k_x8(w, n, k)
-    served_ok = bool((np.abs(oracle.oa_matmul_q4k_x8(x, x8, n) - oracle.oa_matmul(oracle.Q4_K, x, w, n))
-                      <= 1e-3 * np.maximum(np.abs(oracle.oa_matmul(oracle.Q4_K, x, w, n)), 1.0)).all())
-    # working set past the last-level cache: 32 distinct copies = 302 MB
-    copies = [x8.copy() for _ in range(32)]
-    oracle.oa_matmul_q4k_x8(x, copies[0], n)
-    t0 = time.perf_counter()
-    calls = 0
-    while time.perf_counter() - t0 < args.cpu_seconds:
-        for c in copies:
-            oracle.oa_matmul_q4k_x8(x, c, n)
-            calls += 1
-    dt = time.perf_counter() - t0
-    gbs = calls * synth.weight_bytes(lib.TYPE_Q4_K, n, k) / dt / 1e9
+    scalar = oracle.oa_matmul(oracle.Q4_K, x, w, n)
+    served_ok = bool((np.abs(oracle.oa_matmul_q4k_x8(x, x8, n) - scalar) <= 1e-3 * np.maximum(np.abs(scalar), 1.0)).all())
+    copies = rotating_copies(x8, llc)
+    calls, dt, per = timed_calls(lambda c: oracle.oa_matmul_q4k_x8(x, c, n), copies, 0.4 * budget)
+    nbytes = synth.weight_bytes(lib.TYPE_Q4_K, n, k)
+    gbs = calls * nbytes / dt / 1e9
+    rotated = len(copies) * x8.nbytes
+    del copies
+    legs = {}
+
+    # ---- prefill, configuration 2a
+    m2, k2, n2 = 512, 4096, 14336
+    w2 = synth.weight(lib.TYPE_Q4_K, 256, k2, seed=1).reshape(256, -1)
+    w2 = np.ascontiguousarray(np.tile(w2, (n2 // 256, 1)))          # a few generated rows repeated
+    x2 = synth.activation(m2, k2, seed=1)
+    x82 = oracle.repack_q4k_x8(w2, n2, k2)
+    sample = oracle.oa_matmul_q4k_x8_tiled(x2[:8], x82[:(256 // 8) * (k2 // 256) * 1152], 256)
+    ref2 = oracle.oa_matmul(oracle.Q4_K, x2[:8], w2[:256], 256)
+    tiled_ok = bool((np.abs(sample - ref2) <= 1e-3 * np.maximum(np.abs(ref2), 1.0)).all())
+    copies = rotating_copies(x82, llc)
+    calls2, dt2, per2 = timed_calls(lambda c: oracle.oa_matmul_q4k_x8_tiled(x2, c, n2), copies, 0.3 * budget)
+    ops2 = 2.0 * m2 * k2 * n2
+    legs["prefill_2a"] = {"value": round(calls2 * ops2 / dt2 / 1e12, 3), "unit": "TOP/s", "cores": threads, "kind": "port",
+                          "per_call": cpu_spread(per2), "rotated_bytes": len(copies) * x82.nbytes,
+                          "tiled_path_vs_scalar_oracle": "ok" if tiled_ok else "FAILED",
+                          "sample": f"tiled matmul {m2} rows x {k2} -> {n2} Q4_K, {calls2} calls ({dt2:.1f} s): Q8_K rows quantized on "
+                                    f"the pool, one chunk per eight columns, rows in tiles of eight (loken's served CPU prefill "
+                                    f"path, restated in C with AVX2)"}
+    del copies, x82, w2
+
+    # ---- the expert block of configuration 3
+    experts, hidden, ffn, topk, tokens = 128, 2048, 768, 8, 256
+    rng = np.random.default_rng(3)
+
+    def stack(rows, cols, stream):
+        base = synth.weight(lib.TYPE_Q4_K, 256, cols, seed=3, stream=stream).reshape(256, -1)
+        return np.ascontiguousarray(np.tile(base, (rows // 256, 1))).reshape(-1)
+    gate, up, down = stack(experts * ffn, hidden, 1), stack(experts * ffn, hidden, 2), stack(experts * hidden, ffn, 3)
+    xm = synth.activation(tokens, hidden, seed=3)
+    ids = np.stack([rng.permutation(experts)[:topk] for _ in range(tokens)]).astype(np.int32)
+    wts = rng.random((tokens, topk)).astype(np.float32)
+    wts /= wts.sum(axis=1, keepdims=True)
+    block = np.concatenate([gate, up, down])
+    g_end, u_end = gate.size, gate.size + up.size
+    copies = rotating_copies(block, llc)
+    del gate, up, down
+
+    def run_block(c):
+        return oracle.moe_forward_pool(0, oracle.Q4_K, oracle.Q4_K, xm, c[:g_end], c[g_end:u_end], c[u_end:], ids, wts, experts, ffn)
+    calls3, dt3, per3 = timed_calls(run_block, copies, 0.3 * budget)
+    ops3 = 6.0 * tokens * topk * ffn * hidden
+    legs["moe_block_256_tokens"] = {"value": round(calls3 * block.nbytes / dt3 / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+                                    "tops": round(calls3 * ops3 / dt3 / 1e12, 4), "per_call": cpu_spread(per3),
+                                    "rotated_bytes": len(copies) * block.nbytes,
+                                    "sample": f"expert block, {experts} experts {hidden} -> {ffn} -> {hidden} Q4_K, top-{topk}, {tokens} tokens, "
+                                              f"{calls3} calls ({dt3:.1f} s): the scalar block per routed pair (gate and up dots over "
+                                              f"Q8_K rows, SiLU, down dot, weighted sum), chunks of tokens on the pool"}
+    del copies, block
+    oracle.pool_start(1)   # joins the workers: no thread of the pool outlives the measurement
     return {"value": round(gbs, 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "cpu_model": cpu_model(), "physical_cores": physical, "logical_cpus": logical,
+            "last_level_cache_bytes": llc, "last_level_cache_domains": llc_domains, "rotated_bytes": rotated,
             "threads_source": "OMP_NUM_THREADS" if asked > 0 else "one per physical core",
-            "sample": f"Q4_K mat-vec {n}x{k}, batch {b}, {calls} calls over 32 rotating copies of the repacked weights "
-                      f"({dt:.1f} s): Q8_K activation, eight-row repacked weights, group dot per eight columns "
-                      f"(loken's served decode path, restated in C with AVX2), persistent pool of {threads} threads",
+            "per_call": cpu_spread(per),
+            "sample": f"Q4_K mat-vec {n}x{k}, batch {b}, {calls} calls over {rotated // x8.nbytes} rotating copies of the repacked weights "
+                      f"({rotated / 1e6:.0f} MB against {llc / 1e6:.0f} MB of last-level cache; {dt:.1f} s): Q8_K activation, eight-row "
+                      f"repacked weights, group dot per eight columns (loken's served decode path, restated in C with AVX2), "
+                      f"persistent pool of {threads} threads",
             "served_path_vs_scalar_oracle": "ok" if served_ok else "FAILED",
-            "gpu_parity_on_sample": "ok" if ok else "FAILED"}
+            "gpu_parity_on_sample": "ok" if ok else "FAILED",
+            "legs": legs}
 
 
 if __name__ == "__main__":

@@ -177,7 +177,7 @@ def gemv(args, dev):
             check(L.lk_mmvq(wtype, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, b, q.shape[1], n,
                             None, 0, s2), "lk_mmvq")
 
-    us = time_replays(capture(all_copies), max(10, args.launches // n_copies)) / n_copies
+    us = time_replays(capture(all_copies), max(20, -(-args.launches // n_copies))) / n_copies
     med = float(np.median(us))
     value = nbytes / med / 1e3
     roofline = {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -254,10 +254,10 @@ def gemv_4096(args, dev):
              "call_two_launches": dict(spread(two), gbs_median=round(gbs(float(np.median(two))), 1)),
              "call_fused_one_launch": dict(spread(one), gbs_median=round(gbs(float(np.median(one))), 1)),
              "back_to_back_us_per_launch": round(stream_us, 3), "back_to_back_gbs": round(gbs(stream_us), 1),
-             "graph_of_64_rotating_launches": {"us_per_launch_median": round(float(np.median(graph_us)), 3),
-                                               "gbs_median": round(gbs(float(np.median(graph_us))), 1)},
-             "graph_of_64_fused_launches": {"us_per_launch_median": round(float(np.median(graph_fused_us)), 3),
-                                            "gbs_median": round(gbs(float(np.median(graph_fused_us))), 1)},
+             "graph_of_64_rotating_launches": dict(spread(graph_us), us_per_launch_median=round(float(np.median(graph_us)), 3),
+                                                   gbs_median=round(gbs(float(np.median(graph_us))), 1), launches=50 * 64),
+             "graph_of_64_fused_launches": dict(spread(graph_fused_us), us_per_launch_median=round(float(np.median(graph_fused_us)), 3),
+                                                gbs_median=round(gbs(float(np.median(graph_fused_us))), 1), launches=50 * 64),
              "note": "per-launch event pairs and back-to-back eager launches are bounded by the host's launch cost; "
                      "the graph figures are the GPU-side rate, cache-cold (604 MB of rotating copies)"}
     g_med = float(np.median(graph_us))
@@ -309,7 +309,8 @@ def mmq(args, dev):
     # the weight operand), so that unit's dense peak prices it; the int8 fraction is kept beside
     # it because the target is quoted on the int8 peak.
     if wtype == Q4K:
-        kernel, peak, dtype = "q4k_f16_dense_kernel", F16_PEAK_TFLOPS, "f16 operands (exact integers), f32 accumulate"
+        kernel = "q4k_wide_dense_kernel (+ q4k_tokens_f16_kernel once per call)" if m > 128 else "q4k_f16_dense_kernel"
+        peak, dtype = F16_PEAK_TFLOPS, "f16 operands (exact integers), f32 accumulate"
     elif wtype == Q6K:
         kernel, peak, dtype = "mmq_dense_kernel<MmqQ6K,128,1>", INT8_PEAK_TOPS, "int8"
     else:
@@ -399,21 +400,35 @@ def moe_block(args, dev):
     distinct = float(np.mean([int((torch.bincount(c.reshape(-1).to(torch.int64), minlength=experts) > 0).sum())
                               for c in layer_choices]))   # experts a layer's block reads, mean over the layers
     one_matrix = synth.weight_bytes(wt, ffn, hidden)
+    # Both floors of the block: the bytes of the experts it reads at the HBM peak, and its multiply-adds
+    # at the int8 matrix peak. The larger one binds (at 256 tokens every expert is read: 340 MB is
+    # 42 us at 8 TB/s against 4 us of matrix work), and the block is reported against that one.
+    nbytes = 3 * one_matrix * distinct
+    op_count = 6.0 * pairs * ffn * hidden
+    hbm_floor_us, mfma_floor_us = nbytes / HBM_PEAK_GBS / 1e3, op_count / INT8_PEAK_TOPS / 1e6
+    gbs, tops = nbytes / med / 1e3, op_count / med / 1e6
     if tiled:
-        op_count = 6.0 * pairs * ffn * hidden
-        value, unit = op_count / med / 1e6, "TOP/s"
-        roofline = {"bound": "mfma", "achieved": round(value, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                    "frac": round(value / INT8_PEAK_TOPS, 4), "traffic": None,
-                    "kernel": f"q4k_rows_moe_kernel, {name}" if rows_launch else f"mmq_moe_kernel, {name}",
-                    "note": "whole expert block (quantize, two grouped matmuls with the activation in the first, fold)"
-                            if rows_launch else "whole expert block (plan, route, quantize, two grouped matmuls, activation, fold)"}
+        kernel = f"q4k_rows_moe_kernel, {name}" if rows_launch else f"mmq_moe_kernel, {name}"
+        note = ("whole expert block (quantize, two grouped matmuls with the activation in the first, fold)" if rows_launch
+                else "whole expert block (plan, route, quantize, two grouped matmuls, activation, fold)")
     else:
-        nbytes = 3 * one_matrix * distinct
-        value, unit = nbytes / med / 1e3, "GB/s"
-        roofline = {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None, "kernel": f"moe_rows_kernel / moe_rows_legacy_kernel, {name}",
-                    "note": "whole expert block (quantize, gate/up pairs, down pairs, weighted sum); bytes = 3 matrices "
-                            "per distinct expert hit"}
+        kernel = f"moe_rows_kernel / moe_rows_legacy_kernel, {name}"
+        note = "whole expert block (quantize, gate/up pairs, down pairs, weighted sum)"
+    note += "; bytes = 3 matrices per distinct expert read, ops = 6 x pairs x ffn x hidden"
+    if hbm_floor_us >= mfma_floor_us:
+        value, unit = gbs, "GB/s"
+        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "kernel": kernel, "note": note,
+                    "algorithmic_bytes_per_launch": int(nbytes), "avg_launch_us": round(float(us.mean()), 3),
+                    "other_floor": {"bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                                    "frac": round(tops / INT8_PEAK_TOPS, 4)}}
+    else:
+        value, unit = tops, "TOP/s"
+        roofline = {"bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                    "frac": round(tops / INT8_PEAK_TOPS, 4), "traffic": None, "kernel": kernel, "note": note,
+                    "algorithmic_ops_per_launch": int(op_count), "avg_launch_us": round(float(us.mean()), 3),
+                    "other_floor": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                    "frac": round(gbs / HBM_PEAK_GBS, 4)}}
     extra = {"block_in_step_graph": dict(spread(us), blocks_per_graph=layers), "block_graph_replay": spread(single),
              "block_eager_from_python": spread(eager), "path": ("expert-batched rows on the matrix unit" if rows_launch else "expert-batched tiled matmul") if tiled else "mat-vec per routed pair",
              "routed_pairs": pairs, "distinct_experts": distinct,
@@ -614,15 +629,9 @@ def decode_1p7b(args, dev):
         with torch.cuda.graph(graph, stream=side):
             run(cap)
     torch.cuda.synchronize()
-    import time
-    for _ in range(args.warmup):
-        graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        graph.replay()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    # at least 20 warm-up replays and 200 timed ones, each replay between its own pair of events
+    us = time_replays(graph, max(200, args.steps), warm=max(20, args.warmup))
+    ms = float(np.median(us)) * 1e-3
     value = total_bytes / (ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(value / HBM_PEAK_GBS, 4), "traffic": None,
@@ -636,11 +645,12 @@ def decode_1p7b(args, dev):
                               "the Q8_1 rows down reads, down, lm_head; a Q8_1 quantizer launch before the others" if fused_rows
                          else f"linears on the matrix-unit rows kernels: {used['rows']}, as mat-vec slices of eight rows: "
                               f"{used['matvec']}, on the tiled matmul: {used['tiled']}",
-                 "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline)
+                 "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline,
+                {"step_spread": spread(us), "ms_per_step_is": "median of the timed replays"})
 
 
 # ---------------------------------------------------------------------------- short forms for the default line
-def brief_gemv_4096(launches=64, replays=30):
+def brief_gemv_4096(launches=64, replays=50):
     """Config 0 for the default benchmark line: the Q4_K 4096 x 4096 mat-vec at one row as a graph of
     `launches` launches over that many rotating copies (604 MB at 64: past twice the last-level
     cache), from a Q8_1 row and from the f32 row quantized in the kernel."""
@@ -671,17 +681,19 @@ def brief_gemv_4096(launches=64, replays=30):
             check(L.lk_mmvq_fused(Q4K, 1, vx, x.data_ptr(), x.stride(0), dst, lib.TYPE_F32, k, nn, 1, n, None, s2),
                   "lk_mmvq_fused")
 
-    us = float(np.median(time_replays(capture(plain), replays))) / launches
-    us_fused = float(np.median(time_replays(capture(fused), replays))) / launches
-    want = None
+    all_us = time_replays(capture(plain), replays) / launches
+    all_fused = time_replays(capture(fused), replays) / launches
+    us, us_fused = float(np.median(all_us)), float(np.median(all_fused))
     return {"workload": "Q4_K 4096x4096 mat-vec, one row, seed 0, graph of %d launches over %d rotating copies" % (launches, launches),
             "weight_bytes": nbytes, "us_per_launch": round(us, 3), "gbs": round(nbytes / us / 1e3, 1),
             "frac_of_8tbs": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+            "per_launch": dict(spread(all_us), launches=replays * launches),
             "f32_activation_quantized_in_kernel": {"us_per_launch": round(us_fused, 3),
-                                                   "gbs": round(nbytes / us_fused / 1e3, 1)}}
+                                                   "gbs": round(nbytes / us_fused / 1e3, 1),
+                                                   "per_launch": dict(spread(all_fused), launches=replays * launches)}}
 
 
-def brief_mmq(shape, launches=30):
+def brief_mmq(shape, launches=200):
     """Configs 2a / 2b for the default benchmark line: median of event-bracketed launches of the tiled
     matmul alone and of quantizer + matmul."""
     L = lib.load()
@@ -706,12 +718,14 @@ def brief_mmq(shape, launches=30):
                     info["cc"], info["nsm"], info["smpbo"], info["warp_size"], s) == 0:
             raise lib.LokenError(ops.MMQ_LAUNCHER[wtype], lib.LK_ERR_ARG)
 
-    mm = float(np.median(time_launches(lambda i: matmul(), launches, warm=5)))
-    both = float(np.median(time_launches(lambda i: (quant(), matmul()), launches, warm=5)))
+    mm_all = time_launches(lambda i: matmul(), launches)
+    both_all = time_launches(lambda i: (quant(), matmul()), launches)
+    mm, both = float(np.median(mm_all)), float(np.median(both_all))
     op_count = 2.0 * m * k * n
     return {"workload": f"tiled matmul {m} rows x {k} -> {n}, {NAMES[wtype]}", "ops": int(op_count),
-            "kernel": "q4k_f16_dense_kernel (exact integers on f16 operands)" if wtype == Q4K else "mmq_dense_kernel<MmqQ6K,128,1>",
-            "matmul_us": round(mm, 2), "tops": round(op_count / mm / 1e6, 1),
+            "kernel": "q4k_wide_dense_kernel after q4k_tokens_f16_kernel (exact integers on f16 operands)" if wtype == Q4K else "mmq_dense_kernel<MmqQ6K,128,1>",
+            "matmul_us": round(mm, 2), "tops": round(op_count / mm / 1e6, 1), "matmul_launch": spread(mm_all),
+            "call_two_launches": spread(both_all),
             "frac_of_int8_peak": round(op_count / mm / 1e6 / INT8_PEAK_TOPS, 4),
             "quantize_plus_matmul_us": round(both, 2), "tops_with_quantizer": round(op_count / both / 1e6, 1)}
 
@@ -755,8 +769,8 @@ def rows_sweep(args, dev):
             check(L.lk_quantize_q8_1(x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, m, s), "lk_quantize_q8_1")
             check(rows_fn(w.data_ptr(), q.data_ptr(), out.data_ptr(), m, n, k, s), "rows kernel")
 
-        t_tiled = float(np.median(time_replays(capture(tiled), 12, warm=3)))
-        t_rows = float(np.median(time_replays(capture(rows), 12, warm=3)))
+        t_tiled = float(np.median(time_replays(capture(tiled), args.launches)))
+        t_rows = float(np.median(time_replays(capture(rows), args.launches)))
         check(L.lkh_qkernel_matmul_forward(handle, x.data_ptr(), lib.TYPE_F32, m, out.data_ptr(),
                                            torch.cuda.current_stream().cuda_stream, 0), "lkh_qkernel_matmul_forward")
         table.append({"rows": m, "rows_kernel_us": round(t_rows, 1), "tiled_us": round(t_tiled, 1),

@@ -84,6 +84,13 @@ def _declare(l: C.CDLL) -> None:
     l.lko_repack_q4k_x8.argtypes = [_vp, _sz, _sz, _vp]
     l.lko_repack_q4k_x8.restype = None
     l.oa_matmul_q4k_x8.argtypes = [_sz, _sz, _sz, _vp, _vp, _vp]
+    l.oa_matmul_q4k_x8_tiled.argtypes = [_sz, _sz, _sz, _vp, _vp, _vp]
+    l.lko_repack_q6k_x8.argtypes = [_vp, _sz, _sz, _vp]
+    l.lko_repack_q6k_x8.restype = None
+    l.oa_matmul_q6k_x8_tiled.argtypes = [_sz, _sz, _sz, _vp, _vp, _vp]
+    l.lko_gemv_group_q6k_x8_scalar.argtypes = [_vp, _vp, _sz, _vp]
+    l.lko_gemv_group_q6k_x8_scalar.restype = None
+    l.lko_moe_forward_pool.argtypes = [_i, _i, _i, _sz, _sz, _sz, _sz, _sz] + [_vp] * 7
     l.lko_inv_rms_wide.restype = C.c_float
     l.lko_inv_rms_wide.argtypes = [_vp, _sz, C.c_float]
     l.lko_norm_rows.restype = None
@@ -251,6 +258,57 @@ def oa_matmul_q4k_x8(lhs, x8: np.ndarray, n: int) -> np.ndarray:
     dst = np.empty((m, n), np.float32)
     _check(lib().oa_matmul_q4k_x8(m, k, n, _p(lhs), _p(x8), _p(dst)))
     return dst
+
+
+def oa_matmul_q4k_x8_tiled(lhs, x8: np.ndarray, n: int) -> np.ndarray:
+    """The served Q4_K prefill path: one pool chunk per eight columns, rows in tiles of eight."""
+    lhs = _f32(lhs)
+    m, k = lhs.shape
+    dst = np.empty((m, n), np.float32)
+    _check(lib().oa_matmul_q4k_x8_tiled(m, k, n, _p(lhs), _p(x8), _p(dst)))
+    return dst
+
+
+def repack_q6k_x8(rhs, n: int, k: int) -> np.ndarray:
+    """Q6_K rows `[n, k/256]` (n a multiple of 8) -> eight-row group blocks of 1680 bytes."""
+    rhs = _u8(rhs)
+    nb = k // 256
+    out = np.empty((n // 8) * nb * 1680, np.uint8)
+    lib().lko_repack_q6k_x8(_p(rhs), n, nb, _p(out))
+    return out
+
+
+def oa_matmul_q6k_x8_tiled(lhs, x8: np.ndarray, n: int) -> np.ndarray:
+    """The served Q6_K prefill path over repacked weights."""
+    lhs = _f32(lhs)
+    m, k = lhs.shape
+    dst = np.empty((m, n), np.float32)
+    _check(lib().oa_matmul_q6k_x8_tiled(m, k, n, _p(lhs), _p(x8), _p(dst)))
+    return dst
+
+
+def gemv_group_q6k_x8_scalar(x8: np.ndarray, group: int, nb: int, act_q8k: np.ndarray) -> np.ndarray:
+    """Scalar group dot of group `group` against one Q8_K row (`nb` blocks of 292 bytes)."""
+    x8 = _u8(x8)
+    act_q8k = _u8(act_q8k)
+    out = np.empty(8, np.float32)
+    grp = np.ascontiguousarray(x8.reshape(-1)[group * nb * 1680:(group + 1) * nb * 1680])
+    lib().lko_gemv_group_q6k_x8_scalar(_p(grp), _p(act_q8k), nb, _p(out))
+    return out
+
+
+def moe_forward_pool(family: int, dt_gu: int, dt_down: int, x, gate, up, down, ids, weights,
+                     n_experts: int, ffn: int) -> np.ndarray:
+    """`moe_forward` with the tokens spread over the worker pool."""
+    x = _f32(x)
+    tokens, hidden = x.shape
+    ids = np.ascontiguousarray(ids, np.int32)
+    weights = _f32(weights)
+    gate, up, down = _u8(gate), _u8(up), _u8(down)
+    out = np.empty((tokens, hidden), np.float32)
+    _check(lib().lko_moe_forward_pool(family, dt_gu, dt_down, tokens, hidden, ffn, n_experts, ids.shape[1],
+                                      _p(x), _p(gate), _p(up), _p(down), _p(ids), _p(weights), _p(out)))
+    return out
 
 
 def pool_start(threads: int = 0) -> int:

@@ -13,9 +13,12 @@
  * only by float summation order; tests hold it to the reference's own vector-vs-scalar bound
  * 1e-3 * max(|ref|, 1) (avx/parity.rs:50-56).
  *
- * Two drivers: the per-column dot above for every format (oa_matmul_fast), and the path loken
- * actually serves Q4_K with (oa_matmul_q4k_x8): rows repacked eight at a time and one group dot per
- * eight output columns. Both run on ONE persistent pool of workers (no thread is created per call).
+ * Drivers: the per-column dot above for every format (oa_matmul_fast); the path loken actually
+ * serves Q4_K decode with (oa_matmul_q4k_x8): rows repacked eight at a time and one group dot per
+ * eight output columns; and the prefill forms over the same repacked weights, one pool chunk per
+ * column group with the rows in tiles of eight (oa_matmul_q4k_x8_tiled, oa_matmul_q6k_x8_tiled:
+ * matmul_q4k_repacked_tiled / matmul_q6k_repacked_tiled, drivers.rs:231-406). All run on ONE
+ * persistent pool of workers (no thread is created per call).
  *
  * Falls back to the scalar oracle when the CPU lacks AVX2.
  */
@@ -259,6 +262,7 @@ typedef struct {
     int workers;                 /* threads beside the caller */
     atomic_uint generation;      /* bumped once per job */
     atomic_size_t next, done;    /* next chunk to grab; chunks finished */
+    atomic_int active;           /* workers inside pool_drain: a job's state is not reused while one is */
     size_t n_chunks;
     chunk_fn fn;
     void* ctx;
@@ -299,8 +303,13 @@ static void* pool_worker(void* arg) {
             pthread_mutex_unlock(&p->mu);
         }
         if (atomic_load(&p->stop)) return NULL;
+        /* Entering is announced BEFORE the generation is read: pool_run bumps the generation and then
+         * waits for `active` to fall to zero, so either it sees this worker and waits for it, or this
+         * worker sees the new generation's state whole. */
+        atomic_fetch_add(&p->active, 1);
         seen = atomic_load(&p->generation);
         pool_drain(p);
+        atomic_fetch_sub(&p->active, 1);
     }
 }
 
@@ -382,6 +391,10 @@ static void pool_run(size_t n_chunks, chunk_fn fn, void* ctx) {
     }
     pool_drain(p);
     while (atomic_load_explicit(&p->done, memory_order_acquire) < n_chunks) _mm_pause();
+    /* A worker that woke late may still be inside pool_drain (its grab found no chunk left, or it is
+     * about to look): the next job's fn / ctx / counters are written only once nobody is in there,
+     * so a stale grab can never be compared against the next job's chunk count. */
+    while (atomic_load_explicit(&p->active, memory_order_acquire) != 0) _mm_pause();
 }
 
 /* ---------------------------------------------------------------------------------------------
@@ -580,4 +593,235 @@ int oa_matmul_fast(int dtype, size_t m, size_t k, size_t n, const float* lhs,
     pool_run(job.n_chunks, column_chunk, &job);
     free(act);
     return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * The served prefill path: matmul_q4k_repacked_tiled (drivers.rs:231-339). The activation rows
+ * are quantized to Q8_K in parallel over rows (quantize_act_q8k, :179-205), then ONE pool chunk
+ * per group of eight columns computes all m rows of its columns, rows in tiles of eight. Inside a
+ * tile the reference accumulates one row at a time and decodes the weight nibbles again per row
+ * (its comment at :252-259: holding eight rows' partials spills); each row's eight sums are the
+ * decode path's group dot, so the tile is that dot called per row and the result of a row does
+ * not depend on m (the tests hold the driver to that, bit for bit).
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+    size_t k, nb;
+    const float* lhs;
+    uint8_t* act;
+} quant_job_t;
+
+static void quant_row_chunk(void* ctx, size_t r) {
+    const quant_job_t* j = (const quant_job_t*)ctx;
+    lko_quantize_q8_k(j->lhs + r * j->k, j->k, j->act + r * j->nb * LKO_Q8K_BYTES);
+}
+
+static void x8_tiled_chunk(void* ctx, size_t g) {
+    const x8_job_t* j = (const x8_job_t*)ctx;
+    const uint8_t* grp = j->x8 + g * j->nb * LKO_Q4KX8_BYTES;
+    for (size_t r = 0; r < j->m; r += 8) {
+        const size_t mt = j->m - r < 8 ? j->m - r : 8;
+        float local[64];
+        for (size_t t = 0; t < mt; ++t) gemv_group_q4k_x8(grp, j->act + (r + t) * j->nb * LKO_Q8K_BYTES, j->nb, local + 8 * t);
+        for (size_t t = 0; t < mt; ++t) memcpy(j->dst + (r + t) * j->n + g * 8, local + 8 * t, 8 * sizeof(float));
+    }
+}
+
+int oa_matmul_q4k_x8_tiled(size_t m, size_t k, size_t n, const float* lhs, const uint8_t* x8, float* dst) {
+    if (k % LKO_QK_K != 0) return -1;
+    if (n % 8 != 0) return -4;
+    if (!lko_cpu_has_avx2()) return -3;
+    (void)lko_pool_start(g_pool_threads > 0 ? g_pool_threads : 0);
+    x8_job_t job;
+    job.m = m; job.n = n; job.nb = k / LKO_QK_K; job.groups = n / 8; job.x8 = x8; job.dst = dst; job.chunk = 1;
+    uint8_t* act = (uint8_t*)malloc(job.nb * LKO_Q8K_BYTES * (m ? m : 1));
+    if (!act) return -5;
+    quant_job_t qj = {k, job.nb, lhs, act};
+    pool_run(m, quant_row_chunk, &qj);
+    job.act = act;
+    pool_run(job.groups, x8_tiled_chunk, &job);
+    free(act);
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Q6_K repacked eight rows at a time (BlockQ6Kx8, repack_q6k.rs:17-64: the planes are copied per
+ * column, nothing is re-laid) and its prefill driver matmul_q6k_repacked_tiled (drivers.rs:
+ * 341-406). Group block: 8 f16 d, 8 x 16 int8 scales, 8 x 128 bytes ql, 8 x 64 bytes qh.
+ * The group dot follows gemm_group_avx2 (repack_q6k.rs:139-212): a column's 256 codes are decoded
+ * ONCE per tile as unsigned 0..63, meet every row of the tile, and the zero point 32 comes off per
+ * row as 32 * sum_g scale_g * bsum_g from the Q8_K row's sums of sixteen. Integers exact:
+ *   out[r][j] += d_j * act_r.d * (sum_g scale_jg * dot_jg(unsigned) - 32 * sum_g scale_jg * bsum_rg)
+ * ------------------------------------------------------------------------------------------- */
+#define LKO_Q6KX8_BYTES (16 + 128 + 1024 + 512)
+
+void lko_repack_q6k_x8(const uint8_t* rhs, size_t n, size_t nb, uint8_t* out) {
+    for (size_t g = 0; g < n / 8; ++g)
+        for (size_t b = 0; b < nb; ++b) {
+            uint8_t* dst = out + (g * nb + b) * LKO_Q6KX8_BYTES;
+            for (size_t j = 0; j < 8; ++j) {
+                /* a Q6_K block: ql[128], qh[64], scales[16], d */
+                const uint8_t* src = rhs + ((g * 8 + j) * nb + b) * LKO_Q6K_BYTES;
+                memcpy(dst + 2 * j, src + 208, 2);
+                memcpy(dst + 16 + 16 * j, src + 192, 16);
+                memcpy(dst + 144 + 128 * j, src, 128);
+                memcpy(dst + 1168 + 64 * j, src + 128, 64);
+            }
+        }
+}
+
+/* One group's `nb` blocks against `mt` (1..8) Q8_K rows: out[r * 8 + j], added to. */
+static void gemm_group_q6k_x8(const uint8_t* grp, const uint8_t* const* rows, size_t mt, size_t nb, float* out) {
+    const __m256i m4 = _mm256_set1_epi8(0xF), m2 = _mm256_set1_epi8(3);
+    for (size_t l = 0; l < nb; ++l) {
+        const uint8_t* blk = grp + l * LKO_Q6KX8_BYTES;
+        for (int j = 0; j < 8; ++j) {
+            const uint8_t* qlp = blk + 144 + 128 * j;
+            const uint8_t* qhp = blk + 1168 + 64 * j;
+            const int8_t* scp = (const int8_t*)(blk + 16 + 16 * j);
+            __m256i wdec[8];
+            for (int half = 0; half < 2; ++half) {
+                const __m256i ql1 = _mm256_loadu_si256((const __m256i*)(qlp + 64 * half));
+                const __m256i ql2 = _mm256_loadu_si256((const __m256i*)(qlp + 64 * half + 32));
+                const __m256i qh = _mm256_loadu_si256((const __m256i*)(qhp + 32 * half));
+                const __m256i h0 = _mm256_slli_epi16(_mm256_and_si256(qh, m2), 4);
+                const __m256i h1 = _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(qh, 2), m2), 4);
+                const __m256i h2 = _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(qh, 4), m2), 4);
+                const __m256i h3 = _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(qh, 6), m2), 4);
+                wdec[4 * half + 0] = _mm256_or_si256(_mm256_and_si256(ql1, m4), h0);
+                wdec[4 * half + 1] = _mm256_or_si256(_mm256_and_si256(ql2, m4), h1);
+                wdec[4 * half + 2] = _mm256_or_si256(_mm256_and_si256(_mm256_srli_epi16(ql1, 4), m4), h2);
+                wdec[4 * half + 3] = _mm256_or_si256(_mm256_and_si256(_mm256_srli_epi16(ql2, 4), m4), h3);
+            }
+            /* chunk c of 32 codes spans the groups 2c (low sixteen) and 2c + 1 (high sixteen) */
+            __m256i sv[8];
+            for (int c = 0; c < 8; ++c)
+                sv[c] = _mm256_insertf128_si256(_mm256_castsi128_si256(_mm_set1_epi16(scp[2 * c])), _mm_set1_epi16(scp[2 * c + 1]), 1);
+            const __m256i scales16 = _mm256_cvtepi8_epi16(_mm_loadu_si128((const __m128i*)scp));
+            const float dj = f16_to_f32_hw(rd16(blk + 2 * j));
+            for (size_t r = 0; r < mt; ++r) {
+                const uint8_t* yb = rows[r] + l * LKO_Q8K_BYTES;
+                float yd;
+                memcpy(&yd, yb, 4);
+                const int8_t* q8 = (const int8_t*)(yb + 4);
+                __m256i sumi = _mm256_setzero_si256();
+                for (int c = 0; c < 8; ++c) {
+                    const __m256i q = _mm256_loadu_si256((const __m256i*)(q8 + 32 * c));
+                    sumi = _mm256_add_epi32(sumi, _mm256_madd_epi16(_mm256_maddubs_epi16(wdec[c], q), sv[c]));
+                }
+                const __m256i bsums = _mm256_loadu_si256((const __m256i*)(yb + 260));
+                const __m256i corr = _mm256_slli_epi32(_mm256_madd_epi16(bsums, scales16), 5);
+                const int32_t s = hsum_i32_8(_mm256_sub_epi32(sumi, corr));
+                out[r * 8 + j] += dj * yd * (float)s;
+            }
+        }
+    }
+}
+
+typedef struct {
+    size_t m, n, nb;
+    const uint8_t* x8;
+    const uint8_t* act;
+    float* dst;
+} q6x8_job_t;
+
+static void q6x8_tiled_chunk(void* ctx, size_t g) {
+    const q6x8_job_t* j = (const q6x8_job_t*)ctx;
+    const uint8_t* grp = j->x8 + g * j->nb * LKO_Q6KX8_BYTES;
+    for (size_t r = 0; r < j->m; r += 8) {
+        const size_t mt = j->m - r < 8 ? j->m - r : 8;
+        const uint8_t* rows[8];
+        for (size_t t = 0; t < mt; ++t) rows[t] = j->act + (r + t) * j->nb * LKO_Q8K_BYTES;
+        float local[64];
+        memset(local, 0, sizeof local);
+        gemm_group_q6k_x8(grp, rows, mt, j->nb, local);
+        for (size_t t = 0; t < mt; ++t) memcpy(j->dst + (r + t) * j->n + g * 8, local + 8 * t, 8 * sizeof(float));
+    }
+}
+
+int oa_matmul_q6k_x8_tiled(size_t m, size_t k, size_t n, const float* lhs, const uint8_t* x8, float* dst) {
+    if (k % LKO_QK_K != 0) return -1;
+    if (n % 8 != 0) return -4;
+    if (!lko_cpu_has_avx2()) return -3;
+    (void)lko_pool_start(g_pool_threads > 0 ? g_pool_threads : 0);
+    q6x8_job_t job;
+    job.m = m; job.n = n; job.nb = k / LKO_QK_K; job.x8 = x8; job.dst = dst;
+    uint8_t* act = (uint8_t*)malloc(job.nb * LKO_Q8K_BYTES * (m ? m : 1));
+    if (!act) return -5;
+    quant_job_t qj = {k, job.nb, lhs, act};
+    pool_run(m, quant_row_chunk, &qj);
+    job.act = act;
+    pool_run(n / 8, q6x8_tiled_chunk, &job);
+    free(act);
+    return 0;
+}
+
+/* The scalar statement of the Q6_K group dot (gemv_group_scalar, repack_q6k.rs:96-123: "THE ORACLE"):
+ * signed codes, one float fold per block and column. */
+void lko_gemv_group_q6k_x8_scalar(const uint8_t* grp, const uint8_t* y, size_t nb, float out[8]) {
+    float sumf[8] = {0};
+    for (size_t l = 0; l < nb; ++l) {
+        const uint8_t* blk = grp + l * LKO_Q6KX8_BYTES;
+        const uint8_t* yb = y + l * LKO_Q8K_BYTES;
+        float yd;
+        memcpy(&yd, yb, 4);
+        const int8_t* a = (const int8_t*)(yb + 4);
+        for (int j = 0; j < 8; ++j) {
+            const uint8_t* ql = blk + 144 + 128 * j;
+            const uint8_t* qh = blk + 1168 + 64 * j;
+            const int8_t* sc = (const int8_t*)(blk + 16 + 16 * j);
+            int8_t aux[256];
+            for (int jj = 0; jj < 256; jj += 128) {
+                const uint8_t* q4 = ql + jj / 2;
+                const uint8_t* qhh = qh + jj / 4;
+                for (int e = 0; e < 32; ++e) {
+                    aux[jj + e] = (int8_t)((int)((q4[e] & 0xF) | ((qhh[e] & 3) << 4)) - 32);
+                    aux[jj + e + 32] = (int8_t)((int)((q4[e + 32] & 0xF) | (((qhh[e] >> 2) & 3) << 4)) - 32);
+                    aux[jj + e + 64] = (int8_t)((int)((q4[e] >> 4) | (((qhh[e] >> 4) & 3) << 4)) - 32);
+                    aux[jj + e + 96] = (int8_t)((int)((q4[e + 32] >> 4) | (((qhh[e] >> 6) & 3) << 4)) - 32);
+                }
+            }
+            int32_t sumi = 0;
+            for (int g = 0; g < 16; ++g) {
+                int32_t gs = 0;
+                for (int e = 0; e < 16; ++e) gs += (int32_t)aux[16 * g + e] * (int32_t)a[16 * g + e];
+                sumi += (int32_t)sc[g] * gs;
+            }
+            sumf[j] += f16_to_f32_hw(rd16(blk + 2 * j)) * yd * (float)sumi;
+        }
+    }
+    memcpy(out, sumf, sizeof sumf);
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * The MoE block on the pool: the scalar oracle's block (lko_moe_forward) over chunks of tokens, a
+ * token's result depending on its own routed pairs only. The timed CPU figure beside the card's.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct {
+    int family, dt_gu, dt_down, rc;
+    size_t tokens, hidden, ffn, n_experts, topk, per;
+    const float* x;
+    const uint8_t *gate, *up, *down;
+    const int32_t* ids;
+    const float* weights;
+    float* out;
+} moe_job_t;
+
+static void moe_chunk(void* ctx, size_t c) {
+    moe_job_t* j = (moe_job_t*)ctx;
+    const size_t t0 = c * j->per, t1 = t0 + j->per < j->tokens ? t0 + j->per : j->tokens;
+    const int rc = lko_moe_forward(j->family, j->dt_gu, j->dt_down, t1 - t0, j->hidden, j->ffn, j->n_experts, j->topk,
+                                   j->x + t0 * j->hidden, j->gate, j->up, j->down, j->ids + t0 * j->topk,
+                                   j->weights + t0 * j->topk, NULL, j->out + t0 * j->hidden);
+    if (rc) j->rc = rc;
+}
+
+int lko_moe_forward_pool(int family, int dt_gu, int dt_down, size_t tokens, size_t hidden, size_t ffn, size_t n_experts,
+                         size_t topk, const float* x, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+                         const int32_t* ids, const float* weights, float* out) {
+    const int threads = lko_pool_start(g_pool_threads > 0 ? g_pool_threads : 0);
+    moe_job_t job = {family, dt_gu, dt_down, 0, tokens, hidden, ffn, n_experts, topk, 1, x, gate, up, down, ids, weights, out};
+    job.per = (tokens + (size_t)threads * 4 - 1) / ((size_t)threads * 4);
+    if (job.per < 1) job.per = 1;
+    pool_run((tokens + job.per - 1) / job.per, moe_chunk, &job);
+    return job.rc;
 }

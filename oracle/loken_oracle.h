@@ -168,6 +168,17 @@ int lko_logical_cpus(void);
 void lko_repack_q4k_x8(const uint8_t* rhs, size_t n, size_t nb, uint8_t* out);
 /* The served Q4_K path over the repacked weights (matmul_q4k_plain_pre, drivers.rs:61-95). */
 int oa_matmul_q4k_x8(size_t m, size_t k, size_t n, const float* lhs, const uint8_t* x8, float* dst);
+/* The served prefill forms over repacked weights (matmul_q4k_repacked_tiled / matmul_q6k_repacked_tiled,
+ * src/tensor/quant_cpu/drivers.rs:231-406): one pool chunk per group of eight columns, rows in tiles of
+ * eight; and the Q6_K repack (repack_q6k.rs:41-64) with its scalar group dot (:96-123). Same returns. */
+int oa_matmul_q4k_x8_tiled(size_t m, size_t k, size_t n, const float* lhs, const uint8_t* x8, float* dst);
+void lko_repack_q6k_x8(const uint8_t* rhs, size_t n, size_t nb, uint8_t* out);
+int oa_matmul_q6k_x8_tiled(size_t m, size_t k, size_t n, const float* lhs, const uint8_t* x8, float* dst);
+void lko_gemv_group_q6k_x8_scalar(const uint8_t* grp, const uint8_t* y, size_t nb, float out[8]);
+/* lko_moe_forward over chunks of tokens on the pool (the timed CPU figure beside the card's block). */
+int lko_moe_forward_pool(int family, int dt_gu, int dt_down, size_t tokens, size_t hidden, size_t ffn, size_t n_experts,
+                         size_t topk, const float* x, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+                         const int32_t* ids, const float* weights, float* out);
 int oa_matmul_fast(int dtype, size_t m, size_t k, size_t n, const float* lhs,
                    const uint8_t* rhs, size_t rhs_bytes, float* dst, int threads);
 
