@@ -90,7 +90,7 @@ def parse_args():
     ap.add_argument("--shape", choices=["2a", "2b"], default="2a", help="--workload mmq: 512x4096->14336 Q4_K or 2048x14336->4096 Q6_K")
     ap.add_argument("--mmq-wtype", default=None, help="--workload mmq: the shape in another format of the tiled matmul "
                     "(q8_0 q4_0 q4_1 q5_0 q5_1 q2_k q3_k q5_k)")
-    ap.add_argument("--wtype", default="q4_0", help="--workload gemv: q4_0 q4_1 q5_0 q5_1 iq4_nl mxfp4 q8_0 q2_k q3_k q4_k q5_k q6_k iq4_xs")
+    ap.add_argument("--wtype", default="q4_0", help="--workload gemv: q4_0 q4_1 q5_0 q5_1 iq4_nl mxfp4 q8_0 q2_k q3_k q4_k q5_k q6_k iq4_xs iq2_xxs iq3_xxs iq3_s iq2_s q2_0")
     ap.add_argument("--rows-n", type=int, default=14336, help="--workload gemv: weight rows")
     ap.add_argument("--cols-k", type=int, default=4096, help="--workload gemv: values per row")
     ap.add_argument("--tokens", type=int, default=256, help="--workload moe: rows through the expert block")

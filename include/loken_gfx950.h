@@ -41,10 +41,15 @@ extern "C" {
 #define LK_TYPE_Q4_K 12
 #define LK_TYPE_Q5_K 13
 #define LK_TYPE_Q6_K 14
+#define LK_TYPE_IQ2_XXS 16
+#define LK_TYPE_IQ3_XXS 18
 #define LK_TYPE_IQ4_NL 20
+#define LK_TYPE_IQ3_S 21
+#define LK_TYPE_IQ2_S 22
 #define LK_TYPE_IQ4_XS 23
 #define LK_TYPE_BF16 30
 #define LK_TYPE_MXFP4 39
+#define LK_TYPE_Q2_0 42
 
 #define LK_OK 0
 #define LK_ERR_ARG 1        /* a size, stride or pointer the kernels cannot take */
@@ -79,7 +84,9 @@ int lk_quantize_q8_1(const void* x, int x_type, void* vy, int kx, int kx_padded,
 
 /* dst[j, row] = weight row `row` . activation row j, j < batch (1..8).
  *   wtype          LK_TYPE_Q4_K | LK_TYPE_Q5_K | LK_TYPE_Q6_K | LK_TYPE_Q8_0, and (this launcher and
- *                  lk_mmvq_subdots only) the 32-value nibble formats LK_TYPE_Q4_0 | Q4_1 | Q5_0 | Q5_1 | IQ4_NL | MXFP4 and Q2_K | Q3_K | IQ4_XS
+ *                  lk_mmvq_subdots only) the 32-value nibble formats LK_TYPE_Q4_0 | Q4_1 | Q5_0 | Q5_1 | IQ4_NL | MXFP4, Q2_K | Q3_K | IQ4_XS
+ *                  and the codebook formats IQ2_XXS | IQ3_XXS | IQ3_S | IQ2_S | Q2_0 (lk_mmvq_subdots: two integers per run
+ *                  of 32 values, its halves)
  *   vx             nrows_x rows of ncols_x / block_len blocks (Q4_K / Q5_K 16-byte aligned, Q2_K / IQ4_XS
  *                  4-byte, MXFP4 any address, every other format 2-byte; else LK_ERR_ARG)
  *   vy_q8_1        batch rows of Q8_1 blocks, `stride_col_y` blocks apart (k_padded / 32)
@@ -383,6 +390,27 @@ int launch_mmq_moe_gguf_iq4_xs(const void* x, const void* x_second, int64_t dst_
                                int n_experts, int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc,
                                int64_t smpbo, int warp_size, void* stream);
 
+/* The codebook formats only mixtures store: IQ3_XXS (98-byte blocks), IQ3_S (110), IQ2_S (82), all of 256
+ * values, and Q2_0 (18 bytes, 64 values, stride_row_x in those blocks); weights 2-byte aligned. Replaces
+ * launch_mmq_moe_gguf_{iq3_xxs,iq3_s,iq2_s,q2_0} (src/tensor/quantized/mmq.rs:335-343; kernels
+ * cuda/mmq_gguf/mmq_instance_iq3_xxs.cu and siblings, dequantizers cuda/moe/gguf_iq.cuh:126-196). */
+int launch_mmq_moe_gguf_iq3_xxs(const void* x, const void* x_second, int64_t dst_second, const void* y,
+        void* dst, const int* expert_bounds, const int* ids_dst, int64_t stride_expert_x, int64_t ncols_x,
+        int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, int n_experts,
+        int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc, int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_iq3_s(const void* x, const void* x_second, int64_t dst_second, const void* y,
+        void* dst, const int* expert_bounds, const int* ids_dst, int64_t stride_expert_x, int64_t ncols_x,
+        int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, int n_experts,
+        int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc, int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_iq2_s(const void* x, const void* x_second, int64_t dst_second, const void* y,
+        void* dst, const int* expert_bounds, const int* ids_dst, int64_t stride_expert_x, int64_t ncols_x,
+        int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, int n_experts,
+        int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc, int64_t smpbo, int warp_size, void* stream);
+int launch_mmq_moe_gguf_q2_0(const void* x, const void* x_second, int64_t dst_second, const void* y,
+        void* dst, const int* expert_bounds, const int* ids_dst, int64_t stride_expert_x, int64_t ncols_x,
+        int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, int n_experts,
+        int64_t ncols_max, int64_t ncols_hint, int mmq_x, int cc, int64_t smpbo, int warp_size, void* stream);
+
 /* Replaces launch_mmq_moe_gguf_q2_k (src/tensor/quantized/mmq.rs:280). */
 int launch_mmq_moe_gguf_q2_k(const void* x, const void* x_second, int64_t dst_second, const void* y,
                              void* dst, const int* expert_bounds, const int* ids_dst,
@@ -421,7 +449,8 @@ void loken_moe_mmq_fold(const float* pairs, const float* weights, const int32_t*
  * (token * topk + choice) slot of routed pair i, expert_ids[i] its expert; size_m = pairs,
  * size_n = output rows per expert, size_k = reduction length; quant_type is loken's wire id
  * (0 = Q8_0, 1 = Q4_K, 2 = Q2_K, 3 = Q3_K, 4 = Q5_K, 5 = Q6_K, 6 = Q5_0, 7 = MXFP4, 8 = Q5_1, 9 = IQ4_NL,
- * 10 = IQ4_XS; the codebook formats 11..15 return LK_ERR_TYPE). Weights are stacks [num_experts][size_n][size_k / block].
+ * 10 = IQ4_XS, 11 = IQ3_XXS, 12 = IQ3_S, 13 = IQ2_S, 14 = Q2_0, 15 = IQ2_XXS: src/inference/moe_cuda/gemm.rs:23-39).
+ * Weights are stacks [num_experts][size_n][size_k / block].
  * These launchers quantize the f32 activation themselves into a per-(device, stream)
  * grow-only scratch (the one allocation in this library; growing is refused with
  * LK_ERR_NOMEM while the stream is being captured). Return 0 or an LK_ERR_* code.

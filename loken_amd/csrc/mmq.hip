@@ -27,6 +27,7 @@
 
 #include "mmq_problem.h"
 #include "legacy_blocks.h"
+#include "codebook_blocks.h"
 
 #include <cstdlib>
 
@@ -533,6 +534,58 @@ struct MmqIq4Xs {
     }
 };
 
+// The codebook formats of the expert tables (IQ3_XXS, IQ3_S, IQ2_S, Q2_0; codebook_blocks.h): a run of 32
+// values decodes to int8 weights under an odd integer scale times the block's float, so the tiles take them
+// as they take IQ4_XS; IQ2_S scales its halves apart and takes Q6_K's shape of two scales per sub-block. A
+// thread takes (row, run) items; Q2_0's blocks of 64 values go four to a step.
+template <int ID>
+struct MmqCodebook {
+    using C = codebook::Fmt<ID>;
+    static constexpr int ALIGN = 2;
+    static constexpr int BLOCK_BYTES = C::BYTES;
+    static constexpr int NS = ID == 22 ? 16 : 8;
+    static constexpr bool HAS_MIN = false;
+    static constexpr int MIN_RANK = 0;
+    static constexpr bool F16_TILES = false;
+    static constexpr int BLOCKS_PER_STEP = 8 / C::RUNS;
+    static constexpr int PER = TN * 8 / MMQ_WG;
+
+    struct Frag {
+        codebook::Raw raw[PER];
+    };
+    static __device__ __forceinline__ void fetch(Frag& f, const uint8_t* __restrict__ w, int64_t nb, int kb,
+                                                 int n0, int n) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, j = idx & 7;
+            const int gn = min(n0 + row, n - 1);
+            const uint8_t* bp = w + ((int64_t)gn * nb + (int64_t)kb * BLOCKS_PER_STEP + j / C::RUNS) * BLOCK_BYTES;
+            f.raw[i] = codebook::fetch<ID>(bp, j % C::RUNS);
+        }
+    }
+    static __device__ __forceinline__ void commit(const Frag& f, int n0, int n, int8_t* wq, float* wsc, float* wmn) {
+        (void)wmn;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = threadIdx.x + i * MMQ_WG, row = idx >> 3, j = idx & 7;
+            const codebook::Run r = codebook::decode<ID>(f.raw[i], j % C::RUNS);
+            *(uint4*)(wq + (j * TN + row) * 32) = r.lo;
+            *(uint4*)(wq + (j * TN + row) * 32 + 16) = r.hi;
+            const float d = n0 + row < n ? r.d : 0.f;
+            if (NS == 16) {
+                wsc[(2 * j) * TN + row] = d * (float)r.sc0;
+                wsc[(2 * j + 1) * TN + row] = d * (float)r.sc1;
+            } else {
+                wsc[j * TN + row] = d * (float)r.sc0;
+            }
+        }
+    }
+};
+using MmqIq3Xxs = MmqCodebook<18>;
+using MmqIq3S = MmqCodebook<21>;
+using MmqIq2S = MmqCodebook<22>;
+using MmqQ2_0 = MmqCodebook<42>;
+
 // Token rows [m0, m0+TM) of block kb (record layout above). Rows at or past m_end read as zeros.
 // S16: the weight format has a minimum per 16 values (Q2_K), so the sums are formed per chunk of 16
 // codes from the codes themselves (the record holds them per 32) and each chunk's thread reads its scale.
@@ -1037,3 +1090,7 @@ LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_mxfp4, MmqMxfp4)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q3_k, MmqQ3K)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq4_xs, MmqIq4Xs)
 LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q2_k, MmqQ2K)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq3_xxs, MmqIq3Xxs)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq3_s, MmqIq3S)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_iq2_s, MmqIq2S)
+LK_MMQ_MOE_ENTRY(launch_mmq_moe_gguf_q2_0, MmqQ2_0)

@@ -28,6 +28,7 @@
 // table; the kernels are plain statements without the register pipelines of the K-quant engines.
 
 #include "legacy_blocks.h"
+#include "codebook_blocks.h"
 
 namespace {
 
@@ -152,6 +153,15 @@ __global__ __launch_bounds__(64) void subdots_legacy_kernel(const uint8_t* __res
 // j = bytes 16 j .. + 16 of qs as IQ4_NL levels (low nibbles values 0..15, high 16..31), one
 // six-bit scale less 32 for the run.
 // ---------------------------------------------------------------------------------------------
+// Bytes of a block and runs of 32 values in it, by ggml type id: Q2_K, Q3_K, IQ4_XS and the codebook formats
+// (IQ2_XXS 16, IQ3_XXS 18, IQ3_S 21, IQ2_S 22, Q2_0 42: codebook_blocks.h), which ride the same kernels: a run
+// decodes to 32 int8 weights, an odd integer scale per half and the block's float.
+template <int ID> struct Lowbit { static constexpr int BYTES = codebook::Fmt<ID>::BYTES, RUNS = codebook::Fmt<ID>::RUNS; };
+template <> struct Lowbit<10> { static constexpr int BYTES = 84, RUNS = 8; };
+template <> struct Lowbit<11> { static constexpr int BYTES = 110, RUNS = 8; };
+template <> struct Lowbit<23> { static constexpr int BYTES = 136, RUNS = 8; };
+static constexpr bool is_lowbit(int id) { return id == 10 || id == 11 || id == 23 || codebook::is_codebook(id); }
+
 struct LowbitBlock {
     uint4 lo, hi;         // the block's codes 0..3, values 0..15 and 16..31
     uint4 nlo, nhi;       // Q3_K: 1 where the high bit is clear
@@ -178,6 +188,18 @@ static __device__ __forceinline__ void load_run32(const uint8_t* p, uint4& lo, u
 template <int ID>
 static __device__ __forceinline__ LowbitBlock lowbit_block(const uint8_t* __restrict__ bp, int j) {
     LowbitBlock r;
+    if constexpr (codebook::is_codebook(ID)) {
+        const codebook::Run run = codebook::decode<ID>(codebook::fetch<ID>(bp, j), j);
+        r.lo = run.lo;
+        r.hi = run.hi;
+        r.sc0 = run.sc0;
+        r.sc1 = run.sc1;
+        r.mn0 = r.mn1 = 0;
+        r.d = run.d;
+        r.dmin = 0.f;
+        r.nlo = r.nhi = make_uint4(0, 0, 0, 0);
+        return r;
+    }
     if (ID == 23) {
         const uint4 q = *(const uint4_a4*)(bp + 8 + 16 * j);
         r.lo = make_uint4(levels_of<1>(q.x & 0x0F0F0F0Fu), levels_of<1>(q.y & 0x0F0F0F0Fu), levels_of<1>(q.z & 0x0F0F0F0Fu),
@@ -261,11 +283,11 @@ template <int ID, int B, typename T, bool STAGED>
 __global__ __launch_bounds__(LWG) void mmvq_lowbit_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
                                                           T* __restrict__ dst, const float* __restrict__ bias, int nb, int n,
                                                           int stride_col_y, int stride_col_dst) {
-    constexpr int BYTES = ID == 10 ? 84 : ID == 11 ? 110 : 136;
+    constexpr int BYTES = Lowbit<ID>::BYTES, RUNS = Lowbit<ID>::RUNS;
     extern __shared__ __align__(16) uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int k32 = nb * 8;
+    const int k32 = nb * RUNS;
     if (STAGED) stage_acts(lds, vy, B, k32, stride_col_y);
     for (int row = blockIdx.x * LWAVES + wave; row < n; row += gridDim.x * LWAVES) {
         const uint8_t* wrow = vx + (size_t)row * nb * BYTES;
@@ -273,7 +295,7 @@ __global__ __launch_bounds__(LWG) void mmvq_lowbit_kernel(const uint8_t* __restr
 #pragma unroll
         for (int c = 0; c < B; ++c) acc[c] = 0.f;
         for (int idx = lane; idx < k32; idx += 64) {
-            const LowbitBlock w = lowbit_block<ID>(wrow + (size_t)(idx >> 3) * BYTES, idx & 7);
+            const LowbitBlock w = lowbit_block<ID>(wrow + (size_t)(idx / RUNS) * BYTES, idx % RUNS);
 #pragma unroll
             for (int c = 0; c < B; ++c)
                 acc[c] += lowbit_share<ID>(w, act_block<STAGED>(lds, vy, B * k32, k32, stride_col_y, c, idx));
@@ -289,17 +311,17 @@ __global__ __launch_bounds__(LWG) void mmvq_lowbit_kernel(const uint8_t* __restr
 template <int ID>
 __global__ __launch_bounds__(64) void subdots_lowbit_kernel(const uint8_t* __restrict__ vx, const uint8_t* __restrict__ vy,
                                                             int32_t* __restrict__ dots, int nb) {
-    constexpr int BYTES = ID == 10 ? 84 : ID == 11 ? 110 : 136;
+    constexpr int BYTES = Lowbit<ID>::BYTES, RUNS = Lowbit<ID>::RUNS;
     const int row = blockIdx.y, idx = blockIdx.x * 64 + threadIdx.x;
-    if (idx >= nb * 8) return;
-    const LowbitBlock w = lowbit_block<ID>(vx + ((size_t)row * nb + (idx >> 3)) * BYTES, idx & 7);
+    if (idx >= nb * RUNS) return;
+    const LowbitBlock w = lowbit_block<ID>(vx + ((size_t)row * nb + (idx / RUNS)) * BYTES, idx % RUNS);
     int dot0, dot1;
     lowbit_dots<ID>(w, act_from_memory(vy + (size_t)idx * Q81_BYTES), dot0, dot1);
     if (ID == 23) {   // one integer per run of 32
         dots[(size_t)row * nb * 8 + idx] = dot0 + dot1;
         return;
     }
-    int32_t* out = dots + (size_t)row * nb * 16 + 2 * idx;
+    int32_t* out = dots + (size_t)row * nb * 2 * RUNS + 2 * idx;
     out[0] = dot0;
     out[1] = dot1;
 }
@@ -325,10 +347,10 @@ template <int ID>
 static __device__ __forceinline__ float staged_row_share(const uint8_t* __restrict__ wrow, int nb, const uint8_t* lds,
                                                          int k32, int lane) {
     float acc = 0.f;
-    if constexpr (ID == 10 || ID == 11 || ID == 23) {
-        constexpr int BYTES = ID == 10 ? 84 : ID == 11 ? 110 : 136;
+    if constexpr (is_lowbit(ID)) {
+        constexpr int BYTES = Lowbit<ID>::BYTES, RUNS = Lowbit<ID>::RUNS;
         for (int idx = lane; idx < k32; idx += 64) {
-            const LowbitBlock w = lowbit_block<ID>(wrow + (size_t)(idx >> 3) * BYTES, idx & 7);
+            const LowbitBlock w = lowbit_block<ID>(wrow + (size_t)(idx / RUNS) * BYTES, idx % RUNS);
             acc += lowbit_share<ID>(w, act_block<true>(lds, nullptr, k32, k32, 0, 0, idx));
         }
     } else {
@@ -348,10 +370,8 @@ static __device__ __forceinline__ float staged_row_share(const uint8_t* __restri
     return acc;
 }
 
-template <int ID> struct BytesOf { static constexpr int V = Legacy<ID>::BYTES; };
-template <> struct BytesOf<10> { static constexpr int V = 84; };
-template <> struct BytesOf<11> { static constexpr int V = 110; };
-template <> struct BytesOf<23> { static constexpr int V = 136; };
+template <int ID, bool LOW = is_lowbit(ID)> struct BytesOf { static constexpr int V = Legacy<ID>::BYTES, RUNS = 1; };
+template <int ID> struct BytesOf<ID, true> { static constexpr int V = Lowbit<ID>::BYTES, RUNS = Lowbit<ID>::RUNS; };
 
 template <int ID, int MODE>
 __global__ __launch_bounds__(LWG) void moe_rows_legacy_kernel(const uint8_t* __restrict__ w0, const uint8_t* __restrict__ w1,
@@ -405,8 +425,7 @@ __global__ __launch_bounds__(LWG) void moe_rows_legacy_kernel(const uint8_t* __r
 template <int ID>
 static int launch_moe(int mode, const uint8_t* w0, const uint8_t* w1, const uint8_t* acts, const int32_t* sti,
                       const int32_t* eid, const float* tw, const float* bias, float* out, MoeLegacyDims d, hipStream_t s) {
-    constexpr bool LOWBIT = ID == 10 || ID == 11 || ID == 23;
-    d.k32 = LOWBIT ? d.nb * 8 : d.nb;
+    d.k32 = d.nb * BytesOf<ID>::RUNS;
     d.slab_bytes = (int64_t)d.slab_rows * d.nb * BytesOf<ID>::V;
     const size_t lds_bytes = (size_t)d.k32 * ACT_LDS_PER_BLOCK;
     if (lds_bytes > 48 * 1024 || d.pairs > 65535) return LK_ERR_ARG;
@@ -431,8 +450,8 @@ static int launch(const void* vx, const void* vy, void* dst, const float* bias, 
                   int stride_col_dst, hipStream_t s) {
     const int need = (n + LWAVES - 1) / LWAVES, cap = lk_device().cus * 8;
     const dim3 grid(need < cap ? need : cap);
-    constexpr bool LOWBIT = ID == 10 || ID == 11 || ID == 23;
-    const int k32 = LOWBIT ? nb * 8 : nb;
+    constexpr bool LOWBIT = is_lowbit(ID);
+    const int k32 = nb * BytesOf<ID>::RUNS;
     const size_t lds_bytes = (size_t)B * k32 * ACT_LDS_PER_BLOCK;
     const auto run = [&](auto kernel, size_t lds) {
         hipLaunchKernelGGL(kernel, grid, dim3(LWG), lds, s, (const uint8_t*)vx, (const uint8_t*)vy, (T*)dst, bias, nb, n,
@@ -482,14 +501,15 @@ static int by_type(int dst_type, int batch, const void* vx, const void* vy, void
 bool lk_is_legacy_type(int wtype) {
     return wtype == LK_TYPE_Q4_0 || wtype == LK_TYPE_Q4_1 || wtype == LK_TYPE_Q5_0 || wtype == LK_TYPE_Q5_1 ||
            wtype == LK_TYPE_IQ4_NL || wtype == LK_TYPE_MXFP4 || wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K ||
-           wtype == LK_TYPE_IQ4_XS;
+           wtype == LK_TYPE_IQ4_XS || codebook::is_codebook(wtype);
 }
 
 // lk_mmvq for the 32-value nibble formats (the caller has told them apart with lk_is_legacy_type).
 int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, int dst_type, int ncols_x, int nrows_x,
                    int batch, int stride_col_y, int stride_col_dst, const float* bias, hipStream_t s) {
     if (nrows_x == 0) return LK_OK;
-    const int block_len = wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K || wtype == LK_TYPE_IQ4_XS ? 256 : 32;
+    const int block_len = wtype == LK_TYPE_Q2_0 ? 64
+                          : wtype == LK_TYPE_Q2_K || wtype == LK_TYPE_Q3_K || wtype == LK_TYPE_IQ4_XS || codebook::is_codebook(wtype) ? 256 : 32;
     if (!vx || !vy_q8_1 || !dst || ncols_x <= 0 || ncols_x % block_len != 0 || nrows_x < 0) return LK_ERR_ARG;
     if (batch < 1 || batch > 8 || stride_col_y < ncols_x / 32 || stride_col_dst < nrows_x) return LK_ERR_ARG;
     if ((wtype != LK_TYPE_MXFP4 && ((uintptr_t)vx & 1) != 0) || ((uintptr_t)vy_q8_1 & 3) != 0) return LK_ERR_ARG;
@@ -500,6 +520,11 @@ int lk_mmvq_legacy(int wtype, const void* vx, const void* vy_q8_1, void* dst, in
         case LK_TYPE_Q2_K: return by_type<10>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q3_K: return by_type<11>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_IQ4_XS: return by_type<23>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_IQ2_XXS: return by_type<16>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_IQ3_XXS: return by_type<18>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_IQ3_S: return by_type<21>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_IQ2_S: return by_type<22>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
+        case LK_TYPE_Q2_0: return by_type<42>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q4_0: return by_type<2>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q4_1: return by_type<3>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
         case LK_TYPE_Q5_0: return by_type<6>(dst_type, batch, vx, vy_q8_1, dst, bias, nb, nrows_x, stride_col_y, stride_col_dst, s);
@@ -524,6 +549,21 @@ int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32
         else hipLaunchKernelGGL(subdots_lowbit_kernel<23>, gridk, dim3(64), 0, s, w, y, dots, nbk);
         return lk_launch_status();
     }
+    if (codebook::is_codebook(wtype)) {
+        // two integers per run of 32: its halves
+        const int len = wtype == LK_TYPE_Q2_0 ? 64 : 256;
+        if (ncols_x % len != 0 || ((uintptr_t)vx & 1) != 0) return LK_ERR_ARG;
+        const int nbc = ncols_x / len;
+        const dim3 gridc((ncols_x / 32 + 63) / 64, nrows_x);
+        switch (wtype) {
+            case LK_TYPE_IQ2_XXS: hipLaunchKernelGGL(subdots_lowbit_kernel<16>, gridc, dim3(64), 0, s, w, y, dots, nbc); break;
+            case LK_TYPE_IQ3_XXS: hipLaunchKernelGGL(subdots_lowbit_kernel<18>, gridc, dim3(64), 0, s, w, y, dots, nbc); break;
+            case LK_TYPE_IQ3_S: hipLaunchKernelGGL(subdots_lowbit_kernel<21>, gridc, dim3(64), 0, s, w, y, dots, nbc); break;
+            case LK_TYPE_IQ2_S: hipLaunchKernelGGL(subdots_lowbit_kernel<22>, gridc, dim3(64), 0, s, w, y, dots, nbc); break;
+            default: hipLaunchKernelGGL(subdots_lowbit_kernel<42>, gridc, dim3(64), 0, s, w, y, dots, nbc); break;
+        }
+        return lk_launch_status();
+    }
     const int nb = ncols_x / 32;
     const dim3 grid((nb + 63) / 64, nrows_x);
     switch (wtype) {
@@ -542,6 +582,8 @@ int lk_mmvq_subdots_legacy(int wtype, const void* vx, const void* vy_q8_1, int32
 int lk_moe_wire_block_len_legacy(int quant_type) {
     switch (quant_type) {
         case 2: case 3: case 10: return 256;       // Q2_K, Q3_K, IQ4_XS
+        case 11: case 12: case 13: case 15: return 256;   // IQ3_XXS, IQ3_S, IQ2_S, IQ2_XXS
+        case 14: return 64;                        // Q2_0
         case 6: case 7: case 8: case 9: return 32; // Q5_0, MXFP4, Q5_1, IQ4_NL
         default: return 0;
     }
@@ -566,6 +608,11 @@ int lk_moe_rows_legacy(int mode, int quant_type, const uint8_t* w0, const uint8_
         case 7: return launch_moe<39>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
         case 8: return launch_moe<7>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
         case 9: return launch_moe<20>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 11: return launch_moe<18>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 12: return launch_moe<21>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 13: return launch_moe<22>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 14: return launch_moe<42>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
+        case 15: return launch_moe<16>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
         default: return launch_moe<23>(mode, w0, w1, acts_q8_1, sorted_token_ids, expert_ids, topk_weights, down_bias, out, d, s);
     }
 }

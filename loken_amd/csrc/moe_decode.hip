@@ -250,7 +250,8 @@ static int launch_format(int quant_type, const uint8_t* w0, const uint8_t* w1, c
             return d.nb <= 8 ? launch_mode<EngQ6KShort, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s)
                              : launch_mode<EngQ6K, MODE>(w0, w1, acts, sti, eid, tw, bias, out, d, s);
         default:
-            // Q2_K, Q3_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS: the wave-per-row kernels over Q8_1 rows
+            // Q2_K, Q3_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS and the codebook formats IQ3_XXS, IQ3_S, IQ2_S, Q2_0,
+            // IQ2_XXS: the wave-per-row kernels over Q8_1 rows
             if (d.act_f32) return LK_ERR_ARG;
             return lk_moe_rows_legacy(MODE, quant_type, w0, w1, acts, sti, eid, tw, bias, out, d.experts, d.topk,
                                       d.pairs, d.cols, size_k, d.k32, d.act, (int)slab_rows, d.live, d.alt, s);
@@ -458,8 +459,9 @@ extern "C" int loken_moe_gemm_gguf_gate_up_gelu_mul_concat(const float* inputs, 
     if (bl == 0) return LK_ERR_TYPE;
     if (!gate_up_weights || size_n <= 0 || size_k <= 0 || size_k % bl != 0) return size_m == 0 ? LK_OK : LK_ERR_ARG;
     // an expert's slab holds the gate's size_n rows, then the up's
-    // block bytes by wire id: Q8_0, Q4_K, Q2_K, Q3_K, Q5_K, Q6_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS
-    static const int bytes_of_wire[] = {34, 144, 84, 110, 176, 210, 22, 17, 24, 18, 136};
+    // block bytes by wire id: Q8_0, Q4_K, Q2_K, Q3_K, Q5_K, Q6_K, Q5_0, MXFP4, Q5_1, IQ4_NL, IQ4_XS, IQ3_XXS, IQ3_S,
+    // IQ2_S, Q2_0, IQ2_XXS
+    static const int bytes_of_wire[] = {34, 144, 84, 110, 176, 210, 22, 17, 24, 18, 136, 98, 110, 82, 18, 66};
     const int64_t row_bytes = (int64_t)(size_k / bl) * bytes_of_wire[quant_type];
     const uint8_t* up = (const uint8_t*)gate_up_weights + (int64_t)size_n * row_bytes;
     LkGateAct act;

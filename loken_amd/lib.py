@@ -18,6 +18,7 @@ TYPE_Q4_0, TYPE_Q4_1, TYPE_Q5_0, TYPE_Q5_1 = 2, 3, 6, 7
 TYPE_IQ4_NL, TYPE_MXFP4 = 20, 39
 TYPE_Q2_K, TYPE_Q3_K = 10, 11
 TYPE_IQ4_XS = 23
+TYPE_IQ2_XXS, TYPE_IQ3_XXS, TYPE_IQ3_S, TYPE_IQ2_S, TYPE_Q2_0 = 16, 18, 21, 22, 42
 TYPE_Q8_0, TYPE_Q8_1, TYPE_Q4_K, TYPE_Q5_K, TYPE_Q6_K = 8, 9, 12, 13, 14
 
 
@@ -69,6 +70,10 @@ SIGNATURES.update({
     "launch_mmq_moe_gguf_q3_k": _MOE_MMQ,
     "launch_mmq_moe_gguf_q2_k": _MOE_MMQ,
     "launch_mmq_moe_gguf_iq4_xs": _MOE_MMQ,
+    "launch_mmq_moe_gguf_iq3_xxs": _MOE_MMQ,
+    "launch_mmq_moe_gguf_iq3_s": _MOE_MMQ,
+    "launch_mmq_moe_gguf_iq2_s": _MOE_MMQ,
+    "launch_mmq_moe_gguf_q2_0": _MOE_MMQ,
     "loken_moe_mmq_plan": (None, [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "loken_moe_mmq_route": (None, [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "loken_moe_mmq_silu_mul": (None, [_vp, _vp, _i64, _i, _vp]),

@@ -21,6 +21,9 @@ MMQ_MOE_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_moe_gguf_q4_k", _lib.TYPE_Q5_K: 
                     # the formats only mixtures store (quantized/mmq.rs:326-334)
                     _lib.TYPE_IQ4_NL: "launch_mmq_moe_gguf_iq4_nl", _lib.TYPE_MXFP4: "launch_mmq_moe_gguf_mxfp4",
                     _lib.TYPE_IQ4_XS: "launch_mmq_moe_gguf_iq4_xs",
+                    # the codebook formats (quantized/mmq.rs:335-343)
+                    _lib.TYPE_IQ3_XXS: "launch_mmq_moe_gguf_iq3_xxs", _lib.TYPE_IQ3_S: "launch_mmq_moe_gguf_iq3_s",
+                    _lib.TYPE_IQ2_S: "launch_mmq_moe_gguf_iq2_s", _lib.TYPE_Q2_0: "launch_mmq_moe_gguf_q2_0",
                     _lib.TYPE_Q3_K: "launch_mmq_moe_gguf_q3_k", _lib.TYPE_Q2_K: "launch_mmq_moe_gguf_q2_k"}
 MMQ_X_MIN, GRID_Y_MAX = 8, 65535
 
@@ -177,7 +180,8 @@ class MmqRouting:
 # loken's wire ids for the MoE decode launchers (EXPERT_QUANT_CODES, cuda/moe/gguf.cuh:55-71)
 EXPERT_QUANT_CODES = {_lib.TYPE_Q8_0: 0, _lib.TYPE_Q4_K: 1, _lib.TYPE_Q2_K: 2, _lib.TYPE_Q3_K: 3, _lib.TYPE_Q5_K: 4,
                       _lib.TYPE_Q6_K: 5, _lib.TYPE_Q5_0: 6, _lib.TYPE_MXFP4: 7, _lib.TYPE_Q5_1: 8, _lib.TYPE_IQ4_NL: 9,
-                      _lib.TYPE_IQ4_XS: 10}
+                      _lib.TYPE_IQ4_XS: 10, _lib.TYPE_IQ3_XXS: 11, _lib.TYPE_IQ3_S: 12, _lib.TYPE_IQ2_S: 13, _lib.TYPE_Q2_0: 14,
+                      _lib.TYPE_IQ2_XXS: 15}
 
 
 class ExpertRouting:

@@ -177,7 +177,8 @@ def mmvq_grouped(wtype: int, table: torch.Tensor, q8_1: torch.Tensor, k: int, n:
 
 def mmvq_subdots(wtype: int, weight: torch.Tensor, q8_1_row: torch.Tensor, k: int, n: int):
     """Integer sub-block dots of every weight row against ONE Q8_1 row (parity probe)."""
-    per = 16 if wtype in (_lib.TYPE_Q6_K, _lib.TYPE_Q2_K, _lib.TYPE_Q3_K) else 32
+    per = 16 if wtype in (_lib.TYPE_Q6_K, _lib.TYPE_Q2_K, _lib.TYPE_Q3_K, _lib.TYPE_IQ2_XXS, _lib.TYPE_IQ3_XXS, _lib.TYPE_IQ3_S,
+                          _lib.TYPE_IQ2_S, _lib.TYPE_Q2_0) else 32
     dots = torch.empty((n, k // per), dtype=torch.int32, device=weight.device)
     sums = torch.empty((k // 32,), dtype=torch.int32, device=weight.device)
     _lib.check("lk_mmvq_subdots", _lib.load().lk_mmvq_subdots(
@@ -195,6 +196,8 @@ MMQ_QUANTIZER = {_lib.TYPE_Q4_K: "launch_mmq_quantize_q8_1_DS4", _lib.TYPE_Q5_K:
                  _lib.TYPE_Q5_0: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_Q5_1: "launch_mmq_quantize_q8_1_DS4",
                  _lib.TYPE_IQ4_NL: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_MXFP4: "launch_mmq_quantize_q8_1_D4",
                  _lib.TYPE_Q3_K: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_IQ4_XS: "launch_mmq_quantize_q8_1_D4",
+                 _lib.TYPE_IQ3_XXS: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_IQ3_S: "launch_mmq_quantize_q8_1_D4",
+                 _lib.TYPE_IQ2_S: "launch_mmq_quantize_q8_1_D4", _lib.TYPE_Q2_0: "launch_mmq_quantize_q8_1_D4",
                  _lib.TYPE_Q2_K: "launch_mmq_quantize_q8_1_D2S6"}
 MMQ_LAUNCHER = {_lib.TYPE_Q4_K: "launch_mmq_gguf_q4_k", _lib.TYPE_Q5_K: "launch_mmq_gguf_q5_k",
                 _lib.TYPE_Q6_K: "launch_mmq_gguf_q6_k",

@@ -24,9 +24,10 @@ GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1 = 2, 3, 6, 7
 GGML_IQ4_NL, GGML_MXFP4 = 20, 39
 GGML_Q2_K, GGML_Q3_K = 10, 11
 GGML_IQ4_XS = 23
+GGML_IQ2_XXS, GGML_IQ3_XXS, GGML_IQ3_S, GGML_IQ2_S, GGML_Q2_0 = 16, 18, 21, 22, 42   # the codebook expert formats
 GGML_Q8_0, GGML_Q8_1, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K = 8, 9, 12, 13, 14
-BLOCK_LEN = {GGML_IQ4_XS: 256, GGML_Q2_K: 256, GGML_Q3_K: 256, GGML_IQ4_NL: 32, GGML_MXFP4: 32, GGML_Q4_0: 32, GGML_Q4_1: 32, GGML_Q5_0: 32, GGML_Q5_1: 32, GGML_Q8_0: 32, GGML_Q8_1: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256}
-BLOCK_BYTES = {GGML_IQ4_XS: 136, GGML_Q2_K: 84, GGML_Q3_K: 110, GGML_IQ4_NL: 18, GGML_MXFP4: 17, GGML_Q4_0: 18, GGML_Q4_1: 20, GGML_Q5_0: 22, GGML_Q5_1: 24, GGML_Q8_0: 34, GGML_Q8_1: 36, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210}
+BLOCK_LEN = {GGML_IQ2_XXS: 256, GGML_IQ3_XXS: 256, GGML_IQ3_S: 256, GGML_IQ2_S: 256, GGML_Q2_0: 64, GGML_IQ4_XS: 256, GGML_Q2_K: 256, GGML_Q3_K: 256, GGML_IQ4_NL: 32, GGML_MXFP4: 32, GGML_Q4_0: 32, GGML_Q4_1: 32, GGML_Q5_0: 32, GGML_Q5_1: 32, GGML_Q8_0: 32, GGML_Q8_1: 32, GGML_Q4_K: 256, GGML_Q5_K: 256, GGML_Q6_K: 256}
+BLOCK_BYTES = {GGML_IQ2_XXS: 66, GGML_IQ3_XXS: 98, GGML_IQ3_S: 110, GGML_IQ2_S: 82, GGML_Q2_0: 18, GGML_IQ4_XS: 136, GGML_Q2_K: 84, GGML_Q3_K: 110, GGML_IQ4_NL: 18, GGML_MXFP4: 17, GGML_Q4_0: 18, GGML_Q4_1: 20, GGML_Q5_0: 22, GGML_Q5_1: 24, GGML_Q8_0: 34, GGML_Q8_1: 36, GGML_Q4_K: 144, GGML_Q5_K: 176, GGML_Q6_K: 210}
 
 _G = np.uint64(0x9E3779B97F4A7C15)
 _M1 = np.uint64(0xBF58476D1CE4E5B9)
@@ -159,7 +160,20 @@ def legacy_blocks(dtype: int, n_blocks: int, seed: int = 0, stream: int = 0) -> 
     return out
 
 
-_MAKERS = {GGML_IQ4_XS: lambda n, seed=0, stream=0: lowbit_blocks(GGML_IQ4_XS, n, seed, stream),
+def codebook_blocks(dtype: int, n_blocks: int, seed: int = 0, stream: int = 0) -> np.ndarray:
+    """Random blocks of the codebook formats (IQ2_XXS, IQ3_XXS, IQ3_S, IQ2_S, Q2_0): an f16 d sized so that
+    the weights come out around 1e-2, every other byte uniform (each is a code, a sign pattern or scale bits)."""
+    s = stream * 8
+    nbytes = BLOCK_BYTES[dtype]
+    out = rand_bytes(seed, s + 0, n_blocks * nbytes).reshape(n_blocks, nbytes).copy()
+    scale = {GGML_IQ2_XXS: 1e-4, GGML_IQ2_S: 1e-4, GGML_IQ3_XXS: 5e-5, GGML_IQ3_S: 5e-5, GGML_Q2_0: 1e-2}[dtype]
+    out[:, 0:2] = _f16_bytes(np.abs(normal(seed, s + 1, n_blocks)) * np.float32(scale))
+    return out
+
+
+_MAKERS = {**{t: (lambda n, seed=0, stream=0, t=t: codebook_blocks(t, n, seed, stream))
+              for t in (GGML_IQ2_XXS, GGML_IQ3_XXS, GGML_IQ3_S, GGML_IQ2_S, GGML_Q2_0)},
+           GGML_IQ4_XS: lambda n, seed=0, stream=0: lowbit_blocks(GGML_IQ4_XS, n, seed, stream),
            GGML_Q2_K: lambda n, seed=0, stream=0: lowbit_blocks(GGML_Q2_K, n, seed, stream),
            GGML_Q3_K: lambda n, seed=0, stream=0: lowbit_blocks(GGML_Q3_K, n, seed, stream),
            GGML_IQ4_NL: lambda n, seed=0, stream=0: legacy_blocks(GGML_IQ4_NL, n, seed, stream),

@@ -154,7 +154,8 @@ def check(rc, what):
 # ---------------------------------------------------------------------------- gemv (any format)
 WTYPES = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
           "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "q8_0": lib.TYPE_Q8_0, "q4_k": lib.TYPE_Q4_K,
-          "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "iq4_xs": lib.TYPE_IQ4_XS}
+          "q5_k": lib.TYPE_Q5_K, "q6_k": lib.TYPE_Q6_K, "q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "iq4_xs": lib.TYPE_IQ4_XS,
+          "iq2_xxs": lib.TYPE_IQ2_XXS, "iq3_xxs": lib.TYPE_IQ3_XXS, "iq3_s": lib.TYPE_IQ3_S, "iq2_s": lib.TYPE_IQ2_S, "q2_0": lib.TYPE_Q2_0}
 
 
 def gemv(args, dev):

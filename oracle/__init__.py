@@ -18,9 +18,11 @@ Q4_0, Q4_1, Q5_0, Q5_1 = 2, 3, 6, 7
 IQ4_NL, MXFP4 = 20, 39
 Q2_K, Q3_K = 10, 11
 IQ4_XS = 23
+IQ2_XXS, IQ3_XXS, IQ3_S, IQ2_S, Q2_0 = 16, 18, 21, 22, 42   # the codebook expert formats
+CODEBOOK = (IQ2_XXS, IQ3_XXS, IQ3_S, IQ2_S, Q2_0)
 Q8_0, Q8_1, Q4_K, Q5_K, Q6_K, Q8_K = 8, 9, 12, 13, 14, 15
-BLOCK_LEN = {IQ4_XS: 256, Q2_K: 256, Q3_K: 256, IQ4_NL: 32, MXFP4: 32, Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
-BLOCK_BYTES = {IQ4_XS: 136, Q2_K: 84, Q3_K: 110, IQ4_NL: 18, MXFP4: 17, Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
+BLOCK_LEN = {IQ2_XXS: 256, IQ3_XXS: 256, IQ3_S: 256, IQ2_S: 256, Q2_0: 64, IQ4_XS: 256, Q2_K: 256, Q3_K: 256, IQ4_NL: 32, MXFP4: 32, Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32, Q4_K: 256, Q5_K: 256, Q6_K: 256, Q8_K: 256}
+BLOCK_BYTES = {IQ2_XXS: 66, IQ3_XXS: 98, IQ3_S: 110, IQ2_S: 82, Q2_0: 18, IQ4_XS: 136, Q2_K: 84, Q3_K: 110, IQ4_NL: 18, MXFP4: 17, Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36, Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_K: 292}
 
 
 def build(force: bool = False) -> Path:
@@ -69,6 +71,9 @@ def _declare(l: C.CDLL) -> None:
         fn.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp]
         fn.restype = _i
     l.ob_subdots.argtypes = [_i, _sz, _sz, _vp, _vp, _vp, _vp]
+    l.lko_cb_run.argtypes = [_i, _vp, _i, _vp, _vp]
+    l.lko_cb_table.argtypes = [_i, _vp]
+    l.lko_cb_table.restype = _vp
     l.ob_matmul_q8_1.argtypes = [_i, _sz, _sz, _sz, _vp, _sz, _vp, _vp]
     l.ob_matmul.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp]
     l.ob_matmul_f64.argtypes = [_i, _sz, _sz, _sz, _vp, _vp, _vp]
@@ -349,11 +354,27 @@ def ob_matmul_f64(dtype: int, lhs, rhs, n: int) -> np.ndarray:
 def ob_subdots(dtype: int, k: int, n: int, rhs, act_q8_1) -> tuple[np.ndarray, np.ndarray]:
     """(dots[n, k/32 or k/16], sums[k/32]) of weight rows against one Q8_1 activation row."""
     rhs, act = _u8(rhs), _u8(act_q8_1)
-    per = 16 if dtype in (Q6_K, Q2_K, Q3_K) else 32
+    per = 16 if dtype in (Q6_K, Q2_K, Q3_K) or dtype in CODEBOOK else 32
     dots = np.empty((n, k // per), np.int32)
     sums = np.empty(k // 32, np.int32)
     _check(lib().ob_subdots(dtype, k, n, _p(rhs), _p(act), _p(dots), _p(sums)))
     return dots, sums
+
+
+def codebook_run(dtype: int, block, run: int) -> tuple[np.ndarray, np.ndarray]:
+    """(32 signed integer weights, the scales of the two halves) of run `run` of one block."""
+    block = _u8(block)
+    v = np.empty(32, np.int8)
+    s = np.empty(2, np.float32)
+    _check(lib().lko_cb_run(dtype, _p(block), run, _p(v), _p(s)))
+    return v, s
+
+
+def codebook_table(dtype: int) -> bytes:
+    """The expanded grid of a codebook format, little-endian entries."""
+    n = C.c_size_t(0)
+    ptr = lib().lko_cb_table(dtype, C.byref(n))
+    return C.string_at(ptr, n.value)
 
 
 def topk_softmax(logits, topk: int, renorm: bool = True) -> tuple[np.ndarray, np.ndarray]:

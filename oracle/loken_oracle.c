@@ -6,6 +6,7 @@
  * neither may this file.
  */
 #include "loken_oracle.h"
+#include "codebook_formats.h"
 
 #include <math.h>
 #include <stdlib.h>
@@ -82,7 +83,7 @@ int lko_block_len(int dtype) {
         case LKO_Q8_0: case LKO_Q8_1: case LKO_Q4_0: case LKO_Q4_1: case LKO_Q5_0: case LKO_Q5_1:
         case LKO_IQ4_NL: case LKO_MXFP4: return 32;
         case LKO_Q2_K: case LKO_Q3_K: case LKO_Q4_K: case LKO_Q5_K: case LKO_Q6_K: case LKO_Q8_K: case LKO_IQ4_XS: return 256;
-        default: return 0;
+        default: return lko_cb_block_len(dtype);
     }
 }
 
@@ -103,7 +104,7 @@ int lko_block_bytes(int dtype) {
         case LKO_Q5_K: return LKO_Q5K_BYTES;
         case LKO_Q6_K: return LKO_Q6K_BYTES;
         case LKO_Q8_K: return LKO_Q8K_BYTES;
-        default: return 0;
+        default: return lko_cb_block_bytes(dtype);
     }
 }
 
@@ -258,6 +259,8 @@ int lko_dequantize(int dtype, const uint8_t* blocks, size_t n_blocks, float* out
         return lowbit_dequantize(dtype, blocks, n_blocks, out);
     case LKO_IQ4_XS:
         return iq4xs_dequantize(blocks, n_blocks, out);
+    case LKO_IQ2_XXS: case LKO_IQ3_XXS: case LKO_IQ3_S: case LKO_IQ2_S: case LKO_Q2_0:
+        return lko_cb_dequantize(dtype, blocks, n_blocks, out);
     default:
         return legacy_dequantize(dtype, blocks, n_blocks, out);
     }
@@ -870,6 +873,24 @@ static float dot_iq4xs(const uint8_t* w, const uint8_t* y, size_t nb) {
 
 typedef float (*row_dot_fn)(const uint8_t* w, const uint8_t* y, size_t nb);
 
+/* the codebook formats (codebook_formats.c): one statement serves both families, the activation
+ * codes being the same on either side */
+static float dot_iq2xxs(const uint8_t* w, const uint8_t* y, size_t nb) { return lko_cb_dot(LKO_IQ2_XXS, w, y, nb); }
+static float dot_iq3xxs(const uint8_t* w, const uint8_t* y, size_t nb) { return lko_cb_dot(LKO_IQ3_XXS, w, y, nb); }
+static float dot_iq3s(const uint8_t* w, const uint8_t* y, size_t nb) { return lko_cb_dot(LKO_IQ3_S, w, y, nb); }
+static float dot_iq2s(const uint8_t* w, const uint8_t* y, size_t nb) { return lko_cb_dot(LKO_IQ2_S, w, y, nb); }
+static float dot_q20(const uint8_t* w, const uint8_t* y, size_t nb) { return lko_cb_dot(LKO_Q2_0, w, y, nb); }
+static row_dot_fn cb_dot_of(int dtype) {
+    switch (dtype) {
+        case LKO_IQ2_XXS: return dot_iq2xxs;
+        case LKO_IQ3_XXS: return dot_iq3xxs;
+        case LKO_IQ3_S: return dot_iq3s;
+        case LKO_IQ2_S: return dot_iq2s;
+        case LKO_Q2_0: return dot_q20;
+        default: return NULL;
+    }
+}
+
 static row_dot_fn oa_dot_of(int dtype) {
     switch (dtype) {
         case LKO_Q2_K: return oa_dot_q2k;
@@ -885,7 +906,7 @@ static row_dot_fn oa_dot_of(int dtype) {
         case LKO_Q5_1: return oa_dot_q51;
         case LKO_IQ4_NL: return oa_dot_iq4nl;
         case LKO_MXFP4: return oa_dot_mxfp4;
-        default: return NULL;
+        default: return cb_dot_of(dtype);
     }
 }
 static row_dot_fn ob_dot_of(int dtype) {
@@ -903,7 +924,7 @@ static row_dot_fn ob_dot_of(int dtype) {
         case LKO_Q5_1: return ob_dot_q51;
         case LKO_IQ4_NL: return ob_dot_iq4nl;
         case LKO_MXFP4: return ob_dot_mxfp4;
-        default: return NULL;
+        default: return cb_dot_of(dtype);
     }
 }
 
@@ -911,13 +932,13 @@ static row_dot_fn ob_dot_of(int dtype) {
 static size_t oa_act_row_bytes(int dtype, size_t k) {
     if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0 || dtype == LKO_IQ4_NL || dtype == LKO_MXFP4)
         return (k / 32) * LKO_Q80_BYTES;
-    if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1 || dtype == LKO_IQ4_XS) return (k / 32) * LKO_Q81_BYTES;   /* q4_1.rs: BlockQ8_1 */
+    if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1 || dtype == LKO_IQ4_XS || lko_cb_is(dtype)) return (k / 32) * LKO_Q81_BYTES;   /* q4_1.rs: BlockQ8_1 */
     return (k / 256) * LKO_Q8K_BYTES;
 }
 static void oa_quantize_act(int dtype, const float* x, size_t k, uint8_t* out) {
     if (dtype == LKO_Q8_0 || dtype == LKO_Q4_0 || dtype == LKO_Q5_0 || dtype == LKO_IQ4_NL || dtype == LKO_MXFP4)
         lko_quantize_q8_0(x, k, out);
-    else if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1 || dtype == LKO_IQ4_XS) lko_quantize_q8_1(x, k, out);
+    else if (dtype == LKO_Q4_1 || dtype == LKO_Q5_1 || dtype == LKO_IQ4_XS || lko_cb_is(dtype)) lko_quantize_q8_1(x, k, out);
     else lko_quantize_q8_k(x, k, out);
 }
 
@@ -1017,7 +1038,7 @@ int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t*
     const size_t blk = (size_t)lko_block_len(dtype);
     legacy_layout ll;
     const int legacy = legacy_layout_of(dtype, &ll);
-    if (blk == 0 || (!legacy && dtype != LKO_IQ4_XS && dtype != LKO_Q2_K && dtype != LKO_Q3_K && dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
+    if (blk == 0 || (!legacy && !lko_cb_is(dtype) && dtype != LKO_IQ4_XS && dtype != LKO_Q2_K && dtype != LKO_Q3_K && dtype != LKO_Q4_K && dtype != LKO_Q5_K && dtype != LKO_Q6_K && dtype != LKO_Q8_0)) return -3;
     if (k % blk != 0) return -1;
     const size_t nb = k / blk;
     const size_t wrow = nb * (size_t)lko_block_bytes(dtype);
@@ -1041,6 +1062,12 @@ int ob_subdots(int dtype, size_t k, size_t n, const uint8_t* rhs, const uint8_t*
                 for (int s = 0; s < 8; ++s)
                     dots[c * (k / 32) + b * 8 + s] = iq4xs_sub_dot(
                         w + b * 136, s, (const int8_t*)(act + (b * 8 + s) * LKO_Q81_BYTES + 4));
+        } else if (lko_cb_is(dtype)) {   /* two integers per run of 32: its halves */
+            const size_t runs = blk / 32;
+            for (size_t b = 0; b < nb; ++b)
+                for (size_t r = 0; r < runs; ++r)
+                    lko_cb_half_dots(dtype, w + b * (size_t)lko_block_bytes(dtype), (int)r,
+                                     (const int8_t*)(act + (b * runs + r) * LKO_Q81_BYTES + 4), dots + c * (k / 16) + 2 * (b * runs + r));
         } else if (dtype == LKO_Q2_K || dtype == LKO_Q3_K) {
             for (size_t b = 0; b < nb; ++b)
                 for (int s = 0; s < 16; ++s) {
@@ -1148,6 +1175,7 @@ static int dequant_row_f64(int dtype, const uint8_t* w, size_t nb, double* out) 
         }
         return 0;
     }
+    if (lko_cb_is(dtype)) return lko_cb_dequantize_f64(dtype, w, nb, out);
     if (dtype == LKO_IQ4_XS) {
         for (size_t b = 0; b < nb; ++b) {
             const uint8_t* x = w + b * 136;

@@ -151,7 +151,10 @@ def test_legacy_matvec_within_the_reference_envelope(name):
     assert (np.abs(oracle.oa_matmul(wtype, x, w, n) - truth) <= envelope).all()
 
 
-LOWBIT = {"q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "iq4_xs": lib.TYPE_IQ4_XS}
+LOWBIT = {"q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "iq4_xs": lib.TYPE_IQ4_XS,
+          # the codebook expert formats: runs of 32 under a scale per half (two integers per run)
+          "iq2_xxs": lib.TYPE_IQ2_XXS, "iq3_xxs": lib.TYPE_IQ3_XXS, "iq3_s": lib.TYPE_IQ3_S, "iq2_s": lib.TYPE_IQ2_S,
+          "q2_0": lib.TYPE_Q2_0}
 
 
 @pytest.mark.parametrize("name", sorted(LOWBIT))

@@ -91,7 +91,9 @@ def test_expert_batched_block_matches_oracle(tokens, hidden, ffn, n_experts, top
 
 NIBBLE_TILES = {"q4_0": lib.TYPE_Q4_0, "q4_1": lib.TYPE_Q4_1, "q5_0": lib.TYPE_Q5_0, "q5_1": lib.TYPE_Q5_1,
                 "iq4_nl": lib.TYPE_IQ4_NL, "mxfp4": lib.TYPE_MXFP4, "iq4_xs": lib.TYPE_IQ4_XS, "q3_k": lib.TYPE_Q3_K,
-                "q2_k": lib.TYPE_Q2_K}
+                "q2_k": lib.TYPE_Q2_K,
+                # the codebook formats only mixtures store (src/tensor/quantized/mmq.rs:335-343)
+                "iq3_xxs": lib.TYPE_IQ3_XXS, "iq3_s": lib.TYPE_IQ3_S, "iq2_s": lib.TYPE_IQ2_S, "q2_0": lib.TYPE_Q2_0}
 
 
 @pytest.mark.parametrize("tokens,hidden,ffn,n_experts,topk", [(40, 1024, 512, 8, 3), (70, 512, 768, 16, 4),
@@ -255,6 +257,8 @@ def test_per_pair_decode_block_matches_oracle(tokens, hidden, ffn, n_experts, to
 # the rows of the reference's expert table (src/inference/moe_cuda/gemm.rs:23-39) beyond the K-quant engines
 TABLE_TAIL = {"q2_k": lib.TYPE_Q2_K, "q3_k": lib.TYPE_Q3_K, "q5_0": lib.TYPE_Q5_0, "mxfp4": lib.TYPE_MXFP4,
               "q5_1": lib.TYPE_Q5_1, "iq4_nl": lib.TYPE_IQ4_NL, "iq4_xs": lib.TYPE_IQ4_XS,
+              "iq3_xxs": lib.TYPE_IQ3_XXS, "iq3_s": lib.TYPE_IQ3_S, "iq2_s": lib.TYPE_IQ2_S, "q2_0": lib.TYPE_Q2_0,
+              "iq2_xxs": lib.TYPE_IQ2_XXS,   # wire ids 11..15
               "q5_k": lib.TYPE_Q5_K}   # and Q5_K on the K-quant engine, short rows and long
 
 

@@ -364,7 +364,7 @@ def test_driver_error_conditions():
     with pytest.raises(oracle.OracleError, match="byte length"):
         oracle.oa_matmul(oracle.Q4_K, np.zeros((1, 512), np.float32), w, 5)
     with pytest.raises(oracle.OracleError, match="not handled"):
-        oracle.oa_matmul(16, np.zeros((1, 512), np.float32), w, 4)   # IQ2_XXS: no statement of it here
+        oracle.oa_matmul(19, np.zeros((1, 512), np.float32), w, 4)   # IQ1_S: no statement of it here
 
 
 def test_empty_rows_and_columns():

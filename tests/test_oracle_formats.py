@@ -21,7 +21,9 @@ def test_dequantize_matches_ggml_bits(ggml_vectors, name):
 
 
 @pytest.mark.parametrize("name,dtype", [("q2_k", oracle.Q2_K), ("q3_k", oracle.Q3_K), ("iq4_nl", oracle.IQ4_NL), ("iq4_xs", oracle.IQ4_XS), ("mxfp4", oracle.MXFP4), ("q4_0", oracle.Q4_0), ("q4_1", oracle.Q4_1), ("q5_0", oracle.Q5_0), ("q5_1", oracle.Q5_1),
-                                        ("q4_k", oracle.Q4_K), ("q5_k", oracle.Q5_K), ("q6_k", oracle.Q6_K), ("q8_0", oracle.Q8_0)])
+                                        ("q4_k", oracle.Q4_K), ("q5_k", oracle.Q5_K), ("q6_k", oracle.Q6_K), ("q8_0", oracle.Q8_0),
+                                        ("iq2_xxs", oracle.IQ2_XXS), ("iq3_xxs", oracle.IQ3_XXS), ("iq3_s", oracle.IQ3_S), ("iq2_s", oracle.IQ2_S),
+                                        ("q2_0", oracle.Q2_0)])
 def test_ggml_written_blocks_decode_to_ggml_rows(ggml_encode, name, dtype):
     f = ggml_encode["formats"][name]
     cols, read = ggml_encode["cols"], ggml_encode["read"]
@@ -32,7 +34,75 @@ def test_ggml_written_blocks_decode_to_ggml_rows(ggml_encode, name, dtype):
     # and the decoded rows are a quantization of x, not of something else
     x = ggml_encode["x"][: read * cols]
     # (MXFP4's sixteen levels step by up to a third of a value)
-    assert np.abs(got - x).max() <= {"mxfp4": 0.2, "q2_k": 0.4, "q3_k": 0.2}.get(name, 0.1) * np.abs(x).max()
+    # (the two- and three-bit codebooks step wider still; q2_0 has four levels)
+    loose = {"mxfp4": 0.2, "q2_k": 0.4, "q3_k": 0.2, "iq2_xxs": 0.6, "iq2_s": 0.6, "iq3_xxs": 0.4, "iq3_s": 0.4, "q2_0": 1.0}
+    assert np.abs(got - x).max() <= loose.get(name, 0.1) * np.abs(x).max()
+
+
+# ---- the codebook expert formats ----
+CODEBOOK = {"IQ3_XXS": oracle.IQ3_XXS, "IQ3_S": oracle.IQ3_S, "IQ2_S": oracle.IQ2_S, "Q2_0": oracle.Q2_0}
+
+
+@pytest.mark.parametrize("name", sorted(CODEBOOK))
+def test_blocks_cut_from_real_files_decode_to_their_readers_values(name):
+    """The reference's own known answers (tests/vectors/ggml_low_bit_blocks.json, held to by
+    src/tensor/quant_cpu/format/iq_read.rs:212-260): four blocks of an expert tensor and what ggml's reader gives."""
+    import json
+    from pathlib import Path
+    rec = json.loads((Path(__file__).parent / "golden" / "low_bit_blocks.json").read_text())[name]
+    dtype = CODEBOOK[name]
+    assert rec["block_bytes"] == oracle.BLOCK_BYTES[dtype] and rec["values"] == oracle.BLOCK_LEN[dtype]
+    got = oracle.dequantize(dtype, np.frombuffer(bytes.fromhex(rec["bytes"]), np.uint8))
+    want = np.array(rec["decoded"], np.float32)
+    assert got.size == want.size and got.view(np.uint32).tolist() == want.view(np.uint32).tolist()
+
+
+def test_codebooks_are_the_published_tables():
+    """sha256 of each expanded grid (little-endian entries) against the digest of the published table, and the
+    structure a grid has: distinct entries, every byte one of the grid's magnitudes."""
+    import hashlib
+    want = {oracle.IQ2_XXS: (256, 8, {8, 25, 43}, "05826b5d3e472a3a78f196be62ac78acf81df0f909626e12ab9fa2a5d490dd54"),
+            oracle.IQ2_S: (1024, 8, {8, 25, 43}, "e1aa1473412b0552c2174c30ef22ab4073f6a181b85a17056e8249bd2932fd88"),
+            oracle.IQ3_XXS: (256, 4, {4, 12, 20, 28, 36, 44, 52, 62}, "46e35f5a997efdee6c99ce57854c8a0d4f0ff8ca57e5e8a60c0793ea580acf5d"),
+            oracle.IQ3_S: (512, 4, {1, 3, 5, 7, 9, 11, 13, 15}, "bd1af4945a1717c65610b0284e4628b9a1ba3b306fae3a06f6e5f597356e349f")}
+    for dtype, (entries, width, levels, digest) in want.items():
+        raw = oracle.codebook_table(dtype)
+        assert len(raw) == entries * width
+        assert hashlib.sha256(raw).hexdigest() == digest
+        rows = np.frombuffer(raw, np.uint8).reshape(entries, width)
+        assert set(np.unique(rows).tolist()) == levels
+        assert len({r.tobytes() for r in rows}) == entries
+
+
+@pytest.mark.parametrize("dtype", oracle.CODEBOOK)
+def test_codebook_dots_are_the_real_number_products(dtype):
+    """The row dot against Q8_1 rows is sum(weight value * d8 * code) to f32 rounding: brute force in f64 from the
+    dequantized weights (pinned above) and the activation's own codes and scales."""
+    from loken_amd import synth
+    n, k = 5, 1024
+    w = synth.weight(dtype, n, k, seed=31)
+    x = synth.activation(3, k, seed=31)
+    got = oracle.ob_matmul(dtype, x, w, n)
+    assert np.array_equal(got, oracle.oa_matmul(dtype, x, w, n))   # one statement serves both families
+    wv = oracle.dequantize(dtype, w).astype(np.float64).reshape(n, k)
+    q = oracle.quantize_q8_1(x).reshape(3, k // 32, 36)
+    d8 = q[:, :, 0:2].copy().view(np.float16).astype(np.float64)          # [3, k/32, 1]
+    av = (q[:, :, 4:].view(np.int8).astype(np.float64) * d8).reshape(3, k)
+    want = av @ wv.T
+    scale = np.abs(av) @ np.abs(wv).T
+    assert (np.abs(got - want) <= 2e-6 * scale + 1e-30).all()
+    # the integer halves: run values against the codes, by numpy
+    dots, _ = oracle.ob_subdots(dtype, k, n, w, q[0])
+    runs = oracle.BLOCK_LEN[dtype] // 32
+    blocks = w.reshape(n, -1, oracle.BLOCK_BYTES[dtype])
+    codes = q[0, :, 4:].view(np.int8).astype(np.int64)
+    for row in range(n):
+        for b in range(blocks.shape[1]):
+            for r in range(runs):
+                v, s = oracle.codebook_run(dtype, blocks[row, b], r)
+                a = codes[b * runs + r]
+                half = [int((v[:16].astype(np.int64) * a[:16]).sum()), int((v[16:].astype(np.int64) * a[16:]).sum())]
+                assert dots[row, 2 * (b * runs + r):2 * (b * runs + r) + 2].tolist() == half
 
 
 def test_f16_round_trip_is_exhaustively_consistent():
