@@ -11,7 +11,9 @@
 // sub-block's lane groups; lane l, register v is (weight row l % 16, activation row 4 ((l / 16) % 2) + v,
 // sub-block s + 2 (l / 32)). Up to sixteen rows: the slots are rows and every set of weight codes runs
 // twice, against s (the activation live in groups 0, 1) and against s + 2; lane l, register v is (weight
-// row l % 16, activation row 4 (l / 16) + v) for both.
+// row l % 16, activation row 4 (l / 16) + v) for both, and the minimums go through v_mfma_f32_16x16x4_f32 as
+// a product over the sub-blocks, (d8 * sum of codes)[row, sub-block] x (-dmin * min)[sub-block, weight row],
+// four sub-blocks an instruction, straight into the sums (a third of the per-result vector work otherwise).
 #pragma once
 #include "lk_common.h"
 
@@ -188,6 +190,13 @@ struct Core {
         auto fold = [&](int ch, const v4i& c, float dsc, float dmm, int sub) {
             const float off = -MAGIC * dsc;
             const float4 t = *(const float4*)(t_blk + ch * t_chunk + sub * 2 * TOKS);
+            if constexpr (T16) {   // (the minimums: below, on the matrix unit)
+                acc[ch][0] = fmaf(fmaf(__int_as_float(c[0]), dsc, off), t.x, acc[ch][0]);
+                acc[ch][1] = fmaf(fmaf(__int_as_float(c[1]), dsc, off), t.y, acc[ch][1]);
+                acc[ch][2] = fmaf(fmaf(__int_as_float(c[2]), dsc, off), t.z, acc[ch][2]);
+                acc[ch][3] = fmaf(fmaf(__int_as_float(c[3]), dsc, off), t.w, acc[ch][3]);
+                return;
+            }
             const float4 s = *(const float4*)(t_blk + ch * t_chunk + sub * 2 * TOKS + TOKS);
             acc[ch][0] = fmaf(fmaf(__int_as_float(c[0]), dsc, off), t.x, fmaf(dmm, s.x, acc[ch][0]));
             acc[ch][1] = fmaf(fmaf(__int_as_float(c[1]), dsc, off), t.y, fmaf(dmm, s.y, acc[ch][1]));
@@ -225,6 +234,25 @@ struct Core {
                         const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, magic, 0, 0, 0);
                         fold(ch, c, dsc0, dmm0, 4 * c2 + nib);
                     }
+                }
+            }
+        }
+        if constexpr (T16) {
+            // lane (row l16 of the activation, sub-block 4 h + grp) of d8 * S against lane (weight row l16,
+            // sub-block 4 h + grp) of -dmin * min; mn_lo / mn_hi hold the minimums of sub-blocks 0..3 / 4..7
+            const float* s_blk = table + kb * 8 * 2 * TOKS + TOKS + l16;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const float bmin = -(dmin * (float)(((h ? mn_hi : mn_lo) >> (8 * grp)) & 0xFFu));
+#pragma unroll
+                for (int ch = 0; ch < CHUNKS; ++ch) {
+                    const float amin = s_blk[ch * t_chunk + (4 * h + grp) * 2 * TOKS];
+                    v4f c = {acc[ch][0], acc[ch][1], acc[ch][2], acc[ch][3]};
+                    c = __builtin_amdgcn_mfma_f32_16x16x4f32(amin, bmin, c, 0, 0, 0);
+                    acc[ch][0] = c[0];
+                    acc[ch][1] = c[1];
+                    acc[ch][2] = c[2];
+                    acc[ch][3] = c[3];
                 }
             }
         }

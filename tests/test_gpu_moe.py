@@ -399,13 +399,13 @@ def test_experts_over_two_tensors_match_the_one_tensor_launch(name):
     assert torch.equal(moe_gemm_gguf_down_pairs_over(dt, want_h, d0, d0, cut, routing, flat_w, n_experts, hidden, more_at=at_d), rows)
 
 
-def test_decode_launchers_refuse_the_codebook_formats():
+def test_decode_launchers_refuse_wire_ids_outside_the_table():
     tokens, hidden, ffn, n_experts, topk = 2, 512, 256, 4, 2
     gate, up, down, x, ids, w = make_layer(tokens, hidden, ffn, n_experts, topk, seed=62)
     routing = ExpertRouting(dev(ids))
     L = lib.load()
     out = torch.empty((tokens * topk, ffn), device="cuda")
-    for wire in (11, 12, 13, 14, 15, 16, -1):
+    for wire in (16, 17, 99, -1):   # the table ends at 15 (src/inference/moe_cuda/gemm.rs:23-39)
         rc = L.loken_moe_gemm_gguf(dev(x).data_ptr(), dev(gate).data_ptr(), routing.sorted_token_ids.data_ptr(),
                                    routing.expert_ids.data_ptr(), None, out.data_ptr(), n_experts, topk,
                                    tokens * topk, ffn, hidden, wire, None)
@@ -548,7 +548,7 @@ def test_launchers_report_bad_arguments_and_formats():
     l = lib.load()
     buf = torch.zeros(4096, dtype=torch.uint8, device="cuda")
     p, s = buf.data_ptr(), torch.cuda.current_stream().cuda_stream
-    assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 4, 8, 256, 11, s) == lib.LK_ERR_TYPE    # IQ3_XXS: not served
+    assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 4, 8, 256, 16, s) == lib.LK_ERR_TYPE    # past the table's last row
     assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 4, 8, 250, 1, s) == lib.LK_ERR_ARG      # k not whole blocks
     assert l.loken_moe_gemm_gguf(p, p, p, p, None, p, 4, 2, 5, 8, 256, 1, s) == lib.LK_ERR_ARG      # pairs % topk
     assert l.loken_moe_gemm_gguf_down_reduce(p, p, p, p, None, p, 4, 2, 4, 8, 256, 1, None, None, s) == lib.LK_ERR_ARG
