@@ -11,9 +11,7 @@
 // sub-block's lane groups; lane l, register v is (weight row l % 16, activation row 4 ((l / 16) % 2) + v,
 // sub-block s + 2 (l / 32)). Up to sixteen rows: the slots are rows and every set of weight codes runs
 // twice, against s (the activation live in groups 0, 1) and against s + 2; lane l, register v is (weight
-// row l % 16, activation row 4 (l / 16) + v) for both, and the minimums go through v_mfma_f32_16x16x4_f32 as
-// a product over the sub-blocks, (d8 * sum of codes)[row, sub-block] x (-dmin * min)[sub-block, weight row],
-// four sub-blocks an instruction, straight into the sums (a third of the per-result vector work otherwise).
+// row l % 16, activation row 4 (l / 16) + v) for both.
 #pragma once
 #include "lk_common.h"
 
@@ -54,6 +52,10 @@ template <bool Q5, bool T16>
 struct Core {
     static constexpr int TOKS = T16 ? 16 : 8;
     static constexpr int PER = 2;   // staging entries a thread has in flight
+    // The minimums as a product over the sub-blocks on v_mfma_f32_16x16x4_f32, (d8 * sum of codes)[row, sub-block]
+    // x (-dmin * min)[sub-block, weight row], four sub-blocks an instruction, straight into the sums: a third
+    // of the per-result vector work otherwise.
+    static constexpr bool MIN_ON_MATRIX_UNIT = true;
 
     uint8_t *codes, *zeros;
     float* table;
@@ -190,7 +192,7 @@ struct Core {
         auto fold = [&](int ch, const v4i& c, float dsc, float dmm, int sub) {
             const float off = -MAGIC * dsc;
             const float4 t = *(const float4*)(t_blk + ch * t_chunk + sub * 2 * TOKS);
-            if constexpr (T16) {   // (the minimums: below, on the matrix unit)
+            if constexpr (MIN_ON_MATRIX_UNIT) {   // (the minimums: below)
                 acc[ch][0] = fmaf(fmaf(__int_as_float(c[0]), dsc, off), t.x, acc[ch][0]);
                 acc[ch][1] = fmaf(fmaf(__int_as_float(c[1]), dsc, off), t.y, acc[ch][1]);
                 acc[ch][2] = fmaf(fmaf(__int_as_float(c[2]), dsc, off), t.z, acc[ch][2]);
@@ -237,16 +239,20 @@ struct Core {
                 }
             }
         }
-        if constexpr (T16) {
+        if constexpr (MIN_ON_MATRIX_UNIT) {
             // lane (row l16 of the activation, sub-block 4 h + grp) of d8 * S against lane (weight row l16,
-            // sub-block 4 h + grp) of -dmin * min; mn_lo / mn_hi hold the minimums of sub-blocks 0..3 / 4..7
-            const float* s_blk = table + kb * 8 * 2 * TOKS + TOKS + l16;
+            // sub-block 4 h + grp) of -dmin * min. Up to eight rows: rows 8..15 of the product are nobody's
+            // (their lanes' sums join those of rows 0..7 in the end): their operand is zero.
+            const uint32_t mins_lo = w2 & 0x3F3F3F3Fu, mins_hi = ((w3 >> 4) & 0x0F0F0F0Fu) | ((w2 >> 2) & 0x30303030u);
+            const float* s_blk = table + kb * 8 * 2 * TOKS + TOKS + (l16 & (TOKS - 1));
+            const bool real = T16 || l16 < TOKS;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const float bmin = -(dmin * (float)(((h ? mn_hi : mn_lo) >> (8 * grp)) & 0xFFu));
+                const float bmin = -(dmin * (float)(((h ? mins_hi : mins_lo) >> (8 * grp)) & 0xFFu));
 #pragma unroll
                 for (int ch = 0; ch < CHUNKS; ++ch) {
-                    const float amin = s_blk[ch * t_chunk + (4 * h + grp) * 2 * TOKS];
+                    const float at = s_blk[ch * t_chunk + (4 * h + grp) * 2 * TOKS];
+                    const float amin = real ? at : 0.f;
                     v4f c = {acc[ch][0], acc[ch][1], acc[ch][2], acc[ch][3]};
                     c = __builtin_amdgcn_mfma_f32_16x16x4f32(amin, bmin, c, 0, 0, 0);
                     acc[ch][0] = c[0];

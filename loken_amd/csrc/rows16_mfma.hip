@@ -187,17 +187,19 @@ __global__ __launch_bounds__(256 * TW, TW == 4 ? 1 : 2) void q4k_rows16_kernel(L
         }
         stage();
         for (; pair < n_pairs; pair += stride) {
-            if (mine) {
-#pragma unroll
-                for (int d = 0; d < STEPS; ++d) compute(f[d], kq + d * KSPLIT);
-            }
-            // the next tile's loads go out into the registers just read, and fly under the reduction
+            // the next tile's loads go out into each set of registers as it has been read: they fly under
+            // the arithmetic of the sets still to come, and under the reduction
             const int next = TW * (pair + stride) + tsel;
             const bool next_mine = next < n_vt;
-            if (next_mine) {
-                const uint8_t* bp = block0(next);
+            const uint8_t* bp = next_mine ? block0(next) : nullptr;
 #pragma unroll
-                for (int d = 0; d < STEPS; ++d) loadw(f[d], bp + d * STEP_BYTES);
+            for (int d = 0; d < STEPS; ++d) {
+                if (mine) compute(f[d], kq + d * KSPLIT);
+                if (next_mine) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    loadw(f[d], bp + d * STEP_BYTES);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             finish_pair(TW * pair);
             mine = next_mine;
