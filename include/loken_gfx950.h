@@ -560,8 +560,12 @@ int loken_moe_gemm_gguf_down_reduce(const float* inputs, const void* weights,
  * size_m * size_n * 4 bytes plus, for the formats that read Q8_1 rows,
  * size_m * pad512(size_k) / 32 * 36 bytes rounded up to 256, returns LK_ERR_SIZE and launches
  * nothing. Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
- * streams, or two host threads) race; calls on one stream are ordered and safe. No counterpart in
- * the reference. */
+ * streams, or two host threads) race; calls on one stream are ordered and safe. The array keeps the
+ * last call's contents and nothing is cleared: like the allocating entry point, the call relies on
+ * sorted_token_ids naming every slot once (every named slot's row is written, zeros for a pair whose
+ * expert is out of range). The first call on a device asks the runtime for the array's address there:
+ * make it before a capture begins; later calls may be recorded into a graph (kernels only, no memset
+ * node). No counterpart in the reference. */
 int loken_moe_gemm_gguf_down_reduce_static(const float* inputs, const void* weights,
                                            const int32_t* sorted_token_ids, const int32_t* expert_ids,
                                            const float* topk_weights, float* outputs, int num_experts,

@@ -510,11 +510,9 @@ static int down_impl(const float* inputs, const void* weights, const int32_t* so
         if (!base) return LK_ERR_NOMEM;
     }
     float* pairs = pair_rows ? pair_rows : (float*)(base + act_bytes);
-    if (from_static && !live) {
-        // the array keeps the last call's rows: a pair the routing leaves out must read as zero
-        const size_t n = (size_t)size_m * size_n;
-        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, pairs, n);
-    }
+    // (The fixed array keeps the last call's rows. Nothing is cleared: sorted_token_ids names every slot once,
+    // as the allocating path and the reference assume (cuda/moe/moe_gguf.cu:785-786), and the kernels write
+    // every named slot's row, zeros for a pair whose expert is out of range.)
     if (!as_f32)
         if (int rc = lk_quantize_q8_1(inputs, LK_TYPE_F32, base, size_k, kp, size_m, stream)) return rc;
     if (live) {

@@ -62,3 +62,41 @@ def test_static_scratch_entry_refuses_what_does_not_fit():
     torch.cuda.synchronize()
     assert rc == lib.LK_ERR_SIZE
     assert (out == 5.0).all()
+
+
+def test_static_scratch_entry_recorded_into_a_graph_replays_to_the_eager_bits():
+    """What the entry point is for: the call recorded into a HIP graph (after one eager call on the device,
+    which resolves the fixed array's address), replayed three times with the program's own eager work and
+    synchronizations between the replays, every replay bit for bit the eager result."""
+    n_experts, hidden, ffn, topk, tokens = 8, 512, 256, 2, 9
+    for wtype in (lib.TYPE_Q4_K, lib.TYPE_Q5_0):
+        wire = moe.EXPERT_QUANT_CODES[wtype]
+        down = dev(synth.weight(wtype, n_experts * hidden, ffn, seed=95, stream=3))
+        h = dev(synth.activation(tokens * topk, ffn, seed=96) * np.float32(3.0))
+        ids, w = oracle.topk_softmax(synth.activation(tokens, n_experts, seed=96, stream=7), topk)
+        routing = moe.ExpertRouting(dev(ids))
+        wd = dev(w.reshape(-1))
+        add = dev(synth.activation(tokens, hidden, seed=97, stream=9))
+        rc, want = call("loken_moe_gemm_gguf_down_reduce_static", wire, h, down, routing, wd, n_experts, hidden, None, add)
+        assert rc == 0
+        l = lib.load()
+        out = torch.zeros((tokens, hidden), dtype=torch.float32, device="cuda")
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                rc = l.loken_moe_gemm_gguf_down_reduce_static(
+                    h.data_ptr(), down.data_ptr(), routing.sorted_token_ids.data_ptr(), routing.expert_ids.data_ptr(),
+                    wd.data_ptr(), out.data_ptr(), n_experts, topk, tokens * topk, hidden, ffn, wire, None, add.data_ptr(),
+                    side.cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        for replay in range(3):
+            out.fill_(7.0)
+            # eager work of the program between the replays: another call through the same array, smaller
+            rc2, _ = call("loken_moe_gemm_gguf_down_reduce_static", wire, h[: 2 * topk], down,
+                          moe.ExpertRouting(dev(ids[:2])), dev(w[:2].reshape(-1)), n_experts, hidden, None, add[:2].contiguous())
+            assert rc2 == 0
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want), f"replay {replay}"
