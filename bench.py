@@ -487,6 +487,27 @@ def main() -> int:
                 "timed_as": (f"{reps} graph replays of the mix of {len(q4k_plan)} launches, each replay between its own events; "
                              f"per-launch figures are a replay's time over its launches") if q4k_graph is not None else "eager launches"}
     q4k_launch_bytes = sorted({int(a_bytes) for a_bytes in q4k_launch_sizes})
+    # The mix kernel by kernel: the launches of one size (q + k + v; o; gate + up) over the layers' own weights
+    # as a graph of their own, timed the same way. The gate + up launch is the step's largest share of time.
+    if q4k_graph is not None and not args.brief:
+        by_kernel = {}
+        for nbytes in q4k_launch_bytes:
+            items = [it for it, sz in zip(q4k_plan, q4k_launch_sizes) if int(sz) == nbytes]
+            side3 = torch.cuda.Stream()
+            g3 = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side3):
+                cap = [(fn, a[:-1] + (side3.cuda_stream,)) for fn, a in items]
+                run(cap)
+                side3.synchronize()
+                with torch.cuda.graph(g3, stream=side3):
+                    run(cap)
+            torch.cuda.synchronize()
+            us3 = wl.time_launches(lambda i: g3.replay(), 200, warm=20) / len(items)
+            gbs3 = nbytes / float(us3.mean()) / 1e3
+            by_kernel[str(nbytes)] = dict(wl.spread(us3), launches_per_replay=len(items), avg_launch_us=round(float(us3.mean()), 3),
+                                          achieved_gbs=round(gbs3, 1), frac=round(gbs3 / HBM_PEAK_GBS, 4))
+            del g3
+        roofline["by_launch_size"] = by_kernel
 
     # ------------------------------------------------------------------ the rest of the metric, and measured denominators
     extras = {}
