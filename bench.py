@@ -33,7 +33,7 @@ Two more measurements ride in the same JSON line:
                 configuration 2a and the expert block of configuration 3 on the pool.
   gemv_4096     the benchmark set's configuration 0 (Q4_K 4096 x 4096, one row) over rotating copies.
   mmq           configurations 2a / 2b, the tiled matmul, against the int8 matrix peak.
-  rows-sweep    one --wtype q4_k|q6_k matrix (--rows-n x --cols-k) at 16..2048 rows: the matrix-unit
+  rows-sweep    one --wtype q4_k|q5_k|q6_k matrix (--rows-n x --cols-k) at 16..2048 rows: the matrix-unit
                 rows kernel against the tiled matmul, and the path QKernelMatMul::forward's mirror takes.
   other_configs the step at 4 and 8 rows, the MoE block at 1 / 16 / 256 tokens and the Qwen3-1.7B step at
                 1 / 16 / 64 rows (configurations 1, 3, 4), each from a child run of this file.

@@ -236,8 +236,17 @@ void launch_mmq_quantize_q8_1_D2S6(const void* x, const int32_t* ids, void* vy, 
 /* dst[col, row] (f32, rows `stride_col_dst` floats apart) = weight row `row` . token `col`.
  *   x = weights [nrows_x][stride_row_x blocks], y = workspace of ncols_y rows, ncols_x = k.
  * Returns the token-tile width launched (32, 64 or 128), 0 when nothing ran (bad sizes, or k
- * not a multiple of 256). tmp_fixup, cc, nsm, smpbo, warp_size are accepted and unused: there
- * is no stream-k fixup pass and one device family.
+ * not a multiple of 256). cc, nsm, smpbo, warp_size are accepted and unused: one device family.
+ * tmp_fixup: null, or the 16 MiB buffer the reference's workspace keeps for its stream-k partial
+ * tiles (FIXUP_BYTES = 256 * 128 * 128 * 4, src/tensor/quantized/kernel_matmul/mmq.rs:42; 16-byte
+ * aligned, contents irrelevant on entry, overwritten). With it, a product whose tiles would leave
+ * most of the chip idle is launched with K cut into ranges of blocks: each workgroup writes its
+ * partial tile there and a second launch adds the ranges in ascending order into dst (same integers,
+ * a fixed order of f32 sums: the result does not depend on scheduling; it differs from the null
+ * call's in the last bits). Used only when every partial product fits the 16 MiB, nrows_x and
+ * stride_col_dst are multiples of 4 and dst is 16-byte aligned. Calls sharing one buffer must not
+ * overlap on the card (the reference holds its workspace mutex across quantize and matmul,
+ * kernel_matmul/mmq.rs:43-86). Both launches are capturable.
  * Replaces launch_mmq_gguf_{q4_k,q5_k,q6_k,q8_0} (cuda/mmq_gguf/mmq_launch.cuh:61-206). */
 int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,
                          int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,

@@ -178,15 +178,19 @@ int matvec_rows(int dtype, int k) {
 // Rows the matrix-unit rows kernels take before the tiled matmul does. Measured on MI355X over
 // n = 2048 ... 151936 and k = 2048 ... 14336: a rows kernel re-reads the weights for every 32
 // activation rows but fills the chip from the first pass; a tiled launch holds a 128- or 256-row weight
-// block per workgroup and leaves most of the chip idle until n x rows gives it enough tiles. The two
-// meet near n x rows = 1.75 M for Q4_K / Q5_K (4096 x 4096: 480 rows; 14336 x 4096: 110; 128256 x 4096:
-// the rows kernel still wins at 16) and 4 M for Q6_K (4096 x 14336: 1000 rows; 151936 x 2048: under 32).
+// block per workgroup, cuts K into ranges while its tiles are fewer than the chip's workgroup slots
+// (mmq_problem.h) and pays one more pass over the partial products for that. Up to 16 rows the 16-row
+// tiles stay; above, the two meet near n x rows = 450 K at k <= 4096 and in proportion earlier for
+// longer rows (quantizer + kernel, rows kernel against tiled):
+//   Q4_K  4096 x 4096: 128 rows 36 us against 39, 256 rows 49 against 43; 14336 x 4096: 32 rows 36
+//         against 36, 128 rows 75 against 53; 4096 x 14336: 32 rows 52 against 39, 512 rows 207 against 127
+//   Q6_K  4096 x 4096: 64 rows 32 against 35, 256 rows 64 against 51; 14336 x 4096: 32 rows 44 against 40,
+//         256 rows 161 against 114; 4096 x 14336: 32 rows 54 against 42, 1024 rows 568 against 360
+//   Q5_K  4096 x 4096: 128 rows 37 against 41, 256 rows 52 against 48; 4096 x 14336: 128 rows 80 against 63
 // `bench.py --workload rows-sweep` prints the table for a shape.
-static bool rows_kernel_serves(int dtype, int n, int rows) {
-    const long long work = (long long)n * rows;
-    if (dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K) return rows <= 16 || work <= 1750000;
-    if (dtype == LK_TYPE_Q6_K) return work <= (4ll << 20);
-    return false;
+static bool rows_kernel_serves(int dtype, int n, int k, int rows) {
+    if (dtype != LK_TYPE_Q4_K && dtype != LK_TYPE_Q5_K && dtype != LK_TYPE_Q6_K) return false;
+    return rows <= 16 || (long long)n * rows * (k > 4096 ? k : 4096) <= 450000ll * 4096;
 }
 
 // The K-quants at 3 to 8 f32 rows: the 16-row tiles of the matrix-unit kernels (their time hardly moves
@@ -263,7 +267,7 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
 
     // --- a handful of rows (or a matrix too small to fill the chip with tiles): matrix unit, weights
     //     straight from HBM
-    if (rows_kernel_serves(dtype_, n_, rows) && rows_kernel_fits) {
+    if (rows_kernel_serves(dtype_, n_, k_, rows) && rows_kernel_fits) {
         const int blocks = k_ / 32;
         int rc;
         {

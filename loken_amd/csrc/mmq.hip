@@ -117,6 +117,7 @@ struct MmqQ45K {
     static constexpr int BLOCK_BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES;
     static constexpr int QS0 = Q5 ? 48 : 16;
     static constexpr bool F16_TILES = !Q5;   // Q4_K above 64 tokens: the f16 tile kernel
+    static constexpr int WIDE_FROM = 384;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int NS = 8;          // one weight scale per 32 values
     static constexpr bool HAS_MIN = true;
     static constexpr int MIN_RANK = 8;   // one minimum per 32 values
@@ -201,6 +202,7 @@ struct MmqQ6K {
     static constexpr bool HAS_MIN = false;
     static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
+    static constexpr int WIDE_FROM = 384;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int BLOCKS_PER_STEP = 1;
     static constexpr int QCH = TN * 8 / MMQ_WG;
 
@@ -266,6 +268,7 @@ struct MmqQ80 {
     static constexpr bool HAS_MIN = false;
     static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
+    static constexpr int WIDE_FROM = 96;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int BLOCKS_PER_STEP = 8;
     static constexpr int QCH = TN * 16 / MMQ_WG, DCH = TN * 8 / MMQ_WG;
 
@@ -317,6 +320,7 @@ struct MmqLegacy {
     static constexpr bool HAS_MIN = L::M_AT >= 0;
     static constexpr int MIN_RANK = HAS_MIN ? 8 : 0;
     static constexpr bool F16_TILES = false;
+    static constexpr int WIDE_FROM = 300;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int BLOCKS_PER_STEP = 8;
     static constexpr int ALIGN = L::BYTES % 2 ? 1 : 2;
     static constexpr int PER = TN * 8 / MMQ_WG;
@@ -379,6 +383,7 @@ struct MmqQ3K {
     static constexpr bool HAS_MIN = false;
     static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
+    static constexpr int WIDE_FROM = 384;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int BLOCKS_PER_STEP = 1;
     static_assert(TN * 2 == MMQ_WG, "one (row, half) per thread");
 
@@ -447,6 +452,7 @@ struct MmqQ2K {
     static constexpr bool HAS_MIN = true;
     static constexpr int MIN_RANK = 16;
     static constexpr bool F16_TILES = false;
+    static constexpr int WIDE_FROM = 384;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int BLOCKS_PER_STEP = 1;
     static_assert(TN * 2 == MMQ_WG, "one (row, half) per thread");
 
@@ -497,6 +503,7 @@ struct MmqIq4Xs {
     static constexpr bool HAS_MIN = false;
     static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
+    static constexpr int WIDE_FROM = 300;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int BLOCKS_PER_STEP = 1;
     static constexpr int PER = TN * 8 / MMQ_WG;
 
@@ -547,6 +554,7 @@ struct MmqCodebook {
     static constexpr bool HAS_MIN = false;
     static constexpr int MIN_RANK = 0;
     static constexpr bool F16_TILES = false;
+    static constexpr int WIDE_FROM = 300;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int BLOCKS_PER_STEP = 8 / C::RUNS;
     static constexpr int PER = TN * 8 / MMQ_WG;
 
@@ -642,7 +650,7 @@ struct TokenFrag {
 };
 
 template <class F, int TM, int WAVES_M>
-static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, int m0, uint8_t* lds) {
+static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, int m0, uint8_t* lds, int kb0, int kb1) {
     constexpr int WAVES_N = 4 / WAVES_M;
     constexpr int JT = TN / (32 * WAVES_N), IT = TM / (32 * WAVES_M);
     static_assert(JT >= 1 && IT >= 1, "tile does not split over four waves");
@@ -673,15 +681,15 @@ static __device__ __forceinline__ void mmq_tile(const MmqProblem& pb, int n0, in
 
     typename F::Frag wf;
     TokenFrag<TM, F::MIN_RANK == 16> tf;
-    F::fetch(wf, pb.w, pb.row_blocks, 0, n0, pb.n);
-    tf.fetch(pb.y, pb.rows_total, 0, m0, pb.m_end);
+    F::fetch(wf, pb.w, pb.row_blocks, kb0, n0, pb.n);
+    tf.fetch(pb.y, pb.rows_total, kb0, m0, pb.m_end);
 
-    for (int kb = 0; kb < pb.nb; ++kb) {
+    for (int kb = kb0; kb < kb1; ++kb) {
         __syncthreads();  // the previous step's readers are done with the tiles
         F::commit(wf, n0, pb.n, wq, wsc, wmn);
         tf.template commit<F::HAS_MIN>(aq, ad8, ads);
         __syncthreads();
-        if (kb + 1 < pb.nb) {  // next step's loads fly under this step's arithmetic
+        if (kb + 1 < kb1) {  // next step's loads fly under this step's arithmetic
             F::fetch(wf, pb.w, pb.row_blocks, kb + 1, n0, pb.n);
             tf.fetch(pb.y, pb.rows_total, kb + 1, m0, pb.m_end);
         }
@@ -870,7 +878,48 @@ __global__ __launch_bounds__(MMQ_WG, 2) void mmq_dense_kernel(MmqProblem pb, int
     const int m_tile = seq % m_tiles;
     const int n_tile = (seq / m_tiles) * 8 + xcd;
     if (n_tile >= n_tiles) return;
-    mmq_tile<F, TM, WAVES_M>(pb, n_tile * TN, pb.m_begin + m_tile * TM, lds);
+    mmq_tile<F, TM, WAVES_M>(pb, n_tile * TN, pb.m_begin + m_tile * TM, lds, 0, (int)pb.nb);
+}
+
+// The dense product with K cut into `splits` ranges of blocks, for shapes whose tiles alone leave most
+// of the chip idle (4096 weight rows x 128 token rows are 32 tiles for 256 CUs, each walking all of K).
+// A workgroup walks one range and writes its partial tile to part[split] ([token][n] floats, token
+// rows n floats apart); mmq_split_sum_kernel then adds the ranges in ascending order, so a result does
+// not depend on which workgroup finished when. Ids: the m tiles of one (n tile, range) back to back
+// on one XCD, as above.
+template <class F, int TM, int WAVES_M>
+__global__ __launch_bounds__(MMQ_WG, 2) void mmq_dense_split_kernel(MmqProblem pb, int n_tiles, int m_tiles, int splits,
+                                                                   float* part, int64_t part_stride) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int id = blockIdx.x;
+    const int xcd = id & 7;
+    int seq = id >> 3;
+    const int m_tile = seq % m_tiles;
+    seq /= m_tiles;
+    const int split = seq % splits;
+    const int n_tile = (seq / splits) * 8 + xcd;
+    if (n_tile >= n_tiles) return;
+    const int kb0 = (int)(pb.nb * split / splits), kb1 = (int)(pb.nb * (split + 1) / splits);
+    pb.dst = part + split * part_stride;
+    pb.ldd = pb.n;
+    mmq_tile<F, TM, WAVES_M>(pb, n_tile * TN, pb.m_begin + m_tile * TM, lds, kb0, kb1);
+}
+
+// dst[token][c] = part[0][token][c] + part[1][token][c] + ... in that order; four columns a thread.
+__global__ __launch_bounds__(256) void mmq_split_sum_kernel(const float* __restrict__ part, int splits, int64_t part_stride,
+                                                            float* __restrict__ dst, int64_t count, int n, int64_t ldd) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= count) return;
+    float4 a = *(const float4*)(part + i);
+    for (int s = 1; s < splits; ++s) {
+        const float4 b = *(const float4*)(part + s * part_stride + i);
+        a.x += b.x;
+        a.y += b.y;
+        a.z += b.z;
+        a.w += b.w;
+    }
+    const int64_t row = i / n, col = i - row * n;
+    *(float4*)(dst + row * ldd + col) = a;
 }
 
 // Expert-batched product: expert e's slab against the sorted rows [bounds[e], bounds[e+1]).
@@ -888,24 +937,33 @@ __global__ __launch_bounds__(MMQ_WG, 2) void mmq_moe_kernel(MmqProblem pb, const
     pb.w = (stack ? w_second : pb.w) + (int64_t)e * stride_expert;
     if (stack) pb.dst += dst_second;
     for (int m0 = pb.m_begin + blockIdx.y * TM; m0 < pb.m_end; m0 += gridDim.y * TM)
-        mmq_tile<F, TM, WAVES_M>(pb, blockIdx.x * TN, m0, lds);
+        mmq_tile<F, TM, WAVES_M>(pb, blockIdx.x * TN, m0, lds, 0, (int)pb.nb);
 }
 
 template <class F, int TM, int WAVES_M>
-static int launch_dense_tm(const MmqProblem& pb, hipStream_t s) {
-    auto kernel = mmq_dense_kernel<F, TM, WAVES_M>;
+static int launch_dense_tm(const MmqProblem& pb, hipStream_t s, void* fixup = nullptr) {
     constexpr int lds_bytes = mmq_lds_bytes<F, TM>();
-    if (mmq_prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
     const int n_tiles = (pb.n + TN - 1) / TN;
     const int m_tiles = (pb.m_end - pb.m_begin + TM - 1) / TM;
     const int n_groups = (n_tiles + 7) / 8;
+    const int splits = mmq_splits(pb, (int64_t)n_tiles * m_tiles, 2 * lk_device().cus, fixup);   // two workgroups fit a CU
+    if (splits > 1) {
+        auto kernel = mmq_dense_split_kernel<F, TM, WAVES_M>;
+        if (mmq_prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
+        const int64_t count = (int64_t)pb.m_end * pb.n;
+        hipLaunchKernelGGL(kernel, dim3(n_groups * 8 * m_tiles * splits), dim3(MMQ_WG), lds_bytes, s, pb, n_tiles, m_tiles,
+                           splits, (float*)fixup, count);
+        return lk_mmq_split_sum((const float*)fixup, splits, pb, s) == LK_OK ? TM : 0;
+    }
+    auto kernel = mmq_dense_kernel<F, TM, WAVES_M>;
+    if (mmq_prepare_kernel(kernel, lds_bytes) != LK_OK) return 0;
     const int grid = n_groups * 8 * m_tiles;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(MMQ_WG), lds_bytes, s, pb, n_tiles, m_tiles);
     return hipGetLastError() == hipSuccess ? TM : 0;
 }
 
 template <class F>
-static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x, int64_t nrows_x,
+static int launch_dense(void* fixup, const void* x, const void* y, void* dst, int64_t ncols_x, int64_t nrows_x,
                         int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, void* stream) {
     if (!x || !y || !dst || ncols_x <= 0 || nrows_x <= 0 || ncols_y <= 0) return 0;
     if ((uintptr_t)x % F::ALIGN != 0) return 0;
@@ -914,29 +972,42 @@ static int launch_dense(const void* x, const void* y, void* dst, int64_t ncols_x
     MmqProblem pb{(const uint8_t*)x, (const uint8_t*)y, (float*)dst, nullptr, ncols_x / 256, stride_row_x,
                   ncols_y, stride_col_dst, (int)nrows_x, 0, (int)ncols_y};
     hipStream_t s = (hipStream_t)stream;
-    if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s);
+    if (ncols_y <= 32) return launch_dense_tm<F, 32, 1>(pb, s, fixup);
     // (Q2_K stays on 64-token tiles: with the rank-16 minimum its 128-token tile spills and runs 512 x
     // 4096 -> 14336 in 344 us against 240, 2048 x 14336 -> 4096 in 1155 against 742; every other format
     // is 3 to 40 % faster on the wide tile)
-    if (ncols_y <= 64 || F::MIN_RANK == 16) return launch_dense_tm<F, 64, 2>(pb, s);
+    if (ncols_y <= 64 || F::MIN_RANK == 16) return launch_dense_tm<F, 64, 2>(pb, s, fixup);
     if constexpr (F::F16_TILES) {   // Q4_K: scales folded into f16 operands
         if (!lk_env_flag("LK_MMQ_I8")) {
             // 128-token tiles with the token side expanded once per call, where they pad the rows at most a
-            // tenth more than the 64-token tiles would (512 x 4096 -> 14336: 105 us against 123)
+            // tenth more than the 64-token tiles would (512 x 4096 -> 14336: 105 us against 123) and are
+            // enough to occupy half the CUs (fewer: the 64-token tiles, which can cut K)
             const int64_t pad128 = (ncols_y + 127) / 128 * 128, pad64 = (ncols_y + 63) / 64 * 64;
-            if (ncols_y > 128 && 10 * pad128 <= 11 * pad64 && !lk_env_flag("LK_MMQ_NO_WIDE")) {
+            const int64_t wide_tiles = (nrows_x + 255) / 256 * (pad128 / 128);
+            if (ncols_y > 128 && 10 * pad128 <= 11 * pad64 && 2 * wide_tiles > lk_device().cus && !lk_env_flag("LK_MMQ_NO_WIDE")) {
                 const int tm = lk_mmq_q4k_wide_dense(pb, s);
                 if (tm >= 0) return tm;
             }
-            const int tm = lk_mmq_q4k_f16_dense(pb, s);
+            const int tm = lk_mmq_q4k_f16_dense(pb, s, fixup);
             if (tm >= 0) return tm;
         }
     }
+    // 128-token tiles where there are F::WIDE_FROM of them or more, else 64-token tiles, twice as many and
+    // with K cut where those are still few. Quantizer + matmul, 64- against 128-token tiles:
+    //   Q6_K  4096 x 14336 at 128 / 512 / 1024 rows (32 / 128 / 256 tiles) 70 / 215 / 393 us against 99 / 307 /
+    //         577, at 2048 rows (512) 724 against 639; 14336 x 4096 at 384 rows (336) 182 against 196, at 512
+    //         (448) 211 against 197. Q5_K and Q3_K alike.
+    //   Q4_0  14336 x 4096 at 256 rows (224) 115 against 120, at 384 (336) 178 against 155
+    //   Q8_0  4096 x 4096 at 256 rows (64) 61.5 against 62.1, at 384 (96) 92 against 87, at 2048 (512) 299 against 190
+    // LK_TUNE_MMQ_TM = 64 / 128 forces one in measurement runs.
+    const int forced_tm = lk_tune_env("LK_TUNE_MMQ_TM");
+    const int64_t tiles128 = (nrows_x + TN - 1) / TN * ((ncols_y + 127) / 128);
+    if (forced_tm == 64 || (forced_tm != 128 && tiles128 < F::WIDE_FROM)) return launch_dense_tm<F, 64, 2>(pb, s, fixup);
     // 128-token tile: a wave takes all four token tiles of one 32-row weight tile (measured against
     // a 2 x 2 patch per wave: Q4_K 366 against 334 TOP/s at 512 rows, 434 against 364 at 2048;
     // Q6_K 320 against 313; Q8_0 305 against 304)
     constexpr int WAVES_M = 1;
-    return launch_dense_tm<F, 128, WAVES_M>(pb, s);
+    return launch_dense_tm<F, 128, WAVES_M>(pb, s, fixup);
 }
 
 template <class F, int TM, int WAVES_M>
@@ -999,6 +1070,13 @@ static int launch_moe(const void* x, const void* x_second, int64_t dst_second, c
 
 }  // namespace
 
+int lk_mmq_split_sum(const float* part, int splits, const MmqProblem& pb, hipStream_t s) {
+    const int64_t count = (int64_t)pb.m_end * pb.n;
+    hipLaunchKernelGGL(mmq_split_sum_kernel, dim3((unsigned)((count / 4 + 255) / 256)), dim3(256), 0, s, part, splits, count,
+                       pb.dst, count, pb.n, pb.ldd);
+    return lk_launch_status();
+}
+
 extern "C" void launch_mmq_quantize_q8_1_D4(const void* x, const int32_t* ids, void* vy, int type_x,
                                             int64_t ne00, int64_t s01, int64_t s02, int64_t s03,
                                             int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3, void* stream) {
@@ -1021,40 +1099,40 @@ extern "C" int launch_mmq_gguf_q4_k(void* tmp_fixup, const void* x, const void* 
                                     int64_t ncols_x, int64_t nrows_x, int64_t ncols_y,
                                     int64_t stride_row_x, int64_t stride_col_dst, int cc, int nsm,
                                     int64_t smpbo, int warp_size, void* stream) {
-    (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
-    return launch_dense<MmqQ4K>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
+    (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
+    return launch_dense<MmqQ4K>(tmp_fixup, x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
 }
 
 extern "C" int launch_mmq_gguf_q5_k(void* tmp_fixup, const void* x, const void* y, void* dst,
                                     int64_t ncols_x, int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x,
                                     int64_t stride_col_dst, int cc, int nsm, int64_t smpbo, int warp_size,
                                     void* stream) {
-    (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
-    return launch_dense<MmqQ5K>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
+    (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
+    return launch_dense<MmqQ5K>(tmp_fixup, x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
 }
 
 extern "C" int launch_mmq_gguf_q6_k(void* tmp_fixup, const void* x, const void* y, void* dst,
                                     int64_t ncols_x, int64_t nrows_x, int64_t ncols_y,
                                     int64_t stride_row_x, int64_t stride_col_dst, int cc, int nsm,
                                     int64_t smpbo, int warp_size, void* stream) {
-    (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
-    return launch_dense<MmqQ6K>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
+    (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
+    return launch_dense<MmqQ6K>(tmp_fixup, x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
 }
 
 extern "C" int launch_mmq_gguf_q8_0(void* tmp_fixup, const void* x, const void* y, void* dst,
                                     int64_t ncols_x, int64_t nrows_x, int64_t ncols_y,
                                     int64_t stride_row_x, int64_t stride_col_dst, int cc, int nsm,
                                     int64_t smpbo, int warp_size, void* stream) {
-    (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
-    return launch_dense<MmqQ80>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
+    (void)cc; (void)nsm; (void)smpbo; (void)warp_size;
+    return launch_dense<MmqQ80>(tmp_fixup, x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream);
 }
 
 #define LK_MMQ_DENSE_ENTRY(NAME, FMT)                                                                   \
     extern "C" int NAME(void* tmp_fixup, const void* x, const void* y, void* dst, int64_t ncols_x,     \
                         int64_t nrows_x, int64_t ncols_y, int64_t stride_row_x, int64_t stride_col_dst, \
                         int cc, int nsm, int64_t smpbo, int warp_size, void* stream) {                 \
-        (void)tmp_fixup; (void)cc; (void)nsm; (void)smpbo; (void)warp_size;                            \
-        return launch_dense<FMT>(x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream); \
+        (void)cc; (void)nsm; (void)smpbo; (void)warp_size;                            \
+        return launch_dense<FMT>(tmp_fixup, x, y, dst, ncols_x, nrows_x, ncols_y, stride_row_x, stride_col_dst, stream); \
     }
 
 LK_MMQ_DENSE_ENTRY(launch_mmq_gguf_q4_0, MmqQ40)

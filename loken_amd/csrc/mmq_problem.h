@@ -38,10 +38,33 @@ static int mmq_prepare_kernel(K kernel, int lds_bytes) {
     return LK_OK;
 }
 
-// Q4_K against 65 or more token rows (mmq_q4k_f16.hip). Return the token-tile width launched,
+// What the caller's tmp_fixup holds (FIXUP_BYTES, src/tensor/quantized/kernel_matmul/mmq.rs:42): the
+// reference's kernels keep their stream-k partial tiles there, these the partial products of a cut K.
+constexpr int64_t MMQ_FIXUP_BYTES = 256ll * 128 * 128 * 4;
+
+// A dense product whose tiles alone leave most of the chip idle is launched with K cut into ranges of
+// blocks: a workgroup walks one range and writes its partial tile to part[range] ([token][n] floats in
+// the caller's tmp_fixup), and lk_mmq_split_sum adds the ranges in ascending order, so a result does
+// not depend on which workgroup finished when. mmq_splits: how many ranges, for `tiles` tiles on a chip
+// that holds `slots` workgroups of the kernel at once: as many as bring tiles x ranges to the slots,
+// while a range keeps at least two blocks and every partial product fits the buffer. 1 = the plain launch.
+static inline int mmq_splits(const MmqProblem& pb, int64_t tiles, int64_t slots, const void* fixup) {
+    const int forced = lk_tune_env("LK_TUNE_MMQ_SPLITS");   // measurement runs: -1 never, n > 0 that many where they fit
+    if (!fixup || forced < 0 || pb.ids_dst || pb.m_begin != 0) return 1;
+    if (pb.n % 4 != 0 || pb.ldd % 4 != 0 || (uintptr_t)pb.dst % 16 != 0 || (uintptr_t)fixup % 16 != 0) return 1;
+    const int64_t fit = MMQ_FIXUP_BYTES / ((int64_t)pb.m_end * pb.n * 4);
+    int64_t want = forced > 0 ? forced : slots / tiles;
+    if (want > fit) want = fit;
+    if (want > pb.nb / 2) want = pb.nb / 2;
+    return want < 2 ? 1 : (int)want;
+}
+// dst[token][c] = part[0][token][c] + part[1][token][c] + ..., part[i] m_end x n floats; LK_* status.
+int lk_mmq_split_sum(const float* part, int splits, const MmqProblem& pb, hipStream_t s);
+
+// Q4_K against 65 or more token rows (mmq_q4k_f16.hip); `fixup`: the caller's tmp_fixup or null. Return the token-tile width launched,
 // 0 when the launch failed, -1 when the operands do not suit these kernels (16-byte alignment,
 // 32-bit record offsets) and the caller should take the int8 tiles.
-int lk_mmq_q4k_f16_dense(const MmqProblem& pb, hipStream_t s);
+int lk_mmq_q4k_f16_dense(const MmqProblem& pb, hipStream_t s, void* fixup);
 // Q4_K against 129 or more token rows on the f16 tiles with four token tiles per wave (mmq_q4k_wide.hip); same returns.
 int lk_mmq_q4k_wide_dense(const MmqProblem& pb, hipStream_t s);
 void lk_mmq_q4k_wide_release(int device);

@@ -407,6 +407,27 @@ __global__ __launch_bounds__(Wide::THREADS, 1) void q4k_f16_dense_kernel(MmqProb
     q4k_f16_tile(pb, n_tile * Wide::TN, pb.m_begin + m_tile * Wide::TM, lds);
 }
 
+// The same tiles over one of `splits` ranges of K each, the partial tile to part[range].
+__global__ __launch_bounds__(Wide::THREADS, 1) void q4k_f16_dense_split_kernel(MmqProblem pb, int n_tiles, int m_tiles,
+                                                                              int splits, float* part, int64_t part_stride) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int id = blockIdx.x;
+    const int xcd = id & 7;
+    int seq = id >> 3;
+    const int m_tile = seq % m_tiles;
+    seq /= m_tiles;
+    const int split = seq % splits;
+    const int n_tile = (seq / splits) * 8 + xcd;
+    if (n_tile >= n_tiles) return;
+    const int64_t kb0 = pb.nb * split / splits, kb1 = pb.nb * (split + 1) / splits;
+    pb.w += kb0 * Q4K_BYTES;
+    pb.y += kb0 * pb.rows_total * MMQ_REC_BYTES;
+    pb.nb = kb1 - kb0;
+    pb.dst = part + split * part_stride;
+    pb.ldd = pb.n;
+    q4k_f16_tile(pb, n_tile * Wide::TN, pb.m_begin + m_tile * Wide::TM, lds);
+}
+
 // Expert-batched: expert e's slab against the sorted rows [bounds[e], bounds[e+1]).
 __global__ __launch_bounds__(Wide::THREADS, 1) void q4k_f16_moe_kernel(MmqProblem pb, const uint8_t* w_second,
                                                                       int64_t dst_second,
@@ -427,12 +448,19 @@ __global__ __launch_bounds__(Wide::THREADS, 1) void q4k_f16_moe_kernel(MmqProble
 
 }  // namespace
 
-int lk_mmq_q4k_f16_dense(const MmqProblem& pb, hipStream_t s) {
+int lk_mmq_q4k_f16_dense(const MmqProblem& pb, hipStream_t s, void* fixup) {
     using C = Wide;
     if (((uintptr_t)pb.w | (uintptr_t)pb.y) % 16 != 0 || pb.rows_total > (1 << 23)) return -1;
-    if (mmq_prepare_kernel(q4k_f16_dense_kernel, C::LDS) != LK_OK) return 0;
     const int n_tiles = (pb.n + C::TN - 1) / C::TN;
     const int m_tiles = (pb.m_end - pb.m_begin + C::TM - 1) / C::TM;
+    const int splits = mmq_splits(pb, (int64_t)n_tiles * m_tiles, lk_device().cus, fixup);   // one workgroup a CU
+    if (splits > 1) {
+        if (mmq_prepare_kernel(q4k_f16_dense_split_kernel, C::LDS) != LK_OK) return 0;
+        hipLaunchKernelGGL(q4k_f16_dense_split_kernel, dim3((n_tiles + 7) / 8 * 8 * m_tiles * splits), dim3(C::THREADS), C::LDS,
+                           s, pb, n_tiles, m_tiles, splits, (float*)fixup, (int64_t)pb.m_end * pb.n);
+        return lk_mmq_split_sum((const float*)fixup, splits, pb, s) == LK_OK ? C::TM : 0;
+    }
+    if (mmq_prepare_kernel(q4k_f16_dense_kernel, C::LDS) != LK_OK) return 0;
     const int grid = (n_tiles + 7) / 8 * 8 * m_tiles;
     hipLaunchKernelGGL(q4k_f16_dense_kernel, dim3(grid), dim3(C::THREADS), C::LDS, s, pb, n_tiles, m_tiles);
     return hipGetLastError() == hipSuccess ? C::TM : 0;

@@ -264,15 +264,31 @@ def mmq_quantize(wtype: int, x: torch.Tensor, gather: torch.Tensor | None = None
     return ws
 
 
-def mmq_forward(wtype: int, weight: torch.Tensor, x: torch.Tensor, n: int) -> torch.Tensor:
+MMQ_FIXUP_BYTES = 256 * 128 * 128 * 4   # FIXUP_BYTES of MmqWorkspace (kernel_matmul/mmq.rs:42)
+_mmq_fixup = {}
+
+
+def mmq_fixup(device) -> torch.Tensor:
+    """The card's ``tmp_fixup`` buffer of MmqWorkspace (kernel_matmul/mmq.rs:42-60), made on first use and kept:
+    the tiled launchers hold the partial products of a cut K there (calls that share it must not overlap,
+    as with the reference's workspace)."""
+    key = torch.device(device)
+    if key not in _mmq_fixup:
+        _mmq_fixup[key] = torch.empty(MMQ_FIXUP_BYTES, dtype=torch.uint8, device=key)
+    return _mmq_fixup[key]
+
+
+def mmq_forward(wtype: int, weight: torch.Tensor, x: torch.Tensor, n: int, fixup: bool = True) -> torch.Tensor:
     """``[rows, k]`` x weight ``[n, k]`` -> ``[rows, n]`` f32 through the tiled kernels, the two
-    launches of QKernelMatMul::mmq_forward (kernel_matmul/mmq.rs:103-136)."""
+    launches of QKernelMatMul::mmq_forward (kernel_matmul/mmq.rs:103-136). ``fixup`` false passes no
+    ``tmp_fixup``: the launcher then never cuts K."""
     rows, k = x.shape
     ws = mmq_quantize(wtype, x)
     out = torch.empty((rows, n), dtype=torch.float32, device=x.device)
     fn = getattr(_lib.load(), MMQ_LAUNCHER[wtype])
     i = MMQ_DEVICE_INFO
-    launched = fn(None, weight.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, rows, k // BLOCK_LEN[wtype], n,
+    fix = mmq_fixup(x.device).data_ptr() if fixup else None
+    launched = fn(fix, weight.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, rows, k // BLOCK_LEN[wtype], n,
                   i["cc"], i["nsm"], i["smpbo"], i["warp_size"], _stream())
     if launched == 0:
         raise _lib.LokenError(MMQ_LAUNCHER[wtype], _lib.LK_ERR_ARG)

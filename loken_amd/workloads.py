@@ -294,7 +294,7 @@ def mmq(args, dev):
         quantizer(x.data_ptr(), None, ws.data_ptr(), 0, k, x.stride(0), 0, 0, k_padded, m, 1, 1, s)
 
     def matmul():
-        if launcher(None, w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
+        if launcher(ops.mmq_fixup(dev).data_ptr(), w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
                     info["cc"], info["nsm"], info["smpbo"], info["warp_size"], s) == 0:
             raise lib.LokenError(ops.MMQ_LAUNCHER[wtype], lib.LK_ERR_ARG)
 
@@ -604,7 +604,7 @@ def decode_1p7b(args, dev):
                 out = torch.empty((b, n), device=dev)
                 keep.append(out)
                 plan.append(("tile", getattr(L, ops.MMQ_LAUNCHER[wtype]),
-                             (None, w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, b, k // 256, n, info["cc"],
+                             (ops.mmq_fixup(dev).data_ptr(), w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, b, k // 256, n, info["cc"],
                               info["nsm"], info["smpbo"], info["warp_size"], s)))
 
     for _ in range(layers):
@@ -715,7 +715,7 @@ def brief_mmq(shape, launches=200):
         quantizer(x.data_ptr(), None, ws.data_ptr(), 0, k, x.stride(0), 0, 0, k_padded, m, 1, 1, s)
 
     def matmul():
-        if launcher(None, w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
+        if launcher(ops.mmq_fixup(dev).data_ptr(), w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
                     info["cc"], info["nsm"], info["smpbo"], info["warp_size"], s) == 0:
             raise lib.LokenError(ops.MMQ_LAUNCHER[wtype], lib.LK_ERR_ARG)
 
@@ -738,15 +738,15 @@ def rows_sweep(args, dev):
     mirror of QKernelMatMul::forward takes. The crossover constants in host_qmatmul.hip come from
     these tables."""
     L = lib.load()
-    wtype = {"q4_k": Q4K, "q6_k": Q6K}.get(args.wtype)
+    wtype = {"q4_k": Q4K, "q5_k": WTYPES["q5_k"], "q6_k": Q6K}.get(args.wtype)
     if wtype is None:
-        raise SystemExit("--workload rows-sweep: --wtype q4_k or q6_k")
+        raise SystemExit("--workload rows-sweep: --wtype q4_k, q5_k or q6_k")
     n, k = args.rows_n, args.cols_k
     mk = Maker(dev)
     w = mk.make(wtype, n, k)
     quantizer = getattr(L, ops.MMQ_QUANTIZER[wtype])
     launcher = getattr(L, ops.MMQ_LAUNCHER[wtype])
-    rows_fn = L.lk_dense_q4k_rows if wtype == Q4K else L.lk_dense_q6k_rows
+    rows_fn = {Q4K: L.lk_dense_q4k_rows, Q6K: L.lk_dense_q6k_rows}.get(wtype, L.lk_dense_q5k_rows)
     info = ops.MMQ_DEVICE_INFO
     k_padded = ops.pad_to(ops.pad_to(k, 512), 128)
     handle = L.lkh_qkernel_matmul_new(wtype, n, k, w.data_ptr(), dev.index or 0)
@@ -761,7 +761,7 @@ def rows_sweep(args, dev):
         def tiled():
             s = torch.cuda.current_stream().cuda_stream
             quantizer(x.data_ptr(), None, ws.data_ptr(), 0, k, x.stride(0), 0, 0, k_padded, m, 1, 1, s)
-            if launcher(None, w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
+            if launcher(ops.mmq_fixup(dev).data_ptr(), w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
                         info["cc"], info["nsm"], info["smpbo"], info["warp_size"], s) == 0:
                 raise lib.LokenError(ops.MMQ_LAUNCHER[wtype], lib.LK_ERR_ARG)
 

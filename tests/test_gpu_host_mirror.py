@@ -55,12 +55,12 @@ def close(got, want, rtol=1e-3, atol=1e-4):
     # a handful of rows over a matrix large enough to pay for staging them in every workgroup
     ("q4_k", 2, 4000, "matvec-fused"), ("q4_k", 3, 4000, "rows-on-matrix-unit"), ("q4_k", 8, 1100, "rows-on-matrix-unit"),
     ("q5_k", 4, 2100, "rows-on-matrix-unit"), ("q5_k", 4, 2000, "matvec"),
-    # above 64 rows the rows kernel keeps a matrix too small to fill the chip with tiles (n x rows up to 1.75 M)
+    # above 16 rows the rows kernel keeps a matrix too small to fill the chip with tiles (n x rows up to 450 thousand)
     ("q4_k", 80, 200, "rows-on-matrix-unit"), ("q4_k", 80, 24000, "tiled"),
     ("q6_k", 1, 200, "matvec-fused"), ("q6_k", 8, 200, "matvec"), ("q6_k", 20, 200, "rows-on-matrix-unit"),
     ("q6_k", 40, 200, "rows-on-matrix-unit"), ("q6_k", 200, 24000, "tiled"),
     ("q8_0", 3, 200, "matvec"), ("q8_0", 33, 200, "tiled"), ("q5_k", 1, 200, "matvec-fused"), ("q5_k", 8, 200, "matvec"),
-    ("q5_k", 20, 200, "rows-on-matrix-unit"), ("q5_k", 200, 200, "rows-on-matrix-unit"), ("q5_k", 80, 24000, "tiled"),
+    ("q5_k", 20, 200, "rows-on-matrix-unit"), ("q5_k", 200, 200, "rows-on-matrix-unit"), ("q5_k", 80, 24000, "tiled"), ("q5_k", 18, 24000, "rows-on-matrix-unit"),
     ("q4_0", 1, 200, "matvec"), ("q4_0", 40, 200, "matvec"), ("q5_1", 9, 200, "matvec"), ("iq4_nl", 3, 200, "matvec"),
     # four of the 32-value formats have tiles: from 49 rows, or n x rows of 300 thousand
     ("q4_0", 50, 200, "tiled"), ("q5_0", 64, 200, "tiled"), ("q5_1", 30, 12000, "tiled"), ("q4_1", 20, 12000, "matvec"),

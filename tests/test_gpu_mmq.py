@@ -99,6 +99,47 @@ def test_tiled_matmul_agrees_with_matvec_family(name):
     assert (tiled - rows).abs().max().item() <= 2e-5 * scale
 
 
+@pytest.mark.parametrize("name", SERVED)
+@pytest.mark.parametrize("m,k,n", [(20, 1280, 132), (64, 2048, 256), (100, 1280, 512), (300, 3584, 264), (7, 7168, 8)])
+def test_cut_k_follows_the_oracle_and_the_plain_launch(name, m, k, n):
+    # Given the caller's tmp_fixup (FIXUP_BYTES of src/tensor/quantized/kernel_matmul/mmq.rs:42) a product of
+    # few tiles is launched over ranges of K (5, 8, 14 and 28 blocks here: uneven ranges too) and the
+    # partial products are added in ascending order: the same integers, another order of f32 sums, and
+    # nothing that depends on which workgroup finished first.
+    wtype = DT[name]
+    w = dev(synth.weight(wtype, n, k, seed=47, stream=5))
+    xh = synth.activation(m, k, seed=47)
+    x = dev(xh)
+    plain = ops.mmq_forward(wtype, w, x, n, fixup=False)
+    cut = ops.mmq_forward(wtype, w, x, n)
+    again = ops.mmq_forward(wtype, w, x, n)
+    assert torch.equal(cut, again)
+    assert_close(cut.cpu().numpy(), oracle.ob_matmul(wtype, xh, w.cpu().numpy(), n))
+    assert (cut - plain).abs().max().item() <= 2e-5 * plain.abs().max().item()
+
+
+@pytest.mark.parametrize("name,splits", [("q4_k", 3), ("q6_k", 7), ("q8_0", 2), ("q4_k", 64)])
+def test_forced_range_counts_and_what_keeps_k_whole(name, splits, knobs):
+    # LK_TUNE_MMQ_SPLITS asks for a range count (capped so that a range keeps two blocks); -1, no buffer,
+    # or a row length that is not a multiple of four floats leave K whole: then the bits are the plain launch's.
+    wtype = DT[name]
+    m, k, n = 70, 2560, 260
+    w = dev(synth.weight(wtype, n, k, seed=48, stream=6))
+    xh = synth.activation(m, k, seed=48)
+    x = dev(xh)
+    plain = ops.mmq_forward(wtype, w, x, n, fixup=False)
+    knobs.set("LK_TUNE_MMQ_SPLITS", str(splits))
+    cut = ops.mmq_forward(wtype, w, x, n)
+    knobs.set("LK_TUNE_MMQ_SPLITS", "-1")
+    whole = ops.mmq_forward(wtype, w, x, n)
+    knobs.clear("LK_TUNE_MMQ_SPLITS")
+    assert torch.equal(whole, plain)
+    assert not torch.equal(cut, plain)
+    assert_close(cut.cpu().numpy(), oracle.ob_matmul(wtype, xh, w.cpu().numpy(), n))
+    w_odd = dev(synth.weight(wtype, 130, k, seed=48, stream=7))
+    assert torch.equal(ops.mmq_forward(wtype, w_odd, x, 130), ops.mmq_forward(wtype, w_odd, x, 130, fixup=False))
+
+
 @pytest.mark.parametrize("m,k,n", [(65, 256, 33), (130, 2048, 520), (300, 1024, 128)])
 def test_q4k_wide_tiles_agree_with_int8_tiles_and_matvec(m, k, n, knobs):
     # Above 64 token rows Q4_K forms its sub-block dots on the f16 matrix unit (scale folded into
