@@ -456,8 +456,8 @@ def decode_1p7b(args, dev):
     matvec = b <= 8
     used = {"rows": 0, "matvec": 0, "tiled": 0}
 
-    def rows_kernel_serves(wtype, n, rows):   # the rule of host_qmatmul.hip
-        return (rows <= 16 or n * rows <= 1750000) if wtype == Q4K else n * rows <= (4 << 20)
+    def rows_kernel_serves(wtype, n, k, rows):   # the rule of host_qmatmul.hip
+        return rows <= 16 or n * rows * max(k, 4096) <= 450000 * 4096
 
     # 3 to 16 rows: the 16-row-tile kernels on the matrix unit, the matrices that share an activation in
     # one launch (q + k + v; gate + up with the activation on top, as dense_q4k_imma_m8_act_mul of the
@@ -468,8 +468,8 @@ def decode_1p7b(args, dev):
     rows_h_q81 = torch.empty((b, ffn // 32, 36), dtype=torch.uint8, device=dev) if fused_rows else None
     # above 16 rows, while the rows kernels serve gate + up and down: the same hand-over
     mid_h_q81 = (torch.empty((b, ffn // 32, 36), dtype=torch.uint8, device=dev)
-                 if (not fused_rows and not matvec and args.mid_rows == "auto" and rows_kernel_serves(Q4K, ffn, b)
-                     and rows_kernel_serves(Q6K, hidden, b)) else None)
+                 if (not fused_rows and not matvec and args.mid_rows == "auto" and rows_kernel_serves(Q4K, ffn, hidden, b)
+                     and rows_kernel_serves(Q6K, hidden, ffn, b)) else None)
 
     def add_fused_rows(g, k, wtype, ns):
         nonlocal total_bytes
@@ -547,7 +547,7 @@ def decode_1p7b(args, dev):
                 keep.append(out)
                 plan.append(("status", L.lk_mmvq, (wtype, w.data_ptr(), q.data_ptr(), out.data_ptr(), lib.TYPE_F32, k, n, b,
                                          q.shape[1], n, None, 0, s)))
-        elif args.mid_rows == "auto" and all(rows_kernel_serves(wtype, n, b) for n in ns):
+        elif args.mid_rows == "auto" and all(rows_kernel_serves(wtype, n, k, b) for n in ns):
             # the host mirror's choice (host_qmatmul.hip): the matrix-unit rows kernels, no weight staging
             if g == "h" and mid_h_q81 is not None:   # `down` reads the Q8_1 rows the gate + up launch wrote
                 out = torch.empty((b, ns[0]), device=dev)
