@@ -155,15 +155,15 @@ bool tiled_serves(int dtype, int k) {
            k % 256 == 0;
 }
 
-// Q4_0 / Q4_1 / Q5_0 / Q5_1: rows from which one tiled launch beats mat-vec launches of eight rows each.
-// Measured on MI355X (Q4_0 and Q5_1 alike): 2048 x 2048 and 4096 x 4096 from 56-64 rows (48 rows: 67 us
-// against 77), 4096 x 14336 likewise, 14336 x 4096 from 24 (74 us against 60; 16 rows: 50 against 60).
-// Q3_K (and Q2_K, taken alike), whose mat-vec is slower: 4096 x 4096 from 48 rows (89 us against 85; 32 rows: 60 against 61),
-// 14336 x 4096 from 16 (78 against 61; 9 rows: 52 against 60).
+// Q4_0 / Q4_1 / Q5_0 / Q5_1, Q3_K and Q2_K above eight rows: one tiled launch (with K cut into ranges
+// where its tiles are few, mmq_problem.h) against mat-vec launches of eight rows each. Measured on MI355X,
+// quantizer included, mat-vec against tiled: Q4_0 4096 x 4096 at 9 / 16 / 32 rows 29 / 35 / 55 us against
+// 31 / 27 / 29; 14336 x 4096 at 9 / 16 rows 42 / 58 against 37 / 38; 4096 x 14336 at 9 rows 57 against 41;
+// 1024 x 4096 at 9 / 16 rows 27 / 31 against 33 / 26. Q5_1, Q3_K and Q2_K alike (Q3_K 4096 x 4096 at 9 / 16
+// rows 31 / 40 against 29 / 27). So: from 16 rows, and from 9 on a matrix of 48 M weights or more.
 bool nibble_tiles_pay(int dtype, int n, int k, int rows) {
     if (!nibble_tiles(dtype) || k % 256 != 0) return false;
-    if (dtype == LK_TYPE_Q3_K || dtype == LK_TYPE_Q2_K) return rows > 40 || (long long)rows * n >= 200000;
-    return rows > 48 || (long long)rows * n >= 300000;
+    return rows >= 16 || (long long)n * k >= (48ll << 20);
 }
 
 size_t elem_bytes(int type) { return type == LK_TYPE_F32 ? 4 : 2; }
@@ -172,7 +172,9 @@ size_t elem_bytes(int type) { return type == LK_TYPE_F32 ? 4 : 2; }
 
 int matvec_rows(int dtype, int k) {
     if ((dtype == LK_TYPE_Q4_K || dtype == LK_TYPE_Q5_K || dtype == LK_TYPE_Q6_K) && k % 256 == 0) return 8;
-    return dtype == LK_TYPE_Q8_0 && tiled_serves(dtype, k) ? 32 : 8;
+    // Q8_0, mat-vec launches of eight rows against the tiled matmul: 4096 x 4096 at 16 / 24 / 32 rows 32 / 40 /
+    // 49 us against 32 / 32 / 32; 14336 x 4096 51 / 70 / 89 against 56 / 56 / 58
+    return dtype == LK_TYPE_Q8_0 && tiled_serves(dtype, k) ? 16 : 8;
 }
 
 // Rows the matrix-unit rows kernels take before the tiled matmul does. Measured on MI355X over

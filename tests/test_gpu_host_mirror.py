@@ -59,11 +59,12 @@ def close(got, want, rtol=1e-3, atol=1e-4):
     ("q4_k", 80, 200, "rows-on-matrix-unit"), ("q4_k", 80, 24000, "tiled"),
     ("q6_k", 1, 200, "matvec-fused"), ("q6_k", 8, 200, "matvec"), ("q6_k", 20, 200, "rows-on-matrix-unit"),
     ("q6_k", 40, 200, "rows-on-matrix-unit"), ("q6_k", 200, 24000, "tiled"),
-    ("q8_0", 3, 200, "matvec"), ("q8_0", 33, 200, "tiled"), ("q5_k", 1, 200, "matvec-fused"), ("q5_k", 8, 200, "matvec"),
+    ("q8_0", 3, 200, "matvec"), ("q8_0", 16, 200, "matvec"), ("q8_0", 17, 200, "tiled"), ("q5_k", 1, 200, "matvec-fused"), ("q5_k", 8, 200, "matvec"),
     ("q5_k", 20, 200, "rows-on-matrix-unit"), ("q5_k", 200, 200, "rows-on-matrix-unit"), ("q5_k", 80, 24000, "tiled"), ("q5_k", 18, 24000, "rows-on-matrix-unit"),
-    ("q4_0", 1, 200, "matvec"), ("q4_0", 40, 200, "matvec"), ("q5_1", 9, 200, "matvec"), ("iq4_nl", 3, 200, "matvec"),
-    # four of the 32-value formats have tiles: from 49 rows, or n x rows of 300 thousand
-    ("q4_0", 50, 200, "tiled"), ("q5_0", 64, 200, "tiled"), ("q5_1", 30, 12000, "tiled"), ("q4_1", 20, 12000, "matvec"),
+    ("q4_0", 1, 200, "matvec"), ("q4_0", 12, 200, "matvec"), ("q5_1", 9, 200, "matvec"), ("iq4_nl", 3, 200, "matvec"),
+    # four of the 32-value formats have tiles: from 16 rows, or from 9 over 48 M weights
+    ("q4_0", 50, 200, "tiled"), ("q5_0", 16, 200, "tiled"), ("q5_1", 30, 12000, "tiled"), ("q4_1", 12, 12000, "matvec"),
+    ("q4_0", 9, 49152, "tiled"),
     ("q4_1", 130, 300, "tiled"), ("iq4_nl", 60, 200, "matvec"), ("q3_k", 41, 200, "tiled"), ("q3_k", 17, 12000, "tiled"),
     ("q2_k", 50, 200, "tiled"),
     ("mxfp4", 17, 200, "matvec"), ("q2_k", 12, 200, "matvec"), ("q3_k", 1, 200, "matvec")])
@@ -175,7 +176,7 @@ def test_workspace_grows_outside_a_capture_only_and_replays_then():
 def test_argument_errors_are_status_codes():
     l = lib.load()
     assert l.lkh_matvec_rows(lib.TYPE_Q4_K, 4096) == 8 and l.lkh_matvec_rows(lib.TYPE_Q6_K, 4096) == 8
-    assert l.lkh_matvec_rows(lib.TYPE_Q8_0, 4096) == 32
+    assert l.lkh_matvec_rows(lib.TYPE_Q8_0, 4096) == 16
     h = l.lkh_qkernel_matmul_new(99, 8, 256, 16, 0)
     assert l.lkh_qkernel_matmul_forward(h, 16, lib.TYPE_F32, 1, 16, None, 0) == lib.LK_ERR_TYPE
     l.lkh_qkernel_matmul_free(h)
