@@ -35,6 +35,8 @@ Two more measurements ride in the same JSON line:
   mmq           configurations 2a / 2b, the tiled matmul, against the int8 matrix peak.
   rows-sweep    one --wtype q4_k|q5_k|q6_k matrix (--rows-n x --cols-k) at 16..2048 rows: the matrix-unit
                 rows kernel against the tiled matmul, and the path QKernelMatMul::forward's mirror takes.
+  prefill-layer the quantized linears of one Llama-3-8B layer at --tokens rows, each through the host mirror of
+                QKernelMatMul::forward (--layers of them, each with its own weights, a graph replay).
   other_configs the step at 4 and 8 rows, the MoE block at 1 / 16 / 256 tokens and the Qwen3-1.7B step at
                 1 / 16 / 64 rows (configurations 1, 3, 4), each from a child run of this file.
   roofline.peak_measured / mmq.peak_measured: what a read-only launch and a register-resident
@@ -84,7 +86,7 @@ def parse_args():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of 1 GiB before the steps: the dispatch of known size that "
                          "scales the FETCH_SIZE / WRITE_SIZE counters of a profiled run")
-    ap.add_argument("--workload", choices=["decode", "gemv", "gemv-4096", "mmq", "moe", "decode-1p7b", "rows-sweep"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemv", "gemv-4096", "mmq", "moe", "decode-1p7b", "rows-sweep", "prefill-layer"], default="decode",
                     help="decode (default): the Llama-3-8B step described above; the others are the further measured "
                          "workloads of loken_amd/workloads.py, one JSON line each")
     ap.add_argument("--shape", choices=["2a", "2b"], default="2a", help="--workload mmq: 512x4096->14336 Q4_K or 2048x14336->4096 Q6_K")
@@ -93,7 +95,7 @@ def parse_args():
     ap.add_argument("--wtype", default="q4_0", help="--workload gemv: q4_0 q4_1 q5_0 q5_1 iq4_nl mxfp4 q8_0 q2_k q3_k q4_k q5_k q6_k iq4_xs iq2_xxs iq3_xxs iq3_s iq2_s q2_0")
     ap.add_argument("--rows-n", type=int, default=14336, help="--workload gemv: weight rows")
     ap.add_argument("--cols-k", type=int, default=4096, help="--workload gemv: values per row")
-    ap.add_argument("--tokens", type=int, default=256, help="--workload moe: rows through the expert block")
+    ap.add_argument("--tokens", type=int, default=256, help="--workload moe / prefill-layer: rows through the expert block / the layer")
     ap.add_argument("--moe-wtype", default="q4_k", help="--workload moe: the experts' format (as --wtype)")
     ap.add_argument("--moe-path", choices=["auto", "tiled", "rows", "pairs"], default="auto",
                     help="--workload moe: expert-batched tiled matmul, expert-batched rows on the matrix unit, mat-vec per "

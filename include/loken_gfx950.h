@@ -57,6 +57,7 @@ extern "C" {
 #define LK_ERR_LAUNCH 3     /* the HIP runtime refused the launch */
 #define LK_ERR_NOMEM 4      /* scratch could not be reserved (MoE decode launchers only) */
 #define LK_ERR_SIZE 5       /* the call needs more than the fixed scratch of an entry point that allocates nothing */
+#define LK_NOT_TAKEN 6      /* host mirror only: forward would serve this call another way (the reference's None) */
 
 /* Bytes of the per-device fixed scratch array behind loken_moe_gemm_gguf_down_reduce_static. */
 #define LK_STATIC_SCRATCH_BYTES (8u << 20)

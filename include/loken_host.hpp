@@ -54,11 +54,37 @@ public:
      * Returns LK_OK or an LK_ERR_* code; never throws, never aborts. */
     int forward(const void* x, int x_type, int rows, void* out, void* stream, bool decode_order = false);
 
+    /* An activation quantized to Q8_1 once, for every mat-vec over the same k on the same card
+     * (QuantizedActivation of the reference, kernel_matmul.rs:105-117). The caller owns `q81`:
+     * quantized_bytes(k, rows) bytes of device memory, 4-byte aligned. */
+    struct QuantizedActivation {
+        const void* q81 = nullptr;
+        int k = 0, rows = 0, device = -1;
+        int x_type = 0;   /* the type the rows were in, and so the type each product comes back in */
+    };
+    static size_t quantized_bytes(int k, int rows);
+
+    /* quantize_for_matvec (kernel_matmul.rs:695-748): x [rows, k] into `q81` the way forward quantizes it
+     * for the mat-vec kernels, so that several weights over the same rows quantize them once. LK_OK and `a`
+     * filled, or LK_NOT_TAKEN where forward would not take those kernels for this row count (the
+     * reference's None): more rows than matvec_rows without `decode_order`, or a matrix whose few rows go
+     * to the matrix-unit rows kernels. */
+    int quantize_for_matvec(const void* x, int x_type, int rows, void* q81, void* stream, QuantizedActivation* a,
+                            bool decode_order = false) const;
+    /* forward_quantized (kernel_matmul.rs:750-812): out [rows, n] in a.x_type, the bits forward gives on the
+     * rows `a` was made from. LK_NOT_TAKEN where forward would take another path. */
+    int forward_quantized(const QuantizedActivation& a, void* out, void* stream, bool decode_order = false);
+    /* forward_quantized_pair (kernel_matmul.rs:814-876): this weight and `other` over ONE f32-born activation
+     * row in one launch, each output with the bits of its own forward_quantized. LK_NOT_TAKEN where the pair
+     * is not two weights of one format and one k on one card that the mat-vec family serves together. */
+    int forward_quantized_pair(QKernelMatMul& other, const QuantizedActivation& a, void* out0, void* out1, void* stream);
+
     Path last_path() const { return last_path_; }
     int n() const { return n_; }
     int k() const { return k_; }
 
 private:
+    bool takes_matvec(int rows, bool decode_order) const;
     int dtype_, n_, k_, device_;
     const void* blob_;
     Path last_path_ = Path::None;
@@ -172,6 +198,14 @@ void lkh_qkernel_matmul_free(void* handle);
 int lkh_qkernel_matmul_forward(void* handle, const void* x, int x_type, int rows, void* out, void* stream,
                                int decode_order);
 int lkh_qkernel_matmul_last_path(void* handle);
+/* QuantizedActivation through plain pointers: the caller keeps (q81, x_type, rows) and passes them back. */
+size_t lkh_quantized_activation_bytes(int k, int rows);
+int lkh_qkernel_matmul_quantize_for_matvec(void* handle, const void* x, int x_type, int rows, void* q81, void* stream,
+                                           int decode_order);
+int lkh_qkernel_matmul_forward_quantized(void* handle, const void* q81, int x_type, int rows, void* out, void* stream,
+                                         int decode_order);
+int lkh_qkernel_matmul_forward_quantized_pair(void* handle, void* other, const void* q81, void* out0, void* out1,
+                                              void* stream);
 int lkh_matvec_rows(int dtype, int k);
 void lkh_release_workspaces(void);
 

@@ -333,6 +333,88 @@ int QKernelMatMul::forward(const void* x, int x_type, int rows, void* out, void*
     return LK_OK;
 }
 
+// takes_matvec of the reference (kernel_matmul.rs:1069-1075) with this mirror's own exceptions: the
+// K-quants' few rows over a large matrix go to the 16-row tiles, and the formats with tiles leave the
+// mat-vec launches from nibble_tiles_pay's row counts.
+bool QKernelMatMul::takes_matvec(int rows, bool decode_order) const {
+    if (!blob_ || rows < 1) return false;
+    if (decode_order && rows > 1) return true;
+    const bool plain = matvec_only(dtype_);
+    if (plain) return !nibble_tiles_pay(dtype_, n_, k_, rows) || rows <= matvec_rows(dtype_, k_);
+    if (rows > matvec_rows(dtype_, k_)) return false;
+    const bool rows_kernel_fits = k_ % 256 == 0 && ((uintptr_t)blob_ & (dtype_ == LK_TYPE_Q6_K ? 1 : 15)) == 0;
+    return !(rows_kernel_fits && small_rows_kernel_pays(dtype_, n_, k_, rows));
+}
+
+size_t QKernelMatMul::quantized_bytes(int k, int rows) {
+    return k > 0 && rows > 0 ? (size_t)rows * (pad_to((size_t)k, 512) / 32) * Q81_BLOCK : 0;
+}
+
+int QKernelMatMul::quantize_for_matvec(const void* x, int x_type, int rows, void* q81, void* stream, QuantizedActivation* a,
+                                       bool decode_order) const {
+    if (!x || !q81 || !a || rows <= 0) return LK_ERR_ARG;
+    if (x_type != LK_TYPE_F32 && x_type != LK_TYPE_F16 && x_type != LK_TYPE_BF16) return LK_ERR_TYPE;
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess || current != device_) {
+        (void)hipGetLastError();
+        return LK_ERR_ARG;
+    }
+    if (!takes_matvec(rows, decode_order)) return LK_NOT_TAKEN;
+    const int k_padded = (int)pad_to((size_t)k_, 512);
+    if (int rc = lk_quantize_q8_1(x, x_type, q81, k_, k_padded, rows, stream)) return rc;
+    a->q81 = q81;
+    a->k = k_;
+    a->rows = rows;
+    a->device = device_;
+    a->x_type = x_type;
+    return LK_OK;
+}
+
+int QKernelMatMul::forward_quantized(const QuantizedActivation& a, void* out, void* stream, bool decode_order) {
+    last_path_ = Path::None;
+    if (!a.q81 || !out) return LK_ERR_ARG;
+    if (a.k != k_ || a.device != device_ || !takes_matvec(a.rows, decode_order)) return LK_NOT_TAKEN;
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess || current != device_) {
+        (void)hipGetLastError();
+        return LK_ERR_ARG;
+    }
+    const int blocks = (int)pad_to((size_t)k_, 512) / 32;
+    for (int r0 = 0; r0 < a.rows; r0 += 8) {
+        const int b = a.rows - r0 < 8 ? a.rows - r0 : 8;
+        const int rc = lk_mmvq(dtype_, blob_, (const uint8_t*)a.q81 + (size_t)r0 * blocks * Q81_BLOCK,
+                               (uint8_t*)out + (size_t)r0 * n_ * elem_bytes(a.x_type), a.x_type, k_, n_, b, blocks, n_,
+                               nullptr, decode_order ? 1 : 0, stream);
+        if (rc) return rc;
+    }
+    last_path_ = Path::MatVec;
+    return LK_OK;
+}
+
+int QKernelMatMul::forward_quantized_pair(QKernelMatMul& other, const QuantizedActivation& a, void* out0, void* out1,
+                                          void* stream) {
+    last_path_ = other.last_path_ = Path::None;
+    if (!a.q81 || !out0 || !out1) return LK_ERR_ARG;
+    if (a.k != k_ || other.k_ != k_ || a.rows != 1 || a.x_type != LK_TYPE_F32 || dtype_ != other.dtype_ ||
+        device_ != other.device_ || a.device != device_ || !takes_matvec(1, false) || !other.takes_matvec(1, false))
+        return LK_NOT_TAKEN;
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess || current != device_) {
+        (void)hipGetLastError();
+        return LK_ERR_ARG;
+    }
+    const void* vx[2] = {blob_, other.blob_};
+    void* dst[2] = {out0, out1};
+    const int nn[2] = {n_, other.n_};
+    const int blocks = (int)pad_to((size_t)k_, 512) / 32;
+    const int rc = lk_mmvq_multi(dtype_, 2, vx, a.q81, dst, LK_TYPE_F32, k_, nn, 1, blocks, n_ > other.n_ ? n_ : other.n_, nullptr,
+                                 stream);
+    if (rc == LK_ERR_TYPE) return LK_NOT_TAKEN;   // a format without the several-matrices launch
+    if (rc) return rc;
+    last_path_ = other.last_path_ = Path::MatVec;
+    return LK_OK;
+}
+
 void release_workspaces() {
     std::lock_guard<std::mutex> lock(g_slots_mu);
     int current = 0;
@@ -370,6 +452,37 @@ extern "C" int lkh_qkernel_matmul_forward(void* handle, const void* x, int x_typ
 }
 extern "C" int lkh_qkernel_matmul_last_path(void* handle) {
     return handle ? (int)((loken::QKernelMatMul*)handle)->last_path() : 0;
+}
+extern "C" size_t lkh_quantized_activation_bytes(int k, int rows) { return loken::QKernelMatMul::quantized_bytes(k, rows); }
+extern "C" int lkh_qkernel_matmul_quantize_for_matvec(void* handle, const void* x, int x_type, int rows, void* q81, void* stream,
+                                                      int decode_order) {
+    if (!handle) return LK_ERR_ARG;
+    loken::QKernelMatMul::QuantizedActivation a;
+    return ((loken::QKernelMatMul*)handle)->quantize_for_matvec(x, x_type, rows, q81, stream, &a, decode_order != 0);
+}
+namespace {
+loken::QKernelMatMul::QuantizedActivation activation_of(const loken::QKernelMatMul& m, const void* q81, int x_type, int rows) {
+    loken::QKernelMatMul::QuantizedActivation a;
+    a.q81 = q81;
+    a.k = m.k();
+    a.rows = rows;
+    a.x_type = x_type;
+    (void)hipGetDevice(&a.device);   // the rows were quantized on the current card
+    return a;
+}
+}  // namespace
+extern "C" int lkh_qkernel_matmul_forward_quantized(void* handle, const void* q81, int x_type, int rows, void* out, void* stream,
+                                                    int decode_order) {
+    if (!handle) return LK_ERR_ARG;
+    if (x_type != LK_TYPE_F32 && x_type != LK_TYPE_F16 && x_type != LK_TYPE_BF16) return LK_ERR_TYPE;
+    auto* m = (loken::QKernelMatMul*)handle;
+    return m->forward_quantized(activation_of(*m, q81, x_type, rows), out, stream, decode_order != 0);
+}
+extern "C" int lkh_qkernel_matmul_forward_quantized_pair(void* handle, void* other, const void* q81, void* out0, void* out1,
+                                                         void* stream) {
+    if (!handle || !other) return LK_ERR_ARG;
+    auto* m = (loken::QKernelMatMul*)handle;
+    return m->forward_quantized_pair(*(loken::QKernelMatMul*)other, activation_of(*m, q81, LK_TYPE_F32, 1), out0, out1, stream);
 }
 extern "C" int lkh_matvec_rows(int dtype, int k) { return loken::matvec_rows(dtype, k); }
 extern "C" void lkh_release_workspaces(void) { loken::release_workspaces(); }

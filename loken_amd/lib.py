@@ -9,8 +9,8 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libloken_gfx950.so"
 
-LK_OK, LK_ERR_ARG, LK_ERR_TYPE, LK_ERR_LAUNCH, LK_ERR_NOMEM, LK_ERR_SIZE = 0, 1, 2, 3, 4, 5
-_ERR_NAMES = {1: "LK_ERR_ARG", 2: "LK_ERR_TYPE", 3: "LK_ERR_LAUNCH", 4: "LK_ERR_NOMEM", 5: "LK_ERR_SIZE"}
+LK_OK, LK_ERR_ARG, LK_ERR_TYPE, LK_ERR_LAUNCH, LK_ERR_NOMEM, LK_ERR_SIZE, LK_NOT_TAKEN = 0, 1, 2, 3, 4, 5, 6
+_ERR_NAMES = {1: "LK_ERR_ARG", 2: "LK_ERR_TYPE", 3: "LK_ERR_LAUNCH", 4: "LK_ERR_NOMEM", 5: "LK_ERR_SIZE", 6: "LK_NOT_TAKEN"}
 STATIC_SCRATCH_BYTES = 8 << 20
 
 TYPE_F32, TYPE_F16, TYPE_BF16 = 0, 1, 30
@@ -102,6 +102,10 @@ SIGNATURES.update({
     "lkh_qkernel_matmul_forward": (_i, [_vp, _vp, _i, _i, _vp, _vp, _i]),
     "lkh_qkernel_matmul_last_path": (_i, [_vp]),
     "lkh_matvec_rows": (_i, [_i, _i]),
+    "lkh_quantized_activation_bytes": (C.c_size_t, [_i, _i]),
+    "lkh_qkernel_matmul_quantize_for_matvec": (_i, [_vp, _vp, _i, _i, _vp, _vp, _i]),
+    "lkh_qkernel_matmul_forward_quantized": (_i, [_vp, _vp, _i, _i, _vp, _vp, _i]),
+    "lkh_qkernel_matmul_forward_quantized_pair": (_i, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "lkh_release_workspaces": (None, []),
     "lkh_gguf_open": (_vp, [_cp, _vp, _i]),
     "lkh_gguf_over": (_vp, [_vp, _u64, _vp, _i]),

@@ -785,6 +785,58 @@ def rows_sweep(args, dev):
                 None, {"table": table})
 
 
+# ---------------------------------------------------------------------------- prefill-layer
+def prefill_layer(args, dev):
+    """The quantized linears of one Llama-3-8B layer (Q4_K_M: q, k, v, o, gate, up Q4_K; down Q6_K) at
+    `--tokens` rows, each through the host mirror of QKernelMatMul::forward (which picks the kernel
+    family by row count), over `--layers` layers with their own weights, as one HIP graph."""
+    L = lib.load()
+    m = args.tokens
+    hidden, kv, ffn = 4096, 1024, 14336
+    linears = [("q", Q4K, hidden, hidden, "x"), ("k", Q4K, kv, hidden, "x"), ("v", Q4K, kv, hidden, "x"),
+               ("o", Q4K, hidden, hidden, "attn"), ("gate", Q4K, ffn, hidden, "x2"), ("up", Q4K, ffn, hidden, "x2"),
+               ("down", Q6K, hidden, ffn, "h")]
+    layers = max(1, args.layers)
+    mk = Maker(dev)
+    acts = {"x": mk.randn(m, hidden), "attn": mk.randn(m, hidden), "x2": mk.randn(m, hidden), "h": mk.randn(m, ffn)}
+    paths = {1: "matvec-fused", 2: "matvec", 3: "rows-on-matrix-unit", 4: "tiled"}
+    keep, handles, per_layer = [], [], []
+    for _ in range(layers):
+        row = []
+        for name, wtype, n, k, src in linears:
+            w = mk.make(wtype, n, k)
+            out = torch.empty((m, n), device=dev)
+            h = L.lkh_qkernel_matmul_new(wtype, n, k, w.data_ptr(), dev.index or 0)
+            keep.extend([w, out])
+            handles.append(h)
+            row.append((name, h, acts[src], out, wtype, n, k))
+        per_layer.append(row)
+
+    def one(h, x, out):
+        check(L.lkh_qkernel_matmul_forward(h, x.data_ptr(), lib.TYPE_F32, m, out.data_ptr(),
+                                           torch.cuda.current_stream().cuda_stream, 0), "lkh_qkernel_matmul_forward")
+
+    def step():
+        for row in per_layer:
+            for _, h, x, out, *_ in row:
+                one(h, x, out)
+
+    us = time_replays(capture(step), max(20, args.launches))
+    table = []
+    for name, h, x, out, wtype, n, k in per_layer[0]:
+        t = float(np.median(time_replays(capture(lambda: one(h, x, out)), 50)))
+        table.append({"linear": name, "wtype": NAMES[wtype], "n": n, "k": k, "us": round(t, 1),
+                      "path": paths.get(L.lkh_qkernel_matmul_last_path(h), "none"),
+                      "tops": round(2.0 * m * n * k / t / 1e6, 1)})
+    for h in handles:
+        L.lkh_qkernel_matmul_free(h)
+    ops_layer = sum(2.0 * m * n * k for _, _, n, k, _ in linears)
+    med = float(np.median(us)) / layers
+    return line(args, ops_layer / med / 1e6, "TOP/s", med * 1e-3, "int8 / f16 operands (exact integers), f32 accumulate",
+                {"workload": f"Llama-3-8B layer, quantized linears at {m} rows through forward(), {layers} layers a graph replay"},
+                None, {"per_layer_us": spread(us / layers), "ops_per_layer": ops_layer, "linears": table})
+
+
 def run(args) -> int:
     if not torch.cuda.is_available():
         raise SystemExit("bench.py: no GPU visible")
@@ -792,4 +844,4 @@ def run(args) -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     return {"gemv": gemv, "gemv-4096": gemv_4096, "mmq": mmq, "moe": moe_block, "decode-1p7b": decode_1p7b,
-            "rows-sweep": rows_sweep}[args.workload](args, dev)
+            "rows-sweep": rows_sweep, "prefill-layer": prefill_layer}[args.workload](args, dev)

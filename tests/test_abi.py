@@ -13,7 +13,7 @@ def declared_symbols():
     host = (ROOT / "include" / "loken_host.hpp").read_text()
     text += host[host.index('extern "C" {'):]
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(?:int|void\s*\*?)\s*(\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(?:int|size_t|void\s*\*?)\s*(\w+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():

@@ -206,3 +206,72 @@ def test_rows_too_long_for_the_matrix_unit_rows_kernel_go_to_the_tiles():
         lin.close()
     with pytest.raises(lib.LokenError):
         ops.dense_q4k_rows(dev(w), dev(x), n)
+
+
+@pytest.mark.parametrize("name,rows,n", [("q4_k", 1, 300), ("q4_k", 2, 300), ("q4_k", 7, 300), ("q6_k", 5, 260), ("q8_0", 12, 200),
+                                        ("q5_k", 1, 130), ("q4_0", 6, 200), ("q3_k", 3, 200)])
+@pytest.mark.parametrize("xt", [torch.float32, torch.float16])
+def test_an_activation_quantized_once_serves_several_weights_with_the_bits_of_forward(name, rows, n, xt):
+    # quantize_for_matvec / forward_quantized of the reference (src/tensor/quantized/kernel_matmul.rs:695-812):
+    # the Q8_1 rows are made once and every weight over them returns what its own forward returns
+    l = lib.load()
+    wtype, k = DT[name], 1024
+    lins = [Linear(wtype, dev(synth.weight(wtype, n + 8 * i, k, seed=90 + i, stream=1)), n + 8 * i, k) for i in range(2)]
+    x = dev(synth.activation(rows, k, seed=90)).to(xt)
+    q81 = torch.empty(l.lkh_quantized_activation_bytes(k, rows), dtype=torch.uint8, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    try:
+        assert l.lkh_qkernel_matmul_quantize_for_matvec(lins[0].h, x.data_ptr(), X_TYPES[xt], rows, q81.data_ptr(), s, 0) == 0
+        for lin in lins:
+            out = torch.empty((rows, lin.n), dtype=xt, device="cuda")
+            assert l.lkh_qkernel_matmul_forward_quantized(lin.h, q81.data_ptr(), X_TYPES[xt], rows, out.data_ptr(), s, 0) == 0
+            assert lin.path == "matvec"
+            assert torch.equal(out, lin(x))
+    finally:
+        for lin in lins:
+            lin.close()
+
+
+def test_a_pair_of_weights_over_one_quantized_row_in_one_launch():
+    # forward_quantized_pair (kernel_matmul.rs:814-876): one f32-born row, two weights of one format and k
+    l = lib.load()
+    k = 2048
+    a = Linear(lib.TYPE_Q4_K, dev(synth.weight(lib.TYPE_Q4_K, 520, k, seed=91, stream=1)), 520, k)
+    b = Linear(lib.TYPE_Q4_K, dev(synth.weight(lib.TYPE_Q4_K, 136, k, seed=92, stream=1)), 136, k)
+    c = Linear(lib.TYPE_Q6_K, dev(synth.weight(lib.TYPE_Q6_K, 136, k, seed=93, stream=1)), 136, k)
+    x = dev(synth.activation(1, k, seed=91))
+    q81 = torch.empty(l.lkh_quantized_activation_bytes(k, 1), dtype=torch.uint8, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    try:
+        assert l.lkh_qkernel_matmul_quantize_for_matvec(a.h, x.data_ptr(), lib.TYPE_F32, 1, q81.data_ptr(), s, 0) == 0
+        oa, ob = torch.empty((1, 520), device="cuda"), torch.empty((1, 136), device="cuda")
+        assert l.lkh_qkernel_matmul_forward_quantized_pair(a.h, b.h, q81.data_ptr(), oa.data_ptr(), ob.data_ptr(), s) == 0
+        assert torch.equal(oa, a(x)) and torch.equal(ob, b(x))
+        # two formats do not pair: the reference's None
+        assert l.lkh_qkernel_matmul_forward_quantized_pair(a.h, c.h, q81.data_ptr(), oa.data_ptr(), ob.data_ptr(), s) == lib.LK_NOT_TAKEN
+    finally:
+        for lin in (a, b, c):
+            lin.close()
+
+
+def test_rows_that_forward_serves_another_way_are_not_quantized_for_the_matvec():
+    l = lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    k = 1024
+    x = dev(synth.activation(40, k, seed=94))
+    q81 = torch.empty(l.lkh_quantized_activation_bytes(k, 40), dtype=torch.uint8, device="cuda")
+    out = torch.empty((40, 4000), device="cuda")
+    big = Linear(lib.TYPE_Q4_K, dev(synth.weight(lib.TYPE_Q4_K, 4000, k, seed=94, stream=1)), 4000, k)
+    try:
+        # 40 rows go to the matrix-unit kernels, 4 rows over this matrix to the 16-row tiles
+        for rows in (40, 4):
+            assert l.lkh_qkernel_matmul_quantize_for_matvec(big.h, x.data_ptr(), lib.TYPE_F32, rows, q81.data_ptr(), s, 0) == lib.LK_NOT_TAKEN
+            assert l.lkh_qkernel_matmul_forward_quantized(big.h, q81.data_ptr(), lib.TYPE_F32, rows, out.data_ptr(), s, 0) == lib.LK_NOT_TAKEN
+        # in decode order every row count stays on the mat-vec kernels
+        assert l.lkh_qkernel_matmul_quantize_for_matvec(big.h, x.data_ptr(), lib.TYPE_F32, 40, q81.data_ptr(), s, 1) == 0
+        assert l.lkh_qkernel_matmul_forward_quantized(big.h, q81.data_ptr(), lib.TYPE_F32, 40, out.data_ptr(), s, 1) == 0
+        assert torch.equal(out, big(x, decode_order=True))
+        assert l.lkh_qkernel_matmul_quantize_for_matvec(big.h, x.data_ptr(), 77, 2, q81.data_ptr(), s, 0) == lib.LK_ERR_TYPE
+        assert l.lkh_qkernel_matmul_quantize_for_matvec(big.h, None, lib.TYPE_F32, 2, q81.data_ptr(), s, 0) == lib.LK_ERR_ARG
+    finally:
+        big.close()
