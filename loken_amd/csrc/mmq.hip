@@ -978,7 +978,9 @@ static int launch_dense(void* fixup, const void* x, const void* y, void* dst, in
     // is 3 to 40 % faster on the wide tile)
     if (ncols_y <= 64 || F::MIN_RANK == 16) return launch_dense_tm<F, 64, 2>(pb, s, fixup);
     if constexpr (F::F16_TILES) {   // Q4_K: scales folded into f16 operands
-        if (!lk_env_flag("LK_MMQ_I8")) {
+        // (under 2048 weight rows the 256-row f16 tiles are too few even with K cut: 1024 x 4096 at 512 / 1024 /
+        // 2048 rows 48 / 63 / 93 us against 38 / 49 / 73 on the int8 tiles)
+        if (!lk_env_flag("LK_MMQ_I8") && nrows_x >= 2048) {
             // 128-token tiles with the token side expanded once per call, where they pad the rows at most a
             // tenth more than the 64-token tiles would (512 x 4096 -> 14336: 105 us against 123) and are
             // enough to occupy half the CUs (fewer: the 64-token tiles, which can cut K)

@@ -457,7 +457,7 @@ def decode_1p7b(args, dev):
     used = {"rows": 0, "matvec": 0, "tiled": 0}
 
     def rows_kernel_serves(wtype, n, k, rows):   # the rule of host_qmatmul.hip
-        return rows <= 16 or n * rows * max(k, 4096) <= 450000 * 4096
+        return rows <= 16 or n * rows * max(k, 4096) <= 450000 * 4096 * (2048 // max(n, 1) if n < 2048 else 1)
 
     # 3 to 16 rows: the 16-row-tile kernels on the matrix unit, the matrices that share an activation in
     # one launch (q + k + v; gate + up with the activation on top, as dense_q4k_imma_m8_act_mul of the
