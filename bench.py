@@ -37,8 +37,9 @@ Two more measurements ride in the same JSON line:
                 rows kernel against the tiled matmul, and the path QKernelMatMul::forward's mirror takes.
   prefill-layer the quantized linears of one Llama-3-8B layer at --tokens rows, each through the host mirror of
                 QKernelMatMul::forward (--layers of them, each with its own weights, a graph replay).
-  other_configs the step at 4 and 8 rows, the MoE block at 1 / 16 / 256 tokens and the Qwen3-1.7B step at
-                1 / 16 / 64 rows (configurations 1, 3, 4), each from a child run of this file.
+  other_configs the step at 4 and 8 rows, the MoE block at 1 / 16 / 256 tokens, the Qwen3-1.7B step at
+                1 / 16 / 64 rows (configurations 1, 3, 4) and a Llama-3-8B layer's linears at 128 / 512 rows
+                through forward(), each from a child run of this file.
   roofline.peak_measured / mmq.peak_measured: what a read-only launch and a register-resident
                 matrix-instruction loop reach on this card (loken_amd/probes.py).
 """
@@ -124,9 +125,11 @@ def other_configs():
                     if "whole_step" in d:
                         out["whole_step_gbs"] = d["whole_step"]["gbs"]
                         out["spread"] = d["whole_step"]["per_step"]
-                    for key in ("step_spread", "block_in_step_graph"):
+                    for key in ("step_spread", "block_in_step_graph", "per_layer_us"):
                         if key in d:
                             out["spread"] = d[key]
+                    if "linears" in d:
+                        out["linears_us"] = {r["linear"]: [r["us"], r["path"]] for r in d["linears"]}
                     if d.get("roofline"):
                         out["roofline"] = {k: d["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac") if k in d["roofline"]}
                     return out
@@ -140,6 +143,8 @@ def other_configs():
         "llama3_8b_step_by_rows": {str(b): child(["--brief", "--batch", str(b)]) for b in (4, 8)},
         "moe_block_128x2048x768_top8_by_tokens": {str(t): child(["--workload", "moe", "--tokens", str(t)]) for t in (1, 16, 256)},
         "qwen3_1p7b_step_by_rows": {str(b): child(["--workload", "decode-1p7b", "--batch", str(b)]) for b in (1, 16, 64)},
+        "llama3_8b_layer_linears_through_forward_by_rows": {
+            str(t): child(["--workload", "prefill-layer", "--tokens", str(t), "--layers", "4"]) for t in (128, 512)},
     }
 
 
