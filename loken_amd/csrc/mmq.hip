@@ -116,7 +116,7 @@ struct MmqQ45K {
     static constexpr int ALIGN = 4;   // whole-header reads
     static constexpr int BLOCK_BYTES = Q5 ? Q5K_BYTES : Q4K_BYTES;
     static constexpr int QS0 = Q5 ? 48 : 16;
-    static constexpr bool F16_TILES = !Q5;   // Q4_K above 64 tokens: the f16 tile kernel
+    static constexpr bool F16_TILES = !Q5;   // Q4_K above 32 tokens (dense) or 64 (expert-batched): the f16 tile kernels
     static constexpr int WIDE_FROM = 384;   // 128-token tiles from this many of them (launch_dense)
     static constexpr int NS = 8;          // one weight scale per 32 values
     static constexpr bool HAS_MIN = true;
@@ -976,7 +976,10 @@ static int launch_dense(void* fixup, const void* x, const void* y, void* dst, in
     // (Q2_K stays on 64-token tiles: with the rank-16 minimum its 128-token tile spills and runs 512 x
     // 4096 -> 14336 in 344 us against 240, 2048 x 14336 -> 4096 in 1155 against 742; every other format
     // is 3 to 40 % faster on the wide tile)
-    if (ncols_y <= 64 || F::MIN_RANK == 16) return launch_dense_tm<F, 64, 2>(pb, s, fixup);
+    // (Q4_K from 33 rows of a matrix of 2048 rows or more goes on to its 64-token f16 tiles: 14336 x 4096 at 64
+    // rows 40.5 us against 46.4 on the int8 tiles, 4096 x 14336 43.8 against 49.1, 4096 x 4096 the same 33)
+    const bool f16_from_33 = F::F16_TILES && nrows_x >= 2048 && !lk_env_flag("LK_MMQ_I8");
+    if ((ncols_y <= 64 && !f16_from_33) || F::MIN_RANK == 16) return launch_dense_tm<F, 64, 2>(pb, s, fixup);
     if constexpr (F::F16_TILES) {   // Q4_K: scales folded into f16 operands
         // (under 2048 weight rows the 256-row f16 tiles are too few even with K cut: 1024 x 4096 at 512 / 1024 /
         // 2048 rows 48 / 63 / 93 us against 38 / 49 / 73 on the int8 tiles)

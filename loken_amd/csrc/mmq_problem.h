@@ -61,7 +61,7 @@ static inline int mmq_splits(const MmqProblem& pb, int64_t tiles, int64_t slots,
 // dst[token][c] = part[0][token][c] + part[1][token][c] + ..., part[i] m_end x n floats; LK_* status.
 int lk_mmq_split_sum(const float* part, int splits, const MmqProblem& pb, hipStream_t s);
 
-// Q4_K against 65 or more token rows (mmq_q4k_f16.hip); `fixup`: the caller's tmp_fixup or null. Return the token-tile width launched,
+// Q4_K against 33 or more token rows (mmq_q4k_f16.hip); `fixup`: the caller's tmp_fixup or null. Return the token-tile width launched,
 // 0 when the launch failed, -1 when the operands do not suit these kernels (16-byte alignment,
 // 32-bit record offsets) and the caller should take the int8 tiles.
 int lk_mmq_q4k_f16_dense(const MmqProblem& pb, hipStream_t s, void* fixup);

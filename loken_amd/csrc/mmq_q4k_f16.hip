@@ -1,4 +1,4 @@
-// Q4_K weight rows against 65 or more Q8_1 token rows: the sub-block dots on the f16 matrix unit.
+// Q4_K weight rows against 33 or more Q8_1 token rows (65 or more where they are an expert's run): the sub-block dots on the f16 matrix unit.
 //
 //   out[token, n] = sum over 256-value blocks of
 //        d[n] * sum_s d8_s[token] * D_s[n, token]  -  dmin[n] * sum_s m_s[n] * (d8_s * S_s)[token]

@@ -118,6 +118,23 @@ def test_cut_k_follows_the_oracle_and_the_plain_launch(name, m, k, n):
     assert (cut - plain).abs().max().item() <= 2e-5 * plain.abs().max().item()
 
 
+@pytest.mark.parametrize("m,k,n", [(100, 1280, 2052), (40, 1792, 2304), (200, 3584, 2048)])
+def test_cut_k_on_the_f16_tiles_of_q4k_follows_the_oracle(m, k, n):
+    # 2048 weight rows or more and 33 token rows or more: the 64-token f16 tiles, here few enough to have K
+    # cut (5, 7 and 14 blocks: uneven ranges)
+    wtype = lib.TYPE_Q4_K
+    wh = synth.weight(wtype, n, k, seed=49, stream=8)
+    xh = synth.activation(m, k, seed=49)
+    w, x = dev(wh), dev(xh)
+    plain = ops.mmq_forward(wtype, w, x, n, fixup=False)
+    cut = ops.mmq_forward(wtype, w, x, n)
+    assert torch.equal(cut, ops.mmq_forward(wtype, w, x, n))
+    assert not torch.equal(cut, plain)
+    pick = np.sort(np.random.default_rng(49).choice(n, 256, replace=False))
+    assert_close(cut.cpu().numpy()[:, pick], oracle.ob_matmul(wtype, xh, wh[pick], len(pick)))
+    assert (cut - plain).abs().max().item() <= 2e-5 * plain.abs().max().item()
+
+
 @pytest.mark.parametrize("name,splits", [("q4_k", 3), ("q6_k", 7), ("q8_0", 2), ("q4_k", 64)])
 def test_forced_range_counts_and_what_keeps_k_whole(name, splits, knobs):
     # LK_TUNE_MMQ_SPLITS asks for a range count (capped so that a range keeps two blocks); -1, no buffer,
@@ -140,11 +157,13 @@ def test_forced_range_counts_and_what_keeps_k_whole(name, splits, knobs):
     assert torch.equal(ops.mmq_forward(wtype, w_odd, x, 130), ops.mmq_forward(wtype, w_odd, x, 130, fixup=False))
 
 
-@pytest.mark.parametrize("m,k,n", [(65, 256, 33), (130, 2048, 520), (300, 1024, 128)])
+@pytest.mark.parametrize("m,k,n", [(65, 256, 2049), (40, 512, 2050), (130, 2048, 2056), (300, 1024, 2304), (500, 512, 8450)])
 def test_q4k_wide_tiles_agree_with_int8_tiles_and_matvec(m, k, n, knobs):
-    # Above 64 token rows Q4_K forms its sub-block dots on the f16 matrix unit (scale folded into
-    # the weight operand); LK_MMQ_I8 sends the same call to the int8 tiles. Same integers either
-    # way, so only the f32 summation order may differ.
+    # Above 32 token rows of a matrix of 2048 rows or more Q4_K forms its sub-block dots on the f16 matrix
+    # unit (scale folded into the weight operand; 64-token tiles, K cut into ranges where they are few; the
+    # last shape has enough 128-token tiles for the kernel that expands the token side once per call);
+    # LK_MMQ_I8 sends the same call to the int8 tiles. Same integers either way, so only the f32
+    # summation order may differ.
     wtype = lib.TYPE_Q4_K
     w = dev(synth.weight(wtype, n, k, seed=46, stream=4))
     x = dev(synth.activation(m, k, seed=46))
