@@ -135,6 +135,37 @@ def test_cut_k_on_the_f16_tiles_of_q4k_follows_the_oracle(m, k, n):
     assert (cut - plain).abs().max().item() <= 2e-5 * plain.abs().max().item()
 
 
+@pytest.mark.parametrize("name,m,k,n", [("q6_k", 48, 2048, 260), ("q4_k", 100, 1792, 2304)])
+def test_cut_k_recorded_into_a_graph_replays_to_the_eager_bits(name, m, k, n):
+    # The cut-K call is two launches and nothing else (no fill, no allocation): recorded into a HIP graph
+    # and replayed three times, with eager calls of another size through the same tmp_fixup between the
+    # replays, every replay carries the eager call's bits.
+    wtype = DT[name]
+    w = dev(synth.weight(wtype, n, k, seed=50, stream=9))
+    x = dev(synth.activation(m, k, seed=50))
+    want = ops.mmq_forward(wtype, w, x, n)
+    assert not torch.equal(want, ops.mmq_forward(wtype, w, x, n, fixup=False))   # K was cut
+    ws = ops.mmq_quantize(wtype, x)
+    out = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    fn = getattr(lib.load(), ops.MMQ_LAUNCHER[wtype])
+    i = ops.MMQ_DEVICE_INFO
+    fix = ops.mmq_fixup(x.device)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            launched = fn(fix.data_ptr(), w.data_ptr(), ws.data_ptr(), out.data_ptr(), k, n, m, k // synth.BLOCK_LEN[wtype], n,
+                          i["cc"], i["nsm"], i["smpbo"], i["warp_size"], side.cuda_stream)
+    assert launched != 0
+    torch.cuda.synchronize()
+    for replay in range(3):
+        out.fill_(7.0)
+        ops.mmq_forward(wtype, w, x[: m // 2].contiguous(), n)   # the program's own work through the same buffer
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {replay}"
+
+
 @pytest.mark.parametrize("name,splits", [("q4_k", 3), ("q6_k", 7), ("q8_0", 2), ("q4_k", 64)])
 def test_forced_range_counts_and_what_keeps_k_whole(name, splits, knobs):
     # LK_TUNE_MMQ_SPLITS asks for a range count (capped so that a range keeps two blocks); -1, no buffer,
