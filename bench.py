@@ -78,6 +78,11 @@ def parse_args():
                          "launch, gate + up in one); auto: fused at one or two rows, except that rows longer than 8192 "
                          "values are quantized by their own launch (every workgroup of a fused launch quantizes the "
                          "whole row), and rows from three rows on")
+    ap.add_argument("--acts", choices=["f32", "norm-q8_1"], default="f32",
+                    help="the rows plan of the step and --workload decode-1p7b above two rows: f32 rows into every group "
+                         "(a Q8_1 quantizer launch each), or q + k + v and gate + up reading Q8_1 rows as a model's "
+                         "RMSNorm launches that also quantize (lk_rmsnorm_q8_1, lk_add_rmsnorm_q8_1) leave them: those "
+                         "launches are the norms' and are not timed, o keeps its quantizer")
     ap.add_argument("--no-graph", action="store_true", help="launch the step eagerly instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=20.0,
                     help="wall-clock budget of the CPU baseline samples together (mat-vec 40 %, prefill 30 %, expert block 30 %)")
@@ -143,6 +148,10 @@ def other_configs():
         "llama3_8b_step_by_rows": {str(b): child(["--brief", "--batch", str(b)]) for b in (4, 8)},
         "moe_block_128x2048x768_top8_by_tokens": {str(t): child(["--workload", "moe", "--tokens", str(t)]) for t in (1, 16, 256)},
         "qwen3_1p7b_step_by_rows": {str(b): child(["--workload", "decode-1p7b", "--batch", str(b)]) for b in (1, 16, 64)},
+        "same_steps_with_q8_1_rows_from_the_norms": {
+            "llama3_8b_8_rows": child(["--brief", "--batch", "8", "--acts", "norm-q8_1"]),
+            "qwen3_1p7b_16_rows": child(["--workload", "decode-1p7b", "--batch", "16", "--acts", "norm-q8_1"]),
+            "qwen3_1p7b_64_rows": child(["--workload", "decode-1p7b", "--batch", "64", "--acts", "norm-q8_1"])},
         "llama3_8b_layer_linears_through_forward_by_rows": {
             str(t): child(["--workload", "prefill-layer", "--tokens", str(t), "--layers", "4"]) for t in (128, 512)},
     }
@@ -222,10 +231,16 @@ def main() -> int:
     q4k_bytes = 0
     keep = []
 
-    def add_quant(g):
+    def add_quant(g, from_norm=False):
         a, q = acts[g], q81[g]
-        plan.append((L.lk_quantize_q8_1, (a.data_ptr(), lib.TYPE_F32, q.data_ptr(), a.shape[1],
-                                          q.shape[1] * 32, b, stream)))
+        item = (L.lk_quantize_q8_1, (a.data_ptr(), lib.TYPE_F32, q.data_ptr(), a.shape[1], q.shape[1] * 32, b, stream))
+        if from_norm and args.acts == "norm-q8_1":
+            # the rows arrive quantized: written once here, outside the step
+            rc = item[0](*item[1])
+            if rc:
+                raise lib.LokenError("lk_quantize_q8_1", rc)
+            return
+        plan.append(item)
 
     def add_gemv(wtype, w, g, n, k):
         nonlocal total_bytes, q4k_bytes
@@ -366,13 +381,13 @@ def main() -> int:
             # quantizer launch wrote
             made = {name: (maker(n, k), wtype, n, k, g) for name, wtype, n, k, maker, g in shapes}
             keep.extend(v[0] for v in made.values())
-            add_quant("x")
+            add_quant("x", from_norm=True)
             out = add_rows_multi([made[nm][0] for nm in ("q", "k", "v")], "x", [made[nm][2] for nm in ("q", "k", "v")], HIDDEN)
             if first_out is None:
                 first_out, first_w = out, made["q"][0]
             add_quant("attn")
             add_rows(made["o"][0], "attn", HIDDEN, HIDDEN)
-            add_quant("x2")
+            add_quant("x2", from_norm=True)
             if b <= 16:
                 # gate + up hands its result on as the Q8_1 rows `down` reads: no f32 round trip, no quantizer launch
                 count_q4k((L.lk_dense_q4k_rows_actmul_q8_1, (made["gate"][0].data_ptr(), made["up"][0].data_ptr(), q81["x2"].data_ptr(),
@@ -563,7 +578,11 @@ def main() -> int:
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"llama3-8b decode-step quantized linears (Q4_K q,k,v,o,gate,up; Q6_K down; "
                                f"Q8_0 lm_head), batch {b}, {args.layers} layers",
-                   "launch_plan": args.plan if kind == args.plan else f"{args.plan} -> {kind}", "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
+                   "launch_plan": args.plan if kind == args.plan else f"{args.plan} -> {kind}",
+                   "acts": "f32 rows into every group" if args.acts == "f32" or kind != "rows"
+                           else "q + k + v and gate + up read Q8_1 rows as the model's RMSNorm launches that also quantize "
+                                "leave them (those launches are not timed); o from f32 rows",
+                   "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),
                    "hip_graph": used_graph},
         "value_is": "Q4_K weight bytes of the step over the time of its Q4_K mat-vec launches (the roofline leg); "
                     "ms_per_step and whole_step are the whole step, Q6_K and Q8_0 matrices included",

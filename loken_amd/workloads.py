@@ -471,6 +471,15 @@ def decode_1p7b(args, dev):
                  if (not fused_rows and not matvec and args.mid_rows == "auto" and rows_kernel_serves(Q4K, ffn, hidden, b)
                      and rows_kernel_serves(Q6K, hidden, ffn, b)) else None)
 
+    def quantize_or_take(g, x, q, k):
+        """The Q8_1 rows of group `g`: a quantizer launch of the step, or (--acts norm-q8_1, the groups a norm
+        feeds) written once here, as the model's RMSNorm launch that also quantizes would leave them."""
+        item = ("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s))
+        if getattr(args, "acts", "f32") == "norm-q8_1" and g in ("x", "x2"):
+            check(item[1](*item[2]), "lk_quantize_q8_1")
+            return
+        plan.append(item)
+
     def add_fused_rows(g, k, wtype, ns):
         nonlocal total_bytes
         weights = [mk.make(wtype, n, k) for n in ns]
@@ -491,7 +500,7 @@ def decode_1p7b(args, dev):
             return
         q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
         keep.append(q)
-        plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s)))
+        quantize_or_take(g, x, q, k)
         if wtype == Q6K:
             for w, n in zip(weights, ns):
                 out = torch.empty((b, n), device=dev)
@@ -557,7 +566,7 @@ def decode_1p7b(args, dev):
                 return
             q = torch.empty((b, k // 32, 36), dtype=torch.uint8, device=dev)
             keep.append(q)
-            plan.append(("status", L.lk_quantize_q8_1, (x.data_ptr(), lib.TYPE_F32, q.data_ptr(), k, k, b, s)))
+            quantize_or_take(g, x, q, k)
             if g == "x2" and wtype == Q4K:
                 # gate and up with the activation on top in one launch (dense_q4k_imma_m8_act_mul of the reference),
                 # its result handed on as the Q8_1 rows `down` reads
@@ -646,6 +655,9 @@ def decode_1p7b(args, dev):
                               "the Q8_1 rows down reads, down, lm_head; a Q8_1 quantizer launch before the others" if fused_rows
                          else f"linears on the matrix-unit rows kernels: {used['rows']}, as mat-vec slices of eight rows: "
                               f"{used['matvec']}, on the tiled matmul: {used['tiled']}",
+                 "acts": "f32 rows into every group" if getattr(args, "acts", "f32") == "f32" or matvec
+                         else "q + k + v and gate + up read Q8_1 rows as the model's RMSNorm launches that also quantize leave them "
+                              "(those launches are not timed); o and lm_head from f32 rows",
                  "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline,
                 {"step_spread": spread(us), "ms_per_step_is": "median of the timed replays"})
 
