@@ -35,7 +35,7 @@ enum class Path : int {
  * of the matrix-unit rows kernels from 3 f32 rows on (Q4_K / Q5_K: n x rows of 57344, or 8192 at
  * k <= 2048; Q6_K: n x k of 48 Mi with k a multiple of 2048); then the matrix-unit rows kernels up to
  * 16 rows, or while n x rows x max(k, 4096) / 4096 <= 450 000 (twice that for a matrix of 1024 rows, and so
- * on: few rows yield few tiles; below that even a tiled launch with K cut
+ * on: few rows yield few tiles; Q4_K / Q5_K rows of 8192 values or more leave them from 9 rows; below that even a tiled launch with K cut
  * into ranges does not beat them), then the tiled matmul; Q8_0 mat-vec slices up to 16 rows, then the
  * tiled matmul; the 32-value nibble formats, Q3_K and Q2_K mat-vec slices up to 15 rows, or 8 over a
  * matrix of 48 Mi weights or more, then the tiled matmul). */

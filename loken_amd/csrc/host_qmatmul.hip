@@ -195,6 +195,10 @@ static bool rows_kernel_serves(int dtype, int n, int k, int rows) {
     // (a matrix of fewer than 2048 rows yields few tiles whatever the cut: Q4_K 1024 x 4096 at 512 rows 38 us
     // against 38, at 1024 rows 55 against 49)
     const long long few = n < 2048 ? 2048 / (n > 0 ? n : 1) : 1;
+    // (Q4_K / Q5_K rows of 8192 values or more at 9 to 16 activation rows: the 16-row tiles' second set of eight
+    // costs them more than the cut K costs the tiled launch: 4096 x 14336 at 9 / 16 rows 42 / 46 us against 37,
+    // Q5_K 44 / 48 against 38; 4096 x 8192 31 / 33 against 30. Q6_K keeps its 16-row tiles: 38 against 40)
+    if (dtype != LK_TYPE_Q6_K && rows > 8 && rows <= 16 && k >= 8192 && n >= 2048) return false;
     return rows <= 16 || (long long)n * rows * (k > 4096 ? k : 4096) <= 450000ll * 4096 * few;
 }
 

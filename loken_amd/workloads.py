@@ -457,6 +457,8 @@ def decode_1p7b(args, dev):
     used = {"rows": 0, "matvec": 0, "tiled": 0}
 
     def rows_kernel_serves(wtype, n, k, rows):   # the rule of host_qmatmul.hip
+        if wtype != Q6K and 8 < rows <= 16 and k >= 8192 and n >= 2048:
+            return False
         return rows <= 16 or n * rows * max(k, 4096) <= 450000 * 4096 * (2048 // max(n, 1) if n < 2048 else 1)
 
     # 3 to 16 rows: the 16-row-tile kernels on the matrix unit, the matrices that share an activation in

@@ -275,3 +275,20 @@ def test_rows_that_forward_serves_another_way_are_not_quantized_for_the_matvec()
         assert l.lkh_qkernel_matmul_quantize_for_matvec(big.h, None, lib.TYPE_F32, 2, q81.data_ptr(), s, 0) == lib.LK_ERR_ARG
     finally:
         big.close()
+
+
+@pytest.mark.parametrize("name,rows,expect", [("q4_k", 12, "tiled"), ("q5_k", 16, "tiled"), ("q6_k", 12, "rows-on-matrix-unit"),
+                                               ("q4_k", 8, "matvec")])
+def test_long_rows_at_nine_to_sixteen_activation_rows(name, rows, expect):
+    # rows of 8192 values: Q4_K / Q5_K leave the 16-row tiles for the tiled matmul (K cut into ranges) from nine rows
+    wtype, n, k = DT[name], 2048, 8192
+    w = synth.weight(wtype, n, k, seed=96, stream=1)
+    x = synth.activation(rows, k, seed=96)
+    lin = Linear(wtype, dev(w), n, k)
+    try:
+        got = lin(dev(x))
+        assert lin.path == expect
+        pick = np.sort(np.random.default_rng(96).choice(n, 200, replace=False))
+        assert close(got.cpu().numpy()[:, pick], oracle.ob_matmul(wtype, x, w[pick], len(pick)))
+    finally:
+        lin.close()
