@@ -79,7 +79,7 @@ def parse_args():
                          "values are quantized by their own launch (every workgroup of a fused launch quantizes the "
                          "whole row), and rows from three rows on")
     ap.add_argument("--acts", choices=["f32", "norm-q8_1"], default="f32",
-                    help="the rows plan of the step and --workload decode-1p7b above two rows: f32 rows into every group "
+                    help="the step (plans auto, fused, rows) and --workload decode-1p7b from three rows: f32 rows into every group "
                          "(a Q8_1 quantizer launch each), or q + k + v and gate + up reading Q8_1 rows as a model's "
                          "RMSNorm launches that also quantize (lk_rmsnorm_q8_1, lk_add_rmsnorm_q8_1) leave them: those "
                          "launches are the norms' and are not timed, o keeps its quantizer")
@@ -149,7 +149,9 @@ def other_configs():
         "moe_block_128x2048x768_top8_by_tokens": {str(t): child(["--workload", "moe", "--tokens", str(t)]) for t in (1, 16, 256)},
         "qwen3_1p7b_step_by_rows": {str(b): child(["--workload", "decode-1p7b", "--batch", str(b)]) for b in (1, 16, 64)},
         "same_steps_with_q8_1_rows_from_the_norms": {
+            "llama3_8b_1_row": child(["--brief", "--acts", "norm-q8_1"]),
             "llama3_8b_8_rows": child(["--brief", "--batch", "8", "--acts", "norm-q8_1"]),
+            "qwen3_1p7b_1_row": child(["--workload", "decode-1p7b", "--batch", "1", "--acts", "norm-q8_1"]),
             "qwen3_1p7b_16_rows": child(["--workload", "decode-1p7b", "--batch", "16", "--acts", "norm-q8_1"]),
             "qwen3_1p7b_64_rows": child(["--workload", "decode-1p7b", "--batch", "64", "--acts", "norm-q8_1"])},
         "llama3_8b_layer_linears_through_forward_by_rows": {
@@ -270,8 +272,14 @@ def main() -> int:
         dst = (C.c_void_p * len(ws))(*[o.data_ptr() for o in outs])
         nn = (C.c_int * len(ws))(*ns)
         keep.extend(outs + [vx, dst, nn])
-        item = (L.lk_mmvq_fused, (wtype, len(ws), vx, a.data_ptr(), a.stride(0), dst, lib.TYPE_F32, k, nn, b,
-                                  stride, None, stream))
+        if args.acts == "norm-q8_1" and g in ("x", "x2") and k <= 8192:
+            # the group's rows arrive as Q8_1 (written once here, outside the step): the same launch over them
+            add_quant(g, from_norm=True)
+            q = q81[g]
+            item = (L.lk_mmvq_multi, (wtype, len(ws), vx, q.data_ptr(), dst, lib.TYPE_F32, k, nn, b, q.shape[1], stride, None, stream))
+        else:
+            item = (L.lk_mmvq_fused, (wtype, len(ws), vx, a.data_ptr(), a.stride(0), dst, lib.TYPE_F32, k, nn, b,
+                                      stride, None, stream))
         plan.append(item)
         nbytes = sum(synth.weight_bytes(wtype, n, k) for n in ns)
         total_bytes += nbytes
@@ -285,8 +293,13 @@ def main() -> int:
         """One launch: silu(gate . x) * (up . x) as Q8_1 rows in q81["h"] (which `down` then reads)."""
         nonlocal total_bytes, q4k_bytes
         a, q = acts[g], q81["h"]
-        item = (L.lk_mmvq_pair_act_q8_1, (wtype, gate.data_ptr(), up.data_ptr(), a.data_ptr(), 1, a.stride(0),
-                                          q.data_ptr(), q.shape[1], k, n, b, 0, stream))
+        if args.acts == "norm-q8_1":
+            add_quant(g, from_norm=True)
+            item = (L.lk_mmvq_pair_act_q8_1, (wtype, gate.data_ptr(), up.data_ptr(), q81[g].data_ptr(), 0, q81[g].shape[1],
+                                              q.data_ptr(), q.shape[1], k, n, b, 0, stream))
+        else:
+            item = (L.lk_mmvq_pair_act_q8_1, (wtype, gate.data_ptr(), up.data_ptr(), a.data_ptr(), 1, a.stride(0),
+                                              q.data_ptr(), q.shape[1], k, n, b, 0, stream))
         plan.append(item)
         nbytes = 2 * synth.weight_bytes(wtype, n, k)
         total_bytes += nbytes
@@ -579,7 +592,7 @@ def main() -> int:
         "config": {"workload": f"llama3-8b decode-step quantized linears (Q4_K q,k,v,o,gate,up; Q6_K down; "
                                f"Q8_0 lm_head), batch {b}, {args.layers} layers",
                    "launch_plan": args.plan if kind == args.plan else f"{args.plan} -> {kind}",
-                   "acts": "f32 rows into every group" if args.acts == "f32" or kind != "rows"
+                   "acts": "f32 rows into every group" if args.acts == "f32" or kind not in ("rows", "auto", "fused")
                            else "q + k + v and gate + up read Q8_1 rows as the model's RMSNorm launches that also quantize "
                                 "leave them (those launches are not timed); o from f32 rows",
                    "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan),

@@ -532,7 +532,16 @@ def decode_1p7b(args, dev):
         keep.extend(weights)
         total_bytes += sum(synth.weight_bytes(wtype, n, k) for n in ns)
         x = acts[g]
-        if paired and g == "x2":
+        from_norm = getattr(args, "acts", "f32") == "norm-q8_1" and g in ("x", "x2") and k <= 8192
+        if from_norm and matvec:
+            # the group's rows arrive as Q8_1, as the model's quantizing norm leaves them: written once here
+            qn = torch.empty((b, ops.pad_to(k, 512) // 32, 36), dtype=torch.uint8, device=dev)
+            keep.append(qn)
+            check(L.lk_quantize_q8_1(x.data_ptr(), lib.TYPE_F32, qn.data_ptr(), k, qn.shape[1] * 32, b, s), "lk_quantize_q8_1")
+        if paired and g == "x2" and from_norm:
+            plan.append(("status", L.lk_mmvq_pair_act_q8_1, (wtype, weights[0].data_ptr(), weights[1].data_ptr(), qn.data_ptr(), 0,
+                                                              qn.shape[1], h_q81.data_ptr(), h_q81.shape[1], k, ns[0], b, 0, s)))
+        elif paired and g == "x2":
             plan.append(("status", L.lk_mmvq_pair_act_q8_1, (wtype, weights[0].data_ptr(), weights[1].data_ptr(), x.data_ptr(), 1,
                                                               x.stride(0), h_q81.data_ptr(), h_q81.shape[1], k, ns[0], b, 0, s)))
         elif paired and g == "h":
@@ -547,8 +556,12 @@ def decode_1p7b(args, dev):
             dst = (lib.C.c_void_p * len(ns))(*[o.data_ptr() for o in outs])
             nn = (lib.C.c_int * len(ns))(*ns)
             keep.extend(outs + [vx, dst, nn])
-            plan.append(("status", L.lk_mmvq_fused, (wtype, len(ns), vx, x.data_ptr(), x.stride(0), dst, lib.TYPE_F32, k, nn, b,
-                                           stride, None, s)))
+            if from_norm:
+                plan.append(("status", L.lk_mmvq_multi, (wtype, len(ns), vx, qn.data_ptr(), dst, lib.TYPE_F32, k, nn, b, qn.shape[1],
+                                                          stride, None, s)))
+            else:
+                plan.append(("status", L.lk_mmvq_fused, (wtype, len(ns), vx, x.data_ptr(), x.stride(0), dst, lib.TYPE_F32, k, nn, b,
+                                                          stride, None, s)))
         elif matvec:
             q = torch.empty((b, ops.pad_to(k, 512) // 32, 36), dtype=torch.uint8, device=dev)
             keep.append(q)
@@ -657,7 +670,7 @@ def decode_1p7b(args, dev):
                               "the Q8_1 rows down reads, down, lm_head; a Q8_1 quantizer launch before the others" if fused_rows
                          else f"linears on the matrix-unit rows kernels: {used['rows']}, as mat-vec slices of eight rows: "
                               f"{used['matvec']}, on the tiled matmul: {used['tiled']}",
-                 "acts": "f32 rows into every group" if getattr(args, "acts", "f32") == "f32" or matvec
+                 "acts": "f32 rows into every group" if getattr(args, "acts", "f32") == "f32"
                          else "q + k + v and gate + up read Q8_1 rows as the model's RMSNorm launches that also quantize leave them "
                               "(those launches are not timed); o and lm_head from f32 rows",
                  "weight_bytes_per_step": total_bytes, "launches_per_step": len(plan), "hip_graph": True}, roofline,
